@@ -1,0 +1,29 @@
+// Internals shared by the translation units of libdali_hip.so.
+#ifndef DALI_HIP_RUNTIME_H
+#define DALI_HIP_RUNTIME_H
+
+#include <hip/hip_runtime.h>
+
+#include <string>
+
+#include "../../include/dali_hip.h"
+
+namespace dali_hip {
+
+// Workspace of the two-stage reductions: kWorkspaceCounters uint32 counters
+// (zero at creation, reset to zero by the block that consumes them) followed by
+// kWorkspacePartialBytes of partial results.
+constexpr int kWorkspaceCounters = 16384;
+constexpr size_t kWorkspaceCounterBytes = (size_t)kWorkspaceCounters * 4;
+constexpr size_t kWorkspacePartialBytes = (size_t)32 << 20;
+constexpr size_t kWorkspaceBytes = kWorkspaceCounterBytes + kWorkspacePartialBytes;
+
+int fail(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+int fail_str(const std::string& s);
+int ensure_init();
+hipStream_t stream();
+char* workspace();
+
+}  // namespace dali_hip
+
+#endif

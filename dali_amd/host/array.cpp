@@ -1,0 +1,837 @@
+// Array handles, buffer views, memory placement and the op:: factories.
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <numeric>
+
+#include "../../include/dali_hip.h"
+#include "expr.h"
+
+namespace dali {
+
+int size_of_dtype(DType dtype) { return dtype == DTYPE_DOUBLE ? 8 : 4; }
+
+std::string dtype_to_cpp_name(DType dtype) {
+    switch (dtype) {
+        case DTYPE_FLOAT: return "float";
+        case DTYPE_DOUBLE: return "double";
+        default: return "int";
+    }
+}
+
+std::string shape_str(const std::vector<int>& shape) {
+    std::ostringstream ss;
+    ss << "[";
+    for (size_t i = 0; i < shape.size(); ++i) ss << (i ? ", " : "") << shape[i];
+    ss << "]";
+    return ss.str();
+}
+
+void check_hip(int status, const char* what) {
+    if (status != 0) throw std::runtime_error(make_message(what, ": ", dali_hip_last_error()));
+}
+
+std::vector<int> contiguous_strides(const std::vector<int>& shape) {
+    std::vector<int> st(shape.size());
+    int64_t v = 1;
+    for (int i = (int)shape.size() - 1; i >= 0; --i) {
+        st[i] = (int)v;
+        v *= shape[i];
+    }
+    return st;
+}
+
+// ------------------------------------------------------------------ memory
+namespace memory {
+
+SynchronizedMemory::SynchronizedMemory(size_t bytes) : bytes_(bytes) {}
+
+SynchronizedMemory::~SynchronizedMemory() {
+    if (host_) std::free(host_);
+    // device blocks go back to the size-keyed bank, not to the driver
+    // (dali/array/memory/synchronized_memory.cpp:76-82)
+    if (device_) dali_hip_bank_deposit(device_, bytes_);
+}
+
+void SynchronizedMemory::lazy_clear() {
+    clear_on_allocation_ = true;
+    host_fresh_ = false;
+    device_fresh_ = false;
+    if (host_) {
+        std::memset(host_, 0, bytes_);
+        host_fresh_ = true;
+    }
+    if (device_) {
+        check_hip(dali_hip_memset_async(device_, 0, bytes_), "memory clear");
+        device_fresh_ = true;
+    }
+}
+
+void SynchronizedMemory::allocate(DeviceT device) {
+    if (device == DEVICE_T_CPU) {
+        if (host_) return;
+        size_t n = bytes_ ? bytes_ : 4;
+        if (posix_memalign(&host_, 64, n) != 0) throw std::runtime_error("host allocation failed");
+    } else {
+        if (device_) return;
+        check_hip(dali_hip_bank_allocate(&device_, bytes_), "device allocation");
+    }
+}
+
+void SynchronizedMemory::move_to(DeviceT device) {
+    bool& fresh = device == DEVICE_T_CPU ? host_fresh_ : device_fresh_;
+    if (fresh) return;
+    allocate(device);
+    bool other_fresh = device == DEVICE_T_CPU ? device_fresh_ : host_fresh_;
+    if (other_fresh) {
+        if (device == DEVICE_T_CPU)
+            check_hip(dali_hip_memcpy_d2h(host_, device_, bytes_), "copy to host");
+        else
+            check_hip(dali_hip_memcpy_h2d(device_, host_, bytes_), "copy to device");
+    } else if (clear_on_allocation_) {
+        if (device == DEVICE_T_CPU)
+            std::memset(host_, 0, bytes_);
+        else
+            check_hip(dali_hip_memset_async(device_, 0, bytes_), "memory clear");
+    }
+    fresh = true;
+}
+
+const void* SynchronizedMemory::readonly_data(DeviceT device) {
+    move_to(device);
+    return device == DEVICE_T_CPU ? host_ : device_;
+}
+
+void* SynchronizedMemory::mutable_data(DeviceT device) {
+    move_to(device);
+    host_fresh_ = device == DEVICE_T_CPU;
+    device_fresh_ = device == DEVICE_T_GPU;
+    return device == DEVICE_T_CPU ? host_ : device_;
+}
+
+void* SynchronizedMemory::overwrite_data(DeviceT device) {
+    allocate(device);
+    host_fresh_ = device == DEVICE_T_CPU;
+    device_fresh_ = device == DEVICE_T_GPU;
+    return device == DEVICE_T_CPU ? host_ : device_;
+}
+
+void* SynchronizedMemory::data(DeviceT device, AM mode) {
+    switch (mode) {
+        case AM_READONLY: return const_cast<void*>(readonly_data(device));
+        case AM_MUTABLE: return mutable_data(device);
+        default: return overwrite_data(device);
+    }
+}
+}  // namespace memory
+
+// ------------------------------------------------------------------- Array
+static std::shared_ptr<Expr> make_buffer(const std::vector<int>& shape, DType dtype) {
+    for (int s : shape) DALI_ASSERT(s >= 0, make_message("negative dimension in shape ", shape_str(shape)));
+    auto e = std::make_shared<Expr>();
+    e->kind = Kind::BUFFER;
+    e->dtype = dtype;
+    e->shape = shape;
+    int64_t n = 1;
+    for (int s : shape) n *= s;
+    DALI_ASSERT(n < ((int64_t)1 << 31), make_message("array of shape ", shape_str(shape), " has too many elements"));
+    e->memory = std::make_shared<memory::SynchronizedMemory>((size_t)n * size_of_dtype(dtype));
+    return e;
+}
+
+Array::Array() : state_(nullptr) {}
+Array::Array(std::shared_ptr<Expr> expr) : state_(std::make_shared<ArrayState>()) { state_->expr = std::move(expr); }
+Array::Array(const std::vector<int>& shape, DType dtype) : Array(make_buffer(shape, dtype)) {}
+
+static std::shared_ptr<Expr> make_scalar(DType dtype, double d, int i) {
+    auto e = std::make_shared<Expr>();
+    e->kind = Kind::SCALAR;
+    e->dtype = dtype;
+    e->dvalue = d;
+    e->ivalue = i;
+    return e;
+}
+Array::Array(double scalar) : Array(make_scalar(DTYPE_DOUBLE, scalar, (int)scalar)) {}
+Array::Array(float scalar) : Array(make_scalar(DTYPE_FLOAT, scalar, (int)scalar)) {}
+Array::Array(int scalar) : Array(make_scalar(DTYPE_INT32, scalar, scalar)) {}
+
+Array Array::zeros(const std::vector<int>& shape, DType dtype) {
+    Array a(shape, dtype);
+    a.state_->expr->memory->lazy_clear();
+    return a;
+}
+
+Array Array::from_host(const void* data, const std::vector<int>& shape, DType dtype) {
+    Array a(shape, dtype);
+    auto& mem = a.state_->expr->memory;
+    void* dst = mem->overwrite_data(memory::DEVICE_T_CPU);
+    std::memcpy(dst, data, mem->bytes());
+    return a;
+}
+
+template <typename T>
+static Array filled(const std::vector<int>& shape, DType dtype, bool ramp) {
+    Array a(shape, dtype);
+    auto& mem = a.state_->expr->memory;
+    T* dst = (T*)mem->overwrite_data(memory::DEVICE_T_CPU);
+    size_t n = mem->bytes() / sizeof(T);
+    for (size_t i = 0; i < n; ++i) dst[i] = ramp ? (T)i : (T)1;
+    return a;
+}
+
+Array Array::ones(const std::vector<int>& shape, DType dtype) {
+    if (dtype == DTYPE_FLOAT) return filled<float>(shape, dtype, false);
+    if (dtype == DTYPE_DOUBLE) return filled<double>(shape, dtype, false);
+    return filled<int>(shape, dtype, false);
+}
+
+Array Array::arange(int n, DType dtype) {
+    if (dtype == DTYPE_FLOAT) return filled<float>({n}, dtype, true);
+    if (dtype == DTYPE_DOUBLE) return filled<double>({n}, dtype, true);
+    return filled<int>({n}, dtype, true);
+}
+
+bool Array::is_stateless() const { return !state_ || !state_->expr; }
+std::shared_ptr<Expr> Array::expression() const {
+    DALI_ASSERT(!is_stateless(), "operation on a stateless Array");
+    return state_->expr;
+}
+bool Array::is_buffer() const { return expression()->kind == Kind::BUFFER; }
+bool Array::is_scalar() const { return expression()->shape.empty(); }
+const std::vector<int>& Array::shape() const { return expression()->shape; }
+int Array::ndim() const { return (int)expression()->shape.size(); }
+DType Array::dtype() const { return expression()->dtype; }
+int Array::number_of_elements() const { return expression()->numel(); }
+const std::vector<int>& Array::strides() const { return expression()->strides; }
+std::vector<int> Array::normalized_strides() const {
+    auto e = expression();
+    return e->strides.empty() ? contiguous_strides(e->shape) : e->strides;
+}
+int Array::offset() const { return expression()->offset; }
+
+bool Array::contiguous_memory() const {
+    auto e = expression();
+    if (e->kind != Kind::BUFFER) return true;
+    if (e->strides.empty()) return true;
+    auto c = contiguous_strides(e->shape);
+    for (size_t i = 0; i < c.size(); ++i)
+        if (e->shape[i] != 1 && e->strides[i] != c[i]) return false;
+    return true;
+}
+
+void Array::eval() const {
+    if (is_buffer() || expression()->kind == Kind::SCALAR) return;
+    evaluate({*this});
+}
+
+void Array::eval_together(const std::vector<Array>& roots) { evaluate(roots); }
+
+static Array buffer_view(const std::shared_ptr<Expr>& base, const std::vector<int>& shape,
+                         const std::vector<int>& strides, int offset) {
+    auto e = std::make_shared<Expr>();
+    e->kind = Kind::BUFFER;
+    e->dtype = base->dtype;
+    e->memory = base->memory;
+    e->shape = shape;
+    e->offset = offset;
+    // store no strides when the view is contiguous (the reference's convention,
+    // dali/array/expression/buffer.cpp:112-175)
+    auto c = contiguous_strides(shape);
+    bool contiguous = true;
+    for (size_t i = 0; i < shape.size(); ++i)
+        if (shape[i] != 1 && strides[i] != c[i]) contiguous = false;
+    if (!contiguous) e->strides = strides;
+    return Array(e);
+}
+
+// a scalar literal viewed as a buffer is materialised first
+static const Array& as_buffer(const Array& a) {
+    if (a.expression()->kind == Kind::SCALAR) {
+        auto e = a.expression();
+        Array b({}, e->dtype);
+        void* p = b.expression()->memory->overwrite_data(memory::DEVICE_T_CPU);
+        if (e->dtype == DTYPE_FLOAT) *(float*)p = (float)e->dvalue;
+        else if (e->dtype == DTYPE_DOUBLE) *(double*)p = e->dvalue;
+        else *(int*)p = e->ivalue;
+        a.state_->expr = b.expression();
+        return a;
+    }
+    a.eval();
+    return a;
+}
+
+Array Array::transpose() const {
+    std::vector<int> axes(ndim());
+    for (int i = 0; i < ndim(); ++i) axes[i] = ndim() - 1 - i;
+    return transpose(axes);
+}
+
+Array Array::transpose(const std::vector<int>& axes) const {
+    DALI_ASSERT((int)axes.size() == ndim(), make_message("transpose needs ", ndim(), " axes (got ", axes.size(), ")."));
+    auto e = as_buffer(*this).expression();
+    auto st = normalized_strides();
+    std::vector<int> nshape(ndim()), nstrides(ndim());
+    std::vector<bool> seen(ndim(), false);
+    for (int i = 0; i < ndim(); ++i) {
+        int ax = axes[i] < 0 ? axes[i] + ndim() : axes[i];
+        DALI_ASSERT(ax >= 0 && ax < ndim() && !seen[ax], "transpose axes must be a permutation");
+        seen[ax] = true;
+        nshape[i] = e->shape[ax];
+        nstrides[i] = st[ax];
+    }
+    return buffer_view(e, nshape, nstrides, e->offset);
+}
+
+Array Array::swapaxes(int a, int b) const {
+    std::vector<int> axes(ndim());
+    std::iota(axes.begin(), axes.end(), 0);
+    if (a < 0) a += ndim();
+    if (b < 0) b += ndim();
+    DALI_ASSERT(a >= 0 && a < ndim() && b >= 0 && b < ndim(), "swapaxes axis out of range");
+    std::swap(axes[a], axes[b]);
+    return transpose(axes);
+}
+
+Array Array::pluck_axis(int axis, int idx) const {
+    if (axis < 0) axis += ndim();
+    DALI_ASSERT(axis >= 0 && axis < ndim(), make_message("pluck_axis axis ", axis, " out of range for ndim ", ndim()));
+    auto e = as_buffer(*this).expression();
+    if (idx < 0) idx += e->shape[axis];
+    DALI_ASSERT(idx >= 0 && idx < e->shape[axis], make_message("index ", idx, " out of range for axis of size ", e->shape[axis]));
+    auto st = normalized_strides();
+    std::vector<int> nshape, nstrides;
+    for (int i = 0; i < ndim(); ++i)
+        if (i != axis) {
+            nshape.push_back(e->shape[i]);
+            nstrides.push_back(st[i]);
+        }
+    return buffer_view(e, nshape, nstrides, e->offset + idx * st[axis]);
+}
+
+Array Array::slice(int axis, int start, int end, int step) const {
+    if (axis < 0) axis += ndim();
+    DALI_ASSERT(axis >= 0 && axis < ndim(), make_message("slice axis ", axis, " out of range for ndim ", ndim()));
+    DALI_ASSERT(step > 0, "slice step must be positive");
+    auto e = as_buffer(*this).expression();
+    int n = e->shape[axis];
+    if (start < 0) start += n;
+    if (end < 0) end += n;
+    DALI_ASSERT(start >= 0 && start <= n && end >= start && end <= n,
+                make_message("slice [", start, ":", end, "] out of range for axis of size ", n));
+    auto st = normalized_strides();
+    std::vector<int> nshape = e->shape, nstrides = st;
+    nshape[axis] = (end - start + step - 1) / step;
+    nstrides[axis] = st[axis] * step;
+    return buffer_view(e, nshape, nstrides, e->offset + start * st[axis]);
+}
+
+Array Array::ascontiguousarray() const {
+    const Array& self = as_buffer(*this);
+    if (self.contiguous_memory()) return self;
+    Array out(shape(), dtype());
+    evaluate_into(out, OPERATOR_T_EQL, op::identity(self));
+    return out;
+}
+
+Array Array::reshape(const std::vector<int>& new_shape) const {
+    std::vector<int> ns = new_shape;
+    int64_t known = 1;
+    int unknown = -1;
+    for (size_t i = 0; i < ns.size(); ++i) {
+        if (ns[i] == -1) {
+            DALI_ASSERT(unknown < 0, "reshape accepts at most one -1");
+            unknown = (int)i;
+        } else {
+            known *= ns[i];
+        }
+    }
+    if (unknown >= 0) ns[unknown] = known ? (int)(number_of_elements() / known) : 0;
+    int64_t total = 1;
+    for (int s : ns) total *= s;
+    DALI_ASSERT(total == number_of_elements(), make_message("cannot reshape ", shape_str(shape()), " into ", shape_str(new_shape)));
+    Array src = as_buffer(*this).contiguous_memory() ? *this : ascontiguousarray();
+    auto e = src.expression();
+    return buffer_view(e, ns, contiguous_strides(ns), e->offset);
+}
+
+Array Array::expand_dims(int axis) const {
+    if (axis < 0) axis += ndim() + 1;
+    DALI_ASSERT(axis >= 0 && axis <= ndim(), make_message("expand_dims axis ", axis, " out of range for ndim ", ndim()));
+    auto e = expression();
+    if (e->kind == Kind::BUFFER) {
+        auto st = normalized_strides();
+        std::vector<int> nshape = e->shape, nstrides = st;
+        nshape.insert(nshape.begin() + axis, 1);
+        nstrides.insert(nstrides.begin() + axis, 0);
+        return buffer_view(e, nshape, nstrides, e->offset);
+    }
+    auto n = std::make_shared<Expr>();
+    n->kind = Kind::EXPAND_DIMS;
+    n->dtype = e->dtype;
+    n->shape = e->shape;
+    n->shape.insert(n->shape.begin() + axis, 1);
+    n->axis = axis;
+    n->args = {*this};
+    return Array(n);
+}
+
+Array Array::squeeze(int axis) const {
+    if (axis < 0) axis += ndim();
+    DALI_ASSERT(axis >= 0 && axis < ndim() && shape()[axis] == 1,
+                make_message("squeeze axis ", axis, " must have size 1 in shape ", shape_str(shape())));
+    return pluck_axis(axis, 0);
+}
+
+void* Array::device_ptr(memory::AM mode) const {
+    auto e = as_buffer(*this).expression();
+    char* base = (char*)e->memory->data(memory::DEVICE_T_GPU, mode);
+    return base + (size_t)e->offset * size_of_dtype(e->dtype);
+}
+
+void Array::to_host(void* out) const {
+    auto e = as_buffer(*this).expression();
+    const char* src = (const char*)e->memory->readonly_data(memory::DEVICE_T_CPU);
+    int es = size_of_dtype(e->dtype);
+    int n = e->numel();
+    if (n == 0) return;
+    if (contiguous_memory()) {
+        std::memcpy(out, src + (size_t)e->offset * es, (size_t)n * es);
+        return;
+    }
+    auto st = normalized_strides();
+    int nd = ndim();
+    std::vector<int> idx(nd, 0);
+    char* dst = (char*)out;
+    for (int i = 0; i < n; ++i) {
+        int64_t off = e->offset;
+        for (int d = 0; d < nd; ++d) off += (int64_t)idx[d] * st[d];
+        std::memcpy(dst + (size_t)i * es, src + off * es, es);
+        for (int d = nd - 1; d >= 0; --d) {
+            if (++idx[d] < e->shape[d]) break;
+            idx[d] = 0;
+        }
+    }
+}
+
+double Array::scalar_value() const {
+    auto e = expression();
+    if (e->kind == Kind::SCALAR) return e->dtype == DTYPE_INT32 ? (double)e->ivalue : e->dvalue;
+    DALI_ASSERT(number_of_elements() >= 1, "scalar_value of an empty array");
+    auto b = as_buffer(*this).expression();
+    const char* src = (const char*)b->memory->readonly_data(memory::DEVICE_T_CPU) + (size_t)b->offset * size_of_dtype(b->dtype);
+    if (b->dtype == DTYPE_FLOAT) return *(const float*)src;
+    if (b->dtype == DTYPE_DOUBLE) return *(const double*)src;
+    return *(const int*)src;
+}
+
+Array& Array::assign(const Array& other) {
+    if (is_stateless()) {
+        other.eval();
+        state_ = std::make_shared<ArrayState>();
+        state_->expr = other.expression();
+        return *this;
+    }
+    evaluate_into(*this, OPERATOR_T_EQL, other);
+    return *this;
+}
+Array& Array::operator+=(const Array& other) { evaluate_into(*this, OPERATOR_T_ADD, other); return *this; }
+Array& Array::operator-=(const Array& other) { evaluate_into(*this, OPERATOR_T_SUB, other); return *this; }
+Array& Array::operator*=(const Array& other) { evaluate_into(*this, OPERATOR_T_MUL, other); return *this; }
+Array& Array::operator/=(const Array& other) { evaluate_into(*this, OPERATOR_T_DIV, other); return *this; }
+
+Array Array::sum() const { return op::sum(*this); }
+Array Array::sum(const std::vector<int>& axes, bool keepdims) const { return op::sum(*this, axes, keepdims); }
+Array Array::max() const { return op::max(*this); }
+Array Array::max(const std::vector<int>& axes, bool keepdims) const { return op::max(*this, axes, keepdims); }
+Array Array::min() const { return op::min(*this); }
+Array Array::min(const std::vector<int>& axes, bool keepdims) const { return op::min(*this, axes, keepdims); }
+Array Array::mean() const { return op::mean(*this); }
+Array Array::mean(const std::vector<int>& axes, bool keepdims) const { return op::mean(*this, axes, keepdims); }
+Array Array::argmax() const { return op::argmax(*this); }
+Array Array::argmax(int axis) const { return op::argmax(*this, axis); }
+Array Array::argmin() const { return op::argmin(*this); }
+Array Array::argmin(int axis) const { return op::argmin(*this, axis); }
+Array Array::exp() const { return op::exp(*this); }
+Array Array::log() const { return op::log(*this); }
+Array Array::tanh() const { return op::tanh(*this); }
+Array Array::sigmoid() const { return op::sigmoid(*this); }
+Array Array::square() const { return op::square(*this); }
+Array Array::dot(const Array& other) const { return op::dot(*this, other); }
+
+Array operator+(const Array& a, const Array& b) { return op::add(a, b); }
+Array operator-(const Array& a, const Array& b) { return op::subtract(a, b); }
+Array operator*(const Array& a, const Array& b) { return op::eltmul(a, b); }
+Array operator/(const Array& a, const Array& b) { return op::eltdiv(a, b); }
+Array operator-(const Array& a) { return op::negate(a); }
+
+// --------------------------------------------------------------------- op::
+namespace op {
+
+static Array make_node(Kind kind, const std::string& name, std::vector<Array> args, const std::vector<int>& shape,
+                       DType dtype) {
+    auto e = std::make_shared<Expr>();
+    e->kind = kind;
+    e->name = name;
+    e->args = std::move(args);
+    e->shape = shape;
+    e->dtype = dtype;
+    return Array(e);
+}
+
+// dali/array/array.cpp:845-865
+static DType type_promotion(const Array& a, const Array& b) {
+    bool as = a.is_scalar(), bs = b.is_scalar();
+    if (as == bs) {
+        if (a.dtype() == DTYPE_DOUBLE || b.dtype() == DTYPE_DOUBLE) return DTYPE_DOUBLE;
+        if (a.dtype() == DTYPE_FLOAT || b.dtype() == DTYPE_FLOAT) return DTYPE_FLOAT;
+        return DTYPE_INT32;
+    }
+    return as ? b.dtype() : a.dtype();
+}
+
+// dali/array/jit/jit_utils.cpp:107-147
+static std::vector<int> common_shape(const Array& a, const Array& b) {
+    const auto& sa = a.shape();
+    const auto& sb = b.shape();
+    if (sa.empty()) return sb;
+    if (sb.empty()) return sa;
+    DALI_ASSERT(sa.size() == sb.size(), "inputs must be scalars or have the same dimensionality.");
+    std::vector<int> out = sa;
+    for (size_t d = 0; d < sa.size(); ++d) {
+        DALI_ASSERT(sa[d] == sb[d] || sa[d] == 1 || sb[d] == 1,
+                    make_message("Could not find a common shape between ", shape_str(sa), " and ", shape_str(sb), "."));
+        if (sb[d] != 1) out[d] = sb[d];
+    }
+    return out;
+}
+
+static Array broadcasted_reshape(const Array& a, const std::vector<int>& shape) {
+    if (a.shape() == shape) return a;
+    return make_node(Kind::BROADCAST, "", {a}, shape, a.dtype());
+}
+
+Array unsafe_cast(Array a, DType dtype) {
+    if (a.dtype() == dtype) return a;
+    auto e = a.expression();
+    if (e->kind == Kind::SCALAR) {
+        // literal: convert on the host
+        if (dtype == DTYPE_INT32) return Array((int)(e->dtype == DTYPE_INT32 ? e->ivalue : e->dvalue));
+        double v = e->dtype == DTYPE_INT32 ? (double)e->ivalue : e->dvalue;
+        if (dtype == DTYPE_FLOAT) return Array((float)v);
+        return Array(v);
+    }
+    return make_node(Kind::ELEMENTWISE, "functor::cast", {a}, a.shape(), dtype);
+}
+
+Array round(Array a) {
+    if (a.dtype() == DTYPE_INT32) return a;
+    auto e = a.expression();
+    if (e->kind == Kind::SCALAR) return Array((int)std::floor(e->dvalue + 0.5));
+    return make_node(Kind::ELEMENTWISE, "functor::round", {a}, a.shape(), DTYPE_INT32);
+}
+
+// dali/array/op/elementwise_operation.cpp:137-139
+Array astype(Array a, DType dtype) { return dtype == DTYPE_INT32 ? round(a) : unsafe_cast(a, dtype); }
+
+Array elementwise(Array a, const std::string& functor_name) {
+    return make_node(Kind::ELEMENTWISE, functor_name, {a}, a.shape(), a.dtype());
+}
+
+// dali/array/op/elementwise_operation.cpp:130-135,162-186
+Array elementwise(Array a, Array b, const std::string& functor_name) {
+    DALI_ASSERT(a.ndim() == b.ndim() || a.is_scalar() || b.is_scalar(),
+                make_message("Arguments to binary operation '", functor_name, "' must have the same rank (got left.ndim = ",
+                             a.ndim(), ", left.shape = ", shape_str(a.shape()), ", and right.ndim = ", b.ndim(),
+                             ", right.shape = ", shape_str(b.shape()), ")."));
+    if (a.dtype() != b.dtype()) {
+        DType t = type_promotion(a, b);
+        a = astype(a, t);
+        b = astype(b, t);
+    }
+    std::vector<int> shape = common_shape(a, b);
+    if (!a.is_scalar()) a = broadcasted_reshape(a, shape);
+    if (!b.is_scalar()) b = broadcasted_reshape(b, shape);
+    return make_node(Kind::ELEMENTWISE, functor_name, {a, b}, shape, a.dtype());
+}
+
+Array add(const Array& a, const Array& b) { return elementwise(a, b, "functor::add"); }
+Array subtract(const Array& a, const Array& b) { return elementwise(a, b, "functor::subtract"); }
+Array eltmul(const Array& a, const Array& b) { return elementwise(a, b, "functor::eltmul"); }
+Array eltdiv(const Array& a, const Array& b) { return elementwise(a, b, "functor::eltdiv"); }
+Array pow(const Array& a, const Array& b) { return elementwise(a, b, "functor::power"); }
+Array equals(const Array& a, const Array& b) { return elementwise(a, b, "functor::equals"); }
+Array prelu(const Array& x, const Array& w) { return elementwise(x, w, "functor::prelu"); }
+Array clip(const Array& x, const Array& c) { return elementwise(x, c, "functor::clip"); }
+Array identity(const Array& x) { return elementwise(x, "functor::identity"); }
+Array sigmoid(const Array& x) { return elementwise(x, "functor::sigmoid"); }
+Array tanh(const Array& x) { return elementwise(x, "functor::tanh"); }
+Array exp(const Array& x) { return elementwise(x, "functor::exp"); }
+Array log(const Array& x) { return elementwise(x, "functor::log"); }
+Array softplus(const Array& x) { return elementwise(x, "functor::softplus"); }
+Array relu(const Array& x) { return elementwise(x, "functor::relu"); }
+Array abs(const Array& x) { return elementwise(x, "functor::abs"); }
+Array sign(const Array& x) { return elementwise(x, "functor::sign"); }
+Array square(const Array& x) { return elementwise(x, "functor::square"); }
+Array cube(const Array& x) { return elementwise(x, "functor::cube"); }
+Array sqrt(const Array& x) { return elementwise(x, "functor::sqrt_f"); }
+Array rsqrt(const Array& x) { return elementwise(x, "functor::rsqrt"); }
+Array eltinv(const Array& x) { return elementwise(x, "functor::inv"); }
+Array negate(const Array& x) { return eltmul(Array(-1), x); }
+Array isnan(const Array& x) { return elementwise(x, "functor::isnotanumber"); }
+Array isinf(const Array& x) { return elementwise(x, "functor::isinfinity"); }
+Array dsigmoid(const Array& x) { return elementwise(x, "functor::dsigmoid"); }
+Array dtanh(const Array& x) { return elementwise(x, "functor::dtanh"); }
+
+Array all_reduce(const Array& a, const std::string& reducer_name) {
+    return make_node(Kind::ALL_REDUCE, reducer_name, {a}, {}, a.dtype());
+}
+
+static Array axis_reduce_last(const Array& a, const std::string& reducer_name) {
+    std::vector<int> shape(a.shape().begin(), a.shape().end() - 1);
+    return make_node(Kind::AXIS_REDUCE, reducer_name, {a}, shape, a.dtype());
+}
+
+// true when buffer axis `axis` and `axis - 1` can be merged into one
+// (dali/array/array.cpp is_axis_collapsible_with_axis_minus_one)
+static bool collapsible_with_axis_minus_one(const Array& a, int axis) {
+    if (!a.is_buffer()) return false;
+    auto st = a.normalized_strides();
+    return st[axis - 1] == st[axis] * a.shape()[axis];
+}
+
+static Array collapse_axis_with_axis_minus_one(const Array& a, int axis) {
+    auto e = a.expression();
+    auto st = a.normalized_strides();
+    std::vector<int> nshape = e->shape, nstrides = st;
+    nshape[axis - 1] *= nshape[axis];
+    nstrides[axis - 1] = st[axis];
+    nshape.erase(nshape.begin() + axis);
+    nstrides.erase(nstrides.begin() + axis);
+    return buffer_view(e, nshape, nstrides, e->offset);
+}
+
+// dali/array/op/reducer_operation.cpp:595-679
+Array axis_reduce(const Array& a, const std::string& reducer_name, const std::vector<int>& axes, bool keepdims) {
+    if (axes.empty()) return a;
+    int ndim = a.ndim();
+    if (ndim == 0) return a;
+    std::vector<int> norm(axes);
+    for (auto& ax : norm) {
+        if (ax < 0) ax += ndim;
+        DALI_ASSERT(ax >= 0 && ax < ndim,
+                    make_message("Reduction axis must strictly positive and less than the number of dimensions of the input (got axis=",
+                                 axes[0], ", ndim=", ndim, ", input.shape = ", shape_str(a.shape()), ")."));
+    }
+    std::vector<bool> reduced(ndim, false);
+    std::sort(norm.begin(), norm.end());
+    for (int ax : norm) {
+        DALI_ASSERT(!reduced[ax], make_message("axis_reduce received duplicate axes to operate on (axis=", ax, ")."));
+        reduced[ax] = true;
+    }
+    if ((int)norm.size() == ndim) return all_reduce(a, reducer_name);
+    int num_low = 0;
+    for (int i = ndim - 1; i >= 0 && reduced[i]; --i) ++num_low;
+    Array res = a;
+    if (num_low != (int)norm.size()) {
+        std::vector<int> order;
+        for (int i = 0; i < ndim; ++i)
+            if (!reduced[i]) order.push_back(i);
+        for (int i = 0; i < ndim; ++i)
+            if (reduced[i]) order.push_back(i);
+        res = res.transpose(order);
+    }
+    int to_reduce = (int)norm.size();
+    int collapsed_ndim = ndim - 1;
+    for (int used = 0; used < to_reduce; ++used) {
+        if (to_reduce - used == 1 || !collapsible_with_axis_minus_one(res, collapsed_ndim)) {
+            res = axis_reduce_last(res, reducer_name);
+        } else {
+            res = collapse_axis_with_axis_minus_one(res, collapsed_ndim);
+        }
+        --collapsed_ndim;
+    }
+    if (keepdims)
+        for (int ax : norm) res = res.expand_dims(ax);
+    return res;
+}
+
+// The reference stores a flat argmax in the INPUT dtype
+// (dali/array/op/reducer_operation.cpp:681-684).
+Array argument_all_reduce(const Array& a, const std::string& reducer_name) {
+    return make_node(Kind::ARG_ALL_REDUCE, reducer_name, {a}, {}, a.dtype());
+}
+
+// dali/array/op/reducer_operation.cpp:686-710
+Array argument_axis_reduce(const Array& a, const std::string& reducer_name, int axis) {
+    int ndim = a.ndim();
+    if (ndim == 0) return Array(0);
+    if (axis < 0) axis += ndim;
+    DALI_ASSERT(axis >= 0 && axis < ndim,
+                make_message("Reduction axis must strictly positive and less than the number of dimensions of the input (got axis=",
+                             axis, ", ndim=", ndim, ")."));
+    if (ndim == 1) return argument_all_reduce(a, reducer_name);
+    Array res = a;
+    if (axis != ndim - 1) res = res.swapaxes(axis, ndim - 1);
+    std::vector<int> shape(res.shape().begin(), res.shape().end() - 1);
+    return make_node(Kind::ARG_AXIS_REDUCE, reducer_name, {res}, shape, DTYPE_INT32);
+}
+
+Array sum(const Array& x) { return all_reduce(x, "reducers::sum"); }
+Array sum(const Array& x, const std::vector<int>& axes, bool keepdims) { return axis_reduce(x, "reducers::sum", axes, keepdims); }
+Array prod(const Array& x) { return all_reduce(x, "reducers::product"); }
+Array prod(const Array& x, const std::vector<int>& axes, bool keepdims) { return axis_reduce(x, "reducers::product", axes, keepdims); }
+Array max(const Array& x) { return all_reduce(x, "reducers::maximum"); }
+Array max(const Array& x, const std::vector<int>& axes, bool keepdims) { return axis_reduce(x, "reducers::maximum", axes, keepdims); }
+Array min(const Array& x) { return all_reduce(x, "reducers::minimum"); }
+Array min(const Array& x, const std::vector<int>& axes, bool keepdims) { return axis_reduce(x, "reducers::minimum", axes, keepdims); }
+
+// dali/array/op/reducers.cpp:32-41
+Array mean(const Array& x) {
+    Array s = all_reduce(x, "reducers::sum");
+    if (s.dtype() == DTYPE_INT32) s = astype(s, DTYPE_DOUBLE);
+    return eltdiv(s, Array(x.number_of_elements()));
+}
+Array mean(const Array& x, const std::vector<int>& axes, bool keepdims) {
+    Array s = axis_reduce(x, "reducers::sum", axes, keepdims);
+    if (s.dtype() == DTYPE_INT32) s = astype(s, DTYPE_DOUBLE);
+    int n = s.number_of_elements();
+    return eltdiv(s, Array(n ? x.number_of_elements() / n : 0));
+}
+Array L2_norm(const Array& x) {
+    Array s = all_reduce(square(x), "reducers::sum");
+    if (s.dtype() == DTYPE_INT32) s = astype(s, DTYPE_DOUBLE);
+    return sqrt(s);
+}
+Array L2_norm(const Array& x, const std::vector<int>& axes, bool keepdims) {
+    Array s = axis_reduce(square(x), "reducers::sum", axes, keepdims);
+    if (s.dtype() == DTYPE_INT32) s = astype(s, DTYPE_DOUBLE);
+    return sqrt(s);
+}
+Array argmax(const Array& x) { return argument_all_reduce(x, "reducers::maximum"); }
+Array argmax(const Array& x, int axis) { return argument_axis_reduce(x, "reducers::maximum", axis); }
+Array argmin(const Array& x) { return argument_all_reduce(x, "reducers::minimum"); }
+Array argmin(const Array& x, int axis) { return argument_axis_reduce(x, "reducers::minimum", axis); }
+
+// dali/array/op/softmax.cpp:5-8
+Array softmax(const Array& logits, int axis) {
+    Array exped = exp(subtract(logits, max(logits, {axis}, true)));
+    return eltdiv(exped, sum(exped, {axis}, true));
+}
+
+// dali/array/op/gather_from_rows.cpp:110-127
+Array gather_from_rows(const Array& source, const Array& indices) {
+    DALI_ASSERT(source.ndim() > 1, make_message("gather must be called on source with ndim >= 2 (got ndim=", source.ndim(), ")."));
+    DALI_ASSERT(indices.dtype() == DTYPE_INT32, "indices must be integers.");
+    DALI_ASSERT(indices.ndim() <= 1, make_message("indices must have rank 1 or lower (got indices.ndim=", indices.ndim(), ")."));
+    DALI_ASSERT(source.ndim() == 2, "gather_from_rows: only 2-D sources are implemented");
+    if (indices.ndim() == 1) {
+        DALI_ASSERT(indices.shape()[0] <= source.shape()[0] || indices.shape()[0] == 1 || source.shape()[0] == 1,
+                    make_message("dimension 1 of indices must be less than or equal to first dimension of source (got indices.shape[0]=",
+                                 indices.shape()[0], ", source.shape[0]=", source.shape()[0], ")"));
+    }
+    std::vector<int> shape = indices.ndim() ? indices.shape() : std::vector<int>{1};
+    return make_node(Kind::GATHER_FROM_ROWS, "", {source, indices}, shape, source.dtype());
+}
+
+// dali/array/op/one_hot.cpp:62-74
+Array one_hot(Array indices, int depth, Array on_value, Array off_value) {
+    DALI_ASSERT(indices.dtype() == DTYPE_INT32, "indices must be integers.");
+    DALI_ASSERT(on_value.is_scalar(), make_message("on_value must be a scalar (got on_value.ndim=", on_value.ndim(), ")."));
+    DALI_ASSERT(off_value.is_scalar(), make_message("off_value must be a scalar (got off_value.ndim=", off_value.ndim(), ")."));
+    DALI_ASSERT(depth > 0, make_message("depth must be strictly positive (got depth=", depth, ")."));
+    if (on_value.dtype() != off_value.dtype()) {
+        DType t = type_promotion(on_value, off_value);
+        on_value = astype(on_value, t);
+        off_value = astype(off_value, t);
+    }
+    std::vector<int> shape = indices.shape();
+    shape.push_back(depth);
+    auto out = make_node(Kind::ONE_HOT, "", {on_value, off_value, indices}, shape, on_value.dtype());
+    out.expression()->depth = depth;
+    return out;
+}
+
+// dali/array/op/dot.cpp:49-67
+Array matmul(Array a, Array b) {
+    DALI_ASSERT(a.ndim() == 2 && b.ndim() == 2,
+                make_message("matmul inputs must be both be 2-dimensional, but got a.ndim = ", a.ndim(), " and b.ndim = ", b.ndim(), "."));
+    DALI_ASSERT(a.shape()[1] == b.shape()[0] || a.shape()[1] == 1 || b.shape()[0] == 1,
+                make_message("matmul shapes not aligned, with a.shape = ", shape_str(a.shape()), " and b.shape = ", shape_str(b.shape()),
+                             ": expected a.shape[1] = ", a.shape()[1], " to equal b.shape[0] = ", b.shape()[0], ", or for either to equal 1."));
+    if (a.shape()[1] != b.shape()[0]) {
+        if (a.shape()[1] == 1)
+            a = broadcasted_reshape(a, {a.shape()[0], b.shape()[0]});
+        else
+            b = broadcasted_reshape(b, {a.shape()[1], b.shape()[1]});
+    }
+    DType t = type_promotion(a, b);
+    if (a.dtype() != t) a = astype(a, t);
+    if (b.dtype() != t) b = astype(b, t);
+    return make_node(Kind::MATMUL, "", {a, b}, {a.shape()[0], b.shape()[1]}, t);
+}
+
+// dali/array/op/dot.cpp:104-124 (tensordot of rank > 2 operands is not part of this path)
+Array dot(const Array& a, const Array& b) {
+    int an = a.ndim(), bn = b.ndim();
+    if (an == 0 || bn == 0) return eltmul(a, b);
+    DALI_ASSERT(an <= 2 && bn <= 2, "dot: operands of rank > 2 (tensordot) are not implemented");
+    if (an == 1 && bn == 1) {
+        DALI_ASSERT(a.shape()[0] == b.shape()[0], make_message("inner input shapes a.shape = ", shape_str(a.shape()),
+                                                               " and b.shape = ", shape_str(b.shape()), " should be equal."));
+        return matmul(a.reshape({1, a.number_of_elements()}), b.reshape({b.number_of_elements(), 1})).reshape({});
+    }
+    if (an == 2 && bn == 2) return matmul(a, b);
+    if (an == 1) {
+        DALI_ASSERT(b.shape()[0] == a.shape()[0], make_message("matrix_vector_dot shape mistmach between a.shape = ", shape_str(a.shape()),
+                                                               " and b.shape = ", shape_str(b.shape()), "."));
+        return matmul(a.reshape({1, a.number_of_elements()}), b).reshape({b.shape()[1]});
+    }
+    DALI_ASSERT(a.shape()[1] == b.shape()[0], make_message("matrix_vector_dot shape mistmach between a.shape = ", shape_str(a.shape()),
+                                                           " and b.shape = ", shape_str(b.shape()), "."));
+    return matmul(a, b.reshape({b.number_of_elements(), 1})).reshape({a.shape()[0]});
+}
+
+CrossEntropyResult softmax_cross_entropy(const Array& logits, const Array& targets) {
+    DALI_ASSERT(logits.ndim() == 2, "softmax_cross_entropy expects 2-D logits");
+    DALI_ASSERT(targets.ndim() == 1 && targets.dtype() == DTYPE_INT32 && targets.shape()[0] == logits.shape()[0],
+                "softmax_cross_entropy expects one int32 target per row");
+    int rows = logits.shape()[0], cols = logits.shape()[1];
+    Array m = max(logits, {-1}, true);
+    Array exped = exp(subtract(logits, m));
+    Array s = sum(exped, {-1}, true);
+    Array grad = subtract(eltdiv(exped, s), one_hot(targets, cols, Array(1.0f), Array(0.0f)));
+    // lse = log(s) + m, shape [rows, 1]; row loss = lse - logits[i, t_i]
+    Array lse = add(log(s), m);
+    Array picked = gather_from_rows(logits, targets).expand_dims(1);
+    Array row_loss = subtract(lse, picked);
+    Array::eval_together({grad, row_loss});
+    Array rows1d = row_loss.reshape({rows});
+    Array mean_loss = mean(rows1d);
+    mean_loss.eval();
+    return {mean_loss, rows1d, grad};
+}
+
+LSTMState lstm_step(const Array& x, const Array& h, const Array& c, const Array& W, const Array& U, const Array& b) {
+    DALI_ASSERT(x.ndim() == 2 && h.ndim() == 2 && c.ndim() == 2 && W.ndim() == 2 && U.ndim() == 2 && b.ndim() == 1,
+                "lstm_step: x, h, c, W, U must be matrices and b a vector");
+    int H = h.shape()[1];
+    DALI_ASSERT(W.shape()[1] == 4 * H && U.shape()[1] == 4 * H && b.shape()[0] == 4 * H && U.shape()[0] == H &&
+                    W.shape()[0] == x.shape()[1] && c.shape() == h.shape() && x.shape()[0] == h.shape()[0],
+                "lstm_step: inconsistent shapes");
+    // pre-activations: one accumulating GEMM pair (X.W + H.U)
+    Array pre = add(dot(x, W), dot(h, U));
+    pre.eval();
+    auto gate = [&](int k) {
+        Array bias = b.slice(0, k * H, (k + 1) * H).expand_dims(0);
+        return add(pre.slice(1, k * H, (k + 1) * H), bias);
+    };
+    Array ig = sigmoid(gate(0)), fg = sigmoid(gate(1)), og = sigmoid(gate(2)), cw = tanh(gate(3));
+    Array c_new = add(eltmul(fg, c), eltmul(ig, cw));
+    Array h_new = eltmul(og, tanh(c_new));
+    Array::eval_together({c_new, h_new});
+    return {c_new, h_new};
+}
+
+}  // namespace op
+}  // namespace dali

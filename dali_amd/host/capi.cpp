@@ -1,0 +1,179 @@
+// Flat C binding of the front-end, declared in include/dali_front.h.
+#include "../../include/dali_front.h"
+
+#include <cstring>
+
+#include "expr.h"
+
+using dali::Array;
+
+static thread_local std::string g_err;
+static thread_local std::string g_kinds;
+
+#include <functional>
+
+namespace dali {
+void set_dry_compile(bool on);
+void set_recording(std::vector<std::function<void()>>* rec);
+}
+
+#define FE_TRY(body, failure)               \
+    try {                                   \
+        body                                \
+    } catch (const std::exception& ex) {    \
+        g_err = ex.what();                  \
+        return failure;                     \
+    }
+
+static Array& A(dali_array_t h) {
+    if (!h) throw std::runtime_error("NULL array handle");
+    return *(Array*)h;
+}
+static dali_array_t wrap(const Array& a) { return (dali_array_t) new Array(a); }
+static std::vector<int> vec(const int* p, int n) { return n > 0 ? std::vector<int>(p, p + n) : std::vector<int>(); }
+
+extern "C" {
+
+const char* dali_fe_last_error(void) { return g_err.c_str(); }
+
+dali_array_t dali_fe_from_host(const void* data, const int* shape, int ndim, int dtype) {
+    FE_TRY(return wrap(Array::from_host(data, vec(shape, ndim), (dali::DType)dtype));, nullptr)
+}
+dali_array_t dali_fe_empty(const int* shape, int ndim, int dtype) {
+    FE_TRY(return wrap(Array(vec(shape, ndim), (dali::DType)dtype));, nullptr)
+}
+dali_array_t dali_fe_zeros(const int* shape, int ndim, int dtype) {
+    FE_TRY(return wrap(Array::zeros(vec(shape, ndim), (dali::DType)dtype));, nullptr)
+}
+dali_array_t dali_fe_scalar_double(double v) { FE_TRY(return wrap(Array(v));, nullptr) }
+dali_array_t dali_fe_scalar_float(float v) { FE_TRY(return wrap(Array(v));, nullptr) }
+dali_array_t dali_fe_scalar_int(int v) { FE_TRY(return wrap(Array(v));, nullptr) }
+dali_array_t dali_fe_clone_handle(dali_array_t a) { FE_TRY(return wrap(A(a));, nullptr) }
+void dali_fe_release(dali_array_t a) { delete (Array*)a; }
+
+int dali_fe_ndim(dali_array_t a) { FE_TRY(return A(a).ndim();, -1) }
+int dali_fe_shape(dali_array_t a, int* out) {
+    FE_TRY(const auto& s = A(a).shape(); for (size_t i = 0; i < s.size(); ++i) out[i] = s[i]; return 0;, 1)
+}
+int dali_fe_dtype(dali_array_t a) { FE_TRY(return (int)A(a).dtype();, -1) }
+int dali_fe_is_buffer(dali_array_t a) { FE_TRY(return A(a).is_buffer() ? 1 : 0;, -1) }
+int dali_fe_is_contiguous(dali_array_t a) { FE_TRY(return A(a).contiguous_memory() ? 1 : 0;, -1) }
+int dali_fe_strides(dali_array_t a, int* out) {
+    FE_TRY(auto s = A(a).normalized_strides(); for (size_t i = 0; i < s.size(); ++i) out[i] = s[i]; return 0;, 1)
+}
+int dali_fe_offset(dali_array_t a) { FE_TRY(return A(a).offset();, -1) }
+
+dali_array_t dali_fe_transpose(dali_array_t a, const int* axes, int naxes) {
+    FE_TRY(return wrap(naxes ? A(a).transpose(vec(axes, naxes)) : A(a).transpose());, nullptr)
+}
+dali_array_t dali_fe_pluck_axis(dali_array_t a, int axis, int idx) { FE_TRY(return wrap(A(a).pluck_axis(axis, idx));, nullptr) }
+dali_array_t dali_fe_slice(dali_array_t a, int axis, int start, int end, int step) {
+    FE_TRY(return wrap(A(a).slice(axis, start, end, step));, nullptr)
+}
+dali_array_t dali_fe_reshape(dali_array_t a, const int* shape, int ndim) { FE_TRY(return wrap(A(a).reshape(vec(shape, ndim)));, nullptr) }
+dali_array_t dali_fe_expand_dims(dali_array_t a, int axis) { FE_TRY(return wrap(A(a).expand_dims(axis));, nullptr) }
+dali_array_t dali_fe_squeeze(dali_array_t a, int axis) { FE_TRY(return wrap(A(a).squeeze(axis));, nullptr) }
+dali_array_t dali_fe_ascontiguousarray(dali_array_t a) { FE_TRY(return wrap(A(a).ascontiguousarray());, nullptr) }
+
+static std::string qualified(const char* name, const char* ns) {
+    std::string s(name);
+    return s.find("::") == std::string::npos ? std::string(ns) + "::" + s : s;
+}
+
+dali_array_t dali_fe_unary(const char* functor_name, dali_array_t a) {
+    FE_TRY(return wrap(dali::op::elementwise(A(a), qualified(functor_name, "functor")));, nullptr)
+}
+dali_array_t dali_fe_binary(const char* functor_name, dali_array_t a, dali_array_t b) {
+    FE_TRY(return wrap(dali::op::elementwise(A(a), A(b), qualified(functor_name, "functor")));, nullptr)
+}
+dali_array_t dali_fe_astype(dali_array_t a, int dtype) { FE_TRY(return wrap(dali::op::astype(A(a), (dali::DType)dtype));, nullptr) }
+dali_array_t dali_fe_all_reduce(const char* r, dali_array_t a) {
+    FE_TRY(return wrap(dali::op::all_reduce(A(a), qualified(r, "reducers")));, nullptr)
+}
+dali_array_t dali_fe_axis_reduce(const char* r, dali_array_t a, const int* axes, int naxes, int keepdims) {
+    FE_TRY(return wrap(dali::op::axis_reduce(A(a), qualified(r, "reducers"), vec(axes, naxes), keepdims != 0));, nullptr)
+}
+dali_array_t dali_fe_arg_all_reduce(const char* r, dali_array_t a) {
+    FE_TRY(return wrap(dali::op::argument_all_reduce(A(a), qualified(r, "reducers")));, nullptr)
+}
+dali_array_t dali_fe_arg_axis_reduce(const char* r, dali_array_t a, int axis) {
+    FE_TRY(return wrap(dali::op::argument_axis_reduce(A(a), qualified(r, "reducers"), axis));, nullptr)
+}
+dali_array_t dali_fe_mean_all(dali_array_t a) { FE_TRY(return wrap(dali::op::mean(A(a)));, nullptr) }
+dali_array_t dali_fe_mean_axes(dali_array_t a, const int* axes, int naxes, int keepdims) {
+    FE_TRY(return wrap(dali::op::mean(A(a), vec(axes, naxes), keepdims != 0));, nullptr)
+}
+dali_array_t dali_fe_softmax(dali_array_t a, int axis) { FE_TRY(return wrap(dali::op::softmax(A(a), axis));, nullptr) }
+dali_array_t dali_fe_gather_from_rows(dali_array_t s, dali_array_t i) { FE_TRY(return wrap(dali::op::gather_from_rows(A(s), A(i)));, nullptr) }
+dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_value, dali_array_t off_value) {
+    FE_TRY(return wrap(dali::op::one_hot(A(indices), depth, A(on_value), A(off_value)));, nullptr)
+}
+dali_array_t dali_fe_dot(dali_array_t a, dali_array_t b) { FE_TRY(return wrap(dali::op::dot(A(a), A(b)));, nullptr) }
+
+int dali_fe_softmax_cross_entropy(dali_array_t logits, dali_array_t targets, dali_array_t* mean_loss, dali_array_t* row_loss,
+                                  dali_array_t* grad) {
+    FE_TRY(auto r = dali::op::softmax_cross_entropy(A(logits), A(targets)); *mean_loss = wrap(r.mean_loss); *row_loss = wrap(r.row_loss);
+           *grad = wrap(r.grad); return 0;
+           , 1)
+}
+int dali_fe_lstm_step(dali_array_t x, dali_array_t h, dali_array_t c, dali_array_t W, dali_array_t U, dali_array_t b,
+                      dali_array_t* c_new, dali_array_t* h_new) {
+    FE_TRY(auto r = dali::op::lstm_step(A(x), A(h), A(c), A(W), A(U), A(b)); *c_new = wrap(r.memory); *h_new = wrap(r.hidden); return 0;, 1)
+}
+
+int dali_fe_eval(dali_array_t a) { FE_TRY(A(a).eval(); return 0;, 1) }
+int dali_fe_eval_together(dali_array_t* roots, int n) {
+    FE_TRY(std::vector<Array> r; for (int i = 0; i < n; ++i) r.push_back(A(roots[i])); Array::eval_together(r); return 0;, 1)
+}
+int dali_fe_assign(dali_array_t dest, int operator_t, dali_array_t source) {
+    FE_TRY(dali::evaluate_into(A(dest), (dali::OPERATOR_T)operator_t, A(source)); return 0;, 1)
+}
+int dali_fe_to_host(dali_array_t a, void* out) { FE_TRY(A(a).to_host(out); return 0;, 1) }
+void* dali_fe_device_ptr(dali_array_t a) { FE_TRY(return A(a).device_ptr();, nullptr) }
+
+int dali_fe_stats(uint64_t* kernels, uint64_t* gemms, uint64_t* evals, uint64_t* plans) {
+    auto& s = dali::jit_stats();
+    if (kernels) *kernels = s.kernels_launched;
+    if (gemms) *gemms = s.gemms_launched;
+    if (evals) *evals = s.evals;
+    if (plans) *plans = s.plans_built;
+    return 0;
+}
+const char* dali_fe_last_kernel_kinds(void) {
+    g_kinds = dali::jit_stats().last_kernel_kinds;
+    return g_kinds.c_str();
+}
+const char* dali_fe_last_source(void) { return dali::last_generated_source().c_str(); }
+
+void* dali_fe_record_begin(void) {
+    auto* rec = new std::vector<std::function<void()>>();
+    dali::set_recording(rec);
+    return rec;
+}
+int dali_fe_record_end(void* recording) {
+    dali::set_recording(nullptr);
+    return recording ? (int)((std::vector<std::function<void()>>*)recording)->size() : -1;
+}
+int dali_fe_replay(void* recording, int times) {
+    FE_TRY(auto* rec = (std::vector<std::function<void()>>*)recording; if (!rec) throw std::runtime_error("NULL recording");
+           for (int t = 0; t < times; ++t) for (auto& f : *rec) f(); return 0;
+           , 1)
+}
+void dali_fe_record_free(void* recording) { delete (std::vector<std::function<void()>>*)recording; }
+
+int dali_fe_generate_only(dali_array_t* roots, int n, int compile) {
+    dali::set_dry_compile(compile != 0);
+    try {
+        std::vector<Array> r;
+        for (int i = 0; i < n; ++i) r.push_back(A(roots[i]));
+        auto srcs = dali::generate_only(r);
+        dali::set_dry_compile(false);
+        return (int)srcs.size();
+    } catch (const std::exception& ex) {
+        dali::set_dry_compile(false);
+        g_err = ex.what();
+        return -1;
+    }
+}
+
+}  // extern "C"

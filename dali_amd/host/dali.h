@@ -1,0 +1,264 @@
+// Host front-end: lazy `Array` expressions and the `op::` factories for the
+// JIT-fused path, mirroring the subset of the reference's public API that the
+// fused-expression hot path needs (dali/array/array.h:18-230, dali/array/op.h).
+// Building an expression computes nothing; `eval()` (or any host read) plans the
+// fused subgraph, generates HIP source for it, has libdali_hip compile/cache it
+// and launches it through the six-array C ABI.
+#ifndef DALI_AMD_HOST_DALI_H
+#define DALI_AMD_HOST_DALI_H
+
+#include <cstdint>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace dali {
+
+// numbering as in dali/array/dtype.h:6-10
+enum DType { DTYPE_FLOAT = 0, DTYPE_DOUBLE = 1, DTYPE_INT32 = 2 };
+int size_of_dtype(DType dtype);
+std::string dtype_to_cpp_name(DType dtype);
+
+// dali/array/expression/operator.h
+enum OPERATOR_T {
+    OPERATOR_T_EQL = 0,
+    OPERATOR_T_ADD = 1,
+    OPERATOR_T_SUB = 2,
+    OPERATOR_T_MUL = 3,
+    OPERATOR_T_DIV = 4
+};
+
+namespace memory {
+// dali/array/memory/access_modes.h:6-10
+enum AM { AM_READONLY = 0, AM_MUTABLE = 1, AM_OVERWRITE = 2 };
+enum DeviceT { DEVICE_T_CPU = 0, DEVICE_T_GPU = 1 };
+
+// Host + device copies of one allocation with freshness flags and lazy
+// migration on access (dali/array/memory/synchronized_memory.h:35-133).
+class SynchronizedMemory {
+  public:
+    explicit SynchronizedMemory(size_t bytes);
+    ~SynchronizedMemory();
+    SynchronizedMemory(const SynchronizedMemory&) = delete;
+    SynchronizedMemory& operator=(const SynchronizedMemory&) = delete;
+
+    size_t bytes() const { return bytes_; }
+    void* data(DeviceT device, AM mode);
+    const void* readonly_data(DeviceT device);
+    void* mutable_data(DeviceT device);
+    void* overwrite_data(DeviceT device);
+    bool is_fresh(DeviceT device) const { return device == DEVICE_T_CPU ? host_fresh_ : device_fresh_; }
+    bool is_allocated(DeviceT device) const { return device == DEVICE_T_CPU ? host_ != nullptr : device_ != nullptr; }
+    void lazy_clear();  // zero on first allocation (dali/array/memory/synchronized_memory.cpp:237-266)
+
+  private:
+    void allocate(DeviceT device);
+    void move_to(DeviceT device);
+    size_t bytes_;
+    void* host_ = nullptr;
+    void* device_ = nullptr;
+    bool host_fresh_ = false, device_fresh_ = false;
+    bool clear_on_allocation_ = false;
+};
+}  // namespace memory
+
+struct Expr;
+struct ArrayState;
+
+class Array {
+  public:
+    Array();
+    Array(const std::vector<int>& shape, DType dtype = DTYPE_FLOAT);
+    Array(double scalar);
+    Array(float scalar);
+    Array(int scalar);
+    explicit Array(std::shared_ptr<Expr> expr);
+
+    static Array zeros(const std::vector<int>& shape, DType dtype = DTYPE_FLOAT);
+    static Array ones(const std::vector<int>& shape, DType dtype = DTYPE_FLOAT);
+    static Array arange(int n, DType dtype = DTYPE_FLOAT);
+    // copies `data` (contiguous, row-major) into a new buffer
+    static Array from_host(const void* data, const std::vector<int>& shape, DType dtype);
+
+    bool is_stateless() const;
+    bool is_buffer() const;
+    bool is_scalar() const;  // ndim == 0
+    const std::vector<int>& shape() const;
+    int ndim() const;
+    DType dtype() const;
+    int number_of_elements() const;
+    // empty for a contiguous buffer, as in the reference
+    const std::vector<int>& strides() const;
+    std::vector<int> normalized_strides() const;
+    int offset() const;
+    bool contiguous_memory() const;
+    std::shared_ptr<Expr> expression() const;
+
+    // views: exact on buffers; a lazy node is evaluated first
+    Array transpose() const;
+    Array transpose(const std::vector<int>& axes) const;
+    Array swapaxes(int a, int b) const;
+    Array pluck_axis(int axis, int idx) const;
+    Array operator[](int idx) const { return pluck_axis(0, idx); }
+    Array slice(int axis, int start, int end, int step = 1) const;
+    Array reshape(const std::vector<int>& shape) const;
+    Array expand_dims(int axis) const;
+    Array squeeze(int axis) const;
+    Array insert_broadcast_axis(int axis) const { return expand_dims(axis); }
+    Array ascontiguousarray() const;
+
+    // evaluation (dali/array/array.cpp:232-245)
+    void eval() const;
+    // evaluate several roots over the same index domain in as few kernels as the
+    // planner can form (shared subexpressions are computed once)
+    static void eval_together(const std::vector<Array>& roots);
+
+    // dst (op)= expression, into this array's existing buffer
+    Array& assign(const Array& other);
+    Array& operator+=(const Array& other);
+    Array& operator-=(const Array& other);
+    Array& operator*=(const Array& other);
+    Array& operator/=(const Array& other);
+
+    // host access: evaluates, migrates and writes the elements row-major
+    void to_host(void* out) const;
+    double scalar_value() const;  // first element as double
+
+    // device pointer of an evaluated buffer (base + offset applied), for interop
+    void* device_ptr(memory::AM mode = memory::AM_READONLY) const;
+
+    // method sugar used by the reference's expressions (dali/array/array.h:196-230)
+    Array sum() const;
+    Array sum(const std::vector<int>& axes, bool keepdims = false) const;
+    Array max() const;
+    Array max(const std::vector<int>& axes, bool keepdims = false) const;
+    Array min() const;
+    Array min(const std::vector<int>& axes, bool keepdims = false) const;
+    Array mean() const;
+    Array mean(const std::vector<int>& axes, bool keepdims = false) const;
+    Array argmax() const;
+    Array argmax(int axis) const;
+    Array argmin() const;
+    Array argmin(int axis) const;
+    Array exp() const;
+    Array log() const;
+    Array tanh() const;
+    Array sigmoid() const;
+    Array square() const;
+    Array dot(const Array& other) const;
+
+    std::shared_ptr<ArrayState> state_;
+};
+
+Array operator+(const Array& a, const Array& b);
+Array operator-(const Array& a, const Array& b);
+Array operator*(const Array& a, const Array& b);
+Array operator/(const Array& a, const Array& b);
+Array operator-(const Array& a);
+
+namespace op {
+// dali/array/op/elementwise_operation.h, unary.h, binary.h
+Array elementwise(Array a, const std::string& functor_name);
+Array elementwise(Array a, Array b, const std::string& functor_name);
+Array astype(Array a, DType dtype);
+Array unsafe_cast(Array a, DType dtype);
+Array round(Array a);
+Array add(const Array& a, const Array& b);
+Array subtract(const Array& a, const Array& b);
+Array eltmul(const Array& a, const Array& b);
+Array eltdiv(const Array& a, const Array& b);
+Array pow(const Array& a, const Array& b);
+Array equals(const Array& a, const Array& b);
+Array prelu(const Array& x, const Array& weights);
+Array clip(const Array& x, const Array& clipping_value);
+Array identity(const Array& x);
+Array sigmoid(const Array& x);
+Array tanh(const Array& x);
+Array exp(const Array& x);
+Array log(const Array& x);
+Array softplus(const Array& x);
+Array relu(const Array& x);
+Array abs(const Array& x);
+Array sign(const Array& x);
+Array square(const Array& x);
+Array cube(const Array& x);
+Array sqrt(const Array& x);
+Array rsqrt(const Array& x);
+Array eltinv(const Array& x);
+Array negate(const Array& x);
+Array isnan(const Array& x);
+Array isinf(const Array& x);
+Array dsigmoid(const Array& x);
+Array dtanh(const Array& x);
+
+// dali/array/op/reducers.h, reducer_operation.h
+Array all_reduce(const Array& a, const std::string& reducer_name);
+Array axis_reduce(const Array& a, const std::string& reducer_name, const std::vector<int>& axes, bool keepdims);
+Array argument_all_reduce(const Array& a, const std::string& reducer_name);
+Array argument_axis_reduce(const Array& a, const std::string& reducer_name, int axis);
+Array sum(const Array& x);
+Array sum(const Array& x, const std::vector<int>& axes, bool keepdims = false);
+Array prod(const Array& x);
+Array prod(const Array& x, const std::vector<int>& axes, bool keepdims = false);
+Array max(const Array& x);
+Array max(const Array& x, const std::vector<int>& axes, bool keepdims = false);
+Array min(const Array& x);
+Array min(const Array& x, const std::vector<int>& axes, bool keepdims = false);
+Array mean(const Array& x);
+Array mean(const Array& x, const std::vector<int>& axes, bool keepdims = false);
+Array L2_norm(const Array& x);
+Array L2_norm(const Array& x, const std::vector<int>& axes, bool keepdims = false);
+Array argmax(const Array& x);
+Array argmax(const Array& x, int axis);
+Array argmin(const Array& x);
+Array argmin(const Array& x, int axis);
+
+// dali/array/op/softmax.h, gather_from_rows.h, one_hot.h, dot.h
+Array softmax(const Array& logits, int axis = -1);
+Array gather_from_rows(const Array& source, const Array& indices);
+Array one_hot(Array indices, int depth, Array on_value, Array off_value);
+Array matmul(Array a, Array b);
+Array dot(const Array& a, const Array& b);
+
+// Softmax cross-entropy with integer targets in log-sum-exp form
+// (definition: dali/tensor/op/cost.cpp:115-133). Returns {mean loss (scalar),
+// per-row loss [N], gradient [N, V] = softmax - one_hot}; the three are evaluated
+// together so the logits are read once.
+struct CrossEntropyResult {
+    Array mean_loss, row_loss, grad;
+};
+CrossEntropyResult softmax_cross_entropy(const Array& logits, const Array& targets);
+
+// One LSTM cell step with the four gates packed i, f, o, g along the columns of
+// W[I,4H], U[H,4H], b[4H] (definition: dali/layers/lstm.cpp:226-261 with
+// StackedInputLayer::activate, dali/layers/layers.cpp:159-161). Returns {c', h'},
+// already evaluated: one accumulating GEMM pair plus one fused gate kernel.
+struct LSTMState {
+    Array memory, hidden;
+};
+LSTMState lstm_step(const Array& x, const Array& h, const Array& c, const Array& W, const Array& U,
+                    const Array& b);
+}  // namespace op
+
+// Observation hooks in the spirit of dali/utils/scope.h: counts of executed
+// computations, used by tests to assert laziness and fusion.
+struct JitStats {
+    uint64_t kernels_launched = 0;  // generated kernels
+    uint64_t gemms_launched = 0;
+    uint64_t evals = 0;
+    uint64_t plans_built = 0;       // planner invocations that had to generate source
+    std::string last_kernel_kinds;  // e.g. "row" or "row,all" for the last eval
+};
+JitStats& jit_stats();
+// HIP source of the kernels generated for the last eval (concatenated)
+const std::string& last_generated_source();
+
+// Plan + generate the HIP source for `roots` without touching a device; returns
+// the sources of the kernels the planner would launch. Used to check code
+// generation on machines without a GPU.
+std::vector<std::string> generate_only(const std::vector<Array>& roots);
+
+}  // namespace dali
+
+#endif

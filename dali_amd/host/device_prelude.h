@@ -1,0 +1,262 @@
+// Device-side support code prepended to every generated kernel: the scalar
+// functors, the reducers and the wave64 / workgroup reduction helpers.
+//
+// The functors restate the arithmetic contract of the reference's
+// dali/array/functor.h (non-CUDA branch, which is what its CPU results come
+// from): float arguments use the float libm entry points, `sigmoid` and the other
+// functors written with double literals evaluate in double and round once.
+// The reducers restate dali/array/jit/reducer_kernels.h:57-169 (init values
+// 0 / -FLT_MAX / FLT_MAX / 1; maximum is `dst > src ? dst : src`).
+#ifndef DALI_AMD_DEVICE_PRELUDE_H
+#define DALI_AMD_DEVICE_PRELUDE_H
+
+namespace dali {
+namespace codegen {
+
+static const char* const kDevicePrelude = R"HIPSRC(
+#define DALI_FLT_MAX 3.402823466e+38f
+#define DALI_DBL_MAX 1.7976931348623157e+308
+#define DALI_INT_MAX 2147483647
+#define DALI_INT_MIN (-2147483647 - 1)
+#define DI __device__ __forceinline__
+
+union dali_slot { int i; float f; double d; };
+
+template <typename T, int N>
+struct alignas(sizeof(T) * N) dali_vec { T v[N]; };
+
+template <typename T, int N>
+DI dali_vec<T, N> dali_load(const T* p) { return *reinterpret_cast<const dali_vec<T, N>*>(p); }
+template <typename T, int N>
+DI void dali_store(T* p, const dali_vec<T, N>& v) { *reinterpret_cast<dali_vec<T, N>*>(p) = v; }
+template <typename T, int N>
+DI dali_vec<T, N> dali_load_nt(const T* p) {
+    dali_vec<T, N> r;
+    if constexpr (sizeof(T) * N == 16) {
+        typedef int i4 __attribute__((ext_vector_type(4)));
+        i4 raw = __builtin_nontemporal_load(reinterpret_cast<const i4*>(p));
+        __builtin_memcpy(&r, &raw, 16);
+    } else {
+        r = *reinterpret_cast<const dali_vec<T, N>*>(p);
+    }
+    return r;
+}
+template <typename T, int N>
+DI void dali_store_nt(T* p, const dali_vec<T, N>& v) {
+    if constexpr (sizeof(T) * N == 16) {
+        typedef int i4 __attribute__((ext_vector_type(4)));
+        i4 raw;
+        __builtin_memcpy(&raw, &v, 16);
+        __builtin_nontemporal_store(raw, reinterpret_cast<i4*>(p));
+    } else {
+        *reinterpret_cast<dali_vec<T, N>*>(p) = v;
+    }
+}
+
+// ------------------------------------------------------------ libm dispatch
+DI float  m_exp(float a)  { return expf(a); }
+DI double m_exp(double a) { return exp(a); }
+DI double m_exp(int a)    { return exp((double)a); }
+DI float  m_log(float a)  { return logf(a); }
+DI double m_log(double a) { return log(a); }
+DI double m_log(int a)    { return log((double)a); }
+DI float  m_tanh(float a)  { return tanhf(a); }
+DI double m_tanh(double a) { return tanh(a); }
+DI double m_tanh(int a)    { return tanh((double)a); }
+DI float  m_abs(float a)  { return fabsf(a); }
+DI double m_abs(double a) { return fabs(a); }
+DI int    m_abs(int a)    { return a < 0 ? -a : a; }
+DI float  m_pow(float a, float b)   { return powf(a, b); }
+DI double m_pow(double a, double b) { return pow(a, b); }
+DI double m_pow(int a, int b)       { return pow((double)a, (double)b); }
+
+namespace functor {
+template <typename R> struct square   { DI static R Map(R a) { return a * a; } };
+template <typename R> struct cube     { DI static R Map(R a) { return a * a * a; } };
+template <typename R> struct fill     { DI static R Map(R a, R filler) { return filler; } };
+template <typename R> struct add      { DI static R Map(R a, R b) { return a + b; } };
+template <typename R> struct equals   { DI static R Map(R a, R b) { return a == b ? 1 : 0; } };
+template <typename R> struct subtract { DI static R Map(R a, R b) { return a - b; } };
+template <typename R> struct eltmul   { DI static R Map(R a, R b) { return a * b; } };
+template <typename R> struct eltdiv   { DI static R Map(R a, R b) { return a / b; } };
+template <typename R> struct sqrt_f   { DI static R Map(R a) { return (R)sqrt((double)a); } };
+template <> struct sqrt_f<float>      { DI static float Map(float a) { return sqrtf(a); } };
+template <typename R> struct rsqrt    { DI static R Map(R a) { return (R)(1.0 / sqrt((double)a)); } };
+template <typename R> struct inv      { DI static R Map(R a) { return ((R)1.0) / a; } };
+template <typename R> struct cast     { template <typename O> DI static R Map(O a) { return R(a); } };
+template <typename R> struct round    { template <typename O> DI static R Map(O a) { return (R)floor((double)a + 0.5); } };
+template <typename R> struct sigmoid  { DI static R Map(R a) { return (R)(1.0 / (1.0 + (double)m_exp(-a))); } };
+template <typename R> struct identity { DI static R Map(R a) { return a; } };
+template <typename R> struct log      { DI static R Map(R a) { return (R)m_log(a); } };
+template <typename R> struct negative_log { DI static R Map(R a) { return (R)(-m_log(a)); } };
+template <typename R> struct safe_entropy_log {
+    DI static R Map(R a) {
+        R s = a;
+        const R lo = (R)1e-6, hi = (R)(1.0 - 1e-6);
+        if (s > hi) s = hi;
+        if (s < lo) s = lo;
+        return (R)m_log(s);
+    }
+};
+template <typename R> struct exp      { DI static R Map(R a) { return (R)m_exp(a); } };
+template <typename R> struct isnotanumber { DI static R Map(R a) { return (R)(a != a); } };
+template <> struct isnotanumber<int>  { DI static int Map(int a) { return 0; } };
+template <typename R> struct isinfinity { DI static R Map(R a) { return (R)(a == a && (a - a) != (a - a)); } };
+template <> struct isinfinity<int>    { DI static int Map(int a) { return 0; } };
+template <typename R> struct div_grad { DI static R Map(R a, R b) { return a / (b * b); } };
+template <typename R> struct dsigmoid { DI static R Map(R a) { return a * (((R)1.0) - a); } };
+template <typename R> struct tanh     { DI static R Map(R a) { return (R)m_tanh(a); } };
+template <typename R> struct inverse_tanh { DI static R Map(R a) { return (R)((m_log(1 + a) - m_log(1 - a)) * 0.5); } };
+template <typename R> struct dtanh    { DI static R Map(R a) { return (R)(1.0 - a * a); } };
+template <typename R> struct power    { DI static R Map(R a, R b) { return (R)m_pow(a, b); } };
+template <typename R> struct abs      { DI static R Map(R a) { return m_abs(a); } };
+template <typename R> struct log_or_zero { DI static R Map(R a) { return a > 0 ? (R)m_log(a) : (R)0; } };
+template <typename R> struct sign     { DI static R Map(R x) { return x > 0.0 ? 1.0 : -1.0; } };
+template <typename R> struct threshold { DI static R Map(R a, R b) { return a < b ? 1.0 : 0.0; } };
+template <typename R> struct max_scalar { DI static R Map(R x, R y) { return x > y ? x : y; } };
+template <typename R> struct min_scalar { DI static R Map(R x, R y) { return x < y ? x : y; } };
+template <typename R> struct steep_sigmoid { DI static R Map(R x, R g) { return (R)(1.0 / (1.0 + (double)m_exp(-g * x))); } };
+template <typename R> struct steep_sigmoid_backward { DI static R Map(R x, R g) { return g * (x - x * x); } };
+template <typename R> struct relu     { DI static R Map(R x) { return x > 0.0 ? x : (R)0.0; } };
+template <typename R> struct clipped_relu { DI static R Map(R x, R c) { return x > 0.0 ? (x > c ? c : x) : (R)0.0; } };
+template <typename R> struct relu_backward { DI static R Map(R x) { return x > 0.0 ? 1.0 : 0.0; } };
+template <typename R> struct clipped_relu_backward { DI static R Map(R x, R c) { return x > 0.0 ? (x > c ? 0.0 : 1.0) : 0.0; } };
+template <typename R> struct clip {
+    DI static R Map(R x, R c) { return x > c ? c : (x < -c ? -c : x); }
+};
+template <typename R> struct lessthanequal { DI static R Map(R x, R u) { return x <= u ? 1 : 0; } };
+template <typename R> struct greaterthanequal { DI static R Map(R x, R l) { return x >= l ? 1 : 0; } };
+template <typename R> struct binary_cross_entropy {
+    DI static R Map(R x, R t) {
+        R d1 = t * (R)m_log(x);
+        R d0 = (R)((1.0 - t) * m_log(1. - (double)x));
+        return -(d1 + d0);
+    }
+};
+template <typename R> struct binary_cross_entropy_grad {
+    DI static R Map(R x, R t) {
+        R num = t - x;
+        R den = (R)(x * (x - 1.0));
+        return num / den;
+    }
+};
+template <typename R> struct softplus {
+    DI static R Map(R x) { return x > 20.0 ? x : (R)m_log((R)1.0 + (R)m_exp(x)); }
+};
+template <typename R> struct softplus_backward {
+    DI static R Map(R x) { return x > 20.0 ? (R)1.0 : (R)((R)m_exp(x) / ((R)1.0 + (R)m_exp(x))); }
+};
+template <typename R> struct prelu { DI static R Map(R x, R w) { return x > 0 ? x : w * x; } };
+template <typename R> struct prelu_backward_weights { DI static R Map(R x, R g) { return x > 0 ? (R)0 : x * g; } };
+template <typename R> struct prelu_backward_inputs { DI static R Map(R x, R w) { return x > 0 ? (R)1.0 : w; } };
+}  // namespace functor
+
+// one_hot element: on*is_on + (1.0 - is_on)*off with is_on in T and the rest in double
+template <typename T>
+DI T dali_one_hot(int index, int column, T on, T off) {
+    T is_on = (T)(index == column);
+    return (T)((double)(on * is_on) + (1.0 - (double)is_on) * (double)off);
+}
+
+// ------------------------------------------------------------------ reducers
+namespace reducers {
+struct sum {
+    template <typename T> DI static T init() { return (T)0; }
+    template <typename T> DI static T step(T d, T s) { return d + s; }
+    template <typename T> DI static bool better(T cand, T cur) { return false; }
+};
+struct product {
+    template <typename T> DI static T init() { return (T)1; }
+    template <typename T> DI static T step(T d, T s) { return d * s; }
+    template <typename T> DI static bool better(T cand, T cur) { return false; }
+};
+template <typename T> DI T lowest();
+template <> DI float lowest<float>() { return -DALI_FLT_MAX; }
+template <> DI double lowest<double>() { return -DALI_DBL_MAX; }
+template <> DI int lowest<int>() { return DALI_INT_MIN; }
+template <typename T> DI T highest();
+template <> DI float highest<float>() { return DALI_FLT_MAX; }
+template <> DI double highest<double>() { return DALI_DBL_MAX; }
+template <> DI int highest<int>() { return DALI_INT_MAX; }
+struct maximum {
+    template <typename T> DI static T init() { return lowest<T>(); }
+    template <typename T> DI static T step(T d, T s) { return d > s ? d : s; }
+    template <typename T> DI static bool better(T cand, T cur) { return cand > cur; }
+};
+struct minimum {
+    template <typename T> DI static T init() { return highest<T>(); }
+    template <typename T> DI static T step(T d, T s) { return d < s ? d : s; }
+    template <typename T> DI static bool better(T cand, T cur) { return cand < cur; }
+};
+}  // namespace reducers
+
+// --------------------------------------------------------- cross-lane helpers
+template <typename T> DI T dali_shfl_xor(T v, int mask) { return __shfl_xor(v, mask, 64); }
+template <> DI double dali_shfl_xor<double>(double v, int mask) {
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __shfl_xor(lo, mask, 64);
+    hi = __shfl_xor(hi, mask, 64);
+    return __hiloint2double(hi, lo);
+}
+
+// Reduce over aligned groups of WIDTH lanes (WIDTH a power of two <= 64); every
+// lane of the group ends with the group's result.
+template <typename R, typename T, int WIDTH>
+DI T dali_group_reduce(T v) {
+#pragma unroll
+    for (int m = WIDTH / 2; m >= 1; m >>= 1) v = R::template step<T>(v, dali_shfl_xor<T>(v, m));
+    return v;
+}
+
+// (value, index) variant: a candidate wins when its value is strictly better, or
+// equal with a lower index, which reproduces "first index on ties" of a sequential scan.
+template <typename R, typename T, int WIDTH>
+DI void dali_group_arg_reduce(T& v, int& idx) {
+#pragma unroll
+    for (int m = WIDTH / 2; m >= 1; m >>= 1) {
+        T ov = dali_shfl_xor<T>(v, m);
+        int oi = __shfl_xor(idx, m, 64);
+        if (R::template better<T>(ov, v) || (ov == v && oi < idx)) { v = ov; idx = oi; }
+    }
+}
+
+// Reduce over the NW waves of a workgroup through LDS. `sm` must hold NW values
+// and be private to this call site (no barrier is needed before reusing other
+// slots). Every thread returns the workgroup's result, combined in wave order.
+template <typename R, typename T, int NW>
+DI T dali_block_reduce(T v, T* sm) {
+    v = dali_group_reduce<R, T, 64>(v);
+    if constexpr (NW == 1) return v;
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) sm[wave] = v;
+    __syncthreads();
+    T r = sm[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) r = R::template step<T>(r, sm[w]);
+    return r;
+}
+
+template <typename R, typename T, int NW>
+DI void dali_block_arg_reduce(T& v, int& idx, T* smv, int* smi) {
+    dali_group_arg_reduce<R, T, 64>(v, idx);
+    if constexpr (NW == 1) return;
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) { smv[wave] = v; smi[wave] = idx; }
+    __syncthreads();
+    T r = smv[0];
+    int ri = smi[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) {
+        T ov = smv[w];
+        int oi = smi[w];
+        if (R::template better<T>(ov, r) || (ov == r && oi < ri)) { r = ov; ri = oi; }
+    }
+    v = r;
+    idx = ri;
+}
+)HIPSRC";
+
+}  // namespace codegen
+}  // namespace dali
+
+#endif

@@ -1,0 +1,84 @@
+// Expression nodes of the lazy graph (internal to the front-end).
+#ifndef DALI_AMD_HOST_EXPR_H
+#define DALI_AMD_HOST_EXPR_H
+
+#include <sstream>
+
+#include "dali.h"
+
+namespace dali {
+
+enum class Kind {
+    BUFFER,            // dali/array/expression/buffer.h
+    SCALAR,            // dali/array/jit/scalar_view.cpp:15-71
+    ELEMENTWISE,       // dali/array/op/elementwise_operation.cpp:35-124
+    AXIS_REDUCE,       // dali/array/op/reducer_operation.cpp:98-156 (reduces the LAST axis)
+    ALL_REDUCE,        // dali/array/op/reducer_operation.cpp:41-88
+    ARG_AXIS_REDUCE,   // dali/array/op/reducer_operation.cpp:193-228
+    ARG_ALL_REDUCE,    // dali/array/op/reducer_operation.cpp:158-191
+    EXPAND_DIMS,       // dali/array/jit/reshape.cpp:156-209
+    BROADCAST,         // dali/array/jit/reshape.cpp:62-154 (BroadcastedReshape)
+    GATHER_FROM_ROWS,  // dali/array/op/gather_from_rows.cpp:21-127
+    ONE_HOT,           // dali/array/op/one_hot.cpp:16-74
+    MATMUL             // dali/array/op/dot.cpp:18-47
+};
+
+struct Expr {
+    Kind kind;
+    DType dtype = DTYPE_FLOAT;
+    std::vector<int> shape;
+    std::vector<Array> args;
+    std::string name;  // functor or reducer, e.g. "functor::exp", "reducers::sum"
+
+    // BUFFER
+    std::shared_ptr<memory::SynchronizedMemory> memory;
+    std::vector<int> strides;  // empty = contiguous row-major
+    int offset = 0;            // in elements
+
+    // SCALAR
+    double dvalue = 0.0;
+    int ivalue = 0;
+
+    int axis = 0;   // EXPAND_DIMS
+    int depth = 0;  // ONE_HOT
+
+    int numel() const {
+        int64_t n = 1;
+        for (int s : shape) n *= s;
+        return (int)n;
+    }
+};
+
+struct ArrayState {
+    std::shared_ptr<Expr> expr;
+};
+
+template <typename... Args>
+std::string make_message(const Args&... args) {
+    std::ostringstream ss;
+    using expander = int[];
+    (void)expander{0, ((void)(ss << args), 0)...};
+    return ss.str();
+}
+
+std::string shape_str(const std::vector<int>& shape);
+
+#define DALI_ASSERT(cond, msg)                         \
+    do {                                               \
+        if (!(cond)) throw std::runtime_error(msg);    \
+    } while (0)
+
+// C-ABI status -> exception
+void check_hip(int status, const char* what);
+
+std::vector<int> contiguous_strides(const std::vector<int>& shape);
+
+// evaluation driver (jit.cpp)
+void evaluate(const std::vector<Array>& roots);
+void evaluate_into(const Array& dest, OPERATOR_T op, const Array& source);
+void set_dry_run(bool on);
+bool dry_run();
+
+}  // namespace dali
+
+#endif

@@ -1,0 +1,153 @@
+"""``op``: the lazy operator factories (``dali/array/op.h`` of the reference)."""
+import ctypes as C
+
+from ._native import front, fe_error
+from .array import Array, as_array, _ints, _wrap, DTYPE_FLOAT, DTYPE_DOUBLE, DTYPE_INT32  # noqa: F401
+
+
+def elementwise(functor_name, a, b=None):
+    a = as_array(a)
+    if b is None:
+        return _wrap(front.dali_fe_unary(functor_name.encode(), a._h), functor_name)
+    b = as_array(b)
+    return _wrap(front.dali_fe_binary(functor_name.encode(), a._h, b._h), functor_name)
+
+
+def _unary(name):
+    def f(x):
+        return elementwise(name, x)
+    f.__name__ = name
+    return f
+
+
+def _binary(name):
+    def f(a, b):
+        return elementwise(name, a, b)
+    f.__name__ = name
+    return f
+
+
+# dali/array/op/unary.h
+identity = _unary("identity")
+sigmoid = _unary("sigmoid")
+tanh = _unary("tanh")
+exp = _unary("exp")
+log = _unary("log")
+softplus = _unary("softplus")
+relu = _unary("relu")
+abs = _unary("abs")
+sign = _unary("sign")
+square = _unary("square")
+cube = _unary("cube")
+sqrt = _unary("sqrt_f")
+rsqrt = _unary("rsqrt")
+eltinv = _unary("inv")
+isnan = _unary("isnotanumber")
+isinf = _unary("isinfinity")
+dsigmoid = _unary("dsigmoid")
+dtanh = _unary("dtanh")
+# dali/array/op/binary.h
+add = _binary("add")
+subtract = _binary("subtract")
+eltmul = _binary("eltmul")
+eltdiv = _binary("eltdiv")
+pow = _binary("power")
+equals = _binary("equals")
+prelu = _binary("prelu")
+clip = _binary("clip")
+
+
+def astype(a, dtype):
+    a = as_array(a)
+    return _wrap(front.dali_fe_astype(a._h, dtype), "astype")
+
+
+def _reduce(reducer, x, axes, keepdims):
+    x = as_array(x)
+    if axes is None:
+        return _wrap(front.dali_fe_all_reduce(reducer.encode(), x._h), reducer)
+    if isinstance(axes, int):
+        axes = [axes]
+    a, n = _ints(axes)
+    return _wrap(front.dali_fe_axis_reduce(reducer.encode(), x._h, a, n, 1 if keepdims else 0), reducer)
+
+
+def sum(x, axes=None, keepdims=False):
+    return _reduce("sum", x, axes, keepdims)
+
+
+def prod(x, axes=None, keepdims=False):
+    return _reduce("product", x, axes, keepdims)
+
+
+def max(x, axes=None, keepdims=False):
+    return _reduce("maximum", x, axes, keepdims)
+
+
+def min(x, axes=None, keepdims=False):
+    return _reduce("minimum", x, axes, keepdims)
+
+
+def mean(x, axes=None, keepdims=False):
+    x = as_array(x)
+    if axes is None:
+        return _wrap(front.dali_fe_mean_all(x._h), "mean")
+    if isinstance(axes, int):
+        axes = [axes]
+    a, n = _ints(axes)
+    return _wrap(front.dali_fe_mean_axes(x._h, a, n, 1 if keepdims else 0), "mean")
+
+
+def _arg(reducer, x, axis):
+    x = as_array(x)
+    if axis is None:
+        return _wrap(front.dali_fe_arg_all_reduce(reducer.encode(), x._h), "arg " + reducer)
+    return _wrap(front.dali_fe_arg_axis_reduce(reducer.encode(), x._h, axis), "arg " + reducer)
+
+
+def argmax(x, axis=None):
+    return _arg("maximum", x, axis)
+
+
+def argmin(x, axis=None):
+    return _arg("minimum", x, axis)
+
+
+# Converted operands are bound to local names for the duration of each native
+# call: a temporary Array would release its handle before the call reads it.
+def softmax(x, axis=-1):
+    x = as_array(x)
+    return _wrap(front.dali_fe_softmax(x._h, axis), "softmax")
+
+
+def gather_from_rows(source, indices):
+    source, indices = as_array(source), as_array(indices)
+    return _wrap(front.dali_fe_gather_from_rows(source._h, indices._h), "gather_from_rows")
+
+
+def one_hot(indices, depth, on_value, off_value):
+    indices, on_value, off_value = as_array(indices), as_array(on_value), as_array(off_value)
+    return _wrap(front.dali_fe_one_hot(indices._h, depth, on_value._h, off_value._h), "one_hot")
+
+
+def dot(a, b):
+    a, b = as_array(a), as_array(b)
+    return _wrap(front.dali_fe_dot(a._h, b._h), "dot")
+
+
+def softmax_cross_entropy(logits, targets):
+    """(mean loss, per-row loss, gradient) of the LSE-form softmax cross-entropy, evaluated together."""
+    outs = [C.c_void_p() for _ in range(3)]
+    logits, targets = as_array(logits), as_array(targets)
+    if front.dali_fe_softmax_cross_entropy(logits._h, targets._h, *[C.byref(o) for o in outs]) != 0:
+        raise fe_error("softmax_cross_entropy")
+    return tuple(Array(o.value) for o in outs)
+
+
+def lstm_step(x, h, c, W, U, b):
+    """One LSTM cell step; returns (c', h') already evaluated."""
+    outs = [C.c_void_p() for _ in range(2)]
+    keep = [as_array(v) for v in (x, h, c, W, U, b)]
+    if front.dali_fe_lstm_step(*[k._h for k in keep], *[C.byref(o) for o in outs]) != 0:
+        raise fe_error("lstm_step")
+    return tuple(Array(o.value) for o in outs)

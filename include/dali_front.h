@@ -1,0 +1,99 @@
+/*
+ * dali_front.h — flat C binding of the C++ host front-end (dali_amd/host/dali.h)
+ * so that scripting languages can build the same lazy expressions a C++ user of
+ * the reference writes with `Array` and `op::` (dali/array/array.h:18-230,
+ * dali/array/op.h:1-26). Handles are opaque; every function that can fail
+ * returns NULL / non-zero and leaves a message in dali_fe_last_error().
+ * The device work itself goes through the C ABI of include/dali_hip.h.
+ */
+#ifndef DALI_FRONT_H
+#define DALI_FRONT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* dali_array_t;
+
+const char* dali_fe_last_error(void);
+
+/* construction (dali/array/array.h:31-62) */
+dali_array_t dali_fe_from_host(const void* data, const int* shape, int ndim, int dtype);
+dali_array_t dali_fe_empty(const int* shape, int ndim, int dtype);
+dali_array_t dali_fe_zeros(const int* shape, int ndim, int dtype);
+dali_array_t dali_fe_scalar_double(double v);
+dali_array_t dali_fe_scalar_float(float v);
+dali_array_t dali_fe_scalar_int(int v);
+dali_array_t dali_fe_clone_handle(dali_array_t a);
+void dali_fe_release(dali_array_t a);
+
+/* inspection */
+int dali_fe_ndim(dali_array_t a);
+int dali_fe_shape(dali_array_t a, int* out);   /* writes ndim ints */
+int dali_fe_dtype(dali_array_t a);
+int dali_fe_is_buffer(dali_array_t a);
+int dali_fe_is_contiguous(dali_array_t a);
+int dali_fe_strides(dali_array_t a, int* out); /* normalized strides, ndim ints */
+int dali_fe_offset(dali_array_t a);
+
+/* views (dali/array/array.h:120-160) */
+dali_array_t dali_fe_transpose(dali_array_t a, const int* axes, int naxes); /* naxes == 0: reverse */
+dali_array_t dali_fe_pluck_axis(dali_array_t a, int axis, int idx);
+dali_array_t dali_fe_slice(dali_array_t a, int axis, int start, int end, int step);
+dali_array_t dali_fe_reshape(dali_array_t a, const int* shape, int ndim);
+dali_array_t dali_fe_expand_dims(dali_array_t a, int axis);
+dali_array_t dali_fe_squeeze(dali_array_t a, int axis);
+dali_array_t dali_fe_ascontiguousarray(dali_array_t a);
+
+/* lazy ops (headers under dali/array/op) */
+dali_array_t dali_fe_unary(const char* functor_name, dali_array_t a);
+dali_array_t dali_fe_binary(const char* functor_name, dali_array_t a, dali_array_t b);
+dali_array_t dali_fe_astype(dali_array_t a, int dtype);
+dali_array_t dali_fe_all_reduce(const char* reducer_name, dali_array_t a);
+dali_array_t dali_fe_axis_reduce(const char* reducer_name, dali_array_t a, const int* axes, int naxes, int keepdims);
+dali_array_t dali_fe_arg_all_reduce(const char* reducer_name, dali_array_t a);
+dali_array_t dali_fe_arg_axis_reduce(const char* reducer_name, dali_array_t a, int axis);
+dali_array_t dali_fe_mean_all(dali_array_t a);
+dali_array_t dali_fe_mean_axes(dali_array_t a, const int* axes, int naxes, int keepdims);
+dali_array_t dali_fe_softmax(dali_array_t a, int axis);
+dali_array_t dali_fe_gather_from_rows(dali_array_t source, dali_array_t indices);
+dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_value, dali_array_t off_value);
+dali_array_t dali_fe_dot(dali_array_t a, dali_array_t b);
+
+/* composites evaluated as one fused group */
+int dali_fe_softmax_cross_entropy(dali_array_t logits, dali_array_t targets, dali_array_t* mean_loss,
+                                  dali_array_t* row_loss, dali_array_t* grad);
+int dali_fe_lstm_step(dali_array_t x, dali_array_t h, dali_array_t c, dali_array_t W, dali_array_t U, dali_array_t b,
+                      dali_array_t* c_new, dali_array_t* h_new);
+
+/* evaluation, assignment, host access */
+int dali_fe_eval(dali_array_t a);
+int dali_fe_eval_together(dali_array_t* roots, int n);
+int dali_fe_assign(dali_array_t dest, int operator_t, dali_array_t source); /* 0 =, 1 +=, 2 -=, 3 *=, 4 /= */
+int dali_fe_to_host(dali_array_t a, void* out);
+void* dali_fe_device_ptr(dali_array_t a);
+
+/* observation (dali/utils/scope.h, dali/array/tests/dot_tests.cpp:17-36) */
+int dali_fe_stats(uint64_t* kernels, uint64_t* gemms, uint64_t* evals, uint64_t* plans);
+const char* dali_fe_last_kernel_kinds(void);
+const char* dali_fe_last_source(void);
+/* Launch recording: between begin and end every kernel and GEMM launch issued by
+ * evaluations is also stored (with the buffers it touches kept alive); replay
+ * re-issues the stored launches `times` times on the library stream without
+ * rebuilding or re-planning the expressions. */
+void* dali_fe_record_begin(void);
+int dali_fe_record_end(void* recording); /* number of stored launches */
+int dali_fe_replay(void* recording, int times);
+void dali_fe_record_free(void* recording);
+
+/* plan + generate (and optionally hipRTC-compile for gfx950) without a device;
+ * returns the number of kernels, -1 on error */
+int dali_fe_generate_only(dali_array_t* roots, int n, int compile);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DALI_FRONT_H */

@@ -1,0 +1,210 @@
+/*
+ * dali_hip.h — C ABI of the MI355X (gfx950) execution backend for Dali's
+ * JIT-fused array expressions.
+ *
+ * Every entry point returns 0 on success and a non-zero status on failure; the
+ * message for the calling thread's last failure is dali_hip_last_error(). The
+ * library never calls exit() and never frees caller memory. All device work is
+ * issued on ONE non-blocking HIP stream owned by the library, so launches are
+ * ordered among themselves; host-visible copies synchronise that stream.
+ *
+ * Each declaration cites the interface of the reference (bzcheeseman/Dali,
+ * paths relative to its repository root) that it replaces.
+ */
+#ifndef DALI_HIP_H
+#define DALI_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DALI_HIP_OK 0
+#define DALI_HIP_ERROR 1
+
+/* scalar / element types; numbering follows dali/array/dtype.h:6-10 */
+#define DALI_HIP_FLOAT 0
+#define DALI_HIP_DOUBLE 1
+#define DALI_HIP_INT32 2
+
+/* ---------------------------------------------------------------- errors */
+
+/* Message of the last failed call on this thread ("" when none). Replaces the
+ * ASSERT2 -> std::runtime_error text of dali/utils/assert2.h:12 and the
+ * exit(EXIT_FAILURE) paths of dali/utils/compiler.h:81-88. */
+const char* dali_hip_last_error(void);
+
+/* ------------------------------------------------ device and placement */
+
+/* Number of HIP devices. Replaces memory::Device::num_gpus,
+ * dali/array/memory/device.cu.cpp:89-129. */
+int dali_hip_device_count(int* count);
+
+/* Select the device all later calls act on and create the library stream for
+ * it. Replaces Device::set_cuda_device, dali/array/memory/device.cu.cpp:89-129. */
+int dali_hip_init(int device);
+
+/* Device marketing name and gcn arch string. Replaces Device::gpu_name,
+ * dali/array/memory/device.cu.cpp:89-129. */
+int dali_hip_device_name(int device, char* name, size_t name_len, char* arch, size_t arch_len);
+
+/* Free and total device memory in bytes. Replaces memory::cuda_available_memory,
+ * dali/array/memory/memory_ops.cu.cpp:134-138. */
+int dali_hip_mem_info(size_t* free_bytes, size_t* total_bytes);
+
+/* Block until everything issued on the library stream has finished. The
+ * reference relies on NULL-stream ordering plus blocking cudaMemcpy
+ * (dali/array/jit/jit.cpp:752, dali/array/memory/memory_ops.cu.cpp:109-126). */
+int dali_hip_sync(void);
+
+/* The library stream as an opaque hipStream_t, for callers that record their own events. */
+void* dali_hip_stream(void);
+
+/* -------------------------------------------------------------- memory */
+
+/* Raw allocation / release. Replace memory::allocate and memory::free,
+ * dali/array/memory/memory_ops.cu.cpp:58-95 (cudaMallocPitch / cudaFree);
+ * byte counts are size_t instead of the reference's int. */
+int dali_hip_malloc(void** ptr, size_t bytes);
+int dali_hip_free(void* ptr);
+
+/* Size-keyed free-list reuse of device blocks. Replace memory::bank::allocate,
+ * deposit and clear, dali/array/memory/memory_bank.cpp:40-81: a deposited block
+ * is handed out again for a request of the same byte size and only returned to
+ * the driver by dali_hip_bank_clear. */
+int dali_hip_bank_allocate(void** ptr, size_t bytes);
+int dali_hip_bank_deposit(void* ptr, size_t bytes);
+int dali_hip_bank_clear(void);
+/* bytes currently parked in the bank / handed out by it and not yet deposited */
+int dali_hip_bank_stats(size_t* parked_bytes, size_t* live_bytes);
+
+/* Zero-fill on the library stream. Replaces memory::clear,
+ * dali/array/memory/memory_ops.cu.cpp:97-107 (cudaMemset). */
+int dali_hip_memset_async(void* ptr, int value, size_t bytes);
+
+/* Copies. Replace memory::copy, dali/array/memory/memory_ops.cu.cpp:109-126
+ * (blocking cudaMemcpy). h2d and d2h return after the data has arrived (they
+ * synchronise the library stream); d2d is asynchronous on the library stream. */
+int dali_hip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
+int dali_hip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);
+int dali_hip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes);
+
+/* ------------------------------------------- runtime-compiled kernels */
+
+/* How the launcher turns the six argument arrays into a grid. */
+#define DALI_HIP_GRID_ELEMS 0  /* 1-D: blocks over prod(iv[work_begin..+work_count)) / work_per_block */
+#define DALI_HIP_GRID_ROWS 1   /* 1-D: one block per work_per_block rows; rows = prod(iv[work_begin..+work_count)) */
+#define DALI_HIP_GRID_COLS 2   /* 2-D: x over kept columns, y splits the reduced rows; partials in the workspace */
+#define DALI_HIP_GRID_ALL 3    /* 1-D: bounded grid, one partial per block in the workspace */
+
+/*
+ * Launch plan of one generated kernel. The generated kernel has the signature
+ *     extern "C" __global__ void <kernel_name>(KArgs args)
+ * where KArgs is laid out by the launcher as
+ *     void*  ws;                   library workspace (partials and counters)
+ *     void*  p[n_arrays];          array_data[i] + offsets[i] * array_elsize[i]
+ *     slot   s[max(1,n_scalars)];  8-byte slots holding *scalar_arguments[j]
+ *     int    iv[...];              per array: sizes[i][0..nd) then, if the array is
+ *                                  declared strided, strides[i][0..nd); then per
+ *                                  shape k: shapes[k][0..shape_ndim[k])
+ * with nd = array_ndim[i]. The grid is computed from iv by grid_kind.
+ */
+typedef struct dali_hip_launch_plan {
+    int32_t n_arrays;
+    int32_t n_scalars;
+    int32_t n_shapes;
+    const int32_t* array_ndim;    /* [n_arrays] max(1, ndim) of each buffer (dali/array/jit/jit.cpp:281-285) */
+    const int32_t* array_strided; /* [n_arrays] 1 when strides[i] is valid (dali/array/jit/jit.cpp:216-232) */
+    const int32_t* array_elsize;  /* [n_arrays] bytes per element */
+    const int32_t* scalar_dtype;  /* [n_scalars] DALI_HIP_FLOAT / DOUBLE / INT32 (dali/array/jit/scalar_view.cpp:39-66) */
+    const int32_t* shape_ndim;    /* [n_shapes] ints read from shapes[k] */
+    int32_t block_threads;        /* workgroup size */
+    int32_t grid_kind;            /* DALI_HIP_GRID_* */
+    int32_t work_begin;           /* first iv index of the extent product (x dimension) */
+    int32_t work_count;           /* number of iv entries multiplied (0 => 1) */
+    int32_t work_per_block;       /* elements / rows / columns covered by one block in x */
+    int32_t max_blocks;           /* upper bound of grid.x (0 => unbounded) */
+    int32_t work2_begin;          /* GRID_COLS: iv index of the reduced extent */
+    int32_t work2_per_block;      /* GRID_COLS: reduced rows per y-block */
+    int32_t max_blocks2;          /* GRID_COLS: upper bound of grid.y */
+    int32_t ws_elsize;            /* GRID_COLS / GRID_ALL: bytes of one partial result (0 = no workspace) */
+} dali_hip_launch_plan;
+
+/*
+ * Make the kernel for `hash` launchable: in-process map, else the on-disk code
+ * object cache (<cache>/<hash>.hsaco), else hipRTC for gfx950. `*was_cached`
+ * (may be NULL) receives 2 for an in-process hit, 1 for a disk hit, 0 after a
+ * compile. Replaces Compiler::load / Compiler::compile / dlopen / dlsym("maker"),
+ * dali/utils/compiler.h:91-173 and dali/utils/compiler.cpp:36-49,86-103,123-227.
+ * The cache directory is $DALI_HIP_CACHE_DIR, else ~/.dali/cache_hip
+ * (dali/utils/compiler.cpp:234-238); DALI_JIT_ALWAYS_RECOMPILE=true forces one
+ * rebuild per hash per process (dali/array/jit/jit.cpp:27-47,1023-1024).
+ */
+int dali_hip_module_load(uint64_t hash, const char* hip_source, const char* kernel_name,
+                         const dali_hip_launch_plan* plan, int* was_cached);
+
+/* 1 when `hash` is already loaded in this process, else 0 (no compile, no disk access). */
+int dali_hip_module_is_loaded(uint64_t hash);
+
+/*
+ * Launch the kernel of `hash` with the reference's six argument arrays, same
+ * order and meaning as `maker(void** array_data, const int* offsets, const int**
+ * sizes, const int** strides, const void** scalar_arguments, const int** shapes)`
+ * (dali/utils/compiler.cpp:190-197, called from dali/array/jit/jit.cpp:1216-1223):
+ * array_data[i] are device pointers, offsets in elements, scalars are host
+ * pointers read at call time.
+ */
+int dali_hip_launch(uint64_t hash, void** array_data, const int* offsets, const int** sizes,
+                    const int** strides, const void** scalar_arguments, const int** shapes);
+
+/* Compile only (no device needed): hipRTC `hip_source` for gfx950 and return the
+ * code object size; used to check generated source on machines without a GPU. */
+int dali_hip_compile_only(const char* hip_source, size_t* code_size);
+
+/* Counters: modules compiled by hipRTC, loaded from disk, and launches so far. */
+int dali_hip_jit_stats(uint64_t* compiled, uint64_t* disk_hits, uint64_t* launches);
+
+/* Set the code-object cache directory (overrides the environment). Replaces
+ * Compiler::set_output_path, dali/utils/compiler.cpp:115-117. */
+int dali_hip_set_cache_dir(const char* path);
+
+/* ---------------------------------------------------------------- GEMM */
+
+/*
+ * fp32 GEMM on the matrix cores, column-major convention of the call it
+ * replaces: cublasSgemm(handle, transB, transA, m, n, k, &alpha, B, ldb, A, lda,
+ * &beta, C, ldc) in dali/array/gemm/cublas_gemm.cu:153-166 (and cblas_sgemm in
+ * dali/array/gemm/cpu_gemm.cpp:59-68): C(m x n, column-major, ldc) =
+ * alpha * op(B)(m x k) * op(A)(k x n) + beta * C, i.e. in row-major terms
+ * C[n, m] = alpha * A[n, k] * B[k, m] + beta * C. trans flags: 0 = no transpose,
+ * 1 = transpose.
+ */
+int dali_hip_sgemm(int transB, int transA, int m, int n, int k, float alpha, const float* B, int ldb,
+                   const float* A, int lda, float beta, float* C, int ldc);
+
+/*
+ * Two products accumulated into one destination in a single launch:
+ * C = alpha * (op(B1) * op(A1) + op(B2) * op(A2)) + beta * C with the same
+ * conventions as dali_hip_sgemm (k1 and k2 are the two inner extents). This is
+ * the shape `dst = X.W; dst += H.U` of StackedInputLayer::activate,
+ * dali/layers/layers.cpp:159-161 via dali/tensor/op/composite.cpp:18-53.
+ */
+int dali_hip_sgemm_pair(int transB1, int transA1, int transB2, int transA2, int m, int n, int k1, int k2,
+                        float alpha, const float* B1, int ldb1, const float* A1, int lda1, const float* B2,
+                        int ldb2, const float* A2, int lda2, float beta, float* C, int ldc);
+
+/* --------------------------------------------------------------- timing */
+
+/* hipEvent wrappers bound to the library stream (the reference times host-side
+ * only, dali/utils/performance_report.cpp:22-149). */
+int dali_hip_event_create(void** event);
+int dali_hip_event_record(void* event);
+int dali_hip_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
+int dali_hip_event_destroy(void* event);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DALI_HIP_H */

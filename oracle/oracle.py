@@ -1,0 +1,249 @@
+"""ctypes loader for the checker libraries (test infrastructure only).
+
+``liboracle.so`` is the CPU restatement (oracle/dali_oracle.c); ``_ref/libdali_ref.so``
+is built from the reference's own headers when the reference checkout is present.
+Only tests, the smoke check and the benchmark's cpu_baseline leg import this module.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SUM, MAX, MIN, PROD = 0, 1, 2, 3
+
+_f = C.POINTER(C.c_float)
+_i32 = C.POINTER(C.c_int32)
+_i64 = C.c_int64
+
+
+def build(force=False):
+    """Compile the checker libraries (gcc only; no GPU toolchain involved)."""
+    so = os.path.join(_HERE, "liboracle.so")
+    if force or not os.path.exists(so) or os.path.getmtime(so) < os.path.getmtime(os.path.join(_HERE, "dali_oracle.c")):
+        subprocess.check_call(["make", "-C", _HERE, "liboracle.so"], stdout=subprocess.DEVNULL)
+    ref = os.path.join(_HERE, "_ref", "libdali_ref.so")
+    if os.path.isdir("/root/reference") and (force or not os.path.exists(ref)):
+        subprocess.check_call(["make", "-C", _HERE, "ref"], stdout=subprocess.DEVNULL)
+
+
+def _load():
+    path = os.path.join(_HERE, "liboracle.so")
+    if not os.path.exists(path):
+        build()
+    lib = C.CDLL(path)
+    lib.orc_unary.argtypes = [C.c_char_p, _f, _f, _i64]
+    lib.orc_binary.argtypes = [C.c_char_p, _f, _i64, _f, _i64, _f, _i64]
+    lib.orc_round_to_int.argtypes = [_f, _i32, _i64]
+    lib.orc_chain.argtypes = [_f, _f, _f, _f, _f, _i64]
+    lib.orc_axis_reduce.argtypes = [C.c_int, _f, _i64, _i64, _i64, _i64, _f]
+    lib.orc_all_reduce.argtypes = [C.c_int, _f, _i64]
+    lib.orc_all_reduce.restype = C.c_float
+    lib.orc_arg_axis_reduce.argtypes = [C.c_int, _f, _i64, _i64, _i64, _i64, _i32]
+    lib.orc_arg_all_reduce.argtypes = [C.c_int, _f, _i64]
+    lib.orc_arg_all_reduce.restype = _i64
+    lib.orc_mean_all.argtypes = [_f, _i64]
+    lib.orc_mean_all.restype = C.c_float
+    lib.orc_softmax.argtypes = [_f, _f, _i64, _i64]
+    lib.orc_gather_from_rows.argtypes = [_f, _i64, _i32, _i64, _f]
+    lib.orc_one_hot.argtypes = [_i32, _i64, C.c_int, C.c_float, C.c_float, _f]
+    lib.orc_softmax_cross_entropy.argtypes = [_f, _i32, _i64, _i64, _f, _f, _f]
+    lib.orc_softmax_cross_entropy_via_probs.argtypes = [_f, _i32, _i64, _i64, _f]
+    for name in ("orc_gemm_f64acc", "orc_gemm_f32seq"):
+        getattr(lib, name).argtypes = [_f, _i64, _i64, _f, _i64, _i64, _f, _i64, C.c_int, C.c_int, C.c_int]
+    lib.orc_gemm_i32.argtypes = [_i32, _i64, _i64, _i32, _i64, _i64, _i32, _i64, C.c_int, C.c_int, C.c_int]
+    lib.orc_lstm_step.argtypes = [_f, _f, _f, _f, _f, _f, C.c_int, C.c_int, C.c_int, C.c_int, _f, _f, _f]
+    return lib
+
+
+lib = _load()
+
+
+def _ref_load():
+    path = os.path.join(_HERE, "_ref", "libdali_ref.so")
+    if not os.path.exists(path):
+        return None
+    r = C.CDLL(path)
+    r.ref_axis_reduce.argtypes = [C.c_int, _f, C.c_int, C.c_int, C.c_int, C.c_int, _f]
+    r.ref_arg_axis_reduce.argtypes = [C.c_int, _f, C.c_int, C.c_int, C.c_int, C.c_int, _i32]
+    r.ref_all_reduce.argtypes = [C.c_int, _f, C.c_int]
+    r.ref_all_reduce.restype = C.c_float
+    r.ref_index_to_dim3.argtypes = [C.c_int, _i32, _i32]
+    r.ref_indices_to_offset3.argtypes = [_i32, _i32]
+    r.ref_indices_to_offset3.restype = C.c_int
+    r.ref_gemm_i32.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _i32, C.c_int, _i32, C.c_int, _i32, C.c_int]
+    r.ref_gemm_f32.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _f, C.c_int, _f, C.c_int, _f, C.c_int]
+    return r
+
+
+ref = _ref_load()
+
+
+def fp(a):
+    return a.ctypes.data_as(_f)
+
+
+def ip(a):
+    return a.ctypes.data_as(_i32)
+
+
+def _c32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def unary(name, x):
+    x = _c32(x)
+    y = np.empty_like(x)
+    if lib.orc_unary(name.encode(), fp(x), fp(y), x.size) != 0:
+        raise KeyError(name)
+    return y
+
+
+def binary(name, a, b):
+    """a, b: same-shape arrays or Python/NumPy scalars (broadcast with stride 0)."""
+    a_arr = _c32(a)
+    b_arr = _c32(b)
+    out_shape = a_arr.shape if a_arr.size >= b_arr.size else b_arr.shape
+    n = max(a_arr.size, b_arr.size)
+    sa = 0 if a_arr.size == 1 and n > 1 else 1
+    sb = 0 if b_arr.size == 1 and n > 1 else 1
+    y = np.empty(out_shape, dtype=np.float32)
+    if lib.orc_binary(name.encode(), fp(a_arr), sa, fp(b_arr), sb, fp(y), n) != 0:
+        raise KeyError(name)
+    return y
+
+
+def round_to_int(x):
+    x = _c32(x)
+    y = np.empty(x.shape, dtype=np.int32)
+    lib.orc_round_to_int(fp(x), ip(y), x.size)
+    return y
+
+
+def chain(a, b, c, d):
+    a, b, c, d = map(_c32, (a, b, c, d))
+    y = np.empty_like(a)
+    lib.orc_chain(fp(a), fp(b), fp(c), fp(d), fp(y), a.size)
+    return y
+
+
+def axis_reduce(reducer, x, axis):
+    """Reduce a 2-D array along `axis` (0 walks the transposed strided view, as the reference does)."""
+    x = _c32(x)
+    rows, cols = x.shape
+    if axis in (1, -1):
+        out = np.empty(rows, dtype=np.float32)
+        lib.orc_axis_reduce(reducer, fp(x), rows, cols, cols, 1, fp(out))
+    else:
+        out = np.empty(cols, dtype=np.float32)
+        lib.orc_axis_reduce(reducer, fp(x), cols, rows, 1, cols, fp(out))
+    return out
+
+
+def all_reduce(reducer, x):
+    x = _c32(x)
+    return np.float32(lib.orc_all_reduce(reducer, fp(x), x.size))
+
+
+def arg_axis_reduce(reducer, x, axis):
+    x = _c32(x)
+    rows, cols = x.shape
+    if axis in (1, -1):
+        out = np.empty(rows, dtype=np.int32)
+        lib.orc_arg_axis_reduce(reducer, fp(x), rows, cols, cols, 1, ip(out))
+    else:
+        out = np.empty(cols, dtype=np.int32)
+        lib.orc_arg_axis_reduce(reducer, fp(x), cols, rows, 1, cols, ip(out))
+    return out
+
+
+def arg_all_reduce(reducer, x):
+    x = _c32(x)
+    return int(lib.orc_arg_all_reduce(reducer, fp(x), x.size))
+
+
+def mean_all(x):
+    x = _c32(x)
+    return np.float32(lib.orc_mean_all(fp(x), x.size))
+
+
+def softmax(a):
+    a = _c32(a)
+    rows = int(np.prod(a.shape[:-1])) if a.ndim > 1 else 1
+    cols = a.shape[-1]
+    out = np.empty_like(a)
+    lib.orc_softmax(fp(a), fp(out), rows, cols)
+    return out
+
+
+def gather_from_rows(source, indices):
+    source = _c32(source)
+    indices = np.ascontiguousarray(indices, dtype=np.int32)
+    out = np.empty(indices.shape[0], dtype=np.float32)
+    lib.orc_gather_from_rows(fp(source), source.shape[1], ip(indices), indices.shape[0], fp(out))
+    return out
+
+
+def one_hot(indices, depth, on=1.0, off=0.0):
+    indices = np.ascontiguousarray(indices, dtype=np.int32)
+    out = np.empty(indices.shape + (depth,), dtype=np.float32)
+    lib.orc_one_hot(ip(indices), indices.size, depth, on, off, fp(out))
+    return out
+
+
+def softmax_cross_entropy(x, t, want_grad=True):
+    x = _c32(x)
+    t = np.ascontiguousarray(t, dtype=np.int32)
+    rows, cols = x.shape
+    loss_rows = np.empty(rows, dtype=np.float32)
+    grad = np.empty_like(x) if want_grad else None
+    mean = C.c_float()
+    lib.orc_softmax_cross_entropy(fp(x), ip(t), rows, cols, fp(loss_rows), fp(grad) if want_grad else None, C.byref(mean))
+    return np.float32(mean.value), loss_rows, grad
+
+
+def softmax_cross_entropy_via_probs(x, t):
+    x = _c32(x)
+    t = np.ascontiguousarray(t, dtype=np.int32)
+    out = np.empty(x.shape[0], dtype=np.float32)
+    lib.orc_softmax_cross_entropy_via_probs(fp(x), ip(t), x.shape[0], x.shape[1], fp(out))
+    return out
+
+
+def _strides(a):
+    return a.strides[0] // a.itemsize, a.strides[1] // a.itemsize
+
+
+def gemm(A, B, mode="f64"):
+    """C = A @ B for 2-D float32 arrays of any (row, col) strides."""
+    assert A.dtype == np.float32 and B.dtype == np.float32
+    M, K = A.shape
+    N = B.shape[1]
+    Cm = np.empty((M, N), dtype=np.float32)
+    ars, acs = _strides(A)
+    brs, bcs = _strides(B)
+    fn = lib.orc_gemm_f64acc if mode == "f64" else lib.orc_gemm_f32seq
+    fn(A.ctypes.data_as(_f), ars, acs, B.ctypes.data_as(_f), brs, bcs, fp(Cm), N, M, N, K)
+    return Cm
+
+
+def gemm_i32(A, B):
+    M, K = A.shape
+    N = B.shape[1]
+    Cm = np.empty((M, N), dtype=np.int32)
+    ars, acs = _strides(A)
+    brs, bcs = _strides(B)
+    lib.orc_gemm_i32(A.ctypes.data_as(_i32), ars, acs, B.ctypes.data_as(_i32), brs, bcs, ip(Cm), N, M, N, K)
+    return Cm
+
+
+def lstm_step(X, H, Cm, W, U, b, f64_gemm=True):
+    X, H, Cm, W, U, b = map(_c32, (X, H, Cm, W, U, b))
+    B, I = X.shape
+    Hd = H.shape[1]
+    gates = np.empty((B, 4 * Hd), dtype=np.float32)
+    c_new = np.empty((B, Hd), dtype=np.float32)
+    h_new = np.empty((B, Hd), dtype=np.float32)
+    lib.orc_lstm_step(fp(X), fp(H), fp(Cm), fp(W), fp(U), fp(b), B, I, Hd, 1 if f64_gemm else 0, fp(gates), fp(c_new), fp(h_new))
+    return gates, c_new, h_new
