@@ -354,6 +354,8 @@ bool classify(Program& P, int id, Cls want, const Domain& dom) {
             if (dom.flat) return false;
             if (want == Cls::SCAL && dom.R == 1) {
                 // single-row domain: the row value is also the scalar
+            } else if (want == Cls::FULL && dom.C == 1) {
+                // single-column domain: one element per row, the row value is the element
             } else if (want != Cls::ROW) {
                 return false;
             }
@@ -363,7 +365,7 @@ bool classify(Program& P, int id, Cls want, const Domain& dom) {
             return classify(P, c, Cls::FULL, dom);
         }
         case Kind::GATHER_FROM_ROWS: {
-            if (want != Cls::ROW) return false;
+            if (want != Cls::ROW && !(want == Cls::FULL && dom.C == 1)) return false;
             int src = n.args[0], idx = n.args[1];
             if (P.nodes[src].kind != Kind::BUFFER) return false;
             if (P.nodes[src].shape.size() != 2 || P.nodes[src].shape[0] < dom.R) return false;
@@ -2095,6 +2097,11 @@ void run_specs(std::vector<DestSpec> specs) {
         if (!has_red) {
             if (try_flat(specs)) return;
             Domain dom = domain_of(specs[0].dest.shape());
+            if (specs[0].dest.ndim() <= 1 && has_kind(specs[0].root, [](Kind k) { return k == Kind::GATHER_FROM_ROWS; })) {
+                // one gathered element per row: a single-column domain
+                dom.R = numel_of(specs[0].dest.shape());
+                dom.C = 1;
+            }
             if (try_row(specs, dom)) return;
             if (try_generic(specs)) return;
             if (specs.size() > 1) {

@@ -1,0 +1,172 @@
+"""CPU-side checks: the C-ABI libraries load and export every declared symbol,
+the host front-end's shape/dtype logic and error behaviour, and the planner +
+code generator for the five benchmark configurations (generated HIP is compiled
+for gfx950 with hipRTC; nothing is launched)."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dali_(?:hip|fe)_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_hip_library_exports_every_declared_symbol(D):
+    from dali_amd._native import hip, HIP_SYMBOLS
+    names = declared_functions("dali_hip.h")
+    assert len(names) >= 29
+    for n in names:
+        assert hasattr(hip, n), "libdali_hip.so does not export %s" % n
+        assert n in HIP_SYMBOLS, "binding table misses %s" % n
+
+
+def test_front_library_exports_every_declared_symbol(D):
+    from dali_amd._native import front, FRONT_SYMBOLS
+    names = declared_functions("dali_front.h")
+    assert len(names) >= 45
+    for n in names:
+        assert hasattr(front, n), "libdali_front.so does not export %s" % n
+        assert n in FRONT_SYMBOLS, "binding table misses %s" % n
+
+
+def test_launch_plan_struct_layout_matches_header(D):
+    from dali_amd._native import LaunchPlan
+    text = open(os.path.join(ROOT, "include", "dali_hip.h")).read()
+    body = re.search(r"typedef struct dali_hip_launch_plan \{(.*?)\} dali_hip_launch_plan;", text, re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = re.findall(r"(?:const\s+)?int32_t\s*\*?\s*([a-z0-9_]+);", body)
+    assert fields == [f[0] for f in LaunchPlan._fields_]
+
+
+def test_compile_only_reports_errors_without_exiting(D):
+    from dali_amd._native import hip
+    size = C.c_size_t()
+    ok = b'extern "C" __global__ void k(float* a) { a[threadIdx.x] = 1.0f; }'
+    assert hip.dali_hip_compile_only(ok, C.byref(size)) == 0 and size.value > 0
+    bad = b'extern "C" __global__ void k(float* a) { a[0] = functor::nope<float>::Map(1.0f); }'
+    assert hip.dali_hip_compile_only(bad, C.byref(size)) != 0
+    msg = hip.dali_hip_last_error().decode()
+    assert "hipRTC" in msg and "nope" in msg  # the compiler log travels with the error (compiler.h:147-150 keeps only a log path)
+
+
+# ------------------------------------------------------------ host front-end
+def test_lazy_until_evaluated_and_shapes(D, rng):
+    op = D.op
+    a = D.Array.from_numpy(rng.randn(3, 5).astype(np.float32))
+    before = D.jit_stats()
+    e = op.exp(a - op.max(a, [-1], True))
+    s = e / op.sum(e, [-1], True)
+    assert not s.is_buffer() and s.shape == (3, 5) and s.dtype == D.DTYPE_FLOAT
+    assert op.sum(a, [0]).shape == (5,) and op.sum(a, [1], True).shape == (3, 1) and op.sum(a).shape == ()
+    assert op.argmax(a, 1).dtype == D.DTYPE_INT32 and op.argmax(a, 0).shape == (5,)
+    assert op.argmax(a).dtype == D.DTYPE_FLOAT  # flat argmax keeps the input dtype (reducer_operation.cpp:681-684)
+    assert op.dot(a, a.T).shape == (3, 3)
+    assert op.one_hot(D.Array.from_numpy(np.zeros(4, np.int32)), 7, 1.0, 0.0).shape == (4, 7)
+    assert D.jit_stats() == before  # nothing ran
+
+
+def test_type_promotion_and_errors(D, rng):
+    op = D.op
+    f = D.Array.from_numpy(rng.randn(2, 3).astype(np.float32))
+    i = D.Array.from_numpy(np.arange(6, dtype=np.int32).reshape(2, 3))
+    d = D.Array.from_numpy(rng.randn(2, 3))
+    assert (f + i).dtype == D.DTYPE_FLOAT and (f + d).dtype == D.DTYPE_DOUBLE and (i + i).dtype == D.DTYPE_INT32
+    assert (i * 2.5).dtype == D.DTYPE_INT32  # array (op) scalar keeps the array dtype (array.cpp:845-865)
+    assert op.mean(i).dtype == D.DTYPE_DOUBLE  # reducers.cpp:32-36
+    with pytest.raises(D.DaliError, match="same rank"):
+        f + D.Array.from_numpy(rng.randn(3).astype(np.float32))
+    with pytest.raises(D.DaliError, match="common shape"):
+        f + D.Array.from_numpy(rng.randn(2, 4).astype(np.float32))
+    with pytest.raises(D.DaliError, match="duplicate axes"):
+        op.sum(f, [0, 0])
+    with pytest.raises(D.DaliError, match="Reduction axis"):
+        op.sum(f, [2])
+    with pytest.raises(D.DaliError, match="indices must be integers"):
+        op.gather_from_rows(f, f)
+    with pytest.raises(D.DaliError, match="not aligned"):
+        op.dot(f, f)
+    with pytest.raises(D.DaliError, match="depth must be strictly positive"):
+        op.one_hot(i, 0, 1.0, 0.0)
+
+
+def test_view_algebra_matches_numpy_strides(D, rng):
+    x = rng.randn(4, 6, 5).astype(np.float32)
+    a = D.Array.from_numpy(x)
+
+    def same(view, ref):
+        assert view.shape == ref.shape
+        assert [s * 4 for s in view.strides] == [st if n > 1 else view.strides[k] * 4 for k, (st, n) in enumerate(zip(ref.strides, ref.shape))]
+        assert view.offset * 4 == ref.__array_interface__["data"][0] - x.__array_interface__["data"][0]
+
+    same(a.transpose(), x.transpose())
+    same(a.transpose(1, 0, 2), x.transpose(1, 0, 2))
+    same(a[1], x[1])
+    same(a[:, 2:5], x[:, 2:5])
+    same(a[:, ::2, 1:4], x[:, ::2, 1:4])
+    same(a.reshape(24, 5), x.reshape(24, 5))
+    assert a[:, 2:5].contiguous_memory() is False and a[1].contiguous_memory() is True
+    assert a.expand_dims(1).shape == (4, 1, 6, 5)
+
+
+# ------------------------------------------------- planner + code generation
+def _cfg_roots(D, rng, small=True):
+    op = D.op
+    f = lambda *s: D.Array.from_numpy(rng.randn(*s).astype(np.float32))
+    cfgs = {}
+    a, b, c, d = f(4096), f(4096), f(4096), f(4096)
+    cfgs["c2_chain"] = ([op.sigmoid(a) * op.tanh(b) + c * d - 0.5 * op.square(a)], "flat")
+    cfgs["c1_softmax"] = ([op.softmax(f(64, 1024))], "row")
+    m = f(128, 256)
+    cfgs["c3_sum_axis1"] = ([op.sum(m, [1])], "row")
+    cfgs["c3_max_axis0"] = ([op.max(m, [0])], "col")
+    cfgs["c3_sum_all"] = ([op.sum(m)], "all")
+    cfgs["c3_argmax_axis1"] = ([op.argmax(m, 1)], "row")
+    x, t = f(16, 32000), D.Array.from_numpy(rng.randint(0, 32000, 16).astype(np.int32))
+    mx = op.max(x, [-1], True)
+    ex = op.exp(x - mx)
+    s = op.sum(ex, [-1], True)
+    grad = ex / s - op.one_hot(t, 32000, np.float32(1), np.float32(0))
+    row_loss = (op.log(s) + mx) - op.gather_from_rows(x, t).expand_dims(1)
+    cfgs["c4_cross_entropy"] = ([grad, row_loss], "row")
+    pre, bias, cell = f(8, 4 * 64), f(4 * 64), f(8, 64)
+    g = lambda k: pre[:, k * 64:(k + 1) * 64] + bias[k * 64:(k + 1) * 64].expand_dims(0)
+    cn = op.sigmoid(g(1)) * cell + op.sigmoid(g(0)) * op.tanh(g(3))
+    cfgs["c5_lstm_gates"] = ([cn, op.sigmoid(g(2)) * op.tanh(cn)], "map2d")
+    return cfgs
+
+
+def test_five_configs_plan_into_single_fused_kernels_that_compile(D, rng):
+    for name, (roots, kind) in _cfg_roots(D, rng).items():
+        n = D.generate_only(roots, compile=True)  # hipRTC for gfx950, no device needed
+        assert (n, D.last_kernel_kinds()) == (1, kind), name
+        src = D.last_source()
+        assert 'extern "C" __global__' in src and "KArgs" in src, name
+
+
+def test_softmax_kernel_reads_the_row_once_and_keeps_exp_in_registers(D, rng):
+    roots, _ = _cfg_roots(D, rng)["c1_softmax"]
+    D.generate_only(roots)
+    src = D.last_source()
+    body = src[src.index("dali_row_kernel"):]
+    assert body.count("dali_load<float, 4>(q1") == 1  # one global read of the input
+    assert body.count("functor::exp<float>::Map") == 1  # exp computed once, reused from registers
+    assert "dali_group_reduce<reducers::maximum, float, 64>" in body  # wave64 cross-lane reduction
+
+
+def test_planner_splits_what_cannot_fuse(D, rng):
+    op = D.op
+    m = D.Array.from_numpy(rng.randn(6, 8).astype(np.float32))
+    n = D.generate_only([2 + (op.sum(m) - op.max(m))])
+    assert D.last_kernel_kinds().split(",").count("all") == 2 and n == 3
+    x3 = D.Array.from_numpy(rng.randn(3, 4, 5).astype(np.float32))
+    D.generate_only([op.sum(x3, [1])], compile=True)
+    assert D.last_kernel_kinds() == "generic,row"  # middle axis: strided copy, then a trailing-axis reduction
+    D.generate_only([op.mean(m)], compile=True)
+    assert D.last_kernel_kinds() == "all"  # the division by the count is folded into the last block

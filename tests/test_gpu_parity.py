@@ -1,0 +1,490 @@
+"""Parity of the HIP path against the CPU checker, on a real MI355X.
+
+Everything here goes through the C ABI (include/dali_hip.h): either directly
+(memory, raw module load + six-array launch, sgemm) or through the C++ front-end,
+which plans, generates HIP source and calls dali_hip_module_load / dali_hip_launch.
+
+Tolerances (fp32): elementwise, softmax, log-sum-exp, gradients: rel 1e-5 (+ atol
+1e-6 near zero); sums: |gpu - cpu| <= 1e-5 * sum|x| over the reduced set (the CPU
+reference accumulates sequentially, a tree is differently rounded); GEMM: rel 1e-4
+of max|C| against an fp64-accumulated product. Index results (argmax, gather,
+one_hot, astype) are bit-exact.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from conftest import golden
+
+pytestmark = pytest.mark.gpu
+
+FLT_MAX = np.finfo(np.float32).max
+
+
+def arr(D, x):
+    return D.Array.from_numpy(np.asarray(x))
+
+
+def close(got, want, rtol=1e-5, atol=1e-6):
+    np.testing.assert_allclose(np.asarray(got, np.float64), np.asarray(want, np.float64), rtol=rtol, atol=atol)
+
+
+def seq_sum_rtol(n):
+    """Tolerance against the CPU checker for a value normalised by a length-n fp32 sum of positive terms.
+
+    The reference accumulates left to right in fp32; its own a-priori error bound is (n - 1) * 2^-24 (and long
+    rows do lose small terms to stagnation), while the GPU folds a tree. Against fp64 truth the GPU result is
+    held to a plain rel 1e-5; against the sequential checker the checker's bound is added."""
+    return 1e-5 + (n - 1) * 2.0 ** -24
+
+
+# ------------------------------------------------------------ C ABI directly
+def test_memory_abi_roundtrip_and_bank(gpu, rng):
+    hip = gpu
+    n = 1 << 20
+    host = rng.randn(n).astype(np.float32)
+    p, q = C.c_void_p(), C.c_void_p()
+    assert hip.dali_hip_malloc(C.byref(p), n * 4) == 0 and hip.dali_hip_malloc(C.byref(q), n * 4) == 0
+    assert hip.dali_hip_memcpy_h2d(p, host.ctypes.data_as(C.c_void_p), n * 4) == 0
+    assert hip.dali_hip_memcpy_d2d(q, p, n * 4) == 0
+    back = np.empty_like(host)
+    assert hip.dali_hip_memcpy_d2h(back.ctypes.data_as(C.c_void_p), q, n * 4) == 0
+    assert np.array_equal(back, host)
+    assert hip.dali_hip_memset_async(q, 0, n * 4) == 0
+    assert hip.dali_hip_memcpy_d2h(back.ctypes.data_as(C.c_void_p), q, n * 4) == 0
+    assert not back.any()
+    assert hip.dali_hip_free(p) == 0 and hip.dali_hip_free(q) == 0
+    # size-keyed bank: a deposited block is handed out again for the same size (memory_bank.cpp:40-64)
+    a, b = C.c_void_p(), C.c_void_p()
+    assert hip.dali_hip_bank_allocate(C.byref(a), 12345 * 4) == 0
+    assert hip.dali_hip_bank_deposit(a, 12345 * 4) == 0
+    assert hip.dali_hip_bank_allocate(C.byref(b), 12345 * 4) == 0
+    assert a.value == b.value
+    assert hip.dali_hip_bank_deposit(b, 12345 * 4) == 0
+    free_b, total_b = C.c_size_t(), C.c_size_t()
+    assert hip.dali_hip_mem_info(C.byref(free_b), C.byref(total_b)) == 0 and total_b.value > (100 << 30)
+    name, arch = C.create_string_buffer(128), C.create_string_buffer(64)
+    assert hip.dali_hip_device_name(0, name, 128, arch, 64) == 0 and arch.value.startswith(b"gfx950")
+
+
+def test_raw_module_load_and_six_array_launch(gpu, rng):
+    """A hand-written kernel in the generated-kernel convention, driven with the reference's six arrays."""
+    from dali_amd._native import LaunchPlan
+    hip = gpu
+    src = b"""
+    union dali_slot { int i; float f; double d; };
+    struct KArgs { void* ws; void* p[2]; dali_slot s[2]; int iv[3]; };
+    extern "C" __global__ void saxpb(KArgs A) {
+        // dst[i] = s0 * src[i * stride] + s1 ; iv = {n_dst, n_src, stride_src}
+        long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+        if (i < A.iv[0]) ((float*)A.p[0])[i] = A.s[0].f * ((const float*)A.p[1])[i * A.iv[2]] + (float)A.s[1].d;
+    }"""
+    n = 1000
+    i32 = lambda *v: (C.c_int32 * len(v))(*v)
+    plan = LaunchPlan(n_arrays=2, n_scalars=2, n_shapes=0, array_ndim=i32(1, 1), array_strided=i32(0, 1), array_elsize=i32(4, 4),
+                      scalar_dtype=i32(0, 1), shape_ndim=None, block_threads=256, grid_kind=0, work_begin=0, work_count=1,
+                      work_per_block=256, max_blocks=0)
+    cached = C.c_int(-1)
+    h = 0xD411D411D411
+    assert hip.dali_hip_module_load(h, src, b"saxpb", C.byref(plan), C.byref(cached)) == 0, hip.dali_hip_last_error()
+    assert cached.value in (0, 1) and hip.dali_hip_module_is_loaded(h) == 1
+    assert hip.dali_hip_module_load(h, None, b"saxpb", C.byref(plan), C.byref(cached)) == 0 and cached.value == 2
+    host = rng.randn(2 * n + 7).astype(np.float32)
+    dsrc, ddst = C.c_void_p(), C.c_void_p()
+    hip.dali_hip_malloc(C.byref(dsrc), host.nbytes)
+    hip.dali_hip_malloc(C.byref(ddst), n * 4)
+    hip.dali_hip_memcpy_h2d(dsrc, host.ctypes.data_as(C.c_void_p), host.nbytes)
+    data = (C.c_void_p * 2)(ddst, dsrc)
+    offsets = i32(0, 5)  # element offset of the source view
+    sizes = (C.POINTER(C.c_int) * 2)(i32(n), i32(n))
+    strides = (C.POINTER(C.c_int) * 2)(None, i32(2))
+    s0, s1 = C.c_float(1.5), C.c_double(-0.25)
+    scalars = (C.c_void_p * 2)(C.cast(C.byref(s0), C.c_void_p), C.cast(C.byref(s1), C.c_void_p))
+    assert hip.dali_hip_launch(h, data, offsets, sizes, strides, scalars, None) == 0, hip.dali_hip_last_error()
+    out = np.empty(n, np.float32)
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), ddst, n * 4)
+    assert np.array_equal(out, np.float32(1.5) * host[5:5 + 2 * n:2] + np.float32(-0.25))
+    # error paths return a status and a message, never exit (compiler.h:81-88 exits)
+    assert hip.dali_hip_launch(0x1234, data, offsets, sizes, strides, scalars, None) != 0
+    assert b"no module" in hip.dali_hip_last_error()
+    assert hip.dali_hip_module_load(0x77, b"this is not HIP", b"k", C.byref(plan), None) != 0
+    hip.dali_hip_free(dsrc)
+    hip.dali_hip_free(ddst)
+
+
+def _dev(hip, a):
+    p = C.c_void_p()
+    assert hip.dali_hip_malloc(C.byref(p), max(a.nbytes, 4)) == 0
+    assert hip.dali_hip_memcpy_h2d(p, a.ctypes.data_as(C.c_void_p), a.nbytes) == 0
+    return p
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (5, 11, 7), (64, 64, 64), (65, 130, 33), (256, 4096, 128), (300, 200, 100)])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
+    """dali_hip_sgemm(transB, transA, m, n, k, alpha, B, ldb, A, lda, beta, C, ldc) as cublasSgemm is called in
+    cublas_gemm.cu:153-166: row-major C[n, m] = alpha * A[n, k] . B[k, m] + beta * C."""
+    hip = gpu
+    A = rng.randn(M, K).astype(np.float32)  # row-major lhs  (n = M rows)
+    B = rng.randn(K, N).astype(np.float32)  # row-major rhs  (m = N cols)
+    C0 = rng.randn(M, N + 3).astype(np.float32)  # padded destination rows: ldc = N + 3
+    Astore = np.ascontiguousarray(A.T) if ta else A
+    Bstore = np.ascontiguousarray(B.T) if tb else B
+    lda = Astore.shape[1]
+    ldb = Bstore.shape[1]
+    dA, dB, dC = _dev(hip, Astore), _dev(hip, Bstore), _dev(hip, C0)
+    alpha, beta = 0.75, -0.5
+    st = hip.dali_hip_sgemm(tb, ta, N, M, K, alpha, dB, ldb, dA, lda, beta, dC, N + 3)
+    assert st == 0, hip.dali_hip_last_error()
+    out = np.empty_like(C0)
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+    want = alpha * (A.astype(np.float64) @ B.astype(np.float64)) + beta * C0[:, :N]
+    scale = np.abs(want).max() + 1e-6
+    assert np.abs(out[:, :N] - want).max() <= 1e-4 * scale
+    assert np.array_equal(out[:, N:], C0[:, N:])  # padding untouched
+    for p in (dA, dB, dC):
+        hip.dali_hip_free(p)
+
+
+def test_sgemm_pair_accumulates_two_products(gpu, rng):
+    hip = gpu
+    M, N, K1, K2 = 48, 200, 96, 40
+    A1, B1 = rng.randn(M, K1).astype(np.float32), rng.randn(K1, N).astype(np.float32)
+    A2, B2 = rng.randn(M, K2).astype(np.float32), rng.randn(K2, N).astype(np.float32)
+    dA1, dB1, dA2, dB2 = (_dev(hip, x) for x in (A1, B1, A2, B2))
+    out = np.zeros((M, N), np.float32)
+    dC = _dev(hip, out)
+    st = hip.dali_hip_sgemm_pair(0, 0, 0, 0, N, M, K1, K2, 1.0, dB1, N, dA1, K1, dB2, N, dA2, K2, 0.0, dC, N)
+    assert st == 0, hip.dali_hip_last_error()
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, out.nbytes)
+    want = A1.astype(np.float64) @ B1 + A2.astype(np.float64) @ B2
+    assert np.abs(out - want).max() <= 1e-4 * np.abs(want).max()
+    assert hip.dali_hip_sgemm(0, 0, N, M, K1, 1.0, dB1, N - 1, dA1, K1, 0.0, dC, N) != 0  # ld smaller than the row
+    for p in (dA1, dB1, dA2, dB2, dC):
+        hip.dali_hip_free(p)
+
+
+# ---------------------------------------------------------------- functors
+UNARY = ["sigmoid", "tanh", "exp", "log", "negative_log", "square", "cube", "sqrt_f", "rsqrt", "inv", "identity", "abs", "sign",
+         "relu", "relu_backward", "dsigmoid", "dtanh", "softplus", "softplus_backward", "log_or_zero", "isnotanumber", "isinfinity",
+         "safe_entropy_log"]
+
+
+@pytest.mark.parametrize("name", UNARY)
+def test_unary_functors_match_oracle(gpu, D, O, name):
+    # tests.cpp:1015-1073 uses (arange(50) + 1).reshape(5, 10); a signed and a (0, 1) range widen it
+    xs = [(np.arange(50, dtype=np.float32) + 1).reshape(5, 10), np.linspace(-6, 6, 1003).astype(np.float32),
+          np.linspace(0.02, 0.98, 257).astype(np.float32)]
+    if name in ("log", "negative_log", "sqrt_f", "rsqrt", "inv"):
+        xs = [xs[0], xs[2]]
+    if name == "exp":
+        xs = [xs[1], xs[2]]
+    for x in xs:
+        got = D.op.elementwise(name, arr(D, x)).numpy()
+        close(got, O.unary(name, x).reshape(x.shape), rtol=1e-5, atol=1e-6)
+
+
+def test_binary_functors_scalars_and_promotion(gpu, D, O, rng):
+    op = D.op
+    a = rng.uniform(-3, 3, (7, 9)).astype(np.float32)
+    b = rng.uniform(0.5, 3, (7, 9)).astype(np.float32)
+    A, B = arr(D, a), arr(D, b)
+    for name in ["add", "subtract", "eltmul", "eltdiv", "equals", "max_scalar", "min_scalar", "prelu", "clip", "div_grad", "threshold"]:
+        close(op.elementwise(name, A, B).numpy(), O.binary(name, a, b), rtol=1e-5)
+    close(op.pow(arr(D, np.abs(a) + 0.1), B).numpy(), O.binary("power", np.abs(a) + np.float32(0.1), b), rtol=1e-5)
+    # array (op) scalar, both orders (tests.cpp:1075-1117); the double literal is cast to the array dtype
+    close((A - 2.5).numpy(), O.binary("subtract", a, 2.5))
+    close((2.5 - A).numpy(), O.binary("subtract", 2.5, a))
+    close((A / 3).numpy(), O.binary("eltdiv", a, 3.0))
+    close((-A).numpy(), -a, rtol=0, atol=0)
+    # int32 arithmetic and astype rounding floor(x + 0.5) (tests.cpp:854-872)
+    g = golden("reference_known_answers.json")["astype_round"]
+    assert op.astype(arr(D, np.array(g["input"], np.float32)), D.DTYPE_INT32).numpy().tolist() == g["expected"]
+    i = np.arange(12, dtype=np.int32).reshape(3, 4)
+    assert np.array_equal((arr(D, i) * arr(D, i) + 3).numpy(), i * i + 3)
+    assert (arr(D, i) + A[:3, :4]).dtype == D.DTYPE_FLOAT
+    d = rng.randn(3, 4)
+    close((arr(D, d) * 2.0 + arr(D, i)).numpy(), d * 2.0 + i, rtol=1e-12, atol=0)  # fp64 path
+    # broadcast [3,1] + [3,5] and [1,5] + [3,5] (tests.cpp:1599-1620)
+    col, rowv, full = rng.randn(3, 1).astype(np.float32), rng.randn(1, 5).astype(np.float32), rng.randn(3, 5).astype(np.float32)
+    assert np.array_equal((arr(D, col) + arr(D, full)).numpy(), col + full)
+    assert np.array_equal((arr(D, rowv) * arr(D, full)).numpy(), rowv * full)
+
+
+def test_chain_small_and_ragged(gpu, D, O, rng):
+    op = D.op
+    for n in (1, 3, 1000, 4099, 1 << 16):
+        a, b, c, d = [rng.uniform(-4, 4, n).astype(np.float32) for _ in range(4)]
+        A, B, Cc, Dd = (arr(D, v) for v in (a, b, c, d))
+        y = (op.sigmoid(A) * op.tanh(B) + Cc * Dd - 0.5 * op.square(A)).numpy()
+        assert D.last_kernel_kinds() == "flat"
+        scale = np.abs(np.tanh(b)) + np.abs(c * d) + 0.5 * a * a
+        assert np.all(np.abs(y - O.chain(a, b, c, d)) <= 1e-5 * scale + 1e-6)
+    assert op.exp(arr(D, np.zeros((0,), np.float32))).numpy().shape == (0,)  # empty input
+
+
+def test_assignment_operators_and_strided_views(gpu, D, rng):
+    """BinaryTests.add / add_strided / add_strided_nd / chained_add (tests.cpp:1410-1528, 1580-1597)."""
+    op = D.op
+    x = rng.randn(6, 10).astype(np.float32)
+    y = rng.randn(6, 10).astype(np.float32)
+    for k, f in enumerate([lambda u, v: v, lambda u, v: u + v, lambda u, v: u - v, lambda u, v: u * v, lambda u, v: u / v]):
+        dst = arr(D, x)
+        dst.assign(arr(D, y) * 2.0, k)
+        close(dst.numpy(), f(x, y * 2.0), rtol=1e-6)
+    # strided destination and sources
+    dst, want = arr(D, x), x.copy()
+    dst[::2, 1:9:3].assign(arr(D, y)[1::2, 0:9:3] + 1.0, 1)
+    want[::2, 1:9:3] += y[1::2, 0:9:3] + 1.0
+    assert np.array_equal(dst.numpy(), want)
+    # N-D strided, transposed operands
+    z = rng.randn(3, 4, 5).astype(np.float32)
+    assert np.array_equal((arr(D, z).transpose(2, 0, 1) + arr(D, z.transpose(2, 0, 1).copy())).numpy(), 2 * z.transpose(2, 0, 1))
+    assert np.array_equal(arr(D, z)[:, 1:3, ::2].ascontiguousarray().numpy(), z[:, 1:3, ::2])
+    # a chain of additions is one kernel
+    before = D.jit_stats()["kernels"]
+    s = (arr(D, x) + arr(D, y) + arr(D, x) + arr(D, y)).numpy()
+    assert D.jit_stats()["kernels"] - before == 1
+    close(s, 2 * (x + y), rtol=1e-6)
+    # scalar fill
+    f = D.Array.empty((4, 7))
+    f.assign(3.25)
+    assert np.array_equal(f.numpy(), np.full((4, 7), 3.25, np.float32))
+
+
+# ---------------------------------------------------------------- reducers
+def sum_tol(x, axis=None):
+    return 1e-5 * np.abs(np.asarray(x, np.float64)).sum(axis=axis) + 1e-6
+
+
+def test_reducer_closed_forms(gpu, D):
+    op = D.op
+    g = golden("reference_known_answers.json")
+    for n in (1, 2, 5, 100, 1000):
+        assert float(op.sum(arr(D, np.arange(n, dtype=np.float32))).numpy()) == n * (n - 1) / 2
+        assert int(op.sum(arr(D, np.arange(n, dtype=np.int32))).numpy()) == n * (n - 1) // 2
+    assert float(op.prod(arr(D, np.array(g["all_reduce_prod"]["input"], np.float32))).numpy()) == 120
+    mm = arr(D, np.array(g["all_reduce_max_min"]["input"], np.float32))
+    assert float(op.max(mm).numpy()) == 41 and float(op.min(mm).numpy()) == -100
+    a = g["axis_argmax_argmin"]
+    x = arr(D, np.arange(20, dtype=np.float32).reshape(4, 5))
+    assert op.argmax(x, 0).numpy().tolist() == a["argmax_axis0"] and op.argmax(x, 1).numpy().tolist() == a["argmax_axis1"]
+    assert op.argmin(x, 0).numpy().tolist() == a["argmin_axis0"] and op.argmin(x, 1).numpy().tolist() == a["argmin_axis1"]
+    ramp = arr(D, np.arange(-100, 42, dtype=np.float32))
+    assert float(op.argmax(ramp).numpy()) == 141 and float(op.argmin(ramp).numpy()) == 0
+    r4 = arr(D, np.arange(120, dtype=np.float32).reshape(2, 3, 4, 5))
+    assert float(op.argmax(r4).numpy()) == 119 and float(op.argmin(r4).numpy()) == 0
+    # reductions of ones over low / high / middle / several axes (tests.cpp:1215-1239)
+    ones = arr(D, np.ones((2, 3, 4, 5), np.float32))
+    for axes in ([3], [0], [1], [2], [2, 3], [0, 1], [1, 2], [0, 3], [0, 1, 2]):
+        want = np.ones((2, 3, 4, 5)).sum(axis=tuple(axes))
+        assert np.array_equal(op.sum(ones, axes).numpy(), want), axes
+        assert op.sum(ones, axes, True).shape == np.ones((2, 3, 4, 5)).sum(axis=tuple(axes), keepdims=True).shape
+    # mean promotes int to double, L2 norm (tests.cpp:1166-1178)
+    assert float(op.mean(arr(D, np.arange(10, dtype=np.int32))).numpy()) == 4.5
+    assert float(op.sqrt(op.sum(op.square(arr(D, np.array([3.0, 4.0], np.float32))))).numpy()) == 5.0
+    # mixed expression with two full reductions (tests.cpp:1198-1204)
+    av, bv = np.arange(6, dtype=np.float32), np.arange(9, dtype=np.float32) - 3
+    assert float((2 + (op.sum(arr(D, av)) - op.max(arr(D, bv)))).numpy()) == 2 + (15 - 5)
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (1, 7), (9, 1), (37, 53), (64, 1000), (33, 4096), (5, 10001), (300, 517), (3, 70000)])
+def test_axis_and_all_reductions_match_oracle(gpu, D, O, rng, shape):
+    op = D.op
+    x = rng.randn(*shape).astype(np.float32)
+    X = arr(D, x)
+    for name, red in (("sum", O.SUM), ("max", O.MAX), ("min", O.MIN)):
+        f = getattr(op, name)
+        for axis in (0, 1):
+            got, want = f(X, [axis]).numpy(), O.axis_reduce(red, x, axis)
+            if red == O.SUM:
+                assert np.all(np.abs(got - want) <= sum_tol(x, axis)), (name, axis)
+                assert np.all(np.abs(got - x.astype(np.float64).sum(axis)) <= sum_tol(x, axis))
+            else:
+                assert np.array_equal(got, want), (name, axis)
+        got, want = f(X).numpy(), O.all_reduce(red, x)
+        assert abs(float(got) - float(want)) <= (float(sum_tol(x)) if red == O.SUM else 0.0)
+    for axis in (0, 1):
+        assert np.array_equal(op.argmax(X, axis).numpy(), O.arg_axis_reduce(O.MAX, x, axis))
+        assert np.array_equal(op.argmin(X, axis).numpy(), O.arg_axis_reduce(O.MIN, x, axis))
+    assert int(op.argmax(X).numpy()) == O.arg_all_reduce(O.MAX, x)
+    assert abs(float(op.mean(X).numpy()) - float(O.mean_all(x))) <= float(sum_tol(x)) / x.size + 1e-7
+
+
+def test_argmax_ties_and_sentinels_are_bit_exact(gpu, D, O, rng):
+    op = D.op
+    # few distinct values -> many ties; widths straddle the one-wave / multi-wave / streaming row layouts
+    for cols in (5, 64, 257, 1024, 4100, 70001):
+        x = rng.randint(0, 4, size=(23, cols)).astype(np.float32)
+        X = arr(D, x)
+        assert np.array_equal(op.argmax(X, 1).numpy(), O.arg_axis_reduce(O.MAX, x, 1)), cols
+        assert np.array_equal(op.argmin(X, 1).numpy(), O.arg_axis_reduce(O.MIN, x, 1)), cols
+        assert np.array_equal(op.argmax(X, 0).numpy(), O.arg_axis_reduce(O.MAX, x, 0)), cols
+        assert int(op.argmax(X).numpy()) == O.arg_all_reduce(O.MAX, x)
+        assert int(op.argmin(X).numpy()) == O.arg_all_reduce(O.MIN, x)
+    s = np.full((3, 300), -FLT_MAX, np.float32)
+    s[1, 200] = -1e30
+    s[2, :] = -np.inf
+    assert op.argmax(arr(D, s), 1).numpy().tolist() == O.arg_axis_reduce(O.MAX, s, 1).tolist() == [0, 200, 0]
+    assert np.array_equal(op.max(arr(D, s), [1]).numpy(), O.axis_reduce(O.MAX, s, 1))
+
+
+def test_reductions_over_strided_and_broadcast_inputs(gpu, D, O, rng):
+    """all_reduce_sum_with_broadcast / _with_strides, advanced_striding_with_reductions (tests.cpp:923-952, 1180-1213)."""
+    op = D.op
+    x = rng.randn(12, 40).astype(np.float32)
+    X = arr(D, x)
+    v = X[::2, 4:36:3]
+    nv = x[::2, 4:36:3]
+    assert np.all(np.abs(op.sum(v, [1]).numpy() - nv.astype(np.float64).sum(1)) <= sum_tol(nv, 1))
+    assert np.all(np.abs(op.sum(v, [0]).numpy() - nv.astype(np.float64).sum(0)) <= sum_tol(nv, 0))
+    assert abs(float(op.sum(v).numpy()) - nv.astype(np.float64).sum()) <= sum_tol(nv)
+    assert np.array_equal(op.max(X.T, [1]).numpy(), x.max(0))
+    b = arr(D, rng.randn(12, 1).astype(np.float32))
+    got = op.sum(X * b, [1]).numpy()
+    want = (x.astype(np.float64) * b.numpy()).sum(1)
+    assert np.all(np.abs(got - want) <= sum_tol(x * b.numpy(), 1))
+    # reduce of a fused elementwise expression, result fed through keepdims back into an elementwise op
+    centered = X - op.mean(X, [1], True)
+    close(centered.numpy(), x - x.astype(np.float64).mean(1, keepdims=True), rtol=1e-5, atol=1e-5)
+    assert D.last_kernel_kinds() == "row"
+
+
+# ----------------------------------------------------------------- softmax
+@pytest.mark.parametrize("shape", [(2, 5), (7, 33), (4, 1024), (64, 1000), (3, 32000), (2, 100003), (2, 3, 50)])
+def test_fused_softmax_matches_oracle(gpu, D, O, rng, shape):
+    x = (rng.randn(*shape) * 3).astype(np.float32)
+    before = D.jit_stats()["kernels"]
+    s = D.op.softmax(arr(D, x)).numpy()
+    assert D.jit_stats()["kernels"] - before == 1 and D.last_kernel_kinds() == "row"
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(-1, keepdims=True))
+    close(s, e / e.sum(-1, keepdims=True), rtol=1e-5, atol=1e-12)  # fp64 truth
+    close(s, O.softmax(x), rtol=seq_sum_rtol(shape[-1]), atol=1e-12)
+    close(s.sum(-1), 1.0, rtol=0, atol=2e-6)
+
+
+def test_fused_softmax_equals_staged(gpu, D, rng):
+    """JITCachedReduction.fused_softmax (tests.cpp:1622-1664): U(-20,20) [2,5], atol 1e-6."""
+    op = D.op
+    x = arr(D, rng.uniform(-20, 20, (2, 5)).astype(np.float32))
+    fused = op.softmax(x).numpy()
+    m = op.max(x, [-1], True)
+    m.eval()
+    e = op.exp(x - m)
+    e.eval()
+    s = op.sum(e, [-1], True)
+    s.eval()
+    staged = (e / s).numpy()
+    np.testing.assert_allclose(fused, staged, atol=1e-6, rtol=0)
+    sm0 = op.softmax(x, 0).numpy()  # softmax along the leading axis
+    close(sm0.sum(0), 1.0, rtol=0, atol=1e-6)
+
+
+# ------------------------------------------------- gather / one_hot / loss
+def test_gather_from_rows_and_one_hot(gpu, D, O, rng):
+    op = D.op
+    g = golden("reference_known_answers.json")["gather_from_rows_3d"]
+    src = np.arange(5 * 6 * 7, dtype=np.float32).reshape(5, 6, 7)
+    idx = arr(D, np.arange(5, dtype=np.int32))
+    table = np.stack([op.gather_from_rows(arr(D, np.ascontiguousarray(src[:, :, j])), idx).numpy() for j in range(7)], 1)
+    assert table.astype(np.int64).tolist() == g["expected"]
+    s2 = rng.randn(40, 13).astype(np.float32)
+    i2 = rng.randint(0, 13, 40).astype(np.int32)
+    assert np.array_equal(op.gather_from_rows(arr(D, s2), arr(D, i2)).numpy(), O.gather_from_rows(s2, i2))
+    # gather from a strided (column-sliced) source, fused with arithmetic
+    got = (op.gather_from_rows(arr(D, s2)[:, 2:9], arr(D, i2 % 7)) * 2.0).numpy()
+    assert np.array_equal(got, s2[:, 2:9][np.arange(40), i2 % 7] * 2.0)
+    # one_hot with on 112.2 / off 42.0, depth 7 (tests.cpp:984-1012)
+    ind = rng.randint(0, 6, (2, 3)).astype(np.int32)
+    oh = op.one_hot(arr(D, ind), 7, 112.2, 42.0)
+    assert oh.dtype == D.DTYPE_DOUBLE
+    want = np.full((2, 3, 7), 42.0)
+    for r in range(2):
+        for c in range(3):
+            want[r, c, ind[r, c]] = 112.2
+    assert np.array_equal(oh.numpy(), want)
+    assert np.array_equal(op.one_hot(arr(D, i2), 13, np.float32(1), np.float32(0)).numpy(), O.one_hot(i2, 13))
+
+
+@pytest.mark.parametrize("shape", [(5, 97), (37, 1000), (16, 32000), (3, 50001)])
+def test_softmax_cross_entropy_matches_oracle(gpu, D, O, rng, shape):
+    x = (rng.randn(*shape) * 2).astype(np.float32)
+    t = rng.randint(0, shape[1], shape[0]).astype(np.int32)
+    k0 = D.jit_stats()["kernels"]
+    mean, rows, grad = D.op.softmax_cross_entropy(arr(D, x), arr(D, t))
+    assert D.jit_stats()["kernels"] - k0 == 2  # one fused row pass (gradient + row losses) + the mean
+    omean, orows, ograd = O.softmax_cross_entropy(x, t)
+    close(rows.numpy(), orows, rtol=1e-5, atol=shape[1] * 2.0 ** -24)  # log of the row sum: the sum's relative error is absolute here
+    close(mean.numpy(), omean, rtol=1e-5, atol=shape[1] * 2.0 ** -24)
+    close(grad.numpy(), ograd, rtol=seq_sum_rtol(shape[1]), atol=1e-7)
+    x64 = x.astype(np.float64)
+    lse = np.log(np.exp(x64 - x64.max(1, keepdims=True)).sum(1)) + x64.max(1)
+    close(rows.numpy(), lse - x64[np.arange(shape[0]), t], rtol=1e-5, atol=2e-6)  # fp64 truth
+    sm = np.exp(x64 - lse[:, None])
+    sm[np.arange(shape[0]), t] -= 1.0
+    close(grad.numpy(), sm, rtol=1e-5, atol=1e-7)
+    close(grad.numpy().astype(np.float64).sum(1), 0.0, rtol=0, atol=1e-5)
+    # the reference's own forward, -log(gather_from_rows(softmax(x), t)) (cost.cpp:121-122), built from its ops
+    fwd = (-1.0 * D.op.log(D.op.gather_from_rows(D.op.softmax(arr(D, x)), arr(D, t)))).numpy()
+    close(fwd, O.softmax_cross_entropy_via_probs(x, t), rtol=1e-5, atol=1e-5 + shape[1] * 2.0 ** -24)
+
+
+# --------------------------------------------------------------------- dot
+def test_dot_known_answers_and_laziness(gpu, D, rng):
+    """ArrayDotTests.dot / dot_T / dot_strided / matrix-vector (dot_tests.cpp:9-118)."""
+    op = D.op
+    g = golden("reference_known_answers.json")["dot_known"]
+    a = arr(D, np.ones((2, 3), np.float32))
+    b = arr(D, np.arange(12, dtype=np.float32).reshape(3, 4))
+    before = D.jit_stats()
+    c = op.dot(a, b)
+    assert D.jit_stats() == before and not c.is_buffer()  # lazy
+    assert c.numpy().tolist() == g["ones_2x3_times_arange_3x4"]
+    assert D.jit_stats()["gemms"] - before["gemms"] == 1 and D.jit_stats()["kernels"] == before["kernels"]  # exactly one computation
+    bt = arr(D, np.arange(12, dtype=np.float32).reshape(3, 4).T.copy())
+    assert op.dot(a, bt.T).numpy().tolist() == g["ones_2x3_times_arange_3x4"]
+    wide = arr(D, np.tile(np.arange(12, dtype=np.float32).reshape(3, 4), (1, 2)))
+    assert op.dot(a, wide[:, 4:8]).numpy().tolist() == g["ones_2x3_times_arange_3x4"]  # row-strided operand
+    m = arr(D, np.arange(12, dtype=np.float32).reshape(4, 3))
+    v = arr(D, np.arange(3, dtype=np.float32))
+    assert op.dot(m, v).numpy().tolist() == g["arange_4x3_times_arange_3"]
+    assert op.dot(v, m.T).numpy().tolist() == g["arange_4x3_times_arange_3"]
+    assert float(op.dot(v, v).numpy()) == 5.0
+    # fused around the product: bias and non-linearity see the GEMM result as a buffer
+    x = rng.randn(9, 20).astype(np.float32)
+    w = rng.randn(20, 8).astype(np.float32)
+    bias = rng.randn(1, 8).astype(np.float32)
+    y = op.tanh(op.dot(arr(D, x), arr(D, w)) + arr(D, bias)).numpy()
+    close(y, np.tanh(x.astype(np.float64) @ w + bias), rtol=1e-4, atol=1e-5)
+    # dst += dot(a, b) accumulates (MatMul::supports_operator admits +=, dot.cpp:43-47)
+    dst = arr(D, np.ones((2, 4), np.float32))
+    dst += op.dot(a, b)
+    assert dst.numpy().tolist() == [[13, 16, 19, 22], [13, 16, 19, 22]]
+
+
+@pytest.mark.parametrize("B,I,H", [(3, 8, 8), (32, 100, 64), (17, 33, 20)])
+def test_lstm_step_matches_oracle(gpu, D, O, rng, B, I, H):
+    X, Hp, Cp = (rng.randn(B, n).astype(np.float32) for n in (I, H, H))
+    lim = np.sqrt(6.0 / (I + 4 * H))
+    W, U = (rng.uniform(-lim, lim, (n, 4 * H)).astype(np.float32) for n in (I, H))
+    b = (rng.randn(4 * H) * 0.1).astype(np.float32)
+    before = D.jit_stats()
+    cn, hn = D.op.lstm_step(*(arr(D, v) for v in (X, Hp, Cp, W, U, b)))
+    after = D.jit_stats()
+    assert after["gemms"] - before["gemms"] == 1 and after["kernels"] - before["kernels"] == 1  # one GEMM pair + one gate kernel
+    _, ocn, ohn = O.lstm_step(X, Hp, Cp, W, U, b)
+    close(cn.numpy(), ocn, rtol=1e-4, atol=1e-5)
+    close(hn.numpy(), ohn, rtol=1e-4, atol=1e-5)
+
+
+def test_recording_replays_the_same_device_work(gpu, D, rng):
+    x = arr(D, rng.randn(50, 300).astype(np.float32))
+    with D.Recording() as rec:
+        s = D.op.softmax(x)
+        s.eval()
+    assert rec.launches == 1
+    first = s.numpy()
+    rec.replay(3)
+    assert np.array_equal(s.numpy(), first)

@@ -1,0 +1,349 @@
+"""Pins the CPU checker (oracle/) before anything is compared against it.
+
+Every function of the oracle is checked against (i) the expected values the
+reference's own tests hold (tests/golden/reference_known_answers.json, with
+file:line), (ii) the pieces of the reference compiled from its own headers
+(oracle/_ref, when built), and (iii) independent mathematics: fp64 libm closed
+forms, invariants and brute force with planted ties. None of these retype the
+oracle's own formula.
+"""
+import math
+
+import numpy as np
+import pytest
+
+from conftest import golden
+
+FLT_MAX = np.finfo(np.float32).max
+
+
+def f64(x):
+    return np.asarray(x, dtype=np.float64)
+
+
+# ------------------------------------------------------------------ functors
+UNARY_TRUTH = {
+    "sigmoid": lambda x: 1.0 / (1.0 + np.exp(-x)),
+    "tanh": np.tanh,
+    "exp": np.exp,
+    "log": np.log,
+    "negative_log": lambda x: -np.log(x),
+    "square": lambda x: x * x,
+    "cube": lambda x: x * x * x,
+    "sqrt_f": np.sqrt,
+    "rsqrt": lambda x: 1.0 / np.sqrt(x),
+    "inv": lambda x: 1.0 / x,
+    "identity": lambda x: x,
+    "abs": np.abs,
+    "sign": lambda x: np.where(x > 0, 1.0, -1.0),
+    "relu": lambda x: np.where(x > 0, x, 0.0),
+    "relu_backward": lambda x: np.where(x > 0, 1.0, 0.0),
+    "dsigmoid": lambda x: x * (1.0 - x),
+    "dtanh": lambda x: 1.0 - x * x,
+    "softplus": lambda x: np.where(x > 20.0, x, np.log1p(np.exp(np.minimum(x, 30.0)))),
+    "softplus_backward": lambda x: np.where(x > 20.0, 1.0, 1.0 / (1.0 + np.exp(-x))),
+    "log_or_zero": lambda x: np.where(x > 0, np.log(np.where(x > 0, x, 1.0)), 0.0),
+    "inverse_tanh": lambda x: np.arctanh(x),
+    "safe_entropy_log": lambda x: np.log(np.clip(x, 1e-6, 1.0 - 1e-6)),
+}
+
+
+@pytest.mark.parametrize("name", sorted(UNARY_TRUTH))
+def test_unary_against_fp64_closed_form(O, name):
+    # the reference's own unary tests use x = arange(50)+1 (tests.cpp:1015-1073); a
+    # signed range and a (0,1) range cover the functors defined only there
+    xs = [np.arange(1, 51, dtype=np.float32), np.linspace(-6, 6, 97).astype(np.float32), np.linspace(0.02, 0.98, 49).astype(np.float32)]
+    if name in ("log", "negative_log", "sqrt_f", "rsqrt", "inv"):
+        xs = [xs[0], xs[2]]
+    if name in ("inverse_tanh", "safe_entropy_log", "dsigmoid"):
+        xs = [xs[2]]
+    if name in ("exp", "cube"):
+        xs = [xs[1], xs[2]]
+    for x in xs:
+        got = O.unary(name, x)
+        want = UNARY_TRUTH[name](f64(x))
+        np.testing.assert_allclose(got, want, rtol=3e-6, atol=1e-6, err_msg=name)
+
+
+def test_sigmoid_is_the_double_precision_formula(O):
+    # functor.h:157-162: 1.0 / (1.0 + expf(-a)) in double, rounded once; the float-only
+    # formula differs in the last place on part of the range, so this catches dropping the double
+    x = np.linspace(-10, 10, 20001).astype(np.float32)
+    got = O.unary("sigmoid", x)
+    e = np.exp(-x.astype(np.float32)).astype(np.float32)  # float expf
+    want = (1.0 / (1.0 + e.astype(np.float64))).astype(np.float32)
+    # numpy's float32 exp may differ from glibc expf by an ulp: compare through that slack
+    assert np.max(np.abs(got.astype(np.float64) - want.astype(np.float64))) <= 1.2e-7
+    assert got[10000] == np.float32(0.5)
+
+
+def test_round_matches_reference_astype(O):
+    g = golden("reference_known_answers.json")["astype_round"]
+    got = O.round_to_int(np.array(g["input"], dtype=np.float32))
+    assert got.tolist() == g["expected"]
+
+
+def test_binary_closed_forms(O, rng):
+    a = rng.uniform(-3, 3, 200).astype(np.float32)
+    b = rng.uniform(0.5, 3, 200).astype(np.float32)
+    A, B = f64(a), f64(b)
+    checks = {
+        "add": A + B, "subtract": A - B, "eltmul": A * B, "eltdiv": A / B,
+        "equals": (A == B).astype(np.float64), "max_scalar": np.maximum(A, B), "min_scalar": np.minimum(A, B),
+        "threshold": (A < B).astype(np.float64), "lessthanequal": (A <= B).astype(np.float64),
+        "greaterthanequal": (A >= B).astype(np.float64), "prelu": np.where(A > 0, A, B * A),
+        "clip": np.clip(A, -B, B), "div_grad": A / (B * B), "fill": B,
+        "prelu_backward_inputs": np.where(A > 0, 1.0, B), "prelu_backward_weights": np.where(A > 0, 0.0, A * B),
+        "steep_sigmoid": 1.0 / (1.0 + np.exp(-B * A)), "steep_sigmoid_backward": B * (A - A * A),
+        "clipped_relu": np.where(A > 0, np.minimum(A, B), 0.0),
+        "clipped_relu_backward": np.where(A > 0, np.where(A > B, 0.0, 1.0), 0.0),
+    }
+    for name, want in checks.items():
+        np.testing.assert_allclose(O.binary(name, a, b), want, rtol=3e-6, atol=1e-6, err_msg=name)
+    np.testing.assert_allclose(O.binary("power", np.abs(a) + 0.1, b), (np.abs(A) + np.float64(np.float32(0.1))) ** B, rtol=1e-5)
+    p = rng.uniform(0.05, 0.95, 100).astype(np.float32)
+    t = rng.randint(0, 2, 100).astype(np.float32)
+    P, T = f64(p), f64(t)
+    np.testing.assert_allclose(O.binary("binary_cross_entropy", p, t), -(T * np.log(P) + (1 - T) * np.log(1 - P)), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(O.binary("binary_cross_entropy_grad", p, t), (T - P) / (P * (P - 1)), rtol=1e-5)
+    # scalar broadcast on either side (tests.cpp:1075-1117)
+    np.testing.assert_allclose(O.binary("subtract", a, 2.0), A - 2.0, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(O.binary("subtract", 2.0, a), 2.0 - A, rtol=1e-6, atol=1e-6)
+
+
+def test_chain_matches_fp64_truth_and_its_parts(O, rng):
+    a, b, c, d = [rng.uniform(-4, 4, 5000).astype(np.float32) for _ in range(4)]
+    got = O.chain(a, b, c, d)
+    A, B, Cc, Dd = map(f64, (a, b, c, d))
+    want = 1.0 / (1.0 + np.exp(-A)) * np.tanh(B) + Cc * Dd - 0.5 * A * A
+    scale = np.abs(np.tanh(B)) + np.abs(Cc * Dd) + 0.5 * A * A
+    assert np.all(np.abs(got - want) <= 3e-7 * scale + 1e-7)
+    # dropping or flipping a term is far outside that bound
+    assert np.max(np.abs((want + A * A) - got)) > 1.0
+    # and it is exactly the composition of the single-functor entry points, each rounded to fp32
+    comp = O.binary("subtract", O.binary("add", O.binary("eltmul", O.unary("sigmoid", a), O.unary("tanh", b)), O.binary("eltmul", c, d)),
+                    O.binary("eltmul", np.float32(0.5), O.unary("square", a)))
+    assert np.array_equal(comp, got)
+
+
+# ------------------------------------------------------------------ reducers
+def test_all_reduce_closed_forms(O):
+    g = golden("reference_known_answers.json")
+    for n in (1, 2, 5, 100, 1000):
+        assert float(O.all_reduce(O.SUM, np.arange(n, dtype=np.float32))) == n * (n - 1) / 2
+    assert float(O.all_reduce(O.PROD, np.array(g["all_reduce_prod"]["input"], np.float32))) == g["all_reduce_prod"]["expected"]
+    mm = np.array(g["all_reduce_max_min"]["input"], np.float32)
+    assert float(O.all_reduce(O.MAX, mm)) == g["all_reduce_max_min"]["max"]
+    assert float(O.all_reduce(O.MIN, mm)) == g["all_reduce_max_min"]["min"]
+    # init values: empty reductions return the reducer's neutral element (reducer_kernels.h)
+    e = np.zeros(0, np.float32)
+    assert float(O.all_reduce(O.SUM, e)) == 0.0 and float(O.all_reduce(O.PROD, e)) == 1.0
+    assert O.all_reduce(O.MAX, e) == -FLT_MAX and O.all_reduce(O.MIN, e) == FLT_MAX
+
+
+def test_sum_is_strictly_sequential_fp32(O):
+    # 1 followed by many 2^-24: a left-to-right fp32 sum never leaves 1.0, pairwise or fp64 sums do
+    x = np.full(1 + 4096, 2.0 ** -24, dtype=np.float32)
+    x[0] = 1.0
+    assert float(O.all_reduce(O.SUM, x)) == 1.0
+    assert float(O.axis_reduce(O.SUM, x.reshape(1, -1), 1)[0]) == 1.0
+    # reversed order accumulates the small terms first
+    assert float(O.all_reduce(O.SUM, x[::-1].copy())) > 1.0
+
+
+def test_axis_reduce_ones_and_strided_view(O, rng):
+    # tests.cpp:1215-1239: reductions of ones give the reduced extent
+    ones = np.ones((7, 13), np.float32)
+    assert np.array_equal(O.axis_reduce(O.SUM, ones, 1), np.full(7, 13, np.float32))
+    assert np.array_equal(O.axis_reduce(O.SUM, ones, 0), np.full(13, 7, np.float32))
+    x = rng.randn(37, 53).astype(np.float32)
+    np.testing.assert_allclose(O.axis_reduce(O.SUM, x, 0), f64(x).sum(0), atol=1e-5 * np.abs(x).sum(0).max())
+    np.testing.assert_allclose(O.axis_reduce(O.SUM, x, 1), f64(x).sum(1), atol=1e-5 * np.abs(x).sum(1).max())
+    assert np.array_equal(O.axis_reduce(O.MAX, x, 0), x.max(0)) and np.array_equal(O.axis_reduce(O.MAX, x, 1), x.max(1))
+    assert np.array_equal(O.axis_reduce(O.MIN, x, 0), x.min(0)) and np.array_equal(O.axis_reduce(O.MIN, x, 1), x.min(1))
+    # axis 0 must equal axis 1 of the materialised transpose bit for bit (same sequential order)
+    assert np.array_equal(O.axis_reduce(O.SUM, x, 0), O.axis_reduce(O.SUM, np.ascontiguousarray(x.T), 1))
+    np.testing.assert_allclose(O.axis_reduce(O.PROD, x[:5, :6], 1), np.prod(f64(x[:5, :6]), 1), rtol=1e-5)
+
+
+def test_argmax_reference_vectors_and_ties(O):
+    g = golden("reference_known_answers.json")["axis_argmax_argmin"]
+    x = np.arange(20, dtype=np.float32).reshape(4, 5)
+    assert O.arg_axis_reduce(O.MAX, x, 0).tolist() == g["argmax_axis0"]
+    assert O.arg_axis_reduce(O.MAX, x, 1).tolist() == g["argmax_axis1"]
+    assert O.arg_axis_reduce(O.MIN, x, 0).tolist() == g["argmin_axis0"]
+    assert O.arg_axis_reduce(O.MIN, x, 1).tolist() == g["argmin_axis1"]
+    # flat argmax / argmin (tests.cpp:1141-1148): ramp -100..99 -> max at the end, min at 0
+    ramp = np.arange(-100, 42, dtype=np.float32)
+    assert O.arg_all_reduce(O.MAX, ramp) == 141 and O.arg_all_reduce(O.MIN, ramp) == 0
+    # planted ties: the FIRST of equal extrema wins (all_reduce_kernel_utils.cpp:217-219)
+    t = np.array([[1, 7, 3, 7, 7], [5, 5, 5, 5, 5], [-2, -9, -9, 0, -9]], np.float32)
+    assert O.arg_axis_reduce(O.MAX, t, 1).tolist() == [1, 0, 3]
+    assert O.arg_axis_reduce(O.MIN, t, 1).tolist() == [0, 0, 1]
+    # brute force over every length-4 row of {0,1,2}
+    import itertools
+    rows = np.array(list(itertools.product([0, 1, 2], repeat=4)), np.float32)
+    assert O.arg_axis_reduce(O.MAX, rows, 1).tolist() == [int(np.argmax(r)) for r in rows]
+    assert O.arg_axis_reduce(O.MIN, rows, 1).tolist() == [int(np.argmin(r)) for r in rows]
+    # sentinel: a row of -FLT_MAX (or -inf) never replaces the initial value, index stays 0
+    s = np.array([[-FLT_MAX, -FLT_MAX], [-np.inf, -np.inf]], np.float32)
+    assert O.arg_axis_reduce(O.MAX, s, 1).tolist() == [0, 0]
+
+
+def test_reducers_against_reference_headers(O, rng):
+    if O.ref is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    import ctypes as C
+    x = rng.randn(19, 23).astype(np.float32)
+    x[3, 5] = x[3, 11] = 9.0  # tie
+    for red in (O.SUM, O.MAX, O.MIN, O.PROD):
+        for (rows, cols, rs, cs, axis) in ((19, 23, 23, 1, 1), (23, 19, 1, 23, 0)):
+            want = np.empty(rows, np.float32)
+            O.ref.ref_axis_reduce(red, O.fp(x), rows, cols, rs, cs, O.fp(want))
+            assert np.array_equal(O.axis_reduce(red, x, axis), want)
+        assert O.all_reduce(red, x) == np.float32(O.ref.ref_all_reduce(red, O.fp(x), x.size))
+    for red in (O.MAX, O.MIN):
+        for (rows, cols, rs, cs, axis) in ((19, 23, 23, 1, 1), (23, 19, 1, 23, 0)):
+            want = np.empty(rows, np.int32)
+            O.ref.ref_arg_axis_reduce(red, O.fp(x), rows, cols, rs, cs, O.ip(want))
+            assert np.array_equal(O.arg_axis_reduce(red, x, axis), want)
+
+
+def test_reference_index_arithmetic(O):
+    if O.ref is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    shape = np.array([3, 4, 5], np.int32)
+    out = np.empty(3, np.int32)
+    for idx in (0, 7, 23, 59):
+        O.ref.ref_index_to_dim3(idx, O.ip(shape), O.ip(out))
+        assert tuple(out) == np.unravel_index(idx, (3, 4, 5))
+        assert O.ref.ref_indices_to_offset3(O.ip(shape), O.ip(out)) == idx
+
+
+def test_mean(O):
+    x = np.arange(10, dtype=np.float32)
+    assert float(O.mean_all(x)) == 4.5
+
+
+# -------------------------------------------------------- softmax and friends
+def test_softmax_invariants(O, rng):
+    x = (rng.randn(7, 33) * 3).astype(np.float32)
+    s = O.softmax(x)
+    e = np.exp(f64(x) - f64(x).max(1, keepdims=True))
+    np.testing.assert_allclose(s, e / e.sum(1, keepdims=True), rtol=2e-6)
+    np.testing.assert_allclose(s.sum(1), 1.0, atol=1e-6)
+    # shift invariance holds up to the rounding of x + c; an exact power-of-two-friendly case is bit-identical
+    xi = rng.randint(-8, 8, size=(5, 16)).astype(np.float32)
+    assert np.array_equal(O.softmax(xi), O.softmax(xi + 4.0))
+    # one dominant logit
+    big = np.array([[0.0, 100.0, 0.0]], np.float32)
+    assert O.softmax(big)[0, 1] == 1.0
+    # the staged computation of tests.cpp:1622-1664 on U(-20,20) [2,5]
+    u = rng.uniform(-20, 20, (2, 5)).astype(np.float32)
+    staged = O.binary("eltdiv", O.unary("exp", u - u.max(1, keepdims=True)),
+                      np.repeat(O.axis_reduce(O.SUM, O.unary("exp", u - u.max(1, keepdims=True)), 1)[:, None], 5, 1))
+    np.testing.assert_allclose(O.softmax(u), staged, atol=1e-6)
+
+
+def test_gather_from_rows_reference_table(O):
+    g = golden("reference_known_answers.json")["gather_from_rows_3d"]
+    src = np.arange(5 * 6 * 7, dtype=np.float32).reshape(5, 6, 7)
+    idx = np.arange(5, dtype=np.int32)
+    # the 3-D case gathers whole trailing rows; column j of the table is a 2-D gather on source[:, :, j]
+    got = np.stack([O.gather_from_rows(np.ascontiguousarray(src[:, :, j]), idx) for j in range(7)], axis=1)
+    assert got.astype(np.int64).tolist() == g["expected"]
+    src2 = np.arange(30, dtype=np.float32).reshape(5, 6)
+    assert O.gather_from_rows(src2, idx).tolist() == [src2[i, i] for i in range(5)]
+
+
+def test_one_hot_reference_semantics(O, rng):
+    # tests.cpp:984-1012: depth 7, on 112.2, off 42.0 compared with an explicit scatter
+    idx = rng.randint(0, 6, size=6).astype(np.int32)
+    got = O.one_hot(idx, 7, 112.2, 42.0)
+    want = np.full((6, 7), np.float32(42.0), np.float32)
+    want[np.arange(6), idx] = np.float32(112.2)
+    assert np.array_equal(got, want)
+
+
+def test_cross_entropy_identities(O, rng):
+    x = (rng.randn(5, 97) * 2).astype(np.float32)
+    t = rng.randint(0, 97, size=5).astype(np.int32)
+    mean, rows, grad = O.softmax_cross_entropy(x, t)
+    X = f64(x)
+    lse = np.log(np.exp(X - X.max(1, keepdims=True)).sum(1)) + X.max(1)
+    want_rows = lse - X[np.arange(5), t]
+    np.testing.assert_allclose(rows, want_rows, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(mean, want_rows.mean(), rtol=1e-5)
+    sm = np.exp(X - lse[:, None])
+    oh = np.zeros_like(X)
+    oh[np.arange(5), t] = 1
+    np.testing.assert_allclose(grad, sm - oh, atol=2e-6)
+    np.testing.assert_allclose(grad.sum(1), 0.0, atol=1e-5)  # rows of softmax - onehot sum to zero
+    # agrees with the reference's own forward -log(softmax[i, t]) (cost.cpp:121-122)
+    np.testing.assert_allclose(O.softmax_cross_entropy_via_probs(x, t), rows, rtol=1e-5, atol=2e-6)
+    # a wrong sign in the gather term or a missing max would break this: loss of a one-hot-dominant row is ~0
+    z = np.zeros((1, 4), np.float32)
+    z[0, 2] = 50
+    assert abs(float(O.softmax_cross_entropy(z, np.array([2], np.int32))[1][0])) < 1e-6
+
+
+# --------------------------------------------------------------------- gemm
+def test_gemm_known_answers(O):
+    g = golden("reference_known_answers.json")["dot_known"]
+    a = np.ones((2, 3), np.float32)
+    b = np.arange(12, dtype=np.float32).reshape(3, 4)
+    for mode in ("f64", "f32"):
+        assert O.gemm(a, b, mode).tolist() == g["ones_2x3_times_arange_3x4"]
+    m = np.arange(12, dtype=np.float32).reshape(4, 3)
+    v = np.arange(3, dtype=np.float32).reshape(3, 1)
+    assert O.gemm(m, v)[:, 0].tolist() == g["arange_4x3_times_arange_3"]
+    ai = np.arange(6, dtype=np.int32).reshape(2, 3)
+    bi = np.arange(12, dtype=np.int32).reshape(3, 4)
+    assert np.array_equal(O.gemm_i32(ai, bi), ai @ bi)
+
+
+def test_gemm_layouts_against_numpy_fp64(O, rng):
+    A = rng.randn(5, 7).astype(np.float32)
+    B = rng.randn(7, 11).astype(np.float32)
+    want = f64(A) @ f64(B)
+    At = np.ascontiguousarray(A.T).T  # transposed storage
+    Bt = np.ascontiguousarray(B.T).T
+    wide = rng.randn(5, 20).astype(np.float32)
+    As = wide[:, 3:10]  # row-strided view
+    for (a, b, w) in ((A, B, want), (At, B, want), (A, Bt, want), (At, Bt, want), (As, B, f64(As) @ f64(B))):
+        np.testing.assert_allclose(O.gemm(a, b, "f64"), w, rtol=1e-6, atol=1e-6)
+        np.testing.assert_allclose(O.gemm(a, b, "f32"), w, rtol=1e-4, atol=1e-5)
+
+
+def test_gemm_against_reference_template(O, rng):
+    if O.ref is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    # igemm call of cpu_gemm.cpp:14-20,52-58 for row-major lhs[n,k] . rhs[k,m]: (!rhs_T, !lhs_T, m, n, k, rhs, ldr, lhs, ldl, dst, ldd)
+    lhs = rng.randint(-5, 5, size=(4, 6)).astype(np.int32)
+    rhs = rng.randint(-5, 5, size=(6, 3)).astype(np.int32)
+    dst = np.zeros((4, 3), np.int32)
+    O.ref.ref_gemm_i32(1, 1, 3, 4, 6, O.ip(rhs), 3, O.ip(lhs), 6, O.ip(dst), 3)
+    assert np.array_equal(dst, lhs @ rhs)
+    assert np.array_equal(O.gemm_i32(lhs, rhs), dst)
+    fl, fr = lhs.astype(np.float32) * 0.37, rhs.astype(np.float32) * 1.3
+    fd = np.zeros((4, 3), np.float32)
+    O.ref.ref_gemm_f32(1, 1, 3, 4, 6, O.fp(fr), 3, O.fp(fl), 6, O.fp(fd), 3)
+    assert np.array_equal(O.gemm(fl, fr, "f32"), fd)  # same sequential fp32 accumulation order
+
+
+# --------------------------------------------------------------------- lstm
+def test_lstm_step_composition(O, rng):
+    B, I, H = 3, 8, 8
+    X, Hp, Cp = rng.randn(B, I).astype(np.float32), rng.randn(B, H).astype(np.float32), rng.randn(B, H).astype(np.float32)
+    W, U = (rng.randn(I, 4 * H) * 0.3).astype(np.float32), (rng.randn(H, 4 * H) * 0.3).astype(np.float32)
+    b = (rng.randn(4 * H) * 0.1).astype(np.float32)
+    gates, c_new, h_new = O.lstm_step(X, Hp, Cp, W, U, b)
+    G = f64(b) + f64(X) @ f64(W) + f64(Hp) @ f64(U)
+    np.testing.assert_allclose(gates, G, rtol=1e-5, atol=1e-6)
+    sig = lambda z: 1.0 / (1.0 + np.exp(-z))
+    i, f, o, g = sig(G[:, :H]), sig(G[:, H:2 * H]), sig(G[:, 2 * H:3 * H]), np.tanh(G[:, 3 * H:])
+    c = f * f64(Cp) + i * g
+    np.testing.assert_allclose(c_new, c, rtol=1e-5, atol=2e-6)
+    np.testing.assert_allclose(h_new, o * np.tanh(c), rtol=1e-5, atol=2e-6)
+    # gate order matters: swapping o and g changes the answer
+    assert np.max(np.abs(h_new - sig(G[:, 3 * H:]) * np.tanh(c))) > 1e-2
