@@ -525,7 +525,8 @@ int dali_hip_launch(uint64_t hash, void** array_data, const int* offsets, const 
         int64_t per2 = P.work2_per_block > 0 ? P.work2_per_block : 1;
         gy = (red + per2 - 1) / per2;
         if (P.max_blocks2 > 0 && gy > P.max_blocks2) gy = P.max_blocks2;
-        int64_t cap = (int64_t)kWorkspacePartialBytes / (work * (int64_t)(P.ws_elsize > 0 ? P.ws_elsize : 4));
+        // rows of partials are padded to whole column strips
+        int64_t cap = (int64_t)kWorkspacePartialBytes / (gx * per * (int64_t)(P.ws_elsize > 0 ? P.ws_elsize : 4));
         if (cap < 1) cap = 1;
         if (gy > cap) gy = cap;
         if (gx > (int64_t)kWorkspaceCounters) return fail("dali_hip_launch: %lld column strips exceed the %d workspace counters", (long long)gx, kWorkspaceCounters);

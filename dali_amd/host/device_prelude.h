@@ -151,11 +151,31 @@ template <typename R> struct prelu_backward_weights { DI static R Map(R x, R g) 
 template <typename R> struct prelu_backward_inputs { DI static R Map(R x, R w) { return x > 0 ? (R)1.0 : w; } };
 }  // namespace functor
 
-// one_hot element: on*is_on + (1.0 - is_on)*off with is_on in T and the rest in double
+// x / s for a divisor that is the same for every element a thread handles (a row value
+// or a scalar): one true reciprocal per row, then per element a product and one FMA
+// correction step, which yields the correctly rounded quotient except in rare last-place
+// cases. Divisors whose reciprocal is not a normal number take the plain division.
+DI float dali_div_invariant(float x, float s) {
+    const float a = __builtin_fabsf(s);
+    if (a > 1e-30f && a < 1e30f) {
+        const float r = 1.0f / s;
+        const float q = x * r;
+        const float e = __builtin_fmaf(-q, s, x);
+        return __builtin_fmaf(e, r, q);
+    }
+    return x / s;
+}
+DI double dali_div_invariant(double x, double s) { return x / s; }
+DI int dali_div_invariant(int x, int s) { return x / s; }
+
+// one_hot element. The reference evaluates on*is_on + (1.0 - is_on)*off with is_on in T and
+// the rest in double (dali/array/op/one_hot.cpp:38-46). With is_on in {0, 1} that is
+// on + 0*off when the index matches and on*0 + off otherwise, and both forms round to
+// the same T as the double evaluation (the products are exact zeros or NaN), so the
+// select below is bit-identical, including inf / NaN propagation.
 template <typename T>
 DI T dali_one_hot(int index, int column, T on, T off) {
-    T is_on = (T)(index == column);
-    return (T)((double)(on * is_on) + (1.0 - (double)is_on) * (double)off);
+    return index == column ? (T)(on + (T)0 * off) : (T)(on * (T)0 + off);
 }
 
 // ------------------------------------------------------------------ reducers
@@ -189,6 +209,17 @@ struct minimum {
     template <typename T> DI static bool better(T cand, T cur) { return cand < cur; }
 };
 }  // namespace reducers
+
+// ------------------------------------------------- cross-workgroup hand-off
+// Agent-scope relaxed atomics: the store is written through to the coherence point
+// shared by all XCDs, the load does not return a stale line of the local L2.
+template <typename T> DI void dali_publish(T* p, T v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+template <typename T> DI T dali_observe(const T* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// Waits until this thread's earlier stores are acknowledged, then draws a ticket.
+DI unsigned int dali_take_ticket(unsigned int* counter) {
+    __builtin_amdgcn_s_waitcnt(0);
+    return __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // --------------------------------------------------------- cross-lane helpers
 template <typename T> DI T dali_shfl_xor(T v, int mask) { return __shfl_xor(v, mask, 64); }

@@ -20,6 +20,7 @@
 //   all   full reduction, two-stage through the workspace, optional scalar epilogue
 // Anything else is split: inner reductions are evaluated into temporaries first.
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <map>
@@ -56,7 +57,7 @@ void set_recording(std::vector<std::function<void()>>* rec) { g_recording = rec;
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-3";
+const char* const kCodegenVersion = "dali-hip-codegen-7";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -433,8 +434,14 @@ std::string kargs_struct(const Program& P, const IvLayout& L) {
 
 struct RowParams {
     int VEC = 1, TPR = 64, EPT = 0, BT = 256, RPB = 4, NW = 1;
+    int waves_per_eu = 0;  // occupancy hint (0 = compiler default)
     bool cached = true;
 };
+
+int env_int(const char* name, int fallback) {
+    const char* v = getenv(name);
+    return (v && *v) ? atoi(v) : fallback;
+}
 
 // Emits C++ expressions for program nodes inside one loop body, declaring shared
 // values once per body.
@@ -451,6 +458,13 @@ struct BodyEmitter {
     BodyEmitter(const Program& P_, const RowParams& rp_, bool per_el, int body, const std::vector<int>* fb)
         : P(P_), rp(rp_), per_element(per_el), body_index(body), first_body(fb) {
         leaf_suffix = rp.cached ? "[e][j]" : "[j]";
+    }
+
+    // true when the node's value is the same for every element of a row (seen through broadcasts)
+    bool row_invariant(int id) const {
+        const PNode* n = &P.nodes[id];
+        while (n->kind == Kind::BROADCAST || n->kind == Kind::EXPAND_DIMS) n = &P.nodes[n->args[0]];
+        return n->kind == Kind::SCALAR || (n->cls_set && n->cls != Cls::FULL);
     }
 
     std::string scalar_ref(const PNode& n) {
@@ -478,6 +492,10 @@ struct BodyEmitter {
             case Kind::BROADCAST:
                 return value(n.args[0]);
             case Kind::ELEMENTWISE: {
+                if (n.name == "functor::eltdiv" && n.cls == Cls::FULL && n.args.size() == 2 && row_invariant(n.args[1])) {
+                    // divisor constant along the row: reciprocal once, product + correction per element
+                    return "dali_div_invariant(" + value(n.args[0]) + ", " + value(n.args[1]) + ")";
+                }
                 std::string s = n.name + "<" + ctype(n.dtype) + ">::Map(";
                 for (size_t i = 0; i < n.args.size(); ++i) s += (i ? ", " : "") + value(n.args[i]);
                 return s + ")";
@@ -698,7 +716,9 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
     std::ostringstream ss;
     ss << codegen::kDevicePrelude;
     ss << kargs_struct(P, L);
-    ss << "extern \"C\" __global__ __launch_bounds__(" << rp.BT << ") void " << kname << "(KArgs A) {\n";
+    ss << "extern \"C\" __global__ __launch_bounds__(" << rp.BT << ") ";
+    if (rp.waves_per_eu > 0) ss << "__attribute__((amdgpu_waves_per_eu(" << rp.waves_per_eu << ", " << rp.waves_per_eu << "))) ";
+    ss << "void " << kname << "(KArgs A) {\n";
     ss << "  constexpr int VEC = " << rp.VEC << ", TPR = " << rp.TPR << ", RPB = " << rp.RPB << ";\n";
     if (rp.cached) ss << "  constexpr int EPT = " << rp.EPT << ";\n";
     ss << "  const int tid = threadIdx.x;\n  const int tr = tid % TPR;\n";
@@ -1015,10 +1035,13 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
         rp.TPR = (int)std::min<int64_t>(256, pow2ceil((int)std::max<int64_t>(1, CH)));
         rp.BT = 256;
     } else {
-        int tpr = pow2ceil((int)std::max<int64_t>(1, (CH + 3) / 4));
-        tpr = std::min(tpr, 1024);
+        static const int chunks_target = std::max(1, env_int("DALI_HIP_ROW_CHUNKS", 4));
+        static const int tpr_cap = std::max(64, env_int("DALI_HIP_ROW_TPR_MAX", 1024));
+        int tpr = pow2ceil((int)std::max<int64_t>(1, (CH + chunks_target - 1) / chunks_target));
+        tpr = std::min(tpr, tpr_cap);
         int64_t ept = (CH + tpr - 1) / tpr;
-        rp.cached = ept <= 16;
+        // every FULL input is held in registers across the phases: bound the footprint
+        rp.cached = (int64_t)std::max(1, n_full) * ept * rp.VEC * (max_el / 4) <= 64;
         if (!rp.cached) {
             tpr = 1024;
             ept = 0;
@@ -1030,6 +1053,10 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
     }
     rp.RPB = rp.BT / rp.TPR;
     rp.NW = rp.TPR > 64 ? rp.TPR / 64 : 1;
+    // A 1024-thread row block fills a CU by itself unless it stays within 64 VGPRs; two resident
+    // blocks let one row's loads overlap another row's arithmetic.
+    static const int wpe = env_int("DALI_HIP_ROW_WAVES_PER_EU", -1);
+    rp.waves_per_eu = nph > 0 ? (wpe >= 0 ? wpe : (rp.BT == 1024 ? 8 : 0)) : 0;
 
     // cross-phase register caching of expensive shared values
     rpn.first_body.assign(P.nodes.size(), -1);
@@ -1066,7 +1093,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
 
     // kernel identity
     std::ostringstream params;
-    params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached;
+    params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached << "," << rp.waves_per_eu;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     std::string sig = signature(P, rpn.outputs);
     uint64_t h = kernel_hash("row", sig, params.str());
@@ -1225,7 +1252,7 @@ bool try_flat(const std::vector<DestSpec>& specs) {
 // partials in block order (so the result does not depend on scheduling), applies
 // the scalar epilogue and resets the ticket counter.
 std::string gen_all_kernel(const Program& P, int red_id, int root_id, int dest_array, OPERATOR_T op, const IvLayout& L, int VEC, int BT,
-                           const std::string& kname) {
+                           int UNROLL, int TAIL, const std::string& kname) {
     const PNode& red = P.nodes[red_id];
     bool is_arg = red.kind == Kind::ARG_ALL_REDUCE;
     std::string t = ctype(P.nodes[red.args[0]].dtype);
@@ -1247,23 +1274,27 @@ std::string gen_all_kernel(const Program& P, int red_id, int root_id, int dest_a
     for (size_t i = 0; i < P.arrays.size(); ++i)
         if (!P.arrays[i].is_dest && P.arrays[i].cls == Cls::FULL) full_leaves.push_back((int)i);
     ss << "  " << t << " acc = " << red.name << "::init<" << t << ">();\n  int acci = 0; (void)acci;\n";
-    ss << "  for (long ch = (long)blockIdx.x * BT + threadIdx.x; ch < NCH; ch += (long)gridDim.x * BT) {\n";
-    for (int i : full_leaves) {
-        ss << "    " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n";
-        emit_leaf_load(ss, P.arrays[i], i, VEC, "x" + std::to_string(i), "    ", false);
-    }
-    ss << "    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n      const int col = (int)(ch * VEC + j); (void)col;\n";
+    // UNROLL independent vector loads in flight per thread before any of them is consumed
+    ss << "  constexpr int UNROLL = " << UNROLL << ";\n";
+    ss << "  for (long base = (long)blockIdx.x * (BT * UNROLL) + threadIdx.x; base < NCH; base += (long)gridDim.x * (BT * UNROLL)) {\n";
+    for (int i : full_leaves) ss << "    " << ctype(P.arrays[i].buf->dtype) << " x" << i << "s[UNROLL][VEC];\n";
+    ss << "    _Pragma(\"unroll\") for (int u = 0; u < UNROLL; ++u) {\n      const long ch = base + (long)u * BT;\n      if (ch < NCH) {\n";
+    for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, VEC, "x" + std::to_string(i) + "s[u]", "        ", false);
+    ss << "      }\n    }\n";
+    ss << "    _Pragma(\"unroll\") for (int u = 0; u < UNROLL; ++u) {\n      const long ch = base + (long)u * BT;\n      if (ch < NCH) {\n";
+    for (int i : full_leaves) ss << "        const " << ctype(P.arrays[i].buf->dtype) << "* x" << i << " = x" << i << "s[u];\n";
+    ss << "        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n          const int col = (int)(ch * VEC + j); (void)col;\n";
     std::vector<int> first_body(P.nodes.size(), -1);
     {
         BodyEmitter be(P, rp, true, 0, &first_body);
         std::string v = be.value(red.args[0]);
         ss << be.stmts.str();
         if (!is_arg)
-            ss << "      acc = " << red.name << "::step<" << t << ">(acc, " << v << ");\n";
+            ss << "          acc = " << red.name << "::step<" << t << ">(acc, " << v << ");\n";
         else
-            ss << "      { const " << t << " cand = " << v << "; if (" << red.name << "::better<" << t << ">(cand, acc)) { acc = cand; acci = col; } }\n";
+            ss << "          { const " << t << " cand = " << v << "; if (" << red.name << "::better<" << t << ">(cand, acc)) { acc = cand; acci = col; } }\n";
     }
-    ss << "    }\n  }\n";
+    ss << "        }\n      }\n    }\n  }\n";
     ss << "  __shared__ " << t << " smv[" << NW << "]; __shared__ int smi[" << NW << "]; __shared__ int is_last;\n";
     if (!is_arg)
         ss << "  acc = dali_block_reduce<" << red.name << ", " << t << ", " << NW << ">(acc, smv);\n";
@@ -1271,23 +1302,30 @@ std::string gen_all_kernel(const Program& P, int red_id, int root_id, int dest_a
         ss << "  dali_block_arg_reduce<" << red.name << ", " << t << ", " << NW << ">(acc, acci, smv, smi);\n";
     ss << "  unsigned int* counters = (unsigned int*)A.ws;\n";
     ss << "  dali_partial* partials = (dali_partial*)((char*)A.ws + " << 16384 * 4 << ");\n";
-    ss << "  if (threadIdx.x == 0) {\n    partials[blockIdx.x].v = acc; partials[blockIdx.x].i = acci;\n    __threadfence();\n"
-          "    unsigned int ticket = atomicAdd(&counters[0], 1u);\n    is_last = (ticket == gridDim.x - 1);\n  }\n  __syncthreads();\n";
-    ss << "  if (!is_last) return;\n  __threadfence();\n";
+    // Cross-block hand-off without cache-wide fences: partials are written with agent-scope
+    // atomic stores (written through to the device coherence point, never left dirty in one
+    // XCD's L2), s_waitcnt 0 holds the ticket back until those stores are acknowledged, and the
+    // last block reads them with agent-scope atomic loads (which do not hit stale lines).
+    ss << "  if (threadIdx.x == 0) {\n    dali_publish(&partials[blockIdx.x].v, acc); dali_publish(&partials[blockIdx.x].i, acci);\n"
+          "    is_last = dali_take_ticket(&counters[0]) == gridDim.x - 1;\n  }\n  __syncthreads();\n";
+    ss << "  if (!is_last) return;\n";
     ss << "  acc = " << red.name << "::init<" << t << ">(); acci = 0;\n";
-    ss << "  // fixed combination order: thread k folds partials k, k+BT, ... then the block folds in wave order\n";
-    ss << "  for (unsigned int b = threadIdx.x; b < gridDim.x; b += BT) {\n";
-    ss << "    const " << t << " pv = __builtin_nontemporal_load(&partials[b].v); const int pi = __builtin_nontemporal_load(&partials[b].i); (void)pi;\n";
+    ss << "  // fixed combination order: thread k folds partials k, k+BT, ... (all loads issued first), then the block folds in wave order\n";
+    ss << "  {\n    constexpr int TAIL = " << TAIL << ";\n    " << t << " pv[TAIL]; int pi[TAIL];\n";
+    ss << "    _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) {\n      const unsigned int b = threadIdx.x + k * BT;\n"
+          "      if (b < gridDim.x) { pv[k] = dali_observe(&partials[b].v); pi[k] = dali_observe(&partials[b].i); }\n    }\n";
+    ss << "    _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) {\n      const unsigned int b = threadIdx.x + k * BT;\n      if (b < gridDim.x) {\n";
     if (!is_arg)
-        ss << "    acc = " << red.name << "::step<" << t << ">(acc, pv);\n";
+        ss << "        acc = " << red.name << "::step<" << t << ">(acc, pv[k]);\n";
     else
-        ss << "    if (" << red.name << "::better<" << t << ">(pv, acc) || (pv == acc && pi < acci)) { acc = pv; acci = pi; }\n";
-    ss << "  }\n  __syncthreads();\n";
+        ss << "        if (" << red.name << "::better<" << t << ">(pv[k], acc) || (pv[k] == acc && pi[k] < acci)) { acc = pv[k]; acci = pi[k]; }\n";
+    ss << "      }\n    }\n  }\n  __syncthreads();\n";
+
     if (!is_arg)
         ss << "  acc = dali_block_reduce<" << red.name << ", " << t << ", " << NW << ">(acc, smv);\n";
     else
         ss << "  dali_block_arg_reduce<" << red.name << ", " << t << ", " << NW << ">(acc, acci, smv, smi);\n";
-    ss << "  if (threadIdx.x == 0) {\n    counters[0] = 0;\n";
+    ss << "  if (threadIdx.x == 0) {\n    dali_publish(&counters[0], 0u);\n";
     // the reference stores a flat arg index in the input dtype
     if (!is_arg)
         ss << "    const " << ctype(red.dtype) << " red" << red_id << " = acc;\n";
@@ -1383,13 +1421,17 @@ bool try_all(const DestSpec& spec) {
     for (const ArrayArg& a : P.arrays)
         if (a.cls == Cls::FULL && a.buf->offset % 4 != 0) vec = false;
     int VEC = vec ? 4 : 1, BT = 256;
+    int max_el_all = 4;
+    for (const ArrayArg& a : P.arrays) max_el_all = std::max(max_el_all, size_of_dtype(a.buf->dtype));
+    const int UNROLL = max_el_all == 8 ? 4 : 8;  // vector loads in flight per thread
+    const int TAIL = 2, MAX_BLOCKS = TAIL * BT;  // 512 blocks; the last one folds every partial in one unrolled pass
     std::vector<Output> outs(1);
     outs[0].root = root_id;
     outs[0].array = dest_array;
     outs[0].op = spec.op;
     outs[0].cls = Cls::SCAL;
     std::ostringstream params;
-    params << VEC << "," << BT << "," << red_id;
+    params << VEC << "," << BT << "," << red_id << "," << UNROLL << "," << TAIL;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("all", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& K = specs_cache[h];
@@ -1405,12 +1447,12 @@ bool try_all(const DestSpec& spec) {
         K->plan.grid_kind = DALI_HIP_GRID_ALL;
         K->plan.work_begin = L.shape_pos[0];
         K->plan.work_count = 1;
-        K->plan.work_per_block = BT * VEC * 8;
-        K->plan.max_blocks = 2048;
+        K->plan.work_per_block = BT * VEC * UNROLL;
+        K->plan.max_blocks = MAX_BLOCKS;
         K->plan.ws_elsize = 16;
     }
     std::vector<std::vector<int>> shapes = {{(int)n}};
-    load_and_launch(*K, [&]() { return gen_all_kernel(P, red_id, root_id, dest_array, spec.op, L, VEC, BT, K->name); }, P, shapes);
+    load_and_launch(*K, [&]() { return gen_all_kernel(P, red_id, root_id, dest_array, spec.op, L, VEC, BT, UNROLL, TAIL, K->name); }, P, shapes);
     return true;
 }
 
@@ -1450,7 +1492,8 @@ bool col_eligible(const Array& a, int64_t K, int64_t X, std::set<const Expr*>& s
     }
 }
 
-std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATOR_T op, const IvLayout& L, int VEC, const std::string& kname) {
+std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATOR_T op, const IvLayout& L, int VEC, int UNR, int TAIL, int RG,
+                           const std::string& kname) {
     const PNode& red = P.nodes[red_id];
     std::string t = ctype(red.dtype);
     std::string dt = ctype(P.arrays[dest_array].buf->dtype);
@@ -1461,18 +1504,17 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     ss << codegen::kDevicePrelude;
     ss << kargs_struct(P, L);
     ss << "extern \"C\" __global__ __launch_bounds__(256) void " << kname << "(KArgs A) {\n";
-    ss << "  constexpr int VEC = " << VEC << ", NWAVE = 4, UNR = 4;\n";
+    // the 256 threads form RG row groups of TPP threads; a group reads TPP*VEC adjacent kept columns of one memory row
+    ss << "  constexpr int VEC = " << VEC << ", NWAVE = " << RG << ", TPP = " << 256 / RG << ", UNR = " << UNR << ", TAIL = " << TAIL << ";\n";
     ss << "  const long K = A.iv[" << L.shape_pos[0] << "], X = A.iv[" << L.shape_pos[0] + 1 << "];\n";
     ss << "  const long row = 0; const long C = K; (void)row; (void)C;\n";
-    ss << "  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;\n";
-    ss << "  const long k0 = ((long)blockIdx.x * 64 + lane) * VEC;\n";
+    ss << "  const int lane = threadIdx.x % TPP, wave = threadIdx.x / TPP;\n";
+    ss << "  const long k0 = ((long)blockIdx.x * TPP + lane) * VEC;\n";
     ss << "  const bool k_ok = k0 < K;\n";
-    // leaves: pointer to column k0, stride ld along the reduced axis
     for (size_t i = 0; i < P.arrays.size(); ++i) {
         const ArrayArg& a = P.arrays[i];
         std::string ty = ctype(a.buf->dtype);
         if (a.is_dest) {
-            std::string s = a.strided ? " * (long)A.iv[" + std::to_string(L.stride_pos[i]) + "]" : "";
             ss << "  " << ty << "* q" << i << " = (" << ty << "*)A.p[" << i << "];\n  const long ds" << i << " = " << (a.strided ? "A.iv[" + std::to_string(L.stride_pos[i]) + "]" : "1") << ";\n";
         } else if (a.cls == Cls::FULL) {
             ss << "  const " << ty << "* q" << i << " = (const " << ty << "*)A.p[" << i << "] + (k_ok ? k0 : 0);\n";
@@ -1485,29 +1527,33 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     for (size_t i = 0; i < P.arrays.size(); ++i)
         if (!P.arrays[i].is_dest && P.arrays[i].cls == Cls::FULL) full_leaves.push_back((int)i);
     ss << "  " << t << " acc[VEC];\n  _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = " << red.name << "::init<" << t << ">();\n";
-    ss << "  const long xstep = (long)gridDim.y * NWAVE;\n";
-    ss << "  if (k_ok) {\n    long x = (long)blockIdx.y * NWAVE + wave;\n";
+    // contiguous share of the reduced axis for this y-block, interleaved over its waves
+    ss << "  const long per_y = (X + gridDim.y - 1) / gridDim.y;\n";
+    ss << "  const long x_begin = (long)blockIdx.y * per_y, x_end = x_begin + per_y < X ? x_begin + per_y : X;\n";
+    ss << "  if (k_ok) {\n    long x = x_begin + wave;\n";
     std::vector<int> first_body(P.nodes.size(), -1);
-    auto body = [&](const std::string& xs, const std::string& indent, const std::string& sfx) {
-        for (int i : full_leaves) {
-            std::string ty = ctype(P.arrays[i].buf->dtype);
-            ss << indent << ty << " x" << i << sfx << "[VEC];\n";
-            ss << indent << "{ dali_vec<" << ty << ", VEC> tmp = dali_load<" << ty << ", VEC>(q" << i << " + (" << xs << ") * ld" << i << "); _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) x" << i << sfx << "[j] = tmp.v[j]; }\n";
-        }
-    };
-    // unrolled main loop: UNR independent row fetches in flight per lane
-    ss << "    for (; x + (UNR - 1) * xstep < X; x += UNR * xstep) {\n";
-    for (int u = 0; u < 4; ++u) body("x + " + std::to_string(u) + " * xstep", "      ", "u" + std::to_string(u));
-    for (int u = 0; u < 4; ++u) {
-        ss << "      {\n";
-        for (int i : full_leaves) ss << "        const " << ctype(P.arrays[i].buf->dtype) << "* x" << i << " = x" << i << "u" << u << ";\n";
-        ss << "        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n          const int col = 0; (void)col;\n";
+    // main loop: UNR independent row fetches in flight per lane
+    ss << "    for (; x + (UNR - 1) * NWAVE < x_end; x += UNR * NWAVE) {\n";
+    for (int i : full_leaves) {
+        std::string ty = ctype(P.arrays[i].buf->dtype);
+        ss << "      " << ty << " x" << i << "s[UNR][VEC];\n";
+        ss << "      _Pragma(\"unroll\") for (int u = 0; u < UNR; ++u) { dali_vec<" << ty << ", VEC> tmp = dali_load<" << ty << ", VEC>(q" << i
+           << " + (x + u * NWAVE) * ld" << i << "); _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) x" << i << "s[u][j] = tmp.v[j]; }\n";
+    }
+    ss << "      _Pragma(\"unroll\") for (int u = 0; u < UNR; ++u) {\n";
+    for (int i : full_leaves) ss << "        const " << ctype(P.arrays[i].buf->dtype) << "* x" << i << " = x" << i << "s[u];\n";
+    ss << "        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n          const int col = 0; (void)col;\n";
+    {
         BodyEmitter be(P, rp, true, 0, &first_body);
         std::string v = be.value(red.args[0]);
         ss << be.stmts.str() << "          acc[j] = " << red.name << "::step<" << t << ">(acc[j], " << v << ");\n        }\n      }\n";
     }
-    ss << "    }\n    for (; x < X; x += xstep) {\n";
-    body("x", "      ", "");
+    ss << "    }\n    for (; x < x_end; x += NWAVE) {\n";
+    for (int i : full_leaves) {
+        std::string ty = ctype(P.arrays[i].buf->dtype);
+        ss << "      " << ty << " x" << i << "[VEC];\n";
+        ss << "      { dali_vec<" << ty << ", VEC> tmp = dali_load<" << ty << ", VEC>(q" << i << " + x * ld" << i << "); _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) x" << i << "[j] = tmp.v[j]; }\n";
+    }
     ss << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        const int col = 0; (void)col;\n";
     {
         BodyEmitter be(P, rp, true, 0, &first_body);
@@ -1515,10 +1561,10 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
         ss << be.stmts.str() << "        acc[j] = " << red.name << "::step<" << t << ">(acc[j], " << v << ");\n      }\n";
     }
     ss << "    }\n  }\n";
-    // fold the 4 waves of the block in wave order
-    ss << "  __shared__ " << t << " sm[NWAVE][64 * VEC];\n  __shared__ int is_last;\n";
-    ss << "  _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) sm[wave][lane * VEC + j] = acc[j];\n  __syncthreads();\n";
-    ss << "  if (wave == 0) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n      " << t << " r = sm[0][lane * VEC + j];\n"
+    // fold the row groups of the block in group order
+    ss << "  __shared__ " << t << " sm[NWAVE][TPP * VEC];\n  __shared__ int is_last;\n";
+    ss << "  if (NWAVE > 1) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) sm[wave][lane * VEC + j] = acc[j];\n    __syncthreads();\n  }\n";
+    ss << "  if (NWAVE > 1 && wave == 0) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n      " << t << " r = sm[0][lane * VEC + j];\n"
        << "      _Pragma(\"unroll\") for (int w = 1; w < NWAVE; ++w) r = " << red.name << "::step<" << t << ">(r, sm[w][lane * VEC + j]);\n      acc[j] = r;\n    }\n  }\n";
     auto emit_store = [&](const std::string& indent) {
         ss << indent << "_Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) if (k0 + j < K) { " << dt << "* dp = q" << dest_array << " + (k0 + j) * ds" << dest_array
@@ -1529,17 +1575,24 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     ss << "    }\n    return;\n  }\n";
     ss << "  unsigned int* counters = (unsigned int*)A.ws;\n";
     ss << "  " << t << "* partials = (" << t << "*)((char*)A.ws + " << 16384 * 4 << ");\n";
-    ss << "  const long KP = (long)gridDim.x * 64 * VEC;  // padded kept extent of the partial rows\n";
-    ss << "  if (wave == 0) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) partials[(long)blockIdx.y * KP + ((long)blockIdx.x * 64 + lane) * VEC + j] = acc[j];\n"
-          "    __threadfence();\n  }\n  __syncthreads();\n";
-    ss << "  if (threadIdx.x == 0) { unsigned int ticket = atomicAdd(&counters[blockIdx.x], 1u); is_last = (ticket == gridDim.y - 1); }\n  __syncthreads();\n";
-    ss << "  if (!is_last) return;\n  __threadfence();\n";
+    ss << "  const long KP = (long)gridDim.x * TPP * VEC;  // padded kept extent of one row of partials\n";
+    ss << "  const long pcol = ((long)blockIdx.x * TPP + lane) * VEC;\n";
+    // same fence-free hand-off as the full reduction: agent-scope atomic stores, wait for their
+    // acknowledgement, then the ticket; the last block of the strip observes with agent-scope loads
+    ss << "  if (wave == 0) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) dali_publish(partials + (long)blockIdx.y * KP + pcol + j, acc[j]);\n"
+          "    __builtin_amdgcn_s_waitcnt(0);\n  }\n  __syncthreads();\n";
+    ss << "  if (threadIdx.x == 0) is_last = dali_take_ticket(&counters[blockIdx.x]) == gridDim.y - 1;\n  __syncthreads();\n";
+    ss << "  if (!is_last) return;\n";
     ss << "  if (wave == 0) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = " << red.name << "::init<" << t << ">();\n";
-    ss << "    for (unsigned int y = 0; y < gridDim.y; ++y) {\n      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = " << red.name << "::step<" << t
-       << ">(acc[j], __builtin_nontemporal_load(&partials[(long)y * KP + ((long)blockIdx.x * 64 + lane) * VEC + j]));\n    }\n";
+    ss << "    // partial rows are folded in y order; TAIL of them are in flight at a time\n";
+    ss << "    for (unsigned int y0 = 0; y0 < gridDim.y; y0 += TAIL) {\n      dali_vec<" << t << ", VEC> pv[TAIL];\n";
+    ss << "      _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) if (y0 + k < gridDim.y) {\n"
+          "        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) pv[k].v[j] = dali_observe(partials + (long)(y0 + k) * KP + pcol + j);\n      }\n";
+    ss << "      _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) if (y0 + k < gridDim.y) {\n        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = "
+       << red.name << "::step<" << t << ">(acc[j], pv[k].v[j]);\n      }\n    }\n";
     ss << "    if (k_ok) {\n";
     emit_store("      ");
-    ss << "    }\n  }\n  if (threadIdx.x == 0) counters[blockIdx.x] = 0;\n}\n";
+    ss << "    }\n  }\n  if (threadIdx.x == 0) dali_publish(&counters[blockIdx.x], 0u);\n}\n";
     return ss.str();
 }
 
@@ -1611,13 +1664,17 @@ bool try_col(const DestSpec& spec) {
     for (const ArrayArg& a : P.arrays)
         if (!a.is_dest && a.cls == Cls::FULL && (a.buf->offset % 4 != 0 || a.col_stride % 4 != 0)) vec = false;
     int VEC = vec ? 4 : 1;
+    const int UNR = 8, TAIL = 16;
+    // widest row piece the kept extent can fill: 1 group of 256 threads for wide matrices, up to 4 groups of 64
+    int RG = 1;
+    while (RG < 4 && (int64_t)(256 / RG) * VEC > K) RG *= 2;
     std::vector<Output> outs(1);
     outs[0].root = red_id;
     outs[0].array = dest_array;
     outs[0].op = spec.op;
     outs[0].cls = Cls::ROW;
     std::ostringstream params;
-    params << VEC;
+    params << VEC << "," << UNR << "," << TAIL << "," << RG;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("col", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& Kp = specs_cache[h];
@@ -1633,14 +1690,14 @@ bool try_col(const DestSpec& spec) {
         Kp->plan.grid_kind = DALI_HIP_GRID_COLS;
         Kp->plan.work_begin = L.shape_pos[0];
         Kp->plan.work_count = 1;
-        Kp->plan.work_per_block = 64 * VEC;
+        Kp->plan.work_per_block = (256 / RG) * VEC;
         Kp->plan.work2_begin = L.shape_pos[0] + 1;
-        Kp->plan.work2_per_block = 128;  // reduced rows per y-block
-        Kp->plan.max_blocks2 = 64;
+        Kp->plan.work2_per_block = 256;  // reduced rows per y-block
+        Kp->plan.max_blocks2 = 256;
         Kp->plan.ws_elsize = size_of_dtype(re->dtype);
     }
     std::vector<std::vector<int>> shapes = {{(int)K, (int)X}};
-    load_and_launch(*Kp, [&]() { return gen_col_kernel(P, red_id, dest_array, spec.op, L, VEC, Kp->name); }, P, shapes);
+    load_and_launch(*Kp, [&]() { return gen_col_kernel(P, red_id, dest_array, spec.op, L, VEC, UNR, TAIL, RG, Kp->name); }, P, shapes);
     return true;
 }
 
