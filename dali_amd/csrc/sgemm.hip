@@ -1,5 +1,5 @@
-// fp32 GEMM on the CDNA4 matrix cores (v_mfma_f32_32x32x2_f32), LDS-staged and
-// software-pipelined, for dali_hip_sgemm / dali_hip_sgemm_pair.
+// fp32 GEMM on the CDNA4 matrix cores (v_mfma_f32_32x32x2_f32), LDS-staged with
+// a multi-slab register prefetch, for dali_hip_sgemm / dali_hip_sgemm_pair.
 //
 // Row-major view used inside this file: C[M,N] = alpha * sum_s A_s[M,K_s] * B_s[K_s,N] + beta * C
 // for one or two (A_s, B_s) segments. The column-major entry points map onto it
@@ -7,14 +7,27 @@
 // calls a column-major BLAS (dali/array/gemm/cpu_gemm.cpp:43-68).
 //
 // Work decomposition: a 256-thread workgroup (4 waves, 2x2) owns a BM x BN tile
-// of C; each wave owns (BM/2) x (BN/2), built from 32x32 MFMA accumulators.
-// Operand tiles are staged as As[k][m] and Bs[k][n] so that the MFMA operand
-// fetch (lane l reads element l%32 of row k + l/32) is a conflict-free 32-float
-// row read. The next K-slab is fetched from global memory into registers while
-// the current one is consumed from LDS (two LDS buffers, one barrier per slab).
+// of C; each wave owns (BM/2) x (BN/2), built from 32x32 MFMA accumulators. K is
+// walked in slabs of BK (32 or 64).
+//
+// LDS layout.  As[m][k]: rows of BK floats in 16-byte granules, granule g of row m
+// stored in slot (g & ~7) | ((g ^ m) & 7). A lane's MFMA operands for four consecutive
+// MFMAs are one ds_read_b128 (granule 2t + h of its row), and the eight lanes the
+// LDS serves per cycle hit eight different slots, so the read is conflict-free.
+// Bs[k][n]: natural rows; lane l reads column l % 32 of row k, a conflict-free
+// 32-float row read. Within a group of eight k the two half-waves (h = lane / 32)
+// take k = 8t + 4h + c for c = 0..3, the same assignment for A and B, so every
+// MFMA still sums two distinct k.
+//
+// Latency.  One workgroup per CU means one wave per SIMD, so nothing hides a
+// global-memory round trip except distance: slabs are fetched into registers
+// DEPTH slabs ahead of their use, written to the other LDS buffer one slab ahead,
+// and consumed from LDS while the MFMA pipe works (one barrier per slab).
 #include "runtime.h"
 
+#include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 namespace dali_hip {
 
@@ -33,21 +46,31 @@ struct GemmArgs {
     float* C;
     int ldc;
     float alpha, beta;
+    // split-K: gridDim.z workgroups share one tile of C, each walking a contiguous share of the
+    // slabs; partial tiles and the per-tile ticket counters live in the library workspace
+    unsigned int* counters;
+    float* partials;
 };
 
-constexpr int BK = 16;
+__device__ __forceinline__ void publish(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float observe(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-template <int BM, int BN, bool TA, bool TB, bool VEC>
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int DEPTH, bool EDGE>
 __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
-    constexpr int PAD = 4;
     constexpr int WTM = BM / 2, WTN = BN / 2;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr int A_F4 = BM * BK / 4 / 256;  // float4 fetches per thread for the A slab
     constexpr int B_F4 = BN * BK / 4 / 256;
+    constexpr int BPAD = 4;
+    // a lone accumulator per wave would serialise dependent MFMAs: split k over two chains
+    constexpr int CHAINS = (TM * TN == 1) ? 2 : 1;
     static_assert(A_F4 >= 1 && B_F4 >= 1, "tile too small for 256 threads");
 
-    __shared__ float As[2][BK][BM + PAD];
-    __shared__ float Bs[2][BK][BN + PAD];
+    __shared__ __attribute__((aligned(16))) float As[2][BM][BK];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK][BN + BPAD];
+
+    // slot of 16-byte granule `gr` in row m: the low three bits are permuted per row
+    auto swz = [](int gr, int m) { return (gr & ~7) | ((gr ^ m) & 7); };
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -57,103 +80,117 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const int M = g.M, N = g.N;
 
-    floatx16 acc[TM][TN];
+    floatx16 acc[CHAINS][TM][TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int c = 0; c < CHAINS; ++c)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[c][i][j][v] = 0.f;
 
-    float4 ra[A_F4], rb[B_F4];
+    float4 ra[DEPTH][A_F4], rb[DEPTH][B_F4];
 
-    // fetch one BK-deep slab of segment s starting at k0 into registers
-    auto fetch = [&](const GemmSeg& s, int k0) {
+    // flat list of slabs over the segments
+    const int slabs0 = (g.seg[0].K + BK - 1) / BK;
+    const int slabs1 = g.nseg > 1 ? (g.seg[1].K + BK - 1) / BK : 0;
+    const int nslab_all = slabs0 + slabs1;
+    // this workgroup's share of the slabs (all of them without split-K)
+    const int s_begin = (int)((long)blockIdx.z * nslab_all / gridDim.z);
+    const int nslab = (int)((long)(blockIdx.z + 1) * nslab_all / gridDim.z) - s_begin;
+
+    // Per-thread source coordinates of its fetches within a slab (fixed for the whole kernel).
+    // A: row `ar` (or k row for the transposed storage), 4-float granule starting at column `ac`.
+    int a_r[A_F4], a_c[A_F4], b_r[B_F4], b_c[B_F4];
+#pragma unroll
+    for (int t = 0; t < A_F4; ++t) {
+        int idx = tid + t * 256;
+        if (!TA) {
+            a_r[t] = m0 + idx / (BK / 4);        // m
+            a_c[t] = (idx % (BK / 4)) * 4;       // k offset inside the slab
+        } else {
+            a_r[t] = idx / (BM / 4);             // k offset inside the slab
+            a_c[t] = m0 + (idx % (BM / 4)) * 4;  // m
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < B_F4; ++t) {
+        int idx = tid + t * 256;
+        if (!TB) {
+            b_r[t] = idx / (BN / 4);             // k offset inside the slab
+            b_c[t] = n0 + (idx % (BN / 4)) * 4;  // n
+        } else {
+            b_r[t] = n0 + idx / (BK / 4);        // n
+            b_c[t] = (idx % (BK / 4)) * 4;       // k offset inside the slab
+        }
+    }
+
+    // One 4-float granule at row r, columns c..c+3 of a row-major array with `rows` x `cols`
+    // valid entries. Interior tiles (EDGE == false) load unconditionally; edge tiles clamp the
+    // address and zero what lies outside, without branching.
+    auto load4 = [&](const float* base, int ld, int r, int c, int rows, int cols) -> float4 {
+        if (!EDGE) return *(const float4*)(base + (size_t)r * ld + c);
+        const bool rv = r < rows;
+        const size_t ro = (size_t)(rv ? r : 0) * ld;
+        if (VEC) {
+            // cols is a multiple of 4 here or the granule is cut: handle both with per-element masks
+            const bool full = rv && c + 3 < cols;
+            const float4 v = *(const float4*)(base + ro + (full ? c : 0));
+            if (full) return v;
+        }
+        float4 v;
+        v.x = base[ro + ((rv && c + 0 < cols) ? c + 0 : 0)];
+        v.y = base[ro + ((rv && c + 1 < cols) ? c + 1 : 0)];
+        v.z = base[ro + ((rv && c + 2 < cols) ? c + 2 : 0)];
+        v.w = base[ro + ((rv && c + 3 < cols) ? c + 3 : 0)];
+        v.x = (rv && c + 0 < cols) ? v.x : 0.f;
+        v.y = (rv && c + 1 < cols) ? v.y : 0.f;
+        v.z = (rv && c + 2 < cols) ? v.z : 0.f;
+        v.w = (rv && c + 3 < cols) ? v.w : 0.f;
+        return v;
+    };
+
+    // fetch slab `i` (index into the flat slab list) into register stage S
+    auto fetch = [&](auto S, int i) {
+        constexpr int st = decltype(S)::value;
+        const bool first = i < slabs0;
+        const float* sa = first ? g.seg[0].A : g.seg[1].A;
+        const float* sb = first ? g.seg[0].B : g.seg[1].B;
+        const int lda = first ? g.seg[0].lda : g.seg[1].lda;
+        const int ldb = first ? g.seg[0].ldb : g.seg[1].ldb;
+        const int K = first ? g.seg[0].K : g.seg[1].K;
+        const int k0 = (first ? i : i - slabs0) * BK;
 #pragma unroll
         for (int t = 0; t < A_F4; ++t) {
-            int idx = tid + t * 256;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (!TA) {
-                // A[m][k], k contiguous: 4 consecutive k of one row
-                int m = m0 + idx / (BK / 4), k = k0 + (idx % (BK / 4)) * 4;
-                if (m < M) {
-                    const float* p = s.A + (size_t)m * s.lda + k;
-                    if (VEC && k + 3 < s.K) {
-                        v = *(const float4*)p;
-                    } else {
-                        if (k + 0 < s.K) v.x = p[0];
-                        if (k + 1 < s.K) v.y = p[1];
-                        if (k + 2 < s.K) v.z = p[2];
-                        if (k + 3 < s.K) v.w = p[3];
-                    }
-                }
-            } else {
-                // A stored as [K][M], m contiguous: 4 consecutive m of one k
-                int k = k0 + idx / (BM / 4), m = m0 + (idx % (BM / 4)) * 4;
-                if (k < s.K) {
-                    const float* p = s.A + (size_t)k * s.lda + m;
-                    if (VEC && m + 3 < M) {
-                        v = *(const float4*)p;
-                    } else {
-                        if (m + 0 < M) v.x = p[0];
-                        if (m + 1 < M) v.y = p[1];
-                        if (m + 2 < M) v.z = p[2];
-                        if (m + 3 < M) v.w = p[3];
-                    }
-                }
-            }
-            ra[t] = v;
+            if (!TA)
+                ra[st][t] = load4(sa, lda, a_r[t], k0 + a_c[t], M, K);
+            else
+                ra[st][t] = load4(sa, lda, k0 + a_r[t], a_c[t], K, M);
         }
 #pragma unroll
         for (int t = 0; t < B_F4; ++t) {
-            int idx = tid + t * 256;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (!TB) {
-                // B[k][n], n contiguous
-                int k = k0 + idx / (BN / 4), n = n0 + (idx % (BN / 4)) * 4;
-                if (k < s.K) {
-                    const float* p = s.B + (size_t)k * s.ldb + n;
-                    if (VEC && n + 3 < N) {
-                        v = *(const float4*)p;
-                    } else {
-                        if (n + 0 < N) v.x = p[0];
-                        if (n + 1 < N) v.y = p[1];
-                        if (n + 2 < N) v.z = p[2];
-                        if (n + 3 < N) v.w = p[3];
-                    }
-                }
-            } else {
-                // B stored as [N][K], k contiguous
-                int n = n0 + idx / (BK / 4), k = k0 + (idx % (BK / 4)) * 4;
-                if (n < N) {
-                    const float* p = s.B + (size_t)n * s.ldb + k;
-                    if (VEC && k + 3 < s.K) {
-                        v = *(const float4*)p;
-                    } else {
-                        if (k + 0 < s.K) v.x = p[0];
-                        if (k + 1 < s.K) v.y = p[1];
-                        if (k + 2 < s.K) v.z = p[2];
-                        if (k + 3 < s.K) v.w = p[3];
-                    }
-                }
-            }
-            rb[t] = v;
+            if (!TB)
+                rb[st][t] = load4(sb, ldb, k0 + b_r[t], b_c[t], K, N);
+            else
+                rb[st][t] = load4(sb, ldb, b_r[t], k0 + b_c[t], N, K);
         }
     };
 
-    auto stage = [&](int buf) {
+    // register stage S -> LDS buffer `buf`
+    auto stage = [&](auto S, int buf) {
+        constexpr int st = decltype(S)::value;
 #pragma unroll
         for (int t = 0; t < A_F4; ++t) {
             int idx = tid + t * 256;
             if (!TA) {
-                int m = idx / (BK / 4), k = (idx % (BK / 4)) * 4;
-                As[buf][k + 0][m] = ra[t].x;
-                As[buf][k + 1][m] = ra[t].y;
-                As[buf][k + 2][m] = ra[t].z;
-                As[buf][k + 3][m] = ra[t].w;
+                int m = idx / (BK / 4), gr = idx % (BK / 4);
+                *(float4*)&As[buf][m][swz(gr, m) * 4] = ra[st][t];
             } else {
                 int k = idx / (BM / 4), m = (idx % (BM / 4)) * 4;
-                *(float4*)&As[buf][k][m] = ra[t];
+                const float vals[4] = {ra[st][t].x, ra[st][t].y, ra[st][t].z, ra[st][t].w};
+#pragma unroll
+                for (int c = 0; c < 4; ++c) As[buf][m + c][(swz(k >> 2, m + c) << 2) | (k & 3)] = vals[c];
             }
         }
 #pragma unroll
@@ -161,82 +198,175 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
             int idx = tid + t * 256;
             if (!TB) {
                 int k = idx / (BN / 4), n = (idx % (BN / 4)) * 4;
-                *(float4*)&Bs[buf][k][n] = rb[t];
+                *(float4*)&Bs[buf][k][n] = rb[st][t];
             } else {
                 int n = idx / (BK / 4), k = (idx % (BK / 4)) * 4;
-                Bs[buf][k + 0][n] = rb[t].x;
-                Bs[buf][k + 1][n] = rb[t].y;
-                Bs[buf][k + 2][n] = rb[t].z;
-                Bs[buf][k + 3][n] = rb[t].w;
+                Bs[buf][k + 0][n] = rb[st][t].x;
+                Bs[buf][k + 1][n] = rb[st][t].y;
+                Bs[buf][k + 2][n] = rb[st][t].z;
+                Bs[buf][k + 3][n] = rb[st][t].w;
             }
         }
     };
 
-    // flat list of slabs over the segments
-    int slabs0 = (g.seg[0].K + BK - 1) / BK;
-    int slabs1 = g.nseg > 1 ? (g.seg[1].K + BK - 1) / BK : 0;
-    int nslab = slabs0 + slabs1;
-    auto fetch_slab = [&](int i) {
-        if (i < slabs0)
-            fetch(g.seg[0], i * BK);
-        else
-            fetch(g.seg[1], (i - slabs0) * BK);
+    // MFMA operands of k-group t (eight k): one granule of A per 32-row block, four B values per
+    // 32-column block.
+    auto load_ops = [&](int buf, int t, float4 (&a4)[TM], float (&b)[TN][4]) {
+#pragma unroll
+        for (int ii = 0; ii < TM; ++ii) {
+            int m = wm * WTM + ii * 32 + l32;
+            a4[ii] = *(const float4*)&As[buf][m][swz(2 * t + h, m) << 2];
+        }
+#pragma unroll
+        for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) b[jj][c] = Bs[buf][8 * t + 4 * h + c][wn * WTN + jj * 32 + l32];
     };
 
-    if (nslab > 0) {
-        fetch_slab(0);
-        stage(0);
-    }
-    __syncthreads();
-    for (int i = 0; i < nslab; ++i) {
-        int cur = i & 1;
-        if (i + 1 < nslab) fetch_slab(i + 1);
+    // With a single 32x32 accumulator tile per wave the LDS reads of group t+1 are issued before
+    // the MFMAs of group t and kept there (scheduling barriers), so an LDS round trip hides
+    // behind a full group of MFMAs instead of being waited for in front of every pair. Larger
+    // wave tiles have enough independent MFMAs per group and are left to the compiler's scheduler.
+    auto compute = [&](int buf) {
+        float4 a4[2][TM];
+        float b[2][TN][4];
+        load_ops(buf, 0, a4[0], b[0]);
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-            float a[TM], b[TN];
+        for (int t = 0; t < BK / 8; ++t) {
+            const int cur = t & 1;
+            if (t + 1 < BK / 8) load_ops(buf, t + 1, a4[cur ^ 1], b[cur ^ 1]);
+            if (TM * TN == 1) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int ii = 0; ii < TM; ++ii) a[ii] = As[cur][kk + h][wm * WTM + ii * 32 + l32];
+            for (int c = 0; c < 4; ++c)
 #pragma unroll
-            for (int jj = 0; jj < TN; ++jj) b[jj] = Bs[cur][kk + h][wn * WTN + jj * 32 + l32];
+                for (int ii = 0; ii < TM; ++ii) {
+                    const float a = c == 0 ? a4[cur][ii].x : (c == 1 ? a4[cur][ii].y : (c == 2 ? a4[cur][ii].z : a4[cur][ii].w));
 #pragma unroll
-            for (int ii = 0; ii < TM; ++ii)
-#pragma unroll
-                for (int jj = 0; jj < TN; ++jj)
-                    acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ii], b[jj], acc[ii][jj], 0, 0, 0);
+                    for (int jj = 0; jj < TN; ++jj) {
+                        const int ch = CHAINS == 2 ? (c & 1) : 0;
+                        acc[ch][ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b[cur][jj][c], acc[ch][ii][jj], 0, 0, 0);
+                    }
+                }
+            if (TM * TN == 1) __builtin_amdgcn_sched_barrier(0);
         }
-        if (i + 1 < nslab) stage(cur ^ 1);
-        __syncthreads();
+    };
+
+    // prologue: slabs 0 .. DEPTH-1 in flight, slab 0 staged
+    auto for_stages = [&](auto f) {
+        f(std::integral_constant<int, 0>{});
+        if constexpr (DEPTH > 1) f(std::integral_constant<int, 1>{});
+        if constexpr (DEPTH > 2) f(std::integral_constant<int, 2>{});
+        if constexpr (DEPTH > 3) f(std::integral_constant<int, 3>{});
+    };
+    for_stages([&](auto S) {
+        if (decltype(S)::value < nslab) fetch(S, s_begin + decltype(S)::value);
+    });
+    if (nslab > 0) stage(std::integral_constant<int, 0>{}, 0);
+    __syncthreads();
+
+    // slab i lives in register stage i % DEPTH until it is staged; the loop is
+    // unrolled DEPTH times so that the stage index is a compile-time constant
+    for (int base = 0; base < nslab; base += DEPTH) {
+        for_stages([&](auto S) {
+            constexpr int st = decltype(S)::value;
+            const int i = base + st;
+            if (i < nslab) {
+                const int cur = i & 1;
+                // stage slab i+1 (already in registers) into the other buffer, then reuse
+                // the registers slab i occupied for slab i+DEPTH
+                if (i + 1 < nslab) stage(std::integral_constant<int, (st + 1) % DEPTH>{}, cur ^ 1);
+                if (i + DEPTH < nslab) fetch(S, s_begin + i + DEPTH);
+                compute(cur);
+                __syncthreads();
+            }
+        });
     }
 
     // epilogue: lane holds column l32 and rows 8*(v/4) + 4*h + v%4 of each 32x32 tile
     const float alpha = g.alpha, beta = g.beta;
+    const bool split = gridDim.z > 1;
+    float* part = nullptr;
+    const int tile_id = blockIdx.y * gridDim.x + blockIdx.x;
+    if (split) {
+        // every share publishes its partial tile (agent-scope stores, no cache-wide fence); the
+        // workgroup that draws the last ticket folds all shares in z order, so the sum does not
+        // depend on which share finished last
+        part = g.partials + (size_t)tile_id * gridDim.z * (BM * BN);
+        float* mine = part + (size_t)blockIdx.z * (BM * BN);
+#pragma unroll
+        for (int ii = 0; ii < TM; ++ii)
+#pragma unroll
+            for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int lm = wm * WTM + ii * 32 + 8 * (v / 4) + 4 * h + (v % 4), ln = wn * WTN + jj * 32 + l32;
+                    float sum = acc[0][ii][jj][v];
+                    if (CHAINS == 2) sum += acc[CHAINS - 1][ii][jj][v];
+                    publish(mine + lm * BN + ln, sum);
+                }
+        __builtin_amdgcn_s_waitcnt(0);
+        __shared__ int is_last;
+        __syncthreads();
+        if (tid == 0) {
+            unsigned int ticket = __hip_atomic_fetch_add(g.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = ticket == gridDim.z - 1;
+        }
+        __syncthreads();
+        if (!is_last) return;
+    }
 #pragma unroll
     for (int ii = 0; ii < TM; ++ii)
 #pragma unroll
         for (int jj = 0; jj < TN; ++jj) {
             int n = n0 + wn * WTN + jj * 32 + l32;
-            if (n >= N) continue;
+            if (EDGE && n >= N) continue;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 int m = m0 + wm * WTM + ii * 32 + 8 * (v / 4) + 4 * h + (v % 4);
-                if (m < M) {
+                if (!EDGE || m < M) {
                     float* c = g.C + (size_t)m * g.ldc + n;
-                    float r = alpha * acc[ii][jj][v];
+                    float sum;
+                    if (split) {
+                        int lm = m - m0, ln = n - n0;
+                        sum = 0.f;
+                        for (unsigned z = 0; z < gridDim.z; ++z) sum += observe(part + (size_t)z * (BM * BN) + lm * BN + ln);
+                    } else {
+                        sum = acc[0][ii][jj][v];
+                        if (CHAINS == 2) sum += acc[CHAINS - 1][ii][jj][v];
+                    }
+                    float r = alpha * sum;
                     if (beta != 0.f) r += beta * *c;
                     *c = r;
                 }
             }
         }
+    if (split && tid == 0) __hip_atomic_store(g.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int BM, int BN>
-static int launch_tile(const GemmArgs& g, bool ta, bool tb, bool vec) {
+template <int BM, int BN, int BK, int DEPTH>
+static int launch_tile(GemmArgs g, bool ta, bool tb, bool vec, int split_k) {
+    // interior-only problems (every tile and slab full, 16-byte aligned rows) take the unchecked kernel
+    bool edge = !vec || g.M % BM != 0 || g.N % BN != 0;
+    for (int s = 0; s < g.nseg; ++s) edge = edge || g.seg[s].K % BK != 0;
     dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM);
+    int nslab = 0;
+    for (int s = 0; s < g.nseg; ++s) nslab += (g.seg[s].K + BK - 1) / BK;
+    size_t tiles = (size_t)grid.x * grid.y;
+    if (split_k > nslab) split_k = nslab > 0 ? nslab : 1;
+    if (split_k > 1 && (tiles > (size_t)kWorkspaceCounters || tiles * split_k * BM * BN * sizeof(float) > kWorkspacePartialBytes)) split_k = 1;
+    grid.z = split_k;
+    g.counters = (unsigned int*)workspace();
+    g.partials = (float*)(workspace() + kWorkspaceCounterBytes);
     dim3 block(256);
     hipStream_t st = stream();
-#define DALI_GEMM_CASE(TA_, TB_, V_)                                                   \
-    if (ta == TA_ && tb == TB_ && vec == V_) {                                         \
-        hipLaunchKernelGGL((sgemm_kernel<BM, BN, TA_, TB_, V_>), grid, block, 0, st, g); \
+    static const int pad_env = getenv("DALI_HIP_GEMM_PAD_LDS") ? atoi(getenv("DALI_HIP_GEMM_PAD_LDS")) : 0;
+    const unsigned pad_lds = (unsigned)pad_env;
+#define DALI_GEMM_CASE(TA_, TB_, V_)                                                                        \
+    if (ta == TA_ && tb == TB_ && vec == V_) {                                                              \
+        if (edge)                                                                                           \
+            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, TA_, TB_, V_, DEPTH, true>), grid, block, pad_lds, st, g);  \
+        else if (V_)                                                                                        \
+            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, TA_, TB_, true, DEPTH, false>), grid, block, pad_lds, st, g); \
     }
     DALI_GEMM_CASE(false, false, true)
     DALI_GEMM_CASE(false, false, false)
@@ -295,8 +425,17 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         vec = false;
     }
     long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-    if (tiles128 >= 192) return launch_tile<128, 128>(g, ta, tb, vec);
-    return launch_tile<64, 64>(g, ta, tb, vec);
+    static const int variant = getenv("DALI_HIP_GEMM_VARIANT") ? atoi(getenv("DALI_HIP_GEMM_VARIANT")) : 0;
+    if (tiles128 >= 192) return launch_tile<128, 128, 32, 2>(g, ta, tb, vec, 1);
+    // Small grids: 64x64 tiles, and when even those leave CUs with a single workgroup, split K so
+    // that two workgroups share a CU and one's barriers and memory waits hide behind the other's MFMAs.
+    long tiles64 = (long)((M + 63) / 64) * ((N + 63) / 64);
+    static const int split_env = getenv("DALI_HIP_GEMM_SPLITK") ? atoi(getenv("DALI_HIP_GEMM_SPLITK")) : 0;
+    int split_k = split_env > 0 ? split_env : 1;
+    (void)tiles64;
+    if (variant == 1) return launch_tile<64, 64, 32, 3>(g, ta, tb, vec, split_k);
+    if (variant == 2) return launch_tile<64, 64, 64, 3>(g, ta, tb, vec, split_k);
+    return launch_tile<64, 64, 64, 2>(g, ta, tb, vec, split_k);
 }
 
 }  // namespace dali_hip
