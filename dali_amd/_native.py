@@ -82,6 +82,10 @@ HIP_SYMBOLS = {
     "dali_hip_set_cache_dir": (_i, [C.c_char_p]),
     "dali_hip_sgemm": (_i, [_i, _i, _i, _i, _i, C.c_float, H, _i, H, _i, C.c_float, H, _i]),
     "dali_hip_sgemm_pair": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, C.c_float, H, _i, H, _i, H, _i, H, _i, C.c_float, H, _i]),
+    "dali_hip_capture_begin": (_i, []),
+    "dali_hip_capture_end": (_i, [C.POINTER(H)]),
+    "dali_hip_graph_launch": (_i, [H]),
+    "dali_hip_graph_destroy": (_i, [H]),
     "dali_hip_event_create": (_i, [C.POINTER(H)]),
     "dali_hip_event_record": (_i, [H]),
     "dali_hip_event_elapsed_ms": (_i, [H, H, C.POINTER(C.c_float)]),
@@ -138,10 +142,12 @@ FRONT_SYMBOLS = {
     "dali_fe_device_ptr": (H, [H]),
     "dali_fe_stats": (_i, [C.POINTER(_u64)] * 4),
     "dali_fe_last_kernel_kinds": (C.c_char_p, []),
+    "dali_fe_last_kernel_names": (C.c_char_p, []),
     "dali_fe_last_source": (C.c_char_p, []),
     "dali_fe_generate_only": (_i, [_HP, _i, _i]),
     "dali_fe_record_begin": (H, []),
     "dali_fe_record_end": (_i, [H]),
+    "dali_fe_record_make_graph": (_i, [H]),
     "dali_fe_replay": (_i, [H, _i]),
     "dali_fe_record_free": (None, [H]),
 }

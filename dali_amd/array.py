@@ -272,6 +272,10 @@ def last_kernel_kinds():
     return front.dali_fe_last_kernel_kinds().decode()
 
 
+def last_kernel_names():
+    return front.dali_fe_last_kernel_names().decode()
+
+
 def last_source():
     return front.dali_fe_last_source().decode()
 
@@ -299,6 +303,12 @@ class Recording(object):
     def __exit__(self, *exc):
         self.launches = front.dali_fe_record_end(self._rec)
         return False
+
+    def make_graph(self):
+        """Instantiate a HIP graph of the stored launches; later replays launch the graph."""
+        if front.dali_fe_record_make_graph(self._rec) != 0:
+            raise fe_error("make_graph")
+        return self
 
     def replay(self, times=1):
         if front.dali_fe_replay(self._rec, times) != 0:

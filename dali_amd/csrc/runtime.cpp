@@ -537,9 +537,40 @@ int dali_hip_launch(uint64_t hash, void** array_data, const int* offsets, const 
     if (gx > 2147483647LL || gy > 65535) return fail("dali_hip_launch: grid %lld x %lld too large", (long long)gx, (long long)gy);
     size_t karg = m->karg_bytes;
     void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, buf, HIP_LAUNCH_PARAM_BUFFER_SIZE, &karg, HIP_LAUNCH_PARAM_END};
-    hipError_t e = hipModuleLaunchKernel(m->fn, (unsigned)gx, (unsigned)gy, 1, (unsigned)P.block_threads, 1, 1, 0,
+    static const unsigned lds_pad = getenv("DALI_HIP_LAUNCH_LDS_PAD") ? (unsigned)atoi(getenv("DALI_HIP_LAUNCH_LDS_PAD")) : 0u;
+    hipError_t e = hipModuleLaunchKernel(m->fn, (unsigned)gx, (unsigned)gy, 1, (unsigned)P.block_threads, 1, 1, lds_pad,
                                          r.stream, nullptr, extra);
     if (e != hipSuccess) return fail("hipModuleLaunchKernel failed: %s", hipGetErrorString(e));
+    return DALI_HIP_OK;
+}
+
+int dali_hip_capture_begin(void) {
+    if (ensure_init()) return DALI_HIP_ERROR;
+    HIP_TRY(hipStreamBeginCapture(rt().stream, hipStreamCaptureModeThreadLocal));
+    return DALI_HIP_OK;
+}
+
+int dali_hip_capture_end(void** graph_exec) {
+    hipGraph_t graph = nullptr;
+    HIP_TRY(hipStreamEndCapture(rt().stream, &graph));
+    if (!graph) return fail("dali_hip_capture_end: nothing was captured");
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return fail("hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    *graph_exec = (void*)exec;
+    return DALI_HIP_OK;
+}
+
+int dali_hip_graph_launch(void* graph_exec) {
+    HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph_exec, rt().stream));
+    return DALI_HIP_OK;
+}
+
+int dali_hip_graph_destroy(void* graph_exec) {
+    if (!graph_exec) return DALI_HIP_OK;
+    HIP_TRY(hipStreamSynchronize(rt().stream));
+    HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
     return DALI_HIP_OK;
 }
 

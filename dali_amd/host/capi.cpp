@@ -3,6 +3,7 @@
 
 #include <cstring>
 
+#include "../../include/dali_hip.h"
 #include "expr.h"
 
 using dali::Array;
@@ -143,23 +144,48 @@ const char* dali_fe_last_kernel_kinds(void) {
     g_kinds = dali::jit_stats().last_kernel_kinds;
     return g_kinds.c_str();
 }
+const char* dali_fe_last_kernel_names(void) {
+    static thread_local std::string names;
+    names = dali::jit_stats().last_kernel_names;
+    return names.c_str();
+}
 const char* dali_fe_last_source(void) { return dali::last_generated_source().c_str(); }
 
+struct Recording {
+    std::vector<std::function<void()>> launches;
+    void* graph = nullptr;  // hipGraphExec_t once instantiated
+};
+
 void* dali_fe_record_begin(void) {
-    auto* rec = new std::vector<std::function<void()>>();
-    dali::set_recording(rec);
+    auto* rec = new Recording();
+    dali::set_recording(&rec->launches);
     return rec;
 }
 int dali_fe_record_end(void* recording) {
     dali::set_recording(nullptr);
-    return recording ? (int)((std::vector<std::function<void()>>*)recording)->size() : -1;
+    return recording ? (int)((Recording*)recording)->launches.size() : -1;
 }
-int dali_fe_replay(void* recording, int times) {
-    FE_TRY(auto* rec = (std::vector<std::function<void()>>*)recording; if (!rec) throw std::runtime_error("NULL recording");
-           for (int t = 0; t < times; ++t) for (auto& f : *rec) f(); return 0;
+int dali_fe_record_make_graph(void* recording) {
+    FE_TRY(auto* rec = (Recording*)recording; if (!rec) throw std::runtime_error("NULL recording");
+           if (rec->graph) return 0;
+           if (rec->launches.empty()) throw std::runtime_error("recording holds no launches");
+           dali::check_hip(dali_hip_capture_begin(), "graph capture begin");
+           try { for (auto& f : rec->launches) f(); } catch (...) { void* junk = nullptr; dali_hip_capture_end(&junk); if (junk) dali_hip_graph_destroy(junk); throw; }
+           dali::check_hip(dali_hip_capture_end(&rec->graph), "graph capture end");
+           return 0;
            , 1)
 }
-void dali_fe_record_free(void* recording) { delete (std::vector<std::function<void()>>*)recording; }
+int dali_fe_replay(void* recording, int times) {
+    FE_TRY(auto* rec = (Recording*)recording; if (!rec) throw std::runtime_error("NULL recording");
+           if (rec->graph) { for (int t = 0; t < times; ++t) dali::check_hip(dali_hip_graph_launch(rec->graph), "graph launch"); return 0; }
+           for (int t = 0; t < times; ++t) for (auto& f : rec->launches) f(); return 0;
+           , 1)
+}
+void dali_fe_record_free(void* recording) {
+    auto* rec = (Recording*)recording;
+    if (rec && rec->graph) dali_hip_graph_destroy(rec->graph);
+    delete rec;
+}
 
 int dali_fe_generate_only(dali_array_t* roots, int n, int compile) {
     dali::set_dry_compile(compile != 0);

@@ -249,6 +249,7 @@ struct JitStats {
     uint64_t evals = 0;
     uint64_t plans_built = 0;       // planner invocations that had to generate source
     std::string last_kernel_kinds;  // e.g. "row" or "row,all" for the last eval
+    std::string last_kernel_names;  // entry-point names of the generated kernels of the last eval
 };
 JitStats& jit_stats();
 // HIP source of the kernels generated for the last eval (concatenated)

@@ -20,6 +20,7 @@
 //   all   full reduction, two-stage through the workspace, optional scalar epilogue
 // Anything else is split: inner reductions are evaluated into temporaries first.
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <functional>
@@ -57,7 +58,7 @@ void set_recording(std::vector<std::function<void()>>* rec) { g_recording = rec;
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-7";
+const char* const kCodegenVersion = "dali-hip-codegen-8";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -436,6 +437,8 @@ struct RowParams {
     int VEC = 1, TPR = 64, EPT = 0, BT = 256, RPB = 4, NW = 1;
     int waves_per_eu = 0;  // occupancy hint (0 = compiler default)
     bool cached = true;
+    bool nt_loads = false;   // inputs are streamed once: bypass cache allocation
+    bool nt_stores = true;   // outputs are not re-read by this kernel: streaming stores
 };
 
 int env_int(const char* name, int fallback) {
@@ -738,7 +741,7 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
             ss << "  " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[EPT][VEC];\n";
         }
         ss << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n    if (ch < CH) {\n";
-        for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i) + "[e]", "      ", false);
+        for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i) + "[e]", "      ", rp.nt_loads);
         ss << "    }\n  }\n";
         for (size_t id = 0; id < P.nodes.size(); ++id)
             if (P.nodes[id].kept) ss << "  " << ctype(P.nodes[id].dtype) << " t" << id << "[EPT][VEC];\n";
@@ -750,7 +753,7 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
             o << "  for (int ch = tr; ch < CH; ch += TPR) {\n    {\n";
             for (int i : full_leaves) {
                 o << "      " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n";
-                emit_leaf_load(o, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", false);
+                emit_leaf_load(o, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", rp.nt_loads);
             }
         }
     };
@@ -820,7 +823,7 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
             if (rp.VEC > 1) {
                 pre << "        dali_vec<" << t << ", VEC> " << ov << ";\n";
                 if (o.op != OPERATOR_T_EQL) pre << "        " << ov << " = dali_load<" << t << ", VEC>(q" << o.array << " + (long)ch * VEC);\n";
-                post << "        dali_store<" << t << ", VEC>(q" << o.array << " + (long)ch * VEC, " << ov << ");\n";
+                post << "        " << (rp.nt_stores ? "dali_store_nt<" : "dali_store<") << t << ", VEC>(q" << o.array << " + (long)ch * VEC, " << ov << ");\n";
             } else {
                 std::string cs = d.strided ? " * cs" + std::to_string(o.array) : "";
                 pre << "        dali_vec<" << t << ", 1> " << ov << ";\n";
@@ -870,6 +873,13 @@ uint64_t kernel_hash(const std::string& kind, const std::string& sig, const std:
     return Hasher().add(std::string(kCodegenVersion)).add(kind).add(sig).add(params).value();
 }
 
+// entry-point name: shape + hash, so that a profile tells the generated kernels apart
+std::string kernel_name(const std::string& kind, uint64_t hash) {
+    char buf[64];
+    snprintf(buf, sizeof(buf), "dali_%s_%016llx", kind.c_str(), (unsigned long long)hash);
+    return buf;
+}
+
 struct Launch {
     KernelSpec* K;
 };
@@ -880,6 +890,8 @@ void load_and_launch(KernelSpec& K, const std::function<std::string()>& gen, con
     JitStats& st = jit_stats();
     if (!st.last_kernel_kinds.empty()) st.last_kernel_kinds += ",";
     st.last_kernel_kinds += K.kind;
+    if (!st.last_kernel_names.empty()) st.last_kernel_names += ",";
+    st.last_kernel_names += K.name;
     bool need_source = g_dry_run || !loaded_hashes().count(K.hash);
     if (g_dry_run) {
         std::string src = gen();
@@ -1093,7 +1105,13 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
 
     // kernel identity
     std::ostringstream params;
-    params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached << "," << rp.waves_per_eu;
+    // Streaming policy: outputs always leave with non-temporal stores; inputs bypass cache
+    // allocation once the operands are too large to be found in a cache again (64 MiB).
+    static const int nt_l = env_int("DALI_HIP_ROW_NT_LOADS", -1), nt_s = env_int("DALI_HIP_ROW_NT_STORES", -1);
+    rp.nt_loads = nt_l >= 0 ? nt_l != 0 : dom.R * dom.C * (int64_t)max_el >= ((int64_t)64 << 20);
+    rp.nt_stores = nt_s >= 0 ? nt_s != 0 : true;
+    params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached << "," << rp.waves_per_eu << ","
+           << rp.nt_loads << rp.nt_stores;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     std::string sig = signature(P, rpn.outputs);
     uint64_t h = kernel_hash("row", sig, params.str());
@@ -1104,7 +1122,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
         K = std::make_shared<KernelSpec>();
         K->hash = h;
         K->kind = nph == 0 ? "map2d" : "row";
-        K->name = "dali_row_kernel";
+        K->name = kernel_name(K->kind, h);
         fill_plan_arrays(*K, P, shape_ndims);
         K->plan.block_threads = rp.BT;
         K->plan.grid_kind = DALI_HIP_GRID_ROWS;
@@ -1232,7 +1250,7 @@ bool try_flat(const std::vector<DestSpec>& specs) {
         K = std::make_shared<KernelSpec>();
         K->hash = h;
         K->kind = "flat";
-        K->name = "dali_flat_kernel";
+        K->name = kernel_name(K->kind, h);
         fill_plan_arrays(*K, P, shape_ndims);
         K->plan.block_threads = BT;
         K->plan.grid_kind = DALI_HIP_GRID_ELEMS;
@@ -1252,7 +1270,7 @@ bool try_flat(const std::vector<DestSpec>& specs) {
 // partials in block order (so the result does not depend on scheduling), applies
 // the scalar epilogue and resets the ticket counter.
 std::string gen_all_kernel(const Program& P, int red_id, int root_id, int dest_array, OPERATOR_T op, const IvLayout& L, int VEC, int BT,
-                           int UNROLL, int TAIL, const std::string& kname) {
+                           int UNROLL, int TAIL, bool NT, const std::string& kname) {
     const PNode& red = P.nodes[red_id];
     bool is_arg = red.kind == Kind::ARG_ALL_REDUCE;
     std::string t = ctype(P.nodes[red.args[0]].dtype);
@@ -1279,7 +1297,7 @@ std::string gen_all_kernel(const Program& P, int red_id, int root_id, int dest_a
     ss << "  for (long base = (long)blockIdx.x * (BT * UNROLL) + threadIdx.x; base < NCH; base += (long)gridDim.x * (BT * UNROLL)) {\n";
     for (int i : full_leaves) ss << "    " << ctype(P.arrays[i].buf->dtype) << " x" << i << "s[UNROLL][VEC];\n";
     ss << "    _Pragma(\"unroll\") for (int u = 0; u < UNROLL; ++u) {\n      const long ch = base + (long)u * BT;\n      if (ch < NCH) {\n";
-    for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, VEC, "x" + std::to_string(i) + "s[u]", "        ", false);
+    for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, VEC, "x" + std::to_string(i) + "s[u]", "        ", NT);
     ss << "      }\n    }\n";
     ss << "    _Pragma(\"unroll\") for (int u = 0; u < UNROLL; ++u) {\n      const long ch = base + (long)u * BT;\n      if (ch < NCH) {\n";
     for (int i : full_leaves) ss << "        const " << ctype(P.arrays[i].buf->dtype) << "* x" << i << " = x" << i << "s[u];\n";
@@ -1431,7 +1449,8 @@ bool try_all(const DestSpec& spec) {
     outs[0].op = spec.op;
     outs[0].cls = Cls::SCAL;
     std::ostringstream params;
-    params << VEC << "," << BT << "," << red_id << "," << UNROLL << "," << TAIL;
+    const bool NT = n * (int64_t)max_el_all >= ((int64_t)64 << 20);
+    params << VEC << "," << BT << "," << red_id << "," << UNROLL << "," << TAIL << "," << NT;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("all", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& K = specs_cache[h];
@@ -1441,7 +1460,7 @@ bool try_all(const DestSpec& spec) {
         K = std::make_shared<KernelSpec>();
         K->hash = h;
         K->kind = "all";
-        K->name = "dali_all_kernel";
+        K->name = kernel_name(K->kind, h);
         fill_plan_arrays(*K, P, shape_ndims);
         K->plan.block_threads = BT;
         K->plan.grid_kind = DALI_HIP_GRID_ALL;
@@ -1452,7 +1471,7 @@ bool try_all(const DestSpec& spec) {
         K->plan.ws_elsize = 16;
     }
     std::vector<std::vector<int>> shapes = {{(int)n}};
-    load_and_launch(*K, [&]() { return gen_all_kernel(P, red_id, root_id, dest_array, spec.op, L, VEC, BT, UNROLL, TAIL, K->name); }, P, shapes);
+    load_and_launch(*K, [&]() { return gen_all_kernel(P, red_id, root_id, dest_array, spec.op, L, VEC, BT, UNROLL, TAIL, NT, K->name); }, P, shapes);
     return true;
 }
 
@@ -1492,8 +1511,9 @@ bool col_eligible(const Array& a, int64_t K, int64_t X, std::set<const Expr*>& s
     }
 }
 
-std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATOR_T op, const IvLayout& L, int VEC, int UNR, int TAIL, int RG,
+std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATOR_T op, const IvLayout& L, int VEC, int UNR, int TAIL, int RG, bool NT,
                            const std::string& kname) {
+    const std::string ld = NT ? "dali_load_nt<" : "dali_load<";
     const PNode& red = P.nodes[red_id];
     std::string t = ctype(red.dtype);
     std::string dt = ctype(P.arrays[dest_array].buf->dtype);
@@ -1537,7 +1557,7 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     for (int i : full_leaves) {
         std::string ty = ctype(P.arrays[i].buf->dtype);
         ss << "      " << ty << " x" << i << "s[UNR][VEC];\n";
-        ss << "      _Pragma(\"unroll\") for (int u = 0; u < UNR; ++u) { dali_vec<" << ty << ", VEC> tmp = dali_load<" << ty << ", VEC>(q" << i
+        ss << "      _Pragma(\"unroll\") for (int u = 0; u < UNR; ++u) { dali_vec<" << ty << ", VEC> tmp = " << ld << ty << ", VEC>(q" << i
            << " + (x + u * NWAVE) * ld" << i << "); _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) x" << i << "s[u][j] = tmp.v[j]; }\n";
     }
     ss << "      _Pragma(\"unroll\") for (int u = 0; u < UNR; ++u) {\n";
@@ -1552,7 +1572,7 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     for (int i : full_leaves) {
         std::string ty = ctype(P.arrays[i].buf->dtype);
         ss << "      " << ty << " x" << i << "[VEC];\n";
-        ss << "      { dali_vec<" << ty << ", VEC> tmp = dali_load<" << ty << ", VEC>(q" << i << " + x * ld" << i << "); _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) x" << i << "[j] = tmp.v[j]; }\n";
+        ss << "      { dali_vec<" << ty << ", VEC> tmp = " << ld << ty << ", VEC>(q" << i << " + x * ld" << i << "); _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) x" << i << "[j] = tmp.v[j]; }\n";
     }
     ss << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        const int col = 0; (void)col;\n";
     {
@@ -1674,7 +1694,8 @@ bool try_col(const DestSpec& spec) {
     outs[0].op = spec.op;
     outs[0].cls = Cls::ROW;
     std::ostringstream params;
-    params << VEC << "," << UNR << "," << TAIL << "," << RG;
+    const bool NT = K * X * (int64_t)size_of_dtype(re->dtype) >= ((int64_t)64 << 20);
+    params << VEC << "," << UNR << "," << TAIL << "," << RG << "," << NT;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("col", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& Kp = specs_cache[h];
@@ -1684,7 +1705,7 @@ bool try_col(const DestSpec& spec) {
         Kp = std::make_shared<KernelSpec>();
         Kp->hash = h;
         Kp->kind = "col";
-        Kp->name = "dali_col_kernel";
+        Kp->name = kernel_name(Kp->kind, h);
         fill_plan_arrays(*Kp, P, shape_ndims);
         Kp->plan.block_threads = 256;
         Kp->plan.grid_kind = DALI_HIP_GRID_COLS;
@@ -1697,7 +1718,7 @@ bool try_col(const DestSpec& spec) {
         Kp->plan.ws_elsize = size_of_dtype(re->dtype);
     }
     std::vector<std::vector<int>> shapes = {{(int)K, (int)X}};
-    load_and_launch(*Kp, [&]() { return gen_col_kernel(P, red_id, dest_array, spec.op, L, VEC, UNR, TAIL, RG, Kp->name); }, P, shapes);
+    load_and_launch(*Kp, [&]() { return gen_col_kernel(P, red_id, dest_array, spec.op, L, VEC, UNR, TAIL, RG, NT, Kp->name); }, P, shapes);
     return true;
 }
 
@@ -1865,7 +1886,7 @@ bool try_generic(const std::vector<DestSpec>& specs) {
         K = std::make_shared<KernelSpec>();
         K->hash = h;
         K->kind = "generic";
-        K->name = "dali_generic_kernel";
+        K->name = kernel_name(K->kind, h);
         fill_plan_arrays(*K, P, shape_ndims);
         K->plan.block_threads = 256;
         K->plan.grid_kind = DALI_HIP_GRID_ELEMS;
@@ -2245,6 +2266,7 @@ void run_specs(std::vector<DestSpec> specs) {
 void evaluate(const std::vector<Array>& roots) {
     jit_stats().evals++;
     jit_stats().last_kernel_kinds.clear();
+    jit_stats().last_kernel_names.clear();
     g_last_source.clear();
     std::vector<DestSpec> specs;
     std::map<const Expr*, Array> memo;
@@ -2272,6 +2294,7 @@ void evaluate_into(const Array& dest, OPERATOR_T op, const Array& source) {
     DALI_ASSERT(dest.is_buffer(), "assignment destination must be an evaluated buffer");
     jit_stats().evals++;
     jit_stats().last_kernel_kinds.clear();
+    jit_stats().last_kernel_names.clear();
     g_last_source.clear();
     Array src = source;
     if (src.dtype() != dest.dtype()) src = op::astype(src, dest.dtype());

@@ -79,6 +79,7 @@ void* dali_fe_device_ptr(dali_array_t a);
 /* observation (dali/utils/scope.h, dali/array/tests/dot_tests.cpp:17-36) */
 int dali_fe_stats(uint64_t* kernels, uint64_t* gemms, uint64_t* evals, uint64_t* plans);
 const char* dali_fe_last_kernel_kinds(void);
+const char* dali_fe_last_kernel_names(void);
 const char* dali_fe_last_source(void);
 /* Launch recording: between begin and end every kernel and GEMM launch issued by
  * evaluations is also stored (with the buffers it touches kept alive); replay
@@ -86,6 +87,8 @@ const char* dali_fe_last_source(void);
  * rebuilding or re-planning the expressions. */
 void* dali_fe_record_begin(void);
 int dali_fe_record_end(void* recording); /* number of stored launches */
+/* instantiate a HIP graph of the stored launches; later replays launch the graph */
+int dali_fe_record_make_graph(void* recording);
 int dali_fe_replay(void* recording, int times);
 void dali_fe_record_free(void* recording);
 

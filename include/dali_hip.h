@@ -195,6 +195,21 @@ int dali_hip_sgemm_pair(int transB1, int transA1, int transB2, int transA2, int 
                         float alpha, const float* B1, int ldb1, const float* A1, int lda1, const float* B2,
                         int ldb2, const float* A2, int lda2, float beta, float* C, int ldc);
 
+/* ---------------------------------------------------------- HIP graphs */
+
+/*
+ * Capture the launches issued on the library stream between begin and end into
+ * a HIP graph and replay it with one call; for launch-bound steady-state loops
+ * (the reference has no counterpart: it launches every kernel eagerly from
+ * dali/array/jit/jit.cpp:1216-1223). Only kernel launches and device-to-device
+ * copies may be issued while capturing: allocation, host copies and
+ * dali_hip_sync are errors until dali_hip_capture_end.
+ */
+int dali_hip_capture_begin(void);
+int dali_hip_capture_end(void** graph_exec);
+int dali_hip_graph_launch(void* graph_exec);
+int dali_hip_graph_destroy(void* graph_exec);
+
 /* --------------------------------------------------------------- timing */
 
 /* hipEvent wrappers bound to the library stream (the reference times host-side

@@ -154,7 +154,7 @@ def test_softmax_kernel_reads_the_row_once_and_keeps_exp_in_registers(D, rng):
     roots, _ = _cfg_roots(D, rng)["c1_softmax"]
     D.generate_only(roots)
     src = D.last_source()
-    body = src[src.index("dali_row_kernel"):]
+    body = src[src.index("void dali_row_"):]
     assert body.count("dali_load<float, 4>(q1") == 1  # one global read of the input
     assert body.count("functor::exp<float>::Map") == 1  # exp computed once, reused from registers
     assert "dali_group_reduce<reducers::maximum, float, 64>" in body  # wave64 cross-lane reduction
