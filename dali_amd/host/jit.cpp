@@ -1047,7 +1047,11 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
         rp.TPR = (int)std::min<int64_t>(256, pow2ceil((int)std::max<int64_t>(1, CH)));
         rp.BT = 256;
     } else {
-        static const int chunks_target = std::max(1, env_int("DALI_HIP_ROW_CHUNKS", 4));
+        // vectors per thread: latency-bound problems (everything in flight at once, one generation
+        // of waves) want more threads per row, streaming-size problems more work per thread
+        static const int chunks_env = env_int("DALI_HIP_ROW_CHUNKS", 0);
+        const bool big = dom.R * dom.C * (int64_t)max_el >= ((int64_t)64 << 20);
+        const int chunks_target = chunks_env > 0 ? chunks_env : (!big ? 2 : (nph >= 2 ? 8 : 4));
         static const int tpr_cap = std::max(64, env_int("DALI_HIP_ROW_TPR_MAX", 1024));
         int tpr = pow2ceil((int)std::max<int64_t>(1, (CH + chunks_target - 1) / chunks_target));
         tpr = std::min(tpr, tpr_cap);
