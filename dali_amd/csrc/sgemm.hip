@@ -6,8 +6,9 @@
 // by swapping the operands (C^T = B^T A^T), exactly as the reference does when it
 // calls a column-major BLAS (dali/array/gemm/cpu_gemm.cpp:43-68).
 //
-// Work decomposition: a 256-thread workgroup (4 waves, 2x2) owns a BM x BN tile
-// of C; each wave owns (BM/2) x (BN/2), built from 32x32 MFMA accumulators. K is
+// Work decomposition: a workgroup of KW wave sets (4 waves each, 2x2) owns a BM x BN
+// tile of C; each wave owns (BM/2) x (BN/2), built from 32x32 MFMA accumulators, and
+// the KW sets split the k-groups of every slab (summed through LDS at the end). K is
 // walked in slabs of BK (32 or 64).
 //
 // LDS layout.  As[m][k]: rows of BK floats in 16-byte granules, granule g of row m
@@ -55,16 +56,20 @@ struct GemmArgs {
 __device__ __forceinline__ void publish(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float observe(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int DEPTH, bool EDGE>
-__global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int DEPTH, bool EDGE, int KW>
+__global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
+    // KW wave sets share the tile: set kw takes every KW-th k-group of a slab, so each SIMD holds
+    // KW waves that cover each other's LDS and barrier waits; the sets are summed through LDS at the end
+    constexpr int THREADS = 256 * KW;
     constexpr int WTM = BM / 2, WTN = BN / 2;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int A_F4 = BM * BK / 4 / 256;  // float4 fetches per thread for the A slab
-    constexpr int B_F4 = BN * BK / 4 / 256;
+    constexpr int A_F4 = BM * BK / 4 / THREADS;  // float4 fetches per thread for the A slab
+    constexpr int B_F4 = BN * BK / 4 / THREADS;
     constexpr int BPAD = 4;
     // a lone accumulator per wave would serialise dependent MFMAs: split k over two chains
     constexpr int CHAINS = (TM * TN == 1) ? 2 : 1;
-    static_assert(A_F4 >= 1 && B_F4 >= 1, "tile too small for 256 threads");
+    static_assert(A_F4 >= 1 && B_F4 >= 1, "tile too small for the workgroup");
+    static_assert((BK / 8) % KW == 0, "k-groups must divide among the wave sets");
 
     __shared__ __attribute__((aligned(16))) float As[2][BM][BK];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK][BN + BPAD];
@@ -74,7 +79,8 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = (tid >> 6) & 3;
+    const int kw = tid >> 8;  // wave set
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, h = lane >> 5;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
@@ -105,7 +111,7 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
     int a_r[A_F4], a_c[A_F4], b_r[B_F4], b_c[B_F4];
 #pragma unroll
     for (int t = 0; t < A_F4; ++t) {
-        int idx = tid + t * 256;
+        int idx = tid + t * THREADS;
         if (!TA) {
             a_r[t] = m0 + idx / (BK / 4);        // m
             a_c[t] = (idx % (BK / 4)) * 4;       // k offset inside the slab
@@ -116,7 +122,7 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
     }
 #pragma unroll
     for (int t = 0; t < B_F4; ++t) {
-        int idx = tid + t * 256;
+        int idx = tid + t * THREADS;
         if (!TB) {
             b_r[t] = idx / (BN / 4);             // k offset inside the slab
             b_c[t] = n0 + (idx % (BN / 4)) * 4;  // n
@@ -182,7 +188,7 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
         constexpr int st = decltype(S)::value;
 #pragma unroll
         for (int t = 0; t < A_F4; ++t) {
-            int idx = tid + t * 256;
+            int idx = tid + t * THREADS;
             if (!TA) {
                 int m = idx / (BK / 4), gr = idx % (BK / 4);
                 *(float4*)&As[buf][m][swz(gr, m) * 4] = ra[st][t];
@@ -195,7 +201,7 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
         }
 #pragma unroll
         for (int t = 0; t < B_F4; ++t) {
-            int idx = tid + t * 256;
+            int idx = tid + t * THREADS;
             if (!TB) {
                 int k = idx / (BN / 4), n = (idx % (BN / 4)) * 4;
                 *(float4*)&Bs[buf][k][n] = rb[st][t];
@@ -230,11 +236,11 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
     auto compute = [&](int buf) {
         float4 a4[2][TM];
         float b[2][TN][4];
-        load_ops(buf, 0, a4[0], b[0]);
+        load_ops(buf, kw, a4[0], b[0]);
 #pragma unroll
-        for (int t = 0; t < BK / 8; ++t) {
-            const int cur = t & 1;
-            if (t + 1 < BK / 8) load_ops(buf, t + 1, a4[cur ^ 1], b[cur ^ 1]);
+        for (int tt = 0; tt < BK / 8 / KW; ++tt) {
+            const int cur = tt & 1;
+            if (tt + 1 < BK / 8 / KW) load_ops(buf, (tt + 1) * KW + kw, a4[cur ^ 1], b[cur ^ 1]);
             if (TM * TN == 1) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int c = 0; c < 4; ++c)
@@ -282,6 +288,37 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
         });
     }
 
+    if (CHAINS == 2) {
+#pragma unroll
+        for (int ii = 0; ii < TM; ++ii)
+#pragma unroll
+            for (int jj = 0; jj < TN; ++jj) acc[0][ii][jj] += acc[CHAINS - 1][ii][jj];
+    }
+    if (KW > 1) {
+        // wave sets 1.. hand their accumulators to set 0 through LDS (the slab buffers are free now)
+        float* red = &As[0][0][0];
+        static_assert(sizeof(As) >= (size_t)(KW - 1) * BM * BN * sizeof(float), "LDS too small for the wave-set fold");
+        if (kw > 0) {
+#pragma unroll
+            for (int ii = 0; ii < TM; ++ii)
+#pragma unroll
+                for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        red[(size_t)(kw - 1) * BM * BN + ((wave * TM + ii) * TN + jj) * 1024 + v * 64 + lane] = acc[0][ii][jj][v];
+        }
+        __syncthreads();
+        if (kw > 0) return;
+#pragma unroll
+        for (int s2 = 1; s2 < KW; ++s2)
+#pragma unroll
+            for (int ii = 0; ii < TM; ++ii)
+#pragma unroll
+                for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        acc[0][ii][jj][v] += red[(size_t)(s2 - 1) * BM * BN + ((wave * TM + ii) * TN + jj) * 1024 + v * 64 + lane];
+    }
     // epilogue: lane holds column l32 and rows 8*(v/4) + 4*h + v%4 of each 32x32 tile
     const float alpha = g.alpha, beta = g.beta;
     const bool split = gridDim.z > 1;
@@ -300,9 +337,7 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     int lm = wm * WTM + ii * 32 + 8 * (v / 4) + 4 * h + (v % 4), ln = wn * WTN + jj * 32 + l32;
-                    float sum = acc[0][ii][jj][v];
-                    if (CHAINS == 2) sum += acc[CHAINS - 1][ii][jj][v];
-                    publish(mine + lm * BN + ln, sum);
+                    publish(mine + lm * BN + ln, acc[0][ii][jj][v]);
                 }
         __builtin_amdgcn_s_waitcnt(0);
         __shared__ int is_last;
@@ -332,7 +367,6 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
                         for (unsigned z = 0; z < gridDim.z; ++z) sum += observe(part + (size_t)z * (BM * BN) + lm * BN + ln);
                     } else {
                         sum = acc[0][ii][jj][v];
-                        if (CHAINS == 2) sum += acc[CHAINS - 1][ii][jj][v];
                     }
                     float r = alpha * sum;
                     if (beta != 0.f) r += beta * *c;
@@ -343,8 +377,9 @@ __global__ __launch_bounds__(256) void sgemm_kernel(GemmArgs g) {
     if (split && tid == 0) __hip_atomic_store(g.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int BM, int BN, int BK, int DEPTH>
+template <int BM, int BN, int BK, int DEPTH, int KW = 1>
 static int launch_tile(GemmArgs g, bool ta, bool tb, bool vec, int split_k) {
+    if (KW > 1) split_k = 1;  // the wave-set fold and the cross-workgroup fold are alternatives
     // interior-only problems (every tile and slab full, 16-byte aligned rows) take the unchecked kernel
     bool edge = !vec || g.M % BM != 0 || g.N % BN != 0;
     for (int s = 0; s < g.nseg; ++s) edge = edge || g.seg[s].K % BK != 0;
@@ -357,16 +392,16 @@ static int launch_tile(GemmArgs g, bool ta, bool tb, bool vec, int split_k) {
     grid.z = split_k;
     g.counters = (unsigned int*)workspace();
     g.partials = (float*)(workspace() + kWorkspaceCounterBytes);
-    dim3 block(256);
+    dim3 block(256 * KW);
     hipStream_t st = stream();
     static const int pad_env = getenv("DALI_HIP_GEMM_PAD_LDS") ? atoi(getenv("DALI_HIP_GEMM_PAD_LDS")) : 0;
     const unsigned pad_lds = (unsigned)pad_env;
 #define DALI_GEMM_CASE(TA_, TB_, V_)                                                                        \
     if (ta == TA_ && tb == TB_ && vec == V_) {                                                              \
         if (edge)                                                                                           \
-            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, TA_, TB_, V_, DEPTH, true>), grid, block, pad_lds, st, g);  \
+            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, TA_, TB_, V_, DEPTH, true, KW>), grid, block, pad_lds, st, g);  \
         else if (V_)                                                                                        \
-            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, TA_, TB_, true, DEPTH, false>), grid, block, pad_lds, st, g); \
+            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, TA_, TB_, true, DEPTH, false, KW>), grid, block, pad_lds, st, g); \
     }
     DALI_GEMM_CASE(false, false, true)
     DALI_GEMM_CASE(false, false, false)
@@ -433,9 +468,14 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
     static const int split_env = getenv("DALI_HIP_GEMM_SPLITK") ? atoi(getenv("DALI_HIP_GEMM_SPLITK")) : 0;
     int split_k = split_env > 0 ? split_env : 1;
     (void)tiles64;
+    if (variant == 3) return launch_tile<64, 64, 64, 2, 2>(g, ta, tb, vec, split_k);
+    if (variant == 6) return launch_tile<64, 64, 128, 2, 2>(g, ta, tb, vec, split_k);
+    if (variant == 4) return launch_tile<64, 64, 64, 3, 2>(g, ta, tb, vec, split_k);
     if (variant == 1) return launch_tile<64, 64, 32, 3>(g, ta, tb, vec, split_k);
     if (variant == 2) return launch_tile<64, 64, 64, 3>(g, ta, tb, vec, split_k);
-    return launch_tile<64, 64, 64, 2>(g, ta, tb, vec, split_k);
+    if (variant == 8) return launch_tile<64, 64, 64, 2>(g, ta, tb, vec, split_k);
+    // default for small grids: two wave sets per 64x64 tile (two waves per SIMD)
+    return launch_tile<64, 64, 64, 2, 2>(g, ta, tb, vec, split_k);
 }
 
 }  // namespace dali_hip

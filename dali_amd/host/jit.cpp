@@ -1688,7 +1688,8 @@ bool try_col(const DestSpec& spec) {
     for (const ArrayArg& a : P.arrays)
         if (!a.is_dest && a.cls == Cls::FULL && (a.buf->offset % 4 != 0 || a.col_stride % 4 != 0)) vec = false;
     int VEC = vec ? 4 : 1;
-    const int UNR = 8, TAIL = 16;
+    static const int unr_env = env_int("DALI_HIP_COL_UNR", 8), rows_env = env_int("DALI_HIP_COL_ROWS", 256);
+    const int UNR = unr_env, TAIL = 16;
     // widest row piece the kept extent can fill: 1 group of 256 threads for wide matrices, up to 4 groups of 64
     int RG = 1;
     while (RG < 4 && (int64_t)(256 / RG) * VEC > K) RG *= 2;
@@ -1717,7 +1718,7 @@ bool try_col(const DestSpec& spec) {
         Kp->plan.work_count = 1;
         Kp->plan.work_per_block = (256 / RG) * VEC;
         Kp->plan.work2_begin = L.shape_pos[0] + 1;
-        Kp->plan.work2_per_block = 256;  // reduced rows per y-block
+        Kp->plan.work2_per_block = rows_env;  // reduced rows per y-block
         Kp->plan.max_blocks2 = 256;
         Kp->plan.ws_elsize = size_of_dtype(re->dtype);
     }
