@@ -516,7 +516,7 @@ int dali_hip_launch(uint64_t hash, void** array_data, const int* offsets, const 
     if (work <= 0) return DALI_HIP_OK;  // empty arrays: nothing to do
     int64_t per = P.work_per_block > 0 ? P.work_per_block : 1;
     int64_t gx = (work + per - 1) / per;
-    if (P.max_blocks > 0 && gx > P.max_blocks) gx = P.max_blocks;
+    if (P.grid_kind != DALI_HIP_GRID_COLS && P.max_blocks > 0 && gx > P.max_blocks) gx = P.max_blocks;
     int64_t gy = 1;
     if (P.grid_kind == DALI_HIP_GRID_COLS) {
         if (P.work2_begin < 0 || P.work2_begin >= m->n_iv) return fail("dali_hip_launch: plan reduced extent out of range");
@@ -525,6 +525,8 @@ int dali_hip_launch(uint64_t hash, void** array_data, const int* offsets, const 
         int64_t per2 = P.work2_per_block > 0 ? P.work2_per_block : 1;
         gy = (red + per2 - 1) / per2;
         if (P.max_blocks2 > 0 && gy > P.max_blocks2) gy = P.max_blocks2;
+        // every column strip needs its block, so the bound on the whole grid is met by the y split alone
+        if (P.max_blocks > 0 && gx * gy > P.max_blocks) gy = P.max_blocks / gx > 0 ? P.max_blocks / gx : 1;
         // rows of partials are padded to whole column strips
         int64_t cap = (int64_t)kWorkspacePartialBytes / (gx * per * (int64_t)(P.ws_elsize > 0 ? P.ws_elsize : 4));
         if (cap < 1) cap = 1;

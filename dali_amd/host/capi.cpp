@@ -15,7 +15,7 @@ static thread_local std::string g_kinds;
 
 namespace dali {
 void set_dry_compile(bool on);
-void set_recording(std::vector<std::function<void()>>* rec);
+void set_recording(std::vector<std::function<void()>>* rec, std::vector<std::shared_ptr<memory::SynchronizedMemory>>* written);
 }
 
 #define FE_TRY(body, failure)               \
@@ -153,16 +153,21 @@ const char* dali_fe_last_source(void) { return dali::last_generated_source().c_s
 
 struct Recording {
     std::vector<std::function<void()>> launches;
+    std::vector<std::shared_ptr<dali::memory::SynchronizedMemory>> written;
     void* graph = nullptr;  // hipGraphExec_t once instantiated
+    // the replayed kernels write device memory behind the front-end's back: host copies become stale
+    void invalidate_host_copies() {
+        for (auto& m : written) m->mutable_data(dali::memory::DEVICE_T_GPU);
+    }
 };
 
 void* dali_fe_record_begin(void) {
     auto* rec = new Recording();
-    dali::set_recording(&rec->launches);
+    dali::set_recording(&rec->launches, &rec->written);
     return rec;
 }
 int dali_fe_record_end(void* recording) {
-    dali::set_recording(nullptr);
+    dali::set_recording(nullptr, nullptr);
     return recording ? (int)((Recording*)recording)->launches.size() : -1;
 }
 int dali_fe_record_make_graph(void* recording) {
@@ -177,6 +182,7 @@ int dali_fe_record_make_graph(void* recording) {
 }
 int dali_fe_replay(void* recording, int times) {
     FE_TRY(auto* rec = (Recording*)recording; if (!rec) throw std::runtime_error("NULL recording");
+           if (times > 0) rec->invalidate_host_copies();
            if (rec->graph) { for (int t = 0; t < times; ++t) dali::check_hip(dali_hip_graph_launch(rec->graph), "graph launch"); return 0; }
            for (int t = 0; t < times; ++t) for (auto& f : rec->launches) f(); return 0;
            , 1)

@@ -53,12 +53,24 @@ const std::string& last_generated_source() { return g_last_source; }
 // touches) so that a steady-state loop can re-issue exactly the same device work
 // without rebuilding and re-planning the expression.
 static std::vector<std::function<void()>>* g_recording = nullptr;
-void set_recording(std::vector<std::function<void()>>* rec) { g_recording = rec; }
+// memories the recorded launches write: a replay bypasses the access-mode calls of a
+// normal evaluation, so their host copies must be declared stale by the replayer
+static std::vector<std::shared_ptr<memory::SynchronizedMemory>>* g_recording_written = nullptr;
+void set_recording(std::vector<std::function<void()>>* rec, std::vector<std::shared_ptr<memory::SynchronizedMemory>>* written) {
+    g_recording = rec;
+    g_recording_written = written;
+}
+static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory>& m) {
+    if (!g_recording_written) return;
+    for (auto& w : *g_recording_written)
+        if (w == m) return;
+    g_recording_written->push_back(m);
+}
 
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-8";
+const char* const kCodegenVersion = "dali-hip-codegen-9";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -940,6 +952,8 @@ void load_and_launch(KernelSpec& K, const std::function<std::string()>& gen, con
               "kernel launch");
     st.kernels_launched++;
     if (g_recording) {
+        for (const ArrayArg& a : P.arrays)
+            if (a.is_dest) note_recorded_write(a.buf->memory);
         uint64_t hash = K.hash;
         auto arrays = std::make_shared<std::vector<ArrayArg>>(P.arrays);
         auto scal = std::make_shared<std::vector<ScalarArg>>(P.scalars);
@@ -1516,7 +1530,7 @@ bool col_eligible(const Array& a, int64_t K, int64_t X, std::set<const Expr*>& s
 }
 
 std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATOR_T op, const IvLayout& L, int VEC, int UNR, int TAIL, int RG, bool NT,
-                           const std::string& kname) {
+                           int IL, const std::string& kname) {
     const std::string ld = NT ? "dali_load_nt<" : "dali_load<";
     const PNode& red = P.nodes[red_id];
     std::string t = ctype(red.dtype);
@@ -1552,17 +1566,35 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
         if (!P.arrays[i].is_dest && P.arrays[i].cls == Cls::FULL) full_leaves.push_back((int)i);
     ss << "  " << t << " acc[VEC];\n  _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = " << red.name << "::init<" << t << ">();\n";
     // contiguous share of the reduced axis for this y-block, interleaved over its waves
-    ss << "  const long per_y = (X + gridDim.y - 1) / gridDim.y;\n";
-    ss << "  const long x_begin = (long)blockIdx.y * per_y, x_end = x_begin + per_y < X ? x_begin + per_y : X;\n";
-    ss << "  if (k_ok) {\n    long x = x_begin + wave;\n";
+    // Which memory rows a y-block reads. 0: one contiguous share of the reduced axis. 1: single rows dealt
+    // round-robin. 2: chunks of UNR*NWAVE consecutive rows dealt round-robin, so that the grid as a whole reads
+    // one contiguous band of memory at any moment while the loads of one lane stay within a few pages.
+    if (IL == 2) {
+        ss << "  constexpr long XS = NWAVE;\n";
+        ss << "  const long n_chunks = X / (UNR * NWAVE);\n";
+        ss << "  const long x_end = X;\n";
+        ss << "  if (k_ok) {\n";
+    } else if (IL == 1) {
+        ss << "  const long XS = (long)gridDim.y * NWAVE;\n";
+        ss << "  const long x_end = X;\n";
+        ss << "  if (k_ok) {\n    long x = (long)blockIdx.y * NWAVE + wave;\n";
+    } else {
+        ss << "  constexpr long XS = NWAVE;\n";
+        ss << "  const long per_y = (X + gridDim.y - 1) / gridDim.y;\n";
+        ss << "  const long x_begin = (long)blockIdx.y * per_y, x_end = x_begin + per_y < X ? x_begin + per_y : X;\n";
+        ss << "  if (k_ok) {\n    long x = x_begin + wave;\n";
+    }
     std::vector<int> first_body(P.nodes.size(), -1);
     // main loop: UNR independent row fetches in flight per lane
-    ss << "    for (; x + (UNR - 1) * NWAVE < x_end; x += UNR * NWAVE) {\n";
+    if (IL == 2)
+        ss << "    for (long ch = blockIdx.y; ch < n_chunks; ch += gridDim.y) {\n      const long x = ch * (UNR * NWAVE) + wave;\n";
+    else
+        ss << "    for (; x + (UNR - 1) * XS < x_end; x += UNR * XS) {\n";
     for (int i : full_leaves) {
         std::string ty = ctype(P.arrays[i].buf->dtype);
         ss << "      " << ty << " x" << i << "s[UNR][VEC];\n";
         ss << "      _Pragma(\"unroll\") for (int u = 0; u < UNR; ++u) { dali_vec<" << ty << ", VEC> tmp = " << ld << ty << ", VEC>(q" << i
-           << " + (x + u * NWAVE) * ld" << i << "); _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) x" << i << "s[u][j] = tmp.v[j]; }\n";
+           << " + (x + u * XS) * ld" << i << "); _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) x" << i << "s[u][j] = tmp.v[j]; }\n";
     }
     ss << "      _Pragma(\"unroll\") for (int u = 0; u < UNR; ++u) {\n";
     for (int i : full_leaves) ss << "        const " << ctype(P.arrays[i].buf->dtype) << "* x" << i << " = x" << i << "s[u];\n";
@@ -1572,7 +1604,10 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
         std::string v = be.value(red.args[0]);
         ss << be.stmts.str() << "          acc[j] = " << red.name << "::step<" << t << ">(acc[j], " << v << ");\n        }\n      }\n";
     }
-    ss << "    }\n    for (; x < x_end; x += NWAVE) {\n";
+    if (IL == 2)
+        ss << "    }\n    for (long x = n_chunks * (UNR * NWAVE) + (long)blockIdx.y * NWAVE + wave; x < x_end; x += (long)gridDim.y * NWAVE) {\n";
+    else
+        ss << "    }\n    for (; x < x_end; x += XS) {\n";
     for (int i : full_leaves) {
         std::string ty = ctype(P.arrays[i].buf->dtype);
         ss << "      " << ty << " x" << i << "[VEC];\n";
@@ -1607,16 +1642,22 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
           "    __builtin_amdgcn_s_waitcnt(0);\n  }\n  __syncthreads();\n";
     ss << "  if (threadIdx.x == 0) is_last = dali_take_ticket(&counters[blockIdx.x]) == gridDim.y - 1;\n  __syncthreads();\n";
     ss << "  if (!is_last) return;\n";
-    ss << "  if (wave == 0) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = " << red.name << "::init<" << t << ">();\n";
-    ss << "    // partial rows are folded in y order; TAIL of them are in flight at a time\n";
-    ss << "    for (unsigned int y0 = 0; y0 < gridDim.y; y0 += TAIL) {\n      dali_vec<" << t << ", VEC> pv[TAIL];\n";
-    ss << "      _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) if (y0 + k < gridDim.y) {\n"
-          "        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) pv[k].v[j] = dali_observe(partials + (long)(y0 + k) * KP + pcol + j);\n      }\n";
-    ss << "      _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) if (y0 + k < gridDim.y) {\n        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = "
-       << red.name << "::step<" << t << ">(acc[j], pv[k].v[j]);\n      }\n    }\n";
-    ss << "    if (k_ok) {\n";
-    emit_store("      ");
-    ss << "    }\n  }\n  if (threadIdx.x == 0) dali_publish(&counters[blockIdx.x], 0u);\n}\n";
+    // every row group of the last block folds a contiguous share of the partial rows in y order (TAIL of them in
+    // flight at a time); the groups are then joined in group order through LDS
+    ss << "  _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = " << red.name << "::init<" << t << ">();\n";
+    ss << "  const unsigned int y_per = (gridDim.y + NWAVE - 1) / NWAVE;\n";
+    ss << "  const unsigned int y_begin = wave * y_per, y_end = y_begin + y_per < gridDim.y ? y_begin + y_per : gridDim.y;\n";
+    ss << "  for (unsigned int y0 = y_begin; y0 < y_end; y0 += TAIL) {\n    dali_vec<" << t << ", VEC> pv[TAIL];\n";
+    ss << "    _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) if (y0 + k < y_end) {\n"
+          "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) pv[k].v[j] = dali_observe(partials + (long)(y0 + k) * KP + pcol + j);\n    }\n";
+    ss << "    _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) if (y0 + k < y_end) {\n      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = "
+       << red.name << "::step<" << t << ">(acc[j], pv[k].v[j]);\n    }\n  }\n";
+    ss << "  if (NWAVE > 1) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) sm[wave][lane * VEC + j] = acc[j];\n    __syncthreads();\n"
+       << "    if (wave == 0) {\n      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        " << t << " r = sm[0][lane * VEC + j];\n"
+       << "        _Pragma(\"unroll\") for (int w = 1; w < NWAVE; ++w) r = " << red.name << "::step<" << t << ">(r, sm[w][lane * VEC + j]);\n        acc[j] = r;\n      }\n    }\n  }\n";
+    ss << "  if (wave == 0 && k_ok) {\n";
+    emit_store("    ");
+    ss << "  }\n  if (threadIdx.x == 0) dali_publish(&counters[blockIdx.x], 0u);\n}\n";
     return ss.str();
 }
 
@@ -1688,11 +1729,17 @@ bool try_col(const DestSpec& spec) {
     for (const ArrayArg& a : P.arrays)
         if (!a.is_dest && a.cls == Cls::FULL && (a.buf->offset % 4 != 0 || a.col_stride % 4 != 0)) vec = false;
     int VEC = vec ? 4 : 1;
-    static const int unr_env = env_int("DALI_HIP_COL_UNR", 8), rows_env = env_int("DALI_HIP_COL_ROWS", 256);
-    const int UNR = unr_env, TAIL = 16;
-    // widest row piece the kept extent can fill: 1 group of 256 threads for wide matrices, up to 4 groups of 64
-    int RG = 1;
-    while (RG < 4 && (int64_t)(256 / RG) * VEC > K) RG *= 2;
+    static const int IL = env_int("DALI_HIP_COL_INTERLEAVE", 2);
+    static const int rg_env = env_int("DALI_HIP_COL_RG", 0), tail_env = env_int("DALI_HIP_COL_TAIL", 16);
+    static const int unr_env = env_int("DALI_HIP_COL_UNR", 8), rows_env = env_int("DALI_HIP_COL_ROWS", 0);
+    static const int blocks_env = env_int("DALI_HIP_COL_BLOCKS", 256);
+    const int UNR = unr_env;
+    // four row groups of one wave each: a wave reads 1 KiB pieces of memory rows, a block owns a 256-column strip.
+    // Narrow strips and few y-blocks measured best (8192x8192: 53 us with 1024-column strips x 32 y-blocks,
+    // 41 us with 256-column strips x 8 y-blocks).
+    int RG = 4;
+    if (rg_env > 0) RG = rg_env;
+    const int TAIL = tail_env;
     std::vector<Output> outs(1);
     outs[0].root = red_id;
     outs[0].array = dest_array;
@@ -1700,7 +1747,8 @@ bool try_col(const DestSpec& spec) {
     outs[0].cls = Cls::ROW;
     std::ostringstream params;
     const bool NT = K * X * (int64_t)size_of_dtype(re->dtype) >= ((int64_t)64 << 20);
-    params << VEC << "," << UNR << "," << TAIL << "," << RG << "," << NT;
+    static const int maxy_env = env_int("DALI_HIP_COL_MAXY", 256);
+    params << VEC << "," << UNR << "," << TAIL << "," << RG << "," << NT << "," << IL;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("col", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& Kp = specs_cache[h];
@@ -1718,12 +1766,13 @@ bool try_col(const DestSpec& spec) {
         Kp->plan.work_count = 1;
         Kp->plan.work_per_block = (256 / RG) * VEC;
         Kp->plan.work2_begin = L.shape_pos[0] + 1;
-        Kp->plan.work2_per_block = rows_env;  // reduced rows per y-block
-        Kp->plan.max_blocks2 = 256;
+        Kp->plan.work2_per_block = rows_env > 0 ? rows_env : UNR * RG;  // fewest reduced rows per y-block
+        Kp->plan.max_blocks2 = maxy_env;
+        Kp->plan.max_blocks = blocks_env;  // one block per CU: the y split fills what the column strips leave
         Kp->plan.ws_elsize = size_of_dtype(re->dtype);
     }
     std::vector<std::vector<int>> shapes = {{(int)K, (int)X}};
-    load_and_launch(*Kp, [&]() { return gen_col_kernel(P, red_id, dest_array, spec.op, L, VEC, UNR, TAIL, RG, NT, Kp->name); }, P, shapes);
+    load_and_launch(*Kp, [&]() { return gen_col_kernel(P, red_id, dest_array, spec.op, L, VEC, UNR, TAIL, RG, NT, IL, Kp->name); }, P, shapes);
     return true;
 }
 
@@ -1972,6 +2021,7 @@ void run_gemm(const Array& dst, const Expr* mm, const Expr* mm2, float beta) {
         float* dp = (float*)dst.device_ptr(mode);
         check_hip(dali_hip_sgemm(g.rt, g.lt, m, n, k, 1.0f, rp, g.rld, lp, g.lld, beta, dp, ldc), "sgemm");
         if (g_recording) {
+            note_recorded_write(dst.expression()->memory);
             GemmOperands keep = g;
             Array dkeep = dst;
             g_recording->push_back([=]() {
@@ -1991,6 +2041,7 @@ void run_gemm(const Array& dst, const Expr* mm, const Expr* mm2, float beta) {
         check_hip(dali_hip_sgemm_pair(g.rt, g.lt, h.rt, h.lt, m, n, k, k2, 1.0f, rp, g.rld, lp, g.lld, rp2, h.rld, lp2, h.lld, beta, dp, ldc),
                   "sgemm_pair");
         if (g_recording) {
+            note_recorded_write(dst.expression()->memory);
             Array dkeep = dst;
             g_recording->push_back([=]() {
                 (void)dkeep;

@@ -125,7 +125,7 @@ typedef struct dali_hip_launch_plan {
     int32_t work_begin;           /* first iv index of the extent product (x dimension) */
     int32_t work_count;           /* number of iv entries multiplied (0 => 1) */
     int32_t work_per_block;       /* elements / rows / columns covered by one block in x */
-    int32_t max_blocks;           /* upper bound of grid.x (0 => unbounded) */
+    int32_t max_blocks;           /* upper bound of grid.x (0 => unbounded); GRID_COLS: of grid.x * grid.y, met by shrinking grid.y */
     int32_t work2_begin;          /* GRID_COLS: iv index of the reduced extent */
     int32_t work2_per_block;      /* GRID_COLS: reduced rows per y-block */
     int32_t max_blocks2;          /* GRID_COLS: upper bound of grid.y */

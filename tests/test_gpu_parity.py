@@ -488,3 +488,59 @@ def test_recording_replays_the_same_device_work(gpu, D, rng):
     first = s.numpy()
     rec.replay(3)
     assert np.array_equal(s.numpy(), first)
+
+
+def test_graph_replays_match_eager_on_every_replay(gpu, D, O, rng):
+    # cross-entropy: a row kernel plus a two-stage `all` kernel (tickets and partials in the persistent
+    # workspace, which must come back to zero after each replay), then a column reduction
+    n, v = 96, 700
+    logits = arr(D, rng.randn(n, v).astype(np.float32))
+    targets = arr(D, rng.randint(0, v, n).astype(np.int32))
+    with D.Recording() as rec:
+        mean_loss, row_loss, grad = D.op.softmax_cross_entropy(logits, targets)
+        colsum = D.op.sum(grad, [0])
+        colsum.eval()
+    assert rec.launches >= 3
+    rec.make_graph()
+    for it in range(4):
+        fresh = rng.randn(n, v).astype(np.float32)
+        logits.assign(arr(D, fresh))  # eager work between replays changes the graph's input in place
+        rec.replay(1)
+        got = [a.numpy() for a in (mean_loss, row_loss, grad, colsum)]
+        e_mean, e_row, e_grad = D.op.softmax_cross_entropy(arr(D, fresh), targets)
+        e_col = D.op.sum(e_grad, [0])
+        for g, e in zip(got, (e_mean, e_row, e_grad, e_col)):
+            assert np.array_equal(g, e.numpy()), "replay %d differs from the eager evaluation" % it
+        o_loss = O.softmax_cross_entropy(fresh, targets.numpy())[1]
+        close(got[1], o_loss, rtol=1e-5 + v * 2.0 ** -24, atol=1e-6)
+
+
+def test_cabi_graph_capture_of_gemm(gpu, D, rng):
+    # dali_hip_capture_begin / _end / _graph_launch around dali_hip_sgemm, with C-ABI calls only
+    import ctypes as C
+    from dali_amd import _native
+    hip = _native.hip
+    m, n, k = 64, 96, 128
+    b = rng.randn(k, n).astype(np.float32)
+    out = np.empty((m, n), np.float32)
+    ptrs = [C.c_void_p() for _ in range(3)]
+    for p, nbytes in zip(ptrs, (m * k * 4, k * n * 4, m * n * 4)):
+        assert hip.dali_hip_malloc(C.byref(p), nbytes) == 0
+    pa, pb, pc = ptrs
+    assert hip.dali_hip_memcpy_h2d(pb, b.ctypes.data_as(C.c_void_p), b.nbytes) == 0
+    assert hip.dali_hip_capture_begin() == 0
+    # row-major C = A·B as the column-major product Cᵀ = Bᵀ·Aᵀ (the reference's operand swap, cublas_gemm.cu:153-166)
+    rc = hip.dali_hip_sgemm(0, 0, n, m, k, C.c_float(1.0), pb, n, pa, k, C.c_float(0.0), pc, n)
+    graph = C.c_void_p()
+    assert hip.dali_hip_capture_end(C.byref(graph)) == 0 and rc == 0 and graph.value
+    try:
+        for it in range(3):
+            a = rng.randn(m, k).astype(np.float32)
+            assert hip.dali_hip_memcpy_h2d(pa, a.ctypes.data_as(C.c_void_p), a.nbytes) == 0
+            assert hip.dali_hip_graph_launch(graph) == 0
+            assert hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), pc, out.nbytes) == 0
+            close(out, a.astype(np.float64) @ b, rtol=1e-4, atol=1e-4)
+    finally:
+        assert hip.dali_hip_graph_destroy(graph) == 0
+        for p in ptrs:
+            assert hip.dali_hip_free(p) == 0
