@@ -33,6 +33,18 @@
 namespace dali_hip {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// 16-byte accesses through the native vector type (an aggregate float4 copy is a memcpy to the
+// optimiser, which keeps the register stages from being promoted out of private memory)
+__device__ __forceinline__ float4 ld16(const void* p) {
+    const floatx4 v = *(const floatx4*)p;
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void st16(void* p, const float4& v) {
+    floatx4 w = {v.x, v.y, v.z, v.w};
+    *(floatx4*)p = w;
+}
 
 struct GemmSeg {
     const float* A;
@@ -56,7 +68,7 @@ struct GemmArgs {
 __device__ __forceinline__ void publish(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float observe(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int DEPTH, bool EDGE, int KW>
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int DEPTH, bool EDGE, int KW, bool MIDB>
 __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     // KW wave sets share the tile: set kw takes every KW-th k-group of a slab, so each SIMD holds
     // KW waves that cover each other's LDS and barrier waits; the sets are summed through LDS at the end
@@ -65,17 +77,26 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr int A_F4 = BM * BK / 4 / THREADS;  // float4 fetches per thread for the A slab
     constexpr int B_F4 = BN * BK / 4 / THREADS;
-    constexpr int BPAD = 4;
+    constexpr int BPAD = 8;  // rows 4 apart (the two half-waves of a B operand read) land 32 banks apart
     // a lone accumulator per wave would serialise dependent MFMAs: split k over two chains
     constexpr int CHAINS = (TM * TN == 1) ? 2 : 1;
     static_assert(A_F4 >= 1 && B_F4 >= 1, "tile too small for the workgroup");
     static_assert((BK / 8) % KW == 0, "k-groups must divide among the wave sets");
 
-    __shared__ __attribute__((aligned(16))) float As[2][BM][BK];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BK][BN + BPAD];
+    // The small-tile interior kernel runs a software pipeline with the workgroup barrier in the middle of a slab
+    // (see its loop below), which needs a third slab buffer.
+    constexpr int G = BK / 8 / KW;  // k-groups of a slab per wave set
+    constexpr bool PIPE = !EDGE && TM * TN == 1 && DEPTH == 2 && G >= 2 && G % 2 == 0;
+    constexpr int NBUF = PIPE && MIDB ? 4 : 2;
+    // one LDS block: the A slab buffers, the B slab buffers; reused for the wave-set fold at the end
+    constexpr int AS_FLOATS = NBUF * BM * BK, BS_FLOATS = NBUF * BK * (BN + BPAD), RED_FLOATS = (KW - 1) * BM * BN;
+    constexpr int LDS_FLOATS = AS_FLOATS + BS_FLOATS > RED_FLOATS ? AS_FLOATS + BS_FLOATS : RED_FLOATS;
+    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
+    float (*As)[BM][BK] = reinterpret_cast<float (*)[BM][BK]>(lds);
+    float (*Bs)[BK][BN + BPAD] = reinterpret_cast<float (*)[BK][BN + BPAD]>(lds + AS_FLOATS);
 
     // slot of 16-byte granule `gr` in row m: the low three bits are permuted per row
-    auto swz = [](int gr, int m) { return (gr & ~7) | ((gr ^ m) & 7); };
+    auto swz = [](int gr, int m) __attribute__((always_inline)) { return (gr & ~7) | ((gr ^ m) & 7); };
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -135,14 +156,14 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     // One 4-float granule at row r, columns c..c+3 of a row-major array with `rows` x `cols`
     // valid entries. Interior tiles (EDGE == false) load unconditionally; edge tiles clamp the
     // address and zero what lies outside, without branching.
-    auto load4 = [&](const float* base, int ld, int r, int c, int rows, int cols) -> float4 {
-        if (!EDGE) return *(const float4*)(base + (size_t)r * ld + c);
+    auto load4 = [&](const float* base, int ld, int r, int c, int rows, int cols) __attribute__((always_inline)) -> float4 {
+        if (!EDGE) return ld16(base + (size_t)r * ld + c);
         const bool rv = r < rows;
         const size_t ro = (size_t)(rv ? r : 0) * ld;
         if (VEC) {
             // cols is a multiple of 4 here or the granule is cut: handle both with per-element masks
             const bool full = rv && c + 3 < cols;
-            const float4 v = *(const float4*)(base + ro + (full ? c : 0));
+            const float4 v = ld16(base + ro + (full ? c : 0));
             if (full) return v;
         }
         float4 v;
@@ -158,7 +179,7 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     };
 
     // fetch slab `i` (index into the flat slab list) into register stage S
-    auto fetch = [&](auto S, int i) {
+    auto fetch = [&](auto S, int i) __attribute__((always_inline)) {
         constexpr int st = decltype(S)::value;
         const bool first = i < slabs0;
         const float* sa = first ? g.seg[0].A : g.seg[1].A;
@@ -183,15 +204,15 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
         }
     };
 
-    // register stage S -> LDS buffer `buf`
-    auto stage = [&](auto S, int buf) {
+    // register stage S -> LDS buffer `buf`, the A half and the B half
+    auto stageA = [&](auto S, int buf) __attribute__((always_inline)) {
         constexpr int st = decltype(S)::value;
 #pragma unroll
         for (int t = 0; t < A_F4; ++t) {
             int idx = tid + t * THREADS;
             if (!TA) {
                 int m = idx / (BK / 4), gr = idx % (BK / 4);
-                *(float4*)&As[buf][m][swz(gr, m) * 4] = ra[st][t];
+                st16(&As[buf][m][swz(gr, m) * 4], ra[st][t]);
             } else {
                 int k = idx / (BM / 4), m = (idx % (BM / 4)) * 4;
                 const float vals[4] = {ra[st][t].x, ra[st][t].y, ra[st][t].z, ra[st][t].w};
@@ -199,12 +220,15 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
                 for (int c = 0; c < 4; ++c) As[buf][m + c][(swz(k >> 2, m + c) << 2) | (k & 3)] = vals[c];
             }
         }
+    };
+    auto stageB = [&](auto S, int buf) __attribute__((always_inline)) {
+        constexpr int st = decltype(S)::value;
 #pragma unroll
         for (int t = 0; t < B_F4; ++t) {
             int idx = tid + t * THREADS;
             if (!TB) {
                 int k = idx / (BN / 4), n = (idx % (BN / 4)) * 4;
-                *(float4*)&Bs[buf][k][n] = rb[st][t];
+                st16(&Bs[buf][k][n], rb[st][t]);
             } else {
                 int n = idx / (BK / 4), k = (idx % (BK / 4)) * 4;
                 Bs[buf][k + 0][n] = rb[st][t].x;
@@ -214,14 +238,18 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
             }
         }
     };
+    auto stage = [&](auto S, int buf) __attribute__((always_inline)) {
+        stageA(S, buf);
+        stageB(S, buf);
+    };
 
     // MFMA operands of k-group t (eight k): one granule of A per 32-row block, four B values per
     // 32-column block.
-    auto load_ops = [&](int buf, int t, float4 (&a4)[TM], float (&b)[TN][4]) {
+    auto load_ops = [&](int buf, int t, float4 (&a4)[TM], float (&b)[TN][4]) __attribute__((always_inline)) {
 #pragma unroll
         for (int ii = 0; ii < TM; ++ii) {
             int m = wm * WTM + ii * 32 + l32;
-            a4[ii] = *(const float4*)&As[buf][m][swz(2 * t + h, m) << 2];
+            a4[ii] = ld16(&As[buf][m][swz(2 * t + h, m) << 2]);
         }
 #pragma unroll
         for (int jj = 0; jj < TN; ++jj)
@@ -233,7 +261,7 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     // the MFMAs of group t and kept there (scheduling barriers), so an LDS round trip hides
     // behind a full group of MFMAs instead of being waited for in front of every pair. Larger
     // wave tiles have enough independent MFMAs per group and are left to the compiler's scheduler.
-    auto compute = [&](int buf) {
+    auto compute = [&](int buf) __attribute__((always_inline)) {
         float4 a4[2][TM];
         float b[2][TN][4];
         load_ops(buf, kw, a4[0], b[0]);
@@ -257,35 +285,177 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
         }
     };
 
-    // prologue: slabs 0 .. DEPTH-1 in flight, slab 0 staged
-    auto for_stages = [&](auto f) {
-        f(std::integral_constant<int, 0>{});
-        if constexpr (DEPTH > 1) f(std::integral_constant<int, 1>{});
-        if constexpr (DEPTH > 2) f(std::integral_constant<int, 2>{});
-        if constexpr (DEPTH > 3) f(std::integral_constant<int, 3>{});
-    };
-    for_stages([&](auto S) {
-        if (decltype(S)::value < nslab) fetch(S, s_begin + decltype(S)::value);
-    });
-    if (nslab > 0) stage(std::integral_constant<int, 0>{}, 0);
-    __syncthreads();
-
-    // slab i lives in register stage i % DEPTH until it is staged; the loop is
-    // unrolled DEPTH times so that the stage index is a compile-time constant
-    for (int base = 0; base < nslab; base += DEPTH) {
-        for_stages([&](auto S) {
-            constexpr int st = decltype(S)::value;
-            const int i = base + st;
-            if (i < nslab) {
-                const int cur = i & 1;
-                // stage slab i+1 (already in registers) into the other buffer, then reuse
-                // the registers slab i occupied for slab i+DEPTH
-                if (i + 1 < nslab) stage(std::integral_constant<int, (st + 1) % DEPTH>{}, cur ^ 1);
-                if (i + DEPTH < nslab) fetch(S, s_begin + i + DEPTH);
-                compute(cur);
-                __syncthreads();
+    if constexpr (PIPE) {
+        // Interior problems on the small tile: a wave owns a single 32x32 accumulator pair and a slab costs it
+        // 4 * G MFMAs, so everything else has to run in the shadow of those MFMAs. The loads of slab i+2, the
+        // LDS writes of slab i+1 and the operand reads of the next k-group are placed between the MFMAs of
+        // slab i, one piece per MFMA, and pinned there. The workgroup barrier sits in the middle of the slab,
+        // after the writes of slab i+1: the operands of the k-groups behind it were read in front of it, and
+        // the first operands of slab i+1 are read during the last k-group of slab i, so no wave leaves the
+        // barrier with nothing to feed the matrix pipe. A wave that is past the barrier of slab i may write
+        // slab i+2 while a slower one still reads slab i, hence more than two LDS buffers (four, so that buffer indices repeat with the unrolled loop). Addresses are a
+        // wave-uniform base pointer that advances per slab plus a per-thread 32-bit byte offset that never
+        // changes (no vector address arithmetic in the loop). The steady-state loop has no branch around a
+        // load, so the wait for the registers of slab i+1 can leave the four younger loads of slab i+2 in
+        // flight; the last slabs are peeled into branch-free copies for the same reason.
+        unsigned a_off[A_F4], b_off[B_F4];
+        const char* ap = nullptr;
+        const char* bp = nullptr;
+        long a_step = 0, b_step = 0;
+        int fj = s_begin;  // next flat slab to fetch
+        // both segments share their leading dimensions here (the launcher checks it), so the offsets and the
+        // per-slab steps are loop constants and a segment switch only replaces the two base pointers
+        const int lda = g.seg[0].lda, ldb = g.seg[0].ldb;
+#pragma unroll
+        for (int t = 0; t < A_F4; ++t) a_off[t] = (unsigned)(((size_t)a_r[t] * lda + a_c[t]) * sizeof(float));
+#pragma unroll
+        for (int t = 0; t < B_F4; ++t) b_off[t] = (unsigned)(((size_t)b_r[t] * ldb + b_c[t]) * sizeof(float));
+        a_step = (TA ? (long)BK * lda : (long)BK) * (long)sizeof(float);
+        b_step = (TB ? (long)BK : (long)BK * ldb) * (long)sizeof(float);
+        {
+            const bool second = s_begin >= slabs0;
+            const int local_slab = second ? s_begin - slabs0 : s_begin;
+            ap = (const char*)(second ? g.seg[1].A : g.seg[0].A) + (long)local_slab * a_step;
+            bp = (const char*)(second ? g.seg[1].B : g.seg[0].B) + (long)local_slab * b_step;
+        }
+        auto fetchA = [&](auto S) __attribute__((always_inline)) {
+#pragma unroll
+            for (int t = 0; t < A_F4; ++t) ra[decltype(S)::value][t] = ld16(ap + a_off[t]);
+        };
+        auto fetchB = [&](auto S) __attribute__((always_inline)) {
+#pragma unroll
+            for (int t = 0; t < B_F4; ++t) rb[decltype(S)::value][t] = ld16(bp + b_off[t]);
+        };
+        auto advance = [&]() __attribute__((always_inline)) {
+            ++fj;
+            ap += a_step;
+            bp += b_step;
+            if (fj == slabs0 && slabs1 > 0) {
+                ap = (const char*)g.seg[1].A;
+                bp = (const char*)g.seg[1].B;
             }
+        };
+        float4 a4[2][TM];
+        float b[2][TN][4];
+        auto mfma = [&](int o, int c) __attribute__((always_inline)) {
+            const float a = c == 0 ? a4[o][0].x : (c == 1 ? a4[o][0].y : (c == 2 ? a4[o][0].z : a4[o][0].w));
+            acc[c & 1][0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b[o][0][c], acc[c & 1][0][0], 0, 0, 0);
+        };
+        // Slab i sits in LDS buffer `cur`, its k-group 0 operands are in a4[0] / b[0], the loads of slab i+1
+        // are in flight into register stage ST ^ 1. H1 / H2: slabs i+1 / i+2 exist.
+        // P: position of the step in the unrolled loop; it fixes the register stage (P % 2) and the LDS
+        // buffers (slab i in P % NBUF, slab i+1 in the next one) at compile time.
+        auto slab_step = [&](auto P, auto H1, auto H2) __attribute__((always_inline)) {
+            constexpr int ST = decltype(P)::value % 2;
+            constexpr int cur = decltype(P)::value % NBUF, nxt = (decltype(P)::value + 1) % NBUF;
+            constexpr bool has1 = decltype(H1)::value, has2 = decltype(H2)::value;
+            using S = std::integral_constant<int, ST>;
+            using NX = std::integral_constant<int, ST ^ 1>;
+            constexpr int WT = MIDB ? G / 2 - 1 : G - 1;  // k-group that carries the LDS writes and the barrier
+#pragma unroll
+            for (int tt = 0; tt < G; ++tt) {
+                const int o = tt & 1;
+                mfma(o, 0);
+                if (tt + 1 < G)
+                    load_ops(cur, (tt + 1) * KW + kw, a4[o ^ 1], b[o ^ 1]);
+                else if (has1 && MIDB)
+                    load_ops(nxt, kw, a4[0], b[0]);  // G is even: the last group used a4[1] / b[1]
+                __builtin_amdgcn_sched_barrier(0);
+                mfma(o, 1);
+                if (has2 && tt == 0) fetchA(S{});
+                if (has1 && tt == WT) stageA(NX{}, nxt);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma(o, 2);
+                if (has2 && tt == 0) fetchB(S{});
+                if (has1 && tt == WT) stageB(NX{}, nxt);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma(o, 3);
+                __builtin_amdgcn_sched_barrier(0);
+                if (tt == WT) {
+                    if (has2) advance();
+                    if (has1) __syncthreads();
+                }
+            }
+            if (has1 && !MIDB) load_ops(nxt, kw, a4[0], b[0]);
+        };
+        constexpr int U = NBUF;  // steps per trip of the unrolled loop (even)
+        // the last `r` slabs, r <= U + 1, starting at position 0
+        auto tail_step = [&](auto J, auto R) __attribute__((always_inline)) {
+            constexpr int j = decltype(J)::value, r = decltype(R)::value;
+            if constexpr (j < r)
+                slab_step(std::integral_constant<int, j % U>{}, std::integral_constant<bool, (j + 1 < r)>{},
+                          std::integral_constant<bool, (j + 2 < r)>{});
+        };
+        auto run_tail = [&](auto R) __attribute__((always_inline)) {
+            tail_step(std::integral_constant<int, 0>{}, R);
+            tail_step(std::integral_constant<int, 1>{}, R);
+            tail_step(std::integral_constant<int, 2>{}, R);
+            tail_step(std::integral_constant<int, 3>{}, R);
+            tail_step(std::integral_constant<int, 4>{}, R);
+        };
+        static_assert(U + 1 <= 5, "run_tail covers five steps");
+        using S0 = std::integral_constant<int, 0>;
+        using S1 = std::integral_constant<int, 1>;
+        using Yes = std::true_type;
+        if (nslab > 0) {
+            fetchA(S0{});
+            fetchB(S0{});
+            advance();
+            if (nslab > 1) {
+                fetchA(S1{});
+                fetchB(S1{});
+                advance();
+            }
+            stage(S0{}, 0);
+            __syncthreads();
+            load_ops(0, kw, a4[0], b[0]);
+            int i = 0;
+            for (; i + U + 1 < nslab; i += U) {
+                slab_step(std::integral_constant<int, 0>{}, Yes{}, Yes{});
+                slab_step(std::integral_constant<int, 1>{}, Yes{}, Yes{});
+                if constexpr (U > 2) {
+                    slab_step(std::integral_constant<int, 2>{}, Yes{}, Yes{});
+                    slab_step(std::integral_constant<int, 3>{}, Yes{}, Yes{});
+                }
+            }
+            const int rest = nslab - i;  // 1 .. U + 1
+            if (rest == 1) run_tail(std::integral_constant<int, 1>{});
+            else if (rest == 2) run_tail(std::integral_constant<int, 2>{});
+            else if (rest == 3) run_tail(std::integral_constant<int, 3>{});
+            else if (U > 2 && rest == 4) run_tail(std::integral_constant<int, (U > 2 ? 4 : 1)>{});
+            else if (U > 2 && rest == 5) run_tail(std::integral_constant<int, (U > 2 ? 5 : 1)>{});
+        }
+    } else {
+        // prologue: slabs 0 .. DEPTH-1 in flight, slab 0 staged
+        auto for_stages = [&](auto f) __attribute__((always_inline)) {
+            f(std::integral_constant<int, 0>{});
+            if constexpr (DEPTH > 1) f(std::integral_constant<int, 1>{});
+            if constexpr (DEPTH > 2) f(std::integral_constant<int, 2>{});
+            if constexpr (DEPTH > 3) f(std::integral_constant<int, 3>{});
+        };
+        for_stages([&](auto S) __attribute__((always_inline)) {
+            if (decltype(S)::value < nslab) fetch(S, s_begin + decltype(S)::value);
         });
+        if (nslab > 0) stage(std::integral_constant<int, 0>{}, 0);
+        __syncthreads();
+
+        // slab i lives in register stage i % DEPTH until it is staged; the loop is
+        // unrolled DEPTH times so that the stage index is a compile-time constant
+        for (int base = 0; base < nslab; base += DEPTH) {
+            for_stages([&](auto S) __attribute__((always_inline)) {
+                constexpr int st = decltype(S)::value;
+                const int i = base + st;
+                if (i < nslab) {
+                    const int cur = i & 1;
+                    // stage slab i+1 (already in registers) into the other buffer, then reuse
+                    // the registers slab i occupied for slab i+DEPTH
+                    if (i + 1 < nslab) stage(std::integral_constant<int, (st + 1) % DEPTH>{}, cur ^ 1);
+                    if (i + DEPTH < nslab) fetch(S, s_begin + i + DEPTH);
+                    compute(cur);
+                    __syncthreads();
+                }
+            });
+        }
     }
 
     if (CHAINS == 2) {
@@ -296,8 +466,8 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     }
     if (KW > 1) {
         // wave sets 1.. hand their accumulators to set 0 through LDS (the slab buffers are free now)
-        float* red = &As[0][0][0];
-        static_assert(sizeof(As) >= (size_t)(KW - 1) * BM * BN * sizeof(float), "LDS too small for the wave-set fold");
+        float* red = lds;
+        __syncthreads();  // the last slab's operand reads are done in every wave
         if (kw > 0) {
 #pragma unroll
             for (int ii = 0; ii < TM; ++ii)
@@ -377,12 +547,20 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     if (split && tid == 0) __hip_atomic_store(g.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int BM, int BN, int BK, int DEPTH, int KW = 1>
+template <int BM, int BN, int BK, int DEPTH, int KW = 1, bool MIDB = false>
 static int launch_tile(GemmArgs g, bool ta, bool tb, bool vec, int split_k) {
     if (KW > 1) split_k = 1;  // the wave-set fold and the cross-workgroup fold are alternatives
     // interior-only problems (every tile and slab full, 16-byte aligned rows) take the unchecked kernel
     bool edge = !vec || g.M % BM != 0 || g.N % BN != 0;
-    for (int s = 0; s < g.nseg; ++s) edge = edge || g.seg[s].K % BK != 0;
+    for (int s = 0; s < g.nseg; ++s) {
+        edge = edge || g.seg[s].K % BK != 0;
+        // the unchecked kernel addresses a slab through 32-bit byte offsets from its base pointer
+        const size_t a_span = ((size_t)(ta ? BK : g.M) * g.seg[s].lda + (ta ? g.M : BK)) * sizeof(float);
+        const size_t b_span = ((size_t)(tb ? g.N : BK) * g.seg[s].ldb + (tb ? BK : g.N)) * sizeof(float);
+        edge = edge || a_span >= ((size_t)1 << 32) || b_span >= ((size_t)1 << 32);
+        // and keeps one set of offsets for both segments
+        edge = edge || g.seg[s].lda != g.seg[0].lda || g.seg[s].ldb != g.seg[0].ldb;
+    }
     dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM);
     int nslab = 0;
     for (int s = 0; s < g.nseg; ++s) nslab += (g.seg[s].K + BK - 1) / BK;
@@ -399,9 +577,9 @@ static int launch_tile(GemmArgs g, bool ta, bool tb, bool vec, int split_k) {
 #define DALI_GEMM_CASE(TA_, TB_, V_)                                                                        \
     if (ta == TA_ && tb == TB_ && vec == V_) {                                                              \
         if (edge)                                                                                           \
-            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, TA_, TB_, V_, DEPTH, true, KW>), grid, block, pad_lds, st, g);  \
+            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, TA_, TB_, V_, DEPTH, true, KW, false>), grid, block, pad_lds, st, g);  \
         else if (V_)                                                                                        \
-            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, TA_, TB_, true, DEPTH, false, KW>), grid, block, pad_lds, st, g); \
+            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, TA_, TB_, true, DEPTH, false, KW, MIDB>), grid, block, pad_lds, st, g); \
     }
     DALI_GEMM_CASE(false, false, true)
     DALI_GEMM_CASE(false, false, false)
@@ -468,12 +646,9 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
     static const int split_env = getenv("DALI_HIP_GEMM_SPLITK") ? atoi(getenv("DALI_HIP_GEMM_SPLITK")) : 0;
     int split_k = split_env > 0 ? split_env : 1;
     (void)tiles64;
-    if (variant == 3) return launch_tile<64, 64, 64, 2, 2>(g, ta, tb, vec, split_k);
-    if (variant == 6) return launch_tile<64, 64, 128, 2, 2>(g, ta, tb, vec, split_k);
-    if (variant == 4) return launch_tile<64, 64, 64, 3, 2>(g, ta, tb, vec, split_k);
-    if (variant == 1) return launch_tile<64, 64, 32, 3>(g, ta, tb, vec, split_k);
-    if (variant == 2) return launch_tile<64, 64, 64, 3>(g, ta, tb, vec, split_k);
     if (variant == 8) return launch_tile<64, 64, 64, 2>(g, ta, tb, vec, split_k);
+    if (variant == 5) return launch_tile<64, 64, 64, 2, 2, true>(g, ta, tb, vec, split_k);
+    if (variant == 9) return launch_tile<64, 64, 64, 2, 4>(g, ta, tb, vec, split_k);
     // default for small grids: two wave sets per 64x64 tile (two waves per SIMD)
     return launch_tile<64, 64, 64, 2, 2>(g, ta, tb, vec, split_k);
 }
