@@ -152,6 +152,21 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
             b_c[t] = (idx % (BK / 4)) * 4;       // k offset inside the slab
         }
     }
+    if (!EDGE) {
+        // Tiles that hang over the edge of C read the last valid row (or 4-column granule) instead: what
+        // they compute for rows and columns outside C is never stored, so no zeros are needed, only
+        // addresses inside the operands. Granules along M or N are whole here (the launcher checks).
+#pragma unroll
+        for (int t = 0; t < A_F4; ++t) {
+            if (!TA) a_r[t] = a_r[t] < M ? a_r[t] : M - 1;
+            else a_c[t] = a_c[t] < M ? a_c[t] : M - 4;
+        }
+#pragma unroll
+        for (int t = 0; t < B_F4; ++t) {
+            if (!TB) b_c[t] = b_c[t] < N ? b_c[t] : N - 4;
+            else b_r[t] = b_r[t] < N ? b_r[t] : N - 1;
+        }
+    }
 
     // One 4-float granule at row r, columns c..c+3 of a row-major array with `rows` x `cols`
     // valid entries. Interior tiles (EDGE == false) load unconditionally; edge tiles clamp the
@@ -524,11 +539,11 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
 #pragma unroll
         for (int jj = 0; jj < TN; ++jj) {
             int n = n0 + wn * WTN + jj * 32 + l32;
-            if (EDGE && n >= N) continue;
+            if (n >= N) continue;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 int m = m0 + wm * WTM + ii * 32 + 8 * (v / 4) + 4 * h + (v % 4);
-                if (!EDGE || m < M) {
+                if (m < M) {
                     float* c = g.C + (size_t)m * g.ldc + n;
                     float sum;
                     if (split) {
@@ -548,19 +563,9 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
 }
 
 template <int BM, int BN, int BK, int DEPTH, int KW = 1, bool MIDB = false>
-static int launch_tile(GemmArgs g, bool ta, bool tb, bool vec, int split_k) {
+static int launch_tile(GemmArgs g, bool ta, bool tb, bool vec, int split_k, bool edge) {
     if (KW > 1) split_k = 1;  // the wave-set fold and the cross-workgroup fold are alternatives
-    // interior-only problems (every tile and slab full, 16-byte aligned rows) take the unchecked kernel
-    bool edge = !vec || g.M % BM != 0 || g.N % BN != 0;
-    for (int s = 0; s < g.nseg; ++s) {
-        edge = edge || g.seg[s].K % BK != 0;
-        // the unchecked kernel addresses a slab through 32-bit byte offsets from its base pointer
-        const size_t a_span = ((size_t)(ta ? BK : g.M) * g.seg[s].lda + (ta ? g.M : BK)) * sizeof(float);
-        const size_t b_span = ((size_t)(tb ? g.N : BK) * g.seg[s].ldb + (tb ? BK : g.N)) * sizeof(float);
-        edge = edge || a_span >= ((size_t)1 << 32) || b_span >= ((size_t)1 << 32);
-        // and keeps one set of offsets for both segments
-        edge = edge || g.seg[s].lda != g.seg[0].lda || g.seg[s].ldb != g.seg[0].ldb;
-    }
+    if (!vec) edge = true;
     dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM);
     int nslab = 0;
     for (int s = 0; s < g.nseg; ++s) nslab += (g.seg[s].K + BK - 1) / BK;
@@ -593,6 +598,46 @@ static int launch_tile(GemmArgs g, bool ta, bool tb, bool vec, int split_k) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("sgemm launch failed: %s", hipGetErrorString(e));
     return DALI_HIP_OK;
+}
+
+// One product on one tile configuration. When the operands allow the unchecked kernel (16-byte aligned rows,
+// whole 4-column granules along M / N where a granule runs along them, offsets that fit 32 bits, one pair of
+// leading dimensions), the whole slabs of every segment go through it, whatever M and N are; what is left of
+// K (less than one slab per segment) is added by a second, checked launch with beta = 1.
+template <int BM, int BN, int BK, int DEPTH, int KW = 1, bool MIDB = false>
+static int run_tile(const GemmArgs& g, bool ta, bool tb, bool vec, int split_k) {
+    bool fast = vec && g.nseg > 0 && (!ta || g.M % 4 == 0) && (tb || g.N % 4 == 0);
+    for (int s = 0; s < g.nseg && fast; ++s) {
+        const size_t a_span = ((size_t)(ta ? BK : g.M) * g.seg[s].lda + (ta ? g.M : BK)) * sizeof(float);
+        const size_t b_span = ((size_t)(tb ? g.N : BK) * g.seg[s].ldb + (tb ? BK : g.N)) * sizeof(float);
+        fast = fast && a_span < ((size_t)1 << 32) && b_span < ((size_t)1 << 32);
+        fast = fast && g.seg[s].lda == g.seg[0].lda && g.seg[s].ldb == g.seg[0].ldb;
+    }
+    if (!fast) return launch_tile<BM, BN, BK, DEPTH, KW, MIDB>(g, ta, tb, vec, split_k, true);
+    GemmArgs whole = g, rest = g;
+    whole.nseg = rest.nseg = 0;
+    for (int s = 0; s < g.nseg; ++s) {
+        const GemmSeg& sg = g.seg[s];
+        const int kw = sg.K / BK * BK, kr = sg.K - kw;
+        if (kw > 0) {
+            GemmSeg& d = whole.seg[whole.nseg++];
+            d = sg;
+            d.K = kw;
+        }
+        if (kr > 0) {
+            GemmSeg& d = rest.seg[rest.nseg++];
+            d = sg;
+            d.A = sg.A + (ta ? (size_t)kw * sg.lda : (size_t)kw);
+            d.B = sg.B + (tb ? (size_t)kw : (size_t)kw * sg.ldb);
+            d.K = kr;
+        }
+    }
+    if (whole.nseg > 0) {
+        int st = launch_tile<BM, BN, BK, DEPTH, KW, MIDB>(whole, ta, tb, true, split_k, false);
+        if (st || rest.nseg == 0) return st;
+        rest.beta = 1.0f;
+    }
+    return launch_tile<BM, BN, BK, DEPTH, KW, MIDB>(rest, ta, tb, true, 1, true);
 }
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
@@ -639,18 +684,18 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
     }
     long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     static const int variant = getenv("DALI_HIP_GEMM_VARIANT") ? atoi(getenv("DALI_HIP_GEMM_VARIANT")) : 0;
-    if (tiles128 >= 192) return launch_tile<128, 128, 32, 2>(g, ta, tb, vec, 1);
+    if (tiles128 >= 192) return run_tile<128, 128, 32, 2>(g, ta, tb, vec, 1);
     // Small grids: 64x64 tiles, and when even those leave CUs with a single workgroup, split K so
     // that two workgroups share a CU and one's barriers and memory waits hide behind the other's MFMAs.
     long tiles64 = (long)((M + 63) / 64) * ((N + 63) / 64);
     static const int split_env = getenv("DALI_HIP_GEMM_SPLITK") ? atoi(getenv("DALI_HIP_GEMM_SPLITK")) : 0;
     int split_k = split_env > 0 ? split_env : 1;
     (void)tiles64;
-    if (variant == 8) return launch_tile<64, 64, 64, 2>(g, ta, tb, vec, split_k);
-    if (variant == 5) return launch_tile<64, 64, 64, 2, 2, true>(g, ta, tb, vec, split_k);
-    if (variant == 9) return launch_tile<64, 64, 64, 2, 4>(g, ta, tb, vec, split_k);
+    if (variant == 8) return run_tile<64, 64, 64, 2>(g, ta, tb, vec, split_k);
+    if (variant == 5) return run_tile<64, 64, 64, 2, 2, true>(g, ta, tb, vec, split_k);
+    if (variant == 9) return run_tile<64, 64, 64, 2, 4>(g, ta, tb, vec, split_k);
     // default for small grids: two wave sets per 64x64 tile (two waves per SIMD)
-    return launch_tile<64, 64, 64, 2, 2>(g, ta, tb, vec, split_k);
+    return run_tile<64, 64, 64, 2, 2>(g, ta, tb, vec, split_k);
 }
 
 }  // namespace dali_hip

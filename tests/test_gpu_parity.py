@@ -120,7 +120,8 @@ def _dev(hip, a):
     return p
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (5, 11, 7), (64, 64, 64), (65, 130, 33), (256, 4096, 128), (300, 200, 100)])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (5, 11, 7), (64, 64, 64), (65, 130, 33), (256, 4096, 128), (300, 200, 100),
+                                   (132, 72, 640), (252, 1000, 1000), (1100, 2300, 260), (2052, 2052, 132)])
 @pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
 def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
     """dali_hip_sgemm(transB, transA, m, n, k, alpha, B, ldb, A, lda, beta, C, ldc) as cublasSgemm is called in
@@ -147,9 +148,9 @@ def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
         hip.dali_hip_free(p)
 
 
-def test_sgemm_pair_accumulates_two_products(gpu, rng):
+@pytest.mark.parametrize("M,N,K1,K2", [(48, 200, 96, 40), (100, 260, 200, 200), (256, 512, 128, 192), (250, 1000, 100, 100)])
+def test_sgemm_pair_accumulates_two_products(gpu, rng, M, N, K1, K2):
     hip = gpu
-    M, N, K1, K2 = 48, 200, 96, 40
     A1, B1 = rng.randn(M, K1).astype(np.float32), rng.randn(K1, N).astype(np.float32)
     A2, B2 = rng.randn(M, K2).astype(np.float32), rng.randn(K2, N).astype(np.float32)
     dA1, dB1, dA2, dB2 = (_dev(hip, x) for x in (A1, B1, A2, B2))
