@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     // The small-tile interior kernel runs a software pipeline with the workgroup barrier in the middle of a slab
     // (see its loop below), which needs a third slab buffer.
     constexpr int G = BK / 8 / KW;  // k-groups of a slab per wave set
-    constexpr bool PIPE = !EDGE && TM * TN == 1 && DEPTH == 2 && G >= 2 && G % 2 == 0;
+    constexpr bool PIPE = !EDGE && DEPTH == 2 && G >= 2 && G % 2 == 0;
     constexpr int NBUF = PIPE && MIDB ? 4 : 2;
     // one LDS block: the A slab buffers, the B slab buffers; reused for the wave-set fold at the end
     constexpr int AS_FLOATS = NBUF * BM * BK, BS_FLOATS = NBUF * BK * (BN + BPAD), RED_FLOATS = (KW - 1) * BM * BN;
@@ -301,8 +301,8 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     };
 
     if constexpr (PIPE) {
-        // Interior problems on the small tile: a wave owns a single 32x32 accumulator pair and a slab costs it
-        // 4 * G MFMAs, so everything else has to run in the shadow of those MFMAs. The loads of slab i+2, the
+        // Unchecked kernel: every instruction that is not an MFMA has to run in the shadow of the MFMAs (vector
+        // ALU instructions in particular take issue time from the matrix pipe, measured ~6 cycles each). The loads of slab i+2, the
         // LDS writes of slab i+1 and the operand reads of the next k-group are placed between the MFMAs of
         // slab i, one piece per MFMA, and pinned there. The workgroup barrier sits in the middle of the slab,
         // after the writes of slab i+1: the operands of the k-groups behind it were read in front of it, and
@@ -352,12 +352,18 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
         };
         float4 a4[2][TM];
         float b[2][TN][4];
+        // the TM x TN MFMAs of one k (two k, one per half-wave) of the current k-group
         auto mfma = [&](int o, int c) __attribute__((always_inline)) {
-            const float a = c == 0 ? a4[o][0].x : (c == 1 ? a4[o][0].y : (c == 2 ? a4[o][0].z : a4[o][0].w));
-            acc[c & 1][0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b[o][0][c], acc[c & 1][0][0], 0, 0, 0);
+#pragma unroll
+            for (int ii = 0; ii < TM; ++ii) {
+                const float a = c == 0 ? a4[o][ii].x : (c == 1 ? a4[o][ii].y : (c == 2 ? a4[o][ii].z : a4[o][ii].w));
+#pragma unroll
+                for (int jj = 0; jj < TN; ++jj) {
+                    const int ch = CHAINS == 2 ? (c & 1) : 0;
+                    acc[ch][ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b[o][jj][c], acc[ch][ii][jj], 0, 0, 0);
+                }
+            }
         };
-        // Slab i sits in LDS buffer `cur`, its k-group 0 operands are in a4[0] / b[0], the loads of slab i+1
-        // are in flight into register stage ST ^ 1. H1 / H2: slabs i+1 / i+2 exist.
         // P: position of the step in the unrolled loop; it fixes the register stage (P % 2) and the LDS
         // buffers (slab i in P % NBUF, slab i+1 in the next one) at compile time.
         auto slab_step = [&](auto P, auto H1, auto H2) __attribute__((always_inline)) {
