@@ -230,6 +230,29 @@ def main():
                                                  "gemm_pair_us": round(gemm_us, 2),
                                                  "gemm_TFLOP/s": round(flops / gemm_us / 1e6, 2),
                                                  "gemm_frac_fp32_mfma": round(flops / gemm_us / 1e6 / MFMA_FP32_PEAK_TFLOPS, 4)}
+        del X, Hp, Cp, W, U, bias, rec, grec
+
+        # rows beyond the five configs: embedding-style gather and its scatter-add (table [32000, 1024], 8192 indices)
+        V, Dm, Nidx = 32000, 1024, 8192
+        table = D.Array.from_numpy(np.random.RandomState(14).randn(V, Dm).astype(np.float32))
+        ids = D.Array.from_numpy(np.random.RandomState(15).randint(0, V, Nidx).astype(np.int32))
+        upd = D.Array.from_numpy(np.random.RandomState(16).randn(Nidx, Dm).astype(np.float32))
+        with D.Recording() as rec:
+            op.gather(table, ids).eval()
+        us = time_recording(rec, 50)
+        gbytes = 2 * Nidx * Dm * 4
+        nxt = {"gather_32000x1024_8192": {"us": round(us, 2), "GB/s": round(gbytes / us / 1e3, 1),
+                                          "frac_hbm": round(gbytes / us / 1e3 / HBM_PEAK_GBS, 4), "kernels": rec.launches}}
+        with D.Recording() as rec:
+            g = table[ids]
+            g += upd
+        us = time_recording(rec, 50)
+        uniq = int(np.unique(ids.numpy()).size)
+        sbytes = Nidx * Dm * 4 + 2 * uniq * Dm * 4  # values once, every touched table row read and written once
+        nxt["scatter_add_32000x1024_8192"] = {"us": round(us, 2), "GB/s": round(sbytes / us / 1e3, 1),
+                                              "frac_hbm": round(sbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                                              "launches_incl_index_sort": rec.launches, "distinct_rows": uniq}
+        configs["beyond_the_five_configs"] = nxt
         result["configs"] = configs
 
     # --------------------------------------------------------- CPU baseline

@@ -82,6 +82,7 @@ HIP_SYMBOLS = {
     "dali_hip_set_cache_dir": (_i, [C.c_char_p]),
     "dali_hip_sgemm": (_i, [_i, _i, _i, _i, _i, C.c_float, H, _i, H, _i, C.c_float, H, _i]),
     "dali_hip_sgemm_pair": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, C.c_float, H, _i, H, _i, H, _i, H, _i, C.c_float, H, _i]),
+    "dali_hip_argsort_i32": (_i, [H, C.c_int64, C.c_int32, H, H]),
     "dali_hip_capture_begin": (_i, []),
     "dali_hip_capture_end": (_i, [C.POINTER(H)]),
     "dali_hip_graph_launch": (_i, [H]),
@@ -131,6 +132,8 @@ FRONT_SYMBOLS = {
     "dali_fe_mean_axes": (H, [H, _ip, _i, _i]),
     "dali_fe_softmax": (H, [H, _i]),
     "dali_fe_gather_from_rows": (H, [H, H]),
+    "dali_fe_gather": (H, [H, H]),
+    "dali_fe_autoreduce_assign": (_i, [H, H]),
     "dali_fe_one_hot": (H, [H, _i, H, H]),
     "dali_fe_dot": (H, [H, H]),
     "dali_fe_softmax_cross_entropy": (_i, [H, H, _HP, _HP, _HP]),

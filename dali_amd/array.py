@@ -131,6 +131,9 @@ class Array(object):
 
     def __getitem__(self, key):
         """Integers pluck an axis, slices make strided views (buffers only evaluate lazily built nodes first)."""
+        if isinstance(key, Array):
+            from . import op
+            return op.gather(self, key)
         if not isinstance(key, tuple):
             key = (key,)
         out, axis = self, 0
@@ -189,6 +192,17 @@ class Array(object):
 
     def __itruediv__(self, other):
         return self.assign(other, 4)
+
+    def __ilshift__(self, other):
+        """dst <<= src: add the sum of ``src`` over the axes where ``dst`` has extent 1."""
+        other = as_array(other)
+        if front.dali_fe_autoreduce_assign(self._h, other._h) != 0:
+            raise fe_error("autoreduce_assign")
+        return self
+
+    def gather_from_rows(self, indices):
+        from . import op
+        return op.gather_from_rows(self, indices)
 
     # ---- arithmetic sugar
     def __add__(self, o):

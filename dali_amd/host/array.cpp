@@ -439,6 +439,9 @@ Array& Array::operator+=(const Array& other) { evaluate_into(*this, OPERATOR_T_A
 Array& Array::operator-=(const Array& other) { evaluate_into(*this, OPERATOR_T_SUB, other); return *this; }
 Array& Array::operator*=(const Array& other) { evaluate_into(*this, OPERATOR_T_MUL, other); return *this; }
 Array& Array::operator/=(const Array& other) { evaluate_into(*this, OPERATOR_T_DIV, other); return *this; }
+Array& Array::operator<<=(const Array& other) { return op::autoreduce_assign(*this, other); }
+Array Array::operator[](const Array& indices) const { return op::gather(*this, indices); }
+Array Array::gather_from_rows(const Array& indices) const { return op::gather_from_rows(*this, indices); }
 
 Array Array::sum() const { return op::sum(*this); }
 Array Array::sum(const std::vector<int>& axes, bool keepdims) const { return op::sum(*this, axes, keepdims); }
@@ -732,6 +735,38 @@ Array gather_from_rows(const Array& source, const Array& indices) {
     }
     std::vector<int> shape = indices.ndim() ? indices.shape() : std::vector<int>{1};
     return make_node(Kind::GATHER_FROM_ROWS, "", {source, indices}, shape, source.dtype());
+}
+
+// dali/array/op/gather.cpp:163-171: out[i..., rest...] = source[indices[i...], rest...]. The node keeps the
+// source as a 2-D [V, D] view and the indices as a 1-D vector; its own shape is indices.shape + source.shape[1:].
+// Assigning to the lazy node scatters into the source buffer (gather.cpp:126-143).
+Array gather(const Array& source, const Array& indices) {
+    DALI_ASSERT(source.ndim() > 0, make_message("gather must be called on source with ndim > 0 (got ndim=", source.ndim(), ")."));
+    DALI_ASSERT(indices.dtype() == DTYPE_INT32, make_message("indices must be integers (got dtype=", dtype_to_cpp_name(indices.dtype()), ")."));
+    Array src2 = source;
+    if (source.ndim() == 1) src2 = source.expand_dims(1);
+    else if (source.ndim() > 2) src2 = source.reshape({source.shape()[0], -1});
+    Array idx1 = indices.ndim() == 1 ? indices : indices.reshape({-1});
+    std::vector<int> shape = indices.shape();
+    shape.insert(shape.end(), source.shape().begin() + 1, source.shape().end());
+    return make_node(Kind::GATHER, "", {src2, idx1}, shape, source.dtype());
+}
+
+// dali/array/expression/assignment.cpp:92-126: left += sum of right over the axes where left has extent 1
+Array& autoreduce_assign(Array& left, const Array& right) {
+    DALI_ASSERT(left.ndim() == right.ndim(), make_message("destination for autoreduce_assign must have the same dimensionality as the input (destination.ndim = ",
+                                                          left.ndim(), " vs input.ndim = ", right.ndim()));
+    std::vector<int> reduction_axes;
+    for (int i = 0; i < right.ndim(); ++i) {
+        if (left.shape()[i] != right.shape()[i]) {
+            DALI_ASSERT(left.shape()[i] == 1, make_message("Could not autoreduce_assign: destination must have all dimensions equal input dimensions or equal 1, but destination.shape[",
+                                                           i, "] = ", left.shape()[i], " vs input.shape[", i, "] = ", right.shape()[i]));
+            reduction_axes.push_back(i);
+        }
+    }
+    Array r = reduction_axes.empty() ? right : sum(right, reduction_axes, /*keepdims=*/true);
+    left += r;
+    return left;
 }
 
 // dali/array/op/one_hot.cpp:62-74

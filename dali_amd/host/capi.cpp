@@ -106,6 +106,8 @@ dali_array_t dali_fe_mean_axes(dali_array_t a, const int* axes, int naxes, int k
 }
 dali_array_t dali_fe_softmax(dali_array_t a, int axis) { FE_TRY(return wrap(dali::op::softmax(A(a), axis));, nullptr) }
 dali_array_t dali_fe_gather_from_rows(dali_array_t s, dali_array_t i) { FE_TRY(return wrap(dali::op::gather_from_rows(A(s), A(i)));, nullptr) }
+dali_array_t dali_fe_gather(dali_array_t s, dali_array_t i) { FE_TRY(return wrap(dali::op::gather(A(s), A(i)));, nullptr) }
+int dali_fe_autoreduce_assign(dali_array_t dest, dali_array_t source) { FE_TRY(dali::op::autoreduce_assign(A(dest), A(source)); return 0;, 1) }
 dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_value, dali_array_t off_value) {
     FE_TRY(return wrap(dali::op::one_hot(A(indices), depth, A(on_value), A(off_value)));, nullptr)
 }

@@ -120,6 +120,12 @@ class Array {
     Array& operator-=(const Array& other);
     Array& operator*=(const Array& other);
     Array& operator/=(const Array& other);
+    // dst += sum of `other` over the axes where dst has extent 1 (dali/array/array.h, operator<<=)
+    Array& operator<<=(const Array& other);
+    // rows picked by an int32 index array; assigning to the result scatters into this array
+    // (dali/array/array.h:139, dali/array/op/gather.cpp)
+    Array operator[](const Array& indices) const;
+    Array gather_from_rows(const Array& indices) const;
 
     // host access: evaluates, migrates and writes the elements row-major
     void to_host(void* out) const;
@@ -217,6 +223,8 @@ Array argmin(const Array& x, int axis);
 // dali/array/op/softmax.h, gather_from_rows.h, one_hot.h, dot.h
 Array softmax(const Array& logits, int axis = -1);
 Array gather_from_rows(const Array& source, const Array& indices);
+Array gather(const Array& source, const Array& indices);
+Array& autoreduce_assign(Array& left, const Array& right);
 Array one_hot(Array indices, int depth, Array on_value, Array off_value);
 Array matmul(Array a, Array b);
 Array dot(const Array& a, const Array& b);

@@ -19,6 +19,7 @@ enum class Kind {
     EXPAND_DIMS,       // dali/array/jit/reshape.cpp:156-209
     BROADCAST,         // dali/array/jit/reshape.cpp:62-154 (BroadcastedReshape)
     GATHER_FROM_ROWS,  // dali/array/op/gather_from_rows.cpp:21-127
+    GATHER,            // dali/array/op/gather.cpp:31-160 (rows of a 2-D source picked by a 1-D index)
     ONE_HOT,           // dali/array/op/one_hot.cpp:16-74
     MATMUL             // dali/array/op/dot.cpp:18-47
 };

@@ -123,6 +123,7 @@ struct ArrayArg {
     bool strided = false;
     std::vector<int> sizes, strides;
     int64_t row_stride = 0, col_stride = 1;
+    int row_index = -1;  // FULL presentation of a gather source: array whose per-row value picks the source row
 };
 
 struct ScalarArg {
@@ -288,7 +289,9 @@ int add_array(Program& P, const std::shared_ptr<Expr>& b, Cls cls, bool gather, 
     if (!is_dest) {
         std::string key = array_key(b.get(), cls, gather);
         for (size_t i = 0; i < P.arrays.size(); ++i)
-            if (!P.arrays[i].is_dest && array_key(P.arrays[i].buf.get(), P.arrays[i].cls, P.arrays[i].gather_source) == key) return (int)i;
+            if (!P.arrays[i].is_dest && P.arrays[i].row_index < 0 &&
+                array_key(P.arrays[i].buf.get(), P.arrays[i].cls, P.arrays[i].gather_source) == key)
+                return (int)i;
     }
     P.arrays.push_back(a);
     return (int)P.arrays.size() - 1;
@@ -388,6 +391,37 @@ bool classify(Program& P, int id, Cls want, const Domain& dom) {
             if (ai < 0) return false;
             P.nodes[id].array = ai;  // the gather node owns the source presentation
             return classify(P, idx, Cls::ROW, dom);
+        }
+        case Kind::GATHER: {
+            // out[r, c] = source[indices[r], c]: the source is an ordinary FULL leaf whose row pointer goes
+            // through the index (dali/array/op/gather.cpp:49-52)
+            if (want != Cls::FULL || dom.flat) return false;
+            int src = n.args[0], idx = n.args[1];
+            if (P.nodes[src].kind != Kind::BUFFER || P.nodes[idx].kind != Kind::BUFFER) return false;
+            const std::vector<int>& ss = P.nodes[src].shape;
+            if (ss.size() != 2 || ss[1] != dom.C || numel_of(P.nodes[idx].shape) != dom.R) return false;
+            if (P.nodes[idx].dtype != DTYPE_INT32) return false;
+            if (!classify(P, idx, Cls::ROW, dom)) return false;
+            ArrayArg a;
+            a.buf = P.nodes[src].src;
+            a.cls = Cls::FULL;
+            a.nd = 2;
+            a.sizes = ss;
+            auto st = strides_of(a.buf.get());
+            a.row_stride = st[0];
+            a.col_stride = st[1];
+            a.strided = !(st[1] == 1 && st[0] == dom.C);
+            a.strides = {st[0], st[1]};
+            a.row_index = P.nodes[idx].array;
+            for (size_t i = 0; i < P.arrays.size(); ++i)
+                if (!P.arrays[i].is_dest && P.arrays[i].row_index == a.row_index &&
+                    array_key(P.arrays[i].buf.get(), Cls::FULL, false) == array_key(a.buf.get(), Cls::FULL, false)) {
+                    P.nodes[id].array = (int)i;
+                    return true;
+                }
+            P.arrays.push_back(a);
+            P.nodes[id].array = (int)P.arrays.size() - 1;
+            return true;
         }
         case Kind::ONE_HOT: {
             if (want != Cls::FULL || n.depth != dom.C) return false;
@@ -522,6 +556,8 @@ struct BodyEmitter {
                 return "((const " + t + "*)A.p[" + std::to_string(n.array) + "])[row * g_rs" + std::to_string(n.array) + " + (long)(" +
                        value(n.args[1]) + ") * g_cs" + std::to_string(n.array) + "]";
             }
+            case Kind::GATHER:
+                return "x" + std::to_string(n.array) + leaf_suffix;
             case Kind::ONE_HOT:
                 return "dali_one_hot<" + ctype(n.dtype) + ">(" + value(n.args[2]) + ", col, (" + ctype(n.dtype) + ")" + value(n.args[0]) +
                        ", (" + ctype(n.dtype) + ")" + value(n.args[1]) + ")";
@@ -656,7 +692,7 @@ std::string signature(const Program& P, const std::vector<Output>& outs) {
         ss << ");";
     }
     ss << "#";
-    for (const ArrayArg& a : P.arrays) ss << a.nd << (a.strided ? "s" : "c") << (int)a.cls << (a.gather_source ? "g" : "") << (int)a.buf->dtype << ";";
+    for (const ArrayArg& a : P.arrays) ss << a.nd << (a.strided ? "s" : "c") << (int)a.cls << (a.gather_source ? "g" : "") << (a.row_index >= 0 ? "i" + std::to_string(a.row_index) : std::string()) << (int)a.buf->dtype << ";";
     ss << "#";
     for (const ScalarArg& s : P.scalars) ss << (int)s.dtype << ";";
     ss << "#";
@@ -685,6 +721,18 @@ void fill_plan_arrays(KernelSpec& K, const Program& P, const std::vector<int>& s
 
 // Declarations of row pointers and per-row values shared by the row and flat templates.
 void emit_row_prologue(std::ostringstream& ss, const Program& P, const IvLayout& L) {
+    // per-row and scalar input values first: a gathered source's row pointer needs its index value
+    for (size_t i = 0; i < P.arrays.size(); ++i) {
+        const ArrayArg& a = P.arrays[i];
+        std::string t = ctype(a.buf->dtype);
+        if (a.gather_source || a.is_dest) continue;
+        if (a.cls == Cls::ROW) {
+            std::string s = a.strided ? " * (long)A.iv[" + std::to_string(L.stride_pos[i]) + "]" : "";
+            ss << "  const " << t << " rl" << i << " = ((const " << t << "*)A.p[" << i << "])[row" << s << "];\n";
+        } else if (a.cls == Cls::SCAL) {
+            ss << "  const " << t << " sl" << i << " = ((const " << t << "*)A.p[" << i << "])[0];\n";
+        }
+    }
     for (size_t i = 0; i < P.arrays.size(); ++i) {
         const ArrayArg& a = P.arrays[i];
         std::string t = ctype(a.buf->dtype);
@@ -695,19 +743,14 @@ void emit_row_prologue(std::ostringstream& ss, const Program& P, const IvLayout&
                 ss << "  const long g_rs" << i << " = A.iv[" << L.size_pos[i] + 1 << "], g_cs" << i << " = 1;\n";
         } else if (a.cls == Cls::FULL) {
             std::string rs = a.strided ? "(long)A.iv[" + std::to_string(L.stride_pos[i]) + "]" : "C";
-            ss << "  " << (a.is_dest ? "" : "const ") << t << "* q" << i << " = (" << (a.is_dest ? "" : "const ") << t << "*)A.p[" << i << "] + row * " << rs << ";\n";
+            std::string r = a.row_index >= 0 ? "(long)rl" + std::to_string(a.row_index) : std::string("row");
+            ss << "  " << (a.is_dest ? "" : "const ") << t << "* q" << i << " = (" << (a.is_dest ? "" : "const ") << t << "*)A.p[" << i << "] + " << r << " * " << rs << ";\n";
             if (a.strided) ss << "  const long cs" << i << " = A.iv[" << L.stride_pos[i] + 1 << "];\n";
         } else if (a.cls == Cls::ROW) {
             std::string s = a.strided ? " * (long)A.iv[" + std::to_string(L.stride_pos[i]) + "]" : "";
-            if (a.is_dest)
-                ss << "  " << t << "* q" << i << " = (" << t << "*)A.p[" << i << "] + row" << s << ";\n";
-            else
-                ss << "  const " << t << " rl" << i << " = ((const " << t << "*)A.p[" << i << "])[row" << s << "];\n";
+            if (a.is_dest) ss << "  " << t << "* q" << i << " = (" << t << "*)A.p[" << i << "] + row" << s << ";\n";
         } else {
-            if (a.is_dest)
-                ss << "  " << t << "* q" << i << " = (" << t << "*)A.p[" << i << "];\n";
-            else
-                ss << "  const " << t << " sl" << i << " = ((const " << t << "*)A.p[" << i << "])[0];\n";
+            if (a.is_dest) ss << "  " << t << "* q" << i << " = (" << t << "*)A.p[" << i << "];\n";
         }
     }
 }
@@ -2104,11 +2147,33 @@ Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root) {
             std::vector<Array> args;
             bool changed = false;
             for (const Array& x : e->args) {
-                Array c = clean(x, memo, false);
+                Array c = clean(x, memo, is_root && x.shape() == e->shape);
                 changed = changed || c.expression().get() != x.expression().get();
                 args.push_back(c);
             }
             if (changed) out = rebuild(e, args);
+            break;
+        }
+        case Kind::GATHER: {
+            // source and index are presented as buffers; the gather itself stays lazy only where the row
+            // kernel can read through it: a [N, D] node that is the root or sits under same-shape
+            // elementwise nodes of the root. Everything else is evaluated through the [N, D] form.
+            Array src = clean(e->args[0], memo, false);
+            if (src.expression()->kind != Kind::BUFFER) src = materialize(src);
+            Array idx = clean(e->args[1], memo, false);
+            if (idx.expression()->kind != Kind::BUFFER) idx = materialize(idx);
+            const int n_idx = numel_of(idx.shape()), d2 = src.shape()[1];
+            const bool two_d = e->shape.size() == 2 && e->shape[0] == n_idx && e->shape[1] == d2;
+            if (is_root && two_d) {
+                out = rebuild(e, {src, idx});
+            } else {
+                auto n2 = std::make_shared<Expr>(*e);
+                n2->args = {src, idx};
+                n2->shape = {n_idx, d2};
+                Array g2(n2);
+                evaluate({g2});
+                out = g2.reshape(e->shape);
+            }
             break;
         }
         case Kind::GATHER_FROM_ROWS: {
@@ -2317,6 +2382,208 @@ void run_specs(std::vector<DestSpec> specs) {
     throw std::runtime_error("planner did not converge");
 }
 
+// ---------------------------------------------------------------- scatter
+// Assignment through a gather: dest[indices[i], :] (op)= values[i, :] for i in input order
+// (dali/array/op/gather.cpp:89-97,126-143). The indices are ordered by a stable sort; one workgroup per run of
+// equal indices reads the destination row once, applies the run's contributions one after the other in input
+// order (the order of the reference's sequential CPU loop) and writes the row once. No atomics, and the result
+// does not depend on scheduling.
+ArrayArg manual_arg(const Array& buf, Cls cls, bool is_dest, int nd, const std::vector<int>& sizes, const std::vector<int>& strides) {
+    ArrayArg a;
+    a.buf = buf.expression();
+    a.cls = cls;
+    a.is_dest = is_dest;
+    a.nd = nd;
+    a.sizes = sizes;
+    a.strided = !strides.empty();
+    a.strides = strides;
+    return a;
+}
+
+std::string gen_scatter_rows_kernel(const Program& P, const IvLayout& L, OPERATOR_T op, bool scalar_value, int VEC, const std::string& kname) {
+    std::string t = ctype(P.arrays[0].buf->dtype);
+    std::ostringstream ss;
+    ss << codegen::kDevicePrelude;
+    ss << kargs_struct(P, L);
+    ss << "extern \"C\" __global__ __launch_bounds__(256) void " << kname << "(KArgs A) {\n";
+    ss << "  constexpr int VEC = " << VEC << ";\n";
+    ss << "  const long N = A.iv[" << L.shape_pos[0] << "], D = A.iv[" << L.shape_pos[0] + 1 << "];\n";
+    ss << "  const int* sk = (const int*)A.p[1];\n  const int* pm = (const int*)A.p[2];\n";
+    ss << "  const long p = blockIdx.x;\n  const int key = sk[p];\n";
+    ss << "  if (p > 0 && sk[p - 1] == key) return;  // only the head of a run of equal indices works\n";
+    ss << "  long q_end = p + 1;\n  while (q_end < N && sk[q_end] == key) ++q_end;\n";
+    ss << "  const long drs = A.iv[" << L.stride_pos[0] << "], dcs = A.iv[" << L.stride_pos[0] + 1 << "];\n";
+    ss << "  " << t << "* drow = (" << t << "*)A.p[0] + (long)key * drs;\n";
+    if (scalar_value) {
+        ss << "  const " << t << " sv = ((const " << t << "*)A.p[3])[0];\n";
+    } else {
+        ss << "  const long vrs = A.iv[" << L.stride_pos[3] << "], vcs = A.iv[" << L.stride_pos[3] + 1 << "];\n";
+        ss << "  const " << t << "* vals = (const " << t << "*)A.p[3];\n";
+    }
+    ss << "  for (long c = (long)threadIdx.x * VEC; c < D; c += 256 * VEC) {\n";
+    if (VEC > 1) {
+        ss << "    dali_vec<" << t << ", VEC> acc = dali_load<" << t << ", VEC>(drow + c);\n";
+        ss << "    for (long q = p; q < q_end; ++q) {\n";
+        if (!scalar_value) ss << "      const dali_vec<" << t << ", VEC> v = dali_load_nt<" << t << ", VEC>(vals + (long)pm[q] * vrs + c);\n";
+        ss << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc.v[j] = " << op_combine(op, "acc.v[j]", scalar_value ? "sv" : "v.v[j]") << ";\n";
+        ss << "    }\n    dali_store<" << t << ", VEC>(drow + c, acc);\n";
+    } else {
+        ss << "    " << t << " acc = drow[c * dcs];\n";
+        ss << "    for (long q = p; q < q_end; ++q) {\n";
+        if (!scalar_value) ss << "      const " << t << " v = vals[(long)pm[q] * vrs + c * vcs];\n";
+        ss << "      acc = " << op_combine(op, "acc", scalar_value ? "sv" : "v") << ";\n";
+        ss << "    }\n    drow[c * dcs] = acc;\n";
+    }
+    ss << "  }\n}\n";
+    return ss.str();
+}
+
+// dest2d: [V, D] view of the destination buffer; idx: int32 [N] buffer; values: [N, D] buffer or one element
+void run_scatter_rows(const Array& dest2d, const Array& idx, OPERATOR_T op, const Array& values) {
+    const int N = numel_of(idx.shape()), D = dest2d.shape()[1], V = dest2d.shape()[0];
+    if (N == 0 || D == 0) return;
+    const bool scalar_value = numel_of(values.shape()) == 1;
+    Array idx_c = idx.contiguous_memory() ? idx : idx.ascontiguousarray();
+    Array skeys({N}, DTYPE_INT32), perm({N}, DTYPE_INT32);
+    if (!g_dry_run) {
+        check_hip(dali_hip_argsort_i32((const int32_t*)idx_c.device_ptr(), N, V, (int32_t*)skeys.device_ptr(memory::AM_OVERWRITE),
+                                       (int32_t*)perm.device_ptr(memory::AM_OVERWRITE)),
+                  "index sort for scatter");
+        if (g_recording) {
+            note_recorded_write(skeys.expression()->memory);
+            note_recorded_write(perm.expression()->memory);
+            Array k1 = idx_c, k2 = skeys, k3 = perm;
+            const int32_t* kp = (const int32_t*)idx_c.device_ptr();
+            int32_t* sp = (int32_t*)skeys.device_ptr(memory::AM_MUTABLE);
+            int32_t* pp = (int32_t*)perm.device_ptr(memory::AM_MUTABLE);
+            g_recording->push_back([=]() {
+                (void)k1;
+                (void)k2;
+                (void)k3;
+                check_hip(dali_hip_argsort_i32(kp, N, V, sp, pp), "index sort replay");
+            });
+        }
+    }
+    auto dst = strides_of(dest2d.expression().get());
+    Program P;
+    P.arrays.push_back(manual_arg(dest2d, Cls::FULL, true, 2, dest2d.shape(), {dst[0], dst[1]}));
+    P.arrays.push_back(manual_arg(skeys, Cls::ROW, false, 1, {N}, {}));
+    P.arrays.push_back(manual_arg(perm, Cls::ROW, false, 1, {N}, {}));
+    bool vec = D % 4 == 0 && dst[1] == 1 && dst[0] % 4 == 0 && dest2d.offset() % 4 == 0;
+    if (scalar_value) {
+        P.arrays.push_back(manual_arg(values, Cls::SCAL, false, 1, {1}, {}));
+    } else {
+        auto vst = strides_of(values.expression().get());
+        P.arrays.push_back(manual_arg(values, Cls::FULL, false, 2, {N, D}, {vst[0], vst[1]}));
+        vec = vec && vst[1] == 1 && vst[0] % 4 == 0 && values.offset() % 4 == 0;
+    }
+    const int VEC = vec ? 4 : 1;
+    std::ostringstream sig;
+    sig << "scatter_rows|" << (int)dest2d.dtype() << "|" << (int)op << "|" << scalar_value << "|" << VEC;
+    static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
+    uint64_t h = kernel_hash("scatter", sig.str(), "");
+    std::shared_ptr<KernelSpec>& K = specs_cache[h];
+    std::vector<int> shape_ndims = {2};
+    IvLayout L = layout_iv(P, shape_ndims);
+    if (!K) {
+        K = std::make_shared<KernelSpec>();
+        K->hash = h;
+        K->kind = "scatter";
+        K->name = kernel_name(K->kind, h);
+        fill_plan_arrays(*K, P, shape_ndims);
+        K->plan.block_threads = 256;
+        K->plan.grid_kind = DALI_HIP_GRID_ROWS;  // one workgroup per sorted position
+        K->plan.work_begin = L.shape_pos[0];
+        K->plan.work_count = 1;
+        K->plan.work_per_block = 1;
+    }
+    std::vector<std::vector<int>> shapes = {{N, D}};
+    load_and_launch(*K, [&]() { return gen_scatter_rows_kernel(P, L, op, scalar_value, VEC, K->name); }, P, shapes);
+}
+
+// Assignment through gather_from_rows: dest[i, indices[i]] (op)= values[i]; one element per row, so no two
+// contributions meet (dali/array/op/gather_from_rows.cpp:41-51,66-78).
+std::string gen_scatter_to_rows_kernel(const Program& P, const IvLayout& L, OPERATOR_T op, bool scalar_value, const std::string& kname) {
+    std::string t = ctype(P.arrays[0].buf->dtype);
+    std::ostringstream ss;
+    ss << codegen::kDevicePrelude;
+    ss << kargs_struct(P, L);
+    ss << "extern \"C\" __global__ __launch_bounds__(256) void " << kname << "(KArgs A) {\n";
+    ss << "  const long N = A.iv[" << L.shape_pos[0] << "];\n";
+    ss << "  const long drs = A.iv[" << L.stride_pos[0] << "], dcs = A.iv[" << L.stride_pos[0] + 1 << "];\n";
+    ss << "  const long is = A.iv[" << L.stride_pos[1] << "];\n";
+    if (!scalar_value) ss << "  const long vs = A.iv[" << L.stride_pos[2] << "];\n";
+    ss << "  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < N; i += (long)gridDim.x * 256) {\n";
+    ss << "    " << t << "* d = (" << t << "*)A.p[0] + i * drs + (long)((const int*)A.p[1])[i * is] * dcs;\n";
+    ss << "    const " << t << " v = ((const " << t << "*)A.p[2])[" << (scalar_value ? "0" : "i * vs") << "];\n";
+    ss << "    *d = " << op_combine(op, "(*d)", "v") << ";\n  }\n}\n";
+    return ss.str();
+}
+
+void run_scatter_to_rows(const Array& dest2d, const Array& idx, OPERATOR_T op, const Array& values) {
+    const int N = numel_of(idx.shape());
+    if (N == 0) return;
+    const bool scalar_value = numel_of(values.shape()) == 1;
+    auto dst = strides_of(dest2d.expression().get());
+    auto ist = strides_of(idx.expression().get());
+    Program P;
+    P.arrays.push_back(manual_arg(dest2d, Cls::FULL, true, 2, dest2d.shape(), {dst[0], dst[1]}));
+    P.arrays.push_back(manual_arg(idx, Cls::ROW, false, 1, {N}, {ist.empty() ? 1 : ist[0]}));
+    if (scalar_value) {
+        P.arrays.push_back(manual_arg(values, Cls::SCAL, false, 1, {1}, {}));
+    } else {
+        auto vst = strides_of(values.expression().get());
+        P.arrays.push_back(manual_arg(values, Cls::ROW, false, 1, {N}, {vst.empty() ? 1 : vst[0]}));
+    }
+    std::ostringstream sig;
+    sig << "scatter_to_rows|" << (int)dest2d.dtype() << "|" << (int)op << "|" << scalar_value;
+    static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
+    uint64_t h = kernel_hash("scatter", sig.str(), "");
+    std::shared_ptr<KernelSpec>& K = specs_cache[h];
+    std::vector<int> shape_ndims = {1};
+    IvLayout L = layout_iv(P, shape_ndims);
+    if (!K) {
+        K = std::make_shared<KernelSpec>();
+        K->hash = h;
+        K->kind = "scatter";
+        K->name = kernel_name(K->kind, h);
+        fill_plan_arrays(*K, P, shape_ndims);
+        K->plan.block_threads = 256;
+        K->plan.grid_kind = DALI_HIP_GRID_ELEMS;
+        K->plan.work_begin = L.shape_pos[0];
+        K->plan.work_count = 1;
+        K->plan.work_per_block = 256;
+        K->plan.max_blocks = 65536;
+    }
+    std::vector<std::vector<int>> shapes = {{N}};
+    load_and_launch(*K, [&]() { return gen_scatter_to_rows_kernel(P, L, op, scalar_value, K->name); }, P, shapes);
+}
+
+// dest is a lazy gather / gather_from_rows node over a buffer: write through it
+void scatter_assign(const Array& dest, OPERATOR_T op, const Array& source) {
+    auto de = dest.expression();
+    Array target = de->args[0], idx = de->args[1];
+    DALI_ASSERT(target.is_buffer(), "assignment through a gather needs an evaluated buffer as its source (dali/array/op/gather.cpp:126-128)");
+    if (!idx.is_buffer()) idx.eval();
+    Array values = source;
+    if (values.dtype() != dest.dtype()) values = op::astype(values, dest.dtype());
+    const int64_t n_dest = numel_of(dest.shape());
+    DALI_ASSERT(numel_of(values.shape()) == 1 || numel_of(values.shape()) == n_dest,
+                make_message("Cannot assign result of shape ", shape_str(values.shape()), " to a location of shape ", shape_str(dest.shape()), "."));
+    if (values.expression()->kind == Kind::SCALAR) values = op::identity(values);  // scalars have no buffer of their own
+    values.eval();
+    DALI_ASSERT(values.is_buffer(), "internal: scatter values were not evaluated into a buffer");
+    if (de->kind == Kind::GATHER) {
+        const int N = numel_of(idx.shape()), D = target.shape()[1];
+        if (numel_of(values.shape()) != 1) values = values.reshape({N, D});
+        run_scatter_rows(target, idx, op, values);
+    } else {
+        DALI_ASSERT(target.ndim() == 2 && idx.ndim() == 1, "assignment through gather_from_rows is implemented for 2-D sources and 1-D indices");
+        if (numel_of(values.shape()) != 1) values = values.reshape({(int)n_dest});
+        run_scatter_to_rows(target, idx, op, values);
+    }
+}
+
 }  // namespace
 
 void evaluate(const std::vector<Array>& roots) {
@@ -2347,6 +2614,10 @@ void evaluate(const std::vector<Array>& roots) {
 }
 
 void evaluate_into(const Array& dest, OPERATOR_T op, const Array& source) {
+    if (!dest.is_buffer() && (dest.expression()->kind == Kind::GATHER || dest.expression()->kind == Kind::GATHER_FROM_ROWS)) {
+        scatter_assign(dest, op, source);
+        return;
+    }
     DALI_ASSERT(dest.is_buffer(), "assignment destination must be an evaluated buffer");
     jit_stats().evals++;
     jit_stats().last_kernel_kinds.clear();

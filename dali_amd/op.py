@@ -120,6 +120,12 @@ def softmax(x, axis=-1):
     return _wrap(front.dali_fe_softmax(x._h, axis), "softmax")
 
 
+def gather(source, indices):
+    """source[indices[...], ...]; assigning to the lazy result scatters into ``source``."""
+    source, indices = as_array(source), as_array(indices)
+    return _wrap(front.dali_fe_gather(source._h, indices._h), "gather")
+
+
 def gather_from_rows(source, indices):
     source, indices = as_array(source), as_array(indices)
     return _wrap(front.dali_fe_gather_from_rows(source._h, indices._h), "gather_from_rows")

@@ -60,6 +60,10 @@ dali_array_t dali_fe_mean_all(dali_array_t a);
 dali_array_t dali_fe_mean_axes(dali_array_t a, const int* axes, int naxes, int keepdims);
 dali_array_t dali_fe_softmax(dali_array_t a, int axis);
 dali_array_t dali_fe_gather_from_rows(dali_array_t source, dali_array_t indices);
+/* op::gather (dali/array/op/gather.cpp:163-171); assigning to the lazy result scatters into `source` */
+dali_array_t dali_fe_gather(dali_array_t source, dali_array_t indices);
+/* dest <<= source (dali/array/expression/assignment.cpp:92-126) */
+int dali_fe_autoreduce_assign(dali_array_t dest, dali_array_t source);
 dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_value, dali_array_t off_value);
 dali_array_t dali_fe_dot(dali_array_t a, dali_array_t b);
 

@@ -195,6 +195,18 @@ int dali_hip_sgemm_pair(int transB1, int transA1, int transB2, int transA2, int 
                         float alpha, const float* B1, int ldb1, const float* A1, int lda1, const float* B2,
                         int ldb2, const float* A2, int lda2, float beta, float* C, int ldc);
 
+/* ------------------------------------------------------------- scatter */
+/*
+ * Stable ordering of n int32 keys held in device memory: sorted_keys[p] is the p-th smallest key and
+ * perm[p] its position in `keys`; equal keys keep their input order. key_limit > 0 promises that every
+ * key lies in [0, key_limit) (fewer bits to sort); pass 0 for arbitrary keys. Runs on the library stream.
+ * It serves assignment through a gather (`dest[indices] += values`, dali/array/op/gather.cpp:89-97,
+ * 126-143): the reference's GPU code adds duplicates with atomicAdd in arrival order (gather.cpp:14-28);
+ * the generated scatter kernel instead walks each destination row's contributions in input order,
+ * the order of the reference's sequential CPU loop, so the result does not depend on scheduling.
+ */
+int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_limit, int32_t* sorted_keys, int32_t* perm);
+
 /* ---------------------------------------------------------- HIP graphs */
 
 /*

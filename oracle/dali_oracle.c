@@ -312,6 +312,46 @@ void orc_gather_from_rows(const float* source, int64_t cols, const int32_t* indi
     for (int64_t i = 0; i < n; ++i) out[i] = source[i * cols + indices[i]];
 }
 
+/* out[i, :] = source[indices[i], :] (dali/array/op/gather.cpp:49-52, 2-D form). */
+void orc_gather_rows(const float* source, int64_t cols, const int32_t* indices, int64_t n, float* out) {
+    for (int64_t i = 0; i < n; ++i)
+        for (int64_t j = 0; j < cols; ++j) out[i * cols + j] = source[(int64_t)indices[i] * cols + j];
+}
+
+/* Assignment through a gather on the CPU: the generated loop nest walks the destination view in index order
+ * and applies `dst (op)= src` element by element (dali/array/op/gather.cpp:89-97 with the non-atomic branch),
+ * so duplicates of an index are combined in input order. op: 0 =, 1 +=, 2 -=, 3 *=, 4 /=. values holds n*cols
+ * floats, or a single float when value_is_scalar. */
+void orc_scatter_rows(float* dest, int64_t cols, const int32_t* indices, int64_t n, const float* values, int value_is_scalar, int op) {
+    for (int64_t i = 0; i < n; ++i)
+        for (int64_t j = 0; j < cols; ++j) {
+            float* d = dest + (int64_t)indices[i] * cols + j;
+            const float v = value_is_scalar ? values[0] : values[i * cols + j];
+            switch (op) {
+                case 0: *d = v; break;
+                case 1: *d += v; break;
+                case 2: *d -= v; break;
+                case 3: *d *= v; break;
+                default: *d /= v; break;
+            }
+        }
+}
+
+/* dest[i, indices[i]] (op)= values[i] (dali/array/op/gather_from_rows.cpp:41-51,66-78). */
+void orc_scatter_to_rows(float* dest, int64_t cols, const int32_t* indices, int64_t n, const float* values, int value_is_scalar, int op) {
+    for (int64_t i = 0; i < n; ++i) {
+        float* d = dest + i * cols + indices[i];
+        const float v = value_is_scalar ? values[0] : values[i];
+        switch (op) {
+            case 0: *d = v; break;
+            case 1: *d += v; break;
+            case 2: *d -= v; break;
+            case 3: *d *= v; break;
+            default: *d /= v; break;
+        }
+    }
+}
+
 /* is_on = (indices[i] == j); on*is_on + (1.0 - is_on)*off, evaluated with T = float
  * for is_on and the 1.0 in double (dali/array/op/one_hot.cpp:38-46). */
 void orc_one_hot(const int32_t* indices, int64_t n, int depth, float on, float off, float* out) {

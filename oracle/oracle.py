@@ -47,6 +47,9 @@ def _load():
     lib.orc_mean_all.restype = C.c_float
     lib.orc_softmax.argtypes = [_f, _f, _i64, _i64]
     lib.orc_gather_from_rows.argtypes = [_f, _i64, _i32, _i64, _f]
+    lib.orc_gather_rows.argtypes = [_f, _i64, _i32, _i64, _f]
+    lib.orc_scatter_rows.argtypes = [_f, _i64, _i32, _i64, _f, C.c_int, C.c_int]
+    lib.orc_scatter_to_rows.argtypes = [_f, _i64, _i32, _i64, _f, C.c_int, C.c_int]
     lib.orc_one_hot.argtypes = [_i32, _i64, C.c_int, C.c_float, C.c_float, _f]
     lib.orc_softmax_cross_entropy.argtypes = [_f, _i32, _i64, _i64, _f, _f, _f]
     lib.orc_softmax_cross_entropy_via_probs.argtypes = [_f, _i32, _i64, _i64, _f]
@@ -209,6 +212,34 @@ def softmax_cross_entropy_via_probs(x, t):
     out = np.empty(x.shape[0], dtype=np.float32)
     lib.orc_softmax_cross_entropy_via_probs(fp(x), ip(t), x.shape[0], x.shape[1], fp(out))
     return out
+
+
+def gather_rows(source, indices):
+    source = _c32(source)
+    idx = np.ascontiguousarray(indices, dtype=np.int32).ravel()
+    cols = source.shape[1]
+    out = np.empty((idx.size, cols), dtype=np.float32)
+    lib.orc_gather_rows(fp(source), cols, ip(idx), idx.size, fp(out))
+    return out
+
+
+def scatter_rows(dest, indices, values, op=1):
+    """dest[indices[i], :] (op)= values[i, :] in input order; returns the updated copy of ``dest``."""
+    dest = _c32(dest).copy()
+    idx = np.ascontiguousarray(indices, dtype=np.int32).ravel()
+    vals = _c32(np.asarray(values, dtype=np.float32))
+    scalar = vals.size == 1
+    lib.orc_scatter_rows(fp(dest), dest.shape[1], ip(idx), idx.size, fp(vals), 1 if scalar else 0, op)
+    return dest
+
+
+def scatter_to_rows(dest, indices, values, op=1):
+    dest = _c32(dest).copy()
+    idx = np.ascontiguousarray(indices, dtype=np.int32).ravel()
+    vals = _c32(np.asarray(values, dtype=np.float32))
+    scalar = vals.size == 1
+    lib.orc_scatter_to_rows(fp(dest), dest.shape[1], ip(idx), idx.size, fp(vals), 1 if scalar else 0, op)
+    return dest
 
 
 def _strides(a):

@@ -172,3 +172,19 @@ def test_planner_splits_what_cannot_fuse(D, rng):
     assert D.last_kernel_kinds() == "generic,row"  # middle axis: strided copy, then a trailing-axis reduction
     D.generate_only([op.mean(m)], compile=True)
     assert D.last_kernel_kinds() == "all"  # the division by the count is folded into the last block
+
+
+def test_gather_plans_as_an_indirect_row_leaf_and_checks_its_arguments(D, rng):
+    table = D.Array.from_numpy(rng.randn(100, 64).astype(np.float32))
+    idx = D.Array.from_numpy(np.arange(10, dtype=np.int32))
+    g = D.op.gather(table, idx)
+    assert g.shape == (10, 64) and not g.is_buffer()
+    assert D.generate_only([D.op.tanh(g) * 2.0], compile=True) == 1  # one kernel: the map reads through the gather
+    src = D.last_source()
+    assert "(long)rl" in src  # the source row pointer goes through the per-row index value
+    assert D.op.gather(table, D.Array.from_numpy(np.zeros((2, 3), np.int32))).shape == (2, 3, 64)
+    with pytest.raises(RuntimeError, match="indices must be integers"):
+        D.op.gather(table, D.Array.from_numpy(np.zeros(3, np.float32)))
+    with pytest.raises(RuntimeError, match="same dimensionality"):
+        t = D.Array.zeros((3,))
+        t <<= D.Array.from_numpy(np.ones((3, 4), np.float32))

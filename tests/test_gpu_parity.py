@@ -545,3 +545,140 @@ def test_cabi_graph_capture_of_gemm(gpu, D, rng):
         assert hip.dali_hip_graph_destroy(graph) == 0
         for p in ptrs:
             assert hip.dali_hip_free(p) == 0
+
+
+# ---------------------------------------------------------------- gather / scatter / <<=
+def test_gather_reference_cases(gpu, D, O, rng):
+    # GatherTests.gather_simple / gather_simple_elementwise (tests.cpp:1266-1281)
+    idx = arr(D, np.arange(5, dtype=np.int32))
+    src = np.arange(30, dtype=np.float32).reshape(5, 6)
+    assert np.array_equal(D.op.gather(arr(D, src), idx).numpy(), src)
+    src3 = np.arange(5 * 6 * 7, dtype=np.float32).reshape(5, 6, 7)
+    g3 = D.op.gather(arr(D, src3), idx)
+    assert g3.shape == (5, 6, 7) and np.array_equal(g3.numpy(), src3)
+    before = D.jit_stats()
+    fused = D.op.sigmoid(D.op.gather(arr(D, src), idx))
+    close(fused.numpy(), 1.0 / (1.0 + np.exp(-src.astype(np.float64))), rtol=1e-6, atol=1e-7)
+    assert D.jit_stats()["kernels"] - before["kernels"] == 1  # the elementwise map reads through the gather
+
+
+@pytest.mark.parametrize("V,Dm,N", [(7, 1, 20), (50, 33, 64), (1000, 256, 777), (32000, 1024, 4096)])
+def test_gather_matches_oracle(gpu, D, O, rng, V, Dm, N):
+    src = rng.randn(V, Dm).astype(np.float32)
+    idx = rng.randint(0, V, N).astype(np.int32)
+    assert np.array_equal(D.op.gather(arr(D, src), arr(D, idx)).numpy(), O.gather_rows(src, idx))
+    # indices of any rank, 1-D sources, strided sources
+    idx2 = idx[: (N // 4) * 4].reshape(4, -1)
+    got = D.op.gather(arr(D, src), arr(D, idx2)).numpy()
+    assert got.shape == idx2.shape + (Dm,) and np.array_equal(got, src[idx2])
+    assert np.array_equal(arr(D, src[:, 0].copy())[arr(D, idx)].numpy(), src[idx, 0])
+    if Dm >= 8:
+        view = arr(D, src)[:, 4:8]
+        assert np.array_equal(D.op.gather(view, arr(D, idx)).numpy(), src[idx, 4:8])
+
+
+def test_scatter_reference_cases(gpu, D):
+    # GatherTests.scatter_simple (tests.cpp:1316-1331)
+    idx = arr(D, np.array([0, 0, 1, 1, 1, 2], np.int32))
+    dest = D.Array.zeros((3,), D.DTYPE_INT32)
+    gathered = dest[idx]
+    assert gathered.shape == (6,)
+    gathered += 1
+    assert not gathered.is_buffer()
+    assert dest.numpy().tolist() == [2, 3, 1]
+    # GatherTests.scatter_to_rows_simple (tests.cpp:1333-1361)
+    dest2 = arr(D, np.full((7, 3), 42, np.int32))
+    g2 = dest2.gather_from_rows(idx)
+    assert g2.shape == (6,)
+    g2 += 1
+    assert not g2.is_buffer()
+    want = np.full((7, 3), 42, np.int32)
+    want[np.arange(6), [0, 0, 1, 1, 1, 2]] += 1
+    assert np.array_equal(dest2.numpy(), want)
+
+
+@pytest.mark.parametrize("V,Dm,N", [(5, 1, 200), (64, 33, 300), (1000, 256, 5000), (32000, 1024, 8192)])
+@pytest.mark.parametrize("operator_t", [1, 2, 0])
+def test_scatter_rows_is_the_sequential_loop_bit_for_bit(gpu, D, O, rng, V, Dm, N, operator_t):
+    dest = rng.randn(V, Dm).astype(np.float32)
+    idx = rng.randint(0, V, N).astype(np.int32)
+    idx[: N // 3] = idx[0]  # one heavily repeated row
+    rng.shuffle(idx)
+    vals = (rng.randn(N, Dm) * 10).astype(np.float32)
+    d = arr(D, dest)
+    d[arr(D, idx)].assign(arr(D, vals), operator_t)
+    # duplicates are combined in input order, as in the reference's CPU loop: exact equality
+    assert np.array_equal(d.numpy(), O.scatter_rows(dest, idx, vals, op=operator_t))
+    # scalar right-hand side
+    d2 = arr(D, dest)
+    g = d2[arr(D, idx)]
+    g += 0.5
+    assert np.array_equal(d2.numpy(), O.scatter_rows(dest, idx, np.float32(0.5), op=1))
+
+
+@pytest.mark.parametrize("R,Cn", [(6, 3), (300, 1000), (8192, 32000)])
+def test_scatter_to_rows_matches_oracle(gpu, D, O, rng, R, Cn):
+    dest = rng.randn(R, Cn).astype(np.float32)
+    idx = rng.randint(0, Cn, R).astype(np.int32)
+    vals = rng.randn(R).astype(np.float32)
+    d = arr(D, dest)
+    g = d.gather_from_rows(arr(D, idx))
+    g -= arr(D, vals)
+    assert np.array_equal(d.numpy(), O.scatter_to_rows(dest, idx, vals, op=2))
+    g -= 1.0  # the backward step of the cross-entropy: dx[i, t_i] -= dout (cost.cpp:127-129)
+    assert np.array_equal(d.numpy(), O.scatter_to_rows(O.scatter_to_rows(dest, idx, vals, op=2), idx, np.float32(1.0), op=2))
+
+
+def test_autoreduce_assign_reference_cases(gpu, D, rng):
+    # ArrayTests.lse_and_addition, lse, broadcasted_lse, broadcasted_lse2, ReducerTests.lse_reduce (tests.cpp:803-851,1241-1247)
+    i32 = D.DTYPE_INT32
+    t = D.Array.zeros((3, 4), i32)
+    t <<= arr(D, np.ones((3, 4), np.int32)) + arr(D, np.ones((3, 4), np.int32))
+    assert np.array_equal(t.numpy(), np.full((3, 4), 2))
+    t = D.Array.zeros((3, 4), i32)
+    t <<= arr(D, np.arange(12, dtype=np.int32).reshape(3, 4))
+    assert t.numpy().ravel().tolist() == list(range(12))
+    base = D.Array.zeros((3,), i32)
+    t = base[:, None]
+    t <<= arr(D, np.ones((3, 4), np.int32))
+    assert base.numpy().tolist() == [4, 4, 4]
+    base = D.Array.zeros((4,), i32)
+    t = base[None, :]
+    t <<= arr(D, np.ones((3, 4), np.int32))
+    assert base.numpy().tolist() == [3, 3, 3, 3]
+    a = D.Array.zeros((2,), i32).expand_dims(1)
+    a <<= arr(D, np.ones((2, 5), np.int32))
+    assert a.numpy().tolist() == [[5], [5]]
+    # fp32, both axes at once, accumulating on top of existing contents
+    x = rng.randn(37, 53).astype(np.float32)
+    acc = arr(D, np.full((1, 1), 2.0, np.float32))
+    acc <<= arr(D, x)
+    close(acc.numpy(), 2.0 + x.astype(np.float64).sum(), rtol=1e-5, atol=1e-5 * np.abs(x).sum())
+    with pytest.raises(RuntimeError):
+        t = D.Array.zeros((3, 2), i32)
+        t <<= arr(D, np.ones((3, 4), np.int32))
+
+
+@pytest.mark.parametrize("n", [1, 7, 1000, 1024, 1025, 5000, 8192, 8193, 100000])
+def test_cabi_argsort_is_stable(gpu, rng, n):
+    hip = gpu
+    keys = rng.randint(-50, 50, n).astype(np.int32)
+    keys[rng.randint(0, n, max(1, n // 10))] = np.iinfo(np.int32).max  # collides with the padding value of the block sort
+    keys[rng.randint(0, n, max(1, n // 10))] = np.iinfo(np.int32).min
+    dk = _dev(hip, keys)
+    ds, dp = _dev(hip, np.zeros(n, np.int32)), _dev(hip, np.zeros(n, np.int32))
+    sk, pm = np.empty(n, np.int32), np.empty(n, np.int32)
+
+    def check(keys, limit):
+        hip.dali_hip_memcpy_h2d(dk, keys.ctypes.data_as(C.c_void_p), n * 4)
+        assert hip.dali_hip_argsort_i32(dk, n, limit, ds, dp) == 0, hip.dali_hip_last_error()
+        hip.dali_hip_memcpy_d2h(sk.ctypes.data_as(C.c_void_p), ds, n * 4)
+        hip.dali_hip_memcpy_d2h(pm.ctypes.data_as(C.c_void_p), dp, n * 4)
+        order = np.argsort(keys, kind="stable")
+        assert np.array_equal(pm, order) and np.array_equal(sk, keys[order])
+
+    check(keys, 0)
+    for limit in (1, 2, 1000, 32000, 32768):  # bounded keys: only the low bits are sorted
+        check(rng.randint(0, limit, n).astype(np.int32), limit)
+    for p in (dk, ds, dp):
+        hip.dali_hip_free(p)

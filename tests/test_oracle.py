@@ -347,3 +347,50 @@ def test_lstm_step_composition(O, rng):
     np.testing.assert_allclose(h_new, o * np.tanh(c), rtol=1e-5, atol=2e-6)
     # gate order matters: swapping o and g changes the answer
     assert np.max(np.abs(h_new - sig(G[:, 3 * H:]) * np.tanh(c))) > 1e-2
+
+
+# ---------------------------------------------------------------- gather / scatter
+def test_gather_rows_is_fancy_indexing(O, rng):
+    src = rng.randn(11, 7).astype(np.float32)
+    idx = rng.randint(0, 11, 23).astype(np.int32)
+    assert np.array_equal(O.gather_rows(src, idx), src[idx])
+    # reference_gather of tests.cpp:1251-1272: arange source, arange indices reproduce the source
+    a = np.arange(30, dtype=np.float32).reshape(5, 6)
+    assert np.array_equal(O.gather_rows(a, np.arange(5)), a)
+
+
+def test_scatter_rows_reference_known_answers_and_duplicates(O, rng):
+    # GatherTests.scatter_simple (tests.cpp:1316-1331): dest[{0,0,1,1,1,2}] += 1 on zeros(3) -> 2, 3, 1
+    out = O.scatter_rows(np.zeros((3, 1), np.float32), [0, 0, 1, 1, 1, 2], 1.0, op=1)
+    assert out.ravel().tolist() == [2.0, 3.0, 1.0]
+    # integer-valued data: any order gives the same sums, numpy's unbuffered add is the library answer
+    dest = rng.randint(-5, 5, (9, 4)).astype(np.float32)
+    idx = rng.randint(0, 9, 40).astype(np.int32)
+    vals = rng.randint(-3, 3, (40, 4)).astype(np.float32)
+    want = dest.copy()
+    np.add.at(want, idx, vals)
+    assert np.array_equal(O.scatter_rows(dest, idx, vals, op=1), want)
+    want = dest.copy()
+    np.subtract.at(want, idx, vals)
+    assert np.array_equal(O.scatter_rows(dest, idx, vals, op=2), want)
+    # plain assignment: the last writer in input order wins
+    got = O.scatter_rows(dest, idx, vals, op=0)
+    for r in range(9):
+        hits = np.nonzero(idx == r)[0]
+        assert np.array_equal(got[r], vals[hits[-1]] if hits.size else dest[r])
+    # fp32 with duplicates: input-order accumulation, restated as an explicit python loop on one column
+    d1 = rng.randn(5, 1).astype(np.float32)
+    i1 = rng.randint(0, 5, 200).astype(np.int32)
+    v1 = (rng.randn(200, 1) * 1e3).astype(np.float32)
+    acc = d1.copy()
+    for i in range(200):
+        acc[i1[i], 0] = np.float32(acc[i1[i], 0] + v1[i, 0])
+    assert np.array_equal(O.scatter_rows(d1, i1, v1, op=1), acc)
+
+
+def test_scatter_to_rows_reference_known_answer(O):
+    # GatherTests.scatter_to_rows_simple (tests.cpp:1333-1361): 42 everywhere, +1 at (i, vals[i])
+    vals = [0, 0, 1, 1, 1, 2]
+    out = O.scatter_to_rows(np.full((7, 3), 42, np.float32)[:6], vals, 1.0, op=1)
+    for i, v in enumerate(vals):
+        assert out[i].tolist() == [43.0 if j == v else 42.0 for j in range(3)]
