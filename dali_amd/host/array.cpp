@@ -585,6 +585,31 @@ Array isnan(const Array& x) { return elementwise(x, "functor::isnotanumber"); }
 Array isinf(const Array& x) { return elementwise(x, "functor::isinfinity"); }
 Array dsigmoid(const Array& x) { return elementwise(x, "functor::dsigmoid"); }
 Array dtanh(const Array& x) { return elementwise(x, "functor::dtanh"); }
+// the rest of dali/array/op/unary.cpp and binary.cpp: thin names over the functors
+Array softplus_backward(const Array& x) { return elementwise(x, "functor::softplus_backward"); }
+Array relu_backward(const Array& x) { return elementwise(x, "functor::relu_backward"); }
+Array log_or_zero(const Array& x) { return elementwise(x, "functor::log_or_zero"); }
+Array inverse_tanh(const Array& x) { return elementwise(x, "functor::inverse_tanh"); }
+Array clipped_relu(const Array& x, const Array& upper_bound) { return elementwise(x, upper_bound, "functor::clipped_relu"); }
+Array clipped_relu_backward(const Array& x, const Array& upper_bound) { return elementwise(x, upper_bound, "functor::clipped_relu_backward"); }
+Array steep_sigmoid(const Array& x, const Array& aggressiveness) { return elementwise(x, aggressiveness, "functor::steep_sigmoid"); }
+Array steep_sigmoid_backward(const Array& x, const Array& aggressiveness) { return elementwise(x, aggressiveness, "functor::steep_sigmoid_backward"); }
+Array prelu_backward_weights(const Array& a, const Array& grad) { return elementwise(a, grad, "functor::prelu_backward_weights"); }
+Array prelu_backward_inputs(const Array& a, const Array& weights) { return elementwise(a, weights, "functor::prelu_backward_inputs"); }
+Array lessthanequal(const Array& a, const Array& b) { return elementwise(a, b, "functor::lessthanequal"); }
+Array greaterthanequal(const Array& a, const Array& b) { return elementwise(a, b, "functor::greaterthanequal"); }
+Array maximum(const Array& a, const Array& b) { return elementwise(a, b, "functor::max_scalar"); }
+Array minimum(const Array& a, const Array& b) { return elementwise(a, b, "functor::min_scalar"); }
+Array binary_cross_entropy(const Array& a, const Array& b) { return elementwise(a, b, "functor::binary_cross_entropy"); }
+Array binary_cross_entropy_grad(const Array& a, const Array& b) { return elementwise(a, b, "functor::binary_cross_entropy_grad"); }
+Array close(const Array& left, const Array& right, const Array& atolerance) { return lessthanequal(abs(subtract(left, right)), atolerance); }
+// dali/array/op/binary.cpp:9-11,45-60 (sum of many arrays as one fused chain)
+Array add(const std::vector<Array>& arrays) {
+    DALI_ASSERT(!arrays.empty(), "add must have at least one Array to add but got 0.");
+    Array out = arrays[0];
+    for (size_t i = 1; i < arrays.size(); ++i) out = add(out, arrays[i]);
+    return out;
+}
 
 Array all_reduce(const Array& a, const std::string& reducer_name) {
     return make_node(Kind::ALL_REDUCE, reducer_name, {a}, {}, a.dtype());
@@ -715,6 +740,13 @@ Array argmax(const Array& x) { return argument_all_reduce(x, "reducers::maximum"
 Array argmax(const Array& x, int axis) { return argument_axis_reduce(x, "reducers::maximum", axis); }
 Array argmin(const Array& x) { return argument_all_reduce(x, "reducers::minimum"); }
 Array argmin(const Array& x, int axis) { return argument_axis_reduce(x, "reducers::minimum", axis); }
+// dali/array/op/reducers.cpp:61-72, binary.cpp:7-12
+Array any_isnan(const Array& x) { return max(isnan(x)); }
+Array any_isinf(const Array& x) { return max(isinf(x)); }
+Array any_isnan(const Array& x, const std::vector<int>& axes, bool keepdims) { return max(isnan(x), axes, keepdims); }
+Array any_isinf(const Array& x, const std::vector<int>& axes, bool keepdims) { return max(isinf(x), axes, keepdims); }
+Array all_equals(const Array& left, const Array& right) { return prod(equals(left, right)); }
+Array all_close(const Array& left, const Array& right, const Array& atolerance) { return prod(close(left, right, atolerance)); }
 
 // dali/array/op/softmax.cpp:5-8
 Array softmax(const Array& logits, int axis) {

@@ -197,6 +197,24 @@ Array isnan(const Array& x);
 Array isinf(const Array& x);
 Array dsigmoid(const Array& x);
 Array dtanh(const Array& x);
+Array softplus_backward(const Array& x);
+Array relu_backward(const Array& x);
+Array log_or_zero(const Array& x);
+Array inverse_tanh(const Array& x);
+Array clipped_relu(const Array& x, const Array& upper_bound);
+Array clipped_relu_backward(const Array& x, const Array& upper_bound);
+Array steep_sigmoid(const Array& x, const Array& aggressiveness);
+Array steep_sigmoid_backward(const Array& x, const Array& aggressiveness);
+Array prelu_backward_weights(const Array& a, const Array& grad);
+Array prelu_backward_inputs(const Array& a, const Array& weights);
+Array lessthanequal(const Array& a, const Array& b);
+Array greaterthanequal(const Array& a, const Array& b);
+Array maximum(const Array& a, const Array& b);
+Array minimum(const Array& a, const Array& b);
+Array binary_cross_entropy(const Array& a, const Array& b);
+Array binary_cross_entropy_grad(const Array& a, const Array& b);
+Array close(const Array& left, const Array& right, const Array& atolerance);
+Array add(const std::vector<Array>& arrays);
 
 // dali/array/op/reducers.h, reducer_operation.h
 Array all_reduce(const Array& a, const std::string& reducer_name);
@@ -219,6 +237,12 @@ Array argmax(const Array& x);
 Array argmax(const Array& x, int axis);
 Array argmin(const Array& x);
 Array argmin(const Array& x, int axis);
+Array any_isnan(const Array& x);
+Array any_isinf(const Array& x);
+Array any_isnan(const Array& x, const std::vector<int>& axes, bool keepdims = false);
+Array any_isinf(const Array& x, const std::vector<int>& axes, bool keepdims = false);
+Array all_equals(const Array& left, const Array& right);
+Array all_close(const Array& left, const Array& right, const Array& atolerance);
 
 // dali/array/op/softmax.h, gather_from_rows.h, one_hot.h, dot.h
 Array softmax(const Array& logits, int axis = -1);

@@ -85,6 +85,7 @@ template <typename R> struct rsqrt    { DI static R Map(R a) { return (R)(1.0 / 
 template <typename R> struct inv      { DI static R Map(R a) { return ((R)1.0) / a; } };
 template <typename R> struct cast     { template <typename O> DI static R Map(O a) { return R(a); } };
 template <typename R> struct round    { template <typename O> DI static R Map(O a) { return (R)floor((double)a + 0.5); } };
+template <typename R> struct ceil     { template <typename O> DI static R Map(O a) { return (R)::ceil((double)a); } };
 template <typename R> struct sigmoid  { DI static R Map(R a) { return (R)(1.0 / (1.0 + (double)m_exp(-a))); } };
 template <typename R> struct identity { DI static R Map(R a) { return a; } };
 template <typename R> struct log      { DI static R Map(R a) { return (R)m_log(a); } };

@@ -46,6 +46,10 @@ isnan = _unary("isnotanumber")
 isinf = _unary("isinfinity")
 dsigmoid = _unary("dsigmoid")
 dtanh = _unary("dtanh")
+softplus_backward = _unary("softplus_backward")
+relu_backward = _unary("relu_backward")
+log_or_zero = _unary("log_or_zero")
+inverse_tanh = _unary("inverse_tanh")
 # dali/array/op/binary.h
 add = _binary("add")
 subtract = _binary("subtract")
@@ -55,6 +59,23 @@ pow = _binary("power")
 equals = _binary("equals")
 prelu = _binary("prelu")
 clip = _binary("clip")
+clipped_relu = _binary("clipped_relu")
+clipped_relu_backward = _binary("clipped_relu_backward")
+steep_sigmoid = _binary("steep_sigmoid")
+steep_sigmoid_backward = _binary("steep_sigmoid_backward")
+prelu_backward_weights = _binary("prelu_backward_weights")
+prelu_backward_inputs = _binary("prelu_backward_inputs")
+lessthanequal = _binary("lessthanequal")
+greaterthanequal = _binary("greaterthanequal")
+maximum = _binary("max_scalar")
+minimum = _binary("min_scalar")
+binary_cross_entropy = _binary("binary_cross_entropy")
+binary_cross_entropy_grad = _binary("binary_cross_entropy_grad")
+
+
+def close(left, right, atolerance):
+    """|left - right| <= atolerance, elementwise (dali/array/op/binary.cpp:16-18)."""
+    return lessthanequal(abs(subtract(left, right)), atolerance)
 
 
 def astype(a, dtype):
@@ -157,3 +178,20 @@ def lstm_step(x, h, c, W, U, b):
     if front.dali_fe_lstm_step(*[k._h for k in keep], *[C.byref(o) for o in outs]) != 0:
         raise fe_error("lstm_step")
     return tuple(Array(o.value) for o in outs)
+
+
+# dali/array/op/reducers.cpp:61-72, binary.cpp:7-12
+def any_isnan(x, axes=None, keepdims=False):
+    return max(isnan(x), axes, keepdims)
+
+
+def any_isinf(x, axes=None, keepdims=False):
+    return max(isinf(x), axes, keepdims)
+
+
+def all_equals(left, right):
+    return prod(equals(left, right))
+
+
+def all_close(left, right, atolerance):
+    return prod(close(left, right, atolerance))

@@ -682,3 +682,23 @@ def test_cabi_argsort_is_stable(gpu, rng, n):
         check(rng.randint(0, limit, n).astype(np.int32), limit)
     for p in (dk, ds, dp):
         hip.dali_hip_free(p)
+
+
+def test_named_comparison_and_any_all_helpers(gpu, D, rng):
+    # ArrayTests/BinaryTests of the reference use these through Array::equals / allclose (binary.cpp:7-18, reducers.cpp:61-72)
+    op = D.op
+    a = rng.randn(33, 17).astype(np.float32)
+    b = a.copy()
+    b[5, 3] += 1e-3
+    A, B = arr(D, a), arr(D, b)
+    assert float(op.all_equals(A, arr(D, a.copy())).numpy()) == 1.0 and float(op.all_equals(A, B).numpy()) == 0.0
+    assert float(op.all_close(A, B, 1e-2).numpy()) == 1.0 and float(op.all_close(A, B, 1e-4).numpy()) == 0.0
+    assert np.array_equal(op.maximum(A, B).numpy(), np.maximum(a, b)) and np.array_equal(op.minimum(A, B).numpy(), np.minimum(a, b))
+    assert np.array_equal(op.lessthanequal(A, B).numpy(), (a <= b).astype(np.float32))
+    assert np.array_equal(op.greaterthanequal(A, B).numpy(), (a >= b).astype(np.float32))
+    c = a.copy()
+    assert float(op.any_isnan(arr(D, c)).numpy()) == 0.0 and float(op.any_isinf(arr(D, c)).numpy()) == 0.0
+    c[7, 7] = np.nan
+    c[9, 2] = np.inf
+    assert float(op.any_isnan(arr(D, c)).numpy()) == 1.0 and float(op.any_isinf(arr(D, c)).numpy()) == 1.0
+    assert op.any_isnan(arr(D, c), [1]).numpy().tolist() == [1.0 if r == 7 else 0.0 for r in range(33)]
