@@ -575,7 +575,8 @@ struct BodyEmitter {
             if (declared.count(id)) return var;
             declared.insert(id);
             if ((*first_body)[id] == body_index) {
-                stmts << "const " << ctype(n.dtype) << " " << var << " = " << raw(id) << "; t" << id << "[e][j] = " << var << ";\n";
+                const std::string r = raw(id);  // may itself append statements (nested kept or shared nodes): before ours
+                stmts << "const " << ctype(n.dtype) << " " << var << " = " << r << "; t" << id << "[e][j] = " << var << ";\n";
             } else {
                 stmts << "const " << ctype(n.dtype) << " " << var << " = t" << id << "[e][j];\n";
             }

@@ -1,0 +1,207 @@
+"""Seeded random expression trees through the planner, checked against numpy in float64.
+
+The trees mix the node classes of the fused path (elementwise maps, keepdims and plain axis reductions, full
+reductions, broadcasts of row / column vectors and scalars, strided views) over ragged shapes, so that every kernel
+shape and most of the planner's splitting rules are visited. Operations are chosen to be well conditioned (positive
+summands, bounded arguments), so a relative tolerance of 1e-5 plus the summation bound is meaningful.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def arr(D, x):
+    return D.Array.from_numpy(np.ascontiguousarray(x))
+
+
+UNARY = [
+    ("sigmoid", lambda v: 1.0 / (1.0 + np.exp(-v))),
+    ("tanh", np.tanh),
+    ("abs", np.abs),
+    ("square", lambda v: v * v),
+    ("softplus", lambda v: np.where(v > 20.0, v, np.log1p(np.exp(np.minimum(v, 20.0))))),
+    ("relu", lambda v: np.maximum(v, 0.0)),
+]
+
+
+class Gen(object):
+    def __init__(self, D, rng, shape):
+        self.D, self.rng, self.shape = D, rng, shape
+        self.size_terms = 0  # number of summed terms feeding the result (for the tolerance)
+
+    def leaf(self, shape):
+        kind = self.rng.randint(0, 5)
+        x = self.rng.uniform(-2.0, 2.0, shape).astype(np.float32)
+        if kind == 0 and len(shape) == 2 and shape[1] > 1:
+            # strided view: every other column of a wider buffer
+            wide = self.rng.uniform(-2.0, 2.0, (shape[0], 2 * shape[1])).astype(np.float32)
+            return arr(self.D, wide)[:, ::2], wide[:, ::2].astype(np.float64)
+        if kind == 1 and len(shape) == 2:
+            # transposed storage
+            xt = np.ascontiguousarray(x.T)
+            return arr(self.D, xt).T, x.astype(np.float64)
+        return arr(self.D, x), x.astype(np.float64)
+
+    def full(self, depth):
+        """An expression of the generator's full shape."""
+        D, rng, op = self.D, self.rng, self.D.op
+        if depth == 0:
+            return self.leaf(self.shape)
+        choice = rng.randint(0, 7)
+        if choice <= 1:
+            name, f = UNARY[rng.randint(len(UNARY))]
+            a, ra = self.full(depth - 1)
+            return op.elementwise(name, a), f(ra)
+        if choice == 2:
+            a, ra = self.full(depth - 1)
+            b, rb = self.full(depth - 1)
+            if rng.randint(2):
+                return a + op.abs(b), ra + np.abs(rb)
+            return a * b, ra * rb
+        if choice == 3:
+            # broadcast of a row-wise (keepdims) reduction back onto the rows
+            a, ra = self.full(depth - 1)
+            axis = len(self.shape) - 1
+            if rng.randint(2):
+                return a - op.max(a, [axis], True), ra - ra.max(axis=axis, keepdims=True)
+            self.size_terms = max(self.size_terms, self.shape[axis])
+            pos, rpos = op.abs(a) + 0.5, np.abs(ra) + 0.5
+            return pos / op.sum(pos, [axis], True), rpos / rpos.sum(axis=axis, keepdims=True)
+        if choice == 4 and len(self.shape) == 2:
+            # column vector [1, C] and row vector [R, 1] operands
+            a, ra = self.full(depth - 1)
+            cv = rng.uniform(0.5, 1.5, (1, self.shape[1])).astype(np.float32)
+            rv = rng.uniform(0.5, 1.5, (self.shape[0], 1)).astype(np.float32)
+            return a * arr(D, cv) + arr(D, rv), ra * cv.astype(np.float64) + rv.astype(np.float64)
+        if choice == 5:
+            a, ra = self.full(depth - 1)
+            s = float(rng.uniform(0.5, 2.0))
+            return a * s + 0.25, ra * np.float64(np.float32(s)) + 0.25
+        a, ra = self.full(depth - 1)
+        # a full reduction used as a scalar
+        self.size_terms = max(self.size_terms, int(np.prod(self.shape)))
+        pos, rpos = op.abs(a) + 0.5, np.abs(ra) + 0.5
+        return pos / op.sum(pos), rpos / rpos.sum()
+
+    def root(self, depth):
+        """Either a full-shape expression or a reduction of one."""
+        D, rng, op = self.D, self.rng, self.D.op
+        a, ra = self.full(depth)
+        kind = rng.randint(0, 6)
+        nd = len(self.shape)
+        if kind == 0:
+            return a, ra
+        if kind == 1:
+            axis = rng.randint(nd)
+            self.size_terms = max(self.size_terms, self.shape[axis])
+            return op.sum(op.abs(a), [axis]), np.abs(ra).sum(axis=axis)
+        if kind == 2:
+            axis = rng.randint(nd)
+            return op.max(a, [axis]), ra.max(axis=axis)
+        if kind == 3:
+            self.size_terms = max(self.size_terms, int(np.prod(self.shape)))
+            return op.mean(op.abs(a)), np.abs(ra).mean()
+        if kind == 4:
+            return op.min(a), ra.min()
+        axis = rng.randint(nd)
+        return op.max(a, [axis], True) - op.min(a, [axis], True), ra.max(axis=axis, keepdims=True) - ra.min(axis=axis, keepdims=True)
+
+
+SHAPES = [(1, 1), (3, 5), (17, 64), (64, 17), (129, 1000), (5, 4096), (300, 301), (2, 3, 50), (7,), (1025,), (4, 8, 16)]
+
+
+@pytest.mark.parametrize("seed", range(150))
+def test_random_expression_matches_numpy(gpu, D, seed):
+    rng = np.random.RandomState(1000 + seed)
+    shape = SHAPES[seed % len(SHAPES)]
+    g = Gen(D, rng, shape)
+    expr, want = g.root(depth=1 + seed % 3)
+    got = expr.numpy().astype(np.float64)
+    want = np.asarray(want, np.float64)
+    if len(shape) == 1 and want.shape == (1,):
+        # a keepdims reduction over every axis is the plain full reduction, shape {} (reducer_operation.cpp:627-630)
+        want = want.reshape(())
+    assert got.shape == want.shape, (got.shape, want.shape, D.last_kernel_kinds())
+    tol = 2e-5 + max(g.size_terms - 1, 0) * 2.0 ** -24
+    err = np.abs(got - want)
+    bound = tol * np.maximum(np.abs(want), 1e-3) + 1e-6
+    assert (err <= bound).all(), "seed %d shape %s kinds %s: max err %g at %s (want %g)" % (
+        seed, shape, D.last_kernel_kinds(), err.max(), np.unravel_index(err.argmax(), err.shape), want.flat[err.argmax()])
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_assignment_into_views(gpu, D, seed):
+    """dst (op)= expression with dst a whole buffer, a row/column slice or a transposed view."""
+    rng = np.random.RandomState(5000 + seed)
+    R, Cn = [(4, 6), (33, 65), (128, 257), (300, 1000)][seed % 4]
+    base = rng.uniform(1.0, 2.0, (R, Cn)).astype(np.float32)
+    d = arr(D, base)
+    want = base.astype(np.float64)
+    view_kind = rng.randint(0, 4)
+    if view_kind == 0:
+        dv, wv = d, want
+    elif view_kind == 1:
+        r0, r1 = sorted(rng.choice(R + 1, 2, replace=False))
+        dv, wv = d[int(r0):int(r1)], want[r0:r1]
+    elif view_kind == 2:
+        c0, c1 = sorted(rng.choice(Cn + 1, 2, replace=False))
+        dv, wv = d[:, int(c0):int(c1)], want[:, c0:c1]
+    else:
+        dv, wv = d.T, want.T
+    g = Gen(D, rng, wv.shape)
+    if wv.size == 0:
+        return
+    expr, ref = g.full(depth=1 + seed % 2)
+    operator_t = int(rng.randint(0, 5))
+    if operator_t == 4:
+        expr, ref = D.op.abs(expr) + 1.0, np.abs(ref) + 1.0
+    dv.assign(expr, operator_t)
+    if operator_t == 0:
+        wv[...] = ref
+    elif operator_t == 1:
+        wv += ref
+    elif operator_t == 2:
+        wv -= ref
+    elif operator_t == 3:
+        wv *= ref
+    else:
+        wv /= ref
+    got = d.numpy().astype(np.float64)
+    tol = 3e-5 + max(g.size_terms - 1, 0) * 2.0 ** -24
+    assert (np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-3) + 1e-6).all(), (seed, view_kind, operator_t, D.last_kernel_kinds())
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_index_and_dtype_nodes(gpu, D, seed):
+    """argmax / argmin along either axis, one_hot, gather and gather_from_rows over int32, float32 and float64."""
+    rng = np.random.RandomState(9000 + seed)
+    op = D.op
+    R, Cn = [(5, 7), (64, 100), (257, 33), (100, 2048)][seed % 4]
+    dtype = [np.float32, np.float64, np.int32][seed % 3]
+    if dtype is np.int32:
+        x = rng.randint(-50, 50, (R, Cn)).astype(np.int32)  # many ties: first index must win
+    else:
+        x = rng.randn(R, Cn).astype(dtype)
+    X = arr(D, x)
+    assert np.array_equal(op.argmax(X, 1).numpy(), x.argmax(axis=1))
+    assert np.array_equal(op.argmin(X, 0).numpy(), x.argmin(axis=0))
+    assert np.array_equal(op.max(X, [0]).numpy(), x.max(axis=0)) and np.array_equal(op.min(X, [1]).numpy(), x.min(axis=1))
+    idx = rng.randint(0, Cn, R).astype(np.int32)
+    assert np.array_equal(op.gather_from_rows(X, arr(D, idx)).numpy(), x[np.arange(R), idx])
+    rows = rng.randint(0, R, 3 * R).astype(np.int32)
+    assert np.array_equal(op.gather(X, arr(D, rows)).numpy(), x[rows])
+    oh = op.one_hot(arr(D, idx), Cn, 1.0, 0.0).numpy()
+    assert np.array_equal(oh, np.eye(Cn, dtype=oh.dtype)[idx])
+    if dtype is np.int32:
+        assert np.array_equal(op.sum(X, [1]).numpy(), x.sum(axis=1)) and int(op.sum(X).numpy()) == int(x.sum())
+        assert np.array_equal((X * 3 - X).numpy(), x * 2)
+    else:
+        s = op.sum(op.abs(X), [0]).numpy()
+        want = np.abs(x.astype(np.float64)).sum(axis=0)
+        rt = (1e-5 + R * 2.0 ** -24) if dtype is np.float32 else 1e-12
+        assert (np.abs(s - want) <= rt * want + 1e-12).all()
+        sm = op.softmax(X).numpy()
+        e = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True))
+        ref = e / e.sum(axis=1, keepdims=True)
+        assert (np.abs(sm - ref) <= ((1e-5 + Cn * 2.0 ** -24) if dtype is np.float32 else 1e-12) * ref + 1e-30).all()
