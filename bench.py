@@ -252,6 +252,14 @@ def main():
         nxt["scatter_add_32000x1024_8192"] = {"us": round(us, 2), "GB/s": round(sbytes / us / 1e3, 1),
                                               "frac_hbm": round(sbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                                               "launches_incl_index_sort": rec.launches, "distinct_rows": uniq}
+        del table, ids, upd, g, rec
+        sm = D.Array.from_numpy(np.random.RandomState(17).uniform(0.5, 1.5, (8192, 8192)).astype(np.float32))
+        with D.Recording() as rec:
+            op.cumsum(sm).eval()
+        us = time_recording(rec, 20)
+        nxt["cumsum_8192x8192"] = {"us": round(us, 2), "GB/s": round(2 * 8192 * 8192 * 4 / us / 1e3, 1),
+                                   "frac_hbm": round(2 * 8192 * 8192 * 4 / us / 1e3 / HBM_PEAK_GBS, 4), "kernels": rec.launches}
+        del sm, rec
         configs["beyond_the_five_configs"] = nxt
         result["configs"] = configs
 

@@ -133,6 +133,10 @@ FRONT_SYMBOLS = {
     "dali_fe_softmax": (H, [H, _i]),
     "dali_fe_gather_from_rows": (H, [H, H]),
     "dali_fe_gather": (H, [H, H]),
+    "dali_fe_axis_scan": (H, [H, C.c_char_p, _i]),
+    "dali_fe_arange": (H, [H, H, H]),
+    "dali_fe_diag": (H, [H, _i, _i]),
+    "dali_fe_outer": (H, [H, H]),
     "dali_fe_autoreduce_assign": (_i, [H, H]),
     "dali_fe_one_hot": (H, [H, _i, H, H]),
     "dali_fe_dot": (H, [H, H]),

@@ -801,6 +801,60 @@ Array& autoreduce_assign(Array& left, const Array& right) {
     return left;
 }
 
+// dali/array/op/scan.cpp:183-194
+Array axis_scan(const Array& a, const std::string& reducer_name, bool inclusive) {
+    std::vector<int> shape = a.shape();
+    if (!inclusive) {
+        if (shape.empty()) shape = {2};
+        else shape.back() += 1;
+    }
+    Array n = make_node(Kind::AXIS_SCAN, reducer_name, {a}, shape, a.dtype());
+    n.expression()->depth = inclusive ? 1 : 0;
+    return n;
+}
+Array cumsum(const Array& a, bool inclusive) { return axis_scan(a, "reducers::sum", inclusive); }
+Array cumprod(const Array& a, bool inclusive) { return axis_scan(a, "reducers::product", inclusive); }
+
+// dali/array/op/arange.cpp:41-57
+Array arange(const Array& start, const Array& stop, const Array& step) {
+    DALI_ASSERT(start.ndim() == 0, make_message("arange's start argument must be a scalar but got start.shape = ", shape_str(start.shape()), "."));
+    DALI_ASSERT(stop.ndim() == 0, make_message("arange's stop argument must be a scalar but got stop.shape = ", shape_str(stop.shape()), "."));
+    DALI_ASSERT(step.ndim() == 0, make_message("arange's step argument must be a scalar but got step.shape = ", shape_str(step.shape()), "."));
+    const double b = start.scalar_value(), e = stop.scalar_value(), st = step.scalar_value();
+    const int size = (int)std::ceil((e - b) / st);
+    DALI_ASSERT(size > 0, make_message("arange's size must be strictly positive (got start = ", b, ", stop = ", e, ", step = ", st, ")."));
+    return make_node(Kind::ARANGE, "", {start, step}, {size}, start.dtype());
+}
+Array arange(int start, int stop) { return arange(Array(start), Array(stop), Array(1)); }
+Array arange(int size) { return arange(0, size); }
+
+// dali/array/op/eye.cpp:46-77
+Array diag(const Array& array, int rows, int cols) {
+    DALI_ASSERT(rows > 0 && cols > 0, make_message("diag's rows and cols must > 0 (got rows = ", rows, ", cols = ", cols, ")."));
+    DALI_ASSERT(array.ndim() <= 1, make_message("diag's argument must be a scalar or a vector (got array.shape = ", shape_str(array.shape()), ")."));
+    if (array.ndim() == 1) {
+        DALI_ASSERT(array.shape()[0] >= std::min(rows, cols), make_message("diag's argument is smaller than the maximal diagonal item (array.shape = ",
+                                                                           shape_str(array.shape()), ", rows = ", rows, ", cols = ", cols, ")."));
+    }
+    return make_node(Kind::DIAG, "", {array}, {rows, cols}, array.dtype());
+}
+Array diag(const Array& array, int rows) { return diag(array, rows, rows); }
+Array diag(const Array& array) {
+    DALI_ASSERT(array.ndim() == 1, "diag without an extent needs a vector");
+    return diag(array, array.shape()[0], array.shape()[0]);
+}
+Array eye(int rows, int cols) {
+    DALI_ASSERT(rows > 0 && cols > 0, make_message("eye's rows and cols must > 0 (got rows = ", rows, ", cols = ", cols, ")."));
+    return diag(Array(1.0f), rows, cols);
+}
+Array eye(int size) { return eye(size, size); }
+
+// dali/array/op/outer.cpp:8-36: out[i, j] = a[i] * b[j], expressed through the broadcasting elementwise map
+Array outer(const Array& a, const Array& b) {
+    DALI_ASSERT(a.ndim() == 1 && b.ndim() == 1, make_message("outer takes two vectors (got a.ndim = ", a.ndim(), ", b.ndim = ", b.ndim(), ")."));
+    return eltmul(a.expand_dims(1), b.expand_dims(0));
+}
+
 // dali/array/op/one_hot.cpp:62-74
 Array one_hot(Array indices, int depth, Array on_value, Array off_value) {
     DALI_ASSERT(indices.dtype() == DTYPE_INT32, "indices must be integers.");

@@ -108,6 +108,14 @@ dali_array_t dali_fe_softmax(dali_array_t a, int axis) { FE_TRY(return wrap(dali
 dali_array_t dali_fe_gather_from_rows(dali_array_t s, dali_array_t i) { FE_TRY(return wrap(dali::op::gather_from_rows(A(s), A(i)));, nullptr) }
 dali_array_t dali_fe_gather(dali_array_t s, dali_array_t i) { FE_TRY(return wrap(dali::op::gather(A(s), A(i)));, nullptr) }
 int dali_fe_autoreduce_assign(dali_array_t dest, dali_array_t source) { FE_TRY(dali::op::autoreduce_assign(A(dest), A(source)); return 0;, 1) }
+dali_array_t dali_fe_axis_scan(dali_array_t a, const char* reducer, int inclusive) {
+    FE_TRY(return wrap(dali::op::axis_scan(A(a), reducer, inclusive != 0));, nullptr)
+}
+dali_array_t dali_fe_arange(dali_array_t start, dali_array_t stop, dali_array_t step) {
+    FE_TRY(return wrap(dali::op::arange(A(start), A(stop), A(step)));, nullptr)
+}
+dali_array_t dali_fe_diag(dali_array_t diagonal, int rows, int cols) { FE_TRY(return wrap(dali::op::diag(A(diagonal), rows, cols));, nullptr) }
+dali_array_t dali_fe_outer(dali_array_t a, dali_array_t b) { FE_TRY(return wrap(dali::op::outer(A(a), A(b)));, nullptr) }
 dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_value, dali_array_t off_value) {
     FE_TRY(return wrap(dali::op::one_hot(A(indices), depth, A(on_value), A(off_value)));, nullptr)
 }

@@ -248,6 +248,19 @@ Array all_close(const Array& left, const Array& right, const Array& atolerance);
 Array softmax(const Array& logits, int axis = -1);
 Array gather_from_rows(const Array& source, const Array& indices);
 Array gather(const Array& source, const Array& indices);
+// dali/array/op/scan.h, arange.h, eye.h, outer.h
+Array axis_scan(const Array& a, const std::string& reducer_name, bool inclusive = true);
+Array cumsum(const Array& a, bool inclusive = true);
+Array cumprod(const Array& a, bool inclusive = true);
+Array arange(int size);
+Array arange(int start, int stop);
+Array arange(const Array& start, const Array& stop, const Array& step);
+Array eye(int size);
+Array eye(int rows, int cols);
+Array diag(const Array& diagonal);
+Array diag(const Array& diagonal, int rows);
+Array diag(const Array& diagonal, int rows, int cols);
+Array outer(const Array& a, const Array& b);
 Array& autoreduce_assign(Array& left, const Array& right);
 Array one_hot(Array indices, int depth, Array on_value, Array off_value);
 Array matmul(Array a, Array b);

@@ -231,6 +231,32 @@ template <> DI double dali_shfl_xor<double>(double v, int mask) {
     return __hiloint2double(hi, lo);
 }
 
+template <typename T> DI T dali_shfl_up(T v, int delta) { return __shfl_up(v, delta, 64); }
+template <> DI double dali_shfl_up<double>(double v, int delta) {
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __shfl_up(lo, delta, 64);
+    hi = __shfl_up(hi, delta, 64);
+    return __hiloint2double(hi, lo);
+}
+template <typename T> DI T dali_shfl(T v, int lane) { return __shfl(v, lane, 64); }
+template <> DI double dali_shfl<double>(double v, int lane) {
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __shfl(lo, lane, 64);
+    hi = __shfl(hi, lane, 64);
+    return __hiloint2double(hi, lo);
+}
+// Inclusive scan over the 64 lanes of a wave: lane l ends with step(v_0, ..., v_l), combined left to right.
+template <typename R, typename T>
+DI T dali_wave_scan(T v) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const T o = dali_shfl_up<T>(v, d);
+        if (lane >= d) v = R::template step<T>(o, v);
+    }
+    return v;
+}
+
 // Reduce over aligned groups of WIDTH lanes (WIDTH a power of two <= 64); every
 // lane of the group ends with the group's result.
 template <typename R, typename T, int WIDTH>

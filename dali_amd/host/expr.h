@@ -20,6 +20,9 @@ enum class Kind {
     BROADCAST,         // dali/array/jit/reshape.cpp:62-154 (BroadcastedReshape)
     GATHER_FROM_ROWS,  // dali/array/op/gather_from_rows.cpp:21-127
     GATHER,            // dali/array/op/gather.cpp:31-160 (rows of a 2-D source picked by a 1-D index)
+    AXIS_SCAN,         // dali/array/op/scan.cpp:19-194 (name = reducer, depth = 1 when inclusive)
+    ARANGE,            // dali/array/op/arange.cpp:8-39 (args: start, step scalars)
+    DIAG,              // dali/array/op/eye.cpp:8-44 (args: diagonal vector or scalar)
     ONE_HOT,           // dali/array/op/one_hot.cpp:16-74
     MATMUL             // dali/array/op/dot.cpp:18-47
 };

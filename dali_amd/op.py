@@ -195,3 +195,47 @@ def all_equals(left, right):
 
 def all_close(left, right, atolerance):
     return prod(close(left, right, atolerance))
+
+
+# dali/array/op/scan.h, arange.h, eye.h, outer.h
+def axis_scan(a, reducer, inclusive=True):
+    a = as_array(a)
+    return _wrap(front.dali_fe_axis_scan(a._h, reducer.encode(), 1 if inclusive else 0), "axis_scan")
+
+
+def cumsum(a, inclusive=True):
+    return axis_scan(a, "reducers::sum", inclusive)
+
+
+def cumprod(a, inclusive=True):
+    return axis_scan(a, "reducers::product", inclusive)
+
+
+def arange(*args):
+    """arange(size), arange(start, stop) or arange(start, stop, step) over python scalars."""
+    if len(args) == 1:
+        start, stop, step = 0, args[0], 1
+    elif len(args) == 2:
+        start, stop, step = args[0], args[1], 1
+    else:
+        start, stop, step = args
+    s0, s1, s2 = as_array(start), as_array(stop), as_array(step)
+    return _wrap(front.dali_fe_arange(s0._h, s1._h, s2._h), "arange")
+
+
+def diag(diagonal, rows=None, cols=None):
+    d = as_array(diagonal)
+    if rows is None:
+        rows = d.shape[0]
+    if cols is None:
+        cols = rows
+    return _wrap(front.dali_fe_diag(d._h, int(rows), int(cols)), "diag")
+
+
+def eye(rows, cols=None):
+    return diag(1.0, rows, rows if cols is None else cols)
+
+
+def outer(a, b):
+    a, b = as_array(a), as_array(b)
+    return _wrap(front.dali_fe_outer(a._h, b._h), "outer")

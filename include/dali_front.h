@@ -62,6 +62,14 @@ dali_array_t dali_fe_softmax(dali_array_t a, int axis);
 dali_array_t dali_fe_gather_from_rows(dali_array_t source, dali_array_t indices);
 /* op::gather (dali/array/op/gather.cpp:163-171); assigning to the lazy result scatters into `source` */
 dali_array_t dali_fe_gather(dali_array_t source, dali_array_t indices);
+/* op::axis_scan (dali/array/op/scan.cpp:183-194): reducer "reducers::sum" / "reducers::product" / ... along the last axis */
+dali_array_t dali_fe_axis_scan(dali_array_t a, const char* reducer, int inclusive);
+/* op::arange over 0-d start / stop / step (dali/array/op/arange.cpp:47-57) */
+dali_array_t dali_fe_arange(dali_array_t start, dali_array_t stop, dali_array_t step);
+/* op::diag / op::eye (dali/array/op/eye.cpp:46-77): `diagonal` is a vector or a 0-d value */
+dali_array_t dali_fe_diag(dali_array_t diagonal, int rows, int cols);
+/* op::outer (dali/array/op/outer.cpp:33-36) */
+dali_array_t dali_fe_outer(dali_array_t a, dali_array_t b);
 /* dest <<= source (dali/array/expression/assignment.cpp:92-126) */
 int dali_fe_autoreduce_assign(dali_array_t dest, dali_array_t source);
 dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_value, dali_array_t off_value);

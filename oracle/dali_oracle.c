@@ -352,6 +352,25 @@ void orc_scatter_to_rows(float* dest, int64_t cols, const int32_t* indices, int6
     }
 }
 
+/* Running reduction along the last axis, the CPU loop of dali/array/op/scan.cpp:52-75: so_far starts at the
+ * reducer's init value and takes the row's elements one by one. kind: 0 sum, 1 product, 2 maximum, 3 minimum.
+ * inclusive: out has `cols` entries per row; exclusive: cols + 1, the first being the init value. */
+void orc_axis_scan(int kind, const float* x, int64_t rows, int64_t cols, int inclusive, float* out) {
+    const int64_t oc = cols + (inclusive ? 0 : 1);
+    for (int64_t r = 0; r < rows; ++r) {
+        float so_far = kind == 0 ? 0.0f : (kind == 1 ? 1.0f : (kind == 2 ? -FLT_MAX : FLT_MAX));
+        if (!inclusive) out[r * oc] = so_far;
+        for (int64_t i = 0; i < cols; ++i) {
+            const float v = x[r * cols + i];
+            if (kind == 0) so_far += v;
+            else if (kind == 1) so_far *= v;
+            else if (kind == 2) so_far = so_far > v ? so_far : v;
+            else so_far = so_far < v ? so_far : v;
+            out[r * oc + i + (inclusive ? 0 : 1)] = so_far;
+        }
+    }
+}
+
 /* is_on = (indices[i] == j); on*is_on + (1.0 - is_on)*off, evaluated with T = float
  * for is_on and the 1.0 in double (dali/array/op/one_hot.cpp:38-46). */
 void orc_one_hot(const int32_t* indices, int64_t n, int depth, float on, float off, float* out) {

@@ -50,6 +50,7 @@ def _load():
     lib.orc_gather_rows.argtypes = [_f, _i64, _i32, _i64, _f]
     lib.orc_scatter_rows.argtypes = [_f, _i64, _i32, _i64, _f, C.c_int, C.c_int]
     lib.orc_scatter_to_rows.argtypes = [_f, _i64, _i32, _i64, _f, C.c_int, C.c_int]
+    lib.orc_axis_scan.argtypes = [C.c_int, _f, _i64, _i64, C.c_int, _f]
     lib.orc_one_hot.argtypes = [_i32, _i64, C.c_int, C.c_float, C.c_float, _f]
     lib.orc_softmax_cross_entropy.argtypes = [_f, _i32, _i64, _i64, _f, _f, _f]
     lib.orc_softmax_cross_entropy_via_probs.argtypes = [_f, _i32, _i64, _i64, _f]
@@ -211,6 +212,17 @@ def softmax_cross_entropy_via_probs(x, t):
     t = np.ascontiguousarray(t, dtype=np.int32)
     out = np.empty(x.shape[0], dtype=np.float32)
     lib.orc_softmax_cross_entropy_via_probs(fp(x), ip(t), x.shape[0], x.shape[1], fp(out))
+    return out
+
+
+def axis_scan(kind, x, inclusive=True):
+    """kind: 'sum' | 'product' | 'maximum' | 'minimum'; scans the last axis."""
+    x = _c32(x)
+    cols = x.shape[-1] if x.ndim else 1
+    rows = x.size // cols if cols else 0
+    out_shape = x.shape[:-1] + (cols + (0 if inclusive else 1),) if x.ndim else ((), (2,))[0 if inclusive else 1]
+    out = np.empty(out_shape, dtype=np.float32)
+    lib.orc_axis_scan({"sum": 0, "product": 1, "maximum": 2, "minimum": 3}[kind], fp(x), rows, cols, 1 if inclusive else 0, fp(out))
     return out
 
 

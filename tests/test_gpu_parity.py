@@ -702,3 +702,75 @@ def test_named_comparison_and_any_all_helpers(gpu, D, rng):
     c[9, 2] = np.inf
     assert float(op.any_isnan(arr(D, c)).numpy()) == 1.0 and float(op.any_isinf(arr(D, c)).numpy()) == 1.0
     assert op.any_isnan(arr(D, c), [1]).numpy().tolist() == [1.0 if r == 7 else 0.0 for r in range(33)]
+
+
+# ---------------------------------------------------------------- scan / arange / diag / outer
+def test_scan_reference_cases(gpu, D):
+    # ScanTests.cumsum / cumprod (tests.cpp:1737-1786) on int32 arange: exact
+    op = D.op
+    for inclusive in (True, False):
+        a = op.arange(0, 20)
+        want = np.cumsum(np.arange(20))
+        if not inclusive:
+            want = np.concatenate([[0], want])
+        assert np.array_equal(op.cumsum(a, inclusive).numpy(), want)
+        a2 = np.arange(20, dtype=np.int32).reshape(2, 10)
+        w2 = np.cumsum(a2, axis=1)
+        if not inclusive:
+            w2 = np.concatenate([np.zeros((2, 1), np.int64), w2], axis=1)
+        assert np.array_equal(op.cumsum(arr(D, a2), inclusive).numpy(), w2)
+        p = op.arange(1, 11)
+        wp = np.cumprod(np.arange(1, 11))
+        if not inclusive:
+            wp = np.concatenate([[1], wp])
+        assert np.array_equal(op.cumprod(p, inclusive).numpy(), wp)
+
+
+@pytest.mark.parametrize("shape", [(1,), (7,), (3, 64), (5, 257), (33, 1000), (4, 4096), (2, 100003), (3, 262144), (300, 1021), (2, 3, 50)])
+@pytest.mark.parametrize("inclusive", [True, False])
+def test_scan_matches_oracle(gpu, D, O, rng, shape, inclusive):
+    x = rng.uniform(0.5, 1.5, shape).astype(np.float32)
+    n = shape[-1]
+    got = D.op.cumsum(arr(D, x), inclusive).numpy()
+    want = O.axis_scan("sum", x, inclusive)
+    assert got.shape == want.shape
+    truth = np.cumsum(x.astype(np.float64), axis=-1)
+    if not inclusive:
+        truth = np.concatenate([np.zeros(shape[:-1] + (1,)), truth], axis=-1)
+    # all summands are positive: 1e-5 relative to the exact prefix, plus the sequential checker's own bound
+    assert (np.abs(got - truth) <= 1e-5 * np.abs(truth) + 1e-30).all()
+    assert (np.abs(got - want) <= (1e-5 + n * 2.0 ** -24) * np.abs(truth) + 1e-30).all()
+    # order-free reducers are exact
+    y = rng.randn(*shape).astype(np.float32)
+    assert np.array_equal(D.op.axis_scan(arr(D, y), "reducers::maximum", inclusive).numpy(), O.axis_scan("maximum", y, inclusive))
+    small = rng.uniform(0.99, 1.01, shape).astype(np.float32)  # the running product stays far from under- and overflow
+    gp = D.op.cumprod(arr(D, small), inclusive).numpy()
+    wp = O.axis_scan("product", small, inclusive)
+    assert (np.abs(gp - wp) <= (2e-5 + n * 2.0 ** -23) * np.abs(wp)).all()
+    # a strided argument (every other row)
+    if len(shape) == 2 and shape[0] >= 4:
+        v = arr(D, x)[::2]
+        assert np.array_equal(D.op.cumsum(v, inclusive).numpy(), D.op.cumsum(arr(D, x[::2].copy()), inclusive).numpy())
+
+
+def test_arange_diag_outer(gpu, D, rng):
+    op = D.op
+    assert op.arange(5).numpy().tolist() == [0, 1, 2, 3, 4] and op.arange(5).numpy().dtype == np.int32
+    assert op.arange(3, 9).numpy().tolist() == [3, 4, 5, 6, 7, 8]
+    assert op.arange(1, 10, 3).numpy().tolist() == [1, 4, 7]
+    f = op.arange(0.5, 3.0, 0.25).numpy()
+    assert f.dtype == np.float64 and np.array_equal(f, np.arange(0.5, 3.0, 0.25))
+    big = op.arange(1000003).numpy()
+    assert np.array_equal(big, np.arange(1000003, dtype=np.int32))
+    assert np.array_equal(op.eye(4).numpy(), np.eye(4, dtype=np.float32))
+    assert np.array_equal(op.eye(3, 7).numpy(), np.eye(3, 7, dtype=np.float32))
+    d = rng.randn(9).astype(np.float32)
+    assert np.array_equal(op.diag(arr(D, d)).numpy(), np.diag(d))
+    assert np.array_equal(op.diag(arr(D, d), 4, 6).numpy(), np.diag(d)[:4, :6])
+    assert np.array_equal((op.eye(5) * 3.0 + 1.0).numpy(), np.eye(5, dtype=np.float32) * 3 + 1)
+    a, b = rng.randn(37).astype(np.float32), rng.randn(1001).astype(np.float32)
+    assert np.array_equal(op.outer(arr(D, a), arr(D, b)).numpy(), np.outer(a, b))
+    # OuterTests-style use with arange (dali/array/op/outer.cpp:18): integer operands stay exact
+    assert np.array_equal(op.outer(op.arange(4), op.arange(6)).numpy(), np.outer(np.arange(4), np.arange(6)))
+    with pytest.raises(RuntimeError, match="strictly positive"):
+        op.arange(5, 2)

@@ -394,3 +394,19 @@ def test_scatter_to_rows_reference_known_answer(O):
     out = O.scatter_to_rows(np.full((7, 3), 42, np.float32)[:6], vals, 1.0, op=1)
     for i, v in enumerate(vals):
         assert out[i].tolist() == [43.0 if j == v else 42.0 for j in range(3)]
+
+
+def test_axis_scan_known_answers(O, rng):
+    # ScanTests.cumsum / cumprod (tests.cpp:1737-1786): arange inputs, 1-D and [2, 10], inclusive and exclusive
+    a = np.arange(20, dtype=np.float32)
+    assert np.array_equal(O.axis_scan("sum", a), np.cumsum(a))
+    assert np.array_equal(O.axis_scan("sum", a, False), np.concatenate([[0], np.cumsum(a)]))
+    assert np.array_equal(O.axis_scan("sum", a.reshape(2, 10)), np.cumsum(a.reshape(2, 10), axis=1))
+    p = np.arange(1, 11, dtype=np.float32)  # 10! is exact in fp32
+    assert np.array_equal(O.axis_scan("product", p), np.cumprod(p.astype(np.float64)).astype(np.float32))
+    assert np.array_equal(O.axis_scan("product", p, False)[0:2], [1.0, 1.0])
+    x = rng.randn(3, 50).astype(np.float32)
+    assert np.array_equal(O.axis_scan("maximum", x), np.maximum.accumulate(x, axis=1))
+    assert np.array_equal(O.axis_scan("minimum", x), np.minimum.accumulate(x, axis=1))
+    # fp32 sums: numpy's cumsum is the same left-to-right fp32 accumulation
+    assert np.array_equal(O.axis_scan("sum", x), np.cumsum(x, axis=1, dtype=np.float32))
