@@ -82,6 +82,7 @@ HIP_SYMBOLS = {
     "dali_hip_set_cache_dir": (_i, [C.c_char_p]),
     "dali_hip_sgemm": (_i, [_i, _i, _i, _i, _i, C.c_float, H, _i, H, _i, C.c_float, H, _i]),
     "dali_hip_sgemm_pair": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, C.c_float, H, _i, H, _i, H, _i, H, _i, C.c_float, H, _i]),
+    "dali_hip_lstm_step": (_i, [_i, _i, _i, H, _i, H, _i, H, H, _i, H, _i, H, H, H]),
     "dali_hip_argsort_i32": (_i, [H, C.c_int64, C.c_int32, H, H]),
     "dali_hip_capture_begin": (_i, []),
     "dali_hip_capture_end": (_i, [C.POINTER(H)]),

@@ -63,12 +63,19 @@ struct GemmArgs {
     // slabs; partial tiles and the per-tile ticket counters live in the library workspace
     unsigned int* counters;
     float* partials;
+    // fused LSTM gate epilogue (GATES kernels): C is not written; the tile's pre-activations go through the
+    // gate arithmetic with bias[4H], c_prev[M, H] and leave as c_out[M, H], h_out[M, H]
+    const float* bias;
+    const float* c_prev;
+    float* c_out;
+    float* h_out;
+    int H;
 };
 
 __device__ __forceinline__ void publish(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float observe(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int DEPTH, bool EDGE, int KW, bool MIDB>
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int DEPTH, bool EDGE, int KW, bool MIDB, bool GATES = false>
 __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     // KW wave sets share the tile: set kw takes every KW-th k-group of a slab, so each SIMD holds
     // KW waves that cover each other's LDS and barrier waits; the sets are summed through LDS at the end
@@ -147,6 +154,12 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
         if (!TB) {
             b_r[t] = idx / (BN / 4);             // k offset inside the slab
             b_c[t] = n0 + (idx % (BN / 4)) * 4;  // n
+            if (GATES) {
+                // tile column n' = 16 * gate + j stands for column gate * H + 16 * blockIdx.x + j of the packed weights:
+                // the four gates of sixteen hidden units meet in one workgroup
+                const int np = (idx % (BN / 4)) * 4;
+                b_c[t] = (np / 16) * g.H + blockIdx.x * 16 + np % 16;
+            }
         } else {
             b_r[t] = n0 + idx / (BK / 4);        // n
             b_c[t] = (idx % (BK / 4)) * 4;       // k offset inside the slab
@@ -299,6 +312,20 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
             if (TM * TN == 1) __builtin_amdgcn_sched_barrier(0);
         }
     };
+
+    // gate epilogue operands, requested now so that they have arrived long before the epilogue
+    constexpr int GATE_PAIRS = GATES ? BM * 16 / THREADS : 1;
+    float gate_bias[GATE_PAIRS][4], gate_c[GATE_PAIRS];
+    if constexpr (GATES) {
+#pragma unroll
+        for (int q = 0; q < GATE_PAIRS; ++q) {
+            const int e = tid + q * THREADS, r = e / 16, j = e % 16, hu = blockIdx.x * 16 + j;
+            const int m = m0 + r < M ? m0 + r : M - 1;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) gate_bias[q][k] = g.bias[k * g.H + hu];
+            gate_c[q] = g.c_prev[(size_t)m * g.H + hu];
+        }
+    }
 
     if constexpr (PIPE) {
         // Unchecked kernel: every instruction that is not an MFMA has to run in the shadow of the MFMAs (vector
@@ -499,7 +526,8 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
                         red[(size_t)(kw - 1) * BM * BN + ((wave * TM + ii) * TN + jj) * 1024 + v * 64 + lane] = acc[0][ii][jj][v];
         }
         __syncthreads();
-        if (kw > 0) return;
+        if (kw > 0 && !GATES) return;  // with the gate epilogue the other wave sets stay to share its arithmetic
+        if (kw == 0)
 #pragma unroll
         for (int s2 = 1; s2 < KW; ++s2)
 #pragma unroll
@@ -509,6 +537,45 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
                         acc[0][ii][jj][v] += red[(size_t)(s2 - 1) * BM * BN + ((wave * TM + ii) * TN + jj) * 1024 + v * 64 + lane];
+    }
+    if constexpr (GATES) {
+        // The sums go to LDS as a [BM][BN] tile of pre-activations (behind the fold area), then every thread of
+        // the workgroup finishes its (row, hidden unit) pairs: gate = pre + bias, i / f / o = sigmoid, g = tanh,
+        // c' = f * c + i * g, h' = o * tanh(c'), each operation rounded on its own like the generated gate kernel
+        // (dali/layers/lstm.cpp:238-261). Bias and previous cell values were fetched before the main loop.
+        static_assert(BM == 64 && BN == 64 && TM * TN == 1, "gate epilogue is written for the 64x64 tile");
+        static_assert(LDS_FLOATS >= RED_FLOATS + BM * BN, "no room for the pre-activation tile");
+        float* tile = lds + RED_FLOATS;
+        if (kw == 0) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int lm = wm * WTM + 8 * (v / 4) + 4 * h + (v % 4), ln = wn * WTN + l32;
+                tile[lm * BN + ln] = acc[0][0][0][v];
+            }
+        }
+        __syncthreads();
+        const int H = g.H;
+#pragma unroll
+        for (int q = 0; q < GATE_PAIRS; ++q) {
+#pragma clang fp contract(off)
+            const int e = tid + q * THREADS, r = e / 16, j = e % 16, m = m0 + r;
+            if (m >= M) continue;
+            const float gi = tile[r * BN + j] + gate_bias[q][0];
+            const float gf = tile[r * BN + 16 + j] + gate_bias[q][1];
+            const float go = tile[r * BN + 32 + j] + gate_bias[q][2];
+            const float gg = tile[r * BN + 48 + j] + gate_bias[q][3];
+            const float iv = (float)(1.0 / (1.0 + (double)expf(-gi)));
+            const float fv = (float)(1.0 / (1.0 + (double)expf(-gf)));
+            const float ov = (float)(1.0 / (1.0 + (double)expf(-go)));
+            const float gv = tanhf(gg);
+            const float fc = fv * gate_c[q];
+            const float ig = iv * gv;
+            const float cn = fc + ig;
+            const size_t o = (size_t)m * H + blockIdx.x * 16 + j;
+            g.c_out[o] = cn;
+            g.h_out[o] = ov * tanhf(cn);
+        }
+        return;
     }
     // epilogue: lane holds column l32 and rows 8*(v/4) + 4*h + v%4 of each 32x32 tile
     const float alpha = g.alpha, beta = g.beta;
@@ -738,6 +805,47 @@ int dali_hip_sgemm_pair(int transB1, int transA1, int transB2, int transA2, int 
     const float* Bs[2] = {B1, B2};
     int Ks[2] = {k1, k2}, ldas[2] = {lda1, lda2}, ldbs[2] = {ldb1, ldb2};
     return sgemm_rowmajor(2, transA1 != 0, transB1 != 0, n, m, Ks, As, ldas, Bs, ldbs, alpha, beta, C, ldc);
+}
+
+int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx, const float* Hprev, int ldh,
+                       const float* Cprev, const float* W, int ldw, const float* U, int ldu, const float* bias,
+                       float* Cout, float* Hout) {
+    if (ensure_init()) return DALI_HIP_ERROR;
+    if (batch <= 0 || input <= 0 || hidden <= 0) return fail("lstm_step: extents must be positive (batch=%d, input=%d, hidden=%d)", batch, input, hidden);
+    if (!X || !Hprev || !Cprev || !W || !U || !bias || !Cout || !Hout) return fail("lstm_step: NULL argument");
+    const bool ok = hidden % 64 == 0 && input % 64 == 0 && ldx == ldh && ldw == ldu && ldx % 4 == 0 && ldw % 4 == 0 && ldx >= input &&
+                    ldh >= hidden && ldw >= 4 * hidden && aligned16(X) && aligned16(Hprev) && aligned16(W) && aligned16(U) &&
+                    (size_t)64 * ldw * sizeof(float) + (size_t)4 * hidden * sizeof(float) < ((size_t)1 << 32) &&
+                    ((size_t)batch * ldx + 64) * sizeof(float) < ((size_t)1 << 32);
+    if (!ok)
+        return fail("lstm_step: the fused kernel needs input and hidden sizes that are multiples of 64, 16-byte aligned operands and "
+                    "equal leading dimensions for X / Hprev and for W / U");
+    GemmArgs g = {};
+    g.nseg = 2;
+    g.seg[0].A = X;
+    g.seg[0].B = W;
+    g.seg[0].lda = ldx;
+    g.seg[0].ldb = ldw;
+    g.seg[0].K = input;
+    g.seg[1].A = Hprev;
+    g.seg[1].B = U;
+    g.seg[1].lda = ldh;
+    g.seg[1].ldb = ldu;
+    g.seg[1].K = hidden;
+    g.M = batch;
+    g.N = 4 * hidden;
+    g.alpha = 1.0f;
+    g.beta = 0.0f;
+    g.bias = bias;
+    g.c_prev = Cprev;
+    g.c_out = Cout;
+    g.h_out = Hout;
+    g.H = hidden;
+    dim3 grid(4 * hidden / 64, (batch + 63) / 64);
+    hipLaunchKernelGGL((sgemm_kernel<64, 64, 64, false, false, true, 2, false, 2, false, true>), grid, dim3(512), 0, stream(), g);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("lstm_step launch failed: %s", hipGetErrorString(e));
+    return DALI_HIP_OK;
 }
 
 }  // extern "C"

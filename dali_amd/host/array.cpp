@@ -940,6 +940,17 @@ LSTMState lstm_step(const Array& x, const Array& h, const Array& c, const Array&
     DALI_ASSERT(W.shape()[1] == 4 * H && U.shape()[1] == 4 * H && b.shape()[0] == 4 * H && U.shape()[0] == H &&
                     W.shape()[0] == x.shape()[1] && c.shape() == h.shape() && x.shape()[0] == h.shape()[0],
                 "lstm_step: inconsistent shapes");
+    // one launch when the fused kernel applies: the gate arithmetic runs in the GEMM's epilogue
+    static const bool fused_off = getenv("DALI_HIP_LSTM_UNFUSED") != nullptr;
+    const int Bn = x.shape()[0], In = x.shape()[1];
+    auto dense = [](const Array& a) { return a.is_buffer() && a.contiguous_memory() && a.dtype() == DTYPE_FLOAT; };
+    for (const Array* a : {&x, &h, &c, &W, &U, &b}) a->eval();
+    if (!fused_off && !dry_run() && H % 64 == 0 && In == H && dense(x) && dense(h) && dense(c) && dense(W) && dense(U) && dense(b) &&
+        x.offset() % 4 == 0 && h.offset() % 4 == 0 && W.offset() % 4 == 0 && U.offset() % 4 == 0) {
+        Array c_new({Bn, H}, DTYPE_FLOAT), h_new({Bn, H}, DTYPE_FLOAT);
+        lstm_step_fused(x, h, c, W, U, b, c_new, h_new);
+        return {c_new, h_new};
+    }
     // pre-activations: one accumulating GEMM pair (X.W + H.U)
     Array pre = add(dot(x, W), dot(h, U));
     pre.eval();

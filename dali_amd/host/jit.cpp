@@ -2853,6 +2853,31 @@ void scatter_assign(const Array& dest, OPERATOR_T op, const Array& source) {
 
 }  // namespace
 
+void lstm_step_fused(const Array& x, const Array& h, const Array& c, const Array& W, const Array& U, const Array& b, const Array& c_new,
+                     const Array& h_new) {
+    const int Bn = x.shape()[0], In = x.shape()[1], H = h.shape()[1];
+    const float* xp = (const float*)x.device_ptr();
+    const float* hp = (const float*)h.device_ptr();
+    const float* cp = (const float*)c.device_ptr();
+    const float* wp = (const float*)W.device_ptr();
+    const float* up = (const float*)U.device_ptr();
+    const float* bp = (const float*)b.device_ptr();
+    float* co = (float*)c_new.device_ptr(memory::AM_OVERWRITE);
+    float* ho = (float*)h_new.device_ptr(memory::AM_OVERWRITE);
+    jit_stats().gemms_launched++;
+    jit_stats().last_kernel_kinds = "lstm_fused";
+    check_hip(dali_hip_lstm_step(Bn, In, H, xp, In, hp, H, cp, wp, 4 * H, up, 4 * H, bp, co, ho), "fused lstm step");
+    if (g_recording) {
+        note_recorded_write(c_new.expression()->memory);
+        note_recorded_write(h_new.expression()->memory);
+        std::vector<Array> keep = {x, h, c, W, U, b, c_new, h_new};
+        g_recording->push_back([=]() {
+            (void)keep;
+            check_hip(dali_hip_lstm_step(Bn, In, H, xp, In, hp, H, cp, wp, 4 * H, up, 4 * H, bp, co, ho), "fused lstm step replay");
+        });
+    }
+}
+
 void evaluate(const std::vector<Array>& roots) {
     jit_stats().evals++;
     jit_stats().last_kernel_kinds.clear();

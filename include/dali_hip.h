@@ -195,6 +195,20 @@ int dali_hip_sgemm_pair(int transB1, int transA1, int transB2, int transA2, int 
                         float alpha, const float* B1, int ldb1, const float* A1, int lda1, const float* B2,
                         int ldb2, const float* A2, int lda2, float beta, float* C, int ldc);
 
+/*
+ * One LSTM cell step in a single launch: pre = X[batch, input] . W[input, 4 hidden] + Hprev[batch, hidden] .
+ * U[hidden, 4 hidden] (row-major, gates packed i, f, o, g along the columns), then per element
+ * i, f, o = sigmoid(pre + bias), g = tanh(pre + bias), Cout = f * Cprev + i * g, Hout = o * tanh(Cout)
+ * (dali/layers/lstm.cpp:226-261 with StackedInputLayer::activate, dali/layers/layers.cpp:159-161). The MFMA tile of
+ * a workgroup gathers the four gate columns of sixteen hidden units, so the pre-activations never leave the chip;
+ * every operation is rounded as in the two-launch form (dali_hip_sgemm_pair followed by the generated gate
+ * kernel). Needs input and hidden to be multiples of 64, 16-byte aligned operands, ldx == ldh and ldw == ldu;
+ * otherwise it fails and the caller uses the two-launch form. Cprev, Cout, Hout are dense [batch, hidden].
+ */
+int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx, const float* Hprev, int ldh,
+                       const float* Cprev, const float* W, int ldw, const float* U, int ldu, const float* bias,
+                       float* Cout, float* Hout);
+
 /* ------------------------------------------------------------- scatter */
 /*
  * Stable ordering of n int32 keys held in device memory: sorted_keys[p] is the p-th smallest key and

@@ -774,3 +774,30 @@ def test_arange_diag_outer(gpu, D, rng):
     assert np.array_equal(op.outer(op.arange(4), op.arange(6)).numpy(), np.outer(np.arange(4), np.arange(6)))
     with pytest.raises(RuntimeError, match="strictly positive"):
         op.arange(5, 2)
+
+
+@pytest.mark.parametrize("B,H", [(64, 64), (256, 128), (100, 192), (7, 256), (256, 1024)])
+def test_fused_lstm_step_equals_the_two_launch_form(gpu, D, O, rng, B, H):
+    """input == hidden, multiples of 64: the gate arithmetic runs in the GEMM epilogue (one launch) and must give
+    what the GEMM pair followed by the generated gate kernel gives."""
+    op = D.op
+    X, Hp, Cp = (rng.randn(B, H).astype(np.float32) for _ in range(3))
+    lim = np.sqrt(6.0 / (H + 4 * H))
+    W, U = (rng.uniform(-lim, lim, (H, 4 * H)).astype(np.float32) for _ in range(2))
+    b = (rng.randn(4 * H) * 0.1).astype(np.float32)
+    dX, dH, dC, dW, dU, db = (arr(D, v) for v in (X, Hp, Cp, W, U, b))
+    before = D.jit_stats()
+    cn, hn = op.lstm_step(dX, dH, dC, dW, dU, db)
+    after = D.jit_stats()
+    assert after["gemms"] - before["gemms"] == 1 and after["kernels"] == before["kernels"] and D.last_kernel_kinds() == "lstm_fused"
+    # the same step spelled out with op::dot and the elementwise operators
+    pre = op.dot(dX, dW) + op.dot(dH, dU)
+    pre.eval()
+    gate = lambda k: pre[:, k * H:(k + 1) * H] + db[k * H:(k + 1) * H][None, :]
+    c2 = op.sigmoid(gate(1)) * dC + op.sigmoid(gate(0)) * op.tanh(gate(3))
+    h2 = op.sigmoid(gate(2)) * op.tanh(c2)
+    D.eval_together([c2, h2])
+    assert np.array_equal(cn.numpy(), c2.numpy()) and np.array_equal(hn.numpy(), h2.numpy())
+    _, ocn, ohn = O.lstm_step(X, Hp, Cp, W, U, b)
+    close(cn.numpy(), ocn, rtol=1e-4, atol=1e-5)
+    close(hn.numpy(), ohn, rtol=1e-4, atol=1e-5)
