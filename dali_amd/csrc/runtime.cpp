@@ -51,9 +51,12 @@ struct Runtime {
     std::string arch = "gfx950";
     // workspace: [counters | partials]
     char* ws = nullptr;
-    // bank: size -> parked blocks
+    // bank: size class -> parked blocks. Blocks up to kSlabBlockMax are carved out of large slabs (a driver
+    // allocation costs tens to hundreds of microseconds whatever its size); larger ones are driver allocations
     std::unordered_map<size_t, std::vector<void*>> bank;
     size_t bank_parked = 0, bank_live = 0;
+    std::vector<char*> slabs;
+    size_t slab_used = 0;  // bytes handed out from the newest slab
     // modules
     struct Module {
         hipModule_t module = nullptr;
@@ -233,10 +236,23 @@ int dali_hip_free(void* ptr) {
     return DALI_HIP_OK;
 }
 
+// Size class of a request: four classes per power of two above 256 bytes (at most 25% slack), so that
+// requests of nearly equal size share parked blocks.
+static size_t bank_class(size_t bytes) {
+    if (bytes <= 256) return 256;
+    size_t p = 256;
+    while (p * 2 < bytes) p *= 2;  // p < bytes <= 2p
+    const size_t step = p / 4;
+    return p + (bytes - p + step - 1) / step * step;
+}
+
+constexpr size_t kSlabBytes = (size_t)64 << 20;
+constexpr size_t kSlabBlockMax = (size_t)2 << 20;
+
 int dali_hip_bank_allocate(void** ptr, size_t bytes) {
     if (ensure_init()) return DALI_HIP_ERROR;
     Runtime& r = rt();
-    if (bytes == 0) bytes = 4;
+    bytes = bank_class(bytes);
     {
         std::lock_guard<std::mutex> lock(r.mu);
         auto it = r.bank.find(bytes);
@@ -246,6 +262,26 @@ int dali_hip_bank_allocate(void** ptr, size_t bytes) {
             r.bank_parked -= bytes;
             r.bank_live += bytes;
             return DALI_HIP_OK;
+        }
+        if (bytes <= kSlabBlockMax) {
+            if (r.slabs.empty() || r.slab_used + bytes > kSlabBytes) {
+                void* slab = nullptr;
+                hipError_t se = hipMalloc(&slab, kSlabBytes);
+                if (se != hipSuccess) {
+                    (void)hipGetLastError();
+                    slab = nullptr;  // fall through to a plain allocation of the block
+                } else {
+                    r.slabs.push_back((char*)slab);
+                    r.slab_used = 0;
+                }
+            }
+            if (!r.slabs.empty() && r.slab_used + bytes <= kSlabBytes) {
+                *ptr = r.slabs.back() + r.slab_used;
+                r.slab_used += bytes;  // classes are multiples of 64 bytes above 256: blocks stay 256-byte aligned
+                r.slab_used = (r.slab_used + 255) / 256 * 256;
+                r.bank_live += bytes;
+                return DALI_HIP_OK;
+            }
         }
     }
     *ptr = nullptr;
@@ -265,7 +301,7 @@ int dali_hip_bank_allocate(void** ptr, size_t bytes) {
 int dali_hip_bank_deposit(void* ptr, size_t bytes) {
     if (!ptr) return DALI_HIP_OK;
     Runtime& r = rt();
-    if (bytes == 0) bytes = 4;
+    bytes = bank_class(bytes);
     std::lock_guard<std::mutex> lock(r.mu);
     // Same-stream ordering makes immediate reuse safe: a later kernel that
     // receives this block runs after every kernel already queued on it.
@@ -280,12 +316,19 @@ int dali_hip_bank_clear(void) {
     if (!r.ready) return DALI_HIP_OK;
     HIP_TRY(hipStreamSynchronize(r.stream));
     std::lock_guard<std::mutex> lock(r.mu);
-    for (auto& kv : r.bank) {
-        for (void* p : kv.second) (void)hipFree(p);
-        kv.second.clear();
+    // parked driver allocations go back to the driver; blocks carved from slabs stay parked (a slab is only
+    // released as a whole, at process end)
+    size_t kept = 0;
+    for (auto it = r.bank.begin(); it != r.bank.end();) {
+        if (it->first > kSlabBlockMax) {
+            for (void* p : it->second) (void)hipFree(p);
+            it = r.bank.erase(it);
+        } else {
+            kept += it->first * it->second.size();
+            ++it;
+        }
     }
-    r.bank.clear();
-    r.bank_parked = 0;
+    r.bank_parked = kept;
     return DALI_HIP_OK;
 }
 

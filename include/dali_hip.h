@@ -70,10 +70,12 @@ void* dali_hip_stream(void);
 int dali_hip_malloc(void** ptr, size_t bytes);
 int dali_hip_free(void* ptr);
 
-/* Size-keyed free-list reuse of device blocks. Replace memory::bank::allocate,
- * deposit and clear, dali/array/memory/memory_bank.cpp:40-81: a deposited block
- * is handed out again for a request of the same byte size and only returned to
- * the driver by dali_hip_bank_clear. */
+/* Free-list reuse of device blocks. Replace memory::bank::allocate, deposit and clear,
+ * dali/array/memory/memory_bank.cpp:40-81: a deposited block is handed to the next request of its size.
+ * Here sizes are rounded up to classes (four per power of two, at most 25% slack) so that nearly equal
+ * requests share blocks, and blocks of up to 2 MiB are carved out of 64 MiB slabs instead of costing a driver
+ * allocation each. dali_hip_bank_clear returns the parked driver allocations; slab blocks stay parked.
+ * Same-stream ordering makes immediate reuse safe. */
 int dali_hip_bank_allocate(void** ptr, size_t bytes);
 int dali_hip_bank_deposit(void* ptr, size_t bytes);
 int dali_hip_bank_clear(void);

@@ -62,6 +62,29 @@ def test_memory_abi_roundtrip_and_bank(gpu, rng):
     assert hip.dali_hip_bank_allocate(C.byref(b), 12345 * 4) == 0
     assert a.value == b.value
     assert hip.dali_hip_bank_deposit(b, 12345 * 4) == 0
+    # requests of the same size class share blocks; small blocks come out of slabs (distinct, aligned, reusable)
+    assert hip.dali_hip_bank_allocate(C.byref(b), 12345 * 4 - 100) == 0 and a.value == b.value
+    assert hip.dali_hip_bank_deposit(b, 12345 * 4 - 100) == 0
+    blocks = []
+    for i in range(64):
+        blk = C.c_void_p()
+        assert hip.dali_hip_bank_allocate(C.byref(blk), 1000 + 37 * i) == 0 and blk.value % 256 == 0
+        blocks.append((blk.value, 1000 + 37 * i))
+    assert len(set(v for v, _ in blocks)) == 64
+    spans = sorted(blocks)
+    assert all(spans[i][0] + spans[i][1] <= spans[i + 1][0] for i in range(63))  # no overlap
+    pat = np.arange(250, dtype=np.float32)
+    for v, _ in blocks[:4]:
+        assert hip.dali_hip_memcpy_h2d(C.c_void_p(v), pat.ctypes.data_as(C.c_void_p), 1000) == 0
+    out4 = np.empty(250, np.float32)
+    for v, _ in blocks[:4]:
+        assert hip.dali_hip_memcpy_d2h(out4.ctypes.data_as(C.c_void_p), C.c_void_p(v), 1000) == 0 and np.array_equal(out4, pat)
+    for v, n_b in blocks:
+        assert hip.dali_hip_bank_deposit(C.c_void_p(v), n_b) == 0
+    big1, big2 = C.c_void_p(), C.c_void_p()
+    assert hip.dali_hip_bank_allocate(C.byref(big1), 5 << 20) == 0 and hip.dali_hip_bank_deposit(big1, 5 << 20) == 0
+    assert hip.dali_hip_bank_clear() == 0  # parked driver allocations are released, slab blocks stay
+    assert hip.dali_hip_bank_allocate(C.byref(big2), 5 << 20) == 0 and hip.dali_hip_bank_deposit(big2, 5 << 20) == 0
     free_b, total_b = C.c_size_t(), C.c_size_t()
     assert hip.dali_hip_mem_info(C.byref(free_b), C.byref(total_b)) == 0 and total_b.value > (100 << 30)
     name, arch = C.create_string_buffer(128), C.create_string_buffer(64)
