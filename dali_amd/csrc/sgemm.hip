@@ -112,6 +112,11 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, h = lane >> 5;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    // Gate epilogue: first of the sixteen hidden units of this workgroup. Workgroups are dealt to the eight XCDs
+    // round-robin, so consecutive groups of hidden units go to workgroups of the same XCD: the two 64-byte
+    // halves of a 128-byte line of the weights are then asked for by the same L2.
+    const int hu_base = GATES ? 16 * (gridDim.x % 8 == 0 ? (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8 : blockIdx.x) : 0;
+    (void)hu_base;
     const int M = g.M, N = g.N;
 
     floatx16 acc[CHAINS][TM][TN];
@@ -158,7 +163,7 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
                 // tile column n' = 16 * gate + j stands for column gate * H + 16 * blockIdx.x + j of the packed weights:
                 // the four gates of sixteen hidden units meet in one workgroup
                 const int np = (idx % (BN / 4)) * 4;
-                b_c[t] = (np / 16) * g.H + blockIdx.x * 16 + np % 16;
+                b_c[t] = (np / 16) * g.H + hu_base + np % 16;
             }
         } else {
             b_r[t] = n0 + idx / (BK / 4);        // n
@@ -319,7 +324,7 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     if constexpr (GATES) {
 #pragma unroll
         for (int q = 0; q < GATE_PAIRS; ++q) {
-            const int e = tid + q * THREADS, r = e / 16, j = e % 16, hu = blockIdx.x * 16 + j;
+            const int e = tid + q * THREADS, r = e / 16, j = e % 16, hu = hu_base + j;
             const int m = m0 + r < M ? m0 + r : M - 1;
 #pragma unroll
             for (int k = 0; k < 4; ++k) gate_bias[q][k] = g.bias[k * g.H + hu];
@@ -571,7 +576,7 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
             const float fc = fv * gate_c[q];
             const float ig = iv * gv;
             const float cn = fc + ig;
-            const size_t o = (size_t)m * H + blockIdx.x * 16 + j;
+            const size_t o = (size_t)m * H + hu_base + j;
             g.c_out[o] = cn;
             g.h_out[o] = ov * tanhf(cn);
         }
