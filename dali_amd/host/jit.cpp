@@ -70,7 +70,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-9";
+const char* const kCodegenVersion = "dali-hip-codegen-10";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -1577,8 +1577,14 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
                            int IL, const std::string& kname) {
     const std::string ld = NT ? "dali_load_nt<" : "dali_load<";
     const PNode& red = P.nodes[red_id];
-    std::string t = ctype(red.dtype);
+    const bool ARG = red.kind == Kind::ARG_AXIS_REDUCE;  // carries (value, row index); ties keep the lower index
+    std::string t = ctype(P.nodes[red.args[0]].dtype);
     std::string dt = ctype(P.arrays[dest_array].buf->dtype);
+    const std::string Rd = red.name;
+    // fold candidate (cv, ci) into (av, ai)
+    auto take = [&](const std::string& av, const std::string& ai, const std::string& cv, const std::string& ci) {
+        return "if (" + Rd + "::better<" + t + ">(" + cv + ", " + av + ") || (" + cv + " == " + av + " && " + ci + " < " + ai + ")) { " + av + " = " + cv + "; " + ai + " = " + ci + "; }";
+    };
     RowParams rp;
     rp.cached = false;
     rp.VEC = VEC;
@@ -1609,6 +1615,7 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     for (size_t i = 0; i < P.arrays.size(); ++i)
         if (!P.arrays[i].is_dest && P.arrays[i].cls == Cls::FULL) full_leaves.push_back((int)i);
     ss << "  " << t << " acc[VEC];\n  _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = " << red.name << "::init<" << t << ">();\n";
+    if (ARG) ss << "  int acci[VEC];\n  _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acci[j] = 0;\n";
     // contiguous share of the reduced axis for this y-block, interleaved over its waves
     // Which memory rows a y-block reads. 0: one contiguous share of the reduced axis. 1: single rows dealt
     // round-robin. 2: chunks of UNR*NWAVE consecutive rows dealt round-robin, so that the grid as a whole reads
@@ -1646,7 +1653,11 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     {
         BodyEmitter be(P, rp, true, 0, &first_body);
         std::string v = be.value(red.args[0]);
-        ss << be.stmts.str() << "          acc[j] = " << red.name << "::step<" << t << ">(acc[j], " << v << ");\n        }\n      }\n";
+        if (ARG)
+            // a thread meets its rows in increasing order: a strictly better value is the first index of its kind
+            ss << be.stmts.str() << "          { const " << t << " cv = " << v << "; if (" << Rd << "::better<" << t << ">(cv, acc[j])) { acc[j] = cv; acci[j] = (int)(x + u * XS); } }\n        }\n      }\n";
+        else
+            ss << be.stmts.str() << "          acc[j] = " << red.name << "::step<" << t << ">(acc[j], " << v << ");\n        }\n      }\n";
     }
     if (IL == 2)
         ss << "    }\n    for (long x = n_chunks * (UNR * NWAVE) + (long)blockIdx.y * NWAVE + wave; x < x_end; x += (long)gridDim.y * NWAVE) {\n";
@@ -1661,17 +1672,32 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     {
         BodyEmitter be(P, rp, true, 0, &first_body);
         std::string v = be.value(red.args[0]);
-        ss << be.stmts.str() << "        acc[j] = " << red.name << "::step<" << t << ">(acc[j], " << v << ");\n      }\n";
+        if (ARG)
+            ss << be.stmts.str() << "        { const " << t << " cv = " << v << "; if (" << Rd << "::better<" << t << ">(cv, acc[j])) { acc[j] = cv; acci[j] = (int)x; } }\n      }\n";
+        else
+            ss << be.stmts.str() << "        acc[j] = " << red.name << "::step<" << t << ">(acc[j], " << v << ");\n      }\n";
     }
     ss << "    }\n  }\n";
     // fold the row groups of the block in group order
     ss << "  __shared__ " << t << " sm[NWAVE][TPP * VEC];\n  __shared__ int is_last;\n";
-    ss << "  if (NWAVE > 1) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) sm[wave][lane * VEC + j] = acc[j];\n    __syncthreads();\n  }\n";
-    ss << "  if (NWAVE > 1 && wave == 0) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n      " << t << " r = sm[0][lane * VEC + j];\n"
-       << "      _Pragma(\"unroll\") for (int w = 1; w < NWAVE; ++w) r = " << red.name << "::step<" << t << ">(r, sm[w][lane * VEC + j]);\n      acc[j] = r;\n    }\n  }\n";
+    if (ARG) ss << "  __shared__ int smi[NWAVE][TPP * VEC];\n";
+    auto emit_group_fold = [&](const std::string& ind) {
+        ss << ind << "if (NWAVE > 1) {\n" << ind << "  _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) { sm[wave][lane * VEC + j] = acc[j];" << (ARG ? " smi[wave][lane * VEC + j] = acci[j];" : "")
+           << " }\n" << ind << "  __syncthreads();\n";
+        ss << ind << "  if (wave == 0) {\n" << ind << "    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n" << ind << "      " << t << " r = sm[0][lane * VEC + j];\n";
+        if (ARG) {
+            ss << ind << "      int ri = smi[0][lane * VEC + j];\n";
+            ss << ind << "      _Pragma(\"unroll\") for (int w = 1; w < NWAVE; ++w) { const " << t << " ov = sm[w][lane * VEC + j]; const int oi = smi[w][lane * VEC + j]; " << take("r", "ri", "ov", "oi") << " }\n";
+            ss << ind << "      acc[j] = r; acci[j] = ri;\n";
+        } else {
+            ss << ind << "      _Pragma(\"unroll\") for (int w = 1; w < NWAVE; ++w) r = " << red.name << "::step<" << t << ">(r, sm[w][lane * VEC + j]);\n" << ind << "      acc[j] = r;\n";
+        }
+        ss << ind << "    }\n" << ind << "  }\n" << ind << "}\n";
+    };
+    emit_group_fold("  ");
     auto emit_store = [&](const std::string& indent) {
         ss << indent << "_Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) if (k0 + j < K) { " << dt << "* dp = q" << dest_array << " + (k0 + j) * ds" << dest_array
-           << "; *dp = " << op_combine(op, "(*dp)", "(" + dt + ")acc[j]") << "; }\n";
+           << "; *dp = " << op_combine(op, "(*dp)", std::string("(") + dt + ")" + (ARG ? "acci[j]" : "acc[j]")) << "; }\n";
     };
     ss << "  if (gridDim.y == 1) {\n    if (wave == 0 && k_ok) {\n";
     emit_store("      ");
@@ -1682,23 +1708,31 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     ss << "  const long pcol = ((long)blockIdx.x * TPP + lane) * VEC;\n";
     // same fence-free hand-off as the full reduction: agent-scope atomic stores, wait for their
     // acknowledgement, then the ticket; the last block of the strip observes with agent-scope loads
-    ss << "  if (wave == 0) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) dali_publish(partials + (long)blockIdx.y * KP + pcol + j, acc[j]);\n"
+    if (ARG) ss << "  int* pidx = (int*)(partials + (long)gridDim.y * KP);  // the indices follow the values\n";
+    ss << "  if (wave == 0) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) { dali_publish(partials + (long)blockIdx.y * KP + pcol + j, acc[j]);"
+       << (ARG ? " dali_publish(pidx + (long)blockIdx.y * KP + pcol + j, acci[j]);" : "") << " }\n"
           "    __builtin_amdgcn_s_waitcnt(0);\n  }\n  __syncthreads();\n";
     ss << "  if (threadIdx.x == 0) is_last = dali_take_ticket(&counters[blockIdx.x]) == gridDim.y - 1;\n  __syncthreads();\n";
     ss << "  if (!is_last) return;\n";
     // every row group of the last block folds a contiguous share of the partial rows in y order (TAIL of them in
     // flight at a time); the groups are then joined in group order through LDS
     ss << "  _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = " << red.name << "::init<" << t << ">();\n";
+    if (ARG) ss << "  _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acci[j] = 2147483647;\n";
     ss << "  const unsigned int y_per = (gridDim.y + NWAVE - 1) / NWAVE;\n";
     ss << "  const unsigned int y_begin = wave * y_per, y_end = y_begin + y_per < gridDim.y ? y_begin + y_per : gridDim.y;\n";
     ss << "  for (unsigned int y0 = y_begin; y0 < y_end; y0 += TAIL) {\n    dali_vec<" << t << ", VEC> pv[TAIL];\n";
+    if (ARG) ss << "    dali_vec<int, VEC> pi[TAIL];\n";
     ss << "    _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) if (y0 + k < y_end) {\n"
-          "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) pv[k].v[j] = dali_observe(partials + (long)(y0 + k) * KP + pcol + j);\n    }\n";
-    ss << "    _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) if (y0 + k < y_end) {\n      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = "
-       << red.name << "::step<" << t << ">(acc[j], pv[k].v[j]);\n    }\n  }\n";
-    ss << "  if (NWAVE > 1) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) sm[wave][lane * VEC + j] = acc[j];\n    __syncthreads();\n"
-       << "    if (wave == 0) {\n      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        " << t << " r = sm[0][lane * VEC + j];\n"
-       << "        _Pragma(\"unroll\") for (int w = 1; w < NWAVE; ++w) r = " << red.name << "::step<" << t << ">(r, sm[w][lane * VEC + j]);\n        acc[j] = r;\n      }\n    }\n  }\n";
+          "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) { pv[k].v[j] = dali_observe(partials + (long)(y0 + k) * KP + pcol + j);"
+       << (ARG ? " pi[k].v[j] = dali_observe(pidx + (long)(y0 + k) * KP + pcol + j);" : "") << " }\n    }\n";
+    if (ARG)
+        // the y-blocks hold interleaved chunks of rows: equal values are settled by the index itself
+        ss << "    _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) if (y0 + k < y_end) {\n      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) { "
+           << take("acc[j]", "acci[j]", "pv[k].v[j]", "pi[k].v[j]") << " }\n    }\n  }\n";
+    else
+        ss << "    _Pragma(\"unroll\") for (int k = 0; k < TAIL; ++k) if (y0 + k < y_end) {\n      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = "
+           << red.name << "::step<" << t << ">(acc[j], pv[k].v[j]);\n    }\n  }\n";
+    emit_group_fold("  ");
     ss << "  if (wave == 0 && k_ok) {\n";
     emit_store("    ");
     ss << "  }\n  if (threadIdx.x == 0) dali_publish(&counters[blockIdx.x], 0u);\n}\n";
@@ -1709,7 +1743,8 @@ bool try_col(const DestSpec& spec) {
     Array root = spec.root;
     while (root.expression()->kind == Kind::EXPAND_DIMS) root = root.expression()->args[0];
     auto re = root.expression();
-    if (re->kind != Kind::AXIS_REDUCE) return false;
+    if (re->kind != Kind::AXIS_REDUCE && re->kind != Kind::ARG_AXIS_REDUCE) return false;
+    const bool is_arg = re->kind == Kind::ARG_AXIS_REDUCE;
     Array arg = re->args[0];
     if (arg.ndim() != 2) return false;
     int64_t K = arg.shape()[0], X = arg.shape()[1];
@@ -1790,7 +1825,7 @@ bool try_col(const DestSpec& spec) {
     outs[0].op = spec.op;
     outs[0].cls = Cls::ROW;
     std::ostringstream params;
-    const bool NT = K * X * (int64_t)size_of_dtype(re->dtype) >= ((int64_t)64 << 20);
+    const bool NT = K * X * (int64_t)size_of_dtype(arg.dtype()) >= ((int64_t)64 << 20);
     static const int maxy_env = env_int("DALI_HIP_COL_MAXY", 256);
     params << VEC << "," << UNR << "," << TAIL << "," << RG << "," << NT << "," << IL;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
@@ -1813,7 +1848,7 @@ bool try_col(const DestSpec& spec) {
         Kp->plan.work2_per_block = rows_env > 0 ? rows_env : UNR * RG;  // fewest reduced rows per y-block
         Kp->plan.max_blocks2 = maxy_env;
         Kp->plan.max_blocks = blocks_env;  // one block per CU: the y split fills what the column strips leave
-        Kp->plan.ws_elsize = size_of_dtype(re->dtype);
+        Kp->plan.ws_elsize = size_of_dtype(arg.dtype()) + (is_arg ? 4 : 0);  // a partial is a value, plus its index
     }
     std::vector<std::vector<int>> shapes = {{(int)K, (int)X}};
     load_and_launch(*Kp, [&]() { return gen_col_kernel(P, red_id, dest_array, spec.op, L, VEC, UNR, TAIL, RG, NT, IL, Kp->name); }, P, shapes);

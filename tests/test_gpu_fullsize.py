@@ -53,6 +53,18 @@ def test_c3_reductions_8192x8192(gpu, D, O):
     assert float(op.max(X).numpy()) == x.max()
     am = op.argmax(X, 1).numpy()
     assert am.dtype == np.int32 and np.array_equal(am, O.arg_axis_reduce(O.MAX, x, 1))
+    # argmax with planted ties, both axes: the first index must win (all_reduce_kernel_utils.cpp:217-219)
+    xt = x.copy()
+    peak = np.float32(np.abs(x).max() + 1.0)
+    for c in range(0, 8192, 97):
+        xt[[5000 + c % 100, 17 + c % 50, 8191], c] = peak  # three equal maxima in column c
+    for r in range(0, 8192, 89):
+        xt[r, [8000, 3 + r % 64, 4096]] = peak + 1.0
+    XT = arr(D, xt)
+    a0, a1 = op.argmax(XT, 0).numpy(), op.argmax(XT, 1).numpy()
+    assert a0.dtype == np.int32 and np.array_equal(a0, xt.argmax(0)) and np.array_equal(a1, xt.argmax(1))
+    assert np.array_equal(a0, O.arg_axis_reduce(O.MAX, xt, 0))
+    assert np.array_equal(op.argmin(XT, 0).numpy(), xt.argmin(0))
     # checksum of checksums: the row sums and the column sums add up to the same total
     assert abs(s1.astype(np.float64).sum() - s0.astype(np.float64).sum()) <= 1e-5 * np.abs(x64).sum()
 
