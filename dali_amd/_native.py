@@ -138,6 +138,7 @@ FRONT_SYMBOLS = {
     "dali_fe_arange": (H, [H, H, H]),
     "dali_fe_diag": (H, [H, _i, _i]),
     "dali_fe_outer": (H, [H, H]),
+    "dali_fe_circular_convolution": (H, [H, H]),
     "dali_fe_autoreduce_assign": (_i, [H, H]),
     "dali_fe_one_hot": (H, [H, _i, H, H]),
     "dali_fe_dot": (H, [H, H]),

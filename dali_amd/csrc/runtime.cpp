@@ -582,8 +582,7 @@ int dali_hip_launch(uint64_t hash, void** array_data, const int* offsets, const 
     if (gx > 2147483647LL || gy > 65535) return fail("dali_hip_launch: grid %lld x %lld too large", (long long)gx, (long long)gy);
     size_t karg = m->karg_bytes;
     void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, buf, HIP_LAUNCH_PARAM_BUFFER_SIZE, &karg, HIP_LAUNCH_PARAM_END};
-    static const unsigned lds_pad = getenv("DALI_HIP_LAUNCH_LDS_PAD") ? (unsigned)atoi(getenv("DALI_HIP_LAUNCH_LDS_PAD")) : 0u;
-    hipError_t e = hipModuleLaunchKernel(m->fn, (unsigned)gx, (unsigned)gy, 1, (unsigned)P.block_threads, 1, 1, lds_pad,
+    hipError_t e = hipModuleLaunchKernel(m->fn, (unsigned)gx, (unsigned)gy, 1, (unsigned)P.block_threads, 1, 1, 0,
                                          r.stream, nullptr, extra);
     if (e != hipSuccess) return fail("hipModuleLaunchKernel failed: %s", hipGetErrorString(e));
     return DALI_HIP_OK;

@@ -855,6 +855,21 @@ Array outer(const Array& a, const Array& b) {
     return eltmul(a.expand_dims(1), b.expand_dims(0));
 }
 
+// dali/array/op/circular_convolution.cpp:82-86: out[..., x] = sum_s content[..., (x + s) mod n] * weights[..., s]
+Array circular_convolution(Array x, Array weights) {
+    if (x.dtype() != weights.dtype()) {
+        DType t = type_promotion(x, weights);
+        x = astype(x, t);
+        weights = astype(weights, t);
+    }
+    DALI_ASSERT(x.ndim() == weights.ndim() && x.ndim() >= 1, "circular_convolution: content and weights must have the same (non-zero) number of dimensions");
+    std::vector<int> shape = common_shape(x, weights);
+    // both operands are presented at the common shape (a broadcast operand is written out once)
+    Array xb = x.shape() == shape ? x : identity(broadcasted_reshape(x, shape));
+    Array wb = weights.shape() == shape ? weights : identity(broadcasted_reshape(weights, shape));
+    return make_node(Kind::CIRCULAR_CONV, "", {xb, wb}, shape, x.dtype());
+}
+
 // dali/array/op/one_hot.cpp:62-74
 Array one_hot(Array indices, int depth, Array on_value, Array off_value) {
     DALI_ASSERT(indices.dtype() == DTYPE_INT32, "indices must be integers.");

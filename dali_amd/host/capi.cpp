@@ -115,6 +115,7 @@ dali_array_t dali_fe_arange(dali_array_t start, dali_array_t stop, dali_array_t 
     FE_TRY(return wrap(dali::op::arange(A(start), A(stop), A(step)));, nullptr)
 }
 dali_array_t dali_fe_diag(dali_array_t diagonal, int rows, int cols) { FE_TRY(return wrap(dali::op::diag(A(diagonal), rows, cols));, nullptr) }
+dali_array_t dali_fe_circular_convolution(dali_array_t x, dali_array_t w) { FE_TRY(return wrap(dali::op::circular_convolution(A(x), A(w)));, nullptr) }
 dali_array_t dali_fe_outer(dali_array_t a, dali_array_t b) { FE_TRY(return wrap(dali::op::outer(A(a), A(b)));, nullptr) }
 dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_value, dali_array_t off_value) {
     FE_TRY(return wrap(dali::op::one_hot(A(indices), depth, A(on_value), A(off_value)));, nullptr)

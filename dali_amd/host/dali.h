@@ -261,6 +261,8 @@ Array diag(const Array& diagonal);
 Array diag(const Array& diagonal, int rows);
 Array diag(const Array& diagonal, int rows, int cols);
 Array outer(const Array& a, const Array& b);
+// dali/array/op/circular_convolution.h
+Array circular_convolution(Array x, Array weights);
 Array& autoreduce_assign(Array& left, const Array& right);
 Array one_hot(Array indices, int depth, Array on_value, Array off_value);
 Array matmul(Array a, Array b);

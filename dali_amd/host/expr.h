@@ -23,6 +23,7 @@ enum class Kind {
     AXIS_SCAN,         // dali/array/op/scan.cpp:19-194 (name = reducer, depth = 1 when inclusive)
     ARANGE,            // dali/array/op/arange.cpp:8-39 (args: start, step scalars)
     DIAG,              // dali/array/op/eye.cpp:8-44 (args: diagonal vector or scalar)
+    CIRCULAR_CONV,     // dali/array/op/circular_convolution.cpp:8-86 (args: content, weights, both of the node's shape)
     ONE_HOT,           // dali/array/op/one_hot.cpp:16-74
     MATMUL             // dali/array/op/dot.cpp:18-47
 };

@@ -2151,6 +2151,7 @@ bool is_plain_matmul(const Array& a) { return a.expression()->kind == Kind::MATM
 // gather sources that are not buffers.
 Array run_scan(const Array& arg_in, const std::string& reducer, bool inclusive);
 Array run_fill(const std::shared_ptr<Expr>& e);
+Array run_circular_convolution(const Array& x, const Array& w);
 
 Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root) {
     auto e = a.expression();
@@ -2203,6 +2204,11 @@ Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root) {
         case Kind::DIAG:
             out = run_fill(e);
             break;
+        case Kind::CIRCULAR_CONV: {
+            Array x = clean(e->args[0], memo, false), w = clean(e->args[1], memo, false);
+            out = run_circular_convolution(x, w);
+            break;
+        }
         case Kind::GATHER: {
             // source and index are presented as buffers; the gather itself stays lazy only where the row
             // kernel can read through it: a [N, D] node that is the root or sits under same-shape
@@ -2776,6 +2782,65 @@ Array run_scan(const Array& arg_in, const std::string& reducer, bool inclusive) 
         P.arrays.push_back(manual_arg(totals, Cls::FULL, false, 2, {(int)R, (int)S}, {}));
         launch(2, 256, P, {(int)(R * S), C, (int)S, (int)SL});
     }
+    return dest;
+}
+
+// ------------------------------------------------------- circular convolution
+// out[r, x] = sum over s of content[r, (x + s) mod n] * weights[r, s] (dali/array/op/circular_convolution.cpp:22-38).
+// One workgroup per row keeps the row of both operands in LDS; a thread owns outputs x = tid, tid + 256, ... and
+// walks s upwards, so every output is the same left-to-right fp32 sum as the reference's loop. The content reads of
+// a wave are consecutive LDS words, the weight is a broadcast.
+Array run_circular_convolution(const Array& x_in, const Array& w_in) {
+    Array x = x_in, w = w_in;
+    if (!x.is_buffer()) x = materialize(x);
+    if (!w.is_buffer()) w = materialize(w);
+    if (!x.contiguous_memory()) x = x.ascontiguousarray();
+    if (!w.contiguous_memory()) w = w.ascontiguousarray();
+    Array dest(x.shape(), x.dtype());
+    const int n = x.shape().back();
+    const int64_t R = n ? numel_of(x.shape()) / n : 0;
+    if (R == 0 || n == 0) return dest;
+    const int el = size_of_dtype(x.dtype());
+    DALI_ASSERT((int64_t)2 * n * el <= 128 * 1024, make_message("circular_convolution: rows of ", n, " elements do not fit the on-chip staging (limit ", 64 * 1024 / el, ")"));
+    Program P;
+    P.arrays.push_back(manual_arg(dest, Cls::FULL, true, 2, {(int)R, n}, {}));
+    P.arrays.push_back(manual_arg(x, Cls::FULL, false, 2, {(int)R, n}, {}));
+    P.arrays.push_back(manual_arg(w, Cls::FULL, false, 2, {(int)R, n}, {}));
+    std::string t = ctype(x.dtype());
+    std::ostringstream sig;
+    int CAP = 256;  // LDS capacity of the specialisation, in elements per operand row
+    while (CAP < n) CAP *= 2;
+    sig << "circconv|" << (int)x.dtype() << "|" << CAP;
+    static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
+    uint64_t h = kernel_hash("circconv", sig.str(), "");
+    std::shared_ptr<KernelSpec>& K = specs_cache[h];
+    std::vector<int> shape_ndims = {2};
+    IvLayout L = layout_iv(P, shape_ndims);
+    if (!K) {
+        K = std::make_shared<KernelSpec>();
+        K->hash = h;
+        K->kind = "circconv";
+        K->name = kernel_name(K->kind, h);
+        fill_plan_arrays(*K, P, shape_ndims);
+        K->plan.block_threads = 256;
+        K->plan.grid_kind = DALI_HIP_GRID_ROWS;
+        K->plan.work_begin = L.shape_pos[0];
+        K->plan.work_count = 1;
+        K->plan.work_per_block = 1;
+    }
+    load_and_launch(*K, [&]() {
+        std::ostringstream ss;
+        ss << codegen::kDevicePrelude << kargs_struct(P, L);
+        ss << "extern \"C\" __global__ __launch_bounds__(256) void " << K->name << "(KArgs A) {\n  typedef " << t << " T;\n";
+        ss << "  __shared__ T c[" << CAP << "];\n  __shared__ T w[" << CAP << "];\n";
+        ss << "  const int n = A.iv[" << L.shape_pos[0] + 1 << "];\n  const long row = blockIdx.x;\n";
+        ss << "  const T* cg = (const T*)A.p[1] + row * n;\n  const T* wg = (const T*)A.p[2] + row * n;\n";
+        ss << "  for (int i = threadIdx.x; i < n; i += 256) { c[i] = cg[i]; w[i] = wg[i]; }\n  __syncthreads();\n";
+        ss << "  T* out = (T*)A.p[0] + row * n;\n";
+        ss << "  for (int x = threadIdx.x; x < n; x += 256) {\n    T res = (T)0;\n    int off = x;\n";
+        ss << "    for (int s = 0; s < n; ++s) {\n      res += c[off] * w[s];\n      off = off + 1 == n ? 0 : off + 1;\n    }\n    out[x] = res;\n  }\n}\n";
+        return ss.str();
+    }, P, {{(int)R, n}});
     return dest;
 }
 

@@ -239,3 +239,9 @@ def eye(rows, cols=None):
 def outer(a, b):
     a, b = as_array(a), as_array(b)
     return _wrap(front.dali_fe_outer(a._h, b._h), "outer")
+
+
+def circular_convolution(x, weights):
+    """out[..., i] = sum_s x[..., (i + s) mod n] * weights[..., s] (dali/array/op/circular_convolution.cpp)."""
+    x, weights = as_array(x), as_array(weights)
+    return _wrap(front.dali_fe_circular_convolution(x._h, weights._h), "circular_convolution")

@@ -68,6 +68,8 @@ dali_array_t dali_fe_axis_scan(dali_array_t a, const char* reducer, int inclusiv
 dali_array_t dali_fe_arange(dali_array_t start, dali_array_t stop, dali_array_t step);
 /* op::diag / op::eye (dali/array/op/eye.cpp:46-77): `diagonal` is a vector or a 0-d value */
 dali_array_t dali_fe_diag(dali_array_t diagonal, int rows, int cols);
+/* op::circular_convolution (dali/array/op/circular_convolution.cpp:82-86) */
+dali_array_t dali_fe_circular_convolution(dali_array_t x, dali_array_t weights);
 /* op::outer (dali/array/op/outer.cpp:33-36) */
 dali_array_t dali_fe_outer(dali_array_t a, dali_array_t b);
 /* dest <<= source (dali/array/expression/assignment.cpp:92-126) */

@@ -371,6 +371,21 @@ void orc_axis_scan(int kind, const float* x, int64_t rows, int64_t cols, int inc
     }
 }
 
+/* out[r, x] = sum over s = 0..n-1 of content[r, (x + s) mod n] * weights[r, s], accumulated in that order
+ * (dali/array/op/circular_convolution.cpp:22-38). */
+void orc_circular_convolution(const float* content, const float* weights, int64_t rows, int64_t n, float* out) {
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t x = 0; x < n; ++x) {
+            float res = 0.0f;
+            for (int64_t s = 0; s < n; ++s) {
+                int64_t off = x + s;
+                if (off >= n) off -= n;
+                res += content[r * n + off] * weights[r * n + s];
+            }
+            out[r * n + x] = res;
+        }
+}
+
 /* is_on = (indices[i] == j); on*is_on + (1.0 - is_on)*off, evaluated with T = float
  * for is_on and the 1.0 in double (dali/array/op/one_hot.cpp:38-46). */
 void orc_one_hot(const int32_t* indices, int64_t n, int depth, float on, float off, float* out) {

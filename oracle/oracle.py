@@ -51,6 +51,7 @@ def _load():
     lib.orc_scatter_rows.argtypes = [_f, _i64, _i32, _i64, _f, C.c_int, C.c_int]
     lib.orc_scatter_to_rows.argtypes = [_f, _i64, _i32, _i64, _f, C.c_int, C.c_int]
     lib.orc_axis_scan.argtypes = [C.c_int, _f, _i64, _i64, C.c_int, _f]
+    lib.orc_circular_convolution.argtypes = [_f, _f, _i64, _i64, _f]
     lib.orc_one_hot.argtypes = [_i32, _i64, C.c_int, C.c_float, C.c_float, _f]
     lib.orc_softmax_cross_entropy.argtypes = [_f, _i32, _i64, _i64, _f, _f, _f]
     lib.orc_softmax_cross_entropy_via_probs.argtypes = [_f, _i32, _i64, _i64, _f]
@@ -223,6 +224,15 @@ def axis_scan(kind, x, inclusive=True):
     out_shape = x.shape[:-1] + (cols + (0 if inclusive else 1),) if x.ndim else ((), (2,))[0 if inclusive else 1]
     out = np.empty(out_shape, dtype=np.float32)
     lib.orc_axis_scan({"sum": 0, "product": 1, "maximum": 2, "minimum": 3}[kind], fp(x), rows, cols, 1 if inclusive else 0, fp(out))
+    return out
+
+
+def circular_convolution(content, weights):
+    content, weights = np.broadcast_arrays(np.asarray(content, np.float32), np.asarray(weights, np.float32))
+    content, weights = _c32(content), _c32(weights)
+    n = content.shape[-1]
+    out = np.empty_like(content)
+    lib.orc_circular_convolution(fp(content), fp(weights), content.size // n, n, fp(out))
     return out
 
 

@@ -824,3 +824,18 @@ def test_fused_lstm_step_equals_the_two_launch_form(gpu, D, O, rng, B, H):
     _, ocn, ohn = O.lstm_step(X, Hp, Cp, W, U, b)
     close(cn.numpy(), ocn, rtol=1e-4, atol=1e-5)
     close(hn.numpy(), ohn, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(3,), (2, 3, 4), (5, 257), (64, 1024), (3, 5000)])
+def test_circular_convolution_matches_oracle(gpu, D, O, rng, shape):
+    # JITTests.circular_convolution / _broadcast / _1d (circular_convolution_tests.cpp:54-89)
+    x = rng.uniform(-1, 1, shape).astype(np.float32)
+    w = rng.uniform(-1, 1, shape).astype(np.float32)
+    got = D.op.circular_convolution(arr(D, x), arr(D, w)).numpy()
+    assert np.array_equal(got, O.circular_convolution(x, w))  # same left-to-right fp32 sums
+    if len(shape) >= 2:
+        wb = w[..., :1]  # weights broadcast along the convolved axis
+        assert np.array_equal(D.op.circular_convolution(arr(D, x), arr(D, wb)).numpy(), O.circular_convolution(x, wb))
+    if len(shape) == 1:
+        wide = rng.uniform(-1, 1, 2 * shape[0]).astype(np.float32)
+        assert np.array_equal(D.op.circular_convolution(arr(D, x), arr(D, wide)[::2]).numpy(), O.circular_convolution(x, wide[::2]))

@@ -410,3 +410,21 @@ def test_axis_scan_known_answers(O, rng):
     assert np.array_equal(O.axis_scan("minimum", x), np.minimum.accumulate(x, axis=1))
     # fp32 sums: numpy's cumsum is the same left-to-right fp32 accumulation
     assert np.array_equal(O.axis_scan("sum", x), np.cumsum(x, axis=1, dtype=np.float32))
+
+
+def test_circular_convolution_is_a_circular_correlation(O, rng):
+    # integer-valued data: exact against the definition written with numpy's roll
+    c = rng.randint(-4, 5, (3, 11)).astype(np.float32)
+    w = rng.randint(-4, 5, (3, 11)).astype(np.float32)
+    want = np.stack([sum(np.roll(c[r], -s) * w[r, s] for s in range(11)) for r in range(3)])
+    assert np.array_equal(O.circular_convolution(c, w), want)
+    # a one-hot weight at position s shifts the content left by s (circular_convolution.cpp:31-36)
+    e = np.zeros(7, np.float32)
+    e[2] = 1.0
+    x = np.arange(7, dtype=np.float32)
+    assert np.array_equal(O.circular_convolution(x, e), np.roll(x, -2))
+    # the circular-correlation theorem pins the general case: FFT(out) = FFT(c) * conj(FFT(w)) for real w
+    cf, wf = rng.randn(2, 64), rng.randn(2, 64)
+    got = O.circular_convolution(cf, wf).astype(np.float64)
+    ref = np.fft.ifft(np.fft.fft(cf.astype(np.float32)) * np.conj(np.fft.fft(wf.astype(np.float32)))).real
+    assert np.abs(got - ref).max() < 1e-4
