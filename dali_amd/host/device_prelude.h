@@ -166,6 +166,16 @@ DI float dali_div_invariant(float x, float s) {
     }
     return x / s;
 }
+// The same with the reciprocal and the range test hoisted out of the element loop by the kernel generator.
+DI bool dali_div_ok(float s) {
+    const float a = __builtin_fabsf(s);
+    return a > 1e-30f && a < 1e30f;
+}
+DI float dali_div_fast(float x, float s, float r) {
+    const float q = x * r;
+    const float e = __builtin_fmaf(-q, s, x);
+    return __builtin_fmaf(e, r, q);
+}
 DI double dali_div_invariant(double x, double s) { return x / s; }
 DI int dali_div_invariant(int x, int s) { return x / s; }
 

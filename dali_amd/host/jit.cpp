@@ -20,6 +20,7 @@
 //   all   full reduction, two-stage through the workspace, optional scalar epilogue
 // Anything else is split: inner reductions are evaluated into temporaries first.
 #include <algorithm>
+#include <cctype>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -70,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-10";
+const char* const kCodegenVersion = "dali-hip-codegen-11";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -485,6 +486,7 @@ struct RowParams {
     bool cached = true;
     bool nt_loads = false;   // inputs are streamed once: bypass cache allocation
     bool nt_stores = true;   // outputs are not re-read by this kernel: streaming stores
+    bool exact = false;      // register-cached rows: C == TPR * EPT * VEC, the chunk guards fall away
 };
 
 int env_int(const char* name, int fallback) {
@@ -503,6 +505,23 @@ struct BodyEmitter {
     std::string leaf_suffix;  // "[e][j]" (cached) or "[j]" (streaming)
     int body_index;  // phase number, or number of phases for the output body
     const std::vector<int>* first_body;  // per node: first body that evaluates a kept node
+    // Divisions by a row constant: the generator hoists one reciprocal and one range test per divisor out of
+    // the element loop and emits the loop twice, `div_mode` 1 with product + FMA correction, 2 with the plain
+    // quotient; 0 keeps the self-contained per-element form. `divisors` collects the divisor expressions.
+    int div_mode = 0;
+    std::vector<std::string>* divisors = nullptr;
+    int divisor_index(const std::string& dv) {
+        for (size_t k = 0; k < divisors->size(); ++k)
+            if ((*divisors)[k] == dv) return (int)k;
+        divisors->push_back(dv);
+        return (int)divisors->size() - 1;
+    }
+    static bool simple_token(const std::string& s) {
+        if (s.empty()) return false;
+        for (char c : s)
+            if (!(isalnum((unsigned char)c) || c == '_' || c == '.' || c == '[' || c == ']')) return false;
+        return true;
+    }
 
     BodyEmitter(const Program& P_, const RowParams& rp_, bool per_el, int body, const std::vector<int>* fb)
         : P(P_), rp(rp_), per_element(per_el), body_index(body), first_body(fb) {
@@ -543,7 +562,13 @@ struct BodyEmitter {
             case Kind::ELEMENTWISE: {
                 if (n.name == "functor::eltdiv" && n.cls == Cls::FULL && n.args.size() == 2 && row_invariant(n.args[1])) {
                     // divisor constant along the row: reciprocal once, product + correction per element
-                    return "dali_div_invariant(" + value(n.args[0]) + ", " + value(n.args[1]) + ")";
+                    const std::string x = value(n.args[0]), dv = value(n.args[1]);
+                    if (divisors && n.dtype == DTYPE_FLOAT && P.nodes[n.args[1]].dtype == DTYPE_FLOAT && simple_token(dv)) {
+                        const int k = divisor_index(dv);
+                        if (div_mode == 1) return "dali_div_fast(" + x + ", " + dv + ", dr" + std::to_string(k) + ")";
+                        if (div_mode == 2) return "(" + x + " / " + dv + ")";
+                    }
+                    return "dali_div_invariant(" + x + ", " + dv + ")";
                 }
                 std::string s = n.name + "<" + ctype(n.dtype) + ">::Map(";
                 for (size_t i = 0; i < n.args.size(); ++i) s += (i ? ", " : "") + value(n.args[i]);
@@ -783,9 +808,14 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
     ss << "  const int tid = threadIdx.x;\n  const int tr = tid % TPR;\n";
     ss << "  const long R = A.iv[" << L.shape_pos[0] << "], C = A.iv[" << L.shape_pos[0] + 1 << "];\n";
     ss << "  long row = (long)blockIdx.x * RPB + tid / TPR;\n";
-    ss << "  const bool row_ok = row < R;\n  if (!row_ok) row = R - 1;\n";
-    ss << "  const int CH = (int)(C / VEC);\n";
+    if (rp.RPB == 1)
+        ss << "  constexpr bool row_ok = true;  // one row per workgroup: the grid has exactly R of them\n  (void)R;\n";
+    else
+        ss << "  const bool row_ok = row < R;\n  if (!row_ok) row = R - 1;\n";
+    ss << "  const int CH = (int)(C / VEC); (void)CH;\n";
     emit_row_prologue(ss, P, L);
+    // register-cached rows whose length fills every chunk need no chunk guard
+    const std::string chunk_guard = rp.cached && rp.exact ? "    {\n" : "    if (ch < CH) {\n";
 
     // FULL leaves (inputs)
     std::vector<int> full_leaves;
@@ -796,7 +826,7 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
         for (int i : full_leaves) {
             ss << "  " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[EPT][VEC];\n";
         }
-        ss << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n    if (ch < CH) {\n";
+        ss << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n" << chunk_guard;
         for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i) + "[e]", "      ", rp.nt_loads);
         ss << "    }\n  }\n";
         for (size_t id = 0; id < P.nodes.size(); ++id)
@@ -804,7 +834,7 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
     }
     auto open_loop = [&](std::ostringstream& o) {
         if (rp.cached) {
-            o << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n    if (ch < CH) {\n";
+            o << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n" << chunk_guard;
         } else {
             o << "  for (int ch = tr; ch < CH; ch += TPR) {\n    {\n";
             for (int i : full_leaves) {
@@ -812,6 +842,30 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
                 emit_leaf_load(o, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", rp.nt_loads);
             }
         }
+    };
+
+    // A loop whose body divides by row constants is emitted twice behind one wave-uniform test: with the
+    // reciprocals (product + FMA correction per element) when every divisor of the wave's rows has a normal
+    // reciprocal, with plain quotients otherwise. Neither copy has a branch per element.
+    int div_plans = 0;
+    auto emit_with_division_plan = [&](std::ostringstream& o, const std::function<void(std::ostringstream&, int, std::vector<std::string>*)>& emit_loop) {
+        std::vector<std::string> divisors;
+        std::ostringstream probe;
+        emit_loop(probe, 1, &divisors);
+        if (divisors.empty()) {
+            emit_loop(o, 0, nullptr);
+            return;
+        }
+        const int plan = div_plans++;
+        o << "  bool div_ok" << plan << " = true;\n";
+        o << "  {\n";
+        // the reciprocals live in this scope together with both copies of the loop
+        for (size_t k = 0; k < divisors.size(); ++k)
+            o << "  const float dr" << k << " = 1.0f / " << divisors[k] << ";\n  div_ok" << plan << " = div_ok" << plan << " && dali_div_ok(" << divisors[k] << ");\n";
+        o << "  if (__all(div_ok" << plan << ")) {\n" << probe.str() << "  } else {\n";
+        std::vector<std::string> again;
+        emit_loop(o, 2, &again);
+        o << "  }\n  }\n";
     };
 
     // reduction phases
@@ -823,24 +877,29 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
             ss << "  " << t << " acc" << id << " = " << n.name << "::init<" << t << ">();\n";
             if (n.kind == Kind::ARG_AXIS_REDUCE) ss << "  int acci" << id << " = 0;\n";
         }
-        open_loop(ss);
-        ss << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        const int col = ch * VEC + j; (void)col;\n";
-        BodyEmitter be(P, rp, true, p, &rpn.first_body);
-        std::vector<std::string> updates;
-        for (int id : reds) {
-            const PNode& n = P.nodes[id];
-            std::string t = ctype(P.nodes[n.args[0]].dtype);
-            std::string v = be.value(n.args[0]);
-            if (n.kind == Kind::AXIS_REDUCE) {
-                updates.push_back("acc" + std::to_string(id) + " = " + n.name + "::step<" + t + ">(acc" + std::to_string(id) + ", " + v + ");");
-            } else {
-                updates.push_back("{ const " + t + " cand = " + v + "; if (" + n.name + "::better<" + t + ">(cand, acc" + std::to_string(id) +
-                                  ")) { acc" + std::to_string(id) + " = cand; acci" + std::to_string(id) + " = col; } }");
+        auto emit_phase_loop = [&](std::ostringstream& o, int div_mode, std::vector<std::string>* divisors) {
+            open_loop(o);
+            o << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        const int col = ch * VEC + j; (void)col;\n";
+            BodyEmitter be(P, rp, true, p, &rpn.first_body);
+            be.div_mode = div_mode;
+            be.divisors = divisors;
+            std::vector<std::string> updates;
+            for (int id : reds) {
+                const PNode& n = P.nodes[id];
+                std::string t = ctype(P.nodes[n.args[0]].dtype);
+                std::string v = be.value(n.args[0]);
+                if (n.kind == Kind::AXIS_REDUCE) {
+                    updates.push_back("acc" + std::to_string(id) + " = " + n.name + "::step<" + t + ">(acc" + std::to_string(id) + ", " + v + ");");
+                } else {
+                    updates.push_back("{ const " + t + " cand = " + v + "; if (" + n.name + "::better<" + t + ">(cand, acc" + std::to_string(id) +
+                                      ")) { acc" + std::to_string(id) + " = cand; acci" + std::to_string(id) + " = col; } }");
+                }
             }
-        }
-        ss << be.stmts.str();
-        for (auto& u : updates) ss << "        " << u << "\n";
-        ss << "      }\n    }\n  }\n";
+            o << be.stmts.str();
+            for (auto& u : updates) o << "        " << u << "\n";
+            o << "      }\n    }\n  }\n";
+        };
+        emit_with_division_plan(ss, emit_phase_loop);
         for (int id : reds) {
             const PNode& n = P.nodes[id];
             std::string t = ctype(P.nodes[n.args[0]].dtype);
@@ -867,33 +926,38 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
     bool any_full = false;
     for (const Output& o : rpn.outputs) any_full = any_full || o.cls == Cls::FULL;
     if (any_full) {
-        open_loop(ss);
-        ss << "      if (row_ok) {\n";
-        BodyEmitter be(P, rp, true, rpn.n_phases, &rpn.first_body);
-        std::ostringstream pre, body, post;
-        for (const Output& o : rpn.outputs) {
-            if (o.cls != Cls::FULL) continue;
-            const ArrayArg& d = P.arrays[o.array];
-            std::string t = ctype(d.buf->dtype);
-            std::string ov = "o" + std::to_string(o.array);
-            if (rp.VEC > 1) {
-                pre << "        dali_vec<" << t << ", VEC> " << ov << ";\n";
-                if (o.op != OPERATOR_T_EQL) pre << "        " << ov << " = dali_load<" << t << ", VEC>(q" << o.array << " + (long)ch * VEC);\n";
-                post << "        " << (rp.nt_stores ? "dali_store_nt<" : "dali_store<") << t << ", VEC>(q" << o.array << " + (long)ch * VEC, " << ov << ");\n";
-            } else {
-                std::string cs = d.strided ? " * cs" + std::to_string(o.array) : "";
-                pre << "        dali_vec<" << t << ", 1> " << ov << ";\n";
-                if (o.op != OPERATOR_T_EQL) pre << "        " << ov << ".v[0] = q" << o.array << "[(long)ch" << cs << "];\n";
-                post << "        q" << o.array << "[(long)ch" << cs << "] = " << ov << ".v[0];\n";
+        auto emit_output_loop = [&](std::ostringstream& os, int div_mode, std::vector<std::string>* divisors) {
+            open_loop(os);
+            os << "      if (row_ok) {\n";
+            BodyEmitter be(P, rp, true, rpn.n_phases, &rpn.first_body);
+            be.div_mode = div_mode;
+            be.divisors = divisors;
+            std::ostringstream pre, body, post;
+            for (const Output& o : rpn.outputs) {
+                if (o.cls != Cls::FULL) continue;
+                const ArrayArg& d = P.arrays[o.array];
+                std::string t = ctype(d.buf->dtype);
+                std::string ov = "o" + std::to_string(o.array);
+                if (rp.VEC > 1) {
+                    pre << "        dali_vec<" << t << ", VEC> " << ov << ";\n";
+                    if (o.op != OPERATOR_T_EQL) pre << "        " << ov << " = dali_load<" << t << ", VEC>(q" << o.array << " + (long)ch * VEC);\n";
+                    post << "        " << (rp.nt_stores ? "dali_store_nt<" : "dali_store<") << t << ", VEC>(q" << o.array << " + (long)ch * VEC, " << ov << ");\n";
+                } else {
+                    std::string cs = d.strided ? " * cs" + std::to_string(o.array) : "";
+                    pre << "        dali_vec<" << t << ", 1> " << ov << ";\n";
+                    if (o.op != OPERATOR_T_EQL) pre << "        " << ov << ".v[0] = q" << o.array << "[(long)ch" << cs << "];\n";
+                    post << "        q" << o.array << "[(long)ch" << cs << "] = " << ov << ".v[0];\n";
+                }
+                std::string v = be.value(o.root);
+                body << "          " << ov << ".v[j] = " << op_combine(o.op, ov + ".v[j]", "(" + t + ")(" + v + ")") << ";\n";
             }
-            std::string v = be.value(o.root);
-            body << "          " << ov << ".v[j] = " << op_combine(o.op, ov + ".v[j]", "(" + t + ")(" + v + ")") << ";\n";
-        }
-        ss << pre.str();
-        ss << "        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n          const int col = ch * VEC + j; (void)col;\n";
-        ss << be.stmts.str() << body.str();
-        ss << "        }\n" << post.str();
-        ss << "      }\n    }\n  }\n";
+            os << pre.str();
+            os << "        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n          const int col = ch * VEC + j; (void)col;\n";
+            os << be.stmts.str() << body.str();
+            os << "        }\n" << post.str();
+            os << "      }\n    }\n  }\n";
+        };
+        emit_with_division_plan(ss, emit_output_loop);
     }
     // ROW / SCAL destinations: one thread per row writes
     bool any_row = false;
@@ -1127,6 +1191,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
     }
     rp.RPB = rp.BT / rp.TPR;
     rp.NW = rp.TPR > 64 ? rp.TPR / 64 : 1;
+    rp.exact = nph > 0 && rp.cached && dom.C == (int64_t)rp.TPR * rp.EPT * rp.VEC;
     // A 1024-thread row block fills a CU by itself unless it stays within 64 VGPRs; two resident
     // blocks let one row's loads overlap another row's arithmetic.
     static const int wpe = env_int("DALI_HIP_ROW_WAVES_PER_EU", -1);
@@ -1173,7 +1238,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
     rp.nt_loads = nt_l >= 0 ? nt_l != 0 : dom.R * dom.C * (int64_t)max_el >= ((int64_t)64 << 20);
     rp.nt_stores = nt_s >= 0 ? nt_s != 0 : true;
     params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached << "," << rp.waves_per_eu << ","
-           << rp.nt_loads << rp.nt_stores;
+           << rp.nt_loads << rp.nt_stores << rp.exact;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     std::string sig = signature(P, rpn.outputs);
     uint64_t h = kernel_hash("row", sig, params.str());
