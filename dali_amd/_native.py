@@ -139,6 +139,14 @@ FRONT_SYMBOLS = {
     "dali_fe_diag": (H, [H, _i, _i]),
     "dali_fe_outer": (H, [H, H]),
     "dali_fe_circular_convolution": (H, [H, H]),
+    "dali_fe_im2col": (H, [H] + [_i] * 8 + [C.c_char_p]),
+    "dali_fe_col2im": (H, [H, _ip, _i, _i, _i, _i, _i, C.c_char_p]),
+    "dali_fe_conv2d": (H, [H, H, _i, _i, _i, C.c_char_p]),
+    "dali_fe_conv2d_backward_input": (H, [H, H, _i, _i, _ip, _i, C.c_char_p]),
+    "dali_fe_conv2d_backward_filters": (H, [H, H, _i, _i, _ip, _i, C.c_char_p]),
+    "dali_fe_conv2d_backward_bias": (H, [H, C.c_char_p]),
+    "dali_fe_pool2d": (H, [H, _i, _i, _i, _i, _i, _i, C.c_char_p]),
+    "dali_fe_pool2d_backward": (H, [H, H, H, _i, _i, _i, _i, _i, _i, C.c_char_p]),
     "dali_fe_autoreduce_assign": (_i, [H, H]),
     "dali_fe_one_hot": (H, [H, _i, H, H]),
     "dali_fe_dot": (H, [H, H]),

@@ -870,6 +870,262 @@ Array circular_convolution(Array x, Array weights) {
     return make_node(Kind::CIRCULAR_CONV, "", {xb, wb}, shape, x.dtype());
 }
 
+// ---------------------------------------------------------------- sliding windows
+// dali/array/op/spatial_utils.cpp:33-50
+void check_data_format(const std::string& data_format, int* n_dim, int* c_dim, int* h_dim, int* w_dim) {
+    DALI_ASSERT(data_format.size() == 4, make_message("data_format should be a 4 character string containing the letters N, C, H and W (got ",
+                                                      data_format, ")."));
+    const char letters[4] = {'N', 'C', 'H', 'W'};
+    int* outs[4] = {n_dim, c_dim, h_dim, w_dim};
+    for (int k = 0; k < 4; ++k) {
+        size_t pos = data_format.find(letters[k]);
+        DALI_ASSERT(pos != std::string::npos, make_message("data_format should contain character '", letters[k], "' (got ", data_format, ")."));
+        *outs[k] = (int)pos;
+    }
+}
+
+static int int_ceil(int numerator, int denominator) { return (numerator + denominator - 1) / denominator; }
+
+// dali/array/op/spatial_utils.cpp:52-91
+template <typename Info>
+static Info sliding_window_info(const std::vector<int>& input_shape, int window_h, int window_w, int stride_h, int stride_w, PADDING_T padding,
+                                const std::string& data_format) {
+    int n_dim, c_dim, h_dim, w_dim;
+    check_data_format(data_format, &n_dim, &c_dim, &h_dim, &w_dim);
+    DALI_ASSERT(input_shape.size() == 4, make_message("sliding-window geometry needs a 4 dimensional shape (got ", shape_str(input_shape), ")."));
+    DALI_ASSERT(stride_h > 0 && stride_w > 0, make_message("strides must be strictly positive (got stride_h=", stride_h, ", stride_w=", stride_w, ")."));
+    DALI_ASSERT(padding == PADDING_T_SAME || padding == PADDING_T_VALID, make_message("expected padding to be SAME or VALID (got ", (int)padding, ")."));
+    Info info;
+    info.batch_size = input_shape[n_dim];
+    info.in_channels = input_shape[c_dim];
+    info.in_h = input_shape[h_dim];
+    info.in_w = input_shape[w_dim];
+    if (padding == PADDING_T_SAME) {
+        info.out_h = int_ceil(info.in_h, stride_h);
+        info.out_w = int_ceil(info.in_w, stride_w);
+        info.padding_h = std::max(0, (info.out_h - 1) * stride_h + window_h - info.in_h);
+        info.padding_w = std::max(0, (info.out_w - 1) * stride_w + window_w - info.in_w);
+    } else {
+        info.out_h = int_ceil(info.in_h - window_h + 1, stride_h);
+        info.out_w = int_ceil(info.in_w - window_w + 1, stride_w);
+        info.padding_h = 0;
+        info.padding_w = 0;
+    }
+    info.odd_padding_h = info.padding_h % 2;
+    info.odd_padding_w = info.padding_w % 2;
+    info.padding_h /= 2;
+    info.padding_w /= 2;
+    info.stride_h = stride_h;
+    info.stride_w = stride_w;
+    return info;
+}
+
+PoolFunctionInfo compute_pool_info(const std::vector<int>& input_shape, int window_h, int window_w, int stride_h, int stride_w,
+                                   PADDING_T padding, const std::string& data_format) {
+    PoolFunctionInfo info = sliding_window_info<PoolFunctionInfo>(input_shape, window_h, window_w, stride_h, stride_w, padding, data_format);
+    info.window_h = window_h;
+    info.window_w = window_w;
+    return info;
+}
+
+// dali/array/op/spatial_utils.cpp:110-131
+ConvFunctionInfo compute_conv2d_info(const std::vector<int>& input_shape, const std::vector<int>& filters_shape, int stride_h,
+                                     int stride_w, PADDING_T padding, const std::string& data_format) {
+    int n_dim, c_dim, h_dim, w_dim;
+    check_data_format(data_format, &n_dim, &c_dim, &h_dim, &w_dim);
+    DALI_ASSERT(filters_shape.size() == 4, make_message("filters must be 4 dimensional (got ", shape_str(filters_shape), ")."));
+    const int filter_h = filters_shape[h_dim], filter_w = filters_shape[w_dim];
+    ConvFunctionInfo info = sliding_window_info<ConvFunctionInfo>(input_shape, filter_h, filter_w, stride_h, stride_w, padding, data_format);
+    DALI_ASSERT(info.in_channels == filters_shape[c_dim],
+                make_message("conv2d input and filters need to have the same number of input channels (got filters input channels = ",
+                             filters_shape[c_dim], ", and image input channels = ", info.in_channels, ")."));
+    info.filter_h = filter_h;
+    info.filter_w = filter_w;
+    info.out_channels = filters_shape[n_dim];
+    return info;
+}
+
+// a 3-D image has no N dimension: the positions of the other letters close up
+static std::vector<int> with_batch_axis(const std::vector<int>& shape, int n_dim) {
+    std::vector<int> s = shape;
+    if (s.size() == 3) s.insert(s.begin() + n_dim, 1);
+    return s;
+}
+
+// dali/array/op/im2col.cpp:151-188
+std::vector<int> im2col_shape(const std::vector<int>& src_shape, int filter_h, int filter_w, int stride_h, int stride_w, int dilate_h,
+                              int dilate_w, int prepad_h, int prepad_w, int postpad_h, int postpad_w, const std::string& data_format) {
+    int n_dim, c_dim, h_dim, w_dim;
+    check_data_format(data_format, &n_dim, &c_dim, &h_dim, &w_dim);
+    const std::vector<int> s = with_batch_axis(src_shape, n_dim);
+    const int i_height = s[h_dim] + prepad_h + postpad_h, i_width = s[w_dim] + prepad_w + postpad_w;
+    const int o_height = (i_height - (dilate_h * (filter_h - 1) + 1)) / stride_h + 1;
+    const int o_width = (i_width - (dilate_w * (filter_w - 1) + 1)) / stride_w + 1;
+    return {filter_h * filter_w * s[c_dim], o_height * o_width * s[n_dim]};
+}
+
+// dali/array/op/im2col.cpp:190-267
+Array im2col(const Array& image_in, int filter_h, int filter_w, int stride_h, int stride_w, int padding_h, int padding_w, int postpad_h,
+             int postpad_w, const std::string& data_format) {
+    const int image_ndim = image_in.ndim();
+    DALI_ASSERT(image_ndim == 3 || image_ndim == 4, make_message("im2col takes an image with ndim == 3 or ndim == 4 (got ndim=", image_ndim, ")."));
+    int n_dim, c_dim, h_dim, w_dim;
+    check_data_format(data_format, &n_dim, &c_dim, &h_dim, &w_dim);
+    Array image = image_ndim == 3 ? image_in.expand_dims(n_dim) : image_in;
+    const int image_h = image.shape()[h_dim], image_w = image.shape()[w_dim];
+    DALI_ASSERT(image_w >= filter_w && image_h >= filter_h,
+                make_message("the image of im2col with data_format=", data_format, " should not be smaller than the filter (filter_h=", filter_h,
+                             " vs. image_h=", image_h, ", filter_w=", filter_w, " vs. image_w=", image_w, ")."));
+    DALI_ASSERT(filter_h > 0 && filter_w > 0 && stride_h > 0 && stride_w > 0, "im2col: filter sizes and strides must be strictly positive.");
+    DALI_ASSERT(padding_h >= 0, make_message("padding_h should be a positive value (got ", padding_h, ")."));
+    DALI_ASSERT(padding_w >= 0, make_message("padding_w should be a positive value (got ", padding_w, ")."));
+    DALI_ASSERT(postpad_h >= 0, make_message("postpad_h should be a positive value (got ", postpad_h, ")."));
+    DALI_ASSERT(postpad_w >= 0, make_message("postpad_w should be a positive value (got ", postpad_w, ")."));
+    const int dilate_h = 1, dilate_w = 1;
+    Array out = make_node(Kind::IM2COL, "", {image},
+                          im2col_shape(image.shape(), filter_h, filter_w, stride_h, stride_w, dilate_h, dilate_w, padding_h, padding_w,
+                                       postpad_h, postpad_w, data_format),
+                          image.dtype());
+    out.expression()->geom = {filter_h, filter_w, stride_h, stride_w, dilate_h, dilate_w, padding_h, padding_w, postpad_h, postpad_w};
+    out.expression()->data_format = data_format;
+    return out;
+}
+
+// dali/array/op/col2im.cpp:165-233
+Array col2im(const Array& input, const std::vector<int>& image_shape_in, int filter_h, int filter_w, int stride_h, int stride_w,
+             const std::string& data_format) {
+    DALI_ASSERT(input.ndim() == 2, make_message("col2im takes a 2D input (got ", input.ndim(), ")."));
+    const int image_ndim = (int)image_shape_in.size();
+    DALI_ASSERT(image_ndim == 3 || image_ndim == 4, make_message("col2im's image_shape should have size == 3 or 4 (got ", shape_str(image_shape_in), ")."));
+    int n_dim, c_dim, h_dim, w_dim;
+    check_data_format(data_format, &n_dim, &c_dim, &h_dim, &w_dim);
+    const std::vector<int> image_shape = with_batch_axis(image_shape_in, n_dim);
+    const int image_h = image_shape[h_dim], image_w = image_shape[w_dim], channels = image_shape[c_dim], batch = image_shape[n_dim];
+    DALI_ASSERT(filter_h > 0 && filter_w > 0 && stride_h > 0 && stride_w > 0, "col2im: filter sizes and strides must be strictly positive.");
+    DALI_ASSERT(image_w >= filter_w && image_h >= filter_h,
+                make_message("the image shape of col2im with data_format=", data_format, " should not be smaller than the filter (filter_h=",
+                             filter_h, " vs. image_h=", image_h, ", filter_w=", filter_w, " vs. image_w=", image_w, ")."));
+    DALI_ASSERT(filter_h * filter_w * channels == input.shape()[0],
+                make_message("col2im with data_format ", data_format, "'s input must have its first dimension be filter_h * filter_w * i_channel = ",
+                             filter_h * filter_w * channels, " (got ", input.shape()[0], ")."));
+    const int o_height = (image_h - filter_h) / stride_h + 1, o_width = (image_w - filter_w) / stride_w + 1;
+    DALI_ASSERT(o_height * o_width * batch == input.shape()[1],
+                make_message("col2im with data_format ", data_format, "'s input must have its second dimension be ", o_height * o_width * batch,
+                             " = out_h [", o_height, "] * out_w [", o_width, "] * batch_size [", batch, "] (got ", input.shape()[1], ")."));
+    Array out = make_node(Kind::COL2IM, "", {input}, image_shape, input.dtype());
+    out.expression()->geom = {filter_h, filter_w, stride_h, stride_w, 1, 1, 0, 0, 0, 0};
+    out.expression()->data_format = data_format;
+    // the 4-D form is what the kernel fills; a 3-D request is that buffer without its batch axis
+    return image_ndim == 3 ? out.squeeze(n_dim) : out;
+}
+
+static void check_nchw_or_nhwc(const char* name, const std::string& data_format) {
+    DALI_ASSERT(data_format == "NCHW" || data_format == "NHWC", make_message(name, "'s data_format must be NCHW or NHWC but got ", data_format, " instead."));
+}
+
+static void check_ndim4(const char* name, const char* array_name, const Array& a) {
+    DALI_ASSERT(a.ndim() == 4, make_message(name, "'s ", array_name, " must be 4 dimensional but got ", array_name, " with ndim = ", a.ndim(), "."));
+}
+
+// dali/array/op/conv.cpp:223-276: filters [out, ...] flattened to a matrix times the patch matrix
+Array conv2d(const Array& input, const Array& filters, int stride_h, int stride_w, PADDING_T padding, const std::string& data_format) {
+    DALI_ASSERT(input.ndim() == 3 || input.ndim() == 4, make_message("Input argument to conv2d must be 3D or 4D (got input.ndim=", input.ndim(), ")."));
+    check_ndim4("conv2d", "filters", filters);
+    int n_dim, c_dim, h_dim, w_dim;
+    check_data_format(data_format, &n_dim, &c_dim, &h_dim, &w_dim);
+    check_nchw_or_nhwc("conv2d", data_format);
+    ConvFunctionInfo info = compute_conv2d_info(with_batch_axis(input.shape(), n_dim), filters.shape(), stride_h, stride_w, padding, data_format);
+    Array filters_nxxx = filters.swapaxes(n_dim, 0);
+    Array filters_nX = filters_nxxx.reshape({filters_nxxx.shape()[0], -1});
+    Array patches = im2col(input, info.filter_h, info.filter_w, stride_h, stride_w, info.padding_h, info.padding_w,
+                           info.padding_h + info.odd_padding_h, info.padding_w + info.odd_padding_w, data_format);
+    if (data_format == "NCHW")
+        return dot(filters_nX, patches).reshape({info.out_channels, info.batch_size, info.out_h, info.out_w}).swapaxes(0, 1);
+    return dot(patches.transpose(), filters_nX.transpose()).reshape({info.batch_size, info.out_h, info.out_w, info.out_channels});
+}
+
+// dali/array/op/conv.cpp:278-336. The adjoint of im2col takes no padding (col2im.cpp:217-232), so, like the
+// reference, this is defined for convolutions whose windows tile the image without padding.
+Array conv2d_backward_input(Array filters, Array out_dw, int stride_h, int stride_w, const std::vector<int>& result_shape, PADDING_T padding,
+                            const std::string& data_format) {
+    check_ndim4("conv2d_backward_input", "out_dw", out_dw);
+    check_ndim4("conv2d_backward_input", "filters", filters);
+    check_nchw_or_nhwc("conv2d_backward_input", data_format);
+    DALI_ASSERT(result_shape.size() == 4, make_message("conv2d_backward_input's result_shape must be of size 4, but got ", shape_str(result_shape), "."));
+    ConvFunctionInfo info = compute_conv2d_info(result_shape, filters.shape(), stride_h, stride_w, padding, data_format);
+    Array filters2d = filters.reshape({filters.shape()[0], -1});  // [out, filter_h * filter_w * in]
+    if (data_format == "NCHW") {
+        Array out_dw_cnhw = out_dw.swapaxes(0, 1);
+        out_dw_cnhw = out_dw_cnhw.reshape({out_dw_cnhw.shape()[0], -1});
+        return col2im(dot(filters2d.transpose(), out_dw_cnhw), result_shape, info.filter_h, info.filter_w, stride_h, stride_w, data_format);
+    }
+    // NHWC: the patch-matrix gradient Filters^T . dOut^T is formed patch-major, as [N*h*w, window*c] = dOut . Filters, and handed
+    // over as its transposed view: the same numbers, laid out so that the channel run of a pixel is contiguous
+    Array out_dw2d = out_dw.reshape({-1, out_dw.shape()[3]});  // [N*h*w, out]
+    return col2im(dot(out_dw2d, filters2d).transpose(), result_shape, info.filter_h, info.filter_w, stride_h, stride_w, data_format);
+}
+
+// dali/array/op/conv.cpp:338-393
+Array conv2d_backward_filters(Array input, Array out_dw, int stride_h, int stride_w, const std::vector<int>& filters_shape, PADDING_T padding,
+                              const std::string& data_format) {
+    check_ndim4("conv2d_backward_filters", "out_dw", out_dw);
+    check_ndim4("conv2d_backward_filters", "input", input);
+    check_nchw_or_nhwc("conv2d_backward_filters", data_format);
+    DALI_ASSERT(filters_shape.size() == 4, make_message("conv2d_backward_filters's filters_shape must be of size 4, but got ", shape_str(filters_shape), "."));
+    ConvFunctionInfo info = compute_conv2d_info(input.shape(), filters_shape, stride_h, stride_w, padding, data_format);
+    Array patches_t = im2col(input, info.filter_h, info.filter_w, stride_h, stride_w, info.padding_h, info.padding_w,
+                             info.padding_h + info.odd_padding_h, info.padding_w + info.odd_padding_w, data_format).transpose();
+    if (data_format == "NCHW") {
+        Array out_dw_cnhw = out_dw.swapaxes(1, 0);
+        out_dw_cnhw = out_dw_cnhw.reshape({out_dw_cnhw.shape()[0], -1});
+        return dot(out_dw_cnhw, patches_t).reshape(filters_shape);
+    }
+    out_dw = out_dw.reshape({-1, out_dw.shape()[3]}).transpose();
+    return dot(out_dw, patches_t).reshape(filters_shape);
+}
+
+// dali/array/op/conv.cpp:395-401
+Array conv2d_backward_bias(Array out_dw, const std::string& data_format) {
+    check_ndim4("conv2d_backward_bias", "out_dw", out_dw);
+    int n_dim, c_dim, h_dim, w_dim;
+    check_data_format(data_format, &n_dim, &c_dim, &h_dim, &w_dim);
+    return sum(out_dw, {n_dim, h_dim, w_dim});
+}
+
+// dali/array/op/conv.cpp:403-428
+Array pool2d(const Array& input, int window_h, int window_w, int stride_h, int stride_w, POOLING_T pooling_mode, PADDING_T padding,
+             const std::string& data_format) {
+    check_ndim4("pool2d", "input", input);
+    check_nchw_or_nhwc("pool2d", data_format);
+    DALI_ASSERT(window_h > 0 && window_w > 0, make_message("pool2d windows must be strictly positive (got ", window_h, " x ", window_w, ")."));
+    PoolFunctionInfo info = compute_pool_info(input.shape(), window_h, window_w, stride_h, stride_w, padding, data_format);
+    const bool nchw = data_format == "NCHW";
+    std::vector<int> shape = nchw ? std::vector<int>{info.batch_size, info.in_channels, info.out_h, info.out_w}
+                                  : std::vector<int>{info.batch_size, info.out_h, info.out_w, info.in_channels};
+    Array out = make_node(Kind::POOL2D, pooling_mode == POOLING_T_MAX ? "reducers::maximum" : "reducers::avg", {input}, shape, input.dtype());
+    out.expression()->geom = {info.window_h, info.window_w, info.stride_h, info.stride_w, info.padding_h, info.padding_w};
+    out.expression()->data_format = data_format;
+    out.expression()->depth = pooling_mode == POOLING_T_AVG ? 1 : 0;
+    return out;
+}
+
+// dali/array/op/conv.cpp:430-456
+Array pool2d_backward(const Array& y, const Array& dy, const Array& x, int window_h, int window_w, int stride_h, int stride_w,
+                      POOLING_T pooling_mode, PADDING_T padding, const std::string& data_format) {
+    check_ndim4("pool2d_backward", "y", y);
+    check_ndim4("pool2d_backward", "dy", dy);
+    check_ndim4("pool2d_backward", "x", x);
+    check_nchw_or_nhwc("pool2d_backward", data_format);
+    PoolFunctionInfo info = compute_pool_info(x.shape(), window_h, window_w, stride_h, stride_w, padding, data_format);
+    DALI_ASSERT(y.shape() == dy.shape(), make_message("pool2d_backward: y ", shape_str(y.shape()), " and dy ", shape_str(dy.shape()), " must have the same shape."));
+    DALI_ASSERT(y.dtype() == dy.dtype() && y.dtype() == x.dtype(), "pool2d_backward: y, dy and x must have the same dtype.");
+    Array out = make_node(Kind::POOL2D_BACKWARD, pooling_mode == POOLING_T_MAX ? "reducers::maximum" : "reducers::avg", {y, dy, x}, x.shape(), y.dtype());
+    out.expression()->geom = {info.window_h, info.window_w, info.stride_h, info.stride_w, info.padding_h, info.padding_w};
+    out.expression()->data_format = data_format;
+    out.expression()->depth = pooling_mode == POOLING_T_AVG ? 1 : 0;
+    return out;
+}
+
 // dali/array/op/one_hot.cpp:62-74
 Array one_hot(Array indices, int depth, Array on_value, Array off_value) {
     DALI_ASSERT(indices.dtype() == DTYPE_INT32, "indices must be integers.");

@@ -116,6 +116,47 @@ dali_array_t dali_fe_arange(dali_array_t start, dali_array_t stop, dali_array_t 
 }
 dali_array_t dali_fe_diag(dali_array_t diagonal, int rows, int cols) { FE_TRY(return wrap(dali::op::diag(A(diagonal), rows, cols));, nullptr) }
 dali_array_t dali_fe_circular_convolution(dali_array_t x, dali_array_t w) { FE_TRY(return wrap(dali::op::circular_convolution(A(x), A(w)));, nullptr) }
+dali_array_t dali_fe_im2col(dali_array_t image, int filter_h, int filter_w, int stride_h, int stride_w, int padding_h, int padding_w,
+                            int postpad_h, int postpad_w, const char* data_format) {
+    FE_TRY(return wrap(dali::op::im2col(A(image), filter_h, filter_w, stride_h, stride_w, padding_h, padding_w, postpad_h, postpad_w, data_format));
+           , nullptr)
+}
+dali_array_t dali_fe_col2im(dali_array_t input, const int* image_shape, int image_ndim, int filter_h, int filter_w, int stride_h,
+                            int stride_w, const char* data_format) {
+    FE_TRY(return wrap(dali::op::col2im(A(input), std::vector<int>(image_shape, image_shape + image_ndim), filter_h, filter_w, stride_h, stride_w,
+                                        data_format));
+           , nullptr)
+}
+dali_array_t dali_fe_conv2d(dali_array_t input, dali_array_t filters, int stride_h, int stride_w, int padding, const char* data_format) {
+    FE_TRY(return wrap(dali::op::conv2d(A(input), A(filters), stride_h, stride_w, (dali::PADDING_T)padding, data_format));, nullptr)
+}
+dali_array_t dali_fe_conv2d_backward_input(dali_array_t filters, dali_array_t out_dw, int stride_h, int stride_w, const int* input_shape,
+                                           int padding, const char* data_format) {
+    FE_TRY(return wrap(dali::op::conv2d_backward_input(A(filters), A(out_dw), stride_h, stride_w, std::vector<int>(input_shape, input_shape + 4),
+                                                       (dali::PADDING_T)padding, data_format));
+           , nullptr)
+}
+dali_array_t dali_fe_conv2d_backward_filters(dali_array_t input, dali_array_t out_dw, int stride_h, int stride_w, const int* filters_shape,
+                                             int padding, const char* data_format) {
+    FE_TRY(return wrap(dali::op::conv2d_backward_filters(A(input), A(out_dw), stride_h, stride_w,
+                                                         std::vector<int>(filters_shape, filters_shape + 4), (dali::PADDING_T)padding, data_format));
+           , nullptr)
+}
+dali_array_t dali_fe_conv2d_backward_bias(dali_array_t out_dw, const char* data_format) {
+    FE_TRY(return wrap(dali::op::conv2d_backward_bias(A(out_dw), data_format));, nullptr)
+}
+dali_array_t dali_fe_pool2d(dali_array_t input, int window_h, int window_w, int stride_h, int stride_w, int pooling, int padding,
+                            const char* data_format) {
+    FE_TRY(return wrap(dali::op::pool2d(A(input), window_h, window_w, stride_h, stride_w, (dali::POOLING_T)pooling, (dali::PADDING_T)padding,
+                                        data_format));
+           , nullptr)
+}
+dali_array_t dali_fe_pool2d_backward(dali_array_t out, dali_array_t out_dw, dali_array_t in, int window_h, int window_w, int stride_h,
+                                     int stride_w, int pooling, int padding, const char* data_format) {
+    FE_TRY(return wrap(dali::op::pool2d_backward(A(out), A(out_dw), A(in), window_h, window_w, stride_h, stride_w, (dali::POOLING_T)pooling,
+                                                 (dali::PADDING_T)padding, data_format));
+           , nullptr)
+}
 dali_array_t dali_fe_outer(dali_array_t a, dali_array_t b) { FE_TRY(return wrap(dali::op::outer(A(a), A(b)));, nullptr) }
 dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_value, dali_array_t off_value) {
     FE_TRY(return wrap(dali::op::one_hot(A(indices), depth, A(on_value), A(off_value)));, nullptr)

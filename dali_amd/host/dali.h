@@ -66,6 +66,10 @@ class SynchronizedMemory {
 struct Expr;
 struct ArrayState;
 
+// dali/array/op/spatial_enums.h
+enum PADDING_T { PADDING_T_SAME = 0, PADDING_T_VALID = 1 };
+enum POOLING_T { POOLING_T_MAX = 0, POOLING_T_AVG = 1 };
+
 class Array {
   public:
     Array();
@@ -263,6 +267,42 @@ Array diag(const Array& diagonal, int rows, int cols);
 Array outer(const Array& a, const Array& b);
 // dali/array/op/circular_convolution.h
 Array circular_convolution(Array x, Array weights);
+
+// dali/array/op/spatial_utils.h: geometry of sliding-window operators
+void check_data_format(const std::string& data_format, int* n_dim, int* c_dim, int* h_dim, int* w_dim);
+struct SlidingWindowFunctionInfo {
+    int out_w, out_h, batch_size, in_channels, in_h, in_w;
+    int padding_h, padding_w, odd_padding_h, odd_padding_w, stride_h, stride_w;
+};
+struct PoolFunctionInfo : SlidingWindowFunctionInfo {
+    int window_h, window_w;
+};
+struct ConvFunctionInfo : SlidingWindowFunctionInfo {
+    int filter_h, filter_w, out_channels;
+};
+PoolFunctionInfo compute_pool_info(const std::vector<int>& input_shape, int window_h, int window_w, int stride_h, int stride_w,
+                                   PADDING_T padding, const std::string& data_format);
+ConvFunctionInfo compute_conv2d_info(const std::vector<int>& input_shape, const std::vector<int>& filters_shape, int stride_h,
+                                     int stride_w, PADDING_T padding, const std::string& data_format);
+// dali/array/op/im2col.h, col2im.h: the patch matrix [filter_h * filter_w * C, N * out_h * out_w] of an image whose
+// dimensions come in the order of the letters of data_format, and its adjoint
+std::vector<int> im2col_shape(const std::vector<int>& src_shape, int filter_h, int filter_w, int stride_h, int stride_w, int dilate_h,
+                              int dilate_w, int prepad_h, int prepad_w, int postpad_h, int postpad_w, const std::string& data_format);
+Array im2col(const Array& image, int filter_h, int filter_w, int stride_h, int stride_w, int padding_h, int padding_w, int postpad_h,
+             int postpad_w, const std::string& data_format);
+Array col2im(const Array& input, const std::vector<int>& image_shape, int filter_h, int filter_w, int stride_h, int stride_w,
+             const std::string& data_format);
+// dali/array/op/conv.h: convolution as im2col + one matrix product, and pooling
+Array conv2d(const Array& input, const Array& filters, int stride_h, int stride_w, PADDING_T padding, const std::string& data_format);
+Array conv2d_backward_input(Array filters, Array out_dw, int stride_h, int stride_w, const std::vector<int>& input_shape,
+                            PADDING_T padding, const std::string& data_format);
+Array conv2d_backward_filters(Array input, Array out_dw, int stride_h, int stride_w, const std::vector<int>& filters_shape,
+                              PADDING_T padding, const std::string& data_format);
+Array conv2d_backward_bias(Array out_dw, const std::string& data_format);
+Array pool2d(const Array& input, int window_h, int window_w, int stride_h, int stride_w, POOLING_T pooling_mode, PADDING_T padding,
+             const std::string& data_format);
+Array pool2d_backward(const Array& out, const Array& out_dw, const Array& in, int window_h, int window_w, int stride_h, int stride_w,
+                      POOLING_T pooling_mode, PADDING_T padding, const std::string& data_format);
 Array& autoreduce_assign(Array& left, const Array& right);
 Array one_hot(Array indices, int depth, Array on_value, Array off_value);
 Array matmul(Array a, Array b);

@@ -24,6 +24,10 @@ enum class Kind {
     ARANGE,            // dali/array/op/arange.cpp:8-39 (args: start, step scalars)
     DIAG,              // dali/array/op/eye.cpp:8-44 (args: diagonal vector or scalar)
     CIRCULAR_CONV,     // dali/array/op/circular_convolution.cpp:8-86 (args: content, weights, both of the node's shape)
+    IM2COL,            // dali/array/op/im2col.cpp:11-148 (args: image; geom, data_format)
+    COL2IM,            // dali/array/op/col2im.cpp:27-162 (args: patch matrix; shape = image shape)
+    POOL2D,            // dali/array/op/conv.cpp:12-112 (name = reducer, depth = 1 for the average)
+    POOL2D_BACKWARD,   // dali/array/op/conv.cpp:114-212 (args: y, dy, x)
     ONE_HOT,           // dali/array/op/one_hot.cpp:16-74
     MATMUL             // dali/array/op/dot.cpp:18-47
 };
@@ -46,6 +50,11 @@ struct Expr {
 
     int axis = 0;   // EXPAND_DIMS
     int depth = 0;  // ONE_HOT
+
+    // sliding-window nodes. IM2COL / COL2IM: filter_h, filter_w, stride_h, stride_w, dilate_h, dilate_w, prepad_h,
+    // prepad_w, postpad_h, postpad_w; POOL2D / POOL2D_BACKWARD: window_h, window_w, stride_h, stride_w, prepad_h, prepad_w
+    std::vector<int> geom;
+    std::string data_format;  // a permutation of "NCHW": the order of the image's dimensions
 
     int numel() const {
         int64_t n = 1;

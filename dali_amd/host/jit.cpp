@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-11";
+const char* const kCodegenVersion = "dali-hip-codegen-12";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -2217,6 +2217,10 @@ bool is_plain_matmul(const Array& a) { return a.expression()->kind == Kind::MATM
 Array run_scan(const Array& arg_in, const std::string& reducer, bool inclusive);
 Array run_fill(const std::shared_ptr<Expr>& e);
 Array run_circular_convolution(const Array& x, const Array& w);
+Array run_im2col(const Expr& e, const Array& image);
+Array run_col2im(const Expr& e, const Array& patches);
+Array run_pool2d(const Expr& e, const Array& x);
+Array run_pool2d_backward(const Expr& e, const Array& y, const Array& dy, const Array& x);
 
 Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root) {
     auto e = a.expression();
@@ -2274,6 +2278,18 @@ Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root) {
             out = run_circular_convolution(x, w);
             break;
         }
+        case Kind::IM2COL:
+            out = run_im2col(*e, clean(e->args[0], memo, false));
+            break;
+        case Kind::COL2IM:
+            out = run_col2im(*e, clean(e->args[0], memo, false));
+            break;
+        case Kind::POOL2D:
+            out = run_pool2d(*e, clean(e->args[0], memo, false));
+            break;
+        case Kind::POOL2D_BACKWARD:
+            out = run_pool2d_backward(*e, clean(e->args[0], memo, false), clean(e->args[1], memo, false), clean(e->args[2], memo, false));
+            break;
         case Kind::GATHER: {
             // source and index are presented as buffers; the gather itself stays lazy only where the row
             // kernel can read through it: a [N, D] node that is the root or sits under same-shape
@@ -2906,6 +2922,349 @@ Array run_circular_convolution(const Array& x_in, const Array& w_in) {
         ss << "    for (int s = 0; s < n; ++s) {\n      res += c[off] * w[s];\n      off = off + 1 == n ? 0 : off + 1;\n    }\n    out[x] = res;\n  }\n}\n";
         return ss.str();
     }, P, {{(int)R, n}});
+    return dest;
+}
+
+// ------------------------------------------------------------ sliding windows
+// im2col, col2im and the pooling pair (dali/array/op/im2col.cpp, col2im.cpp, conv.cpp:12-212) are index remaps
+// bound by memory traffic. Images are read and written as dense arrays whose dimensions come in the order of
+// the data format's letters; the kernels take the four extents and element strides as (N, C, H, W), so one
+// source serves every layout. Index arithmetic is 32-bit (extents are ints, element counts below 2^31).
+struct ImageGeom {
+    int ext[4];     // N, C, H, W
+    int stride[4];  // element strides of a dense array in data_format order, as (N, C, H, W)
+};
+
+ImageGeom image_geom(const std::vector<int>& shape, const std::string& fmt) {
+    ImageGeom g;
+    const char letters[4] = {'N', 'C', 'H', 'W'};
+    std::vector<int> st = contiguous_strides(shape);
+    for (int k = 0; k < 4; ++k) {
+        const int pos = (int)fmt.find(letters[k]);
+        g.ext[k] = shape[pos];
+        g.stride[k] = st[pos];
+    }
+    return g;
+}
+
+Array dense_buffer(const Array& a) {
+    Array b = a.is_buffer() ? a : materialize(a);
+    return b.contiguous_memory() ? b : b.ascontiguousarray();
+}
+
+// The letters other than N, last to first: the digits of a patch-row index, fastest first
+// (dali/array/op/im2col.cpp:76-80 for N in position 0 or 1, where those lines name three different letters).
+std::string row_letters(const std::string& fmt) {
+    std::string r;
+    for (int p = 3; p >= 0; --p)
+        if (fmt[p] != 'N') r.push_back(fmt[p]);
+    return r;
+}
+
+// Source text: `row` -> c, kh, kw (im2col.cpp:93-110) and back (col2im.cpp:86-94); C, FH, FW are in scope.
+std::string emit_split_row(const std::string& fmt, const std::string& row) {
+    std::string l = row_letters(fmt), out = "unsigned rest_ = (unsigned)(" + row + ");\n";
+    for (int k = 0; k < 3; ++k) {
+        std::string ext = l[k] == 'C' ? "C" : (l[k] == 'H' ? "FH" : "FW"), name = l[k] == 'C' ? "c" : (l[k] == 'H' ? "kh" : "kw");
+        if (k < 2) out += "      const int " + name + " = (int)(rest_ % (unsigned)" + ext + "); rest_ /= (unsigned)" + ext + ";\n";
+        else out += "      const int " + name + " = (int)rest_;\n";
+    }
+    return out;
+}
+
+std::string emit_join_row(const std::string& fmt) {
+    std::string l = row_letters(fmt), expr;
+    for (int k = 2; k >= 0; --k) {
+        std::string ext = l[k] == 'C' ? "C" : (l[k] == 'H' ? "FH" : "FW"), name = l[k] == 'C' ? "c" : (l[k] == 'H' ? "kh" : "kw");
+        expr = expr.empty() ? name : "(" + expr + ") * " + ext + " + " + name;
+    }
+    return expr;
+}
+
+// One launch of a hand-laid-out kernel: `blocks` workgroups of 256 threads (the kernels stride over blocks, so a
+// capped grid still covers the work); `geom` travels as the integers behind the arrays' sizes.
+void launch_special(const char* kind, const std::string& sig, const Program& P, int64_t blocks, const std::vector<int>& geom,
+                    const std::function<std::string(const std::string&, const IvLayout&)>& gen) {
+    static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
+    uint64_t h = kernel_hash(kind, sig, "");
+    std::shared_ptr<KernelSpec>& K = specs_cache[h];
+    std::vector<int> shape_ndims = {2, (int)geom.size()};
+    IvLayout L = layout_iv(P, shape_ndims);
+    if (!K) {
+        K = std::make_shared<KernelSpec>();
+        K->hash = h;
+        K->kind = kind;
+        K->name = kernel_name(K->kind, h);
+        fill_plan_arrays(*K, P, shape_ndims);
+        K->plan.block_threads = 256;
+        K->plan.grid_kind = DALI_HIP_GRID_ELEMS;
+        K->plan.work_begin = L.shape_pos[0];
+        K->plan.work_count = 2;
+        K->plan.work_per_block = 256;
+        K->plan.max_blocks = 1 << 20;
+    }
+    const int nblocks = (int)std::min<int64_t>(std::max<int64_t>(blocks, 1), 1 << 20);
+    load_and_launch(*K, [&]() { return gen(K->name, L); }, P, {{nblocks, 256}, geom});
+}
+
+std::string special_head(const Program& P, const IvLayout& L, const std::string& kname, const std::string& t, int n_geom, const char* const* names) {
+    std::ostringstream ss;
+    ss << codegen::kDevicePrelude << kargs_struct(P, L);
+    ss << "extern \"C\" __global__ __launch_bounds__(256) void " << kname << "(KArgs A) {\n  typedef " << t << " T;\n";
+    for (int k = 0; k < n_geom; ++k) ss << "  const int " << names[k] << " = A.iv[" << L.shape_pos[1] + k << "]; (void)" << names[k] << ";\n";
+    return ss.str();
+}
+
+const char* const kPatchGeomNames[] = {"N", "C", "H", "W", "SN", "SC", "SH", "SW", "FH", "FW", "STH", "STW", "DH", "DW",
+                                       "PH", "PW", "OH", "OW", "ORS", "OCS"};
+
+std::vector<int> patch_geom(const Expr& e, const ImageGeom& g, int o_h, int o_w, int mat_row_stride, int mat_col_stride) {
+    return {g.ext[0], g.ext[1], g.ext[2], g.ext[3], g.stride[0], g.stride[1], g.stride[2], g.stride[3], e.geom[0], e.geom[1],
+            e.geom[2], e.geom[3], e.geom[4], e.geom[5], e.geom[6], e.geom[7], o_h, o_w, mat_row_stride, mat_col_stride};
+}
+
+// im2col. Two layouts of the same matrix, chosen so that both the gather and the store run along memory:
+//  - formats ending in "WC" (NHWC): for a patch and a filter row kh, the filter_w * C values are one contiguous
+//    run of the image, and they are consecutive rows (kh, kw, c) of one column. The matrix is stored patch-major
+//    ([N*out_h*out_w, filter_h*filter_w*C], returned as its transposed view): one wave copies one run.
+//  - every other format: row-major [filter_h*filter_w*C, N*out_h*out_w]; a thread owns a column (consecutive
+//    columns are consecutive output pixels, i.e. consecutive W) and walks a group of rows, whose decomposition
+//    into (c, kh, kw) is uniform over the workgroup.
+Array run_im2col(const Expr& e, const Array& image_in) {
+    Array image = dense_buffer(image_in);
+    const std::string& fmt = e.data_format;
+    ImageGeom g = image_geom(image.shape(), fmt);
+    const int fh = e.geom[0], fw = e.geom[1], sth = e.geom[2], stw = e.geom[3], dh = e.geom[4], dw = e.geom[5];
+    const int o_h = (g.ext[2] + e.geom[6] + e.geom[8] - (dh * (fh - 1) + 1)) / sth + 1;
+    const int o_w = (g.ext[3] + e.geom[7] + e.geom[9] - (dw * (fw - 1) + 1)) / stw + 1;
+    const int64_t rows = e.shape[0], cols = e.shape[1];
+    DALI_ASSERT(rows == (int64_t)fh * fw * g.ext[1] && cols == (int64_t)g.ext[0] * o_h * o_w, "internal: im2col shape does not match its geometry");
+    const bool patch_major = fmt[2] == 'W' && fmt[3] == 'C' && dh == 1 && dw == 1;
+    Array store = patch_major ? Array({(int)cols, (int)rows}, e.dtype) : Array({(int)rows, (int)cols}, e.dtype);
+    Array result = patch_major ? store.transpose() : store;
+    if (rows * cols == 0) return result;
+    DALI_ASSERT(rows * cols < ((int64_t)1 << 31), "im2col: the patch matrix must hold fewer than 2^31 elements");
+    std::string t = ctype(e.dtype);
+    Program P;
+    P.arrays.push_back(manual_arg(store, Cls::FULL, true, 2, store.shape(), {}));
+    P.arrays.push_back(manual_arg(image, Cls::FULL, false, 1, {(int)numel_of(image.shape())}, {}));
+    std::vector<int> geom = patch_geom(e, g, o_h, o_w, patch_major ? 1 : (int)cols, patch_major ? (int)rows : 1);
+    if (patch_major) {
+        const int VEC = (g.ext[1] % 4 == 0 && size_of_dtype(e.dtype) == 4 && image.offset() % 4 == 0) ? 4 : 1;
+        std::ostringstream sig;
+        sig << "im2col_wc|" << (int)e.dtype << "|" << VEC;
+        const int64_t units = cols * fh;  // (patch, filter row) pairs, one wave each
+        launch_special("im2col", sig.str(), P, (units + 3) / 4, geom, [&](const std::string& kname, const IvLayout& L) {
+            std::ostringstream ss;
+            ss << special_head(P, L, kname, t, 20, kPatchGeomNames);
+            ss << "  constexpr int VEC = " << VEC << ";\n";
+            ss << "  T* out = (T*)A.p[0];\n  const T* img = (const T*)A.p[1];\n";
+            ss << "  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;\n";
+            ss << "  const unsigned units = (unsigned)(N * OH * OW) * (unsigned)FH;\n  const int run = FW * C, rows = FH * run;\n";
+            ss << "  for (unsigned u = blockIdx.x * 4u + wave; u < units; u += gridDim.x * 4u) {\n";
+            ss << "    const unsigned col = u / (unsigned)FH; const int kh = (int)(u % (unsigned)FH);\n";
+            ss << "    const int ow = (int)(col % (unsigned)OW); const unsigned t1 = col / (unsigned)OW;\n";
+            ss << "    const int oh = (int)(t1 % (unsigned)OH), n = (int)(t1 / (unsigned)OH);\n";
+            ss << "    const int h = oh * STH - PH + kh, w0 = ow * STW - PW;\n";
+            ss << "    T* dst = out + (long)col * rows + kh * run;\n";
+            ss << "    // the run covers image columns w0 .. w0 + FW - 1 of row h: element j is valid when that column lies inside the image\n";
+            ss << "    const bool row_ok = h >= 0 && h < H;\n";
+            ss << "    const int jlo = w0 < 0 ? -w0 * C : 0, jhi = (W - w0) * C < run ? (W - w0) * C : run;\n";
+            ss << "    const T* src = img + (long)n * SN + (long)(row_ok ? h : 0) * SH + (long)w0 * C;\n";
+            ss << "    for (int j = lane * VEC; j < run; j += 64 * VEC) {\n";
+            ss << "      dali_vec<T, VEC> v;\n";
+            ss << "      if (row_ok && j >= jlo && j < jhi) v = dali_load<T, VEC>(src + j);\n";
+            ss << "      else { _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) v.v[k] = (T)0; }\n";
+            ss << "      dali_store<T, VEC>(dst + j, v);\n    }\n  }\n}\n";
+            return ss.str();
+        });
+    } else {
+        const int RB = 8;  // rows per workgroup
+        const int64_t col_tiles = (cols + 255) / 256, row_groups = (rows + RB - 1) / RB;
+        std::ostringstream sig;
+        sig << "im2col_rows|" << (int)e.dtype << "|" << row_letters(fmt);
+        launch_special("im2col", sig.str(), P, col_tiles * row_groups, geom, [&](const std::string& kname, const IvLayout& L) {
+            std::ostringstream ss;
+            ss << special_head(P, L, kname, t, 20, kPatchGeomNames);
+            ss << "  constexpr int RB = " << RB << ";\n";
+            ss << "  T* out = (T*)A.p[0];\n  const T* img = (const T*)A.p[1];\n";
+            ss << "  const unsigned cols = (unsigned)(N * OH * OW); const int rows = FH * FW * C;\n";
+            ss << "  const unsigned col_tiles = (cols + 255u) / 256u, total = col_tiles * (unsigned)((rows + RB - 1) / RB);\n";
+            ss << "  for (unsigned b = blockIdx.x; b < total; b += gridDim.x) {\n";
+            ss << "    const unsigned col = (b % col_tiles) * 256u + threadIdx.x; const int r0 = (int)(b / col_tiles) * RB;\n";
+            ss << "    if (col >= cols) continue;\n";
+            ss << "    const int ow = (int)(col % (unsigned)OW); const unsigned t1 = col / (unsigned)OW;\n";
+            ss << "    const int oh = (int)(t1 % (unsigned)OH), n = (int)(t1 / (unsigned)OH);\n";
+            ss << "    const int h0 = oh * STH - PH, w0 = ow * STW - PW;\n    const T* img_n = img + (long)n * SN;\n";
+            ss << "    for (int r = r0; r < r0 + RB && r < rows; ++r) {\n      " << emit_split_row(fmt, "r");
+            ss << "      const int h = h0 + kh * DH, w = w0 + kw * DW;\n";
+            ss << "      T v = (T)0;\n      if (h >= 0 && h < H && w >= 0 && w < W) v = img_n[(long)c * SC + (long)h * SH + (long)w * SW];\n";
+            ss << "      out[(long)r * cols + col] = v;\n    }\n  }\n}\n";
+            return ss.str();
+        });
+    }
+    return result;
+}
+
+// col2im: every image element sums, patch rows outermost, the entries of the patch matrix that im2col would have
+// copied it to (col2im.cpp:103-141): the same additions in the same order as the reference's loop. The patch
+// matrix is read through its strides, so the patch-major form produced for NHWC needs no copy.
+Array run_col2im(const Expr& e, const Array& patches_in) {
+    Array patches = patches_in.is_buffer() ? patches_in : materialize(patches_in);
+    const std::string& fmt = e.data_format;
+    Array dest(e.shape, e.dtype);
+    ImageGeom g = image_geom(e.shape, fmt);
+    const int fh = e.geom[0], fw = e.geom[1], sth = e.geom[2], stw = e.geom[3];
+    const int o_h = (g.ext[2] - fh) / sth + 1, o_w = (g.ext[3] - fw) / stw + 1;
+    const int64_t n = numel_of(e.shape);
+    if (n == 0) return dest;
+    std::vector<int> pst = patches.normalized_strides();
+    DALI_ASSERT((int64_t)patches.shape()[0] * patches.shape()[1] < ((int64_t)1 << 31), "col2im: the patch matrix must hold fewer than 2^31 elements");
+    std::string t = ctype(e.dtype);
+    Program P;
+    P.arrays.push_back(manual_arg(dest, Cls::FULL, true, 1, {(int)n}, {}));
+    P.arrays.push_back(manual_arg(patches, Cls::FULL, false, 2, patches.shape(), {pst[0], pst[1]}));
+    std::vector<int> geom = patch_geom(e, g, o_h, o_w, pst[0], pst[1]);
+    std::ostringstream sig;
+    sig << "col2im|" << (int)e.dtype << "|" << fmt;
+    launch_special("col2im", sig.str(), P, (n + 255) / 256, geom, [&](const std::string& kname, const IvLayout& L) {
+        std::ostringstream ss;
+        ss << special_head(P, L, kname, t, 20, kPatchGeomNames);
+        ss << "  T* image = (T*)A.p[0];\n  const T* in = (const T*)A.p[1];\n";
+        ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(H * W);\n";
+        ss << "  const int patch_h = DH * (FH - 1) + 1, patch_w = DW * (FW - 1) + 1;\n";
+        ss << "  for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {\n";
+        ss << "    unsigned rest = i; int q[4];\n";
+        // dimensions in memory order, slowest first: peel the fastest off first
+        for (int p = 3; p >= 1; --p) {
+            const char* ext = fmt[p] == 'N' ? "N" : (fmt[p] == 'C' ? "C" : (fmt[p] == 'H' ? "H" : "W"));
+            ss << "    q[" << p << "] = (int)(rest % (unsigned)" << ext << "); rest /= (unsigned)" << ext << ";\n";
+        }
+        ss << "    q[0] = (int)rest;\n";
+        ss << "    const int n = q[" << fmt.find('N') << "], c = q[" << fmt.find('C') << "];\n";
+        ss << "    const int h = q[" << fmt.find('H') << "] + PH, w = q[" << fmt.find('W') << "] + PW;\n";
+        ss << "    const int ph_min = h < patch_h ? h % DH : (h - patch_h + STH) / STH;\n";
+        ss << "    const int pw_min = w < patch_w ? w % DW : (w - patch_w + STW) / STW;\n";
+        ss << "    const int ph_max = (h + STH) / STH < OH ? (h + STH) / STH : OH;\n";
+        ss << "    const int pw_max = (w + STW) / STW < OW ? (w + STW) / STW : OW;\n";
+        ss << "    T res = (T)0;\n";
+        ss << "    for (int ph = ph_min; ph < ph_max; ph += DH)\n      for (int pw = pw_min; pw < pw_max; pw += DW) {\n";
+        ss << "        const int kh = (h - ph * STH) / DH, kw = (w - pw * STW) / DW;\n";
+        ss << "        const int row = " << emit_join_row(fmt) << ";\n";
+        ss << "        res += in[(long)row * ORS + (long)((n * OH + ph) * OW + pw) * OCS];\n      }\n";
+        ss << "    image[i] = res;\n  }\n}\n";
+        return ss.str();
+    });
+    return dest;
+}
+
+const char* const kPoolGeomNames[] = {"N", "C", "H", "W", "SN", "SC", "SH", "SW", "WH", "WW", "STH", "STW", "PH", "PW",
+                                      "OH", "OW", "YSN", "YSC", "YSH", "YSW"};
+
+std::vector<int> pool_geom(const Expr& e, const ImageGeom& gx, const ImageGeom& gy) {
+    return {gx.ext[0], gx.ext[1], gx.ext[2], gx.ext[3], gx.stride[0], gx.stride[1], gx.stride[2], gx.stride[3], e.geom[0], e.geom[1],
+            e.geom[2], e.geom[3], e.geom[4], e.geom[5], gy.ext[2], gy.ext[3], gy.stride[0], gy.stride[1], gy.stride[2], gy.stride[3]};
+}
+
+// Source text: linear index `i` of a dense array in `fmt` order -> n, c, and the two spatial coordinates
+std::string emit_decompose(const std::string& fmt, const char* eh, const char* ew, const char* nh, const char* nw) {
+    std::ostringstream ss;
+    ss << "    unsigned rest = i; int q[4];\n";
+    for (int p = 3; p >= 1; --p) {
+        std::string ext = fmt[p] == 'N' ? "N" : (fmt[p] == 'C' ? "C" : (fmt[p] == 'H' ? eh : ew));
+        ss << "    q[" << p << "] = (int)(rest % (unsigned)" << ext << "); rest /= (unsigned)" << ext << ";\n";
+    }
+    ss << "    q[0] = (int)rest;\n";
+    ss << "    const int n = q[" << fmt.find('N') << "], c = q[" << fmt.find('C') << "], " << nh << " = q[" << fmt.find('H') << "], " << nw << " = q["
+       << fmt.find('W') << "];\n";
+    return ss.str();
+}
+
+// pool2d: one thread per output element; the window is clipped to the image and walked columns outermost, as the
+// reference's loop does (conv.cpp:66-89), so an average is the same sequence of fp32 additions.
+Array run_pool2d(const Expr& e, const Array& x_in) {
+    Array x = dense_buffer(x_in);
+    const std::string& fmt = e.data_format;
+    Array dest(e.shape, e.dtype);
+    const int64_t n = numel_of(e.shape);
+    if (n == 0) return dest;
+    ImageGeom gx = image_geom(x.shape(), fmt), gy = image_geom(e.shape, fmt);
+    const bool average = e.depth != 0;
+    std::string t = ctype(e.dtype);
+    Program P;
+    P.arrays.push_back(manual_arg(dest, Cls::FULL, true, 1, {(int)n}, {}));
+    P.arrays.push_back(manual_arg(x, Cls::FULL, false, 1, {(int)numel_of(x.shape())}, {}));
+    std::ostringstream sig;
+    sig << "pool2d|" << (int)e.dtype << "|" << fmt << "|" << average;
+    launch_special("pool2d", sig.str(), P, (n + 255) / 256, pool_geom(e, gx, gy), [&](const std::string& kname, const IvLayout& L) {
+        std::ostringstream ss;
+        ss << special_head(P, L, kname, t, 20, kPoolGeomNames);
+        ss << "  T* y = (T*)A.p[0];\n  const T* x = (const T*)A.p[1];\n";
+        ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(OH * OW);\n";
+        ss << "  for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {\n";
+        ss << emit_decompose(fmt, "OH", "OW", "oh", "ow");
+        ss << "    int w_start = ow * STW, w_end = w_start + WW;\n";
+        ss << "    w_start = w_start - PW > 0 ? w_start - PW : 0;\n    w_end = w_end - PW < W ? w_end - PW : W;\n";
+        ss << "    int h_start = oh * STH, h_end = h_start + WH;\n";
+        ss << "    h_start = h_start - PH > 0 ? h_start - PH : 0;\n    h_end = h_end - PH < H ? h_end - PH : H;\n";
+        ss << "    const T* xp = x + (long)n * SN + (long)c * SC;\n";
+        ss << "    T res = " << (average ? "(T)0" : "reducers::lowest<T>()") << ";\n";
+        ss << "    for (int w = w_start; w < w_end; ++w)\n      for (int h = h_start; h < h_end; ++h) {\n";
+        ss << "        const T v = xp[(long)h * SH + (long)w * SW];\n";
+        ss << "        res = " << (average ? "res + v" : "res > v ? res : v") << ";\n      }\n";
+        if (average) ss << "    res = res / ((h_end - h_start) * (w_end - w_start));\n";
+        ss << "    y[i] = res;\n  }\n}\n";
+        return ss.str();
+    });
+    return dest;
+}
+
+// pool2d_backward: one thread per input element, summing over the windows that hold it, window rows outermost
+// (conv.cpp:133-172).
+Array run_pool2d_backward(const Expr& e, const Array& y_in, const Array& dy_in, const Array& x_in) {
+    Array y = dense_buffer(y_in), dy = dense_buffer(dy_in), x = dense_buffer(x_in);
+    const std::string& fmt = e.data_format;
+    Array dest(e.shape, e.dtype);
+    const int64_t n = numel_of(e.shape);
+    if (n == 0) return dest;
+    ImageGeom gx = image_geom(x.shape(), fmt), gy = image_geom(y.shape(), fmt);
+    const bool average = e.depth != 0;
+    std::string t = ctype(e.dtype);
+    Program P;
+    P.arrays.push_back(manual_arg(dest, Cls::FULL, true, 1, {(int)n}, {}));
+    P.arrays.push_back(manual_arg(y, Cls::FULL, false, 1, {(int)numel_of(y.shape())}, {}));
+    P.arrays.push_back(manual_arg(dy, Cls::FULL, false, 1, {(int)numel_of(dy.shape())}, {}));
+    P.arrays.push_back(manual_arg(x, Cls::FULL, false, 1, {(int)numel_of(x.shape())}, {}));
+    std::ostringstream sig;
+    sig << "pool2d_backward|" << (int)e.dtype << "|" << fmt << "|" << average;
+    launch_special("pool2d_backward", sig.str(), P, (n + 255) / 256, pool_geom(e, gx, gy), [&](const std::string& kname, const IvLayout& L) {
+        std::ostringstream ss;
+        ss << special_head(P, L, kname, t, 20, kPoolGeomNames);
+        ss << "  T* dx = (T*)A.p[0];\n  const T* y = (const T*)A.p[1];\n  const T* dy = (const T*)A.p[2];\n  const T* x = (const T*)A.p[3];\n";
+        ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(H * W);\n";
+        ss << "  for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {\n";
+        ss << emit_decompose(fmt, "H", "W", "h", "w");
+        ss << "    const T src = x[i];\n";
+        ss << "    const int ph_start = (h + PH) < WH ? 0 : (h + PH - WH) / STH + 1;\n";
+        ss << "    const int pw_start = (w + PW) < WW ? 0 : (w + PW - WW) / STW + 1;\n";
+        ss << "    const int ph_end = (h + PH) / STH + 1 < OH ? (h + PH) / STH + 1 : OH;\n";
+        ss << "    const int pw_end = (w + PW) / STW + 1 < OW ? (w + PW) / STW + 1 : OW;\n";
+        ss << "    const long base = (long)n * YSN + (long)c * YSC;\n";
+        ss << "    T grad = (T)0;\n";
+        ss << "    for (int ph = ph_start; ph < ph_end; ++ph)\n      for (int pw = pw_start; pw < pw_end; ++pw) {\n";
+        ss << "        const long q = base + (long)ph * YSH + (long)pw * YSW;\n";
+        if (average) {
+            ss << "        int hstart = ph * STH - PH, wstart = pw * STW - PW;\n";
+            ss << "        const int hend = hstart + WH < H ? hstart + WH : H, wend = wstart + WW < W ? wstart + WW : W;\n";
+            ss << "        hstart = hstart > 0 ? hstart : 0; wstart = wstart > 0 ? wstart : 0;\n";
+            ss << "        const int pool_size = (hend - hstart) * (wend - wstart);\n";
+            ss << "        grad += ((T)1 * dy[q]) / pool_size;\n      }\n";
+        } else {
+            ss << "        grad += (y[q] == src ? (T)1 : (T)0) * dy[q];\n      }\n";
+        }
+        ss << "    dx[i] = grad;\n  }\n}\n";
+        return ss.str();
+    });
     return dest;
 }
 

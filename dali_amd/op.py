@@ -245,3 +245,70 @@ def circular_convolution(x, weights):
     """out[..., i] = sum_s x[..., (i + s) mod n] * weights[..., s] (dali/array/op/circular_convolution.cpp)."""
     x, weights = as_array(x), as_array(weights)
     return _wrap(front.dali_fe_circular_convolution(x._h, weights._h), "circular_convolution")
+
+
+# dali/array/op/spatial_enums.h
+PADDING_T_SAME, PADDING_T_VALID = 0, 1
+POOLING_T_MAX, POOLING_T_AVG = 0, 1
+
+
+def _padding(p):
+    return {"same": PADDING_T_SAME, "valid": PADDING_T_VALID}.get(p.lower(), None) if isinstance(p, str) else int(p)
+
+
+def _pooling(p):
+    return {"max": POOLING_T_MAX, "avg": POOLING_T_AVG}.get(p.lower(), None) if isinstance(p, str) else int(p)
+
+
+def im2col(image, filter_h, filter_w, stride_h, stride_w, padding_h=0, padding_w=0, postpad_h=0, postpad_w=0, data_format="NCHW"):
+    """Patch matrix [filter_h*filter_w*C, N*out_h*out_w] of a 3-D or 4-D image (dali/array/op/im2col.cpp:190-267)."""
+    image = as_array(image)
+    return _wrap(front.dali_fe_im2col(image._h, filter_h, filter_w, stride_h, stride_w, padding_h, padding_w, postpad_h, postpad_w,
+                                      data_format.encode()), "im2col")
+
+
+def col2im(patches, image_shape, filter_h, filter_w, stride_h, stride_w, data_format="NCHW"):
+    """The adjoint of im2col: sums the patch matrix back into an image of ``image_shape`` (dali/array/op/col2im.cpp:165-233)."""
+    patches = as_array(patches)
+    s, n = _ints(image_shape)
+    return _wrap(front.dali_fe_col2im(patches._h, s, n, filter_h, filter_w, stride_h, stride_w, data_format.encode()), "col2im")
+
+
+def conv2d(x, filters, stride_h=1, stride_w=1, padding="valid", data_format="NCHW"):
+    x, filters = as_array(x), as_array(filters)
+    return _wrap(front.dali_fe_conv2d(x._h, filters._h, stride_h, stride_w, _padding(padding), data_format.encode()), "conv2d")
+
+
+def conv2d_backward_input(filters, out_dw, stride_h, stride_w, input_shape, padding="valid", data_format="NCHW"):
+    filters, out_dw = as_array(filters), as_array(out_dw)
+    s, n = _ints(input_shape)
+    if n != 4:
+        raise ValueError("conv2d_backward_input's result shape must be of size 4")
+    return _wrap(front.dali_fe_conv2d_backward_input(filters._h, out_dw._h, stride_h, stride_w, s, _padding(padding), data_format.encode()),
+                 "conv2d_backward_input")
+
+
+def conv2d_backward_filters(x, out_dw, stride_h, stride_w, filters_shape, padding="valid", data_format="NCHW"):
+    x, out_dw = as_array(x), as_array(out_dw)
+    s, n = _ints(filters_shape)
+    if n != 4:
+        raise ValueError("conv2d_backward_filters's filters shape must be of size 4")
+    return _wrap(front.dali_fe_conv2d_backward_filters(x._h, out_dw._h, stride_h, stride_w, s, _padding(padding), data_format.encode()),
+                 "conv2d_backward_filters")
+
+
+def conv2d_backward_bias(out_dw, data_format="NCHW"):
+    out_dw = as_array(out_dw)
+    return _wrap(front.dali_fe_conv2d_backward_bias(out_dw._h, data_format.encode()), "conv2d_backward_bias")
+
+
+def pool2d(x, window_h, window_w, stride_h, stride_w, pooling="max", padding="valid", data_format="NCHW"):
+    x = as_array(x)
+    return _wrap(front.dali_fe_pool2d(x._h, window_h, window_w, stride_h, stride_w, _pooling(pooling), _padding(padding), data_format.encode()),
+                 "pool2d")
+
+
+def pool2d_backward(y, dy, x, window_h, window_w, stride_h, stride_w, pooling="max", padding="valid", data_format="NCHW"):
+    y, dy, x = as_array(y), as_array(dy), as_array(x)
+    return _wrap(front.dali_fe_pool2d_backward(y._h, dy._h, x._h, window_h, window_w, stride_h, stride_w, _pooling(pooling), _padding(padding),
+                                               data_format.encode()), "pool2d_backward")

@@ -70,6 +70,26 @@ dali_array_t dali_fe_arange(dali_array_t start, dali_array_t stop, dali_array_t 
 dali_array_t dali_fe_diag(dali_array_t diagonal, int rows, int cols);
 /* op::circular_convolution (dali/array/op/circular_convolution.cpp:82-86) */
 dali_array_t dali_fe_circular_convolution(dali_array_t x, dali_array_t weights);
+/* Sliding-window operators. data_format is a permutation of "NCHW" naming the order of the image's dimensions
+ * (conv2d and the pooling pair accept "NCHW" and "NHWC"); padding: 0 = SAME, 1 = VALID and pooling: 0 = max, 1 = average,
+ * the values of dali/array/op/spatial_enums.h.
+ * op::im2col (dali/array/op/im2col.cpp:190-267), op::col2im (dali/array/op/col2im.cpp:165-233) */
+dali_array_t dali_fe_im2col(dali_array_t image, int filter_h, int filter_w, int stride_h, int stride_w, int padding_h, int padding_w,
+                            int postpad_h, int postpad_w, const char* data_format);
+dali_array_t dali_fe_col2im(dali_array_t input, const int* image_shape, int image_ndim, int filter_h, int filter_w, int stride_h,
+                            int stride_w, const char* data_format);
+/* op::conv2d and its three gradients (dali/array/op/conv.cpp:223-401) */
+dali_array_t dali_fe_conv2d(dali_array_t input, dali_array_t filters, int stride_h, int stride_w, int padding, const char* data_format);
+dali_array_t dali_fe_conv2d_backward_input(dali_array_t filters, dali_array_t out_dw, int stride_h, int stride_w, const int* input_shape,
+                                           int padding, const char* data_format);
+dali_array_t dali_fe_conv2d_backward_filters(dali_array_t input, dali_array_t out_dw, int stride_h, int stride_w, const int* filters_shape,
+                                             int padding, const char* data_format);
+dali_array_t dali_fe_conv2d_backward_bias(dali_array_t out_dw, const char* data_format);
+/* op::pool2d / op::pool2d_backward (dali/array/op/conv.cpp:403-456) */
+dali_array_t dali_fe_pool2d(dali_array_t input, int window_h, int window_w, int stride_h, int stride_w, int pooling, int padding,
+                            const char* data_format);
+dali_array_t dali_fe_pool2d_backward(dali_array_t out, dali_array_t out_dw, dali_array_t in, int window_h, int window_w, int stride_h,
+                                     int stride_w, int pooling, int padding, const char* data_format);
 /* op::outer (dali/array/op/outer.cpp:33-36) */
 dali_array_t dali_fe_outer(dali_array_t a, dali_array_t b);
 /* dest <<= source (dali/array/expression/assignment.cpp:92-126) */

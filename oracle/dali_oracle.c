@@ -24,6 +24,12 @@
  *     loop. The reference's fp32 GEMM is an un-vendored BLAS (cblas_sgemm), so its
  *     rounding on random fp32 inputs is PARITY UNPINNED; the fp64-accumulated product
  *     is used as truth with rel 1e-4.
+ *   - im2col / col2im / pool2d / conv2d: the slice-and-ravel definition of
+ *     dali/array/op/im2col_tests.cpp:7-39 on NHWC, NCHW and WNCH images, the TensorFlow
+ *     tables of dali/array/tests/conv_tests.cpp:132-216 (VALID and SAME), a direct
+ *     convolution loop, <im2col(x), y> == <x, col2im(y)> on integers, the patch-count
+ *     identity col2im(im2col(x)) == x * count, and the window loops of
+ *     dali/array/tests/conv_tests.cpp:422-640 for the pooling pair;
  *   - lstm step: composition of the above per dali/layers/lstm.cpp:226-261
  *     (no test in the reference pins LSTM values: PARITY UNPINNED beyond the
  *     composition of pinned parts).
@@ -384,6 +390,179 @@ void orc_circular_convolution(const float* content, const float* weights, int64_
             }
             out[r * n + x] = res;
         }
+}
+
+/* ---- sliding-window nodes ------------------------------------------------------------------
+ * Images are dense arrays whose four dimensions come in the order of the letters of `fmt` (a permutation of
+ * "NCHW"); dims[k] is the extent of dimension k. */
+static int fmt_pos(const char* fmt, char letter) {
+    for (int k = 0; k < 4; ++k)
+        if (fmt[k] == letter) return k;
+    return -1;
+}
+
+static int64_t image_index(const int* dims, const char* fmt, int n, int c, int h, int w) {
+    int64_t idx = 0;
+    for (int k = 0; k < 4; ++k) {
+        const int v = fmt[k] == 'N' ? n : (fmt[k] == 'C' ? c : (fmt[k] == 'H' ? h : w));
+        idx = idx * dims[k] + v;
+    }
+    return idx;
+}
+
+/* The three letters other than N, last to first: the digits of a patch-row index from the fastest to the
+ * slowest (dali/array/op/im2col.cpp:76-80; the same letters for N in position 0 or 1, the positions for which
+ * those three lines name three different letters). */
+static void row_letters(const char* fmt, char out[3]) {
+    int k = 0;
+    for (int p = 3; p >= 0; --p)
+        if (fmt[p] != 'N') out[k++] = fmt[p];
+}
+
+static int letter_extent(char letter, int channels, int fh, int fw) { return letter == 'C' ? channels : (letter == 'H' ? fh : fw); }
+
+/* row -> (c, kh, kw): dali/array/op/im2col.cpp:93-110 (offsets before the dilation factor is applied) */
+static void split_row(const char* fmt, int row, int channels, int fh, int fw, int* c, int* kh, int* kw) {
+    char l[3];
+    row_letters(fmt, l);
+    int rest = row;
+    for (int k = 0; k < 3; ++k) {
+        const int e = letter_extent(l[k], channels, fh, fw);
+        const int v = rest % e;
+        rest /= e;
+        if (l[k] == 'C') *c = v;
+        else if (l[k] == 'H') *kh = v;
+        else *kw = v;
+    }
+}
+
+/* (c, kh, kw) -> row: dali/array/op/col2im.cpp:86-94 */
+static int join_row(const char* fmt, int channels, int fh, int fw, int c, int kh, int kw) {
+    char l[3];
+    row_letters(fmt, l);
+    int row = 0;
+    for (int k = 2; k >= 0; --k) {
+        const int v = l[k] == 'C' ? c : (l[k] == 'H' ? kh : kw);
+        row = row * letter_extent(l[k], channels, fh, fw) + v;
+    }
+    return row;
+}
+
+/* out[fh*fw*C, N*o_h*o_w]: every column is one patch of the zero-padded image
+ * (dali/array/op/im2col.cpp:112-128). geom = {fh, fw, sh, sw, dh, dw, pre_h, pre_w, post_h, post_w}. */
+void orc_im2col(const float* image, const int* dims, const char* fmt, const int* geom, float* out) {
+    const int fh = geom[0], fw = geom[1], sh = geom[2], sw = geom[3], dh = geom[4], dw = geom[5];
+    const int pre_h = geom[6], pre_w = geom[7], post_h = geom[8], post_w = geom[9];
+    const int N = dims[fmt_pos(fmt, 'N')], Cc = dims[fmt_pos(fmt, 'C')], H = dims[fmt_pos(fmt, 'H')], W = dims[fmt_pos(fmt, 'W')];
+    const int o_h = (H + pre_h + post_h - (dh * (fh - 1) + 1)) / sh + 1;
+    const int o_w = (W + pre_w + post_w - (dw * (fw - 1) + 1)) / sw + 1;
+    const int64_t rows = (int64_t)fh * fw * Cc, cols = (int64_t)N * o_h * o_w;
+    for (int64_t q0 = 0; q0 < rows; ++q0) {
+        int c = 0, kh = 0, kw = 0;
+        split_row(fmt, (int)q0, Cc, fh, fw, &c, &kh, &kw);
+        for (int64_t q1 = 0; q1 < cols; ++q1) {
+            const int n = (int)(q1 / ((int64_t)o_h * o_w));
+            const int w = (int)(q1 % o_w) * sw + kw * dw - pre_w;
+            const int h = (int)((q1 / o_w) % o_h) * sh + kh * dh - pre_h;
+            out[q0 * cols + q1] = (0 <= w && w < W && 0 <= h && h < H) ? image[image_index(dims, fmt, n, c, h, w)] : 0.0f;
+        }
+    }
+}
+
+/* The adjoint: every image element collects, patch rows outermost, the entries of the patch matrix that im2col
+ * would have copied it to (dali/array/op/col2im.cpp:103-141). `dims` is the shape of the image to form. */
+void orc_col2im(const float* input, const int* dims, const char* fmt, const int* geom, float* image) {
+    const int fh = geom[0], fw = geom[1], sh = geom[2], sw = geom[3], dh = geom[4], dw = geom[5];
+    const int pre_h = geom[6], pre_w = geom[7], post_h = geom[8], post_w = geom[9];
+    const int N = dims[fmt_pos(fmt, 'N')], Cc = dims[fmt_pos(fmt, 'C')], H = dims[fmt_pos(fmt, 'H')], W = dims[fmt_pos(fmt, 'W')];
+    const int o_h = (H + pre_h + post_h - (dh * (fh - 1) + 1)) / sh + 1;
+    const int o_w = (W + pre_w + post_w - (dw * (fw - 1) + 1)) / sw + 1;
+    const int64_t cols = (int64_t)N * o_h * o_w;
+    const int patch_h = dh * (fh - 1) + 1, patch_w = dw * (fw - 1) + 1;
+    for (int n = 0; n < N; ++n)
+        for (int c = 0; c < Cc; ++c)
+            for (int h0 = 0; h0 < H; ++h0)
+                for (int w0 = 0; w0 < W; ++w0) {
+                    const int h = h0 + pre_h, w = w0 + pre_w;
+                    const int ph_min = h < patch_h ? h % dh : (h - patch_h + sh) / sh;
+                    const int pw_min = w < patch_w ? w % dw : (w - patch_w + sw) / sw;
+                    const int ph_max = (h + sh) / sh < o_h ? (h + sh) / sh : o_h;
+                    const int pw_max = (w + sw) / sw < o_w ? (w + sw) / sw : o_w;
+                    float res = 0.0f;
+                    for (int ph = ph_min; ph < ph_max; ph += dh)
+                        for (int pw = pw_min; pw < pw_max; pw += dw) {
+                            const int row = join_row(fmt, Cc, fh, fw, c, (h - ph * sh) / dh, (w - pw * sw) / dw);
+                            res += input[(int64_t)row * cols + ((int64_t)n * o_h + ph) * o_w + pw];
+                        }
+                    image[image_index(dims, fmt, n, c, h0, w0)] = res;
+                }
+}
+
+/* Pooling over the window clipped to the image, columns outermost (dali/array/op/conv.cpp:66-89).
+ * average = 0: maximum from -FLT_MAX; 1: the sum divided by the clipped window's area, converted to float.
+ * x has dims (fmt is "NCHW" or "NHWC"); out has the same layout with (out_h, out_w). */
+void orc_pool2d(const float* x, const int* dims, const char* fmt, int window_h, int window_w, int stride_h, int stride_w, int prepad_h,
+                int prepad_w, int out_h, int out_w, int average, float* out) {
+    const int N = dims[fmt_pos(fmt, 'N')], Cc = dims[fmt_pos(fmt, 'C')], H = dims[fmt_pos(fmt, 'H')], W = dims[fmt_pos(fmt, 'W')];
+    int odims[4];
+    for (int k = 0; k < 4; ++k) odims[k] = fmt[k] == 'H' ? out_h : (fmt[k] == 'W' ? out_w : dims[k]);
+    for (int n = 0; n < N; ++n)
+        for (int c = 0; c < Cc; ++c)
+            for (int i = 0; i < out_h; ++i)
+                for (int j = 0; j < out_w; ++j) {
+                    int w_start = j * stride_w, w_end = w_start + window_w;
+                    w_start = w_start - prepad_w > 0 ? w_start - prepad_w : 0;
+                    w_end = w_end - prepad_w < W ? w_end - prepad_w : W;
+                    int h_start = i * stride_h, h_end = h_start + window_h;
+                    h_start = h_start - prepad_h > 0 ? h_start - prepad_h : 0;
+                    h_end = h_end - prepad_h < H ? h_end - prepad_h : H;
+                    float res = average ? 0.0f : -FLT_MAX;
+                    for (int w = w_start; w < w_end; ++w)
+                        for (int h = h_start; h < h_end; ++h) {
+                            const float v = x[image_index(dims, fmt, n, c, h, w)];
+                            if (average) res += v;
+                            else res = res > v ? res : v;
+                        }
+                    if (average) res = res / (float)((h_end - h_start) * (w_end - w_start));
+                    out[image_index(odims, fmt, n, c, i, j)] = res;
+                }
+}
+
+/* dx[n,c,h,w] = sum over the windows (ph outer, pw inner) that hold (h, w) of PartialGrad(x, y[ph,pw]) *
+ * dy[ph,pw], divided by the clipped window area for the average (dali/array/op/conv.cpp:133-172;
+ * PartialGrad: jit/reducer_kernels.h:71-73 sum -> 1, :107-109 maximum -> y == x). */
+void orc_pool2d_backward(const float* y, const float* dy, const float* x, const int* dims, const char* fmt, int window_h, int window_w,
+                         int stride_h, int stride_w, int prepad_h, int prepad_w, int out_h, int out_w, int average, float* dx) {
+    const int N = dims[fmt_pos(fmt, 'N')], Cc = dims[fmt_pos(fmt, 'C')], H = dims[fmt_pos(fmt, 'H')], W = dims[fmt_pos(fmt, 'W')];
+    int odims[4];
+    for (int k = 0; k < 4; ++k) odims[k] = fmt[k] == 'H' ? out_h : (fmt[k] == 'W' ? out_w : dims[k]);
+    for (int n = 0; n < N; ++n)
+        for (int c = 0; c < Cc; ++c)
+            for (int h = 0; h < H; ++h)
+                for (int w = 0; w < W; ++w) {
+                    const float src = x[image_index(dims, fmt, n, c, h, w)];
+                    const int ph_start = (h + prepad_h) < window_h ? 0 : (h + prepad_h - window_h) / stride_h + 1;
+                    const int pw_start = (w + prepad_w) < window_w ? 0 : (w + prepad_w - window_w) / stride_w + 1;
+                    const int ph_end = (h + prepad_h) / stride_h + 1 < out_h ? (h + prepad_h) / stride_h + 1 : out_h;
+                    const int pw_end = (w + prepad_w) / stride_w + 1 < out_w ? (w + prepad_w) / stride_w + 1 : out_w;
+                    float grad = 0.0f;
+                    for (int ph = ph_start; ph < ph_end; ++ph)
+                        for (int pw = pw_start; pw < pw_end; ++pw) {
+                            const int64_t q = image_index(odims, fmt, n, c, ph, pw);
+                            if (average) {
+                                int hstart = ph * stride_h - prepad_h, wstart = pw * stride_w - prepad_w;
+                                const int hend = hstart + window_h < H ? hstart + window_h : H;
+                                const int wend = wstart + window_w < W ? wstart + window_w : W;
+                                hstart = hstart > 0 ? hstart : 0;
+                                wstart = wstart > 0 ? wstart : 0;
+                                const int pool_size = (hend - hstart) * (wend - wstart);
+                                grad += (1.0f * dy[q]) / (float)pool_size;
+                            } else {
+                                grad += (y[q] == src ? 1.0f : 0.0f) * dy[q];
+                            }
+                        }
+                    dx[image_index(dims, fmt, n, c, h, w)] = grad;
+                }
 }
 
 /* is_on = (indices[i] == j); on*is_on + (1.0 - is_on)*off, evaluated with T = float

@@ -53,6 +53,11 @@ def _load():
     lib.orc_axis_scan.argtypes = [C.c_int, _f, _i64, _i64, C.c_int, _f]
     lib.orc_circular_convolution.argtypes = [_f, _f, _i64, _i64, _f]
     lib.orc_one_hot.argtypes = [_i32, _i64, C.c_int, C.c_float, C.c_float, _f]
+    _ip = C.POINTER(C.c_int)
+    lib.orc_im2col.argtypes = [_f, _ip, C.c_char_p, _ip, _f]
+    lib.orc_col2im.argtypes = [_f, _ip, C.c_char_p, _ip, _f]
+    lib.orc_pool2d.argtypes = [_f, _ip, C.c_char_p] + [C.c_int] * 9 + [_f]
+    lib.orc_pool2d_backward.argtypes = [_f, _f, _f, _ip, C.c_char_p] + [C.c_int] * 9 + [_f]
     lib.orc_softmax_cross_entropy.argtypes = [_f, _i32, _i64, _i64, _f, _f, _f]
     lib.orc_softmax_cross_entropy_via_probs.argtypes = [_f, _i32, _i64, _i64, _f]
     for name in ("orc_gemm_f64acc", "orc_gemm_f32seq"):
@@ -262,6 +267,85 @@ def scatter_to_rows(dest, indices, values, op=1):
     scalar = vals.size == 1
     lib.orc_scatter_to_rows(fp(dest), dest.shape[1], ip(idx), idx.size, fp(vals), 1 if scalar else 0, op)
     return dest
+
+
+def _ints(values):
+    return (C.c_int * len(values))(*[int(v) for v in values])
+
+
+def _out_extent(size, pre, post, filt, stride, dilate=1):
+    return (size + pre + post - (dilate * (filt - 1) + 1)) // stride + 1
+
+
+def im2col(image, filter_h, filter_w, stride_h, stride_w, prepad_h=0, prepad_w=0, postpad_h=0, postpad_w=0, data_format="NCHW",
+           dilate_h=1, dilate_w=1):
+    """Patch matrix [filter_h*filter_w*C, N*out_h*out_w] of a 4-D image laid out as ``data_format`` says."""
+    image = _c32(image)
+    H, W = image.shape[data_format.index("H")], image.shape[data_format.index("W")]
+    Cc, N = image.shape[data_format.index("C")], image.shape[data_format.index("N")]
+    o_h = _out_extent(H, prepad_h, postpad_h, filter_h, stride_h, dilate_h)
+    o_w = _out_extent(W, prepad_w, postpad_w, filter_w, stride_w, dilate_w)
+    out = np.empty((filter_h * filter_w * Cc, N * o_h * o_w), dtype=np.float32)
+    geom = _ints([filter_h, filter_w, stride_h, stride_w, dilate_h, dilate_w, prepad_h, prepad_w, postpad_h, postpad_w])
+    lib.orc_im2col(fp(image), _ints(image.shape), data_format.encode(), geom, fp(out))
+    return out
+
+
+def col2im(patches, image_shape, filter_h, filter_w, stride_h, stride_w, data_format="NCHW"):
+    patches = _c32(patches)
+    out = np.empty(tuple(image_shape), dtype=np.float32)
+    geom = _ints([filter_h, filter_w, stride_h, stride_w, 1, 1, 0, 0, 0, 0])
+    lib.orc_col2im(fp(patches), _ints(image_shape), data_format.encode(), geom, fp(out))
+    return out
+
+
+def sliding_window_info(in_h, in_w, window_h, window_w, stride_h, stride_w, padding):
+    """out_h, out_w, padding_h, padding_w, odd_padding_h, odd_padding_w (dali/array/op/spatial_utils.cpp:64-91)."""
+    ceil = lambda a, b: (a + b - 1) // b
+    if padding == "same":
+        out_h, out_w = ceil(in_h, stride_h), ceil(in_w, stride_w)
+        pad_h = max(0, (out_h - 1) * stride_h + window_h - in_h)
+        pad_w = max(0, (out_w - 1) * stride_w + window_w - in_w)
+    else:
+        out_h, out_w = ceil(in_h - window_h + 1, stride_h), ceil(in_w - window_w + 1, stride_w)
+        pad_h = pad_w = 0
+    return out_h, out_w, pad_h // 2, pad_w // 2, pad_h % 2, pad_w % 2
+
+
+def conv2d(x, filters, stride_h, stride_w, padding="valid", data_format="NCHW", gemm_mode="f64"):
+    """im2col followed by one matrix product, laid out as dali/array/op/conv.cpp:223-276 does."""
+    x, filters = _c32(x), _c32(filters)
+    n_dim, c_dim, h_dim, w_dim = (data_format.index(l) for l in "NCHW")
+    fh, fw, oc = filters.shape[h_dim], filters.shape[w_dim], filters.shape[n_dim]
+    out_h, out_w, ph, pw, odd_h, odd_w = sliding_window_info(x.shape[h_dim], x.shape[w_dim], fh, fw, stride_h, stride_w, padding)
+    patches = im2col(x, fh, fw, stride_h, stride_w, ph, pw, ph + odd_h, pw + odd_w, data_format)
+    f2 = np.ascontiguousarray(np.swapaxes(filters, n_dim, 0)).reshape(oc, -1)
+    batch = x.shape[n_dim]
+    if data_format == "NCHW":
+        return np.ascontiguousarray(gemm(f2, patches, gemm_mode).reshape(oc, batch, out_h, out_w).swapaxes(0, 1))
+    return gemm(np.ascontiguousarray(patches.T), np.ascontiguousarray(f2.T), gemm_mode).reshape(batch, out_h, out_w, oc)
+
+
+def pool2d(x, window_h, window_w, stride_h, stride_w, mode="max", padding="valid", data_format="NCHW"):
+    x = _c32(x)
+    H, W = x.shape[data_format.index("H")], x.shape[data_format.index("W")]
+    out_h, out_w, ph, pw, _, _ = sliding_window_info(H, W, window_h, window_w, stride_h, stride_w, padding)
+    oshape = list(x.shape)
+    oshape[data_format.index("H")], oshape[data_format.index("W")] = out_h, out_w
+    out = np.empty(tuple(oshape), dtype=np.float32)
+    lib.orc_pool2d(fp(x), _ints(x.shape), data_format.encode(), window_h, window_w, stride_h, stride_w, ph, pw, out_h, out_w,
+                   1 if mode == "avg" else 0, fp(out))
+    return out
+
+
+def pool2d_backward(y, dy, x, window_h, window_w, stride_h, stride_w, mode="max", padding="valid", data_format="NCHW"):
+    y, dy, x = _c32(y), _c32(dy), _c32(x)
+    H, W = x.shape[data_format.index("H")], x.shape[data_format.index("W")]
+    out_h, out_w, ph, pw, _, _ = sliding_window_info(H, W, window_h, window_w, stride_h, stride_w, padding)
+    dx = np.empty_like(x)
+    lib.orc_pool2d_backward(fp(y), fp(dy), fp(x), _ints(x.shape), data_format.encode(), window_h, window_w, stride_h, stride_w, ph, pw,
+                            out_h, out_w, 1 if mode == "avg" else 0, fp(dx))
+    return dx
 
 
 def _strides(a):

@@ -428,3 +428,145 @@ def test_circular_convolution_is_a_circular_correlation(O, rng):
     got = O.circular_convolution(cf, wf).astype(np.float64)
     ref = np.fft.ifft(np.fft.fft(cf.astype(np.float32)) * np.conj(np.fft.fft(wf.astype(np.float32)))).real
     assert np.abs(got - ref).max() < 1e-4
+
+
+# ------------------------------------------------------------------ sliding windows
+def _patches_by_slicing(image_nhwc, fh, fw, sh, sw):
+    """The definition the reference's test uses (im2col_tests.cpp:7-39): every window of the NHWC image, raveled."""
+    n, h, w, _ = image_nhwc.shape
+    cols = []
+    for b in range(n):
+        for i in range(0, h - fh + 1, sh):
+            for j in range(0, w - fw + 1, sw):
+                cols.append(image_nhwc[b, i:i + fh, j:j + fw].ravel())
+    return np.stack(cols, axis=1)
+
+
+def test_im2col_matches_the_slicing_definition(O, rng):
+    # JITTests.im2col_without_channels (im2col_tests.cpp:41-72): arange image [2,1,3,4], 3x3 windows, three layouts
+    nchw = np.arange(24, dtype=np.float32).reshape(2, 1, 3, 4)
+    nhwc = nchw.transpose(0, 2, 3, 1)
+    want = _patches_by_slicing(nhwc, 3, 3, 1, 1)
+    assert np.array_equal(O.im2col(nhwc, 3, 3, 1, 1, data_format="NHWC"), want)
+    assert np.array_equal(O.im2col(nchw, 3, 3, 1, 1, data_format="NCHW"), want)
+    wnch = O.im2col(nchw.transpose(3, 0, 1, 2), 3, 3, 1, 1, data_format="WNCH")
+    assert np.array_equal(wnch.reshape(3, 1, 3, -1).transpose(1, 2, 0, 3).reshape(9, -1), want)
+    # with channels and strides: NHWC rows run (kh, kw, c), NCHW rows run (c, kh, kw)
+    for sh, sw in ((1, 1), (2, 1), (2, 3)):
+        x = rng.randint(-9, 10, (3, 7, 9, 4)).astype(np.float32)
+        want = _patches_by_slicing(x, 3, 2, sh, sw)
+        assert np.array_equal(O.im2col(x, 3, 2, sh, sw, data_format="NHWC"), want)
+        got = O.im2col(x.transpose(0, 3, 1, 2), 3, 2, sh, sw, data_format="NCHW")
+        assert np.array_equal(got.reshape(4, 3, 2, -1).transpose(1, 2, 0, 3).reshape(24, -1), want)
+    # padding = im2col of the zero-padded image
+    x = rng.randint(-9, 10, (2, 5, 6, 3)).astype(np.float32)
+    padded = np.pad(x, ((0, 0), (1, 2), (2, 1), (0, 0)))
+    assert np.array_equal(O.im2col(x, 3, 3, 1, 2, 1, 2, 2, 1, "NHWC"), _patches_by_slicing(padded, 3, 3, 1, 2))
+
+
+def _direct_conv2d(x_nchw, w_oihw, sh, sw, padding):
+    """Direct convolution (the loop of conv_tests.cpp:57-126), fp64."""
+    n, c, h, w = x_nchw.shape
+    o, _, fh, fw = w_oihw.shape
+    if padding == "same":
+        oh, ow = -(-h // sh), -(-w // sw)
+        ph, pw = max(0, (oh - 1) * sh + fh - h), max(0, (ow - 1) * sw + fw - w)
+        x_nchw = np.pad(x_nchw, ((0, 0), (0, 0), (ph // 2, ph - ph // 2), (pw // 2, pw - pw // 2)))
+    else:
+        oh, ow = -(-(h - fh + 1) // sh), -(-(w - fw + 1) // sw)
+    out = np.zeros((n, o, oh, ow))
+    for i in range(oh):
+        for j in range(ow):
+            win = x_nchw[:, :, i * sh:i * sh + fh, j * sw:j * sw + fw].astype(np.float64)
+            out[:, :, i, j] = np.einsum("nchw,ochw->no", win, w_oihw.astype(np.float64))
+    return out
+
+
+def test_conv2d_tensorflow_tables_and_direct_loop(O, rng):
+    g = golden("reference_known_answers.json")["conv2d_tensorflow"]
+    image = np.arange(2 * 3 * 7 * 5, dtype=np.float32).reshape(2, 3, 7, 5)
+    filters = np.arange(4 * 3 * 6 * 5, dtype=np.float32).reshape(3, 6, 5, 4).transpose(3, 0, 1, 2)
+    for mode in ("f64", "f32"):  # every partial sum is an integer below 2^24: exact either way
+        assert np.array_equal(O.conv2d(image, filters, 1, 1, "valid", "NHWC", mode).ravel(), np.array(g["valid"], np.float32))
+        assert np.array_equal(O.conv2d(image, filters, 1, 1, "same", "NHWC", mode).ravel(), np.array(g["same"], np.float32))
+    # ConvTests.conv2d_forward (conv_tests.cpp:348-410): strides 1..3, both layouts, both paddings
+    for sh in (1, 2, 3):
+        for sw in (1, 2, 3):
+            for padding in ("valid", "same"):
+                x = rng.uniform(-1, 1, (5, 3, 6, 8)).astype(np.float32)
+                w = rng.uniform(-1, 1, (2, 3, 2, 4)).astype(np.float32)
+                want = _direct_conv2d(x, w, sh, sw, padding)
+                got = O.conv2d(x, w, sh, sw, padding, "NCHW")
+                assert got.shape == want.shape and np.abs(got - want).max() < 1e-5
+                got = O.conv2d(x.transpose(0, 2, 3, 1), w.transpose(0, 2, 3, 1), sh, sw, padding, "NHWC")
+                assert np.abs(got.transpose(0, 3, 1, 2) - want).max() < 1e-5
+
+
+def test_col2im_is_the_adjoint_of_im2col(O, rng):
+    for fmt, perm in (("NCHW", (0, 1, 2, 3)), ("NHWC", (0, 2, 3, 1))):
+        for fh, fw, sh, sw in ((3, 3, 1, 1), (2, 3, 2, 1), (2, 2, 2, 2), (3, 2, 2, 3)):
+            shape_nchw = (2, 3, 7, 8)
+            # sizes for which the windows tile exactly, as op::col2im requires (col2im.cpp:204-215)
+            x = rng.randint(-5, 6, shape_nchw).astype(np.float32).transpose(perm)
+            px = O.im2col(x, fh, fw, sh, sw, data_format=fmt)
+            y = rng.randint(-5, 6, px.shape).astype(np.float32)
+            back = O.col2im(y, x.shape, fh, fw, sh, sw, fmt)
+            # <im2col(x), y> == <x, col2im(y)> exactly on small integers
+            assert float((px.astype(np.float64) * y).sum()) == float((x.astype(np.float64) * back).sum())
+            # col2im(im2col(x)) = x times the number of windows that hold each pixel
+            count = O.col2im(np.ones_like(px), x.shape, fh, fw, sh, sw, fmt)
+            assert np.array_equal(O.col2im(px, x.shape, fh, fw, sh, sw, fmt), x * count)
+            oh, ow = (7 - fh) // sh + 1, (8 - fw) // sw + 1
+            assert count.sum() == 2 * 3 * oh * ow * fh * fw
+    # JITTests.col2im_without_channels (col2im_tests.cpp:9-35): the two layouts agree
+    nchw = np.arange(24, dtype=np.float32).reshape(2, 1, 3, 4)
+    nchw[1] *= -1.0
+    nhwc = np.ascontiguousarray(nchw.transpose(0, 2, 3, 1))
+    a = O.col2im(O.im2col(nchw, 3, 3, 1, 1, data_format="NCHW"), nchw.shape, 3, 3, 1, 1, "NCHW")
+    b = O.col2im(O.im2col(nhwc, 3, 3, 1, 1, data_format="NHWC"), nhwc.shape, 3, 3, 1, 1, "NHWC")
+    assert np.array_equal(a.transpose(0, 2, 3, 1), b)
+
+
+def _pool_windows(h, w, wh, ww, sh, sw, padding):
+    ceil = lambda a, b: -(-a // b)
+    if padding == "same":
+        oh, ow = ceil(h, sh), ceil(w, sw)
+        ph, pw = max(0, (oh - 1) * sh + wh - h) // 2, max(0, (ow - 1) * sw + ww - w) // 2
+    else:
+        oh, ow, ph, pw = ceil(h - wh + 1, sh), ceil(w - ww + 1, sw), 0, 0
+    for i in range(oh):
+        for j in range(ow):
+            yield i, j, max(i * sh - ph, 0), min(i * sh + wh - ph, h), max(j * sw - pw, 0), min(j * sw + ww - pw, w)
+
+
+def test_pool2d_pair_against_window_loops(O, rng):
+    # the loops of reference_pool2d / reference_pool2d_backward (conv_tests.cpp:422-545), in fp64, NCHW and NHWC
+    for wh in (1, 2, 3):
+        for ww in (1, 2, 3):
+            for sh, sw in ((1, 1), (2, 1), (2, 2)):
+                for padding in ("valid", "same"):
+                    for mode in ("max", "avg"):
+                        x = rng.uniform(-1, 1, (2, 3, 6, 8)).astype(np.float32)
+                        wins = list(_pool_windows(6, 8, wh, ww, sh, sw, padding))
+                        oh, ow = wins[-1][0] + 1, wins[-1][1] + 1
+                        want = np.zeros((2, 3, oh, ow))
+                        for i, j, h0, h1, w0, w1 in wins:
+                            win = x[:, :, h0:h1, w0:w1].astype(np.float64).reshape(2, 3, -1)
+                            want[:, :, i, j] = win.max(-1) if mode == "max" else win.mean(-1)
+                        y = O.pool2d(x, wh, ww, sh, sw, mode, padding, "NCHW")
+                        assert y.shape == want.shape and np.abs(y - want).max() < 1e-6
+                        xh = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+                        yh = O.pool2d(xh, wh, ww, sh, sw, mode, padding, "NHWC")
+                        assert np.array_equal(yh.transpose(0, 3, 1, 2), y)
+                        dy = rng.uniform(-1, 1, y.shape).astype(np.float32)
+                        dx_want = np.zeros(x.shape)
+                        for i, j, h0, h1, w0, w1 in wins:
+                            if mode == "avg":
+                                dx_want[:, :, h0:h1, w0:w1] += dy[:, :, i, j, None, None].astype(np.float64) / ((h1 - h0) * (w1 - w0))
+                            else:
+                                hit = x[:, :, h0:h1, w0:w1] == y[:, :, i, j, None, None]
+                                dx_want[:, :, h0:h1, w0:w1] += hit * dy[:, :, i, j, None, None].astype(np.float64)
+                        dx = O.pool2d_backward(y, dy, x, wh, ww, sh, sw, mode, padding, "NCHW")
+                        assert np.abs(dx - dx_want).max() < 1e-6
+                        dxh = O.pool2d_backward(yh, np.ascontiguousarray(dy.transpose(0, 2, 3, 1)), xh, wh, ww, sh, sw, mode, padding, "NHWC")
+                        assert np.array_equal(dxh.transpose(0, 3, 1, 2), dx)
