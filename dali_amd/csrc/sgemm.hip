@@ -768,7 +768,16 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
     long tiles64 = (long)((M + 63) / 64) * ((N + 63) / 64);
     static const int split_env = getenv("DALI_HIP_GEMM_SPLITK") ? atoi(getenv("DALI_HIP_GEMM_SPLITK")) : 0;
     int split_k = split_env > 0 ? split_env : 1;
-    (void)tiles64;
+    if (split_env == 0 && variant == 0 && tiles64 <= 128) {
+        // A few tiles over a long inner extent (the weight gradient of a convolution: [out, window] from tens of
+        // thousands of patches) would leave most of the device idle: shares of at least eight slabs, about two
+        // workgroups per CU, folded in a fixed order by the workgroup that finishes last.
+        int nslab64 = 0;
+        for (int s = 0; s < g.nseg; ++s) nslab64 += (g.seg[s].K + 63) / 64;
+        const int want = (int)((512 + tiles64 - 1) / tiles64);
+        const int share = nslab64 / 8 < want ? nslab64 / 8 : want;
+        if (share >= 2) return run_tile<64, 64, 64, 2>(g, ta, tb, vec, share);
+    }
     if (variant == 8) return run_tile<64, 64, 64, 2>(g, ta, tb, vec, split_k);
     if (variant == 5) return run_tile<64, 64, 64, 2, 2, true>(g, ta, tb, vec, split_k);
     if (variant == 9) return run_tile<64, 64, 64, 2, 4>(g, ta, tb, vec, split_k);

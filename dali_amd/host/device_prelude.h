@@ -179,6 +179,12 @@ DI float dali_div_fast(float x, float s, float r) {
 DI double dali_div_invariant(double x, double s) { return x / s; }
 DI int dali_div_invariant(int x, int s) { return x / s; }
 
+// n / d for 0 <= n < 2^31 and a divisor d >= 1 that the host knows at launch. With 2^(s-1) < d <= 2^s the host
+// passes m = ceil(2^(31+s) / d), which fits 32 bits. Then n * m / 2^(31+s) = n / d + n * e / (d * 2^(31+s)) with
+// 0 <= e < d <= 2^s, and the second term is below 1 / d, the distance from n / d to the next integer, so the
+// floor of the product is floor(n / d).
+DI unsigned dali_udiv(unsigned n, unsigned m, int s) { return (unsigned)(((unsigned long long)n * m) >> (31 + s)); }
+
 // one_hot element. The reference evaluates on*is_on + (1.0 - is_on)*off with is_on in T and
 // the rest in double (dali/array/op/one_hot.cpp:38-46). With is_on in {0, 1} that is
 // on + 0*off when the index matches and on*0 + off otherwise, and both forms round to

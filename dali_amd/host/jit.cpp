@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-12";
+const char* const kCodegenVersion = "dali-hip-codegen-14";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -2927,9 +2927,12 @@ Array run_circular_convolution(const Array& x_in, const Array& w_in) {
 
 // ------------------------------------------------------------ sliding windows
 // im2col, col2im and the pooling pair (dali/array/op/im2col.cpp, col2im.cpp, conv.cpp:12-212) are index remaps
-// bound by memory traffic. Images are read and written as dense arrays whose dimensions come in the order of
-// the data format's letters; the kernels take the four extents and element strides as (N, C, H, W), so one
-// source serves every layout. Index arithmetic is 32-bit (extents are ints, element counts below 2^31).
+// bound by memory traffic. Images are dense arrays whose dimensions come in the order of the data format's
+// letters; the kernels take extents and element strides as (N, C, H, W), so one source serves every layout.
+// At streaming rates a vector instruction slot is worth a few bytes, so index arithmetic is kept off the
+// per-element path: it is 32-bit, divisions by extents go through multipliers computed here on the host
+// (dali_udiv), per-patch and per-row parts are computed once per wave or workgroup, and layouts whose channels
+// are contiguous move four channels per thread.
 struct ImageGeom {
     int ext[4];     // N, C, H, W
     int stride[4];  // element strides of a dense array in data_format order, as (N, C, H, W)
@@ -2952,6 +2955,36 @@ Array dense_buffer(const Array& a) {
     return b.contiguous_memory() ? b : b.ascontiguousarray();
 }
 
+// Named integers of a kernel's geometry; a divisor brings its multiplier and shift along (see dali_udiv).
+struct GeomInts {
+    std::vector<std::string> names;
+    std::vector<int> values;
+    void add(const std::string& name, int v) {
+        names.push_back(name);
+        values.push_back(v);
+    }
+    void add_div(const std::string& name, int d) {
+        DALI_ASSERT(d >= 1, make_message("internal: divisor ", name, " must be positive (got ", d, ")"));
+        int sft = 0;
+        while (((int64_t)1 << sft) < d) ++sft;
+        const uint64_t m = (((uint64_t)1 << (31 + sft)) + (uint64_t)d - 1) / (uint64_t)d;
+        add(name, d);
+        add(name + "_M", (int)(uint32_t)m);
+        add(name + "_S", sft);
+    }
+    void add_image(const ImageGeom& g) {
+        const char* ext[4] = {"N", "C", "H", "W"};
+        const char* str[4] = {"SN", "SC", "SH", "SW"};
+        for (int k = 0; k < 4; ++k) add_div(ext[k], g.ext[k]);
+        for (int k = 0; k < 4; ++k) add(str[k], g.stride[k]);
+    }
+};
+
+// q = n / D, r = n % D in generated source
+std::string divmod(const std::string& q, const std::string& r, const std::string& n, const std::string& D) {
+    return "const unsigned " + q + " = dali_udiv(" + n + ", " + D + "_M, " + D + "_S); const int " + r + " = (int)(" + n + " - " + q + " * (unsigned)" + D + ");";
+}
+
 // The letters other than N, last to first: the digits of a patch-row index, fastest first
 // (dali/array/op/im2col.cpp:76-80 for N in position 0 or 1, where those lines name three different letters).
 std::string row_letters(const std::string& fmt) {
@@ -2961,34 +2994,32 @@ std::string row_letters(const std::string& fmt) {
     return r;
 }
 
-// Source text: `row` -> c, kh, kw (im2col.cpp:93-110) and back (col2im.cpp:86-94); C, FH, FW are in scope.
+const char* row_digit_extent(char letter) { return letter == 'C' ? "C" : (letter == 'H' ? "FH" : "FW"); }
+const char* row_digit_name(char letter) { return letter == 'C' ? "c" : (letter == 'H' ? "kh" : "kw"); }
+
+// Source text: `row` -> c, kh, kw (im2col.cpp:93-110) and back (col2im.cpp:86-94)
 std::string emit_split_row(const std::string& fmt, const std::string& row) {
-    std::string l = row_letters(fmt), out = "unsigned rest_ = (unsigned)(" + row + ");\n";
-    for (int k = 0; k < 3; ++k) {
-        std::string ext = l[k] == 'C' ? "C" : (l[k] == 'H' ? "FH" : "FW"), name = l[k] == 'C' ? "c" : (l[k] == 'H' ? "kh" : "kw");
-        if (k < 2) out += "      const int " + name + " = (int)(rest_ % (unsigned)" + ext + "); rest_ /= (unsigned)" + ext + ";\n";
-        else out += "      const int " + name + " = (int)rest_;\n";
-    }
+    std::string l = row_letters(fmt), out;
+    out += "      " + divmod("rq1_", row_digit_name(l[0]), "(unsigned)(" + row + ")", row_digit_extent(l[0])) + "\n";
+    out += "      " + divmod("rq2_", row_digit_name(l[1]), "rq1_", row_digit_extent(l[1])) + "\n";
+    out += std::string("      const int ") + row_digit_name(l[2]) + " = (int)rq2_;\n";
     return out;
 }
 
 std::string emit_join_row(const std::string& fmt) {
     std::string l = row_letters(fmt), expr;
-    for (int k = 2; k >= 0; --k) {
-        std::string ext = l[k] == 'C' ? "C" : (l[k] == 'H' ? "FH" : "FW"), name = l[k] == 'C' ? "c" : (l[k] == 'H' ? "kh" : "kw");
-        expr = expr.empty() ? name : "(" + expr + ") * " + ext + " + " + name;
-    }
+    for (int k = 2; k >= 0; --k) expr = expr.empty() ? row_digit_name(l[k]) : "(" + expr + ") * " + row_digit_extent(l[k]) + " + " + row_digit_name(l[k]);
     return expr;
 }
 
 // One launch of a hand-laid-out kernel: `blocks` workgroups of 256 threads (the kernels stride over blocks, so a
-// capped grid still covers the work); `geom` travels as the integers behind the arrays' sizes.
-void launch_special(const char* kind, const std::string& sig, const Program& P, int64_t blocks, const std::vector<int>& geom,
-                    const std::function<std::string(const std::string&, const IvLayout&)>& gen) {
+// capped grid still covers the work); the geometry travels as the integers behind the arrays' sizes.
+void launch_special(const char* kind, const std::string& sig, const Program& P, int64_t blocks, const GeomInts& G,
+                    const std::function<void(std::ostringstream&)>& body) {
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash(kind, sig, "");
     std::shared_ptr<KernelSpec>& K = specs_cache[h];
-    std::vector<int> shape_ndims = {2, (int)geom.size()};
+    std::vector<int> shape_ndims = {2, (int)G.values.size()};
     IvLayout L = layout_iv(P, shape_ndims);
     if (!K) {
         K = std::make_shared<KernelSpec>();
@@ -3004,32 +3035,49 @@ void launch_special(const char* kind, const std::string& sig, const Program& P, 
         K->plan.max_blocks = 1 << 20;
     }
     const int nblocks = (int)std::min<int64_t>(std::max<int64_t>(blocks, 1), 1 << 20);
-    load_and_launch(*K, [&]() { return gen(K->name, L); }, P, {{nblocks, 256}, geom});
+    load_and_launch(*K, [&]() {
+        std::ostringstream ss;
+        ss << codegen::kDevicePrelude << kargs_struct(P, L);
+        ss << "extern \"C\" __global__ __launch_bounds__(256) void " << K->name << "(KArgs A) {\n  typedef " << ctype(P.arrays[0].buf->dtype) << " T;\n";
+        for (size_t k = 0; k < G.names.size(); ++k) {
+            const bool mult = G.names[k].size() > 2 && G.names[k].compare(G.names[k].size() - 2, 2, "_M") == 0;
+            ss << "  const " << (mult ? "unsigned " : "int ") << G.names[k] << " = " << (mult ? "(unsigned)" : "") << "A.iv[" << L.shape_pos[1] + k
+               << "]; (void)" << G.names[k] << ";\n";
+        }
+        body(ss);
+        return ss.str();
+    }, P, {{nblocks, 256}, G.values});
 }
 
-std::string special_head(const Program& P, const IvLayout& L, const std::string& kname, const std::string& t, int n_geom, const char* const* names) {
+// Source text: index `i` of a dense array in `fmt` order whose innermost dimension is taken in groups of VEC
+// -> n, c and the two spatial coordinates. `eh` / `ew` name the extents of the H and W positions.
+std::string emit_decompose(const std::string& fmt, const std::string& eh, const std::string& ew, const std::string& nh, const std::string& nw,
+                           bool inner_groups) {
     std::ostringstream ss;
-    ss << codegen::kDevicePrelude << kargs_struct(P, L);
-    ss << "extern \"C\" __global__ __launch_bounds__(256) void " << kname << "(KArgs A) {\n  typedef " << t << " T;\n";
-    for (int k = 0; k < n_geom; ++k) ss << "  const int " << names[k] << " = A.iv[" << L.shape_pos[1] + k << "]; (void)" << names[k] << ";\n";
+    auto ext = [&](int p) { return fmt[p] == 'N' ? std::string("N") : (fmt[p] == 'C' ? std::string("C") : (fmt[p] == 'H' ? eh : ew)); };
+    ss << "    " << divmod("dq3_", "q3", "i", inner_groups ? "INNER_GROUPS" : ext(3)) << "\n";
+    ss << "    " << divmod("dq2_", "q2", "dq3_", ext(2)) << "\n";
+    ss << "    " << divmod("dq1_", "q1", "dq2_", ext(1)) << "\n";
+    ss << "    const int q0 = (int)dq1_;\n";
+    const char* qn[4] = {"q0", "q1", "q2", "q3"};
+    auto coord = [&](char letter) {
+        const int p = (int)fmt.find(letter);
+        return p == 3 && inner_groups ? std::string("q3 * VEC") : std::string(qn[p]);
+    };
+    ss << "    const int n = " << coord('N') << ", c = " << coord('C') << ", " << nh << " = " << coord('H') << ", " << nw << " = " << coord('W') << ";\n";
     return ss.str();
 }
 
-const char* const kPatchGeomNames[] = {"N", "C", "H", "W", "SN", "SC", "SH", "SW", "FH", "FW", "STH", "STW", "DH", "DW",
-                                       "PH", "PW", "OH", "OW", "ORS", "OCS"};
-
-std::vector<int> patch_geom(const Expr& e, const ImageGeom& g, int o_h, int o_w, int mat_row_stride, int mat_col_stride) {
-    return {g.ext[0], g.ext[1], g.ext[2], g.ext[3], g.stride[0], g.stride[1], g.stride[2], g.stride[3], e.geom[0], e.geom[1],
-            e.geom[2], e.geom[3], e.geom[4], e.geom[5], e.geom[6], e.geom[7], o_h, o_w, mat_row_stride, mat_col_stride};
-}
+bool four_byte_vectors(DType dtype, const Array& a, int inner) { return size_of_dtype(dtype) == 4 && inner % 4 == 0 && a.offset() % 4 == 0; }
 
 // im2col. Two layouts of the same matrix, chosen so that both the gather and the store run along memory:
 //  - formats ending in "WC" (NHWC): for a patch and a filter row kh, the filter_w * C values are one contiguous
 //    run of the image, and they are consecutive rows (kh, kw, c) of one column. The matrix is stored patch-major
-//    ([N*out_h*out_w, filter_h*filter_w*C], returned as its transposed view): one wave copies one run.
+//    ([N*out_h*out_w, filter_h*filter_w*C], returned as its transposed view): one wave copies one patch, whose
+//    position is computed once, on the scalar unit.
 //  - every other format: row-major [filter_h*filter_w*C, N*out_h*out_w]; a thread owns a column (consecutive
 //    columns are consecutive output pixels, i.e. consecutive W) and walks a group of rows, whose decomposition
-//    into (c, kh, kw) is uniform over the workgroup.
+//    into (c, kh, kw) is the same for the whole workgroup.
 Array run_im2col(const Expr& e, const Array& image_in) {
     Array image = dense_buffer(image_in);
     const std::string& fmt = e.data_format;
@@ -3044,63 +3092,70 @@ Array run_im2col(const Expr& e, const Array& image_in) {
     Array result = patch_major ? store.transpose() : store;
     if (rows * cols == 0) return result;
     DALI_ASSERT(rows * cols < ((int64_t)1 << 31), "im2col: the patch matrix must hold fewer than 2^31 elements");
-    std::string t = ctype(e.dtype);
     Program P;
     P.arrays.push_back(manual_arg(store, Cls::FULL, true, 2, store.shape(), {}));
     P.arrays.push_back(manual_arg(image, Cls::FULL, false, 1, {(int)numel_of(image.shape())}, {}));
-    std::vector<int> geom = patch_geom(e, g, o_h, o_w, patch_major ? 1 : (int)cols, patch_major ? (int)rows : 1);
+    GeomInts G;
+    G.add_image(g);
+    G.add_div("FH", fh);
+    G.add_div("FW", fw);
+    G.add("STH", sth);
+    G.add("STW", stw);
+    G.add("DH", dh);
+    G.add("DW", dw);
+    G.add("PH", e.geom[6]);
+    G.add("PW", e.geom[7]);
+    G.add_div("OH", o_h);
+    G.add_div("OW", o_w);
     if (patch_major) {
-        const int VEC = (g.ext[1] % 4 == 0 && size_of_dtype(e.dtype) == 4 && image.offset() % 4 == 0) ? 4 : 1;
+        const int VEC = four_byte_vectors(e.dtype, image, g.ext[1]) ? 4 : 1;
+        G.add_div("RUN", fw * g.ext[1]);
         std::ostringstream sig;
         sig << "im2col_wc|" << (int)e.dtype << "|" << VEC;
-        const int64_t units = cols * fh;  // (patch, filter row) pairs, one wave each
-        launch_special("im2col", sig.str(), P, (units + 3) / 4, geom, [&](const std::string& kname, const IvLayout& L) {
-            std::ostringstream ss;
-            ss << special_head(P, L, kname, t, 20, kPatchGeomNames);
+        launch_special("im2col", sig.str(), P, (cols + 3) / 4, G, [&](std::ostringstream& ss) {
             ss << "  constexpr int VEC = " << VEC << ";\n";
             ss << "  T* out = (T*)A.p[0];\n  const T* img = (const T*)A.p[1];\n";
-            ss << "  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;\n";
-            ss << "  const unsigned units = (unsigned)(N * OH * OW) * (unsigned)FH;\n  const int run = FW * C, rows = FH * run;\n";
-            ss << "  for (unsigned u = blockIdx.x * 4u + wave; u < units; u += gridDim.x * 4u) {\n";
-            ss << "    const unsigned col = u / (unsigned)FH; const int kh = (int)(u % (unsigned)FH);\n";
-            ss << "    const int ow = (int)(col % (unsigned)OW); const unsigned t1 = col / (unsigned)OW;\n";
-            ss << "    const int oh = (int)(t1 % (unsigned)OH), n = (int)(t1 / (unsigned)OH);\n";
-            ss << "    const int h = oh * STH - PH + kh, w0 = ow * STW - PW;\n";
-            ss << "    T* dst = out + (long)col * rows + kh * run;\n";
-            ss << "    // the run covers image columns w0 .. w0 + FW - 1 of row h: element j is valid when that column lies inside the image\n";
-            ss << "    const bool row_ok = h >= 0 && h < H;\n";
-            ss << "    const int jlo = w0 < 0 ? -w0 * C : 0, jhi = (W - w0) * C < run ? (W - w0) * C : run;\n";
-            ss << "    const T* src = img + (long)n * SN + (long)(row_ok ? h : 0) * SH + (long)w0 * C;\n";
-            ss << "    for (int j = lane * VEC; j < run; j += 64 * VEC) {\n";
+            ss << "  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);\n";
+            ss << "  const unsigned cols = (unsigned)(N * OH * OW);\n  const int rows = FH * RUN;\n";
+            ss << "  for (unsigned col = blockIdx.x * 4u + wave; col < cols; col += gridDim.x * 4u) {\n";
+            ss << "    " << divmod("t1", "ow", "col", "OW") << "\n";
+            ss << "    " << divmod("n", "oh", "t1", "OH") << "\n";
+            ss << "    const int h0 = oh * STH - PH, w0 = ow * STW - PW;\n";
+            ss << "    // a run covers image columns w0 .. w0 + FW - 1 of one image row: element j is valid when that column lies inside the image\n";
+            ss << "    const int jlo = w0 < 0 ? -w0 * C : 0, jhi = (W - w0) * C < RUN ? (W - w0) * C : RUN;\n";
+            ss << "    T* dst = out + (long)col * rows;\n";
+            ss << "    const T* src0 = img + (long)n * SN + (long)w0 * C;\n";
+            ss << "    for (int e = lane * VEC; e < rows; e += 64 * VEC) {\n";
+            ss << "      " << divmod("kh", "j", "(unsigned)e", "RUN") << "\n";
+            ss << "      const int h = h0 + (int)kh;\n";
             ss << "      dali_vec<T, VEC> v;\n";
-            ss << "      if (row_ok && j >= jlo && j < jhi) v = dali_load<T, VEC>(src + j);\n";
+            ss << "      if (h >= 0 && h < H && j >= jlo && j < jhi) v = dali_load<T, VEC>(src0 + (long)h * SH + j);\n";
             ss << "      else { _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) v.v[k] = (T)0; }\n";
-            ss << "      dali_store<T, VEC>(dst + j, v);\n    }\n  }\n}\n";
-            return ss.str();
+            ss << "      dali_store_nt<T, VEC>(dst + e, v);\n    }\n  }\n}\n";
         });
     } else {
-        const int RB = 8;  // rows per workgroup
+        const int RB = 16;  // rows per workgroup
         const int64_t col_tiles = (cols + 255) / 256, row_groups = (rows + RB - 1) / RB;
+        G.add_div("COL_TILES", (int)col_tiles);
         std::ostringstream sig;
         sig << "im2col_rows|" << (int)e.dtype << "|" << row_letters(fmt);
-        launch_special("im2col", sig.str(), P, col_tiles * row_groups, geom, [&](const std::string& kname, const IvLayout& L) {
-            std::ostringstream ss;
-            ss << special_head(P, L, kname, t, 20, kPatchGeomNames);
+        launch_special("im2col", sig.str(), P, col_tiles * row_groups, G, [&](std::ostringstream& ss) {
             ss << "  constexpr int RB = " << RB << ";\n";
             ss << "  T* out = (T*)A.p[0];\n  const T* img = (const T*)A.p[1];\n";
             ss << "  const unsigned cols = (unsigned)(N * OH * OW); const int rows = FH * FW * C;\n";
-            ss << "  const unsigned col_tiles = (cols + 255u) / 256u, total = col_tiles * (unsigned)((rows + RB - 1) / RB);\n";
+            ss << "  const unsigned total = (unsigned)COL_TILES * (unsigned)((rows + RB - 1) / RB);\n";
             ss << "  for (unsigned b = blockIdx.x; b < total; b += gridDim.x) {\n";
-            ss << "    const unsigned col = (b % col_tiles) * 256u + threadIdx.x; const int r0 = (int)(b / col_tiles) * RB;\n";
+            ss << "    " << divmod("rg", "ct", "b", "COL_TILES") << "\n";
+            ss << "    const unsigned col = (unsigned)ct * 256u + threadIdx.x; const int r0 = (int)rg * RB;\n";
             ss << "    if (col >= cols) continue;\n";
-            ss << "    const int ow = (int)(col % (unsigned)OW); const unsigned t1 = col / (unsigned)OW;\n";
-            ss << "    const int oh = (int)(t1 % (unsigned)OH), n = (int)(t1 / (unsigned)OH);\n";
+            ss << "    " << divmod("t1", "ow", "col", "OW") << "\n";
+            ss << "    " << divmod("n", "oh", "t1", "OH") << "\n";
             ss << "    const int h0 = oh * STH - PH, w0 = ow * STW - PW;\n    const T* img_n = img + (long)n * SN;\n";
-            ss << "    for (int r = r0; r < r0 + RB && r < rows; ++r) {\n      " << emit_split_row(fmt, "r");
+            ss << "    T* out_c = out + col;\n";
+            ss << "    for (int r = r0; r < r0 + RB && r < rows; ++r) {\n" << emit_split_row(fmt, "r");
             ss << "      const int h = h0 + kh * DH, w = w0 + kw * DW;\n";
             ss << "      T v = (T)0;\n      if (h >= 0 && h < H && w >= 0 && w < W) v = img_n[(long)c * SC + (long)h * SH + (long)w * SW];\n";
-            ss << "      out[(long)r * cols + col] = v;\n    }\n  }\n}\n";
-            return ss.str();
+            ss << "      __builtin_nontemporal_store(v, out_c + (long)r * cols);\n    }\n  }\n}\n";
         });
     }
     return result;
@@ -3108,7 +3163,8 @@ Array run_im2col(const Expr& e, const Array& image_in) {
 
 // col2im: every image element sums, patch rows outermost, the entries of the patch matrix that im2col would have
 // copied it to (col2im.cpp:103-141): the same additions in the same order as the reference's loop. The patch
-// matrix is read through its strides, so the patch-major form produced for NHWC needs no copy.
+// matrix is read through its strides, so the patch-major form produced for NHWC needs no copy, and there four
+// channels (four consecutive matrix rows, contiguous in that form) travel per thread.
 Array run_col2im(const Expr& e, const Array& patches_in) {
     Array patches = patches_in.is_buffer() ? patches_in : materialize(patches_in);
     const std::string& fmt = e.data_format;
@@ -3120,68 +3176,78 @@ Array run_col2im(const Expr& e, const Array& patches_in) {
     if (n == 0) return dest;
     std::vector<int> pst = patches.normalized_strides();
     DALI_ASSERT((int64_t)patches.shape()[0] * patches.shape()[1] < ((int64_t)1 << 31), "col2im: the patch matrix must hold fewer than 2^31 elements");
-    std::string t = ctype(e.dtype);
+    const bool channel_vectors = fmt[3] == 'C' && pst[0] == 1 && pst[1] % 4 == 0 && row_letters(fmt)[0] == 'C' && four_byte_vectors(e.dtype, patches, g.ext[1]);
+    const int VEC = channel_vectors ? 4 : 1;
     Program P;
     P.arrays.push_back(manual_arg(dest, Cls::FULL, true, 1, {(int)n}, {}));
     P.arrays.push_back(manual_arg(patches, Cls::FULL, false, 2, patches.shape(), {pst[0], pst[1]}));
-    std::vector<int> geom = patch_geom(e, g, o_h, o_w, pst[0], pst[1]);
+    GeomInts G;
+    G.add_image(g);
+    G.add("PH", e.geom[6]);
+    G.add("PW", e.geom[7]);
+    G.add("OH", o_h);
+    G.add("OW", o_w);
+    G.add("ORS", pst[0]);
+    G.add("OCS", pst[1]);
+    G.add_div("INNER_GROUPS", std::max(1, e.shape[3] / VEC));
+    // filter, stride and dilation are compile-time: the loops over the covering patches unroll into independent
+    // loads (a loop with run-time bounds would wait for each load in turn), and the divisions by them fold
+    const int dh = e.geom[4], dw = e.geom[5];
+    const int max_ph = (dh * (fh - 1) + sth) / sth, max_pw = (dw * (fw - 1) + stw) / stw;  // ceil(patch extent / stride)
     std::ostringstream sig;
-    sig << "col2im|" << (int)e.dtype << "|" << fmt;
-    launch_special("col2im", sig.str(), P, (n + 255) / 256, geom, [&](const std::string& kname, const IvLayout& L) {
-        std::ostringstream ss;
-        ss << special_head(P, L, kname, t, 20, kPatchGeomNames);
+    sig << "col2im|" << (int)e.dtype << "|" << fmt << "|" << VEC << "|" << fh << "," << fw << "," << sth << "," << stw << "," << dh << "," << dw;
+    launch_special("col2im", sig.str(), P, (n / VEC + 255) / 256, G, [&](std::ostringstream& ss) {
+        ss << "  constexpr int VEC = " << VEC << ", FH = " << fh << ", FW = " << fw << ", STH = " << sth << ", STW = " << stw << ", DH = " << dh
+           << ", DW = " << dw << ", MAX_PH = " << max_ph << ", MAX_PW = " << max_pw << ";\n";
         ss << "  T* image = (T*)A.p[0];\n  const T* in = (const T*)A.p[1];\n";
-        ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(H * W);\n";
-        ss << "  const int patch_h = DH * (FH - 1) + 1, patch_w = DW * (FW - 1) + 1;\n";
+        ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(H * W) / VEC;\n";
+        ss << "  constexpr int patch_h = DH * (FH - 1) + 1, patch_w = DW * (FW - 1) + 1;\n";
         ss << "  for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {\n";
-        ss << "    unsigned rest = i; int q[4];\n";
-        // dimensions in memory order, slowest first: peel the fastest off first
-        for (int p = 3; p >= 1; --p) {
-            const char* ext = fmt[p] == 'N' ? "N" : (fmt[p] == 'C' ? "C" : (fmt[p] == 'H' ? "H" : "W"));
-            ss << "    q[" << p << "] = (int)(rest % (unsigned)" << ext << "); rest /= (unsigned)" << ext << ";\n";
-        }
-        ss << "    q[0] = (int)rest;\n";
-        ss << "    const int n = q[" << fmt.find('N') << "], c = q[" << fmt.find('C') << "];\n";
-        ss << "    const int h = q[" << fmt.find('H') << "] + PH, w = q[" << fmt.find('W') << "] + PW;\n";
+        ss << emit_decompose(fmt, "H", "W", "h_", "w_", true);
+        ss << "    const int h = h_ + PH, w = w_ + PW;\n";
         ss << "    const int ph_min = h < patch_h ? h % DH : (h - patch_h + STH) / STH;\n";
         ss << "    const int pw_min = w < patch_w ? w % DW : (w - patch_w + STW) / STW;\n";
         ss << "    const int ph_max = (h + STH) / STH < OH ? (h + STH) / STH : OH;\n";
         ss << "    const int pw_max = (w + STW) / STW < OW ? (w + STW) / STW : OW;\n";
-        ss << "    T res = (T)0;\n";
-        ss << "    for (int ph = ph_min; ph < ph_max; ph += DH)\n      for (int pw = pw_min; pw < pw_max; pw += DW) {\n";
+        ss << "    dali_vec<T, VEC> res;\n    _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) res.v[k] = (T)0;\n";
+        ss << "    // patches in the reference's order (rows outermost); beyond the range the load goes to the matrix's first element and is not added\n";
+        ss << "    _Pragma(\"unroll\") for (int a = 0; a < MAX_PH; ++a) {\n      const int ph = ph_min + a * DH; const bool ph_ok = ph < ph_max;\n";
+        ss << "      _Pragma(\"unroll\") for (int b = 0; b < MAX_PW; ++b) {\n        const int pw = pw_min + b * DW; const bool ok = ph_ok && pw < pw_max;\n";
         ss << "        const int kh = (h - ph * STH) / DH, kw = (w - pw * STW) / DW;\n";
         ss << "        const int row = " << emit_join_row(fmt) << ";\n";
-        ss << "        res += in[(long)row * ORS + (long)((n * OH + ph) * OW + pw) * OCS];\n      }\n";
-        ss << "    image[i] = res;\n  }\n}\n";
-        return ss.str();
+        ss << "        const T* src = ok ? in + ((long)row * ORS + (long)((n * OH + ph) * OW + pw) * OCS) : in;\n";
+        ss << "        const dali_vec<T, VEC> v = dali_load<T, VEC>(src);\n";
+        ss << "        if (ok) { _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) res.v[k] += v.v[k]; }\n      }\n    }\n";
+        ss << "    dali_store<T, VEC>(image + (long)i * VEC, res);\n  }\n}\n";
     });
     return dest;
 }
 
-const char* const kPoolGeomNames[] = {"N", "C", "H", "W", "SN", "SC", "SH", "SW", "WH", "WW", "STH", "STW", "PH", "PW",
-                                      "OH", "OW", "YSN", "YSC", "YSH", "YSW"};
-
-std::vector<int> pool_geom(const Expr& e, const ImageGeom& gx, const ImageGeom& gy) {
-    return {gx.ext[0], gx.ext[1], gx.ext[2], gx.ext[3], gx.stride[0], gx.stride[1], gx.stride[2], gx.stride[3], e.geom[0], e.geom[1],
-            e.geom[2], e.geom[3], e.geom[4], e.geom[5], gy.ext[2], gy.ext[3], gy.stride[0], gy.stride[1], gy.stride[2], gy.stride[3]};
+GeomInts pool_geom(const Expr& e, const ImageGeom& gx, const ImageGeom& gy, int groups) {
+    GeomInts G;
+    G.add_image(gx);
+    G.add("PH", e.geom[4]);
+    G.add("PW", e.geom[5]);
+    G.add_div("OH", gy.ext[2]);
+    G.add_div("OW", gy.ext[3]);
+    G.add("YSN", gy.stride[0]);
+    G.add("YSC", gy.stride[1]);
+    G.add("YSH", gy.stride[2]);
+    G.add("YSW", gy.stride[3]);
+    G.add_div("INNER_GROUPS", std::max(1, groups));
+    return G;
 }
 
-// Source text: linear index `i` of a dense array in `fmt` order -> n, c, and the two spatial coordinates
-std::string emit_decompose(const std::string& fmt, const char* eh, const char* ew, const char* nh, const char* nw) {
+std::string pool_constants(const Expr& e, int VEC) {
     std::ostringstream ss;
-    ss << "    unsigned rest = i; int q[4];\n";
-    for (int p = 3; p >= 1; --p) {
-        std::string ext = fmt[p] == 'N' ? "N" : (fmt[p] == 'C' ? "C" : (fmt[p] == 'H' ? eh : ew));
-        ss << "    q[" << p << "] = (int)(rest % (unsigned)" << ext << "); rest /= (unsigned)" << ext << ";\n";
-    }
-    ss << "    q[0] = (int)rest;\n";
-    ss << "    const int n = q[" << fmt.find('N') << "], c = q[" << fmt.find('C') << "], " << nh << " = q[" << fmt.find('H') << "], " << nw << " = q["
-       << fmt.find('W') << "];\n";
+    ss << "  constexpr int VEC = " << VEC << ", WH = " << e.geom[0] << ", WW = " << e.geom[1] << ", STH = " << e.geom[2] << ", STW = " << e.geom[3] << ";\n";
     return ss.str();
 }
 
-// pool2d: one thread per output element; the window is clipped to the image and walked columns outermost, as the
-// reference's loop does (conv.cpp:66-89), so an average is the same sequence of fp32 additions.
+// pool2d: one thread per output element (four channels of it where the channels are contiguous). The window is
+// walked columns outermost, as the reference's loop does (conv.cpp:66-89), so an average is the same sequence of
+// fp32 additions; window and stride are compile-time, which turns the walk into independent loads at clamped
+// coordinates whose values are used only where the window lies inside the image.
 Array run_pool2d(const Expr& e, const Array& x_in) {
     Array x = dense_buffer(x_in);
     const std::string& fmt = e.data_format;
@@ -3190,37 +3256,35 @@ Array run_pool2d(const Expr& e, const Array& x_in) {
     if (n == 0) return dest;
     ImageGeom gx = image_geom(x.shape(), fmt), gy = image_geom(e.shape, fmt);
     const bool average = e.depth != 0;
-    std::string t = ctype(e.dtype);
+    const int VEC = fmt[3] == 'C' && four_byte_vectors(e.dtype, x, gx.ext[1]) ? 4 : 1;
     Program P;
     P.arrays.push_back(manual_arg(dest, Cls::FULL, true, 1, {(int)n}, {}));
     P.arrays.push_back(manual_arg(x, Cls::FULL, false, 1, {(int)numel_of(x.shape())}, {}));
     std::ostringstream sig;
-    sig << "pool2d|" << (int)e.dtype << "|" << fmt << "|" << average;
-    launch_special("pool2d", sig.str(), P, (n + 255) / 256, pool_geom(e, gx, gy), [&](const std::string& kname, const IvLayout& L) {
-        std::ostringstream ss;
-        ss << special_head(P, L, kname, t, 20, kPoolGeomNames);
+    sig << "pool2d|" << (int)e.dtype << "|" << fmt << "|" << average << "|" << VEC << "|" << e.geom[0] << "," << e.geom[1] << "," << e.geom[2] << "," << e.geom[3];
+    launch_special("pool2d", sig.str(), P, (n / VEC + 255) / 256, pool_geom(e, gx, gy, e.shape[3] / VEC), [&](std::ostringstream& ss) {
+        ss << pool_constants(e, VEC);
         ss << "  T* y = (T*)A.p[0];\n  const T* x = (const T*)A.p[1];\n";
-        ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(OH * OW);\n";
+        ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(OH * OW) / VEC;\n";
         ss << "  for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {\n";
-        ss << emit_decompose(fmt, "OH", "OW", "oh", "ow");
-        ss << "    int w_start = ow * STW, w_end = w_start + WW;\n";
-        ss << "    w_start = w_start - PW > 0 ? w_start - PW : 0;\n    w_end = w_end - PW < W ? w_end - PW : W;\n";
-        ss << "    int h_start = oh * STH, h_end = h_start + WH;\n";
-        ss << "    h_start = h_start - PH > 0 ? h_start - PH : 0;\n    h_end = h_end - PH < H ? h_end - PH : H;\n";
-        ss << "    const T* xp = x + (long)n * SN + (long)c * SC;\n";
-        ss << "    T res = " << (average ? "(T)0" : "reducers::lowest<T>()") << ";\n";
-        ss << "    for (int w = w_start; w < w_end; ++w)\n      for (int h = h_start; h < h_end; ++h) {\n";
-        ss << "        const T v = xp[(long)h * SH + (long)w * SW];\n";
-        ss << "        res = " << (average ? "res + v" : "res > v ? res : v") << ";\n      }\n";
-        if (average) ss << "    res = res / ((h_end - h_start) * (w_end - w_start));\n";
-        ss << "    y[i] = res;\n  }\n}\n";
-        return ss.str();
+        ss << emit_decompose(fmt, "OH", "OW", "oh", "ow", true);
+        ss << "    const int w0 = ow * STW - PW, h0 = oh * STH - PH;\n";
+        ss << "    const int w_start = w0 > 0 ? w0 : 0, w_end = w0 + WW < W ? w0 + WW : W;\n";
+        ss << "    const int h_start = h0 > 0 ? h0 : 0, h_end = h0 + WH < H ? h0 + WH : H;\n";
+        ss << "    const T* xp = x + ((long)n * SN + (long)c * SC);\n";
+        ss << "    dali_vec<T, VEC> res;\n    _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) res.v[k] = " << (average ? "(T)0" : "reducers::lowest<T>()") << ";\n";
+        ss << "    _Pragma(\"unroll\") for (int a = 0; a < WW; ++a) {\n      const int w = w0 + a; const bool w_ok = w >= 0 && w < W; const int wc = w_ok ? w : w_start;\n";
+        ss << "      _Pragma(\"unroll\") for (int b = 0; b < WH; ++b) {\n        const int h = h0 + b; const bool ok = w_ok && h >= 0 && h < H; const int hc = h >= 0 && h < H ? h : h_start;\n";
+        ss << "        const dali_vec<T, VEC> v = dali_load<T, VEC>(xp + (hc * SH + wc * SW));\n";
+        ss << "        if (ok) { _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) res.v[k] = " << (average ? "res.v[k] + v.v[k]" : "res.v[k] > v.v[k] ? res.v[k] : v.v[k]") << "; }\n      }\n    }\n";
+        if (average) ss << "    _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) res.v[k] = res.v[k] / ((h_end - h_start) * (w_end - w_start));\n";
+        ss << "    dali_store<T, VEC>(y + (long)i * VEC, res);\n  }\n}\n";
     });
     return dest;
 }
 
-// pool2d_backward: one thread per input element, summing over the windows that hold it, window rows outermost
-// (conv.cpp:133-172).
+// pool2d_backward: one thread per input element (or four channels of it), summing over the windows that hold it,
+// window rows outermost (conv.cpp:133-172); at most ceil(window / stride) windows per direction, unrolled.
 Array run_pool2d_backward(const Expr& e, const Array& y_in, const Array& dy_in, const Array& x_in) {
     Array y = dense_buffer(y_in), dy = dense_buffer(dy_in), x = dense_buffer(x_in);
     const std::string& fmt = e.data_format;
@@ -3229,41 +3293,44 @@ Array run_pool2d_backward(const Expr& e, const Array& y_in, const Array& dy_in, 
     if (n == 0) return dest;
     ImageGeom gx = image_geom(x.shape(), fmt), gy = image_geom(y.shape(), fmt);
     const bool average = e.depth != 0;
-    std::string t = ctype(e.dtype);
+    const int VEC = fmt[3] == 'C' && four_byte_vectors(e.dtype, x, gx.ext[1]) && y.offset() % 4 == 0 && dy.offset() % 4 == 0 ? 4 : 1;
     Program P;
     P.arrays.push_back(manual_arg(dest, Cls::FULL, true, 1, {(int)n}, {}));
     P.arrays.push_back(manual_arg(y, Cls::FULL, false, 1, {(int)numel_of(y.shape())}, {}));
     P.arrays.push_back(manual_arg(dy, Cls::FULL, false, 1, {(int)numel_of(dy.shape())}, {}));
     P.arrays.push_back(manual_arg(x, Cls::FULL, false, 1, {(int)numel_of(x.shape())}, {}));
     std::ostringstream sig;
-    sig << "pool2d_backward|" << (int)e.dtype << "|" << fmt << "|" << average;
-    launch_special("pool2d_backward", sig.str(), P, (n + 255) / 256, pool_geom(e, gx, gy), [&](const std::string& kname, const IvLayout& L) {
-        std::ostringstream ss;
-        ss << special_head(P, L, kname, t, 20, kPoolGeomNames);
+    sig << "pool2d_backward|" << (int)e.dtype << "|" << fmt << "|" << average << "|" << VEC << "|" << e.geom[0] << "," << e.geom[1] << "," << e.geom[2] << ","
+        << e.geom[3];
+    launch_special("pool2d_backward", sig.str(), P, (n / VEC + 255) / 256, pool_geom(e, gx, gy, e.shape[3] / VEC), [&](std::ostringstream& ss) {
+        ss << pool_constants(e, VEC);
+        ss << "  constexpr int MAX_PH = (WH + STH - 1) / STH, MAX_PW = (WW + STW - 1) / STW;\n";
         ss << "  T* dx = (T*)A.p[0];\n  const T* y = (const T*)A.p[1];\n  const T* dy = (const T*)A.p[2];\n  const T* x = (const T*)A.p[3];\n";
-        ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(H * W);\n";
+        ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(H * W) / VEC;\n";
         ss << "  for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {\n";
-        ss << emit_decompose(fmt, "H", "W", "h", "w");
-        ss << "    const T src = x[i];\n";
+        ss << emit_decompose(fmt, "H", "W", "h", "w", true);
+        ss << "    const dali_vec<T, VEC> src = dali_load<T, VEC>(x + (long)i * VEC);\n";
         ss << "    const int ph_start = (h + PH) < WH ? 0 : (h + PH - WH) / STH + 1;\n";
         ss << "    const int pw_start = (w + PW) < WW ? 0 : (w + PW - WW) / STW + 1;\n";
         ss << "    const int ph_end = (h + PH) / STH + 1 < OH ? (h + PH) / STH + 1 : OH;\n";
         ss << "    const int pw_end = (w + PW) / STW + 1 < OW ? (w + PW) / STW + 1 : OW;\n";
         ss << "    const long base = (long)n * YSN + (long)c * YSC;\n";
-        ss << "    T grad = (T)0;\n";
-        ss << "    for (int ph = ph_start; ph < ph_end; ++ph)\n      for (int pw = pw_start; pw < pw_end; ++pw) {\n";
-        ss << "        const long q = base + (long)ph * YSH + (long)pw * YSW;\n";
+        ss << "    dali_vec<T, VEC> grad;\n    _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) grad.v[k] = (T)0;\n";
+        ss << "    _Pragma(\"unroll\") for (int a = 0; a < MAX_PH; ++a) {\n      const int ph = ph_start + a; const bool ph_ok = ph < ph_end;\n";
+        ss << "      _Pragma(\"unroll\") for (int b = 0; b < MAX_PW; ++b) {\n        const int pw = pw_start + b; const bool ok = ph_ok && pw < pw_end;\n";
+        ss << "        const long q = ok ? base + (ph * YSH + pw * YSW) : 0;  // beyond the range: a valid address, value unused\n";
+        ss << "        const dali_vec<T, VEC> g = dali_load<T, VEC>(dy + q);\n";
         if (average) {
             ss << "        int hstart = ph * STH - PH, wstart = pw * STW - PW;\n";
             ss << "        const int hend = hstart + WH < H ? hstart + WH : H, wend = wstart + WW < W ? wstart + WW : W;\n";
             ss << "        hstart = hstart > 0 ? hstart : 0; wstart = wstart > 0 ? wstart : 0;\n";
             ss << "        const int pool_size = (hend - hstart) * (wend - wstart);\n";
-            ss << "        grad += ((T)1 * dy[q]) / pool_size;\n      }\n";
+            ss << "        if (ok) { _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) grad.v[k] += ((T)1 * g.v[k]) / pool_size; }\n      }\n    }\n";
         } else {
-            ss << "        grad += (y[q] == src ? (T)1 : (T)0) * dy[q];\n      }\n";
+            ss << "        const dali_vec<T, VEC> yv = dali_load<T, VEC>(y + q);\n";
+            ss << "        if (ok) { _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) grad.v[k] += (yv.v[k] == src.v[k] ? (T)1 : (T)0) * g.v[k]; }\n      }\n    }\n";
         }
-        ss << "    dx[i] = grad;\n  }\n}\n";
-        return ss.str();
+        ss << "    dali_store<T, VEC>(dx + (long)i * VEC, grad);\n  }\n}\n";
     });
     return dest;
 }

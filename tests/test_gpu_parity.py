@@ -144,7 +144,9 @@ def _dev(hip, a):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (5, 11, 7), (64, 64, 64), (65, 130, 33), (256, 4096, 128), (300, 200, 100),
-                                   (132, 72, 640), (252, 1000, 1000), (1100, 2300, 260), (2052, 2052, 132)])
+                                   (132, 72, 640), (252, 1000, 1000), (1100, 2300, 260), (2052, 2052, 132),
+                                   # few tiles over a long inner extent: shares of K folded across workgroups
+                                   (64, 64, 8192), (128, 576, 20001), (130, 70, 4100)])
 @pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
 def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
     """dali_hip_sgemm(transB, transA, m, n, k, alpha, B, ldb, A, lda, beta, C, ldc) as cublasSgemm is called in
