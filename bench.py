@@ -249,7 +249,13 @@ def main():
                                                  "gemm_pair_us": round(gemm_us, 2),
                                                  "gemm_TFLOP/s": round(flops / gemm_us / 1e6, 2),
                                                  "gemm_frac_fp32_mfma": round(flops / gemm_us / 1e6 / MFMA_FP32_PEAK_TFLOPS, 4)}
-        del X, Hp, Cp, W, U, bias, rec, grec
+        # the same step along a sequence of 32: fused launches chained through one [T, B, H] buffer
+        Xs = D.Array.from_numpy(np.random.RandomState(23).randn(32, B, H).astype(np.float32))
+        with D.Recording() as srec:
+            op.lstm_sequence(Xs, Hp, Cp, W, U, bias)
+        seq_us = time_recording(srec, 10)
+        configs["c5_lstm_step_256x1024x1024"]["sequence_of_32_us_per_step"] = round(seq_us / 32, 2)
+        del X, Hp, Cp, W, U, bias, rec, grec, Xs, srec
 
         # rows beyond the five configs: embedding-style gather and its scatter-add (table [32000, 1024], 8192 indices)
         V, Dm, Nidx = 32000, 1024, 8192
@@ -279,6 +285,49 @@ def main():
         nxt["cumsum_8192x8192"] = {"us": round(us, 2), "GB/s": round(2 * 8192 * 8192 * 4 / us / 1e3, 1),
                                    "frac_hbm": round(2 * 8192 * 8192 * 4 / us / 1e3 / HBM_PEAK_GBS, 4), "kernels": rec.launches}
         del sm, rec
+        # sliding windows in the channels-last layout: a 3x3 convolution layer (64 -> 128 channels, 32 images of 56x56) as
+        # im2col + one matrix product, its two gradients, and a 3x3 / stride 2 max pooling of 32 images of 112x112x64
+        xi = D.Array.from_numpy(np.random.RandomState(18).randn(32, 56, 56, 64).astype(np.float32))
+        wf = D.Array.from_numpy(np.random.RandomState(19).randn(128, 3, 3, 64).astype(np.float32))
+        with D.Recording() as rec:
+            op.im2col(xi, 3, 3, 1, 1, 1, 1, 1, 1, data_format="NHWC").eval()
+        us = time_recording(rec, 20)
+        ibytes = (32 * 56 * 56 * 64 + 576 * 32 * 56 * 56) * 4
+        nxt["im2col_nhwc_32x56x56x64_3x3"] = {"us": round(us, 2), "GB/s": round(ibytes / us / 1e3, 1),
+                                              "frac_hbm": round(ibytes / us / 1e3 / HBM_PEAK_GBS, 4), "kernels": rec.launches}
+        with D.Recording() as rec:
+            yc = op.conv2d(xi, wf, 1, 1, "same", "NHWC")
+            yc.eval()
+        us = time_recording(rec, 20)
+        cflops = 2.0 * 128 * 576 * 32 * 56 * 56
+        nxt["conv2d_nhwc_64to128_3x3_same"] = {"us": round(us, 2), "TFLOP/s": round(cflops / us / 1e6, 2), "launches": rec.launches,
+                                               "frac_fp32_mfma": round(cflops / us / 1e6 / MFMA_FP32_PEAK_TFLOPS, 4)}
+        dyc = D.Array.from_numpy(np.random.RandomState(20).randn(32, 54, 54, 128).astype(np.float32))
+        vflops = 2.0 * 128 * 576 * 32 * 54 * 54
+        with D.Recording() as rec:
+            op.conv2d_backward_input(wf, dyc, 1, 1, (32, 56, 56, 64), "valid", "NHWC").eval()
+        us = time_recording(rec, 20)
+        nxt["conv2d_backward_input_nhwc_valid"] = {"us": round(us, 2), "TFLOP/s": round(vflops / us / 1e6, 2), "launches": rec.launches}
+        with D.Recording() as rec:
+            op.conv2d_backward_filters(xi, dyc, 1, 1, (128, 3, 3, 64), "valid", "NHWC").eval()
+        us = time_recording(rec, 20)
+        nxt["conv2d_backward_filters_nhwc_valid"] = {"us": round(us, 2), "TFLOP/s": round(vflops / us / 1e6, 2), "launches": rec.launches}
+        del xi, wf, yc, dyc, rec
+        xp = D.Array.from_numpy(np.random.RandomState(21).randn(32, 112, 112, 64).astype(np.float32))
+        with D.Recording() as rec:
+            yp = op.pool2d(xp, 3, 3, 2, 2, "max", "same", "NHWC")
+            yp.eval()
+        us = time_recording(rec, 20)
+        pbytes = (32 * 112 * 112 * 64 + 32 * 56 * 56 * 64) * 4
+        nxt["pool2d_max_nhwc_32x112x112x64_3x3_s2"] = {"us": round(us, 2), "GB/s": round(pbytes / us / 1e3, 1),
+                                                       "frac_hbm": round(pbytes / us / 1e3 / HBM_PEAK_GBS, 4), "kernels": rec.launches}
+        dyp = D.Array.from_numpy(np.random.RandomState(22).randn(32, 56, 56, 64).astype(np.float32))
+        with D.Recording() as rec:
+            op.pool2d_backward(yp, dyp, xp, 3, 3, 2, 2, "max", "same", "NHWC").eval()
+        us = time_recording(rec, 20)
+        nxt["pool2d_max_backward_nhwc"] = {"us": round(us, 2), "GB/s": round(2 * pbytes / us / 1e3, 1),
+                                           "frac_hbm": round(2 * pbytes / us / 1e3 / HBM_PEAK_GBS, 4), "kernels": rec.launches}
+        del xp, yp, dyp, rec
         configs["beyond_the_five_configs"] = nxt
         result["configs"] = configs
 

@@ -1236,5 +1236,67 @@ LSTMState lstm_step(const Array& x, const Array& h, const Array& c, const Array&
     return {c_new, h_new};
 }
 
+// The step above applied along a sequence (dali/layers/lstm.cpp:294-303): xs is [T, B, I]; returns every hidden
+// state as one [T, B, H] buffer plus the final cell state. With the fused kernel each step is one launch that reads
+// h(t-1) from, and writes h(t) into, its slice of that buffer; nothing is copied between steps.
+LSTMSequence lstm_sequence(const Array& xs, const Array& h0, const Array& c0, const Array& W, const Array& U, const Array& b) {
+    DALI_ASSERT(xs.ndim() == 3 && h0.ndim() == 2 && c0.ndim() == 2, "lstm_sequence: xs must be [T, B, I], h0 and c0 [B, H]");
+    const int T = xs.shape()[0], Bn = xs.shape()[1], In = xs.shape()[2], H = h0.shape()[1];
+    DALI_ASSERT(T >= 1, "lstm_sequence: the sequence must hold at least one step");
+    DALI_ASSERT(h0.shape()[0] == Bn && c0.shape() == h0.shape(), "lstm_sequence: inconsistent batch sizes");
+    static const bool fused_off = getenv("DALI_HIP_LSTM_UNFUSED") != nullptr;
+    auto dense = [](const Array& a) { return a.is_buffer() && a.contiguous_memory() && a.dtype() == DTYPE_FLOAT; };
+    for (const Array* a : {&xs, &h0, &c0, &W, &U, &b}) a->eval();
+    Array seq = xs.is_buffer() && xs.contiguous_memory() ? xs : xs.ascontiguousarray();
+    Array hs({T, Bn, H}, DTYPE_FLOAT);
+    Array cells[2] = {Array({Bn, H}, DTYPE_FLOAT), Array({Bn, H}, DTYPE_FLOAT)};
+    const bool fused = !fused_off && !dry_run() && H % 64 == 0 && In == H && dense(seq) && dense(h0) && dense(c0) && dense(W) && dense(U) && dense(b) &&
+                       W.ndim() == 2 && U.ndim() == 2 && b.ndim() == 1 && W.shape()[0] == In && W.shape()[1] == 4 * H && U.shape()[0] == H &&
+                       U.shape()[1] == 4 * H && b.shape()[0] == 4 * H && seq.offset() % 4 == 0 && h0.offset() % 4 == 0 && W.offset() % 4 == 0 &&
+                       U.offset() % 4 == 0 && ((int64_t)Bn * H) % 4 == 0;
+    Array c_prev = c0, h_prev = h0;
+    for (int t = 0; t < T; ++t) {
+        Array x_t = seq[t], h_t = hs[t];
+        if (fused) {
+            lstm_step_fused(x_t, h_prev, c_prev, W, U, b, cells[t % 2], h_t);
+            c_prev = cells[t % 2];
+        } else {
+            LSTMState st = lstm_step(x_t, h_prev, c_prev, W, U, b);
+            h_t.assign(st.hidden);
+            c_prev = st.memory;
+        }
+        h_prev = h_t;
+    }
+    return {hs, c_prev, h_prev};
+}
+
+// One GRU step (dali/layers/gru.cpp:27-44 with StackedInputLayer::activate, dali/layers/layers.cpp:159-161), the
+// three input layers packed reset, update, candidate along the columns of W[I, 3H], U[H, 3H], b[3H]:
+//   r = sigmoid(x.Wr + h.Ur + br);  z = sigmoid(x.Wz + h.Uz + bz);  m = tanh(x.Wc + (r * h).Uc + bc)
+//   h' = h * (1.0 - z) + m * z
+// Three matrix products (the candidate's recurrent product needs r first) and two fused elementwise kernels.
+Array gru_step(const Array& x, const Array& h, const Array& W, const Array& U, const Array& b) {
+    DALI_ASSERT(x.ndim() == 2 && h.ndim() == 2 && W.ndim() == 2 && U.ndim() == 2 && b.ndim() == 1, "gru_step: x, h, W, U must be matrices and b a vector");
+    const int H = h.shape()[1];
+    DALI_ASSERT(W.shape()[1] == 3 * H && U.shape()[1] == 3 * H && b.shape()[0] == 3 * H && U.shape()[0] == H && W.shape()[0] == x.shape()[1] &&
+                    x.shape()[0] == h.shape()[0],
+                "gru_step: inconsistent shapes");
+    for (const Array* a : {&x, &h, &W, &U, &b}) a->eval();
+    Array px = dot(x, W);                          // [B, 3H]
+    Array ph = dot(h, U.slice(1, 0, 2 * H));       // [B, 2H]: reset and update see h itself
+    px.eval();
+    ph.eval();
+    auto bias = [&](int k) { return b.slice(0, k * H, (k + 1) * H).expand_dims(0); };
+    auto cols = [&](const Array& a, int k) { return a.slice(1, k * H, (k + 1) * H); };
+    Array reset_state = eltmul(sigmoid(add(add(cols(px, 0), cols(ph, 0)), bias(0))), h);
+    Array pc = dot(reset_state, U.slice(1, 2 * H, 3 * H));
+    pc.eval();
+    Array update = sigmoid(add(add(cols(px, 1), cols(ph, 1)), bias(1)));
+    Array candidate = tanh(add(add(cols(px, 2), pc), bias(2)));
+    Array h_new = add(eltmul(h, subtract(Array(1.0), update)), eltmul(candidate, update));
+    h_new.eval();
+    return h_new;
+}
+
 }  // namespace op
 }  // namespace dali

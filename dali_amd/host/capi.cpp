@@ -174,6 +174,16 @@ int dali_fe_lstm_step(dali_array_t x, dali_array_t h, dali_array_t c, dali_array
     FE_TRY(auto r = dali::op::lstm_step(A(x), A(h), A(c), A(W), A(U), A(b)); *c_new = wrap(r.memory); *h_new = wrap(r.hidden); return 0;, 1)
 }
 
+int dali_fe_lstm_sequence(dali_array_t xs, dali_array_t h0, dali_array_t c0, dali_array_t W, dali_array_t U, dali_array_t b,
+                          dali_array_t* hidden_states, dali_array_t* memory, dali_array_t* hidden) {
+    FE_TRY(auto r = dali::op::lstm_sequence(A(xs), A(h0), A(c0), A(W), A(U), A(b)); *hidden_states = wrap(r.hidden_states);
+           *memory = wrap(r.memory); *hidden = wrap(r.hidden); return 0;
+           , 1)
+}
+dali_array_t dali_fe_gru_step(dali_array_t x, dali_array_t h, dali_array_t W, dali_array_t U, dali_array_t b) {
+    FE_TRY(return wrap(dali::op::gru_step(A(x), A(h), A(W), A(U), A(b)));, nullptr)
+}
+
 int dali_fe_eval(dali_array_t a) { FE_TRY(A(a).eval(); return 0;, 1) }
 int dali_fe_eval_together(dali_array_t* roots, int n) {
     FE_TRY(std::vector<Array> r; for (int i = 0; i < n; ++i) r.push_back(A(roots[i])); Array::eval_together(r); return 0;, 1)

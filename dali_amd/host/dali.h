@@ -326,6 +326,15 @@ struct LSTMState {
 };
 LSTMState lstm_step(const Array& x, const Array& h, const Array& c, const Array& W, const Array& U,
                     const Array& b);
+// The step along a sequence xs[T, B, I] (dali/layers/lstm.cpp:294-303): all hidden states [T, B, H], the final
+// cell state and the final hidden state (a view of the last slice).
+struct LSTMSequence {
+    Array hidden_states, memory, hidden;
+};
+LSTMSequence lstm_sequence(const Array& xs, const Array& h0, const Array& c0, const Array& W, const Array& U, const Array& b);
+// One GRU step with reset, update and candidate layers packed along the columns of W[I,3H], U[H,3H], b[3H]
+// (dali/layers/gru.cpp:27-44). Returns h', already evaluated.
+Array gru_step(const Array& x, const Array& h, const Array& W, const Array& U, const Array& b);
 }  // namespace op
 
 // Observation hooks in the spirit of dali/utils/scope.h: counts of executed

@@ -180,6 +180,21 @@ def lstm_step(x, h, c, W, U, b):
     return tuple(Array(o.value) for o in outs)
 
 
+def lstm_sequence(xs, h0, c0, W, U, b):
+    """The LSTM step along xs[T, B, I]; returns (hidden_states [T, B, H], final memory, final hidden), evaluated."""
+    outs = [C.c_void_p() for _ in range(3)]
+    keep = [as_array(v) for v in (xs, h0, c0, W, U, b)]
+    if front.dali_fe_lstm_sequence(*[k._h for k in keep], *[C.byref(o) for o in outs]) != 0:
+        raise fe_error("lstm_sequence")
+    return tuple(Array(o.value) for o in outs)
+
+
+def gru_step(x, h, W, U, b):
+    """One GRU step; reset / update / candidate layers packed along the columns of W[I,3H], U[H,3H], b[3H]."""
+    keep = [as_array(v) for v in (x, h, W, U, b)]
+    return _wrap(front.dali_fe_gru_step(*[k._h for k in keep]), "gru_step")
+
+
 # dali/array/op/reducers.cpp:61-72, binary.cpp:7-12
 def any_isnan(x, axes=None, keepdims=False):
     return max(isnan(x), axes, keepdims)

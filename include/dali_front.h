@@ -102,6 +102,12 @@ int dali_fe_softmax_cross_entropy(dali_array_t logits, dali_array_t targets, dal
                                   dali_array_t* row_loss, dali_array_t* grad);
 int dali_fe_lstm_step(dali_array_t x, dali_array_t h, dali_array_t c, dali_array_t W, dali_array_t U, dali_array_t b,
                       dali_array_t* c_new, dali_array_t* h_new);
+/* The LSTM step along xs[T, B, I] (dali/layers/lstm.cpp:294-303): hidden_states [T, B, H], final memory and hidden [B, H] */
+int dali_fe_lstm_sequence(dali_array_t xs, dali_array_t h0, dali_array_t c0, dali_array_t W, dali_array_t U, dali_array_t b,
+                          dali_array_t* hidden_states, dali_array_t* memory, dali_array_t* hidden);
+/* One GRU step, layers packed reset / update / candidate along the columns of W[I,3H], U[H,3H], b[3H]
+ * (dali/layers/gru.cpp:27-44) */
+dali_array_t dali_fe_gru_step(dali_array_t x, dali_array_t h, dali_array_t W, dali_array_t U, dali_array_t b);
 
 /* evaluation, assignment, host access */
 int dali_fe_eval(dali_array_t a);

@@ -384,3 +384,30 @@ def lstm_step(X, H, Cm, W, U, b, f64_gemm=True):
     h_new = np.empty((B, Hd), dtype=np.float32)
     lib.orc_lstm_step(fp(X), fp(H), fp(Cm), fp(W), fp(U), fp(b), B, I, Hd, 1 if f64_gemm else 0, fp(gates), fp(c_new), fp(h_new))
     return gates, c_new, h_new
+
+
+def lstm_sequence(Xs, H0, C0, W, U, b, f64_gemm=True):
+    """lstm_step along Xs[T, B, I] (dali/layers/lstm.cpp:294-303): (all hidden states, final memory)."""
+    h, c, hs = H0, C0, []
+    for t in range(Xs.shape[0]):
+        _, c, h = lstm_step(Xs[t], h, c, W, U, b, f64_gemm)
+        hs.append(h)
+    return np.stack(hs), c
+
+
+def gru_step(X, Hs, W, U, b):
+    """dali/layers/gru.cpp:27-44 with the layers packed reset / update / candidate: products accumulated in fp64, the
+    gate arithmetic through the checker's functors (sigmoid in double, libm tanhf), every operation rounded to fp32.
+    No test of the reference pins GRU values: PARITY UNPINNED beyond the composition of pinned parts."""
+    X, Hs, W, U, b = map(_c32, (X, Hs, W, U, b))
+    Hn = Hs.shape[1]
+    px, ph = gemm(X, W), gemm(Hs, np.ascontiguousarray(U[:, :2 * Hn]))
+    f32 = np.float32
+    pre = lambda k, rec: ((px[:, k * Hn:(k + 1) * Hn] + rec).astype(f32) + b[k * Hn:(k + 1) * Hn]).astype(f32)
+    r = unary("sigmoid", pre(0, ph[:, :Hn]))
+    reset_state = (r * Hs).astype(f32)
+    pc = gemm(reset_state, np.ascontiguousarray(U[:, 2 * Hn:]))
+    z = unary("sigmoid", pre(1, ph[:, Hn:]))
+    m = unary("tanh", pre(2, pc))
+    one_minus = (np.float32(1.0) - z).astype(f32)
+    return ((Hs * one_minus).astype(f32) + (m * z).astype(f32)).astype(f32)

@@ -828,6 +828,50 @@ def test_fused_lstm_step_equals_the_two_launch_form(gpu, D, O, rng, B, H):
     close(hn.numpy(), ohn, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("T,B,I,H", [(5, 48, 128, 128), (3, 7, 24, 40), (12, 256, 64, 64)])
+def test_lstm_sequence_is_the_step_applied_in_turn(gpu, D, O, rng, T, B, I, H):
+    """LSTM::activate_sequence (dali/layers/lstm.cpp:294-303): fused steps chained through one [T, B, H] buffer when
+    input == hidden and both are multiples of 64, the unfused step otherwise."""
+    Xs = rng.randn(T, B, I).astype(np.float32)
+    H0, C0 = (rng.randn(B, H).astype(np.float32) for _ in range(2))
+    lim = np.sqrt(6.0 / (I + 4 * H))
+    W, U = (rng.uniform(-lim, lim, (n, 4 * H)).astype(np.float32) for n in (I, H))
+    b = (rng.randn(4 * H) * 0.1).astype(np.float32)
+    dev = [arr(D, v) for v in (Xs, H0, C0, W, U, b)]
+    with D.Recording() as rec:
+        hs, c_last, h_last = D.op.lstm_sequence(*dev)
+    if I == H and H % 64 == 0:
+        assert rec.launches == T  # one launch per step
+    assert hs.shape == (T, B, H) and np.array_equal(h_last.numpy(), hs.numpy()[-1])
+    # bit-equal to calling the step T times
+    h, c = dev[1], dev[2]
+    for t in range(T):
+        c, h = D.op.lstm_step(arr(D, Xs[t]), h, c, dev[3], dev[4], dev[5])
+        assert np.array_equal(hs.numpy()[t], h.numpy())
+    assert np.array_equal(c_last.numpy(), c.numpy())
+    ohs, oc = O.lstm_sequence(Xs, H0, C0, W, U, b)
+    close(hs.numpy(), ohs, rtol=2e-4, atol=2e-5)
+    close(c_last.numpy(), oc, rtol=2e-4, atol=2e-5)
+    # the recorded launches recompute the same sequence
+    first = hs.numpy().copy()
+    rec.replay(2)
+    assert np.array_equal(hs.numpy(), first)
+
+
+@pytest.mark.parametrize("B,I,H", [(16, 32, 48), (64, 128, 128), (5, 7, 9)])
+def test_gru_step_matches_oracle(gpu, D, O, rng, B, I, H):
+    X, Hp = rng.randn(B, I).astype(np.float32), rng.randn(B, H).astype(np.float32)
+    lim = np.sqrt(6.0 / (I + 3 * H))
+    W, U = (rng.uniform(-lim, lim, (n, 3 * H)).astype(np.float32) for n in (I, H))
+    b = (rng.randn(3 * H) * 0.1).astype(np.float32)
+    got = D.op.gru_step(*(arr(D, v) for v in (X, Hp, W, U, b))).numpy()
+    close(got, O.gru_step(X, Hp, W, U, b), rtol=1e-4, atol=1e-5)
+    # z = 1 everywhere (large update bias) keeps only the candidate; z = 0 keeps the old state
+    b_keep = b.copy()
+    b_keep[H:2 * H] = -60.0
+    assert np.array_equal(D.op.gru_step(*(arr(D, v) for v in (X, Hp, W, U, b_keep))).numpy(), Hp)
+
+
 @pytest.mark.parametrize("shape", [(3,), (2, 3, 4), (5, 257), (64, 1024), (3, 5000)])
 def test_circular_convolution_matches_oracle(gpu, D, O, rng, shape):
     # JITTests.circular_convolution / _broadcast / _1d (circular_convolution_tests.cpp:54-89)

@@ -570,3 +570,26 @@ def test_pool2d_pair_against_window_loops(O, rng):
                         assert np.abs(dx - dx_want).max() < 1e-6
                         dxh = O.pool2d_backward(yh, np.ascontiguousarray(dy.transpose(0, 2, 3, 1)), xh, wh, ww, sh, sw, mode, padding, "NHWC")
                         assert np.array_equal(dxh.transpose(0, 3, 1, 2), dx)
+
+
+def test_gru_step_against_fp64_definition(O, rng):
+    # dali/layers/gru.cpp:27-44 written out in fp64 with numpy; the checker rounds every operation to fp32
+    B, I, H = 6, 10, 8
+    X, Hp = rng.randn(B, I).astype(np.float32), rng.randn(B, H).astype(np.float32)
+    W, U = rng.uniform(-0.4, 0.4, (I, 3 * H)).astype(np.float32), rng.uniform(-0.4, 0.4, (H, 3 * H)).astype(np.float32)
+    b = (rng.randn(3 * H) * 0.1).astype(np.float32)
+    x, h, w, u, bb = (f64(v) for v in (X, Hp, W, U, b))
+    sig = lambda v: 1.0 / (1.0 + np.exp(-v))
+    r = sig(x @ w[:, :H] + h @ u[:, :H] + bb[:H])
+    z = sig(x @ w[:, H:2 * H] + h @ u[:, H:2 * H] + bb[H:2 * H])
+    m = np.tanh(x @ w[:, 2 * H:] + (r * h) @ u[:, 2 * H:] + bb[2 * H:])
+    want = h * (1.0 - z) + m * z
+    assert np.abs(O.gru_step(X, Hp, W, U, b) - want).max() < 2e-6
+    # the sequence wrapper is the step in turn
+    Xs = rng.randn(3, B, H).astype(np.float32)
+    W4, U4 = rng.uniform(-0.3, 0.3, (H, 4 * H)).astype(np.float32), rng.uniform(-0.3, 0.3, (H, 4 * H)).astype(np.float32)
+    b4 = np.zeros(4 * H, np.float32)
+    hs, c = O.lstm_sequence(Xs, Hp, Hp, W4, U4, b4)
+    _, c1, h1 = O.lstm_step(Xs[0], Hp, Hp, W4, U4, b4)
+    _, c2, h2 = O.lstm_step(Xs[1], h1, c1, W4, U4, b4)
+    assert np.array_equal(hs[1], h2) and hs.shape == (3, B, H)
