@@ -74,6 +74,10 @@ HIP_SYMBOLS = {
     "dali_hip_memcpy_h2d": (_i, [H, H, _sz]),
     "dali_hip_memcpy_d2h": (_i, [H, H, _sz]),
     "dali_hip_memcpy_d2d": (_i, [H, H, _sz]),
+    "dali_hip_host_alloc": (_i, [C.POINTER(H), _sz]),
+    "dali_hip_host_free": (_i, [H]),
+    "dali_hip_memcpy_h2d_async": (_i, [H, H, _sz, H]),
+    "dali_hip_memcpy_d2h_async": (_i, [H, H, _sz, H]),
     "dali_hip_module_load": (_i, [_u64, C.c_char_p, C.c_char_p, C.POINTER(LaunchPlan), _ip]),
     "dali_hip_module_is_loaded": (_i, [_u64]),
     "dali_hip_launch": (_i, [_u64, C.POINTER(H), _ip, C.POINTER(_ip), C.POINTER(_ip), C.POINTER(H), C.POINTER(_ip)]),
@@ -92,6 +96,9 @@ HIP_SYMBOLS = {
     "dali_hip_event_record": (_i, [H]),
     "dali_hip_event_elapsed_ms": (_i, [H, H, C.POINTER(C.c_float)]),
     "dali_hip_event_destroy": (_i, [H]),
+    "dali_hip_stream_wait_event": (_i, [H]),
+    "dali_hip_event_synchronize": (_i, [H]),
+    "dali_hip_event_query": (_i, [H, C.POINTER(_i)]),
 }
 for _name, (_res, _args) in HIP_SYMBOLS.items():
     _sig(hip, _name, _res, _args)
@@ -101,6 +108,8 @@ _HP = C.POINTER(H)
 FRONT_SYMBOLS = {
     "dali_fe_last_error": (C.c_char_p, []),
     "dali_fe_from_host": (H, [H, _ip, _i, _i]),
+    "dali_fe_from_host_pinned": (H, [H, _ip, _i, _i]),
+    "dali_fe_prefetch": (_i, [H, _i]),
     "dali_fe_empty": (H, [_ip, _i, _i]),
     "dali_fe_zeros": (H, [_ip, _i, _i]),
     "dali_fe_scalar_double": (H, [C.c_double]),

@@ -47,12 +47,21 @@ class Array(object):
 
     # ---- construction
     @staticmethod
-    def from_numpy(a):
+    def from_numpy(a, pinned=False):
+        """Copy ``a`` into a new buffer. ``pinned=True`` keeps the host copy in page-locked memory (needs an initialised
+        device), so that ``prefetch("gpu")`` / ``prefetch("cpu")`` migrate it without blocking."""
         a = np.ascontiguousarray(a)
         if a.dtype not in _FROM_NP:
             raise TypeError("dtype %s is not one of float32, float64, int32" % a.dtype)
         shape, nd = _ints(a.shape)
-        return _wrap(front.dali_fe_from_host(a.ctypes.data_as(C.c_void_p), shape, nd, _FROM_NP[a.dtype]), "from_numpy")
+        make = front.dali_fe_from_host_pinned if pinned else front.dali_fe_from_host
+        return _wrap(make(a.ctypes.data_as(C.c_void_p), shape, nd, _FROM_NP[a.dtype]), "from_numpy")
+
+    def prefetch(self, device="gpu"):
+        """Start migrating the buffer's fresh copy to ``device`` ("gpu" or "cpu"); blocking unless the host copy is pinned."""
+        if front.dali_fe_prefetch(self._h, 1 if device == "gpu" else 0) != 0:
+            raise fe_error("prefetch")
+        return self
 
     @staticmethod
     def empty(shape, dtype=DTYPE_FLOAT):

@@ -48,6 +48,9 @@ struct Runtime {
     bool ready = false;
     int device = -1;
     hipStream_t stream = nullptr;
+    // migrations that should not stall the compute stream run here (created on first use, default priority)
+    hipStream_t copy_stream = nullptr;
+    hipEvent_t order_event = nullptr;
     std::string arch = "gfx950";
     // workspace: [counters | partials]
     char* ws = nullptr;
@@ -367,6 +370,70 @@ int dali_hip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes) 
     if (ensure_init()) return DALI_HIP_ERROR;
     if (bytes == 0) return DALI_HIP_OK;
     HIP_TRY(hipMemcpyAsync(dst_device, src_device, bytes, hipMemcpyDeviceToDevice, rt().stream));
+    return DALI_HIP_OK;
+}
+
+int dali_hip_host_alloc(void** ptr, size_t bytes) {
+    if (ensure_init()) return DALI_HIP_ERROR;
+    if (!ptr) return fail("dali_hip_host_alloc: ptr is NULL");
+    HIP_TRY(hipHostMalloc(ptr, bytes ? bytes : 4, hipHostMallocDefault));
+    return DALI_HIP_OK;
+}
+
+int dali_hip_host_free(void* ptr) {
+    if (!ptr) return DALI_HIP_OK;
+    HIP_TRY(hipHostFree(ptr));
+    return DALI_HIP_OK;
+}
+
+// The copy stream starts a migration only after the work already issued on the compute stream (which may
+// still read or write the device block), and tells the caller's event when the bytes have arrived.
+static int async_copy(void* dst, const void* src, size_t bytes, hipMemcpyKind kind, void* done_event, const char* what) {
+    if (ensure_init()) return DALI_HIP_ERROR;
+    Runtime& r = rt();
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    HIP_TRY(hipStreamIsCapturing(r.stream, &cs));
+    if (cs != hipStreamCaptureStatusNone) return fail("%s: not allowed while the library stream is being captured", what);
+    {
+        std::lock_guard<std::mutex> lock(r.mu);
+        if (!r.copy_stream) {
+            HIP_TRY(hipStreamCreateWithFlags(&r.copy_stream, hipStreamNonBlocking));
+            HIP_TRY(hipEventCreateWithFlags(&r.order_event, hipEventDisableTiming));
+        }
+    }
+    HIP_TRY(hipEventRecord(r.order_event, r.stream));
+    HIP_TRY(hipStreamWaitEvent(r.copy_stream, r.order_event, 0));
+    if (bytes) HIP_TRY(hipMemcpyAsync(dst, src, bytes, kind, r.copy_stream));
+    if (done_event) HIP_TRY(hipEventRecord((hipEvent_t)done_event, r.copy_stream));
+    return DALI_HIP_OK;
+}
+
+int dali_hip_memcpy_h2d_async(void* dst_device, const void* src_pinned, size_t bytes, void* done_event) {
+    return async_copy(dst_device, src_pinned, bytes, hipMemcpyHostToDevice, done_event, "dali_hip_memcpy_h2d_async");
+}
+
+int dali_hip_memcpy_d2h_async(void* dst_pinned, const void* src_device, size_t bytes, void* done_event) {
+    return async_copy(dst_pinned, src_device, bytes, hipMemcpyDeviceToHost, done_event, "dali_hip_memcpy_d2h_async");
+}
+
+int dali_hip_stream_wait_event(void* event) {
+    if (ensure_init()) return DALI_HIP_ERROR;
+    if (!event) return fail("dali_hip_stream_wait_event: event is NULL");
+    HIP_TRY(hipStreamWaitEvent(rt().stream, (hipEvent_t)event, 0));
+    return DALI_HIP_OK;
+}
+
+int dali_hip_event_synchronize(void* event) {
+    if (!event) return fail("dali_hip_event_synchronize: event is NULL");
+    HIP_TRY(hipEventSynchronize((hipEvent_t)event));
+    return DALI_HIP_OK;
+}
+
+int dali_hip_event_query(void* event, int* done) {
+    if (!event || !done) return fail("dali_hip_event_query: NULL argument");
+    hipError_t e = hipEventQuery((hipEvent_t)event);
+    if (e != hipSuccess && e != hipErrorNotReady) return fail("dali_hip_event_query: %s", hipGetErrorString(e));
+    *done = e == hipSuccess ? 1 : 0;
     return DALI_HIP_OK;
 }
 

@@ -45,13 +45,78 @@ std::vector<int> contiguous_strides(const std::vector<int>& shape) {
 // ------------------------------------------------------------------ memory
 namespace memory {
 
-SynchronizedMemory::SynchronizedMemory(size_t bytes) : bytes_(bytes) {}
+SynchronizedMemory::SynchronizedMemory(size_t bytes, bool pinned_host) : bytes_(bytes), pinned_host_(pinned_host) {}
 
 SynchronizedMemory::~SynchronizedMemory() {
-    if (host_) std::free(host_);
+    // transfers in flight still use both blocks
+    for (void* ev : {to_device_event_, to_host_event_})
+        if (ev) {
+            dali_hip_event_synchronize(ev);
+            dali_hip_event_destroy(ev);
+        }
+    if (host_) {
+        if (pinned_host_) dali_hip_host_free(host_);
+        else std::free(host_);
+    }
     // device blocks go back to the size-keyed bank, not to the driver
     // (dali/array/memory/synchronized_memory.cpp:76-82)
     if (device_) dali_hip_bank_deposit(device_, bytes_);
+}
+
+// Before a side is handed out: a transfer towards the device makes the compute stream wait for it (once); a
+// transfer towards the host, or away from a host block that is about to be written, makes the host wait.
+void SynchronizedMemory::settle(DeviceT device, bool host_will_write) {
+    auto retire = [](void*& ev) {
+        check_hip(dali_hip_event_destroy(ev), "event destroy");
+        ev = nullptr;
+    };
+    if (device == DEVICE_T_GPU) {
+        // a transfer that has not finished yet is put in front of whatever the compute stream does next with the
+        // device block (a copy to the host still reads it, a copy from the host still writes it)
+        for (void** ev : {&to_device_event_, &to_host_event_}) {
+            if (!*ev) continue;
+            int done = 0;
+            check_hip(dali_hip_event_query(*ev, &done), "event query");
+            if (done) {
+                if (ev == &to_device_event_) retire(*ev);  // the host block is free again as well
+                else continue;                             // the host side retires its own event when it reads
+            } else {
+                check_hip(dali_hip_stream_wait_event(*ev), "wait for migration");
+            }
+        }
+    } else {
+        if (to_host_event_) {
+            check_hip(dali_hip_event_synchronize(to_host_event_), "wait for migration");
+            retire(to_host_event_);
+        }
+        if (to_device_event_ && host_will_write) {
+            check_hip(dali_hip_event_synchronize(to_device_event_), "wait for migration");
+            retire(to_device_event_);
+        }
+    }
+}
+
+void SynchronizedMemory::prefetch(DeviceT device) {
+    bool& fresh = device == DEVICE_T_CPU ? host_fresh_ : device_fresh_;
+    if (fresh) return;
+    const bool other_fresh = device == DEVICE_T_CPU ? device_fresh_ : host_fresh_;
+    if (!pinned_host_ || !other_fresh) {
+        move_to(device);
+        return;
+    }
+    allocate(device);
+    void*& slot = device == DEVICE_T_CPU ? to_host_event_ : to_device_event_;
+    if (slot) {
+        check_hip(dali_hip_event_synchronize(slot), "wait for migration");
+        check_hip(dali_hip_event_destroy(slot), "event destroy");
+        slot = nullptr;
+    }
+    void* ev = nullptr;
+    check_hip(dali_hip_event_create(&ev), "event create");
+    if (device == DEVICE_T_GPU) check_hip(dali_hip_memcpy_h2d_async(device_, host_, bytes_, ev), "asynchronous copy to device");
+    else check_hip(dali_hip_memcpy_d2h_async(host_, device_, bytes_, ev), "asynchronous copy to host");
+    slot = ev;
+    fresh = true;
 }
 
 void SynchronizedMemory::lazy_clear() {
@@ -72,7 +137,8 @@ void SynchronizedMemory::allocate(DeviceT device) {
     if (device == DEVICE_T_CPU) {
         if (host_) return;
         size_t n = bytes_ ? bytes_ : 4;
-        if (posix_memalign(&host_, 64, n) != 0) throw std::runtime_error("host allocation failed");
+        if (pinned_host_) check_hip(dali_hip_host_alloc(&host_, n), "pinned host allocation");
+        else if (posix_memalign(&host_, 64, n) != 0) throw std::runtime_error("host allocation failed");
     } else {
         if (device_) return;
         check_hip(dali_hip_bank_allocate(&device_, bytes_), "device allocation");
@@ -100,11 +166,13 @@ void SynchronizedMemory::move_to(DeviceT device) {
 
 const void* SynchronizedMemory::readonly_data(DeviceT device) {
     move_to(device);
+    settle(device, false);
     return device == DEVICE_T_CPU ? host_ : device_;
 }
 
 void* SynchronizedMemory::mutable_data(DeviceT device) {
     move_to(device);
+    settle(device, true);
     host_fresh_ = device == DEVICE_T_CPU;
     device_fresh_ = device == DEVICE_T_GPU;
     return device == DEVICE_T_CPU ? host_ : device_;
@@ -112,6 +180,7 @@ void* SynchronizedMemory::mutable_data(DeviceT device) {
 
 void* SynchronizedMemory::overwrite_data(DeviceT device) {
     allocate(device);
+    settle(device, true);
     host_fresh_ = device == DEVICE_T_CPU;
     device_fresh_ = device == DEVICE_T_GPU;
     return device == DEVICE_T_CPU ? host_ : device_;
@@ -167,6 +236,14 @@ Array Array::from_host(const void* data, const std::vector<int>& shape, DType dt
     auto& mem = a.state_->expr->memory;
     void* dst = mem->overwrite_data(memory::DEVICE_T_CPU);
     std::memcpy(dst, data, mem->bytes());
+    return a;
+}
+
+Array Array::from_host_pinned(const void* data, const std::vector<int>& shape, DType dtype) {
+    Array a(shape, dtype);
+    auto& e = a.state_->expr;
+    e->memory = std::make_shared<memory::SynchronizedMemory>((size_t)e->numel() * size_of_dtype(dtype), true);
+    std::memcpy(e->memory->overwrite_data(memory::DEVICE_T_CPU), data, e->memory->bytes());
     return a;
 }
 
@@ -260,6 +337,9 @@ static const Array& as_buffer(const Array& a) {
     a.eval();
     return a;
 }
+
+void Array::prefetch_to_device() const { as_buffer(*this).expression()->memory->prefetch(memory::DEVICE_T_GPU); }
+void Array::prefetch_to_host() const { as_buffer(*this).expression()->memory->prefetch(memory::DEVICE_T_CPU); }
 
 Array Array::transpose() const {
     std::vector<int> axes(ndim());

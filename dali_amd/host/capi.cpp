@@ -40,6 +40,12 @@ const char* dali_fe_last_error(void) { return g_err.c_str(); }
 dali_array_t dali_fe_from_host(const void* data, const int* shape, int ndim, int dtype) {
     FE_TRY(return wrap(Array::from_host(data, vec(shape, ndim), (dali::DType)dtype));, nullptr)
 }
+dali_array_t dali_fe_from_host_pinned(const void* data, const int* shape, int ndim, int dtype) {
+    FE_TRY(return wrap(Array::from_host_pinned(data, vec(shape, ndim), (dali::DType)dtype));, nullptr)
+}
+int dali_fe_prefetch(dali_array_t a, int to_device) {
+    FE_TRY(if (to_device) A(a).prefetch_to_device(); else A(a).prefetch_to_host(); return 0;, 1)
+}
 dali_array_t dali_fe_empty(const int* shape, int ndim, int dtype) {
     FE_TRY(return wrap(Array(vec(shape, ndim), (dali::DType)dtype));, nullptr)
 }

@@ -38,7 +38,8 @@ enum DeviceT { DEVICE_T_CPU = 0, DEVICE_T_GPU = 1 };
 // migration on access (dali/array/memory/synchronized_memory.h:35-133).
 class SynchronizedMemory {
   public:
-    explicit SynchronizedMemory(size_t bytes);
+    // pinned_host: the host copy lives in page-locked memory, which lets prefetch() migrate without blocking
+    explicit SynchronizedMemory(size_t bytes, bool pinned_host = false);
     ~SynchronizedMemory();
     SynchronizedMemory(const SynchronizedMemory&) = delete;
     SynchronizedMemory& operator=(const SynchronizedMemory&) = delete;
@@ -51,11 +52,19 @@ class SynchronizedMemory {
     bool is_fresh(DeviceT device) const { return device == DEVICE_T_CPU ? host_fresh_ : device_fresh_; }
     bool is_allocated(DeviceT device) const { return device == DEVICE_T_CPU ? host_ != nullptr : device_ != nullptr; }
     void lazy_clear();  // zero on first allocation (dali/array/memory/synchronized_memory.cpp:237-266)
+    // Start bringing the other side's fresh copy to `device` without waiting for it. With a pinned host copy the
+    // transfer runs beside the compute stream and the next access waits only for this block; otherwise it is the
+    // blocking migration of data().
+    void prefetch(DeviceT device);
 
   private:
     void allocate(DeviceT device);
     void move_to(DeviceT device);
+    void settle(DeviceT device, bool host_will_write);
     size_t bytes_;
+    bool pinned_host_ = false;
+    void* to_device_event_ = nullptr;  // an h2d transfer in flight: the compute stream has not been told to wait yet
+    void* to_host_event_ = nullptr;    // a d2h transfer in flight
     void* host_ = nullptr;
     void* device_ = nullptr;
     bool host_fresh_ = false, device_fresh_ = false;
@@ -84,6 +93,10 @@ class Array {
     static Array arange(int n, DType dtype = DTYPE_FLOAT);
     // copies `data` (contiguous, row-major) into a new buffer
     static Array from_host(const void* data, const std::vector<int>& shape, DType dtype);
+    // the same with the host copy in pinned memory (needs an initialised device): prefetch_to_device() then returns at once
+    static Array from_host_pinned(const void* data, const std::vector<int>& shape, DType dtype);
+    void prefetch_to_device() const;
+    void prefetch_to_host() const;
 
     bool is_stateless() const;
     bool is_buffer() const;

@@ -22,6 +22,11 @@ const char* dali_fe_last_error(void);
 
 /* construction (dali/array/array.h:31-62) */
 dali_array_t dali_fe_from_host(const void* data, const int* shape, int ndim, int dtype);
+/* the same with the host copy in pinned memory, and the non-blocking migration it allows (to_device != 0: host to
+ * device, else device to host); replaces the blocking copy of SynchronizedMemory::move_to
+ * (dali/array/memory/synchronized_memory.cpp:268-314) where the caller asks for it */
+dali_array_t dali_fe_from_host_pinned(const void* data, const int* shape, int ndim, int dtype);
+int dali_fe_prefetch(dali_array_t a, int to_device);
 dali_array_t dali_fe_empty(const int* shape, int ndim, int dtype);
 dali_array_t dali_fe_zeros(const int* shape, int ndim, int dtype);
 dali_array_t dali_fe_scalar_double(double v);

@@ -93,6 +93,19 @@ int dali_hip_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
 int dali_hip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);
 int dali_hip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes);
 
+/* Pinned host memory and migrations that do not block the caller: the alternative to the blocking cudaMemcpy of
+ * memory::copy (dali/array/memory/memory_ops.cu.cpp:109-126) for a caller whose host side lives in memory from
+ * dali_hip_host_alloc. The copy runs on a second stream of the library. It starts after everything already issued
+ * on the compute stream (so kernels that still use the device block are not overtaken) and records `done_event`
+ * (from dali_hip_event_create, may be NULL) when the bytes have arrived. Work issued afterwards on the compute
+ * stream does not wait for the copy unless dali_hip_stream_wait_event(done_event) is called; the host waits with
+ * dali_hip_event_synchronize or polls with dali_hip_event_query. The host block must stay untouched (h2d) or
+ * unread (d2h) until the event has fired. Not allowed during a capture. */
+int dali_hip_host_alloc(void** ptr, size_t bytes);
+int dali_hip_host_free(void* ptr);
+int dali_hip_memcpy_h2d_async(void* dst_device, const void* src_pinned, size_t bytes, void* done_event);
+int dali_hip_memcpy_d2h_async(void* dst_pinned, const void* src_device, size_t bytes, void* done_event);
+
 /* ------------------------------------------- runtime-compiled kernels */
 
 /* How the launcher turns the six argument arrays into a grid. */
@@ -246,6 +259,11 @@ int dali_hip_event_create(void** event);
 int dali_hip_event_record(void* event);
 int dali_hip_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
 int dali_hip_event_destroy(void* event);
+/* the compute stream waits (on the device) for an event recorded by an asynchronous copy or by dali_hip_event_record */
+int dali_hip_stream_wait_event(void* event);
+/* the host waits for / polls an event */
+int dali_hip_event_synchronize(void* event);
+int dali_hip_event_query(void* event, int* done);
 
 #ifdef __cplusplus
 }

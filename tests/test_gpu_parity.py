@@ -143,6 +143,62 @@ def _dev(hip, a):
     return p
 
 
+def test_pinned_memory_and_asynchronous_copies_abi(gpu, rng):
+    """dali_hip_host_alloc + dali_hip_memcpy_{h2d,d2h}_async: the copy runs beside the compute stream, the event says
+    when the bytes have arrived, dali_hip_stream_wait_event puts it in front of later compute work."""
+    hip = gpu
+    n = 1 << 22
+    src, back = C.c_void_p(), C.c_void_p()
+    assert hip.dali_hip_host_alloc(C.byref(src), n * 4) == 0 and hip.dali_hip_host_alloc(C.byref(back), n * 4) == 0
+    host = np.ctypeslib.as_array(C.cast(src, C.POINTER(C.c_float)), (n,))
+    out = np.ctypeslib.as_array(C.cast(back, C.POINTER(C.c_float)), (n,))
+    host[:] = rng.randn(n).astype(np.float32)
+    out[:] = 0
+    dev, dev2 = C.c_void_p(), C.c_void_p()
+    assert hip.dali_hip_malloc(C.byref(dev), n * 4) == 0 and hip.dali_hip_malloc(C.byref(dev2), n * 4) == 0
+    up, down = C.c_void_p(), C.c_void_p()
+    assert hip.dali_hip_event_create(C.byref(up)) == 0 and hip.dali_hip_event_create(C.byref(down)) == 0
+    assert hip.dali_hip_memcpy_h2d_async(dev, src, n * 4, up) == 0, hip.dali_hip_last_error()
+    assert hip.dali_hip_stream_wait_event(up) == 0          # the compute stream's d2d copy reads what the upload wrote
+    assert hip.dali_hip_memcpy_d2d(dev2, dev, n * 4) == 0
+    assert hip.dali_hip_memcpy_d2h_async(back, dev2, n * 4, down) == 0  # starts after the d2d already issued
+    assert hip.dali_hip_event_synchronize(down) == 0
+    done = C.c_int(0)
+    assert hip.dali_hip_event_query(up, C.byref(done)) == 0 and done.value == 1
+    assert np.array_equal(out, host)
+    for ev in (up, down):
+        assert hip.dali_hip_event_destroy(ev) == 0
+    assert hip.dali_hip_free(dev) == 0 and hip.dali_hip_free(dev2) == 0
+    assert hip.dali_hip_host_free(src) == 0 and hip.dali_hip_host_free(back) == 0
+
+
+def test_prefetch_of_pinned_arrays(gpu, D, rng):
+    xs = [rng.randn(1 << 20).astype(np.float32) for _ in range(6)]
+    arrays = [D.Array.from_numpy(x, pinned=True) for x in xs]
+    for a in arrays:
+        a.prefetch("gpu")                      # six uploads in flight
+    sums = [D.op.sum(D.op.abs(a)) for a in arrays]
+    for s, x in zip(sums, xs):
+        np.testing.assert_allclose(float(s.numpy()), np.abs(x.astype(np.float64)).sum(), rtol=1e-5)
+    # results come back the same way: the download starts behind the kernel that produces the values
+    ys = [D.op.tanh(a) for a in arrays]
+    for y in ys:
+        y.eval()
+    outs = [D.Array.from_numpy(np.zeros(1 << 20, np.float32), pinned=True) for _ in ys]
+    for o, y in zip(outs, ys):
+        o.assign(y)
+        o.prefetch("cpu")
+    for o, x in zip(outs, xs):
+        np.testing.assert_allclose(o.numpy(), np.tanh(x.astype(np.float64)), rtol=1e-5, atol=1e-6)
+    # writing the host side of an array whose upload is in flight waits for the upload first
+    a = D.Array.from_numpy(xs[0], pinned=True)
+    a.prefetch("gpu")
+    b = D.Array.from_numpy(xs[1])              # pageable memory: prefetch is the ordinary blocking migration
+    b.prefetch("gpu")
+    np.testing.assert_allclose(float(D.op.sum(a - a).numpy()), 0.0)
+    np.testing.assert_allclose(float(D.op.max(b).numpy()), xs[1].max())
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (5, 11, 7), (64, 64, 64), (65, 130, 33), (256, 4096, 128), (300, 200, 100),
                                    (132, 72, 640), (252, 1000, 1000), (1100, 2300, 260), (2052, 2052, 132),
                                    # few tiles over a long inner extent: shares of K folded across workgroups
