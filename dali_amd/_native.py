@@ -84,6 +84,7 @@ HIP_SYMBOLS = {
     "dali_hip_compile_only": (_i, [C.c_char_p, C.POINTER(_sz)]),
     "dali_hip_jit_stats": (_i, [C.POINTER(_u64), C.POINTER(_u64), C.POINTER(_u64)]),
     "dali_hip_set_cache_dir": (_i, [C.c_char_p]),
+    "dali_hip_cache_warm": (_i, [C.POINTER(_i)]),
     "dali_hip_sgemm": (_i, [_i, _i, _i, _i, _i, C.c_float, H, _i, H, _i, C.c_float, H, _i]),
     "dali_hip_sgemm_pair": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, C.c_float, H, _i, H, _i, H, _i, H, _i, C.c_float, H, _i]),
     "dali_hip_lstm_step": (_i, [_i, _i, _i, H, _i, H, _i, H, H, _i, H, _i, H, H, H]),

@@ -8,6 +8,7 @@
 #include "runtime.h"
 
 #include <hip/hiprtc.h>
+#include <dirent.h>
 #include <sys/stat.h>
 #include <sys/types.h>
 #include <unistd.h>
@@ -71,6 +72,8 @@ struct Runtime {
     };
     std::unordered_map<uint64_t, Module> modules;
     std::unordered_map<uint64_t, bool> recompiled_once;
+    // code objects loaded ahead of their first use by dali_hip_cache_warm (no launch plan yet)
+    std::unordered_map<uint64_t, hipModule_t> preloaded;
     std::string cache_dir;
     uint64_t n_compiled = 0, n_disk = 0, n_launch = 0;
 };
@@ -461,6 +464,37 @@ int dali_hip_jit_stats(uint64_t* compiled, uint64_t* disk_hits, uint64_t* launch
     return DALI_HIP_OK;
 }
 
+int dali_hip_cache_warm(int* loaded) {
+    if (ensure_init()) return DALI_HIP_ERROR;
+    Runtime& r = rt();
+    std::lock_guard<std::mutex> lock(r.mu);
+    if (r.cache_dir.empty()) r.cache_dir = default_cache_dir();
+    const std::string suffix = "-" + r.arch + ".hsaco";
+    int n = 0;
+    DIR* d = opendir(r.cache_dir.c_str());
+    if (d) {
+        while (struct dirent* ent = readdir(d)) {
+            const std::string name = ent->d_name;
+            if (name.size() != 16 + suffix.size() || name.compare(16, suffix.size(), suffix) != 0) continue;
+            char* end = nullptr;
+            const uint64_t hash = strtoull(name.substr(0, 16).c_str(), &end, 16);
+            if (!end || *end != 0 || r.modules.count(hash) || r.preloaded.count(hash)) continue;
+            std::ifstream in(r.cache_dir + "/" + name, std::ios::binary);
+            std::vector<char> code((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
+            hipModule_t mod = nullptr;
+            if (code.empty() || hipModuleLoadData(&mod, code.data()) != hipSuccess) {
+                (void)hipGetLastError();  // a stale or foreign file is rebuilt from source at its first use
+                continue;
+            }
+            r.preloaded[hash] = mod;
+            ++n;
+        }
+        closedir(d);
+    }
+    if (loaded) *loaded = n;
+    return DALI_HIP_OK;
+}
+
 int dali_hip_module_is_loaded(uint64_t hash) {
     Runtime& r = rt();
     std::lock_guard<std::mutex> lock(r.mu);
@@ -490,7 +524,9 @@ int dali_hip_module_load(uint64_t hash, const char* hip_source, const char* kern
     std::string path = r.cache_dir + "/" + hash_hex(hash) + "-" + r.arch + ".hsaco";
     std::vector<char> code;
     int cached = 0;
-    if (!force) {
+    if (!force && r.preloaded.count(hash)) {
+        cached = 1;
+    } else if (!force) {
         std::ifstream in(path, std::ios::binary);
         if (in) {
             code.assign(std::istreambuf_iterator<char>(in), std::istreambuf_iterator<char>());
@@ -520,7 +556,14 @@ int dali_hip_module_load(uint64_t hash, const char* hip_source, const char* kern
     }
 
     Runtime::Module m;
-    hipError_t e = hipModuleLoadData(&m.module, code.data());
+    hipError_t e = hipSuccess;
+    auto pre = r.preloaded.find(hash);
+    if (cached && pre != r.preloaded.end()) {
+        m.module = pre->second;
+        r.preloaded.erase(pre);
+    } else {
+        e = hipModuleLoadData(&m.module, code.data());
+    }
     if (e != hipSuccess && cached && hip_source) {
         // stale or foreign file: rebuild from source
         (void)hipGetLastError();

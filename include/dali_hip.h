@@ -184,6 +184,12 @@ int dali_hip_jit_stats(uint64_t* compiled, uint64_t* disk_hits, uint64_t* launch
 /* Set the code-object cache directory (overrides the environment). Replaces
  * Compiler::set_output_path, dali/utils/compiler.cpp:115-117. */
 int dali_hip_set_cache_dir(const char* path);
+/* Load every code object of the cache directory into the device ahead of its first use (the counterpart of
+ * shipping ~/.dali/cache/<hash>.so files and having dlopen done before the first request,
+ * dali/utils/compiler.cpp:86-103): dali_hip_module_load then only attaches the launch plan. Files that do not
+ * load are skipped and rebuilt from source when their expression is first evaluated. `loaded` (may be NULL)
+ * receives the number of code objects taken in by this call. */
+int dali_hip_cache_warm(int* loaded);
 
 /* ---------------------------------------------------------------- GEMM */
 

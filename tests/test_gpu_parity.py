@@ -143,6 +143,47 @@ def _dev(hip, a):
     return p
 
 
+_WARM_SCRIPT = """
+import ctypes as C, sys, time
+import numpy as np
+import dali_amd as D
+from dali_amd._native import hip, hip_check
+hip_check(hip.dali_hip_init(0), "init")
+assert hip.dali_hip_set_cache_dir(sys.argv[1].encode()) == 0
+n = C.c_int(-1)
+if sys.argv[2] == "warm":
+    assert hip.dali_hip_cache_warm(C.byref(n)) == 0
+x = D.Array.from_numpy(np.linspace(-1, 1, 3 * 700, dtype=np.float32).reshape(3, 700))
+t0 = time.perf_counter()
+y = D.op.softmax(D.op.tanh(x) * 3.0 + 0.125)
+y.eval()
+hip.dali_hip_sync()
+ms = (time.perf_counter() - t0) * 1e3
+c, d, l = (C.c_uint64() for _ in range(3))
+hip.dali_hip_jit_stats(C.byref(c), C.byref(d), C.byref(l))
+print("RESULT", n.value, c.value, d.value, "%.3f" % ms, "%.6f" % float(y.numpy().sum()))
+"""
+
+
+def test_cache_warm_loads_code_objects_ahead_of_first_use(gpu, tmp_path):
+    """Two fresh processes share a cache directory: the first compiles, the second takes the code objects in with
+    dali_hip_cache_warm and neither compiles nor reads the directory again for that expression."""
+    import os, subprocess, sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, PYTHONPATH=root)
+    runs = []
+    for mode in ("cold", "warm"):
+        out = subprocess.run([sys.executable, "-c", _WARM_SCRIPT, str(tmp_path), mode], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                             text=True, timeout=100)
+        assert out.returncode == 0, out.stdout
+        line = [l for l in out.stdout.splitlines() if l.startswith("RESULT")][-1].split()
+        runs.append((int(line[1]), int(line[2]), int(line[3]), float(line[4]), float(line[5])))
+    (_, compiled0, _, ms0, sum0), (loaded, compiled1, disk1, ms1, sum1) = runs
+    assert compiled0 >= 1 and loaded >= compiled0 and compiled1 == 0 and disk1 >= 1
+    assert abs(sum0 - 3.0) < 1e-4 and sum0 == sum1
+    print("first evaluation: %.1f ms cold, %.1f ms after dali_hip_cache_warm" % (ms0, ms1))
+
+
 def test_pinned_memory_and_asynchronous_copies_abi(gpu, rng):
     """dali_hip_host_alloc + dali_hip_memcpy_{h2d,d2h}_async: the copy runs beside the compute stream, the event says
     when the bytes have arrived, dali_hip_stream_wait_event puts it in front of later compute work."""
