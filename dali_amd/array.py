@@ -288,7 +288,10 @@ def eval_together(arrays):
 def jit_stats():
     vals = [C.c_uint64() for _ in range(4)]
     front.dali_fe_stats(*[C.byref(v) for v in vals])
-    return {"kernels": vals[0].value, "gemms": vals[1].value, "evals": vals[2].value, "plans": vals[3].value}
+    pc = [C.c_uint64() for _ in range(2)]
+    front.dali_fe_plan_cache_stats(*[C.byref(v) for v in pc])
+    return {"kernels": vals[0].value, "gemms": vals[1].value, "evals": vals[2].value, "plans": vals[3].value,
+            "plan_cache_hits": pc[0].value, "plan_cache_stored": pc[1].value}
 
 
 def last_kernel_kinds():

@@ -208,6 +208,12 @@ int dali_fe_stats(uint64_t* kernels, uint64_t* gemms, uint64_t* evals, uint64_t*
     if (plans) *plans = s.plans_built;
     return 0;
 }
+int dali_fe_plan_cache_stats(uint64_t* hits, uint64_t* stored) {
+    auto& s = dali::jit_stats();
+    if (hits) *hits = s.plan_cache_hits;
+    if (stored) *stored = s.plan_cache_stored;
+    return 0;
+}
 const char* dali_fe_last_kernel_kinds(void) {
     g_kinds = dali::jit_stats().last_kernel_kinds;
     return g_kinds.c_str();

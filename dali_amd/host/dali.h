@@ -357,6 +357,8 @@ struct JitStats {
     uint64_t gemms_launched = 0;
     uint64_t evals = 0;
     uint64_t plans_built = 0;       // planner invocations that had to generate source
+    uint64_t plan_cache_hits = 0;   // evaluations that reused a stored plan instead of planning
+    uint64_t plan_cache_stored = 0; // plans stored so far
     std::string last_kernel_kinds;  // e.g. "row" or "row,all" for the last eval
     std::string last_kernel_names;  // entry-point names of the generated kernels of the last eval
 };

@@ -123,6 +123,10 @@ void* dali_fe_device_ptr(dali_array_t a);
 
 /* observation (dali/utils/scope.h, dali/array/tests/dot_tests.cpp:17-36) */
 int dali_fe_stats(uint64_t* kernels, uint64_t* gemms, uint64_t* evals, uint64_t* plans);
+/* evaluations that reused a stored plan (same structure: kinds, functors, dtypes, shapes, buffer layouts and sharing)
+ * instead of running the planner, and plans stored so far; DALI_HIP_PLAN_CACHE=0 turns the cache off,
+ * DALI_HIP_PLAN_CACHE_CHECK=1 runs the planner beside every reuse and raises if the two disagree */
+int dali_fe_plan_cache_stats(uint64_t* hits, uint64_t* stored);
 const char* dali_fe_last_kernel_kinds(void);
 const char* dali_fe_last_kernel_names(void);
 const char* dali_fe_last_source(void);

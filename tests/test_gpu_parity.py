@@ -602,6 +602,45 @@ def test_lstm_step_matches_oracle(gpu, D, O, rng, B, I, H):
     close(hn.numpy(), ohn, rtol=1e-4, atol=1e-5)
 
 
+def test_plan_cache_reuses_structure_not_values(gpu, D, rng):
+    """A repeated request skips the planner; buffers, literal values and results are this request's own."""
+    op = D.op
+    before = D.jit_stats()
+    for k in range(6):
+        x = rng.randn(37, 129).astype(np.float32)
+        s = float(rng.uniform(0.5, 2.0))
+        got = (op.softmax(arr(D, x) * s) + (0.25 * k)).numpy()
+        z = x.astype(np.float64) * np.float64(np.float32(s))
+        e = np.exp(z - z.max(axis=1, keepdims=True))
+        close(got, e / e.sum(axis=1, keepdims=True) + 0.25 * k, rtol=1e-5 + 128 * 2.0 ** -24)
+    after = D.jit_stats()
+    assert after["plan_cache_hits"] - before["plan_cache_hits"] >= 5
+    assert after["plans"] - before["plans"] <= 1                 # source was generated once at most
+    # sharing is part of the structure: x + x (one allocation) and x + y (two) are different requests, both right
+    x, y = rng.randn(64, 64).astype(np.float32), rng.randn(64, 64).astype(np.float32)
+    for _ in range(3):
+        ax, ay = arr(D, x), arr(D, y)
+        assert np.array_equal((ax + ax).numpy(), x + x)
+        assert np.array_equal((ax + ay).numpy(), x + y)
+        assert np.array_equal((ax + ax.T).numpy(), x + x.T)
+    # so are in-place updates, and views of one buffer at different distances
+    for _ in range(3):
+        a = arr(D, x)
+        a += a * 2.0
+        assert np.array_equal(a.numpy(), x + x * np.float32(2.0))
+        wide = arr(D, np.concatenate([x, y], axis=1))
+        assert np.array_equal((wide[:, 0:32] - wide[:, 32:64]).numpy(), x[:, 0:32] - x[:, 32:64])
+        assert np.array_equal((wide[:, 0:32] - wide[:, 64:96]).numpy(), x[:, 0:32] - y[:, 0:32])
+        assert np.array_equal((wide[:, 0:32] - wide[:, 0:32]).numpy(), np.zeros((64, 32), np.float32))
+    # reductions, several shapes of the same expression, dtype changes
+    for shape in ((5, 7), (5, 8), (5, 7), (64, 1000), (5, 7)):
+        v = rng.uniform(0.5, 1.5, shape).astype(np.float32)
+        np.testing.assert_allclose(op.sum(arr(D, v), [0]).numpy(), v.astype(np.float64).sum(axis=0), rtol=1e-5)
+        np.testing.assert_allclose(float(op.mean(arr(D, v)).numpy()), v.astype(np.float64).mean(), rtol=1e-5)
+        vi = (v * 10).astype(np.int32)
+        assert np.array_equal(op.max(arr(D, vi), [1]).numpy(), vi.max(axis=1))
+
+
 def test_recording_replays_the_same_device_work(gpu, D, rng):
     x = arr(D, rng.randn(50, 300).astype(np.float32))
     with D.Recording() as rec:
