@@ -149,6 +149,7 @@ FRONT_SYMBOLS = {
     "dali_fe_diag": (H, [H, _i, _i]),
     "dali_fe_outer": (H, [H, H]),
     "dali_fe_circular_convolution": (H, [H, H]),
+    "dali_fe_concatenate": (H, [_HP, _i, _i]),
     "dali_fe_im2col": (H, [H] + [_i] * 8 + [C.c_char_p]),
     "dali_fe_col2im": (H, [H, _ip, _i, _i, _i, _i, _i, C.c_char_p]),
     "dali_fe_conv2d": (H, [H, H, _i, _i, _i, C.c_char_p]),

@@ -950,6 +950,46 @@ Array circular_convolution(Array x, Array weights) {
     return make_node(Kind::CIRCULAR_CONV, "", {xb, wb}, shape, x.dtype());
 }
 
+// dali/array/op/concatenate.cpp:9-73: the arrays written one after the other along `axis` into one new buffer
+// (dimensions of extent 1 on the other axes are broadcast; the result takes the first array's dtype)
+Array concatenate(const std::vector<Array>& arrays, int axis) {
+    DALI_ASSERT(!arrays.empty(), "concatenate must receive at least one array.");
+    if (arrays.size() == 1) return arrays[0];
+    const int nd = arrays[0].ndim();
+    DALI_ASSERT(nd > 0, make_message("cannot concatenate scalar arrays (got ndim = ", nd, ")."));
+    if (axis < 0) axis += nd;
+    DALI_ASSERT(axis >= 0 && axis < nd, make_message("concatenation axis must be >= 0 and < arrays[0].ndim = ", nd, ", but got axis = ", axis, "."));
+    std::vector<int> common = arrays[0].shape();
+    int total = 0;
+    for (const Array& a : arrays) {
+        DALI_ASSERT(a.ndim() == nd, make_message("All arrays in concatenate must have the same dimensionality, but got ndim = ", a.ndim(), " != ", nd, "."));
+        for (int i = 0; i < nd; ++i) {
+            if (i == axis) continue;
+            if (common[i] != a.shape()[i] && common[i] == 1) common[i] = a.shape()[i];
+            DALI_ASSERT(common[i] == a.shape()[i] || a.shape()[i] == 1,
+                        make_message("All shapes must have length-1 or equal dimensions on all axes except the concatenation axis, but got shape ",
+                                     shape_str(a.shape()), " which differs on axis ", i, " from expected = ", common[i], "."));
+        }
+        total += a.shape()[axis];
+    }
+    std::vector<int> shape = common;
+    shape[axis] = total;
+    Array result(shape, arrays[0].dtype());
+    int so_far = 0;
+    for (Array a : arrays) {
+        const int n = a.shape()[axis];
+        if (n == 0) continue;
+        common[axis] = n;
+        if (a.dtype() != result.dtype()) a = astype(a, result.dtype());
+        if (a.shape() != common) a = broadcasted_reshape(a, common);
+        result.slice(axis, so_far, so_far + n).assign(a);
+        so_far += n;
+    }
+    return result;
+}
+Array hstack(const std::vector<Array>& arrays) { return concatenate(arrays, -1); }
+Array vstack(const std::vector<Array>& arrays) { return concatenate(arrays, 0); }
+
 // ---------------------------------------------------------------- sliding windows
 // dali/array/op/spatial_utils.cpp:33-50
 void check_data_format(const std::string& data_format, int* n_dim, int* c_dim, int* h_dim, int* w_dim) {

@@ -122,6 +122,9 @@ dali_array_t dali_fe_arange(dali_array_t start, dali_array_t stop, dali_array_t 
 }
 dali_array_t dali_fe_diag(dali_array_t diagonal, int rows, int cols) { FE_TRY(return wrap(dali::op::diag(A(diagonal), rows, cols));, nullptr) }
 dali_array_t dali_fe_circular_convolution(dali_array_t x, dali_array_t w) { FE_TRY(return wrap(dali::op::circular_convolution(A(x), A(w)));, nullptr) }
+dali_array_t dali_fe_concatenate(dali_array_t* arrays, int n, int axis) {
+    FE_TRY(std::vector<Array> v; for (int i = 0; i < n; ++i) v.push_back(A(arrays[i])); return wrap(dali::op::concatenate(v, axis));, nullptr)
+}
 dali_array_t dali_fe_im2col(dali_array_t image, int filter_h, int filter_w, int stride_h, int stride_w, int padding_h, int padding_w,
                             int postpad_h, int postpad_w, const char* data_format) {
     FE_TRY(return wrap(dali::op::im2col(A(image), filter_h, filter_w, stride_h, stride_w, padding_h, padding_w, postpad_h, postpad_w, data_format));

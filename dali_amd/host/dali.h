@@ -281,6 +281,11 @@ Array outer(const Array& a, const Array& b);
 // dali/array/op/circular_convolution.h
 Array circular_convolution(Array x, Array weights);
 
+// dali/array/op/concatenate.h
+Array concatenate(const std::vector<Array>& arrays, int axis);
+Array hstack(const std::vector<Array>& arrays);
+Array vstack(const std::vector<Array>& arrays);
+
 // dali/array/op/spatial_utils.h: geometry of sliding-window operators
 void check_data_format(const std::string& data_format, int* n_dim, int* c_dim, int* h_dim, int* w_dim);
 struct SlidingWindowFunctionInfo {

@@ -262,6 +262,21 @@ def circular_convolution(x, weights):
     return _wrap(front.dali_fe_circular_convolution(x._h, weights._h), "circular_convolution")
 
 
+def concatenate(arrays, axis):
+    """The arrays one after the other along ``axis`` (dali/array/op/concatenate.cpp:9-73)."""
+    keep = [as_array(a) for a in arrays]
+    hs = (C.c_void_p * len(keep))(*[k._h for k in keep])
+    return _wrap(front.dali_fe_concatenate(hs, len(keep), axis), "concatenate")
+
+
+def hstack(arrays):
+    return concatenate(arrays, -1)
+
+
+def vstack(arrays):
+    return concatenate(arrays, 0)
+
+
 # dali/array/op/spatial_enums.h
 PADDING_T_SAME, PADDING_T_VALID = 0, 1
 POOLING_T_MAX, POOLING_T_AVG = 0, 1

@@ -75,6 +75,8 @@ dali_array_t dali_fe_arange(dali_array_t start, dali_array_t stop, dali_array_t 
 dali_array_t dali_fe_diag(dali_array_t diagonal, int rows, int cols);
 /* op::circular_convolution (dali/array/op/circular_convolution.cpp:82-86) */
 dali_array_t dali_fe_circular_convolution(dali_array_t x, dali_array_t weights);
+/* op::concatenate (dali/array/op/concatenate.cpp:9-73); hstack = axis -1, vstack = axis 0 */
+dali_array_t dali_fe_concatenate(dali_array_t* arrays, int n, int axis);
 /* Sliding-window operators. data_format is a permutation of "NCHW" naming the order of the image's dimensions
  * (conv2d and the pooling pair accept "NCHW" and "NHWC"); padding: 0 = SAME, 1 = VALID and pooling: 0 = max, 1 = average,
  * the values of dali/array/op/spatial_enums.h.

@@ -641,6 +641,34 @@ def test_plan_cache_reuses_structure_not_values(gpu, D, rng):
         assert np.array_equal(op.max(arr(D, vi), [1]).numpy(), vi.max(axis=1))
 
 
+def test_concatenate_reference_cases(gpu, D, rng):
+    # ArrayConcatenateTests (concatenate_tests.cpp:10-92)
+    op = D.op
+    ab = np.arange(14, dtype=np.float32).reshape(2, 7)
+    dab = arr(D, ab)
+    assert np.array_equal(op.hstack([dab[:, 0:3], dab[:, 3:7]]).numpy(), ab)
+    ab3 = np.arange(14, dtype=np.float32).reshape(7, 2, 1)
+    d3 = arr(D, ab3)
+    assert np.array_equal(op.vstack([d3[0:3], d3[3:7]]).numpy(), ab3)
+    m = np.arange(18, dtype=np.float32).reshape(3, 2, 3)
+    dm = arr(D, m)
+    mid = op.concatenate([dm[:, 0:1, :], dm[:, 1:2, :]], 1)
+    assert np.array_equal(mid.numpy(), m)
+    row = np.arange(5, dtype=np.float32)[None, :]
+    other = np.arange(21, dtype=np.float32).reshape(3, 7)
+    res = op.hstack([arr(D, row), arr(D, other)])          # a dimension of extent 1 is broadcast
+    assert res.shape == (3, 12) and np.array_equal(res.numpy(), np.hstack([np.repeat(row, 3, 0), other]))
+    assert np.array_equal(op.concatenate([dab], 0).numpy(), ab)
+    with pytest.raises(Exception):
+        op.concatenate([], 0)
+    with pytest.raises(Exception):
+        op.concatenate([dab, d3], 0)
+    # lazy operands and mixed dtypes: the first array's dtype wins
+    x, y = rng.randn(33, 50).astype(np.float32), rng.randint(-5, 5, (33, 7)).astype(np.int32)
+    got = op.concatenate([op.tanh(arr(D, x)), arr(D, y)], -1).numpy()
+    close(got, np.concatenate([np.tanh(x.astype(np.float64)), y.astype(np.float64)], axis=1))
+
+
 def test_recording_replays_the_same_device_work(gpu, D, rng):
     x = arr(D, rng.randn(50, 300).astype(np.float32))
     with D.Recording() as rec:
