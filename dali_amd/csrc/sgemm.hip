@@ -52,8 +52,10 @@ struct GemmSeg {
     int lda, ldb, K;
 };
 
+constexpr int kMaxSeg = 8;
+
 struct GemmArgs {
-    GemmSeg seg[2];
+    GemmSeg seg[kMaxSeg];
     int nseg;
     int M, N;
     float* C;
@@ -70,12 +72,23 @@ struct GemmArgs {
     float* c_out;
     float* h_out;
     int H;
+    // Output row map (convolution over a padded image computed at every padded position): row m stands for position
+    // (n, i, j) of an [., map_h, map_w] grid; only i < map_oh, j < map_ow are stored, at row (n * map_oh + i) * map_ow + j.
+    // hw = map_h * map_w and map_w come with the multiplier / shift of an exact division (see row_map_div).
+    int map_on;
+    unsigned map_hw, map_hw_m, map_w, map_w_m;
+    int map_hw_s, map_w_s, map_oh, map_ow;
 };
+
+// n / d for n < 2^31: m = ceil(2^(31+s) / d) with 2^(s-1) < d <= 2^s, computed by the launcher
+__device__ __forceinline__ unsigned row_map_div(unsigned n, unsigned m, int s) { return (unsigned)(((unsigned long long)n * m) >> (31 + s)); }
 
 __device__ __forceinline__ void publish(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float observe(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int DEPTH, bool EDGE, int KW, bool MIDB, bool GATES = false>
+// MAXSEG: how many terms the instantiation can walk. Two (the LSTM pair) keeps the segment switch of the main loop a
+// pair of scalar selects; the eight-term form (convolution by filter rows) carries a short select chain instead.
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int DEPTH, bool EDGE, int KW, bool MIDB, bool GATES = false, int MAXSEG = 2>
 __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     // KW wave sets share the tile: set kw takes every KW-th k-group of a slab, so each SIMD holds
     // KW waves that cover each other's LDS and barrier waits; the sets are summed through LDS at the end
@@ -132,9 +145,8 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     float4 ra[DEPTH][A_F4], rb[DEPTH][B_F4];
 
     // flat list of slabs over the segments
-    const int slabs0 = (g.seg[0].K + BK - 1) / BK;
-    const int slabs1 = g.nseg > 1 ? (g.seg[1].K + BK - 1) / BK : 0;
-    const int nslab_all = slabs0 + slabs1;
+    int nslab_all = 0;
+    for (int sg = 0; sg < g.nseg; ++sg) nslab_all += (g.seg[sg].K + BK - 1) / BK;
     // this workgroup's share of the slabs (all of them without split-K)
     const int s_begin = (int)((long)blockIdx.z * nslab_all / gridDim.z);
     const int nslab = (int)((long)(blockIdx.z + 1) * nslab_all / gridDim.z) - s_begin;
@@ -214,13 +226,22 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
     // fetch slab `i` (index into the flat slab list) into register stage S
     auto fetch = [&](auto S, int i) __attribute__((always_inline)) {
         constexpr int st = decltype(S)::value;
-        const bool first = i < slabs0;
-        const float* sa = first ? g.seg[0].A : g.seg[1].A;
-        const float* sb = first ? g.seg[0].B : g.seg[1].B;
-        const int lda = first ? g.seg[0].lda : g.seg[1].lda;
-        const int ldb = first ? g.seg[0].ldb : g.seg[1].ldb;
-        const int K = first ? g.seg[0].K : g.seg[1].K;
-        const int k0 = (first ? i : i - slabs0) * BK;
+        // the segment that holds flat slab i (a uniform walk over at most MAXSEG entries)
+        int sg = 0, first_slab = 0;
+#pragma unroll
+        for (int q = 0; q + 1 < MAXSEG; ++q) {
+            const int here = (g.seg[q].K + BK - 1) / BK;
+            if (sg == q && q + 1 < g.nseg && i >= first_slab + here) {
+                first_slab += here;
+                sg = q + 1;
+            }
+        }
+        const float* sa = g.seg[sg].A;
+        const float* sb = g.seg[sg].B;
+        const int lda = g.seg[sg].lda;
+        const int ldb = g.seg[sg].ldb;
+        const int K = g.seg[sg].K;
+        const int k0 = (i - first_slab) * BK;
 #pragma unroll
         for (int t = 0; t < A_F4; ++t) {
             if (!TA)
@@ -359,11 +380,37 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
         for (int t = 0; t < B_F4; ++t) b_off[t] = (unsigned)(((size_t)b_r[t] * ldb + b_c[t]) * sizeof(float));
         a_step = (TA ? (long)BK * lda : (long)BK) * (long)sizeof(float);
         b_step = (TB ? (long)BK : (long)BK * ldb) * (long)sizeof(float);
+        // Segment bases and slab counts are read into (scalar) registers here, once: a kernel-argument load inside the
+        // main loop would share its wait counter with the LDS operand reads and stall the pipeline at every switch.
+        const char* seg_a[MAXSEG];
+        const char* seg_b[MAXSEG];
+        int seg_slabs[MAXSEG];
+#pragma unroll
+        for (int q = 0; q < MAXSEG; ++q) {
+            const bool used = q < g.nseg;
+            seg_a[q] = used ? (const char*)g.seg[q].A : nullptr;
+            seg_b[q] = used ? (const char*)g.seg[q].B : nullptr;
+            seg_slabs[q] = used ? (g.seg[q].K + BK - 1) / BK : 0;
+        }
+        const int nseg = g.nseg;
+        int seg_i = 0, seg_end = seg_slabs[0];  // current segment and the flat slab index behind its last slab
+        ap = seg_a[0];
+        bp = seg_b[0];
+#pragma unroll
+        for (int q = 1; q < MAXSEG; ++q)
+            if (q < nseg && s_begin >= seg_end) {
+                seg_i = q;
+                ap = seg_a[q];
+                bp = seg_b[q];
+                seg_end += seg_slabs[q];
+            }
         {
-            const bool second = s_begin >= slabs0;
-            const int local_slab = second ? s_begin - slabs0 : s_begin;
-            ap = (const char*)(second ? g.seg[1].A : g.seg[0].A) + (long)local_slab * a_step;
-            bp = (const char*)(second ? g.seg[1].B : g.seg[0].B) + (long)local_slab * b_step;
+            int cur_slabs = seg_slabs[0];
+#pragma unroll
+            for (int q = 1; q < MAXSEG; ++q) cur_slabs = seg_i == q ? seg_slabs[q] : cur_slabs;
+            const int local_slab = s_begin - (seg_end - cur_slabs);
+            ap += (long)local_slab * a_step;
+            bp += (long)local_slab * b_step;
         }
         auto fetchA = [&](auto S) __attribute__((always_inline)) {
 #pragma unroll
@@ -377,9 +424,23 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
             ++fj;
             ap += a_step;
             bp += b_step;
-            if (fj == slabs0 && slabs1 > 0) {
-                ap = (const char*)g.seg[1].A;
-                bp = (const char*)g.seg[1].B;
+            if constexpr (MAXSEG == 2) {
+                // two terms: one compare and two pointer selects
+                if (fj == seg_slabs[0] && seg_slabs[1] > 0) {
+                    ap = seg_a[1];
+                    bp = seg_b[1];
+                }
+            } else {
+                if (fj == seg_end && seg_i + 1 < nseg) {
+                    ++seg_i;
+#pragma unroll
+                    for (int q = 1; q < MAXSEG; ++q)
+                        if (seg_i == q) {
+                            ap = seg_a[q];
+                            bp = seg_b[q];
+                            seg_end += seg_slabs[q];
+                        }
+                }
             }
         };
         float4 a4[2][TM];
@@ -622,7 +683,14 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
             for (int v = 0; v < 16; ++v) {
                 int m = m0 + wm * WTM + ii * 32 + 8 * (v / 4) + 4 * h + (v % 4);
                 if (m < M) {
-                    float* c = g.C + (size_t)m * g.ldc + n;
+                    size_t out_row = (size_t)m;
+                    if (MAXSEG > 2 && g.map_on) {  // only the multi-term kernels carry the map
+                        const unsigned img = row_map_div((unsigned)m, g.map_hw_m, g.map_hw_s), rest = (unsigned)m - img * g.map_hw;
+                        const unsigned i = row_map_div(rest, g.map_w_m, g.map_w_s), j = rest - i * g.map_w;
+                        if ((int)i >= g.map_oh || (int)j >= g.map_ow) continue;
+                        out_row = ((size_t)img * g.map_oh + i) * g.map_ow + j;
+                    }
+                    float* c = g.C + out_row * g.ldc + n;
                     float sum;
                     if (split) {
                         int lm = m - m0, ln = n - n0;
@@ -664,6 +732,23 @@ static int launch_tile(GemmArgs g, bool ta, bool tb, bool vec, int split_k, bool
         else if (V_)                                                                                        \
             hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, TA_, TB_, true, DEPTH, false, KW, MIDB>), grid, block, pad_lds, st, g); \
     }
+#define DALI_GEMM_CASE_TERMS(TB_, V_)                                                                       \
+    if (tb == TB_ && vec == V_) {                                                                           \
+        if (edge)                                                                                           \
+            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, false, TB_, V_, DEPTH, true, KW, false, false, kMaxSeg>), grid, block, pad_lds, st, g);  \
+        else if (V_)                                                                                        \
+            hipLaunchKernelGGL((sgemm_kernel<BM, BN, BK, false, TB_, true, DEPTH, false, KW, MIDB, false, kMaxSeg>), grid, block, pad_lds, st, g); \
+    }
+    if (g.nseg > 2 || g.map_on) {
+        if (ta) return fail("sgemm: more than two terms, or an output row map, need a left operand stored by rows");
+        DALI_GEMM_CASE_TERMS(false, true)
+        DALI_GEMM_CASE_TERMS(false, false)
+        DALI_GEMM_CASE_TERMS(true, true)
+        DALI_GEMM_CASE_TERMS(true, false)
+        hipError_t e2 = hipGetLastError();
+        if (e2 != hipSuccess) return fail("sgemm launch failed: %s", hipGetErrorString(e2));
+        return DALI_HIP_OK;
+    }
     DALI_GEMM_CASE(false, false, true)
     DALI_GEMM_CASE(false, false, false)
     DALI_GEMM_CASE(false, true, true)
@@ -673,6 +758,7 @@ static int launch_tile(GemmArgs g, bool ta, bool tb, bool vec, int split_k, bool
     DALI_GEMM_CASE(true, true, true)
     DALI_GEMM_CASE(true, true, false)
 #undef DALI_GEMM_CASE
+#undef DALI_GEMM_CASE_TERMS
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("sgemm launch failed: %s", hipGetErrorString(e));
     return DALI_HIP_OK;
@@ -724,12 +810,13 @@ static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 // ta: A_s is stored as [K][M]; tb: B_s is stored as [N][K].
 static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K, const float* const* A,
                           const int* lda, const float* const* B, const int* ldb, float alpha, float beta, float* C,
-                          int ldc) {
+                          int ldc, bool rows_may_overlap = false, const int* row_map = nullptr) {
     if (ensure_init()) return DALI_HIP_ERROR;
     if (M < 0 || N < 0) return fail("sgemm: negative extent (M=%d, N=%d)", M, N);
     if (M == 0 || N == 0) return DALI_HIP_OK;
     if (!C) return fail("sgemm: C is NULL");
     if (ldc < N) return fail("sgemm: ldc=%d smaller than row length %d", ldc, N);
+    if (nseg > kMaxSeg) return fail("sgemm: %d terms exceed the limit of %d", nseg, kMaxSeg);
     GemmArgs g = {};
     g.nseg = 0;
     bool vec = true;
@@ -738,7 +825,7 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         if (K[s] == 0) continue;
         if (!A[s] || !B[s]) return fail("sgemm: operand %d is NULL", s);
         int a_row = ta ? M : K[s], b_row = tb ? K[s] : N;
-        if (lda[s] < a_row) return fail("sgemm: leading dimension %d of the left operand is smaller than its row length %d", lda[s], a_row);
+        if (lda[s] < a_row && !(rows_may_overlap && !ta && lda[s] >= 1)) return fail("sgemm: leading dimension %d of the left operand is smaller than its row length %d", lda[s], a_row);
         if (ldb[s] < b_row) return fail("sgemm: leading dimension %d of the right operand is smaller than its row length %d", ldb[s], b_row);
         GemmSeg& sg = g.seg[g.nseg++];
         sg.A = A[s];
@@ -754,6 +841,24 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
     g.ldc = ldc;
     g.alpha = alpha;
     g.beta = beta;
+    if (row_map) {
+        const int map_h = row_map[0], map_w = row_map[1];
+        if (map_h < 1 || map_w < 1 || row_map[2] < 1 || row_map[3] < 1 || row_map[2] > map_h || row_map[3] > map_w || M % (map_h * map_w) != 0)
+            return fail("sgemm: bad output row map [%d x %d] -> [%d x %d] for %d rows", map_h, map_w, row_map[2], row_map[3], M);
+        auto set_div = [](unsigned d, unsigned* m, int* sh) {
+            int sft = 0;
+            while (((unsigned long long)1 << sft) < d) ++sft;
+            *m = (unsigned)((((unsigned long long)1 << (31 + sft)) + d - 1) / d);
+            *sh = sft;
+        };
+        g.map_on = 1;
+        g.map_hw = (unsigned)(map_h * map_w);
+        g.map_w = (unsigned)map_w;
+        set_div(g.map_hw, &g.map_hw_m, &g.map_hw_s);
+        set_div(g.map_w, &g.map_w_m, &g.map_w_s);
+        g.map_oh = row_map[2];
+        g.map_ow = row_map[3];
+    }
     if (g.nseg == 0) {
         // empty inner extent: C = beta * C
         g.nseg = 1;
@@ -819,6 +924,19 @@ int dali_hip_sgemm_pair(int transB1, int transA1, int transB2, int transA2, int 
     const float* Bs[2] = {B1, B2};
     int Ks[2] = {k1, k2}, ldas[2] = {lda1, lda2}, ldbs[2] = {ldb1, ldb2};
     return sgemm_rowmajor(2, transA1 != 0, transB1 != 0, n, m, Ks, As, ldas, Bs, ldbs, alpha, beta, C, ldc);
+}
+
+int dali_hip_sgemm_terms(int nterms, int transA, int transB, int M, int N, const int* K, const float* const* A, int lda,
+                         const float* const* B, int ldb, float alpha, float beta, float* C, int ldc, const int* row_map) {
+    if (nterms < 1 || nterms > kMaxSeg) return fail("dali_hip_sgemm_terms: between 1 and %d terms (got %d)", kMaxSeg, nterms);
+    if (!K || !A || !B) return fail("dali_hip_sgemm_terms: NULL argument");
+    if (M >= (1 << 30) / 2 * 2 && row_map) return fail("dali_hip_sgemm_terms: too many rows for a row map");
+    int ldas[kMaxSeg], ldbs[kMaxSeg];
+    for (int s = 0; s < nterms; ++s) {
+        ldas[s] = lda;
+        ldbs[s] = ldb;
+    }
+    return sgemm_rowmajor(nterms, transA != 0, transB != 0, M, N, K, A, ldas, B, ldbs, alpha, beta, C, ldc, true, row_map);
 }
 
 int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx, const float* Hprev, int ldh,

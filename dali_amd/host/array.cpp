@@ -1155,13 +1155,25 @@ Array conv2d(const Array& input, const Array& filters, int stride_h, int stride_
     check_data_format(data_format, &n_dim, &c_dim, &h_dim, &w_dim);
     check_nchw_or_nhwc("conv2d", data_format);
     ConvFunctionInfo info = compute_conv2d_info(with_batch_axis(input.shape(), n_dim), filters.shape(), stride_h, stride_w, padding, data_format);
+    // channels-last, stride 1: no patch matrix (see conv2d_direct_nhwc); DALI_HIP_CONV_IM2COL=1 keeps the two-step form
+    static const bool two_step = getenv("DALI_HIP_CONV_IM2COL") != nullptr;
+    if (!two_step && !dry_run() && data_format == "NHWC" && stride_h == 1 && stride_w == 1 && input.ndim() == 4 && input.dtype() == DTYPE_FLOAT &&
+        filters.dtype() == DTYPE_FLOAT && info.in_channels % 4 == 0 && info.filter_h <= 8 &&
+        (int64_t)info.batch_size * (info.in_h + 2 * info.padding_h + info.odd_padding_h + info.filter_h) *
+                (info.in_w + 2 * info.padding_w + info.odd_padding_w + info.filter_w) * info.in_channels < ((int64_t)1 << 30)) {
+        input.eval();
+        filters.eval();
+        return conv2d_direct_nhwc(input, filters, info.padding_h, info.padding_w, info.padding_h + info.odd_padding_h,
+                                  info.padding_w + info.odd_padding_w);
+    }
     Array filters_nxxx = filters.swapaxes(n_dim, 0);
     Array filters_nX = filters_nxxx.reshape({filters_nxxx.shape()[0], -1});
     Array patches = im2col(input, info.filter_h, info.filter_w, stride_h, stride_w, info.padding_h, info.padding_w,
                            info.padding_h + info.odd_padding_h, info.padding_w + info.odd_padding_w, data_format);
     if (data_format == "NCHW")
         return dot(filters_nX, patches).reshape({info.out_channels, info.batch_size, info.out_h, info.out_w}).swapaxes(0, 1);
-    return dot(patches.transpose(), filters_nX.transpose()).reshape({info.batch_size, info.out_h, info.out_w, info.out_channels});
+    // the filter matrix is written out transposed (a few hundred KB): the product then reads both operands along their rows
+    return dot(patches.transpose(), filters_nX.transpose().ascontiguousarray()).reshape({info.batch_size, info.out_h, info.out_w, info.out_channels});
 }
 
 // dali/array/op/conv.cpp:278-336. The adjoint of im2col takes no padding (col2im.cpp:217-232), so, like the

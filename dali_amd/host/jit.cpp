@@ -3562,6 +3562,82 @@ Array run_pool2d_backward(const Expr& e, const Array& y_in, const Array& dy_in, 
     return dest;
 }
 
+// Stride-1 convolution of a channels-last image without a patch matrix (dali/array/op/conv.cpp:253-272 forms
+// im2col + one product). The image is copied once into a zero-padded buffer X[N, Hp, Wp, C]; seen as a matrix of
+// pixels with leading dimension C, filter row kh of every patch is the run of filter_w * C values that starts at
+// pixel p + kh * Wp, so the convolution is the sum over kh of the products X(shifted by kh * Wp pixels)[., fw * C] .
+// F[rows of kh, out]: dali_hip_sgemm_terms with overlapping rows, evaluated at all N * Hp * Wp positions, of which
+// the row map stores the out_h x out_w valid ones densely. The patch matrix (filter_h * filter_w times the image) is
+// never written or read.
+Array conv2d_nhwc_direct(const Array& x_in, const Array& filters_in, int pad_top, int pad_left, int pad_bottom, int pad_right) {
+    Array x = dense_buffer(x_in), f = dense_buffer(filters_in);
+    const int N = x.shape()[0], H = x.shape()[1], W = x.shape()[2], C = x.shape()[3];
+    const int O = f.shape()[0], fh = f.shape()[1], fw = f.shape()[2];
+    const int Hp = H + pad_top + pad_bottom, Wp = W + pad_left + pad_right, oh = Hp - fh + 1, ow = Wp - fw + 1;
+    const int64_t pixels = (int64_t)N * Hp * Wp, slack = (int64_t)(fh - 1) * Wp + fw;
+    DALI_ASSERT(oh >= 1 && ow >= 1 && (pixels + slack) * C < ((int64_t)1 << 31), "conv2d: image too large for the direct path");
+    // the filters as a [filter_h * filter_w * C, out] matrix: the product then reads both operands along their rows
+    // (a right operand stored [out][K] costs the kernel a transposing pass through LDS, 211 against 177 us at this size)
+    Array ft = f.reshape({O, fh * fw * C}).transpose().ascontiguousarray();
+    Array xp({(int)(pixels + slack), C}, DTYPE_FLOAT);
+    {
+        Program P;
+        P.arrays.push_back(manual_arg(xp, Cls::FULL, true, 1, {(int)((pixels + slack) * C)}, {}));
+        P.arrays.push_back(manual_arg(x, Cls::FULL, false, 1, {(int)numel_of(x.shape())}, {}));
+        GeomInts G;
+        G.add("PIXELS", (int)pixels);
+        G.add("ALL", (int)(pixels + slack));
+        G.add("H", H);
+        G.add("W", W);
+        G.add("PT", pad_top);
+        G.add("PL", pad_left);
+        G.add_div("HPWP", Hp * Wp);
+        G.add_div("WP", Wp);
+        G.add_div("C4", C / 4);
+        launch_special("pad", "pad_nhwc|f32", P, ((pixels + slack) * (C / 4) + 255) / 256, G, [&](std::ostringstream& ss) {
+            ss << "  T* out = (T*)A.p[0];\n  const T* img = (const T*)A.p[1];\n";
+            ss << "  const unsigned total = (unsigned)ALL * (unsigned)C4;\n";
+            ss << "  for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {\n";
+            ss << "    " << divmod("p", "c4", "i", "C4") << "\n";
+            ss << "    " << divmod("n", "rest", "p", "HPWP") << "\n";
+            ss << "    " << divmod("ip", "jp", "(unsigned)rest", "WP") << "\n";
+            ss << "    const int h = (int)ip - PT, w = jp - PL;\n";
+            ss << "    dali_vec<T, 4> v;\n";
+            ss << "    if (p < (unsigned)PIXELS && h >= 0 && h < H && w >= 0 && w < W) v = dali_load<T, 4>(img + ((((long)n * H + h) * W + w) * C4 + c4) * 4);\n";
+            ss << "    else { _Pragma(\"unroll\") for (int k = 0; k < 4; ++k) v.v[k] = (T)0; }\n";
+            ss << "    dali_store<T, 4>(out + (long)i * 4, v);\n  }\n}\n";
+        });
+    }
+    Array out({N, oh, ow, O}, DTYPE_FLOAT);
+    const float* xpp = (const float*)xp.device_ptr();
+    const float* fp = (const float*)ft.device_ptr();
+    float* op_ = (float*)out.device_ptr(memory::AM_OVERWRITE);
+    const int lda = C, ldb = O, M = (int)pixels;
+    auto issue = [=]() {
+        int K[8];
+        const float* As[8];
+        const float* Bs[8];
+        for (int t = 0; t < fh; ++t) {
+            K[t] = fw * C;
+            As[t] = xpp + (size_t)t * Wp * C;
+            Bs[t] = fp + (size_t)t * fw * C * O;
+        }
+        const int row_map[4] = {Hp, Wp, oh, ow};
+        check_hip(dali_hip_sgemm_terms(fh, 0, 0, M, O, K, As, lda, Bs, ldb, 1.0f, 0.0f, op_, O, row_map), "convolution product");
+    };
+    jit_stats().gemms_launched++;
+    issue();
+    if (g_recording) {
+        note_recorded_write(out.expression()->memory);
+        std::vector<Array> keep = {xp, ft, out};
+        g_recording->push_back([=]() {
+            (void)keep;
+            issue();
+        });
+    }
+    return out;
+}
+
 // ----------------------------------------------------------- index-valued fills
 // arange (dali/array/op/arange.cpp:8-39: start + offset * step, in the operands' own arithmetic) and diag / eye
 // (dali/array/op/eye.cpp:29-36: the diagonal value where row == column, else 0) as one thread per element.
@@ -3670,6 +3746,10 @@ void scatter_assign(const Array& dest, OPERATOR_T op, const Array& source) {
 }
 
 }  // namespace
+
+Array conv2d_direct_nhwc(const Array& x, const Array& filters, int pad_top, int pad_left, int pad_bottom, int pad_right) {
+    return conv2d_nhwc_direct(x, filters, pad_top, pad_left, pad_bottom, pad_right);
+}
 
 void lstm_step_fused(const Array& x, const Array& h, const Array& c, const Array& W, const Array& U, const Array& b, const Array& c_new,
                      const Array& h_new) {

@@ -216,6 +216,17 @@ int dali_hip_sgemm_pair(int transB1, int transA1, int transB2, int transA2, int 
                         float alpha, const float* B1, int ldb1, const float* A1, int lda1, const float* B2,
                         int ldb2, const float* A2, int lda2, float beta, float* C, int ldc);
 
+/* Row-major sum of up to 8 products into one accumulator: C[M, N] = alpha * sum_t op(A_t) . op(B_t) + beta * C, all A_t with
+ * the leading dimension lda and all B_t with ldb (transA: A_t stored [K_t][M]; transB: B_t stored [N][K_t]). Without
+ * transA the rows of A_t may overlap (lda < K_t). That is a stride-1 convolution without a patch matrix: over a
+ * zero-padded channels-last image X[N, Hp, Wp, C], filter row kh is the term A = X + kh * Wp * C, lda = C, K = filter_w * C
+ * against rows [kh * filter_w * C, ...) of the filter matrix, evaluated at every padded position (M = N * Hp * Wp); the image
+ * needs (filter_h - 1) * Wp + filter_w pixels of readable slack behind it. row_map (NULL, or {Hp, Wp, out_h, out_w}) keeps
+ * only the positions i < out_h, j < out_w of each [Hp, Wp] grid and stores them densely, as rows (n * out_h + i) * out_w + j.
+ * Replaces im2col + op::dot in op::conv2d (dali/array/op/conv.cpp:253-272) for the NHWC, stride-1 case. */
+int dali_hip_sgemm_terms(int nterms, int transA, int transB, int M, int N, const int* K, const float* const* A, int lda,
+                         const float* const* B, int ldb, float alpha, float beta, float* C, int ldc, const int* row_map);
+
 /*
  * One LSTM cell step in a single launch: pre = X[batch, input] . W[input, 4 hidden] + Hprev[batch, hidden] .
  * U[hidden, 4 hidden] (row-major, gates packed i, f, o, g along the columns), then per element

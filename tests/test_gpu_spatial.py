@@ -9,6 +9,8 @@ import pytest
 
 from conftest import golden
 
+import ctypes as C
+
 pytestmark = pytest.mark.gpu
 
 
@@ -162,3 +164,68 @@ def test_pool2d_pair_matches_oracle(gpu, D, O, rng, fmt):
     assert np.array_equal(D.op.pool2d(arr(D, x), 3, 3, 2, 2, "max", "same", fmt).numpy(), O.pool2d(x, 3, 3, 2, 2, "max", "same", fmt))
     with pytest.raises(Exception):
         D.op.pool2d(arr(D, x), 2, 2, 2, 2, "max", "valid", "CHWN")
+
+
+def test_sgemm_terms_is_a_convolution_over_overlapping_rows(gpu, rng):
+    """dali_hip_sgemm_terms through the C ABI: filter rows as terms over a padded channels-last image whose pixel rows
+    overlap (lda = C < K), every padded position computed, the row map keeping the valid ones."""
+    hip = gpu
+    N, Hp, Wp, Cc, O, fh, fw = 3, 9, 11, 8, 12, 3, 2
+    oh, ow = Hp - fh + 1, Wp - fw + 1
+    slack = (fh - 1) * Wp + fw
+    xp = np.zeros((N * Hp * Wp + slack, Cc), np.float32)
+    xp[:N * Hp * Wp] = rng.randint(-3, 4, (N * Hp * Wp, Cc))
+    f = rng.randint(-3, 4, (O, fh, fw, Cc)).astype(np.float32)
+
+    def dev(a):
+        p = C.c_void_p()
+        assert hip.dali_hip_malloc(C.byref(p), a.nbytes) == 0
+        assert hip.dali_hip_memcpy_h2d(p, a.ctypes.data_as(C.c_void_p), a.nbytes) == 0
+        return p
+
+    dx, df = dev(xp), dev(f)
+    out = np.full((N, oh, ow, O), 7.0, np.float32)
+    dout = dev(out)
+    K = (C.c_int * fh)(*[fw * Cc] * fh)
+    As = (C.c_void_p * fh)(*[dx.value + t * Wp * Cc * 4 for t in range(fh)])
+    Bs = (C.c_void_p * fh)(*[df.value + t * fw * Cc * 4 for t in range(fh)])
+    row_map = (C.c_int * 4)(Hp, Wp, oh, ow)
+    st = hip.dali_hip_sgemm_terms(fh, 0, 1, N * Hp * Wp, O, K, As, Cc, Bs, fh * fw * Cc, 1.0, 0.0, dout, O, row_map)
+    assert st == 0, hip.dali_hip_last_error()
+    assert hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dout, out.nbytes) == 0
+    img = xp[:N * Hp * Wp].reshape(N, Hp, Wp, Cc).astype(np.float64)
+    want = np.zeros((N, oh, ow, O))
+    for i in range(oh):
+        for j in range(ow):
+            want[:, i, j, :] = np.einsum("nhwc,ohwc->no", img[:, i:i + fh, j:j + fw, :], f.astype(np.float64))
+    assert np.array_equal(out, want)  # small integers: exact
+    # without the map every padded position is stored, the valid ones in place
+    full = np.zeros((N * Hp * Wp, O), np.float32)
+    dfull = dev(full)
+    assert hip.dali_hip_sgemm_terms(fh, 0, 1, N * Hp * Wp, O, K, As, Cc, Bs, fh * fw * Cc, 1.0, 0.0, dfull, O, None) == 0
+    assert hip.dali_hip_memcpy_d2h(full.ctypes.data_as(C.c_void_p), dfull, full.nbytes) == 0
+    assert np.array_equal(full.reshape(N, Hp, Wp, O)[:, :oh, :ow, :], want)
+    bad = (C.c_int * 4)(Hp, Wp, Hp + 1, ow)
+    assert hip.dali_hip_sgemm_terms(fh, 0, 1, N * Hp * Wp, O, K, As, Cc, Bs, fh * fw * Cc, 1.0, 0.0, dout, O, bad) != 0
+    for p in (dx, df, dout, dfull):
+        hip.dali_hip_free(p)
+
+
+def test_conv2d_nhwc_direct_path_equals_the_two_step_form(gpu, D, O, rng):
+    """Channels-last, stride 1: one padding copy + a multi-term product. Same numbers as im2col + one product on
+    integer-valued data, and one kernel plus one product instead of a patch matrix."""
+    for padding in ("valid", "same"):
+        for fh, fw in ((3, 3), (1, 1), (5, 2), (2, 7)):
+            x = rng.randint(-3, 4, (4, 12, 10, 8)).astype(np.float32)
+            w = rng.randint(-3, 4, (16, fh, fw, 8)).astype(np.float32)
+            before = D.jit_stats()
+            y = D.op.conv2d(arr(D, x), arr(D, w), 1, 1, padding, "NHWC")
+            got = y.numpy()
+            after = D.jit_stats()
+            assert "pad" in D.last_kernel_kinds() and after["gemms"] - before["gemms"] == 1
+            assert np.array_equal(got, O.conv2d(x, w, 1, 1, padding, "NHWC"))
+    # channel counts that are not multiples of 4 keep the patch-matrix form
+    x = rng.randint(-3, 4, (2, 6, 7, 3)).astype(np.float32)
+    w = rng.randint(-3, 4, (5, 3, 3, 3)).astype(np.float32)
+    assert np.array_equal(D.op.conv2d(arr(D, x), arr(D, w), 1, 1, "same", "NHWC").numpy(), O.conv2d(x, w, 1, 1, "same", "NHWC"))
+    assert "im2col" in D.last_kernel_kinds() or D.jit_stats()["gemms"] > 0
