@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-14";
+const char* const kCodegenVersion = "dali-hip-codegen-15";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -3520,14 +3520,17 @@ Array run_pool2d_backward(const Expr& e, const Array& y_in, const Array& dy_in, 
     if (n == 0) return dest;
     ImageGeom gx = image_geom(x.shape(), fmt), gy = image_geom(y.shape(), fmt);
     const bool average = e.depth != 0;
-    const int VEC = fmt[3] == 'C' && four_byte_vectors(e.dtype, x, gx.ext[1]) && y.offset() % 4 == 0 && dy.offset() % 4 == 0 ? 4 : 1;
+    const bool channel_vectors = fmt[3] == 'C' && four_byte_vectors(e.dtype, x, gx.ext[1]) && y.offset() % 4 == 0 && dy.offset() % 4 == 0;
+    // formats ending in W: a thread takes four neighbours along W, which share everything but their window columns
+    const bool along_w = fmt[3] == 'W' && four_byte_vectors(e.dtype, x, gx.ext[3]);
+    const int VEC = channel_vectors || along_w ? 4 : 1;
     Program P;
     P.arrays.push_back(manual_arg(dest, Cls::FULL, true, 1, {(int)n}, {}));
     P.arrays.push_back(manual_arg(y, Cls::FULL, false, 1, {(int)numel_of(y.shape())}, {}));
     P.arrays.push_back(manual_arg(dy, Cls::FULL, false, 1, {(int)numel_of(dy.shape())}, {}));
     P.arrays.push_back(manual_arg(x, Cls::FULL, false, 1, {(int)numel_of(x.shape())}, {}));
     std::ostringstream sig;
-    sig << "pool2d_backward|" << (int)e.dtype << "|" << fmt << "|" << average << "|" << VEC << "|" << e.geom[0] << "," << e.geom[1] << "," << e.geom[2] << ","
+    sig << "pool2d_backward|" << (int)e.dtype << "|" << fmt << "|" << average << "|" << VEC << along_w << "|" << e.geom[0] << "," << e.geom[1] << "," << e.geom[2] << ","
         << e.geom[3];
     launch_special("pool2d_backward", sig.str(), P, (n / VEC + 255) / 256, pool_geom(e, gx, gy, e.shape[3] / VEC), [&](std::ostringstream& ss) {
         ss << pool_constants(e, VEC);
@@ -3538,24 +3541,42 @@ Array run_pool2d_backward(const Expr& e, const Array& y_in, const Array& dy_in, 
         ss << emit_decompose(fmt, "H", "W", "h", "w", true);
         ss << "    const dali_vec<T, VEC> src = dali_load<T, VEC>(x + (long)i * VEC);\n";
         ss << "    const int ph_start = (h + PH) < WH ? 0 : (h + PH - WH) / STH + 1;\n";
-        ss << "    const int pw_start = (w + PW) < WW ? 0 : (w + PW - WW) / STW + 1;\n";
         ss << "    const int ph_end = (h + PH) / STH + 1 < OH ? (h + PH) / STH + 1 : OH;\n";
-        ss << "    const int pw_end = (w + PW) / STW + 1 < OW ? (w + PW) / STW + 1 : OW;\n";
         ss << "    const long base = (long)n * YSN + (long)c * YSC;\n";
         ss << "    dali_vec<T, VEC> grad;\n    _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) grad.v[k] = (T)0;\n";
-        ss << "    _Pragma(\"unroll\") for (int a = 0; a < MAX_PH; ++a) {\n      const int ph = ph_start + a; const bool ph_ok = ph < ph_end;\n";
-        ss << "      _Pragma(\"unroll\") for (int b = 0; b < MAX_PW; ++b) {\n        const int pw = pw_start + b; const bool ok = ph_ok && pw < pw_end;\n";
-        ss << "        const long q = ok ? base + (ph * YSH + pw * YSW) : 0;  // beyond the range: a valid address, value unused\n";
-        ss << "        const dali_vec<T, VEC> g = dali_load<T, VEC>(dy + q);\n";
-        if (average) {
-            ss << "        int hstart = ph * STH - PH, wstart = pw * STW - PW;\n";
-            ss << "        const int hend = hstart + WH < H ? hstart + WH : H, wend = wstart + WW < W ? wstart + WW : W;\n";
-            ss << "        hstart = hstart > 0 ? hstart : 0; wstart = wstart > 0 ? wstart : 0;\n";
-            ss << "        const int pool_size = (hend - hstart) * (wend - wstart);\n";
-            ss << "        if (ok) { _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) grad.v[k] += ((T)1 * g.v[k]) / pool_size; }\n      }\n    }\n";
+        // one window (ph, pw) adds to element k (all elements when the vector runs along the channels)
+        auto add_window = [&](const std::string& k_lo, const std::string& k_hi, const std::string& g, const std::string& yv) {
+            if (average) {
+                ss << "          int hstart = ph * STH - PH, wstart = pw * STW - PW;\n";
+                ss << "          const int hend = hstart + WH < H ? hstart + WH : H, wend = wstart + WW < W ? wstart + WW : W;\n";
+                ss << "          hstart = hstart > 0 ? hstart : 0; wstart = wstart > 0 ? wstart : 0;\n";
+                ss << "          const int pool_size = (hend - hstart) * (wend - wstart);\n";
+                ss << "          if (ok) { _Pragma(\"unroll\") for (int k = " << k_lo << "; k < " << k_hi << "; ++k) grad.v[k] += ((T)1 * " << g << ") / pool_size; }\n";
+            } else {
+                ss << "          if (ok) { _Pragma(\"unroll\") for (int k = " << k_lo << "; k < " << k_hi << "; ++k) grad.v[k] += (" << yv << " == src.v[k] ? (T)1 : (T)0) * " << g << "; }\n";
+            }
+        };
+        if (along_w) {
+            ss << "    _Pragma(\"unroll\") for (int e = 0; e < VEC; ++e) {\n      const int we = w + e;\n";
+            ss << "      const int pw_start = (we + PW) < WW ? 0 : (we + PW - WW) / STW + 1;\n";
+            ss << "      const int pw_end = (we + PW) / STW + 1 < OW ? (we + PW) / STW + 1 : OW;\n";
+            ss << "      _Pragma(\"unroll\") for (int a = 0; a < MAX_PH; ++a) {\n        const int ph = ph_start + a; const bool ph_ok = ph < ph_end;\n";
+            ss << "        _Pragma(\"unroll\") for (int b = 0; b < MAX_PW; ++b) {\n          const int pw = pw_start + b; const bool ok = ph_ok && pw < pw_end;\n";
+            ss << "          const long q = ok ? base + (ph * YSH + pw * YSW) : 0;  // beyond the range: a valid address, value unused\n";
+            ss << "          const T g1 = dy[q];\n";
+            if (!average) ss << "          const T y1 = y[q];\n";
+            add_window("e", "e + 1", "g1", "y1");
+            ss << "        }\n      }\n    }\n";
         } else {
-            ss << "        const dali_vec<T, VEC> yv = dali_load<T, VEC>(y + q);\n";
-            ss << "        if (ok) { _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) grad.v[k] += (yv.v[k] == src.v[k] ? (T)1 : (T)0) * g.v[k]; }\n      }\n    }\n";
+            ss << "    const int pw_start = (w + PW) < WW ? 0 : (w + PW - WW) / STW + 1;\n";
+            ss << "    const int pw_end = (w + PW) / STW + 1 < OW ? (w + PW) / STW + 1 : OW;\n";
+            ss << "    _Pragma(\"unroll\") for (int a = 0; a < MAX_PH; ++a) {\n      const int ph = ph_start + a; const bool ph_ok = ph < ph_end;\n";
+            ss << "      _Pragma(\"unroll\") for (int b = 0; b < MAX_PW; ++b) {\n        const int pw = pw_start + b; const bool ok = ph_ok && pw < pw_end;\n";
+            ss << "          const long q = ok ? base + (ph * YSH + pw * YSW) : 0;  // beyond the range: a valid address, value unused\n";
+            ss << "          const dali_vec<T, VEC> g = dali_load<T, VEC>(dy + q);\n";
+            if (!average) ss << "          const dali_vec<T, VEC> yv = dali_load<T, VEC>(y + q);\n";
+            add_window("0", "VEC", "g.v[k]", "yv.v[k]");
+            ss << "      }\n    }\n";
         }
         ss << "    dali_store<T, VEC>(dx + (long)i * VEC, grad);\n  }\n}\n";
     });
