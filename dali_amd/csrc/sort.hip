@@ -20,39 +20,70 @@ __global__ __launch_bounds__(256) void iota_kernel(int32_t* out, long n) {
 }
 
 // A few thousand keys: counting ranks beats any multi-pass sort. The final position of key i is the number of
-// (key, position) pairs that order before it; every workgroup counts, for 256 keys, the smaller pairs within one
-// segment of the input (staged in LDS, read as wave-wide broadcasts), and a second kernel adds the per-segment
-// counts and places the key. n * n comparisons, but spread over the whole chip and two launches in all.
-__device__ __forceinline__ unsigned long long rank_pair(int32_t key, int pos) {
+// (key, position) pairs that order before it. A workgroup counts, for 256 keys, the smaller pairs within one
+// segment of the input (staged in LDS, read as wave-wide broadcasts) and publishes the counts; the workgroup that
+// finishes last for those 256 keys (a ticket per key block) adds the segments' counts and places the keys.
+// n * n comparisons, but spread over the whole chip, in one launch and without an allocation: the counts and the
+// tickets live in the library workspace. When key_limit * 2^ceil(log2 n) fits 32 bits a pair is one 32-bit word
+// (key in the high bits, position in the low ones), which halves the cost of a comparison.
+template <typename W>
+__device__ __forceinline__ W rank_pair(int32_t key, int pos, int shift);
+template <>
+__device__ __forceinline__ unsigned long long rank_pair<unsigned long long>(int32_t key, int pos, int) {
     return ((unsigned long long)((unsigned int)key ^ 0x80000000u) << 32) | (unsigned int)pos;  // signed key order
+}
+template <>
+__device__ __forceinline__ unsigned int rank_pair<unsigned int>(int32_t key, int pos, int shift) {
+    // a key outside [0, key_limit) (an invalid index) is ordered as the largest valid key: whatever the input, the
+    // words stay distinct, so the positions computed from them are a permutation
+    const unsigned int top = (0xFFFFFFFFu >> shift);
+    const unsigned int k = (unsigned int)key < top ? (unsigned int)key : top;
+    return (k << shift) | (unsigned int)pos;
 }
 
 constexpr int kRankSegment = 512;
+constexpr int kRankMaxSegments = 32;  // 16384 keys
 
-__global__ __launch_bounds__(256) void rank_count_kernel(const int32_t* keys, int n, int32_t* partial) {
-    __shared__ unsigned long long tile[kRankSegment];
+template <typename W>
+__global__ __launch_bounds__(256) void rank_sort_kernel(const int32_t* keys, int n, int shift, int segments, int32_t* partial,
+                                                         unsigned int* tickets, int32_t* sorted_keys, int32_t* perm) {
+    __shared__ __attribute__((aligned(16))) W tile[kRankSegment];
+    __shared__ int is_last;
     const int i = blockIdx.x * 256 + threadIdx.x;
     const int j0 = blockIdx.y * kRankSegment;
     for (int t = threadIdx.x; t < kRankSegment; t += 256) {
         const int j = j0 + t;
-        tile[t] = j < n ? rank_pair(keys[j], j) : ~0ull;  // padding orders after every real pair
+        tile[t] = j < n ? rank_pair<W>(keys[j], j, shift) : ~(W)0;  // padding orders after (or with) every real pair
     }
     __syncthreads();
-    const unsigned long long mine = rank_pair(i < n ? keys[i] : 0, i);
+    const int32_t my_key = i < n ? keys[i] : 0;
+    const W mine = rank_pair<W>(my_key, i, shift);
     int count = 0;
 #pragma unroll 16
     for (int t = 0; t < kRankSegment; ++t) count += tile[t] < mine ? 1 : 0;
-    if (i < n) partial[(size_t)blockIdx.y * n + i] = count;
-}
-
-__global__ __launch_bounds__(256) void rank_place_kernel(const int32_t* keys, int n, int segments, const int32_t* partial,
-                                                          int32_t* sorted_keys, int32_t* perm) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    int pos = 0;
-    for (int s = 0; s < segments; ++s) pos += partial[(size_t)s * n + i];
-    sorted_keys[pos] = keys[i];
-    perm[pos] = i;
+    if (i < n) __hip_atomic_store(partial + (size_t)blockIdx.y * n + i, count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned int ticket = __hip_atomic_fetch_add(tickets + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = ticket == (unsigned int)segments - 1;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    if (i < n) {
+        // all segments' counts are requested before the first one is waited for (a loop of run-time length would wait
+        // for every load in turn)
+        int part[kRankMaxSegments];
+#pragma unroll
+        for (int s = 0; s < kRankMaxSegments; ++s)
+            part[s] = s < segments ? __hip_atomic_load(partial + (size_t)s * n + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+        int pos = 0;
+#pragma unroll
+        for (int s = 0; s < kRankMaxSegments; ++s) pos += part[s];
+        sorted_keys[pos] = my_key;
+        perm[pos] = i;
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(tickets + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace dali_hip
@@ -73,14 +104,22 @@ extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_
         while (end_bit < 31 && ((int64_t)1 << end_bit) < (int64_t)key_limit) ++end_bit;
     }
     static const int rank_max = getenv("DALI_HIP_RANK_SORT_MAX") ? atoi(getenv("DALI_HIP_RANK_SORT_MAX")) : 16384;
-    if (n <= rank_max) {
+    if (n <= rank_max && n <= (int64_t)kRankSegment * kRankMaxSegments &&
+        (size_t)((n + kRankSegment - 1) / kRankSegment) * (size_t)n * sizeof(int32_t) <= kWorkspacePartialBytes &&
+        (n + 255) / 256 <= kWorkspaceCounters) {
         const int ni = (int)n, segments = (ni + kRankSegment - 1) / kRankSegment, blocks = (ni + 255) / 256;
-        void* partial = nullptr;
-        if (dali_hip_bank_allocate(&partial, (size_t)segments * ni * sizeof(int32_t))) return DALI_HIP_ERROR;
-        hipLaunchKernelGGL(rank_count_kernel, dim3(blocks, segments), dim3(256), 0, st, keys, ni, (int32_t*)partial);
-        hipLaunchKernelGGL(rank_place_kernel, dim3(blocks), dim3(256), 0, st, keys, ni, segments, (const int32_t*)partial, sorted_keys, perm);
+        unsigned int* tickets = (unsigned int*)workspace();
+        int32_t* partial = (int32_t*)(workspace() + kWorkspaceCounterBytes);
+        int shift = 0;
+        while ((1 << shift) < ni) ++shift;
+        const bool packed = key_limit > 0 && ((unsigned long long)key_limit << shift) <= (1ull << 32);
+        if (packed)
+            hipLaunchKernelGGL(rank_sort_kernel<unsigned int>, dim3(blocks, segments), dim3(256), 0, st, keys, ni, shift, segments, partial, tickets,
+                               sorted_keys, perm);
+        else
+            hipLaunchKernelGGL(rank_sort_kernel<unsigned long long>, dim3(blocks, segments), dim3(256), 0, st, keys, ni, shift, segments, partial,
+                               tickets, sorted_keys, perm);
         hipError_t le = hipGetLastError();
-        dali_hip_bank_deposit(partial, (size_t)segments * ni * sizeof(int32_t));
         if (le != hipSuccess) return fail("rank sort launch failed: %s", hipGetErrorString(le));
         return DALI_HIP_OK;
     }

@@ -250,6 +250,9 @@ int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx
  * 126-143): the reference's GPU code adds duplicates with atomicAdd in arrival order (gather.cpp:14-28);
  * the generated scatter kernel instead walks each destination row's contributions in input order,
  * the order of the reference's sequential CPU loop, so the result does not depend on scheduling.
+ * Up to 16384 keys are ordered by one kernel that allocates nothing (it may be captured); longer inputs take a
+ * radix sort whose temporary blocks come from the bank. With key_limit > 0, keys outside the promised range come
+ * out in an unspecified order, but perm is a permutation for any input.
  */
 int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_limit, int32_t* sorted_keys, int32_t* perm);
 

@@ -869,6 +869,17 @@ def test_cabi_argsort_is_stable(gpu, rng, n):
     check(keys, 0)
     for limit in (1, 2, 1000, 32000, 32768):  # bounded keys: only the low bits are sorted
         check(rng.randint(0, limit, n).astype(np.int32), limit)
+    check(rng.randint(0, 1 << 30, n).astype(np.int32), 1 << 30)  # a bound too wide for one-word pairs
+    check(rng.randint(0, 7, n).astype(np.int32), 7)               # a second call finds the tickets back at zero
+    # keys outside the promised range (invalid indices) may come out in any order, but the result stays a permutation
+    wild = rng.randint(0, 1000, n).astype(np.int32)
+    wild[::3] = np.iinfo(np.int32).max
+    wild[1::7] = -5
+    hip.dali_hip_memcpy_h2d(dk, wild.ctypes.data_as(C.c_void_p), n * 4)
+    assert hip.dali_hip_argsort_i32(dk, n, 1000, ds, dp) == 0
+    hip.dali_hip_memcpy_d2h(sk.ctypes.data_as(C.c_void_p), ds, n * 4)
+    hip.dali_hip_memcpy_d2h(pm.ctypes.data_as(C.c_void_p), dp, n * 4)
+    assert np.array_equal(np.sort(pm), np.arange(n)) and np.array_equal(sk, wild[pm])
     for p in (dk, ds, dp):
         hip.dali_hip_free(p)
 
