@@ -705,6 +705,27 @@ def test_graph_replays_match_eager_on_every_replay(gpu, D, O, rng):
         close(got[1], o_loss, rtol=1e-5 + v * 2.0 ** -24, atol=1e-6)
 
 
+def test_graph_replays_of_a_scatter_add(gpu, D, O, rng):
+    """Assignment through a gather inside a HIP graph: for up to 16384 indices the index ordering allocates nothing,
+    so both of its launches can be captured; every replay adds the same contributions in input order."""
+    V, Dm, N = 300, 64, 500
+    table0 = rng.randn(V, Dm).astype(np.float32)
+    idx = rng.randint(0, V, N).astype(np.int32)
+    upd = rng.randn(N, Dm).astype(np.float32)
+    table, ids, vals = arr(D, table0), arr(D, idx), arr(D, upd)
+    with D.Recording() as rec:
+        g = table[ids]
+        g += vals
+    want = O.scatter_rows(table0, idx, upd, op=1)
+    assert np.array_equal(table.numpy(), want)
+    rec.make_graph()
+    for it in range(3):
+        (D.op.tanh(vals) + 1.0).eval()  # eager work between the replays
+        rec.replay(1)
+        want = O.scatter_rows(want, idx, upd, op=1)
+        assert np.array_equal(table.numpy(), want), "replay %d" % it
+
+
 def test_cabi_graph_capture_of_gemm(gpu, D, rng):
     # dali_hip_capture_begin / _end / _graph_launch around dali_hip_sgemm, with C-ABI calls only
     import ctypes as C
