@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-15";
+const char* const kCodegenVersion = "dali-hip-codegen-18";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -3239,6 +3239,13 @@ std::string emit_join_row(const std::string& fmt) {
     return expr;
 }
 
+// Element loop of the per-element sliding-window kernels. Workgroups are dealt to the eight XCDs round-robin;
+// renumbering them gives every XCD one contiguous band of the index range, so that neighbours which share input rows
+// (overlapping windows, the patches over a pixel) find them in the same L2 instead of fetching them once per XCD.
+const char* const kBandedElementLoop =
+    "  const unsigned nb_ = gridDim.x, vb_ = nb_ % 8u == 0 ? (blockIdx.x % 8u) * (nb_ / 8u) + blockIdx.x / 8u : blockIdx.x;\n"
+    "  for (unsigned i = vb_ * 256u + threadIdx.x; i < total; i += nb_ * 256u) {\n";
+
 // One launch of a hand-laid-out kernel: `blocks` workgroups of 256 threads (the kernels stride over blocks, so a
 // capped grid still covers the work); the geometry travels as the integers behind the arrays' sizes.
 void launch_special(const char* kind, const std::string& sig, const Program& P, int64_t blocks, const GeomInts& G,
@@ -3429,7 +3436,7 @@ Array run_col2im(const Expr& e, const Array& patches_in) {
         ss << "  T* image = (T*)A.p[0];\n  const T* in = (const T*)A.p[1];\n";
         ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(H * W) / VEC;\n";
         ss << "  constexpr int patch_h = DH * (FH - 1) + 1, patch_w = DW * (FW - 1) + 1;\n";
-        ss << "  for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {\n";
+        ss << kBandedElementLoop;
         ss << emit_decompose(fmt, "H", "W", "h_", "w_", true);
         ss << "    const int h = h_ + PH, w = w_ + PW;\n";
         ss << "    const int ph_min = h < patch_h ? h % DH : (h - patch_h + STH) / STH;\n";
@@ -3483,6 +3490,8 @@ Array run_pool2d(const Expr& e, const Array& x_in) {
     if (n == 0) return dest;
     ImageGeom gx = image_geom(x.shape(), fmt), gy = image_geom(e.shape, fmt);
     const bool average = e.depth != 0;
+    // One output per thread for layouts ending in W: four neighbours along W per thread were tried, but a wave's loads then
+    // spread over four times as many cache lines and the kernel ran three times slower.
     const int VEC = fmt[3] == 'C' && four_byte_vectors(e.dtype, x, gx.ext[1]) ? 4 : 1;
     Program P;
     P.arrays.push_back(manual_arg(dest, Cls::FULL, true, 1, {(int)n}, {}));
@@ -3493,13 +3502,16 @@ Array run_pool2d(const Expr& e, const Array& x_in) {
         ss << pool_constants(e, VEC);
         ss << "  T* y = (T*)A.p[0];\n  const T* x = (const T*)A.p[1];\n";
         ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(OH * OW) / VEC;\n";
-        ss << "  for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {\n";
+        ss << kBandedElementLoop;
         ss << emit_decompose(fmt, "OH", "OW", "oh", "ow", true);
-        ss << "    const int w0 = ow * STW - PW, h0 = oh * STH - PH;\n";
-        ss << "    const int w_start = w0 > 0 ? w0 : 0, w_end = w0 + WW < W ? w0 + WW : W;\n";
+        ss << "    const int h0 = oh * STH - PH;\n";
         ss << "    const int h_start = h0 > 0 ? h0 : 0, h_end = h0 + WH < H ? h0 + WH : H;\n";
         ss << "    const T* xp = x + ((long)n * SN + (long)c * SC);\n";
-        ss << "    dali_vec<T, VEC> res;\n    _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) res.v[k] = " << (average ? "(T)0" : "reducers::lowest<T>()") << ";\n";
+        ss << "    dali_vec<T, VEC> res;\n";
+        const std::string init = average ? "(T)0" : "reducers::lowest<T>()";
+        ss << "    const int w0 = ow * STW - PW;\n";
+        ss << "    const int w_start = w0 > 0 ? w0 : 0, w_end = w0 + WW < W ? w0 + WW : W;\n";
+        ss << "    _Pragma(\"unroll\") for (int k = 0; k < VEC; ++k) res.v[k] = " << init << ";\n";
         ss << "    _Pragma(\"unroll\") for (int a = 0; a < WW; ++a) {\n      const int w = w0 + a; const bool w_ok = w >= 0 && w < W; const int wc = w_ok ? w : w_start;\n";
         ss << "      _Pragma(\"unroll\") for (int b = 0; b < WH; ++b) {\n        const int h = h0 + b; const bool ok = w_ok && h >= 0 && h < H; const int hc = h >= 0 && h < H ? h : h_start;\n";
         ss << "        const dali_vec<T, VEC> v = dali_load<T, VEC>(xp + (hc * SH + wc * SW));\n";
@@ -3537,7 +3549,7 @@ Array run_pool2d_backward(const Expr& e, const Array& y_in, const Array& dy_in, 
         ss << "  constexpr int MAX_PH = (WH + STH - 1) / STH, MAX_PW = (WW + STW - 1) / STW;\n";
         ss << "  T* dx = (T*)A.p[0];\n  const T* y = (const T*)A.p[1];\n  const T* dy = (const T*)A.p[2];\n  const T* x = (const T*)A.p[3];\n";
         ss << "  const unsigned total = (unsigned)(N * C) * (unsigned)(H * W) / VEC;\n";
-        ss << "  for (unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {\n";
+        ss << kBandedElementLoop;
         ss << emit_decompose(fmt, "H", "W", "h", "w", true);
         ss << "    const dali_vec<T, VEC> src = dali_load<T, VEC>(x + (long)i * VEC);\n";
         ss << "    const int ph_start = (h + PH) < WH ? 0 : (h + PH - WH) / STH + 1;\n";
