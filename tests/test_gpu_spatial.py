@@ -229,3 +229,30 @@ def test_conv2d_nhwc_direct_path_equals_the_two_step_form(gpu, D, O, rng):
     w = rng.randint(-3, 4, (5, 3, 3, 3)).astype(np.float32)
     assert np.array_equal(D.op.conv2d(arr(D, x), arr(D, w), 1, 1, "same", "NHWC").numpy(), O.conv2d(x, w, 1, 1, "same", "NHWC"))
     assert "im2col" in D.last_kernel_kinds() or D.jit_stats()["gemms"] > 0
+
+
+@pytest.mark.parametrize("fmt", ["NCHW", "NHWC"])
+def test_sliding_windows_in_double_and_int32(gpu, D, O, rng, fmt):
+    """The kernels are generated per dtype: fp64 agrees with the fp32 checker on values that are exact in both,
+    int32 pooling takes the maximum / the truncating integer average of the reference's `res / area` with T = int."""
+    shape = (2, 3, 6, 8) if fmt == "NCHW" else (2, 6, 8, 3)
+    xi = rng.randint(-20, 21, shape).astype(np.int32)
+    for dtype in (np.float64, np.int32):
+        x = xi.astype(dtype)
+        y = D.op.pool2d(arr(D, x), 2, 3, 2, 1, "max", "same", fmt)
+        want = O.pool2d(xi.astype(np.float32), 2, 3, 2, 1, "max", "same", fmt)
+        assert y.numpy().dtype == dtype and np.array_equal(y.numpy(), want.astype(dtype))
+        p = D.op.im2col(arr(D, x), 2, 2, 1, 2, 1, 0, 0, 1, data_format=fmt)
+        assert np.array_equal(p.numpy(), O.im2col(xi.astype(np.float32), 2, 2, 1, 2, 1, 0, 0, 1, data_format=fmt).astype(dtype))
+        back = D.op.col2im(D.op.im2col(arr(D, x), 2, 2, 2, 2, data_format=fmt), shape, 2, 2, 2, 2, fmt)
+        assert np.array_equal(back.numpy(), x)  # windows that tile the image exactly: every pixel once
+    # sums of integers in fp64 and their division by the window area; the int32 average truncates towards zero
+    sums = O.pool2d(xi.astype(np.float32), 2, 2, 2, 2, "avg", "valid", fmt).astype(np.float64) * 4.0
+    got = D.op.pool2d(arr(D, xi.astype(np.float64)), 2, 2, 2, 2, "avg", "valid", fmt).numpy()
+    assert np.array_equal(got, sums / 4.0)
+    goti = D.op.pool2d(arr(D, xi), 2, 2, 2, 2, "avg", "valid", fmt).numpy()
+    assert np.array_equal(goti, np.trunc(sums / 4.0).astype(np.int32))
+    dy = rng.randint(-5, 6, got.shape).astype(np.float64)
+    dx = D.op.pool2d_backward(arr(D, got), arr(D, dy), arr(D, xi.astype(np.float64)), 2, 2, 2, 2, "avg", "valid", fmt).numpy()
+    want_dx = O.pool2d_backward(got.astype(np.float32), dy.astype(np.float32), xi.astype(np.float32), 2, 2, 2, 2, "avg", "valid", fmt)
+    assert np.array_equal(dx, want_dx.astype(np.float64))
