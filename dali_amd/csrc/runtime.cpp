@@ -684,7 +684,9 @@ int dali_hip_launch(uint64_t hash, void** array_data, const int* offsets, const 
         int64_t cap = (int64_t)kWorkspacePartialBytes / (gx * per * (int64_t)(P.ws_elsize > 0 ? P.ws_elsize : 4));
         if (cap < 1) cap = 1;
         if (gy > cap) gy = cap;
-        if (gx > (int64_t)kWorkspaceCounters) return fail("dali_hip_launch: %lld column strips exceed the %d workspace counters", (long long)gx, kWorkspaceCounters);
+        // more strips than tickets: no split of the reduced rows (the kernel then finishes each strip by itself and
+        // touches neither tickets nor partial results)
+        if (gx > (int64_t)kWorkspaceCounters) gy = 1;
     } else if (P.grid_kind == DALI_HIP_GRID_ALL) {
         int64_t cap = (int64_t)kWorkspacePartialBytes / (int64_t)(P.ws_elsize > 0 ? P.ws_elsize : 4);
         if (gx > cap) gx = cap;

@@ -2627,7 +2627,60 @@ void run_specs(std::vector<DestSpec> specs) {
     st.plan_cache_stored++;
 }
 
+// A plain reduction of a buffer whose shape starves the one-pass kernels is done in two passes over a reshaped view:
+//  - few long rows (one workgroup per row leaves most of the device idle): [R, C] is read as [R * S, C / S], reduced
+//    along the rows, and the [R, S] partial results are reduced again;
+//  - the leading axis of a narrow matrix (a strip of 256 columns per workgroup is mostly empty): [R, C] is read as
+//    [R / k, k * C], reduced along the leading axis, and the [k, C] partial results are reduced again.
+// Sums come out in a different (still tree-shaped) order; maxima, minima and products of the same values are unchanged.
+bool try_two_stage_reduce(const DestSpec& spec) {
+    static const bool off = env_int("DALI_HIP_TWO_STAGE_REDUCE", 1) == 0;
+    if (off) return false;
+    auto e = spec.root.expression();
+    if (e->kind != Kind::AXIS_REDUCE) return false;
+    const std::string& red = e->name;
+    if (red != "reducers::sum" && red != "reducers::maximum" && red != "reducers::minimum" && red != "reducers::product") return false;
+    Array arg = e->args[0];
+    if (!arg.is_buffer() || arg.ndim() < 1 || arg.dtype() != e->dtype) return false;
+    const int C_last = arg.shape().back();
+    const int64_t n = numel_of(arg.shape());
+    if (n == 0 || C_last == 0) return false;
+    const int64_t rows = n / C_last;
+    if (arg.contiguous_memory()) {
+        // few long rows
+        if (rows >= 256 || C_last < (1 << 16)) return false;
+        int S = 1;
+        while (S * 2 * rows <= 2048 && C_last % (S * 2 * 4) == 0 && C_last / (S * 2) >= 8192) S *= 2;
+        if (S < 4) return false;
+        Array stage1 = op::axis_reduce(arg.reshape({(int)(rows * S), C_last / S}), red, {1}, false);
+        stage1.eval();
+        std::vector<int> partial_shape = e->shape;  // the leading dimensions of the argument, then the S partial results
+        partial_shape.push_back(S);
+        Array root2 = op::axis_reduce(stage1.reshape(partial_shape), red, {(int)partial_shape.size() - 1}, false);
+        if (root2.shape() != e->shape) return false;
+        run_specs({{spec.dest, spec.op, root2}});
+        return true;
+    }
+    // leading axis of a narrow row-major matrix: the argument is the transposed view [C, R] with strides [1, C]
+    if (arg.ndim() != 2) return false;
+    const int Cn = arg.shape()[0], R = arg.shape()[1];
+    const std::vector<int>& st = arg.strides();
+    if (st.size() != 2 || st[0] != 1 || st[1] != Cn || Cn > 512 || R < 4096) return false;
+    int k = 1;
+    while (k * 2 * (int64_t)Cn <= 4096 && R % (k * 2) == 0 && R / (k * 2) >= 64) k *= 2;
+    if (k < 2) return false;
+    Array matrix = arg.transpose();  // [R, C], contiguous
+    if (!matrix.contiguous_memory()) return false;
+    Array stage1 = op::axis_reduce(matrix.reshape({R / k, k * Cn}), red, {0}, false);
+    stage1.eval();
+    Array root2 = op::axis_reduce(stage1.reshape({k, Cn}), red, {0}, false);
+    if (root2.shape() != e->shape) return false;
+    run_specs({{spec.dest, spec.op, root2}});
+    return true;
+}
+
 void run_specs_planned(std::vector<DestSpec> specs) {
+    if (specs.size() == 1 && try_two_stage_reduce(specs[0])) return;
     // all-reduce roots are planned one by one
     if (specs.size() > 1) {
         bool any_all = false;

@@ -116,3 +116,39 @@ def test_c5_lstm_step_256x1024x1024(gpu, D, O):
     gf = pre.astype(np.float32)
     oc = O.binary("add", O.binary("eltmul", O.unary("sigmoid", gf[:, H:2 * H]), Cp), O.binary("eltmul", O.unary("sigmoid", gf[:, :H]), O.unary("tanh", gf[:, 3 * H:])))
     np.testing.assert_allclose(cn.numpy(), oc.reshape(B, H), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape,axis", [((64, 1 << 20), 1), ((3, 1 << 22), 1), ((2, 5, 1 << 18), 2), ((1 << 20, 64), 0), ((1 << 22, 8), 0),
+                                        ((65536, 100), 0), ((100, 100000), 1)])
+def test_reductions_of_starved_shapes_take_two_passes(gpu, D, rng, shape, axis):
+    """Few long rows and the leading axis of a narrow matrix: reshaped two-stage reductions, same results."""
+    x = rng.uniform(-1.0, 1.0, shape).astype(np.float32)
+    a = D.Array.from_numpy(x)
+    n_red = shape[axis]
+    for name, f in (("sum", np.sum), ("max", np.max), ("min", np.min)):
+        before = D.jit_stats()["kernels"]
+        got = getattr(D.op, name)(a, [axis]).numpy()
+        launched = D.jit_stats()["kernels"] - before
+        want = f(x.astype(np.float64), axis=axis)
+        assert got.shape == want.shape
+        if name == "sum":
+            bound = 1e-5 * np.abs(x.astype(np.float64)).sum(axis=axis) + 1e-6
+            assert (np.abs(got - want) <= bound).all()
+        else:
+            assert np.array_equal(got, want.astype(np.float32))
+        if shape not in ((100, 100000),):
+            assert launched == 2, (name, launched)
+    # accumulate into an existing destination: only the second pass applies the operator
+    acc = D.Array.from_numpy(np.ones(got.shape, np.float32))
+    acc += D.op.max(a, [axis])
+    assert np.array_equal(acc.numpy(), 1.0 + x.max(axis=axis))
+    assert n_red > 0
+
+
+def test_leading_axis_reduction_of_a_very_wide_matrix(gpu, D, rng):
+    """More 256-column strips than the workspace has tickets: the reduced rows are then not split across workgroups."""
+    x = rng.uniform(-1.0, 1.0, (3, (1 << 23) + 12)).astype(np.float32)
+    a = D.Array.from_numpy(x)
+    np.testing.assert_allclose(D.op.sum(a, [0]).numpy(), x.astype(np.float64).sum(axis=0), rtol=1e-6, atol=1e-6)
+    assert np.array_equal(D.op.max(a, [0]).numpy(), x.max(axis=0))
+    assert np.array_equal(D.op.argmax(a, 0).numpy(), x.argmax(axis=0).astype(np.int32))
