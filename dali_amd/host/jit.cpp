@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-19";
+const char* const kCodegenVersion = "dali-hip-codegen-20";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -1224,7 +1224,11 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
     // A 1024-thread row block fills a CU by itself unless it stays within 64 VGPRs; two resident
     // blocks let one row's loads overlap another row's arithmetic.
     static const int wpe = env_int("DALI_HIP_ROW_WAVES_PER_EU", -1);
-    rp.waves_per_eu = nph > 0 ? (wpe >= 0 ? wpe : (rp.BT == 1024 ? 8 : 0)) : 0;
+    // 1024-thread workgroups: two per CU (8 waves per SIMD, 64 registers per thread) as long as the cached row fits that
+    // budget; beyond ~44 cached values per thread the register cap would spill, so one workgroup per CU with twice the
+    // registers ([2048,50257] 362 -> 200 us, [1024,65536] 169 -> 115 us; [8192,32000] stays at two)
+    const int64_t cached_values = rp.cached ? (int64_t)std::max(1, n_full) * rp.EPT * rp.VEC * (max_el / 4) : 0;
+    rp.waves_per_eu = nph > 0 ? (wpe >= 0 ? wpe : (rp.BT == 1024 ? (cached_values > 44 ? 4 : 8) : 0)) : 0;
 
     // cross-phase register caching of expensive shared values
     rpn.first_body.assign(P.nodes.size(), -1);
