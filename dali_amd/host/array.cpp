@@ -349,6 +349,26 @@ Array Array::transpose() const {
 
 Array Array::transpose(const std::vector<int>& axes) const {
     DALI_ASSERT((int)axes.size() == ndim(), make_message("transpose needs ", ndim(), " axes (got ", axes.size(), ")."));
+    {
+        // An elementwise node over operands of its own shape (and literals) stays lazy: its transpose is the same node
+        // over the transposed operands, so a reduction along a leading axis of an expression still fuses with it.
+        auto le = expression();
+        if (le->kind == Kind::ELEMENTWISE && ndim() >= 2) {
+            bool movable = true;
+            for (const Array& x : le->args)
+                movable = movable && (x.shape() == le->shape || x.expression()->kind == Kind::SCALAR) &&
+                          (x.is_buffer() || x.expression()->kind == Kind::SCALAR || x.expression()->kind == Kind::ELEMENTWISE);
+            if (movable) {
+                std::vector<Array> targs;
+                for (const Array& x : le->args) targs.push_back(x.expression()->kind == Kind::SCALAR ? x : x.transpose(axes));
+                auto n = std::make_shared<Expr>(*le);
+                n->args = targs;
+                for (const Array& t : targs)
+                    if (t.expression()->kind != Kind::SCALAR) n->shape = t.shape();
+                return Array(n);
+            }
+        }
+    }
     auto e = as_buffer(*this).expression();
     auto st = normalized_strides();
     std::vector<int> nshape(ndim()), nstrides(ndim());
@@ -740,6 +760,18 @@ Array axis_reduce(const Array& a, const std::string& reducer_name, const std::ve
     if ((int)norm.size() == ndim) return all_reduce(a, reducer_name);
     int num_low = 0;
     for (int i = ndim - 1; i >= 0 && reduced[i]; --i) ++num_low;
+    if (num_low > 0 && num_low < (int)norm.size() && (reducer_name == "reducers::sum" || reducer_name == "reducers::maximum" ||
+                                                      reducer_name == "reducers::minimum" || reducer_name == "reducers::product")) {
+        // Some reduced axes trail, others do not (per-channel sums of [N, C, H*W]): the trailing ones are reduced where they
+        // lie, along memory, and only the much smaller result takes the transposed route for the others. The reference
+        // moves every reduced axis to the back first (reducer_operation.cpp:595-679), i.e. a strided walk over everything.
+        std::vector<int> tail_axes, rest;
+        for (int ax : norm) (ax >= ndim - num_low ? tail_axes : rest).push_back(ax);
+        Array out = axis_reduce(axis_reduce(a, reducer_name, tail_axes, false), reducer_name, rest, false);
+        if (keepdims)
+            for (int ax : norm) out = out.expand_dims(ax);
+        return out;
+    }
     Array res = a;
     if (num_low != (int)norm.size()) {
         std::vector<int> order;

@@ -2426,6 +2426,8 @@ void run_group(std::vector<DestSpec> specs);
 
 // Evaluate one (dest, op, root) after cleaning; splits until a kernel shape fits.
 void run_specs_planned(std::vector<DestSpec> specs);
+bool is_transposed_matrix(const Expr* e);
+void run_transpose_into(const Array& dest, const Array& src);
 
 // ------------------------------------------------------------------ plan cache
 // Planning an expression (classification, kernel parameters, the structural signature and its hash) costs more
@@ -2723,6 +2725,41 @@ void run_specs_planned(std::vector<DestSpec> specs) {
         for (auto& s : specs) has_red = has_red || has_kind(s.root, [](Kind k) { return is_reduce(k); });
         if (!has_red) {
             if (try_flat(specs)) return;
+            if (specs.size() == 1) {
+                // Large transposed matrices among the operands are first written out along memory by a tiled transpose
+                // (both its reads and its writes are coalesced); a map that walked them in place would fetch a cache line
+                // per element ([16384,4096]: x.T + 1 took 721 us, a transposed copy takes 90).
+                DestSpec& sp = specs[0];
+                auto re = sp.root.expression();
+                if (re->kind == Kind::ELEMENTWISE && re->name == "functor::identity" && sp.op == OPERATOR_T_EQL && sp.dest.contiguous_memory() &&
+                    is_transposed_matrix(re->args[0].expression().get()) && re->args[0].dtype() == sp.dest.dtype() &&
+                    re->args[0].shape() == sp.dest.shape()) {
+                    run_transpose_into(sp.dest, re->args[0]);
+                    return;
+                }
+                Array found;
+                std::function<bool(const Array&)> find = [&](const Array& a) {
+                    auto ae = a.expression();
+                    if (ae->kind == Kind::BUFFER) {
+                        if (is_transposed_matrix(ae.get())) {
+                            found = a;
+                            return true;
+                        }
+                        return false;
+                    }
+                    if (ae->kind == Kind::SCALAR) return false;
+                    for (const Array& x : ae->args)
+                        if (find(x)) return true;
+                    return false;
+                };
+                if (find(sp.root)) {
+                    Array copy(found.shape(), found.dtype());
+                    run_transpose_into(copy, found);
+                    std::map<const Expr*, Array> memo;
+                    sp.root = substitute(sp.root, found.expression().get(), copy, memo);
+                    continue;
+                }
+            }
             Domain dom = domain_of(specs[0].dest.shape());
             if (specs[0].dest.ndim() <= 1 && has_kind(specs[0].root, [](Kind k) { return k == Kind::GATHER_FROM_ROWS; })) {
                 // one gathered element per row: a single-column domain
@@ -2779,6 +2816,32 @@ void run_specs_planned(std::vector<DestSpec> specs) {
             if (find_first_reduce(s.root, &first, seen)) break;
         Domain dom = domain_of(first.expression()->args[0].shape());
         if (specs.size() == 1 && try_col(specs[0])) return;
+        if (specs.size() == 1) {
+            // A reduction along the leading axis of row-major operands under further arithmetic (mean = sum / count, a
+            // normalisation by the column maxima): the row kernel would walk the operands against their layout, so
+            // the reduction goes through the column kernel on its own and the rest reads its small result.
+            Array inner;
+            std::set<const Expr*> seen_inner;
+            if (find_innermost_reduce(specs[0].root, &inner, seen_inner) && inner.expression().get() != specs[0].root.expression().get() &&
+                (inner.expression()->kind == Kind::AXIS_REDUCE || inner.expression()->kind == Kind::ARG_AXIS_REDUCE)) {
+                Array red_arg = inner.expression()->args[0];
+                std::set<const Expr*> seen_col;
+                bool has_layout = false;  // at least one genuinely transposed matrix among the operands
+                std::function<void(const Array&)> scan = [&](const Array& a) {
+                    auto ae = a.expression();
+                    if (ae->kind == Kind::BUFFER && ae->shape.size() == 2 && ae->shape[0] > 1 && ae->shape[1] > 1 && strides_of(ae.get())[0] == 1) has_layout = true;
+                    if (ae->kind != Kind::BUFFER && ae->kind != Kind::SCALAR)
+                        for (const Array& x : ae->args) scan(x);
+                };
+                scan(red_arg);
+                if (red_arg.ndim() == 2 && red_arg.shape()[0] > 1 && has_layout && col_eligible(red_arg, red_arg.shape()[0], red_arg.shape()[1], seen_col)) {
+                    Array buf = materialize(inner);
+                    std::map<const Expr*, Array> memo;
+                    specs[0].root = substitute(specs[0].root, inner.expression().get(), buf, memo);
+                    continue;
+                }
+            }
+        }
         if (try_row(specs, dom)) return;
         if (specs.size() > 1) {
             for (auto& s : specs) run_specs({s});
@@ -3734,6 +3797,48 @@ Array conv2d_nhwc_direct(const Array& x_in, const Array& filters_in, int pad_top
         });
     }
     return out;
+}
+
+// ------------------------------------------------------------------ tiled transpose
+// A 2-D view whose first index runs along memory (strides [1, ld]: the transpose of a row-major matrix) and that is
+// large enough for the layout to matter.
+bool is_transposed_matrix(const Expr* e) {
+    if (e->kind != Kind::BUFFER || e->shape.size() != 2 || e->strides.size() != 2) return false;
+    return e->strides[0] == 1 && e->strides[1] >= e->shape[0] && e->shape[0] >= 32 && e->shape[1] >= 32 && (int64_t)e->shape[0] * e->shape[1] >= (1 << 16);
+}
+
+// dest (contiguous [R, C]) = src (a transposed matrix view [R, C]): 64x64 tiles go through LDS, read along the source's
+// memory rows and written along the destination's.
+void run_transpose_into(const Array& dest, const Array& src) {
+    auto se = src.expression();
+    const int R = se->shape[0], Cn = se->shape[1], ld = se->strides[1];
+    Program P;
+    P.arrays.push_back(manual_arg(dest, Cls::FULL, true, 1, {R * Cn}, {}));
+    P.arrays.push_back(manual_arg(src, Cls::FULL, false, 2, {R, Cn}, {1, ld}));
+    GeomInts G;
+    G.add("R", R);
+    G.add("CN", Cn);
+    G.add("LD", ld);
+    G.add_div("TILES_R", (R + 63) / 64);
+    const int64_t tiles = (int64_t)((R + 63) / 64) * ((Cn + 63) / 64);
+    std::ostringstream sig;
+    sig << "transpose|" << (int)se->dtype;
+    launch_special("transpose", sig.str(), P, tiles, G, [&](std::ostringstream& ss) {
+        ss << "  __shared__ T tile[64][65];\n";
+        ss << "  T* out = (T*)A.p[0];\n  const T* in = (const T*)A.p[1];\n";
+        ss << "  const unsigned total = (unsigned)TILES_R * (unsigned)((CN + 63) / 64);\n";
+        ss << "  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;\n";
+        ss << "  for (unsigned b = blockIdx.x; b < total; b += gridDim.x) {\n";
+        ss << "    " << divmod("tc", "tr", "b", "TILES_R") << "\n";
+        ss << "    const int r0 = tr * 64, c0 = (int)tc * 64;\n";
+        ss << "    // the source's memory rows are the view's columns: element (r, c) lives at c * LD + r\n";
+        ss << "    _Pragma(\"unroll\") for (int k = 0; k < 16; ++k) {\n      const int c = c0 + ty + 4 * k, r = r0 + tx;\n";
+        ss << "      if (c < CN && r < R) tile[ty + 4 * k][tx] = in[(long)c * LD + r];\n    }\n";
+        ss << "    __syncthreads();\n";
+        ss << "    _Pragma(\"unroll\") for (int k = 0; k < 16; ++k) {\n      const int r = r0 + ty + 4 * k, c = c0 + tx;\n";
+        ss << "      if (r < R && c < CN) out[(long)r * CN + c] = tile[tx][ty + 4 * k];\n    }\n";
+        ss << "    __syncthreads();\n  }\n}\n";
+    });
 }
 
 // ----------------------------------------------------------- index-valued fills
