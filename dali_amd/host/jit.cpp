@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-20";
+const char* const kCodegenVersion = "dali-hip-codegen-21";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -1647,7 +1647,33 @@ struct ColLeaf {
     int array;
 };
 
-bool col_eligible(const Array& a, int64_t K, int64_t X, std::set<const Expr*>& seen) {
+// Kept axes [0, split) of a [kept..., reduced] view must merge into one batch axis and kept axes
+// [split, n_kept) into one unit-stride axis; the reduced (last) axis may have any stride.
+bool col_buffer_layout(const Expr* e, const std::vector<int>& shape, int split, int64_t* batch_stride) {
+    auto st = strides_of(e);
+    const int nk = (int)shape.size() - 1;
+    int64_t expect = 1;
+    for (int d = nk - 1; d >= split; --d) {
+        if (shape[d] == 1) continue;
+        if (st[d] != expect) return false;
+        expect *= shape[d];
+    }
+    int64_t bs = 0;
+    expect = -1;
+    for (int d = split - 1; d >= 0; --d) {
+        if (shape[d] == 1) continue;
+        if (expect < 0) {
+            bs = st[d];
+        } else if (st[d] != expect) {
+            return false;
+        }
+        expect = (int64_t)st[d] * shape[d];
+    }
+    if (batch_stride) *batch_stride = bs;
+    return true;
+}
+
+bool col_eligible(const Array& a, const std::vector<int>& shape, int split, std::set<const Expr*>& seen) {
     auto e = a.expression();
     if (seen.count(e.get())) return true;
     seen.insert(e.get());
@@ -1655,24 +1681,34 @@ bool col_eligible(const Array& a, int64_t K, int64_t X, std::set<const Expr*>& s
         case Kind::SCALAR: return true;
         case Kind::BUFFER: {
             if (numel_of(e->shape) == 1) return true;
-            if (e->shape.size() != 2 || e->shape[0] != K || e->shape[1] != X) return false;
-            auto st = strides_of(e.get());
-            return st[0] == 1 || K == 1;
+            if (e->shape != shape) return false;
+            return col_buffer_layout(e.get(), shape, split, nullptr);
         }
         case Kind::ELEMENTWISE:
             for (const Array& x : e->args) {
-                if (numel_of(x.shape()) != K * X && numel_of(x.shape()) != 1) return false;
-                if (!col_eligible(x, K, X, seen)) return false;
+                if (numel_of(x.shape()) != numel_of(shape) && numel_of(x.shape()) != 1) return false;
+                if (!col_eligible(x, shape, split, seen)) return false;
             }
             return true;
         case Kind::BROADCAST:
-            return numel_of(e->args[0].shape()) == 1 && col_eligible(e->args[0], K, X, seen);
+            return numel_of(e->args[0].shape()) == 1 && col_eligible(e->args[0], shape, split, seen);
         default: return false;
     }
 }
 
+// The first split of the kept axes into [batch..., unit-stride run...] that every operand of a
+// [kept..., reduced] argument fits (0: no batch axis); -1 when there is none.
+int col_split_of(const Array& arg) {
+    const int nk = arg.ndim() - 1;
+    for (int sp = 0; sp < nk; ++sp) {
+        std::set<const Expr*> seen;
+        if (col_eligible(arg, arg.shape(), sp, seen)) return sp;
+    }
+    return -1;
+}
+
 std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATOR_T op, const IvLayout& L, int VEC, int UNR, int TAIL, int RG, bool NT,
-                           int IL, const std::string& kname) {
+                           int IL, bool BATCHED, const std::string& kname) {
     const std::string ld = NT ? "dali_load_nt<" : "dali_load<";
     const PNode& red = P.nodes[red_id];
     const bool ARG = red.kind == Kind::ARG_AXIS_REDUCE;  // carries (value, row index); ties keep the lower index
@@ -1697,13 +1733,22 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     ss << "  const int lane = threadIdx.x % TPP, wave = threadIdx.x / TPP;\n";
     ss << "  const long k0 = ((long)blockIdx.x * TPP + lane) * VEC;\n";
     ss << "  const bool k_ok = k0 < K;\n";
+    // BATCHED: the kept index runs over [batch, unit-stride run]; a lane's VEC kept elements lie in one run, and
+    // the second shape entry holds the run length followed by the batch stride of every full operand
+    if (BATCHED) ss << "  const long k_run = A.iv[" << L.shape_pos[1] << "], k_batch = k0 / k_run, k_in = k0 - k_batch * k_run;\n";
+    int full_seen = 0;
     for (size_t i = 0; i < P.arrays.size(); ++i) {
         const ArrayArg& a = P.arrays[i];
         std::string ty = ctype(a.buf->dtype);
         if (a.is_dest) {
             ss << "  " << ty << "* q" << i << " = (" << ty << "*)A.p[" << i << "];\n  const long ds" << i << " = " << (a.strided ? "A.iv[" + std::to_string(L.stride_pos[i]) + "]" : "1") << ";\n";
         } else if (a.cls == Cls::FULL) {
-            ss << "  const " << ty << "* q" << i << " = (const " << ty << "*)A.p[" << i << "] + (k_ok ? k0 : 0);\n";
+            if (BATCHED)
+                ss << "  const " << ty << "* q" << i << " = (const " << ty << "*)A.p[" << i << "] + (k_ok ? k_batch * (long)A.iv[" << L.shape_pos[1] + 1 + full_seen
+                   << "] + k_in : 0);\n";
+            else
+                ss << "  const " << ty << "* q" << i << " = (const " << ty << "*)A.p[" << i << "] + (k_ok ? k0 : 0);\n";
+            ++full_seen;
             ss << "  const long ld" << i << " = A.iv[" << L.stride_pos[i] + 1 << "];\n";
         } else {
             ss << "  const " << ty << " sl" << i << " = ((const " << ty << "*)A.p[" << i << "])[0];\n";
@@ -1844,11 +1889,17 @@ bool try_col(const DestSpec& spec) {
     if (re->kind != Kind::AXIS_REDUCE && re->kind != Kind::ARG_AXIS_REDUCE) return false;
     const bool is_arg = re->kind == Kind::ARG_AXIS_REDUCE;
     Array arg = re->args[0];
-    if (arg.ndim() != 2) return false;
-    int64_t K = arg.shape()[0], X = arg.shape()[1];
-    if (K <= 1 || X == 0) return false;
-    std::set<const Expr*> seen;
-    if (!col_eligible(arg, K, X, seen)) return false;
+    if (arg.ndim() < 2) return false;
+    const std::vector<int> arg_shape = arg.shape();
+    const int nk = arg.ndim() - 1;
+    int64_t X = arg_shape[nk], K = numel_of(arg_shape) / std::max<int64_t>(1, X);
+    if (K <= 1 || X == 0 || K * X >= ((int64_t)1 << 31)) return false;
+    // the kept axes [batch..., unit-stride run...]: the first split every operand fits (0: no batch axis)
+    const int split = col_split_of(arg);
+    if (split < 0) return false;
+    int64_t k_run = 1;
+    for (int d = split; d < nk; ++d) k_run *= arg_shape[d];
+    const bool BATCHED = k_run != K;
     if (numel_of(spec.dest.shape()) != K) return false;
     Domain dom;
     dom.R = K;  // ROW-class destination has K entries
@@ -1858,12 +1909,14 @@ bool try_col(const DestSpec& spec) {
     if (dest_array < 0) return false;
     int red_id = add_node(P, root);
     // classify the argument tree: [K, X] buffers are FULL with the kept stride in strides[0]
+    std::vector<int> batch_strides;  // one per FULL operand, in argument order
     std::function<bool(int)> cls = [&](int id) -> bool {
         PNode& nd = P.nodes[id];
         if (nd.cls_set) return true;
         nd.cls_set = true;
         if (nd.kind == Kind::SCALAR) { nd.cls = Cls::SCAL; return true; }
         if (nd.kind == Kind::BUFFER) {
+            int64_t bs = 0;
             ArrayArg a;
             a.buf = nd.src;
             if (numel_of(nd.shape) == 1) {
@@ -1873,13 +1926,14 @@ bool try_col(const DestSpec& spec) {
                 nd.cls = Cls::SCAL;
             } else {
                 auto st = strides_of(nd.src.get());
+                col_buffer_layout(nd.src.get(), arg_shape, split, &bs);
                 a.cls = Cls::FULL;
                 a.nd = 2;
                 a.sizes = {(int)K, (int)X};
                 a.strided = true;
-                a.strides = {st[0], st[1]};
-                a.row_stride = st[0];
-                a.col_stride = st[1];
+                a.strides = {nk == 1 ? st[0] : 1, st[nk]};
+                a.row_stride = a.strides[0];
+                a.col_stride = st[nk];
                 nd.cls = Cls::FULL;
             }
             std::string key = array_key(nd.src.get(), a.cls, false);
@@ -1889,6 +1943,7 @@ bool try_col(const DestSpec& spec) {
                     return true;
                 }
             P.arrays.push_back(a);
+            if (a.cls == Cls::FULL) batch_strides.push_back((int)bs);
             P.nodes[id].array = (int)P.arrays.size() - 1;
             return true;
         }
@@ -1902,9 +1957,11 @@ bool try_col(const DestSpec& spec) {
     P.nodes[red_id].cls_set = true;
     if (!cls(P.nodes[red_id].args[0])) return false;
     count_uses(P, {red_id});
-    bool vec = K % 4 == 0;
+    bool vec = K % 4 == 0 && k_run % 4 == 0;
     for (const ArrayArg& a : P.arrays)
         if (!a.is_dest && a.cls == Cls::FULL && (a.buf->offset % 4 != 0 || a.col_stride % 4 != 0)) vec = false;
+    for (int bs : batch_strides)
+        if (bs % 4 != 0) vec = false;
     int VEC = vec ? 4 : 1;
     static const int IL = env_int("DALI_HIP_COL_INTERLEAVE", 2);
     static const int rg_env = env_int("DALI_HIP_COL_RG", 0), tail_env = env_int("DALI_HIP_COL_TAIL", 16);
@@ -1925,11 +1982,12 @@ bool try_col(const DestSpec& spec) {
     std::ostringstream params;
     const bool NT = K * X * (int64_t)size_of_dtype(arg.dtype()) >= ((int64_t)64 << 20);
     static const int maxy_env = env_int("DALI_HIP_COL_MAXY", 256);
-    params << VEC << "," << UNR << "," << TAIL << "," << RG << "," << NT << "," << IL;
+    params << VEC << "," << UNR << "," << TAIL << "," << RG << "," << NT << "," << IL << "," << BATCHED;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("col", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& Kp = specs_cache[h];
     std::vector<int> shape_ndims = {2};
+    if (BATCHED) shape_ndims.push_back(1 + (int)batch_strides.size());
     IvLayout L = layout_iv(P, shape_ndims);
     if (!Kp) {
         Kp = std::make_shared<KernelSpec>();
@@ -1949,7 +2007,11 @@ bool try_col(const DestSpec& spec) {
         Kp->plan.ws_elsize = size_of_dtype(arg.dtype()) + (is_arg ? 4 : 0);  // a partial is a value, plus its index
     }
     std::vector<std::vector<int>> shapes = {{(int)K, (int)X}};
-    load_and_launch(*Kp, [&]() { return gen_col_kernel(P, red_id, dest_array, spec.op, L, VEC, UNR, TAIL, RG, NT, IL, Kp->name); }, P, shapes);
+    if (BATCHED) {
+        shapes.push_back({(int)k_run});
+        shapes.back().insert(shapes.back().end(), batch_strides.begin(), batch_strides.end());
+    }
+    load_and_launch(*Kp, [&]() { return gen_col_kernel(P, red_id, dest_array, spec.op, L, VEC, UNR, TAIL, RG, NT, IL, BATCHED, Kp->name); }, P, shapes);
     return true;
 }
 
@@ -2825,16 +2887,17 @@ void run_specs_planned(std::vector<DestSpec> specs) {
             if (find_innermost_reduce(specs[0].root, &inner, seen_inner) && inner.expression().get() != specs[0].root.expression().get() &&
                 (inner.expression()->kind == Kind::AXIS_REDUCE || inner.expression()->kind == Kind::ARG_AXIS_REDUCE)) {
                 Array red_arg = inner.expression()->args[0];
-                std::set<const Expr*> seen_col;
-                bool has_layout = false;  // at least one genuinely transposed matrix among the operands
+                bool has_layout = false;  // at least one operand whose reduced axis does not run along memory
                 std::function<void(const Array&)> scan = [&](const Array& a) {
                     auto ae = a.expression();
-                    if (ae->kind == Kind::BUFFER && ae->shape.size() == 2 && ae->shape[0] > 1 && ae->shape[1] > 1 && strides_of(ae.get())[0] == 1) has_layout = true;
+                    if (ae->kind == Kind::BUFFER && ae->shape.size() >= 2 && ae->shape.back() > 1 && numel_of(ae->shape) > ae->shape.back() &&
+                        strides_of(ae.get()).back() != 1)
+                        has_layout = true;
                     if (ae->kind != Kind::BUFFER && ae->kind != Kind::SCALAR)
                         for (const Array& x : ae->args) scan(x);
                 };
                 scan(red_arg);
-                if (red_arg.ndim() == 2 && red_arg.shape()[0] > 1 && has_layout && col_eligible(red_arg, red_arg.shape()[0], red_arg.shape()[1], seen_col)) {
+                if (red_arg.ndim() >= 2 && numel_of(red_arg.shape()) > red_arg.shape().back() && has_layout && col_split_of(red_arg) >= 0) {
                     Array buf = materialize(inner);
                     std::map<const Expr*, Array> memo;
                     specs[0].root = substitute(specs[0].root, inner.expression().get(), buf, memo);

@@ -169,7 +169,11 @@ def test_planner_splits_what_cannot_fuse(D, rng):
     assert D.last_kernel_kinds().split(",").count("all") == 2 and n == 3
     x3 = D.Array.from_numpy(rng.randn(3, 4, 5).astype(np.float32))
     D.generate_only([op.sum(x3, [1])], compile=True)
-    assert D.last_kernel_kinds() == "generic,row"  # middle axis: strided copy, then a trailing-axis reduction
+    assert D.last_kernel_kinds() == "col"  # middle axis: the column kernel over [batch, unit-stride run] kept axes
+    assert "k_batch * (long)A.iv[" in D.last_source()
+    x4 = D.Array.from_numpy(rng.randn(2, 3, 4, 5).astype(np.float32))
+    D.generate_only([op.sum(x4, [0, 2])], compile=True)
+    assert D.last_kernel_kinds() == "generic,row,row"  # kept axes on both sides of a reduced one: strided copy first
     D.generate_only([op.mean(m)], compile=True)
     assert D.last_kernel_kinds() == "all"  # the division by the count is folded into the last block
 

@@ -435,6 +435,39 @@ def test_axis_and_all_reductions_match_oracle(gpu, D, O, rng, shape):
     assert abs(float(op.mean(X).numpy()) - float(O.mean_all(x))) <= float(sum_tol(x)) / x.size + 1e-7
 
 
+@pytest.mark.parametrize("shape", [(3, 4, 5), (2, 7, 64), (5, 300, 36), (17, 33, 130), (4, 1000, 256), (2, 3, 5, 8), (6, 2, 70001), (1, 9, 12), (9, 1, 12)])
+def test_middle_axis_reductions_use_the_batched_column_kernel(gpu, D, O, rng, shape):
+    """A reduced axis between kept ones: op::axis_reduce presents [kept..., reduced] with the unit stride on the last
+    kept axis (reducer_operation.cpp:642-655); the kept index runs over [batch, unit-stride run]."""
+    op = D.op
+    x = rng.randn(*shape).astype(np.float32)
+    X = arr(D, x)
+    axis = 1
+    got = op.sum(X, [axis]).numpy()
+    if shape[0] > 1 and shape[1] > 1:
+        assert D.last_kernel_kinds() == "col"
+    assert np.all(np.abs(got - x.astype(np.float64).sum(axis)) <= sum_tol(x, axis))
+    assert np.array_equal(op.max(X, [axis]).numpy(), x.max(axis))
+    assert np.array_equal(op.min(X, [axis], True).numpy(), x.min(axis, keepdims=True))
+    # ties: first index along the reduced axis, per (batch, column); the reference SWAPS the reduced axis with the
+    # last one (reducer_operation.cpp:699-707), which differs from numpy's order of the kept axes beyond three dims
+    t = rng.randint(0, 3, size=shape).astype(np.float32)
+    moved = np.swapaxes(t, axis, -1)
+    want = O.arg_axis_reduce(O.MAX, np.ascontiguousarray(moved).reshape(-1, shape[axis]), 1).reshape(moved.shape[:-1])
+    assert np.array_equal(op.argmax(arr(D, t), axis).numpy(), want)
+    assert np.array_equal(op.argmin(arr(D, t), axis).numpy(), np.argmin(moved, -1))
+    # under an epilogue and over a fused argument
+    y = rng.randn(*shape).astype(np.float32)
+    got = op.mean(X * arr(D, y) + 1.0, [axis]).numpy()
+    want = (x.astype(np.float64) * y + 1.0).mean(axis)
+    assert np.all(np.abs(got - want) <= sum_tol(x * y + 1.0, axis) / shape[axis] + 1e-6)
+    # a batch stride that is not the dense one: a slice of a larger array along the leading axis and the run
+    if shape[0] > 1 and len(shape) == 3 and shape[2] >= 8:
+        v, nv = X[::2, :, 4:], x[::2, :, 4:]
+        assert np.all(np.abs(op.sum(v, [1]).numpy() - nv.astype(np.float64).sum(1)) <= sum_tol(nv, 1))
+        assert np.array_equal(op.max(v, [1]).numpy(), nv.max(1))
+
+
 def test_argmax_ties_and_sentinels_are_bit_exact(gpu, D, O, rng):
     op = D.op
     # few distinct values -> many ties; widths straddle the one-wave / multi-wave / streaming row layouts
