@@ -53,6 +53,50 @@ DI void dali_store_nt(T* p, const dali_vec<T, N>& v) {
     }
 }
 
+// The same accesses for addresses aligned to the element only (rows whose length is not a multiple of the
+// vector: every row starts at another offset within 16 bytes). Global memory takes multi-dword accesses at any
+// dword address, so these are single instructions too.
+template <typename T, int N>
+struct alignas(sizeof(T)) dali_vecu { T v[N]; };
+template <typename T, int N>
+DI dali_vec<T, N> dali_loadu(const T* p) {
+    const dali_vecu<T, N> u = *reinterpret_cast<const dali_vecu<T, N>*>(p);
+    dali_vec<T, N> r;
+    __builtin_memcpy(&r, &u, sizeof(r));
+    return r;
+}
+template <typename T, int N>
+DI void dali_storeu(T* p, const dali_vec<T, N>& v) {
+    dali_vecu<T, N> u;
+    __builtin_memcpy(&u, &v, sizeof(u));
+    *reinterpret_cast<dali_vecu<T, N>*>(p) = u;
+}
+template <typename T, int N>
+DI dali_vec<T, N> dali_loadu_nt(const T* p) {
+    dali_vec<T, N> r;
+    if constexpr (sizeof(T) * N == 16) {
+        typedef int i4 __attribute__((ext_vector_type(4)));
+        typedef i4 i4u __attribute__((aligned(4)));
+        i4 raw = __builtin_nontemporal_load(reinterpret_cast<const i4u*>(p));
+        __builtin_memcpy(&r, &raw, 16);
+    } else {
+        r = dali_loadu<T, N>(p);
+    }
+    return r;
+}
+template <typename T, int N>
+DI void dali_storeu_nt(T* p, const dali_vec<T, N>& v) {
+    if constexpr (sizeof(T) * N == 16) {
+        typedef int i4 __attribute__((ext_vector_type(4)));
+        typedef i4 i4u __attribute__((aligned(4)));
+        i4 raw;
+        __builtin_memcpy(&raw, &v, 16);
+        __builtin_nontemporal_store(raw, reinterpret_cast<i4u*>(p));
+    } else {
+        dali_storeu<T, N>(p, v);
+    }
+}
+
 // ------------------------------------------------------------ libm dispatch
 DI float  m_exp(float a)  { return expf(a); }
 DI double m_exp(double a) { return exp(a); }

@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-21";
+const char* const kCodegenVersion = "dali-hip-codegen-23";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -489,6 +489,8 @@ struct RowParams {
     bool nt_loads = false;   // inputs are streamed once: bypass cache allocation
     bool nt_stores = true;   // outputs are not re-read by this kernel: streaming stores
     bool exact = false;      // register-cached rows: C == TPR * EPT * VEC, the chunk guards fall away
+    bool ragged = false;     // rows not aligned to the vector: element-aligned vector accesses
+    bool tail = false;       // ragged, and C is no multiple of VEC: the rest of a row is handled one element to a thread
 };
 
 int env_int(const char* name, int fallback) {
@@ -784,9 +786,14 @@ void emit_row_prologue(std::ostringstream& ss, const Program& P, const IvLayout&
 }
 
 // load of FULL leaf `i` for chunk `ch` into dst (dst is "x<i>[e]" or "x<i>")
-void emit_leaf_load(std::ostringstream& ss, const ArrayArg& a, int i, int VEC, const std::string& dst, const std::string& indent, bool nontemporal) {
+void emit_leaf_load(std::ostringstream& ss, const ArrayArg& a, int i, int VEC, const std::string& dst, const std::string& indent, bool nontemporal,
+                    bool ragged = false) {
     std::string t = ctype(a.buf->dtype);
-    if (VEC > 1) {
+    if (VEC > 1 && ragged) {
+        ss << indent << "{ const dali_vec<" << t << ", " << VEC << "> tmp = " << (nontemporal ? "dali_loadu_nt<" : "dali_loadu<") << t << ", " << VEC << ">(q" << i
+           << " + (long)ch * " << VEC << ");\n";
+        ss << indent << "  _Pragma(\"unroll\") for (int j = 0; j < " << VEC << "; ++j) " << dst << "[j] = tmp.v[j]; }\n";
+    } else if (VEC > 1) {
         ss << indent << "{ dali_vec<" << t << ", " << VEC << "> tmp = " << (nontemporal ? "dali_load_nt<" : "dali_load<") << t << ", " << VEC << ">(q" << i
            << " + (long)ch * " << VEC << ");\n";
         ss << indent << "  _Pragma(\"unroll\") for (int j = 0; j < " << VEC << "; ++j) " << dst << "[j] = tmp.v[j]; }\n";
@@ -816,6 +823,10 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
         ss << "  const bool row_ok = row < R;\n  if (!row_ok) row = R - 1;\n";
     ss << "  const int CH = (int)(C / VEC); (void)CH;\n";
     emit_row_prologue(ss, P, L);
+    // ragged rows: the C % VEC elements past the last whole vector go one to a thread, through the same bodies
+    // (slot EPT of the register cache, j = 0)
+    const bool tail = rp.ragged && rp.tail;
+    if (tail) ss << "  const bool tail_on = tr < (int)(C - (long)CH * VEC);\n  const int tail_col = CH * VEC + tr;\n";
     // register-cached rows whose length fills every chunk need no chunk guard
     const std::string chunk_guard = rp.cached && rp.exact ? "    {\n" : "    if (ch < CH) {\n";
 
@@ -826,14 +837,29 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
     // is each leaf referenced? (an array may only be a gather source)
     if (rp.cached) {
         for (int i : full_leaves) {
-            ss << "  " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[EPT][VEC];\n";
+            ss << "  " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[EPT + " << (tail ? 1 : 0) << "][VEC];\n";
         }
         ss << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n" << chunk_guard;
-        for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i) + "[e]", "      ", rp.nt_loads);
+        for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i) + "[e]", "      ", rp.nt_loads, rp.ragged);
         ss << "    }\n  }\n";
+        if (tail) {
+            ss << "  if (tail_on) {\n";
+            for (int i : full_leaves) ss << "    x" << i << "[EPT][0] = q" << i << "[tail_col];\n";
+            ss << "  }\n";
+        }
         for (size_t id = 0; id < P.nodes.size(); ++id)
-            if (P.nodes[id].kept) ss << "  " << ctype(P.nodes[id].dtype) << " t" << id << "[EPT][VEC];\n";
+            if (P.nodes[id].kept) ss << "  " << ctype(P.nodes[id].dtype) << " t" << id << "[EPT + " << (tail ? 1 : 0) << "][VEC];\n";
     }
+    // opens the tail element's scope: the names a body refers to (e, j, col, x<i>) stand for that one element
+    auto open_tail = [&](std::ostringstream& o, const std::string& cond) {
+        o << "  if (" << cond << ") {\n";
+        if (rp.cached) {
+            o << "    constexpr int e = EPT; (void)e;\n";
+        } else {
+            for (int i : full_leaves) o << "    " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n    x" << i << "[0] = q" << i << "[tail_col];\n";
+        }
+        o << "    constexpr int j = 0; (void)j;\n    const int col = tail_col; (void)col;\n";
+    };
     auto open_loop = [&](std::ostringstream& o) {
         if (rp.cached) {
             o << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n" << chunk_guard;
@@ -841,7 +867,7 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
             o << "  for (int ch = tr; ch < CH; ch += TPR) {\n    {\n";
             for (int i : full_leaves) {
                 o << "      " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n";
-                emit_leaf_load(o, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", rp.nt_loads);
+                emit_leaf_load(o, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", rp.nt_loads, rp.ragged);
             }
         }
     };
@@ -900,6 +926,12 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
             o << be.stmts.str();
             for (auto& u : updates) o << "        " << u << "\n";
             o << "      }\n    }\n  }\n";
+            if (tail) {
+                open_tail(o, "tail_on");
+                o << be.stmts.str();
+                for (auto& u : updates) o << "    " << u << "\n";
+                o << "  }\n";
+            }
         };
         emit_with_division_plan(ss, emit_phase_loop);
         for (int id : reds) {
@@ -940,7 +972,11 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
                 const ArrayArg& d = P.arrays[o.array];
                 std::string t = ctype(d.buf->dtype);
                 std::string ov = "o" + std::to_string(o.array);
-                if (rp.VEC > 1) {
+                if (rp.VEC > 1 && rp.ragged) {
+                    pre << "        dali_vec<" << t << ", VEC> " << ov << ";\n";
+                    if (o.op != OPERATOR_T_EQL) pre << "        " << ov << " = dali_loadu<" << t << ", VEC>(q" << o.array << " + (long)ch * VEC);\n";
+                    post << "        " << (rp.nt_stores ? "dali_storeu_nt<" : "dali_storeu<") << t << ", VEC>(q" << o.array << " + (long)ch * VEC, " << ov << ");\n";
+                } else if (rp.VEC > 1) {
                     pre << "        dali_vec<" << t << ", VEC> " << ov << ";\n";
                     if (o.op != OPERATOR_T_EQL) pre << "        " << ov << " = dali_load<" << t << ", VEC>(q" << o.array << " + (long)ch * VEC);\n";
                     post << "        " << (rp.nt_stores ? "dali_store_nt<" : "dali_store<") << t << ", VEC>(q" << o.array << " + (long)ch * VEC, " << ov << ");\n";
@@ -958,6 +994,17 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
             os << be.stmts.str() << body.str();
             os << "        }\n" << post.str();
             os << "      }\n    }\n  }\n";
+            if (tail) {
+                open_tail(os, "tail_on && row_ok");
+                os << be.stmts.str();
+                for (const Output& o : rpn.outputs) {
+                    if (o.cls != Cls::FULL) continue;
+                    std::string t = ctype(P.arrays[o.array].buf->dtype);
+                    const std::string dp = "q" + std::to_string(o.array) + "[tail_col]";
+                    os << "    " << dp << " = " << op_combine(o.op, dp, "(" + t + ")(" + be.value(o.root) + ")") << ";\n";
+                }
+                os << "  }\n";
+            }
         };
         emit_with_division_plan(ss, emit_output_loop);
     }
@@ -1133,6 +1180,17 @@ bool vec4_ok(const Program& P, const Domain& dom) {
     return true;
 }
 
+// Rows of unit column stride whose length, row stride or offset is no multiple of four elements: vector accesses at
+// element alignment with a partial last chunk, instead of one element per access.
+bool ragged_ok(const Program& P, const Domain& dom) {
+    if (dom.C < 16) return false;
+    for (const ArrayArg& a : P.arrays) {
+        if (a.gather_source || a.cls != Cls::FULL) continue;
+        if (a.col_stride != 1) return false;
+    }
+    return true;
+}
+
 bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
     RowPlan rpn;
     Program& P = rpn.P;
@@ -1178,6 +1236,12 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
     // launch geometry
     RowParams& rp = rpn.rp;
     rp.VEC = vec4_ok(P, dom) ? 4 : 1;
+    static const int ragged_env = env_int("DALI_HIP_ROW_RAGGED", 1);
+    if (rp.VEC == 1 && ragged_env && ragged_ok(P, dom)) {
+        rp.VEC = 4;
+        rp.ragged = true;
+        rp.tail = dom.C % rp.VEC != 0;
+    }
     int64_t CH = dom.C / rp.VEC;
     int n_full = 0, max_el = 4;
     for (const ArrayArg& a : P.arrays)
@@ -1205,6 +1269,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
         bool writes_rows = false;
         for (const Output& o : rpn.outputs) writes_rows = writes_rows || o.cls == Cls::FULL;
         if (writes_rows) tpr = std::max(tpr, std::min(64, pow2ceil((int)std::max<int64_t>(1, CH))));
+        if (rp.tail) tpr = std::max(tpr, 4);  // one thread per element past the last whole vector
         tpr = std::min(tpr, tpr_cap);
         int64_t ept = (CH + tpr - 1) / tpr;
         // every FULL input is held in registers across the phases: bound the footprint
@@ -1271,7 +1336,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
     rp.nt_loads = nt_l >= 0 ? nt_l != 0 : dom.R * dom.C * (int64_t)max_el >= ((int64_t)64 << 20);
     rp.nt_stores = nt_s >= 0 ? nt_s != 0 : true;
     params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached << "," << rp.waves_per_eu << ","
-           << rp.nt_loads << rp.nt_stores << rp.exact;
+           << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     std::string sig = signature(P, rpn.outputs);
     uint64_t h = kernel_hash("row", sig, params.str());
