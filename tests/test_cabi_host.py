@@ -162,6 +162,24 @@ def test_softmax_kernel_reads_the_row_once_and_keeps_exp_in_registers(D, rng):
             or "dali_block_reduce<reducers::maximum, float, 2>" in body)
 
 
+def test_rows_off_the_vector_alignment_keep_vector_accesses(D, rng):
+    op = D.op
+    x = D.Array.from_numpy(rng.randn(8, 1001).astype(np.float32))
+    D.generate_only([op.softmax(x)], compile=True)
+    body = D.last_source()
+    body = body[body.index("void dali_row_"):]
+    assert "dali_loadu" in body and "dali_storeu" in body and "tail_on" in body  # whole vectors + one element per thread
+    D.generate_only([op.softmax(x[:, 1:])], compile=True)  # 1000 columns starting one element in: no rest, still unaligned
+    body = D.last_source()
+    body = body[body.index("void dali_row_"):]
+    assert "dali_loadu" in body and "tail_on" not in body
+    D.generate_only([op.softmax(x[:, :1000])], compile=True)  # row stride 1001: rows start at every alignment
+    assert "dali_loadu" in D.last_source()[D.last_source().index("void dali_row_"):]
+    small = D.Array.from_numpy(rng.randn(8, 13).astype(np.float32))
+    D.generate_only([op.softmax(small)], compile=True)  # short rows: one element per access
+    assert "dali_loadu" not in D.last_source()[D.last_source().index("void dali_row_"):]
+
+
 def test_planner_splits_what_cannot_fuse(D, rng):
     op = D.op
     m = D.Array.from_numpy(rng.randn(6, 8).astype(np.float32))

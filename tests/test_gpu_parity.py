@@ -468,6 +468,47 @@ def test_middle_axis_reductions_use_the_batched_column_kernel(gpu, D, O, rng, sh
         assert np.array_equal(op.max(v, [1]).numpy(), nv.max(1))
 
 
+@pytest.mark.parametrize("cols", [16, 17, 18, 19, 63, 127, 257, 1023, 4097, 50257, 300001])
+def test_rows_not_aligned_to_the_vector(gpu, D, O, rng, cols):
+    """Row lengths that are no multiple of four elements, and views that start off a 16-byte boundary: whole vectors
+    at element alignment, the rest of each row one element per thread. Every phase, the register cache and the
+    op-assign destinations see the rest elements."""
+    op = D.op
+    rows = 5 if cols > 5000 else 37
+    x = (rng.randn(rows, cols) * 3).astype(np.float32)
+    X = arr(D, x)
+    s = op.softmax(X).numpy()
+    assert D.last_kernel_kinds() == "row"
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(-1, keepdims=True))
+    close(s, e / e.sum(-1, keepdims=True), rtol=1e-5, atol=1e-12)
+    assert np.array_equal(op.max(X, [1]).numpy(), x.max(1)) and np.array_equal(op.min(X, [1]).numpy(), x.min(1))
+    assert np.all(np.abs(op.sum(X, [1]).numpy() - x64.sum(1)) <= sum_tol(x, 1))
+    # the largest value sits in the rest elements / ties between a whole vector and the rest keep the first
+    t = rng.randint(0, 3, size=(rows, cols)).astype(np.float32)
+    t[0, :] = 0
+    t[0, cols - 1] = 5
+    t[1, :] = 1
+    t[2, cols - 2:] = 7
+    assert np.array_equal(op.argmax(arr(D, t), 1).numpy(), O.arg_axis_reduce(O.MAX, t, 1))
+    assert np.array_equal(op.argmin(arr(D, t), 1).numpy(), O.arg_axis_reduce(O.MIN, t, 1))
+    # a map over views that start one and two elements into the row, written with += into a view of a larger array
+    y = rng.randn(rows, cols + 3).astype(np.float32)
+    dst, want = arr(D, y), y.copy()
+    dst[:, 2:cols + 1].assign(X[:, 1:] * 2.0 + 1.0, 1)
+    want[:, 2:cols + 1] += x[:, 1:] * 2.0 + 1.0
+    assert np.array_equal(dst.numpy(), want)
+    # register-cached rows: a normalisation reads the row in three bodies
+    got = ((X - op.mean(X, [1], True)) / op.sqrt(op.mean(op.square(X), [1], True) + 1.0)).numpy()
+    close(got, (x64 - x64.mean(1, keepdims=True)) / np.sqrt((x64 * x64).mean(1, keepdims=True) + 1.0), rtol=2e-5, atol=2e-5)
+    # double precision and int32 rows
+    xd = rng.randn(rows, cols)
+    assert np.all(np.abs(op.sum(arr(D, xd), [1]).numpy() - xd.sum(1)) <= 1e-12 * np.abs(xd).sum(1) + 1e-12)
+    xi = rng.randint(-1000, 1000, size=(rows, cols)).astype(np.int32)
+    assert np.array_equal(op.sum(arr(D, xi), [1]).numpy(), xi.sum(1))
+    assert np.array_equal((arr(D, xi)[:, 1:] * 3).numpy(), xi[:, 1:] * 3)
+
+
 def test_argmax_ties_and_sentinels_are_bit_exact(gpu, D, O, rng):
     op = D.op
     # few distinct values -> many ties; widths straddle the one-wave / multi-wave / streaming row layouts
