@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-23";
+const char* const kCodegenVersion = "dali-hip-codegen-24";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -1386,7 +1386,9 @@ bool flat_eligible(const Array& a, int64_t n, std::set<const Expr*>& seen) {
     }
 }
 
-std::string gen_flat_kernel(const Program& P, const std::vector<Output>& outs, const IvLayout& L, int VEC, int BT, int UNROLL,
+// UNALIGNED: some operand starts off a 16-byte boundary (element-aligned vector accesses). REST: the element count is
+// no multiple of VEC; the first block's leading threads take one of the last N % VEC elements each.
+std::string gen_flat_kernel(const Program& P, const std::vector<Output>& outs, const IvLayout& L, int VEC, int BT, int UNROLL, bool UNALIGNED, bool REST,
                             const std::string& kname) {
     std::ostringstream ss;
     RowParams rp;
@@ -1405,7 +1407,7 @@ std::string gen_flat_kernel(const Program& P, const std::vector<Output>& outs, c
     ss << "  const long base = (long)blockIdx.x * (BT * UNROLL) + threadIdx.x;\n";
     for (int i : full_leaves) ss << "  " << ctype(P.arrays[i].buf->dtype) << " x" << i << "s[UNROLL][VEC];\n";
     ss << "  _Pragma(\"unroll\") for (int u = 0; u < UNROLL; ++u) {\n    const long ch = base + (long)u * BT;\n    if (ch < NCH) {\n";
-    for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, VEC, "x" + std::to_string(i) + "s[u]", "      ", true);
+    for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, VEC, "x" + std::to_string(i) + "s[u]", "      ", true, UNALIGNED);
     ss << "    }\n  }\n";
     ss << "  _Pragma(\"unroll\") for (int u = 0; u < UNROLL; ++u) {\n    const long ch = base + (long)u * BT;\n    if (ch < NCH) {\n";
     for (int i : full_leaves) ss << "      const " << ctype(P.arrays[i].buf->dtype) << "* x" << i << " = x" << i << "s[u];\n";
@@ -1417,13 +1419,25 @@ std::string gen_flat_kernel(const Program& P, const std::vector<Output>& outs, c
         std::string t = ctype(d.buf->dtype);
         std::string ov = "o" + std::to_string(o.array);
         pre << "      dali_vec<" << t << ", VEC> " << ov << ";\n";
-        if (o.op != OPERATOR_T_EQL) pre << "      " << ov << " = dali_load<" << t << ", VEC>(q" << o.array << " + ch * VEC);\n";
-        post << "      dali_store_nt<" << t << ", VEC>(q" << o.array << " + ch * VEC, " << ov << ");\n";
+        if (o.op != OPERATOR_T_EQL) pre << "      " << ov << " = " << (UNALIGNED ? "dali_loadu<" : "dali_load<") << t << ", VEC>(q" << o.array << " + ch * VEC);\n";
+        post << "      " << (UNALIGNED ? "dali_storeu_nt<" : "dali_store_nt<") << t << ", VEC>(q" << o.array << " + ch * VEC, " << ov << ");\n";
         std::string v = be.value(o.root);
         body << "        " << ov << ".v[j] = " << op_combine(o.op, ov + ".v[j]", "(" + t + ")(" + v + ")") << ";\n";
     }
     ss << pre.str() << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        const int col = (int)(ch * VEC + j); (void)col;\n";
-    ss << be.stmts.str() << body.str() << "      }\n" << post.str() << "    }\n  }\n}\n";
+    ss << be.stmts.str() << body.str() << "      }\n" << post.str() << "    }\n  }\n";
+    if (REST) {
+        ss << "  if (blockIdx.x == 0 && threadIdx.x < (unsigned)(N - NCH * VEC)) {\n    const long rest = NCH * VEC + threadIdx.x;\n";
+        for (int i : full_leaves) ss << "    " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n    x" << i << "[0] = q" << i << "[rest];\n";
+        ss << "    constexpr int j = 0; (void)j;\n    const int col = (int)rest; (void)col;\n" << be.stmts.str();
+        for (const Output& o : outs) {
+            std::string t = ctype(P.arrays[o.array].buf->dtype);
+            const std::string dp = "q" + std::to_string(o.array) + "[rest]";
+            ss << "    " << dp << " = " << op_combine(o.op, dp, "(" + t + ")(" + be.value(o.root) + ")") << ";\n";
+        }
+        ss << "  }\n";
+    }
+    ss << "}\n";
     return ss.str();
 }
 
@@ -1460,12 +1474,13 @@ bool try_flat(const std::vector<DestSpec>& specs) {
     count_uses(P, roots);
     int max_el = 4;
     for (const ArrayArg& a : P.arrays) max_el = std::max(max_el, size_of_dtype(a.buf->dtype));
-    bool vec = n % 4 == 0;
+    bool aligned = true;
     for (const ArrayArg& a : P.arrays)
-        if (a.cls == Cls::FULL && a.buf->offset % 4 != 0) vec = false;
-    int VEC = vec ? 4 : 1, BT = 256, UNROLL = max_el == 8 ? 2 : 4;
+        if (a.cls == Cls::FULL && a.buf->offset % 4 != 0) aligned = false;
+    int VEC = n >= 16 ? 4 : 1, BT = 256, UNROLL = max_el == 8 ? 2 : 4;
+    const bool UNALIGNED = VEC > 1 && !aligned, REST = VEC > 1 && n % VEC != 0;
     std::ostringstream params;
-    params << VEC << "," << BT << "," << UNROLL;
+    params << VEC << "," << BT << "," << UNROLL << "," << UNALIGNED << REST;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("flat", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& K = specs_cache[h];
@@ -1484,7 +1499,7 @@ bool try_flat(const std::vector<DestSpec>& specs) {
         K->plan.work_per_block = BT * UNROLL * VEC;
     }
     std::vector<std::vector<int>> shapes = {{(int)n}};
-    load_and_launch(*K, [&]() { return gen_flat_kernel(P, outs, L, VEC, BT, UNROLL, K->name); }, P, shapes);
+    load_and_launch(*K, [&]() { return gen_flat_kernel(P, outs, L, VEC, BT, UNROLL, UNALIGNED, REST, K->name); }, P, shapes);
     return true;
 }
 
@@ -1495,7 +1510,7 @@ bool try_flat(const std::vector<DestSpec>& specs) {
 // partials in block order (so the result does not depend on scheduling), applies
 // the scalar epilogue and resets the ticket counter.
 std::string gen_all_kernel(const Program& P, int red_id, int root_id, int dest_array, OPERATOR_T op, const IvLayout& L, int VEC, int BT,
-                           int UNROLL, int TAIL, bool NT, const std::string& kname) {
+                           int UNROLL, int TAIL, bool NT, bool UNALIGNED, bool REST, const std::string& kname) {
     const PNode& red = P.nodes[red_id];
     bool is_arg = red.kind == Kind::ARG_ALL_REDUCE;
     std::string t = ctype(P.nodes[red.args[0]].dtype);
@@ -1522,7 +1537,7 @@ std::string gen_all_kernel(const Program& P, int red_id, int root_id, int dest_a
     ss << "  for (long base = (long)blockIdx.x * (BT * UNROLL) + threadIdx.x; base < NCH; base += (long)gridDim.x * (BT * UNROLL)) {\n";
     for (int i : full_leaves) ss << "    " << ctype(P.arrays[i].buf->dtype) << " x" << i << "s[UNROLL][VEC];\n";
     ss << "    _Pragma(\"unroll\") for (int u = 0; u < UNROLL; ++u) {\n      const long ch = base + (long)u * BT;\n      if (ch < NCH) {\n";
-    for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, VEC, "x" + std::to_string(i) + "s[u]", "        ", NT);
+    for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, VEC, "x" + std::to_string(i) + "s[u]", "        ", NT, UNALIGNED);
     ss << "      }\n    }\n";
     ss << "    _Pragma(\"unroll\") for (int u = 0; u < UNROLL; ++u) {\n      const long ch = base + (long)u * BT;\n      if (ch < NCH) {\n";
     for (int i : full_leaves) ss << "        const " << ctype(P.arrays[i].buf->dtype) << "* x" << i << " = x" << i << "s[u];\n";
@@ -1531,13 +1546,21 @@ std::string gen_all_kernel(const Program& P, int red_id, int root_id, int dest_a
     {
         BodyEmitter be(P, rp, true, 0, &first_body);
         std::string v = be.value(red.args[0]);
-        ss << be.stmts.str();
+        std::string update;
         if (!is_arg)
-            ss << "          acc = " << red.name << "::step<" << t << ">(acc, " << v << ");\n";
+            update = "acc = " + red.name + "::step<" + t + ">(acc, " + v + ");\n";
         else
-            ss << "          { const " << t << " cand = " << v << "; if (" << red.name << "::better<" << t << ">(cand, acc)) { acc = cand; acci = col; } }\n";
+            update = "{ const " + t + " cand = " + v + "; if (" + red.name + "::better<" + t + ">(cand, acc)) { acc = cand; acci = col; } }\n";
+        ss << be.stmts.str() << "          " << update;
+        ss << "        }\n      }\n    }\n  }\n";
+        if (REST) {
+            // the last N % VEC elements: one each to the leading threads of the first block, after their vectors (so a
+            // thread still meets its elements in increasing order)
+            ss << "  if (blockIdx.x == 0 && threadIdx.x < (unsigned)(N - NCH * VEC)) {\n    const long rest = NCH * VEC + threadIdx.x;\n";
+            for (int i : full_leaves) ss << "    " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n    x" << i << "[0] = q" << i << "[rest];\n";
+            ss << "    constexpr int j = 0; (void)j;\n    const int col = (int)rest; (void)col;\n" << be.stmts.str() << "    " << update << "  }\n";
+        }
     }
-    ss << "        }\n      }\n    }\n  }\n";
     ss << "  __shared__ " << t << " smv[" << NW << "]; __shared__ int smi[" << NW << "]; __shared__ int is_last;\n";
     if (!is_arg)
         ss << "  acc = dali_block_reduce<" << red.name << ", " << t << ", " << NW << ">(acc, smv);\n";
@@ -1660,10 +1683,11 @@ bool try_all(const DestSpec& spec) {
     };
     if (!cls_epi(root_id)) return false;
     count_uses(P, {root_id});
-    bool vec = n % 4 == 0;
+    bool aligned = true;
     for (const ArrayArg& a : P.arrays)
-        if (a.cls == Cls::FULL && a.buf->offset % 4 != 0) vec = false;
-    int VEC = vec ? 4 : 1, BT = 256;
+        if (a.cls == Cls::FULL && a.buf->offset % 4 != 0) aligned = false;
+    int VEC = n >= 16 ? 4 : 1, BT = 256;
+    const bool UNALIGNED = VEC > 1 && !aligned, REST = VEC > 1 && n % VEC != 0;
     int max_el_all = 4;
     for (const ArrayArg& a : P.arrays) max_el_all = std::max(max_el_all, size_of_dtype(a.buf->dtype));
     const int UNROLL = max_el_all == 8 ? 4 : 8;  // vector loads in flight per thread
@@ -1675,7 +1699,7 @@ bool try_all(const DestSpec& spec) {
     outs[0].cls = Cls::SCAL;
     std::ostringstream params;
     const bool NT = n * (int64_t)max_el_all >= ((int64_t)64 << 20);
-    params << VEC << "," << BT << "," << red_id << "," << UNROLL << "," << TAIL << "," << NT;
+    params << VEC << "," << BT << "," << red_id << "," << UNROLL << "," << TAIL << "," << NT << "," << UNALIGNED << REST;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("all", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& K = specs_cache[h];
@@ -1696,7 +1720,7 @@ bool try_all(const DestSpec& spec) {
         K->plan.ws_elsize = 16;
     }
     std::vector<std::vector<int>> shapes = {{(int)n}};
-    load_and_launch(*K, [&]() { return gen_all_kernel(P, red_id, root_id, dest_array, spec.op, L, VEC, BT, UNROLL, TAIL, NT, K->name); }, P, shapes);
+    load_and_launch(*K, [&]() { return gen_all_kernel(P, red_id, root_id, dest_array, spec.op, L, VEC, BT, UNROLL, TAIL, NT, UNALIGNED, REST, K->name); }, P, shapes);
     return true;
 }
 

@@ -509,6 +509,37 @@ def test_rows_not_aligned_to_the_vector(gpu, D, O, rng, cols):
     assert np.array_equal((arr(D, xi)[:, 1:] * 3).numpy(), xi[:, 1:] * 3)
 
 
+@pytest.mark.parametrize("n", [16, 17, 18, 19, 1023, 65537, 1000003])
+def test_flat_maps_and_full_reductions_off_the_vector_size(gpu, D, O, rng, n):
+    """Element counts that are no multiple of four and views that start off a 16-byte boundary keep vector accesses;
+    the last n % 4 elements go one each to the leading threads of the first block."""
+    op = D.op
+    x, y = rng.randn(n).astype(np.float32), rng.randn(n).astype(np.float32)
+    X, Y = arr(D, x), arr(D, y)
+    assert np.array_equal((X * 2.0 + Y).numpy(), x * np.float32(2.0) + y)
+    assert D.last_kernel_kinds() == "flat"
+    assert np.array_equal((X[1:] - Y[:n - 1]).numpy(), x[1:] - y[:n - 1])
+    dst, want = arr(D, y), y.copy()
+    dst[3:].assign(X[:n - 3] * 3.0, 1)
+    want[3:] += x[:n - 3] * np.float32(3.0)
+    assert np.array_equal(dst.numpy(), want)
+    assert abs(float(op.sum(X * Y).numpy()) - float((x.astype(np.float64) * y).sum())) <= float(sum_tol(x * y))
+    assert abs(float(op.sum(X[3:]).numpy()) - float(x[3:].astype(np.float64).sum())) <= float(sum_tol(x[3:]))
+    assert float(op.max(X).numpy()) == x.max() and float(op.min(X[1:]).numpy()) == x[1:].min()
+    # the extreme value in the rest elements; ties resolved towards the lower flat index
+    t = rng.randint(0, 3, size=n).astype(np.float32)
+    assert int(op.argmax(arr(D, t)).numpy()) == O.arg_all_reduce(O.MAX, t)
+    t[n - 1] = 9
+    assert int(op.argmax(arr(D, t)).numpy()) == n - 1
+    t[n - 2] = 9
+    assert int(op.argmax(arr(D, t)).numpy()) == n - 2
+    assert int(op.argmin(arr(D, -t)).numpy()) == n - 2
+    xi = rng.randint(-1000, 1000, size=n).astype(np.int32)
+    assert int(op.sum(arr(D, xi)).numpy()) == int(xi.sum())
+    xd = rng.randn(n)
+    assert abs(float(op.sum(arr(D, xd)[1:]).numpy()) - xd[1:].sum()) <= 1e-12 * np.abs(xd).sum() + 1e-12
+
+
 def test_argmax_ties_and_sentinels_are_bit_exact(gpu, D, O, rng):
     op = D.op
     # few distinct values -> many ties; widths straddle the one-wave / multi-wave / streaming row layouts
