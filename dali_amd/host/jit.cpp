@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-24";
+const char* const kCodegenVersion = "dali-hip-codegen-25";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -1797,8 +1797,11 @@ int col_split_of(const Array& arg) {
 }
 
 std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATOR_T op, const IvLayout& L, int VEC, int UNR, int TAIL, int RG, bool NT,
-                           int IL, bool BATCHED, const std::string& kname) {
-    const std::string ld = NT ? "dali_load_nt<" : "dali_load<";
+                           int IL, bool BATCHED, bool UNALIGNED, bool SHIFT, const std::string& kname) {
+    // UNALIGNED: memory rows start off a 16-byte boundary (element-aligned vector loads). SHIFT: K is no multiple of
+    // VEC; the lane whose vector would cross the end of the kept axis moves it back to end at K, reduces those VEC
+    // columns like any other lane and stores only the ones its left neighbour does not own.
+    const std::string ld = UNALIGNED ? (NT ? "dali_loadu_nt<" : "dali_loadu<") : (NT ? "dali_load_nt<" : "dali_load<");
     const PNode& red = P.nodes[red_id];
     const bool ARG = red.kind == Kind::ARG_AXIS_REDUCE;  // carries (value, row index); ties keep the lower index
     std::string t = ctype(P.nodes[red.args[0]].dtype);
@@ -1822,6 +1825,7 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     ss << "  const int lane = threadIdx.x % TPP, wave = threadIdx.x / TPP;\n";
     ss << "  const long k0 = ((long)blockIdx.x * TPP + lane) * VEC;\n";
     ss << "  const bool k_ok = k0 < K;\n";
+    ss << "  const long ks = " << (SHIFT ? "k_ok && k0 + VEC > K ? K - VEC : k0" : "k0") << ";  // first kept column this lane reads\n";
     // BATCHED: the kept index runs over [batch, unit-stride run]; a lane's VEC kept elements lie in one run, and
     // the second shape entry holds the run length followed by the batch stride of every full operand
     if (BATCHED) ss << "  const long k_run = A.iv[" << L.shape_pos[1] << "], k_batch = k0 / k_run, k_in = k0 - k_batch * k_run;\n";
@@ -1836,7 +1840,7 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
                 ss << "  const " << ty << "* q" << i << " = (const " << ty << "*)A.p[" << i << "] + (k_ok ? k_batch * (long)A.iv[" << L.shape_pos[1] + 1 + full_seen
                    << "] + k_in : 0);\n";
             else
-                ss << "  const " << ty << "* q" << i << " = (const " << ty << "*)A.p[" << i << "] + (k_ok ? k0 : 0);\n";
+                ss << "  const " << ty << "* q" << i << " = (const " << ty << "*)A.p[" << i << "] + (k_ok ? ks : 0);\n";
             ++full_seen;
             ss << "  const long ld" << i << " = A.iv[" << L.stride_pos[i] + 1 << "];\n";
         } else {
@@ -1928,7 +1932,7 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     };
     emit_group_fold("  ");
     auto emit_store = [&](const std::string& indent) {
-        ss << indent << "_Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) if (k0 + j < K) { " << dt << "* dp = q" << dest_array << " + (k0 + j) * ds" << dest_array
+        ss << indent << "_Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) if (ks + j >= k0 && ks + j < K) { " << dt << "* dp = q" << dest_array << " + (ks + j) * ds" << dest_array
            << "; *dp = " << op_combine(op, "(*dp)", std::string("(") + dt + ")" + (ARG ? "acci[j]" : "acc[j]")) << "; }\n";
     };
     ss << "  if (gridDim.y == 1) {\n    if (wave == 0 && k_ok) {\n";
@@ -2046,12 +2050,15 @@ bool try_col(const DestSpec& spec) {
     P.nodes[red_id].cls_set = true;
     if (!cls(P.nodes[red_id].args[0])) return false;
     count_uses(P, {red_id});
-    bool vec = K % 4 == 0 && k_run % 4 == 0;
+    // a lane's vector lies within one unit-stride run; without a batch axis the last vector may be moved back instead
+    const bool vec = BATCHED ? k_run % 4 == 0 : K >= 16;
+    bool aligned = true;
     for (const ArrayArg& a : P.arrays)
-        if (!a.is_dest && a.cls == Cls::FULL && (a.buf->offset % 4 != 0 || a.col_stride % 4 != 0)) vec = false;
+        if (!a.is_dest && a.cls == Cls::FULL && (a.buf->offset % 4 != 0 || a.col_stride % 4 != 0)) aligned = false;
     for (int bs : batch_strides)
-        if (bs % 4 != 0) vec = false;
+        if (bs % 4 != 0) aligned = false;
     int VEC = vec ? 4 : 1;
+    const bool UNALIGNED = VEC > 1 && !aligned, SHIFT = VEC > 1 && K % VEC != 0;
     static const int IL = env_int("DALI_HIP_COL_INTERLEAVE", 2);
     static const int rg_env = env_int("DALI_HIP_COL_RG", 0), tail_env = env_int("DALI_HIP_COL_TAIL", 16);
     static const int unr_env = env_int("DALI_HIP_COL_UNR", 8), rows_env = env_int("DALI_HIP_COL_ROWS", 0);
@@ -2071,7 +2078,7 @@ bool try_col(const DestSpec& spec) {
     std::ostringstream params;
     const bool NT = K * X * (int64_t)size_of_dtype(arg.dtype()) >= ((int64_t)64 << 20);
     static const int maxy_env = env_int("DALI_HIP_COL_MAXY", 256);
-    params << VEC << "," << UNR << "," << TAIL << "," << RG << "," << NT << "," << IL << "," << BATCHED;
+    params << VEC << "," << UNR << "," << TAIL << "," << RG << "," << NT << "," << IL << "," << BATCHED << UNALIGNED << SHIFT;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("col", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& Kp = specs_cache[h];
@@ -2100,7 +2107,7 @@ bool try_col(const DestSpec& spec) {
         shapes.push_back({(int)k_run});
         shapes.back().insert(shapes.back().end(), batch_strides.begin(), batch_strides.end());
     }
-    load_and_launch(*Kp, [&]() { return gen_col_kernel(P, red_id, dest_array, spec.op, L, VEC, UNR, TAIL, RG, NT, IL, BATCHED, Kp->name); }, P, shapes);
+    load_and_launch(*Kp, [&]() { return gen_col_kernel(P, red_id, dest_array, spec.op, L, VEC, UNR, TAIL, RG, NT, IL, BATCHED, UNALIGNED, SHIFT, Kp->name); }, P, shapes);
     return true;
 }
 

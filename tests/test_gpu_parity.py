@@ -509,6 +509,29 @@ def test_rows_not_aligned_to_the_vector(gpu, D, O, rng, cols):
     assert np.array_equal((arr(D, xi)[:, 1:] * 3).numpy(), xi[:, 1:] * 3)
 
 
+@pytest.mark.parametrize("shape", [(37, 16), (37, 17), (5, 18), (300, 19), (3000, 1001), (64, 4097), (2000, 50257), (7, 300001)])
+def test_leading_axis_reductions_off_the_vector_size(gpu, D, O, rng, shape):
+    """Kept extents that are no multiple of four: memory rows start at every alignment, and the lane whose vector
+    would cross the end of the kept axis reads the last four columns instead and stores only its own."""
+    op = D.op
+    x = rng.randn(*shape).astype(np.float32)
+    X = arr(D, x)
+    got = op.sum(X, [0]).numpy()
+    assert D.last_kernel_kinds() == "col"
+    assert np.all(np.abs(got - x.astype(np.float64).sum(0)) <= sum_tol(x, 0))
+    assert np.array_equal(op.max(X, [0]).numpy(), x.max(0)) and np.array_equal(op.min(X, [0]).numpy(), x.min(0))
+    t = rng.randint(0, 3, size=shape).astype(np.float32)
+    assert np.array_equal(op.argmax(arr(D, t), 0).numpy(), O.arg_axis_reduce(O.MAX, t, 0))
+    assert np.array_equal(op.argmin(arr(D, t), 0).numpy(), O.arg_axis_reduce(O.MIN, t, 0))
+    # += into the destination: the columns shared by the moved lane and its neighbour are written once
+    acc = arr(D, np.ones(shape[1], np.float32))
+    acc.assign(op.max(X, [0]), 1)
+    assert np.array_equal(acc.numpy(), 1 + x.max(0))
+    v, nv = X[:, 1:], x[:, 1:]
+    assert np.array_equal(op.max(v, [0]).numpy(), nv.max(0))
+    assert np.all(np.abs(op.mean(v * v, [0]).numpy() - (nv.astype(np.float64) ** 2).mean(0)) <= sum_tol(nv * nv, 0) / shape[0] + 1e-6)
+
+
 @pytest.mark.parametrize("n", [16, 17, 18, 19, 1023, 65537, 1000003])
 def test_flat_maps_and_full_reductions_off_the_vector_size(gpu, D, O, rng, n):
     """Element counts that are no multiple of four and views that start off a 16-byte boundary keep vector accesses;
