@@ -1434,6 +1434,26 @@ LSTMSequence lstm_sequence(const Array& xs, const Array& h0, const Array& c0, co
     return {hs, c_prev, h_prev};
 }
 
+// dali/layers/stacked_lstm.cpp:219-283 with drop_prob = 0. A shortcut layer's two inputs are laid side by side so that
+// the layer stays one accumulating GEMM pair plus the gate kernel.
+StackedLSTMState stacked_lstm_step(const Array& x, const std::vector<Array>& h, const std::vector<Array>& c, const std::vector<Array>& W,
+                                   const std::vector<Array>& U, const std::vector<Array>& b, bool shortcut) {
+    const size_t layers = W.size();
+    DALI_ASSERT(h.size() == layers && c.size() == layers,
+                make_message("Activating LSTM stack of size ", layers, " with different number of states ", std::min(h.size(), c.size())));
+    DALI_ASSERT(U.size() == layers && b.size() == layers, "stacked_lstm_step: every layer needs its W, U and b");
+    StackedLSTMState out;
+    Array layer_input = x;
+    for (size_t l = 0; l < layers; ++l) {
+        Array in = (shortcut && l > 0) ? concatenate({layer_input, x}, 1) : layer_input;
+        LSTMState st = lstm_step(in, h[l], c[l], W[l], U[l], b[l]);
+        out.memory.push_back(st.memory);
+        out.hidden.push_back(st.hidden);
+        layer_input = st.hidden;
+    }
+    return out;
+}
+
 // One GRU step (dali/layers/gru.cpp:27-44 with StackedInputLayer::activate, dali/layers/layers.cpp:159-161), the
 // three input layers packed reset, update, candidate along the columns of W[I, 3H], U[H, 3H], b[3H]:
 //   r = sigmoid(x.Wr + h.Ur + br);  z = sigmoid(x.Wz + h.Uz + bz);  m = tanh(x.Wc + (r * h).Uc + bc)

@@ -189,6 +189,27 @@ int dali_fe_lstm_sequence(dali_array_t xs, dali_array_t h0, dali_array_t c0, dal
            *memory = wrap(r.memory); *hidden = wrap(r.hidden); return 0;
            , 1)
 }
+static int stacked_lstm_step_impl(dali_array_t x, int layers, const dali_array_t* h, const dali_array_t* c, const dali_array_t* W, const dali_array_t* U,
+                                  const dali_array_t* b, int shortcut, dali_array_t* c_new, dali_array_t* h_new) {
+    std::vector<Array> hv, cv, Wv, Uv, bv;
+    for (int l = 0; l < layers; ++l) {
+        hv.push_back(A(h[l]));
+        cv.push_back(A(c[l]));
+        Wv.push_back(A(W[l]));
+        Uv.push_back(A(U[l]));
+        bv.push_back(A(b[l]));
+    }
+    auto r = dali::op::stacked_lstm_step(A(x), hv, cv, Wv, Uv, bv, shortcut != 0);
+    for (int l = 0; l < layers; ++l) {
+        c_new[l] = wrap(r.memory[l]);
+        h_new[l] = wrap(r.hidden[l]);
+    }
+    return 0;
+}
+int dali_fe_stacked_lstm_step(dali_array_t x, int layers, const dali_array_t* h, const dali_array_t* c, const dali_array_t* W, const dali_array_t* U,
+                              const dali_array_t* b, int shortcut, dali_array_t* c_new, dali_array_t* h_new) {
+    FE_TRY(return stacked_lstm_step_impl(x, layers, h, c, W, U, b, shortcut, c_new, h_new);, 1)
+}
 dali_array_t dali_fe_gru_step(dali_array_t x, dali_array_t h, dali_array_t W, dali_array_t U, dali_array_t b) {
     FE_TRY(return wrap(dali::op::gru_step(A(x), A(h), A(W), A(U), A(b)));, nullptr)
 }

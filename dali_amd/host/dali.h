@@ -350,6 +350,15 @@ struct LSTMSequence {
     Array hidden_states, memory, hidden;
 };
 LSTMSequence lstm_sequence(const Array& xs, const Array& h0, const Array& c0, const Array& W, const Array& U, const Array& b);
+// One step of a stack of LSTM cells (dali/layers/stacked_lstm.cpp:219-283, forward_LSTMs and shortcut_forward_LSTMs
+// without dropout): layer l reads the new hidden state of layer l-1, the first layer reads x. With `shortcut` every
+// layer above the first also reads x; its W[l] is then [H(l-1) + I, 4 H(l)], the rows for the hidden state below
+// first, the rows for x after them (the order LSTM::activate_shortcut passes its inputs, dali/layers/lstm.cpp:281-289).
+struct StackedLSTMState {
+    std::vector<Array> memory, hidden;
+};
+StackedLSTMState stacked_lstm_step(const Array& x, const std::vector<Array>& h, const std::vector<Array>& c, const std::vector<Array>& W,
+                                   const std::vector<Array>& U, const std::vector<Array>& b, bool shortcut);
 // One GRU step with reset, update and candidate layers packed along the columns of W[I,3H], U[H,3H], b[3H]
 // (dali/layers/gru.cpp:27-44). Returns h', already evaluated.
 Array gru_step(const Array& x, const Array& h, const Array& W, const Array& U, const Array& b);

@@ -1,7 +1,7 @@
 """``op``: the lazy operator factories (``dali/array/op.h`` of the reference)."""
 import ctypes as C
 
-from ._native import front, fe_error
+from ._native import front, fe_error, DaliError
 from .array import Array, as_array, _ints, _wrap, DTYPE_FLOAT, DTYPE_DOUBLE, DTYPE_INT32  # noqa: F401
 
 
@@ -187,6 +187,24 @@ def lstm_sequence(xs, h0, c0, W, U, b):
     if front.dali_fe_lstm_sequence(*[k._h for k in keep], *[C.byref(o) for o in outs]) != 0:
         raise fe_error("lstm_sequence")
     return tuple(Array(o.value) for o in outs)
+
+
+def stacked_lstm_step(x, h, c, W, U, b, shortcut=False):
+    """One step of a stack of LSTM cells (dali/layers/stacked_lstm.cpp:219-283, no dropout); h, c, W, U, b are lists with
+    one entry per layer. Returns (list of c', list of h'), evaluated."""
+    layers = len(W)
+    xa = as_array(x)
+    groups = [[as_array(v) for v in g] for g in (h, c, W, U, b)]
+    if any(len(g) != layers for g in groups[2:]):
+        raise ValueError("stacked_lstm_step: every layer needs its W, U and b")
+    if len(groups[0]) != layers or len(groups[1]) != layers:
+        states = len(groups[0]) if len(groups[0]) != layers else len(groups[1])  # (min / max in this module are the reductions)
+        raise DaliError("Activating LSTM stack of size %d with different number of states %d" % (layers, states))
+    handles = [(C.c_void_p * layers)(*[k._h for k in g]) for g in groups]
+    c_new, h_new = (C.c_void_p * layers)(), (C.c_void_p * layers)()
+    if front.dali_fe_stacked_lstm_step(xa._h, layers, *handles, 1 if shortcut else 0, c_new, h_new) != 0:
+        raise fe_error("stacked_lstm_step")
+    return [Array(v) for v in c_new], [Array(v) for v in h_new]
 
 
 def gru_step(x, h, W, U, b):

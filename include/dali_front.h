@@ -112,6 +112,11 @@ int dali_fe_lstm_step(dali_array_t x, dali_array_t h, dali_array_t c, dali_array
 /* The LSTM step along xs[T, B, I] (dali/layers/lstm.cpp:294-303): hidden_states [T, B, H], final memory and hidden [B, H] */
 int dali_fe_lstm_sequence(dali_array_t xs, dali_array_t h0, dali_array_t c0, dali_array_t W, dali_array_t U, dali_array_t b,
                           dali_array_t* hidden_states, dali_array_t* memory, dali_array_t* hidden);
+/* One step of a stack of `layers` LSTM cells (dali/layers/stacked_lstm.cpp:219-283, no dropout): layer l reads the new
+ * hidden state of layer l-1; with `shortcut` the layers above the first also read x and their W is
+ * [H(l-1) + I, 4 H(l)], hidden-state rows first. c_new and h_new receive `layers` handles each. */
+int dali_fe_stacked_lstm_step(dali_array_t x, int layers, const dali_array_t* h, const dali_array_t* c, const dali_array_t* W,
+                              const dali_array_t* U, const dali_array_t* b, int shortcut, dali_array_t* c_new, dali_array_t* h_new);
 /* One GRU step, layers packed reset / update / candidate along the columns of W[I,3H], U[H,3H], b[3H]
  * (dali/layers/gru.cpp:27-44) */
 dali_array_t dali_fe_gru_step(dali_array_t x, dali_array_t h, dali_array_t W, dali_array_t U, dali_array_t b);

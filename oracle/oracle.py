@@ -395,6 +395,23 @@ def lstm_sequence(Xs, H0, C0, W, U, b, f64_gemm=True):
     return np.stack(hs), c
 
 
+def stacked_lstm_step(X, Hs, Cs, Ws, Us, bs, shortcut=False, f64_gemm=True):
+    """forward_LSTMs / shortcut_forward_LSTMs without dropout (dali/layers/stacked_lstm.cpp:219-283): layer l reads
+    the new hidden state of layer l-1; a shortcut layer above the first reads [hidden below, X]
+    (LSTM::activate_shortcut, dali/layers/lstm.cpp:281-289). Returns (list of c', list of h')."""
+    if not (len(Hs) == len(Cs) == len(Ws)):
+        raise ValueError("Activating LSTM stack of size %d with different number of states %d" % (len(Ws), min(len(Hs), len(Cs))))
+    cs, hs = [], []
+    layer_input = np.ascontiguousarray(X, np.float32)
+    for l in range(len(Ws)):
+        inp = np.concatenate([layer_input, X], 1) if (shortcut and l > 0) else layer_input
+        _, c, h = lstm_step(np.ascontiguousarray(inp, np.float32), Hs[l], Cs[l], Ws[l], Us[l], bs[l], f64_gemm)
+        cs.append(c)
+        hs.append(h)
+        layer_input = h
+    return cs, hs
+
+
 def gru_step(X, Hs, W, U, b):
     """dali/layers/gru.cpp:27-44 with the layers packed reset / update / candidate: products accumulated in fp64, the
     gate arithmetic through the checker's functors (sigmoid in double, libm tanhf), every operation rounded to fp32.

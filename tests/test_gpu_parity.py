@@ -1196,6 +1196,32 @@ def test_gru_step_matches_oracle(gpu, D, O, rng, B, I, H):
     assert np.array_equal(D.op.gru_step(*(arr(D, v) for v in (X, Hp, W, U, b_keep))).numpy(), Hp)
 
 
+@pytest.mark.parametrize("B,I,sizes", [(3, 8, [8]), (5, 7, [6, 4, 9]), (32, 64, [64, 64]), (16, 128, [128, 64, 192])])
+@pytest.mark.parametrize("shortcut", [False, True])
+def test_stacked_lstm_step_matches_oracle(gpu, D, O, rng, B, I, sizes, shortcut):
+    """forward_LSTMs / shortcut_forward_LSTMs without dropout (dali/layers/stacked_lstm.cpp:219-283)."""
+    X = rng.randn(B, I).astype(np.float32)
+    Hs = [rng.randn(B, h).astype(np.float32) for h in sizes]
+    Cs = [rng.randn(B, h).astype(np.float32) for h in sizes]
+    ins = [I] + [sizes[l - 1] + (I if shortcut else 0) for l in range(1, len(sizes))]
+    Ws = [(rng.uniform(-1, 1, (n, 4 * h)) / np.sqrt(n + h)).astype(np.float32) for n, h in zip(ins, sizes)]
+    Us = [(rng.uniform(-1, 1, (h, 4 * h)) / np.sqrt(2 * h)).astype(np.float32) for h in sizes]
+    bs = [(rng.randn(4 * h) * 0.1).astype(np.float32) for h in sizes]
+    wrap = lambda vs: [arr(D, v) for v in vs]
+    cs, hs = D.op.stacked_lstm_step(arr(D, X), wrap(Hs), wrap(Cs), wrap(Ws), wrap(Us), wrap(bs), shortcut)
+    want_c, want_h = O.stacked_lstm_step(X, Hs, Cs, Ws, Us, bs, shortcut)
+    assert len(cs) == len(hs) == len(sizes)
+    for l in range(len(sizes)):
+        close(cs[l].numpy(), want_c[l], rtol=1e-4, atol=1e-5)
+        close(hs[l].numpy(), want_h[l], rtol=1e-4, atol=1e-5)
+    # the first layer is the plain step on x
+    c0, h0 = D.op.lstm_step(*(arr(D, v) for v in (X, Hs[0], Cs[0], Ws[0], Us[0], bs[0])))
+    assert np.array_equal(c0.numpy(), cs[0].numpy()) and np.array_equal(h0.numpy(), hs[0].numpy())
+    if len(sizes) > 1:
+        with pytest.raises(D.DaliError, match="Activating LSTM stack of size %d with different number of states %d" % (len(sizes), len(sizes) - 1)):
+            D.op.stacked_lstm_step(arr(D, X), wrap(Hs[:-1]), wrap(Cs[:-1]), wrap(Ws), wrap(Us), wrap(bs), shortcut)
+
+
 @pytest.mark.parametrize("shape", [(3,), (2, 3, 4), (5, 257), (64, 1024), (3, 5000)])
 def test_circular_convolution_matches_oracle(gpu, D, O, rng, shape):
     # JITTests.circular_convolution / _broadcast / _1d (circular_convolution_tests.cpp:54-89)

@@ -593,3 +593,33 @@ def test_gru_step_against_fp64_definition(O, rng):
     _, c1, h1 = O.lstm_step(Xs[0], Hp, Hp, W4, U4, b4)
     _, c2, h2 = O.lstm_step(Xs[1], h1, c1, W4, U4, b4)
     assert np.array_equal(hs[1], h2) and hs.shape == (3, B, H)
+
+
+def test_stacked_lstm_step_against_fp64_definition(O, rng):
+    # dali/layers/stacked_lstm.cpp:219-283 written out in fp64: layer l reads h'(l-1); a shortcut layer reads [h'(l-1), x]
+    B, I, sizes = 5, 7, [6, 4, 9]
+    sig = lambda v: 1.0 / (1.0 + np.exp(-v))
+    for shortcut in (False, True):
+        X = rng.randn(B, I).astype(np.float32)
+        Hs = [rng.randn(B, h).astype(np.float32) for h in sizes]
+        Cs = [rng.randn(B, h).astype(np.float32) for h in sizes]
+        ins = [I] + [sizes[l - 1] + (I if shortcut else 0) for l in range(1, len(sizes))]
+        Ws = [rng.uniform(-0.4, 0.4, (n, 4 * h)).astype(np.float32) for n, h in zip(ins, sizes)]
+        Us = [rng.uniform(-0.4, 0.4, (h, 4 * h)).astype(np.float32) for h in sizes]
+        bs = [(rng.randn(4 * h) * 0.1).astype(np.float32) for h in sizes]
+        cs, hs = O.stacked_lstm_step(X, Hs, Cs, Ws, Us, bs, shortcut)
+        below = f64(X)
+        for l, h in enumerate(sizes):
+            inp = np.concatenate([below, f64(X)], 1) if (shortcut and l > 0) else below
+            g = inp @ f64(Ws[l]) + f64(Hs[l]) @ f64(Us[l]) + f64(bs[l])
+            i_, f_, o_, g_ = sig(g[:, :h]), sig(g[:, h:2 * h]), sig(g[:, 2 * h:3 * h]), np.tanh(g[:, 3 * h:])
+            c = f_ * f64(Cs[l]) + i_ * g_
+            hid = o_ * np.tanh(c)
+            assert np.abs(cs[l] - c).max() < 5e-6 and np.abs(hs[l] - hid).max() < 5e-6, (shortcut, l)
+            below = hid
+    # one layer is the plain step; a different number of states is refused (stacked_lstm.cpp:225-227)
+    _, c1, h1 = O.lstm_step(X, Hs[0], Cs[0], Ws[0], Us[0], bs[0])
+    cs, hs = O.stacked_lstm_step(X, Hs[:1], Cs[:1], Ws[:1], Us[:1], bs[:1])
+    assert np.array_equal(cs[0], c1) and np.array_equal(hs[0], h1)
+    with pytest.raises(ValueError, match="Activating LSTM stack of size 3 with different number of states 2"):
+        O.stacked_lstm_step(X, Hs[:2], Cs[:2], Ws, Us, bs)
