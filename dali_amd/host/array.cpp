@@ -349,18 +349,63 @@ Array Array::transpose() const {
 
 Array Array::transpose(const std::vector<int>& axes) const {
     DALI_ASSERT((int)axes.size() == ndim(), make_message("transpose needs ", ndim(), " axes (got ", axes.size(), ")."));
+    if (expression()->kind == Kind::EXPAND_DIMS) {
+        // Inserted unit axes over a lazy node (a keepdims reduction): when the permutation only moves the inserted axes
+        // among the others, the result is the same node with the unit axes inserted elsewhere, still lazy.
+        const int nd = ndim();
+        std::vector<int> frame(nd);
+        std::iota(frame.begin(), frame.end(), 0);
+        std::vector<bool> inserted(nd, false);
+        Array base = *this;
+        while (base.expression()->kind == Kind::EXPAND_DIMS) {
+            const int k = base.expression()->axis;
+            inserted[frame[k]] = true;
+            frame.erase(frame.begin() + k);
+            base = base.expression()->args[0];
+        }
+        std::vector<int> kept_order;
+        bool valid = true;
+        std::vector<int> norm(nd);
+        for (int i = 0; i < nd; ++i) {
+            norm[i] = axes[i] < 0 ? axes[i] + nd : axes[i];
+            valid = valid && norm[i] >= 0 && norm[i] < nd;
+            if (valid && !inserted[norm[i]]) kept_order.push_back(norm[i]);
+        }
+        if (valid && kept_order == frame) {
+            Array out = base;
+            for (int i = 0; i < nd; ++i)
+                if (inserted[norm[i]]) out = out.expand_dims(i);
+            return out;
+        }
+    }
     {
         // An elementwise node over operands of its own shape (and literals) stays lazy: its transpose is the same node
         // over the transposed operands, so a reduction along a leading axis of an expression still fuses with it.
         auto le = expression();
         if (le->kind == Kind::ELEMENTWISE && ndim() >= 2) {
             bool movable = true;
+            // (an operand broadcast from [.., 1, ..] moves as the broadcast of its transposed source)
+            auto broadcast_of_same_rank = [&](const Array& x) {
+                return x.expression()->kind == Kind::BROADCAST && x.expression()->args[0].ndim() == ndim();
+            };
             for (const Array& x : le->args)
                 movable = movable && (x.shape() == le->shape || x.expression()->kind == Kind::SCALAR) &&
-                          (x.is_buffer() || x.expression()->kind == Kind::SCALAR || x.expression()->kind == Kind::ELEMENTWISE);
+                          (x.is_buffer() || x.expression()->kind == Kind::SCALAR || x.expression()->kind == Kind::ELEMENTWISE ||
+                           x.expression()->kind == Kind::EXPAND_DIMS || broadcast_of_same_rank(x));
             if (movable) {
+                std::vector<int> tshape(ndim());
+                for (int i = 0; i < ndim(); ++i) tshape[i] = le->shape[axes[i] < 0 ? axes[i] + ndim() : axes[i]];
                 std::vector<Array> targs;
-                for (const Array& x : le->args) targs.push_back(x.expression()->kind == Kind::SCALAR ? x : x.transpose(axes));
+                for (const Array& x : le->args) {
+                    if (x.expression()->kind == Kind::SCALAR) targs.push_back(x);
+                    else if (broadcast_of_same_rank(x)) {
+                        auto bn = std::make_shared<Expr>(*x.expression());
+                        bn->args = {x.expression()->args[0].transpose(axes)};
+                        bn->shape = tshape;
+                        targs.push_back(Array(bn));
+                    }
+                    else targs.push_back(x.transpose(axes));
+                }
                 auto n = std::make_shared<Expr>(*le);
                 n->args = targs;
                 for (const Array& t : targs)

@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-25";
+const char* const kCodegenVersion = "dali-hip-codegen-27";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -1076,6 +1076,8 @@ void load_and_launch(KernelSpec& K, const std::function<std::string()>& gen, con
         if (g_capture_compare_only) return;
     }
     JitStats& st = jit_stats();
+    static const bool trace_plan = getenv("DALI_HIP_TRACE_PLAN") != nullptr;  // one line per planned launch on stderr
+    if (trace_plan) fprintf(stderr, "[dali-hip plan] %s\n", K.name.c_str());
     if (!st.last_kernel_kinds.empty()) st.last_kernel_kinds += ",";
     st.last_kernel_kinds += K.kind;
     if (!st.last_kernel_names.empty()) st.last_kernel_names += ",";
@@ -1762,6 +1764,14 @@ bool col_buffer_layout(const Expr* e, const std::vector<int>& shape, int split, 
     return true;
 }
 
+// [kept..., 1] against [kept..., X]
+bool col_kept_vector(const std::vector<int>& s, const std::vector<int>& shape) {
+    if (s.size() != shape.size() || s.empty() || s.back() != 1 || shape.back() == 1) return false;
+    for (size_t d = 0; d + 1 < s.size(); ++d)
+        if (s[d] != shape[d]) return false;
+    return true;
+}
+
 bool col_eligible(const Array& a, const std::vector<int>& shape, int split, std::set<const Expr*>& seen) {
     auto e = a.expression();
     if (seen.count(e.get())) return true;
@@ -1770,8 +1780,10 @@ bool col_eligible(const Array& a, const std::vector<int>& shape, int split, std:
         case Kind::SCALAR: return true;
         case Kind::BUFFER: {
             if (numel_of(e->shape) == 1) return true;
-            if (e->shape != shape) return false;
-            return col_buffer_layout(e.get(), shape, split, nullptr);
+            if (e->shape == shape) return col_buffer_layout(e.get(), shape, split, nullptr);
+            // one value per kept index, constant along the reduced axis ([kept..., 1] under a broadcast)
+            if (col_kept_vector(e->shape, shape)) return col_buffer_layout(e.get(), e->shape, split, nullptr);
+            return false;
         }
         case Kind::ELEMENTWISE:
             for (const Array& x : e->args) {
@@ -1779,8 +1791,11 @@ bool col_eligible(const Array& a, const std::vector<int>& shape, int split, std:
                 if (!col_eligible(x, shape, split, seen)) return false;
             }
             return true;
-        case Kind::BROADCAST:
-            return numel_of(e->args[0].shape()) == 1 && col_eligible(e->args[0], shape, split, seen);
+        case Kind::BROADCAST: {
+            const Array& in = e->args[0];
+            if (numel_of(in.shape()) == 1) return col_eligible(in, shape, split, seen);
+            return e->shape == shape && in.is_buffer() && col_kept_vector(in.shape(), shape) && col_eligible(in, shape, split, seen);
+        }
         default: return false;
     }
 }
@@ -1827,22 +1842,26 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     ss << "  const bool k_ok = k0 < K;\n";
     ss << "  const long ks = " << (SHIFT ? "k_ok && k0 + VEC > K ? K - VEC : k0" : "k0") << ";  // first kept column this lane reads\n";
     // BATCHED: the kept index runs over [batch, unit-stride run]; a lane's VEC kept elements lie in one run, and
-    // the second shape entry holds the run length followed by the batch stride of every full operand
+    // the second shape entry holds the run length followed by one batch stride per array
     if (BATCHED) ss << "  const long k_run = A.iv[" << L.shape_pos[1] << "], k_batch = k0 / k_run, k_in = k0 - k_batch * k_run;\n";
-    int full_seen = 0;
+    std::vector<int> kept_vectors;  // operands with one value per kept index
     for (size_t i = 0; i < P.arrays.size(); ++i) {
         const ArrayArg& a = P.arrays[i];
         std::string ty = ctype(a.buf->dtype);
         if (a.is_dest) {
             ss << "  " << ty << "* q" << i << " = (" << ty << "*)A.p[" << i << "];\n  const long ds" << i << " = " << (a.strided ? "A.iv[" + std::to_string(L.stride_pos[i]) + "]" : "1") << ";\n";
-        } else if (a.cls == Cls::FULL) {
+        } else if (a.cls == Cls::FULL || a.cls == Cls::ROW) {
             if (BATCHED)
-                ss << "  const " << ty << "* q" << i << " = (const " << ty << "*)A.p[" << i << "] + (k_ok ? k_batch * (long)A.iv[" << L.shape_pos[1] + 1 + full_seen
+                ss << "  const " << ty << "* q" << i << " = (const " << ty << "*)A.p[" << i << "] + (k_ok ? k_batch * (long)A.iv[" << L.shape_pos[1] + 1 + i
                    << "] + k_in : 0);\n";
             else
                 ss << "  const " << ty << "* q" << i << " = (const " << ty << "*)A.p[" << i << "] + (k_ok ? ks : 0);\n";
-            ++full_seen;
-            ss << "  const long ld" << i << " = A.iv[" << L.stride_pos[i] + 1 << "];\n";
+            if (a.cls == Cls::FULL) {
+                ss << "  const long ld" << i << " = A.iv[" << L.stride_pos[i] + 1 << "];\n";
+            } else {
+                kept_vectors.push_back((int)i);
+                ss << "  " << ty << " rl" << i << "v[VEC];\n  _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) rl" << i << "v[j] = k_ok ? q" << i << "[j] : (" << ty << ")0;\n";
+            }
         } else {
             ss << "  const " << ty << " sl" << i << " = ((const " << ty << "*)A.p[" << i << "])[0];\n";
         }
@@ -1886,6 +1905,7 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     ss << "      _Pragma(\"unroll\") for (int u = 0; u < UNR; ++u) {\n";
     for (int i : full_leaves) ss << "        const " << ctype(P.arrays[i].buf->dtype) << "* x" << i << " = x" << i << "s[u];\n";
     ss << "        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n          const int col = 0; (void)col;\n";
+    for (int i : kept_vectors) ss << "          const " << ctype(P.arrays[i].buf->dtype) << " rl" << i << " = rl" << i << "v[j];\n";
     {
         BodyEmitter be(P, rp, true, 0, &first_body);
         std::string v = be.value(red.args[0]);
@@ -1905,6 +1925,7 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
         ss << "      { dali_vec<" << ty << ", VEC> tmp = " << ld << ty << ", VEC>(q" << i << " + x * ld" << i << "); _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) x" << i << "[j] = tmp.v[j]; }\n";
     }
     ss << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        const int col = 0; (void)col;\n";
+    for (int i : kept_vectors) ss << "        const " << ctype(P.arrays[i].buf->dtype) << " rl" << i << " = rl" << i << "v[j];\n";
     {
         BodyEmitter be(P, rp, true, 0, &first_body);
         std::string v = be.value(red.args[0]);
@@ -2002,7 +2023,7 @@ bool try_col(const DestSpec& spec) {
     if (dest_array < 0) return false;
     int red_id = add_node(P, root);
     // classify the argument tree: [K, X] buffers are FULL with the kept stride in strides[0]
-    std::vector<int> batch_strides;  // one per FULL operand, in argument order
+    std::vector<int> batch_strides = {0};  // one per array of the program (the destination's is not used)
     std::function<bool(int)> cls = [&](int id) -> bool {
         PNode& nd = P.nodes[id];
         if (nd.cls_set) return true;
@@ -2017,6 +2038,13 @@ bool try_col(const DestSpec& spec) {
                 a.nd = 1;
                 a.sizes = {1};
                 nd.cls = Cls::SCAL;
+            } else if (col_kept_vector(nd.shape, arg_shape)) {
+                // one value per kept index: read once per lane, ahead of the loop over the reduced axis
+                col_buffer_layout(nd.src.get(), nd.shape, split, &bs);
+                a.cls = Cls::ROW;
+                a.nd = 1;
+                a.sizes = {(int)K};
+                nd.cls = Cls::ROW;
             } else {
                 auto st = strides_of(nd.src.get());
                 col_buffer_layout(nd.src.get(), arg_shape, split, &bs);
@@ -2036,7 +2064,8 @@ bool try_col(const DestSpec& spec) {
                     return true;
                 }
             P.arrays.push_back(a);
-            if (a.cls == Cls::FULL) batch_strides.push_back((int)bs);
+            batch_strides.resize(P.arrays.size(), 0);
+            batch_strides.back() = (int)bs;
             P.nodes[id].array = (int)P.arrays.size() - 1;
             return true;
         }
@@ -2083,6 +2112,7 @@ bool try_col(const DestSpec& spec) {
     uint64_t h = kernel_hash("col", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& Kp = specs_cache[h];
     std::vector<int> shape_ndims = {2};
+    batch_strides.resize(P.arrays.size(), 0);
     if (BATCHED) shape_ndims.push_back(1 + (int)batch_strides.size());
     IvLayout L = layout_iv(P, shape_ndims);
     if (!Kp) {
@@ -2389,6 +2419,9 @@ void run_gemm(const Array& dst, const Expr* mm, const Expr* mm2, float beta) {
 
 // ------------------------------------------------------ graph preparation
 Array rebuild(const std::shared_ptr<Expr>& e, const std::vector<Array>& args) {
+    // a unit axis inserted into a buffer is a view of that buffer (an evaluated keepdims reduction reads like any other
+    // [.., 1, ..] operand)
+    if (e->kind == Kind::EXPAND_DIMS && args.size() == 1 && args[0].is_buffer()) return args[0].expand_dims(e->axis);
     auto n = std::make_shared<Expr>(*e);
     n->args = args;
     return Array(n);
@@ -2566,6 +2599,26 @@ Array substitute(const Array& a, const Expr* target, const Array& with, std::map
         changed = changed || c.expression().get() != x.expression().get();
         args.push_back(c);
     }
+    Array out = changed ? rebuild(e, args) : a;
+    memo[e.get()] = out;
+    return out;
+}
+
+// Evaluating a node turns every handle on it into its buffer, so after an inner reduction has been evaluated the tree
+// holds unit axes inserted over a buffer: those become views of the buffer (what `rebuild` makes of them).
+Array fold_expanded_buffers(const Array& a, std::map<const Expr*, Array>& memo) {
+    auto e = a.expression();
+    if (e->kind == Kind::BUFFER || e->kind == Kind::SCALAR) return a;
+    auto it = memo.find(e.get());
+    if (it != memo.end()) return it->second;
+    std::vector<Array> args;
+    bool changed = false;
+    for (const Array& x : e->args) {
+        Array c = fold_expanded_buffers(x, memo);
+        changed = changed || c.expression().get() != x.expression().get();
+        args.push_back(c);
+    }
+    if (e->kind == Kind::EXPAND_DIMS && args.size() == 1 && args[0].is_buffer()) changed = true;
     Array out = changed ? rebuild(e, args) : a;
     memo[e.get()] = out;
     return out;
@@ -2855,6 +2908,10 @@ void run_specs_planned(std::vector<DestSpec> specs) {
         }
     }
     for (int iter = 0; iter < 64; ++iter) {
+        if (iter > 0 && specs.size() == 1) {
+            std::map<const Expr*, Array> fold_memo;
+            specs[0].root = fold_expanded_buffers(specs[0].root, fold_memo);
+        }
         bool has_all = has_kind(specs[0].root, [](Kind k) { return is_all_reduce(k); });
         if (has_all) {
             if (try_all(specs[0])) return;
@@ -2973,6 +3030,40 @@ void run_specs_planned(std::vector<DestSpec> specs) {
         for (auto& s : specs)
             if (find_first_reduce(s.root, &first, seen)) break;
         Domain dom = domain_of(first.expression()->args[0].shape());
+        if (specs.size() == 1) {
+            // The argument of a reduction against the layout of its operands (a candidate for the column kernel) may hold
+            // small unevaluated operands that are broadcast along the reduced axis (the column means inside a variance):
+            // those are evaluated first, so that the column kernel reads them as one value per kept index.
+            Array inner;
+            std::set<const Expr*> seen_inner;
+            if (find_innermost_reduce(specs[0].root, &inner, seen_inner) &&
+                (inner.expression()->kind == Kind::AXIS_REDUCE || inner.expression()->kind == Kind::ARG_AXIS_REDUCE)) {
+                Array red_arg = inner.expression()->args[0];
+                bool against_layout = false, settled = false;
+                std::function<void(const Array&)> scan = [&](const Array& a) {
+                    auto ae = a.expression();
+                    if (ae->kind == Kind::BUFFER && ae->shape.size() >= 2 && ae->shape.back() > 1 && numel_of(ae->shape) > ae->shape.back() &&
+                        strides_of(ae.get()).back() != 1)
+                        against_layout = true;
+                    if (ae->kind != Kind::BUFFER && ae->kind != Kind::SCALAR)
+                        for (const Array& x : ae->args) scan(x);
+                };
+                scan(red_arg);
+                std::function<void(const Array&)> settle = [&](const Array& a) {
+                    auto ae = a.expression();
+                    if (ae->kind == Kind::BUFFER || ae->kind == Kind::SCALAR) return;
+                    if (ae->kind == Kind::BROADCAST && !ae->args[0].is_buffer() && numel_of(ae->args[0].shape()) > 1 &&
+                        col_kept_vector(ae->args[0].shape(), red_arg.shape()) && !has_kind(ae->args[0], [](Kind k) { return is_reduce(k); })) {
+                        materialize(ae->args[0]);
+                        settled = true;
+                        return;
+                    }
+                    for (const Array& x : ae->args) settle(x);
+                };
+                if (against_layout && red_arg.ndim() >= 2) settle(red_arg);
+                if (settled) continue;
+            }
+        }
         if (specs.size() == 1 && try_col(specs[0])) return;
         if (specs.size() == 1) {
             // A reduction along the leading axis of row-major operands under further arithmetic (mean = sum / count, a

@@ -532,6 +532,32 @@ def test_leading_axis_reductions_off_the_vector_size(gpu, D, O, rng, shape):
     assert np.all(np.abs(op.mean(v * v, [0]).numpy() - (nv.astype(np.float64) ** 2).mean(0)) <= sum_tol(nv * nv, 0) / shape[0] + 1e-6)
 
 
+@pytest.mark.parametrize("shape", [(2, 5), (7, 33), (300, 64), (1000, 257), (4096, 1024), (33, 50257), (5, 6, 7), (16, 300, 64), (3, 4, 5, 8)])
+def test_softmax_and_moments_along_a_leading_axis(gpu, D, O, rng, shape):
+    """op::softmax with an axis (dali/array/op/softmax.cpp:5-8) and the mean / variance of columns: reductions whose
+    argument holds operands that are constant along the reduced axis (the column maxima, the column means)."""
+    op = D.op
+    x = (rng.randn(*shape) * 3).astype(np.float32)
+    X = arr(D, x)
+    x64 = x.astype(np.float64)
+    for axis in range(len(shape) - 1):
+        s = op.softmax(X, axis).numpy()
+        e = np.exp(x64 - x64.max(axis, keepdims=True))
+        close(s, e / e.sum(axis, keepdims=True), rtol=1e-5, atol=1e-12)
+        close(s.sum(axis), 1.0, rtol=0, atol=1e-5)
+        if len(shape) == 2 and shape[0] > 1 and shape[1] >= 16:
+            assert D.last_kernel_kinds() == "col,map2d"  # column maxima, column sums of exp(x - max), the quotient
+        mu = op.mean(X, [axis], True)
+        var = op.mean(op.square(X - mu), [axis]).numpy()
+        close(var, x64.var(axis), rtol=2e-5, atol=1e-6)
+        # the same through an evaluated mean, and the largest centred value per column
+        mu.eval()
+        close(op.mean(op.square(X - mu), [axis]).numpy(), x64.var(axis), rtol=2e-5, atol=1e-6)
+        close(op.max(op.abs(X - mu), [axis]).numpy(), np.abs(x64 - x64.mean(axis, keepdims=True)).max(axis), rtol=1e-5, atol=1e-5)
+        z = ((X - mu) / op.sqrt(op.mean(op.square(X - mu), [axis], True) + 1e-5)).numpy()
+        close(z, (x64 - x64.mean(axis, keepdims=True)) / np.sqrt(x64.var(axis, keepdims=True) + 1e-5), rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("n", [16, 17, 18, 19, 1023, 65537, 1000003])
 def test_flat_maps_and_full_reductions_off_the_vector_size(gpu, D, O, rng, n):
     """Element counts that are no multiple of four and views that start off a 16-byte boundary keep vector accesses;
