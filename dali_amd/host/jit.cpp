@@ -2091,7 +2091,13 @@ bool try_col(const DestSpec& spec) {
     static const int IL = env_int("DALI_HIP_COL_INTERLEAVE", 2);
     static const int rg_env = env_int("DALI_HIP_COL_RG", 0), tail_env = env_int("DALI_HIP_COL_TAIL", 16);
     static const int unr_env = env_int("DALI_HIP_COL_UNR", 8), rows_env = env_int("DALI_HIP_COL_ROWS", 0);
-    static const int blocks_env = env_int("DALI_HIP_COL_BLOCKS", 256);
+    static const int blocks_env = env_int("DALI_HIP_COL_BLOCKS", 0);
+    // One 256-thread workgroup per CU keeps eight loads per lane in flight and is best for a bare reduction; with
+    // transcendental arithmetic on every element a single wave per SIMD cannot overlap it with its loads, and two
+    // workgroups per CU are better (sum(exp(x)) along the leading axis of [8192,8192]: 61 -> 45 us; bare sum 40.6 -> 42.1)
+    // (small problems keep one: [4096,1024] 13 us against 20 us with the extra partial results to fold)
+    const bool streaming = K * X * (int64_t)size_of_dtype(arg.dtype()) >= ((int64_t)64 << 20);
+    const int max_blocks = blocks_env > 0 ? blocks_env : (streaming && contains_expensive(P, P.nodes[red_id].args[0]) ? 512 : 256);
     const int UNR = unr_env;
     // four row groups of one wave each: a wave reads 1 KiB pieces of memory rows, a block owns a 256-column strip.
     // Narrow strips and few y-blocks measured best (8192x8192: 53 us with 1024-column strips x 32 y-blocks,
@@ -2107,7 +2113,7 @@ bool try_col(const DestSpec& spec) {
     std::ostringstream params;
     const bool NT = K * X * (int64_t)size_of_dtype(arg.dtype()) >= ((int64_t)64 << 20);
     static const int maxy_env = env_int("DALI_HIP_COL_MAXY", 256);
-    params << VEC << "," << UNR << "," << TAIL << "," << RG << "," << NT << "," << IL << "," << BATCHED << UNALIGNED << SHIFT;
+    params << VEC << "," << UNR << "," << TAIL << "," << RG << "," << NT << "," << IL << "," << BATCHED << UNALIGNED << SHIFT << "," << max_blocks;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("col", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& Kp = specs_cache[h];
@@ -2129,7 +2135,7 @@ bool try_col(const DestSpec& spec) {
         Kp->plan.work2_begin = L.shape_pos[0] + 1;
         Kp->plan.work2_per_block = rows_env > 0 ? rows_env : UNR * RG;  // fewest reduced rows per y-block
         Kp->plan.max_blocks2 = maxy_env;
-        Kp->plan.max_blocks = blocks_env;  // one block per CU: the y split fills what the column strips leave
+        Kp->plan.max_blocks = max_blocks;  // the y split fills what the column strips leave
         Kp->plan.ws_elsize = size_of_dtype(arg.dtype()) + (is_arg ? 4 : 0);  // a partial is a value, plus its index
     }
     std::vector<std::vector<int>> shapes = {{(int)K, (int)X}};
