@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-27";
+const char* const kCodegenVersion = "dali-hip-codegen-28";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -2223,37 +2223,55 @@ bool nd_collect(Program& P, int id, const std::vector<int>& axis_map, int out_nd
     }
 }
 
-std::string gen_generic_kernel(const Program& P, const std::vector<Output>& outs, const IvLayout& L, int nd, const std::string& kname) {
+// VEC > 1: the destination and every operand have stride 1 or 0 (UNIT[a] false: a broadcast) along the last axis, whose
+// extent is a multiple of VEC; a thread decomposes one index for VEC adjacent elements and moves them as one vector at
+// element alignment. NARROW: fewer than 2^31 elements, the decomposition runs in 32-bit arithmetic.
+std::string gen_generic_kernel(const Program& P, const std::vector<Output>& outs, const IvLayout& L, int nd, int VEC, const std::vector<bool>& UNIT, bool NARROW,
+                               const std::string& kname) {
     std::ostringstream ss;
     RowParams rp;
     rp.cached = false;
-    rp.VEC = 1;
+    rp.VEC = VEC;
+    const std::string it = NARROW ? "unsigned int" : "long";
     ss << codegen::kDevicePrelude;
     ss << kargs_struct(P, L);
     ss << "extern \"C\" __global__ __launch_bounds__(256) void " << kname << "(KArgs A) {\n";
-    ss << "  constexpr int ND = " << nd << ";\n";
-    ss << "  long total = 1;\n  _Pragma(\"unroll\") for (int d = 0; d < ND; ++d) total *= A.iv[" << L.shape_pos[0] << " + d];\n";
+    ss << "  constexpr int ND = " << nd << ", VEC = " << VEC << ";\n";
+    ss << "  long total = 1;\n  _Pragma(\"unroll\") for (int d = 0; d < ND; ++d) total *= A.iv[" << L.shape_pos[0] << " + d];\n  total /= VEC;\n";
     ss << "  const long row = 0; (void)row;\n";
     ss << "  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {\n";
-    ss << "    int idx[ND];\n    long rem = i;\n";
-    ss << "    _Pragma(\"unroll\") for (int d = ND - 1; d >= 0; --d) { const int ext = A.iv[" << L.shape_pos[0] << " + d]; idx[d] = (int)(rem % ext); rem /= ext; }\n";
+    ss << "    int idx[ND];\n    " << it << " rem = (" << it << ")i;\n";
+    ss << "    _Pragma(\"unroll\") for (int d = ND - 1; d >= 0; --d) { const " << it << " ext = (" << it << ")A.iv[" << L.shape_pos[0]
+       << " + d] / (d == ND - 1 ? VEC : 1); idx[d] = (int)(rem % ext) * (d == ND - 1 ? VEC : 1); rem /= ext; }\n";
     for (size_t a = 0; a < P.arrays.size(); ++a) {
         ss << "    long off" << a << " = 0;\n    _Pragma(\"unroll\") for (int d = 0; d < ND; ++d) off" << a << " += (long)idx[d] * A.iv[" << L.stride_pos[a] << " + d];\n";
         const ArrayArg& arr = P.arrays[a];
         std::string t = ctype(arr.buf->dtype);
-        if (!arr.is_dest) ss << "    const " << t << " x" << a << "[1] = { ((const " << t << "*)A.p[" << a << "])[off" << a << "] };\n";
+        if (arr.is_dest) continue;
+        if (VEC > 1 && UNIT[a])
+            ss << "    const dali_vec<" << t << ", VEC> xv" << a << " = dali_loadu<" << t << ", VEC>((const " << t << "*)A.p[" << a << "] + off" << a << ");\n    const " << t
+               << "* x" << a << " = xv" << a << ".v;\n";
+        else if (VEC > 1)
+            ss << "    " << t << " x" << a << "[VEC];\n    { const " << t << " one = ((const " << t << "*)A.p[" << a << "])[off" << a
+               << "]; _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) x" << a << "[j] = one; }\n";
+        else
+            ss << "    const " << t << " x" << a << "[1] = { ((const " << t << "*)A.p[" << a << "])[off" << a << "] };\n";
     }
-    ss << "    const int j = 0, col = idx[ND - 1]; (void)j; (void)col;\n";
     std::vector<int> first_body(P.nodes.size(), -1);
     BodyEmitter be(P, rp, true, 0, &first_body);
-    std::ostringstream body;
+    std::ostringstream pre, body, post;
     for (const Output& o : outs) {
         std::string t = ctype(P.arrays[o.array].buf->dtype);
-        std::string dst = "((" + t + "*)A.p[" + std::to_string(o.array) + "])[off" + std::to_string(o.array) + "]";
+        const std::string ptr = "((" + t + "*)A.p[" + std::to_string(o.array) + "] + off" + std::to_string(o.array) + ")";
+        const std::string ov = "o" + std::to_string(o.array);
+        pre << "    dali_vec<" << t << ", VEC> " << ov << ";\n";
+        if (o.op != OPERATOR_T_EQL) pre << "    " << ov << " = dali_loadu<" << t << ", VEC>(" << ptr << ");\n";
         std::string v = be.value(o.root);
-        body << "    " << dst << " = " << op_combine(o.op, dst, "(" + t + ")(" + v + ")") << ";\n";
+        body << "      " << ov << ".v[j] = " << op_combine(o.op, ov + ".v[j]", "(" + t + ")(" + v + ")") << ";\n";
+        post << "    dali_storeu<" << t << ", VEC>(" << ptr << ", " << ov << ");\n";
     }
-    ss << be.stmts.str() << body.str() << "  }\n}\n";
+    ss << pre.str() << "    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n      const int col = idx[ND - 1] + j; (void)col;\n";
+    ss << be.stmts.str() << body.str() << "    }\n" << post.str() << "  }\n}\n";
     return ss.str();
 }
 
@@ -2300,8 +2318,18 @@ bool try_generic(const std::vector<DestSpec>& specs) {
     std::vector<int> ext = shape;
     if (ext.empty()) ext = {1};
     for (ArrayArg& a : P.arrays) a.sizes = ext;
+    // four adjacent elements of the last axis per thread when every array runs along it with stride 1 (or 0)
+    int VEC = ext.back() % 4 == 0 ? 4 : 1;
+    std::vector<bool> UNIT(P.arrays.size(), true);
+    for (size_t a = 0; a < P.arrays.size(); ++a) {
+        const int last = P.arrays[a].strides.empty() ? 0 : P.arrays[a].strides.back();
+        UNIT[a] = last == 1;
+        if (last != 1 && (last != 0 || P.arrays[a].is_dest)) VEC = 1;
+    }
+    const bool NARROW = numel_of(ext) < ((int64_t)1 << 31);
     std::ostringstream params;
-    params << nd;
+    params << nd << "," << VEC << "," << NARROW << ",";
+    for (size_t a = 0; a < UNIT.size(); ++a) params << (VEC > 1 && UNIT[a] ? 'u' : 'b');
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("generic", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& K = specs_cache[h];
@@ -2317,11 +2345,11 @@ bool try_generic(const std::vector<DestSpec>& specs) {
         K->plan.grid_kind = DALI_HIP_GRID_ELEMS;
         K->plan.work_begin = L.shape_pos[0];
         K->plan.work_count = nd;
-        K->plan.work_per_block = 256;
+        K->plan.work_per_block = 256 * VEC;
         K->plan.max_blocks = 65536;
     }
     std::vector<std::vector<int>> shapes = {ext};
-    load_and_launch(*K, [&]() { return gen_generic_kernel(P, outs, L, nd, K->name); }, P, shapes);
+    load_and_launch(*K, [&]() { return gen_generic_kernel(P, outs, L, nd, VEC, UNIT, NARROW, K->name); }, P, shapes);
     return true;
 }
 

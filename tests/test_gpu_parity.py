@@ -558,6 +558,37 @@ def test_softmax_and_moments_along_a_leading_axis(gpu, D, O, rng, shape):
         close(z, (x64 - x64.mean(axis, keepdims=True)) / np.sqrt(x64.var(axis, keepdims=True) + 1e-5), rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("shape", [(3, 5, 8), (7, 6, 20), (4, 3, 5, 12), (16, 33, 260), (5, 4, 7)])
+def test_strided_map_over_broadcast_inner_axes(gpu, D, rng, shape):
+    """N-D maps the 2-D model cannot express (an operand broadcast along a middle axis, strided views): one index
+    decomposition per four adjacent elements of a unit-stride last axis, one per element otherwise."""
+    x = rng.randn(*shape).astype(np.float32)
+    X = arr(D, x)
+    mid = list(shape)
+    mid[1] = 1
+    m = rng.randn(*mid).astype(np.float32)
+    last = list(shape)
+    last[-1] = 1
+    b = rng.randn(*last).astype(np.float32)
+    got = (X - arr(D, m)).numpy()
+    assert D.last_kernel_kinds() == "generic"
+    assert np.array_equal(got, x - m)
+    assert np.array_equal((X * arr(D, b) + arr(D, m)).numpy(), x * b + m)
+    # op-assign into a view that starts off a 16-byte boundary; int32 and fp64 operands
+    y = rng.randn(*shape[:-1], shape[-1] + 4).astype(np.float32)
+    dst, want = arr(D, y), y.copy()
+    dst.slice(len(shape) - 1, 1, shape[-1] + 1).assign(X * arr(D, m), 1)
+    want[..., 1:shape[-1] + 1] += x * m
+    assert np.array_equal(dst.numpy(), want)
+    xi = rng.randint(-50, 50, size=shape).astype(np.int32)
+    mi = rng.randint(-50, 50, size=mid).astype(np.int32)
+    assert np.array_equal((arr(D, xi) * arr(D, mi)).numpy(), xi * mi)
+    xd = rng.randn(*shape)
+    assert np.array_equal((arr(D, xd) + arr(D, m.astype(np.float64))).numpy(), xd + m.astype(np.float64))
+    # strided last axis: one element per thread
+    assert np.array_equal((X[:, 1:, ::2] * 2.0).numpy(), x[:, 1:, ::2] * np.float32(2.0))
+
+
 @pytest.mark.parametrize("n", [16, 17, 18, 19, 1023, 65537, 1000003])
 def test_flat_maps_and_full_reductions_off_the_vector_size(gpu, D, O, rng, n):
     """Element counts that are no multiple of four and views that start off a 16-byte boundary keep vector accesses;
