@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-28";
+const char* const kCodegenVersion = "dali-hip-codegen-29";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -491,6 +491,7 @@ struct RowParams {
     bool exact = false;      // register-cached rows: C == TPR * EPT * VEC, the chunk guards fall away
     bool ragged = false;     // rows not aligned to the vector: element-aligned vector accesses
     bool tail = false;       // ragged, and C is no multiple of VEC: the rest of a row is handled one element to a thread
+    int EPT_L = 0;           // cached rows: the last EPT_L of the EPT vectors a thread holds live in LDS instead of registers
 };
 
 int env_int(const char* name, int fallback) {
@@ -529,7 +530,7 @@ struct BodyEmitter {
 
     BodyEmitter(const Program& P_, const RowParams& rp_, bool per_el, int body, const std::vector<int>* fb)
         : P(P_), rp(rp_), per_element(per_el), body_index(body), first_body(fb) {
-        leaf_suffix = rp.cached ? "[e][j]" : "[j]";
+        leaf_suffix = rp.cached ? (rp.EPT_L > 0 ? "(e, j)" : "[e][j]") : "[j]";
     }
 
     // true when the node's value is the same for every element of a row (seen through broadcasts)
@@ -835,7 +836,35 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
     for (size_t i = 0; i < P.arrays.size(); ++i)
         if (!P.arrays[i].is_dest && P.arrays[i].cls == Cls::FULL && !P.arrays[i].gather_source) full_leaves.push_back((int)i);
     // is each leaf referenced? (an array may only be a gather source)
-    if (rp.cached) {
+    if (rp.cached && rp.EPT_L > 0) {
+        // Hybrid row cache: a thread keeps its first EPT_R vectors in registers and the other EPT_L in LDS (its own
+        // 16 bytes per slot, so no barrier is involved); two 1024-thread workgroups then fit a CU where the registers
+        // alone allow one, and one row's arithmetic overlaps the other's loads. `x<i>(e, j)` picks the storage; `e` is
+        // a constant after unrolling, so the selection folds away.
+        ss << "  constexpr int EPT_L = " << rp.EPT_L << ", EPT_R = EPT - EPT_L;\n";
+        for (int i : full_leaves) {
+            const std::string t = ctype(P.arrays[i].buf->dtype);
+            ss << "  " << t << " xr" << i << "[EPT_R + 1][VEC];\n";
+            ss << "  __shared__ __attribute__((aligned(16))) " << t << " xl" << i << "[EPT_L][" << rp.BT << " * VEC];\n";
+            ss << "#define x" << i << "(e, j) ((e) < EPT_R ? xr" << i << "[(e) < EPT_R ? (e) : 0][j] : ((e) >= EPT ? xr" << i << "[EPT_R][j] : xl" << i
+               << "[(e) >= EPT_R && (e) < EPT ? (e) - EPT_R : 0][tid * VEC + (j)]))\n";
+        }
+        ss << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n" << chunk_guard;
+        for (int i : full_leaves) {
+            const std::string t = ctype(P.arrays[i].buf->dtype);
+            ss << "      " << t << " ld" << i << "[VEC];\n";
+            emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "ld" + std::to_string(i), "      ", rp.nt_loads, rp.ragged);
+            ss << "      if (e < EPT_R) {\n        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) xr" << i << "[e < EPT_R ? e : 0][j] = ld" << i << "[j];\n      } else {\n";
+            ss << "        dali_vec<" << t << ", VEC> lv; _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) lv.v[j] = ld" << i << "[j];\n";
+            ss << "        dali_store<" << t << ", VEC>(&xl" << i << "[e >= EPT_R ? e - EPT_R : 0][tid * VEC], lv);\n      }\n";
+        }
+        ss << "    }\n  }\n";
+        if (tail) {
+            ss << "  if (tail_on) {\n";
+            for (int i : full_leaves) ss << "    xr" << i << "[EPT_R][0] = q" << i << "[tail_col];\n";
+            ss << "  }\n";
+        }
+    } else if (rp.cached) {
         for (int i : full_leaves) {
             ss << "  " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[EPT + " << (tail ? 1 : 0) << "][VEC];\n";
         }
@@ -847,6 +876,8 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
             for (int i : full_leaves) ss << "    x" << i << "[EPT][0] = q" << i << "[tail_col];\n";
             ss << "  }\n";
         }
+    }
+    if (rp.cached) {
         for (size_t id = 0; id < P.nodes.size(); ++id)
             if (P.nodes[id].kept) ss << "  " << ctype(P.nodes[id].dtype) << " t" << id << "[EPT + " << (tail ? 1 : 0) << "][VEC];\n";
     }
@@ -1294,7 +1325,23 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
     // 1024-thread workgroups: two per CU (8 waves per SIMD, 64 registers per thread) as long as the cached row fits that
     // budget; beyond ~44 cached values per thread the register cap would spill, so one workgroup per CU with twice the
     // registers ([2048,50257] 362 -> 200 us, [1024,65536] 169 -> 115 us; [8192,32000] stays at two)
-    const int64_t cached_values = rp.cached ? (int64_t)std::max(1, n_full) * rp.EPT * rp.VEC * (max_el / 4) : 0;
+    int64_t cached_values = rp.cached ? (int64_t)std::max(1, n_full) * rp.EPT * rp.VEC * (max_el / 4) : 0;
+    // ... unless the vectors beyond 40 registers' worth fit 64 KiB of LDS: then two workgroups per CU remain possible and
+    // one row's exponentials overlap the other's loads
+    static const int hybrid_env = env_int("DALI_HIP_ROW_LDS_CACHE", 1);
+    // (measured on softmax: [2048,50257] 201 -> 178 us, [2048,45000] 187 -> 155 us, [2048,38000] 134 -> 124 us; 32 values
+    // in registers where the rest fits the LDS budget, 36 otherwise; more than 36 spilled under the 64-register cap)
+    if (hybrid_env && rp.cached && nph > 0 && rp.BT == 1024 && rp.TPR == 1024 && cached_values > 32 && max_el == 4 && rp.VEC == 4 && n_full >= 1) {
+        for (int regs : {32, 36}) {
+            const int ept_r = regs / (n_full * rp.VEC);
+            const int ept_l = rp.EPT - ept_r;
+            if (ept_r >= 1 && ept_l >= 1 && (int64_t)n_full * ept_l * 1024 * rp.VEC * 4 <= (64 << 10)) {
+                rp.EPT_L = ept_l;
+                cached_values = (int64_t)n_full * ept_r * rp.VEC;
+                break;
+            }
+        }
+    }
     rp.waves_per_eu = nph > 0 ? (wpe >= 0 ? wpe : (rp.BT == 1024 ? (cached_values > 44 ? 4 : 8) : 0)) : 0;
 
     // cross-phase register caching of expensive shared values
@@ -1338,7 +1385,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
     rp.nt_loads = nt_l >= 0 ? nt_l != 0 : dom.R * dom.C * (int64_t)max_el >= ((int64_t)64 << 20);
     rp.nt_stores = nt_s >= 0 ? nt_s != 0 : true;
     params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached << "," << rp.waves_per_eu << ","
-           << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail;
+           << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail << "," << rp.EPT_L;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     std::string sig = signature(P, rpn.outputs);
     uint64_t h = kernel_hash("row", sig, params.str());

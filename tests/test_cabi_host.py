@@ -180,6 +180,18 @@ def test_rows_off_the_vector_alignment_keep_vector_accesses(D, rng):
     assert "dali_loadu" not in D.last_source()[D.last_source().index("void dali_row_"):]
 
 
+def test_long_cached_rows_put_part_of_the_row_into_lds(D, rng):
+    op = D.op
+    x = D.Array.from_numpy(np.zeros((4, 50257), np.float32))
+    D.generate_only([op.softmax(x)], compile=True)
+    body = D.last_source()
+    body = body[body.index("constexpr int EPT_L"):]
+    assert "EPT_L = 4" in body and "amdgpu_waves_per_eu(8, 8)" in D.last_source() and "__shared__ __attribute__((aligned(16))) float xl1[EPT_L][1024 * VEC]" in body
+    short = D.Array.from_numpy(np.zeros((4, 32000), np.float32))
+    D.generate_only([op.softmax(short)], compile=True)
+    assert "EPT_L" not in D.last_source()  # 32 cached values per thread: registers alone
+
+
 def test_planner_splits_what_cannot_fuse(D, rng):
     op = D.op
     m = D.Array.from_numpy(rng.randn(6, 8).astype(np.float32))

@@ -673,6 +673,30 @@ def test_fused_softmax_matches_oracle(gpu, D, O, rng, shape):
     close(s.sum(-1), 1.0, rtol=0, atol=2e-6)
 
 
+@pytest.mark.parametrize("cols", [33000, 36868, 45000, 49152, 50257, 53248, 57341])
+def test_rows_cached_partly_in_lds(gpu, D, O, rng, cols):
+    """Rows of 32K to 57K floats: a thread keeps the first vectors of its share in registers and the rest in LDS, so that
+    two 1024-thread workgroups still fit a CU. Every phase and the output read both parts."""
+    op = D.op
+    x = (rng.randn(3, cols) * 3).astype(np.float32)
+    X = arr(D, x)
+    s = op.softmax(X).numpy()
+    assert D.last_kernel_kinds() == "row"
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(-1, keepdims=True))
+    close(s, e / e.sum(-1, keepdims=True), rtol=1e-5, atol=1e-12)
+    close(s, O.softmax(x), rtol=seq_sum_rtol(cols), atol=1e-12)
+    z = ((X - op.mean(X, [1], True)) / op.sqrt(op.mean(op.square(X), [1], True) + 1.0)).numpy()
+    close(z, (x64 - x64.mean(1, keepdims=True)) / np.sqrt((x64 * x64).mean(1, keepdims=True) + 1.0), rtol=2e-5, atol=2e-5)
+    # += into the destination, int32 rows
+    y = rng.randn(3, cols).astype(np.float32)
+    dst = arr(D, y)
+    dst.assign(X - op.max(X, [1], True), 1)
+    assert np.array_equal(dst.numpy(), y + (x - x.max(1, keepdims=True)))
+    xi = rng.randint(-1000, 1000, size=(3, cols)).astype(np.int32)
+    assert np.array_equal((arr(D, xi) - op.min(arr(D, xi), [1], True)).numpy(), xi - xi.min(1, keepdims=True))
+
+
 def test_fused_softmax_equals_staged(gpu, D, rng):
     """JITCachedReduction.fused_softmax (tests.cpp:1622-1664): U(-20,20) [2,5], atol 1e-6."""
     op = D.op
