@@ -37,7 +37,16 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 // 16-byte accesses through the native vector type (an aggregate float4 copy is a memcpy to the
 // optimiser, which keeps the register stages from being promoted out of private memory)
+// (the load claims element alignment only: global memory takes a 16-byte access at any dword address as one
+// instruction, so operands whose rows start off a 16-byte boundary - an odd leading dimension, a view that starts inside
+// a row - go through the same kernels)
+typedef floatx4 floatx4u __attribute__((aligned(4)));
 __device__ __forceinline__ float4 ld16(const void* p) {
+    const floatx4 v = *(const floatx4u*)p;
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+// 16-byte aligned (LDS)
+__device__ __forceinline__ float4 ld16a(const void* p) {
     const floatx4 v = *(const floatx4*)p;
     return make_float4(v.x, v.y, v.z, v.w);
 }
@@ -303,7 +312,7 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
 #pragma unroll
         for (int ii = 0; ii < TM; ++ii) {
             int m = wm * WTM + ii * 32 + l32;
-            a4[ii] = ld16(&As[buf][m][swz(2 * t + h, m) << 2]);
+            a4[ii] = ld16a(&As[buf][m][swz(2 * t + h, m) << 2]);
         }
 #pragma unroll
         for (int jj = 0; jj < TN; ++jj)
@@ -672,6 +681,37 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
         }
         __syncthreads();
         if (!is_last) return;
+        // The fold: shares in z order per element, but the loads of four shares x sixteen elements are issued before
+        // the first of them is awaited (one awaited load per share and element cost ~270 ns each: 128 shares of a lone
+        // 64x64 tile took 550 us to fold).
+        constexpr int ZB = 4;
+#pragma unroll
+        for (int ii = 0; ii < TM; ++ii)
+#pragma unroll
+            for (int jj = 0; jj < TN; ++jj) {
+                const int ln = wn * WTN + jj * 32 + l32;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[0][ii][jj][v] = 0.f;
+                for (unsigned z0 = 0; z0 < gridDim.z; z0 += ZB) {
+                    float t[ZB][16];
+#pragma unroll
+                    for (int u = 0; u < ZB; ++u) {
+                        const bool on = z0 + u < gridDim.z;
+                        const float* src = part + (size_t)(on ? z0 + u : z0) * (BM * BN);
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int lm = wm * WTM + ii * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+                            t[u][v] = observe(src + lm * BN + ln);
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < ZB; ++u)
+                        if (z0 + u < gridDim.z) {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) acc[0][ii][jj][v] += t[u][v];
+                        }
+                }
+            }
     }
 #pragma unroll
     for (int ii = 0; ii < TM; ++ii)
@@ -691,14 +731,7 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
                         out_row = ((size_t)img * g.map_oh + i) * g.map_ow + j;
                     }
                     float* c = g.C + out_row * g.ldc + n;
-                    float sum;
-                    if (split) {
-                        int lm = m - m0, ln = n - n0;
-                        sum = 0.f;
-                        for (unsigned z = 0; z < gridDim.z; ++z) sum += observe(part + (size_t)z * (BM * BN) + lm * BN + ln);
-                    } else {
-                        sum = acc[0][ii][jj][v];
-                    }
+                    const float sum = acc[0][ii][jj][v];  // (with split-K: the fold above)
                     float r = alpha * sum;
                     if (beta != 0.f) r += beta * *c;
                     *c = r;
@@ -833,7 +866,7 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         sg.lda = lda[s];
         sg.ldb = ldb[s];
         sg.K = K[s];
-        vec = vec && aligned16(A[s]) && aligned16(B[s]) && lda[s] % 4 == 0 && ldb[s] % 4 == 0;
+        (void)aligned16;  // the vector kernels no longer need 16-byte aligned rows
     }
     g.M = M;
     g.N = N;
