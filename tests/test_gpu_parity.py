@@ -589,6 +589,43 @@ def test_strided_map_over_broadcast_inner_axes(gpu, D, rng, shape):
     assert np.array_equal((X[:, 1:, ::2] * 2.0).numpy(), x[:, 1:, ::2] * np.float32(2.0))
 
 
+@pytest.mark.parametrize("R,C", [(256, 256), (300, 517), (1000, 70), (64, 4097), (2048, 1024)])
+def test_map_over_transposed_matrices_is_one_launch(gpu, D, rng, R, C):
+    """Large transposed matrices among the operands of a map into a contiguous matrix: their tiles go through LDS inside
+    the one kernel that computes the map (edges, several transposed operands, op-assign, mixed dtypes, views)."""
+    op = D.op
+    a = rng.randn(C, R).astype(np.float32)   # read as a.T: [R, C]
+    b = rng.randn(R, C).astype(np.float32)
+    c = rng.randn(C, R).astype(np.float32)
+    A_, B_, C_ = arr(D, a), arr(D, b), arr(D, c)
+    before = D.jit_stats()["kernels"]
+    got = (A_.T + 1.0).numpy()
+    assert D.jit_stats()["kernels"] - before == 1 and D.last_kernel_kinds() == "tmap"
+    assert np.array_equal(got, a.T + np.float32(1.0))
+    got = (A_.T * B_ + op.exp(C_.T * 0.1)).numpy()
+    assert D.last_kernel_kinds() == "tmap"
+    close(got, a.T.astype(np.float64) * b + np.exp(c.T.astype(np.float64) * 0.1), rtol=1e-5, atol=1e-6)
+    # += into an existing matrix; a transposed view with a larger leading dimension; a one-element operand
+    dst, want = arr(D, b), b.copy()
+    dst.assign(A_.T * 2.0, 1)
+    want += a.T * np.float32(2.0)
+    assert np.array_equal(dst.numpy(), want)
+    wide = rng.randn(C, R + 8).astype(np.float32)
+    s = arr(D, np.array([[3.0]], np.float32))
+    assert np.array_equal((arr(D, wide)[:, 4:R + 4].T * s).numpy(), wide[:, 4:R + 4].T * np.float32(3.0))
+    # fp64 and int32 operands
+    ad = rng.randn(C, R)
+    assert np.array_equal((arr(D, ad).T - arr(D, b.astype(np.float64))).numpy(), ad.T - b.astype(np.float64))
+    ai = rng.randint(-100, 100, size=(C, R)).astype(np.int32)
+    assert np.array_equal((arr(D, ai).T * 3).numpy(), ai.T * 3)
+    # the destination's own memory among the transposed operands is not a candidate (the result must still be right)
+    if R == C:
+        sq = rng.randn(R, R).astype(np.float32)
+        S = arr(D, sq)
+        S.assign(S.T + 1.0, 0)
+        assert np.array_equal(S.numpy(), sq.T + np.float32(1.0))
+
+
 @pytest.mark.parametrize("n", [16, 17, 18, 19, 1023, 65537, 1000003])
 def test_flat_maps_and_full_reductions_off_the_vector_size(gpu, D, O, rng, n):
     """Element counts that are no multiple of four and views that start off a 16-byte boundary keep vector accesses;
