@@ -60,9 +60,12 @@ class Gen(object):
                 return a + op.abs(b), ra + np.abs(rb)
             return a * b, ra * rb
         if choice == 3:
-            # broadcast of a row-wise (keepdims) reduction back onto the rows
+            # broadcast of a keepdims reduction back onto the operand: along the rows most of the time, along a leading or
+            # middle axis otherwise (column maxima / sums: operands that are constant along the reduced axis)
             a, ra = self.full(depth - 1)
             axis = len(self.shape) - 1
+            if len(self.shape) >= 2 and rng.randint(3) == 0:
+                axis = rng.randint(len(self.shape) - 1)
             if rng.randint(2):
                 return a - op.max(a, [axis], True), ra - ra.max(axis=axis, keepdims=True)
             self.size_terms = max(self.size_terms, self.shape[axis])
