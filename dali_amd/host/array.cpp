@@ -1,5 +1,6 @@
 // Array handles, buffer views, memory placement and the op:: factories.
 #include <algorithm>
+#include <limits>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -756,12 +757,29 @@ Array add(const std::vector<Array>& arrays) {
     return out;
 }
 
+// A reduction over no elements is the reducer's initial value: the reference's loops never run and store what
+// SetInitValue left (dali/array/jit/reducer_kernels.h:57-169, all_reduce_kernel_utils.cpp:105-154). No kernel is
+// planned for it; the result is a buffer filled with that value.
+static Array reduction_of_nothing(const std::vector<int>& shape, const std::string& reducer_name, DType dtype) {
+    Array out(shape, dtype);
+    if (out.number_of_elements() == 0) return out;
+    if (reducer_name == "reducers::sum") return out.assign(Array(0));
+    if (reducer_name == "reducers::product") return out.assign(Array(1));
+    const bool is_max = reducer_name == "reducers::maximum";
+    DALI_ASSERT(is_max || reducer_name == "reducers::minimum", make_message("reduction of an empty array by ", reducer_name));
+    if (dtype == DTYPE_INT32) return out.assign(Array(is_max ? std::numeric_limits<int>::min() : std::numeric_limits<int>::max()));
+    if (dtype == DTYPE_DOUBLE) return out.assign(Array(is_max ? -std::numeric_limits<double>::max() : std::numeric_limits<double>::max()));
+    return out.assign(Array(is_max ? -std::numeric_limits<float>::max() : std::numeric_limits<float>::max()));
+}
+
 Array all_reduce(const Array& a, const std::string& reducer_name) {
+    if (a.number_of_elements() == 0) return reduction_of_nothing({}, reducer_name, a.dtype());
     return make_node(Kind::ALL_REDUCE, reducer_name, {a}, {}, a.dtype());
 }
 
 static Array axis_reduce_last(const Array& a, const std::string& reducer_name) {
     std::vector<int> shape(a.shape().begin(), a.shape().end() - 1);
+    if (a.shape().back() == 0) return reduction_of_nothing(shape, reducer_name, a.dtype());
     return make_node(Kind::AXIS_REDUCE, reducer_name, {a}, shape, a.dtype());
 }
 
@@ -844,6 +862,7 @@ Array axis_reduce(const Array& a, const std::string& reducer_name, const std::ve
 // The reference stores a flat argmax in the INPUT dtype
 // (dali/array/op/reducer_operation.cpp:681-684).
 Array argument_all_reduce(const Array& a, const std::string& reducer_name) {
+    if (a.number_of_elements() == 0) return reduction_of_nothing({}, "reducers::sum", a.dtype());  // the index stays 0
     return make_node(Kind::ARG_ALL_REDUCE, reducer_name, {a}, {}, a.dtype());
 }
 
@@ -859,6 +878,7 @@ Array argument_axis_reduce(const Array& a, const std::string& reducer_name, int 
     Array res = a;
     if (axis != ndim - 1) res = res.swapaxes(axis, ndim - 1);
     std::vector<int> shape(res.shape().begin(), res.shape().end() - 1);
+    if (res.shape().back() == 0) return reduction_of_nothing(shape, "reducers::sum", DTYPE_INT32);  // the index stays 0
     return make_node(Kind::ARG_AXIS_REDUCE, reducer_name, {res}, shape, DTYPE_INT32);
 }
 

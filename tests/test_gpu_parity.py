@@ -1353,3 +1353,57 @@ def test_circular_convolution_matches_oracle(gpu, D, O, rng, shape):
     if len(shape) == 1:
         wide = rng.uniform(-1, 1, 2 * shape[0]).astype(np.float32)
         assert np.array_equal(D.op.circular_convolution(arr(D, x), arr(D, wide)[::2]).numpy(), O.circular_convolution(x, wide[::2]))
+
+
+def test_degenerate_extents(gpu, D, rng):
+    """Zero and unit extents. A reduction over no elements stores the reducer's initial value, which is what the
+    reference's loops leave when they never run (reducer_kernels.h:57-169, all_reduce_kernel_utils.cpp:105-154)."""
+    op, f32 = D.op, np.float32
+    fmax = np.finfo(f32).max
+    none_of_7, five_of_none = np.zeros((0, 7), f32), np.zeros((5, 0), f32)
+    assert op.sum(arr(D, none_of_7), [1]).numpy().shape == (0,)
+    assert np.array_equal(op.sum(arr(D, none_of_7), [0]).numpy(), np.zeros(7, f32))
+    assert np.array_equal(op.sum(arr(D, five_of_none), [1]).numpy(), np.zeros(5, f32))
+    assert np.array_equal(op.prod(arr(D, five_of_none), [1], True).numpy(), np.ones((5, 1), f32))
+    assert np.array_equal(op.max(arr(D, five_of_none), [1]).numpy(), np.full(5, -fmax, f32))
+    assert np.array_equal(op.min(arr(D, five_of_none), [1]).numpy(), np.full(5, fmax, f32))
+    assert np.array_equal(op.max(arr(D, np.zeros((5, 0), np.int32)), [1]).numpy(), np.full(5, np.iinfo(np.int32).min, np.int32))
+    assert np.array_equal(op.min(arr(D, np.zeros((5, 0), np.float64)), [1]).numpy(), np.full(5, np.finfo(np.float64).max))
+    assert float(op.sum(arr(D, np.zeros(0, f32))).numpy()) == 0.0
+    assert float(op.prod(arr(D, np.zeros(0, f32))).numpy()) == 1.0
+    am = op.argmax(arr(D, five_of_none), 1).numpy()
+    assert am.dtype == np.int32 and np.array_equal(am, np.zeros(5, np.int32))
+    assert np.isnan(float(op.mean(arr(D, np.zeros(0, f32))).numpy()))  # 0 / 0
+    x = rng.randn(3, 4).astype(f32)  # an empty reduction under further arithmetic
+    assert np.array_equal((arr(D, x) + op.sum(arr(D, np.zeros((3, 0), f32)), [1], True)).numpy(), x)
+    # maps, softmax and index operators over nothing
+    assert op.softmax(arr(D, none_of_7)).numpy().shape == (0, 7)
+    assert (arr(D, none_of_7).transpose(1, 0) + 1.0).numpy().shape == (7, 0)
+    t = rng.randn(6, 3).astype(f32)
+    nothing = np.zeros(0, np.int32)
+    assert op.gather(arr(D, t), arr(D, nothing)).numpy().shape == (0, 3)
+    assert op.gather_from_rows(arr(D, t), arr(D, nothing)).numpy().shape == (0,)
+    assert op.one_hot(arr(D, nothing), 4, 1.0, 0.0).numpy().shape == (0, 4)
+    assert op.cumsum(arr(D, np.zeros(0, f32))).numpy().shape == (0,)
+    assert op.outer(arr(D, np.zeros(0, f32)), arr(D, t[0])).numpy().shape == (0, 3)
+    assert np.array_equal(op.concatenate([arr(D, t), arr(D, np.zeros((0, 3), f32)), arr(D, t)], 0).numpy(), np.concatenate([t, t], 0))
+    with pytest.raises(D.DaliError, match="arange's size must be strictly positive"):  # arange.cpp:62-66
+        op.arange(0)
+    # products with an empty contraction are zeros, with no rows are empty
+    assert np.array_equal(op.dot(arr(D, np.zeros((3, 0), f32)), arr(D, np.zeros((0, 4), f32))).numpy(), np.zeros((3, 4), f32))
+    assert op.dot(arr(D, np.zeros((0, 3), f32)), arr(D, t.T.copy()[:, :4])).numpy().shape == (0, 4)
+    # unit extents
+    one = rng.randn(5, 1).astype(f32)
+    assert np.array_equal(op.softmax(arr(D, one)).numpy(), np.ones((5, 1), f32))
+    assert np.array_equal(op.cumsum(arr(D, one)).numpy(), one)
+    row = rng.randn(1, 5).astype(f32)
+    assert np.array_equal(op.argmax(arr(D, row), 1).numpy(), row.argmax(1).astype(np.int32))
+    assert np.array_equal(op.argmax(arr(D, row), 0).numpy(), np.zeros(5, np.int32))
+    assert np.array_equal(op.eye(1).numpy(), np.eye(1))
+    # one very long row, one very tall column
+    big = rng.randn(1, 200001).astype(f32)
+    e = np.exp(big.astype(np.float64) - big.max())
+    close(op.softmax(arr(D, big)).numpy(), e / e.sum(), rtol=2e-5, atol=1e-12)
+    tall = rng.randn(200001, 1).astype(f32)
+    assert abs(float(op.sum(arr(D, tall), [0]).numpy()[0]) - tall.astype(np.float64).sum()) <= 1e-5 * np.abs(tall).sum()
+    assert int(op.argmax(arr(D, tall), 0).numpy()[0]) == int(tall.argmax())
