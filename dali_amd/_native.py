@@ -162,6 +162,7 @@ FRONT_SYMBOLS = {
     "dali_fe_autoreduce_assign": (_i, [H, H]),
     "dali_fe_one_hot": (H, [H, _i, H, H]),
     "dali_fe_dot": (H, [H, H]),
+    "dali_fe_tensordot": (H, [H, H, _i, _ip, _ip]),
     "dali_fe_softmax_cross_entropy": (_i, [H, H, _HP, _HP, _HP]),
     "dali_fe_lstm_step": (_i, [H, H, H, H, H, H, _HP, _HP]),
     "dali_fe_lstm_sequence": (_i, [H, H, H, H, H, H, _HP, _HP, _HP]),

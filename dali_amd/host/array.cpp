@@ -1392,11 +1392,86 @@ Array matmul(Array a, Array b) {
     return make_node(Kind::MATMUL, "", {a, b}, {a.shape()[0], b.shape()[1]}, t);
 }
 
-// dali/array/op/dot.cpp:104-124 (tensordot of rank > 2 operands is not part of this path)
+// A [rows, cols] matrix made of `x` with its axes taken in the order `order`, the first `lead` of them forming the rows.
+// Dense buffers whose order is the identity or a rotation become a view (the rotation is a transposed matrix, which the
+// GEMM reads in place); any other order is written out once.
+static Array as_matrix(const Array& x, const std::vector<int>& order, int lead) {
+    const int nd = x.ndim();
+    int64_t rows = 1, cols = 1;
+    for (int i = 0; i < nd; ++i) (i < lead ? rows : cols) *= x.shape()[order[i]];
+    DALI_ASSERT(rows <= std::numeric_limits<int>::max() && cols <= std::numeric_limits<int>::max(), "tensordot: operand too large");
+    bool identity = true, rotation = true;
+    for (int i = 0; i < nd; ++i) {
+        identity = identity && order[i] == i;
+        rotation = rotation && order[i] == (i + (nd - lead)) % nd;
+    }
+    if (identity) return x.reshape({(int)rows, (int)cols});
+    if (rotation && x.is_buffer() && x.contiguous_memory()) return x.reshape({(int)cols, (int)rows}).transpose();
+    return x.transpose(order).reshape({(int)rows, (int)cols});
+}
+
+static void check_tensordot_axes(const Array& x, char name, std::vector<int>& axes) {
+    const int nd = x.ndim();
+    DALI_ASSERT((int)axes.size() <= nd, make_message("tensordot's length of argument ", name, "_reduce_axes should be less than the dimensions of ",
+                                                     name, " (", name, ".ndim = ", nd, ", ", name, "_reduce_axes.size() = ", axes.size(), ")."));
+    std::vector<bool> seen(nd, false);
+    for (int& ax : axes) {
+        if (ax < 0) ax += nd;
+        DALI_ASSERT(ax >= 0 && ax < nd, make_message(name, "_reduce_axes contains reduction dimensions that are greater than or equal to ", name,
+                                                     ".ndim (", name, ".ndim = ", nd, ", and found ", ax, ")."));
+        DALI_ASSERT(!seen[ax], make_message("tensordot: axis ", ax, " of ", name, " is named twice."));
+        seen[ax] = true;
+    }
+}
+
+// dali/array/gemm/tensordot_as_dot.h:120-158: the kept axes of a, then its reduced axes, against the reduced axes of b,
+// then its kept ones; one matrix product; the result has the kept axes of a followed by those of b.
+Array tensordot(const Array& a, const Array& b, const std::vector<int>& a_reduce_axes, const std::vector<int>& b_reduce_axes) {
+    DALI_ASSERT(a_reduce_axes.size() == b_reduce_axes.size(),
+                make_message("tensordot_as_dot must have as many reduction axes for a than b (got a_reduce_axes.size() = ", a_reduce_axes.size(),
+                             " and b_reduce_axes.size() = ", b_reduce_axes.size(), ")."));
+    std::vector<int> ra = a_reduce_axes, rb = b_reduce_axes;
+    check_tensordot_axes(a, 'a', ra);
+    check_tensordot_axes(b, 'b', rb);
+    std::vector<int> order_a, order_b = rb, out_shape;
+    for (int i = 0; i < a.ndim(); ++i)
+        if (std::find(ra.begin(), ra.end(), i) == ra.end()) {
+            order_a.push_back(i);
+            out_shape.push_back(a.shape()[i]);
+        }
+    const int kept_a = (int)order_a.size();
+    order_a.insert(order_a.end(), ra.begin(), ra.end());
+    for (int i = 0; i < b.ndim(); ++i)
+        if (std::find(rb.begin(), rb.end(), i) == rb.end()) {
+            order_b.push_back(i);
+            out_shape.push_back(b.shape()[i]);
+        }
+    for (size_t i = 0; i < ra.size(); ++i)
+        DALI_ASSERT(a.shape()[ra[i]] == b.shape()[rb[i]],
+                    make_message("tensordot shapes not aligned, with a.shape = ", shape_str(a.shape()), " and b.shape = ", shape_str(b.shape()),
+                                 ": a.shape[", ra[i], "] = ", a.shape()[ra[i]], " != b.shape[", rb[i], "] = ", b.shape()[rb[i]], "."));
+    return matmul(as_matrix(a, order_a, kept_a), as_matrix(b, order_b, (int)rb.size())).reshape(out_shape);
+}
+
+// dali/array/gemm/tensordot_as_dot.h:48-118: the last `axis` axes of a against the first `axis` axes of b
+Array tensordot(const Array& a, const Array& b, int axis) {
+    DALI_ASSERT(axis >= 0, make_message("tensordot_as_dot axis must be a non-negative integer (got axis = ", axis, ")."));
+    DALI_ASSERT(axis <= a.ndim(), make_message("tensordot_as_dot axis can not be larger than the dimension of a (a.ndim() = ", a.ndim(), ", axis = ", axis, ")."));
+    DALI_ASSERT(axis <= b.ndim(), make_message("tensordot_as_dot axis can not be larger than the dimension of b (b.ndim() = ", b.ndim(), ", axis = ", axis, ")."));
+    std::vector<int> ra, rb;
+    for (int i = 0; i < axis; ++i) {
+        ra.push_back(a.ndim() - axis + i);
+        rb.push_back(i);
+    }
+    return tensordot(a, b, ra, rb);
+}
+
+// dali/array/op/dot.cpp:104-124
 Array dot(const Array& a, const Array& b) {
     int an = a.ndim(), bn = b.ndim();
     if (an == 0 || bn == 0) return eltmul(a, b);
-    DALI_ASSERT(an <= 2 && bn <= 2, "dot: operands of rank > 2 (tensordot) are not implemented");
+    // a is reduced over its last axis, b over its second to last one (its only one when it is a vector)
+    if (an > 2 || bn > 2) return tensordot(a, b, std::vector<int>{an - 1}, std::vector<int>{std::max(0, bn - 2)});
     if (an == 1 && bn == 1) {
         DALI_ASSERT(a.shape()[0] == b.shape()[0], make_message("inner input shapes a.shape = ", shape_str(a.shape()),
                                                                " and b.shape = ", shape_str(b.shape()), " should be equal."));

@@ -171,6 +171,12 @@ dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_va
     FE_TRY(return wrap(dali::op::one_hot(A(indices), depth, A(on_value), A(off_value)));, nullptr)
 }
 dali_array_t dali_fe_dot(dali_array_t a, dali_array_t b) { FE_TRY(return wrap(dali::op::dot(A(a), A(b)));, nullptr) }
+dali_array_t dali_fe_tensordot(dali_array_t a, dali_array_t b, int n_axes, const int* a_reduce_axes, const int* b_reduce_axes) {
+    FE_TRY(if (!a_reduce_axes || !b_reduce_axes) return wrap(dali::op::tensordot(A(a), A(b), n_axes));
+           return wrap(dali::op::tensordot(A(a), A(b), std::vector<int>(a_reduce_axes, a_reduce_axes + n_axes),
+                                           std::vector<int>(b_reduce_axes, b_reduce_axes + n_axes)));
+           , nullptr)
+}
 
 int dali_fe_softmax_cross_entropy(dali_array_t logits, dali_array_t targets, dali_array_t* mean_loss, dali_array_t* row_loss,
                                   dali_array_t* grad) {

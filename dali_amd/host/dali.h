@@ -325,6 +325,8 @@ Array& autoreduce_assign(Array& left, const Array& right);
 Array one_hot(Array indices, int depth, Array on_value, Array off_value);
 Array matmul(Array a, Array b);
 Array dot(const Array& a, const Array& b);
+Array tensordot(const Array& a, const Array& b, int axis);
+Array tensordot(const Array& a, const Array& b, const std::vector<int>& a_reduce_axes, const std::vector<int>& b_reduce_axes);
 
 // Softmax cross-entropy with integer targets in log-sum-exp form
 // (definition: dali/tensor/op/cost.cpp:115-133). Returns {mean loss (scalar),

@@ -162,6 +162,19 @@ def dot(a, b):
     return _wrap(front.dali_fe_dot(a._h, b._h), "dot")
 
 
+def tensordot(a, b, axes):
+    """``axes`` = a count (the last axes of a against the first of b) or a pair of axis lists (dali/array/op/dot.cpp:92-98)."""
+    a, b = as_array(a), as_array(b)
+    if isinstance(axes, int):
+        return _wrap(front.dali_fe_tensordot(a._h, b._h, axes, None, None), "tensordot")
+    a_axes, b_axes = axes
+    if len(a_axes) != len(b_axes):
+        raise DaliError("tensordot_as_dot must have as many reduction axes for a than b")
+    pa, n = _ints(a_axes)
+    pb, _ = _ints(b_axes)
+    return _wrap(front.dali_fe_tensordot(a._h, b._h, n, pa, pb), "tensordot")
+
+
 def softmax_cross_entropy(logits, targets):
     """(mean loss, per-row loss, gradient) of the LSE-form softmax cross-entropy, evaluated together."""
     outs = [C.c_void_p() for _ in range(3)]

@@ -102,7 +102,13 @@ dali_array_t dali_fe_outer(dali_array_t a, dali_array_t b);
 /* dest <<= source (dali/array/expression/assignment.cpp:92-126) */
 int dali_fe_autoreduce_assign(dali_array_t dest, dali_array_t source);
 dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_value, dali_array_t off_value);
+/* op::dot (dali/array/op/dot.cpp:104-124): scalars multiply, vectors and matrices go to one matrix product, operands of
+ * more than two dimensions to tensordot over a's last axis and b's second to last */
 dali_array_t dali_fe_dot(dali_array_t a, dali_array_t b);
+/* op::tensordot (dali/array/op/dot.cpp:92-98, dali/array/gemm/tensordot_as_dot.h:48-158). With both axis lists NULL the
+ * last n_axes axes of a are summed against the first n_axes axes of b; otherwise axis a_reduce_axes[i] of a against axis
+ * b_reduce_axes[i] of b. The result holds the kept axes of a, then those of b. */
+dali_array_t dali_fe_tensordot(dali_array_t a, dali_array_t b, int n_axes, const int* a_reduce_axes, const int* b_reduce_axes);
 
 /* composites evaluated as one fused group */
 int dali_fe_softmax_cross_entropy(dali_array_t logits, dali_array_t targets, dali_array_t* mean_loss,

@@ -833,6 +833,60 @@ def test_dot_known_answers_and_laziness(gpu, D, rng):
     assert dst.numpy().tolist() == [[13, 16, 19, 22], [13, 16, 19, 22]]
 
 
+def test_tensordot_alignment_rules_and_values(gpu, D, rng):
+    """ArrayDotTests.tensordot_alignment_rules (dot_tests.cpp:157-224): which shapes `dot` accepts and what it returns,
+    and tensordot over two axis pairs against the five-deep loop of dot_tests.cpp:120-148."""
+    op = D.op
+    lefts = [(2,), (2, 4), (6, 2, 4), (8, 6, 2, 4), (10, 8, 6, 2, 4)]
+    rights = [(2,), (4,), (4, 2), (6, 4, 2), (8, 6, 4, 2), (10, 8, 6, 4, 2)]
+    checked = 0
+    for ls in lefts:
+        for rs in rights:
+            inner_l, inner_r = ls[-1], rs[max(0, len(rs) - 2)]
+            a = rng.randint(-3, 4, ls).astype(np.float32)
+            b = rng.randint(-3, 4, rs).astype(np.float32)
+            if inner_l != inner_r:
+                with pytest.raises(D.DaliError):
+                    op.dot(arr(D, a), arr(D, b))
+                continue
+            got = op.dot(arr(D, a), arr(D, b)).numpy()
+            want = np.dot(a, b)  # numpy's dot has the same rule: last axis of a, second to last of b
+            assert got.shape == want.shape == tuple(ls[:-1]) + tuple(rs[:max(0, len(rs) - 2)]) + tuple(rs[len(rs) - 1:] if len(rs) > 1 else ())
+            assert np.array_equal(got, want)  # small integers: exact in any summation order
+            checked += 1
+    assert checked == 21
+    with pytest.raises(D.DaliError):
+        op.dot(arr(D, np.zeros(4, np.float32)), arr(D, np.zeros(2, np.float32)))
+    a = rng.uniform(0, 1, (2, 3, 4)).astype(np.float32)
+    b = rng.uniform(0, 1, (5, 6, 4, 3)).astype(np.float32)
+    want = np.zeros((2, 5, 6))
+    for i in range(2):
+        for j in range(5):
+            for k in range(6):
+                for l in range(3):
+                    for m in range(4):
+                        want[i, j, k] += float(a[i, l, m]) * float(b[j, k, m, l])
+    got = op.tensordot(arr(D, a), arr(D, b), ([1, 2], [3, 2])).numpy()
+    assert got.shape == (2, 5, 6)
+    close(got, want, rtol=1e-5, atol=1e-6)
+    # a count of axes: the trailing axes of a against the leading axes of b; a rotation of a dense operand is read in place
+    x = rng.randn(3, 4, 5).astype(np.float32)
+    y = rng.randn(4, 5, 7).astype(np.float32)
+    close(op.tensordot(arr(D, x), arr(D, y), 2).numpy(), np.tensordot(x.astype(np.float64), y, 2), rtol=1e-4, atol=1e-5)
+    before = D.jit_stats()["kernels"]
+    z = op.tensordot(arr(D, y), arr(D, x), ([0, 1], [1, 2])).numpy()
+    assert D.jit_stats()["kernels"] == before  # no copies: [4,5,7] reduced over its leading axes is a transposed [20,7] matrix
+    close(z, np.tensordot(y.astype(np.float64), x, ([0, 1], [1, 2])), rtol=1e-4, atol=1e-5)
+    close(op.tensordot(arr(D, x), arr(D, y), 0).numpy().reshape(60, 140), np.outer(x.ravel(), y.ravel()), rtol=1e-6)
+    close(op.tensordot(arr(D, x), arr(D, y), ([-1, 1], [1, 0])).numpy(), np.tensordot(x.astype(np.float64), y, ([2, 1], [1, 0])), rtol=1e-4, atol=1e-5)
+    with pytest.raises(D.DaliError, match="not aligned"):
+        op.tensordot(arr(D, x), arr(D, y), ([0], [0]))
+    with pytest.raises(D.DaliError, match="named twice"):
+        op.tensordot(arr(D, x), arr(D, y), ([1, 1], [0, 0]))
+    with pytest.raises(D.DaliError, match="can not be larger"):
+        op.tensordot(arr(D, x), arr(D, y), 4)
+
+
 @pytest.mark.parametrize("B,I,H", [(3, 8, 8), (32, 100, 64), (17, 33, 20)])
 def test_lstm_step_matches_oracle(gpu, D, O, rng, B, I, H):
     X, Hp, Cp = (rng.randn(B, n).astype(np.float32) for n in (I, H, H))
