@@ -162,6 +162,10 @@ FRONT_SYMBOLS = {
     "dali_fe_autoreduce_assign": (_i, [H, H]),
     "dali_fe_one_hot": (H, [H, _i, H, H]),
     "dali_fe_dot": (H, [H, H]),
+    "dali_fe_inner": (H, [H, H]),
+    "dali_fe_matrix_vector_dot": (H, [H, H]),
+    "dali_fe_ceil": (H, [H]),
+    "dali_fe_softmax_temperature": (H, [H, H, _i]),
     "dali_fe_tensordot": (H, [H, H, _i, _ip, _ip]),
     "dali_fe_softmax_cross_entropy": (_i, [H, H, _HP, _HP, _HP]),
     "dali_fe_lstm_step": (_i, [H, H, H, H, H, H, _HP, _HP]),

@@ -680,6 +680,15 @@ Array round(Array a) {
     return make_node(Kind::ELEMENTWISE, "functor::round", {a}, a.shape(), DTYPE_INT32);
 }
 
+// dali/array/op/elementwise_operation.cpp:155-160 (the reference names a functor "ceiling" that functor.h:150-155 defines
+// as "ceil"; the result is int32 like round's)
+Array ceil(Array a) {
+    if (a.dtype() == DTYPE_INT32) return a;
+    auto e = a.expression();
+    if (e->kind == Kind::SCALAR) return Array((int)std::ceil(e->dvalue));
+    return make_node(Kind::ELEMENTWISE, "functor::ceil", {a}, a.shape(), DTYPE_INT32);
+}
+
 // dali/array/op/elementwise_operation.cpp:137-139
 Array astype(Array a, DType dtype) { return dtype == DTYPE_INT32 ? round(a) : unsafe_cast(a, dtype); }
 
@@ -929,6 +938,12 @@ Array all_close(const Array& left, const Array& right, const Array& atolerance) 
 Array softmax(const Array& logits, int axis) {
     Array exped = exp(subtract(logits, max(logits, {axis}, true)));
     return eltdiv(exped, sum(exped, {axis}, true));
+}
+
+// dali/array/op/softmax.cpp:10-13: the reference does not read `temperature`; the result is softmax(logits, axis)
+Array softmax_temperature(const Array& logits, const Array& temperature, int axis) {
+    (void)temperature;
+    return softmax(logits, axis);
 }
 
 // dali/array/op/gather_from_rows.cpp:110-127
@@ -1466,19 +1481,20 @@ Array tensordot(const Array& a, const Array& b, int axis) {
     return tensordot(a, b, ra, rb);
 }
 
-// dali/array/op/dot.cpp:104-124
-Array dot(const Array& a, const Array& b) {
-    int an = a.ndim(), bn = b.ndim();
-    if (an == 0 || bn == 0) return eltmul(a, b);
-    // a is reduced over its last axis, b over its second to last one (its only one when it is a vector)
-    if (an > 2 || bn > 2) return tensordot(a, b, std::vector<int>{an - 1}, std::vector<int>{std::max(0, bn - 2)});
-    if (an == 1 && bn == 1) {
-        DALI_ASSERT(a.shape()[0] == b.shape()[0], make_message("inner input shapes a.shape = ", shape_str(a.shape()),
-                                                               " and b.shape = ", shape_str(b.shape()), " should be equal."));
-        return matmul(a.reshape({1, a.number_of_elements()}), b.reshape({b.number_of_elements(), 1})).reshape({});
-    }
-    if (an == 2 && bn == 2) return matmul(a, b);
-    if (an == 1) {
+// dali/array/op/dot.cpp:100-102
+Array inner(const Array& a, const Array& b) {
+    DALI_ASSERT(a.ndim() == 1 && b.ndim() == 1,
+                make_message("inner expects vector inputs but got a.ndim = ", a.ndim(), " and b.ndim = ", b.ndim(), " arrays."));
+    DALI_ASSERT(a.shape()[0] == b.shape()[0], make_message("inner input shapes a.shape = ", shape_str(a.shape()),
+                                                           " and b.shape = ", shape_str(b.shape()), " should be equal."));
+    return matmul(a.reshape({1, a.number_of_elements()}), b.reshape({b.number_of_elements(), 1})).reshape({});
+}
+
+// dali/array/op/dot.cpp:67-90
+Array matrix_vector_dot(const Array& a, const Array& b) {
+    DALI_ASSERT((a.ndim() == 1 && b.ndim() == 2) || (a.ndim() == 2 && b.ndim() == 1),
+                make_message("matrix_vector_dot inputs must be a vector and a matrix, but got a.ndim = ", a.ndim(), " and b.ndim = ", b.ndim(), "."));
+    if (a.ndim() == 1) {
         DALI_ASSERT(b.shape()[0] == a.shape()[0], make_message("matrix_vector_dot shape mistmach between a.shape = ", shape_str(a.shape()),
                                                                " and b.shape = ", shape_str(b.shape()), "."));
         return matmul(a.reshape({1, a.number_of_elements()}), b).reshape({b.shape()[1]});
@@ -1486,6 +1502,17 @@ Array dot(const Array& a, const Array& b) {
     DALI_ASSERT(a.shape()[1] == b.shape()[0], make_message("matrix_vector_dot shape mistmach between a.shape = ", shape_str(a.shape()),
                                                            " and b.shape = ", shape_str(b.shape()), "."));
     return matmul(a, b.reshape({b.number_of_elements(), 1})).reshape({a.shape()[0]});
+}
+
+// dali/array/op/dot.cpp:104-124
+Array dot(const Array& a, const Array& b) {
+    int an = a.ndim(), bn = b.ndim();
+    if (an == 0 || bn == 0) return eltmul(a, b);
+    // a is reduced over its last axis, b over its second to last one (its only one when it is a vector)
+    if (an > 2 || bn > 2) return tensordot(a, b, std::vector<int>{an - 1}, std::vector<int>{std::max(0, bn - 2)});
+    if (an == 1 && bn == 1) return inner(a, b);
+    if (an == 2 && bn == 2) return matmul(a, b);
+    return matrix_vector_dot(a, b);
 }
 
 CrossEntropyResult softmax_cross_entropy(const Array& logits, const Array& targets) {

@@ -93,6 +93,7 @@ dali_array_t dali_fe_unary(const char* functor_name, dali_array_t a) {
 dali_array_t dali_fe_binary(const char* functor_name, dali_array_t a, dali_array_t b) {
     FE_TRY(return wrap(dali::op::elementwise(A(a), A(b), qualified(functor_name, "functor")));, nullptr)
 }
+dali_array_t dali_fe_ceil(dali_array_t a) { FE_TRY(return wrap(dali::op::ceil(A(a)));, nullptr) }
 dali_array_t dali_fe_astype(dali_array_t a, int dtype) { FE_TRY(return wrap(dali::op::astype(A(a), (dali::DType)dtype));, nullptr) }
 dali_array_t dali_fe_all_reduce(const char* r, dali_array_t a) {
     FE_TRY(return wrap(dali::op::all_reduce(A(a), qualified(r, "reducers")));, nullptr)
@@ -111,6 +112,9 @@ dali_array_t dali_fe_mean_axes(dali_array_t a, const int* axes, int naxes, int k
     FE_TRY(return wrap(dali::op::mean(A(a), vec(axes, naxes), keepdims != 0));, nullptr)
 }
 dali_array_t dali_fe_softmax(dali_array_t a, int axis) { FE_TRY(return wrap(dali::op::softmax(A(a), axis));, nullptr) }
+dali_array_t dali_fe_softmax_temperature(dali_array_t a, dali_array_t temperature, int axis) {
+    FE_TRY(return wrap(dali::op::softmax_temperature(A(a), A(temperature), axis));, nullptr)
+}
 dali_array_t dali_fe_gather_from_rows(dali_array_t s, dali_array_t i) { FE_TRY(return wrap(dali::op::gather_from_rows(A(s), A(i)));, nullptr) }
 dali_array_t dali_fe_gather(dali_array_t s, dali_array_t i) { FE_TRY(return wrap(dali::op::gather(A(s), A(i)));, nullptr) }
 int dali_fe_autoreduce_assign(dali_array_t dest, dali_array_t source) { FE_TRY(dali::op::autoreduce_assign(A(dest), A(source)); return 0;, 1) }
@@ -171,6 +175,8 @@ dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_va
     FE_TRY(return wrap(dali::op::one_hot(A(indices), depth, A(on_value), A(off_value)));, nullptr)
 }
 dali_array_t dali_fe_dot(dali_array_t a, dali_array_t b) { FE_TRY(return wrap(dali::op::dot(A(a), A(b)));, nullptr) }
+dali_array_t dali_fe_inner(dali_array_t a, dali_array_t b) { FE_TRY(return wrap(dali::op::inner(A(a), A(b)));, nullptr) }
+dali_array_t dali_fe_matrix_vector_dot(dali_array_t a, dali_array_t b) { FE_TRY(return wrap(dali::op::matrix_vector_dot(A(a), A(b)));, nullptr) }
 dali_array_t dali_fe_tensordot(dali_array_t a, dali_array_t b, int n_axes, const int* a_reduce_axes, const int* b_reduce_axes) {
     FE_TRY(if (!a_reduce_axes || !b_reduce_axes) return wrap(dali::op::tensordot(A(a), A(b), n_axes));
            return wrap(dali::op::tensordot(A(a), A(b), std::vector<int>(a_reduce_axes, a_reduce_axes + n_axes),

@@ -187,6 +187,7 @@ Array elementwise(Array a, Array b, const std::string& functor_name);
 Array astype(Array a, DType dtype);
 Array unsafe_cast(Array a, DType dtype);
 Array round(Array a);
+Array ceil(Array a);
 Array add(const Array& a, const Array& b);
 Array subtract(const Array& a, const Array& b);
 Array eltmul(const Array& a, const Array& b);
@@ -263,6 +264,7 @@ Array all_close(const Array& left, const Array& right, const Array& atolerance);
 
 // dali/array/op/softmax.h, gather_from_rows.h, one_hot.h, dot.h
 Array softmax(const Array& logits, int axis = -1);
+Array softmax_temperature(const Array& logits, const Array& temperature, int axis = -1);
 Array gather_from_rows(const Array& source, const Array& indices);
 Array gather(const Array& source, const Array& indices);
 // dali/array/op/scan.h, arange.h, eye.h, outer.h
@@ -325,6 +327,8 @@ Array& autoreduce_assign(Array& left, const Array& right);
 Array one_hot(Array indices, int depth, Array on_value, Array off_value);
 Array matmul(Array a, Array b);
 Array dot(const Array& a, const Array& b);
+Array inner(const Array& a, const Array& b);
+Array matrix_vector_dot(const Array& a, const Array& b);
 Array tensordot(const Array& a, const Array& b, int axis);
 Array tensordot(const Array& a, const Array& b, const std::vector<int>& a_reduce_axes, const std::vector<int>& b_reduce_axes);
 

@@ -162,6 +162,26 @@ def dot(a, b):
     return _wrap(front.dali_fe_dot(a._h, b._h), "dot")
 
 
+def inner(a, b):
+    a, b = as_array(a), as_array(b)
+    return _wrap(front.dali_fe_inner(a._h, b._h), "inner")
+
+
+def matrix_vector_dot(a, b):
+    a, b = as_array(a), as_array(b)
+    return _wrap(front.dali_fe_matrix_vector_dot(a._h, b._h), "matrix_vector_dot")
+
+
+def ceil(a):
+    """Rounds up to int32 (dali/array/op/elementwise_operation.cpp:155-160)."""
+    return _wrap(front.dali_fe_ceil(as_array(a)._h), "ceil")
+
+
+def softmax_temperature(x, temperature, axis=-1):
+    """The reference's softmax_temperature does not read its temperature (dali/array/op/softmax.cpp:10-13); neither does this."""
+    return _wrap(front.dali_fe_softmax_temperature(as_array(x)._h, as_array(temperature)._h, axis), "softmax_temperature")
+
+
 def tensordot(a, b, axes):
     """``axes`` = a count (the last axes of a against the first of b) or a pair of axis lists (dali/array/op/dot.cpp:92-98)."""
     a, b = as_array(a), as_array(b)

@@ -64,6 +64,10 @@ dali_array_t dali_fe_arg_axis_reduce(const char* reducer_name, dali_array_t a, i
 dali_array_t dali_fe_mean_all(dali_array_t a);
 dali_array_t dali_fe_mean_axes(dali_array_t a, const int* axes, int naxes, int keepdims);
 dali_array_t dali_fe_softmax(dali_array_t a, int axis);
+/* op::softmax_temperature (dali/array/op/softmax.cpp:10-13): the reference ignores the temperature, and so does this */
+dali_array_t dali_fe_softmax_temperature(dali_array_t a, dali_array_t temperature, int axis);
+/* op::ceil (dali/array/op/elementwise_operation.cpp:155-160): int32 result, int32 operands pass through */
+dali_array_t dali_fe_ceil(dali_array_t a);
 dali_array_t dali_fe_gather_from_rows(dali_array_t source, dali_array_t indices);
 /* op::gather (dali/array/op/gather.cpp:163-171); assigning to the lazy result scatters into `source` */
 dali_array_t dali_fe_gather(dali_array_t source, dali_array_t indices);
@@ -108,6 +112,9 @@ dali_array_t dali_fe_dot(dali_array_t a, dali_array_t b);
 /* op::tensordot (dali/array/op/dot.cpp:92-98, dali/array/gemm/tensordot_as_dot.h:48-158). With both axis lists NULL the
  * last n_axes axes of a are summed against the first n_axes axes of b; otherwise axis a_reduce_axes[i] of a against axis
  * b_reduce_axes[i] of b. The result holds the kept axes of a, then those of b. */
+/* op::inner and op::matrix_vector_dot (dali/array/op/dot.cpp:67-90,100-102) */
+dali_array_t dali_fe_inner(dali_array_t a, dali_array_t b);
+dali_array_t dali_fe_matrix_vector_dot(dali_array_t a, dali_array_t b);
 dali_array_t dali_fe_tensordot(dali_array_t a, dali_array_t b, int n_axes, const int* a_reduce_axes, const int* b_reduce_axes);
 
 /* composites evaluated as one fused group */

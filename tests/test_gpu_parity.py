@@ -833,6 +833,33 @@ def test_dot_known_answers_and_laziness(gpu, D, rng):
     assert dst.numpy().tolist() == [[13, 16, 19, 22], [13, 16, 19, 22]]
 
 
+def test_ceil_softmax_temperature_and_named_products(gpu, D, rng):
+    op = D.op
+    x = np.concatenate([rng.uniform(-50, 50, 997), [-2.0, -0.0, 0.0, 3.0, 2.5, -2.5, 1e-30, -1e-30]]).astype(np.float32)
+    got = op.ceil(arr(D, x)).numpy()
+    assert got.dtype == np.int32 and np.array_equal(got, np.ceil(x).astype(np.int32))  # elementwise_operation.cpp:155-160
+    xd = rng.uniform(-50, 50, (3, 5))
+    assert np.array_equal(op.ceil(arr(D, xd)).numpy(), np.ceil(xd).astype(np.int32))
+    i = np.arange(-3, 4, dtype=np.int32)
+    assert np.array_equal(op.ceil(arr(D, i)).numpy(), i)  # int32 passes through
+    # the reference's softmax_temperature never reads its temperature (softmax.cpp:10-13)
+    l = rng.randn(6, 40).astype(np.float32)
+    assert np.array_equal(op.softmax_temperature(arr(D, l), 3.0).numpy(), op.softmax(arr(D, l)).numpy())
+    assert np.array_equal(op.softmax_temperature(arr(D, l), 0.5, 0).numpy(), op.softmax(arr(D, l), 0).numpy())
+    # dot.cpp:67-102
+    m = np.arange(12, dtype=np.float32).reshape(4, 3)
+    v = np.arange(3, dtype=np.float32)
+    assert op.matrix_vector_dot(arr(D, m), arr(D, v)).numpy().tolist() == [5, 14, 23, 32]  # dot_tests.cpp:94-118
+    assert op.matrix_vector_dot(arr(D, v), arr(D, m.T.copy())).numpy().tolist() == [5, 14, 23, 32]
+    assert float(op.inner(arr(D, v), arr(D, v)).numpy()) == 5.0
+    with pytest.raises(D.DaliError, match="inner expects vector inputs"):
+        op.inner(arr(D, m), arr(D, v))
+    with pytest.raises(D.DaliError, match="should be equal"):
+        op.inner(arr(D, v), arr(D, np.zeros(4, np.float32)))
+    with pytest.raises(D.DaliError, match="must be a vector and a matrix"):
+        op.matrix_vector_dot(arr(D, m), arr(D, m))
+
+
 def test_tensordot_alignment_rules_and_values(gpu, D, rng):
     """ArrayDotTests.tensordot_alignment_rules (dot_tests.cpp:157-224): which shapes `dot` accepts and what it returns,
     and tensordot over two axis pairs against the five-deep loop of dot_tests.cpp:120-148."""
