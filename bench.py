@@ -285,6 +285,13 @@ def main():
         nxt["cumsum_8192x8192"] = {"us": round(us, 2), "GB/s": round(2 * 8192 * 8192 * 4 / us / 1e3, 1),
                                    "frac_hbm": round(2 * 8192 * 8192 * 4 / us / 1e3 / HBM_PEAK_GBS, 4), "kernels": rec.launches}
         del sm, rec
+        # ordering along rows (the reference runs top_k on the CPU only): the 8 largest of 32000 scores in each of 1024 rows
+        sc = D.Array.from_numpy(np.random.RandomState(20).randn(1024, 32000).astype(np.float32))
+        with D.Recording() as rec:
+            op.top_k(sc, 8).eval()
+        us = time_recording(rec, 10)
+        nxt["top_k_8_of_1024x32000"] = {"us": round(us, 2), "Mkeys/s": round(1024 * 32000 / us, 1), "launches": rec.launches}
+        del sc, rec
         # sliding windows in the channels-last layout: a 3x3 convolution layer (64 -> 128 channels, 32 images of 56x56) as
         # im2col + one matrix product, its two gradients, and a 3x3 / stride 2 max pooling of 32 images of 112x112x64
         xi = D.Array.from_numpy(np.random.RandomState(18).randn(32, 56, 56, 64).astype(np.float32))

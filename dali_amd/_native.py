@@ -90,6 +90,7 @@ HIP_SYMBOLS = {
     "dali_hip_sgemm_terms": (_i, [_i, _i, _i, _i, _i, _ip, C.POINTER(H), _i, C.POINTER(H), _i, C.c_float, C.c_float, H, _i, _ip]),
     "dali_hip_lstm_step": (_i, [_i, _i, _i, H, _i, H, _i, H, H, _i, H, _i, H, H, H]),
     "dali_hip_argsort_i32": (_i, [H, C.c_int64, C.c_int32, H, H]),
+    "dali_hip_topk_rows": (_i, [H, _i, C.c_int64, C.c_int32, C.c_int32, _i, _i, H]),
     "dali_hip_capture_begin": (_i, []),
     "dali_hip_capture_end": (_i, [C.POINTER(H)]),
     "dali_hip_graph_launch": (_i, [H]),
@@ -166,6 +167,8 @@ FRONT_SYMBOLS = {
     "dali_fe_matrix_vector_dot": (H, [H, H]),
     "dali_fe_ceil": (H, [H]),
     "dali_fe_softmax_temperature": (H, [H, H, _i]),
+    "dali_fe_top_k": (H, [H, _i, _i, _i]),
+    "dali_fe_argsort": (H, [H, _i, _i]),
     "dali_fe_tensordot": (H, [H, H, _i, _ip, _ip]),
     "dali_fe_softmax_cross_entropy": (_i, [H, H, _HP, _HP, _HP]),
     "dali_fe_lstm_step": (_i, [H, H, H, H, H, H, _HP, _HP]),

@@ -86,9 +86,102 @@ __global__ __launch_bounds__(256) void rank_sort_kernel(const int32_t* keys, int
     if (threadIdx.x == 0) __hip_atomic_store(tickets + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+
+// ---------------------------------------------------------------- ordering along rows (top_k / bottom_k / argsort)
+// Keys of one dense [rows, cols] matrix are copied into a sort buffer beside their column numbers. -0.0 becomes +0.0
+// so that the two compare equal, as they do for the reference's comparators; with `reverse` a row is laid out back to
+// front, so that the stable sort which follows leaves equal keys in descending column order.
+template <typename T>
+__global__ __launch_bounds__(256) void row_keys_kernel(const T* x, long total, int cols, int reverse, T* keys, int32_t* columns) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const long row = i / cols;
+    const int col = (int)(i - row * cols);
+    const int src = reverse ? cols - 1 - col : col;
+    keys[i] = x[row * cols + src] + (T)0;
+    columns[i] = src;
+}
+
+__global__ __launch_bounds__(256) void row_offsets_kernel(int32_t* offsets, int rows, int cols) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i <= rows) offsets[i] = i * cols;
+}
+
+__global__ __launch_bounds__(256) void leading_columns_kernel(const int32_t* in, long total, int cols, int k, int32_t* out) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const long row = i / k;
+    out[i] = in[row * cols + (i - row * k)];
+}
+
+template <typename T>
+int topk_rows(const void* x, int rows, int cols, int k, bool largest, bool ties_by_descending_column, int32_t* out) {
+    hipStream_t st = stream();
+    const long total = (long)rows * cols;
+    const size_t key_bytes = (size_t)total * sizeof(T), col_bytes = (size_t)total * sizeof(int32_t), off_bytes = ((size_t)rows + 1) * sizeof(int32_t);
+    void *keys = nullptr, *keys_sorted = nullptr, *columns = nullptr, *columns_sorted = nullptr, *offsets = nullptr, *temp = nullptr;
+    size_t temp_bytes = 0;
+    int status = DALI_HIP_OK;
+    if (dali_hip_bank_allocate(&keys, key_bytes) || dali_hip_bank_allocate(&keys_sorted, key_bytes) || dali_hip_bank_allocate(&columns, col_bytes) ||
+        dali_hip_bank_allocate(&offsets, off_bytes) || (k < cols && dali_hip_bank_allocate(&columns_sorted, col_bytes)))
+        status = DALI_HIP_ERROR;
+    int32_t* sorted_columns = k < cols ? (int32_t*)columns_sorted : out;
+    if (status == DALI_HIP_OK) {
+        hipLaunchKernelGGL(row_keys_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (const T*)x, total, cols,
+                           ties_by_descending_column ? 1 : 0, (T*)keys, (int32_t*)columns);
+        hipLaunchKernelGGL(row_offsets_kernel, dim3((unsigned)(rows / 256 + 1)), dim3(256), 0, st, (int32_t*)offsets, rows, cols);
+        auto sort = [&](void* t) {
+            const int32_t* off = (const int32_t*)offsets;
+            return largest ? hipcub::DeviceSegmentedRadixSort::SortPairsDescending(t, temp_bytes, (const T*)keys, (T*)keys_sorted, (const int32_t*)columns,
+                                                                                    sorted_columns, (int)total, rows, off, off + 1, 0, (int)sizeof(T) * 8, st)
+                           : hipcub::DeviceSegmentedRadixSort::SortPairs(t, temp_bytes, (const T*)keys, (T*)keys_sorted, (const int32_t*)columns,
+                                                                          sorted_columns, (int)total, rows, off, off + 1, 0, (int)sizeof(T) * 8, st);
+        };
+        hipError_t e = sort(nullptr);
+        if (e != hipSuccess) {
+            status = fail("row sort sizing failed: %s", hipGetErrorString(e));
+        } else if (dali_hip_bank_allocate(&temp, temp_bytes ? temp_bytes : 4)) {
+            status = DALI_HIP_ERROR;
+        } else if ((e = sort(temp)) != hipSuccess) {
+            status = fail("row sort failed: %s", hipGetErrorString(e));
+        } else if (k < cols) {
+            const long kept = (long)rows * k;
+            hipLaunchKernelGGL(leading_columns_kernel, dim3((unsigned)((kept + 255) / 256)), dim3(256), 0, st, (const int32_t*)columns_sorted, kept, cols, k, out);
+        }
+        if (status == DALI_HIP_OK) {
+            hipError_t le = hipGetLastError();
+            if (le != hipSuccess) status = fail("row sort launch failed: %s", hipGetErrorString(le));
+        }
+    }
+    // back to the bank at once: their next user is ordered behind these launches on the stream
+    if (temp) dali_hip_bank_deposit(temp, temp_bytes ? temp_bytes : 4);
+    if (columns_sorted) dali_hip_bank_deposit(columns_sorted, col_bytes);
+    if (offsets) dali_hip_bank_deposit(offsets, off_bytes);
+    if (columns) dali_hip_bank_deposit(columns, col_bytes);
+    if (keys_sorted) dali_hip_bank_deposit(keys_sorted, key_bytes);
+    if (keys) dali_hip_bank_deposit(keys, key_bytes);
+    return status;
+}
+
 }  // namespace dali_hip
 
 using namespace dali_hip;
+
+extern "C" int dali_hip_topk_rows(const void* x, int dtype, int64_t rows, int32_t cols, int32_t k, int largest, int ties_by_descending_column,
+                                  int32_t* out) {
+    if (ensure_init()) return DALI_HIP_ERROR;
+    if (rows < 0 || cols < 0) return fail("dali_hip_topk_rows: negative extent");
+    if (k < 1 || k > cols) return fail("dali_hip_topk_rows: k = %d must lie in [1, %d]", k, cols);
+    if (rows == 0) return DALI_HIP_OK;
+    if (rows * (int64_t)cols > 2147483647LL) return fail("dali_hip_topk_rows: %lld keys exceed the int32 position range", (long long)(rows * cols));
+    if (!x || !out) return fail("dali_hip_topk_rows: NULL argument");
+    switch (dtype) {
+        case 0: return topk_rows<float>(x, (int)rows, cols, k, largest != 0, ties_by_descending_column != 0, out);
+        case 1: return topk_rows<double>(x, (int)rows, cols, k, largest != 0, ties_by_descending_column != 0, out);
+        case 2: return topk_rows<int32_t>(x, (int)rows, cols, k, largest != 0, ties_by_descending_column != 0, out);
+    }
+    return fail("dali_hip_topk_rows: unknown dtype %d (0 = float, 1 = double, 2 = int32)", dtype);
+}
 
 extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_limit, int32_t* sorted_keys, int32_t* perm) {
     if (ensure_init()) return DALI_HIP_ERROR;

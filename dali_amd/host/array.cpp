@@ -1481,6 +1481,40 @@ Array tensordot(const Array& a, const Array& b, int axis) {
     return tensordot(a, b, ra, rb);
 }
 
+// dali/array/op/top_k.cpp:198-233. The reference computes these on the CPU only; here the rows are ordered on the
+// device. Unlike the other factories these evaluate their argument at once.
+static Array k_best(const Array& array, int k, bool largest, const char* name) {
+    DALI_ASSERT(k >= 1, make_message(name, "'s k argument must be >= 1, but got k = ", k, "."));
+    if (array.number_of_elements() == 1) return Array::zeros(array.shape(), DTYPE_INT32);
+    DALI_ASSERT(array.ndim() >= 1, make_message(name, " expects an array with at least one dimension."));
+    const int cols = array.shape().back();
+    DALI_ASSERT(k <= cols, make_message(name, "'s k argument must be <= the last dimension (got k = ", k, ", shape = ", shape_str(array.shape()), ")."));
+    if (k == 1) return (largest ? argmax(array, -1) : argmin(array, -1)).expand_dims(-1);
+    std::vector<int> shape = array.shape();
+    shape.back() = k;
+    // the reference's heap breaks ties of bottom_k towards the higher column (top_k.cpp:118-123), its full sort
+    // (k = the whole row) towards the lower one (top_k.cpp:139-158)
+    return topk_rows(array.reshape({-1, cols}), k, largest, !largest && k < cols).reshape(shape);
+}
+Array top_k(const Array& array, int k, bool sorted) {
+    (void)sorted;  // the unsorted form promises no order; the sorted one is returned for both
+    return k_best(array, k, true, "top_k");
+}
+Array bottom_k(const Array& array, int k, bool sorted) {
+    (void)sorted;
+    return k_best(array, k, false, "bottom_k");
+}
+Array argsort(const Array& array) {
+    Array raveled = array.reshape({-1});
+    return bottom_k(raveled, raveled.number_of_elements(), true);
+}
+Array argsort(const Array& array, int axis) {
+    if (array.ndim() == 0) return Array::zeros({}, DTYPE_INT32);
+    if (axis < 0) axis += array.ndim();
+    DALI_ASSERT(axis >= 0 && axis < array.ndim(), make_message("argsort axis must >= 0 and < ndim (", array.ndim(), "), got axis = ", axis, "."));
+    return bottom_k(array.swapaxes(axis, -1), array.shape()[axis], true).swapaxes(axis, -1);
+}
+
 // dali/array/op/dot.cpp:100-102
 Array inner(const Array& a, const Array& b) {
     DALI_ASSERT(a.ndim() == 1 && b.ndim() == 1,

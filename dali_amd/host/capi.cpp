@@ -177,6 +177,12 @@ dali_array_t dali_fe_one_hot(dali_array_t indices, int depth, dali_array_t on_va
 dali_array_t dali_fe_dot(dali_array_t a, dali_array_t b) { FE_TRY(return wrap(dali::op::dot(A(a), A(b)));, nullptr) }
 dali_array_t dali_fe_inner(dali_array_t a, dali_array_t b) { FE_TRY(return wrap(dali::op::inner(A(a), A(b)));, nullptr) }
 dali_array_t dali_fe_matrix_vector_dot(dali_array_t a, dali_array_t b) { FE_TRY(return wrap(dali::op::matrix_vector_dot(A(a), A(b)));, nullptr) }
+dali_array_t dali_fe_top_k(dali_array_t a, int k, int sorted, int largest) {
+    FE_TRY(return wrap(largest ? dali::op::top_k(A(a), k, sorted != 0) : dali::op::bottom_k(A(a), k, sorted != 0));, nullptr)
+}
+dali_array_t dali_fe_argsort(dali_array_t a, int axis, int flat) {
+    FE_TRY(return wrap(flat ? dali::op::argsort(A(a)) : dali::op::argsort(A(a), axis));, nullptr)
+}
 dali_array_t dali_fe_tensordot(dali_array_t a, dali_array_t b, int n_axes, const int* a_reduce_axes, const int* b_reduce_axes) {
     FE_TRY(if (!a_reduce_axes || !b_reduce_axes) return wrap(dali::op::tensordot(A(a), A(b), n_axes));
            return wrap(dali::op::tensordot(A(a), A(b), std::vector<int>(a_reduce_axes, a_reduce_axes + n_axes),

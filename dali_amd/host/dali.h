@@ -328,6 +328,10 @@ Array one_hot(Array indices, int depth, Array on_value, Array off_value);
 Array matmul(Array a, Array b);
 Array dot(const Array& a, const Array& b);
 Array inner(const Array& a, const Array& b);
+Array top_k(const Array& array, int k, bool sorted = true);
+Array bottom_k(const Array& array, int k, bool sorted = true);
+Array argsort(const Array& array);
+Array argsort(const Array& array, int axis);
 Array matrix_vector_dot(const Array& a, const Array& b);
 Array tensordot(const Array& a, const Array& b, int axis);
 Array tensordot(const Array& a, const Array& b, const std::vector<int>& a_reduce_axes, const std::vector<int>& b_reduce_axes);

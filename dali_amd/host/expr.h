@@ -97,6 +97,8 @@ void lstm_step_fused(const Array& x, const Array& h, const Array& c, const Array
 // stride-1 convolution of a dense float NHWC image [N,H,W,C] (C a multiple of 4) with filters [O,fh,fw,C], fh <= 8:
 // one padding copy and one multi-term product, no patch matrix; returns [N, out_h, out_w, O]
 Array conv2d_direct_nhwc(const Array& x, const Array& filters, int pad_top, int pad_left, int pad_bottom, int pad_right);
+// column numbers of the k best entries of every row of a [rows, cols] matrix, best first (evaluates its argument)
+Array topk_rows(const Array& x2d, int k, bool largest, bool ties_by_descending_column);
 void set_dry_run(bool on);
 bool dry_run();
 

@@ -3262,6 +3262,31 @@ std::string gen_scatter_rows_kernel(const Program& P, const IvLayout& L, OPERATO
     return ss.str();
 }
 
+Array dense_buffer(const Array& a);
+
+// Column numbers of the k best entries of every row of a dense [rows, cols] matrix, best first
+// (dali/array/op/top_k.cpp:96-170). The ordering is a library call on the library stream, not a generated kernel.
+Array topk_rows_impl(const Array& x2d_in, int k, bool largest, bool ties_by_descending_column) {
+    Array x2d = dense_buffer(x2d_in);
+    const int rows = x2d.shape()[0], cols = x2d.shape()[1];
+    Array out({rows, k}, DTYPE_INT32);
+    if (rows == 0 || g_dry_run) return out;
+    const void* xp = x2d.device_ptr();
+    int32_t* op_ = (int32_t*)out.device_ptr(memory::AM_OVERWRITE);
+    const int dtype = (int)x2d.dtype();
+    check_hip(dali_hip_topk_rows(xp, dtype, rows, cols, k, largest, ties_by_descending_column, op_), "ordering of rows");
+    if (g_recording) {
+        note_recorded_write(out.expression()->memory);
+        Array keep_x = x2d, keep_out = out;
+        g_recording->push_back([=]() {
+            (void)keep_x;
+            (void)keep_out;
+            check_hip(dali_hip_topk_rows(xp, dtype, rows, cols, k, largest, ties_by_descending_column, op_), "ordering of rows, replay");
+        });
+    }
+    return out;
+}
+
 // dest2d: [V, D] view of the destination buffer; idx: int32 [N] buffer; values: [N, D] buffer or one element
 void run_scatter_rows(const Array& dest2d, const Array& idx, OPERATOR_T op, const Array& values) {
     const int N = numel_of(idx.shape()), D = dest2d.shape()[1], V = dest2d.shape()[0];
@@ -4450,6 +4475,10 @@ void scatter_assign(const Array& dest, OPERATOR_T op, const Array& source) {
 }
 
 }  // namespace
+
+Array topk_rows(const Array& x2d, int k, bool largest, bool ties_by_descending_column) {
+    return topk_rows_impl(x2d, k, largest, ties_by_descending_column);
+}
 
 Array conv2d_direct_nhwc(const Array& x, const Array& filters, int pad_top, int pad_left, int pad_bottom, int pad_right) {
     return conv2d_nhwc_direct(x, filters, pad_top, pad_left, pad_bottom, pad_right);

@@ -182,6 +182,24 @@ def softmax_temperature(x, temperature, axis=-1):
     return _wrap(front.dali_fe_softmax_temperature(as_array(x)._h, as_array(temperature)._h, axis), "softmax_temperature")
 
 
+def top_k(a, k, sorted=True):
+    """int32 positions of the k largest entries along the last axis, largest first, lower position first among equals
+    (dali/array/op/top_k.cpp:198-208)."""
+    return _wrap(front.dali_fe_top_k(as_array(a)._h, k, 1 if sorted else 0, 1), "top_k")
+
+
+def bottom_k(a, k, sorted=True):
+    """int32 positions of the k smallest entries along the last axis, smallest first (dali/array/op/top_k.cpp:210-220)."""
+    return _wrap(front.dali_fe_top_k(as_array(a)._h, k, 1 if sorted else 0, 0), "bottom_k")
+
+
+def argsort(a, axis=None):
+    """Stable ascending order of the flattened array, or along ``axis`` (dali/array/op/top_k.cpp:222-233)."""
+    if axis is None:
+        return _wrap(front.dali_fe_argsort(as_array(a)._h, 0, 1), "argsort")
+    return _wrap(front.dali_fe_argsort(as_array(a)._h, axis, 0), "argsort")
+
+
 def tensordot(a, b, axes):
     """``axes`` = a count (the last axes of a against the first of b) or a pair of axis lists (dali/array/op/dot.cpp:92-98)."""
     a, b = as_array(a), as_array(b)

@@ -112,6 +112,11 @@ dali_array_t dali_fe_dot(dali_array_t a, dali_array_t b);
 /* op::tensordot (dali/array/op/dot.cpp:92-98, dali/array/gemm/tensordot_as_dot.h:48-158). With both axis lists NULL the
  * last n_axes axes of a are summed against the first n_axes axes of b; otherwise axis a_reduce_axes[i] of a against axis
  * b_reduce_axes[i] of b. The result holds the kept axes of a, then those of b. */
+/* op::top_k (largest != 0) / op::bottom_k (largest == 0): int32 column numbers of the k best entries along the last axis,
+ * best first (dali/array/op/top_k.cpp:198-220); op::argsort over the flattened array (flat != 0) or along an axis
+ * (dali/array/op/top_k.cpp:222-233) */
+dali_array_t dali_fe_top_k(dali_array_t a, int k, int sorted, int largest);
+dali_array_t dali_fe_argsort(dali_array_t a, int axis, int flat);
 /* op::inner and op::matrix_vector_dot (dali/array/op/dot.cpp:67-90,100-102) */
 dali_array_t dali_fe_inner(dali_array_t a, dali_array_t b);
 dali_array_t dali_fe_matrix_vector_dot(dali_array_t a, dali_array_t b);

@@ -256,6 +256,18 @@ int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx
  */
 int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_limit, int32_t* sorted_keys, int32_t* perm);
 
+/*
+ * The column numbers of the k best entries of every row of a dense row-major [rows, cols] matrix, best first, into
+ * out[rows, k]. Replaces the reference's CPU-only CpuTopKImpl (dali/array/op/top_k.cpp:36-196; "add gpu impl of topk"
+ * is a TODO there, :198). dtype: 0 = float, 1 = double, 2 = int32. largest != 0 orders by descending value (top_k),
+ * else ascending (bottom_k, argsort). Equal values come out in ascending column order, or in descending column order
+ * with ties_by_descending_column != 0 (what the reference's heap gives bottom_k for k < cols, top_k.cpp:118-123).
+ * -0.0 and +0.0 are equal; the place of NaNs is unspecified. One segmented radix sort on the library stream; its
+ * buffers (four times the input) come from the bank.
+ */
+int dali_hip_topk_rows(const void* x, int dtype, int64_t rows, int32_t cols, int32_t k, int largest, int ties_by_descending_column,
+                       int32_t* out);
+
 /* ---------------------------------------------------------- HIP graphs */
 
 /*

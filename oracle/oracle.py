@@ -428,3 +428,34 @@ def gru_step(X, Hs, W, U, b):
     m = unary("tanh", pre(2, pc))
     one_minus = (np.float32(1.0) - z).astype(f32)
     return ((Hs * one_minus).astype(f32) + (m * z).astype(f32)).astype(f32)
+
+
+def k_best(x, k, largest):
+    """int32 positions of the k best entries along the last axis, best first (dali/array/op/top_k.cpp:96-220).
+    k = 1 is argmax / argmin (first position on ties, :205,:217); k = the whole axis is the full sort with runs of equal
+    values in ascending position (:139-158); otherwise the heap's comparator decides (:103-135): top_k breaks ties
+    towards the lower position, bottom_k towards the HIGHER one. Stable sorts of (value, position) pairs."""
+    x = np.asarray(x)
+    if x.size == 1:
+        return np.zeros(x.shape, np.int32)
+    n = x.shape[-1]
+    rows = x.reshape(-1, n)
+    out = np.empty((rows.shape[0], k), np.int32)
+    pos = np.arange(n)
+    for r, row in enumerate(rows):
+        if largest:
+            order = np.lexsort((-pos, row))[::-1]  # value descending, position ascending
+        elif k < n and k > 1:
+            order = np.lexsort((-pos, row))  # value ascending, position descending
+        else:
+            order = np.lexsort((pos, row))  # value ascending, position ascending
+        out[r] = order[:k]
+    return out.reshape(x.shape[:-1] + (k,))
+
+
+def argsort(x, axis=None):
+    """dali/array/op/top_k.cpp:222-233: bottom_k over the whole (flattened, or swapped-to-last) axis."""
+    x = np.asarray(x)
+    if axis is None:
+        return k_best(x.reshape(-1), x.size, False)
+    return np.swapaxes(k_best(np.swapaxes(x, axis, -1), x.shape[axis], False), axis, -1)

@@ -860,6 +860,41 @@ def test_ceil_softmax_temperature_and_named_products(gpu, D, rng):
         op.matrix_vector_dot(arr(D, m), arr(D, m))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32])
+def test_top_k_bottom_k_argsort_are_bit_exact(gpu, D, O, rng, dtype):
+    """Positions from the device ordering against the reference's comparators (top_k.cpp:96-233), on rows full of ties."""
+    op = D.op
+    for shape in [(5, 9), (3, 4, 33), (64, 1000), (2, 70001)]:
+        x = rng.randint(-50, 51, shape).astype(dtype)
+        n = shape[-1]
+        for k in sorted({1, 2, min(7, n), n - 1, n}):
+            got = op.top_k(arr(D, x), k).numpy()
+            assert got.dtype == np.int32 and np.array_equal(got, O.k_best(x, k, True)), (shape, k)
+            assert np.array_equal(op.bottom_k(arr(D, x), k).numpy(), O.k_best(x, k, False)), (shape, k)
+    if dtype != np.int32:
+        z = np.array([[0.0, -0.0, 1.0, -0.0, 0.0, -1.0]], dtype)  # the two zeros are equal: positions decide
+        assert op.top_k(arr(D, z), 6).numpy().tolist() == [[2, 0, 1, 3, 4, 5]]
+        assert op.bottom_k(arr(D, z), 6).numpy().tolist() == [[5, 0, 1, 3, 4, 2]]
+        assert op.bottom_k(arr(D, z), 3).numpy().tolist() == [[5, 4, 3]]
+    # ArgsortTests.argsort / argsort_strided (other_tests.cpp:6-62): increasing along the flattened array and along every axis
+    a = rng.uniform(-20, 20, (2, 3, 4, 3)).astype(dtype)
+    view = arr(D, a).transpose(0, 2, 1, 3)[:, ::2]
+    ref = np.ascontiguousarray(a.swapaxes(1, 2)[:, ::2])
+    flat = op.argsort(view).numpy()
+    assert np.array_equal(flat, O.argsort(ref)) and np.all(np.diff(ref.reshape(-1)[flat]) >= 0)
+    for axis in range(4):
+        idx = op.argsort(view, axis).numpy()
+        assert np.array_equal(idx, O.argsort(ref, axis))
+        assert np.all(np.diff(np.take_along_axis(ref, idx.astype(np.int64), axis), axis=axis) >= 0)
+    assert op.argsort(view, -1).numpy().shape == ref.shape
+    # top_k.cpp:200-204
+    assert op.top_k(arr(D, np.array([[7]], dtype)), 3).numpy().tolist() == [[0]]
+    with pytest.raises(D.DaliError, match="k argument must be >= 1"):
+        op.top_k(arr(D, x), 0)
+    with pytest.raises(D.DaliError, match="argsort axis must >= 0 and < ndim"):
+        op.argsort(arr(D, a), 4)
+
+
 def test_tensordot_alignment_rules_and_values(gpu, D, rng):
     """ArrayDotTests.tensordot_alignment_rules (dot_tests.cpp:157-224): which shapes `dot` accepts and what it returns,
     and tensordot over two axis pairs against the five-deep loop of dot_tests.cpp:120-148."""

@@ -623,3 +623,44 @@ def test_stacked_lstm_step_against_fp64_definition(O, rng):
     assert np.array_equal(cs[0], c1) and np.array_equal(hs[0], h1)
     with pytest.raises(ValueError, match="Activating LSTM stack of size 3 with different number of states 2"):
         O.stacked_lstm_step(X, Hs[:2], Cs[:2], Ws, Us, bs)
+
+
+def test_k_best_against_the_reference_comparators(O, rng):
+    """The heap comparators of top_k.cpp:103-135 and the full-sort rule of :139-158, applied by brute force (selection by
+    repeated scans, no sort routine) to rows full of ties; argsort is increasing (other_tests.cpp:6-31)."""
+    def better_top(row, a, b):  # stable_comp(a, b), reversed = false
+        return row[b] < row[a] or (row[b] == row[a] and a < b)
+
+    def better_bottom(row, a, b):  # stable_comp(a, b), reversed = true
+        return row[b] > row[a] or (row[b] == row[a] and a > b)
+
+    def select(row, k, better):
+        left, out = list(range(len(row))), []
+        for _ in range(k):
+            best = left[0]
+            for c in left[1:]:
+                if better(row, c, best):
+                    best = c
+            out.append(best)
+            left.remove(best)
+        return out
+
+    for dtype in (np.float32, np.int32, np.float64):
+        x = rng.randint(-3, 4, (5, 9)).astype(dtype)
+        for k in (2, 3, 8):
+            assert O.k_best(x, k, True).tolist() == [select(r, k, better_top) for r in x]
+            assert O.k_best(x, k, False).tolist() == [select(r, k, better_bottom) for r in x]
+        # the whole row: values in order, equal values in ascending position
+        full_top = O.k_best(x, 9, True)
+        full_bottom = O.k_best(x, 9, False)
+        for r in range(5):
+            assert full_top[r].tolist() == sorted(range(9), key=lambda c: (-float(x[r, c]), c))
+            assert full_bottom[r].tolist() == sorted(range(9), key=lambda c: (float(x[r, c]), c))
+        assert np.array_equal(O.k_best(x, 1, True)[:, 0], x.argmax(1)) and np.array_equal(O.k_best(x, 1, False)[:, 0], x.argmin(1))
+    a = rng.uniform(-20, 20, (2, 3, 4)).astype(np.float32)
+    flat = O.argsort(a)
+    assert flat.dtype == np.int32 and np.all(np.diff(a.reshape(-1)[flat]) >= 0)
+    for axis in range(3):
+        idx = O.argsort(a, axis)
+        assert idx.shape == a.shape and np.all(np.diff(np.take_along_axis(a, idx, axis), axis=axis) >= 0)
+    assert O.k_best(np.array([[7.0]]), 3, True).tolist() == [[0]]  # one element: zeros of the input's shape (top_k.cpp:202-204)
