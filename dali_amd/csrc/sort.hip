@@ -114,9 +114,135 @@ __global__ __launch_bounds__(256) void leading_columns_kernel(const int32_t* in,
     out[i] = in[row * cols + (i - row * k)];
 }
 
+// A few best entries of long rows: selection instead of a sort. One workgroup per row, read once, coalesced. Every wave
+// keeps ONE list of its k best (value, column) pairs, lane i holding the i-th best, and the value of lane k - 1 as a
+// wave-wide threshold: after the first few steps almost every element fails the threshold, which costs one comparison,
+// and the rare one that passes is inserted by all lanes at once (each lane keeps its entry, takes its neighbour's or
+// takes the newcomer). Wave 0 then inserts the other three lists into its own. `better` is the reference's comparator
+// (dali/array/op/top_k.cpp:103-135): by value, then by column, ascending columns first unless ties_desc; it is a strict
+// total order, so the result does not depend on the order in which elements arrive.
+constexpr int kSelectMax = 64;
+
+template <typename T>
+struct Candidate {
+    T value;
+    int32_t column;  // -1: no candidate
+};
+
+template <typename T>
+__device__ __forceinline__ bool better(const Candidate<T>& a, const Candidate<T>& b, bool largest, bool ties_desc) {
+    if (a.column < 0) return false;
+    if (b.column < 0) return true;
+    if (a.value != b.value) return largest ? a.value > b.value : a.value < b.value;
+    return ties_desc ? a.column > b.column : a.column < b.column;
+}
+
+template <typename T>
+__device__ __forceinline__ T lane_value(T v, int src_lane, bool up) {
+    if constexpr (sizeof(T) == 8) {
+        union {
+            T v;
+            int w[2];
+        } u;
+        u.v = v;
+        u.w[0] = up ? __shfl_up(u.w[0], 1, 64) : __shfl(u.w[0], src_lane, 64);
+        u.w[1] = up ? __shfl_up(u.w[1], 1, 64) : __shfl(u.w[1], src_lane, 64);
+        return u.v;
+    } else {
+        return up ? __shfl_up(v, 1, 64) : __shfl(v, src_lane, 64);
+    }
+}
+template <typename T>
+__device__ __forceinline__ Candidate<T> from_lane(const Candidate<T>& c, int src_lane) {
+    Candidate<T> r;
+    r.value = lane_value(c.value, src_lane, false);
+    r.column = __shfl(c.column, src_lane, 64);
+    return r;
+}
+template <typename T>
+__device__ __forceinline__ Candidate<T> from_lane_below(const Candidate<T>& c) {
+    Candidate<T> r;
+    r.value = lane_value(c.value, 0, true);
+    r.column = __shfl_up(c.column, 1, 64);
+    return r;
+}
+
+// `cand` is the same in every lane. Lanes whose entry it beats move one place back; the first of them takes it.
+template <typename T>
+__device__ __forceinline__ void insert_candidate(Candidate<T>& mine, Candidate<T>& worst, const Candidate<T>& cand, int lane, int k, bool largest,
+                                                 bool ties_desc) {
+    const Candidate<T> prev = from_lane_below(mine);
+    const bool beats_here = better(cand, mine, largest, ties_desc);
+    const bool beats_prev = lane > 0 && better(cand, prev, largest, ties_desc);
+    if (beats_prev)
+        mine = prev;
+    else if (beats_here)
+        mine = cand;
+    worst = from_lane(mine, k - 1);
+}
+
+template <typename T, bool largest, bool ties_desc>
+__global__ __launch_bounds__(256) void select_rows_kernel(const T* x, int cols, int k, int32_t* out) {
+    __shared__ Candidate<T> lists[4][64];
+    const T* row = x + (size_t)blockIdx.x * cols;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    Candidate<T> mine, worst;
+    mine.value = worst.value = (T)0;
+    mine.column = worst.column = -1;
+    constexpr int BATCH = sizeof(T) == 8 ? 8 : 16;  // loads in flight per lane: four waves per SIMD must cover the memory latency
+    for (int base = wave * 64; base < cols; base += 256 * BATCH) {
+        Candidate<T> cand[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+            const int c = base + u * 256 + lane;
+            cand[u].column = c < cols ? c : -1;
+            cand[u].value = c < cols ? row[c] : (T)0;
+        }
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+            // the quick test is on the value alone (an equal value may still win on its column); the full comparison
+            // is made once per passing element, below
+            const bool passes = worst.column < 0 || (largest ? cand[u].value >= worst.value : cand[u].value <= worst.value);
+            unsigned long long pending = __ballot(passes && cand[u].column >= 0);
+            while (pending) {
+                const int src = __ffsll((long long)pending) - 1;
+                pending &= pending - 1;
+                const Candidate<T> c = from_lane(cand[u], src);
+                if (better(c, worst, largest, ties_desc)) insert_candidate(mine, worst, c, lane, k, largest, ties_desc);  // the threshold may have risen
+            }
+        }
+    }
+    if (lane >= k) mine.column = -1;
+    lists[wave][lane] = mine;
+    __syncthreads();
+    if (wave != 0) return;
+    for (int w = 1; w < 4; ++w)
+        for (int i = 0; i < k; ++i) {
+            const Candidate<T> c = lists[w][i];
+            if (!better(c, worst, largest, ties_desc)) break;  // the lists are ordered: nothing behind it passes either
+            insert_candidate(mine, worst, c, lane, k, largest, ties_desc);
+        }
+    if (lane < k) out[(size_t)blockIdx.x * k + lane] = mine.column;
+}
+
 template <typename T>
 int topk_rows(const void* x, int rows, int cols, int k, bool largest, bool ties_by_descending_column, int32_t* out) {
     hipStream_t st = stream();
+    static const int select_off = getenv("DALI_HIP_TOPK_SORT_ONLY") != nullptr;
+    if (k <= kSelectMax && cols >= 1024 && !select_off) {
+        const dim3 grid((unsigned)rows), block(256);
+        if (largest && ties_by_descending_column)
+            hipLaunchKernelGGL((select_rows_kernel<T, true, true>), grid, block, 0, st, (const T*)x, cols, k, out);
+        else if (largest)
+            hipLaunchKernelGGL((select_rows_kernel<T, true, false>), grid, block, 0, st, (const T*)x, cols, k, out);
+        else if (ties_by_descending_column)
+            hipLaunchKernelGGL((select_rows_kernel<T, false, true>), grid, block, 0, st, (const T*)x, cols, k, out);
+        else
+            hipLaunchKernelGGL((select_rows_kernel<T, false, false>), grid, block, 0, st, (const T*)x, cols, k, out);
+        hipError_t le = hipGetLastError();
+        if (le != hipSuccess) return fail("row selection launch failed: %s", hipGetErrorString(le));
+        return DALI_HIP_OK;
+    }
     const long total = (long)rows * cols;
     const size_t key_bytes = (size_t)total * sizeof(T), col_bytes = (size_t)total * sizeof(int32_t), off_bytes = ((size_t)rows + 1) * sizeof(int32_t);
     void *keys = nullptr, *keys_sorted = nullptr, *columns = nullptr, *columns_sorted = nullptr, *offsets = nullptr, *temp = nullptr;

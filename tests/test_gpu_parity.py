@@ -864,13 +864,18 @@ def test_ceil_softmax_temperature_and_named_products(gpu, D, rng):
 def test_top_k_bottom_k_argsort_are_bit_exact(gpu, D, O, rng, dtype):
     """Positions from the device ordering against the reference's comparators (top_k.cpp:96-233), on rows full of ties."""
     op = D.op
-    for shape in [(5, 9), (3, 4, 33), (64, 1000), (2, 70001)]:
+    # rows of 1024 and more with k <= 64 go through the selection kernel, everything else through the segmented sort
+    for shape in [(5, 9), (3, 4, 33), (64, 1000), (37, 2048), (2, 70001)]:
         x = rng.randint(-50, 51, shape).astype(dtype)
         n = shape[-1]
-        for k in sorted({1, 2, min(7, n), n - 1, n}):
+        for k in sorted({1, 2, min(7, n), min(17, n), min(64, n), min(65, n), n - 1, n}):
             got = op.top_k(arr(D, x), k).numpy()
             assert got.dtype == np.int32 and np.array_equal(got, O.k_best(x, k, True)), (shape, k)
             assert np.array_equal(op.bottom_k(arr(D, x), k).numpy(), O.k_best(x, k, False)), (shape, k)
+    for x in (np.tile(np.arange(3000), (3, 1)).astype(dtype), np.tile(np.arange(3000)[::-1], (3, 1)).astype(dtype), np.full((3, 3000), 7, dtype)):
+        for k in (5, 64):  # rising, falling and constant rows: every element, or none, passes the selection kernel's threshold
+            assert np.array_equal(op.top_k(arr(D, x), k).numpy(), O.k_best(x, k, True))
+            assert np.array_equal(op.bottom_k(arr(D, x), k).numpy(), O.k_best(x, k, False))
     if dtype != np.int32:
         z = np.array([[0.0, -0.0, 1.0, -0.0, 0.0, -1.0]], dtype)  # the two zeros are equal: positions decide
         assert op.top_k(arr(D, z), 6).numpy().tolist() == [[2, 0, 1, 3, 4, 5]]
