@@ -9,6 +9,7 @@
 #include "runtime.h"
 
 #include <cstdlib>
+#include <type_traits>
 
 #include <hipcub/hipcub.hpp>
 
@@ -137,32 +138,47 @@ __device__ __forceinline__ bool better(const Candidate<T>& a, const Candidate<T>
     return ties_desc ? a.column > b.column : a.column < b.column;
 }
 
+// Entry of one lane, the same lane for the whole wave (a scalar read of the register, no trip through the LDS crossbar)
 template <typename T>
-__device__ __forceinline__ T lane_value(T v, int src_lane, bool up) {
+__device__ __forceinline__ Candidate<T> from_lane(const Candidate<T>& c, int src_lane) {
+    Candidate<T> r;
     if constexpr (sizeof(T) == 8) {
         union {
             T v;
             int w[2];
         } u;
-        u.v = v;
-        u.w[0] = up ? __shfl_up(u.w[0], 1, 64) : __shfl(u.w[0], src_lane, 64);
-        u.w[1] = up ? __shfl_up(u.w[1], 1, 64) : __shfl(u.w[1], src_lane, 64);
-        return u.v;
+        u.v = c.value;
+        u.w[0] = __builtin_amdgcn_readlane(u.w[0], src_lane);
+        u.w[1] = __builtin_amdgcn_readlane(u.w[1], src_lane);
+        r.value = u.v;
     } else {
-        return up ? __shfl_up(v, 1, 64) : __shfl(v, src_lane, 64);
+        union {
+            T v;
+            int w;
+        } u;
+        u.v = c.value;
+        u.w = __builtin_amdgcn_readlane(u.w, src_lane);
+        r.value = u.v;
     }
-}
-template <typename T>
-__device__ __forceinline__ Candidate<T> from_lane(const Candidate<T>& c, int src_lane) {
-    Candidate<T> r;
-    r.value = lane_value(c.value, src_lane, false);
-    r.column = __shfl(c.column, src_lane, 64);
+    r.column = __builtin_amdgcn_readlane(c.column, src_lane);
     return r;
 }
+// Entry of the lane below (lane 0 keeps its own)
 template <typename T>
 __device__ __forceinline__ Candidate<T> from_lane_below(const Candidate<T>& c) {
     Candidate<T> r;
-    r.value = lane_value(c.value, 0, true);
+    if constexpr (sizeof(T) == 8) {
+        union {
+            T v;
+            int w[2];
+        } u;
+        u.v = c.value;
+        u.w[0] = __shfl_up(u.w[0], 1, 64);
+        u.w[1] = __shfl_up(u.w[1], 1, 64);
+        r.value = u.v;
+    } else {
+        r.value = __shfl_up(c.value, 1, 64);
+    }
     r.column = __shfl_up(c.column, 1, 64);
     return r;
 }
@@ -225,20 +241,124 @@ __global__ __launch_bounds__(256) void select_rows_kernel(const T* x, int cols, 
     if (lane < k) out[(size_t)blockIdx.x * k + lane] = mine.column;
 }
 
+// The same selection for 4-byte keys with a candidate packed into one 64-bit word: the value mapped to an unsigned
+// integer of the same order (inverted when the smallest win) in the high half, the column in the low half (inverted when
+// the lower column wins ties), 0 = no candidate. "Better" is then one unsigned 64-bit comparison, which is what the
+// insertions, the bulk of the work for random rows, are made of.
+template <typename T, bool largest, bool ties_desc>
+__device__ __forceinline__ unsigned long long pack_candidate(T value, int column) {
+    unsigned int u;
+    if constexpr (sizeof(T) == 4 && !std::is_integral<T>::value) {
+        const float canonical = value + 0.0f;  // -0.0 becomes +0.0
+        u = __float_as_uint(canonical);
+        u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    } else {
+        u = (unsigned int)value ^ 0x80000000u;
+    }
+    if (!largest) u = ~u;
+    const unsigned int c = ties_desc ? (unsigned int)column + 1u : ~(unsigned int)column;  // never 0 together with u == 0
+    return ((unsigned long long)u << 32) | c;
+}
+template <typename T, bool largest>
+__device__ __forceinline__ T unpack_value(unsigned long long bits) {
+    unsigned int u = (unsigned int)(bits >> 32);
+    if (!largest) u = ~u;
+    if constexpr (sizeof(T) == 4 && !std::is_integral<T>::value) {
+        u = (u & 0x80000000u) ? (u & 0x7FFFFFFFu) : ~u;
+        return __uint_as_float(u);
+    } else {
+        return (T)(u ^ 0x80000000u);
+    }
+}
+template <bool ties_desc>
+__device__ __forceinline__ int packed_column(unsigned long long bits) {
+    return ties_desc ? (int)((unsigned int)bits - 1u) : (int)~(unsigned int)bits;
+}
+__device__ __forceinline__ unsigned long long packed_from_lane(unsigned long long v, int src_lane) {
+    const unsigned int lo = (unsigned int)__builtin_amdgcn_readlane((int)(unsigned int)v, src_lane);
+    const unsigned int hi = (unsigned int)__builtin_amdgcn_readlane((int)(unsigned int)(v >> 32), src_lane);
+    return ((unsigned long long)hi << 32) | lo;
+}
+__device__ __forceinline__ void insert_packed(unsigned long long& mine, unsigned long long& worst, unsigned long long cand, int lane, int k) {
+    const unsigned int lo = (unsigned int)__shfl_up((int)(unsigned int)mine, 1, 64);
+    const unsigned int hi = (unsigned int)__shfl_up((int)(unsigned int)(mine >> 32), 1, 64);
+    const unsigned long long prev = ((unsigned long long)hi << 32) | lo;
+    if (lane > 0 && cand > prev)
+        mine = prev;
+    else if (cand > mine)
+        mine = cand;
+    worst = packed_from_lane(mine, k - 1);
+}
+
+template <typename T, bool largest, bool ties_desc>
+__global__ __launch_bounds__(256) void select_rows_packed_kernel(const T* x, int cols, int k, int32_t* out) {
+    static_assert(sizeof(T) == 4, "packed candidates hold 4-byte values");
+    __shared__ unsigned long long lists[4][64];
+    const T* row = x + (size_t)blockIdx.x * cols;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    unsigned long long mine = 0, worst = 0;
+    constexpr int BATCH = 16;  // loads in flight per lane
+    for (int base = wave * 64; base < cols; base += 256 * BATCH) {
+        T value[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+            const int c = base + u * 256 + lane;
+            value[u] = c < cols ? row[c] : (T)0;
+        }
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+            // the streaming test is on the raw value against the threshold's value (an equal value may still win on its
+            // column); a candidate is packed only once it passes
+            const T threshold = unpack_value<T, largest>(worst);
+            const bool passes = worst == 0ull || (largest ? value[u] >= threshold : value[u] <= threshold);
+            unsigned long long pending = __ballot(passes && base + u * 256 + lane < cols);
+            while (pending) {
+                const int src = __ffsll((long long)pending) - 1;
+                pending &= pending - 1;
+                union {
+                    T v;
+                    int w;
+                } raw;
+                raw.v = value[u];
+                raw.w = __builtin_amdgcn_readlane(raw.w, src);
+                const unsigned long long cnd = pack_candidate<T, largest, ties_desc>(raw.v, base + u * 256 + src);
+                if (cnd > worst) insert_packed(mine, worst, cnd, lane, k);  // the threshold may have risen
+            }
+        }
+    }
+    lists[wave][lane] = lane < k ? mine : 0ull;
+    __syncthreads();
+    if (wave != 0) return;
+    for (int w = 1; w < 4; ++w)
+        for (int i = 0; i < k; ++i) {
+            const unsigned long long cnd = lists[w][i];
+            if (!(cnd > worst)) break;  // the lists are ordered: nothing behind it passes either
+            insert_packed(mine, worst, cnd, lane, k);
+        }
+    if (lane < k) out[(size_t)blockIdx.x * k + lane] = packed_column<ties_desc>(mine);
+}
+
+template <typename T, bool largest, bool ties_desc>
+void launch_select_rows(const T* x, int rows, int cols, int k, int32_t* out, hipStream_t st) {
+    if constexpr (sizeof(T) == 4)
+        hipLaunchKernelGGL((select_rows_packed_kernel<T, largest, ties_desc>), dim3((unsigned)rows), dim3(256), 0, st, x, cols, k, out);
+    else
+        hipLaunchKernelGGL((select_rows_kernel<T, largest, ties_desc>), dim3((unsigned)rows), dim3(256), 0, st, x, cols, k, out);
+}
+
 template <typename T>
 int topk_rows(const void* x, int rows, int cols, int k, bool largest, bool ties_by_descending_column, int32_t* out) {
     hipStream_t st = stream();
     static const int select_off = getenv("DALI_HIP_TOPK_SORT_ONLY") != nullptr;
     if (k <= kSelectMax && cols >= 1024 && !select_off) {
-        const dim3 grid((unsigned)rows), block(256);
         if (largest && ties_by_descending_column)
-            hipLaunchKernelGGL((select_rows_kernel<T, true, true>), grid, block, 0, st, (const T*)x, cols, k, out);
+            launch_select_rows<T, true, true>((const T*)x, rows, cols, k, out, st);
         else if (largest)
-            hipLaunchKernelGGL((select_rows_kernel<T, true, false>), grid, block, 0, st, (const T*)x, cols, k, out);
+            launch_select_rows<T, true, false>((const T*)x, rows, cols, k, out, st);
         else if (ties_by_descending_column)
-            hipLaunchKernelGGL((select_rows_kernel<T, false, true>), grid, block, 0, st, (const T*)x, cols, k, out);
+            launch_select_rows<T, false, true>((const T*)x, rows, cols, k, out, st);
         else
-            hipLaunchKernelGGL((select_rows_kernel<T, false, false>), grid, block, 0, st, (const T*)x, cols, k, out);
+            launch_select_rows<T, false, false>((const T*)x, rows, cols, k, out, st);
         hipError_t le = hipGetLastError();
         if (le != hipSuccess) return fail("row selection launch failed: %s", hipGetErrorString(le));
         return DALI_HIP_OK;
