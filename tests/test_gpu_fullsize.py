@@ -152,3 +152,23 @@ def test_leading_axis_reduction_of_a_very_wide_matrix(gpu, D, rng):
     np.testing.assert_allclose(D.op.sum(a, [0]).numpy(), x.astype(np.float64).sum(axis=0), rtol=1e-6, atol=1e-6)
     assert np.array_equal(D.op.max(a, [0]).numpy(), x.max(axis=0))
     assert np.array_equal(D.op.argmax(a, 0).numpy(), x.argmax(axis=0).astype(np.int32))
+
+
+def test_top_k_over_the_cross_entropy_logits_shape(gpu, D, O):
+    """The 8 largest and the 8 smallest of 32000 scores in each of 8192 rows (the selection kernel at full width): the
+    values at the returned positions are the row's extremes in order, the positions are distinct, and the first rows
+    agree with the checker position for position."""
+    rng = np.random.RandomState(21)
+    x = (rng.randn(8192, 32000) * 2).astype(np.float32)
+    X = arr(D, x)
+    top = D.op.top_k(X, 8).numpy()
+    bottom = D.op.bottom_k(X, 8).numpy()
+    assert top.shape == bottom.shape == (8192, 8) and top.dtype == np.int32
+    part = np.partition(x, (8, 31991), axis=1)
+    want_top = np.sort(part[:, 31992:], axis=1)[:, ::-1]
+    want_bottom = np.sort(part[:, :8], axis=1)
+    assert np.array_equal(np.take_along_axis(x, top.astype(np.int64), 1), want_top)
+    assert np.array_equal(np.take_along_axis(x, bottom.astype(np.int64), 1), want_bottom)
+    assert all(len(set(r)) == 8 for r in top[::64].tolist()) and all(len(set(r)) == 8 for r in bottom[::64].tolist())
+    assert np.array_equal(top[:16], O.k_best(x[:16], 8, True)) and np.array_equal(bottom[:16], O.k_best(x[:16], 8, False))
+    assert np.array_equal(top[:, 0], D.op.argmax(X, 1).numpy())
