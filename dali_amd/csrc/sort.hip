@@ -290,19 +290,21 @@ __device__ __forceinline__ void insert_packed(unsigned long long& mine, unsigned
     worst = packed_from_lane(mine, k - 1);
 }
 
-template <typename T, bool largest, bool ties_desc>
-__global__ __launch_bounds__(256) void select_rows_packed_kernel(const T* x, int cols, int k, int32_t* out) {
+// WAVES waves share a row: four when there are few rows (more loads in flight per row), one when there are thousands
+// (a single list per row sees every element, so it takes a third of the insertions).
+template <typename T, bool largest, bool ties_desc, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void select_rows_packed_kernel(const T* x, int cols, int k, int32_t* out) {
     static_assert(sizeof(T) == 4, "packed candidates hold 4-byte values");
-    __shared__ unsigned long long lists[4][64];
+    __shared__ unsigned long long lists[WAVES][64];
     const T* row = x + (size_t)blockIdx.x * cols;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     unsigned long long mine = 0, worst = 0;
     constexpr int BATCH = 16;  // loads in flight per lane
-    for (int base = wave * 64; base < cols; base += 256 * BATCH) {
+    for (int base = wave * 64; base < cols; base += 64 * WAVES * BATCH) {
         T value[BATCH];
 #pragma unroll
         for (int u = 0; u < BATCH; ++u) {
-            const int c = base + u * 256 + lane;
+            const int c = base + u * (64 * WAVES) + lane;
             value[u] = c < cols ? row[c] : (T)0;
         }
 #pragma unroll
@@ -311,7 +313,7 @@ __global__ __launch_bounds__(256) void select_rows_packed_kernel(const T* x, int
             // column); a candidate is packed only once it passes
             const T threshold = unpack_value<T, largest>(worst);
             const bool passes = worst == 0ull || (largest ? value[u] >= threshold : value[u] <= threshold);
-            unsigned long long pending = __ballot(passes && base + u * 256 + lane < cols);
+            unsigned long long pending = __ballot(passes && base + u * (64 * WAVES) + lane < cols);
             while (pending) {
                 const int src = __ffsll((long long)pending) - 1;
                 pending &= pending - 1;
@@ -321,7 +323,7 @@ __global__ __launch_bounds__(256) void select_rows_packed_kernel(const T* x, int
                 } raw;
                 raw.v = value[u];
                 raw.w = __builtin_amdgcn_readlane(raw.w, src);
-                const unsigned long long cnd = pack_candidate<T, largest, ties_desc>(raw.v, base + u * 256 + src);
+                const unsigned long long cnd = pack_candidate<T, largest, ties_desc>(raw.v, base + u * (64 * WAVES) + src);
                 if (cnd > worst) insert_packed(mine, worst, cnd, lane, k);  // the threshold may have risen
             }
         }
@@ -329,7 +331,7 @@ __global__ __launch_bounds__(256) void select_rows_packed_kernel(const T* x, int
     lists[wave][lane] = lane < k ? mine : 0ull;
     __syncthreads();
     if (wave != 0) return;
-    for (int w = 1; w < 4; ++w)
+    for (int w = 1; w < WAVES; ++w)
         for (int i = 0; i < k; ++i) {
             const unsigned long long cnd = lists[w][i];
             if (!(cnd > worst)) break;  // the lists are ordered: nothing behind it passes either
@@ -340,8 +342,12 @@ __global__ __launch_bounds__(256) void select_rows_packed_kernel(const T* x, int
 
 template <typename T, bool largest, bool ties_desc>
 void launch_select_rows(const T* x, int rows, int cols, int k, int32_t* out, hipStream_t st) {
-    if constexpr (sizeof(T) == 4)
-        hipLaunchKernelGGL((select_rows_packed_kernel<T, largest, ties_desc>), dim3((unsigned)rows), dim3(256), 0, st, x, cols, k, out);
+    if constexpr (sizeof(T) == 4) {
+        if (rows >= 4096)
+            hipLaunchKernelGGL((select_rows_packed_kernel<T, largest, ties_desc, 1>), dim3((unsigned)rows), dim3(64), 0, st, x, cols, k, out);
+        else
+            hipLaunchKernelGGL((select_rows_packed_kernel<T, largest, ties_desc, 4>), dim3((unsigned)rows), dim3(256), 0, st, x, cols, k, out);
+    }
     else
         hipLaunchKernelGGL((select_rows_kernel<T, largest, ties_desc>), dim3((unsigned)rows), dim3(256), 0, st, x, cols, k, out);
 }
