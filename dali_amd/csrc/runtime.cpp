@@ -85,6 +85,7 @@ static Runtime& rt() {
 
 hipStream_t stream() { return rt().stream; }
 char* workspace() { return rt().ws; }
+int bound_device() { return rt().ready ? rt().device : -1; }
 
 int ensure_init() {
     if (rt().ready) return DALI_HIP_OK;
@@ -195,6 +196,7 @@ int dali_hip_init(int device) {
     HIP_TRY(hipMalloc((void**)&r.ws, kWorkspaceBytes));
     HIP_TRY(hipMemsetAsync(r.ws, 0, kWorkspaceBytes, r.stream));
     HIP_TRY(hipStreamSynchronize(r.stream));
+    if (sort_scratch_init(device)) return DALI_HIP_ERROR;
     r.device = device;
     r.ready = true;
     return DALI_HIP_OK;

@@ -23,6 +23,10 @@ int fail_str(const std::string& s);
 int ensure_init();
 hipStream_t stream();
 char* workspace();
+// device the library is bound to, -1 before dali_hip_init
+int bound_device();
+// sort.hip: looks up the device address of its built-in scratch array; called by dali_hip_init with `device` current
+int sort_scratch_init(int device);
 
 }  // namespace dali_hip
 

@@ -415,6 +415,50 @@ int topk_rows(const void* x, int rows, int cols, int k, bool largest, bool ties_
     return status;
 }
 
+// One launch of the rank sort: `tickets` holds one zeroed counter per block of 256 keys (each is set back to zero by the
+// workgroup that consumes it), `partial` room for ceil(n / kRankSegment) * n counts.
+static int launch_rank_sort(const int32_t* keys, int ni, int32_t key_limit, unsigned int* tickets, int32_t* partial, int32_t* sorted_keys,
+                            int32_t* perm, hipStream_t st) {
+    const int segments = (ni + kRankSegment - 1) / kRankSegment, blocks = (ni + 255) / 256;
+    int shift = 0;
+    while ((1 << shift) < ni) ++shift;
+    const bool packed = key_limit > 0 && ((unsigned long long)key_limit << shift) <= (1ull << 32);
+    if (packed)
+        hipLaunchKernelGGL(rank_sort_kernel<unsigned int>, dim3(blocks, segments), dim3(256), 0, st, keys, ni, shift, segments, partial, tickets,
+                           sorted_keys, perm);
+    else
+        hipLaunchKernelGGL(rank_sort_kernel<unsigned long long>, dim3(blocks, segments), dim3(256), 0, st, keys, ni, shift, segments, partial,
+                           tickets, sorted_keys, perm);
+    hipError_t le = hipGetLastError();
+    if (le != hipSuccess) return fail("rank sort launch failed: %s", hipGetErrorString(le));
+    return DALI_HIP_OK;
+}
+
+// ---------------------------------------------------------------- ordering without any allocation
+// dali_hip_argsort_i32_noalloc keeps the tickets and counts of the rank sort in a device array that is part of this
+// library's code object instead of the library workspace: callers that must not allocate (stream capture, serving
+// loops) get the same kernel with memory that exists from the moment the code object is loaded. Each device holds
+// its own copy of the array at its own address; the host-side name below is only a handle for hipGetSymbolAddress,
+// the kernels receive the address that call returned for the current device.
+constexpr int kNoAllocMaxKeys = kRankSegment * kRankMaxSegments;            // 16384 keys
+constexpr size_t kScratchTicketBytes = 256;                                // one ticket per 256 keys: 64 counters
+constexpr size_t kScratchPartialBytes = (size_t)kRankMaxSegments * kNoAllocMaxKeys * sizeof(int32_t);  // 2 MiB
+static_assert((size_t)(kNoAllocMaxKeys / 256) * sizeof(unsigned int) <= kScratchTicketBytes, "tickets do not fit");
+static __device__ __align__(256) unsigned char scratch[kScratchTicketBytes + kScratchPartialBytes];
+
+constexpr int kMaxDevices = 64;
+static unsigned char* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, 0 = not looked up
+
+int sort_scratch_init(int device) {
+    if (device < 0 || device >= kMaxDevices) return fail("sort_scratch_init: device %d out of range", device);
+    if (g_scratch_ptr[device]) return DALI_HIP_OK;
+    void* ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) return fail("hipGetSymbolAddress(scratch) failed on device %d: %s", device, hipGetErrorString(e));
+    g_scratch_ptr[device] = (unsigned char*)ptr;  // zero-initialised with the code object: the tickets start at zero
+    return DALI_HIP_OK;
+}
+
 }  // namespace dali_hip
 
 using namespace dali_hip;
@@ -451,23 +495,9 @@ extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_
     static const int rank_max = getenv("DALI_HIP_RANK_SORT_MAX") ? atoi(getenv("DALI_HIP_RANK_SORT_MAX")) : 16384;
     if (n <= rank_max && n <= (int64_t)kRankSegment * kRankMaxSegments &&
         (size_t)((n + kRankSegment - 1) / kRankSegment) * (size_t)n * sizeof(int32_t) <= kWorkspacePartialBytes &&
-        (n + 255) / 256 <= kWorkspaceCounters) {
-        const int ni = (int)n, segments = (ni + kRankSegment - 1) / kRankSegment, blocks = (ni + 255) / 256;
-        unsigned int* tickets = (unsigned int*)workspace();
-        int32_t* partial = (int32_t*)(workspace() + kWorkspaceCounterBytes);
-        int shift = 0;
-        while ((1 << shift) < ni) ++shift;
-        const bool packed = key_limit > 0 && ((unsigned long long)key_limit << shift) <= (1ull << 32);
-        if (packed)
-            hipLaunchKernelGGL(rank_sort_kernel<unsigned int>, dim3(blocks, segments), dim3(256), 0, st, keys, ni, shift, segments, partial, tickets,
-                               sorted_keys, perm);
-        else
-            hipLaunchKernelGGL(rank_sort_kernel<unsigned long long>, dim3(blocks, segments), dim3(256), 0, st, keys, ni, shift, segments, partial,
-                               tickets, sorted_keys, perm);
-        hipError_t le = hipGetLastError();
-        if (le != hipSuccess) return fail("rank sort launch failed: %s", hipGetErrorString(le));
-        return DALI_HIP_OK;
-    }
+        (n + 255) / 256 <= kWorkspaceCounters)
+        return launch_rank_sort(keys, (int)n, key_limit, (unsigned int*)workspace(), (int32_t*)(workspace() + kWorkspaceCounterBytes), sorted_keys,
+                                perm, st);
     void* positions = nullptr;
     if (dali_hip_bank_allocate(&positions, (size_t)n * sizeof(int32_t))) return DALI_HIP_ERROR;
     hipLaunchKernelGGL(iota_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (int32_t*)positions, (long)n);
@@ -487,4 +517,18 @@ extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_
     if (temp) dali_hip_bank_deposit(temp, temp_bytes ? temp_bytes : 4);
     dali_hip_bank_deposit(positions, (size_t)n * sizeof(int32_t));
     return status;
+}
+
+extern "C" int dali_hip_argsort_i32_noalloc(const int32_t* keys, int64_t n, int32_t key_limit, int32_t* sorted_keys, int32_t* perm) {
+    const int device = bound_device();
+    if (device < 0) return fail("dali_hip_argsort_i32_noalloc: call dali_hip_init first (initialisation allocates, this call must not)");
+    if (n < 0) return fail("dali_hip_argsort_i32_noalloc: negative length %lld", (long long)n);
+    if (n > kNoAllocMaxKeys)
+        return fail("dali_hip_argsort_i32_noalloc: %lld keys exceed the limit of %d keys that the built-in scratch array serves", (long long)n,
+                    kNoAllocMaxKeys);
+    if (n == 0) return DALI_HIP_OK;
+    if (!keys || !sorted_keys || !perm) return fail("dali_hip_argsort_i32_noalloc: NULL argument");
+    unsigned char* base = device < kMaxDevices ? g_scratch_ptr[device] : nullptr;
+    if (!base) return fail("dali_hip_argsort_i32_noalloc: no scratch address for device %d", device);
+    return launch_rank_sort(keys, (int)n, key_limit, (unsigned int*)base, (int32_t*)(base + kScratchTicketBytes), sorted_keys, perm, stream());
 }

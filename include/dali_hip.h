@@ -257,6 +257,18 @@ int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx
 int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_limit, int32_t* sorted_keys, int32_t* perm);
 
 /*
+ * dali_hip_argsort_i32 for callers that cannot allocate: code under HIP graph capture, tight serving loops and
+ * harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments and same result as
+ * dali_hip_argsort_i32, for at most 16384 keys (more is an error, nothing is launched). The tickets and counts of the
+ * ordering kernel live in a 2 MiB + 256 B device array that is part of the library's code object (each device that the
+ * library runs on holds it until the process ends); the call allocates and frees nothing, neither from the driver nor
+ * from the bank. dali_hip_init must have been called before (it allocates; this call does not initialise). All calls
+ * on a device share that array: calls that overlap on one device (from two threads, or on streams other than the
+ * library stream) race; calls issued one after the other are ordered by the library stream.
+ */
+int dali_hip_argsort_i32_noalloc(const int32_t* keys, int64_t n, int32_t key_limit, int32_t* sorted_keys, int32_t* perm);
+
+/*
  * The column numbers of the k best entries of every row of a dense row-major [rows, cols] matrix, best first, into
  * out[rows, k]. Replaces the reference's CPU-only CpuTopKImpl (dali/array/op/top_k.cpp:36-196; "add gpu impl of topk"
  * is a TODO there, :198). dtype: 0 = float, 1 = double, 2 = int32. largest != 0 orders by descending value (top_k),
