@@ -10,8 +10,9 @@ before the timed region started. Steps are issued from a launch recording (the
 expression is planned and hipRTC-compiled once, outside the timed region).
 
 Prints ONE JSON line. `value` is algorithmic bytes (1 read + 1 write of the
-matrix) per second over the K timed steps; `roofline` is the same kernel priced
-against the 8 TB/s HBM peak with HIP events on the library stream; `configs`
+matrix) per second over the K timed steps, timed with HIP events on the library
+stream (host wall time is reported beside it); `roofline` is the same figure
+priced against the 8 TB/s HBM peak; `configs`
 carries the other four BASELINE.json configurations (GB/s, TFLOP/s or us);
 `cpu_baseline` is the CPU checker (a port of the reference's sequential loops)
 timed on one host core on a bounded sample of the same workload.
@@ -20,6 +21,7 @@ import argparse
 import ctypes as C
 import json
 import os
+import re
 import sys
 import time
 
@@ -30,6 +32,20 @@ HBM_PEAK_GBS = 8000.0
 MFMA_FP32_PEAK_TFLOPS = 157.3
 
 
+def traffic_from_profile(kernel):
+    """HBM bytes per launch of `kernel` from the committed counter summary, or None when that summary was made on
+    another kernel (the name carries the hash of the generated code's structure and launch parameters)."""
+    path = os.path.join(ROOT, "profiles", "softmax_c1_hbm_traffic_pmc.md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, "profiles/softmax_c1_hbm_traffic_pmc.md is missing"
+    got = dict(re.findall(r"^(measured_kernel|traffic_bytes_per_launch): (\S+)$", text, re.M))
+    if got.get("measured_kernel") != kernel or "traffic_bytes_per_launch" not in got:
+        return None, "profiles/softmax_c1_hbm_traffic_pmc.md covers %s, this run launched %s" % (got.get("measured_kernel"), kernel)
+    return int(got["traffic_bytes_per_launch"]), "profiles/softmax_c1_hbm_traffic_pmc.md (measured on %s)" % kernel
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -37,6 +53,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-configs", action="store_true", help="skip the other four configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--c1-only", action="store_true",
+                    help="issue only the warm-up and the K timed softmax steps on the rotating pairs (what a kernel trace "
+                         "of the headline should contain) and print a short JSON line")
+    ap.add_argument("--graph", action="store_true", help="issue the timed softmax steps as HIP graph launches (one graph per group of steps)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter-collection helper: 20 softmax steps on rotating buffers, then 20 plain copies of "
                          "16,777,216 floats (64 MiB read + 64 MiB written each), nothing else; prints no JSON")
@@ -110,43 +130,81 @@ def main():
     t_first = time.perf_counter() - t_first
     jit1 = [C.c_uint64() for _ in range(3)]
     hip.dali_hip_jit_stats(*[C.byref(v) for v in jit1])
-    t_eager = time.perf_counter()
-    for _ in range(200):
-        op.softmax(inputs[0]).eval()
-    t_eager = (time.perf_counter() - t_eager) / 200
-    sync()
+    t_eager = 0.0
+    if not args.c1_only:  # (evaluations on one resident pair: kept out of a trace of the rotating steps)
+        t_eager = time.perf_counter()
+        for _ in range(200):
+            op.softmax(inputs[0]).eval()
+        t_eager = (time.perf_counter() - t_eager) / 200
+        sync()
     outside = {"first_eval_ms": round(t_first * 1e3, 1), "first_eval_compiled": int(jit1[0].value - jit0[0].value),
                "first_eval_disk_hits": int(jit1[1].value - jit0[1].value), "eager_eval_host_us": round(t_eager * 1e6, 1)}
-    singles = []
     with D.Recording() as cycle:
         for x in inputs:
             op.softmax(x).eval()
     softmax_kernel = D.last_kernel_names()
-    for x in inputs:
-        with D.Recording() as one:
-            op.softmax(x).eval()
-        singles.append(one)
     assert cycle.launches == n_pairs
 
-    def run_steps(k):
-        cycle.replay(k // n_pairs)
-        for i in range(k % n_pairs):
-            singles[i].replay(1)
+    def steps_recording(first, count):
+        """`count` steps as one recording, on the pairs first, first + 1, ... of the rotation."""
+        with D.Recording() as rec:
+            for i in range(count):
+                op.softmax(inputs[(first + i) % n_pairs]).eval()
+        assert rec.launches == count
+        return rec
 
-    run_steps(args.warmup)
+    # The K timed steps go on from the pair after the last warm-up step, so no timed step finds its buffers in the
+    # 256 MiB Infinity Cache (the 15 pairs touched in between are 480 MiB). They are issued by at most three calls
+    # (the steps up to the start of the rotation, whole rotations, the rest): the host is not in the timed path.
+    first = args.warmup % n_pairs
+    lead_n = min(args.steps, (n_pairs - first) % n_pairs)
+    cycles, tail_n = divmod(args.steps - lead_n, n_pairs)
+    lead = steps_recording(first, lead_n) if lead_n else None
+    tail = steps_recording(0, tail_n) if tail_n else None
+    warm_cycles, warm_rest = divmod(args.warmup, n_pairs)
+    warm_tail = steps_recording(0, warm_rest) if warm_rest else None
+    preroll = steps_recording(first, n_pairs)
+
+    if args.graph:
+        for r in (cycle, lead, tail, preroll):
+            if r:
+                r.make_graph()
+                r.replay(1)
+    cycle.replay(warm_cycles)
+    if warm_tail:
+        warm_tail.replay(1)
     sync()
     t0 = time.perf_counter()
+    # One more untimed rotation is queued in front of the start event and not waited for: while the device works
+    # through it the host records the event and issues the timed steps, so the two events bracket the device's time
+    # for exactly K launches and not the host's call latency (which at K = 20 would be a tenth of the region).
+    preroll.replay(1)
     ev.start()
-    run_steps(args.steps)
-    ev_ms = ev.stop_ms()
+    if lead:
+        lead.replay(1)
+    if cycles:
+        cycle.replay(cycles)
+    if tail:
+        tail.replay(1)
+    ev_ms = ev.stop_ms()  # waits for the stop event: every timed step has finished
     sync()
     wall = time.perf_counter() - t0
-    gbs = step_bytes * args.steps / wall / 1e9
+    # one clock for the headline and for the roofline: HIP events on the library stream around the K launches
     kernel_us = ev_ms * 1e3 / args.steps
-    achieved = step_bytes / (kernel_us * 1e-6) / 1e9
+    gbs = step_bytes / (kernel_us * 1e-6) / 1e9
+    wall_steps = args.steps + n_pairs  # the host clock also saw the untimed rotation in front
+
+    traffic, traffic_note = traffic_from_profile(softmax_kernel)
+
+    if args.c1_only:
+        print(json.dumps({"kernel": softmax_kernel, "steps": args.steps, "warmup": args.warmup,
+                          "avg_launch_us_hip_events": round(kernel_us, 3), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+                          "host_wall_us_per_step": round(wall * 1e6 / wall_steps, 3)}))
+        return
 
     # same kernel on one resident pair (served from the on-chip caches): reported, not the headline
-    resident_us = time_recording(singles[0], 500, 20)
+    resident = steps_recording(0, 1)
+    resident_us = time_recording(resident, 500, 20)
 
     result = {
         "metric": "fused softmax fp32 [4096,1024] achieved HBM GB/s",
@@ -155,12 +213,16 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(wall * 1e3 / args.steps, 6),
+        "ms_per_step": round(kernel_us * 1e-3, 6),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
+        "clock": "value, ms_per_step and roofline: HIP events on the library stream around the K timed launches; "
+                 "host_wall_ms_per_step: time.perf_counter around the same region plus the untimed rotation of %d steps queued "
+                 "in front of the start event and the final synchronisation, per step issued" % n_pairs,
+        "host_wall_ms_per_step": round(wall * 1e3 / wall_steps, 6),
         "config": {
             "workload": "C1 naive fused softmax exp(a-max)/sum over fp32 [4096,1024] ~ N(0,1), rotating over %d distinct "
                         "input/output pairs (512 MiB > 256 MiB Infinity Cache), one fused row kernel per step" % n_pairs,
@@ -172,15 +234,15 @@ def main():
         "roofline": {
             "bound": "hbm",
             "kernel": softmax_kernel,
-            "achieved": round(achieved, 1),
+            "achieved": round(gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "frac": round(gbs / HBM_PEAK_GBS, 4),
             "avg_launch_us": round(kernel_us, 3),
-            # HBM bytes per launch from the committed counter runs (FETCH_SIZE + WRITE_SIZE, each scaled by the
-            # same counter on a copy of known size); a property of the kernel, not re-measured by this script
-            "traffic": 33595354,
-            "traffic_source": "profiles/softmax_c1_hbm_traffic_pmc.md",
+            # HBM bytes per launch from the committed counter runs (FETCH_SIZE + WRITE_SIZE, each scaled by the same
+            # counter on a copy of known size), taken over only when they were made on this very kernel
+            "traffic": traffic,
+            "traffic_source": traffic_note,
         },
     }
 
@@ -189,7 +251,7 @@ def main():
     # ------------------------------------------------- the other four configs
     if not args.no_configs:
         configs = {}
-        del inputs, singles, cycle
+        del inputs, cycle, lead, tail, warm_tail, resident, preroll
 
         # C2 elementwise chain, 4 x 67,108,864 fp32 in, 1 out
         n = 67108864

@@ -131,8 +131,11 @@ static int rtc_compile(const std::string& arch, const char* src, std::vector<cha
     std::string arch_opt = "--offload-arch=" + arch;
     // No fast-math and no contraction: the CPU path this is checked against is
     // built without either (dali/utils/compiler.cpp:137-145).
+    // The leading kernel parameters (up to the 14 scalar registers the hardware offers) arrive preloaded with the wave
+    // instead of through a load at its start.
     const char* opts[] = {arch_opt.c_str(), "-O3", "-ffp-contract=off", "-std=c++17",
-                          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+                          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                          "-mllvm", "-amdgpu-kernarg-preload-count=14"};
     r = hiprtcCompileProgram(prog, (int)(sizeof(opts) / sizeof(opts[0])), opts);
     size_t log_size = 0;
     hiprtcGetProgramLogSize(prog, &log_size);
