@@ -32,6 +32,18 @@
 
 namespace dali_hip {
 
+// exp of the gate epilogue: the same sequence as the exp of the generated kernels (dali_expf in the device prelude of the
+// front-end), so that the fused step and the two-launch form round every gate identically.
+__device__ __forceinline__ float gate_expf(float x) {
+    const float c = 0x1.715476p+0f, cc = 0x1.4ae0bep-26f;
+    const float t = x * c;
+    float r = __builtin_fmaf(x, c, -t);
+    r = __builtin_fmaf(x, cc, r);
+    const float e = __builtin_amdgcn_exp2f(t);
+    const float fixed = __builtin_fmaf(e, r * 0x1.62e430p-1f, e);
+    return __builtin_fabsf(t) < 128.0f ? fixed : e;
+}
+
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
@@ -639,9 +651,9 @@ __global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
             const float gf = tile[r * BN + 16 + j] + gate_bias[q][1];
             const float go = tile[r * BN + 32 + j] + gate_bias[q][2];
             const float gg = tile[r * BN + 48 + j] + gate_bias[q][3];
-            const float iv = (float)(1.0 / (1.0 + (double)expf(-gi)));
-            const float fv = (float)(1.0 / (1.0 + (double)expf(-gf)));
-            const float ov = (float)(1.0 / (1.0 + (double)expf(-go)));
+            const float iv = (float)(1.0 / (1.0 + (double)gate_expf(-gi)));
+            const float fv = (float)(1.0 / (1.0 + (double)gate_expf(-gf)));
+            const float ov = (float)(1.0 / (1.0 + (double)gate_expf(-go)));
             const float gv = tanhf(gg);
             const float fc = fv * gate_c[q];
             const float ig = iv * gv;

@@ -1562,10 +1562,10 @@ CrossEntropyResult softmax_cross_entropy(const Array& logits, const Array& targe
     Array lse = add(log(s), m);
     Array picked = gather_from_rows(logits, targets).expand_dims(1);
     Array row_loss = subtract(lse, picked);
-    Array::eval_together({grad, row_loss});
+    // the mean over the rows rides along in the same launch (its partial sums meet in the library workspace)
+    Array mean_loss = mean(row_loss);
+    Array::eval_together({grad, row_loss, mean_loss});
     Array rows1d = row_loss.reshape({rows});
-    Array mean_loss = mean(rows1d);
-    mean_loss.eval();
     return {mean_loss, rows1d, grad};
 }
 

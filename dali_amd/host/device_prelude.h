@@ -6,7 +6,7 @@
 // from): float arguments use the float libm entry points, `sigmoid` and the other
 // functors written with double literals evaluate in double and round once.
 // The reducers restate dali/array/jit/reducer_kernels.h:57-169 (init values
-// 0 / -FLT_MAX / FLT_MAX / 1; maximum is `dst > src ? dst : src`).
+// 0 / -FLT_MAX / FLT_MAX / 1; maximum of floats is the device branch's fmaxf).
 #ifndef DALI_AMD_DEVICE_PRELUDE_H
 #define DALI_AMD_DEVICE_PRELUDE_H
 
@@ -98,7 +98,23 @@ DI void dali_storeu_nt(T* p, const dali_vec<T, N>& v) {
 }
 
 // ------------------------------------------------------------ libm dispatch
-DI float  m_exp(float a)  { return expf(a); }
+// exp for float arguments. 2^(x * log2 e) on the hardware's exp2 unit, with the rounding error of the product put back:
+// t = fl(x * c), r = x * c - t exactly (one FMA) plus x times the part of log2 e that c lacks, and 2^(t + r) =
+// 2^t * (1 + r ln 2) to first order (|r| < 2^-17). About 1 ulp from the correctly rounded value wherever the result
+// is a normal number, which is what libm's expf delivers; results below the normal range come out as zero. Outside
+// |t| < 128 (overflow, underflow, infinities, NaN) the exp2 unit's own answer is already the right one and the
+// correction (which would be inf * 0 there) is left out. Eleven issue slots against about eighteen for the library
+// routine: a row kernel that exponentiates every element is otherwise bound by the vector ALU, not by memory.
+DI float dali_expf(float x) {
+    const float c = 0x1.715476p+0f, cc = 0x1.4ae0bep-26f;
+    const float t = x * c;
+    float r = __builtin_fmaf(x, c, -t);
+    r = __builtin_fmaf(x, cc, r);
+    const float e = __builtin_amdgcn_exp2f(t);
+    const float fixed = __builtin_fmaf(e, r * 0x1.62e430p-1f, e);
+    return __builtin_fabsf(t) < 128.0f ? fixed : e;
+}
+DI float  m_exp(float a)  { return dali_expf(a); }
 DI double m_exp(double a) { return exp(a); }
 DI double m_exp(int a)    { return exp((double)a); }
 DI float  m_log(float a)  { return logf(a); }
@@ -259,14 +275,23 @@ template <typename T> DI T highest();
 template <> DI float highest<float>() { return DALI_FLT_MAX; }
 template <> DI double highest<double>() { return DALI_DBL_MAX; }
 template <> DI int highest<int>() { return DALI_INT_MAX; }
+// float and double: fmax / fmin, one instruction each, which is also what the reference's device code calls
+// (dali/array/jit/reducer_kernels.h:92-98,127-131 under __CUDACC__); on numbers it equals the host form
+// `dst > src ? dst : src`, the two differ only in which operand survives a NaN.
+DI float dali_max(float d, float s) { return __builtin_fmaxf(d, s); }
+DI double dali_max(double d, double s) { return __builtin_fmax(d, s); }
+DI int dali_max(int d, int s) { return d > s ? d : s; }
+DI float dali_min(float d, float s) { return __builtin_fminf(d, s); }
+DI double dali_min(double d, double s) { return __builtin_fmin(d, s); }
+DI int dali_min(int d, int s) { return d < s ? d : s; }
 struct maximum {
     template <typename T> DI static T init() { return lowest<T>(); }
-    template <typename T> DI static T step(T d, T s) { return d > s ? d : s; }
+    template <typename T> DI static T step(T d, T s) { return dali_max(d, s); }
     template <typename T> DI static bool better(T cand, T cur) { return cand > cur; }
 };
 struct minimum {
     template <typename T> DI static T init() { return highest<T>(); }
-    template <typename T> DI static T step(T d, T s) { return d < s ? d : s; }
+    template <typename T> DI static T step(T d, T s) { return dali_min(d, s); }
     template <typename T> DI static bool better(T cand, T cur) { return cand < cur; }
 };
 }  // namespace reducers
@@ -317,12 +342,52 @@ DI T dali_wave_scan(T v) {
     return v;
 }
 
+// A lane's value as another lane holds it, moved by the data-parallel-primitive path of the vector ALU (a few
+// cycles) instead of through the LDS crossbar that __shfl uses (a round trip of its own per step). CTRL: 0xB1 / 0x4E
+// swap neighbours / pairs inside a quad, 0x141 / 0x140 mirror a half row / a row of 16 lanes, 0x142 / 0x143 hand
+// lane 15 of every row to the next row / lane 31 to the upper half; ROW_MASK picks the rows of 16 lanes that receive
+// (the others keep their value).
+template <int CTRL, int ROW_MASK>
+DI int dali_dpp_word(int v) { return __builtin_amdgcn_update_dpp(v, v, CTRL, ROW_MASK, 0xF, false); }
+template <typename T, int CTRL, int ROW_MASK>
+DI T dali_dpp(T v) {
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, dali_dpp_word<CTRL, ROW_MASK>(__builtin_bit_cast(int, v)));
+    } else {
+        static_assert(sizeof(T) == 8, "4- or 8-byte values");
+        long long w = __builtin_bit_cast(long long, v);
+        const int lo = dali_dpp_word<CTRL, ROW_MASK>((int)w), hi = dali_dpp_word<CTRL, ROW_MASK>((int)(w >> 32));
+        return __builtin_bit_cast(T, ((long long)hi << 32) | (unsigned int)lo);
+    }
+}
+template <typename T>
+DI T dali_readlane(T v, int lane) {
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+    } else {
+        long long w = __builtin_bit_cast(long long, v);
+        const int lo = __builtin_amdgcn_readlane((int)w, lane), hi = __builtin_amdgcn_readlane((int)(w >> 32), lane);
+        return __builtin_bit_cast(T, ((long long)hi << 32) | (unsigned int)lo);
+    }
+}
+
 // Reduce over aligned groups of WIDTH lanes (WIDTH a power of two <= 64); every
-// lane of the group ends with the group's result.
+// lane of the group ends with the group's result. Groups of up to 16 lanes stay inside a row of the data-parallel
+// path (exchange inside quads, then mirrored halves: after every step the lanes that have met hold the same value);
+// 32 lanes add one exchange through the crossbar; a whole wave adds two row hand-offs, which leave the result in
+// lane 63, and reads that lane for everybody (a scalar from there on).
 template <typename R, typename T, int WIDTH>
 DI T dali_group_reduce(T v) {
-#pragma unroll
-    for (int m = WIDTH / 2; m >= 1; m >>= 1) v = R::template step<T>(v, dali_shfl_xor<T>(v, m));
+    if constexpr (WIDTH >= 2) v = R::template step<T>(v, dali_dpp<T, 0xB1, 0xF>(v));
+    if constexpr (WIDTH >= 4) v = R::template step<T>(v, dali_dpp<T, 0x4E, 0xF>(v));
+    if constexpr (WIDTH >= 8) v = R::template step<T>(v, dali_dpp<T, 0x141, 0xF>(v));
+    if constexpr (WIDTH >= 16) v = R::template step<T>(v, dali_dpp<T, 0x140, 0xF>(v));
+    if constexpr (WIDTH == 32) v = R::template step<T>(v, dali_shfl_xor<T>(v, 16));
+    if constexpr (WIDTH == 64) {
+        v = R::template step<T>(v, dali_dpp<T, 0x142, 0xA>(v));
+        v = R::template step<T>(v, dali_dpp<T, 0x143, 0xC>(v));
+        v = dali_readlane<T>(v, 63);
+    }
     return v;
 }
 

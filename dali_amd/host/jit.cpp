@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-32";
+const char* const kCodegenVersion = "dali-hip-codegen-33";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -653,6 +653,9 @@ struct Output {
     int array;       // dest array index
     OPERATOR_T op;
     Cls cls;
+    // row kernel only: the destination is one value for the whole launch, root = [scalar arithmetic over] a full
+    // reduction (this node) of a value the kernel holds per row (the mean of the row losses of a cross-entropy)
+    int total_red = -1;
 };
 
 bool expensive_functor(const std::string& name) {
@@ -742,7 +745,7 @@ std::string signature(const Program& P, const std::vector<Output>& outs) {
     ss << "#";
     for (const ScalarArg& s : P.scalars) ss << (int)s.dtype << ";";
     ss << "#";
-    for (const Output& o : outs) ss << o.root << ">" << o.array << ":" << (int)o.op << ":" << (int)o.cls << ";";
+    for (const Output& o : outs) ss << o.root << ">" << o.array << ":" << (int)o.op << ":" << (int)o.cls << ":" << o.total_red << ";";
     return ss.str();
 }
 
@@ -1002,6 +1005,80 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
         }
     }
 
+    // totals over the rows: value per row -> workgroup (wave order) -> workspace slot -> last workgroup folds the slots
+    std::vector<const Output*> totals;
+    for (const Output& o : rpn.outputs)
+        if (o.total_red >= 0) totals.push_back(&o);
+    const int NWB = rp.BT / 64;
+    // The slot and the ticket go out before the rows are written: the wave that draws the ticket waits for its earlier
+    // memory operations, and after the output loop those would be a whole row of stores (the workgroup would keep
+    // its place on the compute unit until they are acknowledged).
+    auto emit_totals_publish = [&]() {
+        ss << "  constexpr int BT = " << rp.BT << ";\n";
+        ss << "  unsigned int* counters = (unsigned int*)A.ws;\n  char* slots = (char*)A.ws + " << 16384 * 4 << ";\n";
+        ss << "  __shared__ int is_last;\n";
+        for (size_t k = 0; k < totals.size(); ++k) {
+            const PNode& red = P.nodes[totals[k]->total_red];
+            const std::string t = ctype(P.nodes[red.args[0]].dtype);
+            ss << "  " << t << " tot" << k << " = " << red.name << "::init<" << t << ">();\n";
+            ss << "  __shared__ " << t << " smt" << k << "[" << NWB << "];\n";
+        }
+        ss << "  if (tr == 0 && row_ok) {\n";
+        {
+            BodyEmitter be(P, rp, false, rpn.n_phases, &rpn.first_body);
+            std::ostringstream body;
+            for (size_t k = 0; k < totals.size(); ++k) body << "    tot" << k << " = " << be.value(P.nodes[totals[k]->total_red].args[0]) << ";\n";
+            ss << be.stmts.str() << body.str();
+        }
+        ss << "  }\n";
+        for (size_t k = 0; k < totals.size() && rp.RPB > 1; ++k) {  // (one row per workgroup: thread 0 holds its value already)
+            const PNode& red = P.nodes[totals[k]->total_red];
+            const std::string t = ctype(P.nodes[red.args[0]].dtype);
+            ss << "  tot" << k << " = dali_block_reduce<" << red.name << ", " << t << ", " << NWB << ">(tot" << k << ", smt" << k << ");\n";
+        }
+        ss << "  if (tid == 0) {\n";
+        for (size_t k = 0; k < totals.size(); ++k) {
+            const std::string t = ctype(P.nodes[P.nodes[totals[k]->total_red].args[0]].dtype);
+            ss << "    dali_publish((" << t << "*)(slots + ((size_t)" << k << " * gridDim.x + blockIdx.x) * 8), tot" << k << ");\n";
+        }
+        ss << "    is_last = dali_take_ticket(&counters[0]) == gridDim.x - 1;\n  }\n";
+    };
+    auto emit_totals_fold = [&]() {
+        ss << "  __syncthreads();\n  if (!is_last) return;\n";
+        // fixed order: thread t folds slots t, t + BT, ... (eight loads in flight at a time), then the workgroup folds in wave order
+        for (size_t k = 0; k < totals.size(); ++k) {
+            const PNode& red = P.nodes[totals[k]->total_red];
+            const std::string t = ctype(P.nodes[red.args[0]].dtype);
+            ss << "  tot" << k << " = " << red.name << "::init<" << t << ">();\n";
+            ss << "  for (unsigned int base = tid; base < gridDim.x; base += BT * 8) {\n    " << t << " pv[8];\n";
+            ss << "    _Pragma(\"unroll\") for (int u = 0; u < 8; ++u) { const unsigned int b = base + u * BT; if (b < gridDim.x) pv[u] = dali_observe((const " << t
+               << "*)(slots + ((size_t)" << k << " * gridDim.x + b) * 8)); }\n";
+            ss << "    _Pragma(\"unroll\") for (int u = 0; u < 8; ++u) { const unsigned int b = base + u * BT; if (b < gridDim.x) tot" << k << " = " << red.name
+               << "::step<" << t << ">(tot" << k << ", pv[u]); }\n  }\n";
+            ss << "  __syncthreads();\n";
+            ss << "  tot" << k << " = dali_block_reduce<" << red.name << ", " << t << ", " << NWB << ">(tot" << k << ", smt" << k << ");\n";
+        }
+        ss << "  if (tid == 0) {\n    dali_publish(&counters[0], 0u);\n";
+        {
+            BodyEmitter be(P, rp, false, rpn.n_phases + 1, &rpn.first_body);
+            std::ostringstream body;
+            for (size_t k = 0; k < totals.size(); ++k) {
+                const Output& o = *totals[k];
+                const PNode& red = P.nodes[o.total_red];
+                ss << "    const " << ctype(red.dtype) << " red" << o.total_red << " = tot" << k << ";\n";
+            }
+            for (size_t k = 0; k < totals.size(); ++k) {
+                const Output& o = *totals[k];
+                const std::string dt = ctype(P.arrays[o.array].buf->dtype);
+                const std::string v = be.value(o.root);
+                body << "    q" << o.array << "[0] = " << op_combine(o.op, "q" + std::to_string(o.array) + "[0]", "(" + dt + ")(" + v + ")") << ";\n";
+            }
+            ss << be.stmts.str() << body.str();
+        }
+        ss << "  }\n";
+    };
+    if (!totals.empty()) emit_totals_publish();
+
     // output body: FULL destinations
     bool any_full = false;
     for (const Output& o : rpn.outputs) any_full = any_full || o.cls == Cls::FULL;
@@ -1056,19 +1133,20 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
     }
     // ROW / SCAL destinations: one thread per row writes
     bool any_row = false;
-    for (const Output& o : rpn.outputs) any_row = any_row || o.cls != Cls::FULL;
+    for (const Output& o : rpn.outputs) any_row = any_row || (o.cls != Cls::FULL && o.total_red < 0);
     if (any_row) {
         ss << "  if (tr == 0 && row_ok) {\n";
         BodyEmitter be(P, rp, false, rpn.n_phases, &rpn.first_body);
         std::ostringstream body;
         for (const Output& o : rpn.outputs) {
-            if (o.cls == Cls::FULL) continue;
+            if (o.cls == Cls::FULL || o.total_red >= 0) continue;
             std::string t = ctype(P.arrays[o.array].buf->dtype);
             std::string v = be.value(o.root);
             body << "    q" << o.array << "[0] = " << op_combine(o.op, "q" + std::to_string(o.array) + "[0]", "(" + t + ")(" + v + ")") << ";\n";
         }
         ss << be.stmts.str() << body.str() << "  }\n";
     }
+    if (!totals.empty()) emit_totals_fold();
     ss << "}\n";
     return ss.str();
 }
@@ -1239,7 +1317,11 @@ bool ragged_ok(const Program& P, const Domain& dom) {
     return true;
 }
 
-bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
+// `totals`: further requests whose destination holds one element and whose root is [scalar arithmetic over] one full
+// reduction of an expression with one value per row of `dom` (the mean of the row losses next to the gradient of a
+// cross-entropy). They ride along in the same launch: every workgroup publishes the combination of its rows' values,
+// the workgroup that draws the last ticket folds those in workgroup order, applies the scalar arithmetic and stores.
+bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::vector<DestSpec>* totals = nullptr) {
     RowPlan rpn;
     Program& P = rpn.P;
     rpn.dom = dom;
@@ -1262,23 +1344,78 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
         o.root = -1;
         rpn.outputs.push_back(o);
     }
+    const size_t n_totals = totals ? totals->size() : 0;
+    for (size_t k = 0; k < n_totals; ++k) {
+        const DestSpec& s = (*totals)[k];
+        if (numel_of(s.dest.shape()) != 1) return false;
+        int ai = add_array(P, s.dest.expression(), Cls::SCAL, false, dom, true);
+        if (ai < 0) return false;
+        Output o;
+        o.array = ai;
+        o.op = s.op;
+        o.cls = Cls::SCAL;
+        o.root = -1;
+        rpn.outputs.push_back(o);
+    }
     for (size_t i = 0; i < specs.size(); ++i) {
         int r = add_node(P, specs[i].root);
         rpn.outputs[i].root = r;
         roots.push_back(r);
     }
+    for (size_t k = 0; k < n_totals; ++k) {
+        int r = add_node(P, (*totals)[k].root);
+        rpn.outputs[specs.size() + k].root = r;
+        roots.push_back(r);
+    }
     for (size_t i = 0; i < specs.size(); ++i)
         if (!classify(P, roots[i], rpn.outputs[i].cls, dom)) return false;
+    for (size_t k = 0; k < n_totals; ++k) {
+        // the scalar arithmetic above the full reduction, then the reduced expression as one value per row
+        int found = -1;
+        std::function<bool(int)> cls_epi = [&](int id) -> bool {
+            PNode& nd = P.nodes[id];
+            if (nd.kind == Kind::ALL_REDUCE) {
+                if (found >= 0 && found != id) return false;
+                if (nd.cls_set && nd.cls != Cls::SCAL) return false;
+                found = id;
+                nd.cls = Cls::SCAL;
+                nd.cls_set = true;
+                if (numel_of(P.nodes[nd.args[0]].shape) != dom.R || dom.C == 1) return false;
+                return classify(P, nd.args[0], Cls::ROW, dom);
+            }
+            if (numel_of(nd.shape) != 1) return false;
+            if (nd.kind == Kind::SCALAR) { nd.cls = Cls::SCAL; nd.cls_set = true; return true; }
+            if (nd.cls_set) return nd.cls == Cls::SCAL;
+            if (nd.kind == Kind::BUFFER) {
+                nd.cls = Cls::SCAL;
+                nd.cls_set = true;
+                int ai = add_array(P, nd.src, Cls::SCAL, false, dom, false);
+                if (ai < 0) return false;
+                P.nodes[id].array = ai;
+                return true;
+            }
+            if (nd.kind != Kind::ELEMENTWISE && nd.kind != Kind::EXPAND_DIMS && nd.kind != Kind::BROADCAST) return false;
+            nd.cls = Cls::SCAL;
+            nd.cls_set = true;
+            std::vector<int> args = nd.args;
+            for (int a : args)
+                if (!cls_epi(a)) return false;
+            return true;
+        };
+        if (!cls_epi(roots[specs.size() + k]) || found < 0) return false;
+        rpn.outputs[specs.size() + k].total_red = found;
+    }
     // phases
     std::vector<bool> seen(P.nodes.size(), false);
     for (int r : roots) compute_dep(P, r, seen);
     int nph = 0;
+    // (the full reductions of `totals` are no phases of a row: they are folded across workgroups at the end)
     for (size_t id = 0; id < P.nodes.size(); ++id)
-        if (seen[id] && is_reduce(P.nodes[id].kind)) nph = std::max(nph, P.nodes[id].phase + 1);
+        if (seen[id] && is_reduce(P.nodes[id].kind) && !is_all_reduce(P.nodes[id].kind)) nph = std::max(nph, P.nodes[id].phase + 1);
     rpn.n_phases = nph;
     rpn.phase_reduces.assign(nph, {});
     for (size_t id = 0; id < P.nodes.size(); ++id)
-        if (seen[id] && is_reduce(P.nodes[id].kind)) rpn.phase_reduces[P.nodes[id].phase].push_back((int)id);
+        if (seen[id] && is_reduce(P.nodes[id].kind) && !is_all_reduce(P.nodes[id].kind)) rpn.phase_reduces[P.nodes[id].phase].push_back((int)id);
     count_uses(P, roots);
 
     // launch geometry
@@ -1401,6 +1538,12 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom) {
     rp.nt_stores = nt_s >= 0 ? nt_s != 0 : true;
     params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached << "," << rp.waves_per_eu << ","
            << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail << "," << rp.EPT_L;
+    if (n_totals) {
+        // one 8-byte slot per workgroup and total in the workspace's 32 MiB of partial results
+        const int64_t blocks = (dom.R + rp.RPB - 1) / rp.RPB;
+        if (blocks * (int64_t)n_totals * 8 > ((int64_t)32 << 20) || blocks > 2147483647LL) return false;
+        params << ",T" << n_totals;
+    }
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     std::string sig = signature(P, rpn.outputs);
     uint64_t h = kernel_hash("row", sig, params.str());
@@ -2560,9 +2703,10 @@ Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root) {
         case Kind::ALL_REDUCE:
         case Kind::ARG_ALL_REDUCE: {
             Array arg = clean(e->args[0], memo, false);
-            if (has_kind(arg, [](Kind k) { return is_reduce(k); })) arg = materialize(arg);
+            // An argument that holds reductions of its own is evaluated first. Under a root the planner decides: such a
+            // full reduction may join the row kernel of the roots evaluated with it, or is split off there.
+            if (!is_root && has_kind(arg, [](Kind k) { return is_reduce(k); })) arg = materialize(arg);
             if (arg.expression().get() != e->args[0].expression().get()) out = rebuild(e, {arg});
-            (void)is_root;
             break;
         }
         case Kind::ELEMENTWISE: {
@@ -3000,6 +3144,36 @@ void run_specs_planned(std::vector<DestSpec> specs) {
         bool any_all = false;
         for (auto& s : specs) any_all = any_all || has_kind(s.root, [](Kind k) { return is_all_reduce(k); });
         if (any_all) {
+            // Full reductions of per-row values next to requests over the rows themselves (the mean loss beside the
+            // gradient and the row losses of a cross-entropy) join the row kernel of the others: one launch.
+            std::vector<DestSpec> plain, totals;
+            for (auto& s : specs) (has_kind(s.root, [](Kind k) { return is_all_reduce(k); }) ? totals : plain).push_back(s);
+            static const bool fuse_totals = env_int("DALI_HIP_ROW_TOTALS", 1) != 0;
+            bool row_reduces = !plain.empty();
+            for (auto& s : plain) row_reduces = row_reduces && !has_kind(s.root, [](Kind k) { return k == Kind::MATMUL; });
+            if (fuse_totals && row_reduces) {
+                Array first;
+                std::set<const Expr*> seen;
+                bool found = false;
+                for (auto& s : plain)
+                    if (find_first_reduce(s.root, &first, seen)) { found = true; break; }
+                if (found) {
+                    Domain dom = domain_of(first.expression()->args[0].shape());
+                    if (try_row(plain, dom, &totals)) return;
+                }
+            }
+            if (!plain.empty() && !totals.empty()) {
+                // otherwise the others first, together; what they computed is not computed again for the full reductions
+                run_specs(plain);
+                for (auto& t : totals) {
+                    for (auto& p : plain) {
+                        std::map<const Expr*, Array> memo;
+                        t.root = substitute(t.root, p.root.expression().get(), p.dest, memo);
+                    }
+                    run_specs({t});
+                }
+                return;
+            }
             for (auto& s : specs) run_specs({s});
             return;
         }

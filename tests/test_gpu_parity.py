@@ -777,13 +777,13 @@ def test_gather_from_rows_and_one_hot(gpu, D, O, rng):
     assert np.array_equal(op.one_hot(arr(D, i2), 13, np.float32(1), np.float32(0)).numpy(), O.one_hot(i2, 13))
 
 
-@pytest.mark.parametrize("shape", [(5, 97), (37, 1000), (16, 32000), (3, 50001)])
+@pytest.mark.parametrize("shape", [(5, 97), (300, 17), (1000, 64), (4099, 33), (37, 1000), (16, 32000), (3, 50001)])
 def test_softmax_cross_entropy_matches_oracle(gpu, D, O, rng, shape):
     x = (rng.randn(*shape) * 2).astype(np.float32)
     t = rng.randint(0, shape[1], shape[0]).astype(np.int32)
     k0 = D.jit_stats()["kernels"]
     mean, rows, grad = D.op.softmax_cross_entropy(arr(D, x), arr(D, t))
-    assert D.jit_stats()["kernels"] - k0 == 2  # one fused row pass (gradient + row losses) + the mean
+    assert D.jit_stats()["kernels"] - k0 == 1  # one fused row pass: gradient, row losses and their mean
     omean, orows, ograd = O.softmax_cross_entropy(x, t)
     close(rows.numpy(), orows, rtol=1e-5, atol=shape[1] * 2.0 ** -24)  # log of the row sum: the sum's relative error is absolute here
     close(mean.numpy(), omean, rtol=1e-5, atol=shape[1] * 2.0 ** -24)
@@ -798,6 +798,42 @@ def test_softmax_cross_entropy_matches_oracle(gpu, D, O, rng, shape):
     # the reference's own forward, -log(gather_from_rows(softmax(x), t)) (cost.cpp:121-122), built from its ops
     fwd = (-1.0 * D.op.log(D.op.gather_from_rows(D.op.softmax(arr(D, x)), arr(D, t)))).numpy()
     close(fwd, O.softmax_cross_entropy_via_probs(x, t), rtol=1e-5, atol=1e-5 + shape[1] * 2.0 ** -24)
+
+
+@pytest.mark.parametrize("shape", [(7, 33), (300, 17), (1000, 256), (513, 4096), (2, 70001)])
+def test_full_reductions_of_row_values_join_the_row_kernel(gpu, D, O, rng, shape):
+    """Roots evaluated together: per-element and per-row results of a row kernel, and full reductions of per-row values
+    (their total, their maximum, a mean) computed by the same launch through the workspace."""
+    op = D.op
+    x = rng.randn(*shape).astype(np.float32)
+    X = arr(D, x)
+    rs = op.sum(op.exp(X), [-1], True)                 # [R, 1]
+    shifted = X - op.max(X, [-1], True)                # [R, C]
+    total = op.sum(rs)                                 # sum of the row sums
+    biggest = op.max(op.max(X, [-1], True))            # maximum of the row maxima
+    avg = op.mean(op.log(rs))                          # mean of a function of the row sums
+    k0 = D.jit_stats()["kernels"]
+    D.eval_together([shifted, rs, total, biggest, avg])
+    assert D.jit_stats()["kernels"] - k0 == 1 and D.last_kernel_kinds() == "row"
+    x64 = x.astype(np.float64)
+    rows = np.exp(x64).sum(1, keepdims=True)
+    close(shifted.numpy(), x - x.max(1, keepdims=True), rtol=0, atol=0)
+    close(rs.numpy(), rows, rtol=1e-5)
+    close(total.numpy(), rows.sum(), rtol=1e-5)
+    assert float(biggest.numpy()) == x.max()
+    close(avg.numpy(), np.log(rows).mean(), rtol=1e-5, atol=1e-6)
+    # the same roots one by one give the same values (the order of the partial sums is fixed in both forms)
+    X2 = arr(D, x)
+    t2 = op.sum(op.sum(op.exp(X2), [-1], True))
+    close(t2.numpy(), total.numpy(), rtol=1e-6)
+    # a second evaluation finds the ticket counter back at zero
+    D.eval_together([op.sum(op.exp(X2), [-1], True), op.sum(op.sum(op.exp(X2), [-1], True))])
+    # a full reduction that does not range over the rows of the others is planned on its own
+    other = arr(D, rng.randn(11, 5).astype(np.float32))
+    a, b = op.sum(X2, [-1], True), op.sum(other)
+    D.eval_together([a, b])
+    close(a.numpy(), x64.sum(1, keepdims=True), rtol=1e-5, atol=1e-5 * float(np.abs(x64).sum(1).max()))
+    close(b.numpy(), other.numpy().astype(np.float64).sum(), rtol=1e-5, atol=1e-5)
 
 
 # --------------------------------------------------------------------- dot
@@ -1048,8 +1084,9 @@ def test_recording_replays_the_same_device_work(gpu, D, rng):
 
 
 def test_graph_replays_match_eager_on_every_replay(gpu, D, O, rng):
-    # cross-entropy: a row kernel plus a two-stage `all` kernel (tickets and partials in the persistent
-    # workspace, which must come back to zero after each replay), then a column reduction
+    # cross-entropy: a row kernel that also folds the mean loss across workgroups, a two-stage `all` kernel (both keep
+    # tickets and partials in the persistent workspace, which must come back to zero after each replay), then a column
+    # reduction
     n, v = 96, 700
     logits = arr(D, rng.randn(n, v).astype(np.float32))
     targets = arr(D, rng.randint(0, v, n).astype(np.int32))
@@ -1057,16 +1094,19 @@ def test_graph_replays_match_eager_on_every_replay(gpu, D, O, rng):
         mean_loss, row_loss, grad = D.op.softmax_cross_entropy(logits, targets)
         colsum = D.op.sum(grad, [0])
         colsum.eval()
+        total = D.op.sum(D.op.square(grad))
+        total.eval()
     assert rec.launches >= 3
     rec.make_graph()
     for it in range(4):
         fresh = rng.randn(n, v).astype(np.float32)
         logits.assign(arr(D, fresh))  # eager work between replays changes the graph's input in place
         rec.replay(1)
-        got = [a.numpy() for a in (mean_loss, row_loss, grad, colsum)]
+        got = [a.numpy() for a in (mean_loss, row_loss, grad, colsum, total)]
         e_mean, e_row, e_grad = D.op.softmax_cross_entropy(arr(D, fresh), targets)
         e_col = D.op.sum(e_grad, [0])
-        for g, e in zip(got, (e_mean, e_row, e_grad, e_col)):
+        e_total = D.op.sum(D.op.square(e_grad))
+        for g, e in zip(got, (e_mean, e_row, e_grad, e_col, e_total)):
             assert np.array_equal(g, e.numpy()), "replay %d differs from the eager evaluation" % it
         o_loss = O.softmax_cross_entropy(fresh, targets.numpy())[1]
         close(got[1], o_loss, rtol=1e-5 + v * 2.0 ** -24, atol=1e-6)
