@@ -145,6 +145,7 @@ FRONT_SYMBOLS = {
     "dali_fe_mean_all": (H, [H]),
     "dali_fe_mean_axes": (H, [H, _ip, _i, _i]),
     "dali_fe_softmax": (H, [H, _i]),
+    "dali_fe_softmax_naive": (H, [H, _i]),
     "dali_fe_gather_from_rows": (H, [H, H]),
     "dali_fe_gather": (H, [H, H]),
     "dali_fe_axis_scan": (H, [H, C.c_char_p, _i]),

@@ -935,9 +935,21 @@ Array all_equals(const Array& left, const Array& right) { return prod(equals(lef
 Array all_close(const Array& left, const Array& right, const Array& atolerance) { return prod(close(left, right, atolerance)); }
 
 // dali/array/op/softmax.cpp:5-8
-Array softmax(const Array& logits, int axis) {
+Array softmax_naive(const Array& logits, int axis) {
     Array exped = exp(subtract(logits, max(logits, {axis}, true)));
     return eltdiv(exped, sum(exped, {axis}, true));
+}
+// The same expression, kept as one node until it is evaluated: the planner then writes it out as above, or, for shapes
+// that starve the fused row kernel (few very long rows, an axis that runs against memory), computes the maxima and the
+// sums of exponentials in a pass of their own first.
+Array softmax(const Array& logits, int axis) {
+    const int nd = logits.ndim();
+    const int ax = axis < 0 ? axis + nd : axis;
+    if (nd == 0 || ax < 0 || ax >= nd || logits.dtype() == DTYPE_INT32 || logits.number_of_elements() == 0)
+        return softmax_naive(logits, axis);  // (raises the reduction's own error for a bad axis)
+    Array out = make_node(Kind::SOFTMAX, "", {logits}, logits.shape(), logits.dtype());
+    out.expression()->axis = ax;
+    return out;
 }
 
 // dali/array/op/softmax.cpp:10-13: the reference does not read `temperature`; the result is softmax(logits, axis)

@@ -112,6 +112,7 @@ dali_array_t dali_fe_mean_axes(dali_array_t a, const int* axes, int naxes, int k
     FE_TRY(return wrap(dali::op::mean(A(a), vec(axes, naxes), keepdims != 0));, nullptr)
 }
 dali_array_t dali_fe_softmax(dali_array_t a, int axis) { FE_TRY(return wrap(dali::op::softmax(A(a), axis));, nullptr) }
+dali_array_t dali_fe_softmax_naive(dali_array_t a, int axis) { FE_TRY(return wrap(dali::op::softmax_naive(A(a), axis));, nullptr) }
 dali_array_t dali_fe_softmax_temperature(dali_array_t a, dali_array_t temperature, int axis) {
     FE_TRY(return wrap(dali::op::softmax_temperature(A(a), A(temperature), axis));, nullptr)
 }

@@ -264,6 +264,8 @@ Array all_close(const Array& left, const Array& right, const Array& atolerance);
 
 // dali/array/op/softmax.h, gather_from_rows.h, one_hot.h, dot.h
 Array softmax(const Array& logits, int axis = -1);
+// the written-out expression of dali/array/op/softmax.cpp:5-8 (what op::softmax becomes when it is evaluated)
+Array softmax_naive(const Array& logits, int axis = -1);
 Array softmax_temperature(const Array& logits, const Array& temperature, int axis = -1);
 Array gather_from_rows(const Array& source, const Array& indices);
 Array gather(const Array& source, const Array& indices);

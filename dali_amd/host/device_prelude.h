@@ -294,13 +294,58 @@ struct minimum {
     template <typename T> DI static T step(T d, T s) { return dali_min(d, s); }
     template <typename T> DI static bool better(T cand, T cur) { return cand < cur; }
 };
+// Running (maximum, sum of exp(x - maximum)) of a softmax, for reductions against the memory layout where the values
+// cannot stay in registers between a max pass and a sum pass: one pass over the data yields both. Feeding a value
+// costs one exp (of minus the distance between the value and the running maximum; one of the two terms keeps the
+// factor exp(0)); two partial results combine the same way. A fresh accumulator is (-FLT_MAX, 0).
+struct dali_ms { float m, l; };
+struct maxsumexp {
+    template <typename T> DI static dali_ms init() { dali_ms r; r.m = -DALI_FLT_MAX; r.l = 0.0f; return r; }
+    DI static dali_ms feed(dali_ms a, float x) {
+        const float d = x - a.m;
+        const float e = dali_expf(-__builtin_fabsf(d));
+        dali_ms r;
+        r.m = __builtin_fmaxf(a.m, x);
+        r.l = d > 0.0f ? a.l * e + 1.0f : a.l + e;
+        return r;
+    }
+    // N values at once: their maximum first, then one exp per value against the new running maximum and one to carry
+    // the old sum over; the N exponentials are added among themselves before they meet the running sum.
+    template <int N> DI static dali_ms feed_n(dali_ms a, const float* x) {
+        float bm = x[0];
+#pragma unroll
+        for (int u = 1; u < N; ++u) bm = __builtin_fmaxf(bm, x[u]);
+        dali_ms r;
+        r.m = __builtin_fmaxf(a.m, bm);
+        float s = 0.0f;
+#pragma unroll
+        for (int u = 0; u < N; ++u) s += dali_expf(x[u] - r.m);
+        r.l = a.l * dali_expf(a.m - r.m) + s;
+        return r;
+    }
+    template <typename T> DI static dali_ms step(dali_ms a, dali_ms b) {
+        const float d = b.m - a.m;
+        const float e = dali_expf(-__builtin_fabsf(d));
+        dali_ms r;
+        r.m = __builtin_fmaxf(a.m, b.m);
+        r.l = d > 0.0f ? a.l * e + b.l : a.l + b.l * e;
+        return r;
+    }
+};
 }  // namespace reducers
+using reducers::dali_ms;
 
 // ------------------------------------------------- cross-workgroup hand-off
 // Agent-scope relaxed atomics: the store is written through to the coherence point
 // shared by all XCDs, the load does not return a stale line of the local L2.
 template <typename T> DI void dali_publish(T* p, T v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 template <typename T> DI T dali_observe(const T* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+DI void dali_publish(dali_ms* p, dali_ms v) {
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+DI dali_ms dali_observe(const dali_ms* p) {
+    return __builtin_bit_cast(dali_ms, __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
 // Waits until this thread's earlier stores are acknowledged, then draws a ticket.
 DI unsigned int dali_take_ticket(unsigned int* counter) {
     __builtin_amdgcn_s_waitcnt(0);

@@ -29,7 +29,8 @@ enum class Kind {
     POOL2D,            // dali/array/op/conv.cpp:12-112 (name = reducer, depth = 1 for the average)
     POOL2D_BACKWARD,   // dali/array/op/conv.cpp:114-212 (args: y, dy, x)
     ONE_HOT,           // dali/array/op/one_hot.cpp:16-74
-    MATMUL             // dali/array/op/dot.cpp:18-47
+    MATMUL,            // dali/array/op/dot.cpp:18-47
+    SOFTMAX            // dali/array/op/softmax.cpp:5-8 as one node (axis = the normalised axis); written out when evaluated
 };
 
 struct Expr {

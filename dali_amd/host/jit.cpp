@@ -507,6 +507,8 @@ struct RowParams {
     bool ragged = false;     // rows not aligned to the vector: element-aligned vector accesses
     bool tail = false;       // ragged, and C is no multiple of VEC: the rest of a row is handled one element to a thread
     int EPT_L = 0;           // cached rows: the last EPT_L of the EPT vectors a thread holds live in LDS instead of registers
+    bool split = false;      // maps without a reduction over few long rows: every row is cut into S pieces, one workgroup each
+    int band = 0;            // maps with operands broadcast along the rows ([1, C]): a workgroup walks `band` rows and keeps those operands
 };
 
 int env_int(const char* name, int fallback) {
@@ -530,6 +532,10 @@ struct BodyEmitter {
     // quotient; 0 keeps the self-contained per-element form. `divisors` collects the divisor expressions.
     int div_mode = 0;
     std::vector<std::string>* divisors = nullptr;
+    // Band kernels (several rows per workgroup): a divisor that only depends on operands broadcast along the rows is
+    // evaluated once per column chunk into hv<k>[j] with its reciprocal hr<k>[j], ahead of the loop over the rows.
+    std::vector<int>* band_divisors = nullptr;
+    std::function<bool(int)> band_invariant;
     int divisor_index(const std::string& dv) {
         for (size_t k = 0; k < divisors->size(); ++k)
             if ((*divisors)[k] == dv) return (int)k;
@@ -580,6 +586,15 @@ struct BodyEmitter {
             case Kind::BROADCAST:
                 return value(n.args[0]);
             case Kind::ELEMENTWISE: {
+                if (band_divisors && n.name == "functor::eltdiv" && n.cls == Cls::FULL && n.args.size() == 2 && n.dtype == DTYPE_FLOAT &&
+                    P.nodes[n.args[1]].dtype == DTYPE_FLOAT && band_invariant(n.args[1])) {
+                    size_t k = 0;
+                    while (k < band_divisors->size() && (*band_divisors)[k] != n.args[1]) ++k;
+                    if (k == band_divisors->size()) band_divisors->push_back(n.args[1]);
+                    const std::string x = value(n.args[0]), ks = std::to_string(k);
+                    if (div_mode == 1) return "dali_div_fast(" + x + ", hv" + ks + "[j], hr" + ks + "[j])";
+                    return "(" + x + " / hv" + ks + "[j])";
+                }
                 if (n.name == "functor::eltdiv" && n.cls == Cls::FULL && n.args.size() == 2 && row_invariant(n.args[1])) {
                     // divisor constant along the row: reciprocal once, product + correction per element
                     const std::string x = value(n.args[0]), dv = value(n.args[1]);
@@ -806,19 +821,20 @@ void emit_row_prologue(std::ostringstream& ss, const Program& P, const IvLayout&
 
 // load of FULL leaf `i` for chunk `ch` into dst (dst is "x<i>[e]" or "x<i>")
 void emit_leaf_load(std::ostringstream& ss, const ArrayArg& a, int i, int VEC, const std::string& dst, const std::string& indent, bool nontemporal,
-                    bool ragged = false) {
+                    bool ragged = false, const std::string& pointer_prefix = "q") {
     std::string t = ctype(a.buf->dtype);
+    const std::string q = pointer_prefix + std::to_string(i);  // q<i>, or another name where a workgroup walks several rows
     if (VEC > 1 && ragged) {
-        ss << indent << "{ const dali_vec<" << t << ", " << VEC << "> tmp = " << (nontemporal ? "dali_loadu_nt<" : "dali_loadu<") << t << ", " << VEC << ">(q" << i
+        ss << indent << "{ const dali_vec<" << t << ", " << VEC << "> tmp = " << (nontemporal ? "dali_loadu_nt<" : "dali_loadu<") << t << ", " << VEC << ">(" << q
            << " + (long)ch * " << VEC << ");\n";
         ss << indent << "  _Pragma(\"unroll\") for (int j = 0; j < " << VEC << "; ++j) " << dst << "[j] = tmp.v[j]; }\n";
     } else if (VEC > 1) {
-        ss << indent << "{ dali_vec<" << t << ", " << VEC << "> tmp = " << (nontemporal ? "dali_load_nt<" : "dali_load<") << t << ", " << VEC << ">(q" << i
+        ss << indent << "{ dali_vec<" << t << ", " << VEC << "> tmp = " << (nontemporal ? "dali_load_nt<" : "dali_load<") << t << ", " << VEC << ">(" << q
            << " + (long)ch * " << VEC << ");\n";
         ss << indent << "  _Pragma(\"unroll\") for (int j = 0; j < " << VEC << "; ++j) " << dst << "[j] = tmp.v[j]; }\n";
     } else {
         std::string cs = a.strided ? " * cs" + std::to_string(i) : "";
-        ss << indent << dst << "[0] = q" << i << "[(long)ch" << cs << "];\n";
+        ss << indent << dst << "[0] = " << q << "[(long)ch" << cs << "];\n";
     }
 }
 
@@ -834,6 +850,24 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
     ss << "  constexpr int VEC = " << rp.VEC << ", TPR = " << rp.TPR << ", RPB = " << rp.RPB << ";\n";
     if (rp.cached) ss << "  constexpr int EPT = " << rp.EPT << ";\n";
     ss << "  const int tid = threadIdx.x;\n  const int tr = tid % TPR;\n";
+    if (rp.band > 1) {
+        // the shape entry is {strips, bands, R, C}: neighbouring workgroups take neighbouring strips of TPR vectors of the
+        // same band of rows, so that the device as a whole reads whole rows (all memory channels) at any moment
+        ss << "  constexpr int BAND = " << rp.band << ";\n";
+        ss << "  const unsigned int strips = A.iv[" << L.shape_pos[0] << "];\n";
+        ss << "  const long R = A.iv[" << L.shape_pos[0] + 2 << "], C = A.iv[" << L.shape_pos[0] + 3 << "];\n";
+        ss << "  long row = (long)(blockIdx.x / strips) * BAND;  // first row of this workgroup's band\n  constexpr bool row_ok = true; (void)row_ok;\n";
+        ss << "  const int CH = (int)(C / VEC); (void)CH;\n";
+        ss << "  const int ch = (int)(blockIdx.x % strips) * TPR + tr;\n";
+    } else if (rp.split) {
+        // the shape entry is {S, R, C}: workgroup b works on piece b % S of row b / S
+        ss << "  const int S = A.iv[" << L.shape_pos[0] << "];\n";
+        ss << "  const long R = A.iv[" << L.shape_pos[0] + 1 << "], C = A.iv[" << L.shape_pos[0] + 2 << "];\n";
+        ss << "  long row = blockIdx.x / (unsigned)S;\n  const int seg = (int)(blockIdx.x - (unsigned)row * (unsigned)S);\n";
+        ss << "  constexpr bool row_ok = true;\n  (void)R;\n";
+        ss << "  const int CH = (int)(C / VEC); (void)CH;\n";
+        ss << "  const int CHS = (CH + S - 1) / S, ch_begin = seg * CHS, ch_end = ch_begin + CHS < CH ? ch_begin + CHS : CH;\n";
+    } else {
     ss << "  const long R = A.iv[" << L.shape_pos[0] << "], C = A.iv[" << L.shape_pos[0] + 1 << "];\n";
     ss << "  long row = (long)blockIdx.x * RPB + tid / TPR;\n";
     if (rp.RPB == 1)
@@ -841,11 +875,12 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
     else
         ss << "  const bool row_ok = row < R;\n  if (!row_ok) row = R - 1;\n";
     ss << "  const int CH = (int)(C / VEC); (void)CH;\n";
+    }
     emit_row_prologue(ss, P, L);
     // ragged rows: the C % VEC elements past the last whole vector go one to a thread, through the same bodies
     // (slot EPT of the register cache, j = 0)
     const bool tail = rp.ragged && rp.tail;
-    if (tail) ss << "  const bool tail_on = tr < (int)(C - (long)CH * VEC);\n  const int tail_col = CH * VEC + tr;\n";
+    if (tail) ss << "  const bool tail_on = tr < (int)(C - (long)CH * VEC)" << (rp.split ? " && seg == S - 1" : "") << ";\n  const int tail_col = CH * VEC + tr;\n";
     // register-cached rows whose length fills every chunk need no chunk guard
     const std::string chunk_guard = rp.cached && rp.exact ? "    {\n" : "    if (ch < CH) {\n";
 
@@ -913,7 +948,10 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
         if (rp.cached) {
             o << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n" << chunk_guard;
         } else {
-            o << "  for (int ch = tr; ch < CH; ch += TPR) {\n    {\n";
+            if (rp.split)
+                o << "  for (int ch = ch_begin + tr; ch < ch_end; ch += TPR) {\n    {\n";
+            else
+                o << "  for (int ch = tr; ch < CH; ch += TPR) {\n    {\n";
             for (int i : full_leaves) {
                 o << "      " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n";
                 emit_leaf_load(o, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", rp.nt_loads, rp.ragged);
@@ -1079,6 +1117,90 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
     };
     if (!totals.empty()) emit_totals_publish();
 
+    if (rp.band > 1) {
+        // Operands that are broadcast along the rows (row stride 0) are loaded once per column chunk, what depends on them
+        // alone (the reciprocal of such a divisor) is computed there, and the workgroup then walks its band of rows.
+        auto is_colvec = [&](int i) { const ArrayArg& a = P.arrays[i]; return a.cls == Cls::FULL && !a.is_dest && a.strided && a.strides[0] == 0; };
+        std::function<bool(int)> invariant = [&](int id) -> bool {
+            const PNode& n = P.nodes[id];
+            switch (n.kind) {
+                case Kind::SCALAR: return true;
+                case Kind::BUFFER: return P.arrays[n.array].cls == Cls::SCAL || is_colvec(n.array);
+                case Kind::ELEMENTWISE: case Kind::BROADCAST: case Kind::EXPAND_DIMS:
+                    for (int a : n.args) if (!invariant(a)) return false;
+                    return true;
+                default: return false;
+            }
+        };
+        auto row_stride = [&](int i) { return P.arrays[i].strided ? "(long)A.iv[" + std::to_string(L.stride_pos[i]) + "]" : std::string("C"); };
+        std::vector<int> divs;
+        {
+            BodyEmitter probe(P, rp, true, rpn.n_phases, &rpn.first_body);
+            probe.band_divisors = &divs;
+            probe.band_invariant = invariant;
+            probe.div_mode = 1;
+            for (const Output& o : rpn.outputs) (void)probe.value(o.root);
+        }
+        ss << "  if (ch < CH) {\n";
+        for (int i : full_leaves)
+            if (is_colvec(i)) {
+                ss << "    " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n";
+                emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "    ", false, rp.ragged);
+            }
+        if (!divs.empty()) ss << "    bool hok = true;\n";
+        for (size_t k = 0; k < divs.size(); ++k) {
+            ss << "    float hv" << k << "[VEC], hr" << k << "[VEC];\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n      const int col = ch * VEC + j; (void)col;\n";
+            BodyEmitter hb(P, rp, true, rpn.n_phases, &rpn.first_body);
+            const std::string v = hb.value(divs[k]);
+            ss << hb.stmts.str() << "      hv" << k << "[j] = " << v << "; hr" << k << "[j] = 1.0f / hv" << k << "[j]; hok = hok && dali_div_ok(hv" << k << "[j]);\n    }\n";
+        }
+        auto emit_rows = [&](int div_mode) {
+            ss << "    for (int rr = 0; rr < BAND; ++rr) {\n      if (row + rr >= R) break;\n";
+            for (size_t i = 0; i < P.arrays.size(); ++i) {
+                const ArrayArg& a = P.arrays[i];
+                const std::string t = ctype(a.buf->dtype);
+                if (a.cls == Cls::FULL && !is_colvec((int)i))
+                    ss << "      " << (a.is_dest ? "" : "const ") << t << "* w" << i << " = q" << i << " + (long)rr * " << row_stride((int)i) << ";\n";
+                else if (a.cls == Cls::ROW && !a.is_dest)
+                    ss << "      const " << t << " rl" << i << " = ((const " << t << "*)A.p[" << i << "])[(row + rr)" << (a.strided ? " * (long)A.iv[" + std::to_string(L.stride_pos[i]) + "]" : std::string()) << "];\n";
+            }
+            for (int i : full_leaves)
+                if (!is_colvec(i)) {
+                    ss << "      " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n";
+                    emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", rp.nt_loads, rp.ragged, "w");
+                }
+            BodyEmitter be(P, rp, true, rpn.n_phases, &rpn.first_body);
+            std::vector<int> again;
+            be.band_divisors = &again;
+            be.band_invariant = invariant;
+            be.div_mode = div_mode;
+            std::ostringstream pre, body, post;
+            for (const Output& o : rpn.outputs) {
+                const ArrayArg& d = P.arrays[o.array];
+                const std::string t = ctype(d.buf->dtype), ov = "o" + std::to_string(o.array), w = "w" + std::to_string(o.array);
+                const std::string ldf = rp.ragged ? "dali_loadu<" : "dali_load<";
+                const std::string stf = rp.ragged ? (rp.nt_stores ? "dali_storeu_nt<" : "dali_storeu<") : (rp.nt_stores ? "dali_store_nt<" : "dali_store<");
+                pre << "      dali_vec<" << t << ", VEC> " << ov << ";\n";
+                if (o.op != OPERATOR_T_EQL) pre << "      " << ov << " = " << ldf << t << ", VEC>(" << w << " + (long)ch * VEC);\n";
+                post << "      " << stf << t << ", VEC>(" << w << " + (long)ch * VEC, " << ov << ");\n";
+                body << "        " << ov << ".v[j] = " << op_combine(o.op, ov + ".v[j]", "(" + t + ")(" + be.value(o.root) + ")") << ";\n";
+            }
+            ss << pre.str() << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        const int col = ch * VEC + j; (void)col;\n" << be.stmts.str() << body.str()
+               << "      }\n" << post.str() << "    }\n";
+        };
+        if (divs.empty()) {
+            emit_rows(0);
+        } else {
+            ss << "    if (__all(hok)) {\n";
+            emit_rows(1);
+            ss << "    } else {\n";
+            emit_rows(2);
+            ss << "    }\n";
+        }
+        ss << "  }\n}\n";
+        return ss.str();
+    }
+
     // output body: FULL destinations
     bool any_full = false;
     for (const Output& o : rpn.outputs) any_full = any_full || o.cls == Cls::FULL;
@@ -1135,7 +1257,7 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
     bool any_row = false;
     for (const Output& o : rpn.outputs) any_row = any_row || (o.cls != Cls::FULL && o.total_red < 0);
     if (any_row) {
-        ss << "  if (tr == 0 && row_ok) {\n";
+        ss << "  if (tr == 0 && row_ok" << (rp.split ? " && seg == 0" : "") << ") {\n";
         BodyEmitter be(P, rp, false, rpn.n_phases, &rpn.first_body);
         std::ostringstream body;
         for (const Output& o : rpn.outputs) {
@@ -1434,10 +1556,29 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
             n_full++;
             max_el = std::max(max_el, size_of_dtype(a.buf->dtype));
         }
+    int split_S = 1;
     if (nph == 0) {
         rp.cached = false;
         rp.TPR = (int)std::min<int64_t>(256, pow2ceil((int)std::max<int64_t>(1, CH)));
         rp.BT = 256;
+        // few long rows (one workgroup per row would leave most of the device idle): a row is cut into S pieces of at
+        // least 1024 vectors, as many as bring the grid to about 4096 workgroups
+        // operands broadcast along the rows ([1, C] against [R, C]: a bias, per-column statistics): a workgroup walks a band of
+        // rows chunk by chunk and keeps those operands, and the reciprocal of a divisor made of them, in registers
+        static const int band_env = env_int("DALI_HIP_ROW_BAND", 32);
+        bool colvec = false, band_ok = band_env > 1 && rp.VEC == 4 && !rp.tail && rp.TPR == 256 && n_totals == 0 && dom.R >= 2 * band_env;
+        for (const ArrayArg& a : P.arrays) {
+            if (a.cls == Cls::FULL && !a.is_dest && a.strided && a.strides[0] == 0 && !a.gather_source) colvec = true;
+            if (a.gather_source || a.row_index >= 0 || (a.cls == Cls::FULL && a.strided && a.strides[1] != 1)) band_ok = false;
+        }
+        for (const Output& o : rpn.outputs) band_ok = band_ok && o.cls == Cls::FULL;
+        for (const PNode& nd : P.nodes) band_ok = band_ok && nd.kind != Kind::GATHER_FROM_ROWS && nd.kind != Kind::GATHER;
+        if (colvec && band_ok) rp.band = band_env;
+        static const int split_env = env_int("DALI_HIP_ROW_SPLIT", 1);
+        if (split_env && rp.band == 0 && n_totals == 0 && rp.TPR == 256 && dom.R < 1024 && CH >= 4096) {
+            while (split_S * 2 * dom.R <= 4096 && CH / (split_S * 2) >= 1024) split_S *= 2;
+            rp.split = split_S > 1;
+        }
     } else {
         // vectors per thread: latency-bound problems (everything in flight at once, one generation
         // of waves) want more threads per row, streaming-size problems more work per thread
@@ -1537,7 +1678,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
     rp.nt_loads = nt_l >= 0 ? nt_l != 0 : dom.R * dom.C * (int64_t)max_el >= ((int64_t)64 << 20);
     rp.nt_stores = nt_s >= 0 ? nt_s != 0 : true;
     params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached << "," << rp.waves_per_eu << ","
-           << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail << "," << rp.EPT_L;
+           << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail << "," << rp.EPT_L << (rp.split ? "S" : "") << (rp.band > 1 ? "B" + std::to_string(rp.band) : std::string());
     if (n_totals) {
         // one 8-byte slot per workgroup and total in the workspace's 32 MiB of partial results
         const int64_t blocks = (dom.R + rp.RPB - 1) / rp.RPB;
@@ -1548,7 +1689,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
     std::string sig = signature(P, rpn.outputs);
     uint64_t h = kernel_hash("row", sig, params.str());
     std::shared_ptr<KernelSpec>& K = specs_cache[h];
-    std::vector<int> shape_ndims = {2};
+    std::vector<int> shape_ndims = {rp.band > 1 ? 4 : (rp.split ? 3 : 2)};
     IvLayout L = layout_iv(P, shape_ndims);
     if (!K) {
         K = std::make_shared<KernelSpec>();
@@ -1559,11 +1700,13 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
         K->plan.block_threads = rp.BT;
         K->plan.grid_kind = DALI_HIP_GRID_ROWS;
         K->plan.work_begin = L.shape_pos[0];
-        K->plan.work_count = 1;
+        K->plan.work_count = rp.split || rp.band > 1 ? 2 : 1;  // split: the grid covers S * R; bands: strips * bands
         K->plan.work_per_block = rp.RPB;
         K->plan.max_blocks = 0;
     }
     std::vector<std::vector<int>> shapes = {{(int)dom.R, (int)dom.C}};
+    if (rp.split) shapes[0].insert(shapes[0].begin(), split_S);
+    if (rp.band > 1) shapes[0] = {(int)((CH + rp.TPR - 1) / rp.TPR), (int)((dom.R + rp.band - 1) / rp.band), (int)dom.R, (int)dom.C};
     load_and_launch(*K, [&]() { return gen_row_kernel(rpn, L, K->name); }, P, shapes);
     return true;
 }
@@ -2024,7 +2167,11 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     const std::string ld = UNALIGNED ? (NT ? "dali_loadu_nt<" : "dali_loadu<") : (NT ? "dali_load_nt<" : "dali_load<");
     const PNode& red = P.nodes[red_id];
     const bool ARG = red.kind == Kind::ARG_AXIS_REDUCE;  // carries (value, row index); ties keep the lower index
-    std::string t = ctype(P.nodes[red.args[0]].dtype);
+    // softmax statistics: the accumulator is a (maximum, sum of exponentials) pair fed with plain values; the destination
+    // holds the K maxima followed by the K sums
+    const bool PAIR = red.name == "reducers::maxsumexp";
+    std::string t = PAIR ? std::string("dali_ms") : ctype(P.nodes[red.args[0]].dtype);
+    const std::string feed = PAIR ? red.name + "::feed(" : red.name + "::step<" + t + ">(";
     std::string dt = ctype(P.arrays[dest_array].buf->dtype);
     const std::string Rd = red.name;
     // fold candidate (cv, ci) into (av, ai)
@@ -2107,6 +2254,7 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
         ss << "      _Pragma(\"unroll\") for (int u = 0; u < UNR; ++u) { dali_vec<" << ty << ", VEC> tmp = " << ld << ty << ", VEC>(q" << i
            << " + (x + u * XS) * ld" << i << "); _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) x" << i << "s[u][j] = tmp.v[j]; }\n";
     }
+    if (PAIR) ss << "      float vv[VEC][UNR];\n";
     ss << "      _Pragma(\"unroll\") for (int u = 0; u < UNR; ++u) {\n";
     for (int i : full_leaves) ss << "        const " << ctype(P.arrays[i].buf->dtype) << "* x" << i << " = x" << i << "s[u];\n";
     ss << "        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n          const int col = 0; (void)col;\n";
@@ -2118,7 +2266,11 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
             // a thread meets its rows in increasing order: a strictly better value is the first index of its kind
             ss << be.stmts.str() << "          { const " << t << " cv = " << v << "; if (" << Rd << "::better<" << t << ">(cv, acc[j])) { acc[j] = cv; acci[j] = (int)(x + u * XS); } }\n        }\n      }\n";
         else
-            ss << be.stmts.str() << "          acc[j] = " << red.name << "::step<" << t << ">(acc[j], " << v << ");\n        }\n      }\n";
+            if (PAIR)
+                ss << be.stmts.str() << "          vv[j][u] = " << v << ";\n        }\n      }\n      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[j] = "
+                   << red.name << "::feed_n<UNR>(acc[j], vv[j]);\n";
+            else
+            ss << be.stmts.str() << "          acc[j] = " << feed << "acc[j], " << v << ");\n        }\n      }\n";
     }
     if (IL == 2)
         ss << "    }\n    for (long x = n_chunks * (UNR * NWAVE) + (long)blockIdx.y * NWAVE + wave; x < x_end; x += (long)gridDim.y * NWAVE) {\n";
@@ -2137,7 +2289,7 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
         if (ARG)
             ss << be.stmts.str() << "        { const " << t << " cv = " << v << "; if (" << Rd << "::better<" << t << ">(cv, acc[j])) { acc[j] = cv; acci[j] = (int)x; } }\n      }\n";
         else
-            ss << be.stmts.str() << "        acc[j] = " << red.name << "::step<" << t << ">(acc[j], " << v << ");\n      }\n";
+            ss << be.stmts.str() << "        acc[j] = " << feed << "acc[j], " << v << ");\n      }\n";
     }
     ss << "    }\n  }\n";
     // fold the row groups of the block in group order
@@ -2158,6 +2310,11 @@ std::string gen_col_kernel(const Program& P, int red_id, int dest_array, OPERATO
     };
     emit_group_fold("  ");
     auto emit_store = [&](const std::string& indent) {
+        if (PAIR) {
+            ss << indent << "_Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) if (ks + j >= k0 && ks + j < K) { " << dt << "* dp = q" << dest_array << " + (ks + j) * ds"
+               << dest_array << "; dp[0] = acc[j].m; dp[K * ds" << dest_array << "] = acc[j].l; }\n";
+            return;
+        }
         ss << indent << "_Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) if (ks + j >= k0 && ks + j < K) { " << dt << "* dp = q" << dest_array << " + (ks + j) * ds" << dest_array
            << "; *dp = " << op_combine(op, "(*dp)", std::string("(") + dt + ")" + (ARG ? "acci[j]" : "acc[j]")) << "; }\n";
     };
@@ -2219,12 +2376,15 @@ bool try_col(const DestSpec& spec) {
     int64_t k_run = 1;
     for (int d = split; d < nk; ++d) k_run *= arg_shape[d];
     const bool BATCHED = k_run != K;
-    if (numel_of(spec.dest.shape()) != K) return false;
+    const bool pair = re->name == "reducers::maxsumexp";  // K maxima followed by K sums of exponentials, float only
+    if (pair && (is_arg || spec.op != OPERATOR_T_EQL || arg.dtype() != DTYPE_FLOAT || spec.dest.dtype() != DTYPE_FLOAT || !spec.dest.contiguous_memory())) return false;
+    if (numel_of(spec.dest.shape()) != (pair ? 2 * K : K)) return false;
     Domain dom;
     dom.R = K;  // ROW-class destination has K entries
     dom.C = X;
     Program P;
-    int dest_array = add_array(P, spec.dest.expression(), Cls::ROW, false, dom, true);
+    // (the pair form presents the first half of its destination, the maxima; the kernel stores the sums K entries further on)
+    int dest_array = add_array(P, pair ? spec.dest.reshape({2, (int)K})[0].expression() : spec.dest.expression(), Cls::ROW, false, dom, true);
     if (dest_array < 0) return false;
     int red_id = add_node(P, root);
     // classify the argument tree: [K, X] buffers are FULL with the kept stride in strides[0]
@@ -2302,7 +2462,7 @@ bool try_col(const DestSpec& spec) {
     // workgroups per CU are better (sum(exp(x)) along the leading axis of [8192,8192]: 61 -> 45 us; bare sum 40.6 -> 42.1)
     // (small problems keep one: [4096,1024] 13 us against 20 us with the extra partial results to fold)
     const bool streaming = K * X * (int64_t)size_of_dtype(arg.dtype()) >= ((int64_t)64 << 20);
-    const int max_blocks = blocks_env > 0 ? blocks_env : (streaming && contains_expensive(P, P.nodes[red_id].args[0]) ? 512 : 256);
+    const int max_blocks = blocks_env > 0 ? blocks_env : (streaming && (pair || contains_expensive(P, P.nodes[red_id].args[0])) ? 512 : 256);
     const int UNR = unr_env;
     // four row groups of one wave each: a wave reads 1 KiB pieces of memory rows, a block owns a 256-column strip.
     // Narrow strips and few y-blocks measured best (8192x8192: 53 us with 1024-column strips x 32 y-blocks,
@@ -2341,7 +2501,7 @@ bool try_col(const DestSpec& spec) {
         Kp->plan.work2_per_block = rows_env > 0 ? rows_env : UNR * RG;  // fewest reduced rows per y-block
         Kp->plan.max_blocks2 = maxy_env;
         Kp->plan.max_blocks = max_blocks;  // the y split fills what the column strips leave
-        Kp->plan.ws_elsize = size_of_dtype(arg.dtype()) + (is_arg ? 4 : 0);  // a partial is a value, plus its index
+        Kp->plan.ws_elsize = pair ? 8 : size_of_dtype(arg.dtype()) + (is_arg ? 4 : 0);  // a partial is a value, plus its index
     }
     std::vector<std::vector<int>> shapes = {{(int)K, (int)X}};
     if (BATCHED) {
@@ -2685,6 +2845,69 @@ Array run_col2im(const Expr& e, const Array& patches);
 Array run_pool2d(const Expr& e, const Array& x);
 Array run_pool2d_backward(const Expr& e, const Array& y, const Array& dy, const Array& x);
 
+// op::softmax arrives as one node and is written out here. The general form is the reference's expression
+// (dali/array/op/softmax.cpp:5-8), which the row kernel fuses into one pass. Two shapes starve that kernel and get their
+// statistics (maximum and sum of exponentials per slice) from a pass of their own; what is returned is then the lazy map
+// exp(x - maximum) / sum over evaluated buffers, which still fuses with whatever consumes the softmax:
+//  - few long rows (one workgroup per row leaves most of the device idle): the rows are read as S times as many shorter
+//    ones, each yields its own (maximum, sum), and a small second kernel combines the S pairs of a row;
+//  - an axis other than the last (the slices run against memory): the column kernel carries (maximum, sum) pairs, so the
+//    data is read once for both instead of once for the maxima and once more for the sums.
+bool try_col(const DestSpec& spec);
+Array expand_softmax(Array x, int axis) {
+    static const bool staged_off = env_int("DALI_HIP_SOFTMAX_STAGED", 1) == 0;
+    const std::vector<int> shape = x.shape();
+    const int nd = (int)shape.size();
+    const int64_t n = numel_of(shape), Cx = shape[axis];
+    std::vector<int> keep = shape;
+    keep[axis] = 1;
+    if (!staged_off && x.dtype() == DTYPE_FLOAT && n > 0 && Cx > 1) {
+        if (axis == nd - 1) {
+            const int64_t rows = n / Cx;
+            int S = 1;
+            while (rows < 256 && Cx >= 65536 && S * 2 * rows <= 2048 && Cx % (S * 2 * 4) == 0 && Cx / (S * 2) >= 8192) S *= 2;
+            if (S >= 4) {
+                if (!x.is_buffer()) x = materialize(x);
+                if (!x.contiguous_memory()) x = x.ascontiguousarray();
+                Array xr = x.reshape({(int)(rows * S), (int)(Cx / S)});
+                Array mseg = op::max(xr, {-1}, true);
+                Array lseg = op::sum(op::exp(op::subtract(xr, mseg)), {-1}, true);
+                evaluate({mseg, lseg});
+                Array m2 = mseg.reshape({(int)rows, S}), l2 = lseg.reshape({(int)rows, S});
+                Array M = op::max(m2, {-1}, true);
+                Array L = op::sum(op::eltmul(l2, op::exp(op::subtract(m2, M))), {-1}, true);
+                evaluate({M, L});
+                return op::eltdiv(op::exp(op::subtract(x, M.reshape(keep))), L.reshape(keep));
+            }
+        } else if (n >= (1 << 16)) {
+            int64_t inner = 1;
+            for (int d = axis + 1; d < nd; ++d) inner *= shape[d];
+            if (inner >= 16) {
+                if (!x.is_buffer()) x = materialize(x);
+                if (!x.contiguous_memory()) x = x.ascontiguousarray();
+                std::vector<int> order, kept_shape;
+                for (int d = 0; d < nd; ++d)
+                    if (d != axis) { order.push_back(d); kept_shape.push_back(shape[d]); }
+                order.push_back(axis);
+                auto node = std::make_shared<Expr>();
+                node->kind = Kind::AXIS_REDUCE;
+                node->name = "reducers::maxsumexp";
+                node->args = {x.transpose(order)};
+                node->shape = kept_shape;
+                node->dtype = DTYPE_FLOAT;
+                std::vector<int> stats_shape = kept_shape;
+                stats_shape.insert(stats_shape.begin(), 2);
+                Array stats(stats_shape, DTYPE_FLOAT);
+                if (try_col({stats, OPERATOR_T_EQL, Array(node)})) {
+                    jit_stats().evals++;
+                    return op::eltdiv(op::exp(op::subtract(x, stats[0].reshape(keep))), stats[1].reshape(keep));
+                }
+            }
+        }
+    }
+    return op::softmax_naive(x, axis);
+}
+
 Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root) {
     auto e = a.expression();
     auto it = memo.find(e.get());
@@ -2727,6 +2950,9 @@ Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root) {
             if (changed) out = rebuild(e, args);
             break;
         }
+        case Kind::SOFTMAX:
+            out = clean(expand_softmax(clean(e->args[0], memo, false), e->axis), memo, is_root);
+            break;
         case Kind::AXIS_SCAN: {
             // not chainable (dali/array/op/scan.cpp:38-40): the scan is its own kernel, consumers read its buffer
             Array arg = clean(e->args[0], memo, false);

@@ -141,6 +141,13 @@ def softmax(x, axis=-1):
     return _wrap(front.dali_fe_softmax(x._h, axis), "softmax")
 
 
+def softmax_naive(x, axis=-1):
+    """exp(x - max) / sum(exp(x - max)) written out (what ``softmax`` becomes when it is evaluated, except for shapes that
+    get their statistics from a pass of their own)."""
+    x = as_array(x)
+    return _wrap(front.dali_fe_softmax_naive(x._h, axis), "softmax_naive")
+
+
 def gather(source, indices):
     """source[indices[...], ...]; assigning to the lazy result scatters into ``source``."""
     source, indices = as_array(source), as_array(indices)

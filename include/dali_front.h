@@ -64,6 +64,8 @@ dali_array_t dali_fe_arg_axis_reduce(const char* reducer_name, dali_array_t a, i
 dali_array_t dali_fe_mean_all(dali_array_t a);
 dali_array_t dali_fe_mean_axes(dali_array_t a, const int* axes, int naxes, int keepdims);
 dali_array_t dali_fe_softmax(dali_array_t a, int axis);
+/* the written-out expression exp(a - max) / sum(exp(a - max)) of dali/array/op/softmax.cpp:5-8, which dali_fe_softmax turns into when it is evaluated */
+dali_array_t dali_fe_softmax_naive(dali_array_t a, int axis);
 /* op::softmax_temperature (dali/array/op/softmax.cpp:10-13): the reference ignores the temperature, and so does this */
 dali_array_t dali_fe_softmax_temperature(dali_array_t a, dali_array_t temperature, int axis);
 /* op::ceil (dali/array/op/elementwise_operation.cpp:155-160): int32 result, int32 operands pass through */

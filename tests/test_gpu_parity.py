@@ -734,6 +734,48 @@ def test_rows_cached_partly_in_lds(gpu, D, O, rng, cols):
     assert np.array_equal((arr(D, xi) - op.min(arr(D, xi), [1], True)).numpy(), xi - xi.min(1, keepdims=True))
 
 
+@pytest.mark.parametrize("shape,axis", [((8, 262144), -1), ((3, 524288), 1), ((2, 3, 131072), 2), ((4096, 1000), 0), ((513, 257), 0),
+                                        ((16, 300, 64), 1), ((16, 300, 64), 0), ((70000, 16), 0), ((64, 1000), 0)])
+def test_softmax_over_few_long_rows_and_against_the_layout(gpu, D, O, rng, shape, axis):
+    """op::softmax takes any axis (softmax.cpp:5-8). Few very long rows are cut into pieces whose (maximum, sum of
+    exponentials) pairs are combined by a second small kernel; along an axis other than the last the column kernel
+    carries such pairs through one pass over the data. Both must agree with the written-out expression."""
+    op = D.op
+    x = (rng.randn(*shape) * 3).astype(np.float32)
+    x[tuple(rng.randint(0, n) for n in shape)] = 40.0  # one slice with a dominant entry
+    X = arr(D, x)
+    k0 = D.jit_stats()["kernels"]
+    s = op.softmax(X, axis).numpy()
+    launched = D.jit_stats()["kernels"] - k0
+    ax = axis % len(shape)
+    if ax == len(shape) - 1:
+        assert launched == 3 and D.last_kernel_kinds().endswith("map2d")   # piece statistics, their combination, the quotient
+    elif x.size >= 65536:
+        assert launched == 2                                        # (maximum, sum) pairs in one column pass, the quotient
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(ax, keepdims=True))
+    close(s, e / e.sum(ax, keepdims=True), rtol=1e-5, atol=1e-12)   # fp64 truth
+    moved = np.ascontiguousarray(np.moveaxis(x, ax, -1))
+    close(np.moveaxis(s, ax, -1), O.softmax(moved), rtol=seq_sum_rtol(shape[ax]), atol=1e-12)
+    close(s.astype(np.float64).sum(ax), 1.0, rtol=0, atol=2e-6)
+    naive = op.softmax_naive(arr(D, x), axis).numpy() if hasattr(op, "softmax_naive") else None
+    if naive is not None:
+        close(s, naive, rtol=2e-6, atol=1e-12)
+    # still lazy behind the statistics: a consumer fuses with the quotient
+    t = rng.randint(0, shape[ax], 1)[0]
+    k0 = D.jit_stats()["kernels"]
+    shifted = (op.softmax(X, axis) * 2.0 - 1.0).numpy()
+    assert D.jit_stats()["kernels"] - k0 == launched
+    close(shifted, 2.0 * s.astype(np.float64) - 1.0, rtol=1e-6, atol=1e-6)
+    # infinities: a masked entry (-inf) has probability zero
+    y = x.copy()
+    idx = tuple(rng.randint(0, n) for n in shape)
+    y[idx] = -np.inf
+    sy = op.softmax(arr(D, y), axis).numpy()
+    assert sy[idx] == 0.0 and np.isfinite(sy).all()
+    close(sy.astype(np.float64).sum(ax), 1.0, rtol=0, atol=2e-6)
+
+
 def test_fused_softmax_equals_staged(gpu, D, rng):
     """JITCachedReduction.fused_softmax (tests.cpp:1622-1664): U(-20,20) [2,5], atol 1e-6."""
     op = D.op
