@@ -310,6 +310,11 @@ void dali_fe_record_free(void* recording) {
     delete rec;
 }
 
+int dali_fe_set_dry_run(int on, int compile) {
+    dali::set_dry_run(on != 0);
+    dali::set_dry_compile(on != 0 && compile != 0);
+    return 0;
+}
 int dali_fe_generate_only(dali_array_t* roots, int n, int compile) {
     dali::set_dry_compile(compile != 0);
     try {

@@ -168,6 +168,11 @@ int dali_fe_record_make_graph(void* recording);
 int dali_fe_replay(void* recording, int times);
 void dali_fe_record_free(void* recording);
 
+/* While on, evaluations and assignments plan and generate their kernels (and compile them with hipRTC when `compile` is set)
+ * but launch nothing and touch no device: the way to check code generation for statements that are not plain roots, such as
+ * an assignment through a gather. dali_fe_last_source holds the generated text. */
+int dali_fe_set_dry_run(int on, int compile);
+
 /* plan + generate (and optionally hipRTC-compile for gfx950) without a device;
  * returns the number of kernels, -1 on error */
 int dali_fe_generate_only(dali_array_t* roots, int n, int compile);
