@@ -230,9 +230,23 @@ void* dali_hip_stream(void) {
     return (void*)rt().stream;
 }
 
+// true while the library stream records into a graph: what would be baked into the graph and then reused or released
+// behind its back (bank blocks, driver allocations) or is known to misbehave in a replayed graph (memset nodes) is refused
+static bool stream_is_capturing() {
+    Runtime& r = rt();
+    if (!r.ready) return false;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(r.stream, &cs) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return cs != hipStreamCaptureStatusNone;
+}
+
 int dali_hip_malloc(void** ptr, size_t bytes) {
     if (ensure_init()) return DALI_HIP_ERROR;
     *ptr = nullptr;
+    if (stream_is_capturing()) return fail("dali_hip_malloc: not allowed while the library stream is being captured");
     if (bytes == 0) bytes = 4;
     HIP_TRY(hipMalloc(ptr, bytes));
     return DALI_HIP_OK;
@@ -262,6 +276,9 @@ constexpr size_t kSlabBlockMax = (size_t)2 << 20;
 
 int dali_hip_bank_allocate(void** ptr, size_t bytes) {
     if (ensure_init()) return DALI_HIP_ERROR;
+    if (stream_is_capturing())
+        return fail("dali_hip_bank_allocate: not allowed while the library stream is being captured (the block's address would be part of the "
+                    "graph while the bank hands the block to others)");
     Runtime& r = rt();
     bytes = bank_class(bytes);
     {
@@ -354,6 +371,7 @@ int dali_hip_bank_stats(size_t* parked_bytes, size_t* live_bytes) {
 int dali_hip_memset_async(void* ptr, int value, size_t bytes) {
     if (ensure_init()) return DALI_HIP_ERROR;
     if (bytes == 0) return DALI_HIP_OK;
+    if (stream_is_capturing()) return fail("dali_hip_memset_async: not allowed while the library stream is being captured (fill with a kernel instead)");
     HIP_TRY(hipMemsetAsync(ptr, value, bytes, rt().stream));
     return DALI_HIP_OK;
 }

@@ -15,11 +15,6 @@
 
 namespace dali_hip {
 
-__global__ __launch_bounds__(256) void iota_kernel(int32_t* out, long n) {
-    const long i = (long)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) out[i] = (int32_t)i;
-}
-
 // A few thousand keys: counting ranks beats any multi-pass sort. The final position of key i is the number of
 // (key, position) pairs that order before it. A workgroup counts, for 256 keys, the smaller pairs within one
 // segment of the input (staged in LDS, read as wave-wide broadcasts) and publishes the counts; the workgroup that
@@ -87,6 +82,108 @@ __global__ __launch_bounds__(256) void rank_sort_kernel(const int32_t* keys, int
     if (threadIdx.x == 0) __hip_atomic_store(tickets + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+
+// ---------------------------------------------------------------- more than 16384 keys: least-significant-digit radix sort
+// Eight bits per pass over (key, position) pairs. A workgroup owns a tile of 2048 consecutive pairs. Pass = three
+// launches: (1) a histogram of the tile's digits, stored digit-major [256][tiles]; (2) an exclusive scan over that table,
+// which turns every entry into the first output slot of (digit, tile); (3) the move: a pair goes to that slot plus its
+// rank among the tile's pairs with the same digit that come before it. The rank is exact, not "whoever gets there
+// first", so every pass is stable and equal keys end up in input order: a thread holds eight pairs (one per round of 256),
+// a wave finds the lanes with its digit from eight ballots (one per bit), the lowest such lane records how many there
+// are per (round, wave, digit), and a scan over the 32 (round, wave) slots of every digit gives each group its offset.
+constexpr int kRadixTile = 2048;
+
+__device__ __forceinline__ unsigned int radix_digit(int32_t key, int shift, unsigned int flip) { return (((unsigned int)key ^ flip) >> shift) & 255u; }
+
+__global__ __launch_bounds__(256) void radix_hist_kernel(const int32_t* keys, int n, int shift, unsigned int flip, unsigned int* hist, int tiles) {
+    __shared__ unsigned int h[256];
+    h[threadIdx.x] = 0u;
+    __syncthreads();
+    const long base = (long)blockIdx.x * kRadixTile;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const long i = base + r * 256 + threadIdx.x;
+        if (i < n) atomicAdd(&h[radix_digit(keys[i], shift, flip)], 1u);
+    }
+    __syncthreads();
+    hist[(long)threadIdx.x * tiles + blockIdx.x] = h[threadIdx.x];
+}
+
+// exclusive scan of `total` counters in place, by one workgroup: a thread sums a contiguous share, the shares are scanned
+// through the waves and LDS, and the thread walks its share again
+__global__ __launch_bounds__(1024) void radix_scan_kernel(unsigned int* hist, long total) {
+    __shared__ unsigned int wave_sum[16];
+    const long per = (total + 1023) / 1024, begin = (long)threadIdx.x * per, end = begin + per < total ? begin + per : total;
+    unsigned int mine = 0;
+    for (long i = begin; i < end; ++i) mine += hist[i];
+    unsigned int incl = mine;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const unsigned int o = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += o;
+    }
+    if (lane == 63) wave_sum[wave] = incl;
+    __syncthreads();
+    unsigned int before = 0;
+    for (int w = 0; w < wave; ++w) before += wave_sum[w];
+    unsigned int run = before + incl - mine;
+    for (long i = begin; i < end; ++i) {
+        const unsigned int c = hist[i];
+        hist[i] = run;
+        run += c;
+    }
+}
+
+__global__ __launch_bounds__(256) void radix_move_kernel(const int32_t* keys_in, const int32_t* pos_in, int n, int shift, unsigned int flip, const unsigned int* hist,
+                                                         int tiles, int32_t* keys_out, int32_t* pos_out) {
+    __shared__ unsigned short cnt[32][256];
+    __shared__ unsigned int first_slot[256];
+    for (int t = threadIdx.x; t < 32 * 256; t += 256) (&cnt[0][0])[t] = 0;
+    first_slot[threadIdx.x] = hist[(long)threadIdx.x * tiles + blockIdx.x];
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    const long base = (long)blockIdx.x * kRadixTile;
+    int32_t key[8], pos[8];
+    unsigned int digit[8], rank[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const long i = base + r * 256 + threadIdx.x;
+        const bool valid = i < n;
+        key[r] = valid ? keys_in[i] : 0;
+        pos[r] = valid ? (pos_in ? pos_in[i] : (int32_t)i) : 0;
+        digit[r] = radix_digit(key[r], shift, flip);
+        unsigned long long same = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const unsigned long long m = __ballot((digit[r] >> b) & 1u);
+            same &= ((digit[r] >> b) & 1u) ? m : ~m;
+        }
+        rank[r] = (unsigned int)__popcll(same & below);
+        if (valid && rank[r] == 0) cnt[r * 4 + wave][digit[r]] = (unsigned short)__popcll(same);
+    }
+    __syncthreads();
+    {
+        unsigned int run = 0;
+#pragma unroll 8
+        for (int s = 0; s < 32; ++s) {
+            const unsigned int c = cnt[s][threadIdx.x];
+            cnt[s][threadIdx.x] = (unsigned short)run;
+            run += c;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const long i = base + r * 256 + threadIdx.x;
+        if (i < n) {
+            const unsigned int dst = first_slot[digit[r]] + cnt[r * 4 + wave][digit[r]] + rank[r];
+            keys_out[dst] = key[r];
+            pos_out[dst] = pos[r];
+        }
+    }
+}
 
 // ---------------------------------------------------------------- ordering along rows (top_k / bottom_k / argsort)
 // Keys of one dense [rows, cols] matrix are copied into a sort buffer beside their column numbers. -0.0 becomes +0.0
@@ -498,24 +595,35 @@ extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_
         (n + 255) / 256 <= kWorkspaceCounters)
         return launch_rank_sort(keys, (int)n, key_limit, (unsigned int*)workspace(), (int32_t*)(workspace() + kWorkspaceCounterBytes), sorted_keys,
                                 perm, st);
-    void* positions = nullptr;
-    if (dali_hip_bank_allocate(&positions, (size_t)n * sizeof(int32_t))) return DALI_HIP_ERROR;
-    hipLaunchKernelGGL(iota_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (int32_t*)positions, (long)n);
-    size_t temp_bytes = 0;
-    hipError_t e = hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, keys, sorted_keys, (const int32_t*)positions, perm, (int)n, 0, end_bit, st);
+    // radix passes over the bits that can differ; arbitrary keys are ordered as signed numbers (the sign bit is flipped in
+    // the digit). The pairs bounce between the caller's arrays and one temporary block so that the last pass lands in the
+    // caller's.
+    const int passes = (end_bit + 7) / 8, tiles = (int)((n + kRadixTile - 1) / kRadixTile);
+    const unsigned int flip = key_limit > 0 ? 0u : 0x80000000u;
+    const size_t temp_bytes = ((size_t)2 * (size_t)n + (size_t)256 * (size_t)tiles) * sizeof(int32_t);
     void* temp = nullptr;
-    int status = DALI_HIP_OK;
-    if (e != hipSuccess) {
-        status = fail("radix sort sizing failed: %s", hipGetErrorString(e));
-    } else if (dali_hip_bank_allocate(&temp, temp_bytes ? temp_bytes : 4)) {
-        status = DALI_HIP_ERROR;
-    } else {
-        e = hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, keys, sorted_keys, (const int32_t*)positions, perm, (int)n, 0, end_bit, st);
-        if (e != hipSuccess) status = fail("radix sort failed: %s", hipGetErrorString(e));
+    if (dali_hip_bank_allocate(&temp, temp_bytes)) return DALI_HIP_ERROR;
+    int32_t* tkeys = (int32_t*)temp;
+    int32_t* tpos = tkeys + n;
+    unsigned int* hist = (unsigned int*)(tpos + n);
+    const int32_t* src_keys = keys;
+    const int32_t* src_pos = nullptr;  // first pass: a pair's position is its index
+    for (int i = 0; i < passes; ++i) {
+        const bool to_caller = (passes - 1 - i) % 2 == 0;
+        int32_t* dst_keys = to_caller ? sorted_keys : tkeys;
+        int32_t* dst_pos = to_caller ? perm : tpos;
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(256), 0, st, src_keys, (int)n, 8 * i, flip, hist, tiles);
+        hipLaunchKernelGGL(radix_scan_kernel, dim3(1), dim3(1024), 0, st, hist, (long)256 * tiles);
+        hipLaunchKernelGGL(radix_move_kernel, dim3(tiles), dim3(256), 0, st, src_keys, src_pos, (int)n, 8 * i, flip, (const unsigned int*)hist, tiles, dst_keys,
+                           dst_pos);
+        src_keys = dst_keys;
+        src_pos = dst_pos;
     }
-    // the blocks go back to the bank at once: the next user of them is ordered behind the sort on the stream
-    if (temp) dali_hip_bank_deposit(temp, temp_bytes ? temp_bytes : 4);
-    dali_hip_bank_deposit(positions, (size_t)n * sizeof(int32_t));
+    int status = DALI_HIP_OK;
+    hipError_t le = hipGetLastError();
+    if (le != hipSuccess) status = fail("radix sort launch failed: %s", hipGetErrorString(le));
+    // the block goes back to the bank at once: the next user of it is ordered behind the sort on the stream
+    dali_hip_bank_deposit(temp, temp_bytes);
     return status;
 }
 

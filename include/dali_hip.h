@@ -76,6 +76,7 @@ int dali_hip_free(void* ptr);
  * requests share blocks, and blocks of up to 2 MiB are carved out of 64 MiB slabs instead of costing a driver
  * allocation each. dali_hip_bank_clear returns the parked driver allocations; slab blocks stay parked.
  * Same-stream ordering makes immediate reuse safe. */
+/* (dali_hip_malloc, dali_hip_bank_allocate and dali_hip_memset_async fail while the library stream is being captured) */
 int dali_hip_bank_allocate(void** ptr, size_t bytes);
 int dali_hip_bank_deposit(void* ptr, size_t bytes);
 int dali_hip_bank_clear(void);
@@ -251,8 +252,9 @@ int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx
  * the generated scatter kernel instead walks each destination row's contributions in input order,
  * the order of the reference's sequential CPU loop, so the result does not depend on scheduling.
  * Up to 16384 keys are ordered by one kernel that allocates nothing (it may be captured); longer inputs take a
- * radix sort whose temporary blocks come from the bank. With key_limit > 0, keys outside the promised range come
- * out in an unspecified order, but perm is a permutation for any input.
+ * least-significant-digit radix sort (eight bits per pass, three launches per pass) whose temporary block comes from
+ * the bank, so they fail during a capture. With key_limit > 0, keys outside the promised range come out in an
+ * unspecified order, but perm is a permutation for any input.
  */
 int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_limit, int32_t* sorted_keys, int32_t* perm);
 
@@ -274,8 +276,9 @@ int dali_hip_argsort_i32_noalloc(const int32_t* keys, int64_t n, int32_t key_lim
  * is a TODO there, :198). dtype: 0 = float, 1 = double, 2 = int32. largest != 0 orders by descending value (top_k),
  * else ascending (bottom_k, argsort). Equal values come out in ascending column order, or in descending column order
  * with ties_by_descending_column != 0 (what the reference's heap gives bottom_k for k < cols, top_k.cpp:118-123).
- * -0.0 and +0.0 are equal; the place of NaNs is unspecified. One segmented radix sort on the library stream; its
- * buffers (four times the input) come from the bank.
+ * -0.0 and +0.0 are equal; the place of NaNs is unspecified. Rows of at least 1024 entries with k <= 64 take a one-pass
+ * selection kernel that allocates nothing; everything else one segmented radix sort on the library stream whose buffers
+ * (four times the input) come from the bank, so that form fails during a capture.
  */
 int dali_hip_topk_rows(const void* x, int dtype, int64_t rows, int32_t cols, int32_t k, int largest, int ties_by_descending_column,
                        int32_t* out);

@@ -1318,7 +1318,7 @@ def test_autoreduce_assign_reference_cases(gpu, D, rng):
         t <<= arr(D, np.ones((3, 4), np.int32))
 
 
-@pytest.mark.parametrize("n", [1, 7, 1000, 1024, 1025, 5000, 8192, 8193, 100000])
+@pytest.mark.parametrize("n", [1, 7, 1000, 1024, 1025, 5000, 8192, 8193, 16385, 100000, 1000003])
 def test_cabi_argsort_is_stable(gpu, rng, n):
     hip = gpu
     keys = rng.randint(-50, 50, n).astype(np.int32)
@@ -1352,6 +1352,44 @@ def test_cabi_argsort_is_stable(gpu, rng, n):
     assert np.array_equal(np.sort(pm), np.arange(n)) and np.array_equal(sk, wild[pm])
     for p in (dk, ds, dp):
         hip.dali_hip_free(p)
+
+
+def test_graphs_refuse_what_would_allocate_and_memory_calls_refuse_a_capture(gpu, D, O, rng):
+    """A recording whose replay takes temporary blocks from the bank (an index ordering of more than 16384 keys, a top_k by
+    sorting) cannot become a graph: the block addresses would be baked into it while the bank hands the blocks to others.
+    The attempt fails with a clear error, the capture is closed, and eager replays and later work are unaffected."""
+    hip = gpu
+    V, Dm, N = 500, 32, 20000
+    table0 = rng.randn(V, Dm).astype(np.float32)
+    idx = rng.randint(0, V, N).astype(np.int32)
+    upd = rng.randn(N, Dm).astype(np.float32)
+    table, ids, vals = arr(D, table0), arr(D, idx), arr(D, upd)
+    with D.Recording() as rec:
+        g = table[ids]
+        g += vals
+    want = O.scatter_rows(table0, idx, upd, op=1)
+    assert np.array_equal(table.numpy(), want)
+    with pytest.raises(D.DaliError, match="captured"):
+        rec.make_graph()
+    rec.replay(1)  # launch by launch it still works
+    want = O.scatter_rows(want, idx, upd, op=1)
+    assert np.array_equal(table.numpy(), want)
+    scores = arr(D, rng.randn(64, 300).astype(np.float32))
+    with D.Recording() as rec2:
+        top = D.op.top_k(scores, 100)
+        top.eval()
+    with pytest.raises(D.DaliError, match="captured"):
+        rec2.make_graph()
+    # the memory entry points themselves
+    p = C.c_void_p()
+    assert hip.dali_hip_capture_begin() == 0
+    a = hip.dali_hip_bank_allocate(C.byref(p), 4096)
+    b = hip.dali_hip_malloc(C.byref(p), 4096)
+    c = hip.dali_hip_memset_async(C.c_void_p(1), 0, 16)
+    junk = C.c_void_p()
+    hip.dali_hip_capture_end(C.byref(junk))  # nothing was captured: reports that, and the stream is usable again
+    assert a != 0 and b != 0 and c != 0
+    assert np.array_equal((arr(D, idx) + 1).numpy(), idx + 1)
 
 
 def test_named_comparison_and_any_all_helpers(gpu, D, rng):
