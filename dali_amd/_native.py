@@ -82,6 +82,7 @@ HIP_SYMBOLS = {
     "dali_hip_module_is_loaded": (_i, [_u64]),
     "dali_hip_launch": (_i, [_u64, C.POINTER(H), _ip, C.POINTER(_ip), C.POINTER(_ip), C.POINTER(H), C.POINTER(_ip)]),
     "dali_hip_compile_only": (_i, [C.c_char_p, C.POINTER(_sz)]),
+    "dali_hip_rtc_options": (C.c_char_p, []),
     "dali_hip_jit_stats": (_i, [C.POINTER(_u64), C.POINTER(_u64), C.POINTER(_u64)]),
     "dali_hip_set_cache_dir": (_i, [C.c_char_p]),
     "dali_hip_cache_warm": (_i, [C.POINTER(_i)]),

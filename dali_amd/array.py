@@ -152,8 +152,10 @@ class Array(object):
             elif isinstance(k, slice):
                 n = out.shape[axis]
                 start, stop, step = k.indices(n)
-                if step <= 0:
-                    raise IndexError("negative slice steps are not supported")
+                if step < 0:
+                    # numpy walks start, start + step, ... down to above stop; the native slice names the same elements by
+                    # their range [stop + 1, start + 1) and walks it from its last element (dali/array/slice.cpp:27-37)
+                    start, stop = stop + 1, start + 1
                 if stop < start:
                     stop = start
                 if (start, stop, step) != (0, n, 1):

@@ -123,20 +123,21 @@ static bool env_true(const char* name) {
     return s == "true" || s == "1" || s == "TRUE" || s == "True";
 }
 
+// Options every generated kernel is compiled with (besides the target). No fast-math and no contraction: the CPU path
+// this is checked against is built without either (dali/utils/compiler.cpp:137-145). The leading kernel parameters (up
+// to the 14 scalar registers the hardware offers) arrive preloaded with the wave instead of through a load at its start.
+static const char* const kRtcOptions[] = {"-O3", "-ffp-contract=off", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                                          "-mllvm", "-amdgpu-kernarg-preload-count=14"};
+
 // hipRTC: source -> gfx code object
 static int rtc_compile(const std::string& arch, const char* src, std::vector<char>* code, std::string* log) {
     hiprtcProgram prog;
     hiprtcResult r = hiprtcCreateProgram(&prog, src, "dali_jit.hip", 0, nullptr, nullptr);
     if (r != HIPRTC_SUCCESS) return fail("hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
     std::string arch_opt = "--offload-arch=" + arch;
-    // No fast-math and no contraction: the CPU path this is checked against is
-    // built without either (dali/utils/compiler.cpp:137-145).
-    // The leading kernel parameters (up to the 14 scalar registers the hardware offers) arrive preloaded with the wave
-    // instead of through a load at its start.
-    const char* opts[] = {arch_opt.c_str(), "-O3", "-ffp-contract=off", "-std=c++17",
-                          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                          "-mllvm", "-amdgpu-kernarg-preload-count=14"};
-    r = hiprtcCompileProgram(prog, (int)(sizeof(opts) / sizeof(opts[0])), opts);
+    std::vector<const char*> opts = {arch_opt.c_str()};
+    for (const char* o : kRtcOptions) opts.push_back(o);
+    r = hiprtcCompileProgram(prog, (int)opts.size(), opts.data());
     size_t log_size = 0;
     hiprtcGetProgramLogSize(prog, &log_size);
     if (log_size > 1) {
@@ -470,6 +471,15 @@ int dali_hip_set_cache_dir(const char* path) {
     return DALI_HIP_OK;
 }
 
+const char* dali_hip_rtc_options(void) {
+    static const std::string joined = [] {
+        std::string s;
+        for (const char* o : kRtcOptions) s += std::string(o) + " ";
+        return s;
+    }();
+    return joined.c_str();
+}
+
 int dali_hip_compile_only(const char* hip_source, size_t* code_size) {
     std::vector<char> code;
     std::string log;
@@ -600,7 +610,25 @@ int dali_hip_module_load(uint64_t hash, const char* hip_source, const char* kern
     }
     if (e != hipSuccess) return fail("hipModuleLoadData failed: %s", hipGetErrorString(e));
     e = hipModuleGetFunction(&m.fn, m.module, kernel_name);
-    if (e != hipSuccess) return fail("hipModuleGetFunction(%s) failed: %s", kernel_name, hipGetErrorString(e));
+    if (e != hipSuccess && cached && hip_source) {
+        // a cached object without this entry point (written by another build): drop it and rebuild from source
+        (void)hipGetLastError();
+        (void)hipModuleUnload(m.module);
+        m.module = nullptr;
+        std::string log;
+        if (rtc_compile(r.arch, hip_source, &code, &log)) return DALI_HIP_ERROR;
+        std::ofstream out(path, std::ios::binary);
+        out.write(code.data(), (std::streamsize)code.size());
+        r.n_compiled++;
+        cached = 0;
+        e = hipModuleLoadData(&m.module, code.data());
+        if (e != hipSuccess) return fail("hipModuleLoadData failed: %s", hipGetErrorString(e));
+        e = hipModuleGetFunction(&m.fn, m.module, kernel_name);
+    }
+    if (e != hipSuccess) {
+        if (m.module) (void)hipModuleUnload(m.module);
+        return fail("hipModuleGetFunction(%s) failed: %s", kernel_name, hipGetErrorString(e));
+    }
 
     m.plan = *plan;
     m.array_ndim.assign(plan->array_ndim, plan->array_ndim + plan->n_arrays);

@@ -458,7 +458,7 @@ Array Array::pluck_axis(int axis, int idx) const {
 Array Array::slice(int axis, int start, int end, int step) const {
     if (axis < 0) axis += ndim();
     DALI_ASSERT(axis >= 0 && axis < ndim(), make_message("slice axis ", axis, " out of range for ndim ", ndim()));
-    DALI_ASSERT(step > 0, "slice step must be positive");
+    DALI_ASSERT(step != 0, "slice step cannot be zero");
     auto e = as_buffer(*this).expression();
     int n = e->shape[axis];
     if (start < 0) start += n;
@@ -467,9 +467,13 @@ Array Array::slice(int axis, int start, int end, int step) const {
                 make_message("slice [", start, ":", end, "] out of range for axis of size ", n));
     auto st = normalized_strides();
     std::vector<int> nshape = e->shape, nstrides = st;
-    nshape[axis] = (end - start + step - 1) / step;
+    // dali/array/slice.cpp:76-81, dali/array/expression/buffer.cpp:177-209: ceil((end - start) / |step|) elements; a negative
+    // step walks the same range [start, end) from its last element down, i.e. the view starts at end - 1
+    const int astep = step < 0 ? -step : step;
+    nshape[axis] = (end - start + astep - 1) / astep;
     nstrides[axis] = st[axis] * step;
-    return buffer_view(e, nshape, nstrides, e->offset + start * st[axis]);
+    const int first = step > 0 || end == start ? start : end - 1;
+    return buffer_view(e, nshape, nstrides, e->offset + first * st[axis]);
 }
 
 Array Array::ascontiguousarray() const {

@@ -1284,8 +1284,12 @@ std::unordered_map<uint64_t, bool>& loaded_hashes() {
     return m;
 }
 
+// The identity of a generated kernel, also the name of its code object on disk: besides the structure of the request it
+// covers everything else that shapes the code (the generator's version, the device support code prepended to every kernel
+// and the compiler options), so an edit to any of those cannot meet a stale code object.
 uint64_t kernel_hash(const std::string& kind, const std::string& sig, const std::string& params) {
-    return Hasher().add(std::string(kCodegenVersion)).add(kind).add(sig).add(params).value();
+    static const uint64_t toolchain = Hasher().add(std::string(codegen::kDevicePrelude)).add(std::string(dali_hip_rtc_options())).value();
+    return Hasher().add(std::string(kCodegenVersion)).add(toolchain).add(kind).add(sig).add(params).value();
 }
 
 // entry-point name: shape + hash, so that a profile tells the generated kernels apart
@@ -2778,7 +2782,11 @@ void run_gemm(const Array& dst, const Expr* mm, const Expr* mm2, float beta) {
     jit_stats().last_kernel_kinds += mm2 ? "gemm_pair" : "gemm";
     if (g_dry_run) return;
     int ldc = dst.strides().empty() ? dst.shape()[1] : dst.strides()[0];
-    memory::AM mode = beta == 0.0f ? memory::AM_MUTABLE : memory::AM_MUTABLE;
+    // an overwritten destination that spans its whole allocation needs no migration of what it held (a strided or partial
+    // view keeps the elements between and around its rows, so those stay MUTABLE)
+    const bool spans = dst.offset() == 0 && dst.contiguous_memory() &&
+                       (size_t)numel_of(dst.shape()) * (size_t)size_of_dtype(dst.dtype()) == dst.expression()->memory->bytes();
+    memory::AM mode = beta == 0.0f && spans ? memory::AM_OVERWRITE : memory::AM_MUTABLE;
     if (!mm2) {
         const float* rp = (const float*)g.rhs.device_ptr();
         const float* lp = (const float*)g.lhs.device_ptr();

@@ -179,6 +179,10 @@ int dali_hip_launch(uint64_t hash, void** array_data, const int* offsets, const 
  * code object size; used to check generated source on machines without a GPU. */
 int dali_hip_compile_only(const char* hip_source, size_t* code_size);
 
+/* The hipRTC options (besides the target) every generated kernel is compiled with, space-separated: part of what a
+ * caller must fold into `hash` so that code objects built under other options are not taken from the disk cache. */
+const char* dali_hip_rtc_options(void);
+
 /* Counters: modules compiled by hipRTC, loaded from disk, and launches so far. */
 int dali_hip_jit_stats(uint64_t* compiled, uint64_t* disk_hits, uint64_t* launches);
 

@@ -31,8 +31,17 @@ class Gen(object):
         self.size_terms = 0  # number of summed terms feeding the result (for the tolerance)
 
     def leaf(self, shape):
-        kind = self.rng.randint(0, 5)
+        kind = self.rng.randint(0, 7)
         x = self.rng.uniform(-2.0, 2.0, shape).astype(np.float32)
+        if kind >= 5:
+            # views with negative steps: one axis reversed, or every axis reversed with a skip along the last one
+            if kind == 5:
+                axis = self.rng.randint(len(shape))
+                key = tuple(slice(None, None, -1) if d == axis else slice(None) for d in range(len(shape)))
+                return arr(self.D, x)[key], x[key].astype(np.float64)
+            wide = self.rng.uniform(-2.0, 2.0, shape[:-1] + (2 * shape[-1],)).astype(np.float32)
+            key = tuple(slice(None, None, -1) for _ in shape[:-1]) + (slice(None, None, -2),)
+            return arr(self.D, wide)[key], wide[key].astype(np.float64)
         if kind == 0 and len(shape) == 2 and shape[1] > 1:
             # strided view: every other column of a wider buffer
             wide = self.rng.uniform(-2.0, 2.0, (shape[0], 2 * shape[1])).astype(np.float32)

@@ -1392,6 +1392,68 @@ def test_graphs_refuse_what_would_allocate_and_memory_calls_refuse_a_capture(gpu
     assert np.array_equal((arr(D, idx) + 1).numpy(), idx + 1)
 
 
+def test_slices_with_negative_steps(gpu, D, O, rng):
+    """Slice(start, end, step < 0) names ceil((end - start) / |step|) elements of [start, end), walked from end - 1 down
+    (dali/array/slice.cpp:27-37,76-81, expression/buffer.cpp:177-209): the view starts at the range's last element and its
+    stride is negative. The reference's own cases (tests.cpp:345-357,475-479,557-562,922-941, other_tests.cpp:37), then
+    maps, reductions, assignments and products over such views against numpy."""
+    op = D.op
+    # sizes: Slice(0,5,-2) -> 3, Slice(0,6,-3) -> 2, Slice(0,7,-3) -> 3 (tests.cpp:475-479)
+    v = arr(D, np.arange(7, dtype=np.int32))
+    assert v.slice(0, 0, 5, -2).numpy().tolist() == [4, 2, 0]
+    assert v.slice(0, 0, 6, -3).numpy().tolist() == [5, 2]
+    assert v.slice(0, 0, 7, -3).numpy().tolist() == [6, 3, 0]
+    # proper_slicing (tests.cpp:557-562): x[Slice(0,-1)][2][Slice(0,4,-2)] of arange [2,3,4] sums to 20
+    x234 = arr(D, np.arange(24, dtype=np.int32).reshape(2, 3, 4))
+    sliced = x234.slice(0, 0, -1).pluck_axis(1, 2).slice(1, 0, 4, -2)
+    assert int(op.sum(sliced).numpy()) == 20
+    # a reversed vector shares its storage and spans it (tests.cpp:345-350)
+    z = arr(D, np.arange(4, dtype=np.float32))
+    zr = z[::-1]
+    assert zr.numpy().tolist() == [3.0, 2.0, 1.0, 0.0] and zr.strides == (-1,) and zr.offset == 3
+    zr += 10.0  # writes through the view
+    assert z.numpy().tolist() == [10.0, 11.0, 12.0, 13.0]
+    # advanced_striding_with_reductions (tests.cpp:922-941): filling a reversed view element by element undoes the reversal
+    for key in ((slice(None), slice(None, None, -1)), (slice(None, None, -1),)):
+        y = arr(D, np.arange(12, dtype=np.int32).reshape(3, 4))
+        yv = y[key]
+        yv.assign(arr(D, np.arange(12, dtype=np.int32).reshape(3, 4)))
+        assert np.array_equal(y.numpy(), np.arange(12).reshape(3, 4)[key])
+        assert int(op.sum(op.equals(arr(D, np.arange(12, dtype=np.int32).reshape(3, 4)), yv)).numpy()) == 12
+    # against numpy on ragged shapes: maps, reductions along and against the reversed axes, softmax, a product
+    for shape in ((5, 7), (64, 130), (33, 1024), (4, 6, 50)):
+        a = rng.randn(*shape).astype(np.float32)
+        A = arr(D, a)
+        for key in (tuple([slice(None, None, -1)] + [slice(None)] * (len(shape) - 1)),
+                    tuple([slice(None)] * (len(shape) - 1) + [slice(None, None, -1)]),
+                    tuple(slice(None, None, -1) for _ in shape),
+                    tuple([slice(None, None, -2)] + [slice(None)] * (len(shape) - 2) + [slice(None, None, -3)]),
+                    tuple([slice(None)] * (len(shape) - 1) + [slice(shape[-1] - 2, 1, -1)])):
+            view, ref = A[key], a[key]
+            assert view.shape == ref.shape
+            assert np.array_equal(view.numpy(), ref)
+            assert np.array_equal((view * 2.0 + 1.0).numpy(), ref * np.float32(2.0) + np.float32(1.0))
+            ref64 = ref.astype(np.float64)
+            close(op.sum(view, [len(shape) - 1]).numpy(), ref64.sum(-1), rtol=1e-5, atol=1e-5 * np.abs(ref64).sum(-1).max())
+            close(op.sum(view, [0]).numpy(), ref64.sum(0), rtol=1e-5, atol=1e-5 * np.abs(ref64).sum(0).max())
+            assert np.array_equal(op.argmax(view, len(shape) - 1).numpy(), ref.argmax(-1))
+            assert float(op.max(view).numpy()) == ref.max()
+            e = np.exp(ref64 - ref64.max(-1, keepdims=True))
+            close(op.softmax(view).numpy(), e / e.sum(-1, keepdims=True), rtol=1e-5, atol=1e-12)
+            out = arr(D, np.zeros(shape, np.float32))
+            out[key].assign(view)  # reversed destination and reversed source: a plain copy in memory order
+            want = np.zeros(shape, np.float32)
+            want[key] = ref
+            assert np.array_equal(out.numpy(), want)
+        if len(shape) == 2:
+            b = rng.randn(shape[1], 9).astype(np.float32)
+            got = op.dot(A[::-1, ::-1], arr(D, b)[::-1]).numpy()
+            want = a[::-1, ::-1].astype(np.float64) @ b[::-1].astype(np.float64)
+            close(got, want, rtol=1e-4, atol=1e-4 * np.abs(want).max())
+    with pytest.raises(D.DaliError, match="step cannot be zero"):
+        v.slice(0, 0, 3, 0)
+
+
 def test_named_comparison_and_any_all_helpers(gpu, D, rng):
     # ArrayTests/BinaryTests of the reference use these through Array::equals / allclose (binary.cpp:7-18, reducers.cpp:61-72)
     op = D.op
