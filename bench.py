@@ -317,6 +317,26 @@ def main():
             op.lstm_sequence(Xs, Hp, Cp, W, U, bias)
         seq_us = time_recording(srec, 10)
         configs["c5_lstm_step_256x1024x1024"]["sequence_of_32_us_per_step"] = round(seq_us / 32, 2)
+        # small batches: the whole sequence as one product for the input half plus one persistent launch for the recurrent
+        # half (U stays in the LDS, a grid barrier per step), beside the same sequence as one fused launch per step
+        small = {}
+        for Bs in (8, 32, 64):
+            Xq = D.Array.from_numpy(np.random.RandomState(24).randn(32, Bs, H).astype(np.float32))
+            hs0, cs0 = (D.Array.from_numpy(np.random.RandomState(s).randn(Bs, H).astype(np.float32)) for s in (25, 26))
+            row = {}
+            for name, flag in (("persistent", "1"), ("launch_per_step", "0")):
+                os.environ["DALI_HIP_LSTM_PERSISTENT"] = flag
+                with D.Recording() as qrec:
+                    op.lstm_sequence(Xq, hs0, cs0, W, U, bias)
+                row[name + "_us_per_step"] = round(time_recording(qrec, 10) / 32, 2)
+                row[name + "_launches"] = qrec.launches
+            os.environ.pop("DALI_HIP_LSTM_PERSISTENT", None)
+            sflops = 2.0 * Bs * (I + H) * 4 * H
+            row["mfma_fp32_bound_us"] = round(sflops / MFMA_FP32_PEAK_TFLOPS / 1e6, 2)
+            row["weights_from_hbm_bound_us"] = round(2 * 1024 * 4096 * 4 / HBM_PEAK_GBS / 1e3, 2)  # what a launch per step re-reads
+            small["B%d" % Bs] = row
+            del Xq, hs0, cs0, qrec
+        configs["c5_lstm_step_256x1024x1024"]["sequence_of_32_small_batches"] = small
         del X, Hp, Cp, W, U, bias, rec, grec, Xs, srec
 
         # rows beyond the five configs: embedding-style gather and its scatter-add (table [32000, 1024], 8192 indices)

@@ -1,0 +1,285 @@
+// The recurrent half of an LSTM along a whole sequence in ONE launch, for small batches
+// (dali/layers/lstm.cpp:294-303 runs the cell step by step; the reference's third_party/nervana_kernels
+// persistent_rnn_fprop.sass was meant to play this role on its hardware).
+//
+// At batch sizes of a few dozen rows one step is neither bound by the matrix pipe nor by memory: a launch per step
+// spends its time waiting (37 us per step whatever the batch, measured up to 128 rows). What a step needs from memory
+// is the recurrent weight matrix U [H, 4H], the same every step. The 256 compute units of an MI355X have 40 MiB of
+// LDS between them, so U (16 MiB at H = 1024) stays on the chip for the whole sequence: workgroup g (one per compute
+// unit) keeps the 4 * HU columns of U that produce the four gates of its HU hidden units, and per step
+//   1. multiplies the previous hidden state h(t-1) [B, H] (read from global memory: it is the only thing the
+//      workgroups exchange) with its slice of U on the matrix cores (v_mfma_f32_16x16x4_f32, the K range split over
+//      the four waves and folded through LDS),
+//   2. adds the input half of the pre-activations, pre[t] = x(t).W + bias, which does not depend on h and is computed
+//      for all steps at once by one large product before this kernel runs,
+//   3. applies the gates for its hidden units (same arithmetic, operation by operation, as the fused single step:
+//      double-precision sigmoid, tanhf, no contraction) and writes its HU columns of h(t),
+//   4. meets the other workgroups at a barrier (a counter in global memory; release before, acquire after) so that
+//      h(t) is complete before anyone reads it.
+// The cell state of a workgroup's hidden units never leaves its registers.
+//
+// The barrier only works when every workgroup is resident, which holds because the grid has at most one workgroup per
+// compute unit. Its wait is bounded: a workgroup that does not see the others arrive within `spin_limit` polls raises a
+// flag in host-visible memory, every workgroup leaves at its next poll, and the next synchronising call of the
+// library reports the failure instead of hanging the device.
+#include "runtime.h"
+
+#include <cstdint>
+#include <cstdlib>
+
+namespace dali_hip {
+
+// same sequence as the exp of the generated kernels and of the fused single step (sgemm.hip)
+__device__ __forceinline__ float seq_expf(float x) {
+    const float c = 0x1.715476p+0f, cc = 0x1.4ae0bep-26f;
+    const float t = x * c;
+    float r = __builtin_fmaf(x, c, -t);
+    r = __builtin_fmaf(x, cc, r);
+    const float e = __builtin_amdgcn_exp2f(t);
+    const float fixed = __builtin_fmaf(e, r * 0x1.62e430p-1f, e);
+    return __builtin_fabsf(t) < 128.0f ? fixed : e;
+}
+
+struct PersistentArgs {
+    int T, B, H, HU, ldu;
+    const float* pre;   // [T, B, 4H]
+    const float* U;     // [H, 4H], row stride ldu
+    const float* h0;    // [B, H]
+    const float* c0;    // [B, H]
+    float* hs;          // [T, B, H]
+    float* c_out;       // [B, H]
+    unsigned int* bar;  // barrier counter (zero at rest)
+    unsigned int* done; // exit counter (zero at rest)
+    int* status;        // host-visible: set to 1 when a barrier wait gave up
+    unsigned int spin_limit;
+};
+
+constexpr int kPitchPad = 4;  // LDS row pitch of the U slice = 4 * HU + 4 floats: the four k-groups of a wave land 16 banks apart
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+constexpr int kCoherentLoad = 16;  // cache policy of a buffer load: device scope (the sc1 bit)
+
+// MT: 16-row tiles of the batch (B <= 16 * MT); KQ = H / 64: trips of 16 values of k in a wave's quarter of the K range
+template <int MT, int KQ>
+__global__ __launch_bounds__(256) void lstm_persistent_kernel(PersistentArgs a) {
+    extern __shared__ float lds[];
+    const int H = a.H, HU = a.HU, NC = 4 * HU, P = NC + kPitchPad, B = a.B;
+    float* Us = lds;                       // [H][P]
+    float* red = lds + (size_t)H * P;      // [4 waves][MT][16][16]
+    __shared__ int give_up;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // Consecutive workgroups land on different parts of the chip (eight, each with a second-level cache of its own): the
+    // slices are dealt so that one part holds neighbouring columns and the 64-byte lines of U are fetched by one cache only.
+    const int parts = (gridDim.x & 7) == 0 ? 8 : 1;
+    const int slice = (blockIdx.x % parts) * (gridDim.x / parts) + blockIdx.x / parts;
+    const int u0 = slice * HU;
+    // this workgroup's slice of U: local column j = gate * HU + uu  <->  U column gate * H + u0 + uu
+    if (HU == 4 && (a.ldu & 3) == 0 && ((uintptr_t)a.U & 15) == 0) {
+        // one 16-byte load per (k, gate), eight in flight per thread
+        for (int e0 = tid; e0 < H * 4; e0 += 256 * 8) {
+            f4 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int e = e0 + 256 * i, k = e >> 2, gate = e & 3;
+                v[i] = e < H * 4 ? *reinterpret_cast<const f4*>(a.U + (size_t)k * a.ldu + (size_t)gate * H + u0) : (f4){0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int e = e0 + 256 * i, k = e >> 2, gate = e & 3;
+                if (e < H * 4) *reinterpret_cast<f4*>(Us + (size_t)k * P + 4 * gate) = v[i];
+            }
+        }
+    } else {
+        for (int e0 = tid; e0 < H * NC; e0 += 256 * 8) {
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int e = e0 + 256 * i, k = e / NC, j = e - k * NC, gate = j / HU, uu = j - gate * HU;
+                v[i] = e < H * NC ? a.U[(size_t)k * a.ldu + (size_t)gate * H + u0 + uu] : 0.0f;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int e = e0 + 256 * i, k = e / NC, j = e - k * NC;
+                if (e < H * NC) Us[(size_t)k * P + j] = v[i];
+            }
+        }
+    }
+    if (tid == 0) give_up = 0;
+    // the (row, hidden unit) pair this thread finishes every step, and its cell value
+    const int pb = tid / HU, puu = tid - pb * HU;
+    const bool owner = tid < B * HU;
+    float cell = owner ? a.c0[(size_t)pb * H + u0 + puu] : 0.0f;
+    __syncthreads();
+
+    const int KW = H / 4;             // K range of a wave
+    const int arow = lane & 15, kgrp = lane >> 4;
+    // The values of h cross compute units (and their second-level caches) once a step. They are written and read with
+    // device-coherent accesses (stores and loads at agent scope go past the caches that are private to a part of the chip),
+    // so the step needs no cache-wide release or acquire: those fences write back and invalidate the whole second-level
+    // cache and took 15 to 24 us of a step.
+    float pre4[4] = {0.f, 0.f, 0.f, 0.f};
+    auto fetch_pre = [&](int t) {
+        if (owner) {
+#pragma unroll
+            for (int gate = 0; gate < 4; ++gate) pre4[gate] = a.pre[((size_t)t * B + pb) * 4 * H + (size_t)gate * H + u0 + puu];
+        }
+    };
+    fetch_pre(0);
+    for (int t = 0; t < a.T; ++t) {
+        const float* hp = t == 0 ? a.h0 : a.hs + (size_t)(t - 1) * B * H;
+        // rows past the batch are out of the buffer's range and read as zero
+        const __amdgpu_buffer_rsrc_t hrow = __builtin_amdgcn_make_buffer_rsrc((void*)hp, 0, B * H * 4, 0x00027000);
+        f4 acc[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[m] = (f4){0.f, 0.f, 0.f, 0.f};
+        // 16 values of k per trip: a lane fetches four consecutive k of its batch row with one 16-byte load and feeds them
+        // to four matrix instructions; the slice of U is read at the matching rows, so which k sits in which slot of the
+        // instruction does not matter to the sum. Every load of the step is issued before the first product: the step pays
+        // the latency of h(t-1) once.
+        f4 av[KQ][MT];
+#pragma unroll
+        for (int q = 0; q < KQ; ++q) {
+            const int kb = wave * KW + 16 * q + 4 * kgrp;
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+                av[q][m] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(hrow, ((16 * m + arow) * H + kb) * 4, 0, kCoherentLoad));
+        }
+#pragma unroll
+        for (int q = 0; q < KQ; ++q) {
+            const int kb = wave * KW + 16 * q + 4 * kgrp;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float bv = Us[(size_t)(kb + c) * P + arow];  // B operand: row k of the slice, column lane % 16
+#pragma unroll
+                for (int m = 0; m < MT; ++m) acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[q][m][c], bv, acc[m], 0, 0, 0);
+            }
+        }
+        // fold the four waves' partial tiles: lane holds column lane % 16 and rows 4 * (lane / 16) + v
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[((size_t)(wave * MT + m) * 16 + 4 * kgrp + v) * 16 + arow] = acc[m][v];
+        __syncthreads();
+        if (owner) {
+#pragma clang fp contract(off)
+            float g4[4];
+#pragma unroll
+            for (int gate = 0; gate < 4; ++gate) {
+                const int j = gate * HU + puu;
+                float s = 0.0f;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) s += red[((size_t)(w * MT + pb / 16) * 16 + (pb & 15)) * 16 + j];
+                g4[gate] = pre4[gate] + s;
+            }
+            const float iv = (float)(1.0 / (1.0 + (double)seq_expf(-g4[0])));
+            const float fv = (float)(1.0 / (1.0 + (double)seq_expf(-g4[1])));
+            const float ov = (float)(1.0 / (1.0 + (double)seq_expf(-g4[2])));
+            const float gv = tanhf(g4[3]);
+            const float fc = fv * cell;
+            const float ig = iv * gv;
+            cell = fc + ig;
+            __hip_atomic_store(a.hs + ((size_t)t * B + pb) * H + u0 + puu, ov * tanhf(cell), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (t + 1 == a.T) break;
+        // grid barrier: everybody's columns of h(t) have reached device memory before anybody reads row t
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();  // (also: the fold area is free again)
+        if (tid == 0) __hip_atomic_fetch_add(a.bar, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        fetch_pre(t + 1);  // does not depend on h: in flight during the wait
+        if (tid == 0) {
+            const unsigned int target = gridDim.x * (unsigned int)(t + 1);
+            unsigned int polls = 0;
+            while (__hip_atomic_load(a.bar, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+                __builtin_amdgcn_s_sleep(1);
+                if ((++polls & 63u) == 0u && __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) {
+                    give_up = 1;  // somebody else gave up
+                    break;
+                }
+                if (polls >= a.spin_limit) {
+                    __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    give_up = 1;
+                    break;
+                }
+            }
+        }
+        __syncthreads();
+        if (give_up) break;
+    }
+    if (owner) a.c_out[(size_t)pb * H + u0 + puu] = cell;
+    // the counters go back to zero once every workgroup is past its last wait
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned int ticket = __hip_atomic_fetch_add(a.done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (ticket == gridDim.x - 1) {
+            __hip_atomic_store(a.bar, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(a.done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+static int* g_status = nullptr;  // pinned host word the kernel raises on a barrier time-out
+
+int persistent_status_take() {
+    if (!g_status) return 0;
+    const int v = __atomic_exchange_n(g_status, 0, __ATOMIC_RELAXED);
+    return v;
+}
+
+}  // namespace dali_hip
+
+using namespace dali_hip;
+
+extern "C" int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0,
+                                                  const float* c0, float* hs, float* c_out) {
+    if (ensure_init()) return DALI_HIP_ERROR;
+    if (steps < 1 || batch < 1 || hidden < 1) return fail("dali_hip_lstm_recurrent_persistent: steps, batch and hidden must be positive");
+    if (!pre || !U || !h0 || !c0 || !hs || !c_out) return fail("dali_hip_lstm_recurrent_persistent: NULL argument");
+    if (batch > 64) return fail("dali_hip_lstm_recurrent_persistent: batch %d exceeds 64 rows (use one launch per step)", batch);
+    if (hidden % 256 != 0 || hidden > 1024) return fail("dali_hip_lstm_recurrent_persistent: hidden %d must be 256, 512, 768 or 1024", hidden);
+    if (((uintptr_t)h0 | (uintptr_t)hs) % 16 != 0) return fail("dali_hip_lstm_recurrent_persistent: h0 and hs must be 16-byte aligned");
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, bound_device()) != hipSuccess) return fail("dali_hip_lstm_recurrent_persistent: no device properties");
+    const int cus = prop.multiProcessorCount;
+    // fewest hidden units per workgroup that still give every workgroup a compute unit of its own
+    int HU = 1;
+    while (HU <= 4 && !(hidden % HU == 0 && hidden / HU <= cus)) ++HU;
+    // (the four gates of at most 4 hidden units fill the 16 columns of one matrix instruction)
+    if (HU > 4 || batch * HU > 256)
+        return fail("dali_hip_lstm_recurrent_persistent: hidden %d needs more than 4 hidden units per compute unit on %d compute units", hidden, cus);
+    const int grid = hidden / HU, MT = (batch + 15) / 16;
+    const size_t lds_bytes = ((size_t)hidden * (4 * HU + kPitchPad) + (size_t)4 * MT * 256) * sizeof(float);
+    if (lds_bytes > (size_t)160 * 1024 - 1024)
+        return fail("dali_hip_lstm_recurrent_persistent: the slice of U per compute unit (%zu bytes) does not fit the LDS", lds_bytes);
+    if (!g_status) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        (void)hipStreamIsCapturing(stream(), &cs);
+        if (cs != hipStreamCaptureStatusNone) return fail("dali_hip_lstm_recurrent_persistent: first use cannot be inside a capture");
+        if (hipHostMalloc((void**)&g_status, sizeof(int), hipHostMallocMapped) != hipSuccess) return fail("dali_hip_lstm_recurrent_persistent: no pinned status word");
+        *g_status = 0;
+    }
+    PersistentArgs a;
+    a.T = steps; a.B = batch; a.H = hidden; a.HU = HU; a.ldu = ldu;
+    a.pre = pre; a.U = U; a.h0 = h0; a.c0 = c0; a.hs = hs; a.c_out = c_out;
+    // the last two counters of the workspace (zero at rest, like the reduction tickets)
+    a.bar = (unsigned int*)workspace() + kWorkspaceCounters - 2;
+    a.done = (unsigned int*)workspace() + kWorkspaceCounters - 1;
+    a.status = g_status;
+    static const unsigned int spin_env = getenv("DALI_HIP_PERSISTENT_SPIN_LIMIT") ? (unsigned int)atol(getenv("DALI_HIP_PERSISTENT_SPIN_LIMIT")) : (1u << 20);
+    a.spin_limit = spin_env;
+    hipError_t e = hipSuccess;
+    auto launch = [&](auto kernel) {
+        e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e == hipSuccess) hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream(), a);
+    };
+    const int KQ = hidden / 64;
+#define DALI_PERSISTENT_CASE(mt, kq) \
+    if (MT == mt && KQ == kq) launch(lstm_persistent_kernel<mt, kq>);
+    DALI_PERSISTENT_CASE(1, 4) DALI_PERSISTENT_CASE(2, 4) DALI_PERSISTENT_CASE(3, 4) DALI_PERSISTENT_CASE(4, 4)
+    DALI_PERSISTENT_CASE(1, 8) DALI_PERSISTENT_CASE(2, 8) DALI_PERSISTENT_CASE(3, 8) DALI_PERSISTENT_CASE(4, 8)
+    DALI_PERSISTENT_CASE(1, 12) DALI_PERSISTENT_CASE(2, 12) DALI_PERSISTENT_CASE(3, 12) DALI_PERSISTENT_CASE(4, 12)
+    DALI_PERSISTENT_CASE(1, 16) DALI_PERSISTENT_CASE(2, 16) DALI_PERSISTENT_CASE(3, 16) DALI_PERSISTENT_CASE(4, 16)
+#undef DALI_PERSISTENT_CASE
+    if (e == hipSuccess) e = hipGetLastError();
+    if (e != hipSuccess) return fail("dali_hip_lstm_recurrent_persistent launch failed: %s", hipGetErrorString(e));
+    return DALI_HIP_OK;
+}

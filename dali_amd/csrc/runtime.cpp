@@ -220,10 +220,17 @@ int dali_hip_mem_info(size_t* free_bytes, size_t* total_bytes) {
     return DALI_HIP_OK;
 }
 
+// after the stream has drained: did a persistent kernel abandon a grid barrier?
+static int check_persistent_status() {
+    if (persistent_status_take())
+        return fail("a persistent kernel gave up waiting at a grid barrier (its workgroups were not all resident in time); its outputs are undefined");
+    return DALI_HIP_OK;
+}
+
 int dali_hip_sync(void) {
     if (ensure_init()) return DALI_HIP_ERROR;
     HIP_TRY(hipStreamSynchronize(rt().stream));
-    return DALI_HIP_OK;
+    return check_persistent_status();
 }
 
 void* dali_hip_stream(void) {
@@ -390,7 +397,7 @@ int dali_hip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes) {
     if (bytes == 0) return DALI_HIP_OK;
     HIP_TRY(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, rt().stream));
     HIP_TRY(hipStreamSynchronize(rt().stream));
-    return DALI_HIP_OK;
+    return check_persistent_status();
 }
 
 int dali_hip_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes) {

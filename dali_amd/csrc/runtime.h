@@ -27,6 +27,8 @@ char* workspace();
 int bound_device();
 // sort.hip: looks up the device address of its built-in scratch array; called by dali_hip_init with `device` current
 int sort_scratch_init(int device);
+// lstm_persistent.hip: 1 when a persistent kernel's grid barrier gave up since the last call (and clears that)
+int persistent_status_take();
 
 }  // namespace dali_hip
 

@@ -5115,6 +5115,29 @@ void lstm_step_fused(const Array& x, const Array& h, const Array& c, const Array
     }
 }
 
+// the recurrent half of a whole sequence in one launch (records itself like any other launch)
+void lstm_recurrent_persistent(const Array& pre, const Array& U, const Array& h0, const Array& c0, const Array& hs, const Array& c_out) {
+    const int T = hs.shape()[0], Bn = hs.shape()[1], H = hs.shape()[2];
+    const float* pp = (const float*)pre.device_ptr();
+    const float* up = (const float*)U.device_ptr();
+    const float* hp = (const float*)h0.device_ptr();
+    const float* cp = (const float*)c0.device_ptr();
+    float* ho = (float*)hs.device_ptr(memory::AM_OVERWRITE);
+    float* co = (float*)c_out.device_ptr(memory::AM_OVERWRITE);
+    jit_stats().gemms_launched++;
+    jit_stats().last_kernel_kinds = "lstm_persistent";
+    check_hip(dali_hip_lstm_recurrent_persistent(T, Bn, H, pp, up, 4 * H, hp, cp, ho, co), "persistent lstm sequence");
+    if (g_recording) {
+        note_recorded_write(hs.expression()->memory);
+        note_recorded_write(c_out.expression()->memory);
+        std::vector<Array> keep = {pre, U, h0, c0, hs, c_out};
+        g_recording->push_back([=]() {
+            (void)keep;
+            check_hip(dali_hip_lstm_recurrent_persistent(T, Bn, H, pp, up, 4 * H, hp, cp, ho, co), "persistent lstm sequence replay");
+        });
+    }
+}
+
 void evaluate(const std::vector<Array>& roots) {
     jit_stats().evals++;
     jit_stats().last_kernel_kinds.clear();

@@ -246,6 +246,23 @@ int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx
                        const float* Cprev, const float* W, int ldw, const float* U, int ldu, const float* bias,
                        float* Cout, float* Hout);
 
+/*
+ * The recurrent half of an LSTM over a whole sequence in one launch, for batches of at most 64 rows: the loop of
+ * dali/layers/lstm.cpp:294-303 (one cell activation per time step), whose hidden-to-hidden product the reference meant to
+ * hand to a persistent kernel (third_party/nervana_kernels/sass/persistent_rnn_fprop.sass). pre [steps, batch, 4 hidden]
+ * holds the input half of the pre-activations for every step, x(t).W + bias, gates packed i, f, o, g along the columns (one
+ * large product computed beforehand); U [hidden, 4 hidden] (row stride ldu) stays in the LDS of the compute units for the
+ * whole sequence; per step every workgroup forms h(t-1).U for the gate columns of its hidden units, finishes the cell
+ * (same arithmetic as dali_hip_lstm_step) and meets the others at a grid barrier. hs [steps, batch, hidden] receives every
+ * hidden state, c_out [batch, hidden] the last cell state. hidden must be a multiple of 64 whose slice of U per compute
+ * unit fits the LDS (hidden = 1024 on 256 compute units: 80 KiB); h0 and hs 16-byte aligned. The grid has at most one
+ * workgroup per compute unit, so all are resident; a workgroup that still does not see the others arrive within 2^20 polls
+ * (DALI_HIP_PERSISTENT_SPIN_LIMIT) raises a flag, every workgroup leaves, and the next dali_hip_sync or
+ * dali_hip_memcpy_d2h fails with that message instead of the device hanging.
+ */
+int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0,
+                                       const float* c0, float* hs, float* c_out);
+
 /* ------------------------------------------------------------- scatter */
 /*
  * Stable ordering of n int32 keys held in device memory: sorted_keys[p] is the p-th smallest key and

@@ -1603,6 +1603,62 @@ def test_lstm_sequence_is_the_step_applied_in_turn(gpu, D, O, rng, T, B, I, H):
     assert np.array_equal(hs.numpy(), first)
 
 
+@pytest.mark.parametrize("T,B,H", [(2, 1, 256), (5, 8, 256), (4, 17, 512), (3, 40, 768), (3, 64, 1024), (33, 8, 1024)])
+def test_lstm_sequence_in_one_persistent_launch(gpu, D, O, rng, T, B, H):
+    """Small batches: the input half of every step's pre-activations is one product, the recurrent half one launch that
+    keeps U in the LDS of the compute units and steps through the sequence behind grid barriers (the role of the
+    reference's persistent_rnn_fprop kernel for the loop of dali/layers/lstm.cpp:294-303). Same values as the step applied
+    in turn, to the tolerance of a product summed in another order."""
+    Xs = rng.randn(T, B, H).astype(np.float32)
+    H0, C0 = (rng.randn(B, H).astype(np.float32) for _ in range(2))
+    lim = np.sqrt(6.0 / (H + 4 * H))
+    W, U = (rng.uniform(-lim, lim, (H, 4 * H)).astype(np.float32) for _ in range(2))
+    b = (rng.randn(4 * H) * 0.1).astype(np.float32)
+    dev = [arr(D, v) for v in (Xs, H0, C0, W, U, b)]
+    with D.Recording() as rec:
+        hs, c_last, h_last = D.op.lstm_sequence(*dev)
+    assert D.last_kernel_kinds() == "lstm_persistent"
+    assert hs.shape == (T, B, H) and np.array_equal(h_last.numpy(), hs.numpy()[-1])
+    ohs, oc = O.lstm_sequence(Xs, H0, C0, W, U, b)
+    close(hs.numpy(), ohs, rtol=2e-4, atol=2e-5)
+    close(c_last.numpy(), oc, rtol=2e-4, atol=2e-5)
+    # against the step applied in turn (launch per step)
+    h, c = dev[1], dev[2]
+    for t in range(T):
+        c, h = D.op.lstm_step(arr(D, Xs[t]), h, c, dev[3], dev[4], dev[5])
+        close(hs.numpy()[t], h.numpy(), rtol=1e-4, atol=1e-5)
+    # the recording recomputes the same sequence, bit for bit, and the barrier counters are back at rest
+    first, first_c = hs.numpy().copy(), c_last.numpy().copy()
+    rec.replay(2)
+    assert np.array_equal(hs.numpy(), first) and np.array_equal(c_last.numpy(), first_c)
+    # a reduction right behind it finds its own tickets at zero
+    close(D.op.sum(hs).numpy(), first.astype(np.float64).sum(), rtol=1e-5, atol=1e-5 * np.abs(first).sum())
+
+
+def test_persistent_lstm_barrier_gives_up_instead_of_hanging():
+    """With the poll limit forced to one, the first workgroup at the first barrier gives up, raises the flag, every
+    workgroup leaves (the kernel ends normally) and the next synchronising call reports it."""
+    import subprocess, sys, os
+    code = (
+        "import numpy as np, dali_amd as D\n"
+        "from dali_amd._native import hip\n"
+        "rng = np.random.RandomState(0)\n"
+        "T, B, H = 6, 8, 1024\n"
+        "dev = [D.Array.from_numpy(v.astype(np.float32)) for v in (rng.randn(T, B, H), rng.randn(B, H), rng.randn(B, H), rng.randn(H, 4 * H) * 0.01, rng.randn(H, 4 * H) * 0.01, np.zeros(4 * H))]\n"
+        "hs, c, h = D.op.lstm_sequence(*dev)\n"
+        "rc = hip.dali_hip_sync()\n"
+        "print('SYNC', rc, hip.dali_hip_last_error().decode())\n"
+        "print('AGAIN', hip.dali_hip_sync())\n"
+        "x = D.Array.from_numpy(np.ones((4, 4), np.float32))\n"
+        "print('AFTER', float(D.op.sum(x * 2.0).numpy()))\n"
+    )
+    env = dict(os.environ, DALI_HIP_PERSISTENT_SPIN_LIMIT="1", PYTHONPATH=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert "SYNC 1" in out.stdout and "gave up waiting at a grid barrier" in out.stdout, out.stdout
+    assert "AGAIN 0" in out.stdout and "AFTER 32.0" in out.stdout, out.stdout
+
+
 @pytest.mark.parametrize("B,I,H", [(16, 32, 48), (64, 128, 128), (5, 7, 9)])
 def test_gru_step_matches_oracle(gpu, D, O, rng, B, I, H):
     X, Hp = rng.randn(B, I).astype(np.float32), rng.randn(B, H).astype(np.float32)
