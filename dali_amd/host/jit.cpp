@@ -71,7 +71,7 @@ static void note_recorded_write(const std::shared_ptr<memory::SynchronizedMemory
 namespace {
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-33";
+const char* const kCodegenVersion = "dali-hip-codegen-35";
 
 // boost-style combine of the reference (dali/utils/hash_utils.h:12-23)
 struct Hasher {
@@ -508,6 +508,7 @@ struct RowParams {
     bool tail = false;       // ragged, and C is no multiple of VEC: the rest of a row is handled one element to a thread
     int EPT_L = 0;           // cached rows: the last EPT_L of the EPT vectors a thread holds live in LDS instead of registers
     bool split = false;      // maps without a reduction over few long rows: every row is cut into S pieces, one workgroup each
+    int band_unroll = 1;     // rows of a band whose loads are issued together
     int band = 0;            // maps with operands broadcast along the rows ([1, C]): a workgroup walks `band` rows and keeps those operands
 };
 
@@ -1155,20 +1156,33 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
             ss << hb.stmts.str() << "      hv" << k << "[j] = " << v << "; hr" << k << "[j] = 1.0f / hv" << k << "[j]; hok = hok && dali_div_ok(hv" << k << "[j]);\n    }\n";
         }
         auto emit_rows = [&](int div_mode) {
-            ss << "    for (int rr = 0; rr < BAND; ++rr) {\n      if (row + rr >= R) break;\n";
+            // U rows at a time: their loads are all issued before the first row is worked on
+            const int U = rp.band_unroll;
+            auto row_pointer = [&](size_t i, const std::string& rr, const char* indent) {
+                const ArrayArg& a = P.arrays[i];
+                ss << indent << (a.is_dest ? "" : "const ") << ctype(a.buf->dtype) << "* w" << i << " = q" << i << " + (long)(" << rr << ") * " << row_stride((int)i) << ";\n";
+            };
+            ss << "    for (int r0 = 0; r0 < BAND; r0 += " << U << ") {\n      if (row + r0 >= R) break;\n";
+            for (int i : full_leaves)
+                if (!is_colvec(i)) ss << "      " << ctype(P.arrays[i].buf->dtype) << " x" << i << "u[" << U << "][VEC];\n";
+            ss << "      _Pragma(\"unroll\") for (int u = 0; u < " << U << "; ++u) {\n        if (row + r0 + u < R) {\n";
+            for (int i : full_leaves)
+                if (!is_colvec(i)) {
+                    row_pointer((size_t)i, "r0 + u", "          ");
+                    emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i) + "u[u]", "          ", rp.nt_loads, rp.ragged, "w");
+                }
+            ss << "        }\n      }\n";
+            ss << "      _Pragma(\"unroll\") for (int u = 0; u < " << U << "; ++u) {\n      const int rr = r0 + u;\n      if (row + rr >= R) break;\n";
             for (size_t i = 0; i < P.arrays.size(); ++i) {
                 const ArrayArg& a = P.arrays[i];
                 const std::string t = ctype(a.buf->dtype);
-                if (a.cls == Cls::FULL && !is_colvec((int)i))
-                    ss << "      " << (a.is_dest ? "" : "const ") << t << "* w" << i << " = q" << i << " + (long)rr * " << row_stride((int)i) << ";\n";
+                if (a.cls == Cls::FULL && a.is_dest)
+                    row_pointer(i, "rr", "      ");
                 else if (a.cls == Cls::ROW && !a.is_dest)
                     ss << "      const " << t << " rl" << i << " = ((const " << t << "*)A.p[" << i << "])[(row + rr)" << (a.strided ? " * (long)A.iv[" + std::to_string(L.stride_pos[i]) + "]" : std::string()) << "];\n";
             }
             for (int i : full_leaves)
-                if (!is_colvec(i)) {
-                    ss << "      " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n";
-                    emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", rp.nt_loads, rp.ragged, "w");
-                }
+                if (!is_colvec(i)) ss << "      const " << ctype(P.arrays[i].buf->dtype) << "* x" << i << " = x" << i << "u[u];\n";
             BodyEmitter be(P, rp, true, rpn.n_phases, &rpn.first_body);
             std::vector<int> again;
             be.band_divisors = &again;
@@ -1186,7 +1200,7 @@ std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::str
                 body << "        " << ov << ".v[j] = " << op_combine(o.op, ov + ".v[j]", "(" + t + ")(" + be.value(o.root) + ")") << ";\n";
             }
             ss << pre.str() << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        const int col = ch * VEC + j; (void)col;\n" << be.stmts.str() << body.str()
-               << "      }\n" << post.str() << "    }\n";
+               << "      }\n" << post.str() << "      }\n    }\n";
         };
         if (divs.empty()) {
             emit_rows(0);
@@ -1350,7 +1364,7 @@ void load_and_launch(KernelSpec& K, const std::function<std::string()>& gen, con
             cached = 2;
         } else {
             std::string src = gen();
-            g_last_source += src;
+                g_last_source += src;
             st.plans_built++;
             check_hip(dali_hip_module_load(K.hash, src.c_str(), K.name.c_str(), &K.plan, &cached), "JIT module load");
         }
@@ -1569,7 +1583,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
         // least 1024 vectors, as many as bring the grid to about 4096 workgroups
         // operands broadcast along the rows ([1, C] against [R, C]: a bias, per-column statistics): a workgroup walks a band of
         // rows chunk by chunk and keeps those operands, and the reciprocal of a divisor made of them, in registers
-        static const int band_env = env_int("DALI_HIP_ROW_BAND", 32);
+        static const int band_env = env_int("DALI_HIP_ROW_BAND", 4);
         bool colvec = false, band_ok = band_env > 1 && rp.VEC == 4 && !rp.tail && rp.TPR == 256 && n_totals == 0 && dom.R >= 2 * band_env;
         for (const ArrayArg& a : P.arrays) {
             if (a.cls == Cls::FULL && !a.is_dest && a.strided && a.strides[0] == 0 && !a.gather_source) colvec = true;
@@ -1577,7 +1591,11 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
         }
         for (const Output& o : rpn.outputs) band_ok = band_ok && o.cls == Cls::FULL;
         for (const PNode& nd : P.nodes) band_ok = band_ok && nd.kind != Kind::GATHER_FROM_ROWS && nd.kind != Kind::GATHER;
-        if (colvec && band_ok) rp.band = band_env;
+        if (colvec && band_ok) {
+            static const int unroll_env = env_int("DALI_HIP_ROW_BAND_UNROLL", 1);
+            rp.band = band_env;
+            rp.band_unroll = unroll_env >= 1 && band_env % unroll_env == 0 ? unroll_env : 1;
+        }
         static const int split_env = env_int("DALI_HIP_ROW_SPLIT", 1);
         if (split_env && rp.band == 0 && n_totals == 0 && rp.TPR == 256 && dom.R < 1024 && CH >= 4096) {
             while (split_S * 2 * dom.R <= 4096 && CH / (split_S * 2) >= 1024) split_S *= 2;
@@ -1676,13 +1694,15 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
 
     // kernel identity
     std::ostringstream params;
-    // Streaming policy: outputs always leave with non-temporal stores; inputs bypass cache
-    // allocation once the operands are too large to be found in a cache again (64 MiB).
+    // Streaming policy: outputs of a kernel that reduces over its rows leave with non-temporal stores (C1 4.6 against
+    // 5.9 us, cross-entropy [8192, 32000] 357 against 383 us), outputs of a plain map with ordinary stores (x + bias on
+    // [8192, 8192]: 0.88 against 0.72 of the HBM peak); inputs bypass cache allocation once the operands are too large
+    // to be found in a cache again (64 MiB).
     static const int nt_l = env_int("DALI_HIP_ROW_NT_LOADS", -1), nt_s = env_int("DALI_HIP_ROW_NT_STORES", -1);
     rp.nt_loads = nt_l >= 0 ? nt_l != 0 : dom.R * dom.C * (int64_t)max_el >= ((int64_t)64 << 20);
-    rp.nt_stores = nt_s >= 0 ? nt_s != 0 : true;
+    rp.nt_stores = nt_s >= 0 ? nt_s != 0 : rpn.n_phases > 0;
     params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached << "," << rp.waves_per_eu << ","
-           << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail << "," << rp.EPT_L << (rp.split ? "S" : "") << (rp.band > 1 ? "B" + std::to_string(rp.band) : std::string());
+           << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail << "," << rp.EPT_L << (rp.split ? "S" : "") << (rp.band > 1 ? "B" + std::to_string(rp.band) + "u" + std::to_string(rp.band_unroll) : std::string());
     if (n_totals) {
         // one 8-byte slot per workgroup and total in the workspace's 32 MiB of partial results
         const int64_t blocks = (dom.R + rp.RPB - 1) / rp.RPB;
@@ -1743,7 +1763,7 @@ bool flat_eligible(const Array& a, int64_t n, std::set<const Expr*>& seen) {
 // UNALIGNED: some operand starts off a 16-byte boundary (element-aligned vector accesses). REST: the element count is
 // no multiple of VEC; the first block's leading threads take one of the last N % VEC elements each.
 std::string gen_flat_kernel(const Program& P, const std::vector<Output>& outs, const IvLayout& L, int VEC, int BT, int UNROLL, bool UNALIGNED, bool REST,
-                            const std::string& kname) {
+                            const std::string& kname, bool NT_STORES, bool NT_LOADS) {
     std::ostringstream ss;
     RowParams rp;
     rp.cached = false;
@@ -1761,7 +1781,7 @@ std::string gen_flat_kernel(const Program& P, const std::vector<Output>& outs, c
     ss << "  const long base = (long)blockIdx.x * (BT * UNROLL) + threadIdx.x;\n";
     for (int i : full_leaves) ss << "  " << ctype(P.arrays[i].buf->dtype) << " x" << i << "s[UNROLL][VEC];\n";
     ss << "  _Pragma(\"unroll\") for (int u = 0; u < UNROLL; ++u) {\n    const long ch = base + (long)u * BT;\n    if (ch < NCH) {\n";
-    for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, VEC, "x" + std::to_string(i) + "s[u]", "      ", true, UNALIGNED);
+    for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, VEC, "x" + std::to_string(i) + "s[u]", "      ", NT_LOADS, UNALIGNED);
     ss << "    }\n  }\n";
     ss << "  _Pragma(\"unroll\") for (int u = 0; u < UNROLL; ++u) {\n    const long ch = base + (long)u * BT;\n    if (ch < NCH) {\n";
     for (int i : full_leaves) ss << "      const " << ctype(P.arrays[i].buf->dtype) << "* x" << i << " = x" << i << "s[u];\n";
@@ -1774,7 +1794,7 @@ std::string gen_flat_kernel(const Program& P, const std::vector<Output>& outs, c
         std::string ov = "o" + std::to_string(o.array);
         pre << "      dali_vec<" << t << ", VEC> " << ov << ";\n";
         if (o.op != OPERATOR_T_EQL) pre << "      " << ov << " = " << (UNALIGNED ? "dali_loadu<" : "dali_load<") << t << ", VEC>(q" << o.array << " + ch * VEC);\n";
-        post << "      " << (UNALIGNED ? "dali_storeu_nt<" : "dali_store_nt<") << t << ", VEC>(q" << o.array << " + ch * VEC, " << ov << ");\n";
+        post << "      " << (UNALIGNED ? (NT_STORES ? "dali_storeu_nt<" : "dali_storeu<") : (NT_STORES ? "dali_store_nt<" : "dali_store<")) << t << ", VEC>(q" << o.array << " + ch * VEC, " << ov << ");\n";
         std::string v = be.value(o.root);
         body << "        " << ov << ".v[j] = " << op_combine(o.op, ov + ".v[j]", "(" + t + ")(" + v + ")") << ";\n";
     }
@@ -1832,9 +1852,17 @@ bool try_flat(const std::vector<DestSpec>& specs) {
     for (const ArrayArg& a : P.arrays)
         if (a.cls == Cls::FULL && a.buf->offset % 4 != 0) aligned = false;
     int VEC = n >= 16 ? 4 : 1, BT = 256, UNROLL = max_el == 8 ? 2 : 4;
+    static const int unroll_env = env_int("DALI_HIP_FLAT_UNROLL", 0);
+    if (unroll_env > 0) UNROLL = unroll_env;
     const bool UNALIGNED = VEC > 1 && !aligned, REST = VEC > 1 && n % VEC != 0;
     std::ostringstream params;
-    params << VEC << "," << BT << "," << UNROLL << "," << UNALIGNED << REST;
+    // Streaming policy of a map, measured on 64M floats (copy / a + b / a chain of five operands): inputs bypass cache
+    // allocation (plain loads: 0.73 instead of 0.87 of the HBM peak), outputs leave with plain stores (non-temporal stores:
+    // 0.78). Kernels that reduce over cached rows are the other way round for their stores.
+    static const int nt_env = env_int("DALI_HIP_FLAT_NT_STORES", 0);
+    static const int ntl_env = env_int("DALI_HIP_FLAT_NT_LOADS", 1);
+    const bool NT_STORES = nt_env != 0, NT_LOADS = ntl_env != 0;
+    params << VEC << "," << BT << "," << UNROLL << "," << UNALIGNED << REST << "," << NT_STORES << NT_LOADS;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("flat", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& K = specs_cache[h];
@@ -1853,7 +1881,7 @@ bool try_flat(const std::vector<DestSpec>& specs) {
         K->plan.work_per_block = BT * UNROLL * VEC;
     }
     std::vector<std::vector<int>> shapes = {{(int)n}};
-    load_and_launch(*K, [&]() { return gen_flat_kernel(P, outs, L, VEC, BT, UNROLL, UNALIGNED, REST, K->name); }, P, shapes);
+    load_and_launch(*K, [&]() { return gen_flat_kernel(P, outs, L, VEC, BT, UNROLL, UNALIGNED, REST, K->name, NT_STORES, NT_LOADS); }, P, shapes);
     return true;
 }
 

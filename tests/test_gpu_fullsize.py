@@ -79,9 +79,11 @@ def test_c4_cross_entropy_8192x32000(gpu, D, O):
     g, r = grad.numpy(), rl.numpy()
     sel = np.r_[0:64, rows // 2:rows // 2 + 64, rows - 64:rows]
     _, orows, ograd = O.softmax_cross_entropy(x[sel], t[sel])
-    # the checker sums 32000 terms left to right in fp32: its own bound (n-1) * 2^-24 is added to the 1e-5
-    np.testing.assert_allclose(r[sel], orows, rtol=1e-5, atol=vocab * 2.0 ** -24)
-    np.testing.assert_allclose(g[sel], ograd, rtol=1e-5 + vocab * 2.0 ** -24, atol=1e-8)
+    # The checker sums 32000 terms left to right in fp32 and loses small terms to the running sum. Measured on an MI355X
+    # over 768 rows of this input: row losses differ by at most 8.3e-7 relative (9.5e-6 absolute), gradient entries by at
+    # most 1.0e-5 relative. The bounds are four times that (the checker's a-priori bound n * 2^-24 = 1.9e-3 is 190 times it).
+    np.testing.assert_allclose(r[sel], orows, rtol=3.5e-6, atol=0)
+    np.testing.assert_allclose(g[sel], ograd, rtol=4e-5, atol=1e-8)
     x64 = x[sel].astype(np.float64)
     lse = np.log(np.exp(x64 - x64.max(1, keepdims=True)).sum(1)) + x64.max(1)
     np.testing.assert_allclose(r[sel], lse - x64[np.arange(len(sel)), t[sel]], rtol=1e-5, atol=2e-6)  # fp64 truth, plain 1e-5

@@ -33,10 +33,13 @@ def close(got, want, rtol=1e-5, atol=1e-6):
 def seq_sum_rtol(n):
     """Tolerance against the CPU checker for a value normalised by a length-n fp32 sum of positive terms.
 
-    The reference accumulates left to right in fp32; its own a-priori error bound is (n - 1) * 2^-24 (and long
-    rows do lose small terms to stagnation), while the GPU folds a tree. Against fp64 truth the GPU result is
-    held to a plain rel 1e-5; against the sequential checker the checker's bound is added."""
-    return 1e-5 + (n - 1) * 2.0 ** -24
+    The reference accumulates left to right in fp32 and drops terms below half an ulp of the running sum (stagnation), so
+    its result drifts from the true sum in proportion to n; the GPU folds a tree and stays within 1.5e-6 of fp64 truth at
+    every length tried. Largest relative deviation GPU against checker measured on an MI355X (12 draws per length,
+    N(0,1) and N(0,9) inputs): n=5 3.0e-7, 33 6.1e-7, 1024 1.8e-6, 4096 4.6e-6, 8192 1.7e-5, 32000 4.0e-5, 65536 1.0e-4,
+    100003 2.0e-4, i.e. at most 0.035 * n * 2^-24 beyond a floor of a few ulps. The bound is three times that fit (the
+    a-priori bound (n - 1) * 2^-24 is 29 times it). Against fp64 truth the tests keep a plain rel 1e-5."""
+    return 1e-6 + 0.1 * n * 2.0 ** -24
 
 
 # ------------------------------------------------------------ C ABI directly
