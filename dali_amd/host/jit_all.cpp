@@ -192,8 +192,9 @@ bool try_all(const DestSpec& spec) {
     const bool UNALIGNED = VEC > 1 && !aligned, REST = VEC > 1 && n % VEC != 0;
     int max_el_all = 4;
     for (const ArrayArg& a : P.arrays) max_el_all = std::max(max_el_all, size_of_dtype(a.buf->dtype));
-    const int UNROLL = max_el_all == 8 ? 4 : 8;  // vector loads in flight per thread
-    const int TAIL = 2, MAX_BLOCKS = TAIL * BT;  // 512 blocks; the last one folds every partial in one unrolled pass
+    static const int unroll_env = env_int("DALI_HIP_ALL_UNROLL", 0), tail_env = env_int("DALI_HIP_ALL_TAIL", 0);
+    const int UNROLL = unroll_env > 0 ? unroll_env : (max_el_all == 8 ? 4 : 8);  // vector loads in flight per thread
+    const int TAIL = tail_env > 0 ? tail_env : 2, MAX_BLOCKS = TAIL * BT;  // 512 blocks; the last one folds every partial in one unrolled pass
     std::vector<Output> outs(1);
     outs[0].root = root_id;
     outs[0].array = dest_array;
