@@ -339,6 +339,15 @@ def main():
         configs["c5_lstm_step_256x1024x1024"]["sequence_of_32_small_batches"] = small
         del X, Hp, Cp, W, U, bias, rec, grec, Xs, srec
 
+        # the double-precision product (the reference's cublasDgemm branch)
+        dA, dB = (D.Array.from_numpy(np.random.RandomState(s).randn(2048, 2048)) for s in (27, 28))
+        with D.Recording() as drec:
+            op.dot(dA, dB).eval()
+        dus = time_recording(drec, 10)
+        configs["c5_lstm_step_256x1024x1024"]["dot_fp64_2048x2048x2048"] = {"us": round(dus, 2), "TFLOP/s": round(2.0 * 2048 ** 3 / dus / 1e6, 2),
+                                                                           "frac_fp64_mfma": round(2.0 * 2048 ** 3 / dus / 1e6 / 78.6, 4)}
+        del dA, dB, drec
+
         # rows beyond the five configs: embedding-style gather and its scatter-add (table [32000, 1024], 8192 indices)
         V, Dm, Nidx = 32000, 1024, 8192
         table = D.Array.from_numpy(np.random.RandomState(14).randn(V, Dm).astype(np.float32))

@@ -87,6 +87,7 @@ HIP_SYMBOLS = {
     "dali_hip_set_cache_dir": (_i, [C.c_char_p]),
     "dali_hip_cache_warm": (_i, [C.POINTER(_i)]),
     "dali_hip_sgemm": (_i, [_i, _i, _i, _i, _i, C.c_float, H, _i, H, _i, C.c_float, H, _i]),
+    "dali_hip_dgemm": (_i, [_i, _i, _i, _i, _i, C.c_double, H, _i, H, _i, C.c_double, H, _i]),
     "dali_hip_sgemm_pair": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, C.c_float, H, _i, H, _i, H, _i, H, _i, C.c_float, H, _i]),
     "dali_hip_sgemm_terms": (_i, [_i, _i, _i, _i, _i, _ip, C.POINTER(H), _i, C.POINTER(H), _i, C.c_float, C.c_float, H, _i, _ip]),
     "dali_hip_lstm_step": (_i, [_i, _i, _i, H, _i, H, _i, H, H, _i, H, _i, H, H, H]),

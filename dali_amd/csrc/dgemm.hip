@@ -1,0 +1,143 @@
+// fp64 GEMM on the matrix cores of gfx950 (v_mfma_f64_16x16x4f64): the double-precision branch of op::dot, which the
+// reference hands to cublasDgemm (dali/array/gemm/cublas_gemm.cu:167-178, cblas_dgemm in dali/array/gemm/cpu_gemm.cpp).
+//
+// A workgroup of four waves owns a 64 x 64 tile of C; each wave a 32 x 32 quarter as 2 x 2 accumulators of 16 x 16. A slab
+// of 16 values of k is staged in LDS k-major ([k][row] and [k][column]), so that a lane's operand of the instruction (row
+// or column = lane % 16, k = lane / 16) is one 8-byte read and sixteen lanes read sixteen neighbours. Global loads of the
+// next slab are issued before the products of the current one and land in the other LDS buffer: one barrier per slab.
+// The instruction takes 16 passes (64 cycles), so the loads, the LDS traffic and the address arithmetic of a slab hide
+// behind the sixteen instructions each wave issues for it. Operands are addressed through (row stride, k stride) pairs,
+// which covers the four transposition cases; the lane-to-element map of the global loads follows whichever stride is 1.
+#include <cstdint>
+
+#include "runtime.h"
+
+namespace dali_hip {
+namespace {
+
+typedef double d4 __attribute__((ext_vector_type(4)));
+
+constexpr int BM = 64, BN = 64, BK = 16;
+constexpr int PITCH = 64 + 2;  // doubles per LDS row: the four k-groups of an operand read start 4 banks apart
+
+struct DgemmArgs {
+    int M, N, K;              // row-major problem: C[M, N] = alpha * A[M, K] * B[K, N] + beta * C
+    const double* A;
+    long ai, ak;              // element (i, k) of A at A[i * ai + k * ak]
+    const double* B;
+    long bk, bj;              // element (k, j) of B at B[k * bk + j * bj]
+    double* C;
+    long ldc;
+    double alpha, beta;
+};
+
+__global__ __launch_bounds__(256) void dgemm_kernel(DgemmArgs a) {
+    __shared__ double As[2][BK][PITCH];
+    __shared__ double Bs[2][BK][PITCH];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tiles_n = (a.N + BN - 1) / BN;
+    const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+    const int m0 = tm * BM, n0 = tn * BN;
+    // which element of a 64 x 16 tile a thread fetches in its c-th load (c = 0..3): along k when k is the unit stride,
+    // along the rows otherwise
+    const bool a_k_fast = a.ak == 1, b_k_fast = a.bk == 1;
+    int ar[4], akk[4], bc[4], bkk[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        ar[c] = a_k_fast ? tid / 16 + 16 * c : tid % 64;
+        akk[c] = a_k_fast ? tid % 16 : tid / 64 + 4 * c;
+        bc[c] = b_k_fast ? tid / 16 + 16 * c : tid % 64;
+        bkk[c] = b_k_fast ? tid % 16 : tid / 64 + 4 * c;
+    }
+    double ra[4], rb[4];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int i = m0 + ar[c], k = k0 + akk[c];
+            ra[c] = (i < a.M && k < a.K) ? a.A[(long)i * a.ai + (long)k * a.ak] : 0.0;
+            const int j = n0 + bc[c], kb = k0 + bkk[c];
+            rb[c] = (j < a.N && kb < a.K) ? a.B[(long)kb * a.bk + (long)j * a.bj] : 0.0;
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            As[buf][akk[c]][ar[c]] = ra[c];
+            Bs[buf][bkk[c]][bc[c]] = rb[c];
+        }
+    };
+    const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+    const int r = lane & 15, kg = lane >> 4;
+    d4 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = (d4){0.0, 0.0, 0.0, 0.0};
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    const int slabs = (a.K + BK - 1) / BK;
+    for (int s = 0; s < slabs; ++s) {
+        const int buf = s & 1;
+        if (s + 1 < slabs) fetch((s + 1) * BK);
+#pragma unroll
+        for (int ks = 0; ks < BK; ks += 4) {
+            double av[2], bv[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) av[i] = As[buf][ks + kg][wm + 16 * i + r];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) bv[j] = Bs[buf][ks + kg][wn + 16 * j + r];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[i], bv[j], acc[i][j], 0, 0, 0);
+        }
+        if (s + 1 < slabs) stage(buf ^ 1);  // the other buffer: last read before the previous barrier
+        __syncthreads();
+    }
+    // a lane holds column lane % 16 and rows 4 * v + lane / 16 of each 16 x 16 accumulator
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int row = m0 + wm + 16 * i + 4 * v + kg, col = n0 + wn + 16 * j + r;
+                if (row < a.M && col < a.N) {
+                    double* p = a.C + (long)row * a.ldc + col;
+                    const double prod = a.alpha * acc[i][j][v];
+                    *p = a.beta == 0.0 ? prod : prod + a.beta * *p;
+                }
+            }
+}
+
+}  // namespace
+}  // namespace dali_hip
+
+using namespace dali_hip;
+
+extern "C" int dali_hip_dgemm(int transB, int transA, int m, int n, int k, double alpha, const double* B, int ldb, const double* A, int lda,
+                              double beta, double* C, int ldc) {
+    if (ensure_init()) return DALI_HIP_ERROR;
+    if (m < 0 || n < 0 || k < 0) return fail("dali_hip_dgemm: negative extent (m=%d n=%d k=%d)", m, n, k);
+    if (m == 0 || n == 0) return DALI_HIP_OK;
+    if (!C || (k > 0 && (!A || !B))) return fail("dali_hip_dgemm: NULL operand");
+    // row-major view of the column-major call: C[n, m] = alpha * A[n, k] * B[k, m] + beta * C
+    const int rows = n, cols = m;
+    if (ldc < cols) return fail("dali_hip_dgemm: ldc %d is smaller than the row length %d", ldc, cols);
+    if (k > 0) {
+        if (lda < (transA ? rows : k)) return fail("dali_hip_dgemm: lda %d is too small", lda);
+        if (ldb < (transB ? k : cols)) return fail("dali_hip_dgemm: ldb %d is too small", ldb);
+    }
+    DgemmArgs a;
+    a.M = rows; a.N = cols; a.K = k;
+    a.A = A; a.ai = transA ? 1 : lda; a.ak = transA ? lda : 1;
+    a.B = B; a.bk = transB ? 1 : ldb; a.bj = transB ? ldb : 1;
+    a.C = C; a.ldc = ldc; a.alpha = alpha; a.beta = beta;
+    const long tiles = (long)((rows + BM - 1) / BM) * ((cols + BN - 1) / BN);
+    if (tiles > 0x7fffffffL) return fail("dali_hip_dgemm: too many tiles");
+    hipLaunchKernelGGL(dgemm_kernel, dim3((unsigned)tiles), dim3(256), 0, stream(), a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("dali_hip_dgemm launch failed: %s", hipGetErrorString(e));
+    return DALI_HIP_OK;
+}

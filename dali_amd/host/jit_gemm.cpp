@@ -47,8 +47,9 @@ static GemmOperands prepare_gemm(const Expr* mm) {
     GemmOperands g;
     g.lhs = gemm_operand(mm->args[0]);
     g.rhs = gemm_operand(mm->args[1]);
-    DALI_ASSERT(g.lhs.dtype() == DTYPE_FLOAT && g.rhs.dtype() == DTYPE_FLOAT,
-                "op::dot on this backend is implemented for float32 operands (MFMA fp32 GEMM)");
+    DALI_ASSERT(g.lhs.dtype() == g.rhs.dtype() && (g.lhs.dtype() == DTYPE_FLOAT || g.lhs.dtype() == DTYPE_DOUBLE),
+                "op::dot on this backend is implemented for float32 and float64 operands (MFMA GEMM; the reference's integer "
+                "product is a scalar CPU loop)");
     gemm_stride_transpose(g.lhs, &g.lt, &g.lld);
     gemm_stride_transpose(g.rhs, &g.rt, &g.rld);
     return g;
@@ -69,6 +70,34 @@ void run_gemm(const Array& dst, const Expr* mm, const Expr* mm2, float beta) {
     const bool spans = dst.offset() == 0 && dst.contiguous_memory() &&
                        (size_t)numel_of(dst.shape()) * (size_t)size_of_dtype(dst.dtype()) == dst.expression()->memory->bytes();
     memory::AM mode = beta == 0.0f && spans ? memory::AM_OVERWRITE : memory::AM_MUTABLE;
+    if (g.lhs.dtype() == DTYPE_DOUBLE) {
+        // cublasDgemm's branch (dali/array/gemm/cublas_gemm.cu:167-178); a pair of products is two accumulating calls
+        struct Call { int rt, lt, k; const double* rp; int rld; const double* lp; int lld; double beta; };
+        std::vector<Call> calls;
+        std::vector<GemmOperands> keep = {g};
+        calls.push_back({g.rt, g.lt, k, (const double*)g.rhs.device_ptr(), g.rld, (const double*)g.lhs.device_ptr(), g.lld, (double)beta});
+        if (mm2) {
+            GemmOperands h = prepare_gemm(mm2);
+            DALI_ASSERT(h.lhs.dtype() == DTYPE_DOUBLE, "op::dot: the two products of a sum must share a dtype");
+            keep.push_back(h);
+            calls.push_back({h.rt, h.lt, h.rhs.shape()[0], (const double*)h.rhs.device_ptr(), h.rld, (const double*)h.lhs.device_ptr(), h.lld, 1.0});
+        }
+        double* dp = (double*)dst.device_ptr(mode);
+        auto issue = [=]() {
+            for (const Call& c : calls) check_hip(dali_hip_dgemm(c.rt, c.lt, m, n, c.k, 1.0, c.rp, c.rld, c.lp, c.lld, c.beta, dp, ldc), "dgemm");
+        };
+        issue();
+        if (g_recording) {
+            note_recorded_write(dst.expression()->memory);
+            Array dkeep = dst;
+            g_recording->push_back([=]() {
+                (void)keep;
+                (void)dkeep;
+                issue();
+            });
+        }
+        return;
+    }
     if (!mm2) {
         const float* rp = (const float*)g.rhs.device_ptr();
         const float* lp = (const float*)g.lhs.device_ptr();

@@ -125,7 +125,7 @@ Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root) {
         }
         case Kind::ELEMENTWISE: {
             if (e->name == "functor::add" && e->args.size() == 2 && is_plain_matmul(e->args[0]) && is_plain_matmul(e->args[1]) &&
-                e->dtype == DTYPE_FLOAT && e->args[0].shape() == e->args[1].shape()) {
+                (e->dtype == DTYPE_FLOAT || e->dtype == DTYPE_DOUBLE) && e->args[0].shape() == e->args[1].shape()) {
                 Array dst(e->shape, e->dtype);
                 run_gemm(dst, e->args[0].expression().get(), e->args[1].expression().get(), 0.0f);
                 out = dst;
@@ -652,7 +652,7 @@ void evaluate_into(const Array& dest, OPERATOR_T op, const Array& source) {
     std::map<const Expr*, Array> memo;
     auto se = src.expression();
     // dst (+)= dot(a, b): the GEMM writes (accumulates into) the destination directly
-    if (se->kind == Kind::MATMUL && dest.dtype() == DTYPE_FLOAT && dest.ndim() == 2 &&
+    if (se->kind == Kind::MATMUL && (dest.dtype() == DTYPE_FLOAT || dest.dtype() == DTYPE_DOUBLE) && se->dtype == dest.dtype() && dest.ndim() == 2 &&
         (dest.strides().empty() || dest.strides()[1] == 1) && (op == OPERATOR_T_EQL || op == OPERATOR_T_ADD)) {
         run_gemm(dest, se.get(), nullptr, op == OPERATOR_T_ADD ? 1.0f : 0.0f);
         return;

@@ -211,6 +211,16 @@ int dali_hip_sgemm(int transB, int transA, int m, int n, int k, float alpha, con
                    const float* A, int lda, float beta, float* C, int ldc);
 
 /*
+ * fp64 GEMM on the matrix cores, same conventions as dali_hip_sgemm: replaces
+ * cublasDgemm(handle, transB, transA, m, n, k, &alpha, B, ldb, A, lda, &beta, C, ldc)
+ * in dali/array/gemm/cublas_gemm.cu:167-178 (and cblas_dgemm in
+ * dali/array/gemm/cpu_gemm.cpp). Any leading dimensions and alignments; k == 0
+ * scales C by beta.
+ */
+int dali_hip_dgemm(int transB, int transA, int m, int n, int k, double alpha, const double* B, int ldb,
+                   const double* A, int lda, double beta, double* C, int ldc);
+
+/*
  * Two products accumulated into one destination in a single launch:
  * C = alpha * (op(B1) * op(A1) + op(B2) * op(A2)) + beta * C with the same
  * conventions as dali_hip_sgemm (k1 and k2 are the two inner extents). This is

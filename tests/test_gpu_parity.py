@@ -273,6 +273,75 @@ def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
         hip.dali_hip_free(p)
 
 
+@pytest.mark.parametrize("ta", [0, 1])
+@pytest.mark.parametrize("tb", [0, 1])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 5, 7), (64, 64, 16), (65, 63, 17), (100, 260, 200), (256, 512, 1000), (250, 1, 33), (1, 300, 64), (37, 41, 0)])
+def test_dgemm_abi_column_major_convention(gpu, rng, M, N, K, ta, tb):
+    """dali_hip_dgemm(transB, transA, m, n, k, alpha, B, ldb, A, lda, beta, C, ldc) as cublasDgemm is called in
+    cublas_gemm.cu:167-178: row-major C[n, m] = alpha * A[n, k] . B[k, m] + beta * C, in double precision. Checked against
+    the product accumulated in extended precision; the products are summed in another order, hence a few ulps of the scale."""
+    hip = gpu
+    A = rng.randn(M, K)
+    B = rng.randn(K, N)
+    C0 = rng.randn(M, N + 3)  # padded destination rows: ldc = N + 3
+    Astore = np.ascontiguousarray(A.T) if ta else A
+    Bstore = np.ascontiguousarray(B.T) if tb else B
+    lda = max(Astore.shape[1], 1) + 2  # leading dimensions larger than the rows
+    ldb = max(Bstore.shape[1], 1) + 1
+    Apad = np.zeros((max(Astore.shape[0], 1), lda)); Apad[:Astore.shape[0], :Astore.shape[1]] = Astore
+    Bpad = np.zeros((max(Bstore.shape[0], 1), ldb)); Bpad[:Bstore.shape[0], :Bstore.shape[1]] = Bstore
+    dA, dB, dC = _dev(hip, Apad), _dev(hip, Bpad), _dev(hip, C0)
+    alpha, beta = 0.75, -0.5
+    st = hip.dali_hip_dgemm(tb, ta, N, M, K, alpha, dB, ldb, dA, lda, beta, dC, N + 3)
+    assert st == 0, hip.dali_hip_last_error()
+    out = np.empty_like(C0)
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+    want = alpha * (A.astype(np.longdouble) @ B.astype(np.longdouble)) + beta * C0[:, :N]
+    bound = (K + 4) * 2.0 ** -52 * (np.abs(A) @ np.abs(B) + np.abs(C0[:, :N]) + 1e-300)
+    assert np.all(np.abs(out[:, :N] - want) <= bound)
+    assert np.array_equal(out[:, N:], C0[:, N:])  # padding untouched
+    # beta == 0 overwrites whatever the destination held, NaN included
+    nan = np.full_like(C0, np.nan)
+    hip.dali_hip_memcpy_h2d(dC, nan.ctypes.data_as(C.c_void_p), nan.nbytes)
+    assert hip.dali_hip_dgemm(tb, ta, N, M, K, 1.0, dB, ldb, dA, lda, 0.0, dC, N + 3) == 0
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+    assert np.all(np.abs(out[:, :N] - (A.astype(np.longdouble) @ B.astype(np.longdouble))) <= bound)
+    assert hip.dali_hip_dgemm(tb, ta, N, M, K, 1.0, dB, ldb, dA, lda, 0.0, dC, N - 1) != 0 or N == 0  # ldc smaller than the row
+    for p in (dA, dB, dC):
+        hip.dali_hip_free(p)
+
+
+def test_dot_in_double_precision(gpu, D, rng):
+    """op::dot of float64 operands (the cublasDgemm branch, cublas_gemm.cu:167-178): lazy, one product per evaluation,
+    transposed and row-strided operands in place, accumulation into a destination, the sum of two products, promotion of
+    a float32 operand (dot.cpp:49-67 promotes before the node is built)."""
+    op = D.op
+    a, b = rng.randn(70, 130), rng.randn(130, 50)
+    A, B = arr(D, a), arr(D, b)
+    before = D.jit_stats()
+    c = op.dot(A, B)
+    assert D.jit_stats() == before and not c.is_buffer()
+    got = c.numpy()
+    assert got.dtype == np.float64 and D.jit_stats()["gemms"] - before["gemms"] == 1
+    tol = dict(rtol=0, atol=200 * 2.0 ** -52 * (np.abs(a) @ np.abs(b)).max())
+    close(got, a @ b, **tol)
+    close(op.dot(arr(D, a.T.copy()).T, B).numpy(), a @ b, **tol)
+    wide = arr(D, np.tile(b, (1, 2)))
+    close(op.dot(A, wide[:, 50:100]).numpy(), a @ b, **tol)
+    dst = arr(D, np.ones((70, 50)))
+    dst += op.dot(A, B)
+    close(dst.numpy(), 1.0 + a @ b, **tol)
+    a2, b2 = rng.randn(70, 20), rng.randn(20, 50)
+    close((op.dot(A, B) + op.dot(arr(D, a2), arr(D, b2))).numpy(), a @ b + a2 @ b2, rtol=0, atol=2 * tol["atol"])
+    mixed = op.dot(arr(D, a.astype(np.float32)), B).numpy()
+    assert mixed.dtype == np.float64
+    close(mixed, a.astype(np.float32).astype(np.float64) @ b, **tol)
+    y = op.tanh(op.dot(A, B) + arr(D, rng.randn(1, 50))).numpy()
+    assert y.dtype == np.float64 and np.all(np.abs(y) <= 1)
+    with pytest.raises(Exception):
+        op.dot(arr(D, np.ones((2, 3), np.int32)), arr(D, np.ones((3, 2), np.int32))).numpy()
+
+
 @pytest.mark.parametrize("M,N,K1,K2", [(48, 200, 96, 40), (100, 260, 200, 200), (256, 512, 128, 192), (250, 1000, 100, 100)])
 def test_sgemm_pair_accumulates_two_products(gpu, rng, M, N, K1, K2):
     hip = gpu
