@@ -23,15 +23,18 @@ namespace dali_hip {
 // tickets live in the library workspace. When key_limit * 2^ceil(log2 n) fits 32 bits a pair is one 32-bit word
 // (key in the high bits, position in the low ones), which halves the cost of a comparison.
 template <typename W>
-__device__ __forceinline__ W rank_pair(int32_t key, int pos, int shift);
+__device__ __forceinline__ W rank_pair(int32_t key, int pos, int shift, int limit);
 template <>
-__device__ __forceinline__ unsigned long long rank_pair<unsigned long long>(int32_t key, int pos, int) {
+__device__ __forceinline__ unsigned long long rank_pair<unsigned long long>(int32_t key, int pos, int, int limit) {
+    // with a key limit, a key outside [0, limit) is ordered as `limit`: behind every valid key
+    if (limit > 0 && (unsigned int)key >= (unsigned int)limit) key = limit;
     return ((unsigned long long)((unsigned int)key ^ 0x80000000u) << 32) | (unsigned int)pos;  // signed key order
 }
 template <>
-__device__ __forceinline__ unsigned int rank_pair<unsigned int>(int32_t key, int pos, int shift) {
-    // a key outside [0, key_limit) (an invalid index) is ordered as the largest valid key: whatever the input, the
-    // words stay distinct, so the positions computed from them are a permutation
+__device__ __forceinline__ unsigned int rank_pair<unsigned int>(int32_t key, int pos, int shift, int) {
+    // a key outside [0, key_limit) (an invalid index) is ordered behind the largest valid key (the packed form is chosen
+    // only when that value fits): whatever the input, the words stay distinct, so the positions computed from them are
+    // a permutation, and a run of equal valid keys is never interrupted
     const unsigned int top = (0xFFFFFFFFu >> shift);
     const unsigned int k = (unsigned int)key < top ? (unsigned int)key : top;
     return (k << shift) | (unsigned int)pos;
@@ -41,7 +44,7 @@ constexpr int kRankSegment = 512;
 constexpr int kRankMaxSegments = 32;  // 16384 keys
 
 template <typename W>
-__global__ __launch_bounds__(256) void rank_sort_kernel(const int32_t* keys, int n, int shift, int segments, int32_t* partial,
+__global__ __launch_bounds__(256) void rank_sort_kernel(const int32_t* keys, int n, int shift, int limit, int segments, int32_t* partial,
                                                          unsigned int* tickets, int32_t* sorted_keys, int32_t* perm) {
     __shared__ __attribute__((aligned(16))) W tile[kRankSegment];
     __shared__ int is_last;
@@ -49,11 +52,11 @@ __global__ __launch_bounds__(256) void rank_sort_kernel(const int32_t* keys, int
     const int j0 = blockIdx.y * kRankSegment;
     for (int t = threadIdx.x; t < kRankSegment; t += 256) {
         const int j = j0 + t;
-        tile[t] = j < n ? rank_pair<W>(keys[j], j, shift) : ~(W)0;  // padding orders after (or with) every real pair
+        tile[t] = j < n ? rank_pair<W>(keys[j], j, shift, limit) : ~(W)0;  // padding orders after (or with) every real pair
     }
     __syncthreads();
     const int32_t my_key = i < n ? keys[i] : 0;
-    const W mine = rank_pair<W>(my_key, i, shift);
+    const W mine = rank_pair<W>(my_key, i, shift, limit);
     int count = 0;
 #pragma unroll 16
     for (int t = 0; t < kRankSegment; ++t) count += tile[t] < mine ? 1 : 0;
@@ -93,9 +96,15 @@ __global__ __launch_bounds__(256) void rank_sort_kernel(const int32_t* keys, int
 // are per (round, wave, digit), and a scan over the 32 (round, wave) slots of every digit gives each group its offset.
 constexpr int kRadixTile = 2048;
 
-__device__ __forceinline__ unsigned int radix_digit(int32_t key, int shift, unsigned int flip) { return (((unsigned int)key ^ flip) >> shift) & 255u; }
+// With a key limit, every key outside [0, limit) takes the digits of `limit` itself: such keys (invalid indices) end up behind all
+// valid ones, in input order, instead of between the keys that share their low bits.
+__device__ __forceinline__ unsigned int radix_digit(int32_t key, int shift, unsigned int flip, unsigned int limit) {
+    unsigned int k = (unsigned int)key ^ flip;
+    if (limit != 0u && k > limit) k = limit;
+    return (k >> shift) & 255u;
+}
 
-__global__ __launch_bounds__(256) void radix_hist_kernel(const int32_t* keys, int n, int shift, unsigned int flip, unsigned int* hist, int tiles) {
+__global__ __launch_bounds__(256) void radix_hist_kernel(const int32_t* keys, int n, int shift, unsigned int flip, unsigned int limit, unsigned int* hist, int tiles) {
     __shared__ unsigned int h[256];
     h[threadIdx.x] = 0u;
     __syncthreads();
@@ -103,7 +112,7 @@ __global__ __launch_bounds__(256) void radix_hist_kernel(const int32_t* keys, in
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
         const long i = base + r * 256 + threadIdx.x;
-        if (i < n) atomicAdd(&h[radix_digit(keys[i], shift, flip)], 1u);
+        if (i < n) atomicAdd(&h[radix_digit(keys[i], shift, flip, limit)], 1u);
     }
     __syncthreads();
     hist[(long)threadIdx.x * tiles + blockIdx.x] = h[threadIdx.x];
@@ -135,7 +144,7 @@ __global__ __launch_bounds__(1024) void radix_scan_kernel(unsigned int* hist, lo
     }
 }
 
-__global__ __launch_bounds__(256) void radix_move_kernel(const int32_t* keys_in, const int32_t* pos_in, int n, int shift, unsigned int flip, const unsigned int* hist,
+__global__ __launch_bounds__(256) void radix_move_kernel(const int32_t* keys_in, const int32_t* pos_in, int n, int shift, unsigned int flip, unsigned int limit, const unsigned int* hist,
                                                          int tiles, int32_t* keys_out, int32_t* pos_out) {
     __shared__ unsigned short cnt[32][256];
     __shared__ unsigned int first_slot[256];
@@ -153,7 +162,7 @@ __global__ __launch_bounds__(256) void radix_move_kernel(const int32_t* keys_in,
         const bool valid = i < n;
         key[r] = valid ? keys_in[i] : 0;
         pos[r] = valid ? (pos_in ? pos_in[i] : (int32_t)i) : 0;
-        digit[r] = radix_digit(key[r], shift, flip);
+        digit[r] = radix_digit(key[r], shift, flip, limit);
         unsigned long long same = __ballot(valid);
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
@@ -519,12 +528,13 @@ static int launch_rank_sort(const int32_t* keys, int ni, int32_t key_limit, unsi
     const int segments = (ni + kRankSegment - 1) / kRankSegment, blocks = (ni + 255) / 256;
     int shift = 0;
     while ((1 << shift) < ni) ++shift;
-    const bool packed = key_limit > 0 && ((unsigned long long)key_limit << shift) <= (1ull << 32);
+    // (one more key value than the valid ones: invalid keys get a word of their own, behind every valid key)
+    const bool packed = key_limit > 0 && (((unsigned long long)key_limit + 1ull) << shift) <= (1ull << 32);
     if (packed)
-        hipLaunchKernelGGL(rank_sort_kernel<unsigned int>, dim3(blocks, segments), dim3(256), 0, st, keys, ni, shift, segments, partial, tickets,
+        hipLaunchKernelGGL(rank_sort_kernel<unsigned int>, dim3(blocks, segments), dim3(256), 0, st, keys, ni, shift, (int)key_limit, segments, partial, tickets,
                            sorted_keys, perm);
     else
-        hipLaunchKernelGGL(rank_sort_kernel<unsigned long long>, dim3(blocks, segments), dim3(256), 0, st, keys, ni, shift, segments, partial,
+        hipLaunchKernelGGL(rank_sort_kernel<unsigned long long>, dim3(blocks, segments), dim3(256), 0, st, keys, ni, shift, (int)key_limit, segments, partial,
                            tickets, sorted_keys, perm);
     hipError_t le = hipGetLastError();
     if (le != hipSuccess) return fail("rank sort launch failed: %s", hipGetErrorString(le));
@@ -587,7 +597,7 @@ extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_
     int end_bit = 32;
     if (key_limit > 0) {
         end_bit = 1;
-        while (end_bit < 31 && ((int64_t)1 << end_bit) < (int64_t)key_limit) ++end_bit;
+        while (end_bit < 31 && ((int64_t)1 << end_bit) <= (int64_t)key_limit) ++end_bit;  // the digits of key_limit itself included
     }
     static const int rank_max = getenv("DALI_HIP_RANK_SORT_MAX") ? atoi(getenv("DALI_HIP_RANK_SORT_MAX")) : 16384;
     if (n <= rank_max && n <= (int64_t)kRankSegment * kRankMaxSegments &&
@@ -599,7 +609,7 @@ extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_
     // the digit). The pairs bounce between the caller's arrays and one temporary block so that the last pass lands in the
     // caller's.
     const int passes = (end_bit + 7) / 8, tiles = (int)((n + kRadixTile - 1) / kRadixTile);
-    const unsigned int flip = key_limit > 0 ? 0u : 0x80000000u;
+    const unsigned int flip = key_limit > 0 ? 0u : 0x80000000u, limit = key_limit > 0 ? (unsigned int)key_limit : 0u;
     const size_t temp_bytes = ((size_t)2 * (size_t)n + (size_t)256 * (size_t)tiles) * sizeof(int32_t);
     void* temp = nullptr;
     if (dali_hip_bank_allocate(&temp, temp_bytes)) return DALI_HIP_ERROR;
@@ -612,9 +622,9 @@ extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_
         const bool to_caller = (passes - 1 - i) % 2 == 0;
         int32_t* dst_keys = to_caller ? sorted_keys : tkeys;
         int32_t* dst_pos = to_caller ? perm : tpos;
-        hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(256), 0, st, src_keys, (int)n, 8 * i, flip, hist, tiles);
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(256), 0, st, src_keys, (int)n, 8 * i, flip, limit, hist, tiles);
         hipLaunchKernelGGL(radix_scan_kernel, dim3(1), dim3(1024), 0, st, hist, (long)256 * tiles);
-        hipLaunchKernelGGL(radix_move_kernel, dim3(tiles), dim3(256), 0, st, src_keys, src_pos, (int)n, 8 * i, flip, (const unsigned int*)hist, tiles, dst_keys,
+        hipLaunchKernelGGL(radix_move_kernel, dim3(tiles), dim3(256), 0, st, src_keys, src_pos, (int)n, 8 * i, flip, limit, (const unsigned int*)hist, tiles, dst_keys,
                            dst_pos);
         src_keys = dst_keys;
         src_pos = dst_pos;

@@ -250,6 +250,9 @@ DI unsigned dali_udiv(unsigned n, unsigned m, int s) { return (unsigned)(((unsig
 // on + 0*off when the index matches and on*0 + off otherwise, and both forms round to
 // the same T as the double evaluation (the products are exact zeros or NaN), so the
 // select below is bit-identical, including inf / NaN propagation.
+// index into an axis of n entries, held inside it: what a gather reads for an index outside its source
+DI int dali_clamp_index(int i, int n) { return i < 0 ? 0 : (i >= n ? n - 1 : i); }
+
 template <typename T>
 DI T dali_one_hot(int index, int column, T on, T off) {
     return index == column ? (T)(on + (T)0 * off) : (T)(on * (T)0 + off);

@@ -95,9 +95,12 @@ void emit_row_prologue(std::ostringstream& ss, const Program& P, const IvLayout&
                 ss << "  const long g_rs" << i << " = A.iv[" << L.stride_pos[i] << "], g_cs" << i << " = A.iv[" << L.stride_pos[i] + 1 << "];\n";
             else
                 ss << "  const long g_rs" << i << " = A.iv[" << L.size_pos[i] + 1 << "], g_cs" << i << " = 1;\n";
+            ss << "  const int g_n" << i << " = A.iv[" << L.size_pos[i] + 1 << "]; (void)g_n" << i << ";  // columns of the source: a pick outside them reads the nearest one\n";
         } else if (a.cls == Cls::FULL) {
             std::string rs = a.strided ? "(long)A.iv[" + std::to_string(L.stride_pos[i]) + "]" : "C";
-            std::string r = a.row_index >= 0 ? "(long)rl" + std::to_string(a.row_index) : std::string("row");
+            // a gathered source: the row comes from the index value, held inside the source (the reference reads out of bounds)
+            std::string r = a.row_index >= 0 ? "(long)dali_clamp_index(rl" + std::to_string(a.row_index) + ", A.iv[" + std::to_string(L.size_pos[i]) + "])"
+                                             : std::string("row");
             ss << "  " << (a.is_dest ? "" : "const ") << t << "* q" << i << " = (" << (a.is_dest ? "" : "const ") << t << "*)A.p[" << i << "] + " << r << " * " << rs << ";\n";
             if (a.strided) ss << "  const long cs" << i << " = A.iv[" << L.stride_pos[i] + 1 << "];\n";
         } else if (a.cls == Cls::ROW) {

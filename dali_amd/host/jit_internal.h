@@ -235,8 +235,8 @@ struct BodyEmitter {
                 const ArrayArg& a = P.arrays[n.array];
                 std::string t = ctype(n.dtype);
                 (void)a;
-                return "((const " + t + "*)A.p[" + std::to_string(n.array) + "])[row * g_rs" + std::to_string(n.array) + " + (long)(" +
-                       value(n.args[1]) + ") * g_cs" + std::to_string(n.array) + "]";
+                return "((const " + t + "*)A.p[" + std::to_string(n.array) + "])[row * g_rs" + std::to_string(n.array) + " + (long)dali_clamp_index(" +
+                       value(n.args[1]) + ", g_n" + std::to_string(n.array) + ") * g_cs" + std::to_string(n.array) + "]";
             }
             case Kind::GATHER:
                 return "x" + std::to_string(n.array) + leaf_suffix;

@@ -1347,6 +1347,59 @@ def test_scatter_rows_is_the_sequential_loop_bit_for_bit(gpu, D, O, rng, V, Dm, 
     assert np.array_equal(d2.numpy(), O.scatter_rows(dest, idx, np.float32(0.5), op=1))
 
 
+@pytest.mark.parametrize("V,N", [(1000, 300), (1000, 20000), (4096, 16384), (524288, 8192)])
+def test_indices_outside_the_destination_are_skipped(gpu, D, O, rng, V, N):
+    """An index outside [0, rows) updates nothing and disturbs nothing (the reference performs no check and would write out
+    of bounds): the rows named by valid indices get exactly what the sequential loop over the valid part gives them, on
+    the one-launch form (up to 16384 indices), on the ordered form behind the radix sort, and in the ordering itself, where
+    invalid keys must not split a run of equal valid keys (they come out behind all of them)."""
+    hip = gpu
+    Dm = 24
+    dest = rng.randn(V, Dm).astype(np.float32)
+    idx = rng.randint(0, V, N).astype(np.int32)
+    idx[: N // 4] = V - 1  # a long run of the largest valid row
+    bad = rng.choice(N, N // 5, replace=False)
+    idx[bad] = rng.choice(np.array([-1, -V, V, V + 5, V + (1 << 16) + 7, 2 ** 31 - 1, -2 ** 31], np.int64), bad.size).astype(np.int32)
+    rng.shuffle(idx)
+    vals = (rng.randn(N, Dm) * 3).astype(np.float32)
+    ok = (idx >= 0) & (idx < V)
+    want = O.scatter_rows(dest, idx[ok], vals[ok], op=1)
+    d = arr(D, dest)
+    d[arr(D, idx)].assign(arr(D, vals), 1)
+    assert np.array_equal(d.numpy(), want)
+    # the ordering by itself, through the C ABI
+    dk, ds, dp = _dev(hip, idx), _dev(hip, np.zeros(N, np.int32)), _dev(hip, np.zeros(N, np.int32))
+    assert hip.dali_hip_argsort_i32(dk, N, V, ds, dp) == 0, hip.dali_hip_last_error()
+    sk, pm = np.empty(N, np.int32), np.empty(N, np.int32)
+    hip.dali_hip_memcpy_d2h(sk.ctypes.data_as(C.c_void_p), ds, N * 4)
+    hip.dali_hip_memcpy_d2h(pm.ctypes.data_as(C.c_void_p), dp, N * 4)
+    assert np.array_equal(np.sort(pm), np.arange(N)) and np.array_equal(sk, idx[pm])
+    n_ok = int(ok.sum())
+    order = np.argsort(idx[ok], kind="stable")
+    assert np.array_equal(pm[:n_ok], np.flatnonzero(ok)[order])  # valid keys first, ordered, ties in input order
+    assert not ok[pm[n_ok:]].any()
+    for p in (dk, ds, dp):
+        hip.dali_hip_free(p)
+    # columns outside a row, through gather_from_rows
+    R = 500
+    m = rng.randn(R, 40).astype(np.float32)
+    cols = rng.randint(-3, 44, R).astype(np.int32)
+    dm = arr(D, m)
+    g = dm.gather_from_rows(arr(D, cols))
+    g += 1.0
+    okc = (cols >= 0) & (cols < 40)
+    wantm = m.copy()
+    wantm[np.flatnonzero(okc), cols[okc]] += 1.0
+    assert np.array_equal(dm.numpy(), wantm)
+    # reads through an index stay inside the source: an index outside it reads the nearest row / column
+    table = arr(D, dest)
+    some = idx[:257]
+    got = (D.op.gather(table, arr(D, some)) * 1.0).numpy()
+    assert np.array_equal(got, dest[np.clip(some.astype(np.int64), 0, V - 1)])
+    picked = arr(D, m).gather_from_rows(arr(D, cols)).numpy()
+    assert np.array_equal(picked, m[np.arange(R), np.clip(cols, 0, 39)])
+
+
 @pytest.mark.parametrize("R,Cn", [(6, 3), (300, 1000), (8192, 32000)])
 def test_scatter_to_rows_matches_oracle(gpu, D, O, rng, R, Cn):
     dest = rng.randn(R, Cn).astype(np.float32)
