@@ -94,7 +94,9 @@ __global__ __launch_bounds__(256) void rank_sort_kernel(const int32_t* keys, int
 // first", so every pass is stable and equal keys end up in input order: a thread holds eight pairs (one per round of 256),
 // a wave finds the lanes with its digit from eight ballots (one per bit), the lowest such lane records how many there
 // are per (round, wave, digit), and a scan over the 32 (round, wave) slots of every digit gives each group its offset.
-constexpr int kRadixTile = 2048;
+// A workgroup of 256 threads works on a tile of 256 * ROUNDS keys: 8 rounds for long inputs (fewest counters), fewer for
+// short ones so that the tiles still cover the chip (65536 keys in tiles of 2048 are 32 workgroups on 256 CUs).
+constexpr int kRadixMaxTile = 2048;
 
 // With a key limit, every key outside [0, limit) takes the digits of `limit` itself: such keys (invalid indices) end up behind all
 // valid ones, in input order, instead of between the keys that share their low bits.
@@ -104,13 +106,14 @@ __device__ __forceinline__ unsigned int radix_digit(int32_t key, int shift, unsi
     return (k >> shift) & 255u;
 }
 
+template <int ROUNDS>
 __global__ __launch_bounds__(256) void radix_hist_kernel(const int32_t* keys, int n, int shift, unsigned int flip, unsigned int limit, unsigned int* hist, int tiles) {
     __shared__ unsigned int h[256];
     h[threadIdx.x] = 0u;
     __syncthreads();
-    const long base = (long)blockIdx.x * kRadixTile;
+    const long base = (long)blockIdx.x * (256 * ROUNDS);
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
+    for (int r = 0; r < ROUNDS; ++r) {
         const long i = base + r * 256 + threadIdx.x;
         if (i < n) atomicAdd(&h[radix_digit(keys[i], shift, flip, limit)], 1u);
     }
@@ -118,46 +121,71 @@ __global__ __launch_bounds__(256) void radix_hist_kernel(const int32_t* keys, in
     hist[(long)threadIdx.x * tiles + blockIdx.x] = h[threadIdx.x];
 }
 
-// exclusive scan of `total` counters in place, by one workgroup: a thread sums a contiguous share, the shares are scanned
-// through the waves and LDS, and the thread walks its share again
-__global__ __launch_bounds__(1024) void radix_scan_kernel(unsigned int* hist, long total) {
-    __shared__ unsigned int wave_sum[16];
-    const long per = (total + 1023) / 1024, begin = (long)threadIdx.x * per, end = begin + per < total ? begin + per : total;
-    unsigned int mine = 0;
-    for (long i = begin; i < end; ++i) mine += hist[i];
-    unsigned int incl = mine;
+// The counters are laid out digit-major ([digit][tile]); a key's slot is (keys with smaller digits) + (keys of its digit in
+// earlier tiles) + (its rank within the tile). One workgroup per digit scans that digit's row of counters in place
+// (exclusive, coalesced, 256 at a time) and leaves the row's total; the move kernel adds the totals of the smaller digits.
+// (A single workgroup walking all 256 * tiles counters took 300 us for 1024 tiles, more than the rest of the sort.)
+__global__ __launch_bounds__(256) void radix_row_scan_kernel(unsigned int* hist, int tiles, unsigned int* totals) {
+    __shared__ unsigned int wave_sum[4];
+    unsigned int* row = hist + (long)blockIdx.x * tiles;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    unsigned int carry = 0;
+    for (int base = 0; base < tiles; base += 256) {
+        const int i = base + threadIdx.x;
+        const unsigned int v = i < tiles ? row[i] : 0u;
+        unsigned int incl = v;
 #pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const unsigned int o = __shfl_up(incl, d, 64);
-        if (lane >= d) incl += o;
+        for (int d = 1; d < 64; d <<= 1) {
+            const unsigned int o = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += o;
+        }
+        if (lane == 63) wave_sum[wave] = incl;
+        __syncthreads();
+        unsigned int before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            if (w < wave) before += wave_sum[w];
+            total += wave_sum[w];
+        }
+        if (i < tiles) row[i] = carry + before + incl - v;
+        carry += total;
+        __syncthreads();
     }
-    if (lane == 63) wave_sum[wave] = incl;
-    __syncthreads();
-    unsigned int before = 0;
-    for (int w = 0; w < wave; ++w) before += wave_sum[w];
-    unsigned int run = before + incl - mine;
-    for (long i = begin; i < end; ++i) {
-        const unsigned int c = hist[i];
-        hist[i] = run;
-        run += c;
-    }
+    if (threadIdx.x == 0) totals[blockIdx.x] = carry;
 }
 
+template <int ROUNDS>
 __global__ __launch_bounds__(256) void radix_move_kernel(const int32_t* keys_in, const int32_t* pos_in, int n, int shift, unsigned int flip, unsigned int limit, const unsigned int* hist,
-                                                         int tiles, int32_t* keys_out, int32_t* pos_out) {
-    __shared__ unsigned short cnt[32][256];
+                                                         const unsigned int* totals, int tiles, int32_t* keys_out, int32_t* pos_out) {
+    __shared__ unsigned short cnt[ROUNDS * 4][256];
     __shared__ unsigned int first_slot[256];
-    for (int t = threadIdx.x; t < 32 * 256; t += 256) (&cnt[0][0])[t] = 0;
-    first_slot[threadIdx.x] = hist[(long)threadIdx.x * tiles + blockIdx.x];
-    __syncthreads();
+    __shared__ unsigned int wave_total[4];
+    for (int t = threadIdx.x; t < ROUNDS * 4 * 256; t += 256) (&cnt[0][0])[t] = 0;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const unsigned long long below = (1ull << lane) - 1ull;
-    const long base = (long)blockIdx.x * kRadixTile;
-    int32_t key[8], pos[8];
-    unsigned int digit[8], rank[8];
+    {
+        // keys with smaller digits: exclusive scan of the 256 digit totals, thread d for digit d
+        const unsigned int mine = totals[threadIdx.x];
+        unsigned int incl = mine;
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
+        for (int d = 1; d < 64; d <<= 1) {
+            const unsigned int o = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += o;
+        }
+        if (lane == 63) wave_total[wave] = incl;
+        __syncthreads();
+        unsigned int before = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+            if (w < wave) before += wave_total[w];
+        first_slot[threadIdx.x] = before + incl - mine + hist[(long)threadIdx.x * tiles + blockIdx.x];
+    }
+    __syncthreads();
+    const unsigned long long below = (1ull << lane) - 1ull;
+    const long base = (long)blockIdx.x * (256 * ROUNDS);
+    int32_t key[ROUNDS], pos[ROUNDS];
+    unsigned int digit[ROUNDS], rank[ROUNDS];
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
         const long i = base + r * 256 + threadIdx.x;
         const bool valid = i < n;
         key[r] = valid ? keys_in[i] : 0;
@@ -175,8 +203,8 @@ __global__ __launch_bounds__(256) void radix_move_kernel(const int32_t* keys_in,
     __syncthreads();
     {
         unsigned int run = 0;
-#pragma unroll 8
-        for (int s = 0; s < 32; ++s) {
+#pragma unroll
+        for (int s = 0; s < ROUNDS * 4; ++s) {
             const unsigned int c = cnt[s][threadIdx.x];
             cnt[s][threadIdx.x] = (unsigned short)run;
             run += c;
@@ -184,7 +212,7 @@ __global__ __launch_bounds__(256) void radix_move_kernel(const int32_t* keys_in,
     }
     __syncthreads();
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
+    for (int r = 0; r < ROUNDS; ++r) {
         const long i = base + r * 256 + threadIdx.x;
         if (i < n) {
             const unsigned int dst = first_slot[digit[r]] + cnt[r * 4 + wave][digit[r]] + rank[r];
@@ -608,24 +636,35 @@ extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_
     // radix passes over the bits that can differ; arbitrary keys are ordered as signed numbers (the sign bit is flipped in
     // the digit). The pairs bounce between the caller's arrays and one temporary block so that the last pass lands in the
     // caller's.
-    const int passes = (end_bit + 7) / 8, tiles = (int)((n + kRadixTile - 1) / kRadixTile);
+    int rounds = kRadixMaxTile / 256;
+    while (rounds > 1 && n / (256 * rounds) < 1024) rounds /= 2;
+    const int passes = (end_bit + 7) / 8, tiles = (int)((n + 256 * rounds - 1) / (256 * rounds));
     const unsigned int flip = key_limit > 0 ? 0u : 0x80000000u, limit = key_limit > 0 ? (unsigned int)key_limit : 0u;
-    const size_t temp_bytes = ((size_t)2 * (size_t)n + (size_t)256 * (size_t)tiles) * sizeof(int32_t);
+    const size_t temp_bytes = ((size_t)2 * (size_t)n + (size_t)256 * (size_t)tiles + 256) * sizeof(int32_t);
     void* temp = nullptr;
     if (dali_hip_bank_allocate(&temp, temp_bytes)) return DALI_HIP_ERROR;
     int32_t* tkeys = (int32_t*)temp;
     int32_t* tpos = tkeys + n;
     unsigned int* hist = (unsigned int*)(tpos + n);
+    unsigned int* totals = hist + (size_t)256 * (size_t)tiles;
     const int32_t* src_keys = keys;
     const int32_t* src_pos = nullptr;  // first pass: a pair's position is its index
     for (int i = 0; i < passes; ++i) {
         const bool to_caller = (passes - 1 - i) % 2 == 0;
         int32_t* dst_keys = to_caller ? sorted_keys : tkeys;
         int32_t* dst_pos = to_caller ? perm : tpos;
-        hipLaunchKernelGGL(radix_hist_kernel, dim3(tiles), dim3(256), 0, st, src_keys, (int)n, 8 * i, flip, limit, hist, tiles);
-        hipLaunchKernelGGL(radix_scan_kernel, dim3(1), dim3(1024), 0, st, hist, (long)256 * tiles);
-        hipLaunchKernelGGL(radix_move_kernel, dim3(tiles), dim3(256), 0, st, src_keys, src_pos, (int)n, 8 * i, flip, limit, (const unsigned int*)hist, tiles, dst_keys,
-                           dst_pos);
+        auto pass = [&](auto hist_kernel, auto move_kernel) {
+            hipLaunchKernelGGL(hist_kernel, dim3(tiles), dim3(256), 0, st, src_keys, (int)n, 8 * i, flip, limit, hist, tiles);
+            hipLaunchKernelGGL(radix_row_scan_kernel, dim3(256), dim3(256), 0, st, hist, tiles, totals);
+            hipLaunchKernelGGL(move_kernel, dim3(tiles), dim3(256), 0, st, src_keys, src_pos, (int)n, 8 * i, flip, limit, (const unsigned int*)hist,
+                               (const unsigned int*)totals, tiles, dst_keys, dst_pos);
+        };
+        switch (rounds) {
+            case 1: pass(radix_hist_kernel<1>, radix_move_kernel<1>); break;
+            case 2: pass(radix_hist_kernel<2>, radix_move_kernel<2>); break;
+            case 4: pass(radix_hist_kernel<4>, radix_move_kernel<4>); break;
+            default: pass(radix_hist_kernel<8>, radix_move_kernel<8>); break;
+        }
         src_keys = dst_keys;
         src_pos = dst_pos;
     }

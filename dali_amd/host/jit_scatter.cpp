@@ -27,11 +27,16 @@ static std::string gen_scatter_rows_kernel(const Program& P, const IvLayout& L, 
     std::ostringstream ss;
     ss << device_prelude();
     ss << kargs_struct(P, L);
-    ss << "extern \"C\" __global__ __launch_bounds__(256) void " << kname << "(DALI_KERNEL_PARAMS) {\n  DALI_KERNEL_ARGS\n";
+    // One wave per sorted position, sixteen to a workgroup (a workgroup per position was launch-bound: 65536 positions of
+    // 4 KiB rows took 250 us). Only the wave at the head of a run of equal indices works: it reads the destination row once,
+    // applies the run's rows of values in input order and writes the row once.
+    ss << "extern \"C\" __global__ __launch_bounds__(1024) void " << kname << "(DALI_KERNEL_PARAMS) {\n  DALI_KERNEL_ARGS\n";
     ss << "  constexpr int VEC = " << VEC << ";\n";
     ss << "  const long N = A.iv[" << L.shape_pos[0] << "], D = A.iv[" << L.shape_pos[0] + 1 << "];\n";
     ss << "  const int* sk = (const int*)A.p[1];\n  const int* pm = (const int*)A.p[2];\n";
-    ss << "  const long p = blockIdx.x;\n  const int key = sk[p];\n";
+    ss << "  const int lane = threadIdx.x & 63;\n";
+    ss << "  const long p = (long)blockIdx.x * 16 + (long)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));\n  if (p >= N) return;\n";
+    ss << "  const int key = sk[p];\n";
     ss << "  if ((unsigned)key >= (unsigned)A.iv[" << L.shape_pos[0] + 2 << "]) return;  // no such destination row: skipped\n";
     ss << "  if (p > 0 && sk[p - 1] == key) return;  // only the head of a run of equal indices works\n";
     ss << "  long q_end = p + 1;\n  while (q_end < N && sk[q_end] == key) ++q_end;\n";
@@ -43,7 +48,7 @@ static std::string gen_scatter_rows_kernel(const Program& P, const IvLayout& L, 
         ss << "  const long vrs = A.iv[" << L.stride_pos[3] << "], vcs = A.iv[" << L.stride_pos[3] + 1 << "];\n";
         ss << "  const " << t << "* vals = (const " << t << "*)A.p[3];\n";
     }
-    ss << "  for (long c = (long)threadIdx.x * VEC; c < D; c += 256 * VEC) {\n";
+    ss << "  for (long c = (long)lane * VEC; c < D; c += 64 * VEC) {\n";
     if (VEC > 1) {
         ss << "    dali_vec<" << t << ", VEC> acc = dali_load<" << t << ", VEC>(drow + c);\n";
         ss << "    for (long q = p; q < q_end; ++q) {\n";
@@ -290,7 +295,7 @@ static void run_scatter_rows(const Array& dest2d, const Array& idx, OPERATOR_T o
     }
     const int VEC = vec ? 4 : 1;
     std::ostringstream sig;
-    sig << "scatter_rows_guarded|" << (int)dest2d.dtype() << "|" << (int)op << "|" << scalar_value << "|" << VEC;
+    sig << "scatter_rows_wave|" << (int)dest2d.dtype() << "|" << (int)op << "|" << scalar_value << "|" << VEC;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("scatter", sig.str(), "");
     std::shared_ptr<KernelSpec>& K = specs_cache[h];
@@ -302,11 +307,11 @@ static void run_scatter_rows(const Array& dest2d, const Array& idx, OPERATOR_T o
         K->kind = "scatter";
         K->name = kernel_name(K->kind, h);
         fill_plan_arrays(*K, P, shape_ndims);
-        K->plan.block_threads = 256;
-        K->plan.grid_kind = DALI_HIP_GRID_ROWS;  // one workgroup per sorted position
+        K->plan.block_threads = 1024;
+        K->plan.grid_kind = DALI_HIP_GRID_ROWS;  // one wave per sorted position, 16 to a workgroup
         K->plan.work_begin = L.shape_pos[0];
         K->plan.work_count = 1;
-        K->plan.work_per_block = 1;
+        K->plan.work_per_block = 16;
     }
     std::vector<std::vector<int>> shapes = {{N, D, V}};
     load_and_launch(*K, [&]() { return gen_scatter_rows_kernel(P, L, op, scalar_value, VEC, K->name); }, P, shapes);

@@ -283,7 +283,7 @@ int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidden, const f
  * the generated scatter kernel instead walks each destination row's contributions in input order,
  * the order of the reference's sequential CPU loop, so the result does not depend on scheduling.
  * Up to 16384 keys are ordered by one kernel that allocates nothing (it may be captured); longer inputs take a
- * least-significant-digit radix sort (eight bits per pass, three launches per pass) whose temporary block comes from
+ * least-significant-digit radix sort (eight bits per pass; histogram, per-digit scan and ranked move per pass) whose temporary block comes from
  * the bank, so they fail during a capture. With key_limit > 0, keys outside the promised range come out behind
  * every key inside it (among themselves in an unspecified but stable order) and never between two equal valid
  * keys; perm is a permutation for any input.
