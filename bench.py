@@ -337,6 +337,22 @@ def main():
             small["B%d" % Bs] = row
             del Xq, hs0, cs0, qrec
         configs["c5_lstm_step_256x1024x1024"]["sequence_of_32_small_batches"] = small
+        # one step at small batches (a decoder loop through the host): 16-row tiles with every compute unit on its own columns
+        # of the weights, beside the 64-row tiles of the general kernel
+        single = {}
+        for Bs in (1, 8, 32, 64):
+            xq, hq, cq = (D.Array.from_numpy(np.random.RandomState(s).randn(Bs, H).astype(np.float32)) for s in (29, 30, 31))
+            row = {}
+            for name, flag in (("small_batch_kernel_us", "1"), ("general_kernel_us", "0")):
+                os.environ["DALI_HIP_LSTM_SMALL"] = flag
+                with D.Recording() as qrec:
+                    op.lstm_step(xq, hq, cq, W, U, bias)
+                row[name] = round(time_recording(qrec, 100, 10), 2)
+            os.environ.pop("DALI_HIP_LSTM_SMALL", None)
+            row["weights_from_hbm_bound_us"] = round(2 * 1024 * 4096 * 4 / HBM_PEAK_GBS / 1e3, 2)
+            single["B%d" % Bs] = row
+            del xq, hq, cq, qrec
+        configs["c5_lstm_step_256x1024x1024"]["single_step_small_batches"] = single
         del X, Hp, Cp, W, U, bias, rec, grec, Xs, srec
 
         # the double-precision product (the reference's cublasDgemm branch)

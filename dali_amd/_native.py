@@ -91,6 +91,7 @@ HIP_SYMBOLS = {
     "dali_hip_sgemm_pair": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, C.c_float, H, _i, H, _i, H, _i, H, _i, C.c_float, H, _i]),
     "dali_hip_sgemm_terms": (_i, [_i, _i, _i, _i, _i, _ip, C.POINTER(H), _i, C.POINTER(H), _i, C.c_float, C.c_float, H, _i, _ip]),
     "dali_hip_lstm_step": (_i, [_i, _i, _i, H, _i, H, _i, H, H, _i, H, _i, H, H, H]),
+    "dali_hip_lstm_step_small": (_i, [_i, _i, _i, H, _i, H, _i, H, H, _i, H, _i, H, H, H]),
     "dali_hip_lstm_recurrent_persistent": (_i, [_i, _i, _i, H, H, _i, H, H, H, H]),
     "dali_hip_argsort_i32": (_i, [H, C.c_int64, C.c_int32, H, H]),
     "dali_hip_argsort_i32_noalloc": (_i, [H, C.c_int64, C.c_int32, H, H]),

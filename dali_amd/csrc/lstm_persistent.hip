@@ -14,8 +14,8 @@
 //      for all steps at once by one large product before this kernel runs,
 //   3. applies the gates for its hidden units (same arithmetic, operation by operation, as the fused single step:
 //      double-precision sigmoid, tanhf, no contraction) and writes its HU columns of h(t),
-//   4. meets the other workgroups at a barrier (a counter in global memory; release before, acquire after) so that
-//      h(t) is complete before anyone reads it.
+//   4. meets the other workgroups at a barrier (a counter in global memory) so that h(t) is complete before anyone
+//      reads it. h is written and read with device-coherent accesses, so the barrier needs no cache-wide fences.
 // The cell state of a workgroup's hidden units never leaves its registers.
 //
 // The barrier only works when every workgroup is resident, which holds because the grid has at most one workgroup per
@@ -217,6 +217,153 @@ __global__ __launch_bounds__(256) void lstm_persistent_kernel(PersistentArgs a) 
     }
 }
 
+// ------------------------------------------------------------------------------------------------ one step, small batch
+// A single step for a small batch (a decoder that feeds every output back through the host): the tiles of the general
+// product kernel are 64 rows high, so a step of 8 rows costs as much matrix-pipe time as one of 64 and only 64 workgroups
+// share the weights (37 us whatever the batch). What such a step has to do is stream W and U (32 MiB at I = H = 1024) once.
+// Workgroup (unit block, gate, k share) owns 64 consecutive columns of one gate, 256 bytes of every weight row, over a
+// 1 / KS share of the K range of x.W + h.U, the share split over its four waves. The weights go straight from memory into
+// the B operand of the matrix instruction: a lane loads four consecutive columns of row k with one 16-byte load and feeds
+// them to four instructions, whose 16-column tiles are therefore the columns congruent to 0, 1, 2 and 3 modulo 4 (a tile need
+// not be contiguous). Whole cache lines and few load instructions: a first version that gave every workgroup the four gates
+// of four hidden units read 16 bytes of each line, one value per lane and instruction, and took 14 to 32 us. The workgroups
+// of a unit block publish their partial pre-activations in the library workspace and take a ticket; the last of them adds
+// the k shares in order, then bias, gates and cell update as in the fused step.
+struct SmallStepArgs {
+    int B, I, H, KS;
+    const float* X;   // [B, I]
+    const float* Hp;  // [B, H]
+    const float* Cp;  // [B, H]
+    const float* W;   // [I, 4H]
+    const float* U;   // [H, 4H]
+    const float* bias;  // [4H]
+    float* Cout;      // [B, H]
+    float* Hout;      // [B, H]
+    int ldx, ldh, ldw, ldu;
+    unsigned int* tickets;  // one per unit block, zero at rest
+    float* partials;        // [unit blocks][4 gates][KS][B][64]
+};
+
+constexpr int kSmallUnits = 64;  // hidden units (columns of one gate) per workgroup
+constexpr int kSmallMaxShares = 8;  // k shares per unit block at most
+
+template <int MT, int G>
+__global__ __launch_bounds__(256) void lstm_step_small_kernel(SmallStepArgs a) {
+    extern __shared__ float red_flat[];  // [4 waves][4 column tiles][MT][16][16]
+    float (*red)[4][MT][16][16] = reinterpret_cast<float (*)[4][MT][16][16]>(red_flat);
+    __shared__ int is_last;
+    const int H = a.H, B = a.B, I = a.I, KS = a.KS;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int ks = blockIdx.x % KS, gate = (blockIdx.x / KS) & 3, ub = blockIdx.x / (4 * KS);
+    const int col0 = gate * H + ub * kSmallUnits;
+    const int arow = lane & 15, kgrp = lane >> 4;
+    const int KP = (I + H) / KS, KW = KP / 4;  // K range of the workgroup and of a wave (a multiple of 16)
+    const __amdgpu_buffer_rsrc_t xrows = __builtin_amdgcn_make_buffer_rsrc((void*)a.X, 0, ((B - 1) * a.ldx + I) * 4, 0x00027000);
+    const __amdgpu_buffer_rsrc_t hrows = __builtin_amdgcn_make_buffer_rsrc((void*)a.Hp, 0, ((B - 1) * a.ldh + H) * 4, 0x00027000);
+    f4 acc[4][MT];
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[ct][m] = (f4){0.f, 0.f, 0.f, 0.f};
+    for (int q0 = 0; q0 < KW / 16; q0 += G) {
+        f4 av[G][MT];
+        f4 bv[G][4];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int k0 = ks * KP + wave * KW + 16 * (q0 + g);  // wave-uniform; a trip of 16 lies wholly in x.W or in h.U
+            const bool valid = q0 + g < KW / 16;
+            const bool in_x = k0 < I;
+            const int kk = (in_x ? k0 : k0 - I) + 4 * kgrp;
+            const float* wp = (in_x ? a.W + (size_t)kk * a.ldw : a.U + (size_t)kk * a.ldu) + col0 + 4 * arow;
+            const size_t ldk = in_x ? a.ldw : a.ldu;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) bv[g][c] = valid ? *reinterpret_cast<const f4*>(wp + (size_t)c * ldk) : (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const int row = 16 * m + arow;
+                // rows past the batch lie beyond the buffer's range and read as zero
+                const int off = row < B && valid ? (row * (in_x ? a.ldx : a.ldh) + kk) * 4 : 0x7ffffff0;
+                av[g][m] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(in_x ? xrows : hrows, off, 0, 0));
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) acc[ct][m] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[g][m][c], bv[g][c][ct], acc[ct][m], 0, 0, 0);
+    }
+    // a lane holds column lane % 16 (of tile ct: column 4 * (lane % 16) + ct of the block) and rows 4 * (lane / 16) + v
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][ct][m][4 * kgrp + v][arow] = acc[ct][m][v];
+    __syncthreads();
+    // this workgroup's share of the pre-activations of (row b, unit u): the four waves in order
+    float* mine = a.partials + (((size_t)ub * 4 + gate) * KS + ks) * (size_t)B * kSmallUnits;
+    for (int e = tid; e < B * kSmallUnits; e += 256) {
+        const int bb = e / kSmallUnits, u = e % kSmallUnits;
+        float s = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) s += red[w][u & 3][bb / 16][bb & 15][u >> 2];
+        __hip_atomic_store(mine + e, s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned int ticket = __hip_atomic_fetch_add(a.tickets + ub, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = ticket == (unsigned int)(4 * KS - 1);
+    }
+    __syncthreads();
+    if (!is_last) return;
+    // The fold: a thread takes four neighbouring units of one row at a time; the 16-byte shares of all four gates are asked
+    // for (device-coherent loads) before the first is awaited, then added in k order. (Awaiting every 4-byte share in turn
+    // cost a memory round trip each: 90 us for 64 rows.)
+    const float* blockp = a.partials + (size_t)ub * 4 * KS * (size_t)B * kSmallUnits;
+    const __amdgpu_buffer_rsrc_t shares = __builtin_amdgcn_make_buffer_rsrc((void*)blockp, 0, 4 * KS * B * kSmallUnits * 4, 0x00027000);
+    for (int quad = tid; quad < B * (kSmallUnits / 4); quad += 256) {
+#pragma clang fp contract(off)
+        const int bb = quad / (kSmallUnits / 4), u = (quad % (kSmallUnits / 4)) * 4, unit = ub * kSmallUnits + u;
+        f4 pv[4][kSmallMaxShares];
+#pragma unroll
+        for (int gt = 0; gt < 4; ++gt)
+#pragma unroll
+            for (int k = 0; k < kSmallMaxShares; ++k)
+                pv[gt][k] = k < KS ? __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(shares, (((gt * KS + k) * B + bb) * kSmallUnits + u) * 4, 0, kCoherentLoad))
+                                   : (f4){0.f, 0.f, 0.f, 0.f};
+        const f4 cells = *reinterpret_cast<const f4*>(a.Cp + (size_t)bb * H + unit);
+        f4 cn4, hn4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float g4[4];
+#pragma unroll
+            for (int gt = 0; gt < 4; ++gt) {
+                float sum = 0.0f;
+#pragma unroll
+                for (int k = 0; k < kSmallMaxShares; ++k)
+                    if (k < KS) sum += pv[gt][k][j];
+                g4[gt] = sum + a.bias[gt * H + unit + j];
+            }
+            const float iv = (float)(1.0 / (1.0 + (double)seq_expf(-g4[0])));
+            const float fv = (float)(1.0 / (1.0 + (double)seq_expf(-g4[1])));
+            const float ov = (float)(1.0 / (1.0 + (double)seq_expf(-g4[2])));
+            const float gv = tanhf(g4[3]);
+            const float fc = fv * cells[j];
+            const float ig = iv * gv;
+            const float cn = fc + ig;
+            cn4[j] = cn;
+            hn4[j] = ov * tanhf(cn);
+        }
+        *reinterpret_cast<f4*>(a.Cout + (size_t)bb * H + unit) = cn4;
+        *reinterpret_cast<f4*>(a.Hout + (size_t)bb * H + unit) = hn4;
+    }
+    if (tid == 0) __hip_atomic_store(a.tickets + ub, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 static int* g_status = nullptr;  // pinned host word the kernel raises on a barrier time-out
 
 int persistent_status_take() {
@@ -281,5 +428,51 @@ extern "C" int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidd
 #undef DALI_PERSISTENT_CASE
     if (e == hipSuccess) e = hipGetLastError();
     if (e != hipSuccess) return fail("dali_hip_lstm_recurrent_persistent launch failed: %s", hipGetErrorString(e));
+    return DALI_HIP_OK;
+}
+
+extern "C" int dali_hip_lstm_step_small(int batch, int input, int hidden, const float* X, int ldx, const float* Hprev, int ldh, const float* Cprev,
+                                        const float* W, int ldw, const float* U, int ldu, const float* bias, float* Cout, float* Hout) {
+    if (ensure_init()) return DALI_HIP_ERROR;
+    if (batch < 1 || input < 1 || hidden < 1) return fail("dali_hip_lstm_step_small: batch, input and hidden must be positive");
+    if (!X || !Hprev || !Cprev || !W || !U || !bias || !Cout || !Hout) return fail("dali_hip_lstm_step_small: NULL argument");
+    if (batch > 64) return fail("dali_hip_lstm_step_small: batch %d exceeds 64 rows (use dali_hip_lstm_step)", batch);
+    if (hidden % 256 != 0 || hidden > 1024) return fail("dali_hip_lstm_step_small: hidden %d must be 256, 512, 768 or 1024", hidden);
+    // k shares per unit block: as many as bring the grid to about one workgroup per compute unit (256)
+    int KS = 4096 / hidden;
+    if (KS > kSmallMaxShares) KS = kSmallMaxShares;
+    if (KS < 1) KS = 1;
+    while (KS > 1 && (input + hidden) % (64 * KS) != 0) KS /= 2;
+    if (input % 16 != 0 || (input + hidden) % (64 * KS) != 0)
+        return fail("dali_hip_lstm_step_small: input %d must be a multiple of 16 and input + hidden of 64", input);
+    if (ldx < input || ldh < hidden || ldw < 4 * hidden || ldu < 4 * hidden) return fail("dali_hip_lstm_step_small: a leading dimension is smaller than its row");
+    if ((((uintptr_t)X | (uintptr_t)Hprev | (uintptr_t)W | (uintptr_t)U | (uintptr_t)Cprev | (uintptr_t)Cout | (uintptr_t)Hout) & 15) != 0 || ldx % 4 != 0 ||
+        ldh % 4 != 0 || ldw % 4 != 0 || ldu % 4 != 0)
+        return fail("dali_hip_lstm_step_small: the matrices must be 16-byte aligned with leading dimensions that are multiples of 4");
+    if ((size_t)batch * (size_t)(ldx > ldh ? ldx : ldh) * 4 >= 0x7ffffff0u) return fail("dali_hip_lstm_step_small: operand rows beyond the 2 GiB a buffer load addresses");
+    const int unit_blocks = hidden / kSmallUnits;
+    if ((size_t)unit_blocks * 4 * KS * batch * kSmallUnits * sizeof(float) > kWorkspacePartialBytes || unit_blocks > kWorkspaceCounters - 2)
+        return fail("dali_hip_lstm_step_small: partial sums exceed the workspace");
+    SmallStepArgs a;
+    a.B = batch; a.I = input; a.H = hidden; a.KS = KS;
+    a.X = X; a.Hp = Hprev; a.Cp = Cprev; a.W = W; a.U = U; a.bias = bias; a.Cout = Cout; a.Hout = Hout;
+    a.ldx = ldx; a.ldh = ldh; a.ldw = ldw; a.ldu = ldu;
+    a.tickets = (unsigned int*)workspace();
+    a.partials = (float*)(workspace() + kWorkspaceCounterBytes);
+    const int MT = (batch + 15) / 16, grid = unit_blocks * 4 * KS;
+    const size_t lds_bytes = (size_t)4 * 4 * MT * 256 * sizeof(float);
+    hipError_t e = hipSuccess;
+    auto launch = [&](auto kernel) {
+        e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e == hipSuccess) hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream(), a);
+    };
+    switch (MT) {
+        case 1: launch(lstm_step_small_kernel<1, 8>); break;
+        case 2: launch(lstm_step_small_kernel<2, 8>); break;
+        case 3: launch(lstm_step_small_kernel<3, 8>); break;
+        default: launch(lstm_step_small_kernel<4, 8>); break;
+    }
+    if (e == hipSuccess) e = hipGetLastError();
+    if (e != hipSuccess) return fail("dali_hip_lstm_step_small launch failed: %s", hipGetErrorString(e));
     return DALI_HIP_OK;
 }

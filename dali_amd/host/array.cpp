@@ -1597,6 +1597,16 @@ LSTMState lstm_step(const Array& x, const Array& h, const Array& c, const Array&
     const int Bn = x.shape()[0], In = x.shape()[1];
     auto dense = [](const Array& a) { return a.is_buffer() && a.contiguous_memory() && a.dtype() == DTYPE_FLOAT; };
     for (const Array* a : {&x, &h, &c, &W, &U, &b}) a->eval();
+    // up to 64 rows: the 64-row tiles of the general kernel would mostly multiply padding (37 us whatever the batch); 16-row
+    // tiles with every compute unit on its own columns of the weights
+    const char* small_env = getenv("DALI_HIP_LSTM_SMALL");
+    const bool small_off = small_env != nullptr && std::string(small_env) == "0";
+    if (!fused_off && !small_off && !dry_run() && Bn <= 64 && H % 256 == 0 && H <= 1024 && In % 16 == 0 && (In + H) % 64 == 0 && dense(x) && dense(h) &&
+        dense(c) && dense(W) && dense(U) && dense(b) && x.offset() % 4 == 0 && h.offset() % 4 == 0 && W.offset() % 4 == 0 && U.offset() % 4 == 0 && c.offset() % 4 == 0) {
+        Array c_new({Bn, H}, DTYPE_FLOAT), h_new({Bn, H}, DTYPE_FLOAT);
+        lstm_step_small(x, h, c, W, U, b, c_new, h_new);
+        return {c_new, h_new};
+    }
     if (!fused_off && !dry_run() && H % 64 == 0 && In == H && dense(x) && dense(h) && dense(c) && dense(W) && dense(U) && dense(b) &&
         x.offset() % 4 == 0 && h.offset() % 4 == 0 && W.offset() % 4 == 0 && U.offset() % 4 == 0) {
         Array c_new({Bn, H}, DTYPE_FLOAT), h_new({Bn, H}, DTYPE_FLOAT);

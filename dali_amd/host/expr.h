@@ -95,6 +95,8 @@ bool dry_run();
 // one fused launch for the LSTM cell step (records itself like any other launch)
 void lstm_step_fused(const Array& x, const Array& h, const Array& c, const Array& W, const Array& U, const Array& b, const Array& c_new,
                      const Array& h_new);
+void lstm_step_small(const Array& x, const Array& h, const Array& c, const Array& W, const Array& U, const Array& b, const Array& c_new,
+                     const Array& h_new);
 // the recurrent half of an LSTM over a whole sequence in one launch: pre [T, B, 4H] = x.W + bias for every step
 void lstm_recurrent_persistent(const Array& pre, const Array& U, const Array& h0, const Array& c0, const Array& hs, const Array& c_out);
 // stride-1 convolution of a dense float NHWC image [N,H,W,C] (C a multiple of 4) with filters [O,fh,fw,C], fh <= 8:

@@ -164,6 +164,32 @@ void lstm_step_fused(const Array& x, const Array& h, const Array& c, const Array
     }
 }
 
+// one step at a batch of up to 64 rows: 16-row tiles, one workgroup per compute unit (dali_hip_lstm_step_small)
+void lstm_step_small(const Array& x, const Array& h, const Array& c, const Array& W, const Array& U, const Array& b, const Array& c_new,
+                     const Array& h_new) {
+    const int Bn = x.shape()[0], In = x.shape()[1], H = h.shape()[1];
+    const float* xp = (const float*)x.device_ptr();
+    const float* hp = (const float*)h.device_ptr();
+    const float* cp = (const float*)c.device_ptr();
+    const float* wp = (const float*)W.device_ptr();
+    const float* up = (const float*)U.device_ptr();
+    const float* bp = (const float*)b.device_ptr();
+    float* co = (float*)c_new.device_ptr(memory::AM_OVERWRITE);
+    float* ho = (float*)h_new.device_ptr(memory::AM_OVERWRITE);
+    jit_stats().gemms_launched++;
+    jit_stats().last_kernel_kinds = "lstm_small";
+    check_hip(dali_hip_lstm_step_small(Bn, In, H, xp, In, hp, H, cp, wp, 4 * H, up, 4 * H, bp, co, ho), "small-batch lstm step");
+    if (g_recording) {
+        note_recorded_write(c_new.expression()->memory);
+        note_recorded_write(h_new.expression()->memory);
+        std::vector<Array> keep = {x, h, c, W, U, b, c_new, h_new};
+        g_recording->push_back([=]() {
+            (void)keep;
+            check_hip(dali_hip_lstm_step_small(Bn, In, H, xp, In, hp, H, cp, wp, 4 * H, up, 4 * H, bp, co, ho), "small-batch lstm step replay");
+        });
+    }
+}
+
 // the recurrent half of a whole sequence in one launch (records itself like any other launch)
 void lstm_recurrent_persistent(const Array& pre, const Array& U, const Array& h0, const Array& c0, const Array& hs, const Array& c_out) {
     const int T = hs.shape()[0], Bn = hs.shape()[1], H = hs.shape()[2];

@@ -257,6 +257,20 @@ int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx
                        float* Cout, float* Hout);
 
 /*
+ * The same step for batches of up to 64 rows (a decoder that feeds each output back through the host): 16-row tiles on
+ * the matrix cores and about one workgroup per compute unit, each streaming its own 64 columns of one gate of W and U over
+ * a share of the inner extent (whole cache lines, 16-byte loads straight into the matrix operand), instead of the 64-row
+ * tiles of dali_hip_lstm_step, whose time does not fall with the batch. Same arguments and gate arithmetic
+ * (dali/layers/lstm.cpp:226-261); the products are summed in another order, so results agree with dali_hip_lstm_step to
+ * rounding, not bit for bit. hidden must be 256, 512, 768 or 1024, input a multiple of 16 with input + hidden a multiple of
+ * 64; all matrices 16-byte aligned with leading dimensions that are multiples of 4. Partial sums and tickets live in
+ * the library workspace.
+ */
+int dali_hip_lstm_step_small(int batch, int input, int hidden, const float* X, int ldx, const float* Hprev, int ldh,
+                             const float* Cprev, const float* W, int ldw, const float* U, int ldu, const float* bias,
+                             float* Cout, float* Hout);
+
+/*
  * The recurrent half of an LSTM over a whole sequence in one launch, for batches of at most 64 rows: the loop of
  * dali/layers/lstm.cpp:294-303 (one cell activation per time step), whose hidden-to-hidden product the reference meant to
  * hand to a persistent kernel (third_party/nervana_kernels/sass/persistent_rnn_fprop.sass). pre [steps, batch, 4 hidden]

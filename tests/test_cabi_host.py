@@ -215,7 +215,7 @@ def test_gather_plans_as_an_indirect_row_leaf_and_checks_its_arguments(D, rng):
     assert g.shape == (10, 64) and not g.is_buffer()
     assert D.generate_only([D.op.tanh(g) * 2.0], compile=True) == 1  # one kernel: the map reads through the gather
     src = D.last_source()
-    assert "(long)rl" in src  # the source row pointer goes through the per-row index value
+    assert "dali_clamp_index(rl" in src  # the source row pointer goes through the per-row index value, held inside the source
     assert D.op.gather(table, D.Array.from_numpy(np.zeros((2, 3), np.int32))).shape == (2, 3, 64)
     with pytest.raises(RuntimeError, match="indices must be integers"):
         D.op.gather(table, D.Array.from_numpy(np.zeros(3, np.float32)))

@@ -1671,7 +1671,52 @@ def test_arange_diag_outer(gpu, D, rng):
         op.arange(5, 2)
 
 
-@pytest.mark.parametrize("B,H", [(64, 64), (256, 128), (100, 192), (7, 256), (256, 1024)])
+@pytest.mark.parametrize("B,I,H", [(1, 256, 256), (8, 1024, 1024), (17, 512, 512), (40, 768, 768), (64, 1024, 1024), (5, 256, 512), (33, 960, 1024)])
+def test_lstm_step_at_small_batches(gpu, D, O, rng, B, I, H):
+    """Up to 64 rows the step runs on 16-row tiles with one workgroup per compute unit (dali_hip_lstm_step_small) instead of
+    the 64-row tiles of the general kernel: same definition (lstm.cpp:226-261), the products summed in another order."""
+    import os
+    op = D.op
+    X, Hp, Cp = (rng.randn(B, n).astype(np.float32) for n in (I, H, H))
+    lim = np.sqrt(6.0 / (I + 4 * H))
+    W, U = (rng.uniform(-lim, lim, (n, 4 * H)).astype(np.float32) for n in (I, H))
+    b = (rng.randn(4 * H) * 0.1).astype(np.float32)
+    dev = [arr(D, v) for v in (X, Hp, Cp, W, U, b)]
+    before = D.jit_stats()
+    with D.Recording() as rec:
+        cn, hn = op.lstm_step(*dev)
+    after = D.jit_stats()
+    assert after["gemms"] - before["gemms"] == 1 and after["kernels"] == before["kernels"] and D.last_kernel_kinds() == "lstm_small"
+    _, ocn, ohn = O.lstm_step(X, Hp, Cp, W, U, b)
+    close(cn.numpy(), ocn, rtol=1e-4, atol=1e-5)
+    close(hn.numpy(), ohn, rtol=1e-4, atol=1e-5)
+    # against the general kernels of the library
+    os.environ["DALI_HIP_LSTM_SMALL"] = "0"
+    try:
+        c2, h2 = op.lstm_step(*dev)
+        assert D.last_kernel_kinds() != "lstm_small"
+    finally:
+        os.environ.pop("DALI_HIP_LSTM_SMALL")
+    close(cn.numpy(), c2.numpy(), rtol=2e-5, atol=2e-6)
+    close(hn.numpy(), h2.numpy(), rtol=2e-5, atol=2e-6)
+    first = (cn.numpy().copy(), hn.numpy().copy())
+    rec.replay(2)
+    assert np.array_equal(cn.numpy(), first[0]) and np.array_equal(hn.numpy(), first[1])
+    # through the C ABI with padded rows of X and Hprev
+    hip = gpu
+    Xp = np.zeros((B, I + 8), np.float32); Xp[:, :I] = X
+    Hpp = np.zeros((B, H + 4), np.float32); Hpp[:, :H] = Hp
+    ptrs = [_dev(hip, v) for v in (Xp, Hpp, Cp, W, U, b, np.zeros((B, H), np.float32), np.zeros((B, H), np.float32))]
+    assert hip.dali_hip_lstm_step_small(B, I, H, ptrs[0], I + 8, ptrs[1], H + 4, ptrs[2], ptrs[3], 4 * H, ptrs[4], 4 * H, ptrs[5], ptrs[6], ptrs[7]) == 0, hip.dali_hip_last_error()
+    out = np.empty((B, H), np.float32)
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), ptrs[7], out.nbytes)
+    assert np.array_equal(out, first[1])
+    assert hip.dali_hip_lstm_step_small(65, I, H, *ptrs[:2][:1], I + 8, ptrs[1], H + 4, ptrs[2], ptrs[3], 4 * H, ptrs[4], 4 * H, ptrs[5], ptrs[6], ptrs[7]) != 0
+    for p in ptrs:
+        hip.dali_hip_free(p)
+
+
+@pytest.mark.parametrize("B,H", [(64, 64), (256, 128), (100, 192), (7, 192), (256, 1024)])
 def test_fused_lstm_step_equals_the_two_launch_form(gpu, D, O, rng, B, H):
     """input == hidden, multiples of 64: the gate arithmetic runs in the GEMM epilogue (one launch) and must give
     what the GEMM pair followed by the generated gate kernel gives."""
