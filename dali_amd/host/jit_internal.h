@@ -358,6 +358,18 @@ struct GeomInts {
 extern LaunchCapture* g_capture;
 extern bool g_capture_compare_only;
 
+// Memo of a graph rewrite, keyed by node identity. It keeps every node it has seen alive: a rewrite may release nodes
+// (evaluating an operand in place replaces its node by a buffer), and a node created later at the address of a released
+// one would otherwise meet the released node's entry and be replaced by something unrelated.
+struct ExprMemo {
+    std::map<const Expr*, std::pair<std::shared_ptr<Expr>, Array>> entries;
+    const Array* find(const std::shared_ptr<Expr>& e) const {
+        auto it = entries.find(e.get());
+        return it == entries.end() ? nullptr : &it->second.second;
+    }
+    void put(const std::shared_ptr<Expr>& e, const Array& out) { entries[e.get()] = std::make_pair(e, out); }
+};
+
 
 // jit_launch.cpp
 uint64_t kernel_hash(const std::string& kind, const std::string& sig, const std::string& params);
@@ -416,7 +428,7 @@ void run_gemm(const Array& dst, const Expr* mm, const Expr* mm2, float beta);
 
 // jit_planner.cpp
 Array materialize(const Array& a);
-Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root);
+Array clean(const Array& a, ExprMemo& memo, bool is_root);
 void run_specs_planned(std::vector<DestSpec> specs);
 
 // jit_plan_cache.cpp

@@ -99,10 +99,9 @@ static Array expand_softmax(Array x, int axis) {
     return op::softmax_naive(x, axis);
 }
 
-Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root) {
+Array clean(const Array& a, ExprMemo& memo, bool is_root) {
     auto e = a.expression();
-    auto it = memo.find(e.get());
-    if (it != memo.end()) return it->second;
+    if (const Array* known = memo.find(e)) return *known;
     Array out = a;
     switch (e->kind) {
         case Kind::BUFFER:
@@ -213,7 +212,7 @@ Array clean(const Array& a, std::map<const Expr*, Array>& memo, bool is_root) {
             break;
         }
     }
-    memo[e.get()] = out;
+    memo.put(e, out);
     return out;
 }
 
@@ -244,11 +243,10 @@ static bool find_first_reduce(const Array& a, Array* found, std::set<const Expr*
     return false;
 }
 
-static Array substitute(const Array& a, const Expr* target, const Array& with, std::map<const Expr*, Array>& memo) {
+static Array substitute(const Array& a, const Expr* target, const Array& with, ExprMemo& memo) {
     auto e = a.expression();
     if (e.get() == target) return with;
-    auto it = memo.find(e.get());
-    if (it != memo.end()) return it->second;
+    if (const Array* known = memo.find(e)) return *known;
     std::vector<Array> args;
     bool changed = false;
     for (const Array& x : e->args) {
@@ -257,17 +255,16 @@ static Array substitute(const Array& a, const Expr* target, const Array& with, s
         args.push_back(c);
     }
     Array out = changed ? rebuild(e, args) : a;
-    memo[e.get()] = out;
+    memo.put(e, out);
     return out;
 }
 
 // Evaluating a node turns every handle on it into its buffer, so after an inner reduction has been evaluated the tree
 // holds unit axes inserted over a buffer: those become views of the buffer (what `rebuild` makes of them).
-static Array fold_expanded_buffers(const Array& a, std::map<const Expr*, Array>& memo) {
+static Array fold_expanded_buffers(const Array& a, ExprMemo& memo) {
     auto e = a.expression();
     if (e->kind == Kind::BUFFER || e->kind == Kind::SCALAR) return a;
-    auto it = memo.find(e.get());
-    if (it != memo.end()) return it->second;
+    if (const Array* known = memo.find(e)) return *known;
     std::vector<Array> args;
     bool changed = false;
     for (const Array& x : e->args) {
@@ -277,7 +274,7 @@ static Array fold_expanded_buffers(const Array& a, std::map<const Expr*, Array>&
     }
     if (e->kind == Kind::EXPAND_DIMS && args.size() == 1 && args[0].is_buffer()) changed = true;
     Array out = changed ? rebuild(e, args) : a;
-    memo[e.get()] = out;
+    memo.put(e, out);
     return out;
 }
 
@@ -373,7 +370,7 @@ void run_specs_planned(std::vector<DestSpec> specs) {
                 run_specs(plain);
                 for (auto& t : totals) {
                     for (auto& p : plain) {
-                        std::map<const Expr*, Array> memo;
+                        ExprMemo memo;
                         t.root = substitute(t.root, p.root.expression().get(), p.dest, memo);
                     }
                     run_specs({t});
@@ -386,7 +383,7 @@ void run_specs_planned(std::vector<DestSpec> specs) {
     }
     for (int iter = 0; iter < 64; ++iter) {
         if (iter > 0 && specs.size() == 1) {
-            std::map<const Expr*, Array> fold_memo;
+            ExprMemo fold_memo;
             specs[0].root = fold_expanded_buffers(specs[0].root, fold_memo);
         }
         bool has_all = has_kind(specs[0].root, [](Kind k) { return is_all_reduce(k); });
@@ -408,7 +405,7 @@ void run_specs_planned(std::vector<DestSpec> specs) {
                 Array buf({}, rr.dtype());
                 DestSpec ds{buf, OPERATOR_T_EQL, rr};
                 if (!try_all(ds)) throw std::runtime_error("internal: full reduction could not be planned");
-                std::map<const Expr*, Array> memo;
+                ExprMemo memo;
                 specs[0].root = substitute(specs[0].root, r.expression().get(), buf, memo);
             }
             continue;
@@ -448,7 +445,7 @@ void run_specs_planned(std::vector<DestSpec> specs) {
                 if (find(sp.root)) {
                     Array copy(found.shape(), found.dtype());
                     run_transpose_into(copy, found);
-                    std::map<const Expr*, Array> memo;
+                    ExprMemo memo;
                     sp.root = substitute(sp.root, found.expression().get(), copy, memo);
                     continue;
                 }
@@ -564,7 +561,7 @@ void run_specs_planned(std::vector<DestSpec> specs) {
                 scan(red_arg);
                 if (red_arg.ndim() >= 2 && numel_of(red_arg.shape()) > red_arg.shape().back() && has_layout && col_split_of(red_arg) >= 0) {
                     Array buf = materialize(inner);
-                    std::map<const Expr*, Array> memo;
+                    ExprMemo memo;
                     specs[0].root = substitute(specs[0].root, inner.expression().get(), buf, memo);
                     continue;
                 }
@@ -595,7 +592,7 @@ void run_specs_planned(std::vector<DestSpec> specs) {
             continue;
         }
         Array buf = materialize(inner);
-        std::map<const Expr*, Array> memo;
+        ExprMemo memo;
         specs[0].root = substitute(specs[0].root, inner.expression().get(), buf, memo);
     }
     throw std::runtime_error("planner did not converge");
@@ -611,7 +608,7 @@ void evaluate(const std::vector<Array>& roots) {
     jit_stats().last_kernel_names.clear();
     g_last_source.clear();
     std::vector<DestSpec> specs;
-    std::map<const Expr*, Array> memo;
+    ExprMemo memo;
     std::vector<Array> pending;
     for (const Array& r : roots) {
         auto e = r.expression();
@@ -649,7 +646,7 @@ void evaluate_into(const Array& dest, OPERATOR_T op, const Array& source) {
         DALI_ASSERT(numel_of(src.shape()) == 1 || numel_of(src.shape()) == numel_of(dest.shape()),
                     make_message("Cannot assign result of shape ", shape_str(src.shape()), " to a location of shape ", shape_str(dest.shape()), "."));
     }
-    std::map<const Expr*, Array> memo;
+    ExprMemo memo;
     auto se = src.expression();
     // dst (+)= dot(a, b): the GEMM writes (accumulates into) the destination directly
     if (se->kind == Kind::MATMUL && (dest.dtype() == DTYPE_FLOAT || dest.dtype() == DTYPE_DOUBLE) && se->dtype == dest.dtype() && dest.ndim() == 2 &&

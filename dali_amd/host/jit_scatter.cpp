@@ -392,7 +392,7 @@ void scatter_assign(const Array& dest, OPERATOR_T op, const Array& source) {
     if (de->kind == Kind::GATHER && !values.is_buffer()) {
         // the values stay an expression when the scan form of the scatter can evaluate them where they are used
         const int N = numel_of(idx.shape()), D = target.shape()[1];
-        std::map<const Expr*, Array> memo;
+        ExprMemo memo;
         Array lazy = clean(values, memo, true);
         const bool shaped = numel_of(lazy.shape()) == 1 || (lazy.ndim() == 2 && lazy.shape()[0] == N && lazy.shape()[1] == D);
         if (shaped && !lazy.is_buffer() && lazy.expression()->kind != Kind::SCALAR) {

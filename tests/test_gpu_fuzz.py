@@ -142,6 +142,47 @@ def test_random_expression_matches_numpy(gpu, D, seed):
         seed, shape, D.last_kernel_kinds(), err.max(), np.unravel_index(err.argmax(), err.shape), want.flat[err.argmax()])
 
 
+SOFTMAX_CASES = [((2, 65536), 1), ((3, 131072), 1), ((5, 65568), 1), ((2, 70001), 1), ((7, 262144), 1), ((300, 301), 0), ((129, 1000), 0),
+                 ((1024, 64), 0), ((64, 17), 0), ((4, 8, 4096), 1), ((12, 17, 400), 0), ((12, 17, 400), 1), ((4, 8, 4096), 2), ((2, 3, 5, 1024), 1),
+                 ((2, 3, 5, 1024), 2), ((70000,), 0), ((33, 2048), 1), ((2048, 33), 0)]
+
+
+@pytest.mark.parametrize("case", range(len(SOFTMAX_CASES) * 3))
+def test_random_softmax_over_any_axis(gpu, D, case):
+    """op::softmax over every axis of buffers, views and unevaluated expressions, alone and under a consumer: the shapes
+    reach the one-pass row kernel, the pieces of few long rows, the (maximum, sum) pair reducer along leading and middle
+    axes, and the plain expression where none of them applies. Checked against numpy in float64."""
+    shape, axis = SOFTMAX_CASES[case % len(SOFTMAX_CASES)]
+    variant = case // len(SOFTMAX_CASES)
+    rng = np.random.RandomState(7000 + case)
+    op = D.op
+    x = (rng.randn(*shape) * 2.0).astype(np.float32)
+    if variant == 0:
+        X, rx = arr(D, x), x.astype(np.float64)
+    elif variant == 1:
+        # an unevaluated expression over a reversed view
+        key = tuple(slice(None, None, -1) if d == len(shape) - 1 else slice(None) for d in range(len(shape)))
+        y = rng.uniform(0.5, 1.5, shape).astype(np.float32)
+        X, rx = arr(D, x)[key] * arr(D, y) + 0.25, x[key].astype(np.float64) * y + 0.25
+    else:
+        # transposed storage of the two leading axes (a view that is not contiguous)
+        if len(shape) >= 2:
+            perm = (1, 0) + tuple(range(2, len(shape)))
+            X, rx = arr(D, np.ascontiguousarray(x.transpose(perm))).transpose(perm), x.astype(np.float64)
+        else:
+            X, rx = arr(D, x), x.astype(np.float64)
+    e = np.exp(rx - rx.max(axis=axis, keepdims=True))
+    want = e / e.sum(axis=axis, keepdims=True)
+    got = op.softmax(X, axis).numpy().astype(np.float64)
+    assert got.shape == want.shape
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-12, err_msg="shape %s axis %d variant %d kinds %s" % (shape, axis, variant, D.last_kernel_kinds()))
+    np.testing.assert_allclose(got.sum(axis=axis), 1.0, rtol=0, atol=5e-6)
+    # under a consumer the softmax stays lazy and fuses where its shape allows
+    w = rng.uniform(0.5, 1.5, shape).astype(np.float32)
+    got2 = (op.softmax(X, axis) * arr(D, w) + 1.0).numpy().astype(np.float64)
+    np.testing.assert_allclose(got2, want * w + 1.0, rtol=2e-5, atol=1e-7)
+
+
 @pytest.mark.parametrize("seed", range(40))
 def test_random_assignment_into_views(gpu, D, seed):
     """dst (op)= expression with dst a whole buffer, a row/column slice or a transposed view."""
