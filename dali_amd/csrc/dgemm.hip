@@ -31,32 +31,46 @@ struct DgemmArgs {
     double alpha, beta;
 };
 
-__global__ __launch_bounds__(256) void dgemm_kernel(DgemmArgs a) {
-    __shared__ double As[2][BK][PITCH];
-    __shared__ double Bs[2][BK][PITCH];
+// CHECKED: the tile hangs over an edge of C or the last slab of K is short: every load is bounds-tested. Otherwise a
+// thread's loads are a wave-uniform slab pointer plus a constant 32-bit offset, with no vector arithmetic in the loop
+// (vector-ALU instructions between matrix instructions hold the matrix pipe back).
+template <bool CHECKED>
+__device__ __forceinline__ void dgemm_tile(const DgemmArgs& a, double (*As)[BK][PITCH], double (*Bs)[BK][PITCH], int m0, int n0) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int tiles_n = (a.N + BN - 1) / BN;
-    const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
-    const int m0 = tm * BM, n0 = tn * BN;
     // which element of a 64 x 16 tile a thread fetches in its c-th load (c = 0..3): along k when k is the unit stride,
     // along the rows otherwise
     const bool a_k_fast = a.ak == 1, b_k_fast = a.bk == 1;
     int ar[4], akk[4], bc[4], bkk[4];
+    int aoff[4], boff[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         ar[c] = a_k_fast ? tid / 16 + 16 * c : tid % 64;
         akk[c] = a_k_fast ? tid % 16 : tid / 64 + 4 * c;
         bc[c] = b_k_fast ? tid / 16 + 16 * c : tid % 64;
         bkk[c] = b_k_fast ? tid % 16 : tid / 64 + 4 * c;
+        aoff[c] = CHECKED ? 0 : (int)((long)ar[c] * a.ai + (long)akk[c] * a.ak);
+        boff[c] = CHECKED ? 0 : (int)((long)bkk[c] * a.bk + (long)bc[c] * a.bj);
     }
+    const double* Atile = a.A + (long)m0 * a.ai;
+    const double* Btile = a.B + (long)n0 * a.bj;
     double ra[4], rb[4];
     auto fetch = [&](int k0) {
+        if (CHECKED) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int i = m0 + ar[c], k = k0 + akk[c];
-            ra[c] = (i < a.M && k < a.K) ? a.A[(long)i * a.ai + (long)k * a.ak] : 0.0;
-            const int j = n0 + bc[c], kb = k0 + bkk[c];
-            rb[c] = (j < a.N && kb < a.K) ? a.B[(long)kb * a.bk + (long)j * a.bj] : 0.0;
+            for (int c = 0; c < 4; ++c) {
+                const int i = m0 + ar[c], k = k0 + akk[c];
+                ra[c] = (i < a.M && k < a.K) ? a.A[(long)i * a.ai + (long)k * a.ak] : 0.0;
+                const int j = n0 + bc[c], kb = k0 + bkk[c];
+                rb[c] = (j < a.N && kb < a.K) ? a.B[(long)kb * a.bk + (long)j * a.bj] : 0.0;
+            }
+        } else {
+            const double* As0 = Atile + (long)k0 * a.ak;  // wave-uniform
+            const double* Bs0 = Btile + (long)k0 * a.bk;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                ra[c] = As0[aoff[c]];
+                rb[c] = Bs0[boff[c]];
+            }
         }
     };
     auto stage = [&](int buf) {
@@ -103,12 +117,23 @@ __global__ __launch_bounds__(256) void dgemm_kernel(DgemmArgs a) {
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int row = m0 + wm + 16 * i + 4 * v + kg, col = n0 + wn + 16 * j + r;
-                if (row < a.M && col < a.N) {
+                if (!CHECKED || (row < a.M && col < a.N)) {
                     double* p = a.C + (long)row * a.ldc + col;
                     const double prod = a.alpha * acc[i][j][v];
                     *p = a.beta == 0.0 ? prod : prod + a.beta * *p;
                 }
             }
+}
+
+__global__ __launch_bounds__(256) void dgemm_kernel(DgemmArgs a, int offsets_fit) {
+    __shared__ double As[2][BK][PITCH];
+    __shared__ double Bs[2][BK][PITCH];
+    const int tiles_n = (a.N + BN - 1) / BN;
+    const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const bool interior = offsets_fit && m0 + BM <= a.M && n0 + BN <= a.N && a.K % BK == 0 && a.K > 0;  // workgroup-uniform
+    if (interior) dgemm_tile<false>(a, As, Bs, m0, n0);
+    else dgemm_tile<true>(a, As, Bs, m0, n0);
 }
 
 }  // namespace
@@ -136,7 +161,11 @@ extern "C" int dali_hip_dgemm(int transB, int transA, int m, int n, int k, doubl
     a.C = C; a.ldc = ldc; a.alpha = alpha; a.beta = beta;
     const long tiles = (long)((rows + BM - 1) / BM) * ((cols + BN - 1) / BN);
     if (tiles > 0x7fffffffL) return fail("dali_hip_dgemm: too many tiles");
-    hipLaunchKernelGGL(dgemm_kernel, dim3((unsigned)tiles), dim3(256), 0, stream(), a);
+    // a thread's offset inside a 64 x 16 operand tile as a 32-bit number of elements
+    const long span_a = 63 * (a.ai > 0 ? a.ai : -a.ai) + 15 * (a.ak > 0 ? a.ak : -a.ak);
+    const long span_b = 15 * (a.bk > 0 ? a.bk : -a.bk) + 63 * (a.bj > 0 ? a.bj : -a.bj);
+    const int offsets_fit = span_a < (1L << 28) && span_b < (1L << 28);
+    hipLaunchKernelGGL(dgemm_kernel, dim3((unsigned)tiles), dim3(256), 0, stream(), a, offsets_fit);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("dali_hip_dgemm launch failed: %s", hipGetErrorString(e));
     return DALI_HIP_OK;
