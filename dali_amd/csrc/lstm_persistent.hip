@@ -415,7 +415,13 @@ extern "C" int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidd
     a.spin_limit = spin_env;
     hipError_t e = hipSuccess;
     auto launch = [&](auto kernel) {
-        e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        // once per kernel (its LDS need is fixed by the template arguments): later calls, which may be recorded into a graph,
+        // are launches only
+        static bool attribute_set = false;
+        if (!attribute_set) {
+            e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            attribute_set = e == hipSuccess;
+        }
         if (e == hipSuccess) hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream(), a);
     };
     const int KQ = hidden / 64;
@@ -463,7 +469,13 @@ extern "C" int dali_hip_lstm_step_small(int batch, int input, int hidden, const 
     const size_t lds_bytes = (size_t)4 * 4 * MT * 256 * sizeof(float);
     hipError_t e = hipSuccess;
     auto launch = [&](auto kernel) {
-        e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        // once per kernel (its LDS need is fixed by the template arguments): later calls, which may be recorded into a graph,
+        // are launches only
+        static bool attribute_set = false;
+        if (!attribute_set) {
+            e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            attribute_set = e == hipSuccess;
+        }
         if (e == hipSuccess) hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream(), a);
     };
     switch (MT) {

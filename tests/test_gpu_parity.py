@@ -1702,6 +1702,11 @@ def test_lstm_step_at_small_batches(gpu, D, O, rng, B, I, H):
     first = (cn.numpy().copy(), hn.numpy().copy())
     rec.replay(2)
     assert np.array_equal(cn.numpy(), first[0]) and np.array_equal(hn.numpy(), first[1])
+    # as a HIP graph: the launch allocates nothing and its tickets are back at rest after every replay
+    rec.make_graph()
+    for _ in range(3):
+        rec.replay(1)
+        assert np.array_equal(cn.numpy(), first[0]) and np.array_equal(hn.numpy(), first[1])
     # through the C ABI with padded rows of X and Hprev
     hip = gpu
     Xp = np.zeros((B, I + 8), np.float32); Xp[:, :I] = X
@@ -1801,6 +1806,11 @@ def test_lstm_sequence_in_one_persistent_launch(gpu, D, O, rng, T, B, H):
     first, first_c = hs.numpy().copy(), c_last.numpy().copy()
     rec.replay(2)
     assert np.array_equal(hs.numpy(), first) and np.array_equal(c_last.numpy(), first_c)
+    # also as a HIP graph, replayed with eager work in between
+    rec.make_graph()
+    for _ in range(2):
+        rec.replay(1)
+        assert np.array_equal(hs.numpy(), first) and np.array_equal(c_last.numpy(), first_c)
     # a reduction right behind it finds its own tickets at zero
     close(D.op.sum(hs).numpy(), first.astype(np.float64).sum(), rtol=1e-5, atol=1e-5 * np.abs(first).sum())
 
