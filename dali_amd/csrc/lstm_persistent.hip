@@ -16,6 +16,8 @@
 //      double-precision sigmoid, tanhf, no contraction) and writes its HU columns of h(t),
 //   4. meets the other workgroups at a barrier (a counter in global memory) so that h(t) is complete before anyone
 //      reads it. h is written and read with device-coherent accesses, so the barrier needs no cache-wide fences.
+//      Up to 32 rows the barrier is replaced by waiting on the values of h(t-1) themselves (DATA_FLAGS below): a barrier
+//      costs three dependent round trips through memory (4 us), a value that is polled one.
 // The cell state of a workgroup's hidden units never leaves its registers.
 //
 // The barrier only works when every workgroup is resident, which holds because the grid has at most one workgroup per
@@ -58,9 +60,28 @@ constexpr int kPitchPad = 4;  // LDS row pitch of the U slice = 4 * HU + 4 float
 
 typedef float f4 __attribute__((ext_vector_type(4)));
 constexpr int kCoherentLoad = 16;  // cache policy of a buffer load: device scope (the sc1 bit)
+// the same, marked volatile for the compiler: a load that is repeated until its value changes is not to be merged with
+// its earlier instances
+constexpr int kPollLoad = (int)(0x80000000u | 16u);
 
-// MT: 16-row tiles of the batch (B <= 16 * MT); KQ = H / 64: trips of 16 values of k in a wave's quarter of the K range
-template <int MT, int KQ>
+constexpr unsigned int kNotYet = 0xFFFFFFFFu;    // bit pattern that stands for "h not written yet" (a NaN no arithmetic here produces)
+constexpr unsigned int kQuietNaN = 0x7FC00000u;
+
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+// The pattern is the largest unsigned value: one of four words holds it exactly when their maximum does. (The words are
+// taken from the whole vector cast to integers: __builtin_bit_cast applied to one element of a float vector, v[i], reads
+// element 0 whatever i is with this compiler.)
+__device__ __forceinline__ bool any_not_yet(f4 v) {
+    const u4 w = __builtin_bit_cast(u4, v);
+    const unsigned int hi = max(max(w[0], w[1]), max(w[2], w[3]));
+    return hi == kNotYet;
+}
+
+// MT: 16-row tiles of the batch (B <= 16 * MT); KQ = H / 64: trips of 16 values of k in a wave's quarter of the K range.
+// DATA_FLAGS: instead of a grid barrier per step, the rows of hs that the kernel will read are first filled with a bit
+// pattern that means "not written yet" (one barrier, once), and a wave polls the values of h(t-1) it needs until none of
+// them shows that pattern: a step then costs one memory round trip after the producers' stores instead of three.
+template <int MT, int KQ, bool DATA_FLAGS>
 __global__ __launch_bounds__(256) void lstm_persistent_kernel(PersistentArgs a) {
     extern __shared__ float lds[];
     const int H = a.H, HU = a.HU, NC = 4 * HU, P = NC + kPitchPad, B = a.B;
@@ -73,6 +94,19 @@ __global__ __launch_bounds__(256) void lstm_persistent_kernel(PersistentArgs a) 
     const int parts = (gridDim.x & 7) == 0 ? 8 : 1;
     const int slice = (blockIdx.x % parts) * (gridDim.x / parts) + blockIdx.x / parts;
     const int u0 = slice * HU;
+    // the (row, hidden unit) pair this thread finishes every step
+    const int pb = tid / HU, puu = tid - pb * HU;
+    const bool owner = tid < B * HU;
+    if (DATA_FLAGS) {
+        // this workgroup's part of the rows of hs that will be read gets the "not written yet" pattern; the arrival is
+        // counted now and awaited after the slice of U is in LDS, so the round trips of the one barrier hide behind that load
+        if (owner)
+            for (int t = 0; t + 1 < a.T; ++t)
+                __hip_atomic_store(reinterpret_cast<unsigned int*>(a.hs) + ((size_t)t * B + pb) * H + u0 + puu, kNotYet, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) __hip_atomic_fetch_add(a.bar, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     // this workgroup's slice of U: local column j = gate * HU + uu  <->  U column gate * H + u0 + uu
     if (HU == 4 && (a.ldu & 3) == 0 && ((uintptr_t)a.U & 15) == 0) {
         // one 16-byte load per (k, gate), eight in flight per thread
@@ -105,9 +139,6 @@ __global__ __launch_bounds__(256) void lstm_persistent_kernel(PersistentArgs a) 
         }
     }
     if (tid == 0) give_up = 0;
-    // the (row, hidden unit) pair this thread finishes every step, and its cell value
-    const int pb = tid / HU, puu = tid - pb * HU;
-    const bool owner = tid < B * HU;
     float cell = owner ? a.c0[(size_t)pb * H + u0 + puu] : 0.0f;
     __syncthreads();
 
@@ -125,7 +156,25 @@ __global__ __launch_bounds__(256) void lstm_persistent_kernel(PersistentArgs a) 
         }
     };
     fetch_pre(0);
-    for (int t = 0; t < a.T; ++t) {
+    // bounded wait of thread 0 on the barrier counter; false when it (or another workgroup) gave up
+    auto wait_for = [&](unsigned int target) {
+        unsigned int polls = 0;
+        while (__hip_atomic_load(a.bar, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+            __builtin_amdgcn_s_sleep(1);
+            if ((++polls & 63u) == 0u && __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) return false;
+            if (polls >= a.spin_limit) {
+                __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                return false;
+            }
+        }
+        return true;
+    };
+    if (DATA_FLAGS) {
+        // every workgroup's pattern has reached memory before anybody's first h does
+        if (tid == 0 && !wait_for(gridDim.x)) give_up = 1;
+        __syncthreads();
+    }
+    for (int t = 0; t < a.T && !give_up; ++t) {
         const float* hp = t == 0 ? a.h0 : a.hs + (size_t)(t - 1) * B * H;
         // rows past the batch are out of the buffer's range and read as zero
         const __amdgpu_buffer_rsrc_t hrow = __builtin_amdgcn_make_buffer_rsrc((void*)hp, 0, B * H * 4, 0x00027000);
@@ -137,12 +186,59 @@ __global__ __launch_bounds__(256) void lstm_persistent_kernel(PersistentArgs a) 
         // instruction does not matter to the sum. Every load of the step is issued before the first product: the step pays
         // the latency of h(t-1) once.
         f4 av[KQ][MT];
+        auto load_tile = [&](int m) {
 #pragma unroll
-        for (int q = 0; q < KQ; ++q) {
-            const int kb = wave * KW + 16 * q + 4 * kgrp;
+            for (int q = 0; q < KQ; ++q) {
+                const int kb = wave * KW + 16 * q + 4 * kgrp;
+                av[q][m] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(hrow, ((16 * m + arow) * H + kb) * 4, 0, DATA_FLAGS ? kPollLoad : kCoherentLoad));
+            }
+        };
+        if (!DATA_FLAGS || t == 0) {
 #pragma unroll
-            for (int m = 0; m < MT; ++m)
-                av[q][m] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(hrow, ((16 * m + arow) * H + kb) * 4, 0, kCoherentLoad));
+            for (int m = 0; m < MT; ++m) load_tile(m);
+        } else {
+            // every tile is fetched, and a tile in which a lane of this wave still sees the "not written yet" pattern (rows
+            // past the batch read as zero) is fetched again until none does
+            unsigned int polls = 0;
+            bool need[MT];
+#pragma unroll
+            for (int m = 0; m < MT; ++m) need[m] = true;
+            // The waiting is done on one load per lane: a wave that fetched all its tiles again and again would multiply the
+            // traffic of the step (at 64 rows every workgroup reads 256 KiB of h) and slow the producers it waits for.
+            while (polls < a.spin_limit) {
+                const int kb = wave * KW + 4 * kgrp;
+                const f4 probe = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(hrow, (arow * H + kb) * 4, 0, kPollLoad));
+                if (!__any(any_not_yet(probe))) break;
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_sleep(1);
+                ++polls;
+                if ((polls & 15u) == 0u && __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) break;
+            }
+            while (true) {
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+                    if (need[m]) load_tile(m);
+                bool again = false;
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+                    if (need[m]) {
+                        bool missing = false;
+#pragma unroll
+                        for (int q = 0; q < KQ; ++q) missing = missing || any_not_yet(av[q][m]);
+                        need[m] = __any(missing);  // the same for every lane
+                        again = again || need[m];
+                    }
+                if (!again) break;
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_sleep(1);
+                ++polls;
+                const bool others = (polls & 15u) == 0u && __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0;
+                if (others || polls >= a.spin_limit) {
+                    if (!others) __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    give_up = 1;  // (every wave that gives up writes the same value; read behind the next barrier)
+                    break;
+                }
+            }
         }
 #pragma unroll
         for (int q = 0; q < KQ; ++q) {
@@ -160,6 +256,7 @@ __global__ __launch_bounds__(256) void lstm_persistent_kernel(PersistentArgs a) 
 #pragma unroll
             for (int v = 0; v < 4; ++v) red[((size_t)(wave * MT + m) * 16 + 4 * kgrp + v) * 16 + arow] = acc[m][v];
         __syncthreads();
+        if (give_up) break;  // a wave stopped waiting for h(t-1): the sums are meaningless
         if (owner) {
 #pragma clang fp contract(off)
             float g4[4];
@@ -178,32 +275,23 @@ __global__ __launch_bounds__(256) void lstm_persistent_kernel(PersistentArgs a) 
             const float fc = fv * cell;
             const float ig = iv * gv;
             cell = fc + ig;
-            __hip_atomic_store(a.hs + ((size_t)t * B + pb) * H + u0 + puu, ov * tanhf(cell), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            float hv = ov * tanhf(cell);
+            if (DATA_FLAGS && __builtin_bit_cast(unsigned int, hv) == kNotYet) hv = __builtin_bit_cast(float, kQuietNaN);
+            __hip_atomic_store(a.hs + ((size_t)t * B + pb) * H + u0 + puu, hv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         if (t + 1 == a.T) break;
+        if (DATA_FLAGS) {
+            fetch_pre(t + 1);
+            __syncthreads();  // the fold area is free again
+            continue;
+        }
         // grid barrier: everybody's columns of h(t) have reached device memory before anybody reads row t
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();  // (also: the fold area is free again)
         if (tid == 0) __hip_atomic_fetch_add(a.bar, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         fetch_pre(t + 1);  // does not depend on h: in flight during the wait
-        if (tid == 0) {
-            const unsigned int target = gridDim.x * (unsigned int)(t + 1);
-            unsigned int polls = 0;
-            while (__hip_atomic_load(a.bar, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-                __builtin_amdgcn_s_sleep(1);
-                if ((++polls & 63u) == 0u && __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) {
-                    give_up = 1;  // somebody else gave up
-                    break;
-                }
-                if (polls >= a.spin_limit) {
-                    __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                    give_up = 1;
-                    break;
-                }
-            }
-        }
+        if (tid == 0 && !wait_for(gridDim.x * (unsigned int)(t + 1))) give_up = 1;
         __syncthreads();
-        if (give_up) break;
     }
     if (owner) a.c_out[(size_t)pb * H + u0 + puu] = cell;
     // the counters go back to zero once every workgroup is past its last wait
@@ -425,8 +513,16 @@ extern "C" int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidd
         if (e == hipSuccess) hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream(), a);
     };
     const int KQ = hidden / 64;
-#define DALI_PERSISTENT_CASE(mt, kq) \
-    if (MT == mt && KQ == kq) launch(lstm_persistent_kernel<mt, kq>);
+    // Waiting on the values themselves beats the barrier up to 32 rows (3.7 / 4.9 / 8.8 us a step at 1 / 8 / 32 rows of
+    // 1024 units against 6.6 / 7.5 / 10.3); from 33 rows on the tiles that have to be fetched a second time cost more than
+    // the barrier (12.8 against 11.3 us at 33 rows, 17.4 against 13.6 at 64). DALI_HIP_PERSISTENT_DATA_FLAGS=0: always barriers.
+    static const bool flags_allowed = !(getenv("DALI_HIP_PERSISTENT_DATA_FLAGS") && atoi(getenv("DALI_HIP_PERSISTENT_DATA_FLAGS")) == 0);
+    const bool data_flags = flags_allowed && MT <= 2;
+#define DALI_PERSISTENT_CASE(mt, kq)                                              \
+    if (MT == mt && KQ == kq) {                                                   \
+        if (data_flags) launch(lstm_persistent_kernel<mt, kq, (mt <= 2)>);        \
+        else launch(lstm_persistent_kernel<mt, kq, false>);                       \
+    }
     DALI_PERSISTENT_CASE(1, 4) DALI_PERSISTENT_CASE(2, 4) DALI_PERSISTENT_CASE(3, 4) DALI_PERSISTENT_CASE(4, 4)
     DALI_PERSISTENT_CASE(1, 8) DALI_PERSISTENT_CASE(2, 8) DALI_PERSISTENT_CASE(3, 8) DALI_PERSISTENT_CASE(4, 8)
     DALI_PERSISTENT_CASE(1, 12) DALI_PERSISTENT_CASE(2, 12) DALI_PERSISTENT_CASE(3, 12) DALI_PERSISTENT_CASE(4, 12)

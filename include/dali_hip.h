@@ -277,7 +277,9 @@ int dali_hip_lstm_step_small(int batch, int input, int hidden, const float* X, i
  * holds the input half of the pre-activations for every step, x(t).W + bias, gates packed i, f, o, g along the columns (one
  * large product computed beforehand); U [hidden, 4 hidden] (row stride ldu) stays in the LDS of the compute units for the
  * whole sequence; per step every workgroup forms h(t-1).U for the gate columns of its hidden units, finishes the cell
- * (same arithmetic as dali_hip_lstm_step) and meets the others at a grid barrier. hs [steps, batch, hidden] receives every
+ * (same arithmetic as dali_hip_lstm_step) and meets the others at a grid barrier (up to 32 rows: waits until the values of
+ * h(t-1) it needs have replaced a "not written yet" bit pattern that the launch first writes into hs, so hs must not be
+ * read by anybody else while the launch runs). hs [steps, batch, hidden] receives every
  * hidden state, c_out [batch, hidden] the last cell state. hidden must be a multiple of 64 whose slice of U per compute
  * unit fits the LDS (hidden = 1024 on 256 compute units: 80 KiB); h0 and hs 16-byte aligned. The grid has at most one
  * workgroup per compute unit, so all are resident; a workgroup that still does not see the others arrive within 2^20 polls

@@ -1778,12 +1778,14 @@ def test_lstm_sequence_is_the_step_applied_in_turn(gpu, D, O, rng, T, B, I, H):
     assert np.array_equal(hs.numpy(), first)
 
 
-@pytest.mark.parametrize("T,B,H", [(2, 1, 256), (5, 8, 256), (4, 17, 512), (3, 40, 768), (3, 64, 1024), (33, 8, 1024)])
+@pytest.mark.parametrize("T,B,H", [(2, 1, 256), (5, 8, 256), (4, 17, 512), (3, 40, 768), (3, 64, 1024), (33, 8, 1024), (6, 32, 1024), (70, 2, 512),
+                                   (9, 33, 256)])
 def test_lstm_sequence_in_one_persistent_launch(gpu, D, O, rng, T, B, H):
     """Small batches: the input half of every step's pre-activations is one product, the recurrent half one launch that
-    keeps U in the LDS of the compute units and steps through the sequence behind grid barriers (the role of the
-    reference's persistent_rnn_fprop kernel for the loop of dali/layers/lstm.cpp:294-303). Same values as the step applied
-    in turn, to the tolerance of a product summed in another order."""
+    keeps U in the LDS of the compute units and steps through the sequence, waiting for the values of h(t-1) themselves
+    up to 32 rows and behind grid barriers above (the role of the reference's persistent_rnn_fprop kernel for the loop of
+    dali/layers/lstm.cpp:294-303). Same values as the step applied in turn, to the tolerance of a product summed in another
+    order."""
     Xs = rng.randn(T, B, H).astype(np.float32)
     H0, C0 = (rng.randn(B, H).astype(np.float32) for _ in range(2))
     lim = np.sqrt(6.0 / (H + 4 * H))
@@ -1815,15 +1817,17 @@ def test_lstm_sequence_in_one_persistent_launch(gpu, D, O, rng, T, B, H):
     close(D.op.sum(hs).numpy(), first.astype(np.float64).sum(), rtol=1e-5, atol=1e-5 * np.abs(first).sum())
 
 
-def test_persistent_lstm_barrier_gives_up_instead_of_hanging():
+@pytest.mark.parametrize("B", [8, 40])
+def test_persistent_lstm_barrier_gives_up_instead_of_hanging(B):
     """With the poll limit forced to one, the first workgroup at the first barrier gives up, raises the flag, every
-    workgroup leaves (the kernel ends normally) and the next synchronising call reports it."""
+    workgroup leaves (the kernel ends normally) and the next synchronising call reports it. 8 rows: the form that waits
+    for the values (its one barrier comes first); 40 rows: a barrier per step."""
     import subprocess, sys, os
     code = (
         "import numpy as np, dali_amd as D\n"
         "from dali_amd._native import hip\n"
         "rng = np.random.RandomState(0)\n"
-        "T, B, H = 6, 8, 1024\n"
+        "T, B, H = 6, %d, 1024\n" % B +
         "dev = [D.Array.from_numpy(v.astype(np.float32)) for v in (rng.randn(T, B, H), rng.randn(B, H), rng.randn(B, H), rng.randn(H, 4 * H) * 0.01, rng.randn(H, 4 * H) * 0.01, np.zeros(4 * H))]\n"
         "hs, c, h = D.op.lstm_sequence(*dev)\n"
         "rc = hip.dali_hip_sync()\n"
