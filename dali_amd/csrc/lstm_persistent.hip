@@ -472,9 +472,20 @@ extern "C" int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidd
     if (batch > 64) return fail("dali_hip_lstm_recurrent_persistent: batch %d exceeds 64 rows (use one launch per step)", batch);
     if (hidden % 256 != 0 || hidden > 1024) return fail("dali_hip_lstm_recurrent_persistent: hidden %d must be 256, 512, 768 or 1024", hidden);
     if (((uintptr_t)h0 | (uintptr_t)hs) % 16 != 0) return fail("dali_hip_lstm_recurrent_persistent: h0 and hs must be 16-byte aligned");
-    hipDeviceProp_t prop;
-    if (hipGetDeviceProperties(&prop, bound_device()) != hipSuccess) return fail("dali_hip_lstm_recurrent_persistent: no device properties");
-    const int cus = prop.multiProcessorCount;
+    {
+        // rows 0 .. steps-2 of hs are overwritten (with the "not written yet" pattern or with h) while h0, c0 and pre are
+        // still being read
+        const char *lo = (const char*)hs, *hi = lo + (size_t)steps * batch * hidden * sizeof(float);
+        auto inside = [&](const void* p, size_t bytes) { return (const char*)p < hi && (const char*)p + bytes > lo; };
+        if (inside(h0, (size_t)batch * hidden * 4) || inside(c0, (size_t)batch * hidden * 4) || inside(pre, (size_t)steps * batch * hidden * 16))
+            return fail("dali_hip_lstm_recurrent_persistent: hs overlaps an input");
+    }
+    static int cus = 0;  // (the library is bound to one device)
+    if (cus == 0) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, bound_device()) != hipSuccess) return fail("dali_hip_lstm_recurrent_persistent: no device properties");
+        cus = prop.multiProcessorCount;
+    }
     // fewest hidden units per workgroup that still give every workgroup a compute unit of its own
     int HU = 1;
     while (HU <= 4 && !(hidden % HU == 0 && hidden / HU <= cus)) ++HU;

@@ -128,10 +128,15 @@ bool try_flat(const std::vector<DestSpec>& specs) {
     std::ostringstream params;
     // Streaming policy of a map, measured on 64M floats (copy / a + b / a chain of five operands): inputs bypass cache
     // allocation (plain loads: 0.73 instead of 0.87 of the HBM peak), outputs leave with plain stores (non-temporal stores:
-    // 0.78). Kernels that reduce over cached rows are the other way round for their stores.
-    static const int nt_env = env_int("DALI_HIP_FLAT_NT_STORES", 0);
+    // 0.78). Kernels that reduce over cached rows are the other way round for their stores, and so is a map whose outputs
+    // fit the second-level caches (32 MiB between them): with plain stores the whole output is still dirty in cache when
+    // the last wave ends and the write-back is added to the kernel's time (4M floats over sixteen rotating buffer
+    // pairs: copy 7.0 us, with non-temporal stores 6.0; a + b 9.2 -> 9.0; the same from cache-resident pairs: no loss).
+    static const int nt_env = env_int("DALI_HIP_FLAT_NT_STORES", -1);
     static const int ntl_env = env_int("DALI_HIP_FLAT_NT_LOADS", 1);
-    const bool NT_STORES = nt_env != 0, NT_LOADS = ntl_env != 0;
+    long out_bytes = 0;
+    for (const Output& o : outs) out_bytes += n * (long)size_of_dtype(P.arrays[o.array].buf->dtype);
+    const bool NT_STORES = nt_env < 0 ? out_bytes <= (32L << 20) : nt_env != 0, NT_LOADS = ntl_env != 0;
     params << VEC << "," << BT << "," << UNROLL << "," << UNALIGNED << REST << "," << NT_STORES << NT_LOADS;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("flat", signature(P, outs), params.str());

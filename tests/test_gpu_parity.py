@@ -1817,6 +1817,37 @@ def test_lstm_sequence_in_one_persistent_launch(gpu, D, O, rng, T, B, H):
     close(D.op.sum(hs).numpy(), first.astype(np.float64).sum(), rtol=1e-5, atol=1e-5 * np.abs(first).sum())
 
 
+@pytest.mark.parametrize("T,B,H", [(7, 4, 512), (4, 40, 256)])
+def test_persistent_recurrence_through_the_c_abi(gpu, O, rng, T, B, H):
+    """dali_hip_lstm_recurrent_persistent on raw device pointers: pre-activations of the input half from the host, a
+    leading dimension of U larger than its row, twice in a row into the same hs; against the sequential definition, and
+    the argument checks."""
+    hip = gpu
+    Xs = rng.randn(T, B, H).astype(np.float32)
+    H0, C0 = (rng.randn(B, H).astype(np.float32) for _ in range(2))
+    lim = np.sqrt(6.0 / (H + 4 * H))
+    W, U = (rng.uniform(-lim, lim, (H, 4 * H)).astype(np.float32) for _ in range(2))
+    b = (rng.randn(4 * H) * 0.1).astype(np.float32)
+    pre = (Xs.reshape(T * B, H).astype(np.float64) @ W.astype(np.float64) + b).astype(np.float32).reshape(T, B, 4 * H)
+    Up = np.zeros((H, 4 * H + 8), np.float32); Up[:, :4 * H] = U
+    ptrs = [_dev(hip, v) for v in (pre, Up, H0, C0, np.zeros((T, B, H), np.float32), np.zeros((B, H), np.float32))]
+    ohs, oc = O.lstm_sequence(Xs, H0, C0, W, U, b)
+    hs, c = np.empty((T, B, H), np.float32), np.empty((B, H), np.float32)
+    for _ in range(2):
+        assert hip.dali_hip_lstm_recurrent_persistent(T, B, H, ptrs[0], ptrs[1], 4 * H + 8, ptrs[2], ptrs[3], ptrs[4], ptrs[5]) == 0, hip.dali_hip_last_error()
+        assert hip.dali_hip_memcpy_d2h(hs.ctypes.data_as(C.c_void_p), ptrs[4], hs.nbytes) == 0, hip.dali_hip_last_error()
+        assert hip.dali_hip_memcpy_d2h(c.ctypes.data_as(C.c_void_p), ptrs[5], c.nbytes) == 0
+        close(hs, ohs, rtol=2e-4, atol=2e-5)
+        close(c, oc, rtol=2e-4, atol=2e-5)
+    # refused: more than 64 rows, a hidden size without a kernel, hs on top of h0
+    assert hip.dali_hip_lstm_recurrent_persistent(T, 65, H, ptrs[0], ptrs[1], 4 * H + 8, ptrs[2], ptrs[3], ptrs[4], ptrs[5]) != 0
+    assert hip.dali_hip_lstm_recurrent_persistent(T, B, 320, ptrs[0], ptrs[1], 4 * H + 8, ptrs[2], ptrs[3], ptrs[4], ptrs[5]) != 0
+    assert hip.dali_hip_lstm_recurrent_persistent(T, B, H, ptrs[0], ptrs[1], 4 * H + 8, ptrs[4], ptrs[3], ptrs[4], ptrs[5]) != 0
+    assert b"overlaps" in hip.dali_hip_last_error()
+    for p in ptrs:
+        hip.dali_hip_free(p)
+
+
 @pytest.mark.parametrize("B", [8, 40])
 def test_persistent_lstm_barrier_gives_up_instead_of_hanging(B):
     """With the poll limit forced to one, the first workgroup at the first barrier gives up, raises the flag, every
