@@ -188,6 +188,8 @@ FRONT_SYMBOLS = {
     "dali_fe_device_ptr": (H, [H]),
     "dali_fe_stats": (_i, [C.POINTER(_u64)] * 4),
     "dali_fe_plan_cache_stats": (_i, [C.POINTER(_u64)] * 2),
+    "dali_fe_scope_observe": (_i, [C.c_void_p, C.c_void_p, C.c_void_p]),
+    "dali_fe_scope_unobserve": (None, [_i]),
     "dali_fe_last_kernel_kinds": (C.c_char_p, []),
     "dali_fe_last_kernel_names": (C.c_char_p, []),
     "dali_fe_last_source": (C.c_char_p, []),

@@ -317,6 +317,45 @@ def generate_only(arrays, compile=False):
     return n
 
 
+_SCOPE_CB = C.CFUNCTYPE(None, C.c_char_p, C.c_int, C.c_void_p)
+
+
+class ScopeObserver(object):
+    """Calls ``on_enter(name, trace)`` / ``on_exit(name, trace)`` for every named scope the front-end opens inside the
+    ``with`` block (dali/utils/scope.h: ScopeObserver); ``trace`` lists the open scopes, outermost first, the reported
+    one included. ``events`` collects ("enter" | "exit", name, depth) in order."""
+
+    def __init__(self, on_enter=None, on_exit=None):
+        self.events, self.trace = [], []
+        self._on_enter, self._on_exit, self._id = on_enter, on_exit, 0
+
+        def enter(name, depth, _user):
+            name = name.decode()
+            self.trace.append(name)
+            self.events.append(("enter", name, depth))
+            if self._on_enter:
+                self._on_enter(name, list(self.trace))
+
+        def leave(name, depth, _user):
+            name = name.decode()
+            self.events.append(("exit", name, depth))
+            if self._on_exit:
+                self._on_exit(name, list(self.trace))
+            if self.trace and self.trace[-1] == name:
+                self.trace.pop()
+
+        self._enter_cb, self._exit_cb = _SCOPE_CB(enter), _SCOPE_CB(leave)  # kept alive as long as the observer
+
+    def __enter__(self):
+        self._id = front.dali_fe_scope_observe(C.cast(self._enter_cb, C.c_void_p), C.cast(self._exit_cb, C.c_void_p), None)
+        return self
+
+    def __exit__(self, *exc):
+        front.dali_fe_scope_unobserve(self._id)
+        self._id = 0
+        return False
+
+
 class Recording(object):
     """Stores the launches issued inside the ``with`` block; ``replay(n)`` re-issues them."""
 

@@ -315,6 +315,23 @@ int dali_fe_set_dry_run(int on, int compile) {
     dali::set_dry_compile(on != 0 && compile != 0);
     return 0;
 }
+int dali_fe_scope_observe(dali_fe_scope_callback on_enter, dali_fe_scope_callback on_exit, void* user) {
+    // the depth counts the scopes this observer has seen open, the one reported included
+    auto depth = std::make_shared<int>(0);
+    dali::Scope::callback_t enter, leave;
+    enter = [on_enter, user, depth](dali::Scope::name_t n) {
+        ++*depth;
+        if (on_enter) on_enter(n->c_str(), *depth, user);
+    };
+    leave = [on_exit, user, depth](dali::Scope::name_t n) {
+        if (on_exit) on_exit(n->c_str(), *depth, user);
+        if (*depth > 0) --*depth;
+    };
+    return dali::Scope::add_observer(enter, leave);
+}
+
+void dali_fe_scope_unobserve(int id) { dali::Scope::remove_observer(id); }
+
 int dali_fe_generate_only(dali_array_t* roots, int n, int compile) {
     dali::set_dry_compile(compile != 0);
     try {

@@ -8,6 +8,7 @@
 #define DALI_AMD_HOST_DALI_H
 
 #include <cstdint>
+#include <functional>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -376,8 +377,45 @@ StackedLSTMState stacked_lstm_step(const Array& x, const std::vector<Array>& h, 
 Array gru_step(const Array& x, const Array& h, const Array& W, const Array& U, const Array& b);
 }  // namespace op
 
-// Observation hooks in the spirit of dali/utils/scope.h: counts of executed
-// computations, used by tests to assert laziness and fusion.
+// Named scopes (dali/utils/scope.h:11-34): DALI_SCOPE(name) opens a scope that lasts to the end of the block when
+// somebody observes and costs one test otherwise. The front-end opens "JIT[<kernel shape>:<entry point>]" around every
+// generated kernel it launches (the name dali/array/expression/computation.cpp:19 gives a computation), inside it
+// "get_function" when the kernel is not loaded yet and, inside that, "compilation" around the call that builds it from
+// source unless the code-object cache on disk holds it (dali/array/jit/jit.cpp:1015,1025), and "gemm" around a product.
+struct Scope {
+    typedef std::shared_ptr<std::string> name_t;
+    typedef std::function<void(name_t)> callback_t;
+    static bool has_observers();
+    // returns the handle remove_observer takes; either callback may be empty
+    static int add_observer(callback_t on_enter, callback_t on_exit);
+    static void remove_observer(int id);
+    name_t name;
+    explicit Scope(name_t name_);
+    ~Scope();
+    Scope(const Scope&) = delete;
+    Scope& operator=(const Scope&) = delete;
+};
+#define DALI_SCOPE(str)                                                              \
+    std::unique_ptr<::dali::Scope> dali_scope_guard;                                 \
+    if (::dali::Scope::has_observers()) dali_scope_guard.reset(new ::dali::Scope(std::make_shared<std::string>(str)))
+
+// Keeps the stack of open scopes and hands it to two callbacks (dali/utils/scope.h:37-63); observes for as long as it lives.
+struct ScopeObserver {
+    struct State {
+        std::vector<Scope::name_t> trace;  // outermost first; on_exit sees the scope that is being left as the last entry
+    };
+    typedef std::function<void(const State&)> callback_t;
+    ScopeObserver(callback_t on_enter_, callback_t on_exit_);
+    ~ScopeObserver();
+    ScopeObserver(const ScopeObserver&) = delete;
+    ScopeObserver& operator=(const ScopeObserver&) = delete;
+  private:
+    callback_t on_enter, on_exit;
+    State state;
+    int id;
+};
+
+// Counts of executed computations, used by tests to assert laziness and fusion.
 struct JitStats {
     uint64_t kernels_launched = 0;  // generated kernels
     uint64_t gemms_launched = 0;

@@ -58,6 +58,7 @@ static GemmOperands prepare_gemm(const Expr* mm) {
 // dst[n_rows, m] = lhs * rhs through the column-major entry point, argument for
 // argument the call of dali/array/gemm/cublas_gemm.cu:153-166.
 void run_gemm(const Array& dst, const Expr* mm, const Expr* mm2, float beta) {
+    DALI_SCOPE(mm2 ? "gemm_pair" : "gemm");
     GemmOperands g = prepare_gemm(mm);
     int m = g.rhs.shape()[1], n = g.lhs.shape()[0], k = g.rhs.shape()[0];
     jit_stats().gemms_launched++;

@@ -46,6 +46,7 @@ void load_and_launch(KernelSpec& K, const std::function<std::string()>& gen, con
         g_capture->shapes = shapes;
         if (g_capture_compare_only) return;
     }
+    DALI_SCOPE("JIT[" + K.kind + ":" + K.name + "]");
     JitStats& st = jit_stats();
     static const bool trace_plan = getenv("DALI_HIP_TRACE_PLAN") != nullptr;  // one line per planned launch on stderr
     if (trace_plan) fprintf(stderr, "[dali-hip plan] %s\n", K.name.c_str());
@@ -66,13 +67,16 @@ void load_and_launch(KernelSpec& K, const std::function<std::string()>& gen, con
         return;
     }
     if (need_source) {
+        DALI_SCOPE("get_function");
         int cached = 0;
         if (dali_hip_module_is_loaded(K.hash)) {
             cached = 2;
         } else {
             std::string src = gen();
-                g_last_source += src;
+            g_last_source += src;
             st.plans_built++;
+            std::unique_ptr<Scope> compilation;
+            if (Scope::has_observers()) compilation.reset(new Scope(std::make_shared<std::string>("compilation")));
             check_hip(dali_hip_module_load(K.hash, src.c_str(), K.name.c_str(), &K.plan, &cached), "JIT module load");
         }
         loaded_hashes()[K.hash] = true;

@@ -154,6 +154,16 @@ int dali_fe_stats(uint64_t* kernels, uint64_t* gemms, uint64_t* evals, uint64_t*
  * instead of running the planner, and plans stored so far; DALI_HIP_PLAN_CACHE=0 turns the cache off,
  * DALI_HIP_PLAN_CACHE_CHECK=1 runs the planner beside every reuse and raises if the two disagree */
 int dali_fe_plan_cache_stats(uint64_t* hits, uint64_t* stored);
+/* Named scopes around the front-end's work (dali/utils/scope.h: Scope, ScopeObserver): on_enter / on_exit are called
+ * with the scope's name and the number of scopes open (the reported one included) when a scope opens and closes. The
+ * front-end opens "JIT[<kernel shape>:<entry point>]" around every generated kernel it launches
+ * (dali/array/expression/computation.cpp:19), inside it "get_function" while the kernel is not loaded and, inside that,
+ * "compilation" around the build from source (dali/array/jit/jit.cpp:1015,1025), and "gemm" / "gemm_pair" around a
+ * product. Either callback may be NULL. Returns the handle dali_fe_scope_unobserve takes. Without observers a scope
+ * costs one test. */
+typedef void (*dali_fe_scope_callback)(const char* name, int depth, void* user);
+int dali_fe_scope_observe(dali_fe_scope_callback on_enter, dali_fe_scope_callback on_exit, void* user);
+void dali_fe_scope_unobserve(int handle);
 const char* dali_fe_last_kernel_kinds(void);
 const char* dali_fe_last_kernel_names(void);
 const char* dali_fe_last_source(void);

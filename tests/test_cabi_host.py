@@ -222,3 +222,25 @@ def test_gather_plans_as_an_indirect_row_leaf_and_checks_its_arguments(D, rng):
     with pytest.raises(RuntimeError, match="same dimensionality"):
         t = D.Array.zeros((3,))
         t <<= D.Array.from_numpy(np.ones((3, 4), np.float32))
+
+
+def test_scope_observers_see_the_planned_kernels(D, rng):
+    """dali/utils/scope.h: an observer is told when a named scope opens and closes; the front-end names every generated
+    kernel it plans "JIT[<shape>:<entry point>]" (generation only: no device needed). Observers stack and detach."""
+    op = D.op
+    x = D.Array.from_numpy(rng.randn(8, 64).astype(np.float32))
+    seen = []
+    with D.ScopeObserver(lambda name, trace: seen.append(("in", name, tuple(trace))),
+                         lambda name, trace: seen.append(("out", name, tuple(trace)))) as outer:
+        D.generate_only([op.softmax(x)])
+        with D.ScopeObserver() as inner:
+            D.generate_only([op.sum(x * 2.0)])
+        D.generate_only([op.exp(x)])
+    D.generate_only([op.tanh(x)])  # nobody observes any more
+    names = [e[1] for e in outer.events if e[0] == "enter"]
+    assert len(names) == 3 and names[0].startswith("JIT[row:dali_row_") and names[1].startswith("JIT[all:dali_all_") and names[2].startswith("JIT[flat:dali_flat_")
+    assert [e[1] for e in inner.events] == [names[1], names[1]] and [e[0] for e in inner.events] == ["enter", "exit"]
+    # every scope that opened closed again, at the depth it opened at, and the callbacks saw the stack of open scopes
+    assert [e[0] for e in outer.events] == ["enter", "exit"] * 3 and all(e[2] == 1 for e in outer.events)
+    assert seen[0] == ("in", names[0], (names[0],)) and seen[1] == ("out", names[0], (names[0],)) and len(seen) == 6
+    assert outer.trace == [] and names[0].endswith("]")

@@ -950,6 +950,30 @@ def test_full_reductions_of_row_values_join_the_row_kernel(gpu, D, O, rng, shape
     close(b.numpy(), other.numpy().astype(np.float64).sum(), rtol=1e-5, atol=1e-5)
 
 
+def test_scopes_around_launch_load_and_product(gpu, D, rng):
+    """dali/utils/scope.h with the call sites of dali/array/expression/computation.cpp:19 and dali/array/jit/jit.cpp:1015,1025:
+    a kernel met for the first time opens JIT[...] > get_function > compilation (unless it is already loaded in this
+    process), the second evaluation only JIT[...]; a product opens "gemm"."""
+    op = D.op
+    x = D.Array.from_numpy(rng.randn(37, 53).astype(np.float32))
+    expr = lambda: op.tanh(x * 1.25 + 0.75) * op.sigmoid(x - 0.375)
+    with D.ScopeObserver() as first:
+        want = expr().numpy()
+    with D.ScopeObserver() as second:
+        again = expr().numpy()
+        prod = op.dot(x, x.transpose()).numpy()
+    assert np.array_equal(want, again)
+    ev = [(k, n.split(":")[0] if n.startswith("JIT[") else n, d) for k, n, d in first.events]
+    assert ev[0] == ("enter", "JIT[flat", 1) and ev[-1] == ("exit", "JIT[flat", 1)
+    inner = ev[1:-1]
+    # loaded now or earlier in this process; when it is loaded now, from source or from the cache on disk
+    assert inner in ([], [("enter", "get_function", 2), ("exit", "get_function", 2)],
+                     [("enter", "get_function", 2), ("enter", "compilation", 3), ("exit", "compilation", 3), ("exit", "get_function", 2)])
+    ev2 = [(k, n.split(":")[0] if n.startswith("JIT[") else n, d) for k, n, d in second.events]
+    assert ev2 == [("enter", "JIT[flat", 1), ("exit", "JIT[flat", 1), ("enter", "gemm", 1), ("exit", "gemm", 1)]
+    close(prod, x.numpy().astype(np.float64) @ x.numpy().astype(np.float64).T, rtol=1e-5, atol=1e-4)
+
+
 # --------------------------------------------------------------------- dot
 def test_dot_known_answers_and_laziness(gpu, D, rng):
     """ArrayDotTests.dot / dot_T / dot_strided / matrix-vector (dot_tests.cpp:9-118)."""
