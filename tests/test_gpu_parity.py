@@ -275,7 +275,8 @@ def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
 
 @pytest.mark.parametrize("ta", [0, 1])
 @pytest.mark.parametrize("tb", [0, 1])
-@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 5, 7), (64, 64, 16), (65, 63, 17), (100, 260, 200), (256, 512, 1000), (250, 1, 33), (1, 300, 64), (37, 41, 0)])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 5, 7), (64, 64, 16), (65, 63, 17), (100, 260, 200), (256, 512, 1000), (250, 1, 33), (1, 300, 64), (37, 41, 0),
+                                   (2100, 1990, 40), (2048, 2048, 32)])  # the last two: enough 128 x 128 tiles for every compute unit
 def test_dgemm_abi_column_major_convention(gpu, rng, M, N, K, ta, tb):
     """dali_hip_dgemm(transB, transA, m, n, k, alpha, B, ldb, A, lda, beta, C, ldc) as cublasDgemm is called in
     cublas_gemm.cu:167-178: row-major C[n, m] = alpha * A[n, k] . B[k, m] + beta * C, in double precision. Checked against
