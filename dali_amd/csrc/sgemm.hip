@@ -110,7 +110,7 @@ __device__ __forceinline__ float observe(const float* p) { return __hip_atomic_l
 // MAXSEG: how many terms the instantiation can walk. Two (the LSTM pair) keeps the segment switch of the main loop a
 // pair of scalar selects; the eight-term form (convolution by filter rows) carries a short select chain instead.
 template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int DEPTH, bool EDGE, int KW, bool MIDB, bool GATES = false, int MAXSEG = 2>
-__global__ __launch_bounds__(256 * KW) void sgemm_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256 * KW, (BM == 128 && !EDGE && KW == 1) ? 2 : 1) void sgemm_kernel(GemmArgs g) {
     // KW wave sets share the tile: set kw takes every KW-th k-group of a slab, so each SIMD holds
     // KW waves that cover each other's LDS and barrier waits; the sets are summed through LDS at the end
     constexpr int THREADS = 256 * KW;
