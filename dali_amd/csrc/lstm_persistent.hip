@@ -28,6 +28,7 @@
 
 #include <cstdint>
 #include <cstdlib>
+#include <type_traits>
 
 namespace dali_hip {
 
@@ -413,42 +414,61 @@ __global__ __launch_bounds__(256) void lstm_step_small_kernel(SmallStepArgs a) {
     // cost a memory round trip each: 90 us for 64 rows.)
     const float* blockp = a.partials + (size_t)ub * 4 * KS * (size_t)B * kSmallUnits;
     const __amdgpu_buffer_rsrc_t shares = __builtin_amdgcn_make_buffer_rsrc((void*)blockp, 0, 4 * KS * B * kSmallUnits * 4, 0x00027000);
-    for (int quad = tid; quad < B * (kSmallUnits / 4); quad += 256) {
+    // With at most four k shares a thread asks for the shares of two quads at once (the registers that eight shares of one
+    // quad would take): half as many round trips for 17 rows and more.
+    const int quads = B * (kSmallUnits / 4);
+    auto fold = [&](auto per_trip_tag, auto shares_tag) {
+        constexpr int QI = decltype(per_trip_tag)::value, KSM = decltype(shares_tag)::value;
+        for (int quad0 = tid; quad0 < quads; quad0 += 256 * QI) {
 #pragma clang fp contract(off)
-        const int bb = quad / (kSmallUnits / 4), u = (quad % (kSmallUnits / 4)) * 4, unit = ub * kSmallUnits + u;
-        f4 pv[4][kSmallMaxShares];
+            f4 pv[QI][4][KSM];
 #pragma unroll
-        for (int gt = 0; gt < 4; ++gt)
+            for (int i = 0; i < QI; ++i) {
+                const int quad = quad0 + 256 * i;
+                const int bb = quad / (kSmallUnits / 4), u = (quad % (kSmallUnits / 4)) * 4;
 #pragma unroll
-            for (int k = 0; k < kSmallMaxShares; ++k)
-                pv[gt][k] = k < KS ? __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(shares, (((gt * KS + k) * B + bb) * kSmallUnits + u) * 4, 0, kCoherentLoad))
-                                   : (f4){0.f, 0.f, 0.f, 0.f};
-        const f4 cells = *reinterpret_cast<const f4*>(a.Cp + (size_t)bb * H + unit);
-        f4 cn4, hn4;
+                for (int gt = 0; gt < 4; ++gt)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            float g4[4];
-#pragma unroll
-            for (int gt = 0; gt < 4; ++gt) {
-                float sum = 0.0f;
-#pragma unroll
-                for (int k = 0; k < kSmallMaxShares; ++k)
-                    if (k < KS) sum += pv[gt][k][j];
-                g4[gt] = sum + a.bias[gt * H + unit + j];
+                    for (int k = 0; k < KSM; ++k)
+                        pv[i][gt][k] = k < KS && quad < quads
+                                           ? __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(shares, (((gt * KS + k) * B + bb) * kSmallUnits + u) * 4, 0, kCoherentLoad))
+                                           : (f4){0.f, 0.f, 0.f, 0.f};
             }
-            const float iv = (float)(1.0 / (1.0 + (double)seq_expf(-g4[0])));
-            const float fv = (float)(1.0 / (1.0 + (double)seq_expf(-g4[1])));
-            const float ov = (float)(1.0 / (1.0 + (double)seq_expf(-g4[2])));
-            const float gv = tanhf(g4[3]);
-            const float fc = fv * cells[j];
-            const float ig = iv * gv;
-            const float cn = fc + ig;
-            cn4[j] = cn;
-            hn4[j] = ov * tanhf(cn);
+#pragma unroll
+            for (int i = 0; i < QI; ++i) {
+                const int quad = quad0 + 256 * i;
+                if (quad >= quads) break;
+                const int bb = quad / (kSmallUnits / 4), u = (quad % (kSmallUnits / 4)) * 4, unit = ub * kSmallUnits + u;
+                const f4 cells = *reinterpret_cast<const f4*>(a.Cp + (size_t)bb * H + unit);
+                f4 cn4, hn4;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float g4[4];
+#pragma unroll
+                    for (int gt = 0; gt < 4; ++gt) {
+                        float sum = 0.0f;
+#pragma unroll
+                        for (int k = 0; k < KSM; ++k)
+                            if (k < KS) sum += pv[i][gt][k][j];
+                        g4[gt] = sum + a.bias[gt * H + unit + j];
+                    }
+                    const float iv = (float)(1.0 / (1.0 + (double)seq_expf(-g4[0])));
+                    const float fv = (float)(1.0 / (1.0 + (double)seq_expf(-g4[1])));
+                    const float ov = (float)(1.0 / (1.0 + (double)seq_expf(-g4[2])));
+                    const float gv = tanhf(g4[3]);
+                    const float fc = fv * cells[j];
+                    const float ig = iv * gv;
+                    const float cn = fc + ig;
+                    cn4[j] = cn;
+                    hn4[j] = ov * tanhf(cn);
+                }
+                *reinterpret_cast<f4*>(a.Cout + (size_t)bb * H + unit) = cn4;
+                *reinterpret_cast<f4*>(a.Hout + (size_t)bb * H + unit) = hn4;
+            }
         }
-        *reinterpret_cast<f4*>(a.Cout + (size_t)bb * H + unit) = cn4;
-        *reinterpret_cast<f4*>(a.Hout + (size_t)bb * H + unit) = hn4;
-    }
+    };
+    if (KS <= 4 && quads > 256) fold(std::integral_constant<int, 2>(), std::integral_constant<int, 4>());
+    else fold(std::integral_constant<int, 1>(), std::integral_constant<int, kSmallMaxShares>());
     if (tid == 0) __hip_atomic_store(a.tickets + ub, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
