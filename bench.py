@@ -364,6 +364,20 @@ def main():
                                                                            "frac_fp64_mfma": round(2.0 * 2048 ** 3 / dus / 1e6 / 78.6, 4)}
         del dA, dB, drec
 
+        # few rows against a wide weight matrix (the output projection of a decoder step): bound by streaming the weights once
+        Wp = D.Array.from_numpy((np.random.RandomState(29).randn(1024, 32000) * 0.02).astype(np.float32))
+        proj = {}
+        for Bq in (8, 64):
+            hq = D.Array.from_numpy(np.random.RandomState(30 + Bq).randn(Bq, 1024).astype(np.float32))
+            with D.Recording() as prec:
+                op.dot(hq, Wp).eval()
+            pus = time_recording(prec, 20)
+            proj["B%d" % Bq] = {"us": round(pus, 2), "weights_GB/s": round(1024 * 32000 * 4 / pus / 1e3, 1), "frac_hbm": round(1024 * 32000 * 4 / pus / 1e3 / HBM_PEAK_GBS, 4),
+                                "TFLOP/s": round(2.0 * Bq * 1024 * 32000 / pus / 1e6, 2)}
+            del hq, prec
+        configs["c5_lstm_step_256x1024x1024"]["dot_few_rows_Bx1024x32000"] = proj
+        del Wp
+
         # rows beyond the five configs: embedding-style gather and its scatter-add (table [32000, 1024], 8192 indices)
         V, Dm, Nidx = 32000, 1024, 8192
         table = D.Array.from_numpy(np.random.RandomState(14).randn(V, Dm).astype(np.float32))

@@ -205,7 +205,9 @@ int dali_hip_cache_warm(int* loaded);
  * dali/array/gemm/cpu_gemm.cpp:59-68): C(m x n, column-major, ldc) =
  * alpha * op(B)(m x k) * op(A)(k x n) + beta * C, i.e. in row-major terms
  * C[n, m] = alpha * A[n, k] * B[k, m] + beta * C. trans flags: 0 = no transpose,
- * 1 = transpose.
+ * 1 = transpose. With n <= 64 (a few rows of A against a wide B, transA = 0, k a multiple of 4) B is streamed once,
+ * straight from memory into the matrix instruction, instead of being tiled through LDS; the sums are then formed in
+ * another order than the tiled kernels form them (DALI_HIP_GEMM_SKINNY=0 switches this off).
  */
 int dali_hip_sgemm(int transB, int transA, int m, int n, int k, float alpha, const float* B, int ldb,
                    const float* A, int lda, float beta, float* C, int ldc);

@@ -273,6 +273,44 @@ def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
         hip.dali_hip_free(p)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 32000, 1024), (8, 4096, 1024), (64, 1000, 260), (17, 777, 512), (33, 2049, 64), (64, 8192, 2048),
+                                   (5, 40000, 68), (48, 32000, 1024)])
+@pytest.mark.parametrize("tb", [0, 1])
+def test_sgemm_with_few_rows_streams_the_right_operand(gpu, rng, M, N, K, tb):
+    """At most 64 rows against a wide row-major right operand (the output projection of a decoder step): the kernel that
+    reads B straight into the matrix instruction, with and without a split of K across workgroups, B row-major [K, N] or
+    stored transposed as [N, K] (weights kept as [outputs, inputs]). Leading dimensions
+    larger than the rows, with NaN in the padding of both operands and, for beta = 0, in the destination: nothing outside
+    the operands may reach a result. Against the product accumulated in double precision."""
+    hip = gpu
+    A = rng.randn(M, K).astype(np.float32)
+    B = rng.randn(K, N).astype(np.float32)
+    lda, ldb, ldc = K + 4, (K + 8 if tb else N + 5), N + 3
+    Ap = np.full((M, lda), np.nan, np.float32); Ap[:, :K] = A
+    if tb:
+        Bp = np.full((N, ldb), np.nan, np.float32); Bp[:, :K] = B.T
+    else:
+        Bp = np.full((K, ldb), np.nan, np.float32); Bp[:, :N] = B
+    C0 = rng.randn(M, ldc).astype(np.float32)
+    dA, dB, dC = _dev(hip, Ap), _dev(hip, Bp), _dev(hip, C0)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    scale = np.abs(want).max() + 1e-6
+    out = np.empty_like(C0)
+    assert hip.dali_hip_sgemm(tb, 0, N, M, K, 0.75, dB, ldb, dA, lda, -0.5, dC, ldc) == 0, hip.dali_hip_last_error()
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+    assert np.abs(out[:, :N] - (0.75 * want - 0.5 * C0[:, :N])).max() <= 1e-4 * scale
+    assert np.array_equal(out[:, N:], C0[:, N:])  # padding untouched
+    nan = np.full_like(C0, np.nan)
+    hip.dali_hip_memcpy_h2d(dC, nan.ctypes.data_as(C.c_void_p), nan.nbytes)
+    for _ in range(2):  # twice: the tickets of a split of K are back at rest
+        assert hip.dali_hip_sgemm(tb, 0, N, M, K, 1.0, dB, ldb, dA, lda, 0.0, dC, ldc) == 0, hip.dali_hip_last_error()
+        hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+        assert np.abs(out[:, :N] - want).max() <= 1e-4 * scale
+        assert np.isnan(out[:, N:]).all()
+    for p in (dA, dB, dC):
+        hip.dali_hip_free(p)
+
+
 @pytest.mark.parametrize("ta", [0, 1])
 @pytest.mark.parametrize("tb", [0, 1])
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 5, 7), (64, 64, 16), (65, 63, 17), (100, 260, 200), (256, 512, 1000), (250, 1, 33), (1, 300, 64), (37, 41, 0),
