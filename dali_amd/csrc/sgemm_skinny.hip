@@ -171,9 +171,13 @@ int sgemm_skinny(bool tb, int M, int N, int K, float alpha, const float* A, int 
     // idle, so 500 column blocks (32000 columns) stay whole
     int KS = 1;
     while (blocks * KS < 384 && KS < kMaxShares && K / (KS * 2) >= 256) KS *= 2;
-    if (blocks * KS < 128) return 0;  // too little of B per workgroup to stream: the tiled kernel with its split of K
-    // 33 to 64 rows with a split of K: the tiled kernel is as fast or faster (64 x 4096 over K = 4096: 29.8 against 32 us)
-    if (KS > 1 && M > 32) return 0;
+    // a narrow B: shares down to 128 values of k until there are 128 workgroups ([8,1024].[1024,1024]: 7.1 us against 15.4
+    // through the tiled kernel, which walks its sixteen slabs one after the other whatever the number of rows)
+    while (blocks * KS < 128 && KS < kMaxShares && K / (KS * 2) >= 128) KS *= 2;
+    if (blocks * KS < 32) return 0;
+    // 33 to 64 rows with a split of K: the tiled kernel is as fast or faster unless the shares are long
+    // (64 x 4096 over K = 1024: 16.4 against 22.9 us here; 64 x 1024 over K = 32000: 71 against 58 us)
+    if (KS > 1 && M > 32 && K / KS < (M > 48 ? 1536 : 1024)) return 0;
     if (KS > 1 && ((size_t)blocks * KS * M * kCols * sizeof(float) > kWorkspacePartialBytes || blocks > kWorkspaceCounters - 2)) KS = 1;
     SkinnyArgs a;
     a.M = M; a.N = N; a.K = K; a.KS = KS;

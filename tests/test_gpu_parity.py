@@ -274,7 +274,8 @@ def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 32000, 1024), (8, 4096, 1024), (64, 1000, 260), (17, 777, 512), (33, 2049, 64), (64, 8192, 2048),
-                                   (5, 40000, 68), (48, 32000, 1024)])
+                                   (5, 40000, 68), (48, 32000, 1024), (8, 1024, 1024), (8, 256, 1024), (9, 512, 512), (20, 4096, 256),
+                                   (64, 1024, 32000), (40, 1028, 16384)])
 @pytest.mark.parametrize("tb", [0, 1])
 def test_sgemm_with_few_rows_streams_the_right_operand(gpu, rng, M, N, K, tb):
     """At most 64 rows against a wide row-major right operand (the output projection of a decoder step): the kernel that
