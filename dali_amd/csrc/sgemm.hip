@@ -915,6 +915,11 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         const int st = sgemm_skinny(tb, M, N, g.seg[0].K, alpha, g.seg[0].A, g.seg[0].lda, g.seg[0].B, g.seg[0].ldb, beta, C, ldc);
         if (st != 0) return st > 0 ? DALI_HIP_OK : DALI_HIP_ERROR;
     }
+    if (g.nseg == 1 && g.seg[0].K > 0 && g.seg[0].K <= 64 && !row_map && !rows_may_overlap) {
+        // a short inner extent against a large result (the weight gradient of a layer at a small batch)
+        const int st = sgemm_smallk(ta, tb, M, N, g.seg[0].K, alpha, g.seg[0].A, g.seg[0].lda, g.seg[0].B, g.seg[0].ldb, beta, C, ldc);
+        if (st != 0) return st > 0 ? DALI_HIP_OK : DALI_HIP_ERROR;
+    }
     long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     static const int variant = getenv("DALI_HIP_GEMM_VARIANT") ? atoi(getenv("DALI_HIP_GEMM_VARIANT")) : 0;
     if (tiles128 >= 192) return run_tile<128, 128, 32, 2>(g, ta, tb, vec, 1);

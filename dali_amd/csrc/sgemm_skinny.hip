@@ -156,6 +156,87 @@ __global__ __launch_bounds__(256, 2) void sgemm_skinny_kernel(SkinnyArgs a) {
     if (tid == 0) __hip_atomic_store(a.tickets + cb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// ---------------------------------------------------------------------------------------------- short inner extent
+// C[M, N] = alpha * A . B + beta * C with K <= 64, B row-major [K][N], A stored as [K][M] or [M][K]: the weight gradient of
+// a layer, dot(h^T [hidden, batch], g [batch, outputs]), at a small batch, or a layer with few inputs. Such a product is bound by writing C once; the tiled
+// kernel spends a whole 64-deep slab, its prologue and its epilogue on every 64 x 64 tile (1024 x 32000 at K = 8:
+// 51 us for 131 MB). Here a workgroup keeps its 64 columns of A (64 rows of C) in registers in the layout of the
+// instruction's A operand for all of K and walks along a strip of C; per 64 columns a wave loads K/4 16-byte pieces of B
+// (four consecutive columns of row k, feeding the four column tiles congruent to 0..3 modulo 4, as above) and stores its
+// 64 x 64 results as 16-byte pieces: the four tiles' values of a lane are four consecutive columns of one row.
+struct SmallKArgs {
+    int M, N, K, CB;  // CB: 64-column blocks per wave
+    const float* A;
+    const float* B;
+    float* C;
+    int a_row, a_k, a_extent;  // element (row, k) of A at A[row * a_row + k * a_k]; a_extent: elements up to its last one
+    int ldb, ldc;
+    float alpha, beta;
+};
+
+// S: steps of 4 values of k (K <= 4 S)
+template <int S>
+__global__ __launch_bounds__(256, 2) void sgemm_smallk_kernel(SmallKArgs a) {
+    const int M = a.M, N = a.N, K = a.K;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int arow = lane & 15, kgrp = lane >> 4;
+    const int row0 = blockIdx.x * 64;
+    // rows of both operands past K lie outside the ranges and read as zero
+    const __amdgpu_buffer_rsrc_t arows = __builtin_amdgcn_make_buffer_rsrc((void*)a.A, 0, a.a_extent * 4, 0x00027000);
+    const __amdgpu_buffer_rsrc_t brows = __builtin_amdgcn_make_buffer_rsrc((void*)a.B, 0, ((K - 1) * a.ldb + N) * 4, 0x00027000);
+    float av[S][4];
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            const int k = 4 * s + kgrp, row = row0 + 16 * m + arow;
+            av[s][m] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(arows, k < K && row < M ? (k * a.a_k + row * a.a_row) * 4 : kOutside, 0, 0));
+        }
+    const int first = (blockIdx.y * 4 + wave) * a.CB;
+    for (int cb = first; cb < first + a.CB; ++cb) {
+        const int col0 = cb * kCols;
+        if (col0 >= N) break;  // (wave-uniform)
+        const int col = col0 + 4 * arow;
+        f4 bv[S];
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            const int k = 4 * s + kgrp;
+            bv[s] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(brows, k < K ? (k * a.ldb + col) * 4 : kOutside, 0, 0));
+        }
+        f4 acc[4][4];
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+            for (int m = 0; m < 4; ++m) acc[ct][m] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < S; ++s)
+#pragma unroll
+            for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+                for (int m = 0; m < 4; ++m) acc[ct][m] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s][m], bv[s][ct], acc[ct][m], 0, 0, 0);
+        // a lane holds, of tile ct, column 4 * (lane % 16) + ct of the block and rows 16 m + 4 * (lane / 16) + v
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int row = row0 + 16 * m + 4 * kgrp + v;
+                if (row >= M || col >= N) continue;
+                float* p = a.C + (size_t)row * a.ldc + col;
+                f4 r = (f4){a.alpha * acc[0][m][v], a.alpha * acc[1][m][v], a.alpha * acc[2][m][v], a.alpha * acc[3][m][v]};
+                typedef f4 f4u __attribute__((aligned(4)));
+                if (col + 3 < N) {
+                    if (a.beta != 0.0f) {
+                        const f4 old = *reinterpret_cast<const f4u*>(p);
+                        r += a.beta * old;
+                    }
+                    *reinterpret_cast<f4u*>(p) = r;
+                } else {
+                    for (int j = 0; j < 4 && col + j < N; ++j) p[j] = a.beta == 0.0f ? r[j] : r[j] + a.beta * p[j];
+                }
+            }
+    }
+}
+
 }  // namespace
 
 // 1: the product was launched; 0: not a case for this kernel (the caller takes the general path); -1: failure
@@ -215,6 +296,42 @@ int sgemm_skinny(bool tb, int M, int N, int K, float alpha, const float* A, int 
     if (e == hipSuccess) e = hipGetLastError();
     if (e != hipSuccess) {
         fail("sgemm (at most 64 rows) launch failed: %s", hipGetErrorString(e));
+        return -1;
+    }
+    return 1;
+}
+
+
+// the same convention of results as sgemm_skinny; ta: A is stored as [K][M]
+int sgemm_smallk(bool ta, bool tb, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb, float beta, float* C, int ldc) {
+    static const bool enabled = !(getenv("DALI_HIP_GEMM_SMALLK") && atoi(getenv("DALI_HIP_GEMM_SMALLK")) == 0);
+    if (!enabled || tb || K < 1 || K > 64 || M < 64 || N < 256) return 0;
+    if ((size_t)K * ldb * 4 + 4096 >= ((size_t)1 << 31) || (size_t)(ta ? K : M) * lda * 4 + 4096 >= ((size_t)1 << 31)) return 0;
+    if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) % 4 != 0) return 0;
+    const int row_blocks = (M + 63) / 64, col_blocks = (N + kCols - 1) / kCols;
+    // blocks per wave: long strips amortise the registers of A, but keep a few thousand workgroups
+    if ((long)row_blocks * ((col_blocks + 3) / 4) < 256) return 0;  // a small C: the tiled kernel ([1024,1024] at K = 64: 5.9 against 7.7 us)
+    const int enough = K <= 16 ? 1024 : 512;  // (measured: 1024 x 32000 at K = 8 / 64: 22.8 / 51.6 us with 1024, 24.0 / 49.4 with 512)
+    int CB = 1;
+    while (CB < 8 && (long)row_blocks * ((col_blocks + 4 * CB * 2 - 1) / (4 * CB * 2)) >= enough) CB *= 2;
+    const int col_groups = (col_blocks + 4 * CB - 1) / (4 * CB);
+    if (col_groups > 65535) return 0;
+    SmallKArgs a;
+    a.M = M; a.N = N; a.K = K; a.CB = CB;
+    a.A = A; a.B = B; a.C = C;
+    a.a_row = ta ? 1 : lda; a.a_k = ta ? lda : 1;
+    a.a_extent = ta ? (K - 1) * lda + M : (M - 1) * lda + K;
+    a.ldb = ldb; a.ldc = ldc;
+    a.alpha = alpha; a.beta = beta;
+    const dim3 grid((unsigned)row_blocks, (unsigned)col_groups);
+    const int S = (K + 3) / 4;
+    if (S <= 2) hipLaunchKernelGGL(sgemm_smallk_kernel<2>, grid, dim3(256), 0, stream(), a);
+    else if (S <= 4) hipLaunchKernelGGL(sgemm_smallk_kernel<4>, grid, dim3(256), 0, stream(), a);
+    else if (S <= 8) hipLaunchKernelGGL(sgemm_smallk_kernel<8>, grid, dim3(256), 0, stream(), a);
+    else hipLaunchKernelGGL(sgemm_smallk_kernel<16>, grid, dim3(256), 0, stream(), a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        fail("sgemm (inner extent of at most 64) launch failed: %s", hipGetErrorString(e));
         return -1;
     }
     return 1;

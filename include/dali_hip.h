@@ -207,7 +207,8 @@ int dali_hip_cache_warm(int* loaded);
  * C[n, m] = alpha * A[n, k] * B[k, m] + beta * C. trans flags: 0 = no transpose,
  * 1 = transpose. With n <= 64 (a few rows of A against a wide B, transA = 0, k a multiple of 4) B is streamed once,
  * straight from memory into the matrix instruction, instead of being tiled through LDS; the sums are then formed in
- * another order than the tiled kernels form them (DALI_HIP_GEMM_SKINNY=0 switches this off).
+ * another order than the tiled kernels form them (DALI_HIP_GEMM_SKINNY=0 switches this off). With k <= 64 against a
+ * large C (transB = 0) the rows of A stay in registers and C is written once (DALI_HIP_GEMM_SMALLK=0 switches that off).
  */
 int dali_hip_sgemm(int transB, int transA, int m, int n, int k, float alpha, const float* B, int ldb,
                    const float* A, int lda, float beta, float* C, int ldc);

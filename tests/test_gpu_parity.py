@@ -312,6 +312,40 @@ def test_sgemm_with_few_rows_streams_the_right_operand(gpu, rng, M, N, K, tb):
         hip.dali_hip_free(p)
 
 
+@pytest.mark.parametrize("M,N,K", [(1024, 32000, 8), (100, 300, 64), (64, 256, 1), (130, 1000, 33), (512, 4099, 17), (2048, 8192, 48)])
+@pytest.mark.parametrize("ta", [1, 0])
+def test_sgemm_with_a_short_inner_extent(gpu, rng, M, N, K, ta):
+    """C = A . B with K <= 64, B stored as [K, N] and A as [K, M] (the weight gradient dot(h^T, g) of a layer at a small
+    batch) or as [M, K] (a layer with few inputs): the kernel that keeps its columns of A in registers and is bound by writing C. NaN in the padding of the
+    operands and, for beta = 0, in the destination; against the product in double precision."""
+    hip = gpu
+    A = rng.randn(M, K).astype(np.float32)
+    B = rng.randn(K, N).astype(np.float32)
+    lda, ldb, ldc = (M + 3 if ta else K + 1), N + 5, N + 2
+    if ta:
+        Ap = np.full((K, lda), np.nan, np.float32); Ap[:, :M] = A.T
+    else:
+        Ap = np.full((M, lda), np.nan, np.float32); Ap[:, :K] = A
+    Bp = np.full((K, ldb), np.nan, np.float32); Bp[:, :N] = B
+    C0 = rng.randn(M, ldc).astype(np.float32)
+    dA, dB, dC = _dev(hip, Ap), _dev(hip, Bp), _dev(hip, C0)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    scale = np.abs(want).max() + 1e-6
+    out = np.empty_like(C0)
+    assert hip.dali_hip_sgemm(0, ta, N, M, K, 0.75, dB, ldb, dA, lda, -0.5, dC, ldc) == 0, hip.dali_hip_last_error()
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+    assert np.abs(out[:, :N] - (0.75 * want - 0.5 * C0[:, :N])).max() <= 1e-5 * scale
+    assert np.array_equal(out[:, N:], C0[:, N:])  # padding untouched
+    nan = np.full_like(C0, np.nan)
+    hip.dali_hip_memcpy_h2d(dC, nan.ctypes.data_as(C.c_void_p), nan.nbytes)
+    assert hip.dali_hip_sgemm(0, ta, N, M, K, 1.0, dB, ldb, dA, lda, 0.0, dC, ldc) == 0, hip.dali_hip_last_error()
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+    assert np.abs(out[:, :N] - want).max() <= 1e-5 * scale
+    assert np.isnan(out[:, N:]).all()
+    for p in (dA, dB, dC):
+        hip.dali_hip_free(p)
+
+
 @pytest.mark.parametrize("ta", [0, 1])
 @pytest.mark.parametrize("tb", [0, 1])
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (3, 5, 7), (64, 64, 16), (65, 63, 17), (100, 260, 200), (256, 512, 1000), (250, 1, 33), (1, 300, 64), (37, 41, 0),
