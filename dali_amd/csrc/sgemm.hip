@@ -930,12 +930,17 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
     int split_k = split_env > 0 ? split_env : 1;
     if (split_env == 0 && variant == 0 && tiles64 <= 128) {
         // A few tiles over a long inner extent (the weight gradient of a convolution: [out, window] from tens of
-        // thousands of patches) would leave most of the device idle: shares of at least eight slabs, about two
-        // workgroups per CU, folded in a fixed order by the workgroup that finishes last.
+        // thousands of patches) would leave most of the device idle: about two workgroups per CU, folded in a fixed
+        // order by the workgroup that finishes last.
         int nslab64 = 0;
         for (int s = 0; s < g.nseg; ++s) nslab64 += (g.seg[s].K + 63) / 64;
         const int want = (int)((512 + tiles64 - 1) / tiles64);
-        const int share = nslab64 / 8 < want ? nslab64 / 8 : want;
+        // (shares of at least four slabs, two when there are no more than eight: [256,1024] over K = 1024 16.4 -> 12.9 us,
+        // [100,512] over K = 512 12.4 -> 8.9 us against shares of at least eight; shorter shares lose to their fold)
+        // A sum of several products keeps shares of eight: the LSTM pair over short inner extents then stays whole and
+        // bit-equal to the fused step, which sums its slabs in one workgroup.
+        const int min_slabs = g.nseg > 1 ? 8 : nslab64 <= 8 ? 2 : 4;
+        const int share = nslab64 / min_slabs < want ? nslab64 / min_slabs : want;
         if (share >= 2) return run_tile<64, 64, 64, 2>(g, ta, tb, vec, share);
     }
     if (variant == 8) return run_tile<64, 64, 64, 2>(g, ta, tb, vec, split_k);
