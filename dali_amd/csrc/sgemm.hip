@@ -915,6 +915,18 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         const int st = sgemm_skinny(tb, M, N, g.seg[0].K, alpha, g.seg[0].A, g.seg[0].lda, g.seg[0].B, g.seg[0].ldb, beta, C, ldc);
         if (st != 0) return st > 0 ? DALI_HIP_OK : DALI_HIP_ERROR;
     }
+    if (g.nseg == 2 && !ta && !row_map && !rows_may_overlap && M <= 64) {
+        // a sum of two such products (an LSTM's x.W + h.U at a small batch whose sizes the fused kernels do not take): the
+        // first streams its right operand, the second adds to the result
+        const int st = sgemm_skinny(tb, M, N, g.seg[0].K, alpha, g.seg[0].A, g.seg[0].lda, g.seg[0].B, g.seg[0].ldb, beta, C, ldc);
+        if (st < 0) return DALI_HIP_ERROR;
+        if (st > 0) {
+            const int k1[1] = {g.seg[1].K}, lda1[1] = {g.seg[1].lda}, ldb1[1] = {g.seg[1].ldb};
+            const float* a1[1] = {g.seg[1].A};
+            const float* b1[1] = {g.seg[1].B};
+            return sgemm_rowmajor(1, ta, tb, M, N, k1, a1, lda1, b1, ldb1, alpha, 1.0f, C, ldc);
+        }
+    }
     if (g.nseg == 1 && g.seg[0].K > 0 && g.seg[0].K <= 64 && !row_map && !rows_may_overlap) {
         // a short inner extent against a large result (the weight gradient of a layer at a small batch)
         const int st = sgemm_smallk(ta, tb, M, N, g.seg[0].K, alpha, g.seg[0].A, g.seg[0].lda, g.seg[0].B, g.seg[0].ldb, beta, C, ldc);

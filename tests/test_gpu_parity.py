@@ -416,7 +416,9 @@ def test_dot_in_double_precision(gpu, D, rng):
         op.dot(arr(D, np.ones((2, 3), np.int32)), arr(D, np.ones((3, 2), np.int32))).numpy()
 
 
-@pytest.mark.parametrize("M,N,K1,K2", [(48, 200, 96, 40), (100, 260, 200, 200), (256, 512, 128, 192), (250, 1000, 100, 100)])
+@pytest.mark.parametrize("M,N,K1,K2", [(48, 200, 96, 40), (100, 260, 200, 200), (256, 512, 128, 192), (250, 1000, 100, 100),
+                                       # few rows: the first product streams its right operand, the second adds to it
+                                       (8, 8192, 1024, 2048), (33, 4000, 300, 1000), (64, 32000, 64, 128), (16, 8192, 1024, 30)])
 def test_sgemm_pair_accumulates_two_products(gpu, rng, M, N, K1, K2):
     hip = gpu
     A1, B1 = rng.randn(M, K1).astype(np.float32), rng.randn(K1, N).astype(np.float32)
