@@ -312,6 +312,43 @@ def test_sgemm_with_few_rows_streams_the_right_operand(gpu, rng, M, N, K, tb):
         hip.dali_hip_free(p)
 
 
+def test_sgemm_random_shapes_around_the_kernel_boundaries(gpu):
+    """One entry point, three kernels (tiled, few rows, short inner extent) chosen from M, N, K, the transposition flags
+    and the alignment: 160 random products drawn around the limits of that choice (64 rows, an inner extent of 64 and
+    multiples of 4, 64 and 256 columns), with padded leading dimensions, NaN in every padding and random alpha / beta,
+    against the product in double precision."""
+    hip = gpu
+    rng = np.random.RandomState(4242)
+    near = lambda centre, spread: int(max(1, centre + rng.randint(-spread, spread + 1)))
+    for case in range(160):
+        M = near(rng.choice([1, 8, 32, 64, 65, 130, 300]), 3)
+        N = near(rng.choice([48, 64, 256, 300, 1000, 4100]), 5)
+        K = near(rng.choice([4, 32, 64, 68, 128, 260, 1024]), 4)
+        ta, tb = int(rng.randint(2)), int(rng.randint(2))
+        alpha, beta = float(rng.choice([1.0, 0.75, -2.0])), float(rng.choice([0.0, 0.0, 1.0, -0.5]))
+        A = rng.randn(M, K).astype(np.float32)
+        B = rng.randn(K, N).astype(np.float32)
+        Ast, Bst = (A.T if ta else A), (B.T if tb else B)
+        lda, ldb, ldc = Ast.shape[1] + int(rng.randint(0, 6)), Bst.shape[1] + int(rng.randint(0, 6)), N + int(rng.randint(0, 4))
+        Ap = np.full((Ast.shape[0], lda), np.nan, np.float32); Ap[:, :Ast.shape[1]] = Ast
+        Bp = np.full((Bst.shape[0], ldb), np.nan, np.float32); Bp[:, :Bst.shape[1]] = Bst
+        C0 = rng.randn(M, ldc).astype(np.float32)
+        if beta == 0.0:
+            C0[:, :N] = np.nan
+        dA, dB, dC = _dev(hip, Ap), _dev(hip, Bp), _dev(hip, C0)
+        what = "case %d: M=%d N=%d K=%d ta=%d tb=%d lda=%d ldb=%d ldc=%d alpha=%g beta=%g" % (case, M, N, K, ta, tb, lda, ldb, ldc, alpha, beta)
+        assert hip.dali_hip_sgemm(tb, ta, N, M, K, alpha, dB, ldb, dA, lda, beta, dC, ldc) == 0, what + ": " + hip.dali_hip_last_error().decode()
+        out = np.empty_like(C0)
+        hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+        prod = A.astype(np.float64) @ B.astype(np.float64)
+        want = alpha * prod + (beta * C0[:, :N] if beta != 0.0 else 0.0)
+        scale = np.abs(alpha) * (np.abs(A).astype(np.float64) @ np.abs(B)).max() + np.abs(want).max() + 1e-6
+        assert np.abs(out[:, :N] - want).max() <= 2e-6 * scale * max(1.0, np.sqrt(K) / 8), what
+        assert np.array_equal(out[:, N:], C0[:, N:]), what  # padding untouched
+        for p in (dA, dB, dC):
+            hip.dali_hip_free(p)
+
+
 @pytest.mark.parametrize("M,N,K", [(1024, 32000, 8), (100, 300, 64), (64, 256, 1), (130, 1000, 33), (512, 4099, 17), (2048, 8192, 48)])
 @pytest.mark.parametrize("ta", [1, 0])
 def test_sgemm_with_a_short_inner_extent(gpu, rng, M, N, K, ta):
