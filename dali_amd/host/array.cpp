@@ -1727,5 +1727,42 @@ Array gru_step(const Array& x, const Array& h, const Array& W, const Array& U, c
     return h_new;
 }
 
+// GRU::activate_sequence (dali/layers/gru.cpp:59-64): the step applied to every x(t) in turn, the state carried along.
+// What does not depend on the state, x(t).W for all three layers, is one product over the whole sequence; a step is
+// then the recurrent products and the two gate kernels of gru_step.
+GRUSequence gru_sequence(const Array& xs, const Array& h0, const Array& W, const Array& U, const Array& b) {
+    DALI_ASSERT(xs.ndim() == 3 && h0.ndim() == 2 && W.ndim() == 2 && U.ndim() == 2 && b.ndim() == 1,
+                "gru_sequence: xs must be [T, B, I], h0 a matrix, W and U matrices, b a vector");
+    const int T = xs.shape()[0], Bn = xs.shape()[1], In = xs.shape()[2], H = h0.shape()[1];
+    DALI_ASSERT(T >= 1 && h0.shape()[0] == Bn && W.shape()[0] == In && W.shape()[1] == 3 * H && U.shape()[0] == H && U.shape()[1] == 3 * H &&
+                    b.shape()[0] == 3 * H,
+                "gru_sequence: inconsistent shapes");
+    for (const Array* a : {&xs, &h0, &W, &U, &b}) a->eval();
+    Array px_all = dot(xs.reshape({T * Bn, In}), W);  // [T B, 3H]
+    px_all.eval();
+    auto bias = [&](int k) { return b.slice(0, k * H, (k + 1) * H).expand_dims(0); };
+    auto cols = [&](const Array& a, int k) { return a.slice(1, k * H, (k + 1) * H); };
+    Array states = Array({T, Bn, H}, DTYPE_FLOAT);
+    Array h = h0;
+    for (int t = 0; t < T; ++t) {
+        Array px = px_all.slice(0, t * Bn, (t + 1) * Bn);
+        Array ph = dot(h, U.slice(1, 0, 2 * H));
+        ph.eval();
+        Array reset_state = eltmul(sigmoid(add(add(cols(px, 0), cols(ph, 0)), bias(0))), h);
+        Array pc = dot(reset_state, U.slice(1, 2 * H, 3 * H));
+        pc.eval();
+        Array update = sigmoid(add(add(cols(px, 1), cols(ph, 1)), bias(1)));
+        Array candidate = tanh(add(add(cols(px, 2), pc), bias(2)));
+        Array h_t = states.pluck_axis(0, t);
+        h_t.assign(add(eltmul(h, subtract(Array(1.0), update)), eltmul(candidate, update)));
+        h_t.eval();
+        h = h_t;
+    }
+    GRUSequence out;
+    out.states = states;
+    out.last = h;
+    return out;
+}
+
 }  // namespace op
 }  // namespace dali

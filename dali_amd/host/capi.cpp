@@ -229,6 +229,10 @@ int dali_fe_stacked_lstm_step(dali_array_t x, int layers, const dali_array_t* h,
                               const dali_array_t* b, int shortcut, dali_array_t* c_new, dali_array_t* h_new) {
     FE_TRY(return stacked_lstm_step_impl(x, layers, h, c, W, U, b, shortcut, c_new, h_new);, 1)
 }
+int dali_fe_gru_sequence(dali_array_t xs, dali_array_t h0, dali_array_t W, dali_array_t U, dali_array_t b, dali_array_t* states, dali_array_t* last) {
+    FE_TRY(auto r = dali::op::gru_sequence(A(xs), A(h0), A(W), A(U), A(b)); *states = wrap(r.states); *last = wrap(r.last); return 0;, -1)
+}
+
 dali_array_t dali_fe_gru_step(dali_array_t x, dali_array_t h, dali_array_t W, dali_array_t U, dali_array_t b) {
     FE_TRY(return wrap(dali::op::gru_step(A(x), A(h), A(W), A(U), A(b)));, nullptr)
 }

@@ -375,6 +375,12 @@ StackedLSTMState stacked_lstm_step(const Array& x, const std::vector<Array>& h, 
 // One GRU step with reset, update and candidate layers packed along the columns of W[I,3H], U[H,3H], b[3H]
 // (dali/layers/gru.cpp:27-44). Returns h', already evaluated.
 Array gru_step(const Array& x, const Array& h, const Array& W, const Array& U, const Array& b);
+// The step along a whole sequence xs [T, B, I] from the state h0 (GRU::activate_sequence, dali/layers/gru.cpp:59-64, which
+// returns the last state): every state [T, B, H] and the last one (a view of it), already evaluated.
+struct GRUSequence {
+    Array states, last;
+};
+GRUSequence gru_sequence(const Array& xs, const Array& h0, const Array& W, const Array& U, const Array& b);
 }  // namespace op
 
 // Named scopes (dali/utils/scope.h:11-34): DALI_SCOPE(name) opens a scope that lasts to the end of the block when

@@ -265,6 +265,15 @@ def stacked_lstm_step(x, h, c, W, U, b, shortcut=False):
     return [Array(v) for v in c_new], [Array(v) for v in h_new]
 
 
+def gru_sequence(xs, h0, W, U, b):
+    """The GRU step along xs [T, B, I] from the state h0 (GRU::activate_sequence): (states [T, B, H], last state)."""
+    keep = [as_array(v) for v in (xs, h0, W, U, b)]
+    outs = [C.c_void_p(), C.c_void_p()]
+    if front.dali_fe_gru_sequence(*[k._h for k in keep], *[C.byref(o) for o in outs]) != 0:
+        raise fe_error("gru_sequence")
+    return Array(outs[0].value), Array(outs[1].value)
+
+
 def gru_step(x, h, W, U, b):
     """One GRU step; reset / update / candidate layers packed along the columns of W[I,3H], U[H,3H], b[3H]."""
     keep = [as_array(v) for v in (x, h, W, U, b)]

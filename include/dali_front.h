@@ -140,6 +140,9 @@ int dali_fe_stacked_lstm_step(dali_array_t x, int layers, const dali_array_t* h,
 /* One GRU step, layers packed reset / update / candidate along the columns of W[I,3H], U[H,3H], b[3H]
  * (dali/layers/gru.cpp:27-44) */
 dali_array_t dali_fe_gru_step(dali_array_t x, dali_array_t h, dali_array_t W, dali_array_t U, dali_array_t b);
+/* The step along a sequence xs [T, B, I] from the state h0 (GRU::activate_sequence, dali/layers/gru.cpp:59-64): every state
+ * [T, B, H] and the last one; the input half of all steps is one product */
+int dali_fe_gru_sequence(dali_array_t xs, dali_array_t h0, dali_array_t W, dali_array_t U, dali_array_t b, dali_array_t* states, dali_array_t* last);
 
 /* evaluation, assignment, host access */
 int dali_fe_eval(dali_array_t a);

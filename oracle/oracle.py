@@ -430,6 +430,17 @@ def gru_step(X, Hs, W, U, b):
     return ((Hs * one_minus).astype(f32) + (m * z).astype(f32)).astype(f32)
 
 
+def gru_sequence(Xs, H0, W, U, b):
+    """GRU::activate_sequence (dali/layers/gru.cpp:59-64): the step applied to every Xs[t] in turn, the state carried along.
+    Returns every state [T, B, H]."""
+    h = _c32(H0)
+    out = []
+    for x in Xs:
+        h = gru_step(x, h, W, U, b)
+        out.append(h)
+    return np.stack(out)
+
+
 def k_best(x, k, largest):
     """int32 positions of the k best entries along the last axis, best first (dali/array/op/top_k.cpp:96-220).
     k = 1 is argmax / argmin (first position on ties, :205,:217); k = the whole axis is the full sort with runs of equal

@@ -2025,6 +2025,32 @@ def test_gru_step_matches_oracle(gpu, D, O, rng, B, I, H):
     assert np.array_equal(D.op.gru_step(*(arr(D, v) for v in (X, Hp, W, U, b_keep))).numpy(), Hp)
 
 
+@pytest.mark.parametrize("T,B,I,H", [(3, 16, 32, 48), (6, 8, 256, 256), (4, 5, 7, 9), (5, 70, 128, 64)])
+def test_gru_sequence_is_the_step_in_turn(gpu, D, O, rng, T, B, I, H):
+    """GRU::activate_sequence (dali/layers/gru.cpp:59-64): the input half of all steps is one product, so the states equal
+    the step applied in turn to the rounding of that product's other order of summation; against the sequential definition
+    and against op.gru_step step by step; the recorded launches recompute the same states."""
+    Xs = rng.randn(T, B, I).astype(np.float32)
+    H0 = rng.randn(B, H).astype(np.float32)
+    lim = np.sqrt(6.0 / (I + 3 * H))
+    W, U = (rng.uniform(-lim, lim, (n, 3 * H)).astype(np.float32) for n in (I, H))
+    b = (rng.randn(3 * H) * 0.1).astype(np.float32)
+    dev = [arr(D, v) for v in (Xs, H0, W, U, b)]
+    with D.Recording() as rec:
+        states, last = D.op.gru_sequence(*dev)
+    assert states.shape == (T, B, H) and np.array_equal(last.numpy(), states.numpy()[-1])
+    close(states.numpy(), O.gru_sequence(Xs, H0, W, U, b), rtol=2e-4, atol=2e-5)
+    h = dev[1]
+    for t in range(T):
+        h = D.op.gru_step(arr(D, Xs[t]), h, dev[2], dev[3], dev[4])
+        close(states.numpy()[t], h.numpy(), rtol=1e-4, atol=1e-5)
+    first = states.numpy().copy()
+    rec.replay(2)
+    assert np.array_equal(states.numpy(), first)
+    with pytest.raises(Exception):
+        D.op.gru_sequence(dev[0], arr(D, np.zeros((B + 1, H), np.float32)), dev[2], dev[3], dev[4])
+
+
 @pytest.mark.parametrize("B,I,sizes", [(3, 8, [8]), (5, 7, [6, 4, 9]), (32, 64, [64, 64]), (16, 128, [128, 64, 192])])
 @pytest.mark.parametrize("shortcut", [False, True])
 def test_stacked_lstm_step_matches_oracle(gpu, D, O, rng, B, I, sizes, shortcut):

@@ -585,6 +585,16 @@ def test_gru_step_against_fp64_definition(O, rng):
     m = np.tanh(x @ w[:, 2 * H:] + (r * h) @ u[:, 2 * H:] + bb[2 * H:])
     want = h * (1.0 - z) + m * z
     assert np.abs(O.gru_step(X, Hp, W, U, b) - want).max() < 2e-6
+    # GRU::activate_sequence (gru.cpp:59-64) carries the state through the steps: against the fp64 recurrence
+    Xg = rng.randn(4, B, I).astype(np.float32)
+    state = h
+    for t in range(4):
+        xt = f64(Xg[t])
+        r = sig(xt @ w[:, :H] + state @ u[:, :H] + bb[:H])
+        z = sig(xt @ w[:, H:2 * H] + state @ u[:, H:2 * H] + bb[H:2 * H])
+        m = np.tanh(xt @ w[:, 2 * H:] + (r * state) @ u[:, 2 * H:] + bb[2 * H:])
+        state = state * (1.0 - z) + m * z
+        assert np.abs(O.gru_sequence(Xg, Hp, W, U, b)[t] - state).max() < 1e-5
     # the sequence wrapper is the step in turn
     Xs = rng.randn(3, B, H).astype(np.float32)
     W4, U4 = rng.uniform(-0.3, 0.3, (H, 4 * H)).astype(np.float32), rng.uniform(-0.3, 0.3, (H, 4 * H)).astype(np.float32)
