@@ -182,6 +182,7 @@ FRONT_SYMBOLS = {
     "dali_fe_gru_step": (H, [H, H, H, H, H]),
     "dali_fe_gru_sequence": (_i, [H, H, H, H, H, _HP, _HP]),
     "dali_fe_stacked_lstm_step": (_i, [H, _i, _HP, _HP, _HP, _HP, _HP, _i, _HP, _HP]),
+    "dali_fe_stacked_lstm_sequence": (_i, [H, _i, _HP, _HP, _HP, _HP, _HP, _i, _HP, _HP, _HP]),
     "dali_fe_eval": (_i, [H]),
     "dali_fe_eval_together": (_i, [_HP, _i]),
     "dali_fe_assign": (_i, [H, _i, H]),

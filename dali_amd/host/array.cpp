@@ -1699,6 +1699,30 @@ StackedLSTMState stacked_lstm_step(const Array& x, const std::vector<Array>& h, 
     return out;
 }
 
+// AbstractStackedLSTM::activate_sequence (dali/layers/stacked_lstm.cpp:44-51, drop_prob = 0): the stack applied to every
+// x(t) in turn. Layer l at step t needs layer l-1 at step t and itself at step t-1 only, so the loop nest can be turned
+// around: every layer runs over the whole sequence before the next one starts, on the hidden states of the layer below
+// ([T, B, H], beside x(t) for a shortcut stack), which lets each layer take the one-launch recurrence of lstm_sequence.
+StackedLSTMSequence stacked_lstm_sequence(const Array& xs, const std::vector<Array>& h, const std::vector<Array>& c, const std::vector<Array>& W,
+                                          const std::vector<Array>& U, const std::vector<Array>& b, bool shortcut) {
+    const size_t layers = W.size();
+    DALI_ASSERT(xs.ndim() == 3, "stacked_lstm_sequence: xs must be [T, B, I]");
+    DALI_ASSERT(h.size() == layers && c.size() == layers,
+                make_message("Activating LSTM stack of size ", layers, " with different number of states ", std::min(h.size(), c.size())));
+    DALI_ASSERT(U.size() == layers && b.size() == layers && layers >= 1, "stacked_lstm_sequence: every layer needs its W, U and b");
+    StackedLSTMSequence out;
+    Array layer_input = xs;
+    for (size_t l = 0; l < layers; ++l) {
+        Array in = (shortcut && l > 0) ? concatenate({layer_input, xs}, 2) : layer_input;
+        LSTMSequence r = lstm_sequence(in, h[l], c[l], W[l], U[l], b[l]);
+        out.memory.push_back(r.memory);
+        out.hidden.push_back(r.hidden);
+        layer_input = r.hidden_states;
+    }
+    out.top_hidden_states = layer_input;
+    return out;
+}
+
 // One GRU step (dali/layers/gru.cpp:27-44 with StackedInputLayer::activate, dali/layers/layers.cpp:159-161), the
 // three input layers packed reset, update, candidate along the columns of W[I, 3H], U[H, 3H], b[3H]:
 //   r = sigmoid(x.Wr + h.Ur + br);  z = sigmoid(x.Wz + h.Uz + bz);  m = tanh(x.Wc + (r * h).Uc + bc)

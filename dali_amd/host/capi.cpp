@@ -229,6 +229,30 @@ int dali_fe_stacked_lstm_step(dali_array_t x, int layers, const dali_array_t* h,
                               const dali_array_t* b, int shortcut, dali_array_t* c_new, dali_array_t* h_new) {
     FE_TRY(return stacked_lstm_step_impl(x, layers, h, c, W, U, b, shortcut, c_new, h_new);, 1)
 }
+static int stacked_lstm_sequence_impl(dali_array_t xs, int layers, const dali_array_t* h, const dali_array_t* c, const dali_array_t* W,
+                                      const dali_array_t* U, const dali_array_t* b, int shortcut, dali_array_t* c_last, dali_array_t* h_last,
+                                      dali_array_t* top_states) {
+    std::vector<Array> hv, cv, Wv, Uv, bv;
+    for (int l = 0; l < layers; ++l) {
+        hv.push_back(A(h[l]));
+        cv.push_back(A(c[l]));
+        Wv.push_back(A(W[l]));
+        Uv.push_back(A(U[l]));
+        bv.push_back(A(b[l]));
+    }
+    auto r = dali::op::stacked_lstm_sequence(A(xs), hv, cv, Wv, Uv, bv, shortcut != 0);
+    for (int l = 0; l < layers; ++l) {
+        c_last[l] = wrap(r.memory[l]);
+        h_last[l] = wrap(r.hidden[l]);
+    }
+    *top_states = wrap(r.top_hidden_states);
+    return 0;
+}
+int dali_fe_stacked_lstm_sequence(dali_array_t xs, int layers, const dali_array_t* h, const dali_array_t* c, const dali_array_t* W,
+                                  const dali_array_t* U, const dali_array_t* b, int shortcut, dali_array_t* c_last, dali_array_t* h_last,
+                                  dali_array_t* top_states) {
+    FE_TRY(return stacked_lstm_sequence_impl(xs, layers, h, c, W, U, b, shortcut, c_last, h_last, top_states);, 1)
+}
 int dali_fe_gru_sequence(dali_array_t xs, dali_array_t h0, dali_array_t W, dali_array_t U, dali_array_t b, dali_array_t* states, dali_array_t* last) {
     FE_TRY(auto r = dali::op::gru_sequence(A(xs), A(h0), A(W), A(U), A(b)); *states = wrap(r.states); *last = wrap(r.last); return 0;, -1)
 }

@@ -372,6 +372,15 @@ struct StackedLSTMState {
 };
 StackedLSTMState stacked_lstm_step(const Array& x, const std::vector<Array>& h, const std::vector<Array>& c, const std::vector<Array>& W,
                                    const std::vector<Array>& U, const std::vector<Array>& b, bool shortcut);
+// The stack along a whole sequence xs [T, B, I] (AbstractStackedLSTM::activate_sequence, dali/layers/stacked_lstm.cpp:44-51,
+// which returns the final state of every layer): final memory and hidden state per layer and the hidden states of the top
+// layer [T, B, H], already evaluated. Layer by layer, each over the whole sequence.
+struct StackedLSTMSequence {
+    std::vector<Array> memory, hidden;
+    Array top_hidden_states;
+};
+StackedLSTMSequence stacked_lstm_sequence(const Array& xs, const std::vector<Array>& h, const std::vector<Array>& c, const std::vector<Array>& W,
+                                          const std::vector<Array>& U, const std::vector<Array>& b, bool shortcut);
 // One GRU step with reset, update and candidate layers packed along the columns of W[I,3H], U[H,3H], b[3H]
 // (dali/layers/gru.cpp:27-44). Returns h', already evaluated.
 Array gru_step(const Array& x, const Array& h, const Array& W, const Array& U, const Array& b);

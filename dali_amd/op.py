@@ -265,6 +265,24 @@ def stacked_lstm_step(x, h, c, W, U, b, shortcut=False):
     return [Array(v) for v in c_new], [Array(v) for v in h_new]
 
 
+def stacked_lstm_sequence(xs, h, c, W, U, b, shortcut=False):
+    """The stack of LSTM layers along xs [T, B, I] (AbstractStackedLSTM::activate_sequence): h, c, W, U, b are lists with
+    one entry per layer. Returns (list of final c, list of final h, hidden states [T, B, H] of the top layer), evaluated."""
+    layers = len(W)
+    xa = as_array(xs)
+    groups = [[as_array(v) for v in g] for g in (h, c, W, U, b)]
+    if any(len(g) != layers for g in groups[2:]) or layers < 1:
+        raise ValueError("stacked_lstm_sequence: every layer needs its W, U and b")
+    if len(groups[0]) != layers or len(groups[1]) != layers:
+        states = len(groups[0]) if len(groups[0]) != layers else len(groups[1])
+        raise DaliError("Activating LSTM stack of size %d with different number of states %d" % (layers, states))
+    handles = [(C.c_void_p * layers)(*[k._h for k in g]) for g in groups]
+    c_last, h_last, top = (C.c_void_p * layers)(), (C.c_void_p * layers)(), C.c_void_p()
+    if front.dali_fe_stacked_lstm_sequence(xa._h, layers, *handles, 1 if shortcut else 0, c_last, h_last, C.byref(top)) != 0:
+        raise fe_error("stacked_lstm_sequence")
+    return [Array(v) for v in c_last], [Array(v) for v in h_last], Array(top.value)
+
+
 def gru_sequence(xs, h0, W, U, b):
     """The GRU step along xs [T, B, I] from the state h0 (GRU::activate_sequence): (states [T, B, H], last state)."""
     keep = [as_array(v) for v in (xs, h0, W, U, b)]

@@ -137,6 +137,11 @@ int dali_fe_lstm_sequence(dali_array_t xs, dali_array_t h0, dali_array_t c0, dal
  * [H(l-1) + I, 4 H(l)], hidden-state rows first. c_new and h_new receive `layers` handles each. */
 int dali_fe_stacked_lstm_step(dali_array_t x, int layers, const dali_array_t* h, const dali_array_t* c, const dali_array_t* W,
                               const dali_array_t* U, const dali_array_t* b, int shortcut, dali_array_t* c_new, dali_array_t* h_new);
+/* The stack along a sequence xs [T, B, I] (AbstractStackedLSTM::activate_sequence, dali/layers/stacked_lstm.cpp:44-51): the
+ * final memory and hidden state of every layer and the hidden states [T, B, H] of the top layer */
+int dali_fe_stacked_lstm_sequence(dali_array_t xs, int layers, const dali_array_t* h, const dali_array_t* c, const dali_array_t* W,
+                                  const dali_array_t* U, const dali_array_t* b, int shortcut, dali_array_t* c_last, dali_array_t* h_last,
+                                  dali_array_t* top_states);
 /* One GRU step, layers packed reset / update / candidate along the columns of W[I,3H], U[H,3H], b[3H]
  * (dali/layers/gru.cpp:27-44) */
 dali_array_t dali_fe_gru_step(dali_array_t x, dali_array_t h, dali_array_t W, dali_array_t U, dali_array_t b);

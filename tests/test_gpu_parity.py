@@ -2077,6 +2077,37 @@ def test_stacked_lstm_step_matches_oracle(gpu, D, O, rng, B, I, sizes, shortcut)
             D.op.stacked_lstm_step(arr(D, X), wrap(Hs[:-1]), wrap(Cs[:-1]), wrap(Ws), wrap(Us), wrap(bs), shortcut)
 
 
+@pytest.mark.parametrize("T,B,I,sizes,shortcut", [(4, 6, 10, [12, 8], False), (3, 5, 16, [16, 16, 24], True), (5, 8, 256, [256, 256], False),
+                                                  (3, 70, 64, [64], False)])
+def test_stacked_lstm_sequence_is_the_stack_applied_in_turn(gpu, D, O, rng, T, B, I, sizes, shortcut):
+    """AbstractStackedLSTM::activate_sequence (dali/layers/stacked_lstm.cpp:44-51): the stack applied to every x(t) in turn.
+    Here every layer runs over the whole sequence before the next (the same values: layer l at step t needs layer l-1 at
+    step t and itself at step t-1 only), which lets a layer take the one-launch recurrence; checked against the step of the
+    whole stack applied in turn, by the checker and by op.stacked_lstm_step."""
+    Xs = rng.randn(T, B, I).astype(np.float32)
+    Hs = [rng.randn(B, h).astype(np.float32) for h in sizes]
+    Cs = [rng.randn(B, h).astype(np.float32) for h in sizes]
+    ins = [I] + [sizes[l - 1] + (I if shortcut else 0) for l in range(1, len(sizes))]
+    Ws = [(rng.uniform(-1, 1, (n, 4 * h)) / np.sqrt(n + h)).astype(np.float32) for n, h in zip(ins, sizes)]
+    Us = [(rng.uniform(-1, 1, (h, 4 * h)) / np.sqrt(2 * h)).astype(np.float32) for h in sizes]
+    bs = [(rng.randn(4 * h) * 0.1).astype(np.float32) for h in sizes]
+    wrap = lambda vs: [arr(D, v) for v in vs]
+    c_last, h_last, top = D.op.stacked_lstm_sequence(arr(D, Xs), wrap(Hs), wrap(Cs), wrap(Ws), wrap(Us), wrap(bs), shortcut)
+    assert len(c_last) == len(h_last) == len(sizes) and top.shape == (T, B, sizes[-1])
+    want_c, want_h, dev_c, dev_h = Cs, Hs, wrap(Cs), wrap(Hs)
+    for t in range(T):
+        want_c, want_h = O.stacked_lstm_step(Xs[t], want_h, want_c, Ws, Us, bs, shortcut)
+        dev_c, dev_h = D.op.stacked_lstm_step(arr(D, Xs[t]), dev_h, dev_c, wrap(Ws), wrap(Us), wrap(bs), shortcut)
+        close(top.numpy()[t], want_h[-1], rtol=3e-4, atol=3e-5)
+        close(top.numpy()[t], dev_h[-1].numpy(), rtol=2e-4, atol=2e-5)
+    for l in range(len(sizes)):
+        close(c_last[l].numpy(), want_c[l], rtol=3e-4, atol=3e-5)
+        close(h_last[l].numpy(), want_h[l], rtol=3e-4, atol=3e-5)
+    assert np.array_equal(h_last[-1].numpy(), top.numpy()[-1])
+    with pytest.raises(D.DaliError, match="Activating LSTM stack of size %d with different number of states" % len(sizes)):
+        D.op.stacked_lstm_sequence(arr(D, Xs), wrap(Hs) + [arr(D, Hs[0])], wrap(Cs), wrap(Ws), wrap(Us), wrap(bs), shortcut)
+
+
 @pytest.mark.parametrize("shape", [(3,), (2, 3, 4), (5, 257), (64, 1024), (3, 5000)])
 def test_circular_convolution_matches_oracle(gpu, D, O, rng, shape):
     # JITTests.circular_convolution / _broadcast / _1d (circular_convolution_tests.cpp:54-89)
