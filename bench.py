@@ -376,7 +376,29 @@ def main():
                                 "TFLOP/s": round(2.0 * Bq * 1024 * 32000 / pus / 1e6, 2)}
             del hq, prec
         configs["c5_lstm_step_256x1024x1024"]["dot_few_rows_Bx1024x32000"] = proj
-        del Wp
+
+        # a whole decoder step around those pieces: embedding rows, two LSTM layers, the output projection, the loss and its gradient
+        emb = D.Array.from_numpy((np.random.RandomState(40).randn(32000, 1024) * 0.1).astype(np.float32))
+        lim_d = np.sqrt(6.0 / (1024 + 4096))
+        Wd = [D.Array.from_numpy(np.random.RandomState(41 + i).uniform(-lim_d, lim_d, (1024, 4096)).astype(np.float32)) for i in range(4)]
+        bd = [D.Array.zeros((4096,)) for _ in range(2)]
+        step = {}
+        for Bq in (8, 64):
+            rs = np.random.RandomState(50 + Bq)
+            ids, tgt = (D.Array.from_numpy(rs.randint(0, 32000, size=Bq).astype(np.int32)) for _ in range(2))
+            hd = [D.Array.from_numpy(rs.randn(Bq, 1024).astype(np.float32)) for _ in range(2)]
+            cd = [D.Array.from_numpy(rs.randn(Bq, 1024).astype(np.float32)) for _ in range(2)]
+            with D.Recording() as srec:
+                xq = op.gather(emb, ids)
+                c1, h1 = op.lstm_step(xq, hd[0], cd[0], Wd[0], Wd[1], bd[0])
+                c2, h2 = op.lstm_step(h1, hd[1], cd[1], Wd[2], Wd[3], bd[1])
+                lossq = op.softmax_cross_entropy(op.dot(h2, Wp), tgt)
+            sus = time_recording(srec, 20)
+            weights_bytes = (4 * 1024 * 4096 + 1024 * 32000) * 4
+            step["B%d" % Bq] = {"us": round(sus, 2), "launches": srec.launches, "weights_from_hbm_bound_us": round(weights_bytes / HBM_PEAK_GBS / 1e3, 2)}
+            del ids, tgt, hd, cd, srec, xq, c1, h1, c2, h2, lossq
+        configs["c5_lstm_step_256x1024x1024"]["decoder_step_2xLSTM1024_vocab32000"] = step
+        del Wp, emb, Wd, bd
 
         # rows beyond the five configs: embedding-style gather and its scatter-add (table [32000, 1024], 8192 indices)
         V, Dm, Nidx = 32000, 1024, 8192

@@ -28,11 +28,12 @@ static bool col_buffer_layout(const Expr* e, const std::vector<int>& shape, int 
         expect *= shape[d];
     }
     int64_t bs = 0;
-    expect = -1;
+    bool first = true;  // (a flag of its own: with a reversed axis the expected stride is itself negative)
     for (int d = split - 1; d >= 0; --d) {
         if (shape[d] == 1) continue;
-        if (expect < 0) {
+        if (first) {
             bs = st[d];
+            first = false;
         } else if (st[d] != expect) {
             return false;
         }
