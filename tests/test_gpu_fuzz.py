@@ -277,3 +277,143 @@ def test_random_index_and_dtype_nodes(gpu, D, seed):
         e = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True))
         ref = e / e.sum(axis=1, keepdims=True)
         assert (np.abs(sm - ref) <= ((1e-5 + Cn * 2.0 ** -24) if dtype is np.float32 else 1e-12) * ref + 1e-30).all()
+
+
+# ------------------------------------------------------------------------------------------ views under consumers
+# Random chains of view operations (transposes with any permutation, slices with any start, end and step including
+# negative ones, plucked axes, inserted and removed unit axes) over bases of one to five dimensions, mirrored in numpy,
+# then one random consumer: a map against a broadcast operand, sums over any subset of axes, extrema and their
+# positions along any axis, softmax along any axis, a running sum, a normalisation by a kept-dims sum, a mean, a
+# product with a matrix, and assignment (=, +=, -=) into a strided, partly reversed view of a destination.
+VIEW_EXTENTS = [1, 2, 3, 5, 8, 9, 16, 17, 33, 64, 100]
+
+
+def _random_view(D, rng, max_elems=150000):
+    nd = rng.randint(1, 6)
+    while True:
+        shape = tuple(int(VIEW_EXTENTS[rng.randint(len(VIEW_EXTENTS))]) for _ in range(nd))
+        if np.prod(shape) <= max_elems:
+            break
+    x = rng.uniform(-2, 2, shape).astype(np.float32)
+    a, r = D.Array.from_numpy(x), x
+    desc = ["base%s" % (shape,)]
+    for _ in range(rng.randint(0, 4)):
+        kind = rng.randint(0, 6)
+        if kind == 0 and r.ndim >= 2:
+            perm = tuple(int(v) for v in rng.permutation(r.ndim))
+            a, r = a.transpose(*perm), r.transpose(perm)
+            desc.append("T%s" % (perm,))
+        elif kind == 1:
+            ax = rng.randint(r.ndim)
+            n = r.shape[ax]
+            step = int(rng.choice([1, 1, 2, 3, -1, -2]))
+            lo = rng.randint(0, n)
+            hi = rng.randint(lo + 1, n + 1)
+            key = tuple(slice(lo, hi, abs(step)) if d == ax else slice(None) for d in range(r.ndim))
+            a, r = a[key], r[key]
+            if step < 0:
+                key = tuple(slice(None, None, -1) if d == ax else slice(None) for d in range(r.ndim))
+                a, r = a[key], r[key]
+            desc.append("S(ax%d,%d:%d:%d)" % (ax, lo, hi, step))
+        elif kind == 2 and r.ndim >= 2:
+            ax = rng.randint(r.ndim)
+            i = rng.randint(r.shape[ax])
+            a, r = a.pluck_axis(ax, i), np.take(r, i, axis=ax)
+            desc.append("P(ax%d,%d)" % (ax, i))
+        elif kind == 3 and r.ndim <= 4:
+            ax = rng.randint(r.ndim + 1)
+            a, r = a.expand_dims(ax), np.expand_dims(r, ax)
+            desc.append("E(%d)" % ax)
+        elif kind == 4:
+            ones = [d for d in range(r.ndim) if r.shape[d] == 1]
+            if ones and r.ndim >= 2:
+                ax = ones[rng.randint(len(ones))]
+                a, r = a.squeeze(ax), np.squeeze(r, ax)
+                desc.append("Q(%d)" % ax)
+    return a, r, " ".join(desc)
+
+
+def _view_case(D, seed):
+    """One case; returns a description of the failure or None."""
+    op = D.op
+    rng = np.random.RandomState(900000 + seed)
+    a, r, desc = _random_view(D, rng)
+    r64 = r.astype(np.float64)
+    nd = r.ndim
+    kind = rng.randint(0, 10)
+
+    def judge(name, got, want, tol=2e-5, exact=False):
+        got, want = np.asarray(got), np.asarray(want)
+        where = "seed %d %s on %s [%s]" % (seed, name, desc, D.last_kernel_kinds())
+        if got.shape != want.shape and not (got.size == 1 and want.size == 1):
+            return "%s: shape %s, expected %s" % (where, got.shape, want.shape)
+        got = got.reshape(want.shape)
+        if exact:
+            return None if np.array_equal(got, want) else "%s: %d of %d positions differ" % (where, int((got != want).sum()), want.size)
+        err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+        bound = tol * np.abs(want) + 2e-6
+        return None if (err <= bound).all() else "%s: max error %g, %d of %d values off" % (where, err.max(), int((err > bound).sum()), err.size)
+
+    if kind == 0:
+        b = rng.uniform(0.5, 1.5, r.shape).astype(np.float32)
+        if rng.randint(2):
+            ax = rng.randint(nd)
+            bs = list(r.shape); bs[ax] = 1
+            b = rng.uniform(0.5, 1.5, bs).astype(np.float32)
+        return judge("map", (op.tanh(a) * D.Array.from_numpy(b) + 0.25).numpy(), np.tanh(r64) * b + 0.25)
+    if kind == 1:
+        axes = sorted(set(int(v) for v in rng.choice(nd, size=rng.randint(1, nd + 1), replace=False)))
+        keep = bool(rng.randint(2))
+        return judge("sum over %s" % axes, op.sum(op.abs(a), axes, keep).numpy(), np.abs(r64).sum(axis=tuple(axes), keepdims=keep), tol=3e-5)
+    if kind == 2:
+        ax, keep = rng.randint(nd), bool(rng.randint(2))
+        f, nf = ((op.max, np.max) if rng.randint(2) else (op.min, np.min))
+        return judge("extremum along %d" % ax, f(a * 1.5, [ax], keep).numpy(), nf(r64 * 1.5, axis=ax, keepdims=keep))
+    if kind == 3:
+        ax = rng.randint(nd)
+        f, nf = ((op.argmax, np.argmax) if rng.randint(2) else (op.argmin, np.argmin))
+        # the reference swaps the reduced axis with the last one (reducer_operation.cpp:699-707): the kept axes come out in
+        # that order; one dimension: the position as a scalar of the input's dtype (:681-684)
+        want = nf(np.swapaxes(r, ax, -1), axis=-1).astype(np.int32) if nd > 1 else np.float32(nf(r))
+        return judge("position of the extremum along %d" % ax, f(a, ax).numpy(), want, exact=True)
+    if kind == 4:
+        ax = rng.randint(nd)
+        e = np.exp(r64 - r64.max(axis=ax, keepdims=True))
+        return judge("softmax along %d" % ax, op.softmax(a, ax).numpy(), e / e.sum(axis=ax, keepdims=True), tol=3e-5)
+    if kind == 5:
+        return judge("running sum", op.cumsum(op.abs(a)).numpy(), np.cumsum(np.abs(r64), axis=-1), tol=3e-5)
+    if kind == 6:
+        wide = rng.uniform(-1, 1, tuple(2 * s for s in r.shape)).astype(np.float32)
+        dw = D.Array.from_numpy(wide)
+        key = tuple(slice(None, None, 2) for _ in r.shape)
+        if rng.randint(2):
+            key = tuple(slice(1, None, 2) if d % 2 else slice(None, None, -2) for d in range(nd))
+        dest, mode = dw[key], rng.randint(0, 3)
+        expr, ref, val = op.sigmoid(a) * 2.0, wide.astype(np.float64).copy(), 2.0 / (1.0 + np.exp(-r64))
+        if mode == 0:
+            dest.assign(expr); ref[key] = val
+        elif mode == 1:
+            dest += expr; ref[key] += val
+        else:
+            dest -= expr; ref[key] -= val
+        return judge("assignment %d into %s" % (mode, key), dw.numpy(), ref)
+    if kind == 7 and nd >= 2:
+        ax = rng.randint(nd)
+        pos, rpos = op.abs(a) + 0.5, np.abs(r64) + 0.5
+        return judge("normalisation along %d" % ax, (pos / op.sum(pos, [ax], True)).numpy(), rpos / rpos.sum(axis=ax, keepdims=True), tol=3e-5)
+    if kind == 8 and nd == 2:
+        n = int(rng.choice([1, 7, 64, 130]))
+        b = rng.uniform(-1, 1, (r.shape[1], n)).astype(np.float32)
+        db = D.Array.from_numpy(np.ascontiguousarray(b.T)).T if rng.randint(2) else D.Array.from_numpy(b)
+        want = r64 @ b.astype(np.float64)
+        got = op.dot(a, db).numpy()
+        err = np.abs(got - want).max() if want.size else 0.0
+        scale = (np.abs(r64) @ np.abs(b)).max() + 1e-6 if want.size else 1.0
+        return None if err <= 1e-5 * scale else "seed %d product on %s [%s]: max error %g against a scale of %g" % (seed, desc, D.last_kernel_kinds(), err, scale)
+    return judge("mean of squares", op.mean(op.square(a)).numpy(), (r64 * r64).mean(), tol=3e-5)
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_views_under_random_consumers(gpu, D, block):
+    failures = [f for f in (_view_case(D, seed) for seed in range(block * 300, (block + 1) * 300)) if f]
+    assert not failures, "%d of 300 cases failed, the first: %s" % (len(failures), failures[0])
