@@ -989,7 +989,10 @@ Array gather(const Array& source, const Array& indices) {
     Array idx1 = indices.ndim() == 1 ? indices : indices.reshape({-1});
     std::vector<int> shape = indices.shape();
     shape.insert(shape.end(), source.shape().begin() + 1, source.shape().end());
-    return make_node(Kind::GATHER, "", {src2, idx1}, shape, source.dtype());
+    Array node = make_node(Kind::GATHER, "", {src2, idx1}, shape, source.dtype());
+    if (source.ndim() > 2 && source.is_buffer() && !(src2.is_buffer() && src2.expression()->memory == source.expression()->memory))
+        node.expression()->origin = {source};  // the [V, D] form is a copy: assignments go through the view (jit_scatter.cpp)
+    return node;
 }
 
 // dali/array/expression/assignment.cpp:92-126: left += sum of right over the axes where left has extent 1

@@ -49,6 +49,10 @@ struct Expr {
     double dvalue = 0.0;
     int ivalue = 0;
 
+    // GATHER over a source of more than two dimensions whose trailing axes do not merge into one (a strided view): args[0]
+    // is then a dense copy, good for reading; an assignment through the node must reach the view itself, kept here
+    std::vector<Array> origin;
+
     int axis = 0;   // EXPAND_DIMS
     int depth = 0;  // ONE_HOT
 

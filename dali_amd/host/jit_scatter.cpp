@@ -380,6 +380,18 @@ static void run_scatter_to_rows(const Array& dest2d, const Array& idx, OPERATOR_
 // dest is a lazy gather / gather_from_rows node over a buffer: write through it
 void scatter_assign(const Array& dest, OPERATOR_T op, const Array& source) {
     auto de = dest.expression();
+    if (!de->origin.empty()) {
+        // The rows of the destination view are not contiguous pieces of memory (strided trailing axes): the rows are
+        // scattered into a dense copy taken now, which then goes back into the view. (The reference indexes such a view
+        // element by element, dali/array/op/gather.cpp:89-97; here the kernels want [V, D] rows.)
+        const Array view = de->origin[0];
+        Array dense = view.reshape({view.shape()[0], -1});
+        DALI_ASSERT(dense.is_buffer(), "internal: the dense form of a scatter destination is not a buffer");
+        Array through = op::gather(dense, de->args[1]);
+        scatter_assign(through, op, source);
+        evaluate_into(view, OPERATOR_T_EQL, dense.reshape(view.shape()));
+        return;
+    }
     Array target = de->args[0], idx = de->args[1];
     DALI_ASSERT(target.is_buffer(), "assignment through a gather needs an evaluated buffer as its source (dali/array/op/gather.cpp:126-128)");
     if (!idx.is_buffer()) idx.eval();

@@ -417,3 +417,53 @@ def _view_case(D, seed):
 def test_random_views_under_random_consumers(gpu, D, block):
     failures = [f for f in (_view_case(D, seed) for seed in range(block * 300, (block + 1) * 300)) if f]
     assert not failures, "%d of 300 cases failed, the first: %s" % (len(failures), failures[0])
+
+
+# ------------------------------------------------------------------------------------------ gather and scatter through views
+def _gather_case(D, seed):
+    """A table that is a strided, possibly reversed view of one to three dimensions, read and written through an index
+    vector that is itself a strided view (dali/array/op/gather.cpp:14-28,89-143): rows picked, rows added to (with
+    repeated indices) and an expression subtracted, against numpy's take / add.at / subtract.at on the same view."""
+    op = D.op
+    rng = np.random.RandomState(70000 + seed)
+    V = int(rng.choice([1, 3, 17, 100, 1000]))
+    inner = tuple(int(v) for v in rng.choice([1, 2, 5, 16, 33, 64], size=rng.randint(0, 3)))
+    wide = rng.uniform(-1, 1, (2 * V,) + tuple(2 * s for s in inner)).astype(np.float32)
+    tv = rng.randint(0, 4)
+    key = (slice(None, None, 2),) + tuple(slice(None, None, 2) for _ in inner)
+    if tv == 1:
+        key = (slice(1, None, 2),) + tuple(slice(None, None, -2) for _ in inner)
+    if tv == 2:
+        key = (slice(None, None, -2),) + tuple(slice(1, None, 2) for _ in inner)
+    if tv == 3:
+        wide = rng.uniform(-1, 1, (V,) + inner).astype(np.float32)
+        key = tuple(slice(None) for _ in wide.shape)
+    dw = D.Array.from_numpy(wide)
+    table, rt = dw[key], wide[key]
+    n = int(rng.choice([1, 2, 7, 64, 300, 5000]))
+    idx_wide = rng.randint(0, V, size=2 * n).astype(np.int32)
+    ik = slice(None, None, 2) if rng.randint(2) else slice(None, None, -2)
+    idx, ri = D.Array.from_numpy(idx_wide)[ik], idx_wide[ik]
+    what = "seed %d: %d rows of %s, table view %d, %d indices" % (seed, V, inner, tv, n)
+    kind = rng.randint(0, 3)
+    if kind == 0:
+        return None if np.array_equal(op.gather(table, idx).numpy(), rt[ri]) else what + ": picked rows differ [%s]" % D.last_kernel_kinds()
+    vals = rng.uniform(-1, 1, (n,) + rt.shape[1:]).astype(np.float32)
+    ref = wide.astype(np.float64).copy()
+    view = ref[key]
+    g = table[idx]
+    if kind == 1:
+        g += D.Array.from_numpy(vals)
+        np.add.at(view, ri, vals.astype(np.float64))
+    else:
+        g -= op.tanh(D.Array.from_numpy(vals))
+        np.subtract.at(view, ri, np.tanh(vals.astype(np.float64)))
+    err = np.abs(dw.numpy() - ref)
+    most = np.bincount(ri, minlength=V).max()
+    return None if (err <= 4e-6 * (most + 1) + 1e-6).all() else what + ": scatter %d off by %g [%s]" % (kind, err.max(), D.last_kernel_kinds())
+
+
+@pytest.mark.parametrize("block", range(3))
+def test_random_gathers_and_scatters_through_views(gpu, D, block):
+    failures = [f for f in (_gather_case(D, seed) for seed in range(block * 300, (block + 1) * 300)) if f]
+    assert not failures, "%d of 300 cases failed, the first: %s" % (len(failures), failures[0])
