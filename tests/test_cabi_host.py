@@ -244,3 +244,18 @@ def test_scope_observers_see_the_planned_kernels(D, rng):
     assert [e[0] for e in outer.events] == ["enter", "exit"] * 3 and all(e[2] == 1 for e in outer.events)
     assert seen[0] == ("in", names[0], (names[0],)) and seen[1] == ("out", names[0], (names[0],)) and len(seen) == 6
     assert outer.trace == [] and names[0].endswith("]")
+
+
+def test_kept_leading_axes_with_a_reversed_axis_are_not_one_batch_axis(D, rng):
+    """A reduction along a middle axis reads its kept leading axes as one batch axis only when their strides nest. With a
+    reversed axis among them (strides 36, -18 for extents 2, 2) they do not: the plan must not be the batched column kernel
+    (generation only; the values are checked on the device)."""
+    op = D.op
+    x = rng.randn(2, 2, 2, 9).astype(np.float32)
+    D.generate_only([op.max(op.tanh(D.Array.from_numpy(x)), [2], True)])
+    assert D.last_kernel_kinds() == "col" and "k_batch" in D.last_source()  # contiguous: one launch, batched
+    D.generate_only([op.max(op.tanh(D.Array.from_numpy(x)[:, ::-1]), [2], True)])
+    assert "k_batch" not in D.last_source()
+    # reversed along the reduced axis itself, or along the innermost kept axis: the batch axes still nest
+    D.generate_only([op.max(op.tanh(D.Array.from_numpy(x)[:, :, ::-1]), [2], True)])
+    assert D.last_kernel_kinds().count("col") <= 1
