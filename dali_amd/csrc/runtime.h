@@ -32,6 +32,12 @@ int sort_scratch_init(int device);
 int sgemm_skinny(bool tb, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb, float beta, float* C, int ldc);
 // the same for an inner extent of at most 64 against a large C (ta: A stored as [K][M]): bound by writing C once
 int sgemm_smallk(bool ta, bool tb, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb, float beta, float* C, int ldc);
+// sgemm_dma.hip: row-major C[M, N] = alpha * sum_s A_s . B_s + beta * C for one or two terms of whole 64-deep slabs through
+// the kernel whose operand slabs are written into LDS by the loads themselves (ta: A_s stored as [K][M], tb: B_s stored as
+// [N][K]; one pair of leading dimensions). With `bias` the sums go through the LSTM gate arithmetic instead of into C
+// (N = 4 H, columns gathered per hidden unit). 1: launched; 0: not a case for it; -1: failure (message set)
+int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
+              float alpha, float beta, float* C, int ldc, const float* bias, const float* c_prev, float* c_out, float* h_out, int H);
 // lstm_persistent.hip: 1 when a persistent kernel's grid barrier gave up since the last call (and clears that)
 int persistent_status_take();
 

@@ -25,24 +25,13 @@
 // DEPTH slabs ahead of their use, written to the other LDS buffer one slab ahead,
 // and consumed from LDS while the MFMA pipe works (one barrier per slab).
 #include "runtime.h"
+#include "gate_math.h"
 
 #include <cstdlib>
 #include <cstring>
 #include <type_traits>
 
 namespace dali_hip {
-
-// exp of the gate epilogue: the same sequence as the exp of the generated kernels (dali_expf in the device prelude of the
-// front-end), so that the fused step and the two-launch form round every gate identically.
-__device__ __forceinline__ float gate_expf(float x) {
-    const float c = 0x1.715476p+0f, cc = 0x1.4ae0bep-26f;
-    const float t = x * c;
-    float r = __builtin_fmaf(x, c, -t);
-    r = __builtin_fmaf(x, cc, r);
-    const float e = __builtin_amdgcn_exp2f(t);
-    const float fixed = __builtin_fmaf(e, r * 0x1.62e430p-1f, e);
-    return __builtin_fabsf(t) < 128.0f ? fixed : e;
-}
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -842,7 +831,19 @@ static int run_tile(const GemmArgs& g, bool ta, bool tb, bool vec, int split_k) 
         }
     }
     if (whole.nseg > 0) {
-        int st = launch_tile<BM, BN, BK, DEPTH, KW, MIDB>(whole, ta, tb, true, split_k, false);
+        int st = 0;
+        bool done = false;
+        if (BM == 64 && BN == 64 && BK == 64 && KW == 2 && !MIDB && split_k == 1 && whole.nseg <= 2 && !whole.map_on) {
+            // small grids of whole slabs: the kernel that has its operand slabs written into LDS by the loads themselves
+            const float* as[2] = {whole.seg[0].A, whole.seg[1].A};
+            const float* bs[2] = {whole.seg[0].B, whole.seg[1].B};
+            const int ks[2] = {whole.seg[0].K, whole.seg[1].K};
+            const int r = sgemm_dma(ta, tb, whole.M, whole.N, whole.nseg, ks, as, bs, whole.seg[0].lda, whole.seg[0].ldb, whole.alpha, whole.beta,
+                                    whole.C, whole.ldc, nullptr, nullptr, nullptr, nullptr, 0);
+            if (r < 0) return DALI_HIP_ERROR;
+            done = r > 0;
+        }
+        if (!done) st = launch_tile<BM, BN, BK, DEPTH, KW, MIDB>(whole, ta, tb, true, split_k, false);
         if (st || rest.nseg == 0) return st;
         rest.beta = 1.0f;
     }
@@ -1024,6 +1025,14 @@ int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx
     if (!ok)
         return fail("lstm_step: the fused kernel needs input and hidden sizes that are multiples of 64, 16-byte aligned operands and "
                     "equal leading dimensions for X / Hprev and for W / U");
+    {
+        const float* as[2] = {X, Hprev};
+        const float* bs[2] = {W, U};
+        const int ks[2] = {input, hidden};
+        const int r = sgemm_dma(false, false, batch, 4 * hidden, 2, ks, as, bs, ldx, ldw, 1.0f, 0.0f, nullptr, 0, bias, Cprev, Cout, Hout, hidden);
+        if (r < 0) return DALI_HIP_ERROR;
+        if (r > 0) return DALI_HIP_OK;
+    }
     GemmArgs g = {};
     g.nseg = 2;
     g.seg[0].A = X;

@@ -1,0 +1,402 @@
+// fp32 GEMM for small grids (at most a few 64x64 tiles of C per CU; the LSTM step is exactly one): the memory pipeline
+// writes the operand slabs into LDS itself (global_load_lds_dwordx4), four slabs are in flight, and the waves do
+// nothing but read operands from LDS and issue v_mfma_f32_16x16x4_f32.
+//
+// Row-major view: C[M,N] = alpha * sum_s A_s[M,K_s] * B_s[K_s,N] + beta * C for one or two terms (dali_hip_sgemm,
+// dali_hip_sgemm_pair, dali_hip_lstm_step; the reference's call is dali/array/gemm/cublas_gemm.cu:153-166).
+//
+// What shaped it (measured on MI355X with timestamps inside the kernel, one 64x64 tile over K = 2048 per CU):
+//  * with every CU busy the fp32 matrix pipe is held back by power, not by issue: the shader clock settles near
+//    2.05 GHz on random operands (2.25 GHz on zeros), so cycles saved in the loop come back as a lower clock unless
+//    energy is saved with them. Staging through registers (global load, ds_write) and 32x32x2 instructions (which
+//    read and write a 4 KiB accumulator per 4096 flops) both cost energy; loads straight into LDS and 16x16x4
+//    instructions (half the accumulator traffic) gave 44.3 -> 36.4 us for the LSTM pair on the same device.
+//  * one workgroup barrier per slab is enough, and it costs nothing when it sits inside the first k-group of a slab:
+//    at that point a wave has the operands of its next k-group in registers, the barrier proves that every wave's
+//    loads of slab i+1 have landed (they are first read in the second k-group) and that slab i-1 is no longer read,
+//    and the loads of slab i+3 are issued into the buffer of slab i-1 one matrix instruction later (issuing them
+//    right behind the barrier delayed the first instruction after it: 2133 -> 2071 cycles per slab of 2048).
+//  * two wave sets split the k-groups of a slab (two waves per SIMD cover each other's waits: 2316 -> 2071 cycles)
+//    and exchange halves of their sums through LDS at the end.
+//
+// LDS: four slabs of A, then four of B, 16 KiB each, no padding. An operand whose k runs along memory rows
+// (A [M,K], B stored [N,K]) is kept as [row][k] with the 16-byte granule g of row r in slot (g ^ r) & 15: the 16 lanes
+// of an operand read (same granule, consecutive rows) hit 16 different slots. An operand whose k runs across rows
+// (B [K,N], A stored [K,M]) is kept as [k][col] with granule g of row k in slot g ^ (((k >> 2) & 3) << 2): the four lane
+// groups of an operand read (k, k+4, k+8, k+12, sixteen consecutive columns each) hit the four quarters of a bank row.
+// A lane of a load always writes LDS bytes [16 * lane, 16 * lane + 16) of its 1 KiB chunk, so the permutation is
+// applied to the global address the lane fetches.
+#include "runtime.h"
+
+#include <cstdlib>
+#include <type_traits>
+
+#include "gate_math.h"
+
+namespace dali_hip {
+
+namespace {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kStage = 16384;          // bytes of one operand's slab: 64 x 64 floats
+constexpr int kBRegion = 4 * kStage;   // the B slabs follow the four A slabs
+constexpr int kDmaLds = 8 * kStage;
+
+struct DmaArgs {
+    const float* A[2];
+    const float* B[2];
+    int slabs[2];  // 64-deep slabs per term (the second is 0 for a single product)
+    int lda, ldb;
+    int M, N;
+    float* C;
+    int ldc;
+    float alpha, beta;
+    // gate epilogue (GATES): C is not written; see gate_math.h
+    const float* bias;
+    const float* c_prev;
+    float* c_out;
+    float* h_out;
+    int H;
+};
+
+// One 16-byte piece per lane from global memory straight into LDS: lane l writes bytes [16 l, 16 l + 16) behind
+// `lds_addr` (wave-uniform, goes through M0); the source is base + voff.
+__device__ __forceinline__ void dma16(unsigned lds_addr, unsigned voff, const char* base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+// The compiler does not see these loads, so the waits for them are written out; they are also compiler barriers.
+__device__ __forceinline__ void wait_loads_but_4() { asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); }
+__device__ __forceinline__ void wait_loads_but_8() { asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); }
+__device__ __forceinline__ void wait_loads_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// TA: A stored as [K][M]; TB: B stored as [N][K]. 512 threads: waves 0-3 (wave set 0) and 4-7 (set 1) each cover the
+// 64x64 tile as 2x2 wave tiles of 32x32; set kw takes the k-groups (16 k) kw and kw + 2 of every slab.
+template <bool TA, bool TB, bool GATES>
+__global__ __launch_bounds__(512, 1) void sgemm_dma_kernel(DmaArgs g) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = w & 3, kw = w >> 2;
+    const int wm = wave >> 1, wn = wave & 1, l16 = lane & 15, kq = lane >> 4;
+    const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+    const int M = g.M, N = g.N;
+    // Gate epilogue: the tile's columns are the four gates of sixteen hidden units. Workgroups are dealt to the eight
+    // XCDs round-robin, so consecutive groups of hidden units go to workgroups of the same XCD: both 64-byte halves
+    // of a 128-byte line of the weights are then asked for by the same L2.
+    const int hu_base = GATES ? 16 * (gridDim.x % 8 == 0 ? (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8 : blockIdx.x) : 0;
+
+    // gate epilogue operands first: they are then older than every load below, which keeps the counted waits exact
+    float gate_bias[2][4], gate_c[2];
+    if constexpr (GATES) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int e = tid + q * 512, r = e / 16, j = e % 16, hu = hu_base + j;
+            const int m = m0 + r < M ? m0 + r : M - 1;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) gate_bias[q][k] = g.bias[k * g.H + hu];
+            gate_c[q] = g.c_prev[(size_t)m * g.H + hu];
+        }
+    }
+
+    // Sources of this wave's four loads per slab (byte offsets, constant over the kernel) and their LDS chunks.
+    // Tiles that hang over the edge of C fetch the last valid row (or granule) instead: what they compute for rows and
+    // columns outside C is never stored.
+    unsigned a_off[2], b_off[2], a_dst[2], b_dst[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int c = w + 8 * q;                         // 1 KiB chunk: LDS rows 4c .. 4c+3 of the slab
+        const int r = 4 * c + (lane >> 4), s = lane & 15;  // LDS row and slot of this lane's piece
+        if (!TA) {
+            const int row = m0 + r < M ? m0 + r : M - 1;
+            a_off[q] = (unsigned)(((size_t)row * g.lda + 4 * ((s ^ r) & 15)) * sizeof(float));
+        } else {
+            int col = m0 + 4 * (s ^ ((c & 3) << 2));
+            col = col < M ? col : M - 4;
+            a_off[q] = (unsigned)(((size_t)r * g.lda + col) * sizeof(float));
+        }
+        if (!TB) {
+            const int gr = s ^ ((c & 3) << 2);
+            int col = GATES ? (gr / 4) * g.H + hu_base + 4 * (gr % 4) : n0 + 4 * gr;
+            col = col < N ? col : N - 4;
+            b_off[q] = (unsigned)(((size_t)r * g.ldb + col) * sizeof(float));
+        } else {
+            const int row = n0 + r < N ? n0 + r : N - 1;
+            b_off[q] = (unsigned)(((size_t)row * g.ldb + 4 * ((s ^ r) & 15)) * sizeof(float));
+        }
+        a_dst[q] = (unsigned)(c * 1024);
+        b_dst[q] = (unsigned)(kBRegion + c * 1024);
+    }
+    const char* ap = (const char*)g.A[0];
+    const char* bp = (const char*)g.B[0];
+    const long a_step = (TA ? (long)64 * g.lda : 64L) * (long)sizeof(float);
+    const long b_step = (TB ? 64L : (long)64 * g.ldb) * (long)sizeof(float);
+    const int slabs0 = g.slabs[0];
+    const int n = slabs0 + g.slabs[1];
+    int fj = 0;  // next slab to request
+    auto issue = [&](int stage) __attribute__((always_inline)) {
+        dma16(a_dst[0] + stage * kStage, a_off[0], ap);
+        dma16(a_dst[1] + stage * kStage, a_off[1], ap);
+        dma16(b_dst[0] + stage * kStage, b_off[0], bp);
+        dma16(b_dst[1] + stage * kStage, b_off[1], bp);
+        ++fj;
+        ap += a_step;
+        bp += b_step;
+        if (fj == slabs0) {
+            ap = (const char*)g.A[1];
+            bp = (const char*)g.B[1];
+        }
+    };
+    issue(0);
+    if (n > 1) issue(1);
+    if (n > 2) issue(2);
+
+    // operand addresses of this lane: [k-group of the wave set][16-row block of the wave tile]
+    unsigned a_addr[2][2], b_addr[2][2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const int t = kw + 2 * tt;
+            const int ra = wm * 32 + s * 16 + l16, rb = wn * 32 + s * 16 + l16;
+            a_addr[tt][s] = !TA ? (unsigned)(ra * 256 + (((4 * t + kq) ^ ra) & 15) * 16) : (unsigned)((16 * t + 4 * kq) * 256 + ((ra ^ (kq << 4)) * 4));
+            b_addr[tt][s] = kBRegion + (TB ? (unsigned)(rb * 256 + (((4 * t + kq) ^ rb) & 15) * 16) : (unsigned)((16 * t + 4 * kq) * 256 + ((rb ^ (kq << 4)) * 4)));
+        }
+
+    floatx4 acc[2][2];
+#pragma unroll
+    for (int si = 0; si < 2; ++si)
+#pragma unroll
+        for (int sj = 0; sj < 2; ++sj)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[si][sj][v] = 0.f;
+
+    // operands of one k-group: element c of a vector belongs to k = 16 t + 4 kq + c
+    floatx4 a4[2][2], b4[2][2];
+    auto load_ops = [&](auto ST, int tt, int o) __attribute__((always_inline)) {
+        constexpr int st = decltype(ST)::value;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            if (!TA) {
+                a4[o][s] = *(const floatx4*)(lds + a_addr[tt][s] + st * kStage);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) a4[o][s][c] = *(const float*)(lds + a_addr[tt][s] + st * kStage + c * 256);
+            }
+            if (TB) {
+                b4[o][s] = *(const floatx4*)(lds + b_addr[tt][s] + st * kStage);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) b4[o][s][c] = *(const float*)(lds + b_addr[tt][s] + st * kStage + c * 256);
+            }
+        }
+    };
+    auto mfma = [&](int o, int c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int si = 0; si < 2; ++si)
+#pragma unroll
+            for (int sj = 0; sj < 2; ++sj) acc[si][sj] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[o][si][c], b4[o][sj][c], acc[si][sj], 0, 0, 0);
+    };
+    // Slab i lives in LDS stage i % 4 (ST). The barrier inside slab i is for slab i+1; behind it the buffer of slab
+    // i-1 is free and takes slab i+3.
+    auto slab_step = [&](auto ST, auto H1, auto H2, auto H3) __attribute__((always_inline)) {
+        constexpr int st = decltype(ST)::value;
+        constexpr bool has1 = decltype(H1)::value, has2 = decltype(H2)::value, has3 = decltype(H3)::value;  // slabs i+1, i+2, i+3 exist
+        using NX = std::integral_constant<int, (st + 1) % 4>;
+        mfma(0, 0);
+        load_ops(ST, 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(0, 1);
+        if (has1) {
+            // own loads of slab i+1 done (those of slab i+2 may still be in flight), then everybody's
+            if (has2) wait_loads_but_4(); else wait_loads_all();
+            __builtin_amdgcn_s_barrier();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(0, 2);
+        if (has3) issue((st + 3) % 4);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(0, 3);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(1, 0);
+        if (has1) load_ops(NX{}, 0, 0);  // behind the barrier: slab i+1 is complete in LDS
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(1, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(1, 3);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // the last R slabs, starting in stage 0: step J of them
+    auto tail_step = [&](auto J, auto R) __attribute__((always_inline)) {
+        constexpr int j = decltype(J)::value, r = decltype(R)::value;
+        if constexpr (j < r)
+            slab_step(std::integral_constant<int, j % 4>{}, std::integral_constant<bool, (j + 1 < r)>{}, std::integral_constant<bool, (j + 2 < r)>{},
+                      std::integral_constant<bool, (j + 3 < r)>{});
+    };
+    auto run_tail = [&](auto R) __attribute__((always_inline)) {
+        tail_step(std::integral_constant<int, 0>{}, R);
+        tail_step(std::integral_constant<int, 1>{}, R);
+        tail_step(std::integral_constant<int, 2>{}, R);
+        tail_step(std::integral_constant<int, 3>{}, R);
+        tail_step(std::integral_constant<int, 4>{}, R);
+        tail_step(std::integral_constant<int, 5>{}, R);
+    };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+    using S3 = std::integral_constant<int, 3>;
+    using Yes = std::true_type;
+
+    // slab 0 has landed once at most the loads of slabs 1 and 2 are outstanding
+    if (n > 2) wait_loads_but_8();
+    else if (n > 1) wait_loads_but_4();
+    else wait_loads_all();
+    __builtin_amdgcn_s_barrier();
+    load_ops(S0{}, 0, 0);
+    int i = 0;
+    // steady state: slabs that still have three successors, four per trip so that the stage is a constant
+    for (; i + 7 <= n; i += 4) {
+        slab_step(S0{}, Yes{}, Yes{}, Yes{});
+        slab_step(S1{}, Yes{}, Yes{}, Yes{});
+        slab_step(S2{}, Yes{}, Yes{}, Yes{});
+        slab_step(S3{}, Yes{}, Yes{}, Yes{});
+    }
+    const int rest = n - i;  // 1 .. 6
+    if (rest == 1) run_tail(std::integral_constant<int, 1>{});
+    else if (rest == 2) run_tail(std::integral_constant<int, 2>{});
+    else if (rest == 3) run_tail(std::integral_constant<int, 3>{});
+    else if (rest == 4) run_tail(std::integral_constant<int, 4>{});
+    else if (rest == 5) run_tail(std::integral_constant<int, 5>{});
+    else run_tail(std::integral_constant<int, 6>{});
+
+    // The 16 sums of a lane: element e = (si * 2 + sj) * 4 + v is row wm*32 + si*16 + 4*kq + v, column wn*32 + sj*16 + l16
+    // of the tile. The stages n % 4 and (n + 1) % 4 are read by no wave any more (the last two slabs sit in the two
+    // others and every wave has passed the barrier inside slab n - 2, which it reaches after its last read of slab n - 3),
+    // so the exchange needs no barrier in front.
+    float out[16];
+#pragma unroll
+    for (int si = 0; si < 2; ++si)
+#pragma unroll
+        for (int sj = 0; sj < 2; ++sj)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) out[(si * 2 + sj) * 4 + v] = acc[si][sj][v];
+
+    if constexpr (GATES) {
+        // both wave sets write their sums as a [64][64] tile of pre-activations; every thread then finishes two
+        // (row, hidden unit) pairs. Bias and previous cell values were fetched at the start.
+        float* mine = (float*)(lds + ((n + kw) & 3) * kStage);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int r = wm * 32 + (e / 8) * 16 + 4 * kq + (e % 4), c = wn * 32 + ((e / 4) % 2) * 16 + l16;
+            mine[r * 64 + c] = out[e];
+        }
+        __syncthreads();
+        const float* t0 = (const float*)(lds + (n & 3) * kStage);
+        const float* t1 = (const float*)(lds + ((n + 1) & 3) * kStage);
+        const int H = g.H;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int e = tid + q * 512, r = e / 16, j = e % 16, m = m0 + r;
+            if (m >= M) continue;
+            float pre[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) pre[k] = t0[r * 64 + 16 * k + j] + t1[r * 64 + 16 * k + j];
+            const size_t o = (size_t)m * H + hu_base + j;
+            lstm_gates(pre[0], pre[1], pre[2], pre[3], gate_bias[q], gate_c[q], g.c_out + o, g.h_out + o);
+        }
+        return;
+    } else {
+        // wave set 0 keeps the upper 16 rows of every wave tile (e < 8), set 1 the lower; each hands the other half over
+        float* red = (float*)(lds + (n & 3) * kStage);
+#pragma unroll
+        for (int v = 0; v < 8; ++v) red[(kw * 4 + wave) * 512 + v * 64 + lane] = kw == 0 ? out[8 + v] : out[v];
+        __syncthreads();
+        const float alpha = g.alpha, beta = g.beta;
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+            const float other = red[((1 - kw) * 4 + wave) * 512 + v * 64 + lane];
+            // the term of set 0 first, whichever set adds: the sum does not depend on who keeps the element
+            const float sum = kw == 0 ? out[v] + other : other + out[8 + v];
+            const int e = kw * 8 + v;
+            const int m = m0 + wm * 32 + (e / 8) * 16 + 4 * kq + (e % 4), nn = n0 + wn * 32 + ((e / 4) % 2) * 16 + l16;
+            if (m < M && nn < N) {
+                float* c = g.C + (size_t)m * g.ldc + nn;
+                float r = alpha * sum;
+                if (beta != 0.f) r += beta * *c;
+                *c = r;
+            }
+        }
+    }
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+template <bool TA, bool TB, bool GATES>
+int launch(const DmaArgs& g, dim3 grid) {
+    static bool attribute_set = false;  // one flag per instantiation of this function template
+    auto kernel = sgemm_dma_kernel<TA, TB, GATES>;
+    if (!attribute_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kDmaLds);
+        if (e != hipSuccess) return fail("sgemm: cannot reserve %d bytes of LDS: %s", kDmaLds, hipGetErrorString(e));
+        attribute_set = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(512), kDmaLds, stream(), g);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("sgemm launch failed: %s", hipGetErrorString(e));
+    return 1;
+}
+
+}  // namespace
+
+int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
+              float alpha, float beta, float* C, int ldc, const float* bias, const float* c_prev, float* c_out, float* h_out, int H) {
+    static const int enabled = getenv("DALI_HIP_GEMM_DMA") ? atoi(getenv("DALI_HIP_GEMM_DMA")) : 1;
+    if (!enabled || nseg < 1 || nseg > 2 || M < 1 || N < 1) return 0;
+    const bool gates = bias != nullptr;
+    // whole 64-deep slabs, 16-byte pieces that start on 16-byte boundaries and never straddle the end of a row
+    if (lda % 4 != 0 || ldb % 4 != 0 || (ta && M % 4 != 0) || (!tb && N % 4 != 0)) return 0;
+    size_t a_rows = 0, b_rows = 0;
+    for (int s = 0; s < nseg; ++s) {
+        if (K[s] < 64 || K[s] % 64 != 0 || !aligned16(A[s]) || !aligned16(B[s])) return 0;
+        a_rows = ta ? (size_t)K[s] : (size_t)M;
+        b_rows = tb ? (size_t)N : (size_t)K[s];
+        // the per-lane offsets are 32-bit and relative to a pointer that walks along k
+        const size_t a_span = ((size_t)(ta ? 64 : M) * lda + (ta ? M : 64)) * sizeof(float);
+        const size_t b_span = ((size_t)(tb ? N : 64) * ldb + (tb ? 64 : N)) * sizeof(float);
+        if (a_span >= ((size_t)1 << 32) || b_span >= ((size_t)1 << 32)) return 0;
+    }
+    (void)a_rows;
+    (void)b_rows;
+    DmaArgs g = {};
+    for (int s = 0; s < 2; ++s) {
+        g.A[s] = s < nseg ? A[s] : nullptr;
+        g.B[s] = s < nseg ? B[s] : nullptr;
+        g.slabs[s] = s < nseg ? K[s] / 64 : 0;
+    }
+    g.lda = lda;
+    g.ldb = ldb;
+    g.M = M;
+    g.N = N;
+    g.C = C;
+    g.ldc = ldc;
+    g.alpha = alpha;
+    g.beta = beta;
+    g.bias = bias;
+    g.c_prev = c_prev;
+    g.c_out = c_out;
+    g.h_out = h_out;
+    g.H = H;
+    dim3 grid((N + 63) / 64, (M + 63) / 64);
+    if (gates) {
+        if (ta || tb) return 0;
+        return launch<false, false, true>(g, grid);
+    }
+    if (!ta && !tb) return launch<false, false, false>(g, grid);
+    if (!ta && tb) return launch<false, true, false>(g, grid);
+    if (ta && !tb) return launch<true, false, false>(g, grid);
+    return launch<true, true, false>(g, grid);
+}
+
+}  // namespace dali_hip
