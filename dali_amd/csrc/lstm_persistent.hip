@@ -401,7 +401,8 @@ __global__ __launch_bounds__(256) void lstm_step_small_kernel(SmallStepArgs a) {
         for (int w = 0; w < 4; ++w) s += red[w][u & 3][bb / 16][bb & 15][u >> 2];
         __hip_atomic_store(mine + e, s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    __builtin_amdgcn_s_waitcnt(0);
+    // the shares are acknowledged by memory before the ticket is drawn; the clobber keeps the compiler from moving them
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
         const unsigned int ticket = __hip_atomic_fetch_add(a.tickets + ub, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -534,13 +535,7 @@ extern "C" int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidd
     a.spin_limit = spin_env;
     hipError_t e = hipSuccess;
     auto launch = [&](auto kernel) {
-        // once per kernel (its LDS need is fixed by the template arguments): later calls, which may be recorded into a graph,
-        // are launches only
-        static bool attribute_set = false;
-        if (!attribute_set) {
-            e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            attribute_set = e == hipSuccess;
-        }
+        e = reserve_dynamic_lds((const void*)kernel, lds_bytes);
         if (e == hipSuccess) hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream(), a);
     };
     const int KQ = hidden / 64;
@@ -596,13 +591,7 @@ extern "C" int dali_hip_lstm_step_small(int batch, int input, int hidden, const 
     const size_t lds_bytes = (size_t)4 * 4 * MT * 256 * sizeof(float);
     hipError_t e = hipSuccess;
     auto launch = [&](auto kernel) {
-        // once per kernel (its LDS need is fixed by the template arguments): later calls, which may be recorded into a graph,
-        // are launches only
-        static bool attribute_set = false;
-        if (!attribute_set) {
-            e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            attribute_set = e == hipSuccess;
-        }
+        e = reserve_dynamic_lds((const void*)kernel, lds_bytes);
         if (e == hipSuccess) hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream(), a);
     };
     switch (MT) {

@@ -156,6 +156,17 @@ static int rtc_compile(const std::string& arch, const char* src, std::vector<cha
     return DALI_HIP_OK;
 }
 
+hipError_t reserve_dynamic_lds(const void* kernel, size_t bytes) {
+    static std::mutex m;
+    static std::unordered_map<const void*, size_t> reserved;
+    std::lock_guard<std::mutex> lock(m);
+    auto it = reserved.find(kernel);
+    if (it != reserved.end() && it->second >= bytes) return hipSuccess;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess) reserved[kernel] = bytes;
+    return e;
+}
+
 }  // namespace dali_hip
 
 using namespace dali_hip;

@@ -673,7 +673,8 @@ __global__ __launch_bounds__(256 * KW, (BM == 128 && !EDGE && KW == 1) ? 2 : 1) 
                     int lm = wm * WTM + ii * 32 + 8 * (v / 4) + 4 * h + (v % 4), ln = wn * WTN + jj * 32 + l32;
                     publish(mine + lm * BN + ln, acc[0][ii][jj][v]);
                 }
-        __builtin_amdgcn_s_waitcnt(0);
+        // the partial tile is acknowledged by memory before the ticket is drawn; the clobber keeps the compiler from moving the stores
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __shared__ int is_last;
         __syncthreads();
         if (tid == 0) {

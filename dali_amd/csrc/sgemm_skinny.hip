@@ -123,7 +123,8 @@ __global__ __launch_bounds__(256, 2) void sgemm_skinny_kernel(SkinnyArgs a) {
     float* mine = a.partials + ((size_t)cb * KS + ks) * (size_t)M * kCols;
     for (int e = tid; e < M * kCols; e += 256)
         __hip_atomic_store(mine + e, waves_sum(e / kCols, e % kCols), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __builtin_amdgcn_s_waitcnt(0);
+    // the shares are acknowledged by memory before the ticket is drawn; the clobber keeps the compiler from moving them
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
         const unsigned int ticket = __hip_atomic_fetch_add(a.tickets + cb, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -273,12 +274,7 @@ int sgemm_skinny(bool tb, int M, int N, int K, float alpha, const float* A, int 
     const unsigned grid = (unsigned)blocks * KS;
     hipError_t e = hipSuccess;
     auto launch = [&](auto kernel) {
-        // once per kernel: later calls, which may be recorded into a graph, are launches only
-        static bool attribute_set = false;
-        if (!attribute_set) {
-            e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            attribute_set = e == hipSuccess;
-        }
+        e = reserve_dynamic_lds((const void*)kernel, lds_bytes);
         if (e == hipSuccess) hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream(), a);
     };
     // (trips issued together: 1 to 8 measured alike, the compiler pipelines the loop; 4 is the best of them on short K shares)

@@ -61,7 +61,8 @@ __global__ __launch_bounds__(256) void rank_sort_kernel(const int32_t* keys, int
 #pragma unroll 16
     for (int t = 0; t < kRankSegment; ++t) count += tile[t] < mine ? 1 : 0;
     if (i < n) __hip_atomic_store(partial + (size_t)blockIdx.y * n + i, count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __builtin_amdgcn_s_waitcnt(0);
+    // the counts are acknowledged by memory before the ticket is drawn; the clobber keeps the compiler from moving the stores
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
         const unsigned int ticket = __hip_atomic_fetch_add(tickets + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -614,12 +615,20 @@ extern "C" int dali_hip_topk_rows(const void* x, int dtype, int64_t rows, int32_
     return fail("dali_hip_topk_rows: unknown dtype %d (0 = float, 1 = double, 2 = int32)", dtype);
 }
 
+// the outputs are written while other workgroups still read the keys: the three arrays must be distinct
+static bool argsort_arrays_overlap(const int32_t* keys, int64_t n, const int32_t* sorted_keys, const int32_t* perm) {
+    const size_t bytes = (size_t)n * sizeof(int32_t);
+    auto meet = [&](const void* a, const void* b) { return (const char*)a < (const char*)b + bytes && (const char*)b < (const char*)a + bytes; };
+    return meet(keys, sorted_keys) || meet(keys, perm) || meet(sorted_keys, perm);
+}
+
 extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_limit, int32_t* sorted_keys, int32_t* perm) {
     if (ensure_init()) return DALI_HIP_ERROR;
     if (n < 0) return fail("dali_hip_argsort_i32: negative length %lld", (long long)n);
     if (n == 0) return DALI_HIP_OK;
     if (n > 2147483647LL) return fail("dali_hip_argsort_i32: %lld keys exceed the int32 position range", (long long)n);
     if (!keys || !sorted_keys || !perm) return fail("dali_hip_argsort_i32: NULL argument");
+    if (argsort_arrays_overlap(keys, n, sorted_keys, perm)) return fail("dali_hip_argsort_i32: keys, sorted_keys and perm must not overlap");
     hipStream_t st = stream();
     // keys known to lie in [0, key_limit) need only their low bits sorted
     int end_bit = 32;
@@ -685,6 +694,7 @@ extern "C" int dali_hip_argsort_i32_noalloc(const int32_t* keys, int64_t n, int3
                     kNoAllocMaxKeys);
     if (n == 0) return DALI_HIP_OK;
     if (!keys || !sorted_keys || !perm) return fail("dali_hip_argsort_i32_noalloc: NULL argument");
+    if (argsort_arrays_overlap(keys, n, sorted_keys, perm)) return fail("dali_hip_argsort_i32_noalloc: keys, sorted_keys and perm must not overlap");
     unsigned char* base = device < kMaxDevices ? g_scratch_ptr[device] : nullptr;
     if (!base) return fail("dali_hip_argsort_i32_noalloc: no scratch address for device %d", device);
     return launch_rank_sort(keys, (int)n, key_limit, (unsigned int*)base, (int32_t*)(base + kScratchTicketBytes), sorted_keys, perm, stream());

@@ -349,10 +349,16 @@ DI void dali_publish(dali_ms* p, dali_ms v) {
 DI dali_ms dali_observe(const dali_ms* p) {
     return __builtin_bit_cast(dali_ms, __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 }
-// Waits until this thread's earlier stores are acknowledged, then draws a ticket.
+// Waits until this thread's earlier stores are acknowledged by memory; also a compiler barrier for memory operations.
+DI void dali_stores_acknowledged() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
+// Waits until this thread's earlier stores are acknowledged by memory, then draws a ticket. The wait is written as an asm
+// statement that clobbers memory: the compiler may then move neither the published stores behind it nor the ticket (or the
+// loads of the fold that follows it) in front of it.
 DI unsigned int dali_take_ticket(unsigned int* counter) {
-    __builtin_amdgcn_s_waitcnt(0);
-    return __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    const unsigned int ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("" ::: "memory");
+    return ticket;
 }
 
 // --------------------------------------------------------- cross-lane helpers

@@ -261,7 +261,7 @@ static std::string gen_col_kernel(const Program& P, int red_id, int dest_array, 
     if (ARG) ss << "  int* pidx = (int*)(partials + (long)gridDim.y * KP);  // the indices follow the values\n";
     ss << "  if (wave == 0) {\n    _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) { dali_publish(partials + (long)blockIdx.y * KP + pcol + j, acc[j]);"
        << (ARG ? " dali_publish(pidx + (long)blockIdx.y * KP + pcol + j, acci[j]);" : "") << " }\n"
-          "    __builtin_amdgcn_s_waitcnt(0);\n  }\n  __syncthreads();\n";
+          "    dali_stores_acknowledged();\n  }\n  __syncthreads();\n";
     ss << "  if (threadIdx.x == 0) is_last = dali_take_ticket(&counters[blockIdx.x]) == gridDim.y - 1;\n  __syncthreads();\n";
     ss << "  if (!is_last) return;\n";
     // every row group of the last block folds a contiguous share of the partial rows in y order (TAIL of them in

@@ -305,7 +305,8 @@ int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidden, const f
  * least-significant-digit radix sort (eight bits per pass; histogram, per-digit scan and ranked move per pass) whose temporary block comes from
  * the bank, so they fail during a capture. With key_limit > 0, keys outside the promised range come out behind
  * every key inside it (among themselves in an unspecified but stable order) and never between two equal valid
- * keys; perm is a permutation for any input.
+ * keys; perm is a permutation for any input. keys, sorted_keys and perm must not overlap (the outputs are written
+ * while the keys are still being read): a call with overlapping arrays is refused.
  */
 int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_limit, int32_t* sorted_keys, int32_t* perm);
 

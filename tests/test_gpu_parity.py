@@ -1515,6 +1515,10 @@ def test_indices_outside_the_destination_are_skipped(gpu, D, O, rng, V, N):
     order = np.argsort(idx[ok], kind="stable")
     assert np.array_equal(pm[:n_ok], np.flatnonzero(ok)[order])  # valid keys first, ordered, ties in input order
     assert not ok[pm[n_ok:]].any()
+    # the outputs are written while the keys are still read: overlapping arrays are refused, by both entry points
+    for entry in (hip.dali_hip_argsort_i32, hip.dali_hip_argsort_i32_noalloc):
+        assert entry(dk, 1000, V, dk, dp) != 0 and b"must not overlap" in hip.dali_hip_last_error()
+        assert entry(dk, 1000, V, ds, C.c_void_p(ds.value + 400)) != 0 and b"must not overlap" in hip.dali_hip_last_error()
     for p in (dk, ds, dp):
         hip.dali_hip_free(p)
     # columns outside a row, through gather_from_rows
