@@ -46,6 +46,16 @@ def traffic_from_profile(kernel):
     return int(got["traffic_bytes_per_launch"]), "profiles/softmax_c1_hbm_traffic_pmc.md (measured on %s)" % kernel
 
 
+def config_traffic():
+    """kernel name -> HBM bytes per launch from the committed counter summary of the other configurations."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic_all_configs_pmc.md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return {}
+    return {k: int(v) for _, k, v in re.findall(r"^traffic: (\S+) (\S+) (\d+)$", text, re.M)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -58,8 +68,14 @@ def main():
                          "of the headline should contain) and print a short JSON line")
     ap.add_argument("--graph", action="store_true", help="issue the timed softmax steps as HIP graph launches (one graph per group of steps)")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="counter-collection helper: 20 softmax steps on rotating buffers, then 20 plain copies of "
-                         "16,777,216 floats (64 MiB read + 64 MiB written each), nothing else; prints no JSON")
+                    help="counter-collection helper: a few dispatches of every configuration's kernels (32 softmax steps on "
+                         "rotating buffers first) and two plain copies of known size (64 MiB and 1000 MiB each way) that calibrate "
+                         "the byte counters, nothing else; prints which kernel belongs to which configuration and no JSON "
+                         "(with --no-configs: the softmax steps and the small copy only)")
+    ap.add_argument("--copy-sweep", action="store_true",
+                    help="streaming rates of the library's own kernels against size: a plain copy (op::identity) on one buffer "
+                         "pair and on two alternating pairs, a read-only pass (op::sum) and a write-only pass (op::arange), "
+                         "32 MiB to 1000 MiB; prints one JSON line and nothing else")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path runs on ONE GPU (the reference has no multi-device support and this build "
@@ -100,18 +116,74 @@ def main():
         rec.replay(reps)
         return ev.stop_ms() * 1e3 / reps
 
+    if args.copy_sweep:
+        # What bounds the read+write kernels: at which size a copy stops being helped by the 256 MiB Infinity Cache, and
+        # what reads alone and writes alone reach beyond it.
+        rows = []
+        for mib in (32, 64, 128, 192, 256, 320, 384, 512, 768, 1000):
+            n = mib * 262144
+            srcs = [D.Array.from_numpy(np.random.RandomState(40 + i).randn(n).astype(np.float32)) for i in range(2)]
+            reps = 40 if mib < 512 else 16
+            row = {"MiB_each_way": mib}
+            with D.Recording() as rec:
+                kept = [op.identity(srcs[0]).eval()]
+            row["copy_same_pair_frac_hbm"] = round(2.0 * n * 4 / time_recording(rec, reps) / 1e3 / HBM_PEAK_GBS, 4)
+            with D.Recording() as rec:
+                kept = [op.identity(x).eval() for x in srcs]
+            row["copy_alternating_pairs_frac_hbm"] = round(2.0 * n * 4 / (time_recording(rec, reps // 2) / 2) / 1e3 / HBM_PEAK_GBS, 4)
+            with D.Recording() as rec:
+                kept = [op.sum(srcs[0]).eval()]
+            row["read_only_frac_hbm"] = round(1.0 * n * 4 / time_recording(rec, reps) / 1e3 / HBM_PEAK_GBS, 4)
+            with D.Recording() as rec:
+                kept = [op.arange(n).eval()]
+            row["write_only_frac_hbm"] = round(1.0 * n * 4 / time_recording(rec, reps) / 1e3 / HBM_PEAK_GBS, 4)
+            rows.append(row)
+            del srcs, kept, rec
+        print(json.dumps({"copy_sweep": rows, "unit": "fraction of 8 TB/s by algorithmic bytes (copy: read + write)"}))
+        return
+
     if args.pmc_probe:
+        # Every dispatch below belongs to one configuration; "probe_kernel: <tag> <kernel names>" lines on stdout say which
+        # generated kernel is which (their names carry a hash). The two copies calibrate the byte counters.
+        def probe(tag, build, reps):
+            with D.Recording() as rec:
+                kept = build()
+            names = D.last_kernel_names()
+            rec.replay(reps - 1)
+            sync()
+            print("probe_kernel: %s %s launches_per_evaluation=%d evaluations=%d" % (tag, names or "-", rec.launches, reps), flush=True)
+            return kept
+
         rng = np.random.RandomState(1)
         xs = [D.Array.from_numpy(rng.randn(4096, 1024).astype(np.float32)) for _ in range(16)]
-        with D.Recording() as rec:
-            for x in xs:
-                op.softmax(x).eval()
-        rec.replay(1)  # 16 more launches: 32 softmax dispatches in total
+        probe("c1_softmax_4096x1024", lambda: [op.softmax(x).eval() for x in xs], 2)  # 32 dispatches on 16 rotating pairs
         src = D.Array.from_numpy(rng.randn(16777216).astype(np.float32))
-        with D.Recording() as cp:
-            op.identity(src).eval()
-        cp.replay(19)
-        sync()
+        probe("copy_64MiB_each_way", lambda: op.identity(src).eval(), 20)
+        del xs, src
+        if not args.no_configs:
+            n = 67108864
+            a, b, c, d = (D.Array.from_numpy(np.random.RandomState(s).uniform(-4, 4, n).astype(np.float32)) for s in (2, 3, 4, 5))
+            probe("c2_chain_4x67108864", lambda: (op.sigmoid(a) * op.tanh(b) + c * d - 0.5 * op.square(a)).eval(), 6)
+            del a, b, c, d
+            m = D.Array.from_numpy(np.random.RandomState(6).randn(8192, 8192).astype(np.float32))
+            for name, fn in (("sum_axis1", lambda: op.sum(m, [1])), ("max_axis1", lambda: op.max(m, [1])), ("sum_axis0", lambda: op.sum(m, [0])),
+                             ("max_axis0", lambda: op.max(m, [0])), ("sum_all", lambda: op.sum(m)), ("max_all", lambda: op.max(m)),
+                             ("argmax_axis1", lambda: op.argmax(m, 1))):
+                probe("c3_" + name + "_8192x8192", lambda: fn().eval(), 6)
+            del m
+            rows, vocab = 8192, 32000
+            x = D.Array.from_numpy((np.random.RandomState(7).randn(rows, vocab) * 2).astype(np.float32))
+            t = D.Array.from_numpy(np.random.RandomState(8).randint(0, vocab, rows).astype(np.int32))
+            probe("c4_cross_entropy_8192x32000", lambda: op.softmax_cross_entropy(x, t), 6)
+            probe("copy_1000MiB_each_way", lambda: op.identity(x).eval(), 6)  # the plain copy of C4's size: 1,048,576,000 B each way
+            del x, t
+            B, I, H = 256, 1024, 1024
+            X, Hp, Cp = (D.Array.from_numpy(np.random.RandomState(s).randn(B, k).astype(np.float32)) for s, k in ((9, I), (10, H), (11, H)))
+            lim = np.sqrt(6.0 / (1024 + 4096))
+            W, U = (D.Array.from_numpy(np.random.RandomState(s).uniform(-lim, lim, (1024, 4096)).astype(np.float32)) for s in (12, 13))
+            bias = D.Array.zeros((4096,))
+            probe("c5_gemm_pair_256x2048x4096", lambda: (op.dot(X, W) + op.dot(Hp, U)).eval(), 20)
+            probe("c5_lstm_step_fused", lambda: op.lstm_step(X, Hp, Cp, W, U, bias), 20)
         return
 
     # ------------------------------------------------------------ headline: C1
@@ -252,15 +324,24 @@ def main():
     if not args.no_configs:
         configs = {}
         del inputs, cycle, lead, tail, warm_tail, resident, preroll
+        measured = config_traffic()
+
+        def with_traffic(row):
+            """adds the kernel's name and, when the committed counter runs were made on this very kernel, its HBM bytes per launch"""
+            name = D.last_kernel_names()
+            row["kernel"] = name
+            row["traffic"] = measured.get(name)
+            return row
 
         # C2 elementwise chain, 4 x 67,108,864 fp32 in, 1 out
         n = 67108864
         a, b, c, d = (D.Array.from_numpy(np.random.RandomState(s).uniform(-4, 4, n).astype(np.float32)) for s in (2, 3, 4, 5))
         with D.Recording() as rec:
             (op.sigmoid(a) * op.tanh(b) + c * d - 0.5 * op.square(a)).eval()
+        c2_row = with_traffic({})
         us = time_recording(rec, 30)
-        configs["c2_chain_4x67108864"] = {"us": round(us, 2), "GB/s": round(5 * n * 4 / us / 1e3, 1),
-                                          "frac_hbm": round(5 * n * 4 / us / 1e3 / HBM_PEAK_GBS, 4), "kernels": rec.launches}
+        configs["c2_chain_4x67108864"] = dict({"us": round(us, 2), "GB/s": round(5 * n * 4 / us / 1e3, 1),
+                                               "frac_hbm": round(5 * n * 4 / us / 1e3 / HBM_PEAK_GBS, 4), "kernels": rec.launches}, **c2_row)
         del a, b, c, d, rec
 
         # C3 reductions over [8192, 8192]; two matrices alternate (268 MB each) to stay out of the cache
@@ -274,9 +355,10 @@ def main():
             with D.Recording() as rec:
                 for m in mats:
                     fn(m).eval()
+            c3_row = with_traffic({})
             us = time_recording(rec, 20) / len(mats)
-            c3[name] = {"us": round(us, 2), "GB/s": round(nb / us / 1e3, 1), "frac_hbm": round(nb / us / 1e3 / HBM_PEAK_GBS, 4),
-                        "kernels": rec.launches // len(mats)}
+            c3[name] = dict({"us": round(us, 2), "GB/s": round(nb / us / 1e3, 1), "frac_hbm": round(nb / us / 1e3 / HBM_PEAK_GBS, 4),
+                             "kernels": rec.launches // len(mats)}, **c3_row)
         configs["c3_reductions_8192x8192"] = c3
         del mats, rec
 
@@ -286,12 +368,13 @@ def main():
         t = D.Array.from_numpy(np.random.RandomState(8).randint(0, vocab, rows).astype(np.int32))
         with D.Recording() as rec:
             mean, rl, grad = op.softmax_cross_entropy(x, t)
+        c4_row = with_traffic({})
         us = time_recording(rec, 10)
         ce_bytes = 2 * rows * vocab * 4
-        configs["c4_cross_entropy_8192x32000"] = {"us": round(us, 2), "GB/s": round(ce_bytes / us / 1e3, 1),
-                                                  "frac_hbm": round(ce_bytes / us / 1e3 / HBM_PEAK_GBS, 4),
-                                                  "kernels": rec.launches, "passes_over_logits": 1,
-                                                  "mean_loss": round(float(mean.numpy()), 5)}
+        configs["c4_cross_entropy_8192x32000"] = dict({"us": round(us, 2), "GB/s": round(ce_bytes / us / 1e3, 1),
+                                                       "frac_hbm": round(ce_bytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                                                       "kernels": rec.launches, "passes_over_logits": 1,
+                                                       "mean_loss": round(float(mean.numpy()), 5)}, **c4_row)
         del x, t, grad, rl, mean, rec
 
         # C5 LSTM step B=256, I=H=1024
