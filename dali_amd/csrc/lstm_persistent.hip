@@ -485,45 +485,80 @@ int persistent_status_take() {
 
 using namespace dali_hip;
 
+// host-visible status word shared by the persistent kernels (pinned, allocated on first use outside a capture)
+static int ensure_status_word(const char* who) {
+    if (g_status) return DALI_HIP_OK;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(stream(), &cs);
+    if (cs != hipStreamCaptureStatusNone) return fail("%s: first use cannot be inside a capture", who);
+    if (hipHostMalloc((void**)&g_status, sizeof(int), hipHostMallocMapped) != hipSuccess) return fail("%s: no pinned status word", who);
+    *g_status = 0;
+    return DALI_HIP_OK;
+}
+
+static int compute_units() {
+    static int cus = 0;  // (the library is bound to one device)
+    if (cus == 0) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, bound_device()) != hipSuccess) return 0;
+        cus = prop.multiProcessorCount;
+    }
+    return cus;
+}
+
+// the kernel that keeps U in LDS: up to 64 rows of 256, 512, 768 or 1024 hidden units (faster than the phased kernel wherever it
+// runs: 19 against 21 us per step at 64 rows of 1024, 12 against 13.4 at 32)
+static bool lds_kernel_serves(int batch, int hidden, int cus) {
+    // DALI_HIP_PERSISTENT_PHASED=1: never this kernel (for comparisons and tests of the other)
+    static const bool phased_only = getenv("DALI_HIP_PERSISTENT_PHASED") && atoi(getenv("DALI_HIP_PERSISTENT_PHASED")) == 1;
+    if (phased_only || batch > 64 || hidden % 256 != 0 || hidden > 1024) return false;
+    int HU = 1;
+    while (HU <= 4 && !(hidden % HU == 0 && hidden / HU <= cus)) ++HU;
+    return HU <= 4;
+}
+
+extern "C" int dali_hip_lstm_recurrent_persistent_supported(int batch, int hidden) {
+    if (ensure_init()) return 0;
+    const int cus = compute_units();
+    if (cus <= 0 || batch < 1) return 0;
+    if (lds_kernel_serves(batch, hidden, cus)) return 2;
+    if (!recurrent_phased_supported(batch, hidden, cus)) return 0;
+    // measured against one fused launch per step (us per step, 32 steps): 31 / 33 at 96 rows of 1024, 41 / 33 at 128; 53 / 61 at 64 rows of
+    // 2048, 106 / 64 at 128; 15 / 18 at 64 rows of 512, 30 / 18 at 128
+    return batch <= 96 ? 2 : 1;
+}
+
 extern "C" int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0,
                                                   const float* c0, float* hs, float* c_out) {
     if (ensure_init()) return DALI_HIP_ERROR;
     if (steps < 1 || batch < 1 || hidden < 1) return fail("dali_hip_lstm_recurrent_persistent: steps, batch and hidden must be positive");
     if (!pre || !U || !h0 || !c0 || !hs || !c_out) return fail("dali_hip_lstm_recurrent_persistent: NULL argument");
-    if (batch > 64) return fail("dali_hip_lstm_recurrent_persistent: batch %d exceeds 64 rows (use one launch per step)", batch);
-    if (hidden % 256 != 0 || hidden > 1024) return fail("dali_hip_lstm_recurrent_persistent: hidden %d must be 256, 512, 768 or 1024", hidden);
+    if (ldu < 4 * hidden) return fail("dali_hip_lstm_recurrent_persistent: ldu %d is smaller than a row of U (%d)", ldu, 4 * hidden);
     if (((uintptr_t)h0 | (uintptr_t)hs) % 16 != 0) return fail("dali_hip_lstm_recurrent_persistent: h0 and hs must be 16-byte aligned");
     {
-        // rows 0 .. steps-2 of hs are overwritten (with the "not written yet" pattern or with h) while h0, c0 and pre are
-        // still being read
+        // rows 0 .. steps-2 of hs are overwritten while h0, c0 and pre are still being read
         const char *lo = (const char*)hs, *hi = lo + (size_t)steps * batch * hidden * sizeof(float);
         auto inside = [&](const void* p, size_t bytes) { return (const char*)p < hi && (const char*)p + bytes > lo; };
         if (inside(h0, (size_t)batch * hidden * 4) || inside(c0, (size_t)batch * hidden * 4) || inside(pre, (size_t)steps * batch * hidden * 16))
             return fail("dali_hip_lstm_recurrent_persistent: hs overlaps an input");
     }
-    static int cus = 0;  // (the library is bound to one device)
-    if (cus == 0) {
-        hipDeviceProp_t prop;
-        if (hipGetDeviceProperties(&prop, bound_device()) != hipSuccess) return fail("dali_hip_lstm_recurrent_persistent: no device properties");
-        cus = prop.multiProcessorCount;
+    const int cus = compute_units();
+    if (cus == 0) return fail("dali_hip_lstm_recurrent_persistent: no device properties");
+    if (ensure_status_word("dali_hip_lstm_recurrent_persistent")) return DALI_HIP_ERROR;
+    // a launch that finds the flag of an earlier one would leave at its first wait and hand back rows that were never written
+    if (__atomic_load_n(g_status, __ATOMIC_RELAXED) != 0)
+        return fail("dali_hip_lstm_recurrent_persistent: an earlier persistent launch gave up waiting; call dali_hip_sync to collect that error first");
+    if (!lds_kernel_serves(batch, hidden, cus)) {
+        if ((size_t)batch * hidden * 4 >= 0x7ffffff0u) return fail("dali_hip_lstm_recurrent_persistent: state rows beyond the 2 GiB a buffer load addresses");
+        return lstm_recurrent_phased(steps, batch, hidden, pre, U, ldu, h0, c0, hs, c_out, g_status, cus);
     }
     // fewest hidden units per workgroup that still give every workgroup a compute unit of its own
     int HU = 1;
     while (HU <= 4 && !(hidden % HU == 0 && hidden / HU <= cus)) ++HU;
-    // (the four gates of at most 4 hidden units fill the 16 columns of one matrix instruction)
-    if (HU > 4 || batch * HU > 256)
-        return fail("dali_hip_lstm_recurrent_persistent: hidden %d needs more than 4 hidden units per compute unit on %d compute units", hidden, cus);
     const int grid = hidden / HU, MT = (batch + 15) / 16;
     const size_t lds_bytes = ((size_t)hidden * (4 * HU + kPitchPad) + (size_t)4 * MT * 256) * sizeof(float);
     if (lds_bytes > (size_t)160 * 1024 - 1024)
         return fail("dali_hip_lstm_recurrent_persistent: the slice of U per compute unit (%zu bytes) does not fit the LDS", lds_bytes);
-    if (!g_status) {
-        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-        (void)hipStreamIsCapturing(stream(), &cs);
-        if (cs != hipStreamCaptureStatusNone) return fail("dali_hip_lstm_recurrent_persistent: first use cannot be inside a capture");
-        if (hipHostMalloc((void**)&g_status, sizeof(int), hipHostMallocMapped) != hipSuccess) return fail("dali_hip_lstm_recurrent_persistent: no pinned status word");
-        *g_status = 0;
-    }
     PersistentArgs a;
     a.T = steps; a.B = batch; a.H = hidden; a.HU = HU; a.ldu = ldu;
     a.pre = pre; a.U = U; a.h0 = h0; a.c0 = c0; a.hs = hs; a.c_out = c_out;

@@ -42,6 +42,12 @@ int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const floa
 // graph, are launches only. Keyed on the kernel's address (kernels of one signature share a function type, so a flag inside a
 // generic lambda or template would be shared among them).
 hipError_t reserve_dynamic_lds(const void* kernel, size_t bytes);
+// recurrent_phased.hip: the recurrent half of a sequence in one launch for up to 128 rows and hidden sizes that are multiples of
+// 64 up to 2048 (weights in registers, two row blocks taking turns at the grid barrier). `status` is the host-visible word that a
+// workgroup sets when a wait gives up; `cus` the number of compute units of the bound device.
+int recurrent_phased_supported(int batch, int hidden, int cus);
+int lstm_recurrent_phased(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0, const float* c0, float* hs,
+                          float* c_out, int* status, int cus);
 // lstm_persistent.hip: 1 when a persistent kernel's grid barrier gave up since the last call (and clears that)
 int persistent_status_take();
 

@@ -1650,21 +1650,22 @@ LSTMSequence lstm_sequence(const Array& xs, const Array& h0, const Array& c0, co
                        U.offset() % 4 == 0 && ((int64_t)Bn * H) % 4 == 0;
     // Small batches: a launch per step waits more than it works (37 us per step from 1 to 128 rows). The input half of
     // every step's pre-activations is one product over all T * B rows, and the recurrent half runs as one persistent launch
-    // that keeps U in the LDS of the compute units.
+    // that keeps U on the chip (in the LDS or the registers of the compute units).
     const char* persistent_env = getenv("DALI_HIP_LSTM_PERSISTENT");  // read per call: a benchmark times both forms in one process
     const bool persistent_off = persistent_env != nullptr && std::string(persistent_env) == "0";
-    if (fused && !persistent_off && Bn <= 64 && T >= 2 && H <= 1024 && H % 256 == 0 && c0.offset() % 4 == 0) {
+    const bool persistent_ok = !persistent_off && !dry_run() && T >= 2 && dense(seq) && dense(h0) && dense(c0) && dense(W) && dense(U) && dense(b) &&
+                               W.ndim() == 2 && U.ndim() == 2 && b.ndim() == 1 && W.shape()[0] == In && W.shape()[1] == 4 * H && U.shape()[0] == H &&
+                               U.shape()[1] == 4 * H && b.shape()[0] == 4 * H && c0.offset() % 4 == 0 && ((int64_t)Bn * H) % 4 == 0 &&
+                               dali_hip_lstm_recurrent_persistent_supported(Bn, H) == 2;
+    // (a size that the persistent kernels do not serve, or serve more slowly than a launch per step, takes the loop below; a failure of the
+    // launch itself is an error)
+    if (persistent_ok) {
         Array pre = add(dot(seq.reshape({T * Bn, In}), W), b.expand_dims(0));
         pre.eval();
         Array c_last({Bn, H}, DTYPE_FLOAT);
         Array h0c = h0.offset() % 4 == 0 ? h0 : h0.ascontiguousarray();
-        bool launched = true;
-        try {
-            lstm_recurrent_persistent(pre.reshape({T, Bn, 4 * H}), U, h0c, c0, hs, c_last);
-        } catch (const std::exception&) {
-            launched = false;  // a device with fewer compute units or less LDS: one launch per step below
-        }
-        if (launched) return {hs, c_last, hs[T - 1]};
+        lstm_recurrent_persistent(pre.reshape({T, Bn, 4 * H}), U, h0c, c0, hs, c_last);
+        return {hs, c_last, hs[T - 1]};
     }
     Array c_prev = c0, h_prev = h0;
     for (int t = 0; t < T; ++t) {

@@ -274,23 +274,30 @@ int dali_hip_lstm_step_small(int batch, int input, int hidden, const float* X, i
                              float* Cout, float* Hout);
 
 /*
- * The recurrent half of an LSTM over a whole sequence in one launch, for batches of at most 64 rows: the loop of
+ * The recurrent half of an LSTM over a whole sequence in one launch, for batches of at most 128 rows: the loop of
  * dali/layers/lstm.cpp:294-303 (one cell activation per time step), whose hidden-to-hidden product the reference meant to
  * hand to a persistent kernel (third_party/nervana_kernels/sass/persistent_rnn_fprop.sass). pre [steps, batch, 4 hidden]
  * holds the input half of the pre-activations for every step, x(t).W + bias, gates packed i, f, o, g along the columns (one
- * large product computed beforehand); U [hidden, 4 hidden] (row stride ldu) stays in the LDS of the compute units for the
- * whole sequence; per step every workgroup forms h(t-1).U for the gate columns of its hidden units, finishes the cell
- * (same arithmetic as dali_hip_lstm_step) and meets the others at a grid barrier (up to 32 rows: waits until the values of
- * h(t-1) it needs have replaced a "not written yet" bit pattern that the launch first writes into hs, so hs must not be
- * read by anybody else while the launch runs). hs [steps, batch, hidden] receives every
- * hidden state, c_out [batch, hidden] the last cell state. hidden must be a multiple of 64 whose slice of U per compute
- * unit fits the LDS (hidden = 1024 on 256 compute units: 80 KiB); h0 and hs 16-byte aligned. The grid has at most one
- * workgroup per compute unit, so all are resident; a workgroup that still does not see the others arrive within 2^20 polls
- * (DALI_HIP_PERSISTENT_SPIN_LIMIT) raises a flag, every workgroup leaves, and the next dali_hip_sync or
- * dali_hip_memcpy_d2h fails with that message instead of the device hanging.
+ * large product computed beforehand); U [hidden, 4 hidden] (row stride ldu >= 4 hidden) stays on the chip for the whole
+ * sequence, every workgroup holding the gate columns of its hidden units; per step a workgroup forms h(t-1).U for those
+ * columns, finishes the cell (same arithmetic as dali_hip_lstm_step) and meets the others at a grid barrier.
+ * hs [steps, batch, hidden] receives every hidden state, c_out [batch, hidden] the last cell state.
+ * Accepted sizes: hidden a multiple of 64 up to 2048 and at most 128 rows (dali_hip_lstm_recurrent_persistent_supported
+ * answers for the bound device; anything else is refused with an error). Up to 64 rows with hidden = 256, 512, 768 or 1024
+ * the weights sit in LDS (up to 32 rows a step waits for the values of h(t-1) themselves: hs is first filled with a "not
+ * written yet" bit pattern); otherwise the weights sit in registers and the batch is cut into row blocks that take turns,
+ * so that one block's barrier runs while the others are multiplied. h0 and hs must be 16-byte aligned. hs must not overlap h0, c0
+ * or pre (a call where it does is refused) and must not be read by anybody else while the launch runs.
+ * The grid has at most one workgroup per compute unit, so all are resident; a workgroup that still does not see the others
+ * arrive within 2^20 polls (DALI_HIP_PERSISTENT_SPIN_LIMIT) raises a flag, every workgroup leaves, and the next
+ * dali_hip_sync or dali_hip_memcpy_d2h fails with that message instead of the device hanging. Until that error has been
+ * collected, further persistent launches are refused (they would leave at their first wait).
  */
 int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0,
                                        const float* c0, float* hs, float* c_out);
+/* Whether dali_hip_lstm_recurrent_persistent serves this batch and hidden size on the bound device: 0 no (the call would be refused), 1 yes,
+ * 2 yes and it is expected to beat one launch per step (up to 96 rows). No error is set. */
+int dali_hip_lstm_recurrent_persistent_supported(int batch, int hidden);
 
 /* ------------------------------------------------------------- scatter */
 /*

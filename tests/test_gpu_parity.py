@@ -139,6 +139,24 @@ def test_raw_module_load_and_six_array_launch(gpu, rng):
     hip.dali_hip_free(ddst)
 
 
+def lstm_sequence_truth(O, Xs, H0, C0, W, U, b):
+    """(all hidden states, final memory) of the LSTM of dali/layers/lstm.cpp:226-261,294-303: the CPU checker's step in turn where that
+    finishes in seconds (its products are scalar loops), the same recurrence written out in fp64 with numpy beyond."""
+    T, B, I = Xs.shape
+    H = H0.shape[1]
+    if 8.0 * T * B * (I + H) * H < 3e9:
+        return O.lstm_sequence(Xs, H0, C0, W, U, b)
+    h, c, hs = H0.astype(np.float64), C0.astype(np.float64), []
+    W64, U64, b64 = W.astype(np.float64), U.astype(np.float64), b.astype(np.float64)
+    for t in range(T):
+        g = Xs[t].astype(np.float64) @ W64 + h @ U64 + b64
+        i, f, o = (1.0 / (1.0 + np.exp(-g[:, k * H:(k + 1) * H])) for k in range(3))
+        c = f * c + i * np.tanh(g[:, 3 * H:])
+        h = o * np.tanh(c)
+        hs.append(h)
+    return np.stack(hs), c
+
+
 def _dev(hip, a):
     p = C.c_void_p()
     assert hip.dali_hip_malloc(C.byref(p), max(a.nbytes, 4)) == 0
@@ -1889,10 +1907,11 @@ def test_fused_lstm_step_equals_the_two_launch_form(gpu, D, O, rng, B, H):
     close(hn.numpy(), ohn, rtol=1e-4, atol=1e-5)
 
 
-@pytest.mark.parametrize("T,B,I,H", [(5, 48, 128, 128), (3, 7, 24, 40), (12, 256, 64, 64)])
+@pytest.mark.parametrize("T,B,I,H", [(5, 160, 128, 128), (3, 7, 24, 40), (12, 256, 64, 64)])
 def test_lstm_sequence_is_the_step_applied_in_turn(gpu, D, O, rng, T, B, I, H):
-    """LSTM::activate_sequence (dali/layers/lstm.cpp:294-303): fused steps chained through one [T, B, H] buffer when
-    input == hidden and both are multiples of 64, the unfused step otherwise."""
+    """LSTM::activate_sequence (dali/layers/lstm.cpp:294-303) at batches beyond the persistent kernels (more than 96 rows) or
+    hidden sizes they do not take: fused steps chained through one [T, B, H] buffer when input == hidden and both are
+    multiples of 64, the unfused step otherwise."""
     Xs = rng.randn(T, B, I).astype(np.float32)
     H0, C0 = (rng.randn(B, H).astype(np.float32) for _ in range(2))
     lim = np.sqrt(6.0 / (I + 4 * H))
@@ -1919,25 +1938,31 @@ def test_lstm_sequence_is_the_step_applied_in_turn(gpu, D, O, rng, T, B, I, H):
     assert np.array_equal(hs.numpy(), first)
 
 
-@pytest.mark.parametrize("T,B,H", [(2, 1, 256), (5, 8, 256), (4, 17, 512), (3, 40, 768), (3, 64, 1024), (33, 8, 1024), (6, 32, 1024), (70, 2, 512),
-                                   (9, 33, 256)])
-def test_lstm_sequence_in_one_persistent_launch(gpu, D, O, rng, T, B, H):
+@pytest.mark.parametrize("T,B,I,H", [(2, 1, 256, 256), (5, 8, 256, 256), (4, 17, 512, 512), (3, 40, 768, 768), (3, 64, 1024, 1024), (12, 8, 1024, 1024),
+                                     (6, 32, 1024, 1024), (70, 2, 512, 512), (9, 33, 256, 256),
+                                     # sizes of the kernel that keeps the weights in registers: other hidden sizes, more than 64 rows, an input
+                                     # size of its own
+                                     (4, 17, 128, 320), (3, 96, 320, 320), (3, 40, 256, 640), (2, 64, 512, 1536), (2, 96, 256, 2048), (3, 20, 1088, 1088),
+                                     (4, 80, 1024, 1024), (5, 96, 64, 128), (3, 1, 64, 192), (3, 8, 32, 64)])
+def test_lstm_sequence_in_one_persistent_launch(gpu, D, O, rng, T, B, I, H):
     """Small batches: the input half of every step's pre-activations is one product, the recurrent half one launch that
-    keeps U in the LDS of the compute units and steps through the sequence, waiting for the values of h(t-1) themselves
-    up to 32 rows and behind grid barriers above (the role of the reference's persistent_rnn_fprop kernel for the loop of
-    dali/layers/lstm.cpp:294-303). Same values as the step applied in turn, to the tolerance of a product summed in another
-    order."""
-    Xs = rng.randn(T, B, H).astype(np.float32)
+    keeps U on the chip and steps through the sequence (the role of the reference's persistent_rnn_fprop kernel for the loop
+    of dali/layers/lstm.cpp:294-303): in LDS up to 64 rows of 256, 512, 768 or 1024 hidden units (waiting for the values of
+    h(t-1) themselves up to 32 rows, behind grid barriers above), in registers with row blocks that take turns at the barrier
+    for every other multiple of 64 up to 2048 and up to 96 rows. Same values as the step applied in turn, to the tolerance of
+    a product summed in another order."""
+    Xs = rng.randn(T, B, I).astype(np.float32)
     H0, C0 = (rng.randn(B, H).astype(np.float32) for _ in range(2))
     lim = np.sqrt(6.0 / (H + 4 * H))
-    W, U = (rng.uniform(-lim, lim, (H, 4 * H)).astype(np.float32) for _ in range(2))
+    W = rng.uniform(-lim, lim, (I, 4 * H)).astype(np.float32)
+    U = rng.uniform(-lim, lim, (H, 4 * H)).astype(np.float32)
     b = (rng.randn(4 * H) * 0.1).astype(np.float32)
     dev = [arr(D, v) for v in (Xs, H0, C0, W, U, b)]
     with D.Recording() as rec:
         hs, c_last, h_last = D.op.lstm_sequence(*dev)
     assert D.last_kernel_kinds() == "lstm_persistent"
     assert hs.shape == (T, B, H) and np.array_equal(h_last.numpy(), hs.numpy()[-1])
-    ohs, oc = O.lstm_sequence(Xs, H0, C0, W, U, b)
+    ohs, oc = lstm_sequence_truth(O, Xs, H0, C0, W, U, b)
     close(hs.numpy(), ohs, rtol=2e-4, atol=2e-5)
     close(c_last.numpy(), oc, rtol=2e-4, atol=2e-5)
     # against the step applied in turn (launch per step)
@@ -1958,7 +1983,7 @@ def test_lstm_sequence_in_one_persistent_launch(gpu, D, O, rng, T, B, H):
     close(D.op.sum(hs).numpy(), first.astype(np.float64).sum(), rtol=1e-5, atol=1e-5 * np.abs(first).sum())
 
 
-@pytest.mark.parametrize("T,B,H", [(7, 4, 512), (4, 40, 256)])
+@pytest.mark.parametrize("T,B,H", [(7, 4, 512), (4, 40, 256), (3, 128, 1024), (2, 128, 2048), (3, 96, 640), (3, 112, 320)])
 def test_persistent_recurrence_through_the_c_abi(gpu, O, rng, T, B, H):
     """dali_hip_lstm_recurrent_persistent on raw device pointers: pre-activations of the input half from the host, a
     leading dimension of U larger than its row, twice in a row into the same hs; against the sequential definition, and
@@ -1972,7 +1997,7 @@ def test_persistent_recurrence_through_the_c_abi(gpu, O, rng, T, B, H):
     pre = (Xs.reshape(T * B, H).astype(np.float64) @ W.astype(np.float64) + b).astype(np.float32).reshape(T, B, 4 * H)
     Up = np.zeros((H, 4 * H + 8), np.float32); Up[:, :4 * H] = U
     ptrs = [_dev(hip, v) for v in (pre, Up, H0, C0, np.zeros((T, B, H), np.float32), np.zeros((B, H), np.float32))]
-    ohs, oc = O.lstm_sequence(Xs, H0, C0, W, U, b)
+    ohs, oc = lstm_sequence_truth(O, Xs, H0, C0, W, U, b)
     hs, c = np.empty((T, B, H), np.float32), np.empty((B, H), np.float32)
     for _ in range(2):
         assert hip.dali_hip_lstm_recurrent_persistent(T, B, H, ptrs[0], ptrs[1], 4 * H + 8, ptrs[2], ptrs[3], ptrs[4], ptrs[5]) == 0, hip.dali_hip_last_error()
@@ -1980,20 +2005,26 @@ def test_persistent_recurrence_through_the_c_abi(gpu, O, rng, T, B, H):
         assert hip.dali_hip_memcpy_d2h(c.ctypes.data_as(C.c_void_p), ptrs[5], c.nbytes) == 0
         close(hs, ohs, rtol=2e-4, atol=2e-5)
         close(c, oc, rtol=2e-4, atol=2e-5)
-    # refused: more than 64 rows, a hidden size without a kernel, hs on top of h0
-    assert hip.dali_hip_lstm_recurrent_persistent(T, 65, H, ptrs[0], ptrs[1], 4 * H + 8, ptrs[2], ptrs[3], ptrs[4], ptrs[5]) != 0
-    assert hip.dali_hip_lstm_recurrent_persistent(T, B, 320, ptrs[0], ptrs[1], 4 * H + 8, ptrs[2], ptrs[3], ptrs[4], ptrs[5]) != 0
+    # what is served: up to 128 rows, hidden sizes that are multiples of 64 up to 2048 (2: expected to beat a launch per step)
+    assert hip.dali_hip_lstm_recurrent_persistent_supported(B, H) == (2 if B <= 96 else 1)
+    assert hip.dali_hip_lstm_recurrent_persistent_supported(129, 1024) == 0 and hip.dali_hip_lstm_recurrent_persistent_supported(8, 96) == 0
+    assert hip.dali_hip_lstm_recurrent_persistent_supported(8, 2112) == 0 and hip.dali_hip_lstm_recurrent_persistent_supported(128, 2048) == 1
+    # refused: more than 128 rows, a hidden size without a kernel, a leading dimension below the row, hs on top of h0
+    assert hip.dali_hip_lstm_recurrent_persistent(T, 129, H, ptrs[0], ptrs[1], 4 * H + 8, ptrs[2], ptrs[3], ptrs[4], ptrs[5]) != 0
+    assert hip.dali_hip_lstm_recurrent_persistent(T, B, 96, ptrs[0], ptrs[1], 4 * H + 8, ptrs[2], ptrs[3], ptrs[4], ptrs[5]) != 0
+    assert hip.dali_hip_lstm_recurrent_persistent(T, B, H, ptrs[0], ptrs[1], 4 * H - 4, ptrs[2], ptrs[3], ptrs[4], ptrs[5]) != 0
     assert hip.dali_hip_lstm_recurrent_persistent(T, B, H, ptrs[0], ptrs[1], 4 * H + 8, ptrs[4], ptrs[3], ptrs[4], ptrs[5]) != 0
     assert b"overlaps" in hip.dali_hip_last_error()
     for p in ptrs:
         hip.dali_hip_free(p)
 
 
-@pytest.mark.parametrize("B", [8, 40])
+@pytest.mark.parametrize("B", [8, 40, 80])
 def test_persistent_lstm_barrier_gives_up_instead_of_hanging(B):
     """With the poll limit forced to one, the first workgroup at the first barrier gives up, raises the flag, every
     workgroup leaves (the kernel ends normally) and the next synchronising call reports it. 8 rows: the form that waits
-    for the values (its one barrier comes first); 40 rows: a barrier per step."""
+    for the values (its one barrier comes first); 40 rows: a barrier per step; 80 rows: the kernel whose row blocks take
+    turns at their barriers."""
     import subprocess, sys, os
     code = (
         "import numpy as np, dali_amd as D\n"
@@ -2008,7 +2039,8 @@ def test_persistent_lstm_barrier_gives_up_instead_of_hanging(B):
         "x = D.Array.from_numpy(np.ones((4, 4), np.float32))\n"
         "print('AFTER', float(D.op.sum(x * 2.0).numpy()))\n"
     )
-    env = dict(os.environ, DALI_HIP_PERSISTENT_SPIN_LIMIT="1", PYTHONPATH=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    # (the kernel with row blocks looks at a barrier that has usually completed by then: a limit of zero makes its first wait give up unseen)
+    env = dict(os.environ, DALI_HIP_PERSISTENT_SPIN_LIMIT="0" if B > 64 else "1", PYTHONPATH=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
     assert out.returncode == 0, out.stderr[-2000:]
     assert "SYNC 1" in out.stdout and "gave up waiting at a grid barrier" in out.stdout, out.stdout
