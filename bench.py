@@ -420,6 +420,47 @@ def main():
             small["B%d" % Bs] = row
             del Xq, hs0, cs0, qrec
         configs["c5_lstm_step_256x1024x1024"]["sequence_of_32_small_batches"] = small
+        # sizes of the persistent kernel that keeps the weights in registers (other hidden sizes, more than 64 rows), again beside a
+        # fused launch per step
+        other = {}
+        for Bs, Hs in ((96, 1024), (64, 640), (64, 1536), (32, 2048), (64, 2048)):
+            Xq = D.Array.from_numpy(np.random.RandomState(24).randn(32, Bs, Hs).astype(np.float32))
+            hs0, cs0 = (D.Array.from_numpy(np.random.RandomState(s).randn(Bs, Hs).astype(np.float32)) for s in (25, 26))
+            limq = np.sqrt(6.0 / (5 * Hs))
+            Wq, Uq = (D.Array.from_numpy(np.random.RandomState(s).uniform(-limq, limq, (Hs, 4 * Hs)).astype(np.float32)) for s in (12, 13))
+            bq = D.Array.zeros((4 * Hs,))
+            row = {}
+            for name, flag in (("persistent", "1"), ("launch_per_step", "0")):
+                os.environ["DALI_HIP_LSTM_PERSISTENT"] = flag
+                with D.Recording() as qrec:
+                    op.lstm_sequence(Xq, hs0, cs0, Wq, Uq, bq)
+                row[name + "_us_per_step"] = round(time_recording(qrec, 6) / 32, 2)
+                row[name + "_launches"] = qrec.launches
+            os.environ.pop("DALI_HIP_LSTM_PERSISTENT", None)
+            row["mfma_fp32_bound_us"] = round(2.0 * Bs * 2 * Hs * 4 * Hs / MFMA_FP32_PEAK_TFLOPS / 1e6, 2)
+            other["B%d_H%d" % (Bs, Hs)] = row
+            del Xq, hs0, cs0, Wq, Uq, bq, qrec
+        configs["c5_lstm_step_256x1024x1024"]["sequence_of_32_other_sizes"] = other
+        # the GRU (two dependent products per step): the recurrent half as one persistent launch beside the launch-per-step form
+        gru = {}
+        for Bs, Hs in ((8, 1024), (32, 1024), (8, 512)):
+            Xq = D.Array.from_numpy(np.random.RandomState(24).randn(32, Bs, Hs).astype(np.float32))
+            hq = D.Array.from_numpy(np.random.RandomState(25).randn(Bs, Hs).astype(np.float32))
+            limq = np.sqrt(6.0 / (4 * Hs))
+            Wq, Uq = (D.Array.from_numpy(np.random.RandomState(s).uniform(-limq, limq, (Hs, 3 * Hs)).astype(np.float32)) for s in (12, 13))
+            bq = D.Array.zeros((3 * Hs,))
+            row = {}
+            for name, flag in (("persistent", "1"), ("launch_per_step", "0")):
+                os.environ["DALI_HIP_GRU_PERSISTENT"] = flag
+                with D.Recording() as qrec:
+                    op.gru_sequence(Xq, hq, Wq, Uq, bq)
+                row[name + "_us_per_step"] = round(time_recording(qrec, 6) / 32, 2)
+                row[name + "_launches"] = qrec.launches
+            os.environ.pop("DALI_HIP_GRU_PERSISTENT", None)
+            row["weights_from_hbm_bound_us"] = round(2 * Hs * 3 * Hs * 4 / HBM_PEAK_GBS / 1e3, 2)  # what a launch per step re-reads
+            gru["B%d_H%d" % (Bs, Hs)] = row
+            del Xq, hq, Wq, Uq, bq, qrec
+        configs["c5_lstm_step_256x1024x1024"]["gru_sequence_of_32"] = gru
         # one step at small batches (a decoder loop through the host): 16-row tiles with every compute unit on its own columns
         # of the weights, beside the 64-row tiles of the general kernel
         single = {}

@@ -18,6 +18,9 @@ __device__ __forceinline__ float gate_expf(float x) {
     return __builtin_fabsf(t) < 128.0f ? fixed : e;
 }
 
+// the reference's sigmoid (dali/array/functor.h:157-162): 1 / (1 + exp(-x)) in double, rounded to float
+__device__ __forceinline__ float gate_sigmoid(float x) { return (float)(1.0 / (1.0 + (double)gate_expf(-x))); }
+
 // One (row, hidden unit) pair of an LSTM step from its four pre-activations (bias not yet added) and the previous cell
 // value: gate = pre + bias, i / f / o = sigmoid in double, g = tanh, c' = f * c + i * g, h' = o * tanh(c'), each operation
 // rounded on its own like the generated gate kernel (dali/layers/lstm.cpp:238-261).

@@ -594,6 +594,38 @@ extern "C" int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidd
     return DALI_HIP_OK;
 }
 
+extern "C" int dali_hip_gru_recurrent_persistent_supported(int batch, int hidden) {
+    if (ensure_init()) return 0;
+    const int cus = compute_units();
+    if (cus <= 0 || batch < 1 || !recurrent_phased_supported(batch, hidden, cus)) return 0;
+    // measured against the launch-per-step form (us per step): 17 / 25 at 8 rows of 1024, 23 / 32 at 32, 37 / 37 at 64, 57 / 42 at 96; 15 / 18
+    // at 8 rows of 512, 29 / 24 at 64; 46 / 44 at 32 rows of 2048: two barriers per step leave less to win than the LSTM's one
+    return batch <= 48 && hidden <= 1536 ? 2 : 1;
+}
+
+extern "C" int dali_hip_gru_recurrent_persistent(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0, float* hs,
+                                                 float* scratch) {
+    if (ensure_init()) return DALI_HIP_ERROR;
+    if (steps < 1 || batch < 1 || hidden < 1) return fail("dali_hip_gru_recurrent_persistent: steps, batch and hidden must be positive");
+    if (!pre || !U || !h0 || !hs || !scratch) return fail("dali_hip_gru_recurrent_persistent: NULL argument");
+    if (ldu < 3 * hidden) return fail("dali_hip_gru_recurrent_persistent: ldu %d is smaller than a row of U (%d)", ldu, 3 * hidden);
+    if (((uintptr_t)h0 | (uintptr_t)hs | (uintptr_t)scratch) % 16 != 0) return fail("dali_hip_gru_recurrent_persistent: h0, hs and scratch must be 16-byte aligned");
+    {
+        const size_t seq = (size_t)steps * batch * hidden * sizeof(float);
+        auto meet = [](const void* p, size_t pb, const void* q, size_t qb) { return (const char*)p < (const char*)q + qb && (const char*)q < (const char*)p + pb; };
+        if (meet(hs, seq, h0, (size_t)batch * hidden * 4) || meet(hs, seq, pre, 3 * seq) || meet(scratch, seq, h0, (size_t)batch * hidden * 4) ||
+            meet(scratch, seq, pre, 3 * seq) || meet(hs, seq, scratch, seq))
+            return fail("dali_hip_gru_recurrent_persistent: hs and scratch must not overlap each other or an input");
+    }
+    if ((size_t)batch * hidden * 4 >= 0x7ffffff0u) return fail("dali_hip_gru_recurrent_persistent: state rows beyond the 2 GiB a buffer load addresses");
+    const int cus = compute_units();
+    if (cus == 0) return fail("dali_hip_gru_recurrent_persistent: no device properties");
+    if (ensure_status_word("dali_hip_gru_recurrent_persistent")) return DALI_HIP_ERROR;
+    if (__atomic_load_n(g_status, __ATOMIC_RELAXED) != 0)
+        return fail("dali_hip_gru_recurrent_persistent: an earlier persistent launch gave up waiting; call dali_hip_sync to collect that error first");
+    return gru_recurrent_phased(steps, batch, hidden, pre, U, ldu, h0, hs, scratch, g_status, cus);
+}
+
 extern "C" int dali_hip_lstm_step_small(int batch, int input, int hidden, const float* X, int ldx, const float* Hprev, int ldh, const float* Cprev,
                                         const float* W, int ldw, const float* U, int ldu, const float* bias, float* Cout, float* Hout) {
     if (ensure_init()) return DALI_HIP_ERROR;

@@ -54,11 +54,12 @@ struct PhasedArgs {
     const float* c0;           // [B, H]
     float* hs;                 // [T, B, H]
     float* c_out;              // [B, H]
+    float* rh;                 // GRU: [T, B, H] scratch for r * h(t-1), written once per row like hs
     int* status;               // host-visible: set to 1 when a wait gave up
     unsigned int spin_limit;
 };
 
-constexpr int kMaxBar = 8;      // phases at most (128 rows in blocks of 16)
+constexpr int kMaxBar = 16;     // counters: phases (at most 8: 128 rows in blocks of 16) x rounds of a step (two for the GRU)
 constexpr int kBarStride = 64;  // in words: every counter has 256 bytes to itself
 
 // Arrival counters, one per phase, zero at rest (the last workgroup to leave restores that). One arrival per workgroup and one
@@ -256,6 +257,120 @@ __global__ __launch_bounds__(256) void lstm_phased_kernel(PhasedArgs a) {
     }
 }
 
+// The GRU (dali/layers/gru.cpp:27-44) in the same frame. `pre` is [T, B, 3H] = x(t).W + b and U [H, 3H], gates packed reset, update,
+// candidate. A step has two rounds, each a product over all of H and therefore each behind a grid barrier:
+//   A: (r, z) = sigmoid(pre_r,z + h(t-1).U_r,z); r * h(t-1) goes to the scratch rows rh[t] (the candidate needs it for ALL hidden units)
+//   B: c = tanh(pre_c + rh[t].U_c); h(t) = h(t-1) * (1 - z) + c * z goes to hs[t]
+// The turns of a step are A(phase 0), A(1), ..., B(0), B(1), ...: the barrier behind A(p) has the other phases' turns to complete in.
+// Local columns: gate g of hidden unit u0 + uu at g * HU + uu, so that up to four hidden units put all three gates into one
+// 16-column tile and eight put (r, z) into the first tile and the candidate into the second.
+template <int KQB, int NT, int MT>
+__global__ __launch_bounds__(256) void gru_phased_kernel(PhasedArgs a) {
+    __shared__ float red[4][MT][256];
+    __shared__ float hown[128 * 8];  // h(t-1) of this workgroup's (row, hidden unit) pairs: row * HU + unit
+    __shared__ float zown[128 * 8];  // their update gates between the two rounds
+    __shared__ int give_up;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int arow = lane & 15, kgrp = lane >> 4;
+    const int H = a.H, HU = a.HU, B = a.B, KQ = a.KQ, PH = a.PH, kbase = wave * (H / 4);
+    const int parts = (gridDim.x & 7) == 0 ? 8 : 1;
+    const int slice = (blockIdx.x % parts) * (gridDim.x / parts) + blockIdx.x / parts;
+    const int u0 = slice * HU;
+    float wreg[KQB][4][NT];
+    load_weights<KQB, NT>(a.U, a.ldu, H, HU, 3, u0, KQ, kbase, arow, kgrp, 0, wreg);
+    for (int e = tid; e < B * HU; e += 256) hown[e] = a.h0[(size_t)(e / HU) * H + u0 + e % HU];
+    if (tid == 0) give_up = 0;
+    constexpr int ROWS = 16 * MT;
+    static_assert(ROWS * (NT * 4) <= 256, "one (row, hidden unit) pair per thread");
+    extern __shared__ __attribute__((aligned(16))) char stage_all[];
+    const int pitch_bytes = H + 16;
+    const unsigned stage_off = (unsigned)wave * (unsigned)(ROWS * pitch_bytes);
+    const char* stage = stage_all + stage_off;
+    const unsigned stage_base = (unsigned)(uintptr_t)stage_all + stage_off;
+    fetch_rows(a.h0, B, H, 0, ROWS, kbase, lane, stage_base, pitch_bytes);
+    __syncthreads();
+    const int per_step = 2 * PH, turns = a.T * per_step;
+    for (int turn = 0; turn < turns; ++turn) {
+        const int t = turn / per_step, rest = turn - t * per_step, round = rest / PH, p = rest - round * PH, r0 = p * ROWS;
+        const int tn = (turn + 1) / per_step, restn = (turn + 1) - tn * per_step, roundn = restn / PH, pn = restn - roundn * PH;
+        // what the next turn reads: round A the rows of h(tn - 1), complete when counter PH + pn has seen tn rounds of arrivals;
+        // round B the rows of rh[tn], complete when counter pn has seen tn + 1
+        const int next_counter = roundn == 0 ? PH + pn : pn;
+        const unsigned int next_target = gridDim.x * (unsigned int)(roundn == 0 ? tn : tn + 1);
+        unsigned int early = 0;
+        const int e = tid, rr = e / HU, row = r0 + rr, uu = e - rr * HU;
+        const bool mine = rr < ROWS && row < B;
+        float pre_a = 0.0f, pre_b = 0.0f;  // round A: reset and update; round B: candidate
+        if (mine) {
+            const float* pr = a.pre + ((size_t)t * B + row) * 3 * H + u0 + uu;
+            if (round == 0) { pre_a = pr[0]; pre_b = pr[H]; } else { pre_a = pr[2 * H]; }
+        }
+        // round A needs the first tile only when (r, z) fill it (eight hidden units); otherwise every gate sits in tile 0
+        f4 acc[MT][NT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n) acc[m][n] = (f4){0.f, 0.f, 0.f, 0.f};
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's rows have landed in its stage
+        multiply<KQB, NT, MT>(stage, pitch_bytes, KQ, arow, kgrp, wreg, acc);
+        if (tid == 0 && turn + 1 < turns && next_target > 0) early = read_counter(next_counter);
+        // the tile that holds this round's columns: with two tiles, (r, z) are tile 0 and the candidate tile 1
+        const int tile = NT == 2 && round == 1 ? 1 : 0;
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) red[wave][m][(4 * kgrp + v) * 16 + arow] = NT == 2 && tile == 1 ? acc[m][NT - 1][v] : acc[m][0][v];
+        __syncthreads();
+        if (mine) {
+            auto column_sum = [&](int j) {
+                float s = 0.0f;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) s += red[w][rr / 16][(rr & 15) * 16 + (j & 15)];
+                return s;
+            };
+            const float hprev = hown[row * HU + uu];
+            if (round == 0) {
+#pragma clang fp contract(off)
+                const float r = gate_sigmoid(pre_a + column_sum(uu));
+                const float z = gate_sigmoid(pre_b + column_sum(HU + uu));
+                zown[row * HU + uu] = z;
+                __hip_atomic_store(a.rh + ((size_t)t * B + row) * H + u0 + uu, r * hprev, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+#pragma clang fp contract(off)
+                const float c = tanhf(pre_a + column_sum(2 * HU + uu));
+                const float z = zown[row * HU + uu];
+                const float keep = hprev * (1.0f - z);
+                const float take = c * z;
+                const float hn = keep + take;
+                hown[row * HU + uu] = hn;
+                __hip_atomic_store(a.hs + ((size_t)t * B + row) * H + u0 + uu, hn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        // every wave's stores are acknowledged by memory before the workgroup counts its arrival
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();  // (also: the fold area is free again)
+        if (tid == 0 && (round == 0 || t + 1 < a.T)) arrive(round == 0 ? p : PH + p);
+        if (turn + 1 == turns) break;
+        if (tid == 0 && next_target > 0) {
+            if (a.spin_limit == 0u || (early < next_target && !wait_for(a, next_counter, next_target))) {
+                if (a.spin_limit == 0u) __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                give_up = 1;
+            }
+        }
+        __syncthreads();
+        if (give_up) break;
+        const float* src = roundn == 1 ? a.rh + (size_t)tn * B * H : (tn == 0 ? a.h0 : a.hs + (size_t)(tn - 1) * B * H);
+        fetch_rows(src, B, H, pn * ROWS, ROWS, kbase, lane, stage_base, pitch_bytes);
+    }
+    __shared__ int last_out;
+    if (tid == 0) last_out = __hip_atomic_fetch_add(&g_done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1;
+    __syncthreads();
+    if (last_out) {
+        if (tid < kMaxBar) __hip_atomic_store(&g_bar[tid][0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) __hip_atomic_store(&g_done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 template <typename K>
 int launch(K kernel, const PhasedArgs& a, int grid, int rows_per_phase) {
     const size_t lds_bytes = (size_t)rows_per_phase * (a.H + 16) * 4;  // four waves x rows x (H / 4 + 4) floats
@@ -304,6 +419,39 @@ int lstm_recurrent_phased(int steps, int batch, int hidden, const float* pre, co
     if (KQB == kqb && NT == nt) {                                                       \
         if (MT == 1) return launch(lstm_phased_kernel<kqb, nt, 1>, a, grid, 16);        \
         return launch(lstm_phased_kernel<kqb, nt, (kqb <= 16 ? 2 : 1)>, a, grid, 32);   \
+    }
+    DALI_PHASED_CASE(4, 1)
+    DALI_PHASED_CASE(8, 1)
+    DALI_PHASED_CASE(16, 1)
+    DALI_PHASED_CASE(32, 2)
+#undef DALI_PHASED_CASE
+    return fail("persistent recurrence: no kernel for hidden %d", hidden);
+}
+
+
+// hidden units per workgroup for the GRU: three gates of each; the same rule as above
+int gru_recurrent_phased(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0, float* hs, float* scratch,
+                         int* status, int cus) {
+    const int HU = units_per_workgroup(hidden, cus);
+    if (!recurrent_phased_supported(batch, hidden, cus) || HU == 0)
+        return fail("persistent recurrence: %d rows of %d hidden units on %d compute units are outside what it serves (at most 128 rows, hidden a multiple "
+                    "of 64 up to 2048)", batch, hidden, cus);
+    PhasedArgs a = {};
+    a.T = steps; a.B = batch; a.H = hidden; a.HU = HU; a.ldu = ldu; a.KQ = hidden / 64;
+    a.pre = pre; a.U = U; a.h0 = h0; a.hs = hs; a.rh = scratch;
+    a.status = status;
+    static const unsigned int spin_env = getenv("DALI_HIP_PERSISTENT_SPIN_LIMIT") ? (unsigned int)atol(getenv("DALI_HIP_PERSISTENT_SPIN_LIMIT")) : (1u << 20);
+    a.spin_limit = spin_env;
+    const int tiles = (batch + 15) / 16;
+    const int KQB = hidden <= 256 ? 4 : hidden <= 512 ? 8 : hidden <= 1024 ? 16 : 32;
+    const int NT = 3 * HU > 16 ? 2 : 1;
+    const int MT = (KQB <= 16 && tiles >= 4) ? 2 : 1;
+    a.PH = (tiles + MT - 1) / MT;
+    const int grid = hidden / HU;
+#define DALI_PHASED_CASE(kqb, nt)                                                      \
+    if (KQB == kqb && NT == nt) {                                                      \
+        if (MT == 1) return launch(gru_phased_kernel<kqb, nt, 1>, a, grid, 16);        \
+        return launch(gru_phased_kernel<kqb, nt, (kqb <= 16 ? 2 : 1)>, a, grid, 32);   \
     }
     DALI_PHASED_CASE(4, 1)
     DALI_PHASED_CASE(8, 1)

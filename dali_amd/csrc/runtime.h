@@ -48,6 +48,8 @@ hipError_t reserve_dynamic_lds(const void* kernel, size_t bytes);
 int recurrent_phased_supported(int batch, int hidden, int cus);
 int lstm_recurrent_phased(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0, const float* c0, float* hs,
                           float* c_out, int* status, int cus);
+int gru_recurrent_phased(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0, float* hs, float* scratch,
+                         int* status, int cus);
 // lstm_persistent.hip: 1 when a persistent kernel's grid barrier gave up since the last call (and clears that)
 int persistent_status_take();
 

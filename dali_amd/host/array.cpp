@@ -1766,6 +1766,25 @@ GRUSequence gru_sequence(const Array& xs, const Array& h0, const Array& W, const
                     b.shape()[0] == 3 * H,
                 "gru_sequence: inconsistent shapes");
     for (const Array* a : {&xs, &h0, &W, &U, &b}) a->eval();
+    // Small batches: the recurrent half of the whole sequence as one persistent launch (weights in the registers of the compute
+    // units, two grid barriers per step), the input half with the bias as one product in front of it.
+    {
+        auto dense = [](const Array& a) { return a.is_buffer() && a.contiguous_memory() && a.dtype() == DTYPE_FLOAT; };
+        const char* persistent_env = getenv("DALI_HIP_GRU_PERSISTENT");  // read per call: a benchmark times both forms in one process
+        const bool persistent_off = persistent_env != nullptr && std::string(persistent_env) == "0";
+        Array seq = xs.is_buffer() && xs.contiguous_memory() ? xs : xs.ascontiguousarray();
+        if (!persistent_off && !dry_run() && T >= 2 && dense(seq) && dense(h0) && dense(W) && dense(U) && dense(b) && h0.offset() % 4 == 0 &&
+            ((int64_t)Bn * H) % 4 == 0 && dali_hip_gru_recurrent_persistent_supported(Bn, H) == 2) {
+            Array pre = add(dot(seq.reshape({T * Bn, In}), W), b.expand_dims(0));
+            pre.eval();
+            Array states({T, Bn, H}, DTYPE_FLOAT), scratch({T, Bn, H}, DTYPE_FLOAT);
+            gru_recurrent_persistent(pre.reshape({T, Bn, 3 * H}), U, h0, states, scratch);
+            GRUSequence out;
+            out.states = states;
+            out.last = states[T - 1];
+            return out;
+        }
+    }
     Array px_all = dot(xs.reshape({T * Bn, In}), W);  // [T B, 3H]
     px_all.eval();
     auto bias = [&](int k) { return b.slice(0, k * H, (k + 1) * H).expand_dims(0); };

@@ -214,4 +214,27 @@ void lstm_recurrent_persistent(const Array& pre, const Array& U, const Array& h0
     }
 }
 
+
+// the recurrent half of a whole GRU sequence in one launch
+void gru_recurrent_persistent(const Array& pre, const Array& U, const Array& h0, const Array& hs, const Array& scratch) {
+    const int T = hs.shape()[0], Bn = hs.shape()[1], H = hs.shape()[2];
+    const float* pp = (const float*)pre.device_ptr();
+    const float* up = (const float*)U.device_ptr();
+    const float* hp = (const float*)h0.device_ptr();
+    float* ho = (float*)hs.device_ptr(memory::AM_OVERWRITE);
+    float* sp = (float*)scratch.device_ptr(memory::AM_OVERWRITE);
+    jit_stats().gemms_launched++;
+    jit_stats().last_kernel_kinds = "gru_persistent";
+    check_hip(dali_hip_gru_recurrent_persistent(T, Bn, H, pp, up, 3 * H, hp, ho, sp), "persistent gru sequence");
+    if (g_recording) {
+        note_recorded_write(hs.expression()->memory);
+        note_recorded_write(scratch.expression()->memory);
+        std::vector<Array> keep = {pre, U, h0, hs, scratch};
+        g_recording->push_back([=]() {
+            (void)keep;
+            check_hip(dali_hip_gru_recurrent_persistent(T, Bn, H, pp, up, 3 * H, hp, ho, sp), "persistent gru sequence replay");
+        });
+    }
+}
+
 }  // namespace dali

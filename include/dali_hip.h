@@ -299,6 +299,22 @@ int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidden, const f
  * 2 yes and it is expected to beat one launch per step (up to 96 rows). No error is set. */
 int dali_hip_lstm_recurrent_persistent_supported(int batch, int hidden);
 
+/*
+ * The recurrent half of a GRU over a whole sequence in one launch: the loop of dali/layers/gru.cpp:59-64 over
+ * GRU::activate (gru.cpp:27-44). pre [steps, batch, 3 hidden] holds x(t).W + bias for the reset, update and candidate
+ * layers (packed in that order along the columns, one product computed beforehand), U [hidden, 3 hidden] (row stride ldu)
+ * the recurrent weights in the same packing. Per step every workgroup forms (r, z) = sigmoid(pre + h(t-1).U) for its hidden
+ * units, writes r * h(t-1) into scratch [steps, batch, hidden], meets the others at a grid barrier, forms the candidate
+ * tanh(pre + (r * h(t-1)).U) and h(t) = h(t-1) * (1 - z) + candidate * z, and meets them again; hs [steps, batch, hidden]
+ * receives every state. Same sizes, row blocks that take turns at the barriers, bounded waits and error reporting as
+ * dali_hip_lstm_recurrent_persistent (weights in registers). h0, hs and scratch 16-byte aligned; hs and scratch must not
+ * overlap each other or an input, and must not be touched by anybody else while the launch runs.
+ */
+int dali_hip_gru_recurrent_persistent(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0, float* hs,
+                                      float* scratch);
+/* 0: not served; 1: served; 2: served and expected to beat the launch-per-step form */
+int dali_hip_gru_recurrent_persistent_supported(int batch, int hidden);
+
 /* ------------------------------------------------------------- scatter */
 /*
  * Stable ordering of n int32 keys held in device memory: sorted_keys[p] is the p-th smallest key and

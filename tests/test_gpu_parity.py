@@ -2061,11 +2061,16 @@ def test_gru_step_matches_oracle(gpu, D, O, rng, B, I, H):
     assert np.array_equal(D.op.gru_step(*(arr(D, v) for v in (X, Hp, W, U, b_keep))).numpy(), Hp)
 
 
-@pytest.mark.parametrize("T,B,I,H", [(3, 16, 32, 48), (6, 8, 256, 256), (4, 5, 7, 9), (5, 70, 128, 64)])
+@pytest.mark.parametrize("T,B,I,H", [(3, 16, 32, 48), (6, 8, 256, 256), (4, 5, 7, 9), (5, 70, 128, 64),
+                                     # one persistent launch for the recurrent half (up to 48 rows, hidden a multiple of 64 up to 1536)
+                                     (4, 17, 128, 320), (3, 33, 320, 320), (3, 48, 256, 640), (3, 32, 512, 1024), (2, 40, 256, 1536), (3, 20, 256, 1088),
+                                     (9, 1, 64, 192), (5, 8, 1024, 1024)])
 def test_gru_sequence_is_the_step_in_turn(gpu, D, O, rng, T, B, I, H):
     """GRU::activate_sequence (dali/layers/gru.cpp:59-64): the input half of all steps is one product, so the states equal
     the step applied in turn to the rounding of that product's other order of summation; against the sequential definition
-    and against op.gru_step step by step; the recorded launches recompute the same states."""
+    and against op.gru_step step by step; the recorded launches recompute the same states. Up to 48 rows of a hidden size
+    that is a multiple of 64 the recurrent half is one persistent launch (weights in registers, two grid barriers per step,
+    row blocks taking turns at them)."""
     Xs = rng.randn(T, B, I).astype(np.float32)
     H0 = rng.randn(B, H).astype(np.float32)
     lim = np.sqrt(6.0 / (I + 3 * H))
@@ -2074,6 +2079,8 @@ def test_gru_sequence_is_the_step_in_turn(gpu, D, O, rng, T, B, I, H):
     dev = [arr(D, v) for v in (Xs, H0, W, U, b)]
     with D.Recording() as rec:
         states, last = D.op.gru_sequence(*dev)
+    persistent = H % 64 == 0 and B <= 48 and H <= 1536
+    assert (D.last_kernel_kinds() == "gru_persistent") == persistent and (rec.launches == 3 if persistent else rec.launches > 3)
     assert states.shape == (T, B, H) and np.array_equal(last.numpy(), states.numpy()[-1])
     close(states.numpy(), O.gru_sequence(Xs, H0, W, U, b), rtol=2e-4, atol=2e-5)
     h = dev[1]
@@ -2085,6 +2092,45 @@ def test_gru_sequence_is_the_step_in_turn(gpu, D, O, rng, T, B, I, H):
     assert np.array_equal(states.numpy(), first)
     with pytest.raises(Exception):
         D.op.gru_sequence(dev[0], arr(D, np.zeros((B + 1, H), np.float32)), dev[2], dev[3], dev[4])
+
+
+@pytest.mark.parametrize("T,B,H", [(4, 8, 256), (3, 96, 640), (2, 128, 2048), (3, 70, 1024)])
+def test_persistent_gru_through_the_c_abi(gpu, rng, T, B, H):
+    """dali_hip_gru_recurrent_persistent on raw device pointers, a leading dimension of U larger than its row, twice in a row
+    into the same buffers; against the recurrence of dali/layers/gru.cpp:27-44 written out in fp64; the argument checks."""
+    hip = gpu
+    Xs = rng.randn(T, B, H).astype(np.float32)
+    H0 = rng.randn(B, H).astype(np.float32)
+    lim = np.sqrt(6.0 / (4 * H))
+    W, U = (rng.uniform(-lim, lim, (H, 3 * H)).astype(np.float32) for _ in range(2))
+    b = (rng.randn(3 * H) * 0.1).astype(np.float32)
+    pre = (Xs.reshape(T * B, H).astype(np.float64) @ W.astype(np.float64) + b).astype(np.float32).reshape(T, B, 3 * H)
+    Up = np.zeros((H, 3 * H + 4), np.float32); Up[:, :3 * H] = U
+    h, want = H0.astype(np.float64), []
+    sg = lambda v: 1.0 / (1.0 + np.exp(-v))
+    for t in range(T):
+        p64, ph = pre[t].astype(np.float64), h @ U[:, :2 * H].astype(np.float64)
+        r, z = sg(p64[:, :H] + ph[:, :H]), sg(p64[:, H:2 * H] + ph[:, H:])
+        cand = np.tanh(p64[:, 2 * H:] + (r * h) @ U[:, 2 * H:].astype(np.float64))
+        h = h * (1.0 - z) + cand * z
+        want.append(h)
+    want = np.stack(want)
+    ptrs = [_dev(hip, v) for v in (pre, Up, H0, np.zeros((T, B, H), np.float32), np.zeros((T, B, H), np.float32))]
+    got = np.empty((T, B, H), np.float32)
+    for _ in range(2):
+        assert hip.dali_hip_gru_recurrent_persistent(T, B, H, ptrs[0], ptrs[1], 3 * H + 4, ptrs[2], ptrs[3], ptrs[4]) == 0, hip.dali_hip_last_error()
+        assert hip.dali_hip_memcpy_d2h(got.ctypes.data_as(C.c_void_p), ptrs[3], got.nbytes) == 0, hip.dali_hip_last_error()
+        close(got, want, rtol=2e-4, atol=2e-5)
+    assert hip.dali_hip_gru_recurrent_persistent_supported(B, H) == (2 if B <= 48 and H <= 1536 else 1)
+    assert hip.dali_hip_gru_recurrent_persistent_supported(129, H) == 0 and hip.dali_hip_gru_recurrent_persistent_supported(B, 100) == 0
+    # refused: too many rows, a hidden size without a kernel, a leading dimension below the row, states on top of the scratch rows
+    assert hip.dali_hip_gru_recurrent_persistent(T, 129, H, ptrs[0], ptrs[1], 3 * H + 4, ptrs[2], ptrs[3], ptrs[4]) != 0
+    assert hip.dali_hip_gru_recurrent_persistent(T, B, 100, ptrs[0], ptrs[1], 3 * H + 4, ptrs[2], ptrs[3], ptrs[4]) != 0
+    assert hip.dali_hip_gru_recurrent_persistent(T, B, H, ptrs[0], ptrs[1], 3 * H - 4, ptrs[2], ptrs[3], ptrs[4]) != 0
+    assert hip.dali_hip_gru_recurrent_persistent(T, B, H, ptrs[0], ptrs[1], 3 * H + 4, ptrs[2], ptrs[3], ptrs[3]) != 0
+    assert b"overlap" in hip.dali_hip_last_error()
+    for p in ptrs:
+        hip.dali_hip_free(p)
 
 
 @pytest.mark.parametrize("B,I,sizes", [(3, 8, [8]), (5, 7, [6, 4, 9]), (32, 64, [64, 64]), (16, 128, [128, 64, 192])])
