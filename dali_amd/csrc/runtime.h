@@ -38,6 +38,11 @@ int sgemm_smallk(bool ta, bool tb, int M, int N, int K, float alpha, const float
 // (N = 4 H, columns gathered per hidden unit). 1: launched; 0: not a case for it; -1: failure (message set)
 int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
               float alpha, float beta, float* C, int ldc, const float* bias, const float* c_prev, float* c_out, float* h_out, int H);
+// The same pipeline over a stream of work items per workgroup (one workgroup per compute unit walks many tiles, its loads
+// running ahead across tile boundaries); `shares` > 1 cuts every tile's inner extent into that many contiguous shares that meet
+// in the library workspace (single products only). `cus`: compute units of the bound device. Same return values.
+int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
+                     float alpha, float beta, float* C, int ldc, int shares, int cus);
 // hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per kernel: later launches of that kernel, which may be recorded into a
 // graph, are launches only. Keyed on the kernel's address (kernels of one signature share a function type, so a flag inside a
 // generic lambda or template would be shared among them).

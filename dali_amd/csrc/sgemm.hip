@@ -853,6 +853,52 @@ static int run_tile(const GemmArgs& g, bool ta, bool tb, bool vec, int split_k) 
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
+// compute units of the bound device (0 when they cannot be read)
+static int device_cus() {
+    static int cus = -1;
+    if (cus < 0) {
+        int v = 0;
+        cus = hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, bound_device()) == hipSuccess ? v : 0;
+    }
+    return cus;
+}
+
+// The whole slabs of a product of one or two terms through the streaming kernel, what is left of the inner extents by a
+// checked launch that adds to the result. -1: not a case for it (nothing was launched).
+static int stream_product(const GemmArgs& g, bool ta, bool tb, int shares) {
+    GemmArgs whole = g, rest = g;
+    whole.nseg = rest.nseg = 0;
+    for (int s = 0; s < g.nseg; ++s) {
+        const GemmSeg& sg = g.seg[s];
+        const int kw = sg.K / 64 * 64, kr = sg.K - kw;
+        if (kw > 0) {
+            GemmSeg& d = whole.seg[whole.nseg++];
+            d = sg;
+            d.K = kw;
+        }
+        if (kr > 0) {
+            GemmSeg& d = rest.seg[rest.nseg++];
+            d = sg;
+            d.A = sg.A + (ta ? (size_t)kw * sg.lda : (size_t)kw);
+            d.B = sg.B + (tb ? (size_t)kw : (size_t)kw * sg.ldb);
+            d.K = kr;
+        }
+    }
+    if (whole.nseg == 0) return -1;
+    const float* as[2] = {whole.seg[0].A, whole.seg[1].A};
+    const float* bs[2] = {whole.seg[0].B, whole.seg[1].B};
+    const int ks[2] = {whole.seg[0].K, whole.seg[1].K};
+    const int cus = device_cus();
+    if (cus <= 0) return -1;
+    const int r = sgemm_dma_stream(ta, tb, whole.M, whole.N, whole.nseg, ks, as, bs, whole.seg[0].lda, whole.seg[0].ldb, whole.alpha, whole.beta, whole.C,
+                                   whole.ldc, shares, cus);
+    if (r < 0) return DALI_HIP_ERROR;
+    if (r == 0) return -1;
+    if (rest.nseg == 0) return DALI_HIP_OK;
+    rest.beta = 1.0f;
+    return launch_tile<64, 64, 64, 2, 2, false>(rest, ta, tb, true, 1, true);
+}
+
 // Row-major driver: C[M,N] = alpha * sum_s opA_s * opB_s + beta * C.
 // ta: A_s is stored as [K][M]; tb: B_s is stored as [N][K].
 static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K, const float* const* A,
@@ -936,6 +982,13 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
     }
     long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     static const int variant = getenv("DALI_HIP_GEMM_VARIANT") ? atoi(getenv("DALI_HIP_GEMM_VARIANT")) : 0;
+    // >0: that many shares of the inner extent through the streaming kernel for every product it takes; <0: never
+    static const int stream_env = getenv("DALI_HIP_GEMM_STREAM") ? atoi(getenv("DALI_HIP_GEMM_STREAM")) : 0;
+    const bool stream_fits = vec && g.nseg <= 2 && !g.map_on && !rows_may_overlap && (g.nseg == 1 || (g.seg[0].lda == g.seg[1].lda && g.seg[0].ldb == g.seg[1].ldb));
+    if (stream_env > 0 && stream_fits) {
+        const int st = stream_product(g, ta, tb, stream_env);
+        if (st >= 0) return st;
+    }
     if (tiles128 >= 192) return run_tile<128, 128, 32, 2>(g, ta, tb, vec, 1);
     // Small grids: 64x64 tiles, and when even those leave CUs with a single workgroup, split K so
     // that two workgroups share a CU and one's barriers and memory waits hide behind the other's MFMAs.
@@ -948,6 +1001,18 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         // order by the workgroup that finishes last.
         int nslab64 = 0;
         for (int s = 0; s < g.nseg; ++s) nslab64 += (g.seg[s].K + 63) / 64;
+        if (stream_env == 0 && stream_fits && g.nseg == 1) {
+            // one item per compute unit through the kernel whose loads write LDS themselves, in shares of at least four slabs
+            // ([256,1024] over 32000: 145 us against 158 us, against 210 us with B stored as [N][K]; [64,64] over 65536:
+            // 34 us against 65 us)
+            const int cus = device_cus();
+            int shares = cus > 0 ? (int)(cus / tiles64) : 0;
+            if (shares > nslab64 / 4) shares = nslab64 / 4;
+            if (shares >= 2) {
+                const int st = stream_product(g, ta, tb, shares);
+                if (st >= 0) return st;
+            }
+        }
         const int want = (int)((512 + tiles64 - 1) / tiles64);
         // (shares of at least four slabs, two when there are no more than eight: [256,1024] over K = 1024 16.4 -> 12.9 us,
         // [100,512] over K = 512 12.4 -> 8.9 us against shares of at least eight; shorter shares lose to their fold)

@@ -65,6 +65,12 @@ struct DmaArgs {
 __device__ __forceinline__ void dma16(unsigned lds_addr, unsigned voff, const char* base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
 }
+// the same for a base pointer that the compiler cannot prove to be the same in every lane (it is)
+__device__ __forceinline__ void dma16_uniform(unsigned lds_addr, unsigned voff, const char* base) {
+    const unsigned long long b = (unsigned long long)base;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b), hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+    dma16(lds_addr, voff, (const char*)(((unsigned long long)hi << 32) | lo));
+}
 // The compiler does not see these loads, so the waits for them are written out; they are also compiler barriers.
 __device__ __forceinline__ void wait_loads_but_4() { asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); }
 __device__ __forceinline__ void wait_loads_but_8() { asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); }
@@ -331,6 +337,348 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_kernel(DmaArgs g) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------- many tiles
+// The same pipeline over a stream of work items. An item is a 64x64 tile of C, or, with Z > 1, one of Z contiguous shares of
+// a tile's slabs (few tiles over a long inner extent). A workgroup walks its items one after the other and the loads run
+// ahead across the item boundary: while the sums of one item are exchanged and stored, the first slabs of the next are
+// already on their way. What it is for is the second case: [256,1024] over an inner extent of 32000 (a weight gradient of the
+// vocabulary projection) runs as 64 tiles x 4 shares, one item per compute unit, in 145 us (0.73 of the fp32 matrix peak)
+// with either operand order, where the register-staged kernel with shares took 158 us, 210 us with B stored as [N][K].
+// With whole tiles as items it is no faster than one workgroup per tile (4096^3: 1150 us against 1033 us; 8000 tiles of four
+// slabs: 195 us against 198 us): at 64x64x64 per slab every compute unit asks its die's cache for 32 KiB per microsecond,
+// 8 TB/s over the device, which is what those caches deliver, so the product of many tiles stays with the 128x128 kernel.
+// Items are numbered by tile (see tile_at) with the share fastest; the workgroups of one die (every eighth workgroup) take
+// a contiguous band of them, so that tiles worked on together share their operands in that die's second-level cache. Shares of a tile meet in the workspace: each publishes its 64x64 partial sums and draws a
+// ticket, the last one adds them in share order (the order does not depend on who finishes last).
+struct StreamArgs {
+    const float* A[2];
+    const float* B[2];
+    int slabs[2];
+    int lda, ldb;
+    int M, N;
+    float* C;
+    int ldc;
+    float alpha, beta;
+    int tiles_m, tiles_n, Z;
+    unsigned int* counters;  // one ticket counter per tile (zero at rest)
+    float* partials;         // [tile][share][4096]
+};
+
+constexpr int kFoldBytes = 16384;
+constexpr int kStreamLds = kDmaLds + kFoldBytes + 16;  // stages, exchange area, one flag
+
+template <bool TA, bool TB>
+__global__ __launch_bounds__(512, 1) void sgemm_dma_stream_kernel(StreamArgs g) {
+    // (no static LDS beside this: the loads address LDS from offset 0)
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    volatile int& is_last = *(volatile int*)(lds + kDmaLds + kFoldBytes);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = w & 3, kw = w >> 2;
+    const int wm = wave >> 1, wn = wave & 1, l16 = lane & 15, kq = lane >> 4;
+    const int M = g.M, N = g.N, Z = g.Z;
+    const int slabs0 = g.slabs[0], n_all = slabs0 + g.slabs[1];
+    const int items_total = g.tiles_m * g.tiles_n * Z;
+    // this workgroup's items: first, first + stride, ... (count of them)
+    int first, stride, count;
+    {
+        const int G = gridDim.x, b = blockIdx.x;
+        if ((G & 7) == 0) {
+            const int chunk = (items_total + 7) / 8, wgx = G / 8;
+            const int lo = (b & 7) * chunk, hi = lo + chunk < items_total ? lo + chunk : items_total;
+            first = lo + b / 8;
+            stride = wgx;
+            count = first < hi ? (hi - first + wgx - 1) / wgx : 0;
+        } else {
+            first = b;
+            stride = G;
+            count = first < items_total ? (items_total - first + G - 1) / G : 0;
+        }
+    }
+    if (count == 0) return;
+    auto share_begin = [&](int z) __attribute__((always_inline)) { return (int)((long)n_all * z / Z); };
+    // Tiles are numbered in column blocks four tiles wide, by rows inside a block: 32 consecutive tiles (what the 32
+    // workgroups of a die work on together) are 8 x 4 and ask their die's cache for 12 operand slabs per step, not 33.
+    auto tile_at = [&](int tile, int& mt, int& nt) __attribute__((always_inline)) {
+        const int per_block = g.tiles_m * 4, nb = tile / per_block, rem = tile - nb * per_block;
+        const int width = g.tiles_n - 4 * nb < 4 ? g.tiles_n - 4 * nb : 4;
+        mt = rem / width;
+        nt = 4 * nb + (rem - mt * width);
+    };
+    int total = 0;  // slabs of all items of this workgroup
+    for (int r = 0; r < count; ++r) {
+        const int z = (first + r * stride) % Z;
+        total += share_begin(z + 1) - share_begin(z);
+    }
+
+    const long a_step = (TA ? (long)64 * g.lda : 64L) * (long)sizeof(float);
+    const long b_step = (TB ? 64L : (long)64 * g.ldb) * (long)sizeof(float);
+    unsigned a_off[2], b_off[2], a_dst[2], b_dst[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        a_dst[q] = (unsigned)((w + 8 * q) * 1024);
+        b_dst[q] = (unsigned)(kBRegion + (w + 8 * q) * 1024);
+    }
+    // ---- the side that requests slabs
+    int i_r = 0, i_fj = 0, i_n = 0, i_g = 0;  // item, slab within it, its slabs, slab within the tile's inner extent
+    const char* ap = nullptr;
+    const char* bp = nullptr;
+    auto request_item = [&](int r) __attribute__((always_inline)) {
+        const int id = first + r * stride, tile = id / Z, z = id - tile * Z;
+        int mt, nt;
+        tile_at(tile, mt, nt);
+        const int m0 = 64 * mt, n0 = 64 * nt;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int c = w + 8 * q;
+            const int rr = 4 * c + (lane >> 4), s = lane & 15;
+            if (!TA) {
+                const int row = m0 + rr < M ? m0 + rr : M - 1;
+                a_off[q] = (unsigned)(((size_t)row * g.lda + 4 * ((s ^ rr) & 15)) * sizeof(float));
+            } else {
+                int col = m0 + 4 * (s ^ ((c & 3) << 2));
+                col = col < M ? col : M - 4;
+                a_off[q] = (unsigned)(((size_t)rr * g.lda + col) * sizeof(float));
+            }
+            if (!TB) {
+                int col = n0 + 4 * (s ^ ((c & 3) << 2));
+                col = col < N ? col : N - 4;
+                b_off[q] = (unsigned)(((size_t)rr * g.ldb + col) * sizeof(float));
+            } else {
+                const int row = n0 + rr < N ? n0 + rr : N - 1;
+                b_off[q] = (unsigned)(((size_t)row * g.ldb + 4 * ((s ^ rr) & 15)) * sizeof(float));
+            }
+        }
+        i_g = share_begin(z);
+        i_n = share_begin(z + 1) - i_g;
+        i_fj = 0;
+        const bool second = i_g >= slabs0;  // (only with two terms; shares are cut from single products)
+        ap = (const char*)(second ? g.A[1] : g.A[0]) + (long)(i_g - (second ? slabs0 : 0)) * a_step;
+        bp = (const char*)(second ? g.B[1] : g.B[0]) + (long)(i_g - (second ? slabs0 : 0)) * b_step;
+    };
+    auto issue = [&](int stage) __attribute__((always_inline)) {
+        dma16_uniform(a_dst[0] + stage * kStage, a_off[0], ap);
+        dma16_uniform(a_dst[1] + stage * kStage, a_off[1], ap);
+        dma16_uniform(b_dst[0] + stage * kStage, b_off[0], bp);
+        dma16_uniform(b_dst[1] + stage * kStage, b_off[1], bp);
+        ++i_fj;
+        ++i_g;
+        ap += a_step;
+        bp += b_step;
+        if (i_g == slabs0 && g.slabs[1] > 0) {
+            ap = (const char*)g.A[1];
+            bp = (const char*)g.B[1];
+        }
+        if (i_fj == i_n) {
+            ++i_r;
+            if (i_r < count) request_item(i_r);
+        }
+    };
+    request_item(0);
+    issue(0);
+    if (total > 1) issue(1);
+    if (total > 2) issue(2);
+
+    unsigned a_addr[2][2], b_addr[2][2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const int t = kw + 2 * tt;
+            const int ra = wm * 32 + s * 16 + l16, rb = wn * 32 + s * 16 + l16;
+            a_addr[tt][s] = !TA ? (unsigned)(ra * 256 + (((4 * t + kq) ^ ra) & 15) * 16) : (unsigned)((16 * t + 4 * kq) * 256 + ((ra ^ (kq << 4)) * 4));
+            b_addr[tt][s] = kBRegion + (TB ? (unsigned)(rb * 256 + (((4 * t + kq) ^ rb) & 15) * 16) : (unsigned)((16 * t + 4 * kq) * 256 + ((rb ^ (kq << 4)) * 4)));
+        }
+    floatx4 acc[2][2];
+    auto clear = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int si = 0; si < 2; ++si)
+#pragma unroll
+            for (int sj = 0; sj < 2; ++sj)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[si][sj][v] = 0.f;
+    };
+    clear();
+    floatx4 a4[2][2], b4[2][2];
+    auto load_ops = [&](auto ST, int tt, int o) __attribute__((always_inline)) {
+        constexpr int st = decltype(ST)::value;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            if (!TA) {
+                a4[o][s] = *(const floatx4*)(lds + a_addr[tt][s] + st * kStage);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) a4[o][s][c] = *(const float*)(lds + a_addr[tt][s] + st * kStage + c * 256);
+            }
+            if (TB) {
+                b4[o][s] = *(const floatx4*)(lds + b_addr[tt][s] + st * kStage);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) b4[o][s][c] = *(const float*)(lds + b_addr[tt][s] + st * kStage + c * 256);
+            }
+        }
+    };
+    auto mfma = [&](int o, int c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int si = 0; si < 2; ++si)
+#pragma unroll
+            for (int sj = 0; sj < 2; ++sj) acc[si][sj] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[o][si][c], b4[o][sj][c], acc[si][sj], 0, 0, 0);
+    };
+    // ---- the side that multiplies: its item, the slab within it
+    int c_r = 0, c_fj = 0, c_n;
+    {
+        const int z = first % Z;
+        c_n = share_begin(z + 1) - share_begin(z);
+    }
+    // the sums of the finished item leave: exchange between the wave sets, then C (or the tile's partial sums and a ticket)
+    auto finish_item = [&]() __attribute__((always_inline)) {
+        const int id = first + c_r * stride, tile = id / Z, z = id - tile * Z;
+        int mt, nt;
+        tile_at(tile, mt, nt);
+        const int m0 = 64 * mt, n0 = 64 * nt;
+        float out[16];
+#pragma unroll
+        for (int si = 0; si < 2; ++si)
+#pragma unroll
+            for (int sj = 0; sj < 2; ++sj)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) out[(si * 2 + sj) * 4 + v] = acc[si][sj][v];
+        // (the area was last read in the previous item's exchange, which every wave left before the barrier of a later slab)
+        float* red = (float*)(lds + kDmaLds);
+#pragma unroll
+        for (int v = 0; v < 8; ++v) red[(kw * 4 + wave) * 512 + v * 64 + lane] = kw == 0 ? out[8 + v] : out[v];
+        __syncthreads();
+        float sum[8];
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+            const float other = red[((1 - kw) * 4 + wave) * 512 + v * 64 + lane];
+            sum[v] = kw == 0 ? out[v] + other : other + out[8 + v];
+        }
+        const float alpha = g.alpha, beta = g.beta;
+        int last = 1;
+        if (Z > 1) {
+            float* part = g.partials + (size_t)tile * Z * 4096;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) __hip_atomic_store(part + (size_t)z * 4096 + v * 512 + tid, sum[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // the partial sums are acknowledged by memory before the ticket is drawn
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (tid == 0) {
+                const unsigned int ticket = __hip_atomic_fetch_add(g.counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                is_last = ticket == (unsigned int)Z - 1;
+            }
+            __syncthreads();
+            last = __builtin_amdgcn_readfirstlane(is_last);
+            if (last) {
+#pragma unroll
+                for (int v = 0; v < 8; ++v) sum[v] = 0.f;
+                for (int z0 = 0; z0 < Z; z0 += 4) {
+                    float t[4][8];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+#pragma unroll
+                        for (int v = 0; v < 8; ++v)
+                            t[u][v] = __hip_atomic_load(part + (size_t)(z0 + u < Z ? z0 + u : z0) * 4096 + v * 512 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+                        if (z0 + u < Z) {
+#pragma unroll
+                            for (int v = 0; v < 8; ++v) sum[v] += t[u][v];
+                        }
+                }
+                if (tid == 0) __hip_atomic_store(g.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (last) {
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const int e = kw * 8 + v;
+                const int m = m0 + wm * 32 + (e / 8) * 16 + 4 * kq + (e % 4), nn = n0 + wn * 32 + ((e / 4) % 2) * 16 + l16;
+                if (m < M && nn < N) {
+                    float* c = g.C + (size_t)m * g.ldc + nn;
+                    float r = alpha * sum[v];
+                    if (beta != 0.f) r += beta * *c;
+                    *c = r;
+                }
+            }
+        }
+        clear();
+        ++c_r;
+        c_fj = 0;
+        if (c_r < count) {
+            const int zn = (first + c_r * stride) % Z;
+            c_n = share_begin(zn + 1) - share_begin(zn);
+        }
+    };
+    auto slab_step = [&](auto ST, auto H1, auto H2, auto H3) __attribute__((always_inline)) {
+        constexpr int st = decltype(ST)::value;
+        constexpr bool has1 = decltype(H1)::value, has2 = decltype(H2)::value, has3 = decltype(H3)::value;
+        using NX = std::integral_constant<int, (st + 1) % 4>;
+        mfma(0, 0);
+        load_ops(ST, 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(0, 1);
+        if (has1) {
+            if (has2) wait_loads_but_4(); else wait_loads_all();
+            __builtin_amdgcn_s_barrier();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(0, 2);
+        if (has3) issue((st + 3) % 4);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(0, 3);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(1, 0);
+        if (has1) load_ops(NX{}, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(1, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(1, 3);
+        __builtin_amdgcn_sched_barrier(0);
+        if (++c_fj == c_n) finish_item();
+    };
+    auto tail_step = [&](auto J, auto R) __attribute__((always_inline)) {
+        constexpr int j = decltype(J)::value, r = decltype(R)::value;
+        if constexpr (j < r)
+            slab_step(std::integral_constant<int, j % 4>{}, std::integral_constant<bool, (j + 1 < r)>{}, std::integral_constant<bool, (j + 2 < r)>{},
+                      std::integral_constant<bool, (j + 3 < r)>{});
+    };
+    auto run_tail = [&](auto R) __attribute__((always_inline)) {
+        tail_step(std::integral_constant<int, 0>{}, R);
+        tail_step(std::integral_constant<int, 1>{}, R);
+        tail_step(std::integral_constant<int, 2>{}, R);
+        tail_step(std::integral_constant<int, 3>{}, R);
+        tail_step(std::integral_constant<int, 4>{}, R);
+        tail_step(std::integral_constant<int, 5>{}, R);
+    };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+    using S3 = std::integral_constant<int, 3>;
+    using Yes = std::true_type;
+    if (total > 2) wait_loads_but_8();
+    else if (total > 1) wait_loads_but_4();
+    else wait_loads_all();
+    __builtin_amdgcn_s_barrier();
+    load_ops(S0{}, 0, 0);
+    int i = 0;
+    for (; i + 7 <= total; i += 4) {
+        slab_step(S0{}, Yes{}, Yes{}, Yes{});
+        slab_step(S1{}, Yes{}, Yes{}, Yes{});
+        slab_step(S2{}, Yes{}, Yes{}, Yes{});
+        slab_step(S3{}, Yes{}, Yes{}, Yes{});
+    }
+    const int rest = total - i;  // 1 .. 6
+    if (rest == 1) run_tail(std::integral_constant<int, 1>{});
+    else if (rest == 2) run_tail(std::integral_constant<int, 2>{});
+    else if (rest == 3) run_tail(std::integral_constant<int, 3>{});
+    else if (rest == 4) run_tail(std::integral_constant<int, 4>{});
+    else if (rest == 5) run_tail(std::integral_constant<int, 5>{});
+    else run_tail(std::integral_constant<int, 6>{});
+}
+
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 template <bool TA, bool TB, bool GATES>
@@ -348,27 +696,79 @@ int launch(const DmaArgs& g, dim3 grid) {
     return 1;
 }
 
+
+// whole 64-deep slabs, 16-byte pieces that start on 16-byte boundaries and never straddle the end of a row, per-lane offsets
+// (relative to a pointer that walks along k) that fit 32 bits
+bool operands_fit(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb) {
+    if (nseg < 1 || nseg > 2 || M < 1 || N < 1) return false;
+    if (lda % 4 != 0 || ldb % 4 != 0 || (ta && M % 4 != 0) || (!tb && N % 4 != 0)) return false;
+    for (int s = 0; s < nseg; ++s) {
+        if (K[s] < 64 || K[s] % 64 != 0 || !aligned16(A[s]) || !aligned16(B[s])) return false;
+        const size_t a_span = ((size_t)(ta ? 64 : M) * lda + (ta ? M : 64)) * sizeof(float);
+        const size_t b_span = ((size_t)(tb ? N : 64) * ldb + (tb ? 64 : N)) * sizeof(float);
+        if (a_span >= ((size_t)1 << 32) || b_span >= ((size_t)1 << 32)) return false;
+    }
+    return true;
+}
+
+template <bool TA, bool TB>
+int launch_stream(const StreamArgs& g, int workgroups) {
+    auto kernel = sgemm_dma_stream_kernel<TA, TB>;
+    hipError_t e = reserve_dynamic_lds((const void*)kernel, kStreamLds);
+    if (e != hipSuccess) return fail("sgemm: cannot reserve %d bytes of LDS: %s", kStreamLds, hipGetErrorString(e));
+    hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(512), kStreamLds, stream(), g);
+    e = hipGetLastError();
+    if (e != hipSuccess) return fail("sgemm launch failed: %s", hipGetErrorString(e));
+    return 1;
+}
+
 }  // namespace
+
+int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
+                     float alpha, float beta, float* C, int ldc, int shares, int cus) {
+    static const int enabled = getenv("DALI_HIP_GEMM_DMA") ? atoi(getenv("DALI_HIP_GEMM_DMA")) : 1;
+    if (!enabled || cus < 8 || !operands_fit(ta, tb, M, N, nseg, K, A, B, lda, ldb)) return 0;
+    StreamArgs g = {};
+    int slabs = 0;
+    for (int s = 0; s < 2; ++s) {
+        g.A[s] = s < nseg ? A[s] : nullptr;
+        g.B[s] = s < nseg ? B[s] : nullptr;
+        g.slabs[s] = s < nseg ? K[s] / 64 : 0;
+        slabs += g.slabs[s];
+    }
+    g.lda = lda;
+    g.ldb = ldb;
+    g.M = M;
+    g.N = N;
+    g.C = C;
+    g.ldc = ldc;
+    g.alpha = alpha;
+    g.beta = beta;
+    g.tiles_m = (M + 63) / 64;
+    g.tiles_n = (N + 63) / 64;
+    const long tiles = (long)g.tiles_m * g.tiles_n;
+    if (tiles > (1L << 24)) return 0;
+    int Z = shares < 1 ? 1 : shares;
+    if (Z > slabs) Z = slabs;
+    if (Z > 1 && (nseg != 1 || tiles > (long)kWorkspaceCounters || (size_t)tiles * Z * 4096 * sizeof(float) > kWorkspacePartialBytes)) Z = 1;
+    g.Z = Z;
+    g.counters = (unsigned int*)workspace();
+    g.partials = (float*)(workspace() + kWorkspaceCounterBytes);
+    const long items = tiles * Z;
+    // every workgroup has a compute unit to itself (its LDS); a whole number of workgroups per die keeps the bands of tiles
+    int workgroups = cus - cus % 8;
+    if (items < workgroups) workgroups = (int)items;
+    if (!ta && !tb) return launch_stream<false, false>(g, workgroups);
+    if (!ta && tb) return launch_stream<false, true>(g, workgroups);
+    if (ta && !tb) return launch_stream<true, false>(g, workgroups);
+    return launch_stream<true, true>(g, workgroups);
+}
 
 int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
               float alpha, float beta, float* C, int ldc, const float* bias, const float* c_prev, float* c_out, float* h_out, int H) {
     static const int enabled = getenv("DALI_HIP_GEMM_DMA") ? atoi(getenv("DALI_HIP_GEMM_DMA")) : 1;
-    if (!enabled || nseg < 1 || nseg > 2 || M < 1 || N < 1) return 0;
+    if (!enabled || !operands_fit(ta, tb, M, N, nseg, K, A, B, lda, ldb)) return 0;
     const bool gates = bias != nullptr;
-    // whole 64-deep slabs, 16-byte pieces that start on 16-byte boundaries and never straddle the end of a row
-    if (lda % 4 != 0 || ldb % 4 != 0 || (ta && M % 4 != 0) || (!tb && N % 4 != 0)) return 0;
-    size_t a_rows = 0, b_rows = 0;
-    for (int s = 0; s < nseg; ++s) {
-        if (K[s] < 64 || K[s] % 64 != 0 || !aligned16(A[s]) || !aligned16(B[s])) return 0;
-        a_rows = ta ? (size_t)K[s] : (size_t)M;
-        b_rows = tb ? (size_t)N : (size_t)K[s];
-        // the per-lane offsets are 32-bit and relative to a pointer that walks along k
-        const size_t a_span = ((size_t)(ta ? 64 : M) * lda + (ta ? M : 64)) * sizeof(float);
-        const size_t b_span = ((size_t)(tb ? N : 64) * ldb + (tb ? 64 : N)) * sizeof(float);
-        if (a_span >= ((size_t)1 << 32) || b_span >= ((size_t)1 << 32)) return 0;
-    }
-    (void)a_rows;
-    (void)b_rows;
     DmaArgs g = {};
     for (int s = 0; s < 2; ++s) {
         g.A[s] = s < nseg ? A[s] : nullptr;

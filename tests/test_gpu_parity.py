@@ -264,7 +264,11 @@ def test_prefetch_of_pinned_arrays(gpu, D, rng):
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (5, 11, 7), (64, 64, 64), (65, 130, 33), (256, 4096, 128), (300, 200, 100),
                                    (132, 72, 640), (252, 1000, 1000), (1100, 2300, 260), (2052, 2052, 132),
                                    # few tiles over a long inner extent: shares of K folded across workgroups
-                                   (64, 64, 8192), (128, 576, 20001), (130, 70, 4100)])
+                                   (64, 64, 8192), (128, 576, 20001), (130, 70, 4100),
+                                   # the same with whole 64-deep slabs and aligned rows: one share per compute unit through the
+                                   # kernel that walks a list of work items (the last two are the weight and input gradients of a
+                                   # [256]->[32000] projection at 1024 rows)
+                                   (192, 320, 4160), (256, 1024, 32000), (1024, 32000, 256)])
 @pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
 def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
     """dali_hip_sgemm(transB, transA, m, n, k, alpha, B, ldb, A, lda, beta, C, ldc) as cublasSgemm is called in
