@@ -132,6 +132,8 @@ struct RowParams {
     bool exact = false;      // register-cached rows: C == TPR * EPT * VEC, the chunk guards fall away
     bool ragged = false;     // rows not aligned to the vector: element-aligned vector accesses
     bool tail = false;       // ragged, and C is no multiple of VEC: the rest of a row is handled one element to a thread
+    bool peel = false;       // ragged rows that all start at the same offset within 16 bytes: the vectors begin at the first aligned
+                             // element of the row, the 0..3 elements in front of it go with the rest behind the last vector
     int EPT_L = 0;           // cached rows: the last EPT_L of the EPT vectors a thread holds live in LDS instead of registers
     bool split = false;      // maps without a reduction over few long rows: every row is cut into S pieces, one workgroup each
     int band_unroll = 1;     // rows of a band whose loads are issued together
@@ -256,11 +258,12 @@ struct BodyEmitter {
         if (n.kept && rp.cached && per_element) {
             if (declared.count(id)) return var;
             declared.insert(id);
+            const std::string slot = "t" + std::to_string(id) + "[e][j]";
             if ((*first_body)[id] == body_index) {
                 const std::string r = raw(id);  // may itself append statements (nested kept or shared nodes): before ours
-                stmts << "const " << ctype(n.dtype) << " " << var << " = " << r << "; t" << id << "[e][j] = " << var << ";\n";
+                stmts << "const " << ctype(n.dtype) << " " << var << " = " << r << "; " << slot << " = " << var << ";\n";
             } else {
-                stmts << "const " << ctype(n.dtype) << " " << var << " = t" << id << "[e][j];\n";
+                stmts << "const " << ctype(n.dtype) << " " << var << " = " << slot << ";\n";
             }
             return var;
         }

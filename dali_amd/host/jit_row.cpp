@@ -42,21 +42,36 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
         ss << "  constexpr bool row_ok = true;  // one row per workgroup: the grid has exactly R of them\n  (void)R;\n";
     else
         ss << "  const bool row_ok = row < R;\n  if (!row_ok) row = R - 1;\n";
-    ss << "  const int CH = (int)(C / VEC); (void)CH;\n";
+    if (!rp.peel) ss << "  const int CH = (int)(C / VEC); (void)CH;\n";
     }
     emit_row_prologue(ss, P, L);
-    // ragged rows: the C % VEC elements past the last whole vector go one to a thread, through the same bodies
-    // (slot EPT of the register cache, j = 0)
-    const bool tail = rp.ragged && rp.tail;
-    if (tail) ss << "  const bool tail_on = tr < (int)(C - (long)CH * VEC)" << (rp.split ? " && seg == S - 1" : "") << ";\n  const int tail_col = CH * VEC + tr;\n";
-    // register-cached rows whose length fills every chunk need no chunk guard
-    const std::string chunk_guard = rp.cached && rp.exact ? "    {\n" : "    if (ch < CH) {\n";
-
     // FULL leaves (inputs)
     std::vector<int> full_leaves;
     for (size_t i = 0; i < P.arrays.size(); ++i)
         if (!P.arrays[i].is_dest && P.arrays[i].cls == Cls::FULL && !P.arrays[i].gather_source) full_leaves.push_back((int)i);
-    // is each leaf referenced? (an array may only be a gather source)
+    // vector accesses go through v<i>: the row pointer, moved to the row's first 16-byte boundary when the rows are peeled
+    const std::string vp = rp.peel ? "v" : "q";
+    if (rp.peel) {
+        int first = -1;
+        for (size_t i = 0; i < P.arrays.size() && first < 0; ++i)
+            if (P.arrays[i].cls == Cls::FULL && !P.arrays[i].gather_source) first = (int)i;
+        // (rows as wide as a wave or wider: up to the first 128-byte boundary, so that a wave's kilobyte is eight whole cache lines)
+        ss << "  const int head = (int)((0u - (unsigned int)((unsigned long)q" << first << " >> 2)) & " << (rp.TPR >= 64 && rpn.dom.C >= 8192 ? 31 : 3) << "u);  // elements in front of the row's first boundary\n";
+        ss << "  const int CH = (int)((C - head) / VEC); (void)CH;\n";
+        for (size_t i = 0; i < P.arrays.size(); ++i)
+            if (P.arrays[i].cls == Cls::FULL && !P.arrays[i].gather_source)
+                ss << "  " << (P.arrays[i].is_dest ? "" : "const ") << ctype(P.arrays[i].buf->dtype) << "* v" << i << " = q" << i << " + head;\n";
+    }
+    const std::string col_of_ch = rp.peel ? "head + ch * VEC + j" : "ch * VEC + j";
+    // ragged rows: the C % VEC elements past the last whole vector go one to a thread, through the same bodies
+    // (slot EPT of the register cache, j = 0)
+    const bool tail = rp.ragged && rp.tail;
+    // (peeled rows: thread tr < head takes element tr, the others the elements behind the last vector, head + CH * VEC + (tr - head))
+    if (tail) ss << "  const bool tail_on = tr < (int)(C - (long)CH * VEC)" << (rp.split ? " && seg == S - 1" : "") << ";\n  const int tail_col = "
+                 << (rp.peel ? "tr < head ? tr : CH * VEC + tr" : "CH * VEC + tr") << ";\n";
+    // register-cached rows whose length fills every chunk need no chunk guard
+    const std::string chunk_guard = rp.cached && rp.exact ? "    {\n" : "    if (ch < CH) {\n";
+
     if (rp.cached && rp.EPT_L > 0) {
         // Hybrid row cache: a thread keeps its first EPT_R vectors in registers and the other EPT_L in LDS (its own
         // 16 bytes per slot, so no barrier is involved); two 1024-thread workgroups then fit a CU where the registers
@@ -74,7 +89,7 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
         for (int i : full_leaves) {
             const std::string t = ctype(P.arrays[i].buf->dtype);
             ss << "      " << t << " ld" << i << "[VEC];\n";
-            emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "ld" + std::to_string(i), "      ", rp.nt_loads, rp.ragged);
+            emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "ld" + std::to_string(i), "      ", rp.nt_loads, rp.ragged && !rp.peel, vp);
             ss << "      if (e < EPT_R) {\n        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) xr" << i << "[e < EPT_R ? e : 0][j] = ld" << i << "[j];\n      } else {\n";
             ss << "        dali_vec<" << t << ", VEC> lv; _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) lv.v[j] = ld" << i << "[j];\n";
             ss << "        dali_store<" << t << ", VEC>(&xl" << i << "[e >= EPT_R ? e - EPT_R : 0][tid * VEC], lv);\n      }\n";
@@ -90,7 +105,7 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
             ss << "  " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[EPT + " << (tail ? 1 : 0) << "][VEC];\n";
         }
         ss << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n" << chunk_guard;
-        for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i) + "[e]", "      ", rp.nt_loads, rp.ragged);
+        for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i) + "[e]", "      ", rp.nt_loads, rp.ragged && !rp.peel, vp);
         ss << "    }\n  }\n";
         if (tail) {
             ss << "  if (tail_on) {\n";
@@ -122,7 +137,7 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
                 o << "  for (int ch = tr; ch < CH; ch += TPR) {\n    {\n";
             for (int i : full_leaves) {
                 o << "      " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n";
-                emit_leaf_load(o, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", rp.nt_loads, rp.ragged);
+                emit_leaf_load(o, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", rp.nt_loads, rp.ragged && !rp.peel, vp);
             }
         }
     };
@@ -162,7 +177,7 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
         }
         auto emit_phase_loop = [&](std::ostringstream& o, int div_mode, std::vector<std::string>* divisors) {
             open_loop(o);
-            o << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        const int col = ch * VEC + j; (void)col;\n";
+            o << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        const int col = " << col_of_ch << "; (void)col;\n";
             BodyEmitter be(P, rp, true, p, &rpn.first_body);
             be.div_mode = div_mode;
             be.divisors = divisors;
@@ -398,7 +413,11 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
                 const ArrayArg& d = P.arrays[o.array];
                 std::string t = ctype(d.buf->dtype);
                 std::string ov = "o" + std::to_string(o.array);
-                if (rp.VEC > 1 && rp.ragged) {
+                if (rp.VEC > 1 && rp.peel) {
+                    pre << "        dali_vec<" << t << ", VEC> " << ov << ";\n";
+                    if (o.op != OPERATOR_T_EQL) pre << "        " << ov << " = dali_load<" << t << ", VEC>(v" << o.array << " + (long)ch * VEC);\n";
+                    post << "        " << (rp.nt_stores ? "dali_store_nt<" : "dali_store<") << t << ", VEC>(v" << o.array << " + (long)ch * VEC, " << ov << ");\n";
+                } else if (rp.VEC > 1 && rp.ragged) {
                     pre << "        dali_vec<" << t << ", VEC> " << ov << ";\n";
                     if (o.op != OPERATOR_T_EQL) pre << "        " << ov << " = dali_loadu<" << t << ", VEC>(q" << o.array << " + (long)ch * VEC);\n";
                     post << "        " << (rp.nt_stores ? "dali_storeu_nt<" : "dali_storeu<") << t << ", VEC>(q" << o.array << " + (long)ch * VEC, " << ov << ");\n";
@@ -416,7 +435,7 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
                 body << "          " << ov << ".v[j] = " << op_combine(o.op, ov + ".v[j]", "(" + t + ")(" + v + ")") << ";\n";
             }
             os << pre.str();
-            os << "        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n          const int col = ch * VEC + j; (void)col;\n";
+            os << "        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n          const int col = " << col_of_ch << "; (void)col;\n";
             os << be.stmts.str() << body.str();
             os << "        }\n" << post.str();
             os << "      }\n    }\n  }\n";
@@ -474,6 +493,24 @@ static bool ragged_ok(const Program& P, const Domain& dom) {
         if (a.col_stride != 1) return false;
     }
     return true;
+}
+
+// every vector-accessed array starts its rows at the same distance from a 16-byte boundary: 4-byte elements, offsets and row
+// strides congruent modulo 4 (buffers themselves are 256-byte aligned); positions matter to nothing but the element values
+// (no argmax / argmin, whose ties go by the order in which a thread visits its elements)
+static bool peel_ok(const Program& P, const Domain& dom) {
+    if (dom.C < 64) return false;
+    long off = -1, rs = -1;
+    for (const ArrayArg& a : P.arrays) {
+        if (a.gather_source || a.cls != Cls::FULL) continue;
+        if (a.col_stride != 1 || size_of_dtype(a.buf->dtype) != 4 || a.row_index >= 0) return false;
+        const long o = (long)(a.buf->offset % 4), r = (long)(a.row_stride % 4);
+        if (off < 0) { off = o; rs = r; }
+        if (o != off || r != rs) return false;
+    }
+    for (const PNode& n : P.nodes)
+        if (n.kind == Kind::ARG_AXIS_REDUCE || n.kind == Kind::ARG_ALL_REDUCE || n.kind == Kind::GATHER) return false;
+    return off >= 0;
 }
 
 // `totals`: further requests whose destination holds one element and whose root is [scalar arithmetic over] one full
@@ -586,6 +623,19 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
         rp.ragged = true;
         rp.tail = dom.C % rp.VEC != 0;
     }
+    // Rows that are not aligned to the vector but all start at the same offset within 16 bytes (contiguous buffers of odd row
+    // length): vectors from the row's first 16-byte boundary, from its first 128-byte boundary when the row has 8192 elements or
+    // more ([2048,50257] softmax 165 -> 150 us, 163 us with 16-byte boundaries; a wave's unaligned kilobyte touches nine cache
+    // lines instead of eight and writes partial lines at both ends).
+    static const int peel_env = env_int("DALI_HIP_ROW_PEEL", 1);
+    // Long rows whose vectors are aligned but whose length is no whole number of cache lines gain the same way from starting at
+    // a 128-byte boundary ([2048,50256]: 156 -> 154 us, [2048,45000]: 142 -> 137 us).
+    const bool line_rows = rp.VEC == 4 && !rp.ragged && dom.C >= 8192 && dom.C % 32 != 0;
+    if ((rp.ragged || line_rows) && peel_env && nph > 0 && peel_ok(P, dom)) {
+        rp.ragged = true;
+        rp.peel = true;
+        rp.tail = true;
+    }
     int64_t CH = dom.C / rp.VEC;
     int n_full = 0, max_el = 4;
     for (const ArrayArg& a : P.arrays)
@@ -636,7 +686,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
         bool writes_rows = false;
         for (const Output& o : rpn.outputs) writes_rows = writes_rows || o.cls == Cls::FULL;
         if (writes_rows) tpr = std::max(tpr, std::min(64, pow2ceil((int)std::max<int64_t>(1, CH))));
-        if (rp.tail) tpr = std::max(tpr, 4);  // one thread per element past the last whole vector
+        if (rp.tail) tpr = std::max(tpr, rp.peel ? 8 : 4);  // one thread per element outside the whole vectors
         tpr = std::min(tpr, tpr_cap);
         int64_t ept = (CH + tpr - 1) / tpr;
         // every FULL input is held in registers across the phases: bound the footprint
@@ -652,7 +702,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
     }
     rp.RPB = rp.BT / rp.TPR;
     rp.NW = rp.TPR > 64 ? rp.TPR / 64 : 1;
-    rp.exact = nph > 0 && rp.cached && dom.C == (int64_t)rp.TPR * rp.EPT * rp.VEC;
+    rp.exact = nph > 0 && rp.cached && !rp.peel && dom.C == (int64_t)rp.TPR * rp.EPT * rp.VEC;
     // A 1024-thread row block fills a CU by itself unless it stays within 64 VGPRs; two resident
     // blocks let one row's loads overlap another row's arithmetic.
     static const int wpe = env_int("DALI_HIP_ROW_WAVES_PER_EU", -1);
@@ -721,7 +771,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
     rp.nt_loads = nt_l >= 0 ? nt_l != 0 : dom.R * dom.C * (int64_t)max_el >= ((int64_t)64 << 20);
     rp.nt_stores = nt_s >= 0 ? nt_s != 0 : rpn.n_phases > 0;
     params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached << "," << rp.waves_per_eu << ","
-           << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail << "," << rp.EPT_L << (rp.split ? "S" : "") << (rp.band > 1 ? "B" + std::to_string(rp.band) + "u" + std::to_string(rp.band_unroll) : std::string());
+           << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail << rp.peel << "," << rp.EPT_L << (rp.split ? "S" : "") << (rp.band > 1 ? "B" + std::to_string(rp.band) + "u" + std::to_string(rp.band_unroll) : std::string());
     if (n_totals) {
         // one 8-byte slot per workgroup and total in the workspace's 32 MiB of partial results
         const int64_t blocks = (dom.R + rp.RPB - 1) / rp.RPB;

@@ -941,6 +941,41 @@ def test_rows_cached_partly_in_lds(gpu, D, O, rng, cols):
     assert np.array_equal((arr(D, xi) - op.min(arr(D, xi), [1], True)).numpy(), xi - xi.min(1, keepdims=True))
 
 
+@pytest.mark.parametrize("rows,cols,skip", [(5, 50257, 0), (4, 45000, 0), (3, 8200, 0), (7, 8191, 0), (9, 16390, 5), (6, 8300, 2), (40, 67, 0), (33, 1001, 3),
+                                            (4, 9000, 1)])
+def test_rows_that_start_off_the_vector_boundary(gpu, D, O, rng, rows, cols, skip):
+    """Rows whose starts fall anywhere within 16 bytes (an odd row length, a view that drops leading columns), or aligned rows
+    whose length is no whole number of 128-byte lines: the vectors begin at the row's first boundary and the elements in front
+    of it go one to a thread together with the rest behind the last vector. Source and destination here share offset and row
+    stride, so the peeled form applies; the values must not depend on where a row starts."""
+    op = D.op
+    x = (rng.randn(rows, cols) * 3).astype(np.float32)
+    X = arr(D, x)
+    V = X[:, skip:] if skip else X
+    xv = x[:, skip:].astype(np.float64)
+    e = np.exp(xv - xv.max(-1, keepdims=True))
+    want = e / e.sum(-1, keepdims=True)
+    # into a fresh array (for a view: other row stride than the source, the unaligned form), then in place (the peeled form)
+    close(op.softmax(V).numpy(), want, rtol=1e-5, atol=1e-12)
+    assert D.last_kernel_kinds() == "row"
+    V.assign(op.softmax(V), 0)
+    assert D.last_kernel_kinds() == "row"
+    got = X.numpy()
+    close(got[:, skip:], want, rtol=1e-5, atol=1e-12)
+    assert np.array_equal(got[:, :skip], x[:, :skip])  # the columns in front of the view are untouched
+    close(got[:, skip:].sum(-1), 1.0, rtol=0, atol=2e-6)
+    # log-sum-exp per row (a per-row result only) and a row-normalised map with += into the rows
+    y = (rng.randn(rows, cols) * 2).astype(np.float32)
+    Y = arr(D, y)
+    m = op.max(Y, [1], True)
+    lse = (op.log(op.sum(op.exp(Y - m), [1], True)) + m).numpy()
+    y64 = y.astype(np.float64)
+    close(lse[:, 0], np.log(np.exp(y64 - y64.max(1, keepdims=True)).sum(1)) + y64.max(1), rtol=1e-5, atol=1e-5)
+    Z = arr(D, y)
+    Z.assign(Y - op.mean(Y, [1], True), 1)
+    close(Z.numpy(), y64 + (y64 - y64.mean(1, keepdims=True)), rtol=1e-5, atol=2e-5)
+
+
 @pytest.mark.parametrize("shape,axis", [((8, 262144), -1), ((3, 524288), 1), ((2, 3, 131072), 2), ((4096, 1000), 0), ((513, 257), 0),
                                         ((16, 300, 64), 1), ((16, 300, 64), 0), ((70000, 16), 0), ((64, 1000), 0)])
 def test_softmax_over_few_long_rows_and_against_the_layout(gpu, D, O, rng, shape, axis):
