@@ -545,6 +545,18 @@ def main():
                                               "frac_hbm": round(sbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                                               "launches_incl_index_sort": rec.launches, "distinct_rows": uniq}
         del table, ids, upd, g, rec
+        # softmax away from the C1 shape: rows of a vocabulary that is no multiple of anything (one row = 201,028 bytes, every
+        # row starts elsewhere within a cache line) and the middle axis of a 3-D array; bytes = one read + one write
+        for tag, shp, axis in (("softmax_rows_2048x50257", (2048, 50257), -1), ("softmax_middle_axis_256x512x512", (256, 512, 512), 1),
+                               ("softmax_middle_axis_64x1024x1024", (64, 1024, 1024), 1)):
+            xs_ = D.Array.from_numpy(np.random.RandomState(18).randn(*shp).astype(np.float32))
+            with D.Recording() as rec:
+                op.softmax(xs_, axis).eval()
+            us = time_recording(rec, 20)
+            nb = 2.0 * 4 * float(np.prod(shp))
+            nxt[tag] = {"us": round(us, 2), "GB/s": round(nb / us / 1e3, 1), "frac_hbm": round(nb / us / 1e3 / HBM_PEAK_GBS, 4), "launches": rec.launches,
+                        "kernel": D.last_kernel_kinds()}
+            del xs_, rec
         sm = D.Array.from_numpy(np.random.RandomState(17).uniform(0.5, 1.5, (8192, 8192)).astype(np.float32))
         with D.Recording() as rec:
             op.cumsum(sm).eval()

@@ -96,6 +96,8 @@ HIP_SYMBOLS = {
     "dali_hip_lstm_recurrent_persistent_supported": (_i, [_i, _i]),
     "dali_hip_gru_recurrent_persistent": (_i, [_i, _i, _i, H, H, _i, H, H, H]),
     "dali_hip_gru_recurrent_persistent_supported": (_i, [_i, _i]),
+    "dali_hip_softmax_axis": (_i, [H, H, C.c_int64, _i, C.c_int64]),
+    "dali_hip_softmax_axis_supported": (_i, [C.c_int64, _i, C.c_int64]),
     "dali_hip_argsort_i32": (_i, [H, C.c_int64, C.c_int32, H, H]),
     "dali_hip_argsort_i32_noalloc": (_i, [H, C.c_int64, C.c_int32, H, H]),
     "dali_hip_topk_rows": (_i, [H, _i, C.c_int64, C.c_int32, C.c_int32, _i, _i, H]),

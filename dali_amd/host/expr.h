@@ -104,6 +104,8 @@ void lstm_step_small(const Array& x, const Array& h, const Array& c, const Array
 // the recurrent half of an LSTM over a whole sequence in one launch: pre [T, B, 4H] = x.W + bias for every step
 void lstm_recurrent_persistent(const Array& pre, const Array& U, const Array& h0, const Array& c0, const Array& hs, const Array& c_out);
 void gru_recurrent_persistent(const Array& pre, const Array& U, const Array& h0, const Array& hs, const Array& scratch);
+// softmax of a contiguous fp32 buffer seen as [outer, extent, inner] along `extent`, one pass over memory (records itself like any other launch)
+void softmax_axis_launch(const Array& x, const Array& out, long long outer, int extent, long long inner);
 // stride-1 convolution of a dense float NHWC image [N,H,W,C] (C a multiple of 4) with filters [O,fh,fw,C], fh <= 8:
 // one padding copy and one multi-term product, no patch matrix; returns [N, out_h, out_w, O]
 Array conv2d_direct_nhwc(const Array& x, const Array& filters, int pad_top, int pad_left, int pad_bottom, int pad_right);

@@ -237,4 +237,20 @@ void gru_recurrent_persistent(const Array& pre, const Array& U, const Array& h0,
     }
 }
 
+void softmax_axis_launch(const Array& x, const Array& out, long long outer, int extent, long long inner) {
+    const float* xp = (const float*)x.device_ptr();
+    float* op = (float*)out.device_ptr(memory::AM_OVERWRITE);
+    jit_stats().kernels_launched++;
+    jit_stats().last_kernel_kinds = "softmax_axis";
+    check_hip(dali_hip_softmax_axis(xp, op, outer, extent, inner), "softmax along an inner axis");
+    if (g_recording) {
+        note_recorded_write(out.expression()->memory);
+        std::vector<Array> keep = {x, out};
+        g_recording->push_back([=]() {
+            (void)keep;
+            check_hip(dali_hip_softmax_axis(xp, op, outer, extent, inner), "softmax along an inner axis replay");
+        });
+    }
+}
+
 }  // namespace dali

@@ -315,6 +315,18 @@ int dali_hip_gru_recurrent_persistent(int steps, int batch, int hidden, const fl
 /* 0: not served; 1: served; 2: served and expected to beat the launch-per-step form */
 int dali_hip_gru_recurrent_persistent_supported(int batch, int hidden);
 
+/* ------------------------------------------------------------- softmax along an inner axis */
+/*
+ * out = softmax(x) along the middle axis of a contiguous fp32 array seen as [outer, extent, inner]
+ * (reference: op::softmax(logits, axis), dali/array/op/softmax.cpp:5-8, for an axis other than the last; outer = 1 is the
+ * leading axis of a matrix). One pass over memory: a workgroup keeps a strip of the reduced axis in registers. inner must be
+ * a multiple of 4 and at least 16, extent at most 2048 (at most 512 for the widest strips), both arrays 16-byte aligned;
+ * x and out may be the same array. dali_hip_softmax_axis_supported returns 1 for the sizes the kernel takes (the generated
+ * three-pass form serves the others).
+ */
+int dali_hip_softmax_axis(const float* x, float* out, long long outer, int extent, long long inner);
+int dali_hip_softmax_axis_supported(long long outer, int extent, long long inner);
+
 /* ------------------------------------------------------------- scatter */
 /*
  * Stable ordering of n int32 keys held in device memory: sorted_keys[p] is the p-th smallest key and
