@@ -75,8 +75,13 @@ static std::string gen_scatter_rows_kernel(const Program& P, const IvLayout& L, 
 // together make N * N comparisons against LDS, which the device does in the shadow of the memory traffic; no index
 // ordering pass (and no launch for it) is needed. The values are an expression evaluated where they are used, as in the
 // reference's fused scatter kernel (gather.cpp:126-143). Indices outside the destination are skipped.
-static std::string gen_scatter_scan_kernel(const Program& P, const IvLayout& L, OPERATOR_T op, int root, int VEC, int KCAP, const std::string& kname) {
+//
+// `sorted`: for index vectors beyond what LDS holds. P.arrays[1] then holds the indices in ascending order (stable) and
+// P.arrays[2] the input position of each; the wave of a sorted position works when it heads a run of equal indices, and the
+// run's rows of values, still an expression, are evaluated in input order as above.
+static std::string gen_scatter_scan_kernel(const Program& P, const IvLayout& L, OPERATOR_T op, int root, int VEC, int KCAP, const std::string& kname, bool sorted) {
     const std::string t = ctype(P.arrays[0].buf->dtype);
+    const size_t first_operand = sorted ? 3 : 2;
     const int U = VEC == 4 ? 4 : 16;
     RowParams rp;
     rp.cached = false;
@@ -89,6 +94,13 @@ static std::string gen_scatter_scan_kernel(const Program& P, const IvLayout& L, 
     ss << "  constexpr int VEC = " << VEC << ", U = " << U << ", KCAP = " << KCAP << ", TILE = 64 * VEC * U;\n";
     ss << "  const int N = A.iv[" << L.shape_pos[0] << "], D = A.iv[" << L.shape_pos[0] + 1 << "], V = A.iv[" << L.shape_pos[0] + 2 << "];\n";
     ss << "  const long C = D; (void)C;\n";
+    if (sorted) {
+        ss << "  (void)KCAP;\n  const int* sk = (const int*)A.p[1];\n  const int* pm = (const int*)A.p[2];\n";
+        ss << "  const int lane = threadIdx.x & 63;\n  const int p = (int)blockIdx.x * 16 + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));\n";
+        ss << "  if (p >= N) return;\n  const int key = sk[p];\n  const bool valid = (unsigned)key < (unsigned)V;\n";
+        ss << "  if (!valid) return;  // no such destination row: skipped\n  if (p > 0 && sk[p - 1] == key) return;  // only the head of a run of equal indices works\n";
+        ss << "  int q_end = p + 1;\n  while (q_end < N && sk[q_end] == key) ++q_end;\n";
+    } else {
     ss << "  __shared__ __attribute__((aligned(16))) int lk[KCAP];\n";
     ss << "  const int* keys = (const int*)A.p[1];\n";
     ss << "  const int lane = threadIdx.x & 63;\n  const int p = (int)blockIdx.x * 16 + (int)(threadIdx.x >> 6);\n";
@@ -97,7 +109,8 @@ static std::string gen_scatter_scan_kernel(const Program& P, const IvLayout& L, 
     ss << "  constexpr int KF = (KCAP + 4095) / 4096;\n  dali_vec<int, 4> kf[KF];\n";
     ss << "  _Pragma(\"unroll\") for (int f = 0; f < KF; ++f) {\n    const int t = (int)threadIdx.x * 4 + f * 4096;\n"
           "    if (t + 3 < N) kf[f] = dali_loadu<int, 4>(keys + t);\n    else { _Pragma(\"unroll\") for (int b = 0; b < 4; ++b) kf[f].v[b] = t + b < N ? keys[t + b] : -1; }\n  }\n";
-    for (size_t i = 2; i < P.arrays.size(); ++i) {
+    }
+    for (size_t i = first_operand; i < P.arrays.size(); ++i) {
         const ArrayArg& a = P.arrays[i];
         const std::string ty = ctype(a.buf->dtype);
         if (a.cls == Cls::SCAL) ss << "  const " << ty << " sl" << i << " = ((const " << ty << "*)A.p[" << i << "])[0];\n";
@@ -107,7 +120,9 @@ static std::string gen_scatter_scan_kernel(const Program& P, const IvLayout& L, 
     }
     ss << "  const long drs = A.iv[" << L.stride_pos[0] << "], dcs = A.iv[" << L.stride_pos[0] + 1 << "]; (void)dcs;\n";
     ss << "  " << t << "* drow = (" << t << "*)A.p[0] + (long)(valid ? key : 0) * drs;\n";
-    ss << "  " << t << " acc[U][VEC];\n  const dali_vec<int, 4>* lk4 = reinterpret_cast<const dali_vec<int, 4>*>(lk);\n";
+    ss << "  " << t << " acc[U][VEC];\n";
+    if (!sorted) {
+    ss << "  const dali_vec<int, 4>* lk4 = reinterpret_cast<const dali_vec<int, 4>*>(lk);\n";
     ss << "  const int p_lo = p & ~255;\n  unsigned int m_own = 0;  // this lane's positions after p, in p's own chunk, that repeat the index\n";
     // the index vector goes to LDS; then the ownership test
     ss << "  {\n";
@@ -123,10 +138,11 @@ static std::string gen_scatter_scan_kernel(const Program& P, const IvLayout& L, 
     ss << "      const int j0 = p_lo + lane * 4;\n      const dali_vec<int, 4> k4 = lk4[(p_lo >> 2) + lane];\n      int before = 0;\n"
           "      _Pragma(\"unroll\") for (int b = 0; b < 4; ++b) { before |= (k4.v[b] == key && j0 + b < p) ? 1 : 0; m_own |= (k4.v[b] == key && j0 + b > p) ? (1u << b) : 0u; }\n"
           "      if (__any(before)) return;\n  }\n";
+    }
     ss << "  for (int c0 = 0; c0 < D; c0 += TILE) {\n";
     // loads of row `row` of the value expression's operands
     ss << "    auto fetch = [&](const long row) {\n";
-    for (size_t i = 2; i < P.arrays.size(); ++i) {
+    for (size_t i = first_operand; i < P.arrays.size(); ++i) {
         const ArrayArg& a = P.arrays[i];
         const std::string ty = ctype(a.buf->dtype);
         if (a.cls == Cls::ROW)
@@ -135,8 +151,8 @@ static std::string gen_scatter_scan_kernel(const Program& P, const IvLayout& L, 
             ss << "      const " << ty << "* w" << i << " = (const " << ty << "*)A.p[" << i << "] + row * " << (a.strided ? "(long)A.iv[" + std::to_string(L.stride_pos[i]) + "]" : std::string("(long)D")) << ";\n";
     }
     ss << "      _Pragma(\"unroll\") for (int u = 0; u < U; ++u) {\n        const int ch = c0 / VEC + lane + 64 * u;\n        if (ch * VEC < D) {\n";
-    for (size_t i = 2; i < P.arrays.size(); ++i)
-        if (P.arrays[i].cls == Cls::FULL) emit_leaf_load(ss, P.arrays[i], (int)i, VEC, "x" + std::to_string(i) + "[u]", "          ", false, false, "w");
+    for (size_t i = first_operand; i < P.arrays.size(); ++i)
+        if (P.arrays[i].cls == Cls::FULL) emit_leaf_load(ss, P.arrays[i], (int)i, VEC, "x" + std::to_string(i) + "[u]", "          ", sorted, false, "w");
     ss << "        }\n      }\n    };\n";
     ss << "    auto combine = [&]() {\n      _Pragma(\"unroll\") for (int u = 0; u < U; ++u) {\n        const int ch = c0 / VEC + lane + 64 * u;\n        if (ch * VEC < D) {\n";
     {
@@ -152,8 +168,11 @@ static std::string gen_scatter_scan_kernel(const Program& P, const IvLayout& L, 
         ss << "          const dali_vec<" << t << ", VEC> d4 = dali_load<" << t << ", VEC>(drow + (long)ch * VEC);\n          _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) acc[u][j] = d4.v[j];\n";
     else
         ss << "          acc[u][0] = drow[(long)ch * dcs];\n";
-    ss << "        }\n      }\n      fetch(p);\n    }\n";
+    ss << "        }\n      }\n      fetch(" << (sorted ? "pm[p]" : "p") << ");\n    }\n";
     ss << "    combine();\n";
+    if (sorted) {
+        ss << "    for (int q = p + 1; q < q_end; ++q) { fetch(pm[q]); combine(); }\n";
+    } else {
     ss << "    {\n      unsigned long long any = __ballot(m_own != 0);\n      while (any) {\n        const int l = __builtin_ctzll(any);\n        any &= any - 1;\n"
           "        const unsigned int ml = (unsigned int)__builtin_amdgcn_readlane((int)m_own, l);\n"
           "        for (int b = 0; b < 4; ++b) if ((ml >> b) & 1u) { fetch(p_lo + l * 4 + b); combine(); }\n      }\n    }\n";
@@ -165,6 +184,7 @@ static std::string gen_scatter_scan_kernel(const Program& P, const IvLayout& L, 
           "        const int l = __builtin_ctzll(any);\n        any &= any - 1;\n"
           "        if ((a0 >> l) & 1ull) { fetch(base + l * 4); combine(); }\n        if ((a1 >> l) & 1ull) { fetch(base + l * 4 + 1); combine(); }\n"
           "        if ((a2 >> l) & 1ull) { fetch(base + l * 4 + 2); combine(); }\n        if ((a3 >> l) & 1ull) { fetch(base + l * 4 + 3); combine(); }\n      }\n    }\n";
+    }
     ss << "    _Pragma(\"unroll\") for (int u = 0; u < U; ++u) {\n      const int ch = c0 / VEC + lane + 64 * u;\n      if (ch * VEC < D) {\n";
     if (VEC > 1)
         ss << "        dali_vec<" << t << ", VEC> d4;\n        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) d4.v[j] = acc[u][j];\n        dali_store<" << t << ", VEC>(drow + (long)ch * VEC, d4);\n";
@@ -176,10 +196,35 @@ static std::string gen_scatter_scan_kernel(const Program& P, const IvLayout& L, 
 
 // dest2d: [V, D] view of the destination buffer; idx_c: contiguous int32 [N] buffer; values: an expression of [N, D] elements
 // (or of one element) that a fused kernel can evaluate in place. False when this form does not apply.
+// Index vectors beyond 16384 entries are ordered first (a stable sort by the library, on the library stream) and the same
+// kernel then walks runs of equal indices instead of scanning LDS; the values stay an expression in both forms.
+static void order_indices(const Array& idx_c, int N, int V, const Array& skeys, const Array& perm) {
+    if (g_dry_run) return;
+    check_hip(dali_hip_argsort_i32((const int32_t*)idx_c.device_ptr(), N, V, (int32_t*)skeys.device_ptr(memory::AM_OVERWRITE),
+                                   (int32_t*)perm.device_ptr(memory::AM_OVERWRITE)),
+              "index sort for scatter");
+    if (g_recording) {
+        note_recorded_write(skeys.expression()->memory);
+        note_recorded_write(perm.expression()->memory);
+        Array k1 = idx_c, k2 = skeys, k3 = perm;
+        const int32_t* kp = (const int32_t*)idx_c.device_ptr();
+        int32_t* sp = (int32_t*)skeys.device_ptr(memory::AM_MUTABLE);
+        int32_t* pp = (int32_t*)perm.device_ptr(memory::AM_MUTABLE);
+        g_recording->push_back([=]() {
+            (void)k1;
+            (void)k2;
+            (void)k3;
+            check_hip(dali_hip_argsort_i32(kp, N, V, sp, pp), "index sort replay");
+        });
+    }
+}
+
 static bool try_scatter_scan(const Array& dest2d, const Array& idx_c, OPERATOR_T op, const Array& values) {
-    static const int scan_max = env_int("DALI_HIP_SCATTER_SCAN_MAX", 16384);
+    static const int scan_max = std::min(16384, env_int("DALI_HIP_SCATTER_SCAN_MAX", 16384));
+    static const bool sorted_fused = env_int("DALI_HIP_SCATTER_SORTED_FUSED", 1) != 0;
     const int N = numel_of(idx_c.shape()), D = dest2d.shape()[1], V = dest2d.shape()[0];
-    if (N > scan_max || N > 16384 || has_kind(values, [](Kind k) { return is_reduce(k) || is_all_reduce(k) || k == Kind::GATHER || k == Kind::GATHER_FROM_ROWS; }))
+    const bool sorted = N > scan_max;
+    if ((sorted && !sorted_fused) || has_kind(values, [](Kind k) { return is_reduce(k) || is_all_reduce(k) || k == Kind::GATHER || k == Kind::GATHER_FROM_ROWS; }))
         return false;
     Domain dom;
     dom.R = N;
@@ -187,27 +232,36 @@ static bool try_scatter_scan(const Array& dest2d, const Array& idx_c, OPERATOR_T
     Program P;
     auto dst = strides_of(dest2d.expression().get());
     P.arrays.push_back(manual_arg(dest2d, Cls::FULL, true, 2, dest2d.shape(), {dst[0], dst[1]}));
-    P.arrays.push_back(manual_arg(idx_c, Cls::ROW, false, 1, {N}, {}));
+    Array skeys, perm;
+    if (sorted) {
+        skeys = Array({N}, DTYPE_INT32);
+        perm = Array({N}, DTYPE_INT32);
+        P.arrays.push_back(manual_arg(skeys, Cls::ROW, false, 1, {N}, {}));
+        P.arrays.push_back(manual_arg(perm, Cls::ROW, false, 1, {N}, {}));
+    } else {
+        P.arrays.push_back(manual_arg(idx_c, Cls::ROW, false, 1, {N}, {}));
+    }
+    const size_t first_operand = P.arrays.size();
     const bool one_value = numel_of(values.shape()) == 1;
     int root = add_node(P, values);
     if (!classify(P, root, one_value ? Cls::SCAL : Cls::FULL, dom)) return false;
     count_uses(P, {root});
     bool vec = D % 4 == 0 && dst[1] == 1 && dst[0] % 4 == 0 && dest2d.offset() % 4 == 0 && size_of_dtype(dest2d.dtype()) == 4;
-    for (size_t i = 2; i < P.arrays.size(); ++i) {
+    for (size_t i = first_operand; i < P.arrays.size(); ++i) {
         const ArrayArg& a = P.arrays[i];
         if (a.buf->memory.get() == dest2d.expression()->memory.get()) return false;  // values read from the destination: evaluate them first
         if (a.cls == Cls::FULL) vec = vec && a.col_stride == 1 && a.row_stride % 4 == 0 && a.buf->offset % 4 == 0 && size_of_dtype(a.buf->dtype) == 4;
     }
     const int VEC = vec ? 4 : 1;
     int KCAP = 1024;
-    while (KCAP < N) KCAP *= 2;
+    while (!sorted && KCAP < N) KCAP *= 2;
     std::vector<Output> outs(1);
     outs[0].root = root;
     outs[0].array = 0;
     outs[0].op = op;
     outs[0].cls = Cls::FULL;
     std::ostringstream params;
-    params << "scan6," << VEC << "," << KCAP;
+    params << (sorted ? "runs1," : "scan6,") << VEC << "," << KCAP;
     static std::unordered_map<uint64_t, std::shared_ptr<KernelSpec>> specs_cache;
     uint64_t h = kernel_hash("scatter", signature(P, outs), params.str());
     std::shared_ptr<KernelSpec>& K = specs_cache[h];
@@ -225,8 +279,9 @@ static bool try_scatter_scan(const Array& dest2d, const Array& idx_c, OPERATOR_T
         K->plan.work_count = 1;
         K->plan.work_per_block = 16;
     }
+    if (sorted) order_indices(idx_c, N, V, skeys, perm);
     std::vector<std::vector<int>> shapes = {{N, D, V}};
-    load_and_launch(*K, [&]() { return gen_scatter_scan_kernel(P, L, op, root, VEC, KCAP, K->name); }, P, shapes);
+    load_and_launch(*K, [&]() { return gen_scatter_scan_kernel(P, L, op, root, VEC, KCAP, K->name, sorted); }, P, shapes);
     return true;
 }
 
@@ -259,27 +314,10 @@ static void run_scatter_rows(const Array& dest2d, const Array& idx, OPERATOR_T o
     if (N == 0 || D == 0) return;
     const bool scalar_value = numel_of(values.shape()) == 1;
     Array idx_c = idx.contiguous_memory() ? idx : idx.ascontiguousarray();
-    if (try_scatter_scan(dest2d, idx_c, op, op::identity(values))) return;
+    // (rows narrower than a wave's 1 KiB gain nothing from the unrolled form: [1000000,128] with 262144 indices 155 against 170 us)
+    if ((N <= 16384 || D >= 256) && try_scatter_scan(dest2d, idx_c, op, op::identity(values))) return;
     Array skeys({N}, DTYPE_INT32), perm({N}, DTYPE_INT32);
-    if (!g_dry_run) {
-        check_hip(dali_hip_argsort_i32((const int32_t*)idx_c.device_ptr(), N, V, (int32_t*)skeys.device_ptr(memory::AM_OVERWRITE),
-                                       (int32_t*)perm.device_ptr(memory::AM_OVERWRITE)),
-                  "index sort for scatter");
-        if (g_recording) {
-            note_recorded_write(skeys.expression()->memory);
-            note_recorded_write(perm.expression()->memory);
-            Array k1 = idx_c, k2 = skeys, k3 = perm;
-            const int32_t* kp = (const int32_t*)idx_c.device_ptr();
-            int32_t* sp = (int32_t*)skeys.device_ptr(memory::AM_MUTABLE);
-            int32_t* pp = (int32_t*)perm.device_ptr(memory::AM_MUTABLE);
-            g_recording->push_back([=]() {
-                (void)k1;
-                (void)k2;
-                (void)k3;
-                check_hip(dali_hip_argsort_i32(kp, N, V, sp, pp), "index sort replay");
-            });
-        }
-    }
+    order_indices(idx_c, N, V, skeys, perm);
     auto dst = strides_of(dest2d.expression().get());
     Program P;
     P.arrays.push_back(manual_arg(dest2d, Cls::FULL, true, 2, dest2d.shape(), {dst[0], dst[1]}));

@@ -1531,7 +1531,9 @@ def test_scatter_reference_cases(gpu, D):
     assert np.array_equal(dest2.numpy(), want)
 
 
-@pytest.mark.parametrize("V,Dm,N", [(5, 1, 200), (64, 33, 300), (1000, 256, 5000), (32000, 1024, 8192)])
+@pytest.mark.parametrize("V,Dm,N", [(5, 1, 200), (64, 33, 300), (1000, 256, 5000), (32000, 1024, 8192),
+                                    # beyond 16384 indices: ordered first, the values still evaluated inside the kernel
+                                    (32000, 256, 65536), (3000, 36, 20000), (700, 7, 40001)])
 @pytest.mark.parametrize("operator_t", [1, 2, 0])
 def test_scatter_rows_is_the_sequential_loop_bit_for_bit(gpu, D, O, rng, V, Dm, N, operator_t):
     dest = rng.randn(V, Dm).astype(np.float32)
@@ -1543,6 +1545,16 @@ def test_scatter_rows_is_the_sequential_loop_bit_for_bit(gpu, D, O, rng, V, Dm, 
     d[arr(D, idx)].assign(arr(D, vals), operator_t)
     # duplicates are combined in input order, as in the reference's CPU loop: exact equality
     assert np.array_equal(d.numpy(), O.scatter_rows(dest, idx, vals, op=operator_t))
+    assert D.last_kernel_kinds().endswith("scatter")
+    # the values as an expression: evaluated where they are used, no [N, D] array in between (one generated kernel)
+    if operator_t == 1:
+        scale = rng.randn(N, 1).astype(np.float32)
+        d3 = arr(D, dest)
+        k0 = D.jit_stats()["kernels"]
+        d3[arr(D, idx)].assign(arr(D, vals) * arr(D, scale) + 1.0, 1)
+        if Dm > 1:
+            assert D.jit_stats()["kernels"] - k0 == 1 and D.last_kernel_kinds() == "scatter"
+        assert np.array_equal(d3.numpy(), O.scatter_rows(dest, idx, vals * scale + np.float32(1.0), op=1))
     # scalar right-hand side
     d2 = arr(D, dest)
     g = d2[arr(D, idx)]
