@@ -544,6 +544,17 @@ def main():
         nxt["scatter_add_32000x1024_8192"] = {"us": round(us, 2), "GB/s": round(sbytes / us / 1e3, 1),
                                               "frac_hbm": round(sbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                                               "launches_incl_index_sort": rec.launches, "distinct_rows": uniq}
+        # the same with 65536 indices: ordered first (stable radix sort), then one launch that walks runs of equal indices
+        ids = D.Array.from_numpy(np.random.RandomState(15).randint(0, V, 65536).astype(np.int32))
+        upd = D.Array.from_numpy(np.random.RandomState(16).randn(65536, Dm).astype(np.float32))
+        with D.Recording() as rec:
+            g = table[ids]
+            g += upd
+        us = time_recording(rec, 20)
+        uniq = int(np.unique(ids.numpy()).size)
+        sbytes = 65536 * Dm * 4 + 2 * uniq * Dm * 4
+        nxt["scatter_add_32000x1024_65536"] = {"us": round(us, 2), "GB/s": round(sbytes / us / 1e3, 1), "frac_hbm": round(sbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                                               "launches_incl_index_sort": rec.launches, "distinct_rows": uniq}
         del table, ids, upd, g, rec
         # softmax away from the C1 shape: rows of a vocabulary that is no multiple of anything (one row = 201,028 bytes, every
         # row starts elsewhere within a cache line) and the middle axis of a 3-D array; bytes = one read + one write
