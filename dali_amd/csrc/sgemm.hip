@@ -899,6 +899,26 @@ static int stream_product(const GemmArgs& g, bool ta, bool tb, int shares) {
     return launch_tile<64, 64, 64, 2, 2, false>(rest, ta, tb, true, 1, true);
 }
 
+// Many 128x128 tiles of a single product with B stored [K][N]: the whole 32-deep slabs through the kernel that walks a list of
+// tiles per compute unit, what is left of the inner extent by a checked launch that adds to the result. -1: not a case for it.
+static int tiles128_product(const GemmArgs& g, bool ta) {
+    const GemmSeg& sg = g.seg[0];
+    const int kw = sg.K / 32 * 32, kr = sg.K - kw;
+    if (kw == 0) return -1;
+    const int cus = device_cus();
+    if (cus <= 0) return -1;
+    const int r = sgemm_dma128(ta, g.M, g.N, kw, sg.A, sg.lda, sg.B, sg.ldb, g.alpha, g.beta, g.C, g.ldc, cus);
+    if (r < 0) return DALI_HIP_ERROR;
+    if (r == 0) return -1;
+    if (kr == 0) return DALI_HIP_OK;
+    GemmArgs rest = g;
+    rest.seg[0].A = sg.A + (ta ? (size_t)kw * sg.lda : (size_t)kw);
+    rest.seg[0].B = sg.B + (size_t)kw * sg.ldb;
+    rest.seg[0].K = kr;
+    rest.beta = 1.0f;
+    return launch_tile<128, 128, 32, 2>(rest, ta, false, true, 1, true);
+}
+
 // Row-major driver: C[M,N] = alpha * sum_s opA_s * opB_s + beta * C.
 // ta: A_s is stored as [K][M]; tb: B_s is stored as [N][K].
 static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K, const float* const* A,
@@ -989,7 +1009,13 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         const int st = stream_product(g, ta, tb, stream_env);
         if (st >= 0) return st;
     }
-    if (tiles128 >= 192) return run_tile<128, 128, 32, 2>(g, ta, tb, vec, 1);
+    if (tiles128 >= 192) {
+        if (vec && g.nseg == 1 && !tb && !g.map_on && !rows_may_overlap) {
+            const int st = tiles128_product(g, ta);
+            if (st >= 0) return st;
+        }
+        return run_tile<128, 128, 32, 2>(g, ta, tb, vec, 1);
+    }
     // Small grids: 64x64 tiles, and when even those leave CUs with a single workgroup, split K so
     // that two workgroups share a CU and one's barriers and memory waits hide behind the other's MFMAs.
     long tiles64 = (long)((M + 63) / 64) * ((N + 63) / 64);

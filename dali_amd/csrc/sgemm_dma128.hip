@@ -1,0 +1,391 @@
+// fp32 GEMM for grids of many tiles: 128x128 tiles of C, one workgroup per compute unit walking a list of them, operand slabs
+// written into LDS by the loads themselves (global_load_lds_dwordx4), four slabs of 32 in flight.
+//
+// Row-major view: C[M,N] = alpha * A[M,K] * B[K,N] + beta * C with B stored [K][N] and A stored [M][K] or [K][M]
+// (dali_hip_sgemm; the reference's call is dali/array/gemm/cublas_gemm.cu:153-166, and with A stored [K][M] the weight
+// gradient matmul(a.w.transpose(), out_dw) of dali/tensor/op/dot.cpp:17-18).
+//
+// Against the 64x64 kernel of the same kind (sgemm_dma.hip) a tile of 128x128 asks the caches for half as many operand bytes
+// per flop, which is what limits that kernel once every compute unit runs it (32 KiB per microsecond each). Eight waves
+// form 2 x 4 wave tiles of 64 rows x 32 columns; a wave keeps its sums for the whole inner extent, so nothing is exchanged
+// at the end of a tile, and the loads of the next tile's first slabs are under way while the sums of this one are stored.
+//
+// Operands whose k runs across memory rows ([K][N], [K][M]) are read "outer product" fashion: a lane takes a 16-byte piece
+// (8 bytes for B) of row k = 4 kk + lane / 16 and feeds its elements to different matrix instructions, so that the 16x16 tile
+// of instruction u holds the rows (columns) congruent to u modulo 4 (modulo 2). One 16-byte and one 8-byte LDS read feed
+// eight v_mfma_f32_16x16x4_f32; the operand stored [M][K] is read as 16-byte pieces along k, as in the 64x64 kernel, and
+// then sixteen reads feed sixty-four instructions.
+//
+// LDS, per stage of 32 KiB: A (16 KiB) then B. [K][x] operands are kept as rows of 128 x values, 512 bytes, with the
+// sixteen-byte piece p of row k in slot p ^ 8 when bit `swizzle_bit` of k is set: the two rows that one pass of an 8-byte
+// read touches then lie in different halves of the banks. A stored [M][K] is kept as rows of 32 k values, 128 bytes, piece
+// g of row r in slot g ^ ((r >> 1) & 7): the sixteen rows of one pass hit sixteen different slots of a 256-byte bank row.
+// A lane of a load always writes bytes [16 lane, 16 lane + 16) of its 1 KiB chunk, so the permutations are applied to the
+// global address the lane fetches.
+#include <cstdlib>
+#include <type_traits>
+
+#include "runtime.h"
+
+namespace dali_hip {
+namespace {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+constexpr int kStageBytes = 32768;
+constexpr int kBOffset = 16384;
+constexpr int kLdsBytes = 4 * kStageBytes;
+
+struct Args128 {
+    const float* A;
+    const float* B;
+    int slabs;  // 32-deep slabs of the inner extent
+    int lda, ldb;
+    int M, N;
+    float* C;
+    int ldc;
+    float alpha, beta;
+    int tiles_m, tiles_n;
+};
+
+// One 16-byte piece per lane from global memory straight into LDS: lane l writes bytes [16 l, 16 l + 16) behind `lds_addr`
+// (wave-uniform, goes through M0); the source is base + voff. The base is made a scalar by hand: the compiler cannot prove
+// that a pointer which changes with the work item is the same in every lane.
+__device__ __forceinline__ void load_to_lds(unsigned lds_addr, unsigned voff, const char* base) {
+    const unsigned long long b = (unsigned long long)base;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b), hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+    const char* sbase = (const char*)(((unsigned long long)hi << 32) | lo);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+// The compiler does not see these loads, so the waits for them are written out; they are also compiler barriers.
+__device__ __forceinline__ void wait_but_4() { asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); }
+__device__ __forceinline__ void wait_but_8() { asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); }
+__device__ __forceinline__ void wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// TA: A stored as [K][M]
+template <bool TA>
+__global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
+    // (no static LDS beside this: the loads address LDS from offset 0)
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = w >> 2, wn = w & 3, l16 = lane & 15, kq = lane >> 4;
+    const int M = g.M, N = g.N, n = g.slabs;
+    const int tiles = g.tiles_m * g.tiles_n;
+    // this workgroup's tiles: first, first + stride, ... The workgroups of one die (every eighth) take a contiguous band.
+    int first, stride, count;
+    {
+        const int G = gridDim.x, b = blockIdx.x;
+        if ((G & 7) == 0) {
+            const int chunk = (tiles + 7) / 8, wgx = G / 8;
+            const int lo = (b & 7) * chunk, hi = lo + chunk < tiles ? lo + chunk : tiles;
+            first = lo + b / 8;
+            stride = wgx;
+            count = first < hi ? (hi - first + wgx - 1) / wgx : 0;
+        } else {
+            first = b;
+            stride = G;
+            count = first < tiles ? (tiles - first + G - 1) / G : 0;
+        }
+    }
+    if (count == 0) return;
+    const int total = count * n;  // slabs of all tiles of this workgroup
+    // Tiles are numbered in column blocks four tiles wide, by rows inside a block: the 32 tiles that the workgroups of a die
+    // work on together are 8 x 4 and share their operand slabs in that die's cache.
+    auto tile_at = [&](int tile, int& mt, int& nt) __attribute__((always_inline)) {
+        const int per_block = g.tiles_m * 4, nb = tile / per_block, rem = tile - nb * per_block;
+        const int width = g.tiles_n - 4 * nb < 4 ? g.tiles_n - 4 * nb : 4;
+        mt = rem / width;
+        nt = 4 * nb + (rem - mt * width);
+    };
+
+    const long a_step = (TA ? (long)32 * g.lda : 32L) * (long)sizeof(float);
+    const long b_step = (long)32 * g.ldb * (long)sizeof(float);
+    unsigned a_off[2], b_off[2], a_dst[2], b_dst[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        a_dst[q] = (unsigned)((w + 8 * q) * 1024);
+        b_dst[q] = (unsigned)(kBOffset + (w + 8 * q) * 1024);
+    }
+    // ---- the side that requests slabs
+    int i_r = 0, i_fj = 0;
+    const char* ap = nullptr;
+    const char* bp = nullptr;
+    auto request_tile = [&](int r) __attribute__((always_inline)) {
+        int mt, nt;
+        tile_at(first + r * stride, mt, nt);
+        const int m0 = 128 * mt, n0 = 128 * nt;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int c = w + 8 * q;  // 1 KiB chunk of the slab
+            if (!TA) {
+                const int r_in = 8 * c + (lane >> 3), s = lane & 7;
+                const int row = m0 + r_in < M ? m0 + r_in : M - 1;
+                a_off[q] = (unsigned)(((size_t)row * g.lda + 4 * (s ^ ((r_in >> 1) & 7))) * sizeof(float));
+            } else {
+                const int k = 2 * c + (lane >> 5), s = lane & 31;
+                int col = m0 + 4 * s;
+                col = col < M ? col : M - 4;
+                a_off[q] = (unsigned)(((size_t)k * g.lda + col) * sizeof(float));
+            }
+            {
+                const int k = 2 * c + (lane >> 5), s = lane & 31;
+                const int bit = TA ? (k & 1) : ((k >> 2) & 1);
+                int col = n0 + 4 * (s ^ (bit << 3));
+                col = col < N ? col : N - 4;
+                b_off[q] = (unsigned)(((size_t)k * g.ldb + col) * sizeof(float));
+            }
+        }
+        i_fj = 0;
+        ap = (const char*)g.A;
+        bp = (const char*)g.B;
+    };
+    auto issue = [&](int stage) __attribute__((always_inline)) {
+        load_to_lds(a_dst[0] + stage * kStageBytes, a_off[0], ap);
+        load_to_lds(a_dst[1] + stage * kStageBytes, a_off[1], ap);
+        load_to_lds(b_dst[0] + stage * kStageBytes, b_off[0], bp);
+        load_to_lds(b_dst[1] + stage * kStageBytes, b_off[1], bp);
+        ++i_fj;
+        ap += a_step;
+        bp += b_step;
+        if (i_fj == n) {
+            ++i_r;
+            if (i_r < count) request_tile(i_r);
+        }
+    };
+    request_tile(0);
+    issue(0);
+    if (total > 1) issue(1);
+    if (total > 2) issue(2);
+
+    // ---- operand addresses of this lane within a stage
+    // [K][x] operands: row 4 kk + kq of the slab; A [M][K]: row block rb of the wave tile, piece 4 t + kq
+    unsigned a_addr[4], b_addr;
+    if (TA) {
+        a_addr[0] = (unsigned)(kq * 512 + (wm * 64 + 4 * l16) * 4);
+        a_addr[1] = a_addr[2] = a_addr[3] = 0;
+    } else {
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) {
+            const int r_in = wm * 64 + 16 * rb + l16;
+            a_addr[rb] = (unsigned)(r_in * 128 + ((kq ^ ((r_in >> 1) & 7)) * 16));  // piece kq of k-group 0; k-group 1 flips bit 2 of the slot
+        }
+    }
+    // (the swizzle bit of B's row is bit 0 of kq in both forms: k = 4 kk + kq, or (k >> 2) = 4 t + kq)
+    b_addr = (unsigned)(kBOffset + ((wn * 8 + (l16 >> 1)) ^ ((kq & 1) << 3)) * 16 + (l16 & 1) * 8);
+
+    floatx4 acc[4][2];
+    auto clear = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+    };
+    clear();
+    // Operand registers, two sets. TA: set o holds one k-quad (a: 4 rows congruent classes, b: 2 column classes).
+    // !TA: set o holds one k-group of 16 (a[rb]: four k of row block rb, b[c]: row 16 t + 4 kq + c).
+    floatx4 a_tn[2];
+    floatx2 b_tn[2];
+    floatx4 a_nn[2][4];
+    floatx2 b_nn[2][4];
+    auto load_ops = [&](auto ST, int step, int o) __attribute__((always_inline)) {
+        constexpr int st = decltype(ST)::value;
+        const char* base = lds + st * kStageBytes;
+        if (TA) {
+            // step = kk (0..7)
+            a_tn[o] = *(const floatx4*)(base + a_addr[0] + step * 2048);
+            b_tn[o] = *(const floatx2*)(base + b_addr + kq * 512 + step * 2048);
+        } else {
+            // step = t (0..1)
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) a_nn[o][rb] = *(const floatx4*)(base + (a_addr[rb] ^ (unsigned)(step * 64)));
+#pragma unroll
+            for (int c = 0; c < 4; ++c) b_nn[o][c] = *(const floatx2*)(base + b_addr + (16 * step + 4 * kq + c) * 512);
+        }
+    };
+    // eight matrix instructions on independent sums
+    auto mfma_tn = [&](int o) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ua = 0; ua < 4; ++ua)
+#pragma unroll
+            for (int ub = 0; ub < 2; ++ub) acc[ua][ub] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_tn[o][ua], b_tn[o][ub], acc[ua][ub], 0, 0, 0);
+    };
+    auto mfma_nn = [&](int o, int c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+            for (int ub = 0; ub < 2; ++ub) acc[rb][ub] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_nn[o][rb][c], b_nn[o][c][ub], acc[rb][ub], 0, 0, 0);
+    };
+
+    // ---- the side that multiplies
+    int c_r = 0, c_fj = 0;
+    auto finish_tile = [&]() __attribute__((always_inline)) {
+        int mt, nt;
+        tile_at(first + c_r * stride, mt, nt);
+        const int m_base = 128 * mt + wm * 64, nn = 128 * nt + wn * 32 + 2 * l16;
+        const float alpha = g.alpha, beta = g.beta;
+        if (nn < N) {  // (N is a multiple of 4 and nn even: nn + 1 < N as well)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    // TA: the tile of instruction i holds the rows congruent to i modulo 4; else row block i
+                    const int m = m_base + (TA ? 16 * kq + 4 * v + i : 16 * i + 4 * kq + v);
+                    if (m < M) {
+                        floatx2* c = (floatx2*)(g.C + (size_t)m * g.ldc + nn);
+                        floatx2 r;
+                        r[0] = alpha * acc[i][0][v];
+                        r[1] = alpha * acc[i][1][v];
+                        if (beta != 0.f) {
+                            const floatx2 old = *c;
+                            r[0] += beta * old[0];
+                            r[1] += beta * old[1];
+                        }
+                        *c = r;
+                    }
+                }
+        }
+        clear();
+        ++c_r;
+        c_fj = 0;
+    };
+    // Slab i lives in stage i % 4. The barrier inside slab i is for slab i+1 (its loads were issued two slabs earlier); behind
+    // it the buffer of slab i-1 is free and takes slab i+3.
+    auto slab_step = [&](auto ST, auto H1, auto H2, auto H3) __attribute__((always_inline)) {
+        constexpr int st = decltype(ST)::value;
+        constexpr bool has1 = decltype(H1)::value, has2 = decltype(H2)::value, has3 = decltype(H3)::value;
+        using NX = std::integral_constant<int, (st + 1) % 4>;
+        if (TA) {
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                if (kk < 7) load_ops(ST, kk + 1, (kk + 1) & 1);
+                else if (has1) load_ops(NX{}, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_tn(kk & 1);
+                if (kk == 1 && has1) {
+                    if (has2) wait_but_4(); else wait_all();
+                    __builtin_amdgcn_s_barrier();
+                }
+                if (kk == 2 && has3) issue((st + 3) % 4);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            load_ops(ST, 1, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_nn(0, 0);
+            if (has1) {
+                if (has2) wait_but_4(); else wait_all();
+                __builtin_amdgcn_s_barrier();
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_nn(0, 1);
+            if (has3) issue((st + 3) % 4);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_nn(0, 2);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_nn(0, 3);
+            __builtin_amdgcn_sched_barrier(0);
+            if (has1) load_ops(NX{}, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_nn(1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_nn(1, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_nn(1, 2);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_nn(1, 3);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (++c_fj == n) finish_tile();
+    };
+    auto tail_step = [&](auto J, auto R) __attribute__((always_inline)) {
+        constexpr int j = decltype(J)::value, r = decltype(R)::value;
+        if constexpr (j < r)
+            slab_step(std::integral_constant<int, j % 4>{}, std::integral_constant<bool, (j + 1 < r)>{}, std::integral_constant<bool, (j + 2 < r)>{},
+                      std::integral_constant<bool, (j + 3 < r)>{});
+    };
+    auto run_tail = [&](auto R) __attribute__((always_inline)) {
+        tail_step(std::integral_constant<int, 0>{}, R);
+        tail_step(std::integral_constant<int, 1>{}, R);
+        tail_step(std::integral_constant<int, 2>{}, R);
+        tail_step(std::integral_constant<int, 3>{}, R);
+        tail_step(std::integral_constant<int, 4>{}, R);
+        tail_step(std::integral_constant<int, 5>{}, R);
+    };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+    using S3 = std::integral_constant<int, 3>;
+    using Yes = std::true_type;
+    // slab 0 has landed once at most the loads of slabs 1 and 2 are outstanding
+    if (total > 2) wait_but_8();
+    else if (total > 1) wait_but_4();
+    else wait_all();
+    __builtin_amdgcn_s_barrier();
+    load_ops(S0{}, 0, 0);
+    int i = 0;
+    for (; i + 7 <= total; i += 4) {
+        slab_step(S0{}, Yes{}, Yes{}, Yes{});
+        slab_step(S1{}, Yes{}, Yes{}, Yes{});
+        slab_step(S2{}, Yes{}, Yes{}, Yes{});
+        slab_step(S3{}, Yes{}, Yes{}, Yes{});
+    }
+    const int rest = total - i;  // 1 .. 6
+    if (rest == 1) run_tail(std::integral_constant<int, 1>{});
+    else if (rest == 2) run_tail(std::integral_constant<int, 2>{});
+    else if (rest == 3) run_tail(std::integral_constant<int, 3>{});
+    else if (rest == 4) run_tail(std::integral_constant<int, 4>{});
+    else if (rest == 5) run_tail(std::integral_constant<int, 5>{});
+    else run_tail(std::integral_constant<int, 6>{});
+}
+
+bool aligned_to(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+template <bool TA>
+int launch128(const Args128& g, int workgroups) {
+    auto kernel = sgemm_dma128_kernel<TA>;
+    hipError_t e = reserve_dynamic_lds((const void*)kernel, kLdsBytes);
+    if (e != hipSuccess) return fail("sgemm: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
+    hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(512), kLdsBytes, stream(), g);
+    e = hipGetLastError();
+    if (e != hipSuccess) return fail("sgemm launch failed: %s", hipGetErrorString(e));
+    return 1;
+}
+
+}  // namespace
+
+int sgemm_dma128(bool ta, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float alpha, float beta, float* C, int ldc, int cus) {
+    static const int enabled = getenv("DALI_HIP_GEMM_DMA128") ? atoi(getenv("DALI_HIP_GEMM_DMA128")) : 1;
+    if (!enabled || cus < 8 || M < 1 || N < 4 || K < 32 || K % 32 != 0) return 0;
+    // 16-byte pieces that start on 16-byte boundaries and never straddle the end of a row; pairs of results stored as 8 bytes
+    if (lda % 4 != 0 || ldb % 4 != 0 || N % 4 != 0 || (ta && (M % 4 != 0 || M < 4)) || ldc % 2 != 0) return 0;
+    if (!aligned_to(A, 16) || !aligned_to(B, 16) || !aligned_to(C, 8)) return 0;
+    // per-lane offsets are 32-bit and relative to a pointer that walks along k
+    const size_t a_span = ((size_t)(ta ? 32 : M) * lda + (ta ? M : 32)) * sizeof(float);
+    const size_t b_span = ((size_t)32 * ldb + N) * sizeof(float);
+    if (a_span >= ((size_t)1 << 32) || b_span >= ((size_t)1 << 32)) return 0;
+    Args128 g = {};
+    g.A = A;
+    g.B = B;
+    g.slabs = K / 32;
+    g.lda = lda;
+    g.ldb = ldb;
+    g.M = M;
+    g.N = N;
+    g.C = C;
+    g.ldc = ldc;
+    g.alpha = alpha;
+    g.beta = beta;
+    g.tiles_m = (M + 127) / 128;
+    g.tiles_n = (N + 127) / 128;
+    const long tiles = (long)g.tiles_m * g.tiles_n;
+    if (tiles > (1L << 24)) return 0;
+    int workgroups = cus - cus % 8;  // every workgroup has a compute unit to itself (its LDS); whole dies keep the bands of tiles
+    if (tiles < workgroups) workgroups = (int)tiles;
+    return ta ? launch128<true>(g, workgroups) : launch128<false>(g, workgroups);
+}
+
+}  // namespace dali_hip
