@@ -479,6 +479,28 @@ def main():
         configs["c5_lstm_step_256x1024x1024"]["single_step_small_batches"] = single
         del X, Hp, Cp, W, U, bias, rec, grec, Xs, srec
 
+        # the products of the backward pass of dot(h [256,1024], W [1024,32000]) (dali/tensor/op/dot.cpp:17-18): the weight gradient
+        # h^T . g reads its left operand against its rows (inner extent 256), the input gradient g . W^T its right one (32000)
+        bh, bg, bw = (D.Array.from_numpy((np.random.RandomState(s).randn(*shp) * 0.1).astype(np.float32))
+                      for s, shp in ((60, (256, 1024)), (61, (256, 32000)), (62, (1024, 32000))))
+        bwd = {}
+        for tag, make in (("weights_256x1024T_x_256x32000", lambda: op.dot(bh.transpose(), bg)), ("inputs_256x32000_x_1024x32000T", lambda: op.dot(bg, bw.transpose()))):
+            flops = 2.0 * 256 * 1024 * 32000
+            with D.Recording() as brec:
+                make().eval()
+            bus = time_recording(brec, 20)
+            bwd[tag] = {"us": round(bus, 2), "TFLOP/s": round(flops / bus / 1e6, 2), "frac_fp32_mfma": round(flops / bus / 1e6 / 157.3, 4), "launches": brec.launches}
+            del brec
+        configs["c5_lstm_step_256x1024x1024"]["dot_backward_products"] = bwd
+        del bh, bg, bw
+        sq = [D.Array.from_numpy(np.random.RandomState(s).randn(4096, 4096).astype(np.float32)) for s in (63, 64)]
+        with D.Recording() as brec:
+            op.dot(sq[0], sq[1]).eval()
+        bus = time_recording(brec, 5)
+        configs["c5_lstm_step_256x1024x1024"]["dot_4096x4096x4096"] = {"us": round(bus, 2), "TFLOP/s": round(2.0 * 4096 ** 3 / bus / 1e6, 2),
+                                                                      "frac_fp32_mfma": round(2.0 * 4096 ** 3 / bus / 1e6 / 157.3, 4)}
+        del sq, brec
+
         # the double-precision product (the reference's cublasDgemm branch)
         dA, dB = (D.Array.from_numpy(np.random.RandomState(s).randn(2048, 2048)) for s in (27, 28))
         with D.Recording() as drec:

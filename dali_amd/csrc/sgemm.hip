@@ -978,6 +978,14 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         g.seg[0].K = 0;
         vec = false;
     }
+    // More than `low_rows_from` and at most 64 rows against a wide B stored [K][N]: bound by the matrix pipe rather than by
+    // streaming B, so 64-row tiles fed through LDS, one workgroup per compute unit ([64,1024].[1024,32000]: 45 -> 41 us, 0.65 of the fp32 matrix peak; the row-streaming
+    // kernel takes 26 us at 32 rows and grows with the rows, this one takes 38 to 41 us whatever they are)
+    static const int low_rows_from = getenv("DALI_HIP_GEMM_LOW_ROWS") ? atoi(getenv("DALI_HIP_GEMM_LOW_ROWS")) : 52;
+    if (g.nseg == 1 && vec && !ta && !tb && !row_map && !rows_may_overlap && M > low_rows_from && M <= 64 && N >= 8192 && g.seg[0].K >= 256) {
+        const int st = tiles128_product(g, false);
+        if (st >= 0) return st;
+    }
     if (g.nseg == 1 && g.seg[0].K > 0 && !ta && !row_map && !rows_may_overlap && M <= 64) {
         // few rows against a wide right operand: stream it once instead of tiling it through LDS
         const int st = sgemm_skinny(tb, M, N, g.seg[0].K, alpha, g.seg[0].A, g.seg[0].lda, g.seg[0].B, g.seg[0].ldb, beta, C, ldc);

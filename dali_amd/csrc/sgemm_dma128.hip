@@ -59,13 +59,19 @@ __device__ __forceinline__ void load_to_lds(unsigned lds_addr, unsigned voff, co
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
 // The compiler does not see these loads, so the waits for them are written out; they are also compiler barriers.
-__device__ __forceinline__ void wait_but_4() { asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); }
-__device__ __forceinline__ void wait_but_8() { asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); }
+template <int N>
+__device__ __forceinline__ void wait_but() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 __device__ __forceinline__ void wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
-// TA: A stored as [K][M]
-template <bool TA>
+// TA: A stored as [K][M]. TM: rows of a tile, 128, or 64 for products of at most 64 rows against a wide B (the output
+// projection of a decoder step at a batch the row-streaming kernel no longer serves well: such a product is bound by the matrix
+// pipe, 4.2 GFLOP at [64,1024].[1024,32000], and 128-row tiles would double that); the wave tiles are then 32 rows high.
+template <bool TA, int TM>
 __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
+    static_assert(TM == 128 || (TM == 64 && !TA), "64-row tiles are built for A stored [M][K]");
+    constexpr int RB = TM / 32;   // 16-row blocks of a wave tile
+    constexpr int AQ = TM / 64;   // loads of A per wave and slab
+    constexpr int LPS = AQ + 2;   // loads per wave and slab
     // (no static LDS beside this: the loads address LDS from offset 0)
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -115,11 +121,13 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     auto request_tile = [&](int r) __attribute__((always_inline)) {
         int mt, nt;
         tile_at(first + r * stride, mt, nt);
-        const int m0 = 128 * mt, n0 = 128 * nt;
+        const int m0 = TM * mt, n0 = 128 * nt;
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
             const int c = w + 8 * q;  // 1 KiB chunk of the slab
-            if (!TA) {
+            if (q >= AQ) {
+                a_off[q] = 0;
+            } else if (!TA) {
                 const int r_in = 8 * c + (lane >> 3), s = lane & 7;
                 const int row = m0 + r_in < M ? m0 + r_in : M - 1;
                 a_off[q] = (unsigned)(((size_t)row * g.lda + 4 * (s ^ ((r_in >> 1) & 7))) * sizeof(float));
@@ -143,7 +151,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     };
     auto issue = [&](int stage) __attribute__((always_inline)) {
         load_to_lds(a_dst[0] + stage * kStageBytes, a_off[0], ap);
-        load_to_lds(a_dst[1] + stage * kStageBytes, a_off[1], ap);
+        if (AQ > 1) load_to_lds(a_dst[1] + stage * kStageBytes, a_off[1], ap);
         load_to_lds(b_dst[0] + stage * kStageBytes, b_off[0], bp);
         load_to_lds(b_dst[1] + stage * kStageBytes, b_off[1], bp);
         ++i_fj;
@@ -168,17 +176,17 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     } else {
 #pragma unroll
         for (int rb = 0; rb < 4; ++rb) {
-            const int r_in = wm * 64 + 16 * rb + l16;
-            a_addr[rb] = (unsigned)(r_in * 128 + ((kq ^ ((r_in >> 1) & 7)) * 16));  // piece kq of k-group 0; k-group 1 flips bit 2 of the slot
+            const int r_in = wm * (TM / 2) + 16 * rb + l16;
+            a_addr[rb] = rb < RB ? (unsigned)(r_in * 128 + ((kq ^ ((r_in >> 1) & 7)) * 16)) : 0u;  // piece kq of k-group 0; k-group 1 flips bit 2 of the slot
         }
     }
     // (the swizzle bit of B's row is bit 0 of kq in both forms: k = 4 kk + kq, or (k >> 2) = 4 t + kq)
     b_addr = (unsigned)(kBOffset + ((wn * 8 + (l16 >> 1)) ^ ((kq & 1) << 3)) * 16 + (l16 & 1) * 8);
 
-    floatx4 acc[4][2];
+    floatx4 acc[RB][2];
     auto clear = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < RB; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -189,7 +197,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     // !TA: set o holds one k-group of 16 (a[rb]: four k of row block rb, b[c]: row 16 t + 4 kq + c).
     floatx4 a_tn[2];
     floatx2 b_tn[2];
-    floatx4 a_nn[2][4];
+    floatx4 a_nn[2][RB];
     floatx2 b_nn[2][4];
     auto load_ops = [&](auto ST, int step, int o) __attribute__((always_inline)) {
         constexpr int st = decltype(ST)::value;
@@ -201,7 +209,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
         } else {
             // step = t (0..1)
 #pragma unroll
-            for (int rb = 0; rb < 4; ++rb) a_nn[o][rb] = *(const floatx4*)(base + (a_addr[rb] ^ (unsigned)(step * 64)));
+            for (int rb = 0; rb < RB; ++rb) a_nn[o][rb] = *(const floatx4*)(base + (a_addr[rb] ^ (unsigned)(step * 64)));
 #pragma unroll
             for (int c = 0; c < 4; ++c) b_nn[o][c] = *(const floatx2*)(base + b_addr + (16 * step + 4 * kq + c) * 512);
         }
@@ -209,13 +217,13 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     // eight matrix instructions on independent sums
     auto mfma_tn = [&](int o) __attribute__((always_inline)) {
 #pragma unroll
-        for (int ua = 0; ua < 4; ++ua)
+        for (int ua = 0; ua < RB; ++ua)
 #pragma unroll
             for (int ub = 0; ub < 2; ++ub) acc[ua][ub] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_tn[o][ua], b_tn[o][ub], acc[ua][ub], 0, 0, 0);
     };
     auto mfma_nn = [&](int o, int c) __attribute__((always_inline)) {
 #pragma unroll
-        for (int rb = 0; rb < 4; ++rb)
+        for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
             for (int ub = 0; ub < 2; ++ub) acc[rb][ub] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_nn[o][rb][c], b_nn[o][c][ub], acc[rb][ub], 0, 0, 0);
     };
@@ -225,11 +233,11 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     auto finish_tile = [&]() __attribute__((always_inline)) {
         int mt, nt;
         tile_at(first + c_r * stride, mt, nt);
-        const int m_base = 128 * mt + wm * 64, nn = 128 * nt + wn * 32 + 2 * l16;
+        const int m_base = TM * mt + wm * (TM / 2), nn = 128 * nt + wn * 32 + 2 * l16;
         const float alpha = g.alpha, beta = g.beta;
         if (nn < N) {  // (N is a multiple of 4 and nn even: nn + 1 < N as well)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < RB; ++i)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     // TA: the tile of instruction i holds the rows congruent to i modulo 4; else row block i
@@ -266,7 +274,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
                 __builtin_amdgcn_sched_barrier(0);
                 mfma_tn(kk & 1);
                 if (kk == 1 && has1) {
-                    if (has2) wait_but_4(); else wait_all();
+                    if (has2) wait_but<LPS>(); else wait_all();
                     __builtin_amdgcn_s_barrier();
                 }
                 if (kk == 2 && has3) issue((st + 3) % 4);
@@ -277,7 +285,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
             __builtin_amdgcn_sched_barrier(0);
             mfma_nn(0, 0);
             if (has1) {
-                if (has2) wait_but_4(); else wait_all();
+                if (has2) wait_but<LPS>(); else wait_all();
                 __builtin_amdgcn_s_barrier();
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -321,8 +329,8 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     using S3 = std::integral_constant<int, 3>;
     using Yes = std::true_type;
     // slab 0 has landed once at most the loads of slabs 1 and 2 are outstanding
-    if (total > 2) wait_but_8();
-    else if (total > 1) wait_but_4();
+    if (total > 2) wait_but<2 * LPS>();
+    else if (total > 1) wait_but<LPS>();
     else wait_all();
     __builtin_amdgcn_s_barrier();
     load_ops(S0{}, 0, 0);
@@ -344,9 +352,9 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
 
 bool aligned_to(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-template <bool TA>
+template <bool TA, int TM>
 int launch128(const Args128& g, int workgroups) {
-    auto kernel = sgemm_dma128_kernel<TA>;
+    auto kernel = sgemm_dma128_kernel<TA, TM>;
     hipError_t e = reserve_dynamic_lds((const void*)kernel, kLdsBytes);
     if (e != hipSuccess) return fail("sgemm: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
     hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(512), kLdsBytes, stream(), g);
@@ -379,13 +387,15 @@ int sgemm_dma128(bool ta, int M, int N, int K, const float* A, int lda, const fl
     g.ldc = ldc;
     g.alpha = alpha;
     g.beta = beta;
-    g.tiles_m = (M + 127) / 128;
+    const bool low = !ta && M <= 64;  // one row of 64-row tiles
+    g.tiles_m = low ? 1 : (M + 127) / 128;
     g.tiles_n = (N + 127) / 128;
     const long tiles = (long)g.tiles_m * g.tiles_n;
     if (tiles > (1L << 24)) return 0;
     int workgroups = cus - cus % 8;  // every workgroup has a compute unit to itself (its LDS); whole dies keep the bands of tiles
     if (tiles < workgroups) workgroups = (int)tiles;
-    return ta ? launch128<true>(g, workgroups) : launch128<false>(g, workgroups);
+    if (low) return launch128<false, 64>(g, workgroups);
+    return ta ? launch128<true, 128>(g, workgroups) : launch128<false, 128>(g, workgroups);
 }
 
 }  // namespace dali_hip
