@@ -297,7 +297,9 @@ def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
 
 @pytest.mark.parametrize("M,N,K", [(1, 32000, 1024), (8, 4096, 1024), (64, 1000, 260), (17, 777, 512), (33, 2049, 64), (64, 8192, 2048),
                                    (5, 40000, 68), (48, 32000, 1024), (8, 1024, 1024), (8, 256, 1024), (9, 512, 512), (20, 4096, 256),
-                                   (64, 1024, 32000), (40, 1028, 16384)])
+                                   (64, 1024, 32000), (40, 1028, 16384),
+                                   # 53 to 64 rows against B stored [K][N]: 64-row tiles fed through LDS (whole 32-deep slabs, then the rest)
+                                   (60, 32000, 1024), (57, 9000, 300)])
 @pytest.mark.parametrize("tb", [0, 1])
 def test_sgemm_with_few_rows_streams_the_right_operand(gpu, rng, M, N, K, tb):
     """At most 64 rows against a wide row-major right operand (the output projection of a decoder step): the kernel that
@@ -330,6 +332,46 @@ def test_sgemm_with_few_rows_streams_the_right_operand(gpu, rng, M, N, K, tb):
         hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
         assert np.abs(out[:, :N] - want).max() <= 1e-4 * scale
         assert np.isnan(out[:, N:]).all()
+    for p in (dA, dB, dC):
+        hip.dali_hip_free(p)
+
+
+@pytest.mark.parametrize("M,N,K,ta", [(2052, 2052, 132, 0), (2052, 2052, 132, 1), (1024, 32000, 256, 1), (300, 12800, 96, 0), (300, 12800, 32, 1),
+                                      (129, 24704, 64, 0), (132, 24704, 160, 1), (4096, 768, 2048, 0), (60, 32000, 1024, 0), (57, 9000, 300, 0),
+                                      (64, 8192, 256, 0)])
+def test_sgemm_many_tiles_walked_by_one_workgroup_per_compute_unit(gpu, rng, M, N, K, ta):
+    """Products of 192 and more 128x128 tiles (and of 53 to 64 rows against a wide right operand) with B stored [K][N] and
+    operands the loads can write straight into LDS (16-byte aligned rows, an even row length of C): one workgroup per compute
+    unit walks a list of tiles, the part of the inner extent beyond whole 32-deep slabs is added by a second launch. Padded
+    leading dimensions with NaN in every padding (nothing outside the operands may reach a result, tiles that hang over the
+    edges of C included), alpha and beta, then beta = 0 over a destination full of NaN; against the product in double
+    precision, every element."""
+    hip = gpu
+    A = rng.randn(M, K).astype(np.float32)
+    B = rng.randn(K, N).astype(np.float32)
+    lda, ldb, ldc = (M + 4 if ta else K + 4), N + 8, N + 2
+    Ap = np.full((K, lda) if ta else (M, lda), np.nan, np.float32)
+    if ta:
+        Ap[:, :M] = A.T
+    else:
+        Ap[:, :K] = A
+    Bp = np.full((K, ldb), np.nan, np.float32)
+    Bp[:, :N] = B
+    C0 = rng.randn(M, ldc).astype(np.float32)
+    dA, dB, dC = _dev(hip, Ap), _dev(hip, Bp), _dev(hip, C0)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    scale = np.abs(want).max() + 1e-6
+    out = np.empty_like(C0)
+    assert hip.dali_hip_sgemm(0, ta, N, M, K, 0.75, dB, ldb, dA, lda, -0.5, dC, ldc) == 0, hip.dali_hip_last_error()
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+    assert np.abs(out[:, :N] - (0.75 * want - 0.5 * C0[:, :N])).max() <= 1e-4 * scale
+    assert np.array_equal(out[:, N:], C0[:, N:])  # padding untouched
+    nan = np.full_like(C0, np.nan)
+    hip.dali_hip_memcpy_h2d(dC, nan.ctypes.data_as(C.c_void_p), nan.nbytes)
+    assert hip.dali_hip_sgemm(0, ta, N, M, K, 1.0, dB, ldb, dA, lda, 0.0, dC, ldc) == 0, hip.dali_hip_last_error()
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+    assert np.abs(out[:, :N] - want).max() <= 1e-4 * scale
+    assert np.isnan(out[:, N:]).all()
     for p in (dA, dB, dC):
         hip.dali_hip_free(p)
 
