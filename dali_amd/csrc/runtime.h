@@ -44,8 +44,8 @@ int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const floa
 int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
                      float alpha, float beta, float* C, int ldc, int shares, int cus);
 // sgemm_dma128.hip: row-major C[M, N] = alpha * A . B + beta * C over whole 32-deep slabs with 128x128 tiles, one workgroup per
-// compute unit walking a list of tiles (B stored [K][N]; ta: A stored as [K][M]). Same return values.
-int sgemm_dma128(bool ta, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float alpha, float beta, float* C, int ldc, int cus);
+// compute unit walking a list of tiles (ta: A stored as [K][M]; tb: B stored as [N][K]). Same return values.
+int sgemm_dma128(bool ta, bool tb, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float alpha, float beta, float* C, int ldc, int cus);
 // hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per kernel: later launches of that kernel, which may be recorded into a
 // graph, are launches only. Keyed on the kernel's address (kernels of one signature share a function type, so a flag inside a
 // generic lambda or template would be shared among them).

@@ -899,24 +899,24 @@ static int stream_product(const GemmArgs& g, bool ta, bool tb, int shares) {
     return launch_tile<64, 64, 64, 2, 2, false>(rest, ta, tb, true, 1, true);
 }
 
-// Many 128x128 tiles of a single product with B stored [K][N]: the whole 32-deep slabs through the kernel that walks a list of
-// tiles per compute unit, what is left of the inner extent by a checked launch that adds to the result. -1: not a case for it.
-static int tiles128_product(const GemmArgs& g, bool ta) {
+// Many 128x128 tiles of a single product: the whole 32-deep slabs through the kernel that walks a list of tiles per compute
+// unit, what is left of the inner extent by a checked launch that adds to the result. -1: not a case for it.
+static int tiles128_product(const GemmArgs& g, bool ta, bool tb) {
     const GemmSeg& sg = g.seg[0];
     const int kw = sg.K / 32 * 32, kr = sg.K - kw;
     if (kw == 0) return -1;
     const int cus = device_cus();
     if (cus <= 0) return -1;
-    const int r = sgemm_dma128(ta, g.M, g.N, kw, sg.A, sg.lda, sg.B, sg.ldb, g.alpha, g.beta, g.C, g.ldc, cus);
+    const int r = sgemm_dma128(ta, tb, g.M, g.N, kw, sg.A, sg.lda, sg.B, sg.ldb, g.alpha, g.beta, g.C, g.ldc, cus);
     if (r < 0) return DALI_HIP_ERROR;
     if (r == 0) return -1;
     if (kr == 0) return DALI_HIP_OK;
     GemmArgs rest = g;
     rest.seg[0].A = sg.A + (ta ? (size_t)kw * sg.lda : (size_t)kw);
-    rest.seg[0].B = sg.B + (size_t)kw * sg.ldb;
+    rest.seg[0].B = sg.B + (tb ? (size_t)kw : (size_t)kw * sg.ldb);
     rest.seg[0].K = kr;
     rest.beta = 1.0f;
-    return launch_tile<128, 128, 32, 2>(rest, ta, false, true, 1, true);
+    return launch_tile<128, 128, 32, 2>(rest, ta, tb, true, 1, true);
 }
 
 // Row-major driver: C[M,N] = alpha * sum_s opA_s * opB_s + beta * C.
@@ -983,7 +983,7 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
     // kernel takes 26 us at 32 rows and grows with the rows, this one takes 38 to 41 us whatever they are)
     static const int low_rows_from = getenv("DALI_HIP_GEMM_LOW_ROWS") ? atoi(getenv("DALI_HIP_GEMM_LOW_ROWS")) : 52;
     if (g.nseg == 1 && vec && !ta && !tb && !row_map && !rows_may_overlap && M > low_rows_from && M <= 64 && N >= 8192 && g.seg[0].K >= 256) {
-        const int st = tiles128_product(g, false);
+        const int st = tiles128_product(g, false, false);
         if (st >= 0) return st;
     }
     if (g.nseg == 1 && g.seg[0].K > 0 && !ta && !row_map && !rows_may_overlap && M <= 64) {
@@ -1018,8 +1018,8 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         if (st >= 0) return st;
     }
     if (tiles128 >= 192) {
-        if (vec && g.nseg == 1 && !tb && !g.map_on && !rows_may_overlap) {
-            const int st = tiles128_product(g, ta);
+        if (vec && g.nseg == 1 && !g.map_on && !rows_may_overlap) {
+            const int st = tiles128_product(g, ta, tb);
             if (st >= 0) return st;
         }
         return run_tile<128, 128, 32, 2>(g, ta, tb, vec, 1);

@@ -1,9 +1,9 @@
 // fp32 GEMM for grids of many tiles: 128x128 tiles of C, one workgroup per compute unit walking a list of them, operand slabs
 // written into LDS by the loads themselves (global_load_lds_dwordx4), four slabs of 32 in flight.
 //
-// Row-major view: C[M,N] = alpha * A[M,K] * B[K,N] + beta * C with B stored [K][N] and A stored [M][K] or [K][M]
-// (dali_hip_sgemm; the reference's call is dali/array/gemm/cublas_gemm.cu:153-166, and with A stored [K][M] the weight
-// gradient matmul(a.w.transpose(), out_dw) of dali/tensor/op/dot.cpp:17-18).
+// Row-major view: C[M,N] = alpha * A[M,K] * B[K,N] + beta * C with A stored [M][K] or [K][M] and B stored [K][N] or [N][K]
+// (dali_hip_sgemm; the reference's call is dali/array/gemm/cublas_gemm.cu:153-166; with a transposed operand the products
+// matmul(a.w.transpose(), out_dw) and matmul(out_dw, b.w.transpose()) of dali/tensor/op/dot.cpp:17-18).
 //
 // Against the 64x64 kernel of the same kind (sgemm_dma.hip) a tile of 128x128 asks the caches for half as many operand bytes
 // per flop, which is what limits that kernel once every compute unit runs it (32 KiB per microsecond each). Eight waves
@@ -66,9 +66,13 @@ __device__ __forceinline__ void wait_all() { asm volatile("s_waitcnt vmcnt(0)" :
 // TA: A stored as [K][M]. TM: rows of a tile, 128, or 64 for products of at most 64 rows against a wide B (the output
 // projection of a decoder step at a batch the row-streaming kernel no longer serves well: such a product is bound by the matrix
 // pipe, 4.2 GFLOP at [64,1024].[1024,32000], and 128-row tiles would double that); the wave tiles are then 32 rows high.
-template <bool TA, int TM>
+// TB: B stored as [N][K]; it is then kept and read like A stored [M][K], and a lane's two 16-column tiles are two runs of
+// sixteen consecutive columns. With A stored [K][M] as well, A's rows are read one k at a time (k = 16 t + 4 kq + c, the order
+// in which the pieces of B deliver theirs), still four row classes to a 16-byte read.
+template <bool TA, bool TB, int TM>
 __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     static_assert(TM == 128 || (TM == 64 && !TA), "64-row tiles are built for A stored [M][K]");
+    constexpr bool OUTER = TA && !TB;  // both operands run across memory rows: one k-quad per step
     constexpr int RB = TM / 32;   // 16-row blocks of a wave tile
     constexpr int AQ = TM / 64;   // loads of A per wave and slab
     constexpr int LPS = AQ + 2;   // loads per wave and slab
@@ -107,7 +111,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     };
 
     const long a_step = (TA ? (long)32 * g.lda : 32L) * (long)sizeof(float);
-    const long b_step = (long)32 * g.ldb * (long)sizeof(float);
+    const long b_step = (TB ? 32L : (long)32 * g.ldb) * (long)sizeof(float);
     unsigned a_off[2], b_off[2], a_dst[2], b_dst[2];
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
@@ -137,9 +141,13 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
                 col = col < M ? col : M - 4;
                 a_off[q] = (unsigned)(((size_t)k * g.lda + col) * sizeof(float));
             }
-            {
+            if (TB) {
+                const int r_in = 8 * c + (lane >> 3), s = lane & 7;
+                const int row = n0 + r_in < N ? n0 + r_in : N - 1;
+                b_off[q] = (unsigned)(((size_t)row * g.ldb + 4 * (s ^ ((r_in >> 1) & 7))) * sizeof(float));
+            } else {
                 const int k = 2 * c + (lane >> 5), s = lane & 31;
-                const int bit = TA ? (k & 1) : ((k >> 2) & 1);
+                const int bit = OUTER ? (k & 1) : ((k >> 2) & 1);
                 int col = n0 + 4 * (s ^ (bit << 3));
                 col = col < N ? col : N - 4;
                 b_off[q] = (unsigned)(((size_t)k * g.ldb + col) * sizeof(float));
@@ -169,9 +177,9 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
 
     // ---- operand addresses of this lane within a stage
     // [K][x] operands: row 4 kk + kq of the slab; A [M][K]: row block rb of the wave tile, piece 4 t + kq
-    unsigned a_addr[4], b_addr;
+    unsigned a_addr[4], b_addr, b_addr_t[2];
     if (TA) {
-        a_addr[0] = (unsigned)(kq * 512 + (wm * 64 + 4 * l16) * 4);
+        a_addr[0] = (unsigned)(kq * (OUTER ? 512 : 2048) + (wm * 64 + 4 * l16) * 4);  // row kq, or row 4 kq of a k-group
         a_addr[1] = a_addr[2] = a_addr[3] = 0;
     } else {
 #pragma unroll
@@ -182,6 +190,11 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     }
     // (the swizzle bit of B's row is bit 0 of kq in both forms: k = 4 kk + kq, or (k >> 2) = 4 t + kq)
     b_addr = (unsigned)(kBOffset + ((wn * 8 + (l16 >> 1)) ^ ((kq & 1) << 3)) * 16 + (l16 & 1) * 8);
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+        const int r_in = wn * 32 + 16 * cb + l16;
+        b_addr_t[cb] = (unsigned)(kBOffset + r_in * 128 + ((kq ^ ((r_in >> 1) & 7)) * 16));
+    }
 
     floatx4 acc[RB][2];
     auto clear = [&]() __attribute__((always_inline)) {
@@ -197,21 +210,32 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     // !TA: set o holds one k-group of 16 (a[rb]: four k of row block rb, b[c]: row 16 t + 4 kq + c).
     floatx4 a_tn[2];
     floatx2 b_tn[2];
-    floatx4 a_nn[2][RB];
+    floatx4 a_nn[2][4];  // A [M][K]: [row block] with four k; A [K][M] beside B [N][K]: [c] with four row classes
     floatx2 b_nn[2][4];
+    floatx4 b_nt[2][2];  // B [N][K]: [column block] with four k
     auto load_ops = [&](auto ST, int step, int o) __attribute__((always_inline)) {
         constexpr int st = decltype(ST)::value;
         const char* base = lds + st * kStageBytes;
-        if (TA) {
+        if (OUTER) {
             // step = kk (0..7)
             a_tn[o] = *(const floatx4*)(base + a_addr[0] + step * 2048);
             b_tn[o] = *(const floatx2*)(base + b_addr + kq * 512 + step * 2048);
         } else {
             // step = t (0..1)
+            if (TA) {
 #pragma unroll
-            for (int rb = 0; rb < RB; ++rb) a_nn[o][rb] = *(const floatx4*)(base + (a_addr[rb] ^ (unsigned)(step * 64)));
+                for (int c = 0; c < 4; ++c) a_nn[o][c] = *(const floatx4*)(base + a_addr[0] + (16 * step + c) * 512);
+            } else {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) b_nn[o][c] = *(const floatx2*)(base + b_addr + (16 * step + 4 * kq + c) * 512);
+                for (int rb = 0; rb < RB; ++rb) a_nn[o][rb] = *(const floatx4*)(base + (a_addr[rb] ^ (unsigned)(step * 64)));
+            }
+            if (TB) {
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb) b_nt[o][cb] = *(const floatx4*)(base + (b_addr_t[cb] ^ (unsigned)(step * 64)));
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) b_nn[o][c] = *(const floatx2*)(base + b_addr + (16 * step + 4 * kq + c) * 512);
+            }
         }
     };
     // eight matrix instructions on independent sums
@@ -225,7 +249,8 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-            for (int ub = 0; ub < 2; ++ub) acc[rb][ub] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_nn[o][rb][c], b_nn[o][c][ub], acc[rb][ub], 0, 0, 0);
+            for (int ub = 0; ub < 2; ++ub)
+                acc[rb][ub] = __builtin_amdgcn_mfma_f32_16x16x4f32(TA ? a_nn[o][c][rb] : a_nn[o][rb][c], TB ? b_nt[o][ub][c] : b_nn[o][c][ub], acc[rb][ub], 0, 0, 0);
     };
 
     // ---- the side that multiplies
@@ -235,7 +260,25 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
         tile_at(first + c_r * stride, mt, nt);
         const int m_base = TM * mt + wm * (TM / 2), nn = 128 * nt + wn * 32 + 2 * l16;
         const float alpha = g.alpha, beta = g.beta;
-        if (nn < N) {  // (N is a multiple of 4 and nn even: nn + 1 < N as well)
+        if (TB) {
+            // a lane's two sums of a row are sixteen columns apart
+#pragma unroll
+            for (int i = 0; i < RB; ++i)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int m = m_base + (TA ? 16 * kq + 4 * v + i : 16 * i + 4 * kq + v);
+#pragma unroll
+                    for (int cb = 0; cb < 2; ++cb) {
+                        const int col = 128 * nt + wn * 32 + 16 * cb + l16;
+                        if (m < M && col < N) {
+                            float* c = g.C + (size_t)m * g.ldc + col;
+                            float r = alpha * acc[i][cb][v];
+                            if (beta != 0.f) r += beta * *c;
+                            *c = r;
+                        }
+                    }
+                }
+        } else if (nn < N) {  // (N is a multiple of 4 and nn even: nn + 1 < N as well)
 #pragma unroll
             for (int i = 0; i < RB; ++i)
 #pragma unroll
@@ -266,7 +309,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
         constexpr int st = decltype(ST)::value;
         constexpr bool has1 = decltype(H1)::value, has2 = decltype(H2)::value, has3 = decltype(H3)::value;
         using NX = std::integral_constant<int, (st + 1) % 4>;
-        if (TA) {
+        if (OUTER) {
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk) {
                 if (kk < 7) load_ops(ST, kk + 1, (kk + 1) & 1);
@@ -352,9 +395,9 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
 
 bool aligned_to(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-template <bool TA, int TM>
+template <bool TA, bool TB, int TM>
 int launch128(const Args128& g, int workgroups) {
-    auto kernel = sgemm_dma128_kernel<TA, TM>;
+    auto kernel = sgemm_dma128_kernel<TA, TB, TM>;
     hipError_t e = reserve_dynamic_lds((const void*)kernel, kLdsBytes);
     if (e != hipSuccess) return fail("sgemm: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
     hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(512), kLdsBytes, stream(), g);
@@ -365,15 +408,17 @@ int launch128(const Args128& g, int workgroups) {
 
 }  // namespace
 
-int sgemm_dma128(bool ta, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float alpha, float beta, float* C, int ldc, int cus) {
+int sgemm_dma128(bool ta, bool tb, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float alpha, float beta, float* C, int ldc, int cus) {
     static const int enabled = getenv("DALI_HIP_GEMM_DMA128") ? atoi(getenv("DALI_HIP_GEMM_DMA128")) : 1;
     if (!enabled || cus < 8 || M < 1 || N < 4 || K < 32 || K % 32 != 0) return 0;
-    // 16-byte pieces that start on 16-byte boundaries and never straddle the end of a row; pairs of results stored as 8 bytes
-    if (lda % 4 != 0 || ldb % 4 != 0 || N % 4 != 0 || (ta && (M % 4 != 0 || M < 4)) || ldc % 2 != 0) return 0;
-    if (!aligned_to(A, 16) || !aligned_to(B, 16) || !aligned_to(C, 8)) return 0;
+    // 16-byte pieces that start on 16-byte boundaries and never straddle the end of a row; with B stored [K][N] pairs of results
+    // are stored as 8 bytes
+    if (lda % 4 != 0 || ldb % 4 != 0 || (ta && (M % 4 != 0 || M < 4))) return 0;
+    if (!tb && (N % 4 != 0 || ldc % 2 != 0 || !aligned_to(C, 8))) return 0;
+    if (!aligned_to(A, 16) || !aligned_to(B, 16)) return 0;
     // per-lane offsets are 32-bit and relative to a pointer that walks along k
     const size_t a_span = ((size_t)(ta ? 32 : M) * lda + (ta ? M : 32)) * sizeof(float);
-    const size_t b_span = ((size_t)32 * ldb + N) * sizeof(float);
+    const size_t b_span = ((size_t)(tb ? N : 32) * ldb + (tb ? 32 : N)) * sizeof(float);
     if (a_span >= ((size_t)1 << 32) || b_span >= ((size_t)1 << 32)) return 0;
     Args128 g = {};
     g.A = A;
@@ -387,15 +432,18 @@ int sgemm_dma128(bool ta, int M, int N, int K, const float* A, int lda, const fl
     g.ldc = ldc;
     g.alpha = alpha;
     g.beta = beta;
-    const bool low = !ta && M <= 64;  // one row of 64-row tiles
+    const bool low = !ta && !tb && M <= 64;  // one row of 64-row tiles
     g.tiles_m = low ? 1 : (M + 127) / 128;
     g.tiles_n = (N + 127) / 128;
     const long tiles = (long)g.tiles_m * g.tiles_n;
     if (tiles > (1L << 24)) return 0;
     int workgroups = cus - cus % 8;  // every workgroup has a compute unit to itself (its LDS); whole dies keep the bands of tiles
     if (tiles < workgroups) workgroups = (int)tiles;
-    if (low) return launch128<false, 64>(g, workgroups);
-    return ta ? launch128<true, 128>(g, workgroups) : launch128<false, 128>(g, workgroups);
+    if (low) return launch128<false, false, 64>(g, workgroups);
+    if (!ta && !tb) return launch128<false, false, 128>(g, workgroups);
+    if (ta && !tb) return launch128<true, false, 128>(g, workgroups);
+    if (!ta && tb) return launch128<false, true, 128>(g, workgroups);
+    return launch128<true, true, 128>(g, workgroups);
 }
 
 }  // namespace dali_hip

@@ -336,12 +336,14 @@ def test_sgemm_with_few_rows_streams_the_right_operand(gpu, rng, M, N, K, tb):
         hip.dali_hip_free(p)
 
 
-@pytest.mark.parametrize("M,N,K,ta", [(2052, 2052, 132, 0), (2052, 2052, 132, 1), (1024, 32000, 256, 1), (300, 12800, 96, 0), (300, 12800, 32, 1),
-                                      (129, 24704, 64, 0), (132, 24704, 160, 1), (4096, 768, 2048, 0), (60, 32000, 1024, 0), (57, 9000, 300, 0),
-                                      (64, 8192, 256, 0)])
-def test_sgemm_many_tiles_walked_by_one_workgroup_per_compute_unit(gpu, rng, M, N, K, ta):
-    """Products of 192 and more 128x128 tiles (and of 53 to 64 rows against a wide right operand) with B stored [K][N] and
-    operands the loads can write straight into LDS (16-byte aligned rows, an even row length of C): one workgroup per compute
+@pytest.mark.parametrize("M,N,K,ta,tb", [(2052, 2052, 132, 0, 0), (2052, 2052, 132, 1, 0), (1024, 32000, 256, 1, 0), (300, 12800, 96, 0, 0),
+                                         (300, 12800, 32, 1, 0), (129, 24704, 64, 0, 0), (132, 24704, 160, 1, 0), (4096, 768, 2048, 0, 0),
+                                         (60, 32000, 1024, 0, 0), (57, 9000, 300, 0, 0), (64, 8192, 256, 0, 0),
+                                         (2052, 2051, 132, 0, 1), (2052, 2050, 132, 1, 1), (300, 12801, 96, 0, 1), (8192, 1024, 320, 0, 1),
+                                         (132, 24703, 64, 1, 1)])
+def test_sgemm_many_tiles_walked_by_one_workgroup_per_compute_unit(gpu, rng, M, N, K, ta, tb):
+    """Products of 192 and more 128x128 tiles (and of 53 to 64 rows against a wide right operand stored [K][N]) with
+    operands the loads can write straight into LDS (16-byte aligned rows; with B stored [K][N] an even row length of C): one workgroup per compute
     unit walks a list of tiles, the part of the inner extent beyond whole 32-deep slabs is added by a second launch. Padded
     leading dimensions with NaN in every padding (nothing outside the operands may reach a result, tiles that hang over the
     edges of C included), alpha and beta, then beta = 0 over a destination full of NaN; against the product in double
@@ -349,26 +351,29 @@ def test_sgemm_many_tiles_walked_by_one_workgroup_per_compute_unit(gpu, rng, M, 
     hip = gpu
     A = rng.randn(M, K).astype(np.float32)
     B = rng.randn(K, N).astype(np.float32)
-    lda, ldb, ldc = (M + 4 if ta else K + 4), N + 8, N + 2
+    lda, ldb, ldc = (M + 4 if ta else K + 4), (K + 8 if tb else N + 8), N + (3 if tb else 2)
     Ap = np.full((K, lda) if ta else (M, lda), np.nan, np.float32)
     if ta:
         Ap[:, :M] = A.T
     else:
         Ap[:, :K] = A
-    Bp = np.full((K, ldb), np.nan, np.float32)
-    Bp[:, :N] = B
+    Bp = np.full((N, ldb) if tb else (K, ldb), np.nan, np.float32)
+    if tb:
+        Bp[:, :K] = B.T
+    else:
+        Bp[:, :N] = B
     C0 = rng.randn(M, ldc).astype(np.float32)
     dA, dB, dC = _dev(hip, Ap), _dev(hip, Bp), _dev(hip, C0)
     want = A.astype(np.float64) @ B.astype(np.float64)
     scale = np.abs(want).max() + 1e-6
     out = np.empty_like(C0)
-    assert hip.dali_hip_sgemm(0, ta, N, M, K, 0.75, dB, ldb, dA, lda, -0.5, dC, ldc) == 0, hip.dali_hip_last_error()
+    assert hip.dali_hip_sgemm(tb, ta, N, M, K, 0.75, dB, ldb, dA, lda, -0.5, dC, ldc) == 0, hip.dali_hip_last_error()
     hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
     assert np.abs(out[:, :N] - (0.75 * want - 0.5 * C0[:, :N])).max() <= 1e-4 * scale
     assert np.array_equal(out[:, N:], C0[:, N:])  # padding untouched
     nan = np.full_like(C0, np.nan)
     hip.dali_hip_memcpy_h2d(dC, nan.ctypes.data_as(C.c_void_p), nan.nbytes)
-    assert hip.dali_hip_sgemm(0, ta, N, M, K, 1.0, dB, ldb, dA, lda, 0.0, dC, ldc) == 0, hip.dali_hip_last_error()
+    assert hip.dali_hip_sgemm(tb, ta, N, M, K, 1.0, dB, ldb, dA, lda, 0.0, dC, ldc) == 0, hip.dali_hip_last_error()
     hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
     assert np.abs(out[:, :N] - want).max() <= 1e-4 * scale
     assert np.isnan(out[:, N:]).all()
