@@ -168,7 +168,15 @@ def test_rows_off_the_vector_alignment_keep_vector_accesses(D, rng):
     D.generate_only([op.softmax(x)], compile=True)
     body = D.last_source()
     body = body[body.index("void dali_row_"):]
-    assert "dali_loadu" in body and "dali_storeu" in body and "tail_on" in body  # whole vectors + one element per thread
+    # source and destination rows start at the same distance from a 16-byte boundary: aligned vectors from the row's first
+    # boundary, the elements in front of it and behind the last vector one to a thread
+    assert "const int head" in body and "dali_loadu" not in body and "dali_storeu" not in body and "tail_on" in body
+    assert "(v1 + (long)ch * 4)" in body and "tail_col = tr < head ? tr : CH * VEC + tr" in body
+    y = D.Array.from_numpy(rng.randn(8, 1001).astype(np.float32))
+    D.generate_only([op.softmax(x[:, 2:]) * y[:, :999]], compile=True)  # operands that start their rows at different distances
+    body = D.last_source()
+    body = body[body.index("void dali_row_"):]
+    assert "dali_loadu" in body and "dali_storeu" in body and "tail_on" in body  # whole unaligned vectors + one element per thread
     D.generate_only([op.softmax(x[:, 1:])], compile=True)  # 1000 columns starting one element in: no rest, still unaligned
     body = D.last_source()
     body = body[body.index("void dali_row_"):]
