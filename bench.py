@@ -184,6 +184,13 @@ def main():
             bias = D.Array.zeros((4096,))
             probe("c5_gemm_pair_256x2048x4096", lambda: (op.dot(X, W) + op.dot(Hp, U)).eval(), 20)
             probe("c5_lstm_step_fused", lambda: op.lstm_step(X, Hp, Cp, W, U, bias), 20)
+            del X, Hp, Cp, W, U, bias
+            # the products of the backward pass of dot(h [256,1024], W [1024,32000]): many 128x128 tiles walked by one workgroup per
+            # compute unit, and 64 tiles x 4 shares of a long inner extent
+            bh, bg, bw = (D.Array.from_numpy((np.random.RandomState(s).randn(*shp) * 0.1).astype(np.float32))
+                          for s, shp in ((60, (256, 1024)), (61, (256, 32000)), (62, (1024, 32000))))
+            probe("dot_backward_weights_256x1024T_x_256x32000", lambda: op.dot(bh.transpose(), bg).eval(), 10)
+            probe("dot_backward_inputs_256x32000_x_1024x32000T", lambda: op.dot(bg, bw.transpose()).eval(), 10)
         return
 
     # ------------------------------------------------------------ headline: C1
