@@ -35,7 +35,8 @@ typedef float floatx2 __attribute__((ext_vector_type(2)));
 
 constexpr int kStageBytes = 32768;
 constexpr int kBOffset = 16384;
-constexpr int kLdsBytes = 4 * kStageBytes;
+constexpr int kLdsBytes = 4 * kStageBytes + 16;  // four stages and one flag
+constexpr int kDeviceScope = 16;                 // cache policy of a buffer access: device scope (the sc1 bit)
 
 struct Args128 {
     const float* A;
@@ -47,6 +48,12 @@ struct Args128 {
     int ldc;
     float alpha, beta;
     int tiles_m, tiles_n;
+    // The tiles are dealt in `rounds` whole rounds of one tile per workgroup; the `rem` tiles left over (fewer than there are
+    // workgroups) are either worked whole by the first `rem` workgroups (shares = 0) or cut along the inner extent into equal
+    // shares, one per workgroup (boundaries within `min_frag` slabs of a tile's edge move to the edge).
+    int rounds, rem, shares, min_frag;  // shares: workgroups that take a share of the left-over tiles (0: those tiles go whole)
+    unsigned int* counters;  // one ticket counter per left-over tile (zero at rest)
+    float* partials;         // [2 * workgroups][128 * 128]: a workgroup's share that starts inside a tile, then the one that ends inside one
 };
 
 // One 16-byte piece per lane from global memory straight into LDS: lane l writes bytes [16 l, 16 l + 16) behind `lds_addr`
@@ -69,7 +76,9 @@ __device__ __forceinline__ void wait_all() { asm volatile("s_waitcnt vmcnt(0)" :
 // TB: B stored as [N][K]; it is then kept and read like A stored [M][K], and a lane's two 16-column tiles are two runs of
 // sixteen consecutive columns. With A stored [K][M] as well, A's rows are read one k at a time (k = 16 t + 4 kq + c, the order
 // in which the pieces of B deliver theirs), still four row classes to a 16-byte read.
-template <bool TA, bool TB, int TM>
+// SHARE: the launch cuts left-over tiles into shares (the code that publishes and adds them up is left out of the other form,
+// where it would sit, unused, behind every slab of the loop).
+template <bool TA, bool TB, int TM, bool SHARE>
 __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     static_assert(TM == 128 || (TM == 64 && !TA), "64-row tiles are built for A stored [M][K]");
     constexpr bool OUTER = TA && !TB;  // both operands run across memory rows: one k-quad per step
@@ -82,25 +91,52 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = w >> 2, wn = w & 3, l16 = lane & 15, kq = lane >> 4;
     const int M = g.M, N = g.N, n = g.slabs;
-    const int tiles = g.tiles_m * g.tiles_n;
-    // this workgroup's tiles: first, first + stride, ... The workgroups of one die (every eighth) take a contiguous band.
-    int first, stride, count;
-    {
-        const int G = gridDim.x, b = blockIdx.x;
-        if ((G & 7) == 0) {
-            const int chunk = (tiles + 7) / 8, wgx = G / 8;
-            const int lo = (b & 7) * chunk, hi = lo + chunk < tiles ? lo + chunk : tiles;
-            first = lo + b / 8;
-            stride = wgx;
-            count = first < hi ? (hi - first + wgx - 1) / wgx : 0;
-        } else {
-            first = b;
-            stride = G;
-            count = first < tiles ? (tiles - first + G - 1) / G : 0;
+    // This workgroup's work items: one whole tile per round, then its part of the left-over tiles. Workgroups are numbered die by
+    // die (every eighth workgroup runs on the same die): a die takes a contiguous band of the tiles of the whole rounds, and
+    // neighbouring shares of a left-over tile belong to workgroups of one die.
+    const int G = gridDim.x, wg = blockIdx.x;
+    const bool banded = (G & 7) == 0;
+    const int p = banded ? (wg & 7) * (G / 8) + wg / 8 : wg;
+    const int R = g.rounds;
+    const long T2 = (long)g.rem * n;  // slabs of the left-over tiles
+    auto bound = [&](int q) __attribute__((always_inline)) -> long {
+        if (q >= g.shares) return T2;
+        long x = (long)q * T2 / g.shares;
+        const int j = (int)(x % n);
+        if (j < g.min_frag) x -= j;
+        else if (n - j < g.min_frag) x += n - j;
+        return x;
+    };
+    long s2 = 0, e2 = 0;
+    if (g.rem > 0) {
+        if (SHARE) {
+            s2 = bound(p);
+            e2 = bound(p + 1);
+        } else if (p < g.rem) {
+            s2 = (long)p * n;
+            e2 = s2 + n;
         }
     }
+    const int t2_first = (int)(s2 / n), t2_last = e2 > s2 ? (int)((e2 - 1) / n) : -1;
+    const int count2 = e2 > s2 ? t2_last - t2_first + 1 : 0;
+    const int count = count2 + R;
     if (count == 0) return;
-    const int total = count * n;  // slabs of all tiles of this workgroup
+    const int total = R * n + (int)(e2 - s2);  // slabs of all items of this workgroup
+    // item -> tile and slabs [j0, j1) of it. The left-over tiles come first: their shares are then published and added up while
+    // everybody still has whole tiles to do, not at the end of the launch with every workgroup waiting on memory.
+    auto item_at = [&](int idx, int& tile, int& j0, int& j1) __attribute__((always_inline)) {
+        if (idx >= count2) {
+            const int r = idx - count2;
+            tile = banded ? (wg & 7) * (R * (G / 8)) + r * (G / 8) + wg / 8 : r * G + wg;
+            j0 = 0;
+            j1 = n;
+        } else {
+            const int t = t2_first + idx;
+            tile = R * G + t;
+            j0 = idx == 0 ? (int)(s2 - (long)t2_first * n) : 0;
+            j1 = t == t2_last ? (int)(e2 - (long)t * n) : n;
+        }
+    };
     // Tiles are numbered in column blocks four tiles wide, by rows inside a block: the 32 tiles that the workgroups of a die
     // work on together are 8 x 4 and share their operand slabs in that die's cache.
     auto tile_at = [&](int tile, int& mt, int& nt) __attribute__((always_inline)) {
@@ -119,12 +155,13 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
         b_dst[q] = (unsigned)(kBOffset + (w + 8 * q) * 1024);
     }
     // ---- the side that requests slabs
-    int i_r = 0, i_fj = 0;
+    int i_r = 0, i_j = 0, i_j1 = 0;
     const char* ap = nullptr;
     const char* bp = nullptr;
     auto request_tile = [&](int r) __attribute__((always_inline)) {
-        int mt, nt;
-        tile_at(first + r * stride, mt, nt);
+        int tile, j0, mt, nt;
+        item_at(r, tile, j0, i_j1);
+        tile_at(tile, mt, nt);
         const int m0 = TM * mt, n0 = 128 * nt;
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
@@ -153,19 +190,19 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
                 b_off[q] = (unsigned)(((size_t)k * g.ldb + col) * sizeof(float));
             }
         }
-        i_fj = 0;
-        ap = (const char*)g.A;
-        bp = (const char*)g.B;
+        i_j = j0;
+        ap = (const char*)g.A + (long)j0 * a_step;
+        bp = (const char*)g.B + (long)j0 * b_step;
     };
     auto issue = [&](int stage) __attribute__((always_inline)) {
         load_to_lds(a_dst[0] + stage * kStageBytes, a_off[0], ap);
         if (AQ > 1) load_to_lds(a_dst[1] + stage * kStageBytes, a_off[1], ap);
         load_to_lds(b_dst[0] + stage * kStageBytes, b_off[0], bp);
         load_to_lds(b_dst[1] + stage * kStageBytes, b_off[1], bp);
-        ++i_fj;
+        ++i_j;
         ap += a_step;
         bp += b_step;
-        if (i_fj == n) {
+        if (i_j == i_j1) {
             ++i_r;
             if (i_r < count) request_tile(i_r);
         }
@@ -254,13 +291,88 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     };
 
     // ---- the side that multiplies
-    int c_r = 0, c_fj = 0;
+    int c_r = 0, c_tile, c_j0, c_j, c_j1;
+    item_at(0, c_tile, c_j0, c_j1);
+    c_j = c_j0;
+    volatile int& is_last = *(volatile int*)(lds + 4 * kStageBytes);
+    // slabs [c_j0, c_j1) of tile c_tile are summed: a whole tile goes to C; a share of a left-over tile is published in the
+    // workspace and a ticket drawn, and whoever draws the tile's last ticket adds the shares in the order of their slabs (its
+    // own from registers), so the sum does not depend on who that is
     auto finish_tile = [&]() __attribute__((always_inline)) {
+        bool store = true;
+        if (SHARE && (c_j0 != 0 || c_j1 != n)) {
+            const int t = c_tile - R * G;  // left-over tile
+            // the workgroups whose shares meet in this tile: q0 .. q1 (those of them with a share at all)
+            auto owner_of = [&](long it) __attribute__((always_inline)) -> int {
+                int q = (int)(it * g.shares / T2);
+                q = q < 0 ? 0 : (q > g.shares - 1 ? g.shares - 1 : q);
+                while (q + 1 < g.shares && bound(q + 1) <= it) ++q;
+                while (bound(q) > it) --q;
+                return q;
+            };
+            const int q0 = owner_of((long)t * n), q1 = owner_of((long)(t + 1) * n - 1);
+            int sharers = 0;
+            for (int q = q0; q <= q1; ++q) sharers += bound(q + 1) > bound(q) ? 1 : 0;
+            // (16-byte device-scope accesses: written through to, and read from, the memory that all dies share)
+            float* mine = g.partials + (size_t)(c_j0 > 0 ? 2 * p : 2 * p + 1) * 16384;
+            const __amdgpu_buffer_rsrc_t mine_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)mine, 0, 65536, 0x00027000);
+#pragma unroll
+            for (int i = 0; i < RB; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, acc[i][j]), mine_rsrc,
+                                                           ((i * 2 + j) * 512 + tid) * 16, 0, kDeviceScope);
+            // the share is acknowledged by memory before the ticket is drawn
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (tid == 0) {
+                const unsigned int ticket = __hip_atomic_fetch_add(g.counters + t, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                is_last = ticket == (unsigned int)sharers - 1;
+            }
+            __syncthreads();
+            store = __builtin_amdgcn_readfirstlane(is_last) != 0;
+            if (store) {
+                floatx4 sum[RB][2];
+#pragma unroll
+                for (int i = 0; i < RB; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) sum[i][j] = (floatx4){0.f, 0.f, 0.f, 0.f};
+                for (int q = q0; q <= q1; ++q) {
+                    const long qb = bound(q);
+                    if (bound(q + 1) <= qb) continue;
+                    if (q == p) {
+#pragma unroll
+                        for (int i = 0; i < RB; ++i)
+#pragma unroll
+                            for (int j = 0; j < 2; ++j) sum[i][j] += acc[i][j];
+                    } else {
+                        const float* theirs = g.partials + (size_t)(qb > (long)t * n ? 2 * q : 2 * q + 1) * 16384;
+                        const __amdgpu_buffer_rsrc_t their_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)theirs, 0, 65536, 0x00027000);
+                        floatx4 got[RB][2];
+#pragma unroll
+                        for (int i = 0; i < RB; ++i)
+#pragma unroll
+                            for (int j = 0; j < 2; ++j)
+                                got[i][j] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(their_rsrc, ((i * 2 + j) * 512 + tid) * 16, 0, kDeviceScope));
+#pragma unroll
+                        for (int i = 0; i < RB; ++i)
+#pragma unroll
+                            for (int j = 0; j < 2; ++j) sum[i][j] += got[i][j];
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < RB; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) acc[i][j] = sum[i][j];
+                if (tid == 0) __hip_atomic_store(g.counters + t, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
         int mt, nt;
-        tile_at(first + c_r * stride, mt, nt);
+        tile_at(c_tile, mt, nt);
         const int m_base = TM * mt + wm * (TM / 2), nn = 128 * nt + wn * 32 + 2 * l16;
         const float alpha = g.alpha, beta = g.beta;
-        if (TB) {
+        if (!store) {
+        } else if (TB) {
             // a lane's two sums of a row are sixteen columns apart
 #pragma unroll
             for (int i = 0; i < RB; ++i)
@@ -301,7 +413,10 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
         }
         clear();
         ++c_r;
-        c_fj = 0;
+        if (c_r < count) {
+            item_at(c_r, c_tile, c_j0, c_j1);
+            c_j = c_j0;
+        }
     };
     // Slab i lives in stage i % 4. The barrier inside slab i is for slab i+1 (its loads were issued two slabs earlier); behind
     // it the buffer of slab i-1 is free and takes slab i+3.
@@ -350,7 +465,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
             mfma_nn(1, 3);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (++c_fj == n) finish_tile();
+        if (++c_j == c_j1) finish_tile();
     };
     auto tail_step = [&](auto J, auto R) __attribute__((always_inline)) {
         constexpr int j = decltype(J)::value, r = decltype(R)::value;
@@ -395,9 +510,9 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
 
 bool aligned_to(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-template <bool TA, bool TB, int TM>
+template <bool TA, bool TB, int TM, bool SHARE>
 int launch128(const Args128& g, int workgroups) {
-    auto kernel = sgemm_dma128_kernel<TA, TB, TM>;
+    auto kernel = sgemm_dma128_kernel<TA, TB, TM, SHARE>;
     hipError_t e = reserve_dynamic_lds((const void*)kernel, kLdsBytes);
     if (e != hipSuccess) return fail("sgemm: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
     hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(512), kLdsBytes, stream(), g);
@@ -438,12 +553,33 @@ int sgemm_dma128(bool ta, bool tb, int M, int N, int K, const float* A, int lda,
     const long tiles = (long)g.tiles_m * g.tiles_n;
     if (tiles > (1L << 24)) return 0;
     int workgroups = cus - cus % 8;  // every workgroup has a compute unit to itself (its LDS); whole dies keep the bands of tiles
-    if (tiles < workgroups) workgroups = (int)tiles;
-    if (low) return launch128<false, false, 64>(g, workgroups);
-    if (!ta && !tb) return launch128<false, false, 128>(g, workgroups);
-    if (ta && !tb) return launch128<true, false, 128>(g, workgroups);
-    if (!ta && tb) return launch128<false, true, 128>(g, workgroups);
-    return launch128<true, true, 128>(g, workgroups);
+    // Tiles that do not fill a last round are cut along the inner extent into shares, one per workgroup, unless the inner extent
+    // is short (fewer than eight
+    // slabs (3072x1536 over K = 4096, 288 tiles on 256 compute units: 77 -> 112 TFLOP/s).
+    static const int share_env = getenv("DALI_HIP_GEMM_SHARE_REST") ? atoi(getenv("DALI_HIP_GEMM_SHARE_REST")) : 1;
+    const int rest = (int)(tiles % workgroups);
+    // (a share costs about 5 us to publish and 5 us to add up: with no whole round to hide behind, inner extents under 1536 gain nothing)
+    const bool share = share_env && !low && rest > 0 && workgroups <= 256 && g.slabs >= (tiles < workgroups ? 48 : 16) &&
+                       (size_t)2 * workgroups * 16384 * sizeof(float) <= kWorkspacePartialBytes && rest <= kWorkspaceCounters;
+    if (!share && tiles < workgroups) workgroups = (int)tiles;
+    g.rounds = (int)(tiles / workgroups);
+    g.rem = (int)(tiles % workgroups);
+    // at most four workgroups to a tile (a fifth where the cuts fall unevenly): whoever adds the shares up fetches 64 KiB for each
+    g.shares = share ? (4 * rest < workgroups ? 4 * rest : workgroups) : 0;
+    g.min_frag = 2;
+    g.counters = (unsigned int*)workspace();
+    g.partials = (float*)(workspace() + kWorkspaceCounterBytes);
+    if (low) return launch128<false, false, 64, false>(g, workgroups);
+    if (share) {
+        if (!ta && !tb) return launch128<false, false, 128, true>(g, workgroups);
+        if (ta && !tb) return launch128<true, false, 128, true>(g, workgroups);
+        if (!ta && tb) return launch128<false, true, 128, true>(g, workgroups);
+        return launch128<true, true, 128, true>(g, workgroups);
+    }
+    if (!ta && !tb) return launch128<false, false, 128, false>(g, workgroups);
+    if (ta && !tb) return launch128<true, false, 128, false>(g, workgroups);
+    if (!ta && tb) return launch128<false, true, 128, false>(g, workgroups);
+    return launch128<true, true, 128, false>(g, workgroups);
 }
 
 }  // namespace dali_hip
