@@ -414,13 +414,14 @@ def main():
             Xq = D.Array.from_numpy(np.random.RandomState(24).randn(32, Bs, H).astype(np.float32))
             hs0, cs0 = (D.Array.from_numpy(np.random.RandomState(s).randn(Bs, H).astype(np.float32)) for s in (25, 26))
             row = {}
-            for name, flag in (("persistent", "1"), ("launch_per_step", "0")):
+            for name, flag in (("persistent", "2"), ("launch_per_step", "0")):  # "2": wherever the persistent kernels serve the size
                 os.environ["DALI_HIP_LSTM_PERSISTENT"] = flag
                 with D.Recording() as qrec:
                     op.lstm_sequence(Xq, hs0, cs0, W, U, bias)
                 row[name + "_us_per_step"] = round(time_recording(qrec, 10) / 32, 2)
                 row[name + "_launches"] = qrec.launches
             os.environ.pop("DALI_HIP_LSTM_PERSISTENT", None)
+            row["front_end_takes"] = "persistent" if hip.dali_hip_lstm_recurrent_persistent_supported(Bs, H) == 2 else "launch_per_step"
             sflops = 2.0 * Bs * (I + H) * 4 * H
             row["mfma_fp32_bound_us"] = round(sflops / MFMA_FP32_PEAK_TFLOPS / 1e6, 2)
             row["weights_from_hbm_bound_us"] = round(2 * 1024 * 4096 * 4 / HBM_PEAK_GBS / 1e3, 2)  # what a launch per step re-reads
@@ -437,13 +438,14 @@ def main():
             Wq, Uq = (D.Array.from_numpy(np.random.RandomState(s).uniform(-limq, limq, (Hs, 4 * Hs)).astype(np.float32)) for s in (12, 13))
             bq = D.Array.zeros((4 * Hs,))
             row = {}
-            for name, flag in (("persistent", "1"), ("launch_per_step", "0")):
+            for name, flag in (("persistent", "2"), ("launch_per_step", "0")):  # "2": wherever the persistent kernels serve the size
                 os.environ["DALI_HIP_LSTM_PERSISTENT"] = flag
                 with D.Recording() as qrec:
                     op.lstm_sequence(Xq, hs0, cs0, Wq, Uq, bq)
                 row[name + "_us_per_step"] = round(time_recording(qrec, 6) / 32, 2)
                 row[name + "_launches"] = qrec.launches
             os.environ.pop("DALI_HIP_LSTM_PERSISTENT", None)
+            row["front_end_takes"] = "persistent" if hip.dali_hip_lstm_recurrent_persistent_supported(Bs, Hs) == 2 else "launch_per_step"
             row["mfma_fp32_bound_us"] = round(2.0 * Bs * 2 * Hs * 4 * Hs / MFMA_FP32_PEAK_TFLOPS / 1e6, 2)
             other["B%d_H%d" % (Bs, Hs)] = row
             del Xq, hs0, cs0, Wq, Uq, bq, qrec
@@ -474,11 +476,15 @@ def main():
         for Bs in (1, 8, 32, 64):
             xq, hq, cq = (D.Array.from_numpy(np.random.RandomState(s).randn(Bs, H).astype(np.float32)) for s in (29, 30, 31))
             row = {}
-            for name, flag in (("small_batch_kernel_us", "1"), ("general_kernel_us", "0")):
+            # the path the front-end takes (the 16-row-tile kernel up to 16 rows, then the fused step with its inner extent cut into
+            # one share per compute unit), and the fused step whatever the batch
+            for name, flag in (("us", "1"), ("fused_step_us", "0")):
                 os.environ["DALI_HIP_LSTM_SMALL"] = flag
                 with D.Recording() as qrec:
                     op.lstm_step(xq, hq, cq, W, U, bias)
                 row[name] = round(time_recording(qrec, 100, 10), 2)
+                if flag == "1":
+                    row["kernel"] = D.last_kernel_kinds()
             os.environ.pop("DALI_HIP_LSTM_SMALL", None)
             row["weights_from_hbm_bound_us"] = round(2 * 1024 * 4096 * 4 / HBM_PEAK_GBS / 1e3, 2)
             single["B%d" % Bs] = row

@@ -521,11 +521,12 @@ extern "C" int dali_hip_lstm_recurrent_persistent_supported(int batch, int hidde
     if (ensure_init()) return 0;
     const int cus = compute_units();
     if (cus <= 0 || batch < 1) return 0;
-    if (lds_kernel_serves(batch, hidden, cus)) return 2;
-    if (!recurrent_phased_supported(batch, hidden, cus)) return 0;
-    // measured against one fused launch per step (us per step, 32 steps): 31 / 33 at 96 rows of 1024, 41 / 33 at 128; 53 / 61 at 64 rows of
-    // 2048, 106 / 64 at 128; 15 / 18 at 64 rows of 512, 30 / 18 at 128
-    return batch <= 96 ? 2 : 1;
+    if (!lds_kernel_serves(batch, hidden, cus) && !recurrent_phased_supported(batch, hidden, cus)) return 0;
+    // Measured against one fused launch per step, whose inner extent is cut into one share per compute unit at these batches
+    // (us per step over 32 steps, persistent / per step). 1024 hidden units: 6.2 / 16.7 at 8 rows, 11.7 / 17.2 at 32, 16.3 / 17.9 at
+    // 48, 18.8 / 18.3 at 64, 30.8 / 25.0 at 96; 512: 7.3 / 11.4 at 32, 11.7 / 11.7 at 48, 14.0 / 12.0 at 64; 2048: 27.3 / 40.2 at 32,
+    // 40.2 / 40.7 at 48, 52.8 / 40.7 at 64, 104 / 67 at 128.
+    return batch <= 32 || (batch <= 48 && hidden >= 1024) ? 2 : 1;
 }
 
 extern "C" int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0,

@@ -41,8 +41,10 @@ int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const floa
 // The same pipeline over a stream of work items per workgroup (one workgroup per compute unit walks many tiles, its loads
 // running ahead across tile boundaries); `shares` > 1 cuts every tile's inner extent into that many contiguous shares that meet
 // in the library workspace (single products only). `cus`: compute units of the bound device. Same return values.
+// With `bias` the sums go through the LSTM gate arithmetic instead of into C, as in sgemm_dma.
 int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
-                     float alpha, float beta, float* C, int ldc, int shares, int cus);
+                     float alpha, float beta, float* C, int ldc, int shares, int cus, const float* bias = nullptr, const float* c_prev = nullptr,
+                     float* c_out = nullptr, float* h_out = nullptr, int H = 0);
 // sgemm_dma128.hip: row-major C[M, N] = alpha * A . B + beta * C over whole 32-deep slabs with 128x128 tiles, one workgroup per
 // compute unit walking a list of tiles (ta: A stored as [K][M]; tb: B stored as [N][K]). Same return values.
 int sgemm_dma128(bool ta, bool tb, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float alpha, float beta, float* C, int ldc, int cus);

@@ -863,6 +863,16 @@ static int device_cus() {
     return cus;
 }
 
+// shares of the inner extent (64-deep slabs) for a product of `tiles64` 64x64 tiles that leaves compute units idle: one work
+// item per compute unit, at least four slabs each; below 2 the product is not cut
+static int stream_shares(long tiles64, int nslab64) {
+    const int cus = device_cus();
+    if (cus <= 0 || tiles64 <= 0 || tiles64 > cus / 2) return 1;
+    int shares = (int)(cus / tiles64);
+    if (shares > nslab64 / 4) shares = nslab64 / 4;
+    return shares < 1 ? 1 : shares;
+}
+
 // The whole slabs of a product of one or two terms through the streaming kernel, what is left of the inner extents by a
 // checked launch that adds to the result. -1: not a case for it (nothing was launched).
 static int stream_product(const GemmArgs& g, bool ta, bool tb, int shares) {
@@ -1042,13 +1052,12 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         // order by the workgroup that finishes last.
         int nslab64 = 0;
         for (int s = 0; s < g.nseg; ++s) nslab64 += (g.seg[s].K + 63) / 64;
-        if (stream_env == 0 && stream_fits && g.nseg == 1) {
+        if (stream_env == 0 && stream_fits) {
             // one item per compute unit through the kernel whose loads write LDS themselves, in shares of at least four slabs
             // ([256,1024] over 32000: 145 us against 158 us, against 210 us with B stored as [N][K]; [64,64] over 65536:
-            // 34 us against 65 us)
-            const int cus = device_cus();
-            int shares = cus > 0 ? (int)(cus / tiles64) : 0;
-            if (shares > nslab64 / 4) shares = nslab64 / 4;
+            // 34 us against 65 us). A sum of two products is cut the same way as the fused LSTM step of its shape, whose
+            // results it then matches bit for bit.
+            const int shares = stream_shares(tiles64, nslab64);
             if (shares >= 2) {
                 const int st = stream_product(g, ta, tb, shares);
                 if (st >= 0) return st;
@@ -1136,6 +1145,16 @@ int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx
         const float* as[2] = {X, Hprev};
         const float* bs[2] = {W, U};
         const int ks[2] = {input, hidden};
+        // a batch whose tiles leave compute units idle: shares of the inner extent, one work item per compute unit; whoever
+        // draws a tile's last ticket adds the shares and computes the gates (up to 64 rows of 1024: 32 -> 17-19 us, 128 rows: 35 -> 27 us)
+        static const int share_env = getenv("DALI_HIP_LSTM_STEP_SHARES") ? atoi(getenv("DALI_HIP_LSTM_STEP_SHARES")) : 1;
+        const int shares = share_env ? stream_shares((long)((batch + 63) / 64) * (4 * hidden / 64), (input + hidden) / 64) : 1;
+        if (shares >= 2) {
+            const int r = sgemm_dma_stream(false, false, batch, 4 * hidden, 2, ks, as, bs, ldx, ldw, 1.0f, 0.0f, nullptr, 0, shares, device_cus(), bias, Cprev, Cout, Hout,
+                                           hidden);
+            if (r < 0) return DALI_HIP_ERROR;
+            if (r > 0) return DALI_HIP_OK;
+        }
         const int r = sgemm_dma(false, false, batch, 4 * hidden, 2, ks, as, bs, ldx, ldw, 1.0f, 0.0f, nullptr, 0, bias, Cprev, Cout, Hout, hidden);
         if (r < 0) return DALI_HIP_ERROR;
         if (r > 0) return DALI_HIP_OK;

@@ -362,12 +362,18 @@ struct StreamArgs {
     int tiles_m, tiles_n, Z;
     unsigned int* counters;  // one ticket counter per tile (zero at rest)
     float* partials;         // [tile][share][4096]
+    // gate epilogue (GATES): C is not written; a tile's columns are the four gates of sixteen hidden units
+    const float* bias;
+    const float* c_prev;
+    float* c_out;
+    float* h_out;
+    int H;
 };
 
 constexpr int kFoldBytes = 16384;
 constexpr int kStreamLds = kDmaLds + kFoldBytes + 16;  // stages, exchange area, one flag
 
-template <bool TA, bool TB>
+template <bool TA, bool TB, bool GATES>
 __global__ __launch_bounds__(512, 1) void sgemm_dma_stream_kernel(StreamArgs g) {
     // (no static LDS beside this: the loads address LDS from offset 0)
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -441,7 +447,8 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_stream_kernel(StreamArgs g) 
                 a_off[q] = (unsigned)(((size_t)rr * g.lda + col) * sizeof(float));
             }
             if (!TB) {
-                int col = n0 + 4 * (s ^ ((c & 3) << 2));
+                const int gr = s ^ ((c & 3) << 2);
+                int col = GATES ? (gr / 4) * g.H + 16 * nt + 4 * (gr % 4) : n0 + 4 * gr;
                 col = col < N ? col : N - 4;
                 b_off[q] = (unsigned)(((size_t)rr * g.ldb + col) * sizeof(float));
             } else {
@@ -589,7 +596,30 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_stream_kernel(StreamArgs g) 
                 if (tid == 0) __hip_atomic_store(g.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        if (last) {
+        if (GATES) {
+            if (last) {
+                // the sums as a [64][64] tile of pre-activations in the exchange area; every thread then finishes two (row, hidden
+                // unit) pairs with the arithmetic of the fused step
+                __syncthreads();  // the exchange has been read
+#pragma unroll
+                for (int v = 0; v < 8; ++v) {
+                    const int e = kw * 8 + v;
+                    red[(wm * 32 + (e / 8) * 16 + 4 * kq + (e % 4)) * 64 + wn * 32 + ((e / 4) % 2) * 16 + l16] = sum[v];
+                }
+                __syncthreads();
+                const int H = g.H;
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const int e = tid + q * 512, r = e / 16, j = e % 16, m = m0 + r, hu = 16 * nt + j;
+                    if (m >= M) continue;
+                    float gate_bias[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) gate_bias[k] = g.bias[k * H + hu];
+                    const size_t o = (size_t)m * H + hu;
+                    lstm_gates(red[r * 64 + j], red[r * 64 + 16 + j], red[r * 64 + 32 + j], red[r * 64 + 48 + j], gate_bias, g.c_prev[o], g.c_out + o, g.h_out + o);
+                }
+            }
+        } else if (last) {
 #pragma unroll
             for (int v = 0; v < 8; ++v) {
                 const int e = kw * 8 + v;
@@ -711,9 +741,9 @@ bool operands_fit(bool ta, bool tb, int M, int N, int nseg, const int* K, const 
     return true;
 }
 
-template <bool TA, bool TB>
+template <bool TA, bool TB, bool GATES>
 int launch_stream(const StreamArgs& g, int workgroups) {
-    auto kernel = sgemm_dma_stream_kernel<TA, TB>;
+    auto kernel = sgemm_dma_stream_kernel<TA, TB, GATES>;
     hipError_t e = reserve_dynamic_lds((const void*)kernel, kStreamLds);
     if (e != hipSuccess) return fail("sgemm: cannot reserve %d bytes of LDS: %s", kStreamLds, hipGetErrorString(e));
     hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(512), kStreamLds, stream(), g);
@@ -725,7 +755,7 @@ int launch_stream(const StreamArgs& g, int workgroups) {
 }  // namespace
 
 int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
-                     float alpha, float beta, float* C, int ldc, int shares, int cus) {
+                     float alpha, float beta, float* C, int ldc, int shares, int cus, const float* bias, const float* c_prev, float* c_out, float* h_out, int H) {
     static const int enabled = getenv("DALI_HIP_GEMM_DMA") ? atoi(getenv("DALI_HIP_GEMM_DMA")) : 1;
     if (!enabled || cus < 8 || !operands_fit(ta, tb, M, N, nseg, K, A, B, lda, ldb)) return 0;
     StreamArgs g = {};
@@ -750,18 +780,27 @@ int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, con
     if (tiles > (1L << 24)) return 0;
     int Z = shares < 1 ? 1 : shares;
     if (Z > slabs) Z = slabs;
-    if (Z > 1 && (nseg != 1 || tiles > (long)kWorkspaceCounters || (size_t)tiles * Z * 4096 * sizeof(float) > kWorkspacePartialBytes)) Z = 1;
+    if (Z > 1 && (tiles > (long)kWorkspaceCounters || (size_t)tiles * Z * 4096 * sizeof(float) > kWorkspacePartialBytes)) Z = 1;
     g.Z = Z;
+    g.bias = bias;
+    g.c_prev = c_prev;
+    g.c_out = c_out;
+    g.h_out = h_out;
+    g.H = H;
     g.counters = (unsigned int*)workspace();
     g.partials = (float*)(workspace() + kWorkspaceCounterBytes);
     const long items = tiles * Z;
     // every workgroup has a compute unit to itself (its LDS); a whole number of workgroups per die keeps the bands of tiles
     int workgroups = cus - cus % 8;
     if (items < workgroups) workgroups = (int)items;
-    if (!ta && !tb) return launch_stream<false, false>(g, workgroups);
-    if (!ta && tb) return launch_stream<false, true>(g, workgroups);
-    if (ta && !tb) return launch_stream<true, false>(g, workgroups);
-    return launch_stream<true, true>(g, workgroups);
+    if (bias) {
+        if (ta || tb || N != 4 * H || H % 16 != 0) return 0;
+        return launch_stream<false, false, true>(g, workgroups);
+    }
+    if (!ta && !tb) return launch_stream<false, false, false>(g, workgroups);
+    if (!ta && tb) return launch_stream<false, true, false>(g, workgroups);
+    if (ta && !tb) return launch_stream<true, false, false>(g, workgroups);
+    return launch_stream<true, true, false>(g, workgroups);
 }
 
 int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,

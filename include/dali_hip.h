@@ -296,7 +296,7 @@ int dali_hip_lstm_step_small(int batch, int input, int hidden, const float* X, i
 int dali_hip_lstm_recurrent_persistent(int steps, int batch, int hidden, const float* pre, const float* U, int ldu, const float* h0,
                                        const float* c0, float* hs, float* c_out);
 /* Whether dali_hip_lstm_recurrent_persistent serves this batch and hidden size on the bound device: 0 no (the call would be refused), 1 yes,
- * 2 yes and it is expected to beat one launch per step (up to 96 rows). No error is set. */
+ * 2 yes and it is expected to beat one launch of dali_hip_lstm_step per step (up to 32 rows; up to 48 from 1024 hidden units on). No error is set. */
 int dali_hip_lstm_recurrent_persistent_supported(int batch, int hidden);
 
 /*

@@ -1949,8 +1949,9 @@ def test_arange_diag_outer(gpu, D, rng):
 
 @pytest.mark.parametrize("B,I,H", [(1, 256, 256), (8, 1024, 1024), (17, 512, 512), (40, 768, 768), (64, 1024, 1024), (5, 256, 512), (33, 960, 1024)])
 def test_lstm_step_at_small_batches(gpu, D, O, rng, B, I, H):
-    """Up to 64 rows the step runs on 16-row tiles with one workgroup per compute unit (dali_hip_lstm_step_small) instead of
-    the 64-row tiles of the general kernel: same definition (lstm.cpp:226-261), the products summed in another order."""
+    """Up to 16 rows (up to 64 where input != hidden, which the fused step does not take) the step runs on 16-row tiles with one
+    workgroup per compute unit (dali_hip_lstm_step_small); from 17 rows on the fused step, its inner extent cut into one share
+    per compute unit. Same definition (lstm.cpp:226-261), the products summed in another order."""
     import os
     op = D.op
     X, Hp, Cp = (rng.randn(B, n).astype(np.float32) for n in (I, H, H))
@@ -1962,7 +1963,8 @@ def test_lstm_step_at_small_batches(gpu, D, O, rng, B, I, H):
     with D.Recording() as rec:
         cn, hn = op.lstm_step(*dev)
     after = D.jit_stats()
-    assert after["gemms"] - before["gemms"] == 1 and after["kernels"] == before["kernels"] and D.last_kernel_kinds() == "lstm_small"
+    expected = "lstm_fused" if (I == H and B > 16) else "lstm_small"
+    assert after["gemms"] - before["gemms"] == 1 and after["kernels"] == before["kernels"] and D.last_kernel_kinds() == expected
     _, ocn, ohn = O.lstm_step(X, Hp, Cp, W, U, b)
     close(cn.numpy(), ocn, rtol=1e-4, atol=1e-5)
     close(hn.numpy(), ohn, rtol=1e-4, atol=1e-5)
@@ -1991,13 +1993,19 @@ def test_lstm_step_at_small_batches(gpu, D, O, rng, B, I, H):
     assert hip.dali_hip_lstm_step_small(B, I, H, ptrs[0], I + 8, ptrs[1], H + 4, ptrs[2], ptrs[3], 4 * H, ptrs[4], 4 * H, ptrs[5], ptrs[6], ptrs[7]) == 0, hip.dali_hip_last_error()
     out = np.empty((B, H), np.float32)
     hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), ptrs[7], out.nbytes)
-    assert np.array_equal(out, first[1])
+    if expected == "lstm_small":
+        assert np.array_equal(out, first[1])
+    else:  # the front-end took the fused step: the same sums in another order
+        close(out, first[1], rtol=2e-5, atol=2e-6)
+        close(out, ohn, rtol=1e-4, atol=1e-5)
     assert hip.dali_hip_lstm_step_small(65, I, H, *ptrs[:2][:1], I + 8, ptrs[1], H + 4, ptrs[2], ptrs[3], 4 * H, ptrs[4], 4 * H, ptrs[5], ptrs[6], ptrs[7]) != 0
     for p in ptrs:
         hip.dali_hip_free(p)
 
 
-@pytest.mark.parametrize("B,H", [(64, 64), (256, 128), (100, 192), (7, 192), (256, 1024)])
+@pytest.mark.parametrize("B,H", [(64, 64), (256, 128), (100, 192), (7, 192), (256, 1024),
+                                 # batches whose tiles leave compute units idle: both forms cut the inner extent into the same shares
+                                 (128, 1024), (96, 512), (72, 1024), (130, 448)])
 def test_fused_lstm_step_equals_the_two_launch_form(gpu, D, O, rng, B, H):
     """input == hidden, multiples of 64: the gate arithmetic runs in the GEMM epilogue (one launch) and must give
     what the GEMM pair followed by the generated gate kernel gives."""
@@ -2075,8 +2083,18 @@ def test_lstm_sequence_in_one_persistent_launch(gpu, D, O, rng, T, B, I, H):
     U = rng.uniform(-lim, lim, (H, 4 * H)).astype(np.float32)
     b = (rng.randn(4 * H) * 0.1).astype(np.float32)
     dev = [arr(D, v) for v in (Xs, H0, C0, W, U, b)]
-    with D.Recording() as rec:
-        hs, c_last, h_last = D.op.lstm_sequence(*dev)
+    # what the front-end chooses by itself: the persistent launch where it beats a launch of the fused step per step (up to 32
+    # rows, 48 from 1024 hidden units on), and up to 96 rows where the fused step does not apply (input size != hidden size)
+    import os
+    D.op.lstm_sequence(*dev)
+    by_itself = D.last_kernel_kinds() == "lstm_persistent"
+    assert by_itself == (B <= 32 or (B <= 48 and H >= 1024) or (I != H and B <= 96))
+    os.environ["DALI_HIP_LSTM_PERSISTENT"] = "2"  # here: wherever the kernels serve the size
+    try:
+        with D.Recording() as rec:
+            hs, c_last, h_last = D.op.lstm_sequence(*dev)
+    finally:
+        os.environ.pop("DALI_HIP_LSTM_PERSISTENT")
     assert D.last_kernel_kinds() == "lstm_persistent"
     assert hs.shape == (T, B, H) and np.array_equal(h_last.numpy(), hs.numpy()[-1])
     ohs, oc = lstm_sequence_truth(O, Xs, H0, C0, W, U, b)
@@ -2123,7 +2141,7 @@ def test_persistent_recurrence_through_the_c_abi(gpu, O, rng, T, B, H):
         close(hs, ohs, rtol=2e-4, atol=2e-5)
         close(c, oc, rtol=2e-4, atol=2e-5)
     # what is served: up to 128 rows, hidden sizes that are multiples of 64 up to 2048 (2: expected to beat a launch per step)
-    assert hip.dali_hip_lstm_recurrent_persistent_supported(B, H) == (2 if B <= 96 else 1)
+    assert hip.dali_hip_lstm_recurrent_persistent_supported(B, H) == (2 if B <= 32 or (B <= 48 and H >= 1024) else 1)
     assert hip.dali_hip_lstm_recurrent_persistent_supported(129, 1024) == 0 and hip.dali_hip_lstm_recurrent_persistent_supported(8, 96) == 0
     assert hip.dali_hip_lstm_recurrent_persistent_supported(8, 2112) == 0 and hip.dali_hip_lstm_recurrent_persistent_supported(128, 2048) == 1
     # refused: more than 128 rows, a hidden size without a kernel, a leading dimension below the row, hs on top of h0
@@ -2157,7 +2175,8 @@ def test_persistent_lstm_barrier_gives_up_instead_of_hanging(B):
         "print('AFTER', float(D.op.sum(x * 2.0).numpy()))\n"
     )
     # (the kernel with row blocks looks at a barrier that has usually completed by then: a limit of zero makes its first wait give up unseen)
-    env = dict(os.environ, DALI_HIP_PERSISTENT_SPIN_LIMIT="0" if B > 64 else "1", PYTHONPATH=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    # (DALI_HIP_LSTM_PERSISTENT=2: the persistent launch also at 80 rows, where the front-end would take a launch per step)
+    env = dict(os.environ, DALI_HIP_PERSISTENT_SPIN_LIMIT="0" if B > 64 else "1", DALI_HIP_LSTM_PERSISTENT="2", PYTHONPATH=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
     assert out.returncode == 0, out.stderr[-2000:]
     assert "SYNC 1" in out.stdout and "gave up waiting at a grid barrier" in out.stdout, out.stdout
