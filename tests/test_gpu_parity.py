@@ -1755,6 +1755,31 @@ def test_cabi_argsort_is_stable(gpu, rng, n):
         hip.dali_hip_free(p)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 1024, 8192), (1536, 1536, 2048), (3072, 1536, 1024), (2048, 2048, 512)])
+def test_graph_replays_of_products_cut_into_shares(gpu, D, rng, M, N, K):
+    """Products whose tiles meet in the library workspace (shares of the inner extent published, a ticket per tile, the last
+    one adds them up) captured into a HIP graph: every replay, with eager work and synchronisations between the replays, gives
+    the bits of the eager evaluation, and the tickets are back at rest afterwards."""
+    a, b = (arr(D, rng.randn(*shp).astype(np.float32)) for shp in ((M, K), (K, N)))
+    b_by_columns = b.transpose().ascontiguousarray()  # [N, K] in memory: the product below reads its right operand against its rows
+    with D.Recording() as rec:
+        c = D.op.dot(a, b)
+        c.eval()
+        ct = D.op.dot(a, b_by_columns.transpose())
+        ct.eval()
+    first, first_t = c.numpy().copy(), ct.numpy().copy()
+    want = a.numpy().astype(np.float64) @ b.numpy().astype(np.float64)
+    close(first, want, rtol=1e-4, atol=1e-4 * np.abs(want).max())
+    close(first_t, want, rtol=1e-4, atol=1e-4 * np.abs(want).max())
+    rec.make_graph()
+    for i in range(3):
+        rec.replay(1)
+        assert np.array_equal(c.numpy(), first) and np.array_equal(ct.numpy(), first_t)
+        # eager work that uses the same tickets and partial sums in between
+        assert np.isclose(float(D.op.sum(a).numpy()), a.numpy().astype(np.float64).sum(), rtol=1e-4, atol=1e-2)
+        assert np.array_equal(D.op.dot(a, b).numpy(), first)
+
+
 def test_graphs_refuse_what_would_allocate_and_memory_calls_refuse_a_capture(gpu, D, O, rng):
     """A recording whose replay takes temporary blocks from the bank (an index ordering of more than 16384 keys, a top_k by
     sorting) cannot become a graph: the block addresses would be baked into it while the bank hands the blocks to others.
