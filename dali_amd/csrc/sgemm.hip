@@ -867,10 +867,24 @@ static int device_cus() {
 // item per compute unit, at least four slabs each; below 2 the product is not cut
 static int stream_shares(long tiles64, int nslab64) {
     const int cus = device_cus();
-    if (cus <= 0 || tiles64 <= 0 || tiles64 > cus / 2) return 1;
-    int shares = (int)(cus / tiles64);
-    if (shares > nslab64 / 4) shares = nslab64 / 4;
-    return shares < 1 ? 1 : shares;
+    if (cus <= 0 || tiles64 <= 0 || tiles64 >= cus || nslab64 < 8) return 1;
+    // Estimated time in units of one slab (about 1.1 us): rounds x (slabs of a share + what a cut costs: publishing the share,
+    // the ticket and the fetch by whoever adds the shares up, 5 slab times and 0.15 more per share; measured on [64,64] over
+    // K = 65536 and on the LSTM shapes). The cut has to win a tenth to be made.
+    const int most = nslab64 / 4 < 256 ? nslab64 / 4 : 256;
+    int best = 1;
+    double best_time = (double)nslab64;
+    for (int sh = 2; sh <= most; ++sh) {
+        const long items = tiles64 * sh;
+        if (items > 2048) break;  // 16 KiB of partial sums each in the 32 MiB workspace
+        const long rounds = (items + cus - 1) / cus;
+        const double t = (double)rounds * ((double)nslab64 / sh + 5.0 + 0.15 * sh);
+        if (t < best_time) {
+            best = sh;
+            best_time = t;
+        }
+    }
+    return best_time <= 0.9 * nslab64 ? best : 1;
 }
 
 // The whole slabs of a product of one or two terms through the streaming kernel, what is left of the inner extents by a
@@ -1046,6 +1060,16 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
     long tiles64 = (long)((M + 63) / 64) * ((N + 63) / 64);
     static const int split_env = getenv("DALI_HIP_GEMM_SPLITK") ? atoi(getenv("DALI_HIP_GEMM_SPLITK")) : 0;
     int split_k = split_env > 0 ? split_env : 1;
+    if (split_env == 0 && variant == 0 && stream_env == 0 && stream_fits && tiles64 > 128) {
+        // between half a round and a whole one of 64x64 tiles: shares that fill whole rounds (384x1536 over K = 4096, 144 tiles: 66 -> 58 us)
+        int nslab64 = 0;
+        for (int s = 0; s < g.nseg; ++s) nslab64 += (g.seg[s].K + 63) / 64;
+        const int shares = stream_shares(tiles64, nslab64);
+        if (shares >= 2) {
+            const int st = stream_product(g, ta, tb, shares);
+            if (st >= 0) return st;
+        }
+    }
     if (split_env == 0 && variant == 0 && tiles64 <= 128) {
         // A few tiles over a long inner extent (the weight gradient of a convolution: [out, window] from tens of
         // thousands of patches) would leave most of the device idle: about two workgroups per CU, folded in a fixed
