@@ -65,11 +65,12 @@ struct DmaArgs {
 __device__ __forceinline__ void dma16(unsigned lds_addr, unsigned voff, const char* base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
 }
-// the same for a base pointer that the compiler cannot prove to be the same in every lane (it is)
-__device__ __forceinline__ void dma16_uniform(unsigned lds_addr, unsigned voff, const char* base) {
-    const unsigned long long b = (unsigned long long)base;
+// A pointer that is the same in every lane, said so where the compiler cannot prove it (a pointer chosen per work item): what is
+// computed from it afterwards stays on the scalar unit.
+__device__ __forceinline__ const char* wave_uniform(const char* p) {
+    const unsigned long long b = (unsigned long long)p;
     const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b), hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
-    dma16(lds_addr, voff, (const char*)(((unsigned long long)hi << 32) | lo));
+    return (const char*)(((unsigned long long)hi << 32) | lo);
 }
 // The compiler does not see these loads, so the waits for them are written out; they are also compiler barriers.
 __device__ __forceinline__ void wait_loads_but_4() { asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); }
@@ -460,14 +461,14 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_stream_kernel(StreamArgs g) 
         i_n = share_begin(z + 1) - i_g;
         i_fj = 0;
         const bool second = i_g >= slabs0;  // (only with two terms; shares are cut from single products)
-        ap = (const char*)(second ? g.A[1] : g.A[0]) + (long)(i_g - (second ? slabs0 : 0)) * a_step;
-        bp = (const char*)(second ? g.B[1] : g.B[0]) + (long)(i_g - (second ? slabs0 : 0)) * b_step;
+        ap = wave_uniform((const char*)(second ? g.A[1] : g.A[0]) + (long)(i_g - (second ? slabs0 : 0)) * a_step);
+        bp = wave_uniform((const char*)(second ? g.B[1] : g.B[0]) + (long)(i_g - (second ? slabs0 : 0)) * b_step);
     };
     auto issue = [&](int stage) __attribute__((always_inline)) {
-        dma16_uniform(a_dst[0] + stage * kStage, a_off[0], ap);
-        dma16_uniform(a_dst[1] + stage * kStage, a_off[1], ap);
-        dma16_uniform(b_dst[0] + stage * kStage, b_off[0], bp);
-        dma16_uniform(b_dst[1] + stage * kStage, b_off[1], bp);
+        dma16(a_dst[0] + stage * kStage, a_off[0], ap);
+        dma16(a_dst[1] + stage * kStage, a_off[1], ap);
+        dma16(b_dst[0] + stage * kStage, b_off[0], bp);
+        dma16(b_dst[1] + stage * kStage, b_off[1], bp);
         ++i_fj;
         ++i_g;
         ap += a_step;

@@ -57,13 +57,16 @@ struct Args128 {
 };
 
 // One 16-byte piece per lane from global memory straight into LDS: lane l writes bytes [16 l, 16 l + 16) behind `lds_addr`
-// (wave-uniform, goes through M0); the source is base + voff. The base is made a scalar by hand: the compiler cannot prove
-// that a pointer which changes with the work item is the same in every lane.
+// (wave-uniform, goes through M0); the source is base + voff, base in scalar registers.
 __device__ __forceinline__ void load_to_lds(unsigned lds_addr, unsigned voff, const char* base) {
-    const unsigned long long b = (unsigned long long)base;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+// A pointer that is the same in every lane, said so where the compiler cannot prove it (a pointer chosen per work item): what is
+// computed from it afterwards stays on the scalar unit.
+__device__ __forceinline__ const char* wave_uniform(const char* p) {
+    const unsigned long long b = (unsigned long long)p;
     const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b), hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
-    const char* sbase = (const char*)(((unsigned long long)hi << 32) | lo);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+    return (const char*)(((unsigned long long)hi << 32) | lo);
 }
 // The compiler does not see these loads, so the waits for them are written out; they are also compiler barriers.
 template <int N>
@@ -191,8 +194,8 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
             }
         }
         i_j = j0;
-        ap = (const char*)g.A + (long)j0 * a_step;
-        bp = (const char*)g.B + (long)j0 * b_step;
+        ap = wave_uniform((const char*)g.A + (long)j0 * a_step);
+        bp = wave_uniform((const char*)g.B + (long)j0 * b_step);
     };
     auto issue = [&](int stage) __attribute__((always_inline)) {
         load_to_lds(a_dst[0] + stage * kStageBytes, a_off[0], ap);
