@@ -428,6 +428,59 @@ def test_sgemm_random_shapes_around_the_kernel_boundaries(gpu):
             hip.dali_hip_free(p)
 
 
+def test_sgemm_random_shapes_for_the_kernels_that_walk_work_items(gpu):
+    """Random products with operands the loads can write straight into LDS (aligned rows), drawn where the choice between the
+    kernels changes: few 64x64 tiles over a long inner extent (shares of the inner extent, one work item per compute unit),
+    under-filled rounds of 64x64 tiles, many 128x128 tiles with and without a last round that is cut into shares, inner
+    extents with a rest beyond whole slabs, all four operand orders, alpha / beta, NaN in every padding; every element against
+    the product in double precision, and the same bits when the product is repeated."""
+    hip = gpu
+    rng = np.random.RandomState(777)
+    pick = lambda values: int(values[rng.randint(len(values))])
+    for case in range(36):
+        kind = case % 4
+        if kind == 0:    # few tiles, long inner extent
+            M, N, K = pick([64, 100, 128, 256, 320]), pick([64, 192, 576, 1024]), pick([2048, 4100, 8192, 20032])
+        elif kind == 1:  # between half a round and a round of 64x64 tiles, and a little more than whole rounds of 128x128 tiles
+            M, N, K = pick([384, 768, 1100]), pick([1536, 2052, 4096]), pick([1024, 2048, 2080])
+        elif kind == 2:  # many 128x128 tiles
+            M, N, K = pick([1536, 2052, 3072, 4100]), pick([1536, 2048, 2304]), pick([96, 256, 548, 2048])
+        else:            # wide and short
+            M, N, K = pick([256, 640, 1024]), pick([16000, 24704, 32000]), pick([64, 160, 256])
+        ta, tb = int(rng.randint(2)), int(rng.randint(2))
+        if ta:
+            M = (M + 3) // 4 * 4
+        if not tb:
+            N = (N + 3) // 4 * 4
+        alpha, beta = float(rng.choice([1.0, 0.75, -2.0])), float(rng.choice([0.0, 0.0, 1.0, -0.5]))
+        A = rng.randn(M, K).astype(np.float32)
+        B = rng.randn(K, N).astype(np.float32)
+        Ast, Bst = (A.T if ta else A), (B.T if tb else B)
+        lda, ldb, ldc = Ast.shape[1] + 4 * int(rng.randint(0, 3)), Bst.shape[1] + 4 * int(rng.randint(0, 3)), N + 2 * int(rng.randint(0, 3))
+        Ap = np.full((Ast.shape[0], lda), np.nan, np.float32); Ap[:, :Ast.shape[1]] = Ast
+        Bp = np.full((Bst.shape[0], ldb), np.nan, np.float32); Bp[:, :Bst.shape[1]] = Bst
+        C0 = rng.randn(M, ldc).astype(np.float32)
+        if beta == 0.0:
+            C0[:, :N] = np.nan
+        dA, dB, dC = _dev(hip, Ap), _dev(hip, Bp), _dev(hip, C0)
+        what = "case %d: M=%d N=%d K=%d ta=%d tb=%d lda=%d ldb=%d ldc=%d alpha=%g beta=%g" % (case, M, N, K, ta, tb, lda, ldb, ldc, alpha, beta)
+        prod = A.astype(np.float64) @ B.astype(np.float64)
+        want = alpha * prod + (beta * C0[:, :N] if beta != 0.0 else 0.0)
+        scale = np.abs(alpha) * (np.abs(A).astype(np.float64) @ np.abs(B)).max() + np.abs(want).max() + 1e-6
+        outs = []
+        for _ in range(2):
+            hip.dali_hip_memcpy_h2d(dC, C0.ctypes.data_as(C.c_void_p), C0.nbytes)
+            assert hip.dali_hip_sgemm(tb, ta, N, M, K, alpha, dB, ldb, dA, lda, beta, dC, ldc) == 0, what + ": " + hip.dali_hip_last_error().decode()
+            out = np.empty_like(C0)
+            hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+            assert np.abs(out[:, :N] - want).max() <= 2e-6 * scale * max(1.0, np.sqrt(K) / 8), what
+            assert np.array_equal(out[:, N:], C0[:, N:]), what  # padding untouched
+            outs.append(out[:, :N].copy())
+        assert np.array_equal(outs[0], outs[1]), what
+        for p in (dA, dB, dC):
+            hip.dali_hip_free(p)
+
+
 @pytest.mark.parametrize("M,N,K", [(1024, 32000, 8), (100, 300, 64), (64, 256, 1), (130, 1000, 33), (512, 4099, 17), (2048, 8192, 48)])
 @pytest.mark.parametrize("ta", [1, 0])
 def test_sgemm_with_a_short_inner_extent(gpu, rng, M, N, K, ta):
