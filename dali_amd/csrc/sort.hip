@@ -11,8 +11,6 @@
 #include <cstdlib>
 #include <type_traits>
 
-#include <hipcub/hipcub.hpp>
-
 namespace dali_hip {
 
 // A few thousand keys: counting ranks beats any multi-pass sort. The final position of key i is the number of
@@ -99,16 +97,37 @@ __global__ __launch_bounds__(256) void rank_sort_kernel(const int32_t* keys, int
 // short ones so that the tiles still cover the chip (65536 keys in tiles of 2048 are 32 workgroups on 256 CUs).
 constexpr int kRadixMaxTile = 2048;
 
-// With a key limit, every key outside [0, limit) takes the digits of `limit` itself: such keys (invalid indices) end up behind all
-// valid ones, in input order, instead of between the keys that share their low bits.
-__device__ __forceinline__ unsigned int radix_digit(int32_t key, int shift, unsigned int flip, unsigned int limit) {
-    unsigned int k = (unsigned int)key ^ flip;
-    if (limit != 0u && k > limit) k = limit;
-    return (k >> shift) & 255u;
-}
+// Where a pair's digit comes from. The sort itself only needs "the digit of pair i in this pass":
+// IndexDigits: int32 keys. With a key limit, every key outside [0, limit) takes the digits of `limit` itself: such keys (invalid
+// indices) end up behind all valid ones, in input order, instead of between the keys that share their low bits.
+struct IndexDigits {
+    unsigned int flip, limit;
+    __device__ __forceinline__ unsigned int operator()(int32_t key, int32_t, int shift) const {
+        unsigned int k = (unsigned int)key ^ flip;
+        if (limit != 0u && k > limit) k = limit;
+        return (k >> shift) & 255u;
+    }
+};
+// WordDigits: unsigned keys ordered as they stand (values of any type mapped to words of the same order beforehand)
+struct WordDigits {
+    template <typename KEY>
+    __device__ __forceinline__ unsigned int operator()(KEY key, int32_t, int shift) const {
+        return (unsigned int)(key >> shift) & 255u;
+    }
+};
+// RowDigits: the row of a [rows, cols] matrix that the pair started in (its position / cols): stable passes over these
+// digits after the passes over the keys leave every row's pairs together, in key order. The keys are not looked at.
+struct RowDigits {
+    int cols;
+    template <typename KEY>
+    __device__ __forceinline__ unsigned int operator()(KEY, int32_t pos, int shift) const {
+        return ((unsigned int)(pos / cols) >> shift) & 255u;
+    }
+};
 
-template <int ROUNDS>
-__global__ __launch_bounds__(256) void radix_hist_kernel(const int32_t* keys, int n, int shift, unsigned int flip, unsigned int limit, unsigned int* hist, int tiles) {
+// keys == nullptr: the digits come from the positions alone; pos_in == nullptr: a pair's position is its index
+template <int ROUNDS, typename KEY, typename DIGITS>
+__global__ __launch_bounds__(256) void radix_hist_kernel(const KEY* keys, const int32_t* pos_in, int n, int shift, DIGITS digits, unsigned int* hist, int tiles) {
     __shared__ unsigned int h[256];
     h[threadIdx.x] = 0u;
     __syncthreads();
@@ -116,7 +135,7 @@ __global__ __launch_bounds__(256) void radix_hist_kernel(const int32_t* keys, in
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r) {
         const long i = base + r * 256 + threadIdx.x;
-        if (i < n) atomicAdd(&h[radix_digit(keys[i], shift, flip, limit)], 1u);
+        if (i < n) atomicAdd(&h[digits(keys ? keys[i] : (KEY)0, pos_in ? pos_in[i] : (int32_t)i, shift)], 1u);
     }
     __syncthreads();
     hist[(long)threadIdx.x * tiles + blockIdx.x] = h[threadIdx.x];
@@ -155,9 +174,9 @@ __global__ __launch_bounds__(256) void radix_row_scan_kernel(unsigned int* hist,
     if (threadIdx.x == 0) totals[blockIdx.x] = carry;
 }
 
-template <int ROUNDS>
-__global__ __launch_bounds__(256) void radix_move_kernel(const int32_t* keys_in, const int32_t* pos_in, int n, int shift, unsigned int flip, unsigned int limit, const unsigned int* hist,
-                                                         const unsigned int* totals, int tiles, int32_t* keys_out, int32_t* pos_out) {
+template <int ROUNDS, typename KEY, typename DIGITS>
+__global__ __launch_bounds__(256) void radix_move_kernel(const KEY* keys_in, const int32_t* pos_in, int n, int shift, DIGITS digits, const unsigned int* hist,
+                                                         const unsigned int* totals, int tiles, KEY* keys_out, int32_t* pos_out) {
     __shared__ unsigned short cnt[ROUNDS * 4][256];
     __shared__ unsigned int first_slot[256];
     __shared__ unsigned int wave_total[4];
@@ -183,15 +202,16 @@ __global__ __launch_bounds__(256) void radix_move_kernel(const int32_t* keys_in,
     __syncthreads();
     const unsigned long long below = (1ull << lane) - 1ull;
     const long base = (long)blockIdx.x * (256 * ROUNDS);
-    int32_t key[ROUNDS], pos[ROUNDS];
+    KEY key[ROUNDS];
+    int32_t pos[ROUNDS];
     unsigned int digit[ROUNDS], rank[ROUNDS];
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r) {
         const long i = base + r * 256 + threadIdx.x;
         const bool valid = i < n;
-        key[r] = valid ? keys_in[i] : 0;
+        key[r] = valid && keys_in ? keys_in[i] : (KEY)0;
         pos[r] = valid ? (pos_in ? pos_in[i] : (int32_t)i) : 0;
-        digit[r] = radix_digit(key[r], shift, flip, limit);
+        digit[r] = digits(key[r], pos[r], shift);
         unsigned long long same = __ballot(valid);
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
@@ -217,37 +237,87 @@ __global__ __launch_bounds__(256) void radix_move_kernel(const int32_t* keys_in,
         const long i = base + r * 256 + threadIdx.x;
         if (i < n) {
             const unsigned int dst = first_slot[digit[r]] + cnt[r * 4 + wave][digit[r]] + rank[r];
-            keys_out[dst] = key[r];
+            if (keys_in) keys_out[dst] = key[r];
             pos_out[dst] = pos[r];
         }
     }
 }
 
+// One pass of the radix sort over n pairs in tiles of 256 * rounds: histogram, scan, move (see above)
+template <typename KEY, typename DIGITS>
+static void radix_pass(int rounds, const KEY* src_keys, const int32_t* src_pos, int n, int shift, DIGITS digits, unsigned int* hist, unsigned int* totals, int tiles,
+                       KEY* dst_keys, int32_t* dst_pos, hipStream_t st) {
+    auto pass = [&](auto hist_kernel, auto move_kernel) {
+        hipLaunchKernelGGL(hist_kernel, dim3(tiles), dim3(256), 0, st, src_keys, src_pos, n, shift, digits, hist, tiles);
+        hipLaunchKernelGGL(radix_row_scan_kernel, dim3(256), dim3(256), 0, st, hist, tiles, totals);
+        hipLaunchKernelGGL(move_kernel, dim3(tiles), dim3(256), 0, st, src_keys, src_pos, n, shift, digits, (const unsigned int*)hist, (const unsigned int*)totals, tiles,
+                           dst_keys, dst_pos);
+    };
+    switch (rounds) {
+        case 1: pass(radix_hist_kernel<1, KEY, DIGITS>, radix_move_kernel<1, KEY, DIGITS>); break;
+        case 2: pass(radix_hist_kernel<2, KEY, DIGITS>, radix_move_kernel<2, KEY, DIGITS>); break;
+        case 4: pass(radix_hist_kernel<4, KEY, DIGITS>, radix_move_kernel<4, KEY, DIGITS>); break;
+        default: pass(radix_hist_kernel<8, KEY, DIGITS>, radix_move_kernel<8, KEY, DIGITS>); break;
+    }
+}
+
+// tile height for n pairs: 8 rounds for long inputs, fewer while the tiles would not cover the chip
+static int radix_rounds(long n) {
+    int rounds = kRadixMaxTile / 256;
+    while (rounds > 1 && n / (256 * rounds) < 1024) rounds /= 2;
+    return rounds;
+}
+
 // ---------------------------------------------------------------- ordering along rows (top_k / bottom_k / argsort)
-// Keys of one dense [rows, cols] matrix are copied into a sort buffer beside their column numbers. -0.0 becomes +0.0
-// so that the two compare equal, as they do for the reference's comparators; with `reverse` a row is laid out back to
-// front, so that the stable sort which follows leaves equal keys in descending column order.
+// The values of one dense [rows, cols] matrix become unsigned words whose ascending order is the order asked for: the
+// value's bits with the sign bit set for non-negative numbers and all bits inverted for negative ones (two's complement
+// integers: the sign bit flipped), everything inverted once more when the largest come first. -0.0 becomes +0.0 first,
+// so that the two compare equal, as they do for the reference's comparators. With `reverse` a row is laid out back to
+// front, so that the stable sort which follows leaves equal keys in descending column order. The whole matrix is then
+// sorted as one sequence by word (stable passes, lowest digit first) and after that by the row a pair started in: every
+// row's pairs end up together and in order.
 template <typename T>
-__global__ __launch_bounds__(256) void row_keys_kernel(const T* x, long total, int cols, int reverse, T* keys, int32_t* columns) {
+struct OrderedWord;
+template <>
+struct OrderedWord<float> {
+    typedef unsigned int type;
+    static __device__ __forceinline__ type of(float v) {
+        const unsigned int b = __float_as_uint(v + 0.f);
+        return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+    }
+};
+template <>
+struct OrderedWord<double> {
+    typedef unsigned long long type;
+    static __device__ __forceinline__ type of(double v) {
+        const unsigned long long b = (unsigned long long)__double_as_longlong(v + 0.0);
+        return (b >> 63) ? ~b : (b | 0x8000000000000000ull);
+    }
+};
+template <>
+struct OrderedWord<int32_t> {
+    typedef unsigned int type;
+    static __device__ __forceinline__ type of(int32_t v) { return (unsigned int)v ^ 0x80000000u; }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void row_words_kernel(const T* x, long total, int cols, int reverse, int largest, typename OrderedWord<T>::type* words) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const long row = i / cols;
     const int col = (int)(i - row * cols);
     const int src = reverse ? cols - 1 - col : col;
-    keys[i] = x[row * cols + src] + (T)0;
-    columns[i] = src;
+    const typename OrderedWord<T>::type w = OrderedWord<T>::of(x[row * cols + src]);
+    words[i] = largest ? ~w : w;
 }
 
-__global__ __launch_bounds__(256) void row_offsets_kernel(int32_t* offsets, int rows, int cols) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i <= rows) offsets[i] = i * cols;
-}
-
-__global__ __launch_bounds__(256) void leading_columns_kernel(const int32_t* in, long total, int cols, int k, int32_t* out) {
+// The first k positions of every sorted row, as column numbers of the input
+__global__ __launch_bounds__(256) void leading_columns_kernel(const int32_t* pos, long total, int cols, int k, int reverse, int32_t* out) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const long row = i / k;
-    out[i] = in[row * cols + (i - row * k)];
+    const int col = pos[row * cols + (i - row * k)] - (int)(row * cols);
+    out[i] = reverse ? cols - 1 - col : col;
 }
 
 // A few best entries of long rows: selection instead of a sort. One workgroup per row, read once, coalesced. Every wave
@@ -504,49 +574,47 @@ int topk_rows(const void* x, int rows, int cols, int k, bool largest, bool ties_
         if (le != hipSuccess) return fail("row selection launch failed: %s", hipGetErrorString(le));
         return DALI_HIP_OK;
     }
-    const long total = (long)rows * cols;
-    const size_t key_bytes = (size_t)total * sizeof(T), col_bytes = (size_t)total * sizeof(int32_t), off_bytes = ((size_t)rows + 1) * sizeof(int32_t);
-    void *keys = nullptr, *keys_sorted = nullptr, *columns = nullptr, *columns_sorted = nullptr, *offsets = nullptr, *temp = nullptr;
-    size_t temp_bytes = 0;
+    // the whole matrix as one stable sort: by word, then by row
+    typedef typename OrderedWord<T>::type W;
+    const int total = rows * cols;  // (the caller has checked that it fits)
+    const int rounds = radix_rounds(total), tiles = (total + 256 * rounds - 1) / (256 * rounds);
+    int row_bits = 0;
+    while (row_bits < 31 && (1 << row_bits) < rows) ++row_bits;
+    const int key_passes = (int)sizeof(W), row_passes = (row_bits + 7) / 8;
+    const size_t word_bytes = (size_t)total * sizeof(W), pos_bytes = (size_t)total * sizeof(int32_t), hist_bytes = ((size_t)256 * tiles + 256) * sizeof(unsigned int);
+    void *words[2] = {nullptr, nullptr}, *pos[2] = {nullptr, nullptr}, *hist = nullptr;
     int status = DALI_HIP_OK;
-    if (dali_hip_bank_allocate(&keys, key_bytes) || dali_hip_bank_allocate(&keys_sorted, key_bytes) || dali_hip_bank_allocate(&columns, col_bytes) ||
-        dali_hip_bank_allocate(&offsets, off_bytes) || (k < cols && dali_hip_bank_allocate(&columns_sorted, col_bytes)))
+    if (dali_hip_bank_allocate(&words[0], word_bytes) || dali_hip_bank_allocate(&words[1], word_bytes) || dali_hip_bank_allocate(&pos[0], pos_bytes) ||
+        dali_hip_bank_allocate(&pos[1], pos_bytes) || dali_hip_bank_allocate(&hist, hist_bytes))
         status = DALI_HIP_ERROR;
-    int32_t* sorted_columns = k < cols ? (int32_t*)columns_sorted : out;
     if (status == DALI_HIP_OK) {
-        hipLaunchKernelGGL(row_keys_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (const T*)x, total, cols,
-                           ties_by_descending_column ? 1 : 0, (T*)keys, (int32_t*)columns);
-        hipLaunchKernelGGL(row_offsets_kernel, dim3((unsigned)(rows / 256 + 1)), dim3(256), 0, st, (int32_t*)offsets, rows, cols);
-        auto sort = [&](void* t) {
-            const int32_t* off = (const int32_t*)offsets;
-            return largest ? hipcub::DeviceSegmentedRadixSort::SortPairsDescending(t, temp_bytes, (const T*)keys, (T*)keys_sorted, (const int32_t*)columns,
-                                                                                    sorted_columns, (int)total, rows, off, off + 1, 0, (int)sizeof(T) * 8, st)
-                           : hipcub::DeviceSegmentedRadixSort::SortPairs(t, temp_bytes, (const T*)keys, (T*)keys_sorted, (const int32_t*)columns,
-                                                                          sorted_columns, (int)total, rows, off, off + 1, 0, (int)sizeof(T) * 8, st);
-        };
-        hipError_t e = sort(nullptr);
-        if (e != hipSuccess) {
-            status = fail("row sort sizing failed: %s", hipGetErrorString(e));
-        } else if (dali_hip_bank_allocate(&temp, temp_bytes ? temp_bytes : 4)) {
-            status = DALI_HIP_ERROR;
-        } else if ((e = sort(temp)) != hipSuccess) {
-            status = fail("row sort failed: %s", hipGetErrorString(e));
-        } else if (k < cols) {
-            const long kept = (long)rows * k;
-            hipLaunchKernelGGL(leading_columns_kernel, dim3((unsigned)((kept + 255) / 256)), dim3(256), 0, st, (const int32_t*)columns_sorted, kept, cols, k, out);
+        unsigned int* h = (unsigned int*)hist;
+        unsigned int* totals = h + (size_t)256 * tiles;
+        hipLaunchKernelGGL(row_words_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (const T*)x, (long)total, cols,
+                           ties_by_descending_column ? 1 : 0, largest ? 1 : 0, (W*)words[0]);
+        int from = 0;
+        const int32_t* src_pos = nullptr;  // first pass: a pair's position is its index
+        for (int i = 0; i < key_passes; ++i) {
+            radix_pass<W, WordDigits>(rounds, (const W*)words[from], src_pos, total, 8 * i, WordDigits(), h, totals, tiles, (W*)words[1 - from], (int32_t*)pos[1 - from], st);
+            from = 1 - from;
+            src_pos = (const int32_t*)pos[from];
         }
-        if (status == DALI_HIP_OK) {
-            hipError_t le = hipGetLastError();
-            if (le != hipSuccess) status = fail("row sort launch failed: %s", hipGetErrorString(le));
+        for (int i = 0; i < row_passes; ++i) {
+            radix_pass<W, RowDigits>(rounds, (const W*)nullptr, src_pos, total, 8 * i, RowDigits{cols}, h, totals, tiles, (W*)nullptr, (int32_t*)pos[1 - from], st);
+            from = 1 - from;
+            src_pos = (const int32_t*)pos[from];
         }
+        const long kept = (long)rows * k;
+        hipLaunchKernelGGL(leading_columns_kernel, dim3((unsigned)((kept + 255) / 256)), dim3(256), 0, st, src_pos, kept, cols, k, ties_by_descending_column ? 1 : 0, out);
+        hipError_t le = hipGetLastError();
+        if (le != hipSuccess) status = fail("row sort launch failed: %s", hipGetErrorString(le));
     }
     // back to the bank at once: their next user is ordered behind these launches on the stream
-    if (temp) dali_hip_bank_deposit(temp, temp_bytes ? temp_bytes : 4);
-    if (columns_sorted) dali_hip_bank_deposit(columns_sorted, col_bytes);
-    if (offsets) dali_hip_bank_deposit(offsets, off_bytes);
-    if (columns) dali_hip_bank_deposit(columns, col_bytes);
-    if (keys_sorted) dali_hip_bank_deposit(keys_sorted, key_bytes);
-    if (keys) dali_hip_bank_deposit(keys, key_bytes);
+    if (hist) dali_hip_bank_deposit(hist, hist_bytes);
+    if (pos[1]) dali_hip_bank_deposit(pos[1], pos_bytes);
+    if (pos[0]) dali_hip_bank_deposit(pos[0], pos_bytes);
+    if (words[1]) dali_hip_bank_deposit(words[1], word_bytes);
+    if (words[0]) dali_hip_bank_deposit(words[0], word_bytes);
     return status;
 }
 
@@ -645,8 +713,7 @@ extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_
     // radix passes over the bits that can differ; arbitrary keys are ordered as signed numbers (the sign bit is flipped in
     // the digit). The pairs bounce between the caller's arrays and one temporary block so that the last pass lands in the
     // caller's.
-    int rounds = kRadixMaxTile / 256;
-    while (rounds > 1 && n / (256 * rounds) < 1024) rounds /= 2;
+    const int rounds = radix_rounds(n);
     const int passes = (end_bit + 7) / 8, tiles = (int)((n + 256 * rounds - 1) / (256 * rounds));
     const unsigned int flip = key_limit > 0 ? 0u : 0x80000000u, limit = key_limit > 0 ? (unsigned int)key_limit : 0u;
     const size_t temp_bytes = ((size_t)2 * (size_t)n + (size_t)256 * (size_t)tiles + 256) * sizeof(int32_t);
@@ -662,18 +729,7 @@ extern "C" int dali_hip_argsort_i32(const int32_t* keys, int64_t n, int32_t key_
         const bool to_caller = (passes - 1 - i) % 2 == 0;
         int32_t* dst_keys = to_caller ? sorted_keys : tkeys;
         int32_t* dst_pos = to_caller ? perm : tpos;
-        auto pass = [&](auto hist_kernel, auto move_kernel) {
-            hipLaunchKernelGGL(hist_kernel, dim3(tiles), dim3(256), 0, st, src_keys, (int)n, 8 * i, flip, limit, hist, tiles);
-            hipLaunchKernelGGL(radix_row_scan_kernel, dim3(256), dim3(256), 0, st, hist, tiles, totals);
-            hipLaunchKernelGGL(move_kernel, dim3(tiles), dim3(256), 0, st, src_keys, src_pos, (int)n, 8 * i, flip, limit, (const unsigned int*)hist,
-                               (const unsigned int*)totals, tiles, dst_keys, dst_pos);
-        };
-        switch (rounds) {
-            case 1: pass(radix_hist_kernel<1>, radix_move_kernel<1>); break;
-            case 2: pass(radix_hist_kernel<2>, radix_move_kernel<2>); break;
-            case 4: pass(radix_hist_kernel<4>, radix_move_kernel<4>); break;
-            default: pass(radix_hist_kernel<8>, radix_move_kernel<8>); break;
-        }
+        radix_pass<int32_t, IndexDigits>(rounds, src_keys, src_pos, (int)n, 8 * i, IndexDigits{flip, limit}, hist, totals, tiles, dst_keys, dst_pos, st);
         src_keys = dst_keys;
         src_pos = dst_pos;
     }

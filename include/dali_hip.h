@@ -364,8 +364,8 @@ int dali_hip_argsort_i32_noalloc(const int32_t* keys, int64_t n, int32_t key_lim
  * else ascending (bottom_k, argsort). Equal values come out in ascending column order, or in descending column order
  * with ties_by_descending_column != 0 (what the reference's heap gives bottom_k for k < cols, top_k.cpp:118-123).
  * -0.0 and +0.0 are equal; the place of NaNs is unspecified. Rows of at least 1024 entries with k <= 64 take a one-pass
- * selection kernel that allocates nothing; everything else one segmented radix sort on the library stream whose buffers
- * (four times the input) come from the bank, so that form fails during a capture.
+ * selection kernel that allocates nothing; everything else stable radix passes over the whole matrix (by key, then by
+ * row) on the library stream whose buffers (four times the input) come from the bank, so that form fails during a capture.
  */
 int dali_hip_topk_rows(const void* x, int dtype, int64_t rows, int32_t cols, int32_t k, int largest, int ties_by_descending_column,
                        int32_t* out);

@@ -1327,7 +1327,7 @@ def test_ceil_softmax_temperature_and_named_products(gpu, D, rng):
 def test_top_k_bottom_k_argsort_are_bit_exact(gpu, D, O, rng, dtype):
     """Positions from the device ordering against the reference's comparators (top_k.cpp:96-233), on rows full of ties."""
     op = D.op
-    # rows of 1024 and more with k <= 64 go through the selection kernel, everything else through the segmented sort
+    # rows of 1024 and more with k <= 64 go through the selection kernel, everything else through the radix sort of the whole matrix
     for shape in [(5, 9), (3, 4, 33), (64, 1000), (37, 2048), (2, 70001)]:
         x = rng.randint(-50, 51, shape).astype(dtype)
         n = shape[-1]
