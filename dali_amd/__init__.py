@@ -9,5 +9,5 @@ hipRTC compilation and launches all happen in the native libraries
 libraries the import fails, and without a GPU every evaluation raises.
 """
 from ._native import front, hip, DaliError, lib_paths  # noqa: F401
-from .array import Array, DTYPE_FLOAT, DTYPE_DOUBLE, DTYPE_INT32, eval_together, jit_stats, last_kernel_kinds, last_kernel_names, last_source, generate_only, Recording, ScopeObserver  # noqa: F401
+from .array import Array, DTYPE_FLOAT, DTYPE_DOUBLE, DTYPE_INT32, eval_together, jit_stats, last_kernel_kinds, last_kernel_names, last_source, generate_only, generated_source, Recording, ScopeObserver  # noqa: F401
 from . import op  # noqa: F401

@@ -200,6 +200,7 @@ FRONT_SYMBOLS = {
     "dali_fe_last_kernel_kinds": (C.c_char_p, []),
     "dali_fe_last_kernel_names": (C.c_char_p, []),
     "dali_fe_last_source": (C.c_char_p, []),
+    "dali_fe_generated_source": (C.c_char_p, [C.c_int]),
     "dali_fe_generate_only": (_i, [_HP, _i, _i]),
     "dali_fe_set_dry_run": (_i, [_i, _i]),
     "dali_fe_record_begin": (H, []),

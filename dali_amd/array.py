@@ -308,6 +308,11 @@ def last_source():
     return front.dali_fe_last_source().decode()
 
 
+def generated_source(i):
+    """Source of the i-th kernel of the last ``generate_only`` call."""
+    return front.dali_fe_generated_source(i).decode()
+
+
 def generate_only(arrays, compile=False):
     """Plan and generate HIP source for ``arrays`` without touching a device."""
     hs = (C.c_void_p * len(arrays))(*[a._h for a in arrays])

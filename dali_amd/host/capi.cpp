@@ -360,14 +360,18 @@ int dali_fe_scope_observe(dali_fe_scope_callback on_enter, dali_fe_scope_callbac
 
 void dali_fe_scope_unobserve(int id) { dali::Scope::remove_observer(id); }
 
+// every kernel source of the last dali_fe_generate_only call, in the order of the launches they stand for
+static std::vector<std::string> g_generated;
+const char* dali_fe_generated_source(int i) { return i >= 0 && i < (int)g_generated.size() ? g_generated[i].c_str() : ""; }
+
 int dali_fe_generate_only(dali_array_t* roots, int n, int compile) {
     dali::set_dry_compile(compile != 0);
     try {
         std::vector<Array> r;
         for (int i = 0; i < n; ++i) r.push_back(A(roots[i]));
-        auto srcs = dali::generate_only(r);
+        g_generated = dali::generate_only(r);
         dali::set_dry_compile(false);
-        return (int)srcs.size();
+        return (int)g_generated.size();
     } catch (const std::exception& ex) {
         dali::set_dry_compile(false);
         g_err = ex.what();

@@ -406,7 +406,10 @@ void emit_leaf_load(std::ostringstream& ss, const ArrayArg& a, int i, int VEC, c
                     bool ragged = false, const std::string& pointer_prefix = "q");
 
 // jit_row.cpp
-bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::vector<DestSpec>* totals = nullptr);
+// `segments` > 1: the requests are reductions along the rows with one result per row and nothing else; every row is cut into
+// that many pieces, each piece goes to a workgroup of its own, and a destination (a view of `dom.R` elements whose stride is
+// `segments`: one column of an [R, segments] buffer) receives the pieces' results side by side, for the caller to reduce again.
+bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::vector<DestSpec>* totals = nullptr, int segments = 0);
 
 // jit_flat.cpp
 bool flat_eligible(const Array& a, int64_t n, std::set<const Expr*>& seen);

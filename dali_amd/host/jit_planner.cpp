@@ -72,6 +72,19 @@ static Array expand_softmax(Array x, int axis) {
                 evaluate({M, L});
                 return op::eltdiv(op::exp(op::subtract(x, M.reshape(keep))), L.reshape(keep));
             }
+            // the same rows at a length that does not divide that way: the row kernel cuts them into pieces itself, once for
+            // the maxima and once for the sums of the exponentials (see try_segmented_reduce)
+            static const bool pieces_off = env_int("DALI_HIP_SEGMENTED_REDUCE", 1) == 0;
+            if (!pieces_off && rows < 256 && Cx >= 65536 && rows * 8 <= 2048 && Cx / 8 >= 8192) {
+                if (!x.is_buffer()) x = materialize(x);
+                if (!x.contiguous_memory()) x = x.ascontiguousarray();
+                Array x2 = x.reshape({(int)rows, (int)Cx});
+                Array M = op::max(x2, {-1}, false);
+                evaluate({M});
+                Array L = op::sum(op::exp(op::subtract(x2, M.reshape({(int)rows, 1}))), {-1}, false);
+                evaluate({L});
+                return op::eltdiv(op::exp(op::subtract(x, M.reshape(keep))), L.reshape(keep));
+            }
         } else if (n >= (1 << 16)) {
             int64_t inner = 1, outer = 1;
             for (int d = axis + 1; d < nd; ++d) inner *= shape[d];
@@ -356,8 +369,64 @@ static bool try_two_stage_reduce(const DestSpec& spec) {
     return true;
 }
 
+// Few long rows that the reshaped view above cannot serve: rows whose length is no multiple of four elements times the
+// number of pieces, and the position of the best element (dali/array/op/reducer_operation.cpp:193-228,686-710). The row kernel
+// itself cuts every row into S pieces (whole vectors each, the last one with the elements left over), a workgroup per piece,
+// and leaves [R, S] partial results. Position: a piece yields its best value and that value's column in the whole row (the
+// first one among equals); the first piece that holds the row's best value (an argmax over the S values, first among equals
+// again) then names the column, which is the reference's "first index on ties".
+static bool try_segmented_reduce(const DestSpec& spec) {
+    static const bool off = env_int("DALI_HIP_SEGMENTED_REDUCE", 1) == 0;
+    if (off) return false;
+    auto e = spec.root.expression();
+    const bool position = e->kind == Kind::ARG_AXIS_REDUCE;
+    if (e->kind != Kind::AXIS_REDUCE && !position) return false;
+    const std::string& red = e->name;
+    if (position ? (red != "reducers::maximum" && red != "reducers::minimum")
+                 : (red != "reducers::sum" && red != "reducers::maximum" && red != "reducers::minimum" && red != "reducers::product"))
+        return false;
+    Array arg = e->args[0];
+    // a buffer of any rank, or an expression over [R, C] (the exponentials of a softmax's rows: whether it fits the row kernel is
+    // the row kernel's to say)
+    if (arg.ndim() < 1 || size_of_dtype(arg.dtype()) != 4) return false;
+    if (arg.is_buffer() ? !arg.contiguous_memory() : arg.ndim() != 2) return false;
+    if (!position && arg.dtype() != e->dtype) return false;
+    const int C_last = arg.shape().back();
+    const int64_t n = numel_of(arg.shape());
+    if (n == 0 || C_last < (1 << 16)) return false;
+    const int64_t rows = n / C_last;
+    if (rows >= 256) return false;
+    int S = 1;
+    while (S * 2 * rows <= 2048 && C_last / (S * 2) >= 8192) S *= 2;
+    if (S < 4) return false;
+    const int R = (int)rows;
+    Array rows2d = arg.is_buffer() ? arg.reshape({R, C_last}) : arg;
+    const Domain dom = domain_of(rows2d.shape());
+    std::vector<int> partial_shape = e->shape;  // the leading dimensions of the argument, then the S partial results
+    partial_shape.push_back(S);
+    Array best({R, S}, arg.dtype());
+    if (!position) {
+        if (!try_row({{best.pluck_axis(1, 0), OPERATOR_T_EQL, op::axis_reduce(rows2d, red, {1}, false)}}, dom, nullptr, S)) return false;
+        Array root2 = op::axis_reduce(best.reshape(partial_shape), red, {(int)partial_shape.size() - 1}, false);
+        if (root2.shape() != e->shape) return false;
+        run_specs({{spec.dest, spec.op, root2}});
+        return true;
+    }
+    Array where({R, S}, DTYPE_INT32);
+    if (!try_row({{best.pluck_axis(1, 0), OPERATOR_T_EQL, op::axis_reduce(rows2d, red, {1}, false)},
+                  {where.pluck_axis(1, 0), OPERATOR_T_EQL, op::argument_axis_reduce(rows2d, red, 1)}},
+                 dom, nullptr, S))
+        return false;
+    Array piece = op::argument_axis_reduce(best, red, 1);
+    piece.eval();
+    Array root2 = op::gather_from_rows(where, piece);
+    if (e->shape.size() != 1) root2 = root2.reshape(e->shape);
+    run_specs({{spec.dest, spec.op, root2}});
+    return true;
+}
+
 void run_specs_planned(std::vector<DestSpec> specs) {
-    if (specs.size() == 1 && try_two_stage_reduce(specs[0])) return;
+    if (specs.size() == 1 && (try_two_stage_reduce(specs[0]) || try_segmented_reduce(specs[0]))) return;
     // all-reduce roots are planned one by one
     if (specs.size() > 1) {
         bool any_all = false;

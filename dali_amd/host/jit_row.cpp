@@ -132,7 +132,7 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
             o << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n" << chunk_guard;
         } else {
             if (rp.split)
-                o << "  for (int ch = ch_begin + tr; ch < ch_end; ch += TPR) {\n    {\n";
+                o << (rpn.n_phases > 0 ? "  _Pragma(\"unroll 4\")\n" : "") << "  for (int ch = ch_begin + tr; ch < ch_end; ch += TPR) {\n    {\n";
             else
                 o << "  for (int ch = tr; ch < CH; ch += TPR) {\n    {\n";
             for (int i : full_leaves) {
@@ -457,14 +457,17 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
     bool any_row = false;
     for (const Output& o : rpn.outputs) any_row = any_row || (o.cls != Cls::FULL && o.total_red < 0);
     if (any_row) {
-        ss << "  if (tr == 0 && row_ok" << (rp.split ? " && seg == 0" : "") << ") {\n";
+        // (pieces of rows reduced on their own: every piece writes its result, piece `seg` into element `seg` behind the row's first)
+        const bool pieces = rp.split && rpn.n_phases > 0;
+        const std::string slot = pieces ? "[seg]" : "[0]";
+        ss << "  if (tr == 0 && row_ok" << (rp.split && !pieces ? " && seg == 0" : "") << ") {\n";
         BodyEmitter be(P, rp, false, rpn.n_phases, &rpn.first_body);
         std::ostringstream body;
         for (const Output& o : rpn.outputs) {
             if (o.cls == Cls::FULL || o.total_red >= 0) continue;
             std::string t = ctype(P.arrays[o.array].buf->dtype);
             std::string v = be.value(o.root);
-            body << "    q" << o.array << "[0] = " << op_combine(o.op, "q" + std::to_string(o.array) + "[0]", "(" + t + ")(" + v + ")") << ";\n";
+            body << "    q" << o.array << slot << " = " << op_combine(o.op, "q" + std::to_string(o.array) + slot, "(" + t + ")(" + v + ")") << ";\n";
         }
         ss << be.stmts.str() << body.str() << "  }\n";
     }
@@ -517,7 +520,7 @@ static bool peel_ok(const Program& P, const Domain& dom) {
 // reduction of an expression with one value per row of `dom` (the mean of the row losses next to the gradient of a
 // cross-entropy). They ride along in the same launch: every workgroup publishes the combination of its rows' values,
 // the workgroup that draws the last ticket folds those in workgroup order, applies the scalar arithmetic and stores.
-bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::vector<DestSpec>* totals) {
+bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::vector<DestSpec>* totals, int segments) {
     RowPlan rpn;
     Program& P = rpn.P;
     rpn.dom = dom;
@@ -631,7 +634,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
     // Long rows whose vectors are aligned but whose length is no whole number of cache lines gain the same way from starting at
     // a 128-byte boundary ([2048,50256]: 156 -> 154 us, [2048,45000]: 142 -> 137 us).
     const bool line_rows = rp.VEC == 4 && !rp.ragged && dom.C >= 8192 && dom.C % 32 != 0;
-    if ((rp.ragged || line_rows) && peel_env && nph > 0 && peel_ok(P, dom)) {
+    if ((rp.ragged || line_rows) && peel_env && nph > 0 && segments <= 1 && peel_ok(P, dom)) {
         rp.ragged = true;
         rp.peel = true;
         rp.tail = true;
@@ -691,6 +694,15 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
         int64_t ept = (CH + tpr - 1) / tpr;
         // every FULL input is held in registers across the phases: bound the footprint
         rp.cached = (int64_t)std::max(1, n_full) * ept * rp.VEC * (max_el / 4) <= 64;
+        if (segments > 1) {
+            // pieces of rows: one phase, results per row only, streamed (a piece is read once); at least a workgroup's worth of vectors each
+            if (nph != 1 || n_totals != 0 || rp.VEC != 4 || CH / segments < 1024) return false;
+            for (const Output& o : rpn.outputs)
+                if (o.cls != Cls::ROW) return false;
+            rp.cached = false;
+            rp.split = true;
+            split_S = segments;
+        }
         if (!rp.cached) {
             tpr = 1024;
             ept = 0;

@@ -194,6 +194,8 @@ int dali_fe_set_dry_run(int on, int compile);
 /* plan + generate (and optionally hipRTC-compile for gfx950) without a device;
  * returns the number of kernels, -1 on error */
 int dali_fe_generate_only(dali_array_t* roots, int n, int compile);
+/* source of the i-th of those kernels, in launch order ("" outside the range); valid until the next dali_fe_generate_only */
+const char* dali_fe_generated_source(int i);
 
 #ifdef __cplusplus
 }

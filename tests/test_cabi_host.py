@@ -188,6 +188,26 @@ def test_rows_off_the_vector_alignment_keep_vector_accesses(D, rng):
     assert "dali_loadu" not in D.last_source()[D.last_source().index("void dali_row_"):]
 
 
+def test_few_long_ragged_rows_are_cut_into_pieces_inside_the_row_kernel(D, rng):
+    op = D.op
+    x = D.Array.from_numpy(np.zeros((3, 1000001), np.float32))
+    n = D.generate_only([op.argmax(x, 1)], compile=True)
+    assert n == 3                                     # pieces, the first best piece of every row, its column
+    first = D.generated_source(0)
+    first = first[first.index("void dali_row_"):]
+    # S * R workgroups, piece `seg` of a row writes element `seg` behind the row's first; the elements past the last whole
+    # vector belong to the last piece; columns count from the start of the row
+    assert "const int seg" in first and "q0[seg] =" in first and "q1[seg] =" in first and "seg == S - 1" in first
+    assert "const int col = ch * VEC + j" in first and "for (int ch = ch_begin + tr; ch < ch_end; ch += TPR)" in first
+    assert D.generate_only([op.sum(x, [1])], compile=True) == 2
+    assert D.generate_only([op.softmax(x)], compile=True) == 5   # maxima, sums of exponentials (two launches each), the quotient
+    last = D.generated_source(4)
+    assert "void dali_map2d_" in last
+    # rows that divide into equal aligned pieces keep the reshaped view (cached pieces, (maximum, sum) in one pass)
+    y = D.Array.from_numpy(np.zeros((3, 1 << 20), np.float32))
+    assert D.generate_only([op.softmax(y)], compile=True) == 3
+
+
 def test_long_cached_rows_put_part_of_the_row_into_lds(D, rng):
     op = D.op
     x = D.Array.from_numpy(np.zeros((4, 50257), np.float32))

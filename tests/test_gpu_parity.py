@@ -785,13 +785,14 @@ def test_middle_axis_reductions_use_the_batched_column_kernel(gpu, D, O, rng, sh
         assert np.array_equal(op.max(v, [1]).numpy(), nv.max(1))
 
 
-@pytest.mark.parametrize("cols", [16, 17, 18, 19, 63, 127, 257, 1023, 4097, 50257, 300001])
+@pytest.mark.parametrize("cols", [16, 17, 18, 19, 63, 127, 257, 1023, 4097, 50257, 70001])
 def test_rows_not_aligned_to_the_vector(gpu, D, O, rng, cols):
     """Row lengths that are no multiple of four elements, and views that start off a 16-byte boundary: whole vectors
     at element alignment, the rest of each row one element per thread. Every phase, the register cache and the
     op-assign destinations see the rest elements."""
     op = D.op
-    rows = 5 if cols > 5000 else 37
+    # (70001: rows streamed through the kernel three times; 256 of them, fewer would be cut into pieces and reduced in two steps)
+    rows = 256 if cols > 65536 else (5 if cols > 5000 else 37)
     x = (rng.randn(rows, cols) * 3).astype(np.float32)
     X = arr(D, x)
     s = op.softmax(X).numpy()
@@ -824,6 +825,53 @@ def test_rows_not_aligned_to_the_vector(gpu, D, O, rng, cols):
     xi = rng.randint(-1000, 1000, size=(rows, cols)).astype(np.int32)
     assert np.array_equal(op.sum(arr(D, xi), [1]).numpy(), xi.sum(1))
     assert np.array_equal((arr(D, xi)[:, 1:] * 3).numpy(), xi[:, 1:] * 3)
+
+
+@pytest.mark.parametrize("shape", [(7, 300001), (3, 1000003), (1, 524291), (2, 3, 131075), (31, 65537), (5, 262144)])
+def test_few_long_rows_cut_into_pieces_by_the_row_kernel(gpu, D, O, rng, shape):
+    """Reductions along few very long rows whose length does not divide into equal aligned pieces, and the position of the
+    best element at any length (reducer_operation.cpp:98-156,193-228): the row kernel cuts every row into pieces, a second
+    small kernel reduces the pieces' results. Sums within rel 1e-5 of fp64, extrema and positions exact, with equal best values
+    planted in different pieces and next to the pieces' boundaries (the reference keeps the first: all_reduce_kernel_utils.cpp:
+    217-219)."""
+    op = D.op
+    x = rng.randn(*shape).astype(np.float32)
+    C = shape[-1]
+    rows = x.reshape(-1, C)
+    S = 1
+    while S * 2 * rows.shape[0] <= 2048 and C // (S * 2) >= 8192:
+        S *= 2
+    per = (C // 4 + S - 1) // S * 4          # elements of a piece
+    for r in range(rows.shape[0]):
+        # the same best value in three pieces: last element of one, first of the next, and the very last element of the row
+        p = int(rng.randint(1, S - 1)) * per
+        for c in (p - 1, p, C - 1):
+            rows[r, c] = 50.0 + r
+            rows[r, (c + 7) % C] = -50.0 - r if c != C - 1 else rows[r, (c + 7) % C]
+    X = arr(D, x)
+    x64 = x.astype(np.float64)
+    k0 = D.jit_stats()["kernels"]
+    got = op.sum(X, [-1]).numpy()
+    assert D.jit_stats()["kernels"] - k0 == 2
+    close(got, x64.sum(-1), rtol=1e-5, atol=1e-5 * np.sqrt(C))
+    assert np.array_equal(op.max(X, [-1]).numpy(), x.max(-1))
+    assert np.array_equal(op.min(X, [-1]).numpy(), x.min(-1))
+    k0 = D.jit_stats()["kernels"]
+    am = op.argmax(X, -1).numpy()
+    assert D.jit_stats()["kernels"] - k0 <= 4
+    assert am.dtype == np.int32 and np.array_equal(am, x.argmax(-1)) and np.array_equal(am, O.arg_axis_reduce(O.MAX, rows, 1).reshape(am.shape))
+    assert np.array_equal(op.argmin(X, -1).numpy(), O.arg_axis_reduce(O.MIN, rows, 1).reshape(am.shape))
+    # an expression over the rows reduces the same way once its leaves are buffers
+    y = np.abs(x) * 1e-3 + 1.0
+    close(op.prod(arr(D, y[..., :65600]), [-1]).numpy(), y[..., :65600].astype(np.float64).prod(-1), rtol=65600 * 2.0 ** -24 * 0.05)  # (a twentieth of the a-priori bound)
+    # softmax over such rows: maxima in pieces, sums of exponentials in pieces, the quotient as a lazy map
+    k0 = D.jit_stats()["kernels"]
+    s = op.softmax(X).numpy()
+    if C % 32 != 0 or rows.shape[0] * 8 > 2048:
+        assert D.jit_stats()["kernels"] - k0 == 5 and D.last_kernel_kinds().endswith(("map2d", "flat"))  # (flat: a single row)
+    e = np.exp(x64 - x64.max(-1, keepdims=True))
+    close(s, e / e.sum(-1, keepdims=True), rtol=1e-5, atol=1e-12)
+    close(s.astype(np.float64).sum(-1), 1.0, rtol=0, atol=2e-6)
 
 
 @pytest.mark.parametrize("shape", [(37, 16), (37, 17), (5, 18), (300, 19), (3000, 1001), (64, 4097), (2000, 50257), (7, 300001)])
