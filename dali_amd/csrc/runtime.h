@@ -30,6 +30,8 @@ int sort_scratch_init(int device);
 // sgemm_skinny.hip: row-major C[M, N] = alpha * A[M, K] . B[K, N] + beta * C for M <= 64 by streaming B once
 // (tb: B stored as [N][K]). 1: launched; 0: not a case for it (take the tiled kernels); -1: failure (message set)
 int sgemm_skinny(bool tb, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb, float beta, float* C, int ldc);
+// sgemv.hip: y[M] = alpha * A[M, K] . x[K] + beta * y for row-major A, strides in elements; 1 = launched, 0 = not taken, -1 = error
+int sgemv_rows(int M, int K, float alpha, const float* A, int lda, const float* x, int incx, float beta, float* y, int incy);
 // the same for an inner extent of at most 64 against a large C (ta: A stored as [K][M]): bound by writing C once
 int sgemm_smallk(bool ta, bool tb, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb, float beta, float* C, int ldc);
 // sgemm_dma.hip: row-major C[M, N] = alpha * sum_s A_s . B_s + beta * C for one or two terms of whole 64-deep slabs through

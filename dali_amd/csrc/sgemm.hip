@@ -1010,6 +1010,12 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         const int st = tiles128_product(g, false, false);
         if (st >= 0) return st;
     }
+    static const int gemv_on = getenv("DALI_HIP_GEMV") ? atoi(getenv("DALI_HIP_GEMV")) : 1;
+    if (gemv_on && g.nseg == 1 && N == 1 && g.seg[0].K > 0 && !ta && !row_map && !rows_may_overlap && (M >= 64 || g.seg[0].K <= 65536)) {
+        // a matrix times a column: the rows of A streamed once, each against the same vector
+        const int st = sgemv_rows(M, g.seg[0].K, alpha, g.seg[0].A, g.seg[0].lda, g.seg[0].B, tb ? 1 : g.seg[0].ldb, beta, C, ldc);
+        if (st != 0) return st > 0 ? DALI_HIP_OK : DALI_HIP_ERROR;
+    }
     if (g.nseg == 1 && g.seg[0].K > 0 && !ta && !row_map && !rows_may_overlap && M <= 64) {
         // few rows against a wide right operand: stream it once instead of tiling it through LDS
         const int st = sgemm_skinny(tb, M, N, g.seg[0].K, alpha, g.seg[0].A, g.seg[0].lda, g.seg[0].B, g.seg[0].ldb, beta, C, ldc);

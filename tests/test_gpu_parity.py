@@ -295,6 +295,43 @@ def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
         hip.dali_hip_free(p)
 
 
+@pytest.mark.parametrize("M,K", [(4096, 4096), (256, 1024), (2049, 1001), (3000, 7), (5, 3), (1, 70000), (70, 66001), (100000, 64), (2048, 258)])
+@pytest.mark.parametrize("tb", [0, 1])
+def test_sgemm_of_a_matrix_with_a_column_streams_the_rows(gpu, rng, M, K, tb):
+    """A row-major matrix times a single column (dot.cpp:49-67 with b.shape[1] == 1): the rows are streamed once, one wave or
+    one workgroup per row. The column as B stored [K][1] with any leading dimension (a column of a wider matrix) or as [1][K];
+    rows and results with padding (NaN in the operands' padding, and in the destination when beta = 0); rows that start off
+    the 16-byte boundary. Against the product accumulated in double precision."""
+    hip = gpu
+    A = rng.randn(M, K).astype(np.float32)
+    x = rng.randn(K).astype(np.float32)
+    lda, ldb, ldc = K + 3, (K + 2 if tb else 5), 3
+    Ap = np.full((M, lda), np.nan, np.float32); Ap[:, :K] = A
+    if tb:
+        Bp = np.full((1, ldb), np.nan, np.float32); Bp[0, :K] = x
+    else:
+        Bp = np.full((K, ldb), np.nan, np.float32); Bp[:, 0] = x
+    C0 = rng.randn(M, ldc).astype(np.float32)
+    want = A.astype(np.float64) @ x.astype(np.float64)
+    scale = np.abs(want).max() + 1e-6
+    dA, dB = _dev(hip, Ap), _dev(hip, Bp)
+    for alpha, beta in ((1.0, 0.0), (0.75, -0.5)):
+        Cin = C0.copy()
+        if beta == 0.0:
+            Cin[:, 0] = np.nan
+        dC = _dev(hip, Cin)
+        st = hip.dali_hip_sgemm(tb, 0, 1, M, K, alpha, dB, ldb, dA, lda, beta, dC, ldc)
+        assert st == 0, hip.dali_hip_last_error()
+        out = np.empty_like(Cin)
+        hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, Cin.nbytes)
+        ref = alpha * want + (beta * C0[:, 0] if beta != 0.0 else 0.0)
+        assert np.abs(out[:, 0] - ref).max() <= 1e-4 * scale
+        assert np.array_equal(out[:, 1:], C0[:, 1:])  # padding untouched
+        hip.dali_hip_free(dC)
+    for p in (dA, dB):
+        hip.dali_hip_free(p)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 32000, 1024), (8, 4096, 1024), (64, 1000, 260), (17, 777, 512), (33, 2049, 64), (64, 8192, 2048),
                                    (5, 40000, 68), (48, 32000, 1024), (8, 1024, 1024), (8, 256, 1024), (9, 512, 512), (20, 4096, 256),
                                    (64, 1024, 32000), (40, 1028, 16384),
