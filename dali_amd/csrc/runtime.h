@@ -36,15 +36,15 @@ int sgemv_rows(int M, int K, float alpha, const float* A, int lda, const float* 
 int sgemm_smallk(bool ta, bool tb, int M, int N, int K, float alpha, const float* A, int lda, const float* B, int ldb, float beta, float* C, int ldc);
 // sgemm_dma.hip: row-major C[M, N] = alpha * sum_s A_s . B_s + beta * C for one or two terms of whole 64-deep slabs through
 // the kernel whose operand slabs are written into LDS by the loads themselves (ta: A_s stored as [K][M], tb: B_s stored as
-// [N][K]; one pair of leading dimensions). With `bias` the sums go through the LSTM gate arithmetic instead of into C
+// [N][K]; leading dimensions per term). With `bias` the sums go through the LSTM gate arithmetic instead of into C
 // (N = 4 H, columns gathered per hidden unit). 1: launched; 0: not a case for it; -1: failure (message set)
-int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
+int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, const int* lda, const int* ldb,
               float alpha, float beta, float* C, int ldc, const float* bias, const float* c_prev, float* c_out, float* h_out, int H);
 // The same pipeline over a stream of work items per workgroup (one workgroup per compute unit walks many tiles, its loads
 // running ahead across tile boundaries); `shares` > 1 cuts every tile's inner extent into that many contiguous shares that meet
 // in the library workspace (single products only). `cus`: compute units of the bound device. Same return values.
 // With `bias` the sums go through the LSTM gate arithmetic instead of into C, as in sgemm_dma.
-int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
+int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, const int* lda, const int* ldb,
                      float alpha, float beta, float* C, int ldc, int shares, int cus, const float* bias = nullptr, const float* c_prev = nullptr,
                      float* c_out = nullptr, float* h_out = nullptr, int H = 0);
 // sgemm_dma128.hip: row-major C[M, N] = alpha * A . B + beta * C over whole 32-deep slabs with 128x128 tiles, one workgroup per

@@ -806,13 +806,15 @@ static int launch_tile(GemmArgs g, bool ta, bool tb, bool vec, int split_k, bool
 template <int BM, int BN, int BK, int DEPTH, int KW = 1, bool MIDB = false>
 static int run_tile(const GemmArgs& g, bool ta, bool tb, bool vec, int split_k) {
     bool fast = vec && g.nseg > 0 && (!ta || g.M % 4 == 0) && (tb || g.N % 4 == 0);
+    bool same_ld = true;  // the register-staged kernel takes one pair of leading dimensions, the other one a pair per term
     for (int s = 0; s < g.nseg && fast; ++s) {
         const size_t a_span = ((size_t)(ta ? BK : g.M) * g.seg[s].lda + (ta ? g.M : BK)) * sizeof(float);
         const size_t b_span = ((size_t)(tb ? g.N : BK) * g.seg[s].ldb + (tb ? BK : g.N)) * sizeof(float);
         fast = fast && a_span < ((size_t)1 << 32) && b_span < ((size_t)1 << 32);
-        fast = fast && g.seg[s].lda == g.seg[0].lda && g.seg[s].ldb == g.seg[0].ldb;
+        same_ld = same_ld && g.seg[s].lda == g.seg[0].lda && g.seg[s].ldb == g.seg[0].ldb;
     }
-    if (!fast) return launch_tile<BM, BN, BK, DEPTH, KW, MIDB>(g, ta, tb, vec, split_k, true);
+    constexpr bool dma_tile = BM == 64 && BN == 64 && BK == 64 && KW == 2 && !MIDB;
+    if (!fast || (!same_ld && !(dma_tile && split_k == 1 && g.nseg <= 2 && !g.map_on))) return launch_tile<BM, BN, BK, DEPTH, KW, MIDB>(g, ta, tb, vec, split_k, true);
     GemmArgs whole = g, rest = g;
     whole.nseg = rest.nseg = 0;
     for (int s = 0; s < g.nseg; ++s) {
@@ -834,16 +836,19 @@ static int run_tile(const GemmArgs& g, bool ta, bool tb, bool vec, int split_k) 
     if (whole.nseg > 0) {
         int st = 0;
         bool done = false;
-        if (BM == 64 && BN == 64 && BK == 64 && KW == 2 && !MIDB && split_k == 1 && whole.nseg <= 2 && !whole.map_on) {
+        if (dma_tile && split_k == 1 && whole.nseg <= 2 && !whole.map_on) {
             // small grids of whole slabs: the kernel that has its operand slabs written into LDS by the loads themselves
             const float* as[2] = {whole.seg[0].A, whole.seg[1].A};
             const float* bs[2] = {whole.seg[0].B, whole.seg[1].B};
             const int ks[2] = {whole.seg[0].K, whole.seg[1].K};
-            const int r = sgemm_dma(ta, tb, whole.M, whole.N, whole.nseg, ks, as, bs, whole.seg[0].lda, whole.seg[0].ldb, whole.alpha, whole.beta,
+            const int las[2] = {whole.seg[0].lda, whole.seg[1].lda}, lbs[2] = {whole.seg[0].ldb, whole.seg[1].ldb};
+            const int r = sgemm_dma(ta, tb, whole.M, whole.N, whole.nseg, ks, as, bs, las, lbs, whole.alpha, whole.beta,
                                     whole.C, whole.ldc, nullptr, nullptr, nullptr, nullptr, 0);
             if (r < 0) return DALI_HIP_ERROR;
             done = r > 0;
         }
+        // (terms with rows of different lengths that the kernel above did not take: everything through the guarded kernel)
+        if (!done && !same_ld) return launch_tile<BM, BN, BK, DEPTH, KW, MIDB>(g, ta, tb, vec, split_k, true);
         if (!done) st = launch_tile<BM, BN, BK, DEPTH, KW, MIDB>(whole, ta, tb, true, split_k, false);
         if (st || rest.nseg == 0) return st;
         rest.beta = 1.0f;
@@ -914,7 +919,8 @@ static int stream_product(const GemmArgs& g, bool ta, bool tb, int shares) {
     const int ks[2] = {whole.seg[0].K, whole.seg[1].K};
     const int cus = device_cus();
     if (cus <= 0) return -1;
-    const int r = sgemm_dma_stream(ta, tb, whole.M, whole.N, whole.nseg, ks, as, bs, whole.seg[0].lda, whole.seg[0].ldb, whole.alpha, whole.beta, whole.C,
+    const int las[2] = {whole.seg[0].lda, whole.seg[1].lda}, lbs[2] = {whole.seg[0].ldb, whole.seg[1].ldb};
+    const int r = sgemm_dma_stream(ta, tb, whole.M, whole.N, whole.nseg, ks, as, bs, las, lbs, whole.alpha, whole.beta, whole.C,
                                    whole.ldc, shares, cus);
     if (r < 0) return DALI_HIP_ERROR;
     if (r == 0) return -1;
@@ -1011,6 +1017,32 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
         if (st >= 0) return st;
     }
     static const int gemv_on = getenv("DALI_HIP_GEMV") ? atoi(getenv("DALI_HIP_GEMV")) : 1;
+    if (gemv_on && g.nseg >= 1 && g.nseg <= 2 && g.seg[0].K > 0 && !ta && !tb && !row_map && !rows_may_overlap && N % 4 != 0 && N >= 1024 && M > 64) {
+        // A wide row-major B whose row length is no multiple of four (a vocabulary of 50257 words): the kernels that take whole
+        // 16-byte granules along N serve the columns up to the last multiple of four, and the one to three columns left over
+        // are matrix-vector products ([256,1024].[1024,50257]: 334 -> 289 us; the guarded kernel would serve all of it; up to 64 rows the
+        // row-streaming kernel below takes any N)
+        const int N4 = N & ~3;
+        const float* as[kMaxSeg];
+        const float* bs[kMaxSeg];
+        int ks[kMaxSeg], las[kMaxSeg], lbs[kMaxSeg];
+        for (int s = 0; s < g.nseg; ++s) {
+            as[s] = g.seg[s].A;
+            bs[s] = g.seg[s].B;
+            ks[s] = g.seg[s].K;
+            las[s] = g.seg[s].lda;
+            lbs[s] = g.seg[s].ldb;
+        }
+        const int st = sgemm_rowmajor(g.nseg, false, false, M, N4, ks, as, las, bs, lbs, alpha, beta, C, ldc);
+        if (st != DALI_HIP_OK) return st;
+        for (int j = N4; j < N; ++j)
+            for (int s = 0; s < g.nseg; ++s) {
+                const int r = sgemv_rows(M, ks[s], alpha, as[s], las[s], bs[s] + j, lbs[s], s == 0 ? beta : 1.0f, C + j, ldc);
+                if (r < 0) return DALI_HIP_ERROR;
+                if (r == 0) return fail("sgemm: the matrix-vector kernel refused column %d of a validated product", j);
+            }
+        return DALI_HIP_OK;
+    }
     if (gemv_on && g.nseg == 1 && N == 1 && g.seg[0].K > 0 && !ta && !row_map && !rows_may_overlap && (M >= 64 || g.seg[0].K <= 65536)) {
         // a matrix times a column: the rows of A streamed once, each against the same vector
         const int st = sgemv_rows(M, g.seg[0].K, alpha, g.seg[0].A, g.seg[0].lda, g.seg[0].B, tb ? 1 : g.seg[0].ldb, beta, C, ldc);
@@ -1042,7 +1074,7 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
     static const int variant = getenv("DALI_HIP_GEMM_VARIANT") ? atoi(getenv("DALI_HIP_GEMM_VARIANT")) : 0;
     // >0: that many shares of the inner extent through the streaming kernel for every product it takes; <0: never
     static const int stream_env = getenv("DALI_HIP_GEMM_STREAM") ? atoi(getenv("DALI_HIP_GEMM_STREAM")) : 0;
-    const bool stream_fits = vec && g.nseg <= 2 && !g.map_on && !rows_may_overlap && (g.nseg == 1 || (g.seg[0].lda == g.seg[1].lda && g.seg[0].ldb == g.seg[1].ldb));
+    const bool stream_fits = vec && g.nseg <= 2 && !g.map_on && !rows_may_overlap;
     if (stream_env > 0 && stream_fits) {
         const int st = stream_product(g, ta, tb, stream_env);
         if (st >= 0) return st;
@@ -1164,31 +1196,33 @@ int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx
     if (ensure_init()) return DALI_HIP_ERROR;
     if (batch <= 0 || input <= 0 || hidden <= 0) return fail("lstm_step: extents must be positive (batch=%d, input=%d, hidden=%d)", batch, input, hidden);
     if (!X || !Hprev || !Cprev || !W || !U || !bias || !Cout || !Hout) return fail("lstm_step: NULL argument");
-    const bool ok = hidden % 64 == 0 && input % 64 == 0 && ldx == ldh && ldw == ldu && ldx % 4 == 0 && ldw % 4 == 0 && ldx >= input &&
-                    ldh >= hidden && ldw >= 4 * hidden && aligned16(X) && aligned16(Hprev) && aligned16(W) && aligned16(U) &&
-                    (size_t)64 * ldw * sizeof(float) + (size_t)4 * hidden * sizeof(float) < ((size_t)1 << 32) &&
-                    ((size_t)batch * ldx + 64) * sizeof(float) < ((size_t)1 << 32);
+    const bool ok = hidden % 64 == 0 && input % 64 == 0 && ldx % 4 == 0 && ldh % 4 == 0 && ldw % 4 == 0 && ldu % 4 == 0 && ldx >= input &&
+                    ldh >= hidden && ldw >= 4 * hidden && ldu >= 4 * hidden && aligned16(X) && aligned16(Hprev) && aligned16(W) && aligned16(U) &&
+                    (size_t)64 * (ldw > ldu ? ldw : ldu) * sizeof(float) + (size_t)4 * hidden * sizeof(float) < ((size_t)1 << 32) &&
+                    ((size_t)batch * (ldx > ldh ? ldx : ldh) + 64) * sizeof(float) < ((size_t)1 << 32);
     if (!ok)
-        return fail("lstm_step: the fused kernel needs input and hidden sizes that are multiples of 64, 16-byte aligned operands and "
-                    "equal leading dimensions for X / Hprev and for W / U");
+        return fail("lstm_step: the fused kernel needs input and hidden sizes that are multiples of 64 and 16-byte aligned operands whose "
+                    "leading dimensions are multiples of 4");
     {
         const float* as[2] = {X, Hprev};
         const float* bs[2] = {W, U};
-        const int ks[2] = {input, hidden};
+        const int ks[2] = {input, hidden}, las[2] = {ldx, ldh}, lbs[2] = {ldw, ldu};
         // a batch whose tiles leave compute units idle: shares of the inner extent, one work item per compute unit; whoever
         // draws a tile's last ticket adds the shares and computes the gates (up to 64 rows of 1024: 32 -> 17-19 us, 128 rows: 35 -> 27 us)
         static const int share_env = getenv("DALI_HIP_LSTM_STEP_SHARES") ? atoi(getenv("DALI_HIP_LSTM_STEP_SHARES")) : 1;
         const int shares = share_env ? stream_shares((long)((batch + 63) / 64) * (4 * hidden / 64), (input + hidden) / 64) : 1;
         if (shares >= 2) {
-            const int r = sgemm_dma_stream(false, false, batch, 4 * hidden, 2, ks, as, bs, ldx, ldw, 1.0f, 0.0f, nullptr, 0, shares, device_cus(), bias, Cprev, Cout, Hout,
+            const int r = sgemm_dma_stream(false, false, batch, 4 * hidden, 2, ks, as, bs, las, lbs, 1.0f, 0.0f, nullptr, 0, shares, device_cus(), bias, Cprev, Cout, Hout,
                                            hidden);
             if (r < 0) return DALI_HIP_ERROR;
             if (r > 0) return DALI_HIP_OK;
         }
-        const int r = sgemm_dma(false, false, batch, 4 * hidden, 2, ks, as, bs, ldx, ldw, 1.0f, 0.0f, nullptr, 0, bias, Cprev, Cout, Hout, hidden);
+        const int r = sgemm_dma(false, false, batch, 4 * hidden, 2, ks, as, bs, las, lbs, 1.0f, 0.0f, nullptr, 0, bias, Cprev, Cout, Hout, hidden);
         if (r < 0) return DALI_HIP_ERROR;
         if (r > 0) return DALI_HIP_OK;
     }
+    // (the register-staged kernel below takes one pair of leading dimensions)
+    if (ldx != ldh || ldw != ldu) return fail("lstm_step: X / Hprev (or W / U) with different leading dimensions need the kernel that DALI_HIP_GEMM_DMA=0 switches off");
     GemmArgs g = {};
     g.nseg = 2;
     g.seg[0].A = X;

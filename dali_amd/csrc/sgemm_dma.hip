@@ -47,7 +47,7 @@ struct DmaArgs {
     const float* A[2];
     const float* B[2];
     int slabs[2];  // 64-deep slabs per term (the second is 0 for a single product)
-    int lda, ldb;
+    int lda[2], ldb[2];  // per term (x [batch, input] and h [batch, hidden] of an LSTM step have rows of different length)
     int M, N;
     float* C;
     int ldc;
@@ -79,7 +79,7 @@ __device__ __forceinline__ void wait_loads_all() { asm volatile("s_waitcnt vmcnt
 
 // TA: A stored as [K][M]; TB: B stored as [N][K]. 512 threads: waves 0-3 (wave set 0) and 4-7 (set 1) each cover the
 // 64x64 tile as 2x2 wave tiles of 32x32; set kw takes the k-groups (16 k) kw and kw + 2 of every slab.
-template <bool TA, bool TB, bool GATES>
+template <bool TA, bool TB, bool GATES, bool LD2>
 __global__ __launch_bounds__(512, 1) void sgemm_dma_kernel(DmaArgs g) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -109,35 +109,40 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_kernel(DmaArgs g) {
     // Sources of this wave's four loads per slab (byte offsets, constant over the kernel) and their LDS chunks.
     // Tiles that hang over the edge of C fetch the last valid row (or granule) instead: what they compute for rows and
     // columns outside C is never stored.
-    unsigned a_off[2], b_off[2], a_dst[2], b_dst[2];
+    // (the offsets of the second term, whose rows may be of another length, wait in a_next / b_next)
+    unsigned a_off[2], b_off[2], a_next[2], b_next[2], a_dst[2], b_dst[2];
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
         const int c = w + 8 * q;                         // 1 KiB chunk: LDS rows 4c .. 4c+3 of the slab
         const int r = 4 * c + (lane >> 4), s = lane & 15;  // LDS row and slot of this lane's piece
         if (!TA) {
             const int row = m0 + r < M ? m0 + r : M - 1;
-            a_off[q] = (unsigned)(((size_t)row * g.lda + 4 * ((s ^ r) & 15)) * sizeof(float));
+            a_off[q] = (unsigned)(((size_t)row * g.lda[0] + 4 * ((s ^ r) & 15)) * sizeof(float));
+            if (LD2) a_next[q] = (unsigned)(((size_t)row * g.lda[1] + 4 * ((s ^ r) & 15)) * sizeof(float));
         } else {
             int col = m0 + 4 * (s ^ ((c & 3) << 2));
             col = col < M ? col : M - 4;
-            a_off[q] = (unsigned)(((size_t)r * g.lda + col) * sizeof(float));
+            a_off[q] = (unsigned)(((size_t)r * g.lda[0] + col) * sizeof(float));
+            if (LD2) a_next[q] = (unsigned)(((size_t)r * g.lda[1] + col) * sizeof(float));
         }
         if (!TB) {
             const int gr = s ^ ((c & 3) << 2);
             int col = GATES ? (gr / 4) * g.H + hu_base + 4 * (gr % 4) : n0 + 4 * gr;
             col = col < N ? col : N - 4;
-            b_off[q] = (unsigned)(((size_t)r * g.ldb + col) * sizeof(float));
+            b_off[q] = (unsigned)(((size_t)r * g.ldb[0] + col) * sizeof(float));
+            if (LD2) b_next[q] = (unsigned)(((size_t)r * g.ldb[1] + col) * sizeof(float));
         } else {
             const int row = n0 + r < N ? n0 + r : N - 1;
-            b_off[q] = (unsigned)(((size_t)row * g.ldb + 4 * ((s ^ r) & 15)) * sizeof(float));
+            b_off[q] = (unsigned)(((size_t)row * g.ldb[0] + 4 * ((s ^ r) & 15)) * sizeof(float));
+            if (LD2) b_next[q] = (unsigned)(((size_t)row * g.ldb[1] + 4 * ((s ^ r) & 15)) * sizeof(float));
         }
         a_dst[q] = (unsigned)(c * 1024);
         b_dst[q] = (unsigned)(kBRegion + c * 1024);
     }
     const char* ap = (const char*)g.A[0];
     const char* bp = (const char*)g.B[0];
-    const long a_step = (TA ? (long)64 * g.lda : 64L) * (long)sizeof(float);
-    const long b_step = (TB ? 64L : (long)64 * g.ldb) * (long)sizeof(float);
+    long a_step = (TA ? (long)64 * g.lda[0] : 64L) * (long)sizeof(float);
+    long b_step = (TB ? 64L : (long)64 * g.ldb[0]) * (long)sizeof(float);
     const int slabs0 = g.slabs[0];
     const int n = slabs0 + g.slabs[1];
     int fj = 0;  // next slab to request
@@ -152,6 +157,15 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_kernel(DmaArgs g) {
         if (fj == slabs0) {
             ap = (const char*)g.A[1];
             bp = (const char*)g.B[1];
+            if (LD2) {
+                a_step = (TA ? (long)64 * g.lda[1] : 64L) * (long)sizeof(float);
+                b_step = (TB ? 64L : (long)64 * g.ldb[1]) * (long)sizeof(float);
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    a_off[q] = a_next[q];
+                    b_off[q] = b_next[q];
+                }
+            }
         }
     };
     issue(0);
@@ -355,7 +369,7 @@ struct StreamArgs {
     const float* A[2];
     const float* B[2];
     int slabs[2];
-    int lda, ldb;
+    int lda[2], ldb[2];  // per term (x [batch, input] and h [batch, hidden] of an LSTM step have rows of different length)
     int M, N;
     float* C;
     int ldc;
@@ -374,7 +388,7 @@ struct StreamArgs {
 constexpr int kFoldBytes = 16384;
 constexpr int kStreamLds = kDmaLds + kFoldBytes + 16;  // stages, exchange area, one flag
 
-template <bool TA, bool TB, bool GATES>
+template <bool TA, bool TB, bool GATES, bool LD2>
 __global__ __launch_bounds__(512, 1) void sgemm_dma_stream_kernel(StreamArgs g) {
     // (no static LDS beside this: the loads address LDS from offset 0)
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -418,9 +432,13 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_stream_kernel(StreamArgs g) 
         total += share_begin(z + 1) - share_begin(z);
     }
 
-    const long a_step = (TA ? (long)64 * g.lda : 64L) * (long)sizeof(float);
-    const long b_step = (TB ? 64L : (long)64 * g.ldb) * (long)sizeof(float);
-    unsigned a_off[2], b_off[2], a_dst[2], b_dst[2];
+    long a_step = (TA ? (long)64 * g.lda[0] : 64L) * (long)sizeof(float), b_step = (TB ? 64L : (long)64 * g.ldb[0]) * (long)sizeof(float);
+    auto set_steps = [&](int term) __attribute__((always_inline)) {
+        a_step = (TA ? (long)64 * g.lda[term] : 64L) * (long)sizeof(float);
+        b_step = (TB ? 64L : (long)64 * g.ldb[term]) * (long)sizeof(float);
+    };
+    // (the offsets of the second term, whose rows may be of another length, wait in a_next / b_next)
+    unsigned a_off[2], b_off[2], a_next[2], b_next[2], a_dst[2], b_dst[2];
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
         a_dst[q] = (unsigned)((w + 8 * q) * 1024);
@@ -441,26 +459,38 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_stream_kernel(StreamArgs g) 
             const int rr = 4 * c + (lane >> 4), s = lane & 15;
             if (!TA) {
                 const int row = m0 + rr < M ? m0 + rr : M - 1;
-                a_off[q] = (unsigned)(((size_t)row * g.lda + 4 * ((s ^ rr) & 15)) * sizeof(float));
+                a_off[q] = (unsigned)(((size_t)row * g.lda[0] + 4 * ((s ^ rr) & 15)) * sizeof(float));
+                if (LD2) a_next[q] = (unsigned)(((size_t)row * g.lda[1] + 4 * ((s ^ rr) & 15)) * sizeof(float));
             } else {
                 int col = m0 + 4 * (s ^ ((c & 3) << 2));
                 col = col < M ? col : M - 4;
-                a_off[q] = (unsigned)(((size_t)rr * g.lda + col) * sizeof(float));
+                a_off[q] = (unsigned)(((size_t)rr * g.lda[0] + col) * sizeof(float));
+                if (LD2) a_next[q] = (unsigned)(((size_t)rr * g.lda[1] + col) * sizeof(float));
             }
             if (!TB) {
                 const int gr = s ^ ((c & 3) << 2);
                 int col = GATES ? (gr / 4) * g.H + 16 * nt + 4 * (gr % 4) : n0 + 4 * gr;
                 col = col < N ? col : N - 4;
-                b_off[q] = (unsigned)(((size_t)rr * g.ldb + col) * sizeof(float));
+                b_off[q] = (unsigned)(((size_t)rr * g.ldb[0] + col) * sizeof(float));
+                if (LD2) b_next[q] = (unsigned)(((size_t)rr * g.ldb[1] + col) * sizeof(float));
             } else {
                 const int row = n0 + rr < N ? n0 + rr : N - 1;
-                b_off[q] = (unsigned)(((size_t)row * g.ldb + 4 * ((s ^ rr) & 15)) * sizeof(float));
+                b_off[q] = (unsigned)(((size_t)row * g.ldb[0] + 4 * ((s ^ rr) & 15)) * sizeof(float));
+                if (LD2) b_next[q] = (unsigned)(((size_t)row * g.ldb[1] + 4 * ((s ^ rr) & 15)) * sizeof(float));
             }
         }
         i_g = share_begin(z);
         i_n = share_begin(z + 1) - i_g;
         i_fj = 0;
         const bool second = i_g >= slabs0;  // (only with two terms; shares are cut from single products)
+        if (LD2) set_steps(second ? 1 : 0);
+        if (LD2 && second) {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                a_off[q] = a_next[q];
+                b_off[q] = b_next[q];
+            }
+        }
         ap = wave_uniform((const char*)(second ? g.A[1] : g.A[0]) + (long)(i_g - (second ? slabs0 : 0)) * a_step);
         bp = wave_uniform((const char*)(second ? g.B[1] : g.B[0]) + (long)(i_g - (second ? slabs0 : 0)) * b_step);
     };
@@ -476,6 +506,14 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_stream_kernel(StreamArgs g) 
         if (i_g == slabs0 && g.slabs[1] > 0) {
             ap = (const char*)g.A[1];
             bp = (const char*)g.B[1];
+            if (LD2) {
+                set_steps(1);
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    a_off[q] = a_next[q];
+                    b_off[q] = b_next[q];
+                }
+            }
         }
         if (i_fj == i_n) {
             ++i_r;
@@ -712,10 +750,10 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_stream_kernel(StreamArgs g) 
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
-template <bool TA, bool TB, bool GATES>
+template <bool TA, bool TB, bool GATES, bool LD2>
 int launch(const DmaArgs& g, dim3 grid) {
     static bool attribute_set = false;  // one flag per instantiation of this function template
-    auto kernel = sgemm_dma_kernel<TA, TB, GATES>;
+    auto kernel = sgemm_dma_kernel<TA, TB, GATES, LD2>;
     if (!attribute_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kDmaLds);
         if (e != hipSuccess) return fail("sgemm: cannot reserve %d bytes of LDS: %s", kDmaLds, hipGetErrorString(e));
@@ -730,21 +768,22 @@ int launch(const DmaArgs& g, dim3 grid) {
 
 // whole 64-deep slabs, 16-byte pieces that start on 16-byte boundaries and never straddle the end of a row, per-lane offsets
 // (relative to a pointer that walks along k) that fit 32 bits
-bool operands_fit(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb) {
+bool operands_fit(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, const int* lda, const int* ldb) {
     if (nseg < 1 || nseg > 2 || M < 1 || N < 1) return false;
-    if (lda % 4 != 0 || ldb % 4 != 0 || (ta && M % 4 != 0) || (!tb && N % 4 != 0)) return false;
+    if ((ta && M % 4 != 0) || (!tb && N % 4 != 0)) return false;
     for (int s = 0; s < nseg; ++s) {
+        if (lda[s] % 4 != 0 || ldb[s] % 4 != 0) return false;
         if (K[s] < 64 || K[s] % 64 != 0 || !aligned16(A[s]) || !aligned16(B[s])) return false;
-        const size_t a_span = ((size_t)(ta ? 64 : M) * lda + (ta ? M : 64)) * sizeof(float);
-        const size_t b_span = ((size_t)(tb ? N : 64) * ldb + (tb ? 64 : N)) * sizeof(float);
+        const size_t a_span = ((size_t)(ta ? 64 : M) * lda[s] + (ta ? M : 64)) * sizeof(float);
+        const size_t b_span = ((size_t)(tb ? N : 64) * ldb[s] + (tb ? 64 : N)) * sizeof(float);
         if (a_span >= ((size_t)1 << 32) || b_span >= ((size_t)1 << 32)) return false;
     }
     return true;
 }
 
-template <bool TA, bool TB, bool GATES>
+template <bool TA, bool TB, bool GATES, bool LD2>
 int launch_stream(const StreamArgs& g, int workgroups) {
-    auto kernel = sgemm_dma_stream_kernel<TA, TB, GATES>;
+    auto kernel = sgemm_dma_stream_kernel<TA, TB, GATES, LD2>;
     hipError_t e = reserve_dynamic_lds((const void*)kernel, kStreamLds);
     if (e != hipSuccess) return fail("sgemm: cannot reserve %d bytes of LDS: %s", kStreamLds, hipGetErrorString(e));
     hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(512), kStreamLds, stream(), g);
@@ -755,7 +794,7 @@ int launch_stream(const StreamArgs& g, int workgroups) {
 
 }  // namespace
 
-int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
+int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, const int* lda, const int* ldb,
                      float alpha, float beta, float* C, int ldc, int shares, int cus, const float* bias, const float* c_prev, float* c_out, float* h_out, int H) {
     static const int enabled = getenv("DALI_HIP_GEMM_DMA") ? atoi(getenv("DALI_HIP_GEMM_DMA")) : 1;
     if (!enabled || cus < 8 || !operands_fit(ta, tb, M, N, nseg, K, A, B, lda, ldb)) return 0;
@@ -767,8 +806,11 @@ int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, con
         g.slabs[s] = s < nseg ? K[s] / 64 : 0;
         slabs += g.slabs[s];
     }
-    g.lda = lda;
-    g.ldb = ldb;
+    for (int s = 0; s < 2; ++s) {
+        g.lda[s] = lda[s < nseg ? s : 0];
+        g.ldb[s] = ldb[s < nseg ? s : 0];
+    }
+    const bool ld2 = g.lda[0] != g.lda[1] || g.ldb[0] != g.ldb[1];  // (a kernel of its own: the common case keeps its registers)
     g.M = M;
     g.N = N;
     g.C = C;
@@ -796,15 +838,15 @@ int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, con
     if (items < workgroups) workgroups = (int)items;
     if (bias) {
         if (ta || tb || N != 4 * H || H % 16 != 0) return 0;
-        return launch_stream<false, false, true>(g, workgroups);
+        return ld2 ? launch_stream<false, false, true, true>(g, workgroups) : launch_stream<false, false, true, false>(g, workgroups);
     }
-    if (!ta && !tb) return launch_stream<false, false, false>(g, workgroups);
-    if (!ta && tb) return launch_stream<false, true, false>(g, workgroups);
-    if (ta && !tb) return launch_stream<true, false, false>(g, workgroups);
-    return launch_stream<true, true, false>(g, workgroups);
+    if (!ta && !tb) return ld2 ? launch_stream<false, false, false, true>(g, workgroups) : launch_stream<false, false, false, false>(g, workgroups);
+    if (!ta && tb) return ld2 ? launch_stream<false, true, false, true>(g, workgroups) : launch_stream<false, true, false, false>(g, workgroups);
+    if (ta && !tb) return ld2 ? launch_stream<true, false, false, true>(g, workgroups) : launch_stream<true, false, false, false>(g, workgroups);
+    return ld2 ? launch_stream<true, true, false, true>(g, workgroups) : launch_stream<true, true, false, false>(g, workgroups);
 }
 
-int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, int lda, int ldb,
+int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, const int* lda, const int* ldb,
               float alpha, float beta, float* C, int ldc, const float* bias, const float* c_prev, float* c_out, float* h_out, int H) {
     static const int enabled = getenv("DALI_HIP_GEMM_DMA") ? atoi(getenv("DALI_HIP_GEMM_DMA")) : 1;
     if (!enabled || !operands_fit(ta, tb, M, N, nseg, K, A, B, lda, ldb)) return 0;
@@ -815,8 +857,11 @@ int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const floa
         g.B[s] = s < nseg ? B[s] : nullptr;
         g.slabs[s] = s < nseg ? K[s] / 64 : 0;
     }
-    g.lda = lda;
-    g.ldb = ldb;
+    for (int s = 0; s < 2; ++s) {
+        g.lda[s] = lda[s < nseg ? s : 0];
+        g.ldb[s] = ldb[s < nseg ? s : 0];
+    }
+    const bool ld2 = g.lda[0] != g.lda[1] || g.ldb[0] != g.ldb[1];  // (a kernel of its own: the common case keeps its registers)
     g.M = M;
     g.N = N;
     g.C = C;
@@ -831,12 +876,12 @@ int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const floa
     dim3 grid((N + 63) / 64, (M + 63) / 64);
     if (gates) {
         if (ta || tb) return 0;
-        return launch<false, false, true>(g, grid);
+        return ld2 ? launch<false, false, true, true>(g, grid) : launch<false, false, true, false>(g, grid);
     }
-    if (!ta && !tb) return launch<false, false, false>(g, grid);
-    if (!ta && tb) return launch<false, true, false>(g, grid);
-    if (ta && !tb) return launch<true, false, false>(g, grid);
-    return launch<true, true, false>(g, grid);
+    if (!ta && !tb) return ld2 ? launch<false, false, false, true>(g, grid) : launch<false, false, false, false>(g, grid);
+    if (!ta && tb) return ld2 ? launch<false, true, false, true>(g, grid) : launch<false, true, false, false>(g, grid);
+    if (ta && !tb) return ld2 ? launch<true, false, false, true>(g, grid) : launch<true, false, false, false>(g, grid);
+    return ld2 ? launch<true, true, false, true>(g, grid) : launch<true, true, false, false>(g, grid);
 }
 
 }  // namespace dali_hip

@@ -1589,12 +1589,12 @@ CrossEntropyResult softmax_cross_entropy(const Array& logits, const Array& targe
 }
 
 // Whether the recurrent half of a sequence goes into one persistent launch: where the library expects that to beat a launch per
-// step of the fused step (answer 2); where the fused step does not apply (input size != hidden size: two products and a gate
+// step of the fused step (answer 2); where the fused step does not apply (an input or hidden size that is no multiple of 64: two products and a gate
 // kernel per step), wherever it is served up to the batch it was measured to win at against that form; `always`: wherever served.
 static bool persistent_wins(int Bn, int In, int H, bool always) {
     const int served = dali_hip_lstm_recurrent_persistent_supported(Bn, H);
     if (always) return served >= 1;
-    const bool fused_applies = H % 64 == 0 && In == H;
+    const bool fused_applies = H % 64 == 0 && In % 64 == 0;
     return served == 2 || (served == 1 && !fused_applies && Bn <= 96);
 }
 
@@ -1616,14 +1616,14 @@ LSTMState lstm_step(const Array& x, const Array& h, const Array& c, const Array&
     const bool small_off = small_env != nullptr && std::string(small_env) == "0";
     // (from 17 rows on, where the fused step applies, that one is faster: its inner extent is cut into one share per compute unit
     // and it takes 17.3-18.8 us for up to 64 rows of 1024, against 18.4-31.0 us here)
-    const bool fused_applies = H % 64 == 0 && In == H;
+    const bool fused_applies = H % 64 == 0 && In % 64 == 0;
     if (!fused_off && !small_off && !dry_run() && Bn <= (fused_applies ? 16 : 64) && H % 256 == 0 && H <= 1024 && In % 16 == 0 && (In + H) % 64 == 0 && dense(x) && dense(h) &&
         dense(c) && dense(W) && dense(U) && dense(b) && x.offset() % 4 == 0 && h.offset() % 4 == 0 && W.offset() % 4 == 0 && U.offset() % 4 == 0 && c.offset() % 4 == 0) {
         Array c_new({Bn, H}, DTYPE_FLOAT), h_new({Bn, H}, DTYPE_FLOAT);
         lstm_step_small(x, h, c, W, U, b, c_new, h_new);
         return {c_new, h_new};
     }
-    if (!fused_off && !dry_run() && H % 64 == 0 && In == H && dense(x) && dense(h) && dense(c) && dense(W) && dense(U) && dense(b) &&
+    if (!fused_off && !dry_run() && H % 64 == 0 && In % 64 == 0 && dense(x) && dense(h) && dense(c) && dense(W) && dense(U) && dense(b) &&
         x.offset() % 4 == 0 && h.offset() % 4 == 0 && W.offset() % 4 == 0 && U.offset() % 4 == 0) {
         Array c_new({Bn, H}, DTYPE_FLOAT), h_new({Bn, H}, DTYPE_FLOAT);
         lstm_step_fused(x, h, c, W, U, b, c_new, h_new);
@@ -1657,7 +1657,7 @@ LSTMSequence lstm_sequence(const Array& xs, const Array& h0, const Array& c0, co
     Array seq = xs.is_buffer() && xs.contiguous_memory() ? xs : xs.ascontiguousarray();
     Array hs({T, Bn, H}, DTYPE_FLOAT);
     Array cells[2] = {Array({Bn, H}, DTYPE_FLOAT), Array({Bn, H}, DTYPE_FLOAT)};
-    const bool fused = !fused_off && !dry_run() && H % 64 == 0 && In == H && dense(seq) && dense(h0) && dense(c0) && dense(W) && dense(U) && dense(b) &&
+    const bool fused = !fused_off && !dry_run() && H % 64 == 0 && In % 64 == 0 && dense(seq) && dense(h0) && dense(c0) && dense(W) && dense(U) && dense(b) &&
                        W.ndim() == 2 && U.ndim() == 2 && b.ndim() == 1 && W.shape()[0] == In && W.shape()[1] == 4 * H && U.shape()[0] == H &&
                        U.shape()[1] == 4 * H && b.shape()[0] == 4 * H && seq.offset() % 4 == 0 && h0.offset() % 4 == 0 && W.offset() % 4 == 0 &&
                        U.offset() % 4 == 0 && ((int64_t)Bn * H) % 4 == 0;

@@ -252,7 +252,8 @@ int dali_hip_sgemm_terms(int nterms, int transA, int transB, int M, int N, const
  * (dali/layers/lstm.cpp:226-261 with StackedInputLayer::activate, dali/layers/layers.cpp:159-161). The MFMA tile of
  * a workgroup gathers the four gate columns of sixteen hidden units, so the pre-activations never leave the chip;
  * every operation is rounded as in the two-launch form (dali_hip_sgemm_pair followed by the generated gate
- * kernel). Needs input and hidden to be multiples of 64, 16-byte aligned operands, ldx == ldh and ldw == ldu;
+ * kernel). Needs input and hidden to be multiples of 64 and 16-byte aligned operands whose leading dimensions are
+ * multiples of 4 (X and Hprev, W and U may differ in theirs: the input size need not equal the hidden size);
  * otherwise it fails and the caller uses the two-launch form. Cprev, Cout, Hout are dense [batch, hidden].
  */
 int dali_hip_lstm_step(int batch, int input, int hidden, const float* X, int ldx, const float* Hprev, int ldh,
