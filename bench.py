@@ -401,6 +401,15 @@ def main():
                                                  "gemm_pair_us": round(gemm_us, 2),
                                                  "gemm_TFLOP/s": round(flops / gemm_us / 1e6, 2),
                                                  "gemm_frac_fp32_mfma": round(flops / gemm_us / 1e6 / MFMA_FP32_PEAK_TFLOPS, 4)}
+        # the same step with an input size other than the hidden size (rows of x and of h differ in length)
+        X5 = D.Array.from_numpy(np.random.RandomState(24).randn(B, 512).astype(np.float32))
+        W5 = D.Array.from_numpy(np.random.RandomState(25).uniform(-lim, lim, (512, 4096)).astype(np.float32))
+        with D.Recording() as rec5:
+            op.lstm_step(X5, Hp, Cp, W5, U, bias)
+        us5 = time_recording(rec5, 200, 10)
+        configs["c5_lstm_step_256x1024x1024"]["step_input512_hidden1024"] = {"us": round(us5, 2), "launches": rec5.launches,
+                                                                             "TFLOP/s": round(2.0 * B * (512 + H) * 4 * H / us5 / 1e6, 2)}
+        del X5, W5, rec5
         # the same step along a sequence of 32: fused launches chained through one [T, B, H] buffer
         Xs = D.Array.from_numpy(np.random.RandomState(23).randn(32, B, H).astype(np.float32))
         with D.Recording() as srec:
@@ -603,6 +612,27 @@ def main():
             nxt[tag] = {"us": round(us, 2), "GB/s": round(nb / us / 1e3, 1), "frac_hbm": round(nb / us / 1e3 / HBM_PEAK_GBS, 4), "launches": rec.launches,
                         "kernel": D.last_kernel_kinds()}
             del xs_, rec
+        # few very long rows of a length that divides into nothing: the row kernel cuts them into pieces (bytes = one read)
+        few = D.Array.from_numpy(np.random.RandomState(19).randn(7, 9999999).astype(np.float32))
+        rows_few = {}
+        for tag, build in (("sum_axis1", lambda: op.sum(few, [1])), ("argmax_axis1", lambda: op.argmax(few, 1))):
+            with D.Recording() as rec:
+                build().eval()
+            us = time_recording(rec, 20)
+            nb = 4.0 * 7 * 9999999
+            rows_few[tag] = {"us": round(us, 2), "GB/s": round(nb / us / 1e3, 1), "frac_hbm": round(nb / us / 1e3 / HBM_PEAK_GBS, 4), "launches": rec.launches}
+            del rec
+        nxt["reductions_few_long_rows_7x9999999"] = rows_few
+        del few
+        # a matrix times a column: the rows streamed once
+        mv_a = D.Array.from_numpy(np.random.RandomState(20).randn(4096, 4096).astype(np.float32))
+        mv_x = D.Array.from_numpy(np.random.RandomState(21).randn(4096, 1).astype(np.float32))
+        with D.Recording() as rec:
+            op.dot(mv_a, mv_x).eval()
+        us = time_recording(rec, 50)
+        nxt["dot_matrix_column_4096x4096"] = {"us": round(us, 2), "GB/s": round(4096 * 4096 * 4 / us / 1e3, 1), "frac_hbm": round(4096 * 4096 * 4 / us / 1e3 / HBM_PEAK_GBS, 4),
+                                              "launches": rec.launches}
+        del mv_a, mv_x, rec
         sm = D.Array.from_numpy(np.random.RandomState(17).uniform(0.5, 1.5, (8192, 8192)).astype(np.float32))
         with D.Recording() as rec:
             op.cumsum(sm).eval()
