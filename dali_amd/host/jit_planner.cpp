@@ -47,6 +47,9 @@ static bool is_plain_matmul(const Array& a) { return a.expression()->kind == Kin
 //    registers (extent up to 2048) the softmax is computed in one pass by a kernel of the library and arrives as a
 //    buffer; otherwise the column kernel carries (maximum, sum) pairs, so the data is read once for both instead of once
 //    for the maxima and once more for the sums.
+// set while a softmax over few long rows evaluates its statistics: try_segmented_reduce then cuts rows into pieces at any size
+static bool g_segment_whatever_the_size = false;
+
 static Array expand_softmax(Array x, int axis) {
     static const bool staged_off = env_int("DALI_HIP_SOFTMAX_STAGED", 1) == 0;
     const std::vector<int> shape = x.shape();
@@ -75,15 +78,26 @@ static Array expand_softmax(Array x, int axis) {
             // the same rows at a length that does not divide that way: the row kernel cuts them into pieces itself, once for
             // the maxima and once for the sums of the exponentials (see try_segmented_reduce)
             static const bool pieces_off = env_int("DALI_HIP_SEGMENTED_REDUCE", 1) == 0;
-            if (!pieces_off && rows < 256 && Cx >= 65536 && rows * 8 <= 2048 && Cx / 8 >= 8192) {
+            // (five launches against one whose workgroups walk their rows three times: worth it for rows that are few for their
+            // length, [2,100003] 22.5 -> 13.5 us, [32,131073] 29.9 -> 18.5 us, but [64,65537] 13.5 -> 18.1 us; and whenever the rows
+            // together are more than the caches keep between the passes)
+            const bool few_for_their_length = (double)rows < 75.0 - 3.75e6 / (double)Cx;
+            if (!pieces_off && rows < 256 && Cx >= 65536 && rows * 8 <= 2048 && Cx / 8 >= 8192 && (n * 4 >= ((int64_t)64 << 20) || few_for_their_length)) {
                 if (!x.is_buffer()) x = materialize(x);
                 if (!x.contiguous_memory()) x = x.ascontiguousarray();
                 Array x2 = x.reshape({(int)rows, (int)Cx});
-                Array M = op::max(x2, {-1}, false);
-                evaluate({M});
-                Array L = op::sum(op::exp(op::subtract(x2, M.reshape({(int)rows, 1}))), {-1}, false);
-                evaluate({L});
-                return op::eltdiv(op::exp(op::subtract(x, M.reshape(keep))), L.reshape(keep));
+                g_segment_whatever_the_size = true;  // (the rule of the softmax has been applied; the reductions have another)
+                try {
+                    Array M = op::max(x2, {-1}, false);
+                    evaluate({M});
+                    Array L = op::sum(op::exp(op::subtract(x2, M.reshape({(int)rows, 1}))), {-1}, false);
+                    evaluate({L});
+                    g_segment_whatever_the_size = false;
+                    return op::eltdiv(op::exp(op::subtract(x, M.reshape(keep))), L.reshape(keep));
+                } catch (...) {
+                    g_segment_whatever_the_size = false;
+                    throw;
+                }
             }
         } else if (n >= (1 << 16)) {
             int64_t inner = 1, outer = 1;
@@ -396,6 +410,10 @@ static bool try_segmented_reduce(const DestSpec& spec) {
     if (n == 0 || C_last < (1 << 16)) return false;
     const int64_t rows = n / C_last;
     if (rows >= 256) return false;
+    // Two or three launches against one: worth it once a row takes a workgroup longer than the extra launches (from about 200000
+    // elements on: [4,262145] 8.5 -> 6.1 us, [8,131073] 5.2 -> 6.4 us) or the rows together are more than the caches keep between
+    // two uses, where a workgroup streams its row from memory at a fortieth of what the device can ([64,1048577]: 131 -> 41 us).
+    if (!g_segment_whatever_the_size && C_last < 200000 && n * 4 < ((int64_t)64 << 20)) return false;
     int S = 1;
     while (S * 2 * rows <= 2048 && C_last / (S * 2) >= 8192) S *= 2;
     if (S < 4) return false;

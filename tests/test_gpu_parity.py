@@ -869,7 +869,7 @@ def test_rows_not_aligned_to_the_vector(gpu, D, O, rng, cols):
     assert np.array_equal((arr(D, xi)[:, 1:] * 3).numpy(), xi[:, 1:] * 3)
 
 
-@pytest.mark.parametrize("shape", [(7, 300001), (3, 1000003), (1, 524291), (2, 3, 131075), (31, 65537), (5, 262144)])
+@pytest.mark.parametrize("shape", [(7, 300001), (3, 1000003), (1, 524291), (2, 3, 200003), (250, 70001), (5, 262144)])
 def test_few_long_rows_cut_into_pieces_by_the_row_kernel(gpu, D, O, rng, shape):
     """Reductions along few very long rows whose length does not divide into equal aligned pieces, and the position of the
     best element at any length (reducer_operation.cpp:98-156,193-228): the row kernel cuts every row into pieces, a second
@@ -904,12 +904,12 @@ def test_few_long_rows_cut_into_pieces_by_the_row_kernel(gpu, D, O, rng, shape):
     assert am.dtype == np.int32 and np.array_equal(am, x.argmax(-1)) and np.array_equal(am, O.arg_axis_reduce(O.MAX, rows, 1).reshape(am.shape))
     assert np.array_equal(op.argmin(X, -1).numpy(), O.arg_axis_reduce(O.MIN, rows, 1).reshape(am.shape))
     # an expression over the rows reduces the same way once its leaves are buffers
-    y = np.abs(x) * 1e-3 + 1.0
-    close(op.prod(arr(D, y[..., :65600]), [-1]).numpy(), y[..., :65600].astype(np.float64).prod(-1), rtol=65600 * 2.0 ** -24 * 0.05)  # (a twentieth of the a-priori bound)
+    y = np.exp(np.clip(x, -4, 4) * 0.01).astype(np.float32)  # (factors within 1e-4 of one would lose their second-order terms to rounding in any tree)
+    close(op.prod(arr(D, y), [-1]).numpy(), y.astype(np.float64).prod(-1), rtol=C * 2.0 ** -24 * 0.05)  # (a twentieth of the a-priori bound)
     # softmax over such rows: maxima in pieces, sums of exponentials in pieces, the quotient as a lazy map
     k0 = D.jit_stats()["kernels"]
     s = op.softmax(X).numpy()
-    if C % 32 != 0 or rows.shape[0] * 8 > 2048:
+    if C % 32 != 0:
         assert D.jit_stats()["kernels"] - k0 == 5 and D.last_kernel_kinds().endswith(("map2d", "flat"))  # (flat: a single row)
     e = np.exp(x64 - x64.max(-1, keepdims=True))
     close(s, e / e.sum(-1, keepdims=True), rtol=1e-5, atol=1e-12)
@@ -1109,7 +1109,10 @@ def test_fused_softmax_matches_oracle(gpu, D, O, rng, shape):
     x = (rng.randn(*shape) * 3).astype(np.float32)
     before = D.jit_stats()["kernels"]
     s = D.op.softmax(arr(D, x)).numpy()
-    assert D.jit_stats()["kernels"] - before == 1 and D.last_kernel_kinds() == "row"
+    if shape == (2, 100003):  # rows that are few for their length: maxima and sums of exponentials over pieces of the rows, then the quotient
+        assert D.jit_stats()["kernels"] - before == 5 and D.last_kernel_kinds().endswith("map2d")
+    else:
+        assert D.jit_stats()["kernels"] - before == 1 and D.last_kernel_kinds() == "row"
     x64 = x.astype(np.float64)
     e = np.exp(x64 - x64.max(-1, keepdims=True))
     close(s, e / e.sum(-1, keepdims=True), rtol=1e-5, atol=1e-12)  # fp64 truth
