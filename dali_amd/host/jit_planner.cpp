@@ -351,8 +351,9 @@ static bool try_two_stage_reduce(const DestSpec& spec) {
     if (n == 0 || C_last == 0) return false;
     const int64_t rows = n / C_last;
     if (arg.contiguous_memory()) {
-        // few long rows
+        // few long rows (from the size on at which a second launch pays, see try_segmented_reduce)
         if (rows >= 256 || C_last < (1 << 16)) return false;
+        if (C_last < 200000 && n * 4 < ((int64_t)64 << 20)) return false;
         int S = 1;
         while (S * 2 * rows <= 2048 && C_last % (S * 2 * 4) == 0 && C_last / (S * 2) >= 8192) S *= 2;
         if (S < 4) return false;
