@@ -948,10 +948,16 @@ static int stream_product(const GemmArgs& g, bool ta, bool tb, int shares) {
 // unit, what is left of the inner extent by a checked launch that adds to the result. -1: not a case for it.
 static int tiles128_product(const GemmArgs& g, bool ta, bool tb) {
     const GemmSeg& sg = g.seg[0];
-    const int kw = sg.K / 32 * 32, kr = sg.K - kw;
-    if (kw == 0) return -1;
     const int cus = device_cus();
     if (cus <= 0) return -1;
+    if (sg.K % 32 != 0 && sg.K % 4 == 0 && sg.K > 32) {
+        // the kernel fills a partly filled last slab with zeros as it arrives (no second launch for the rest)
+        const int r = sgemm_dma128(ta, tb, g.M, g.N, sg.K, sg.A, sg.lda, sg.B, sg.ldb, g.alpha, g.beta, g.C, g.ldc, cus);
+        if (r < 0) return DALI_HIP_ERROR;
+        if (r > 0) return DALI_HIP_OK;
+    }
+    const int kw = sg.K / 32 * 32, kr = sg.K - kw;
+    if (kw == 0) return -1;
     const int r = sgemm_dma128(ta, tb, g.M, g.N, kw, sg.A, sg.lda, sg.B, sg.ldb, g.alpha, g.beta, g.C, g.ldc, cus);
     if (r < 0) return DALI_HIP_ERROR;
     if (r == 0) return -1;

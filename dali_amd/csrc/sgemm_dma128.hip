@@ -41,7 +41,8 @@ constexpr int kDeviceScope = 16;                 // cache policy of a buffer acc
 struct Args128 {
     const float* A;
     const float* B;
-    int slabs;  // 32-deep slabs of the inner extent
+    int slabs;  // 32-deep slabs of the inner extent, the last one partly filled when ...
+    int ktail;  // ... the inner extent is no multiple of 32: values of k in that slab (a multiple of 4), 0 = the slab is whole
     int lda, ldb;
     int M, N;
     float* C;
@@ -81,7 +82,10 @@ __device__ __forceinline__ void wait_all() { asm volatile("s_waitcnt vmcnt(0)" :
 // in which the pieces of B deliver theirs), still four row classes to a 16-byte read.
 // SHARE: the launch cuts left-over tiles into shares (the code that publishes and adds them up is left out of the other form,
 // where it would sit, unused, behind every slab of the loop).
-template <bool TA, bool TB, int TM, bool SHARE>
+// KT: the last slab of the inner extent is partly filled. Its loads fetch, for the values of k past the end, a piece that exists
+// (the first of the same row, or row 0 of the slab: nothing outside the operands is read), and every lane overwrites what it
+// fetched that way with zeros once its loads have landed, before the barrier that releases the slab.
+template <bool TA, bool TB, int TM, bool SHARE, bool KT>
 __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     static_assert(TM == 128 || (TM == 64 && !TA), "64-row tiles are built for A stored [M][K]");
     constexpr bool OUTER = TA && !TB;  // both operands run across memory rows: one k-quad per step
@@ -197,11 +201,35 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
         ap = wave_uniform((const char*)g.A + (long)j0 * a_step);
         bp = wave_uniform((const char*)g.B + (long)j0 * b_step);
     };
+    // (KT) whether this lane's piece of load q lies past the end of the partly filled slab, and how far in front of it (bytes) the
+    // piece fetched in its place is
+    auto past_end = [&](int q, bool of_b, unsigned* back) __attribute__((always_inline)) -> bool {
+        const int c = w + 8 * q;
+        if (of_b ? TB : !TA) {  // the eight pieces of an LDS row run along k
+            const int r_in = 8 * c + (lane >> 3), pk = (lane & 7) ^ ((r_in >> 1) & 7);
+            *back = 16u * (unsigned)pk;
+            return 4 * pk >= g.ktail;
+        }
+        const int k = 2 * c + (lane >> 5);
+        *back = (unsigned)k * (unsigned)(of_b ? g.ldb : g.lda) * 4u;
+        return k >= g.ktail;
+    };
+    unsigned tail_stages = 0;  // (KT) bit s: the slab in stage s is the partly filled one
     auto issue = [&](int stage) __attribute__((always_inline)) {
-        load_to_lds(a_dst[0] + stage * kStageBytes, a_off[0], ap);
-        if (AQ > 1) load_to_lds(a_dst[1] + stage * kStageBytes, a_off[1], ap);
-        load_to_lds(b_dst[0] + stage * kStageBytes, b_off[0], bp);
-        load_to_lds(b_dst[1] + stage * kStageBytes, b_off[1], bp);
+        if (KT && i_j == n - 1) {
+            unsigned back;
+            tail_stages |= 1u << stage;
+            load_to_lds(a_dst[0] + stage * kStageBytes, past_end(0, false, &back) ? a_off[0] - back : a_off[0], ap);
+            if (AQ > 1) load_to_lds(a_dst[1] + stage * kStageBytes, past_end(1, false, &back) ? a_off[1] - back : a_off[1], ap);
+            load_to_lds(b_dst[0] + stage * kStageBytes, past_end(0, true, &back) ? b_off[0] - back : b_off[0], bp);
+            load_to_lds(b_dst[1] + stage * kStageBytes, past_end(1, true, &back) ? b_off[1] - back : b_off[1], bp);
+        } else {
+            if (KT) tail_stages &= ~(1u << stage);
+            load_to_lds(a_dst[0] + stage * kStageBytes, a_off[0], ap);
+            if (AQ > 1) load_to_lds(a_dst[1] + stage * kStageBytes, a_off[1], ap);
+            load_to_lds(b_dst[0] + stage * kStageBytes, b_off[0], bp);
+            load_to_lds(b_dst[1] + stage * kStageBytes, b_off[1], bp);
+        }
         ++i_j;
         ap += a_step;
         bp += b_step;
@@ -421,6 +449,16 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
             c_j = c_j0;
         }
     };
+    auto zero_past_end = [&](int stage) __attribute__((always_inline)) {
+        const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+        unsigned back;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            if (q < AQ && past_end(q, false, &back)) *(floatx4*)(lds + a_dst[q] + stage * kStageBytes + 16 * lane) = zero;
+            if (past_end(q, true, &back)) *(floatx4*)(lds + b_dst[q] + stage * kStageBytes + 16 * lane) = zero;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
     // Slab i lives in stage i % 4. The barrier inside slab i is for slab i+1 (its loads were issued two slabs earlier); behind
     // it the buffer of slab i-1 is free and takes slab i+3.
     auto slab_step = [&](auto ST, auto H1, auto H2, auto H3) __attribute__((always_inline)) {
@@ -436,6 +474,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
                 mfma_tn(kk & 1);
                 if (kk == 1 && has1) {
                     if (has2) wait_but<LPS>(); else wait_all();
+                    if (KT && ((tail_stages >> ((st + 1) % 4)) & 1u)) zero_past_end((st + 1) % 4);
                     __builtin_amdgcn_s_barrier();
                 }
                 if (kk == 2 && has3) issue((st + 3) % 4);
@@ -447,6 +486,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
             mfma_nn(0, 0);
             if (has1) {
                 if (has2) wait_but<LPS>(); else wait_all();
+                if (KT && ((tail_stages >> ((st + 1) % 4)) & 1u)) zero_past_end((st + 1) % 4);
                 __builtin_amdgcn_s_barrier();
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -493,6 +533,7 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
     if (total > 2) wait_but<2 * LPS>();
     else if (total > 1) wait_but<LPS>();
     else wait_all();
+    if (KT && (tail_stages & 1u)) zero_past_end(0);  // (a share that is the last slab of its tile alone)
     __builtin_amdgcn_s_barrier();
     load_ops(S0{}, 0, 0);
     int i = 0;
@@ -513,9 +554,9 @@ __global__ __launch_bounds__(512, 1) void sgemm_dma128_kernel(Args128 g) {
 
 bool aligned_to(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-template <bool TA, bool TB, int TM, bool SHARE>
+template <bool TA, bool TB, int TM, bool SHARE, bool KT = false>
 int launch128(const Args128& g, int workgroups) {
-    auto kernel = sgemm_dma128_kernel<TA, TB, TM, SHARE>;
+    auto kernel = sgemm_dma128_kernel<TA, TB, TM, SHARE, KT>;
     hipError_t e = reserve_dynamic_lds((const void*)kernel, kLdsBytes);
     if (e != hipSuccess) return fail("sgemm: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
     hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(512), kLdsBytes, stream(), g);
@@ -528,7 +569,8 @@ int launch128(const Args128& g, int workgroups) {
 
 int sgemm_dma128(bool ta, bool tb, int M, int N, int K, const float* A, int lda, const float* B, int ldb, float alpha, float beta, float* C, int ldc, int cus) {
     static const int enabled = getenv("DALI_HIP_GEMM_DMA128") ? atoi(getenv("DALI_HIP_GEMM_DMA128")) : 1;
-    if (!enabled || cus < 8 || M < 1 || N < 4 || K < 32 || K % 32 != 0) return 0;
+    static const int tails_on = getenv("DALI_HIP_GEMM_DMA_TAILS") ? atoi(getenv("DALI_HIP_GEMM_DMA_TAILS")) : 1;
+    if (!enabled || cus < 8 || M < 1 || N < 4 || K < 32 || K % (tails_on ? 4 : 32) != 0) return 0;
     // 16-byte pieces that start on 16-byte boundaries and never straddle the end of a row; with B stored [K][N] pairs of results
     // are stored as 8 bytes
     if (lda % 4 != 0 || ldb % 4 != 0 || (ta && (M % 4 != 0 || M < 4))) return 0;
@@ -541,7 +583,9 @@ int sgemm_dma128(bool ta, bool tb, int M, int N, int K, const float* A, int lda,
     Args128 g = {};
     g.A = A;
     g.B = B;
-    g.slabs = K / 32;
+    g.slabs = (K + 31) / 32;
+    g.ktail = K % 32;
+    const bool kt = g.ktail != 0;
     g.lda = lda;
     g.ldb = ldb;
     g.M = M;
@@ -572,7 +616,16 @@ int sgemm_dma128(bool ta, bool tb, int M, int N, int K, const float* A, int lda,
     g.min_frag = 2;
     g.counters = (unsigned int*)workspace();
     g.partials = (float*)(workspace() + kWorkspaceCounterBytes);
-    if (low) return launch128<false, false, 64, false>(g, workgroups);
+    if (low) return kt ? launch128<false, false, 64, false, true>(g, workgroups) : launch128<false, false, 64, false>(g, workgroups);
+    if (kt) {
+        // (whole tiles only: a product whose left-over tiles would be cut into shares has its whole slabs done that way and the
+        // rest of the inner extent added by the caller)
+        if (share) return 0;
+        if (!ta && !tb) return launch128<false, false, 128, false, true>(g, workgroups);
+        if (ta && !tb) return launch128<true, false, 128, false, true>(g, workgroups);
+        if (!ta && tb) return launch128<false, true, 128, false, true>(g, workgroups);
+        return launch128<true, true, 128, false, true>(g, workgroups);
+    }
     if (share) {
         if (!ta && !tb) return launch128<false, false, 128, true>(g, workgroups);
         if (ta && !tb) return launch128<true, false, 128, true>(g, workgroups);

@@ -487,7 +487,7 @@ def test_sgemm_random_shapes_for_the_kernels_that_walk_work_items(gpu):
         elif kind == 1:  # between half a round and a round of 64x64 tiles, and a little more than whole rounds of 128x128 tiles
             M, N, K = pick([384, 768, 1100]), pick([1536, 2052, 4096]), pick([1024, 2048, 2080])
         elif kind == 2:  # many 128x128 tiles
-            M, N, K = pick([1536, 2052, 3072, 4100]), pick([1536, 2048, 2304]), pick([96, 256, 548, 2048])
+            M, N, K = pick([1536, 2052, 3072, 4100]), pick([1536, 2048, 2304]), pick([96, 132, 256, 548, 1000, 2048])
         else:            # wide and short
             M, N, K = pick([256, 640, 1024]), pick([16000, 24704, 32000]), pick([64, 160, 256])
         ta, tb = int(rng.randint(2)), int(rng.randint(2))
