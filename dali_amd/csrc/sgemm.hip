@@ -1119,6 +1119,18 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
     long tiles64 = (long)((M + 63) / 64) * ((N + 63) / 64);
     static const int split_env = getenv("DALI_HIP_GEMM_SPLITK") ? atoi(getenv("DALI_HIP_GEMM_SPLITK")) : 0;
     int split_k = split_env > 0 ? split_env : 1;
+    {
+        // a short inner extent that ends in a partly filled slab: one launch of the kernel that fills the slab up, rather than
+        // shares of the whole slabs and a second launch for the rest ([256,300].[300,2048]: 17.0 -> 11 us)
+        int nslab64 = 0;
+        bool partly = false, pieces = true;
+        for (int s = 0; s < g.nseg; ++s) {
+            nslab64 += (g.seg[s].K + 63) / 64;
+            partly = partly || g.seg[s].K % 64 != 0;
+            pieces = pieces && g.seg[s].K % 4 == 0 && g.seg[s].K >= 64;
+        }
+        if (split_env == 0 && variant == 0 && stream_env == 0 && stream_fits && partly && pieces && nslab64 <= 16) return run_tile<64, 64, 64, 2, 2>(g, ta, tb, vec, 1);
+    }
     if (split_env == 0 && variant == 0 && stream_env == 0 && stream_fits && tiles64 > 128) {
         // between half a round and a whole one of 64x64 tiles: shares that fill whole rounds (384x1536 over K = 4096, 144 tiles: 66 -> 58 us)
         int nslab64 = 0;
@@ -1129,7 +1141,12 @@ static int sgemm_rowmajor(int nseg, bool ta, bool tb, int M, int N, const int* K
             if (st >= 0) return st;
         }
     }
-    if (split_env == 0 && variant == 0 && tiles64 <= 128) {
+    // (an inner extent of up to four slabs, or up to eight with a tile for half the compute units: nothing to share; one launch of the
+    // kernel that loads into LDS takes [512,256].[256,1024] in 7.1 us against 9.5 us in two shares, [256,512].[512,2048] in 10.9 against 12.6)
+    int nslab64_all = 0;
+    for (int s = 0; s < g.nseg; ++s) nslab64_all += (g.seg[s].K + 63) / 64;
+    const bool nothing_to_share = nslab64_all <= 4 || (tiles64 >= 128 && nslab64_all <= 8);
+    if (split_env == 0 && variant == 0 && tiles64 <= 128 && !nothing_to_share) {
         // A few tiles over a long inner extent (the weight gradient of a convolution: [out, window] from tens of
         // thousands of patches) would leave most of the device idle: about two workgroups per CU, folded in a fixed
         // order by the workgroup that finishes last.
