@@ -262,7 +262,7 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
             const std::string t = ctype(P.nodes[P.nodes[totals[k]->total_red].args[0]].dtype);
             ss << "    dali_publish((" << t << "*)(slots + ((size_t)" << k << " * gridDim.x + blockIdx.x) * 8), tot" << k << ");\n";
         }
-        ss << "    is_last = dali_take_ticket(&counters[0]) == gridDim.x - 1;\n  }\n";
+        ss << "    is_last = dali_last_arrival(counters, blockIdx.x, gridDim.x);\n  }\n";
     };
     auto emit_totals_fold = [&]() {
         ss << "  __syncthreads();\n  if (!is_last) return;\n";
