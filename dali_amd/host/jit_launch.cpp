@@ -10,7 +10,7 @@ namespace jit {
 const char* device_prelude() { return codegen::kDevicePrelude; }
 
 // Bump when generated code changes meaning, so stale on-disk code objects are not reused.
-const char* const kCodegenVersion = "dali-hip-codegen-37";
+const char* const kCodegenVersion = "dali-hip-codegen-38";
 
 static std::unordered_map<uint64_t, bool>& loaded_hashes() {
     static std::unordered_map<uint64_t, bool> m;

@@ -166,8 +166,65 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
         o << "  }\n  }\n";
     };
 
+    // Rows that are streamed (too long for the registers): a maximum followed by the sum of exp(x - maximum), the statistics
+    // of a softmax or a log-sum-exp, are taken in ONE walk over the row. A thread keeps the largest value it has met and the
+    // sum of the exponentials relative to it, and scales the sum when a larger value arrives; the threads' sums are scaled
+    // to the row's maximum before they are added. The row is then read twice in all (statistics, output) instead of three times
+    // ([1024,128256]: 361 -> 292 us, [512,151936]: 209 -> 167 us).
+    int online_max = -1, online_sum = -1, online_arg = -1;
+    static const int online_env = env_int("DALI_HIP_ROW_ONLINE_SOFTMAX", 1);
+    if (online_env && !rp.cached && !rp.split && rpn.n_phases >= 2 && rpn.phase_reduces[0].size() == 1 && rpn.phase_reduces[1].size() == 1) {
+        const int m_id = rpn.phase_reduces[0][0], s_id = rpn.phase_reduces[1][0];
+        const PNode& mx = P.nodes[m_id];
+        const PNode& sm = P.nodes[s_id];
+        auto through_views = [&](int id) {
+            while (P.nodes[id].kind == Kind::BROADCAST || P.nodes[id].kind == Kind::EXPAND_DIMS) id = P.nodes[id].args[0];
+            return id;
+        };
+        if (mx.kind == Kind::AXIS_REDUCE && mx.name == "reducers::maximum" && sm.kind == Kind::AXIS_REDUCE && sm.name == "reducers::sum" &&
+            mx.dtype == DTYPE_FLOAT && sm.dtype == DTYPE_FLOAT) {
+            const PNode& ex = P.nodes[sm.args[0]];
+            if (ex.kind == Kind::ELEMENTWISE && ex.name == "functor::exp" && ex.args.size() == 1) {
+                const PNode& sub = P.nodes[ex.args[0]];
+                if (sub.kind == Kind::ELEMENTWISE && sub.name == "functor::subtract" && sub.args.size() == 2 && sub.args[0] == mx.args[0] &&
+                    through_views(sub.args[1]) == m_id && P.nodes[mx.args[0]].dtype == DTYPE_FLOAT) {
+                    online_max = m_id;
+                    online_sum = s_id;
+                    online_arg = mx.args[0];
+                }
+            }
+        }
+    }
     // reduction phases
     for (int p = 0; p < rpn.n_phases; ++p) {
+        if (online_max >= 0 && p == 0) {
+            const std::string m = "acc" + std::to_string(online_max), l = "acc" + std::to_string(online_sum);
+            ss << "  float " << m << " = reducers::maximum::init<float>();\n  float " << l << " = 0.0f;\n";
+            BodyEmitter be(P, rp, true, 0, &rpn.first_body);
+            const std::string v = be.value(online_arg);
+            const std::string update = "{ const float xv = " + v + "; if (xv > " + m + ") { " + l + " = " + l + " * functor::exp<float>::Map(functor::subtract<float>::Map(" + m +
+                                       ", xv)) + 1.0f; " + m + " = xv; } else { " + l + " += functor::exp<float>::Map(functor::subtract<float>::Map(xv, " + m + ")); } }";
+            open_loop(ss);
+            ss << "      _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) {\n        const int col = " << col_of_ch << "; (void)col;\n";
+            ss << be.stmts.str() << "        " << update << "\n      }\n    }\n  }\n";
+            if (tail) {
+                open_tail(ss, "tail_on");
+                ss << be.stmts.str() << "    " << update << "\n  }\n";
+            }
+            const std::string rm = "red" + std::to_string(online_max), rs = "red" + std::to_string(online_sum);
+            if (rp.NW == 1) {
+                ss << "  const float " << rm << " = dali_group_reduce<reducers::maximum, float, " << std::min(rp.TPR, 64) << ">(" << m << ");\n";
+                ss << "  " << l << " *= functor::exp<float>::Map(functor::subtract<float>::Map(" << m << ", " << rm << "));\n";
+                ss << "  const float " << rs << " = dali_group_reduce<reducers::sum, float, " << std::min(rp.TPR, 64) << ">(" << l << ");\n";
+            } else {
+                ss << "  __shared__ float sm" << online_max << "[" << rp.NW << "];\n  __shared__ float sm" << online_sum << "[" << rp.NW << "];\n";
+                ss << "  const float " << rm << " = dali_block_reduce<reducers::maximum, float, " << rp.NW << ">(" << m << ", sm" << online_max << ");\n";
+                ss << "  " << l << " *= functor::exp<float>::Map(functor::subtract<float>::Map(" << m << ", " << rm << "));\n";
+                ss << "  const float " << rs << " = dali_block_reduce<reducers::sum, float, " << rp.NW << ">(" << l << ", sm" << online_sum << ");\n";
+            }
+            p = 1;  // both phases are done
+            continue;
+        }
         const std::vector<int>& reds = rpn.phase_reduces[p];
         for (int id : reds) {
             const PNode& n = P.nodes[id];
@@ -783,7 +840,7 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
     rp.nt_loads = nt_l >= 0 ? nt_l != 0 : dom.R * dom.C * (int64_t)max_el >= ((int64_t)64 << 20);
     rp.nt_stores = nt_s >= 0 ? nt_s != 0 : rpn.n_phases > 0;
     params << rp.VEC << "," << rp.TPR << "," << rp.EPT << "," << rp.BT << "," << rp.cached << "," << rp.waves_per_eu << ","
-           << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail << rp.peel << "," << rp.EPT_L << (rp.split ? "S" : "") << (rp.band > 1 ? "B" + std::to_string(rp.band) + "u" + std::to_string(rp.band_unroll) : std::string());
+           << rp.nt_loads << rp.nt_stores << rp.exact << rp.ragged << rp.tail << rp.peel << "," << rp.EPT_L << (rp.split ? "S" : "") << (!rp.cached && env_int("DALI_HIP_ROW_ONLINE_SOFTMAX", 1) == 0 ? "w" : "") << (rp.band > 1 ? "B" + std::to_string(rp.band) + "u" + std::to_string(rp.band_unroll) : std::string());
     if (n_totals) {
         // one 8-byte slot per workgroup and total in the workspace's 32 MiB of partial results
         const int64_t blocks = (dom.R + rp.RPB - 1) / rp.RPB;

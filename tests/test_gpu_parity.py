@@ -901,6 +901,44 @@ def test_rows_not_aligned_to_the_vector(gpu, D, O, rng, cols):
     assert np.array_equal((arr(D, xi)[:, 1:] * 3).numpy(), xi[:, 1:] * 3)
 
 
+@pytest.mark.parametrize("shape", [(256, 70001), (300, 131072)])
+def test_streamed_rows_take_maximum_and_sum_of_exponentials_in_one_walk(gpu, D, O, rng, shape):
+    """Rows too long for a workgroup's registers: the maximum and the sum of exp(x - maximum) (softmax.cpp:5-8, the log-sum-exp of
+    cost.cpp:115-133) come from one walk over the row, every thread scaling its running sum when a larger value arrives. Rows
+    with a dominant entry late in the row, with masked (-inf) entries, in ascending and in descending order (a new maximum at
+    every step, never again after the first), against fp64 and the sequential checker."""
+    op = D.op
+    R, C = shape
+    x = (rng.randn(R, C) * 3).astype(np.float32)
+    x[0, C - 3] = 60.0                       # dominant, met last by its thread
+    x[1, ::7] = -np.inf                      # masked entries
+    x[2] = np.sort(x[2])                     # ascending: every element a new maximum for the thread that meets it
+    x[3] = np.sort(x[3])[::-1]               # descending
+    x[4, :] = -1e30                          # nothing beats the first element by much
+    x[4, 5] = -1e30 + 1e24
+    X = arr(D, x)
+    k0 = D.jit_stats()["kernels"]
+    s = op.softmax(X).numpy()
+    assert D.jit_stats()["kernels"] - k0 == 1 and D.last_kernel_kinds() == "row"
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(1, keepdims=True))
+    close(s, e / e.sum(1, keepdims=True), rtol=1e-5, atol=1e-12)
+    close(s.astype(np.float64).sum(1), 1.0, rtol=0, atol=2e-6)
+    assert np.all(s[1, ::7] == 0.0)
+    close(s[:8], O.softmax(x[:8]), rtol=seq_sum_rtol(C), atol=1e-12)
+    m = op.max(X, [1], True)
+    lse = (op.log(op.sum(op.exp(X - m), [1], True)) + m).numpy()
+    close(lse[:, 0], np.log(e.sum(1)) + x64.max(1), rtol=1e-5, atol=1e-5)
+    t = rng.randint(0, C, R).astype(np.int32)
+    mean, rows, grad = op.softmax_cross_entropy(X, arr(D, t))
+    want_rows = np.log(e.sum(1)) + x64.max(1) - x64[np.arange(R), t]
+    finite = np.isfinite(want_rows)
+    close(rows.numpy()[finite], want_rows[finite], rtol=1e-5, atol=2e-5)
+    g = e / e.sum(1, keepdims=True)
+    g[np.arange(R), t] -= 1.0
+    close(grad.numpy(), g, rtol=1e-5, atol=1e-7)
+
+
 @pytest.mark.parametrize("shape", [(7, 300001), (3, 1000003), (1, 524291), (2, 3, 200003), (250, 70001), (5, 262144)])
 def test_few_long_rows_cut_into_pieces_by_the_row_kernel(gpu, D, O, rng, shape):
     """Reductions along few very long rows whose length does not divide into equal aligned pieces, and the position of the
