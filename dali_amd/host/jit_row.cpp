@@ -691,7 +691,10 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
     // Long rows whose vectors are aligned but whose length is no whole number of cache lines gain the same way from starting at
     // a 128-byte boundary ([2048,50256]: 156 -> 154 us, [2048,45000]: 142 -> 137 us).
     const bool line_rows = rp.VEC == 4 && !rp.ragged && dom.C >= 8192 && dom.C % 32 != 0;
-    if ((rp.ragged || line_rows) && peel_env && nph > 0 && segments <= 1 && peel_ok(P, dom)) {
+    // (maps over many long rows as well: `tanh(x + column)` on [2000,50257])
+    static const int peel_maps = env_int("DALI_HIP_ROW_PEEL_MAPS", 1);
+    const bool long_rows_map = nph == 0 && peel_maps && n_totals == 0 && dom.R >= 1024 && dom.C >= 8192;
+    if ((rp.ragged || line_rows) && peel_env && (nph > 0 || long_rows_map) && segments <= 1 && peel_ok(P, dom)) {
         rp.ragged = true;
         rp.peel = true;
         rp.tail = true;

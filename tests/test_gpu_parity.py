@@ -901,6 +901,30 @@ def test_rows_not_aligned_to_the_vector(gpu, D, O, rng, cols):
     assert np.array_equal((arr(D, xi)[:, 1:] * 3).numpy(), xi[:, 1:] * 3)
 
 
+@pytest.mark.parametrize("shape", [(1100, 8195), (1030, 50257), (1024, 8200)])
+def test_maps_over_many_long_rows_off_the_vector_boundary(gpu, D, rng, shape):
+    """A map without a reduction over many long rows whose length is no multiple of four elements (a per-row value added to the
+    logits of an odd vocabulary): vectors from each row's first 128-byte boundary, the elements in front of it and behind the
+    last vector one to a thread. Exact against numpy, also with += into the destination and into a view of a wider array."""
+    op = D.op
+    R, C = shape
+    x = rng.randn(R, C).astype(np.float32)
+    col = rng.randn(R, 1).astype(np.float32)
+    X, Cv = arr(D, x), arr(D, col)
+    got = (X + Cv).numpy()
+    assert D.last_kernel_kinds() == "map2d" and np.array_equal(got, x + col)
+    assert np.array_equal((X * 2.0 - Cv).numpy(), x * 2.0 - col)
+    y = rng.randn(R, C).astype(np.float32)
+    Y = arr(D, y)
+    Y.assign(X * Cv, 1)
+    assert np.array_equal(Y.numpy(), y + x * col)
+    wide = rng.randn(R, C + 5).astype(np.float32)
+    W = arr(D, wide)
+    W[:, 3:C + 3].assign(X + Cv, 0)          # rows of the destination start elsewhere than those of the source
+    want = wide.copy(); want[:, 3:C + 3] = x + col
+    assert np.array_equal(W.numpy(), want)
+
+
 @pytest.mark.parametrize("shape", [(256, 70001), (300, 131072)])
 def test_streamed_rows_take_maximum_and_sum_of_exponentials_in_one_walk(gpu, D, O, rng, shape):
     """Rows too long for a workgroup's registers: the maximum and the sum of exp(x - maximum) (softmax.cpp:5-8, the log-sum-exp of
