@@ -62,6 +62,9 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
             if (P.arrays[i].cls == Cls::FULL && !P.arrays[i].gather_source)
                 ss << "  " << (P.arrays[i].is_dest ? "" : "const ") << ctype(P.arrays[i].buf->dtype) << "* v" << i << " = q" << i << " + head;\n";
     }
+    // an operand broadcast along the rows ([1, C]: row stride 0): with peeled rows its vectors start wherever the rows' do, at
+    // element alignment, and it is read by every row, so it stays in the caches
+    auto along_rows = [&](int i) { const ArrayArg& a = P.arrays[i]; return rp.peel && !a.is_dest && a.strided && a.strides[0] == 0; };
     const std::string col_of_ch = rp.peel ? "head + ch * VEC + j" : "ch * VEC + j";
     // ragged rows: the C % VEC elements past the last whole vector go one to a thread, through the same bodies
     // (slot EPT of the register cache, j = 0)
@@ -89,7 +92,7 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
         for (int i : full_leaves) {
             const std::string t = ctype(P.arrays[i].buf->dtype);
             ss << "      " << t << " ld" << i << "[VEC];\n";
-            emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "ld" + std::to_string(i), "      ", rp.nt_loads, rp.ragged && !rp.peel, vp);
+            emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "ld" + std::to_string(i), "      ", rp.nt_loads && !along_rows(i), rp.ragged && (!rp.peel || along_rows(i)), vp);
             ss << "      if (e < EPT_R) {\n        _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) xr" << i << "[e < EPT_R ? e : 0][j] = ld" << i << "[j];\n      } else {\n";
             ss << "        dali_vec<" << t << ", VEC> lv; _Pragma(\"unroll\") for (int j = 0; j < VEC; ++j) lv.v[j] = ld" << i << "[j];\n";
             ss << "        dali_store<" << t << ", VEC>(&xl" << i << "[e >= EPT_R ? e - EPT_R : 0][tid * VEC], lv);\n      }\n";
@@ -105,7 +108,7 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
             ss << "  " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[EPT + " << (tail ? 1 : 0) << "][VEC];\n";
         }
         ss << "  _Pragma(\"unroll\") for (int e = 0; e < EPT; ++e) {\n    const int ch = tr + e * TPR;\n" << chunk_guard;
-        for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i) + "[e]", "      ", rp.nt_loads, rp.ragged && !rp.peel, vp);
+        for (int i : full_leaves) emit_leaf_load(ss, P.arrays[i], i, rp.VEC, "x" + std::to_string(i) + "[e]", "      ", rp.nt_loads && !along_rows(i), rp.ragged && (!rp.peel || along_rows(i)), vp);
         ss << "    }\n  }\n";
         if (tail) {
             ss << "  if (tail_on) {\n";
@@ -137,7 +140,7 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
                 o << "  for (int ch = tr; ch < CH; ch += TPR) {\n    {\n";
             for (int i : full_leaves) {
                 o << "      " << ctype(P.arrays[i].buf->dtype) << " x" << i << "[VEC];\n";
-                emit_leaf_load(o, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", rp.nt_loads, rp.ragged && !rp.peel, vp);
+                emit_leaf_load(o, P.arrays[i], i, rp.VEC, "x" + std::to_string(i), "      ", rp.nt_loads && !along_rows(i), rp.ragged && (!rp.peel || along_rows(i)), vp);
             }
         }
     };
@@ -564,6 +567,7 @@ static bool peel_ok(const Program& P, const Domain& dom) {
     for (const ArrayArg& a : P.arrays) {
         if (a.gather_source || a.cls != Cls::FULL) continue;
         if (a.col_stride != 1 || size_of_dtype(a.buf->dtype) != 4 || a.row_index >= 0) return false;
+        if (!a.is_dest && a.strided && a.strides[0] == 0) continue;  // broadcast along the rows: read at element alignment
         const long o = (long)(a.buf->offset % 4), r = (long)(a.row_stride % 4);
         if (off < 0) { off = o; rs = r; }
         if (o != off || r != rs) return false;

@@ -914,6 +914,15 @@ def test_maps_over_many_long_rows_off_the_vector_boundary(gpu, D, rng, shape):
     got = (X + Cv).numpy()
     assert D.last_kernel_kinds() == "map2d" and np.array_equal(got, x + col)
     assert np.array_equal((X * 2.0 - Cv).numpy(), x * 2.0 - col)
+    # a bias along the rows ([1, C]): its vectors start where the rows' do, at element alignment
+    bias = rng.randn(1, C).astype(np.float32)
+    Bv = arr(D, bias)
+    assert np.array_equal((X + Bv).numpy(), x + bias) and D.last_kernel_kinds() == "map2d"
+    assert np.array_equal(((X + Bv) * Cv).numpy(), (x + bias) * col)
+    sm = op.softmax(X + Bv).numpy()
+    x64 = (x + bias).astype(np.float64)
+    e = np.exp(x64 - x64.max(1, keepdims=True))
+    close(sm, e / e.sum(1, keepdims=True), rtol=1e-5, atol=1e-12)
     y = rng.randn(R, C).astype(np.float32)
     Y = arr(D, y)
     Y.assign(X * Cv, 1)
