@@ -1378,13 +1378,14 @@ def test_gather_from_rows_and_one_hot(gpu, D, O, rng):
 
 @pytest.mark.parametrize("shape", [(5, 97), (300, 17), (1000, 64), (4099, 33), (37, 1000), (16, 32000), (3, 50001),
                                    # thousands of workgroups meet for the mean: they arrive in groups, each with a counter of its own
-                                   (70001, 40), (9001, 513)])
+                                   (15000, 40), (9001, 513), (70001, 40)])
 def test_softmax_cross_entropy_matches_oracle(gpu, D, O, rng, shape):
     x = (rng.randn(*shape) * 2).astype(np.float32)
     t = rng.randint(0, shape[1], shape[0]).astype(np.int32)
     k0 = D.jit_stats()["kernels"]
     mean, rows, grad = D.op.softmax_cross_entropy(arr(D, x), arr(D, t))
-    assert D.jit_stats()["kernels"] - k0 == 1  # one fused row pass: gradient, row losses and their mean
+    # one fused row pass: gradient, row losses and their mean (tens of thousands of short rows: the mean in a small launch of its own)
+    assert D.jit_stats()["kernels"] - k0 == (2 if shape[0] >= 16384 and shape[1] < 2048 else 1)
     omean, orows, ograd = O.softmax_cross_entropy(x, t)
     close(rows.numpy(), orows, rtol=1e-5, atol=shape[1] * 2.0 ** -24)  # log of the row sum: the sum's relative error is absolute here
     close(mean.numpy(), omean, rtol=1e-5, atol=shape[1] * 2.0 ** -24)
