@@ -95,6 +95,7 @@ std::vector<int> contiguous_strides(const std::vector<int>& shape);
 // evaluation driver (jit.cpp)
 void evaluate(const std::vector<Array>& roots);
 void evaluate_into(const Array& dest, OPERATOR_T op, const Array& source);
+void evaluate_into_together(const std::vector<Array>& dests, const std::vector<Array>& sources);
 bool dry_run();
 // one fused launch for the LSTM cell step (records itself like any other launch)
 void lstm_step_fused(const Array& x, const Array& h, const Array& c, const Array& W, const Array& U, const Array& b, const Array& c_new,

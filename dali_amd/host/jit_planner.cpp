@@ -767,6 +767,26 @@ void evaluate_into(const Array& dest, OPERATOR_T op, const Array& source) {
     run_specs({{dest, op, c}});
 }
 
+// Several assignments dest_i = source_i planned together (one kernel where they fuse): the destinations are buffers or views
+// of buffers of their sources' shapes and dtypes.
+void evaluate_into_together(const std::vector<Array>& dests, const std::vector<Array>& sources) {
+    DALI_ASSERT(dests.size() == sources.size() && !dests.empty(), "evaluate_into_together: one source per destination");
+    jit_stats().evals++;
+    jit_stats().last_kernel_kinds.clear();
+    jit_stats().last_kernel_names.clear();
+    g_last_source.clear();
+    std::vector<DestSpec> specs;
+    ExprMemo memo;
+    for (size_t i = 0; i < dests.size(); ++i) {
+        DALI_ASSERT(dests[i].is_buffer() && dests[i].shape() == sources[i].shape() && dests[i].dtype() == sources[i].dtype(),
+                    "evaluate_into_together: a destination must be an evaluated buffer of its source's shape and dtype");
+        Array c = clean(sources[i], memo, true);
+        if (c.expression()->kind == Kind::SCALAR || c.expression()->kind == Kind::BUFFER) c = op::identity(c);
+        specs.push_back({dests[i], OPERATOR_T_EQL, c});
+    }
+    run_specs(specs);
+}
+
 std::vector<std::string> generate_only(const std::vector<Array>& roots) {
     std::vector<std::string> sources;
     bool prev = g_dry_run;
