@@ -1573,6 +1573,20 @@ CrossEntropyResult softmax_cross_entropy(const Array& logits, const Array& targe
     DALI_ASSERT(targets.ndim() == 1 && targets.dtype() == DTYPE_INT32 && targets.shape()[0] == logits.shape()[0],
                 "softmax_cross_entropy expects one int32 target per row");
     int rows = logits.shape()[0], cols = logits.shape()[1];
+    {
+        // Rows that are few for their length: one launch would give each row to one workgroup, which streams it through a single
+        // compute unit three times ([7,9999999]: 3.5 ms). The statistics come from pieces of the rows instead, and gradient and
+        // losses are then maps over them: the logits are read twice and nothing else is as large.
+        Array x = logits, M, L;
+        if (!dry_run() && few_long_rows_softmax_statistics(&x, &M, &L)) {
+            Array grad = subtract(eltdiv(exp(subtract(x, M)), L), one_hot(targets, cols, Array(1.0f), Array(0.0f)));
+            Array row_loss = subtract(add(log(L), M), gather_from_rows(x, targets).expand_dims(1));
+            Array mean_loss = mean(row_loss);
+            grad.eval();
+            Array::eval_together({row_loss, mean_loss});
+            return {mean_loss, row_loss.reshape({rows}), grad};
+        }
+    }
     Array m = max(logits, {-1}, true);
     Array exped = exp(subtract(logits, m));
     Array s = sum(exped, {-1}, true);

@@ -96,6 +96,9 @@ std::vector<int> contiguous_strides(const std::vector<int>& shape);
 void evaluate(const std::vector<Array>& roots);
 void evaluate_into(const Array& dest, OPERATOR_T op, const Array& source);
 void evaluate_into_together(const std::vector<Array>& dests, const std::vector<Array>& sources);
+// Maximum and sum of exp(x - maximum) of every row, evaluated, as [rows, 1], for rows that are few for their length (cut into
+// pieces that fill the device); *x comes back as the contiguous buffer they were taken from. False for any other shape.
+bool few_long_rows_softmax_statistics(Array* x, Array* maxima, Array* sums);
 bool dry_run();
 // one fused launch for the LSTM cell step (records itself like any other launch)
 void lstm_step_fused(const Array& x, const Array& h, const Array& c, const Array& W, const Array& U, const Array& b, const Array& c_new,

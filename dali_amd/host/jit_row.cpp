@@ -6,6 +6,34 @@
 namespace dali {
 namespace jit {
 
+
+// The statistics of a softmax or a log-sum-exp as two reduction phases: a maximum over the row, then the sum of
+// exp(x - that maximum) over the same values x. Gives the two reduction nodes and the node of x.
+static bool max_then_sum_of_exp(const RowPlan& rpn, int* max_id, int* sum_id, int* arg_id) {
+    const Program& P = rpn.P;
+    if (rpn.n_phases < 2 || rpn.phase_reduces[0].size() != 1 || rpn.phase_reduces[1].size() != 1) return false;
+    const int m_id = rpn.phase_reduces[0][0], s_id = rpn.phase_reduces[1][0];
+    const PNode& mx = P.nodes[m_id];
+    const PNode& sm = P.nodes[s_id];
+    auto through_views = [&](int id) {
+        while (P.nodes[id].kind == Kind::BROADCAST || P.nodes[id].kind == Kind::EXPAND_DIMS) id = P.nodes[id].args[0];
+        return id;
+    };
+    if (mx.kind != Kind::AXIS_REDUCE || mx.name != "reducers::maximum" || sm.kind != Kind::AXIS_REDUCE || sm.name != "reducers::sum" ||
+        mx.dtype != DTYPE_FLOAT || sm.dtype != DTYPE_FLOAT)
+        return false;
+    const PNode& ex = P.nodes[sm.args[0]];
+    if (ex.kind != Kind::ELEMENTWISE || ex.name != "functor::exp" || ex.args.size() != 1) return false;
+    const PNode& sub = P.nodes[ex.args[0]];
+    if (sub.kind != Kind::ELEMENTWISE || sub.name != "functor::subtract" || sub.args.size() != 2 || sub.args[0] != mx.args[0] ||
+        through_views(sub.args[1]) != m_id || P.nodes[mx.args[0]].dtype != DTYPE_FLOAT)
+        return false;
+    *max_id = m_id;
+    *sum_id = s_id;
+    *arg_id = mx.args[0];
+    return true;
+}
+
 static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const std::string& kname) {
     const Program& P = rpn.P;
     const RowParams& rp = rpn.rp;
@@ -176,28 +204,8 @@ static std::string gen_row_kernel(const RowPlan& rpn, const IvLayout& L, const s
     // ([1024,128256]: 361 -> 292 us, [512,151936]: 209 -> 167 us).
     int online_max = -1, online_sum = -1, online_arg = -1;
     static const int online_env = env_int("DALI_HIP_ROW_ONLINE_SOFTMAX", 1);
-    if (online_env && !rp.cached && !rp.split && rpn.n_phases >= 2 && rpn.phase_reduces[0].size() == 1 && rpn.phase_reduces[1].size() == 1) {
-        const int m_id = rpn.phase_reduces[0][0], s_id = rpn.phase_reduces[1][0];
-        const PNode& mx = P.nodes[m_id];
-        const PNode& sm = P.nodes[s_id];
-        auto through_views = [&](int id) {
-            while (P.nodes[id].kind == Kind::BROADCAST || P.nodes[id].kind == Kind::EXPAND_DIMS) id = P.nodes[id].args[0];
-            return id;
-        };
-        if (mx.kind == Kind::AXIS_REDUCE && mx.name == "reducers::maximum" && sm.kind == Kind::AXIS_REDUCE && sm.name == "reducers::sum" &&
-            mx.dtype == DTYPE_FLOAT && sm.dtype == DTYPE_FLOAT) {
-            const PNode& ex = P.nodes[sm.args[0]];
-            if (ex.kind == Kind::ELEMENTWISE && ex.name == "functor::exp" && ex.args.size() == 1) {
-                const PNode& sub = P.nodes[ex.args[0]];
-                if (sub.kind == Kind::ELEMENTWISE && sub.name == "functor::subtract" && sub.args.size() == 2 && sub.args[0] == mx.args[0] &&
-                    through_views(sub.args[1]) == m_id && P.nodes[mx.args[0]].dtype == DTYPE_FLOAT) {
-                    online_max = m_id;
-                    online_sum = s_id;
-                    online_arg = mx.args[0];
-                }
-            }
-        }
-    }
+    // (pieces of rows: each piece ends with its own maximum and its own sum relative to it, which is what its workgroup writes)
+    if (online_env && !rp.cached) max_then_sum_of_exp(rpn, &online_max, &online_sum, &online_arg);
     // reduction phases
     for (int p = 0; p < rpn.n_phases; ++p) {
         if (online_max >= 0 && p == 0) {
@@ -760,9 +768,14 @@ bool try_row(const std::vector<DestSpec>& specs, const Domain& dom, const std::v
         rp.cached = (int64_t)std::max(1, n_full) * ept * rp.VEC * (max_el / 4) <= 64;
         if (segments > 1) {
             // pieces of rows: one phase, results per row only, streamed (a piece is read once); at least a workgroup's worth of vectors each
-            if (nph != 1 || n_totals != 0 || rp.VEC != 4 || CH / segments < 1024) return false;
+            // (or the two phases that one walk takes together, a maximum and the sum of the exponentials relative to it: a piece's
+            // results are then those two reductions themselves, its own maximum and its sum relative to that)
+            int m_id = -1, s_id = -1, x_id = -1;
+            static const int online_env = env_int("DALI_HIP_ROW_ONLINE_SOFTMAX", 1);
+            const bool statistics = nph == 2 && online_env && max_then_sum_of_exp(rpn, &m_id, &s_id, &x_id);
+            if ((nph != 1 && !statistics) || n_totals != 0 || rp.VEC != 4 || CH / segments < 1024) return false;
             for (const Output& o : rpn.outputs)
-                if (o.cls != Cls::ROW) return false;
+                if (o.cls != Cls::ROW || (statistics && o.root != m_id && o.root != s_id)) return false;
             rp.cached = false;
             rp.split = true;
             split_S = segments;
