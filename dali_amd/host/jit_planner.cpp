@@ -717,6 +717,38 @@ void run_specs_planned(std::vector<DestSpec> specs) {
                 }
             }
         }
+        if (specs.size() == 1) {
+            // Reductions along few long rows under further arithmetic (rows minus their means, rows over their norms, a
+            // log-softmax): one launch would give each row to one workgroup, which walks it once per phase through a single
+            // compute unit ([7,9999999] minus the row means: 2.5 ms). The reductions are evaluated on their own instead, in pieces of
+            // the rows that fill the device, and what is left is a map over the rows that reads their small results.
+            static const bool pieces_off = env_int("DALI_HIP_SEGMENTED_REDUCE", 1) == 0;
+            // (a result per row only: the rows are walked once either way, and what counts is the rule of a reduction on its own)
+            const bool map_over_rows = numel_of(specs[0].dest.shape()) == dom.R * dom.C;
+            const bool few_long_rows = dom.R < 256 && dom.C >= 65536 &&
+                                       (dom.R * dom.C * 4 >= ((int64_t)64 << 20) ||
+                                        (map_over_rows ? dom.C >= 131072 && (double)dom.R < 75.0 - 3.75e6 / (double)dom.C : dom.C >= 200000));
+            Array inner;
+            std::set<const Expr*> seen_inner;
+            if (!pieces_off && few_long_rows && find_innermost_reduce(specs[0].root, &inner, seen_inner) &&
+                inner.expression().get() != specs[0].root.expression().get() &&
+                (inner.expression()->kind == Kind::AXIS_REDUCE || inner.expression()->kind == Kind::ARG_AXIS_REDUCE) &&
+                domain_of(inner.expression()->args[0].shape()).C == dom.C) {
+                const bool before = g_segment_whatever_the_size;
+                g_segment_whatever_the_size = true;  // (the rule above has been applied; a reduction on its own has another)
+                Array buf;
+                try {
+                    buf = materialize(inner);
+                } catch (...) {
+                    g_segment_whatever_the_size = before;
+                    throw;
+                }
+                g_segment_whatever_the_size = before;
+                ExprMemo memo;
+                specs[0].root = substitute(specs[0].root, inner.expression().get(), buf, memo);
+                continue;
+            }
+        }
         if (try_row(specs, dom)) return;
         if (specs.size() > 1) {
             for (auto& s : specs) run_specs({s});

@@ -934,6 +934,55 @@ def test_maps_over_many_long_rows_off_the_vector_boundary(gpu, D, rng, shape):
     assert np.array_equal(W.numpy(), want)
 
 
+@pytest.mark.parametrize("shape", [(3, 300001), (2, 1 << 20), (5, 3400003)])
+def test_row_reductions_under_arithmetic_over_few_long_rows(gpu, D, O, rng, shape):
+    """Few rows, each far longer than a workgroup holds: reductions along the rows inside a larger expression are evaluated on
+    their own, over pieces of the rows, and the rest is a map that reads their per-row results (softmax.cpp:5-8 and the
+    reducers of reducer_operation.cpp:595-679 under elementwise arithmetic). Softmax and cross-entropy take each piece's maximum
+    and sum of exponentials from one walk; pieces that are masked out altogether count for nothing."""
+    op = D.op
+    R, C = shape
+    x = (rng.randn(R, C) * 2).astype(np.float32)
+    x[0, :20000] = -np.inf                   # whole pieces of the first row masked
+    x[R - 1, C - 2] = 40.0                   # a dominant entry in the last piece
+    X = arr(D, x)
+    x64 = x.astype(np.float64)
+    k0 = D.jit_stats()["kernels"]
+    s = op.softmax(X).numpy()
+    assert D.jit_stats()["kernels"] - k0 == 3
+    e = np.exp(x64 - x64.max(1, keepdims=True))
+    close(s, e / e.sum(1, keepdims=True), rtol=1e-5, atol=1e-12)
+    assert np.all(s[0, :20000] == 0.0)
+    close(s.astype(np.float64).sum(1), 1.0, rtol=0, atol=2e-6)
+    t = rng.randint(20000, C, R).astype(np.int32)
+    mean, rows, grad = op.softmax_cross_entropy(X, arr(D, t))
+    lse = np.log(e.sum(1)) + x64.max(1)
+    close(rows.numpy(), lse - x64[np.arange(R), t], rtol=1e-5, atol=2e-5)
+    close(mean.numpy(), (lse - x64[np.arange(R), t]).mean(), rtol=1e-5, atol=2e-5)
+    g = e / e.sum(1, keepdims=True)
+    g[np.arange(R), t] -= 1.0
+    close(grad.numpy(), g, rtol=1e-5, atol=3e-7)  # (the target's element is a softmax minus one: a few ulps of one)
+    # rows minus their means, rows over their norms, a log-softmax written out, a mean of squares: reductions first, then a map
+    y = (rng.randn(R, C) * 2).astype(np.float32)
+    Y = arr(D, y)
+    y64 = y.astype(np.float64)
+    k0 = D.jit_stats()["kernels"]
+    centered = (Y - op.mean(Y, [1], True)).numpy()
+    assert D.jit_stats()["kernels"] - k0 == 3 and D.last_kernel_kinds().endswith("map2d")
+    close(centered, y64 - y64.mean(1, keepdims=True), rtol=1e-5, atol=1e-5)
+    unit = (Y / op.sqrt(op.sum(Y * Y, [1], True))).numpy()
+    close(unit, y64 / np.sqrt((y64 * y64).sum(1, keepdims=True)), rtol=1e-5, atol=1e-12)
+    m = op.max(Y, [1], True)
+    k0 = D.jit_stats()["kernels"]
+    logp = (Y - (op.log(op.sum(op.exp(Y - m), [1], True)) + m)).numpy()
+    assert D.jit_stats()["kernels"] - k0 == 5
+    ey = np.exp(y64 - y64.max(1, keepdims=True))
+    close(logp, y64 - (np.log(ey.sum(1, keepdims=True)) + y64.max(1, keepdims=True)), rtol=1e-5, atol=2e-5)
+    close(op.mean(Y * Y, [1]).numpy(), (y64 * y64).mean(1), rtol=1e-5)
+    am = op.argmax(Y * 2.0, 1).numpy()
+    assert np.array_equal(am, (y * 2.0).argmax(1))
+
+
 @pytest.mark.parametrize("shape", [(256, 70001), (300, 131072)])
 def test_streamed_rows_take_maximum_and_sum_of_exponentials_in_one_walk(gpu, D, O, rng, shape):
     """Rows too long for a workgroup's registers: the maximum and the sum of exp(x - maximum) (softmax.cpp:5-8, the log-sum-exp of
