@@ -414,13 +414,17 @@ static bool try_two_stage_reduce(const DestSpec& spec) {
     // (between 513 and 1024 columns only where the second launch is small beside the first: [50000,1000] 38.0 -> 34.5 us, [65536,1024] 46.7 -> 43.0 us)
     if (Cn > 512 && (int64_t)R * Cn * 4 < ((int64_t)64 << 20)) return false;
     int k = 1;
-    while (k * 2 * (int64_t)Cn <= 4096 && R % (k * 2) == 0 && R / (k * 2) >= 64) k *= 2;
+    while (k * 2 * (int64_t)Cn <= 4096 && R / (k * 2) >= 64) k *= 2;
     if (k < 2) return false;
     Array matrix = arg.transpose();  // [R, C], contiguous
     if (!matrix.contiguous_memory()) return false;
-    Array stage1 = op::axis_reduce(matrix.reshape({R / k, k * Cn}), red, {0}, false);
-    stage1.eval();
-    Array root2 = op::axis_reduce(stage1.reshape({k, Cn}), red, {0}, false);
+    // rows beyond the last whole group of k (fewer than k, at most 4096 elements) join the k partial rows as they are:
+    // [9999999,7] has no divisor to go by, and its sum took 555 us through strips of 256 columns that hold seven
+    const int rest = R % k, R0 = R - rest;
+    Array partial({k + rest, Cn}, arg.dtype());
+    evaluate_into(partial.slice(0, 0, k).reshape({k * Cn}), OPERATOR_T_EQL, op::axis_reduce(matrix.slice(0, 0, R0).reshape({R0 / k, k * Cn}), red, {0}, false));
+    if (rest > 0) evaluate_into(partial.slice(0, k, k + rest), OPERATOR_T_EQL, op::identity(matrix.slice(0, R0, R)));
+    Array root2 = op::axis_reduce(partial, red, {0}, false);
     if (root2.shape() != e->shape) return false;
     run_specs({{spec.dest, spec.op, root2}});
     return true;

@@ -1068,6 +1068,32 @@ def test_few_long_rows_cut_into_pieces_by_the_row_kernel(gpu, D, O, rng, shape):
     close(s.astype(np.float64).sum(-1), 1.0, rtol=0, atol=2e-6)
 
 
+@pytest.mark.parametrize("shape", [(100003, 7), (65537, 33), (1000003, 3), (70001, 512), (9973, 100), (4099, 1), (131072, 24)])
+def test_leading_axis_of_tall_narrow_matrices_with_any_number_of_rows(gpu, D, O, rng, shape):
+    """Tall narrow matrices reduced along the leading axis (reducer_operation.cpp:595-679): k neighbouring rows are read as one
+    row of k times as many columns, and the k partial rows are reduced again. The row count need not divide by k: the rows
+    past the last whole group join the partial rows as they are."""
+    op = D.op
+    R, C = shape
+    x = rng.randn(R, C).astype(np.float32)
+    x[R - 1] = 7.5                           # the best value of every column in the very last row
+    x[R - 2, ::2] = -9.25                    # and the smallest of every other column in the one before
+    X = arr(D, x)
+    x64 = x.astype(np.float64)
+    assert np.all(np.abs(op.sum(X, [0]).numpy() - x64.sum(0)) <= sum_tol(x, 0))
+    assert np.array_equal(op.max(X, [0]).numpy(), x.max(0)) and np.array_equal(op.min(X, [0]).numpy(), x.min(0))
+    assert np.all(op.max(X, [0]).numpy() == 7.5) and np.all(op.min(X, [0]).numpy()[::2] == -9.25)
+    close(op.mean(X, [0], True).numpy(), x64.mean(0, keepdims=True), rtol=1e-5, atol=1e-6)
+    close((X - op.mean(X, [0], True)).numpy(), x64 - x64.mean(0, keepdims=True), rtol=1e-5, atol=1e-5)
+    y = np.exp(x[:, : min(C, 16)] * 0.001).astype(np.float32)
+    close(op.prod(arr(D, y), [0]).numpy(), y.astype(np.float64).prod(0), rtol=R * 2.0 ** -24 * 0.1)
+    # a slice of the rows (the matrix does not start where its buffer does)
+    if R > 5000:
+        v, nv = X[3:R - 2], x[3:R - 2]
+        assert np.all(np.abs(op.sum(v, [0]).numpy() - nv.astype(np.float64).sum(0)) <= sum_tol(nv, 0))
+        assert np.array_equal(op.max(v, [0]).numpy(), nv.max(0))
+
+
 @pytest.mark.parametrize("shape", [(37, 16), (37, 17), (5, 18), (300, 19), (3000, 1001), (64, 4097), (2000, 50257), (7, 300001)])
 def test_leading_axis_reductions_off_the_vector_size(gpu, D, O, rng, shape):
     """Kept extents that are no multiple of four: memory rows start at every alignment, and the lane whose vector
