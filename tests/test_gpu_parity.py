@@ -2254,7 +2254,9 @@ def test_scan_reference_cases(gpu, D):
         assert np.array_equal(op.cumprod(p, inclusive).numpy(), wp)
 
 
-@pytest.mark.parametrize("shape", [(1,), (7,), (3, 64), (5, 257), (33, 1000), (4, 4096), (2, 100003), (3, 262144), (300, 1021), (2, 3, 50)])
+@pytest.mark.parametrize("shape", [(1,), (7,), (3, 64), (5, 257), (33, 1000), (4, 4096), (2, 100003), (3, 262144), (300, 1021), (2, 3, 50),
+                                   # rows shorter than a wave's vectors: several rows to a wave (4, 8, 16 and 32 threads per row)
+                                   (1000, 7), (513, 3), (300, 16), (1025, 128), (64, 31), (70001, 5)])
 @pytest.mark.parametrize("inclusive", [True, False])
 def test_scan_matches_oracle(gpu, D, O, rng, shape, inclusive):
     x = rng.uniform(0.5, 1.5, shape).astype(np.float32)
