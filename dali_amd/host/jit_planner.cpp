@@ -490,6 +490,111 @@ static bool try_segmented_reduce(const DestSpec& spec) {
     return true;
 }
 
+// A map over a tall matrix whose rows are short and off the vector size, with operands that hold one value per column (a
+// bias added to [N, 7] features, columns minus their means): the row kernel would read such rows an element per lane
+// ([9999999,7] + [1,7]: 190 us, 0.37 of the HBM peak). k neighbouring rows are read as one row of k * C elements instead, k a
+// multiple of four, against the per-column operands repeated k times; the rows past the last whole group go through the
+// ordinary form. Operands other than [R, C] matrices along memory, per-column vectors and single values: not taken.
+static bool try_narrow_map(const DestSpec& spec) {
+    static const bool off = env_int("DALI_HIP_NARROW_MAP", 1) == 0;
+    const Array& dest = spec.dest;
+    if (off || !dest.is_buffer() || dest.ndim() != 2 || !dest.contiguous_memory()) return false;
+    const int R = dest.shape()[0], C = dest.shape()[1];
+    if (C % 4 == 0 || C >= 256 || C < 2 || (int64_t)R * C < (1 << 20)) return false;
+    const int k = std::max(4, 4 * ((512 / C + 3) / 4));
+    if (R / k < 1024) return false;
+    const int rest = R % k, R0 = R - rest;
+    bool ok = true, per_column = false;
+    // pass 0 only looks; pass 1 builds the grouped rows, pass 2 the rows left over
+    int pass = 0;
+    std::map<const Expr*, Array> tiles, memo;  // per-column operands repeated k times; what a node became in this pass
+    auto mapped = [&](const std::vector<int>& shape, std::vector<int>* out) {
+        const int64_t n = numel_of(shape);
+        if (n == (int64_t)R * C && shape.size() == 2 && shape[0] == R) *out = pass == 2 ? std::vector<int>{rest, C} : std::vector<int>{R0 / k, k * C};
+        else if (n == C && (shape == std::vector<int>{C} || shape == std::vector<int>{1, C})) *out = pass == 2 ? std::vector<int>{1, C} : std::vector<int>{1, k * C};
+        else return false;
+        return true;
+    };
+    std::function<Array(const Array&)> regroup = [&](const Array& a) -> Array {
+        auto e = a.expression();
+        if (!ok || e->kind == Kind::SCALAR || numel_of(e->shape) == 1) return a;  // single values are read as they are
+        auto known = memo.find(e.get());
+        if (known != memo.end()) return known->second;
+        Array out = a;
+        std::vector<int> shape;
+        switch (e->kind) {
+            case Kind::BUFFER:
+                if (!a.contiguous_memory() || !mapped(e->shape, &shape)) {
+                    ok = false;
+                } else if (numel_of(e->shape) == C) {
+                    per_column = true;
+                    if (pass == 1) {
+                        auto made = tiles.find(e.get());
+                        if (made == tiles.end()) {
+                            Array t({1, k * C}, e->dtype);
+                            auto b = std::make_shared<Expr>();
+                            b->kind = Kind::BROADCAST;
+                            b->args = {a.reshape({1, C})};
+                            b->shape = {k, C};
+                            b->dtype = e->dtype;
+                            evaluate_into(t.reshape({k, C}), OPERATOR_T_EQL, op::identity(Array(b)));
+                            made = tiles.emplace(e.get(), t).first;
+                        }
+                        out = made->second;
+                    } else if (pass == 2) {
+                        out = a.reshape({1, C});
+                    }
+                } else if (pass == 1) {
+                    out = a.slice(0, 0, R0).reshape({R0 / k, k * C});
+                } else if (pass == 2) {
+                    out = a.slice(0, R0, R);
+                }
+                break;
+            case Kind::EXPAND_DIMS:
+                out = regroup(e->args[0]);  // ([C] -> [1, C]: the grouped form is two-dimensional already)
+                if (numel_of(e->shape) != C) ok = false;
+                break;
+            case Kind::BROADCAST:
+            case Kind::ELEMENTWISE: {
+                if (!mapped(e->shape, &shape)) {
+                    ok = false;
+                    break;
+                }
+                std::vector<Array> args;
+                for (const Array& x : e->args) args.push_back(regroup(x));
+                if (!ok || pass == 0) break;
+                if (e->kind == Kind::BROADCAST && args[0].shape() == shape) {
+                    out = args[0];
+                    break;
+                }
+                auto n = std::make_shared<Expr>(*e);
+                n->args = args;
+                n->shape = shape;
+                out = Array(n);
+                break;
+            }
+            default: ok = false;
+        }
+        memo[e.get()] = out;
+        return out;
+    };
+    regroup(spec.root);
+    if (!ok || !per_column) return false;
+    pass = 1;
+    memo.clear();
+    Array head = regroup(spec.root);
+    if (!ok) return false;
+    run_specs({{dest.slice(0, 0, R0).reshape({R0 / k, k * C}), spec.op, head}});
+    if (rest > 0) {
+        pass = 2;
+        memo.clear();
+        Array tail = regroup(spec.root);
+        if (!ok) throw std::runtime_error("internal: the rows left over by a grouped map could not be planned");
+        run_specs({{dest.slice(0, R0, R), spec.op, tail}});
+    }
+    return true;
+}
+
 void run_specs_planned(std::vector<DestSpec> specs) {
     if (specs.size() == 1 && (try_two_stage_reduce(specs[0]) || try_segmented_reduce(specs[0]))) return;
     // all-reduce roots are planned one by one
@@ -568,6 +673,7 @@ void run_specs_planned(std::vector<DestSpec> specs) {
         for (auto& s : specs) has_red = has_red || has_kind(s.root, [](Kind k) { return is_reduce(k); });
         if (!has_red) {
             if (try_flat(specs)) return;
+            if (specs.size() == 1 && !g_dry_run && try_narrow_map(specs[0])) return;
             if (specs.size() == 1) {
                 // Large transposed matrices among the operands are first written out along memory by a tiled transpose
                 // (both its reads and its writes are coalesced); a map that walked them in place would fetch a cache line

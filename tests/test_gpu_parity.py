@@ -901,6 +901,41 @@ def test_rows_not_aligned_to_the_vector(gpu, D, O, rng, cols):
     assert np.array_equal((arr(D, xi)[:, 1:] * 3).numpy(), xi[:, 1:] * 3)
 
 
+@pytest.mark.parametrize("shape", [(150001, 7), (65537, 33), (40000, 30), (1048579, 3), (20000, 130)])
+def test_maps_over_tall_narrow_matrices_with_per_column_operands(gpu, D, rng, shape):
+    """A bias added to [N, 7] features, columns minus their means over their deviations (elementwise_operation.cpp:130-186
+    with operands broadcast along the rows): k neighbouring rows are read as one long row against the per-column operands
+    repeated k times, and the rows past the last whole group separately. Every element is the same single fp32 operation
+    as in the ordinary form."""
+    op = D.op
+    R, C = shape
+    x = rng.randn(R, C).astype(np.float32)
+    b = rng.randn(1, C).astype(np.float32)
+    s = rng.uniform(0.5, 2.0, (1, C)).astype(np.float32)
+    X, B, S = arr(D, x), arr(D, b), arr(D, s)
+    assert np.array_equal((X + B).numpy(), x + b)
+    assert np.array_equal(((X - B) / S).numpy(), (x - b) / s)
+    assert np.array_equal((X * 2.0 + arr(D, b[0]).expand_dims(0)).numpy(), x * np.float32(2.0) + b)   # a [C] vector with a unit axis inserted
+    assert np.array_equal((B - X).numpy(), b - x)
+    assert np.array_equal(op.tanh(X * (B * 0.5)).numpy() == 0, np.tanh(x * (b * np.float32(0.5))) == 0)
+    close(op.tanh(X * (B * 0.5)).numpy(), np.tanh(x.astype(np.float64) * (b * np.float32(0.5))), rtol=1e-5, atol=1e-6)
+    # in place, and into a matrix that does not start where its buffer does
+    Y = arr(D, x.copy())
+    Y += X * B
+    assert np.array_equal(Y.numpy(), x + x * b)
+    big = arr(D, np.zeros((R + 3, C), np.float32))
+    view = big[2:R + 2]
+    view.assign(X - B)
+    got = big.numpy()
+    assert np.array_equal(got[2:R + 2], x - b) and not got[:2].any() and not got[R + 2:].any()
+    # integers, and a per-row operand beside the per-column one (not grouped: one value per row has no place in a row of k rows)
+    xi = rng.randint(-1000, 1000, (R, C)).astype(np.int32)
+    bi = rng.randint(-1000, 1000, (1, C)).astype(np.int32)
+    assert np.array_equal((arr(D, xi) + arr(D, bi)).numpy(), xi + bi)
+    col = rng.randn(R, 1).astype(np.float32)
+    assert np.array_equal((X + B + arr(D, col)).numpy(), (x + b) + col)
+
+
 @pytest.mark.parametrize("shape", [(1100, 8195), (1030, 50257), (1024, 8200)])
 def test_maps_over_many_long_rows_off_the_vector_boundary(gpu, D, rng, shape):
     """A map without a reduction over many long rows whose length is no multiple of four elements (a per-row value added to the
