@@ -385,6 +385,31 @@ static bool try_two_stage_reduce(const DestSpec& spec) {
     const std::string& red = e->name;
     if (red != "reducers::sum" && red != "reducers::maximum" && red != "reducers::minimum" && red != "reducers::product") return false;
     Array arg = e->args[0];
+    if (!arg.is_buffer() && arg.ndim() == 2 && arg.dtype() == e->dtype && arg.expression()->kind == Kind::ELEMENTWISE && arg.shape()[0] <= 64 &&
+        numel_of(arg.shape()) >= (1 << 20)) {
+        // The leading axis of a tall narrow expression (the column variances inside a standardisation: squares of [N, 7] minus
+        // its column means): the fused form walks strips of 256 columns that hold seven ([9999999,7]: 700 us). The expression is
+        // written out along memory first, as a map over rows grouped k at a time, and reduced as a buffer: two more passes over
+        // the matrix against one that uses a thirtieth of every strip.
+        Array matrix = arg.transpose();  // the same node over the operands as they lie in memory
+        bool along_memory = matrix.expression()->kind == Kind::ELEMENTWISE;
+        std::function<void(const Array&)> look = [&](const Array& a) {
+            auto ae = a.expression();
+            if (ae->kind == Kind::BUFFER) {
+                if (numel_of(ae->shape) == numel_of(matrix.shape()) && !a.contiguous_memory()) along_memory = false;
+            } else if (ae->kind == Kind::ELEMENTWISE || ae->kind == Kind::BROADCAST || ae->kind == Kind::EXPAND_DIMS) {
+                for (const Array& x : ae->args) look(x);
+            } else if (ae->kind != Kind::SCALAR) {
+                along_memory = false;
+            }
+        };
+        if (along_memory) look(matrix);
+        if (along_memory) {
+            Array buf = materialize(matrix);
+            run_specs({{spec.dest, spec.op, op::axis_reduce(buf, red, {0}, false)}});
+            return true;
+        }
+    }
     if (!arg.is_buffer() || arg.ndim() < 1 || arg.dtype() != e->dtype) return false;
     const int C_last = arg.shape().back();
     const int64_t n = numel_of(arg.shape());

@@ -1122,6 +1122,13 @@ def test_leading_axis_of_tall_narrow_matrices_with_any_number_of_rows(gpu, D, O,
     close((X - op.mean(X, [0], True)).numpy(), x64 - x64.mean(0, keepdims=True), rtol=1e-5, atol=1e-5)
     y = np.exp(x[:, : min(C, 16)] * 0.001).astype(np.float32)
     close(op.prod(arr(D, y), [0]).numpy(), y.astype(np.float64).prod(0), rtol=R * 2.0 ** -24 * 0.1)
+    # the leading axis of an expression (the column variances of a standardisation; from 2**20 elements and up to 64 columns the
+    # expression is written out along memory first), and the standardised matrix
+    mean = op.mean(X, [0], True)
+    var = op.mean(op.square(X - mean), [0], True)
+    close(var.numpy(), x64.var(0, keepdims=True), rtol=1e-4, atol=1e-6)
+    close(((X - mean) / op.sqrt(var)).numpy(), (x64 - x64.mean(0, keepdims=True)) / x64.std(0, keepdims=True), rtol=1e-4, atol=1e-5)
+    assert np.array_equal(op.max(op.abs(X) * 2.0, [0]).numpy(), (np.abs(x) * np.float32(2.0)).max(0))
     # a slice of the rows (the matrix does not start where its buffer does)
     if R > 5000:
         v, nv = X[3:R - 2], x[3:R - 2]
