@@ -145,6 +145,19 @@ static Array expand_softmax(Array x, int axis) {
             for (int d = 0; d < axis; ++d) outer *= shape[d];
             // a reduced axis short enough for a strip of it to live in one workgroup's registers: one pass, read once and
             // written once ([256,512,512] along axis 1: 142 -> 88 us, 0.76 of the HBM peak)
+            static const bool narrow_off = env_int("DALI_HIP_NARROW_MAP", 1) == 0;
+            if (!narrow_off && !g_dry_run && nd == 2 && axis == 0 && shape[1] >= 2 && shape[1] <= 48 && n >= (1 << 20)) {
+                // along the leading axis of a tall narrow matrix: a strip of 256 columns holds a few ([9999999,7]: 1408 us). Column
+                // maxima and column sums go through the grouped forms of such matrices, the exponentials are written out once.
+                if (!x.is_buffer()) x = materialize(x);
+                if (!x.contiguous_memory()) x = x.ascontiguousarray();
+                Array M = op::max(x, {0}, true);
+                evaluate({M});
+                Array E = materialize(op::exp(op::subtract(x, M)));
+                Array L = op::sum(E, {0}, true);
+                evaluate({L});
+                return op::eltdiv(E, L);
+            }
             static const bool one_pass_off = env_int("DALI_HIP_SOFTMAX_AXIS", 1) == 0;
             if (!one_pass_off && !g_dry_run && dali_hip_softmax_axis_supported(outer, (int)Cx, inner)) {
                 if (!x.is_buffer()) x = materialize(x);
@@ -385,7 +398,7 @@ static bool try_two_stage_reduce(const DestSpec& spec) {
     const std::string& red = e->name;
     if (red != "reducers::sum" && red != "reducers::maximum" && red != "reducers::minimum" && red != "reducers::product") return false;
     Array arg = e->args[0];
-    if (!arg.is_buffer() && arg.ndim() == 2 && arg.dtype() == e->dtype && arg.expression()->kind == Kind::ELEMENTWISE && arg.shape()[0] <= 64 &&
+    if (!arg.is_buffer() && arg.ndim() == 2 && arg.dtype() == e->dtype && arg.expression()->kind == Kind::ELEMENTWISE && arg.shape()[0] >= 2 && arg.shape()[0] <= 64 &&
         numel_of(arg.shape()) >= (1 << 20)) {
         // The leading axis of a tall narrow expression (the column variances inside a standardisation: squares of [N, 7] minus
         // its column means): the fused form walks strips of 256 columns that hold seven ([9999999,7]: 700 us). The expression is
@@ -622,6 +635,18 @@ static bool try_narrow_map(const DestSpec& spec) {
 
 void run_specs_planned(std::vector<DestSpec> specs) {
     if (specs.size() == 1 && (try_two_stage_reduce(specs[0]) || try_segmented_reduce(specs[0]))) return;
+    if (specs.size() == 1) {
+        // the same reductions with their reduced axes kept as unit axes (keepdims): unit axes inserted over the reduction,
+        // written through a view of the destination without them
+        Array base = specs[0].root;
+        while (base.expression()->kind == Kind::EXPAND_DIMS) base = base.expression()->args[0];
+        const Kind bk = base.expression()->kind;
+        if (base.expression().get() != specs[0].root.expression().get() && (bk == Kind::AXIS_REDUCE || bk == Kind::ARG_AXIS_REDUCE) &&
+            specs[0].dest.is_buffer() && specs[0].dest.contiguous_memory() && numel_of(specs[0].dest.shape()) == numel_of(base.shape())) {
+            DestSpec plain{specs[0].dest.reshape(base.shape()), specs[0].op, base};
+            if (try_two_stage_reduce(plain) || try_segmented_reduce(plain)) return;
+        }
+    }
     // all-reduce roots are planned one by one
     if (specs.size() > 1) {
         bool any_all = false;

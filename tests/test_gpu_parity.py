@@ -1086,6 +1086,9 @@ def test_few_long_rows_cut_into_pieces_by_the_row_kernel(gpu, D, O, rng, shape):
     assert np.array_equal(op.max(X, [-1]).numpy(), x.max(-1))
     assert np.array_equal(op.min(X, [-1]).numpy(), x.min(-1))
     k0 = D.jit_stats()["kernels"]
+    kept = op.max(X, [-1], True).numpy()     # the reduced axis kept as a unit axis: the same two launches
+    assert D.jit_stats()["kernels"] - k0 == 2 and kept.shape == x.shape[:-1] + (1,) and np.array_equal(kept, x.max(-1, keepdims=True))
+    k0 = D.jit_stats()["kernels"]
     am = op.argmax(X, -1).numpy()
     assert D.jit_stats()["kernels"] - k0 <= 4
     assert am.dtype == np.int32 and np.array_equal(am, x.argmax(-1)) and np.array_equal(am, O.arg_axis_reduce(O.MAX, rows, 1).reshape(am.shape))
@@ -1118,6 +1121,9 @@ def test_leading_axis_of_tall_narrow_matrices_with_any_number_of_rows(gpu, D, O,
     assert np.all(np.abs(op.sum(X, [0]).numpy() - x64.sum(0)) <= sum_tol(x, 0))
     assert np.array_equal(op.max(X, [0]).numpy(), x.max(0)) and np.array_equal(op.min(X, [0]).numpy(), x.min(0))
     assert np.all(op.max(X, [0]).numpy() == 7.5) and np.all(op.min(X, [0]).numpy()[::2] == -9.25)
+    kept = op.max(X, [0], True).numpy()      # the reduced axis kept as a unit axis: the same route
+    assert kept.shape == (1, C) and np.array_equal(kept, x.max(0, keepdims=True))
+    assert np.all(np.abs(op.sum(X, [0], True).numpy() - x64.sum(0, keepdims=True)) <= sum_tol(x, 0))
     close(op.mean(X, [0], True).numpy(), x64.mean(0, keepdims=True), rtol=1e-5, atol=1e-6)
     close((X - op.mean(X, [0], True)).numpy(), x64 - x64.mean(0, keepdims=True), rtol=1e-5, atol=1e-5)
     y = np.exp(x[:, : min(C, 16)] * 0.001).astype(np.float32)
@@ -1402,7 +1408,9 @@ def test_rows_that_start_off_the_vector_boundary(gpu, D, O, rng, rows, cols, ski
 @pytest.mark.parametrize("shape,axis", [((8, 262144), -1), ((3, 524288), 1), ((2, 3, 131072), 2), ((4096, 1000), 0), ((513, 257), 0),
                                         ((16, 300, 64), 1), ((16, 300, 64), 0), ((70000, 16), 0), ((64, 1000), 0),
                                         # strips of 64, 32 and 16 inner positions held in registers, the last strip partly filled
-                                        ((2, 512, 200), 1), ((4, 1000, 96), 1), ((3, 2000, 40), 1), ((1100, 64), 0), ((5, 3, 511, 6, 8), 2)])
+                                        ((2, 512, 200), 1), ((4, 1000, 96), 1), ((3, 2000, 40), 1), ((1100, 64), 0), ((5, 3, 511, 6, 8), 2),
+                                        # tall and narrow, along the leading axis: column maxima, exponentials written out, column sums, quotient
+                                        ((150001, 7), 0), ((1048579, 3), 0)])
 def test_softmax_over_few_long_rows_and_against_the_layout(gpu, D, O, rng, shape, axis):
     """op::softmax takes any axis (softmax.cpp:5-8). Few very long rows are cut into pieces whose (maximum, sum of
     exponentials) pairs are combined by a second small kernel; along an axis other than the last a strip of the reduced axis is
@@ -1418,6 +1426,8 @@ def test_softmax_over_few_long_rows_and_against_the_layout(gpu, D, O, rng, shape
     ax = axis % len(shape)
     if ax == len(shape) - 1:
         assert launched == 3 and D.last_kernel_kinds().endswith("map2d")   # piece statistics, their combination, the quotient
+    elif len(shape) == 2 and 2 <= shape[1] <= 48 and x.size >= 1 << 20:
+        assert launched >= 4 and D.last_kernel_kinds().endswith(("map2d", "flat"))
     elif x.size >= 65536:
         outer, inner = int(np.prod(shape[:ax], dtype=np.int64)), int(np.prod(shape[ax + 1:], dtype=np.int64))
         one_pass = gpu.dali_hip_softmax_axis_supported(outer, shape[ax], inner) == 1
