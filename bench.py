@@ -622,8 +622,34 @@ def main():
             nb = 4.0 * 7 * 9999999
             rows_few[tag] = {"us": round(us, 2), "GB/s": round(nb / us / 1e3, 1), "frac_hbm": round(nb / us / 1e3 / HBM_PEAK_GBS, 4), "launches": rec.launches}
             del rec
+        # maps over the same rows that need row statistics first (bytes = one read and one write)
+        few_t = D.Array.from_numpy(np.random.RandomState(20).randint(0, 9999999, 7).astype(np.int32))
+        for tag, build in (("softmax", lambda: op.softmax(few)), ("cross_entropy_gradient", lambda: op.softmax_cross_entropy(few, few_t)[2]),
+                           ("minus_row_means", lambda: few - op.mean(few, [1], True))):
+            with D.Recording() as rec:
+                build().eval()
+            us = time_recording(rec, 10)
+            nb = 2 * 4.0 * 7 * 9999999
+            rows_few[tag] = {"us": round(us, 2), "GB/s": round(nb / us / 1e3, 1), "frac_hbm": round(nb / us / 1e3 / HBM_PEAK_GBS, 4), "launches": rec.launches}
+            del rec
         nxt["reductions_few_long_rows_7x9999999"] = rows_few
-        del few
+        del few, few_t
+        # a tall narrow matrix whose row count has no divisor to go by: column sums, a bias added, columns standardised,
+        # a cumsum along its rows of seven (bytes = one read, plus one write for the maps)
+        tall = D.Array.from_numpy(np.random.RandomState(21).randn(9999999, 7).astype(np.float32))
+        tall_b = D.Array.from_numpy(np.random.RandomState(22).randn(1, 7).astype(np.float32))
+        rows_tall = {}
+        for tag, passes, build in (("sum_axis0", 1, lambda: op.sum(tall, [0])), ("plus_bias", 2, lambda: tall + tall_b),
+                                   ("minus_column_means", 2, lambda: tall - op.mean(tall, [0], True)), ("softmax_axis0", 2, lambda: op.softmax(tall, 0)),
+                                   ("cumsum_axis1", 2, lambda: op.cumsum(tall))):
+            with D.Recording() as rec:
+                build().eval()
+            us = time_recording(rec, 10)
+            nb = passes * 4.0 * 7 * 9999999
+            rows_tall[tag] = {"us": round(us, 2), "GB/s": round(nb / us / 1e3, 1), "frac_hbm": round(nb / us / 1e3 / HBM_PEAK_GBS, 4), "launches": rec.launches}
+            del rec
+        nxt["tall_narrow_9999999x7"] = rows_tall
+        del tall, tall_b
         # a matrix times a column: the rows streamed once
         mv_a = D.Array.from_numpy(np.random.RandomState(20).randn(4096, 4096).astype(np.float32))
         mv_x = D.Array.from_numpy(np.random.RandomState(21).randn(4096, 1).astype(np.float32))
